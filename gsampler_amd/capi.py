@@ -1,0 +1,218 @@
+"""ctypes binding of the C ABI declared in include/gsampler_hip.h.
+
+Two layers:
+
+* ``lib()`` returns the loaded ``libgsampler_hip.so`` with argument types set,
+  one attribute per exported symbol.  Loading fails loudly when the library has
+  not been built -- there is no fallback path.
+* thin helpers (``col_count``, ``col_slice``, ``sample_uniform``,
+  ``unique_relabel`` ...) that take CUDA ``torch.Tensor`` arguments, allocate
+  outputs and workspaces with torch (plumbing only) and launch on torch's
+  current HIP stream.  They are what the tests and the benchmark call; the
+  C++ operator library (``libgs.so``) binds the same symbols directly.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+from typing import Optional, Tuple
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "lib", "libgsampler_hip.so")
+
+GS_OK = 0
+ALGO_AUTO, ALGO_RESERVOIR, ALGO_FLOYD = 0, 1, 2
+
+_i64 = C.c_int64
+_u64 = C.c_uint64
+_p = C.c_void_p
+_sz = C.c_size_t
+_int = C.c_int
+
+# name -> (restype, argtypes); the single source of truth for the loader and
+# for the "every declared symbol is exported" test.
+SIGNATURES = {
+    "gs_last_error": (C.c_char_p, []),
+    "gs_abi_version": (_int, []),
+    "gs_scan_workspace_bytes": (_sz, [_i64]),
+    "gs_exclusive_scan_i64": (_int, [_p, _p, _i64, _p, _sz, _p]),
+    "gs_csc_col_count": (_int, [_p, _i64, _p, _i64, _i64, _int, _p, _p, _sz, _p]),
+    "gs_csc_col_slice_fill": (_int, [_p, _i64, _p, _p, _i64, _p, _i64, _p, _i64,
+                                     _i64, _p, _p, _p, _p]),
+    "gs_csc_col_sample_uniform_fill": (_int, [_p, _i64, _p, _p, _i64, _i64, _int,
+                                              _int, _u64, _u64, _p, _p, _p, _p,
+                                              _p]),
+    "gs_unique_workspace_bytes": (_sz, [_i64, _i64, _i64]),
+    "gs_unique_count": (_int, [_p, _p, _i64, _p, _p, _i64, _i64, _p, _p, _sz, _p]),
+    "gs_unique_fill": (_int, [_p, _p, _i64, _p, _p, _i64, _i64, _p, _p, _p, _p,
+                              _p, _p, _sz, _p]),
+}
+
+_lib = None
+
+
+class GsError(RuntimeError):
+    pass
+
+
+def lib() -> C.CDLL:
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise GsError(
+                f"{LIB_PATH} is missing: build it with "
+                "`make -C gsampler_amd/csrc` (or __graft_entry__.build())")
+        l = C.CDLL(LIB_PATH)
+        for name, (res, args) in SIGNATURES.items():
+            fn = getattr(l, name)
+            fn.restype = res
+            fn.argtypes = args
+        _lib = l
+    return _lib
+
+
+def check(rc: int) -> None:
+    if rc != GS_OK:
+        raise GsError(f"gsampler_hip error {rc}: {lib().gs_last_error().decode()}")
+
+
+# --------------------------------------------------------------- plumbing
+def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
+    if t is None:
+        return None
+    return t.data_ptr() if t.numel() > 0 else None
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _i64t(t: torch.Tensor, name: str) -> torch.Tensor:
+    if t.dtype != torch.int64 or not t.is_cuda:
+        raise GsError(f"{name} must be a CUDA int64 tensor, got {t.dtype} on {t.device}")
+    return t.contiguous()
+
+
+def _workspace(nbytes: int, device) -> torch.Tensor:
+    return torch.empty(max(int(nbytes), 1), dtype=torch.uint8, device=device)
+
+
+# ---------------------------------------------------------------- helpers
+def exclusive_scan(x: torch.Tensor) -> torch.Tensor:
+    x = _i64t(x, "x")
+    out = torch.empty_like(x)
+    n = x.numel()
+    ws = _workspace(lib().gs_scan_workspace_bytes(n), x.device)
+    check(lib().gs_exclusive_scan_i64(_ptr(x), _ptr(out), n, ws.data_ptr(),
+                                      ws.numel(), _stream()))
+    return out
+
+
+def col_count(indptr: torch.Tensor, column_ids: Optional[torch.Tensor],
+              fanout: int, replace: bool,
+              num_items: Optional[int] = None) -> torch.Tensor:
+    """sub_indptr[num_items + 1] for slicing (fanout < 0) or sampling."""
+    indptr = _i64t(indptr, "indptr")
+    num_cols = indptr.numel() - 1
+    if column_ids is not None:
+        column_ids = _i64t(column_ids, "column_ids")
+        num_items = column_ids.numel()
+    elif num_items is None:
+        num_items = num_cols
+    sub_indptr = torch.empty(num_items + 1, dtype=torch.int64, device=indptr.device)
+    ws = _workspace(lib().gs_scan_workspace_bytes(num_items + 1), indptr.device)
+    check(lib().gs_csc_col_count(_ptr(indptr), num_cols, _ptr(column_ids),
+                                 num_items, fanout, int(replace),
+                                 sub_indptr.data_ptr(), ws.data_ptr(), ws.numel(),
+                                 _stream()))
+    return sub_indptr
+
+
+def col_slice(indptr, indices, column_ids, with_coo=True, batch_ptr=None,
+              encode_stride=0):
+    """A[:, column_ids] -> (sub_indptr, coo_col | None, sub_indices, select_index)."""
+    indptr, indices = _i64t(indptr, "indptr"), _i64t(indices, "indices")
+    column_ids = _i64t(column_ids, "column_ids")
+    num_cols = indptr.numel() - 1
+    n = column_ids.numel()
+    sub_indptr = col_count(indptr, column_ids, -1, False)
+    nnz = int(sub_indptr[-1].item())
+    dev = indptr.device
+    out_idx = torch.empty(nnz, dtype=torch.int64, device=dev)
+    out_sel = torch.empty(nnz, dtype=torch.int64, device=dev)
+    out_col = torch.empty(nnz, dtype=torch.int64, device=dev) if with_coo else None
+    nb = 0
+    if batch_ptr is not None:
+        batch_ptr = _i64t(batch_ptr, "batch_ptr")
+        nb = batch_ptr.numel() - 1
+    check(lib().gs_csc_col_slice_fill(_ptr(indptr), num_cols, _ptr(indices),
+                                      _ptr(column_ids), n, sub_indptr.data_ptr(),
+                                      nnz, _ptr(batch_ptr), nb, encode_stride,
+                                      _ptr(out_col), _ptr(out_idx), _ptr(out_sel),
+                                      _stream()))
+    return sub_indptr, out_col, out_idx, out_sel
+
+
+def sample_uniform(indptr, indices, column_ids, fanout, replace=False,
+                   algo=ALGO_AUTO, seed=7777, call_id=0, with_coo=True):
+    """Uniform per-column sampling, fused with the slice when column_ids is given.
+
+    -> (sub_indptr, coo_col | None, sub_indices, select_index)
+    """
+    indptr, indices = _i64t(indptr, "indptr"), _i64t(indices, "indices")
+    num_cols = indptr.numel() - 1
+    if column_ids is not None:
+        column_ids = _i64t(column_ids, "column_ids")
+        n = column_ids.numel()
+    else:
+        n = num_cols
+    sub_indptr = col_count(indptr, column_ids, fanout, replace, n)
+    nnz = int(sub_indptr[-1].item())
+    dev = indptr.device
+    out_idx = torch.empty(nnz, dtype=torch.int64, device=dev)
+    out_sel = torch.empty(nnz, dtype=torch.int64, device=dev)
+    out_col = torch.empty(nnz, dtype=torch.int64, device=dev) if with_coo else None
+    if nnz > 0:
+        check(lib().gs_csc_col_sample_uniform_fill(
+            _ptr(indptr), num_cols, _ptr(indices), _ptr(column_ids), n, fanout,
+            int(replace), algo, seed, call_id, sub_indptr.data_ptr(),
+            _ptr(out_col), out_idx.data_ptr(), out_sel.data_ptr(), _stream()))
+    return sub_indptr, out_col, out_idx, out_sel
+
+
+def unique_relabel(seeds, rows, seeds_ptr=None, rows_ptr=None, edge_col=None,
+                   want_row=True, want_col=True):
+    """First-occurrence unique of seeds_b ++ rows_b per batch, plus relabel.
+
+    -> (unique, unique_ptr, out_row | None, out_col | None)
+    """
+    seeds, rows = _i64t(seeds, "seeds"), _i64t(rows, "rows")
+    dev = seeds.device
+    S, E = seeds.numel(), rows.numel()
+    if seeds_ptr is not None:
+        seeds_ptr, rows_ptr = _i64t(seeds_ptr, "seeds_ptr"), _i64t(rows_ptr, "rows_ptr")
+        B = seeds_ptr.numel() - 1
+    else:
+        B = 1
+    l = lib()
+    ws = _workspace(l.gs_unique_workspace_bytes(S, E, B), dev)
+    unique_ptr = torch.empty(B + 1, dtype=torch.int64, device=dev)
+    sp = seeds_ptr.data_ptr() if seeds_ptr is not None else None
+    rp = rows_ptr.data_ptr() if rows_ptr is not None else None
+    check(l.gs_unique_count(_ptr(seeds), sp, S, _ptr(rows), rp, E, B,
+                            unique_ptr.data_ptr(), ws.data_ptr(), ws.numel(),
+                            _stream()))
+    U = int(unique_ptr[-1].item())
+    unique = torch.empty(U, dtype=torch.int64, device=dev)
+    want_col = want_col and edge_col is not None
+    out_row = torch.empty(E, dtype=torch.int64, device=dev) if want_row else None
+    out_col = torch.empty(E, dtype=torch.int64, device=dev) if want_col else None
+    if edge_col is not None:
+        edge_col = _i64t(edge_col, "edge_col")
+    check(l.gs_unique_fill(_ptr(seeds), sp, S, _ptr(rows), rp, E, B,
+                           unique_ptr.data_ptr(), _ptr(edge_col), _ptr(unique),
+                           _ptr(out_row), _ptr(out_col), ws.data_ptr(), ws.numel(),
+                           _stream()))
+    return unique, unique_ptr, out_row, out_col

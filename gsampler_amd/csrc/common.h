@@ -1,0 +1,167 @@
+// common.h -- shared device/host helpers for the gfx950 sampling kernels.
+// wave64 everywhere: a wavefront is 64 lanes, sub-wave "groups" are power-of-two
+// slices of one wavefront.
+#ifndef GSAMPLER_CSRC_COMMON_H_
+#define GSAMPLER_CSRC_COMMON_H_
+
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+
+#include "../../include/gsampler_hip.h"
+
+namespace gs {
+
+// ------------------------------------------------------------ error plumbing
+void set_error(const char* fmt, ...);
+int hip_fail(hipError_t e, const char* what, const char* file, int line);
+
+#define GS_REQUIRE(cond, ...)     \
+  do {                            \
+    if (!(cond)) {                \
+      gs::set_error(__VA_ARGS__); \
+      return GS_ERR_INVALID;      \
+    }                             \
+  } while (0)
+
+#define GS_HIP(expr)                                                    \
+  do {                                                                  \
+    hipError_t e__ = (expr);                                            \
+    if (e__ != hipSuccess) return gs::hip_fail(e__, #expr, __FILE__, __LINE__); \
+  } while (0)
+
+// Call right after a kernel launch.
+#define GS_LAUNCH_CHECK() GS_HIP(hipGetLastError())
+
+inline hipStream_t as_stream(gs_stream_t s) { return (hipStream_t)s; }
+
+constexpr int kWave = 64;
+constexpr int kBlock = 256;  // 4 waves; the default block for flat kernels
+
+inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
+inline size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
+
+// Carves aligned sub-buffers out of a caller-supplied workspace.
+struct Carver {
+  char* base;
+  size_t used;
+  explicit Carver(void* p) : base((char*)p), used(0) {}
+  template <typename T>
+  T* take(size_t count) {
+    used = align_up(used, 256);
+    T* r = (T*)(base ? base + used : nullptr);
+    used += count * sizeof(T);
+    return r;
+  }
+  size_t total() const { return align_up(used, 256); }
+};
+
+// ------------------------------------------------------------------- Philox
+// Philox4x32-10 (Salmon et al., SC'11).  One call yields four 32-bit words.
+struct PhiloxKey {
+  uint32_t k0, k1;
+};
+
+__host__ __device__ inline PhiloxKey make_key(uint64_t seed, uint64_t call_id) {
+  uint64_t k = seed + call_id * 0x9E3779B97F4A7C15ull;
+  PhiloxKey r;
+  r.k0 = (uint32_t)k;
+  r.k1 = (uint32_t)(k >> 32);
+  return r;
+}
+
+struct Words4 {
+  uint32_t x, y, z, w;
+};
+
+__device__ __forceinline__ Words4 philox(PhiloxKey key, uint64_t pos,
+                                         uint64_t draw) {
+  uint32_t c0 = (uint32_t)draw, c1 = (uint32_t)(draw >> 32);
+  uint32_t c2 = (uint32_t)pos, c3 = (uint32_t)(pos >> 32);
+  uint32_t k0 = key.k0, k1 = key.k1;
+#pragma unroll
+  for (int r = 0; r < 10; ++r) {
+    uint32_t hi0 = __umulhi(0xD2511F53u, c0), lo0 = 0xD2511F53u * c0;
+    uint32_t hi1 = __umulhi(0xCD9E8D57u, c2), lo1 = 0xCD9E8D57u * c2;
+    c0 = hi1 ^ c1 ^ k0;
+    c1 = lo1;
+    c2 = hi0 ^ c3 ^ k1;
+    c3 = lo0;
+    k0 += 0x9E3779B9u;
+    k1 += 0xBB67AE85u;
+  }
+  return Words4{c0, c1, c2, c3};
+}
+
+// Integer in [0, n): floor(r64 * n / 2^64) with r64 = w1:w0.
+__device__ __forceinline__ uint64_t philox_bounded(PhiloxKey key, uint64_t pos,
+                                                   uint64_t draw, uint64_t n) {
+  Words4 w = philox(key, pos, draw);
+  uint64_t r = ((uint64_t)w.y << 32) | w.x;
+  return __umul64hi(r, n);
+}
+
+// ------------------------------------------------------------- wave helpers
+__device__ __forceinline__ int lane_id() { return (int)__lane_id(); }
+
+// Inclusive scan across the 64 lanes of a wavefront.
+template <typename T>
+__device__ __forceinline__ T wave_inclusive_sum(T v) {
+#pragma unroll
+  for (int d = 1; d < kWave; d <<= 1) {
+    T o = __shfl_up(v, d, kWave);
+    if (lane_id() >= d) v += o;
+  }
+  return v;
+}
+
+// Exclusive block scan for blocks of kBlock threads.  `total` receives the
+// block sum in every thread.  smem must hold kBlock / kWave + 1 elements.
+template <typename T>
+__device__ __forceinline__ T block_exclusive_sum(T v, T* smem, T* total) {
+  const int wave = threadIdx.x / kWave;
+  T inc = wave_inclusive_sum(v);
+  if (lane_id() == kWave - 1) smem[wave] = inc;
+  __syncthreads();
+  T base = 0, sum = 0;
+#pragma unroll
+  for (int w = 0; w < kBlock / kWave; ++w) {
+    T s = smem[w];
+    if (w < wave) base += s;
+    sum += s;
+  }
+  __syncthreads();
+  *total = sum;
+  return base + inc - v;
+}
+
+// Largest b in [0, n) with ptr[b] <= x, for a non-decreasing ptr[0..n] whose
+// first element is <= x (segment lookup in a [n+1] offsets array).
+__device__ __forceinline__ int64_t segment_of(const int64_t* ptr, int64_t n,
+                                              int64_t x) {
+  int64_t lo = 0, hi = n;  // answer in [lo, hi)
+  while (hi - lo > 1) {
+    int64_t mid = (lo + hi) >> 1;
+    if (ptr[mid] <= x)
+      lo = mid;
+    else
+      hi = mid;
+  }
+  return lo;
+}
+
+__device__ __forceinline__ int64_t column_degree(const int64_t* indptr,
+                                                 int64_t num_cols, int64_t c,
+                                                 int64_t* in_start) {
+  if (c < 0 || c >= num_cols) {
+    *in_start = 0;
+    return 0;
+  }
+  int64_t b = indptr[c];
+  *in_start = b;
+  return indptr[c + 1] - b;
+}
+
+}  // namespace gs
+
+#endif  // GSAMPLER_CSRC_COMMON_H_

@@ -1,0 +1,131 @@
+// core.hip -- error plumbing and the device-wide exclusive scan.
+#include <cstdarg>
+#include <cstdio>
+#include <string>
+
+#include "common.h"
+#include "scan.h"
+
+namespace gs {
+
+static thread_local std::string g_last_error;
+
+void set_error(const char* fmt, ...) {
+  char buf[512];
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(buf, sizeof(buf), fmt, ap);
+  va_end(ap);
+  g_last_error = buf;
+}
+
+int hip_fail(hipError_t e, const char* what, const char* file, int line) {
+  set_error("HIP error %d (%s) at %s:%d in %s", (int)e, hipGetErrorString(e),
+            file, line, what);
+  return GS_ERR_HIP;
+}
+
+// ------------------------------------------------------------------ scan
+// Three launches: per-tile sums, a single-block scan of the tile sums, and a
+// per-tile down-sweep.  A tile is kBlock threads x kScanItems consecutive
+// values per thread, so global accesses stay coalesced per thread-vector.
+
+__global__ __launch_bounds__(kBlock) void scan_tile_sums_kernel(
+    const int64_t* __restrict__ in, int64_t n, int64_t* __restrict__ tile_sums) {
+  __shared__ int64_t smem[kBlock / kWave + 1];
+  const int64_t base = (int64_t)blockIdx.x * kScanTile + threadIdx.x * kScanItems;
+  int64_t s = 0;
+#pragma unroll
+  for (int k = 0; k < kScanItems; ++k) {
+    int64_t i = base + k;
+    if (i < n) s += in[i];
+  }
+  int64_t total;
+  block_exclusive_sum(s, smem, &total);
+  if (threadIdx.x == 0) tile_sums[blockIdx.x] = total;
+}
+
+// One block scans `num_tiles` values in place (exclusive), chunk by chunk.
+__global__ __launch_bounds__(kBlock) void scan_spine_kernel(int64_t* tile_sums,
+                                                            int64_t num_tiles) {
+  __shared__ int64_t smem[kBlock / kWave + 1];
+  int64_t carry = 0;
+  for (int64_t start = 0; start < num_tiles; start += kBlock) {
+    int64_t i = start + threadIdx.x;
+    int64_t v = i < num_tiles ? tile_sums[i] : 0;
+    int64_t total;
+    int64_t ex = block_exclusive_sum(v, smem, &total);
+    if (i < num_tiles) tile_sums[i] = carry + ex;
+    carry += total;
+  }
+}
+
+__global__ __launch_bounds__(kBlock) void scan_down_kernel(
+    const int64_t* in, int64_t* out, int64_t n,
+    const int64_t* __restrict__ tile_sums) {
+  __shared__ int64_t smem[kBlock / kWave + 1];
+  const int64_t base = (int64_t)blockIdx.x * kScanTile + threadIdx.x * kScanItems;
+  int64_t v[kScanItems];
+  int64_t s = 0;
+#pragma unroll
+  for (int k = 0; k < kScanItems; ++k) {
+    int64_t i = base + k;
+    v[k] = i < n ? in[i] : 0;
+    s += v[k];
+  }
+  int64_t total;
+  int64_t ex = block_exclusive_sum(s, smem, &total) + tile_sums[blockIdx.x];
+#pragma unroll
+  for (int k = 0; k < kScanItems; ++k) {
+    int64_t i = base + k;
+    if (i < n) out[i] = ex;
+    ex += v[k];
+  }
+}
+
+size_t scan_workspace_bytes(int64_t n) {
+  int64_t tiles = n > 0 ? ceil_div(n, kScanTile) : 1;
+  return align_up((size_t)tiles * sizeof(int64_t), 256);
+}
+
+int exclusive_scan_i64(const int64_t* in, int64_t* out, int64_t n, void* ws,
+                       size_t ws_bytes, hipStream_t stream) {
+  if (n <= 0) return GS_OK;
+  if (ws_bytes < scan_workspace_bytes(n) || ws == nullptr) {
+    set_error("scan workspace too small: %zu < %zu", ws_bytes,
+              scan_workspace_bytes(n));
+    return GS_ERR_WORKSPACE;
+  }
+  int64_t* tile_sums = (int64_t*)ws;
+  const int64_t tiles = ceil_div(n, kScanTile);
+  scan_tile_sums_kernel<<<dim3((unsigned)tiles), dim3(kBlock), 0, stream>>>(
+      in, n, tile_sums);
+  GS_LAUNCH_CHECK();
+  scan_spine_kernel<<<dim3(1), dim3(kBlock), 0, stream>>>(tile_sums, tiles);
+  GS_LAUNCH_CHECK();
+  scan_down_kernel<<<dim3((unsigned)tiles), dim3(kBlock), 0, stream>>>(
+      in, out, n, tile_sums);
+  GS_LAUNCH_CHECK();
+  return GS_OK;
+}
+
+}  // namespace gs
+
+extern "C" {
+
+const char* gs_last_error(void) { return gs::g_last_error.c_str(); }
+
+int gs_abi_version(void) { return 1; }
+
+size_t gs_scan_workspace_bytes(int64_t n) { return gs::scan_workspace_bytes(n); }
+
+int gs_exclusive_scan_i64(const int64_t* in, int64_t* out, int64_t n,
+                          void* workspace, size_t workspace_bytes,
+                          gs_stream_t stream) {
+  GS_REQUIRE(n >= 0, "scan: negative length %lld", (long long)n);
+  GS_REQUIRE(n == 0 || (in && out), "scan: null pointer");
+  return gs::exclusive_scan_i64(in, out, n, workspace, workspace_bytes,
+                                gs::as_stream(stream));
+}
+
+}  // extern "C"

@@ -1,0 +1,170 @@
+// sampling.hip -- uniform per-column sampling, optionally fused with the
+// column slice (the GraphSAGE kernel).
+//
+// Work mapping: a group of G lanes (G a power of two <= 64, a slice of one
+// wavefront) owns one requested column; a wavefront therefore keeps 64 / G
+// independent columns -- and their dependent seed -> indptr -> indices load
+// chains -- in flight at once.  Group-level exchange uses wavefront shuffles
+// only, so divergent columns never meet at a block barrier.
+#include "common.h"
+
+namespace gs {
+
+// Reads a value that other lanes may have updated with an atomic, bypassing
+// the per-CU vector cache.
+__device__ __forceinline__ int64_t load_coherent(const int64_t* p) {
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+template <int G>
+__global__ __launch_bounds__(kBlock) void sample_uniform_kernel(
+    const int64_t* __restrict__ indptr, int64_t num_cols,
+    const int64_t* __restrict__ indices, const int64_t* __restrict__ column_ids,
+    int64_t num_items, int64_t fanout, int replace, int algo, PhiloxKey key,
+    const int64_t* __restrict__ sub_indptr, int64_t* __restrict__ out_coo_col,
+    int64_t* __restrict__ out_indices, int64_t* __restrict__ out_select) {
+  const int lane = threadIdx.x & (G - 1);
+  const int64_t item =
+      ((int64_t)blockIdx.x * kBlock + threadIdx.x) / G;
+  if (item >= num_items) return;  // whole groups leave together
+
+  const int64_t c = column_ids ? column_ids[item] : item;
+  int64_t in_start;
+  const int64_t deg = column_degree(indptr, num_cols, c, &in_start);
+  if (deg == 0) return;
+  const int64_t out_start = sub_indptr[item];
+  const uint64_t pos = (uint64_t)item;
+
+  if (replace) {
+    // slot j takes a uniform position of the column
+    for (int64_t j = lane; j < fanout; j += G) {
+      int64_t p = in_start + (int64_t)philox_bounded(key, pos, (uint64_t)j,
+                                                      (uint64_t)deg);
+      out_indices[out_start + j] = indices[p];
+      out_select[out_start + j] = p;
+      if (out_coo_col) out_coo_col[out_start + j] = item;
+    }
+    return;
+  }
+
+  if (deg <= fanout) {
+    // the whole column, original order
+    for (int64_t j = lane; j < deg; j += G) {
+      int64_t p = in_start + j;
+      out_indices[out_start + j] = indices[p];
+      out_select[out_start + j] = p;
+      if (out_coo_col) out_coo_col[out_start + j] = item;
+    }
+    return;
+  }
+
+  if (algo == GS_ALGO_FLOYD) {
+    // Floyd's subset sampling, one lane per output slot (fanout <= G).
+    // Slot i draws t_i in [0, j_i], j_i = deg - fanout + i, and keeps t_i
+    // unless an earlier slot already holds it, in which case it keeps j_i.
+    // "Already held" <=> some earlier slot drew the same t, or t_i equals the
+    // j_m of an earlier slot m that fell back to j_m; m is then unique
+    // (m = t_i - (deg - fanout)), so the fall-back flags form a chain that is
+    // settled by visiting slots in increasing order.
+    const int K = (int)fanout;
+    const bool active = lane < K;
+    const int64_t base = deg - fanout;
+    const int64_t j = base + lane;
+    int64_t t = -1;
+    if (active)
+      t = (int64_t)philox_bounded(key, pos, (uint64_t)lane, (uint64_t)j + 1);
+    bool dup = false;
+    for (int m = 0; m < K; ++m) {
+      int64_t tm = __shfl(t, m, G);
+      dup |= (m < lane) & (tm == t);
+    }
+    const int64_t mi = t - base;  // slot whose j equals my t, if in [0, lane)
+    for (int m = 0; m < K; ++m) {
+      int dm = __shfl((int)dup, m, G);
+      if (mi == m && m < lane) dup |= (dm != 0);
+    }
+    if (active) {
+      int64_t p = in_start + (dup ? j : t);
+      out_indices[out_start + lane] = indices[p];
+      out_select[out_start + lane] = p;
+      if (out_coo_col) out_coo_col[out_start + lane] = item;
+    }
+    return;
+  }
+
+  // Reservoir (Algorithm R in max-form): slot[j] = j, then every idx in
+  // [fanout, deg) draws num in [0, idx]; if num < fanout the slot keeps the
+  // largest idx that hit it.  The slots live in out_select until the final
+  // gather.  Order-independent, so lanes take idx values strided by G.
+  for (int64_t jj = lane; jj < fanout; jj += G) out_select[out_start + jj] = jj;
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+  __builtin_amdgcn_wave_barrier();
+  for (int64_t idx = fanout + lane; idx < deg; idx += G) {
+    int64_t num = (int64_t)philox_bounded(key, pos, (uint64_t)idx,
+                                          (uint64_t)idx + 1);
+    if (num < fanout)
+      atomicMax((long long*)(out_select + out_start + num), (long long)idx);
+  }
+  __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "agent");
+  __builtin_amdgcn_wave_barrier();
+  for (int64_t jj = lane; jj < fanout; jj += G) {
+    int64_t p = in_start + load_coherent(out_select + out_start + jj);
+    out_indices[out_start + jj] = indices[p];
+    out_select[out_start + jj] = p;
+    if (out_coo_col) out_coo_col[out_start + jj] = item;
+  }
+}
+
+template <int G>
+static int launch_sample_uniform(const int64_t* indptr, int64_t num_cols,
+                                 const int64_t* indices,
+                                 const int64_t* column_ids, int64_t num_items,
+                                 int64_t fanout, int replace, int algo,
+                                 PhiloxKey key, const int64_t* sub_indptr,
+                                 int64_t* out_coo_col, int64_t* out_indices,
+                                 int64_t* out_select, hipStream_t stream) {
+  const int64_t blocks = ceil_div(num_items * G, kBlock);
+  sample_uniform_kernel<G><<<dim3((unsigned)blocks), dim3(kBlock), 0, stream>>>(
+      indptr, num_cols, indices, column_ids, num_items, fanout, replace, algo,
+      key, sub_indptr, out_coo_col, out_indices, out_select);
+  GS_LAUNCH_CHECK();
+  return GS_OK;
+}
+
+}  // namespace gs
+
+extern "C" int gs_csc_col_sample_uniform_fill(
+    const int64_t* indptr, int64_t num_cols, const int64_t* indices,
+    const int64_t* column_ids, int64_t num_items, int64_t fanout, int replace,
+    int algo, uint64_t seed, uint64_t call_id, const int64_t* sub_indptr,
+    int64_t* out_coo_col, int64_t* out_indices, int64_t* out_select,
+    gs_stream_t stream) {
+  using namespace gs;
+  GS_REQUIRE(num_items >= 0 && num_cols >= 0, "sample_uniform: negative size");
+  GS_REQUIRE(fanout >= 0, "sample_uniform: negative fanout %lld",
+             (long long)fanout);
+  GS_REQUIRE(algo == GS_ALGO_AUTO || algo == GS_ALGO_RESERVOIR ||
+                 algo == GS_ALGO_FLOYD,
+             "sample_uniform: unknown algorithm %d", algo);
+  GS_REQUIRE(!(algo == GS_ALGO_FLOYD && fanout > 64),
+             "sample_uniform: Floyd sampling needs fanout <= 64, got %lld",
+             (long long)fanout);
+  if (num_items == 0 || fanout == 0) return GS_OK;
+  GS_REQUIRE(indptr && indices && sub_indptr && out_indices && out_select,
+             "sample_uniform: null pointer");
+  GS_REQUIRE(column_ids != nullptr || num_items <= num_cols,
+             "sample_uniform: %lld items but the matrix has %lld columns",
+             (long long)num_items, (long long)num_cols);
+  if (algo == GS_ALGO_AUTO)
+    algo = fanout <= 64 ? GS_ALGO_FLOYD : GS_ALGO_RESERVOIR;
+  const PhiloxKey key = make_key(seed, call_id);
+  hipStream_t s = as_stream(stream);
+#define GS_SAMPLE_ARGS                                                    \
+  indptr, num_cols, indices, column_ids, num_items, fanout, replace, algo, \
+      key, sub_indptr, out_coo_col, out_indices, out_select, s
+  if (fanout <= 8) return launch_sample_uniform<8>(GS_SAMPLE_ARGS);
+  if (fanout <= 16) return launch_sample_uniform<16>(GS_SAMPLE_ARGS);
+  if (fanout <= 32) return launch_sample_uniform<32>(GS_SAMPLE_ARGS);
+  return launch_sample_uniform<64>(GS_SAMPLE_ARGS);
+#undef GS_SAMPLE_ARGS
+}

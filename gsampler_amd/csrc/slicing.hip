@@ -1,0 +1,103 @@
+// slicing.hip -- per-column counts and the CSC column slice.
+#include "common.h"
+#include "scan.h"
+
+namespace gs {
+
+// One thread per requested column: writes its output count; the scan that
+// follows turns the counts into sub_indptr in place.
+__global__ __launch_bounds__(kBlock) void col_count_kernel(
+    const int64_t* __restrict__ indptr, int64_t num_cols,
+    const int64_t* __restrict__ column_ids, int64_t num_items, int64_t fanout,
+    int replace, int64_t* __restrict__ counts) {
+  const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (i > num_items) return;
+  int64_t cnt = 0;
+  if (i < num_items) {
+    int64_t c = column_ids ? column_ids[i] : i;
+    int64_t in_start;
+    int64_t deg = column_degree(indptr, num_cols, c, &in_start);
+    if (fanout < 0)
+      cnt = deg;
+    else if (replace)
+      cnt = deg == 0 ? 0 : fanout;
+    else
+      cnt = deg < fanout ? deg : fanout;
+  }
+  counts[i] = cnt;  // counts[num_items] = 0 so the scan leaves the total there
+}
+
+// Edge-parallel slice: thread e owns output edge e, finds its column by binary
+// search in sub_indptr (L2-resident) and copies one row id.  Load balance is
+// independent of the degree distribution; reads within a column and all
+// writes are coalesced.
+__global__ __launch_bounds__(kBlock) void col_slice_fill_kernel(
+    const int64_t* __restrict__ indptr, int64_t num_cols,
+    const int64_t* __restrict__ indices, const int64_t* __restrict__ column_ids,
+    int64_t num_items, const int64_t* __restrict__ sub_indptr, int64_t nnz,
+    const int64_t* __restrict__ batch_ptr, int64_t num_batches,
+    int64_t encode_stride, int64_t* __restrict__ out_coo_col,
+    int64_t* __restrict__ out_indices, int64_t* __restrict__ out_select) {
+  const int64_t e = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (e >= nnz) return;
+  const int64_t item = segment_of(sub_indptr, num_items, e);
+  const int64_t c = column_ids ? column_ids[item] : item;
+  const int64_t in_pos = indptr[c] + (e - sub_indptr[item]);
+  int64_t row = indices[in_pos];
+  if (batch_ptr != nullptr && encode_stride > 0)
+    row += segment_of(batch_ptr, num_batches, item) * encode_stride;
+  out_indices[e] = row;
+  out_select[e] = in_pos;
+  if (out_coo_col) out_coo_col[e] = item;
+}
+
+}  // namespace gs
+
+extern "C" {
+
+int gs_csc_col_count(const int64_t* indptr, int64_t num_cols,
+                     const int64_t* column_ids, int64_t num_items,
+                     int64_t fanout, int replace, int64_t* sub_indptr,
+                     void* workspace, size_t workspace_bytes,
+                     gs_stream_t stream) {
+  using namespace gs;
+  GS_REQUIRE(num_items >= 0 && num_cols >= 0, "col_count: negative size");
+  GS_REQUIRE(indptr && sub_indptr, "col_count: null pointer");
+  GS_REQUIRE(column_ids != nullptr || num_items <= num_cols,
+             "col_count: %lld items but the matrix has %lld columns",
+             (long long)num_items, (long long)num_cols);
+  hipStream_t s = as_stream(stream);
+  const int64_t n = num_items + 1;
+  col_count_kernel<<<dim3((unsigned)ceil_div(n, kBlock)), dim3(kBlock), 0, s>>>(
+      indptr, num_cols, column_ids, num_items, fanout, replace, sub_indptr);
+  GS_LAUNCH_CHECK();
+  return exclusive_scan_i64(sub_indptr, sub_indptr, n, workspace,
+                            workspace_bytes, s);
+}
+
+int gs_csc_col_slice_fill(const int64_t* indptr, int64_t num_cols,
+                          const int64_t* indices, const int64_t* column_ids,
+                          int64_t num_items, const int64_t* sub_indptr,
+                          int64_t nnz, const int64_t* batch_ptr,
+                          int64_t num_batches, int64_t encode_stride,
+                          int64_t* out_coo_col, int64_t* out_indices,
+                          int64_t* out_select, gs_stream_t stream) {
+  using namespace gs;
+  GS_REQUIRE(num_items >= 0 && nnz >= 0, "col_slice_fill: negative size");
+  if (nnz == 0 || num_items == 0) return GS_OK;
+  GS_REQUIRE(indptr && indices && sub_indptr && out_indices && out_select,
+             "col_slice_fill: null pointer");
+  GS_REQUIRE(batch_ptr == nullptr || num_batches > 0,
+             "col_slice_fill: batch_ptr given but num_batches = %lld",
+             (long long)num_batches);
+  (void)num_cols;
+  col_slice_fill_kernel<<<dim3((unsigned)ceil_div(nnz, kBlock)), dim3(kBlock), 0,
+                          as_stream(stream)>>>(
+      indptr, num_cols, indices, column_ids, num_items, sub_indptr, nnz,
+      batch_ptr, num_batches, encode_stride, out_coo_col, out_indices,
+      out_select);
+  GS_LAUNCH_CHECK();
+  return GS_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,153 @@
+/*
+ * gsampler_hip.h -- C ABI of the MI355X (gfx950) sampling kernels.
+ *
+ * Every entry point takes raw device pointers, element counts, a HIP stream
+ * (passed as void*, it is a hipStream_t) and returns an int status
+ * (GS_OK == 0).  No entry point allocates device memory: scratch space is a
+ * caller-supplied workspace whose size the matching *_workspace_bytes()
+ * function reports.  All ids, pointers-into-arrays and counts are int64,
+ * all edge weights fp32, exactly as in the reference's tensors.
+ *
+ * Data-dependent output sizes use two phases: a *_count call fills a prefix
+ * array on the device (its last element is the total), the caller reads that
+ * total, allocates the outputs and calls *_fill.
+ *
+ * Random picks are a pure function of (seed, call_id, position of the column
+ * / list element in its input array, draw index): Philox4x32-10 keyed by
+ * seed + call_id * 0x9E3779B97F4A7C15 (mod 2^64), counter
+ * (lo32(draw), hi32(draw), lo32(pos), hi32(pos)).  Launch geometry and
+ * super-batching therefore never change a result.
+ *
+ * Each declaration cites the reference interface it stands in for
+ * (paths relative to the gSampler source tree).
+ */
+#ifndef GSAMPLER_HIP_H_
+#define GSAMPLER_HIP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define GS_OK 0
+#define GS_ERR_INVALID 1     /* bad argument (null pointer, negative size, ...) */
+#define GS_ERR_HIP 2         /* a HIP runtime call failed; see gs_last_error() */
+#define GS_ERR_WORKSPACE 3   /* workspace too small */
+#define GS_ERR_UNSUPPORTED 4 /* valid request this build does not implement */
+
+/* Sampling algorithm for uniform sampling without replacement. */
+#define GS_ALGO_AUTO 0      /* Floyd when fanout <= 64, else reservoir */
+#define GS_ALGO_RESERVOIR 1 /* the reference's Algorithm R in max-form */
+#define GS_ALGO_FLOYD 2     /* Floyd's subset sampling, O(fanout) per column */
+
+typedef void* gs_stream_t;
+
+/* Message of the last error raised on the calling thread ("" if none). */
+const char* gs_last_error(void);
+/* ABI revision; bumped whenever a signature changes. */
+int gs_abi_version(void);
+
+/* ------------------------------------------------------------------------
+ * Exclusive prefix sum of n int64 values, in place allowed (in == out).
+ * Stands in for cub_exclusiveSum, src/cuda/utils.h:18-28.
+ * ---------------------------------------------------------------------- */
+size_t gs_scan_workspace_bytes(int64_t n);
+int gs_exclusive_scan_i64(const int64_t* in, int64_t* out, int64_t n,
+                          void* workspace, size_t workspace_bytes,
+                          gs_stream_t stream);
+
+/* ------------------------------------------------------------------------
+ * Per-column output count + prefix (count phase of slicing and sampling).
+ *   column_ids == NULL : columns 0..num_items-1 of the CSC itself.
+ *   fanout < 0         : whole column (slicing).
+ *   replace            : count = degree == 0 ? 0 : fanout, else min(degree, fanout).
+ * Column ids outside [0, num_cols) count as empty columns.
+ * Writes sub_indptr[num_items + 1]; sub_indptr[num_items] is the edge total.
+ * Stands in for the degree lambda + scan of
+ *   src/cuda/slicing.cu:133-141, src/cuda/sampling.cu:112-124,
+ *   src/cuda/fusion/slice_sampling.cu:111-124, src/cuda/sampling_probs.cu:201-216.
+ * Workspace: gs_scan_workspace_bytes(num_items + 1).
+ * ---------------------------------------------------------------------- */
+int gs_csc_col_count(const int64_t* indptr, int64_t num_cols,
+                     const int64_t* column_ids, int64_t num_items,
+                     int64_t fanout, int replace, int64_t* sub_indptr,
+                     void* workspace, size_t workspace_bytes,
+                     gs_stream_t stream);
+
+/* ------------------------------------------------------------------------
+ * Column slicing A[:, column_ids] (fill phase).
+ *   nnz = sub_indptr[num_items], as read back by the caller.
+ *   out_coo_col   (nullable) : local column id of every output edge.
+ *   out_indices              : global row id of every output edge.
+ *   out_select               : position of the edge in `indices`.
+ *   batch_ptr (nullable)     : [num_batches + 1] offsets into column_ids; with
+ *     encode_stride > 0 the row id of an edge of batch b becomes
+ *     id + b * encode_stride (src/cuda/batch/slicing.cu:25-27).
+ * Stands in for OnIndptrSlicingCUDA (src/cuda/slicing.cu:169-181) and
+ * BatchOnIndptrSlicingCUDA (src/cuda/batch/slicing.cu:100-120).
+ * ---------------------------------------------------------------------- */
+int gs_csc_col_slice_fill(const int64_t* indptr, int64_t num_cols,
+                          const int64_t* indices, const int64_t* column_ids,
+                          int64_t num_items, const int64_t* sub_indptr,
+                          int64_t nnz, const int64_t* batch_ptr,
+                          int64_t num_batches,
+                          int64_t encode_stride, int64_t* out_coo_col,
+                          int64_t* out_indices, int64_t* out_select,
+                          gs_stream_t stream);
+
+/* ------------------------------------------------------------------------
+ * Uniform per-column sampling (fill phase), optionally fused with the column
+ * slice (column_ids != NULL).  sub_indptr comes from gs_csc_col_count with
+ * the same fanout / replace.  Columns with degree <= fanout are copied in
+ * their original order (no replace).  `algo` is one of GS_ALGO_*.
+ * Stands in for CSCColSamplingCUDA (src/cuda/sampling.cu:161-172) and
+ * FusedCSCColSlicingSamplingCUDA (src/cuda/fusion/slice_sampling.cu:164-177).
+ * ---------------------------------------------------------------------- */
+int gs_csc_col_sample_uniform_fill(const int64_t* indptr, int64_t num_cols,
+                                   const int64_t* indices,
+                                   const int64_t* column_ids, int64_t num_items,
+                                   int64_t fanout, int replace, int algo,
+                                   uint64_t seed, uint64_t call_id,
+                                   const int64_t* sub_indptr,
+                                   int64_t* out_coo_col, int64_t* out_indices,
+                                   int64_t* out_select, gs_stream_t stream);
+
+/* ------------------------------------------------------------------------
+ * Unique in first-occurrence order + relabel, for one batch or a super-batch.
+ * For batch b the key sequence is
+ *     seeds[seeds_ptr[b] : seeds_ptr[b+1]] ++ rows[rows_ptr[b] : rows_ptr[b+1]]
+ * (seeds_ptr == rows_ptr == NULL means a single batch holding everything).
+ *
+ * count: builds the per-batch hash tables inside the workspace and writes
+ *   unique_ptr[num_batches + 1] (number of unique keys before each batch;
+ *   the last element is the total U).
+ * fill:  same arguments + the same workspace, untouched in between; writes
+ *   out_unique[U]; out_row[num_rows_keys] = batch-local rank of every row key
+ *   (nullable); out_col[num_rows_keys] = batch-local rank of
+ *   seeds[edge_col[e]] (nullable; edge_col holds positions into `seeds`).
+ * Keys must lie in [0, 2^32 - 2] and one batch may hold at most 2^32 - 2 keys.
+ * Stands in for TensorUniqueCUDA / TensorRelabelCUDA
+ * (src/cuda/unique_reindex.cu:174-199) and BatchCOORelabelCUDA
+ * (src/cuda/batch/batch_relabel.cu:480-498).
+ * ---------------------------------------------------------------------- */
+size_t gs_unique_workspace_bytes(int64_t num_seeds, int64_t num_rows_keys,
+                                 int64_t num_batches);
+int gs_unique_count(const int64_t* seeds, const int64_t* seeds_ptr,
+                    int64_t num_seeds, const int64_t* rows,
+                    const int64_t* rows_ptr, int64_t num_rows_keys,
+                    int64_t num_batches, int64_t* unique_ptr, void* workspace,
+                    size_t workspace_bytes, gs_stream_t stream);
+int gs_unique_fill(const int64_t* seeds, const int64_t* seeds_ptr,
+                   int64_t num_seeds, const int64_t* rows,
+                   const int64_t* rows_ptr, int64_t num_rows_keys,
+                   int64_t num_batches, const int64_t* unique_ptr,
+                   const int64_t* edge_col, int64_t* out_unique,
+                   int64_t* out_row, int64_t* out_col, void* workspace,
+                   size_t workspace_bytes, gs_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* GSAMPLER_HIP_H_ */

@@ -1,0 +1,155 @@
+"""numpy-facing ctypes binding of the CPU oracle (oracle/libgs_oracle.so).
+
+TEST INFRASTRUCTURE ONLY: imported by tests/, __graft_entry__.smoke() and the
+cpu_baseline leg of bench.py.  The shipped package never imports this module.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libgs_oracle.so")
+
+_lib = None
+
+
+def build() -> None:
+    subprocess.check_call(["make", "-C", _HERE, "-s"])
+
+
+def lib() -> C.CDLL:
+    global _lib
+    if _lib is None:
+        src = os.path.join(_HERE, "gs_oracle.cpp")
+        if (not os.path.exists(LIB_PATH)
+                or os.path.getmtime(src) > os.path.getmtime(LIB_PATH)):
+            build()
+        _lib = C.CDLL(LIB_PATH)
+        _lib.gs_num_threads_cpu.restype = C.c_int
+    return _lib
+
+
+def _i64(a) -> np.ndarray:
+    return np.ascontiguousarray(np.asarray(a, dtype=np.int64))
+
+
+def _p(a):
+    if a is None:
+        return None
+    return a.ctypes.data_as(C.c_void_p)
+
+
+def num_threads() -> int:
+    return lib().gs_num_threads_cpu()
+
+
+def philox4x32_10(ctr, key) -> np.ndarray:
+    c = np.asarray(ctr, dtype=np.uint32)
+    k = np.asarray(key, dtype=np.uint32)
+    out = np.zeros(4, dtype=np.uint32)
+    lib().gs_philox4x32_10_cpu(_p(c), _p(k), _p(out))
+    return out
+
+
+def stream_words(seed, call_id, pos, draw) -> np.ndarray:
+    out = np.zeros(4, dtype=np.uint32)
+    lib().gs_stream_words_cpu(C.c_uint64(seed), C.c_uint64(call_id),
+                              C.c_uint64(pos), C.c_uint64(draw), _p(out))
+    return out
+
+
+def exclusive_scan(x) -> np.ndarray:
+    x = _i64(x)
+    out = np.empty_like(x)
+    lib().gs_exclusive_scan_i64_cpu(_p(x), _p(out), C.c_int64(x.size))
+    return out
+
+
+def col_count(indptr, column_ids, fanout, replace, num_items=None) -> np.ndarray:
+    indptr = _i64(indptr)
+    num_cols = indptr.size - 1
+    if column_ids is not None:
+        column_ids = _i64(column_ids)
+        num_items = column_ids.size
+    elif num_items is None:
+        num_items = num_cols
+    out = np.empty(num_items + 1, dtype=np.int64)
+    lib().gs_csc_col_count_cpu(_p(indptr), C.c_int64(num_cols), _p(column_ids),
+                               C.c_int64(num_items), C.c_int64(fanout),
+                               C.c_int(int(replace)), _p(out))
+    return out
+
+
+def col_slice(indptr, indices, column_ids, with_coo=True, batch_ptr=None,
+              encode_stride=0):
+    indptr, indices, column_ids = _i64(indptr), _i64(indices), _i64(column_ids)
+    num_cols = indptr.size - 1
+    n = column_ids.size
+    sub_indptr = col_count(indptr, column_ids, -1, False)
+    nnz = int(sub_indptr[-1])
+    out_idx = np.empty(nnz, dtype=np.int64)
+    out_sel = np.empty(nnz, dtype=np.int64)
+    out_col = np.empty(nnz, dtype=np.int64) if with_coo else None
+    nb = 0
+    if batch_ptr is not None:
+        batch_ptr = _i64(batch_ptr)
+        nb = batch_ptr.size - 1
+    lib().gs_csc_col_slice_fill_cpu(
+        _p(indptr), C.c_int64(num_cols), _p(indices), _p(column_ids),
+        C.c_int64(n), _p(sub_indptr), C.c_int64(nnz), _p(batch_ptr),
+        C.c_int64(nb), C.c_int64(encode_stride), _p(out_col), _p(out_idx),
+        _p(out_sel))
+    return sub_indptr, out_col, out_idx, out_sel
+
+
+def sample_uniform(indptr, indices, column_ids, fanout, replace=False, algo=0,
+                   seed=7777, call_id=0, with_coo=True):
+    indptr, indices = _i64(indptr), _i64(indices)
+    num_cols = indptr.size - 1
+    if column_ids is not None:
+        column_ids = _i64(column_ids)
+        n = column_ids.size
+    else:
+        n = num_cols
+    sub_indptr = col_count(indptr, column_ids, fanout, replace, n)
+    nnz = int(sub_indptr[-1])
+    out_idx = np.empty(nnz, dtype=np.int64)
+    out_sel = np.empty(nnz, dtype=np.int64)
+    out_col = np.empty(nnz, dtype=np.int64) if with_coo else None
+    lib().gs_csc_col_sample_uniform_fill_cpu(
+        _p(indptr), C.c_int64(num_cols), _p(indices), _p(column_ids),
+        C.c_int64(n), C.c_int64(fanout), C.c_int(int(replace)), C.c_int(algo),
+        C.c_uint64(seed), C.c_uint64(call_id), _p(sub_indptr), _p(out_col),
+        _p(out_idx), _p(out_sel))
+    return sub_indptr, out_col, out_idx, out_sel
+
+
+def unique_relabel(seeds, rows, seeds_ptr=None, rows_ptr=None, edge_col=None,
+                   want_row=True, want_col=True):
+    seeds, rows = _i64(seeds), _i64(rows)
+    S, E = seeds.size, rows.size
+    if seeds_ptr is not None:
+        seeds_ptr, rows_ptr = _i64(seeds_ptr), _i64(rows_ptr)
+        B = seeds_ptr.size - 1
+    else:
+        B = 1
+    unique_ptr = np.empty(B + 1, dtype=np.int64)
+    lib().gs_unique_count_cpu(_p(seeds), _p(seeds_ptr), C.c_int64(S), _p(rows),
+                              _p(rows_ptr), C.c_int64(E), C.c_int64(B),
+                              _p(unique_ptr))
+    U = int(unique_ptr[-1])
+    unique = np.empty(U, dtype=np.int64)
+    want_col = want_col and edge_col is not None
+    if edge_col is not None:
+        edge_col = _i64(edge_col)
+    out_row = np.empty(E, dtype=np.int64) if want_row else None
+    out_col = np.empty(E, dtype=np.int64) if want_col else None
+    lib().gs_unique_fill_cpu(_p(seeds), _p(seeds_ptr), C.c_int64(S), _p(rows),
+                             _p(rows_ptr), C.c_int64(E), C.c_int64(B),
+                             _p(unique_ptr), _p(edge_col), _p(unique),
+                             _p(out_row), _p(out_col))
+    return unique, unique_ptr, out_row, out_col

@@ -1,0 +1,348 @@
+// gs_oracle.cpp -- CPU restatement of gSampler's sampling hot path.
+//
+// TEST INFRASTRUCTURE ONLY.  This file is the correctness oracle and the timed
+// host baseline.  Nothing in the shipped package may link, load or call it:
+// only tests/, __graft_entry__.smoke() and bench.py's cpu_baseline leg do.
+//
+// Every function restates what the cited reference kernel computes (paths are
+// relative to the gSampler source tree), written for clarity, parallel over
+// columns / batches / walks with OpenMP.  Exported with a `_cpu` suffix and
+// the same argument meaning as include/gsampler_hip.h, minus stream and
+// workspace.
+//
+// Random numbers.  The reference draws from curand streams whose layout
+// depends on the CUDA launch geometry (src/cuda/sampling.cu:25-26,56), so its
+// exact picks cannot be restated on a CPU.  The convention here (shared with
+// the HIP kernels, implemented independently in both) makes every pick a pure
+// function of (seed, call_id, position, draw):
+//   key     = seed + call_id * 0x9E3779B97F4A7C15  (mod 2^64), split lo/hi
+//   counter = (lo32(draw), hi32(draw), lo32(pos), hi32(pos))
+//   (w0,w1,w2,w3) = Philox4x32-10(counter, key)
+//   r64 = w1:w0,  bounded(n) = floor(r64 * n / 2^64)
+// Pinned by the Random123 known-answer vectors (tests/test_oracle_philox.py).
+//
+// Parity status of each function is listed in oracle/README.md.
+
+#include <algorithm>
+#include <cmath>
+#include <cstdint>
+#include <cstring>
+#include <limits>
+#include <unordered_map>
+#include <vector>
+
+#ifdef _OPENMP
+#include <omp.h>
+#endif
+
+#define GS_ALGO_AUTO 0
+#define GS_ALGO_RESERVOIR 1
+#define GS_ALGO_FLOYD 2
+
+namespace {
+
+// ---------------------------------------------------------------- Philox
+struct U4 {
+  uint32_t v[4];
+};
+
+inline U4 philox4x32_10(U4 ctr, uint32_t k0, uint32_t k1) {
+  const uint64_t M0 = 0xD2511F53u, M1 = 0xCD9E8D57u;
+  for (int r = 0; r < 10; ++r) {
+    uint64_t p0 = M0 * ctr.v[0];
+    uint64_t p1 = M1 * ctr.v[2];
+    U4 n;
+    n.v[0] = (uint32_t)(p1 >> 32) ^ ctr.v[1] ^ k0;
+    n.v[1] = (uint32_t)p1;
+    n.v[2] = (uint32_t)(p0 >> 32) ^ ctr.v[3] ^ k1;
+    n.v[3] = (uint32_t)p0;
+    ctr = n;
+    k0 += 0x9E3779B9u;
+    k1 += 0xBB67AE85u;
+  }
+  return ctr;
+}
+
+struct Stream {
+  uint32_t k0, k1;
+  Stream(uint64_t seed, uint64_t call_id) {
+    uint64_t k = seed + call_id * 0x9E3779B97F4A7C15ull;
+    k0 = (uint32_t)k;
+    k1 = (uint32_t)(k >> 32);
+  }
+  U4 words(uint64_t pos, uint64_t draw) const {
+    U4 c;
+    c.v[0] = (uint32_t)draw;
+    c.v[1] = (uint32_t)(draw >> 32);
+    c.v[2] = (uint32_t)pos;
+    c.v[3] = (uint32_t)(pos >> 32);
+    return philox4x32_10(c, k0, k1);
+  }
+  uint64_t r64(uint64_t pos, uint64_t draw) const {
+    U4 w = words(pos, draw);
+    return ((uint64_t)w.v[1] << 32) | w.v[0];
+  }
+  // integer in [0, n)
+  uint64_t bounded(uint64_t pos, uint64_t draw, uint64_t n) const {
+    return (uint64_t)(((unsigned __int128)r64(pos, draw) * n) >> 64);
+  }
+};
+
+inline int64_t col_degree(const int64_t* indptr, int64_t num_cols, int64_t c) {
+  if (c < 0 || c >= num_cols) return 0;
+  return indptr[c + 1] - indptr[c];
+}
+
+}  // namespace
+
+extern "C" {
+
+// Known-answer hook for the Philox block function.
+void gs_philox4x32_10_cpu(const uint32_t* ctr, const uint32_t* key,
+                          uint32_t* out) {
+  U4 c = {{ctr[0], ctr[1], ctr[2], ctr[3]}};
+  U4 r = philox4x32_10(c, key[0], key[1]);
+  for (int i = 0; i < 4; ++i) out[i] = r.v[i];
+}
+
+// The four words drawn for (seed, call_id, pos, draw).
+void gs_stream_words_cpu(uint64_t seed, uint64_t call_id, uint64_t pos,
+                         uint64_t draw, uint32_t* out) {
+  U4 r = Stream(seed, call_id).words(pos, draw);
+  for (int i = 0; i < 4; ++i) out[i] = r.v[i];
+}
+
+int gs_num_threads_cpu(void) {
+#ifdef _OPENMP
+  return omp_get_max_threads();
+#else
+  return 1;
+#endif
+}
+
+// -------------------------------------------------------------------------
+// Exclusive scan (cub_exclusiveSum, src/cuda/utils.h:18-28).
+void gs_exclusive_scan_i64_cpu(const int64_t* in, int64_t* out, int64_t n) {
+  int64_t acc = 0;
+  for (int64_t i = 0; i < n; ++i) {
+    int64_t v = in[i];
+    out[i] = acc;
+    acc += v;
+  }
+}
+
+// -------------------------------------------------------------------------
+// Per-column counts + prefix.  src/cuda/slicing.cu:133-141 (slice),
+// src/cuda/sampling.cu:112-124 and src/cuda/fusion/slice_sampling.cu:111-124
+// (sample): replace -> deg == 0 ? 0 : K ; else min(deg, K).
+void gs_csc_col_count_cpu(const int64_t* indptr, int64_t num_cols,
+                          const int64_t* column_ids, int64_t num_items,
+                          int64_t fanout, int replace, int64_t* sub_indptr) {
+  int64_t acc = 0;
+  for (int64_t i = 0; i < num_items; ++i) {
+    int64_t c = column_ids ? column_ids[i] : i;
+    int64_t deg = col_degree(indptr, num_cols, c);
+    int64_t cnt;
+    if (fanout < 0)
+      cnt = deg;
+    else if (replace)
+      cnt = deg == 0 ? 0 : fanout;
+    else
+      cnt = std::min(deg, fanout);
+    sub_indptr[i] = acc;
+    acc += cnt;
+  }
+  sub_indptr[num_items] = acc;
+}
+
+// -------------------------------------------------------------------------
+// Column slice, src/cuda/slicing.cu:101-119 (_GetSubIndicesKernel) and the
+// batched form src/cuda/batch/slicing.cu:12-38 (row id + batch * stride).
+void gs_csc_col_slice_fill_cpu(const int64_t* indptr, int64_t num_cols,
+                               const int64_t* indices,
+                               const int64_t* column_ids, int64_t num_items,
+                               const int64_t* sub_indptr, int64_t /*nnz*/,
+                               const int64_t* batch_ptr, int64_t num_batches,
+                               int64_t encode_stride, int64_t* out_coo_col,
+                               int64_t* out_indices, int64_t* out_select) {
+#pragma omp parallel for schedule(dynamic, 256)
+  for (int64_t i = 0; i < num_items; ++i) {
+    int64_t c = column_ids ? column_ids[i] : i;
+    int64_t deg = col_degree(indptr, num_cols, c);
+    if (deg == 0) continue;
+    int64_t in_start = indptr[c];
+    int64_t out_start = sub_indptr[i];
+    int64_t add = 0;
+    if (batch_ptr && encode_stride > 0) {
+      int64_t b = std::upper_bound(batch_ptr, batch_ptr + num_batches + 1, i) -
+                  batch_ptr - 1;
+      add = b * encode_stride;
+    }
+    for (int64_t k = 0; k < deg; ++k) {
+      out_indices[out_start + k] = indices[in_start + k] + add;
+      out_select[out_start + k] = in_start + k;
+      if (out_coo_col) out_coo_col[out_start + k] = i;
+    }
+  }
+}
+
+// -------------------------------------------------------------------------
+// Uniform per-column sampling, src/cuda/sampling.cu:18-101 and the fused form
+// src/cuda/fusion/slice_sampling.cu:14-96.
+//  * replace: slot j takes position r(j) mod deg            (:34-45)
+//  * deg <= K: copy the column in order                      (:64-73)
+//  * reservoir: slot[j] = j; for idx in [K, deg):
+//      num = r(idx) mod (idx+1); if num < K: slot[num] = max(slot[num], idx)
+//                                                            (:75-88)
+//    The reference's `curand() % n` is replaced by the (less biased)
+//    multiply-shift bounded(); the result depends only on idx -> r(idx).
+//  * Floyd (not in the reference; same distribution over K-subsets, O(K)
+//    draws instead of O(deg)): for i in [0,K): j = deg-K+i,
+//      t = r(i) bounded to [0, j]; pick t unless already picked, then pick j.
+void gs_csc_col_sample_uniform_fill_cpu(
+    const int64_t* indptr, int64_t num_cols, const int64_t* indices,
+    const int64_t* column_ids, int64_t num_items, int64_t fanout, int replace,
+    int algo, uint64_t seed, uint64_t call_id, const int64_t* sub_indptr,
+    int64_t* out_coo_col, int64_t* out_indices, int64_t* out_select) {
+  Stream rng(seed, call_id);
+  if (algo == GS_ALGO_AUTO)
+    algo = fanout <= 64 ? GS_ALGO_FLOYD : GS_ALGO_RESERVOIR;
+#pragma omp parallel
+  {
+    std::vector<int64_t> slot((size_t)std::max<int64_t>(fanout, 1));
+#pragma omp for schedule(dynamic, 256)
+    for (int64_t i = 0; i < num_items; ++i) {
+      int64_t c = column_ids ? column_ids[i] : i;
+      int64_t deg = col_degree(indptr, num_cols, c);
+      if (deg == 0) continue;
+      int64_t in_start = indptr[c];
+      int64_t out_start = sub_indptr[i];
+      int64_t cnt = sub_indptr[i + 1] - out_start;
+      if (replace) {
+        for (int64_t j = 0; j < cnt; ++j)
+          slot[j] = (int64_t)rng.bounded((uint64_t)i, (uint64_t)j, (uint64_t)deg);
+      } else if (deg <= fanout) {
+        for (int64_t j = 0; j < cnt; ++j) slot[j] = j;
+      } else if (algo == GS_ALGO_RESERVOIR) {
+        for (int64_t j = 0; j < fanout; ++j) slot[j] = j;
+        for (int64_t idx = fanout; idx < deg; ++idx) {
+          int64_t num = (int64_t)rng.bounded((uint64_t)i, (uint64_t)idx,
+                                             (uint64_t)idx + 1);
+          if (num < fanout) slot[num] = std::max(slot[num], idx);
+        }
+      } else {  // Floyd
+        for (int64_t k = 0; k < fanout; ++k) {
+          int64_t j = deg - fanout + k;
+          int64_t t = (int64_t)rng.bounded((uint64_t)i, (uint64_t)k,
+                                           (uint64_t)j + 1);
+          bool seen = false;
+          for (int64_t m = 0; m < k; ++m)
+            if (slot[m] == t) {
+              seen = true;
+              break;
+            }
+          slot[k] = seen ? j : t;
+        }
+      }
+      for (int64_t j = 0; j < cnt; ++j) {
+        int64_t p = in_start + slot[j];
+        out_indices[out_start + j] = indices[p];
+        out_select[out_start + j] = p;
+        if (out_coo_col) out_coo_col[out_start + j] = i;
+      }
+    }
+  }
+}
+
+// -------------------------------------------------------------------------
+// Unique (first-occurrence order) + relabel.
+//  single batch : Unique / Relabel, src/cuda/unique_reindex.cu:81-172 -- the
+//    table keeps the minimum index per key (:25 AtomicMin), an element is kept
+//    iff it holds that minimum (:113), its rank is the prefix count (:138-139).
+//  super-batch  : src/cuda/batch/batch_relabel.cu:92-377 -- one table per
+//    batch, keys of batch b are seeds_b ++ rows_b (:138-161), ranks are
+//    batch-local, unique_ptr[b] = uniques before batch b (:437-438).
+// out_col[e] = rank of seeds[edge_col[e]] (the reference relabels
+// coo_col = col_seeds[coo.col], src/batch_graph.cc:230, src/graph.cc:582).
+static void batch_bounds(const int64_t* ptr, int64_t total, int64_t nb,
+                         int64_t b, int64_t* lo, int64_t* hi) {
+  if (ptr) {
+    *lo = ptr[b];
+    *hi = ptr[b + 1];
+  } else {
+    *lo = 0;
+    *hi = total;
+    (void)nb;
+  }
+}
+
+// Pass 1 (count): unique_ptr.  Pass 2 (fill): outputs.  Both recompute the
+// per-batch map; the oracle favours obviousness over speed.
+static void unique_batch(const int64_t* seeds, int64_t s_lo, int64_t s_hi,
+                         const int64_t* rows, int64_t r_lo, int64_t r_hi,
+                         std::unordered_map<int64_t, int64_t>* rank,
+                         std::vector<int64_t>* uniq) {
+  rank->clear();
+  uniq->clear();
+  rank->reserve((size_t)((s_hi - s_lo) + (r_hi - r_lo)));
+  for (int64_t i = s_lo; i < s_hi; ++i)
+    if (rank->emplace(seeds[i], (int64_t)uniq->size()).second)
+      uniq->push_back(seeds[i]);
+  for (int64_t i = r_lo; i < r_hi; ++i)
+    if (rank->emplace(rows[i], (int64_t)uniq->size()).second)
+      uniq->push_back(rows[i]);
+}
+
+void gs_unique_count_cpu(const int64_t* seeds, const int64_t* seeds_ptr,
+                         int64_t num_seeds, const int64_t* rows,
+                         const int64_t* rows_ptr, int64_t num_rows_keys,
+                         int64_t num_batches, int64_t* unique_ptr) {
+  std::vector<int64_t> counts((size_t)num_batches);
+#pragma omp parallel
+  {
+    std::unordered_map<int64_t, int64_t> rank;
+    std::vector<int64_t> uniq;
+#pragma omp for schedule(dynamic, 1)
+    for (int64_t b = 0; b < num_batches; ++b) {
+      int64_t s_lo, s_hi, r_lo, r_hi;
+      batch_bounds(seeds_ptr, num_seeds, num_batches, b, &s_lo, &s_hi);
+      batch_bounds(rows_ptr, num_rows_keys, num_batches, b, &r_lo, &r_hi);
+      unique_batch(seeds, s_lo, s_hi, rows, r_lo, r_hi, &rank, &uniq);
+      counts[(size_t)b] = (int64_t)uniq.size();
+    }
+  }
+  int64_t acc = 0;
+  for (int64_t b = 0; b < num_batches; ++b) {
+    unique_ptr[b] = acc;
+    acc += counts[(size_t)b];
+  }
+  unique_ptr[num_batches] = acc;
+}
+
+void gs_unique_fill_cpu(const int64_t* seeds, const int64_t* seeds_ptr,
+                        int64_t num_seeds, const int64_t* rows,
+                        const int64_t* rows_ptr, int64_t num_rows_keys,
+                        int64_t num_batches, const int64_t* unique_ptr,
+                        const int64_t* edge_col, int64_t* out_unique,
+                        int64_t* out_row, int64_t* out_col) {
+#pragma omp parallel
+  {
+    std::unordered_map<int64_t, int64_t> rank;
+    std::vector<int64_t> uniq;
+#pragma omp for schedule(dynamic, 1)
+    for (int64_t b = 0; b < num_batches; ++b) {
+      int64_t s_lo, s_hi, r_lo, r_hi;
+      batch_bounds(seeds_ptr, num_seeds, num_batches, b, &s_lo, &s_hi);
+      batch_bounds(rows_ptr, num_rows_keys, num_batches, b, &r_lo, &r_hi);
+      unique_batch(seeds, s_lo, s_hi, rows, r_lo, r_hi, &rank, &uniq);
+      if (out_unique)
+        std::copy(uniq.begin(), uniq.end(), out_unique + unique_ptr[b]);
+      for (int64_t e = r_lo; e < r_hi; ++e) {
+        if (out_row) out_row[e] = rank[rows[e]];
+        if (out_col) out_col[e] = rank[seeds[edge_col[e]]];
+      }
+    }
+  }
+}
+
+}  // extern "C"

@@ -1,0 +1,154 @@
+"""HIP kernels vs the CPU oracle on the same seeded inputs, called through the
+C ABI.  Integer / index work: bit-exact."""
+import numpy as np
+import pytest
+import torch
+
+from gsampler_amd import capi
+from oracle import binding as orc
+from tests.conftest import random_csc
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def T(a):
+    return None if a is None else torch.as_tensor(np.asarray(a, dtype=np.int64), device=DEV)
+
+
+def N(t):
+    return None if t is None else t.cpu().numpy()
+
+
+def assert_same(got, want):
+    assert len(got) == len(want)
+    for g, w in zip(got, want):
+        if w is None:
+            assert g is None
+        else:
+            assert np.array_equal(N(g), w)
+
+
+@pytest.mark.parametrize("n", [0, 1, 255, 256, 2049, 1 << 20, (1 << 22) + 3])
+def test_scan(n):
+    rng = np.random.default_rng(n)
+    x = rng.integers(0, 1000, size=n)
+    assert np.array_equal(N(capi.exclusive_scan(T(x))), np.cumsum(x) - x)
+
+
+def test_reference_known_answers():
+    indptr, indices = np.arange(21) * 5, np.arange(100)
+    s, c, i, sel = capi.col_slice(T(indptr), T(indices), T([0, 1, 2]))
+    assert N(s).tolist() == [0, 5, 10, 15] and N(i).tolist() == list(range(15))
+    # K > deg, no replace -> identity (tests/test_colwise_sampling.cc test1)
+    s, c, i, sel = capi.sample_uniform(T(indptr), T(indices), None, 6, False)
+    assert np.array_equal(N(s), indptr) and np.array_equal(N(i), indices)
+    for fanout in (6, 4):  # test2 / test3
+        s, c, i, sel = capi.sample_uniform(T(indptr), T(indices), None, fanout, True)
+        assert np.array_equal(N(s), np.arange(21) * fanout)
+        assert np.array_equal(N(sel) // 5, np.repeat(np.arange(20), fanout))
+
+
+@pytest.mark.parametrize("seed", range(3))
+def test_col_slice_parity(seed):
+    rng = np.random.default_rng(seed)
+    indptr, indices = random_csc(rng, 3000, 10**5, 60, hub_deg=50000)
+    cols = rng.integers(-2, 3003, size=2500)  # a few out-of-range ids
+    assert_same(capi.col_slice(T(indptr), T(indices), T(cols)),
+                orc.col_slice(indptr, indices, cols))
+    ptr = np.array([0, 100, 100, 1700, 2500])
+    assert_same(capi.col_slice(T(indptr), T(indices), T(cols), batch_ptr=T(ptr),
+                               encode_stride=10**5),
+                orc.col_slice(indptr, indices, cols, batch_ptr=ptr, encode_stride=10**5))
+    e = np.empty(0, dtype=np.int64)
+    assert_same(capi.col_slice(T(indptr), T(indices), T(e)), orc.col_slice(indptr, indices, e))
+
+
+@pytest.mark.parametrize("algo", [capi.ALGO_AUTO, capi.ALGO_RESERVOIR, capi.ALGO_FLOYD])
+@pytest.mark.parametrize("fanout", [1, 5, 8, 10, 15, 16, 25, 33, 64])
+def test_sample_uniform_parity(algo, fanout):
+    rng = np.random.default_rng(fanout)
+    indptr, indices = random_csc(rng, 5000, 10**6, 90, hub_deg=20000)
+    cols = rng.integers(0, 5000, size=4097)
+    for call_id in (0, 3):
+        assert_same(
+            capi.sample_uniform(T(indptr), T(indices), T(cols), fanout, False, algo,
+                                seed=7777, call_id=call_id),
+            orc.sample_uniform(indptr, indices, cols, fanout, False, algo,
+                               seed=7777, call_id=call_id))
+
+
+@pytest.mark.parametrize("fanout", [3, 20, 100])
+def test_sample_replace_and_unfused_parity(fanout):
+    rng = np.random.default_rng(fanout)
+    indptr, indices = random_csc(rng, 2000, 10**6, 50, hub_deg=3000)
+    cols = rng.integers(0, 2000, size=1500)
+    assert_same(capi.sample_uniform(T(indptr), T(indices), T(cols), fanout, True),
+                orc.sample_uniform(indptr, indices, cols, fanout, True))
+    # column_ids = None: sample the matrix's own columns (un-fused Sampling)
+    for replace in (False, True):
+        assert_same(capi.sample_uniform(T(indptr), T(indices), None, fanout, replace),
+                    orc.sample_uniform(indptr, indices, None, fanout, replace))
+    # reservoir with fanout > 64 (the AUTO choice there)
+    assert_same(capi.sample_uniform(T(indptr), T(indices), T(cols), 100, False),
+                orc.sample_uniform(indptr, indices, cols, 100, False))
+
+
+def _batched_case(rng, B, max_seeds, max_rows, id_range):
+    s_sizes = rng.integers(1, max_seeds, size=B)
+    r_sizes = rng.integers(0, max_rows, size=B)
+    r_sizes[B // 2] = 0
+    sp = np.concatenate([[0], np.cumsum(s_sizes)])
+    rp = np.concatenate([[0], np.cumsum(r_sizes)])
+    seeds = rng.integers(0, id_range, size=sp[-1])
+    rows = rng.integers(0, id_range, size=rp[-1])
+    edge_col = np.concatenate(
+        [rng.integers(sp[b], sp[b + 1], size=r_sizes[b]) for b in range(B)]).astype(np.int64)
+    return seeds, rows, sp, rp, edge_col
+
+
+@pytest.mark.parametrize("id_range", [50, 5000, 2**32 - 2])
+def test_unique_relabel_single_parity(id_range):
+    rng = np.random.default_rng(1)
+    seeds = rng.integers(0, id_range, size=777)
+    rows = rng.integers(0, id_range, size=50000)
+    if id_range > 10**6:
+        rows[:5] = id_range  # the largest admissible key
+    edge_col = rng.integers(0, 777, size=50000)
+    assert_same(capi.unique_relabel(T(seeds), T(rows), edge_col=T(edge_col)),
+                orc.unique_relabel(seeds, rows, edge_col=edge_col))
+    # no seeds / no rows / nothing
+    e = np.empty(0, dtype=np.int64)
+    assert_same(capi.unique_relabel(T(e), T(rows)), orc.unique_relabel(e, rows))
+    assert_same(capi.unique_relabel(T(seeds), T(e)), orc.unique_relabel(seeds, e))
+    assert_same(capi.unique_relabel(T(e), T(e)), orc.unique_relabel(e, e))
+
+
+@pytest.mark.parametrize("B,id_range", [(2, 100), (7, 3000), (64, 10**5)])
+def test_unique_relabel_batched_parity(B, id_range):
+    rng = np.random.default_rng(B)
+    seeds, rows, sp, rp, edge_col = _batched_case(rng, B, 300, 6000, id_range)
+    assert_same(capi.unique_relabel(T(seeds), T(rows), T(sp), T(rp), T(edge_col)),
+                orc.unique_relabel(seeds, rows, sp, rp, edge_col))
+
+
+def test_graphsage_layers_end_to_end():
+    """Three fused slice+sample + unique/relabel layers on an R-MAT graph, super-batch
+    of 8, compared with the oracle layer by layer."""
+    from gsampler_amd.utils import rmat_csc, batched_seeds
+    indptr_t, indices_t = rmat_csc(20000, 400000, seed=1)
+    seeds_t, ptr_t = batched_seeds(20000, 8, 128, seed=2)
+    indptr, indices = indptr_t.numpy(), indices_t.numpy()
+    seeds, ptr = seeds_t.numpy(), ptr_t.numpy()
+    g_seeds, g_ptr = T(seeds), T(ptr)
+    for layer, fanout in enumerate([15, 10, 5]):
+        g = capi.sample_uniform(T(indptr), T(indices), g_seeds, fanout, call_id=layer)
+        o = orc.sample_uniform(indptr, indices, seeds, fanout, call_id=layer)
+        assert_same(g, o)
+        g_eptr = g[0][g_ptr]
+        o_eptr = o[0][ptr]
+        gu = capi.unique_relabel(g_seeds, g[2], g_ptr, g_eptr, g[1])
+        ou = orc.unique_relabel(seeds, o[2], ptr, o_eptr, o[1])
+        assert_same(gu, ou)
+        g_seeds, g_ptr = gu[0], gu[1]
+        seeds, ptr = ou[0], ou[1]
