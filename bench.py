@@ -1,0 +1,210 @@
+#!/usr/bin/env python3
+"""Benchmark of the GraphSAGE sampling hot path on one MI355X.
+
+One "step" = one super-batch through the whole pipeline: for every fanout in
+[15, 10, 5]: fused column slice + uniform sampling without replacement, then
+per-batch unique (first-occurrence order) + relabel; the unique frontier of a
+layer is the seed set of the next.  Inputs (CSC graph, seeds) are resident in
+HBM before the timed region starts.
+
+Prints ONE JSON line.  `value` is sampled edges per second over the timed
+steps; `roofline` describes the kernel with the largest share of GPU time
+(durations from HIP events recorded by the library on the launch stream while
+the same steps run once more); `cpu_baseline` is the CPU oracle timed on a
+bounded sample of the same workload on this machine's host cores.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published peak
+
+WORKLOADS = {
+    # name: (nodes, edges, generator, batches, batch size, fanouts)
+    "c2": dict(nodes=2_450_000, edges=124_000_000, gen="chung_lu", batches=64,
+               batch_size=1024, fanouts=[15, 10, 5],
+               desc="GraphSAGE 3-layer uniform [15,10,5], 64 batches x 1024 seeds per "
+                    "launch, Chung-Lu power-law (exp 2.1) 2.45M nodes / 124M edges, CSC int64"),
+    "c1": dict(nodes=100_000, edges=2_000_000, gen="rmat", batches=1,
+               batch_size=1024, fanouts=[25, 10],
+               desc="GraphSAGE 2-layer uniform [25,10], 1024 seeds, R-MAT 100K nodes / 2M edges"),
+    "tiny": dict(nodes=50_000, edges=1_000_000, gen="chung_lu", batches=8,
+                 batch_size=256, fanouts=[15, 10, 5],
+                 desc="1/50-scale twin of c2 (smoke runs)"),
+}
+
+
+def graphsage_step(be, indptr, indices, seeds, ptr, fanouts, seed, call_base):
+    """The pipeline, written once for both back ends (`be` is gsampler_amd.capi
+    on torch CUDA tensors or oracle.binding on numpy arrays).
+    Returns per-layer (S, E, U) and the last layer's outputs."""
+    sizes, last = [], None
+    for layer, fanout in enumerate(fanouts):
+        sub_indptr, coo_col, rows, sel = be.sample_uniform(
+            indptr, indices, seeds, fanout, False, 0, seed, call_base + layer)
+        edge_ptr = sub_indptr[ptr]
+        uniq, uniq_ptr, out_row, out_col = be.unique_relabel(
+            seeds, rows, ptr, edge_ptr, coo_col)
+        sizes.append((int(seeds.shape[0]), int(rows.shape[0]), int(uniq.shape[0])))
+        last = (uniq, uniq_ptr, out_row, out_col, sel)
+        seeds, ptr = uniq, uniq_ptr
+    return sizes, last
+
+
+def kernel_bytes(name, sizes):
+    """Algorithmic bytes moved by all launches of `name` in one step: the
+    compulsory reads and writes of the kernel's interface (hash-table, scratch
+    and re-read traffic excluded)."""
+    total = 0
+    for S, E, U in sizes:
+        N = S + E
+        total += {
+            "sample_uniform": 32 * S + 32 * E,   # seeds, indptr pair, sub_indptr, gather, 3 outputs
+            "col_count": 32 * S,                 # seeds, indptr pair, counts
+            "unique_insert": 8 * N,              # keys in
+            "unique_flag": 8 * N + N // 8,       # keys in, flag bits out
+            "unique_fill": 8 * N + 8 * U + 8 * S,  # keys in, frontier + seed ranks out
+            "unique_relabel": 32 * E,            # row key + column id in, row + col out
+            "unique_clear": 16 * N,              # table initialisation
+        }.get(name, 0)
+    return total
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=2)
+    ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS))
+    ap.add_argument("--cpu-seconds", type=float, default=15.0,
+                    help="target CPU time of the oracle baseline (0 = skip)")
+    ap.add_argument("--seed", type=int, default=7777)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build drives exactly one GPU (the super-batch is the unit "
+                 "that would be dealt out across GPUs); run with --gpus 1")
+
+    import numpy as np
+    import torch
+    from gsampler_amd import capi
+    from gsampler_amd.utils import batched_seeds, chung_lu_csc, rmat_csc
+
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU visible")
+    capi.lib()  # fail loudly when the kernel library is missing
+    dev = torch.device("cuda:0")
+    wl = WORKLOADS[args.workload]
+
+    t0 = time.time()
+    gen = chung_lu_csc if wl["gen"] == "chung_lu" else rmat_csc
+    indptr, indices = gen(wl["nodes"], wl["edges"], seed=1, device=dev)
+    seeds, ptr = batched_seeds(wl["nodes"], wl["batches"], wl["batch_size"], seed=2, device=dev)
+    torch.cuda.synchronize()
+    t_build = time.time() - t0
+    fanouts = wl["fanouts"]
+
+    def step(i):
+        return graphsage_step(capi, indptr, indices, seeds, ptr, fanouts, args.seed,
+                              i * len(fanouts))
+
+    for i in range(args.warmup):
+        step(i)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    edges = 0
+    sizes = None
+    for i in range(args.steps):
+        sizes, _ = step(args.warmup + i)
+        edges += sum(E for _, E, _ in sizes)
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    ms_per_step = elapsed / args.steps * 1e3
+    edges_per_s = edges / elapsed
+    batches_per_s = wl["batches"] * args.steps / elapsed
+
+    # ---- per-kernel durations: same steps again with the library's event timers on
+    capi.profile_reset()
+    capi.profile_enable(True)
+    prof_sizes = []
+    for i in range(args.steps):
+        s, _ = step(args.warmup + i)
+        prof_sizes.append(s)
+    torch.cuda.synchronize()
+    totals = capi.profile_totals()
+    capi.profile_enable(False)
+    kernels = []
+    for name, (calls, ms) in totals.items():
+        nbytes = sum(kernel_bytes(name, s) for s in prof_sizes)
+        kernels.append(dict(kernel=name, launches=calls, avg_ms=ms / max(calls, 1),
+                            total_ms=ms, algorithmic_bytes=nbytes,
+                            gbs=(nbytes / (ms * 1e-3) / 1e9) if ms > 0 else 0.0))
+    kernels.sort(key=lambda k: -k["total_ms"])
+    dom = kernels[0]
+    traffic = None
+    tpath = os.path.join(ROOT, "profiles", f"traffic_{args.workload}.json")
+    if os.path.exists(tpath):
+        traffic = json.load(open(tpath)).get(dom["kernel"])
+    roofline = dict(bound="hbm", kernel=dom["kernel"], achieved=round(dom["gbs"], 1),
+                    peak=HBM_PEAK_GBS, unit="GB/s", frac=round(dom["gbs"] / HBM_PEAK_GBS, 4),
+                    traffic=traffic, avg_launch_ms=round(dom["avg_ms"], 4),
+                    launches=dom["launches"])
+    pipeline_bytes = sum(40 * S + 56 * E + 8 * U for S, E, U in sizes)
+
+    # ---- CPU baseline: the oracle on the first few batches of the same super-batch
+    cpu = None
+    if args.cpu_seconds > 0:
+        from oracle import binding as orc
+        h_indptr, h_indices = indptr.cpu().numpy(), indices.cpu().numpy()
+        h_seeds, h_ptr = seeds.cpu().numpy(), ptr.cpu().numpy()
+
+        def cpu_run(call_base):
+            t = time.perf_counter()
+            sz, _ = graphsage_step(orc, h_indptr, h_indices, h_seeds, h_ptr, fanouts,
+                                   args.seed, call_base)
+            return time.perf_counter() - t, sum(E for _, E, _ in sz)
+
+        cpu_run(0)  # warm-up (page in the graph, spin up the thread pool)
+        t_cpu, e_cpu, n_cpu = 0.0, 0, 0
+        while t_cpu < args.cpu_seconds and n_cpu < 1000:
+            t, e = cpu_run((n_cpu + 1) * len(fanouts))
+            t_cpu, e_cpu, n_cpu = t_cpu + t, e_cpu + e, n_cpu + 1
+        cpu = dict(value=round(e_cpu / t_cpu, 1), unit="edges/s", cores=orc.num_threads(),
+                   kind="port",
+                   sample=f"{n_cpu} full super-batches ({wl['batches']} batches each, same "
+                          f"graph and seeds, a new sampler call id each) in {t_cpu:.1f} s, "
+                          f"OpenMP oracle after one warm-up pass",
+                   host_cpus=os.cpu_count())
+
+    out = {
+        "metric": "sampled_edges_per_sec", "value": round(edges_per_s, 1), "unit": "edges/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 3), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "int64", "data": "synthetic",
+        "config": {"workload": f"{args.workload}: {wl['desc']}",
+                   "fanouts": fanouts, "batches_per_launch": wl["batches"],
+                   "seeds_per_batch": wl["batch_size"], "sampler_seed": args.seed,
+                   "layer_sizes_S_E_U": sizes},
+        "batches_per_sec": round(batches_per_s, 1),
+        "pipeline_algorithmic_gbs": round(pipeline_bytes / (ms_per_step * 1e-3) / 1e9, 1),
+        "pipeline_frac_of_hbm_peak": round(pipeline_bytes / (ms_per_step * 1e-3) / 1e9
+                                           / HBM_PEAK_GBS, 4),
+        "roofline": roofline,
+        "cpu_baseline": cpu,
+        "gpu_over_cpu": round(edges_per_s / cpu["value"], 1) if cpu else None,
+        "kernels": [{k: (round(v, 4) if isinstance(v, float) else v) for k, v in kk.items()}
+                    for kk in kernels],
+        "graph_build_s": round(t_build, 1),
+    }
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

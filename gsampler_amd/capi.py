@@ -36,6 +36,11 @@ _int = C.c_int
 SIGNATURES = {
     "gs_last_error": (C.c_char_p, []),
     "gs_abi_version": (_int, []),
+    "gs_profile_enable": (None, [_int]),
+    "gs_profile_reset": (None, []),
+    "gs_profile_count": (_int, []),
+    "gs_profile_get": (_int, [_int, C.c_char_p, _sz, C.POINTER(C.c_longlong),
+                              C.POINTER(C.c_double)]),
     "gs_scan_workspace_bytes": (_sz, [_i64]),
     "gs_exclusive_scan_i64": (_int, [_p, _p, _i64, _p, _sz, _p]),
     "gs_csc_col_count": (_int, [_p, _i64, _p, _i64, _i64, _int, _p, _p, _sz, _p]),
@@ -97,6 +102,27 @@ def _i64t(t: torch.Tensor, name: str) -> torch.Tensor:
 
 def _workspace(nbytes: int, device) -> torch.Tensor:
     return torch.empty(max(int(nbytes), 1), dtype=torch.uint8, device=device)
+
+
+# -------------------------------------------------------------- profiling
+def profile_enable(on: bool) -> None:
+    lib().gs_profile_enable(int(on))
+
+
+def profile_reset() -> None:
+    lib().gs_profile_reset()
+
+
+def profile_totals() -> dict:
+    """{kernel name: (launches, total milliseconds)} since the last reset."""
+    l = lib()
+    out = {}
+    for i in range(l.gs_profile_count()):
+        name = C.create_string_buffer(128)
+        calls, ms = C.c_longlong(0), C.c_double(0.0)
+        check(l.gs_profile_get(i, name, 128, C.byref(calls), C.byref(ms)))
+        out[name.value.decode()] = (calls.value, ms.value)
+    return out
 
 
 # ---------------------------------------------------------------- helpers

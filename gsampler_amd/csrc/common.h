@@ -35,6 +35,31 @@ int hip_fail(hipError_t e, const char* what, const char* file, int line);
 
 inline hipStream_t as_stream(gs_stream_t s) { return (hipStream_t)s; }
 
+// Optional per-kernel timing (gs_profile_*): while enabled, every launch that
+// sits inside a ProfScope is bracketed by two HIP events on its own stream.
+bool profile_enabled();
+void profile_begin(const char* name, hipStream_t stream);
+void profile_end(hipStream_t stream);
+struct ProfScope {
+  hipStream_t stream;
+  bool on;
+  ProfScope(const char* name, hipStream_t s) : stream(s), on(profile_enabled()) {
+    if (on) profile_begin(name, s);
+  }
+  ~ProfScope() {
+    if (on) profile_end(stream);
+  }
+};
+// Usage: GS_LAUNCH("name", stream, kernel<<<grid, block, 0, stream>>>(args));
+#define GS_LAUNCH(name, stream, ...)   \
+  do {                                 \
+    {                                  \
+      gs::ProfScope ps__(name, stream); \
+      __VA_ARGS__;                     \
+    }                                  \
+    GS_LAUNCH_CHECK();                 \
+  } while (0)
+
 constexpr int kWave = 64;
 constexpr int kBlock = 256;  // 4 waves; the default block for flat kernels
 

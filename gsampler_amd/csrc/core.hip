@@ -1,7 +1,10 @@
 // core.hip -- error plumbing and the device-wide exclusive scan.
 #include <cstdarg>
 #include <cstdio>
+#include <cstring>
+#include <mutex>
 #include <string>
+#include <vector>
 
 #include "common.h"
 #include "scan.h"
@@ -23,6 +26,74 @@ int hip_fail(hipError_t e, const char* what, const char* file, int line) {
   set_error("HIP error %d (%s) at %s:%d in %s", (int)e, hipGetErrorString(e),
             file, line, what);
   return GS_ERR_HIP;
+}
+
+// ------------------------------------------------------------- profiling
+namespace {
+struct ProfPending {
+  const char* name;
+  hipEvent_t start, stop;
+};
+struct ProfTotal {
+  std::string name;
+  long long calls;
+  double ms;
+};
+std::mutex g_prof_mutex;
+bool g_prof_on = false;
+std::vector<ProfPending> g_prof_pending;
+std::vector<hipEvent_t> g_prof_pool;
+std::vector<ProfTotal> g_prof_totals;
+
+hipEvent_t prof_event() {
+  if (!g_prof_pool.empty()) {
+    hipEvent_t e = g_prof_pool.back();
+    g_prof_pool.pop_back();
+    return e;
+  }
+  hipEvent_t e = nullptr;
+  (void)hipEventCreate(&e);
+  return e;
+}
+
+// Folds finished event pairs into the per-name totals (waits for them).
+void prof_drain() {
+  for (ProfPending& p : g_prof_pending) {
+    float ms = 0.f;
+    if (p.start && p.stop && hipEventSynchronize(p.stop) == hipSuccess &&
+        hipEventElapsedTime(&ms, p.start, p.stop) == hipSuccess) {
+      ProfTotal* t = nullptr;
+      for (ProfTotal& x : g_prof_totals)
+        if (x.name == p.name) t = &x;
+      if (!t) {
+        g_prof_totals.push_back(ProfTotal{p.name, 0, 0.0});
+        t = &g_prof_totals.back();
+      }
+      t->calls += 1;
+      t->ms += ms;
+    }
+    if (p.start) g_prof_pool.push_back(p.start);
+    if (p.stop) g_prof_pool.push_back(p.stop);
+  }
+  g_prof_pending.clear();
+}
+}  // namespace
+
+bool profile_enabled() { return g_prof_on; }
+
+void profile_begin(const char* name, hipStream_t stream) {
+  std::lock_guard<std::mutex> lock(g_prof_mutex);
+  ProfPending p{name, prof_event(), prof_event()};
+  if (p.start) (void)hipEventRecord(p.start, stream);
+  g_prof_pending.push_back(p);
+}
+
+void profile_end(hipStream_t stream) {
+  std::lock_guard<std::mutex> lock(g_prof_mutex);
+  if (g_prof_pending.empty()) return;
+  ProfPending& p = g_prof_pending.back();
+  if (p.stop) (void)hipEventRecord(p.stop, stream);
+  if (g_prof_pending.size() >= 4096) prof_drain();
 }
 
 // ------------------------------------------------------------------ scan
@@ -98,14 +169,15 @@ int exclusive_scan_i64(const int64_t* in, int64_t* out, int64_t n, void* ws,
   }
   int64_t* tile_sums = (int64_t*)ws;
   const int64_t tiles = ceil_div(n, kScanTile);
-  scan_tile_sums_kernel<<<dim3((unsigned)tiles), dim3(kBlock), 0, stream>>>(
-      in, n, tile_sums);
-  GS_LAUNCH_CHECK();
-  scan_spine_kernel<<<dim3(1), dim3(kBlock), 0, stream>>>(tile_sums, tiles);
-  GS_LAUNCH_CHECK();
-  scan_down_kernel<<<dim3((unsigned)tiles), dim3(kBlock), 0, stream>>>(
-      in, out, n, tile_sums);
-  GS_LAUNCH_CHECK();
+  GS_LAUNCH("scan_tile_sums", stream,
+            scan_tile_sums_kernel<<<dim3((unsigned)tiles), dim3(kBlock), 0,
+                                    stream>>>(in, n, tile_sums));
+  GS_LAUNCH("scan_spine", stream,
+            scan_spine_kernel<<<dim3(1), dim3(kBlock), 0, stream>>>(tile_sums,
+                                                                    tiles));
+  GS_LAUNCH("scan_down", stream,
+            scan_down_kernel<<<dim3((unsigned)tiles), dim3(kBlock), 0, stream>>>(
+                in, out, n, tile_sums));
   return GS_OK;
 }
 
@@ -116,6 +188,40 @@ extern "C" {
 const char* gs_last_error(void) { return gs::g_last_error.c_str(); }
 
 int gs_abi_version(void) { return 1; }
+
+void gs_profile_enable(int on) {
+  std::lock_guard<std::mutex> lock(gs::g_prof_mutex);
+  gs::g_prof_on = on != 0;
+}
+
+void gs_profile_reset(void) {
+  std::lock_guard<std::mutex> lock(gs::g_prof_mutex);
+  gs::prof_drain();
+  gs::g_prof_totals.clear();
+}
+
+int gs_profile_count(void) {
+  std::lock_guard<std::mutex> lock(gs::g_prof_mutex);
+  gs::prof_drain();
+  return (int)gs::g_prof_totals.size();
+}
+
+int gs_profile_get(int index, char* name, size_t name_bytes, long long* calls,
+                   double* total_ms) {
+  std::lock_guard<std::mutex> lock(gs::g_prof_mutex);
+  if (index < 0 || index >= (int)gs::g_prof_totals.size()) {
+    gs::set_error("profile_get: index %d out of range", index);
+    return GS_ERR_INVALID;
+  }
+  const auto& t = gs::g_prof_totals[(size_t)index];
+  if (name && name_bytes > 0) {
+    strncpy(name, t.name.c_str(), name_bytes - 1);
+    name[name_bytes - 1] = 0;
+  }
+  if (calls) *calls = t.calls;
+  if (total_ms) *total_ms = t.ms;
+  return GS_OK;
+}
 
 size_t gs_scan_workspace_bytes(int64_t n) { return gs::scan_workspace_bytes(n); }
 

@@ -124,10 +124,12 @@ static int launch_sample_uniform(const int64_t* indptr, int64_t num_cols,
                                  int64_t* out_coo_col, int64_t* out_indices,
                                  int64_t* out_select, hipStream_t stream) {
   const int64_t blocks = ceil_div(num_items * G, kBlock);
-  sample_uniform_kernel<G><<<dim3((unsigned)blocks), dim3(kBlock), 0, stream>>>(
-      indptr, num_cols, indices, column_ids, num_items, fanout, replace, algo,
-      key, sub_indptr, out_coo_col, out_indices, out_select);
-  GS_LAUNCH_CHECK();
+  GS_LAUNCH("sample_uniform", stream,
+            sample_uniform_kernel<G><<<dim3((unsigned)blocks), dim3(kBlock), 0,
+                                       stream>>>(
+                indptr, num_cols, indices, column_ids, num_items, fanout,
+                replace, algo, key, sub_indptr, out_coo_col, out_indices,
+                out_select));
   return GS_OK;
 }
 

@@ -32,8 +32,7 @@ __global__ __launch_bounds__(kBlock) void col_count_kernel(
 // independent of the degree distribution; reads within a column and all
 // writes are coalesced.
 __global__ __launch_bounds__(kBlock) void col_slice_fill_kernel(
-    const int64_t* __restrict__ indptr, int64_t num_cols,
-    const int64_t* __restrict__ indices, const int64_t* __restrict__ column_ids,
+    const int64_t* __restrict__ indptr, const int64_t* __restrict__ indices, const int64_t* __restrict__ column_ids,
     int64_t num_items, const int64_t* __restrict__ sub_indptr, int64_t nnz,
     const int64_t* __restrict__ batch_ptr, int64_t num_batches,
     int64_t encode_stride, int64_t* __restrict__ out_coo_col,
@@ -68,9 +67,10 @@ int gs_csc_col_count(const int64_t* indptr, int64_t num_cols,
              (long long)num_items, (long long)num_cols);
   hipStream_t s = as_stream(stream);
   const int64_t n = num_items + 1;
-  col_count_kernel<<<dim3((unsigned)ceil_div(n, kBlock)), dim3(kBlock), 0, s>>>(
-      indptr, num_cols, column_ids, num_items, fanout, replace, sub_indptr);
-  GS_LAUNCH_CHECK();
+  GS_LAUNCH("col_count", s,
+            col_count_kernel<<<dim3((unsigned)ceil_div(n, kBlock)), dim3(kBlock),
+                               0, s>>>(indptr, num_cols, column_ids, num_items,
+                                       fanout, replace, sub_indptr));
   return exclusive_scan_i64(sub_indptr, sub_indptr, n, workspace,
                             workspace_bytes, s);
 }
@@ -90,13 +90,13 @@ int gs_csc_col_slice_fill(const int64_t* indptr, int64_t num_cols,
   GS_REQUIRE(batch_ptr == nullptr || num_batches > 0,
              "col_slice_fill: batch_ptr given but num_batches = %lld",
              (long long)num_batches);
-  (void)num_cols;
-  col_slice_fill_kernel<<<dim3((unsigned)ceil_div(nnz, kBlock)), dim3(kBlock), 0,
-                          as_stream(stream)>>>(
-      indptr, num_cols, indices, column_ids, num_items, sub_indptr, nnz,
-      batch_ptr, num_batches, encode_stride, out_coo_col, out_indices,
-      out_select);
-  GS_LAUNCH_CHECK();
+  hipStream_t s = as_stream(stream);
+  GS_LAUNCH("col_slice_fill", s,
+            col_slice_fill_kernel<<<dim3((unsigned)ceil_div(nnz, kBlock)),
+                                    dim3(kBlock), 0, s>>>(
+                indptr, indices, column_ids, num_items, sub_indptr, nnz,
+                batch_ptr, num_batches, encode_stride, out_coo_col, out_indices,
+                out_select));
   return GS_OK;
 }
 

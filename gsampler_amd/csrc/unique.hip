@@ -299,35 +299,38 @@ int gs_unique_count(const int64_t* seeds, const int64_t* seeds_ptr,
   hipStream_t s = as_stream(stream);
   const int64_t N = S + E;
   if (N == 0) {
-    unique_clear_kernel<<<dim3((unsigned)ceil_div(B + 1, kBlock)), dim3(kBlock),
-                          0, s>>>((uint64_t*)unique_ptr, B + 1, 0ull);
-    GS_LAUNCH_CHECK();
+    GS_LAUNCH("unique_clear", s,
+              unique_clear_kernel<<<dim3((unsigned)ceil_div(B + 1, kBlock)),
+                                    dim3(kBlock), 0, s>>>((uint64_t*)unique_ptr,
+                                                          B + 1, 0ull));
     return GS_OK;
   }
   const int64_t nblocks = ceil_div(N, kBlock);
-  unique_flat_ptr_kernel<<<dim3((unsigned)ceil_div(B + 1, kBlock)), dim3(kBlock),
-                           0, s>>>(seeds_ptr, S, rows_ptr, E, B, w.flat_ptr);
-  GS_LAUNCH_CHECK();
+  GS_LAUNCH("unique_flat_ptr", s,
+            unique_flat_ptr_kernel<<<dim3((unsigned)ceil_div(B + 1, kBlock)),
+                                     dim3(kBlock), 0, s>>>(seeds_ptr, S, rows_ptr,
+                                                           E, B, w.flat_ptr));
   {
     const int64_t slots = 2 * N;
     int64_t blocks = ceil_div(slots, kBlock * 8);
-    unique_clear_kernel<<<dim3((unsigned)blocks), dim3(kBlock), 0, s>>>(
-        w.table, slots, kEmptySlot);
-    GS_LAUNCH_CHECK();
+    GS_LAUNCH("unique_clear", s,
+              unique_clear_kernel<<<dim3((unsigned)blocks), dim3(kBlock), 0, s>>>(
+                  w.table, slots, kEmptySlot));
   }
-  unique_insert_kernel<<<dim3((unsigned)nblocks), dim3(kBlock), 0, s>>>(
-      w.flat_ptr, B, seeds, seeds_ptr, S, rows, rows_ptr, N, w.table);
-  GS_LAUNCH_CHECK();
-  unique_flag_kernel<<<dim3((unsigned)nblocks), dim3(kBlock), 0, s>>>(
-      w.flat_ptr, B, seeds, seeds_ptr, S, rows, rows_ptr, N, w.table, w.flags,
-      w.block_off);
-  GS_LAUNCH_CHECK();
+  GS_LAUNCH("unique_insert", s,
+            unique_insert_kernel<<<dim3((unsigned)nblocks), dim3(kBlock), 0, s>>>(
+                w.flat_ptr, B, seeds, seeds_ptr, S, rows, rows_ptr, N, w.table));
+  GS_LAUNCH("unique_flag", s,
+            unique_flag_kernel<<<dim3((unsigned)nblocks), dim3(kBlock), 0, s>>>(
+                w.flat_ptr, B, seeds, seeds_ptr, S, rows, rows_ptr, N, w.table,
+                w.flags, w.block_off));
   rc = exclusive_scan_i64(w.block_off, w.block_off, nblocks + 1, w.scan_ws,
                           w.scan_ws_bytes, s);
   if (rc != GS_OK) return rc;
-  unique_ptr_kernel<<<dim3((unsigned)ceil_div(B + 1, kBlock)), dim3(kBlock), 0,
-                      s>>>(w.flat_ptr, B, w.flags, w.block_off, unique_ptr);
-  GS_LAUNCH_CHECK();
+  GS_LAUNCH("unique_ptr", s,
+            unique_ptr_kernel<<<dim3((unsigned)ceil_div(B + 1, kBlock)),
+                                dim3(kBlock), 0, s>>>(w.flat_ptr, B, w.flags,
+                                                      w.block_off, unique_ptr));
   return GS_OK;
 }
 
@@ -355,16 +358,16 @@ int gs_unique_fill(const int64_t* seeds, const int64_t* seeds_ptr,
   GS_REQUIRE(out_unique, "unique_fill: null out_unique");
   hipStream_t s = as_stream(stream);
   const int64_t nblocks = ceil_div(N, kBlock);
-  unique_fill_kernel<<<dim3((unsigned)nblocks), dim3(kBlock), 0, s>>>(
-      w.flat_ptr, B, seeds, seeds_ptr, S, rows, rows_ptr, N, w.table, w.flags,
-      w.block_off, unique_ptr, out_unique, w.seed_rank);
-  GS_LAUNCH_CHECK();
+  GS_LAUNCH("unique_fill", s,
+            unique_fill_kernel<<<dim3((unsigned)nblocks), dim3(kBlock), 0, s>>>(
+                w.flat_ptr, B, seeds, seeds_ptr, S, rows, rows_ptr, N, w.table,
+                w.flags, w.block_off, unique_ptr, out_unique, w.seed_rank));
   if (E > 0 && (out_row || out_col)) {
-    unique_relabel_kernel<<<dim3((unsigned)ceil_div(E, kBlock)), dim3(kBlock), 0,
-                            s>>>(w.flat_ptr, B, seeds, rows, rows_ptr, E,
-                                 w.table, w.seed_rank, edge_col, out_row,
-                                 out_col);
-    GS_LAUNCH_CHECK();
+    GS_LAUNCH("unique_relabel", s,
+              unique_relabel_kernel<<<dim3((unsigned)ceil_div(E, kBlock)),
+                                      dim3(kBlock), 0, s>>>(
+                  w.flat_ptr, B, seeds, rows, rows_ptr, E, w.table, w.seed_rank,
+                  edge_col, out_row, out_col));
   }
   return GS_OK;
 }

@@ -50,6 +50,18 @@ const char* gs_last_error(void);
 int gs_abi_version(void);
 
 /* ------------------------------------------------------------------------
+ * Per-kernel timing with HIP events on the launch stream (measurement aid; no
+ * counterpart in the reference, which is profiled externally with Nsight).
+ * While enabled every kernel launch is bracketed by two events; totals are
+ * kept per kernel name.  gs_profile_count() waits for outstanding events.
+ * ---------------------------------------------------------------------- */
+void gs_profile_enable(int on);
+void gs_profile_reset(void);
+int gs_profile_count(void);
+int gs_profile_get(int index, char* name, size_t name_bytes, long long* calls,
+                   double* total_ms);
+
+/* ------------------------------------------------------------------------
  * Exclusive prefix sum of n int64 values, in place allowed (in == out).
  * Stands in for cub_exclusiveSum, src/cuda/utils.h:18-28.
  * ---------------------------------------------------------------------- */
