@@ -51,8 +51,13 @@ SIGNATURES = {
                                               _p]),
     "gs_unique_workspace_bytes": (_sz, [_i64, _i64, _i64]),
     "gs_unique_count": (_int, [_p, _p, _i64, _p, _p, _i64, _i64, _p, _p, _sz, _p]),
-    "gs_unique_fill": (_int, [_p, _p, _i64, _p, _p, _i64, _i64, _p, _p, _p, _p,
-                              _p, _p, _sz, _p]),
+    "gs_unique_fill": (_int, [_p, _p, _i64, _p, _p, _i64, _i64, _p, _p, _p, _sz, _p]),
+    "gs_unique_relabel": (_int, [_p, _p, _i64, _p, _p, _i64, _i64, _p, _p, _p, _p,
+                                 _sz, _p]),
+    "gs_csc2coo": (_int, [_p, _i64, _i64, _p, _p]),
+    "gs_sorted_to_indptr": (_int, [_p, _i64, _i64, _p, _p]),
+    "gs_decode_batch_ids": (_int, [_p, _i64, _i64, _p, _p, _p]),
+    "gs_split_indptr": (_int, [_p, _p, _i64, _i64, _p, _p]),
 }
 
 _lib = None
@@ -238,7 +243,48 @@ def unique_relabel(seeds, rows, seeds_ptr=None, rows_ptr=None, edge_col=None,
     if edge_col is not None:
         edge_col = _i64t(edge_col, "edge_col")
     check(l.gs_unique_fill(_ptr(seeds), sp, S, _ptr(rows), rp, E, B,
-                           unique_ptr.data_ptr(), _ptr(edge_col), _ptr(unique),
-                           _ptr(out_row), _ptr(out_col), ws.data_ptr(), ws.numel(),
-                           _stream()))
+                           unique_ptr.data_ptr(), _ptr(unique), ws.data_ptr(),
+                           ws.numel(), _stream()))
+    if want_row or want_col:
+        check(l.gs_unique_relabel(_ptr(seeds), sp, S, _ptr(rows), rp, E, B,
+                                  _ptr(edge_col), _ptr(out_row), _ptr(out_col),
+                                  ws.data_ptr(), ws.numel(), _stream()))
     return unique, unique_ptr, out_row, out_col
+
+
+def csc2coo(indptr: torch.Tensor, nnz: Optional[int] = None) -> torch.Tensor:
+    """Column id of every edge of a CSC matrix."""
+    indptr = _i64t(indptr, "indptr")
+    if nnz is None:
+        nnz = int(indptr[-1].item())
+    out = torch.empty(nnz, dtype=torch.int64, device=indptr.device)
+    check(lib().gs_csc2coo(_ptr(indptr), indptr.numel() - 1, nnz, _ptr(out), _stream()))
+    return out
+
+
+def sorted_to_indptr(sorted_ids: torch.Tensor, num_cols: int) -> torch.Tensor:
+    sorted_ids = _i64t(sorted_ids, "sorted_ids")
+    out = torch.empty(num_cols + 1, dtype=torch.int64, device=sorted_ids.device)
+    check(lib().gs_sorted_to_indptr(_ptr(sorted_ids), sorted_ids.numel(), num_cols,
+                                    out.data_ptr(), _stream()))
+    return out
+
+
+def decode_batch_ids(encoded: torch.Tensor, stride: int):
+    """-> (orig, batch) for ids encoded as id + batch * stride."""
+    encoded = _i64t(encoded, "encoded")
+    orig, batch = torch.empty_like(encoded), torch.empty_like(encoded)
+    check(lib().gs_decode_batch_ids(_ptr(encoded), encoded.numel(), stride,
+                                    _ptr(orig), _ptr(batch), _stream()))
+    return orig, batch
+
+
+def split_indptr(indptr: torch.Tensor, offset: torch.Tensor) -> torch.Tensor:
+    """Per-batch indptr arrays rebased to 0, concatenated."""
+    indptr, offset = _i64t(indptr, "indptr"), _i64t(offset, "offset")
+    nb = offset.numel() - 1
+    total = int((offset[-1] - offset[0]).item()) + nb
+    out = torch.empty(total, dtype=torch.int64, device=indptr.device)
+    check(lib().gs_split_indptr(_ptr(indptr), _ptr(offset), nb, total, _ptr(out),
+                                _stream()))
+    return out

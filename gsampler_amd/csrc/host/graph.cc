@@ -1,0 +1,372 @@
+// graph.cc -- format management and the extract / select / finalize operators
+// of gs_classes.Graph.  Each operator validates its tensors, sizes outputs and
+// workspaces through torch, and calls the C ABI on the current HIP stream.
+#include "graph.h"
+
+#include "abi_call.h"
+
+namespace gs {
+
+RandomState& random_state() {
+  static RandomState state;
+  return state;
+}
+
+static uint64_t next_call_id() { return random_state().next_call++; }
+
+// ------------------------------------------------------------------ loading
+void Graph::LoadCSC(torch::Tensor indptr, torch::Tensor indices) {
+  auto m = std::make_shared<Compressed>();
+  m->indptr = ids(indptr, "indptr");
+  m->indices = ids(indices, "indices");
+  TORCH_CHECK(m->indptr.numel() == num_cols_ + 1, "LoadCSC: indptr has ",
+              indptr.numel(), " entries for ", num_cols_, " columns");
+  csc_ = m;
+  num_edges_ = indices.numel();
+}
+
+void Graph::LoadCSR(torch::Tensor indptr, torch::Tensor indices) {
+  auto m = std::make_shared<Compressed>();
+  m->indptr = ids(indptr, "indptr");
+  m->indices = ids(indices, "indices");
+  TORCH_CHECK(m->indptr.numel() == num_rows_ + 1, "LoadCSR: indptr has ",
+              indptr.numel(), " entries for ", num_rows_, " rows");
+  csr_ = m;
+  num_edges_ = indices.numel();
+}
+
+void Graph::LoadCOO(torch::Tensor row, torch::Tensor col, bool row_sorted,
+                    bool col_sorted) {
+  auto m = std::make_shared<Coordinate>();
+  m->row = ids(row, "row");
+  m->col = ids(col, "col");
+  TORCH_CHECK(row.numel() == col.numel(), "LoadCOO: row and col differ in length");
+  m->row_sorted = row_sorted;
+  m->col_sorted = col_sorted;
+  coo_ = m;
+  num_edges_ = row.numel();
+}
+
+// --------------------------------------------------------- format conversion
+// CSC/CSR -> COO: the id on the compressed axis of every edge position.
+static torch::Tensor expand_indptr(const torch::Tensor& indptr, int64_t nnz) {
+  torch::Tensor out = new_ids(nnz, indptr);
+  GS_CALL(gs_csc2coo(cptr(indptr), indptr.numel() - 1, nnz, mptr(out),
+                     cur_stream()));
+  return out;
+}
+
+// COO -> CSC/CSR along `major`: stable sort by the major id (the permutation is
+// kept as e_ids, like the reference's COO2CSC, src/cuda/format_transform.cu:
+// 121-142), then indptr by binary search.
+static std::shared_ptr<Compressed> compress(const Coordinate& coo, bool by_col,
+                                            int64_t num_major) {
+  const torch::Tensor& major = by_col ? coo.col : coo.row;
+  const torch::Tensor& minor = by_col ? coo.row : coo.col;
+  const bool sorted = by_col ? coo.col_sorted : coo.row_sorted;
+  auto out = std::make_shared<Compressed>();
+  torch::Tensor sorted_major;
+  if (sorted) {
+    sorted_major = major;
+    out->indices = minor;
+    out->e_ids = coo.e_ids;
+  } else {
+    torch::Tensor perm = torch::argsort(major, /*stable=*/true, /*dim=*/0);
+    sorted_major = major.index_select(0, perm);
+    out->indices = minor.index_select(0, perm);
+    out->e_ids = coo.e_ids.has_value() ? coo.e_ids.value().index_select(0, perm)
+                                       : perm;
+  }
+  out->indptr = new_ids(num_major + 1, major);
+  GS_CALL(gs_sorted_to_indptr(cptr(sorted_major), sorted_major.numel(),
+                              num_major, mptr(out->indptr), cur_stream()));
+  return out;
+}
+
+static std::shared_ptr<Coordinate> expand(const Compressed& m, bool is_csc) {
+  auto coo = std::make_shared<Coordinate>();
+  torch::Tensor major = expand_indptr(m.indptr, m.indices.numel());
+  coo->row = is_csc ? m.indices : major;
+  coo->col = is_csc ? major : m.indices;
+  coo->e_ids = m.e_ids;
+  coo->col_sorted = is_csc;
+  coo->row_sorted = !is_csc;
+  return coo;
+}
+
+void Graph::CreateSparseFormat(int64_t format) {
+  TORCH_CHECK(csc_ || csr_ || coo_, "the graph holds no sparse format yet");
+  if (format == kCOO) {
+    if (coo_) return;
+    coo_ = csc_ ? expand(*csc_, true) : expand(*csr_, false);
+  } else if (format == kCSC) {
+    if (csc_) return;
+    if (!coo_) coo_ = expand(*csr_, false);
+    csc_ = compress(*coo_, true, num_cols_);
+  } else if (format == kCSR) {
+    if (csr_) return;
+    if (!coo_) coo_ = expand(*csc_, true);
+    csr_ = compress(*coo_, false, num_rows_);
+  } else {
+    TORCH_CHECK(false, "unsupported sparse format ", format);
+  }
+}
+
+static torch::Tensor or_empty(const c10::optional<torch::Tensor>& t) {
+  return t.has_value() ? t.value() : torch::Tensor();
+}
+
+torch::Tensor Graph::GetCSCIndptr() { CreateSparseFormat(kCSC); return csc_->indptr; }
+torch::Tensor Graph::GetCSCIndices() { CreateSparseFormat(kCSC); return csc_->indices; }
+torch::Tensor Graph::GetCSCEids() { CreateSparseFormat(kCSC); return or_empty(csc_->e_ids); }
+torch::Tensor Graph::GetCOORows() { CreateSparseFormat(kCOO); return coo_->row; }
+torch::Tensor Graph::GetCOOCols() { CreateSparseFormat(kCOO); return coo_->col; }
+torch::Tensor Graph::GetCOOEids() { CreateSparseFormat(kCOO); return or_empty(coo_->e_ids); }
+torch::Tensor Graph::GetCSRIndptr() { CreateSparseFormat(kCSR); return csr_->indptr; }
+torch::Tensor Graph::GetCSRIndices() { CreateSparseFormat(kCSR); return csr_->indices; }
+torch::Tensor Graph::GetCSREids() { CreateSparseFormat(kCSR); return or_empty(csr_->e_ids); }
+
+const Compressed& Graph::compressed(int64_t format) {
+  CreateSparseFormat(format);
+  return format == kCSC ? *csc_ : *csr_;
+}
+
+// ---------------------------------------------------- operators, major axis
+MajorResult major_slice(const Compressed& m, const torch::Tensor& picked,
+                               bool with_coo, const torch::Tensor& batch_ptr,
+                               int64_t encode_stride) {
+  const int64_t num_major = m.indptr.numel() - 1;
+  const int64_t n = picked.numel();
+  MajorResult r;
+  r.indptr = new_ids(n + 1, m.indptr);
+  torch::Tensor ws = new_workspace(gs_scan_workspace_bytes(n + 1), m.indptr);
+  GS_CALL(gs_csc_col_count(cptr(m.indptr), num_major, cptr(picked), n, -1, 0,
+                           mptr(r.indptr), ws.data_ptr(), ws.numel(),
+                           cur_stream()));
+  const int64_t nnz = read_last(r.indptr);
+  r.minor_ids = new_ids(nnz, m.indptr);
+  r.select = new_ids(nnz, m.indptr);
+  if (with_coo) r.major_ids = new_ids(nnz, m.indptr);
+  const int64_t nb = batch_ptr.defined() ? batch_ptr.numel() - 1 : 0;
+  GS_CALL(gs_csc_col_slice_fill(
+      cptr(m.indptr), num_major, cptr(m.indices), cptr(picked), n,
+      cptr(r.indptr), nnz, nb > 0 ? cptr(batch_ptr) : nullptr, nb,
+      encode_stride, with_coo ? mptr(r.major_ids) : nullptr, mptr(r.minor_ids),
+      mptr(r.select), cur_stream()));
+  return r;
+}
+
+// picked undefined: sample every column of the matrix itself.
+MajorResult major_sample_uniform(const Compressed& m,
+                                        const torch::Tensor& picked,
+                                        int64_t fanout, bool replace,
+                                        bool with_coo) {
+  TORCH_CHECK(fanout >= 0, "fanout must be non-negative, got ", fanout);
+  const int64_t num_major = m.indptr.numel() - 1;
+  const bool fused = picked.defined();
+  const int64_t n = fused ? picked.numel() : num_major;
+  MajorResult r;
+  r.indptr = new_ids(n + 1, m.indptr);
+  torch::Tensor ws = new_workspace(gs_scan_workspace_bytes(n + 1), m.indptr);
+  GS_CALL(gs_csc_col_count(cptr(m.indptr), num_major,
+                           fused ? cptr(picked) : nullptr, n, fanout,
+                           replace ? 1 : 0, mptr(r.indptr), ws.data_ptr(),
+                           ws.numel(), cur_stream()));
+  const int64_t nnz = read_last(r.indptr);
+  r.minor_ids = new_ids(nnz, m.indptr);
+  r.select = new_ids(nnz, m.indptr);
+  if (with_coo) r.major_ids = new_ids(nnz, m.indptr);
+  const RandomState& rs = random_state();
+  GS_CALL(gs_csc_col_sample_uniform_fill(
+      cptr(m.indptr), num_major, cptr(m.indices),
+      fused ? cptr(picked) : nullptr, n, fanout, replace ? 1 : 0, (int)rs.algo,
+      rs.seed, next_call_id(), cptr(r.indptr),
+      with_coo ? mptr(r.major_ids) : nullptr, mptr(r.minor_ids), mptr(r.select),
+      cur_stream()));
+  return r;
+}
+
+// Wraps a MajorResult into a new Graph in the requested output formats
+// (bit-OR of kCOO and the format the operator ran on).
+GraphPtr Graph::derive(int64_t on_format, int64_t output_format,
+                       const MajorResult& r, int64_t new_rows,
+                       int64_t new_cols) {
+  auto g = c10::make_intrusive<Graph>(new_rows, new_cols);
+  const bool is_csc = on_format == kCSC;
+  if (output_format & on_format) {
+    auto c = std::make_shared<Compressed>();
+    c->indptr = r.indptr;
+    c->indices = r.minor_ids;
+    (is_csc ? g->csc_ : g->csr_) = c;
+  }
+  if (output_format & kCOO) {
+    auto coo = std::make_shared<Coordinate>();
+    coo->row = is_csc ? r.minor_ids : r.major_ids;
+    coo->col = is_csc ? r.major_ids : r.minor_ids;
+    coo->col_sorted = is_csc;
+    coo->row_sorted = !is_csc;
+    g->coo_ = coo;
+  }
+  g->num_edges_ = r.select.numel();
+  return g;
+}
+
+torch::Tensor Graph::edge_index(const c10::optional<torch::Tensor>& parent_eids,
+                                const torch::Tensor& select) {
+  return parent_eids.has_value() ? parent_eids.value().index_select(0, select)
+                                 : select;
+}
+
+static void check_out_format(int64_t on_format, int64_t output_format,
+                             const char* op) {
+  TORCH_CHECK(on_format == kCSC || on_format == kCSR || on_format == kCOO, op,
+              ": unknown on_format ", on_format);
+  const int64_t other = on_format == kCSC ? kCSR : kCSC;
+  TORCH_CHECK(on_format == kCOO || output_format != other, op,
+              ": on_format ", on_format, " cannot produce output_format ",
+              output_format);
+}
+
+// axis 0 = rows, axis 1 = columns (src/graph.cc:88-89 of the reference).
+GraphAndIndex Graph::Slicing(torch::Tensor seeds, int64_t axis,
+                             int64_t on_format, int64_t output_format) {
+  check_out_format(on_format, output_format, "Slicing");
+  TORCH_CHECK(axis == 0 || axis == 1, "Slicing: axis must be 0 or 1");
+  seeds = ids(seeds, "seeds");
+  const int64_t new_rows = axis == 0 ? seeds.numel() : num_rows_;
+  const int64_t new_cols = axis == 0 ? num_cols_ : seeds.numel();
+  if (on_format == kCOO) return slice_coo(seeds, axis, new_rows, new_cols);
+  const Compressed& m = compressed(on_format);
+  const bool with_coo = output_format & kCOO;
+  const bool along_major = (on_format == kCSC) == (axis == 1);
+  MajorResult r = along_major ? major_slice(m, seeds, with_coo, {}, 0)
+                              : minor_slice(m, seeds, with_coo);
+  GraphPtr g = derive(on_format, output_format, r, new_rows, new_cols);
+  return {g, edge_index(m.e_ids, r.select)};
+}
+
+GraphAndIndex Graph::Sampling(int64_t axis, int64_t fanout, bool replace,
+                              int64_t on_format, int64_t output_format) {
+  check_out_format(on_format, output_format, "Sampling");
+  TORCH_CHECK((axis == 1 && on_format == kCSC) || (axis == 0 && on_format == kCSR),
+              "Sampling: not implemented for axis ", axis, " on format ",
+              on_format);
+  const Compressed& m = compressed(on_format);
+  MajorResult r = major_sample_uniform(m, {}, fanout, replace, output_format & kCOO);
+  GraphPtr g = derive(on_format, output_format, r, num_rows_, num_cols_);
+  return {g, edge_index(m.e_ids, r.select)};
+}
+
+GraphAndIndex Graph::FusedSlicingSampling(int64_t axis, torch::Tensor seeds,
+                                          int64_t fanout, bool replace,
+                                          int64_t on_format,
+                                          int64_t output_format) {
+  check_out_format(on_format, output_format, "FusedSlicingSampling");
+  TORCH_CHECK((axis == 1 && on_format == kCSC) || (axis == 0 && on_format == kCSR),
+              "FusedSlicingSampling: not implemented for axis ", axis,
+              " on format ", on_format);
+  seeds = ids(seeds, "seeds");
+  const Compressed& m = compressed(on_format);
+  MajorResult r = major_sample_uniform(m, seeds, fanout, replace, output_format & kCOO);
+  const int64_t new_rows = axis == 0 ? seeds.numel() : num_rows_;
+  const int64_t new_cols = axis == 0 ? num_cols_ : seeds.numel();
+  GraphPtr g = derive(on_format, output_format, r, new_rows, new_cols);
+  return {g, edge_index(m.e_ids, r.select)};
+}
+
+// ------------------------------------------------------- unique and relabel
+bool Graph::Frontier::matches(const torch::Tensor& s, const torch::Tensor& r,
+                              const torch::Tensor& sp,
+                              const torch::Tensor& rp) const {
+  auto same = [](const torch::Tensor& a, const torch::Tensor& b) {
+    if (!a.defined() || !b.defined()) return a.defined() == b.defined();
+    return a.is_same(b) ||
+           (a.data_ptr() == b.data_ptr() && a.numel() == b.numel());
+  };
+  return same(seeds, s) && same(rows, r) && same(seeds_ptr, sp) &&
+         same(rows_ptr, rp) && seeds_version == (int64_t)s._version() &&
+         rows_version == (int64_t)r._version();
+}
+
+// Unique (first-occurrence order) of seeds_b ++ rows_b per batch; the hash
+// tables stay in the workspace for the relabel pass.
+Graph::Frontier& Graph::frontier_for(const torch::Tensor& seeds,
+                                     const torch::Tensor& rows,
+                                     const torch::Tensor& seeds_ptr,
+                                     const torch::Tensor& rows_ptr) {
+  if (frontier_ && frontier_->matches(seeds, rows, seeds_ptr, rows_ptr))
+    return *frontier_;
+  auto f = std::make_unique<Frontier>();
+  f->seeds = seeds;
+  f->rows = rows;
+  f->seeds_ptr = seeds_ptr;
+  f->rows_ptr = rows_ptr;
+  f->seeds_version = seeds._version();
+  f->rows_version = rows._version();
+  const int64_t B = seeds_ptr.defined() ? seeds_ptr.numel() - 1 : 1;
+  TORCH_CHECK(B >= 1, "unique: at least one batch is required");
+  f->num_batches = B;
+  const int64_t S = seeds.numel(), E = rows.numel();
+  f->workspace = new_workspace(gs_unique_workspace_bytes(S, E, B), rows);
+  f->unique_ptr = new_ids(B + 1, rows);
+  GS_CALL(gs_unique_count(cptr(seeds), cptr(seeds_ptr), S, cptr(rows),
+                          cptr(rows_ptr), E, B, mptr(f->unique_ptr),
+                          f->workspace.data_ptr(), f->workspace.numel(),
+                          cur_stream()));
+  const int64_t U = read_last(f->unique_ptr);
+  f->unique = new_ids(U, rows);
+  GS_CALL(gs_unique_fill(cptr(seeds), cptr(seeds_ptr), S, cptr(rows),
+                         cptr(rows_ptr), E, B, cptr(f->unique_ptr),
+                         mptr(f->unique), f->workspace.data_ptr(),
+                         f->workspace.numel(), cur_stream()));
+  frontier_ = std::move(f);
+  return *frontier_;
+}
+
+// row_ids[base] when row_ids is non-empty (rows of a compacted or row-sliced
+// matrix are local ids), else base.  The gathered tensor is kept so that
+// all_nodes() and to_dgl_block() on the same matrix share one frontier.
+torch::Tensor Graph::mapped_rows(const torch::Tensor& base,
+                                 const torch::Tensor& row_ids) {
+  if (row_ids.numel() == 0) return base;
+  torch::Tensor table = ids(row_ids, "row_ids");
+  if (!(mapped_out_.defined() && mapped_from_.is_same(base) &&
+        mapped_by_.is_same(row_ids))) {
+    mapped_out_ = table.index_select(0, base);
+    mapped_from_ = base;
+    mapped_by_ = row_ids;
+  }
+  return mapped_out_;
+}
+
+std::tuple<torch::Tensor, torch::Tensor, torch::Tensor,
+           c10::optional<torch::Tensor>>
+Graph::GraphRelabel(torch::Tensor col_seeds, torch::Tensor row_ids) {
+  CreateSparseFormat(kCOO);
+  col_seeds = ids(col_seeds, "col_seeds");
+  TORCH_CHECK(col_seeds.numel() > 0 || coo_->col.numel() == 0,
+              "GraphRelabel: the matrix has edges but col_seeds is empty");
+  torch::Tensor rows = mapped_rows(coo_->row, row_ids);
+  Frontier& f = frontier_for(col_seeds, rows, {}, {});
+  const int64_t E = rows.numel();
+  torch::Tensor out_row = new_ids(E, rows), out_col = new_ids(E, rows);
+  GS_CALL(gs_unique_relabel(cptr(col_seeds), nullptr, col_seeds.numel(),
+                            cptr(rows), nullptr, E, 1, cptr(coo_->col),
+                            mptr(out_row), mptr(out_col),
+                            f.workspace.data_ptr(), f.workspace.numel(),
+                            cur_stream()));
+  return {f.unique, out_row, out_col, coo_->e_ids};
+}
+
+torch::Tensor Graph::GetValidNodes(torch::Tensor col_seeds,
+                                   torch::Tensor row_ids) {
+  col_seeds = ids(col_seeds, "col_seeds");
+  // Row ids in CSC order equal the column-sorted COO rows, so both formats
+  // give the same first-occurrence order (src/graph.cc:593-608).
+  if (!csc_) CreateSparseFormat(kCOO);
+  const torch::Tensor& base = csc_ ? csc_->indices : coo_->row;
+  torch::Tensor rows = mapped_rows(base, row_ids);
+  return frontier_for(col_seeds, rows, {}, {}).unique;
+}
+
+}  // namespace gs

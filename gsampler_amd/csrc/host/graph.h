@@ -1,0 +1,223 @@
+// graph.h -- the `gs_classes.Graph` operator object: one sparse matrix held in
+// up to three formats, plus the super-batch bookkeeping.  Method names,
+// argument order and return shapes follow the reference's class
+// (src/graph.h:11-232 of gSampler) because its Python layer and JIT address
+// them by name and position; the bodies call the C ABI of gsampler_hip.h.
+#ifndef GS_HOST_GRAPH_H_
+#define GS_HOST_GRAPH_H_
+
+#include <torch/custom_class.h>
+#include <torch/script.h>
+
+#include <memory>
+#include <string>
+#include <tuple>
+#include <vector>
+
+namespace gs {
+
+// Format bit flags (src/graph_storage.h:31-33).
+constexpr int64_t kCOO = 1, kCSC = 2, kCSR = 4;
+
+// CSC or CSR: `indptr` over the compressed ("major") axis, `indices` holds the
+// ids on the other ("minor") axis.
+struct Compressed {
+  torch::Tensor indptr, indices;
+  c10::optional<torch::Tensor> e_ids;
+};
+
+struct Coordinate {
+  torch::Tensor row, col;
+  c10::optional<torch::Tensor> e_ids;
+  bool row_sorted = false, col_sorted = false;
+};
+
+// Output of an operator that works along the compressed axis.
+struct MajorResult {
+  torch::Tensor indptr;     // [items + 1]
+  torch::Tensor major_ids;  // local id on the compressed axis per edge (COO), may be undefined
+  torch::Tensor minor_ids;  // id on the other axis per edge
+  torch::Tensor select;     // position of the edge in the parent's `indices`
+};
+
+// Process-wide sampler state: every sampling call consumes one call id, so
+// successive layers / epochs draw from disjoint Philox streams while a fixed
+// seed reproduces a whole run.
+struct RandomState {
+  uint64_t seed = 7777;  // the reference's literal, src/cuda/sampling.cu:143
+  uint64_t next_call = 0;
+  int64_t algo = 0;      // GS_ALGO_AUTO
+};
+RandomState& random_state();
+
+class Graph;
+using GraphPtr = c10::intrusive_ptr<Graph>;
+using GraphAndIndex = std::tuple<GraphPtr, torch::Tensor>;
+
+class Graph : public torch::CustomClassHolder {
+ public:
+  Graph(int64_t num_rows, int64_t num_cols)
+      : num_rows_(num_rows), num_cols_(num_cols) {}
+
+  // ---- loading and inspection
+  void LoadCSC(torch::Tensor indptr, torch::Tensor indices);
+  void LoadCOO(torch::Tensor row, torch::Tensor col, bool row_sorted,
+               bool col_sorted);
+  void LoadCSR(torch::Tensor indptr, torch::Tensor indices);
+  int64_t GetNumRows() { return num_rows_; }
+  int64_t GetNumCols() { return num_cols_; }
+  int64_t GetNumEdges() { return num_edges_; }
+  torch::Tensor GetCSCIndptr();
+  torch::Tensor GetCSCIndices();
+  torch::Tensor GetCSCEids();
+  torch::Tensor GetCOORows();
+  torch::Tensor GetCOOCols();
+  torch::Tensor GetCOOEids();
+  torch::Tensor GetCSRIndptr();
+  torch::Tensor GetCSRIndices();
+  torch::Tensor GetCSREids();
+  void CreateSparseFormat(int64_t format);
+
+  // ---- extract / select operators
+  GraphAndIndex Slicing(torch::Tensor seeds, int64_t axis, int64_t on_format,
+                        int64_t output_format);
+  GraphAndIndex Sampling(int64_t axis, int64_t fanout, bool replace,
+                         int64_t on_format, int64_t output_format);
+  GraphAndIndex SamplingProbs(int64_t axis, torch::Tensor edge_probs,
+                              int64_t fanout, bool replace, int64_t on_format,
+                              int64_t output_format);
+  GraphAndIndex FusedSlicingSampling(int64_t axis, torch::Tensor seeds,
+                                     int64_t fanout, bool replace,
+                                     int64_t on_format, int64_t output_format);
+  GraphAndIndex Compact(int64_t axis);
+  torch::Tensor RandomWalk(torch::Tensor seeds, int64_t walk_length);
+  torch::Tensor Node2Vec(torch::Tensor seeds, int64_t walk_length, double p,
+                         double q);
+  void SortCSCIndices();
+
+  // ---- compute operators
+  void SDDMM(const std::string& op, torch::Tensor lhs, torch::Tensor rhs,
+             torch::Tensor out, int64_t lhs_target, int64_t rhs_target,
+             int64_t on_format);
+  void SpMM(const std::string& op, const std::string& reduce,
+            torch::Tensor ufeat, torch::Tensor efeat, torch::Tensor out,
+            torch::Tensor argu, torch::Tensor arge, int64_t u_target,
+            int64_t on_format);
+  void FusedUOPV(const std::string& op, torch::Tensor lhs1, torch::Tensor rhs1,
+                 torch::Tensor out1, torch::Tensor lhs2, torch::Tensor rhs2,
+                 torch::Tensor out2, int64_t on_format);
+  void FusedESquareSum(const std::string& op, const std::string& reduce,
+                       torch::Tensor ufeat, torch::Tensor efeat,
+                       torch::Tensor out, torch::Tensor argu,
+                       torch::Tensor arge, int64_t u_target, int64_t on_format);
+  void FusedEDivUSum(const std::string& op, const std::string& reduce,
+                     torch::Tensor ufeat, torch::Tensor efeat,
+                     torch::Tensor out, torch::Tensor argu, torch::Tensor arge,
+                     int64_t u_target, int64_t on_format);
+
+  // ---- finalize operators
+  std::tuple<torch::Tensor, torch::Tensor, torch::Tensor,
+             c10::optional<torch::Tensor>>
+  GraphRelabel(torch::Tensor col_seeds, torch::Tensor row_ids);
+  torch::Tensor GetValidNodes(torch::Tensor col_seeds, torch::Tensor row_ids);
+
+  // ---- super-batch interface
+  void SetEdgeBptr(torch::Tensor p) { edge_bptr_ = p; }
+  void SetColBptr(torch::Tensor p) { col_bptr_ = p; }
+  void SetRowBptr(torch::Tensor p) { row_bptr_ = p; }
+  void SetOrigRowIds(torch::Tensor t) { orig_row_ids_ = t; }
+  void SetOrigColIds(torch::Tensor t) { orig_col_ids_ = t; }
+  torch::Tensor GetEdgeBptr() { return edge_bptr_; }
+  torch::Tensor GetColBptr() { return col_bptr_; }
+  torch::Tensor GetRowBptr() { return row_bptr_; }
+  std::tuple<torch::Tensor, torch::Tensor> BatchGetRows() {
+    return {orig_row_ids_, row_bptr_};
+  }
+  std::tuple<torch::Tensor, torch::Tensor> BatchGetCols() {
+    return {orig_col_ids_, col_bptr_};
+  }
+  std::tuple<torch::Tensor, torch::Tensor> BatchGetCSCIndptr();
+  std::tuple<torch::Tensor, torch::Tensor> BatchGetCSCIndices();
+  std::tuple<torch::Tensor, torch::Tensor> BatchGetCSCEids();
+  std::tuple<torch::Tensor, torch::Tensor> BatchGetCOORows();
+  std::tuple<torch::Tensor, torch::Tensor> BatchGetCOOCols();
+  std::tuple<torch::Tensor, torch::Tensor> BatchGetCOOEids();
+  std::vector<int64_t> BatchGetColCounts();
+  GraphAndIndex BatchColSlicing(torch::Tensor seeds, torch::Tensor col_bptr,
+                                bool encoding);
+  GraphAndIndex BatchColRowSlcing(torch::Tensor col, torch::Tensor col_bptr,
+                                  torch::Tensor row, torch::Tensor row_bptr);
+  GraphAndIndex BatchRowSlicing(torch::Tensor row_ids, torch::Tensor row_bptr);
+  GraphAndIndex BatchRowSampling(int64_t fanout, bool replace);
+  GraphAndIndex BatchRowSamplingProbs(int64_t fanout, bool replace,
+                                      torch::Tensor edge_probs);
+  GraphAndIndex BatchFusedSlicingSampling(torch::Tensor seeds,
+                                          torch::Tensor col_bptr,
+                                          int64_t fanout, bool replace);
+  std::tuple<torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor,
+             c10::optional<torch::Tensor>, torch::Tensor>
+  BatchGraphRelabel(torch::Tensor col_seeds, torch::Tensor row_ids);
+  std::tuple<torch::Tensor, torch::Tensor> BatchGetValidNodes(
+      torch::Tensor col_seeds, torch::Tensor row_ids);
+
+ private:
+  // Unique/relabel state shared by all_nodes() and to_dgl_block(): the
+  // frontier is computed once, the relabel pass reuses the hash tables.
+  struct Frontier {
+    torch::Tensor seeds, rows, seeds_ptr, rows_ptr;  // the keys it was built from
+    int64_t seeds_version = -1, rows_version = -1;
+    torch::Tensor workspace, unique, unique_ptr;
+    int64_t num_batches = 0;
+    bool matches(const torch::Tensor& s, const torch::Tensor& r,
+                 const torch::Tensor& sp, const torch::Tensor& rp) const;
+  };
+  Frontier& frontier_for(const torch::Tensor& seeds, const torch::Tensor& rows,
+                         const torch::Tensor& seeds_ptr,
+                         const torch::Tensor& rows_ptr);
+
+  const Compressed& compressed(int64_t format);
+  torch::Tensor mapped_rows(const torch::Tensor& base, const torch::Tensor& row_ids);
+  GraphAndIndex slice_coo(const torch::Tensor& seeds, int64_t axis,
+                          int64_t new_rows, int64_t new_cols);
+  GraphPtr derive(int64_t on_format, int64_t output_format,
+                  const MajorResult& r, int64_t new_rows, int64_t new_cols);
+  torch::Tensor edge_index(const c10::optional<torch::Tensor>& parent_eids,
+                           const torch::Tensor& select);
+  void copy_batch_state_to(Graph& g, bool with_rows);
+  torch::Tensor batch_rows_for_relabel(const torch::Tensor& row_ids);
+
+  int64_t num_rows_ = 0, num_cols_ = 0, num_edges_ = 0;
+  std::shared_ptr<Compressed> csc_, csr_;
+  std::shared_ptr<Coordinate> coo_;
+  torch::Tensor col_bptr_, row_bptr_, edge_bptr_;
+  torch::Tensor orig_row_ids_, orig_col_ids_;
+  int64_t row_encoding_size_ = 0;
+  std::unique_ptr<Frontier> frontier_;
+  torch::Tensor mapped_out_, mapped_from_, mapped_by_;
+};
+
+// Operators along the compressed axis (graph.cc) and across it (slicing.cc).
+MajorResult major_slice(const Compressed& m, const torch::Tensor& picked,
+                        bool with_coo, const torch::Tensor& batch_ptr,
+                        int64_t encode_stride);
+MajorResult major_sample_uniform(const Compressed& m, const torch::Tensor& picked,
+                                 int64_t fanout, bool replace, bool with_coo);
+MajorResult minor_slice(const Compressed& m, const torch::Tensor& picked,
+                        bool with_coo);
+
+// ---- free operators (gs_ops)
+torch::Tensor ListSampling(int64_t num_items, int64_t num_picks, bool replace);
+torch::Tensor ListSamplingProbs(torch::Tensor probs, int64_t num_picks,
+                                bool replace);
+std::tuple<torch::Tensor, torch::Tensor> BatchListSamplingProbs(
+    torch::Tensor probs, int64_t num_picks, bool replace, torch::Tensor range);
+std::tuple<torch::Tensor, torch::Tensor> BatchListSampling(
+    int64_t num_picks, bool replace, torch::Tensor range);
+std::vector<torch::Tensor> SplitByOffset(torch::Tensor data,
+                                         torch::Tensor offset);
+std::vector<torch::Tensor> SplitIndptrByOffset(torch::Tensor indptr,
+                                               torch::Tensor offset);
+
+}  // namespace gs
+
+#endif  // GS_HOST_GRAPH_H_

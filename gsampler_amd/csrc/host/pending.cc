@@ -1,0 +1,70 @@
+// pending.cc -- operators of the reference interface whose kernels are not
+// built yet.  Each raises a clear error instead of computing on a fallback
+// path.  This file shrinks as kernels land.
+#include "abi_call.h"
+#include "graph.h"
+
+namespace gs {
+
+#define GS_PENDING(what) \
+  TORCH_CHECK(false, what, " is not implemented in this build of gsampler_amd")
+
+MajorResult minor_slice(const Compressed&, const torch::Tensor&, bool) {
+  GS_PENDING("slicing across the compressed axis");
+}
+GraphAndIndex Graph::slice_coo(const torch::Tensor&, int64_t, int64_t, int64_t) {
+  GS_PENDING("COO slicing");
+}
+GraphAndIndex Graph::SamplingProbs(int64_t, torch::Tensor, int64_t, bool, int64_t,
+                                   int64_t) {
+  GS_PENDING("weighted per-column sampling");
+}
+GraphAndIndex Graph::Compact(int64_t) { GS_PENDING("Compact"); }
+torch::Tensor Graph::RandomWalk(torch::Tensor, int64_t) { GS_PENDING("RandomWalk"); }
+torch::Tensor Graph::Node2Vec(torch::Tensor, int64_t, double, double) {
+  GS_PENDING("Node2Vec");
+}
+void Graph::SortCSCIndices() { GS_PENDING("SortCSCIndices"); }
+void Graph::SDDMM(const std::string&, torch::Tensor, torch::Tensor, torch::Tensor,
+                  int64_t, int64_t, int64_t) {
+  GS_PENDING("SDDMM");
+}
+void Graph::SpMM(const std::string&, const std::string&, torch::Tensor,
+                 torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor,
+                 int64_t, int64_t) {
+  GS_PENDING("SpMM");
+}
+void Graph::FusedUOPV(const std::string&, torch::Tensor, torch::Tensor,
+                      torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor,
+                      int64_t) {
+  GS_PENDING("FusedUOPV");
+}
+void Graph::FusedESquareSum(const std::string&, const std::string&, torch::Tensor,
+                            torch::Tensor, torch::Tensor, torch::Tensor,
+                            torch::Tensor, int64_t, int64_t) {
+  GS_PENDING("FusedESquareSum");
+}
+void Graph::FusedEDivUSum(const std::string&, const std::string&, torch::Tensor,
+                          torch::Tensor, torch::Tensor, torch::Tensor,
+                          torch::Tensor, int64_t, int64_t) {
+  GS_PENDING("FusedEDivUSum");
+}
+GraphAndIndex Graph::BatchColRowSlcing(torch::Tensor, torch::Tensor, torch::Tensor,
+                                       torch::Tensor) {
+  GS_PENDING("BatchColRowSlcing");
+}
+torch::Tensor ListSampling(int64_t, int64_t, bool) { GS_PENDING("ListSampling"); }
+torch::Tensor ListSamplingProbs(torch::Tensor, int64_t, bool) {
+  GS_PENDING("ListSamplingProbs");
+}
+std::tuple<torch::Tensor, torch::Tensor> BatchListSamplingProbs(torch::Tensor,
+                                                                int64_t, bool,
+                                                                torch::Tensor) {
+  GS_PENDING("BatchListSamplingProbs");
+}
+std::tuple<torch::Tensor, torch::Tensor> BatchListSampling(int64_t, bool,
+                                                           torch::Tensor) {
+  GS_PENDING("BatchListSampling");
+}
+
+}  // namespace gs

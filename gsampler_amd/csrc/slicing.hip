@@ -90,6 +90,7 @@ int gs_csc_col_slice_fill(const int64_t* indptr, int64_t num_cols,
   GS_REQUIRE(batch_ptr == nullptr || num_batches > 0,
              "col_slice_fill: batch_ptr given but num_batches = %lld",
              (long long)num_batches);
+  (void)num_cols;  // ids were validated by the count phase
   hipStream_t s = as_stream(stream);
   GS_LAUNCH("col_slice_fill", s,
             col_slice_fill_kernel<<<dim3((unsigned)ceil_div(nnz, kBlock)),

@@ -338,16 +338,13 @@ int gs_unique_fill(const int64_t* seeds, const int64_t* seeds_ptr,
                    int64_t num_seeds, const int64_t* rows,
                    const int64_t* rows_ptr, int64_t num_rows_keys,
                    int64_t num_batches, const int64_t* unique_ptr,
-                   const int64_t* edge_col, int64_t* out_unique,
-                   int64_t* out_row, int64_t* out_col, void* workspace,
-                   size_t workspace_bytes, gs_stream_t stream) {
+                   int64_t* out_unique, void* workspace, size_t workspace_bytes,
+                   gs_stream_t stream) {
   using namespace gs;
   const int64_t S = num_seeds, E = num_rows_keys, B = num_batches;
   int rc = check_unique_args(seeds, seeds_ptr, S, rows, rows_ptr, E, B);
   if (rc != GS_OK) return rc;
   GS_REQUIRE(unique_ptr, "unique_fill: null unique_ptr");
-  GS_REQUIRE(out_col == nullptr || edge_col != nullptr,
-             "unique_fill: out_col needs edge_col");
   UniqueWs w = carve_unique(workspace, S, E, B);
   if (workspace == nullptr || workspace_bytes < w.total) {
     set_error("unique workspace too small: %zu < %zu", workspace_bytes, w.total);
@@ -362,6 +359,27 @@ int gs_unique_fill(const int64_t* seeds, const int64_t* seeds_ptr,
             unique_fill_kernel<<<dim3((unsigned)nblocks), dim3(kBlock), 0, s>>>(
                 w.flat_ptr, B, seeds, seeds_ptr, S, rows, rows_ptr, N, w.table,
                 w.flags, w.block_off, unique_ptr, out_unique, w.seed_rank));
+  return GS_OK;
+}
+
+int gs_unique_relabel(const int64_t* seeds, const int64_t* seeds_ptr,
+                      int64_t num_seeds, const int64_t* rows,
+                      const int64_t* rows_ptr, int64_t num_rows_keys,
+                      int64_t num_batches, const int64_t* edge_col,
+                      int64_t* out_row, int64_t* out_col, void* workspace,
+                      size_t workspace_bytes, gs_stream_t stream) {
+  using namespace gs;
+  const int64_t S = num_seeds, E = num_rows_keys, B = num_batches;
+  int rc = check_unique_args(seeds, seeds_ptr, S, rows, rows_ptr, E, B);
+  if (rc != GS_OK) return rc;
+  GS_REQUIRE(out_col == nullptr || edge_col != nullptr,
+             "unique_relabel: out_col needs edge_col");
+  UniqueWs w = carve_unique(workspace, S, E, B);
+  if (workspace == nullptr || workspace_bytes < w.total) {
+    set_error("unique workspace too small: %zu < %zu", workspace_bytes, w.total);
+    return GS_ERR_WORKSPACE;
+  }
+  hipStream_t s = as_stream(stream);
   if (E > 0 && (out_row || out_col)) {
     GS_LAUNCH("unique_relabel", s,
               unique_relabel_kernel<<<dim3((unsigned)ceil_div(E, kBlock)),

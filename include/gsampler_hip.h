@@ -136,9 +136,11 @@ int gs_csc_col_sample_uniform_fill(const int64_t* indptr, int64_t num_cols,
  *   unique_ptr[num_batches + 1] (number of unique keys before each batch;
  *   the last element is the total U).
  * fill:  same arguments + the same workspace, untouched in between; writes
- *   out_unique[U]; out_row[num_rows_keys] = batch-local rank of every row key
- *   (nullable); out_col[num_rows_keys] = batch-local rank of
- *   seeds[edge_col[e]] (nullable; edge_col holds positions into `seeds`).
+ *   out_unique[U] and turns the tables into key -> batch-local rank maps.
+ * relabel: after fill, same workspace; out_row[num_rows_keys] = batch-local
+ *   rank of every row key (nullable); out_col[num_rows_keys] = batch-local rank
+ *   of seeds[edge_col[e]] (nullable; edge_col holds positions into `seeds`).
+ *   May be called any number of times while the workspace is kept.
  * Keys must lie in [0, 2^32 - 2] and one batch may hold at most 2^32 - 2 keys.
  * Stands in for TensorUniqueCUDA / TensorRelabelCUDA
  * (src/cuda/unique_reindex.cu:174-199) and BatchCOORelabelCUDA
@@ -155,9 +157,46 @@ int gs_unique_fill(const int64_t* seeds, const int64_t* seeds_ptr,
                    int64_t num_seeds, const int64_t* rows,
                    const int64_t* rows_ptr, int64_t num_rows_keys,
                    int64_t num_batches, const int64_t* unique_ptr,
-                   const int64_t* edge_col, int64_t* out_unique,
-                   int64_t* out_row, int64_t* out_col, void* workspace,
-                   size_t workspace_bytes, gs_stream_t stream);
+                   int64_t* out_unique, void* workspace, size_t workspace_bytes,
+                   gs_stream_t stream);
+int gs_unique_relabel(const int64_t* seeds, const int64_t* seeds_ptr,
+                      int64_t num_seeds, const int64_t* rows,
+                      const int64_t* rows_ptr, int64_t num_rows_keys,
+                      int64_t num_batches, const int64_t* edge_col,
+                      int64_t* out_row, int64_t* out_col, void* workspace,
+                      size_t workspace_bytes, gs_stream_t stream);
+
+/* ------------------------------------------------------------------------
+ * Format conversion.
+ *  gs_csc2coo: out_col[e] = column that owns edge position e
+ *    (CSC2COOCUDA, src/cuda/format_transform.cu:24-46).
+ *  gs_sorted_to_indptr: indptr[c] = #entries < c of a sorted id array, for
+ *    c in [0, num_cols]; the COO -> CSC step after the sort by column
+ *    (COO2CSCCUDA, src/cuda/format_transform.cu:109-142).  The sort itself is
+ *    done by the caller.
+ * ---------------------------------------------------------------------- */
+int gs_csc2coo(const int64_t* indptr, int64_t num_cols, int64_t nnz,
+               int64_t* out_col, gs_stream_t stream);
+int gs_sorted_to_indptr(const int64_t* sorted_ids, int64_t nnz, int64_t num_cols,
+                        int64_t* out_indptr, gs_stream_t stream);
+
+/* ------------------------------------------------------------------------
+ * Super-batch bookkeeping.
+ *  gs_decode_batch_ids: ids encoded as id + batch * stride -> out_batch =
+ *    id / stride, out_orig = id - batch * stride (either output nullable).
+ *    With gs_sorted_to_indptr over out_batch this is GetBatchOffsets,
+ *    src/cuda/batch/encoding_decoding.cu:99-122.
+ *  gs_split_indptr: batch b gets indptr[offset[b] .. offset[b+1]] rebased to
+ *    start at 0, written at out[offset[b] + b ...]; out_len =
+ *    offset[num_batches] - offset[0] + num_batches.  SplitIndptrByOffsetCUDA,
+ *    src/cuda/batch/batch_split.cu:53-94.
+ * ---------------------------------------------------------------------- */
+int gs_decode_batch_ids(const int64_t* encoded, int64_t n, int64_t stride,
+                        int64_t* out_orig, int64_t* out_batch,
+                        gs_stream_t stream);
+int gs_split_indptr(const int64_t* indptr, const int64_t* offset,
+                    int64_t num_batches, int64_t out_len, int64_t* out,
+                    gs_stream_t stream);
 
 #ifdef __cplusplus
 }

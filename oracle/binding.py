@@ -150,6 +150,44 @@ def unique_relabel(seeds, rows, seeds_ptr=None, rows_ptr=None, edge_col=None,
     out_col = np.empty(E, dtype=np.int64) if want_col else None
     lib().gs_unique_fill_cpu(_p(seeds), _p(seeds_ptr), C.c_int64(S), _p(rows),
                              _p(rows_ptr), C.c_int64(E), C.c_int64(B),
-                             _p(unique_ptr), _p(edge_col), _p(unique),
-                             _p(out_row), _p(out_col))
+                             _p(unique_ptr), _p(unique))
+    if want_row or want_col:
+        lib().gs_unique_relabel_cpu(_p(seeds), _p(seeds_ptr), C.c_int64(S), _p(rows),
+                                    _p(rows_ptr), C.c_int64(E), C.c_int64(B),
+                                    _p(edge_col), _p(out_row), _p(out_col))
     return unique, unique_ptr, out_row, out_col
+
+
+def csc2coo(indptr, nnz=None) -> np.ndarray:
+    indptr = _i64(indptr)
+    if nnz is None:
+        nnz = int(indptr[-1])
+    out = np.empty(nnz, dtype=np.int64)
+    lib().gs_csc2coo_cpu(_p(indptr), C.c_int64(indptr.size - 1), C.c_int64(nnz), _p(out))
+    return out
+
+
+def sorted_to_indptr(sorted_ids, num_cols) -> np.ndarray:
+    sorted_ids = _i64(sorted_ids)
+    out = np.empty(num_cols + 1, dtype=np.int64)
+    lib().gs_sorted_to_indptr_cpu(_p(sorted_ids), C.c_int64(sorted_ids.size),
+                                  C.c_int64(num_cols), _p(out))
+    return out
+
+
+def decode_batch_ids(encoded, stride):
+    encoded = _i64(encoded)
+    orig, batch = np.empty_like(encoded), np.empty_like(encoded)
+    lib().gs_decode_batch_ids_cpu(_p(encoded), C.c_int64(encoded.size),
+                                  C.c_int64(stride), _p(orig), _p(batch))
+    return orig, batch
+
+
+def split_indptr(indptr, offset) -> np.ndarray:
+    indptr, offset = _i64(indptr), _i64(offset)
+    nb = offset.size - 1
+    total = int(offset[-1] - offset[0]) + nb
+    out = np.empty(total, dtype=np.int64)
+    lib().gs_split_indptr_cpu(_p(indptr), _p(offset), C.c_int64(nb),
+                              C.c_int64(total), _p(out))
+    return out

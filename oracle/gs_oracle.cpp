@@ -323,8 +323,7 @@ void gs_unique_fill_cpu(const int64_t* seeds, const int64_t* seeds_ptr,
                         int64_t num_seeds, const int64_t* rows,
                         const int64_t* rows_ptr, int64_t num_rows_keys,
                         int64_t num_batches, const int64_t* unique_ptr,
-                        const int64_t* edge_col, int64_t* out_unique,
-                        int64_t* out_row, int64_t* out_col) {
+                        int64_t* out_unique) {
 #pragma omp parallel
   {
     std::unordered_map<int64_t, int64_t> rank;
@@ -335,13 +334,72 @@ void gs_unique_fill_cpu(const int64_t* seeds, const int64_t* seeds_ptr,
       batch_bounds(seeds_ptr, num_seeds, num_batches, b, &s_lo, &s_hi);
       batch_bounds(rows_ptr, num_rows_keys, num_batches, b, &r_lo, &r_hi);
       unique_batch(seeds, s_lo, s_hi, rows, r_lo, r_hi, &rank, &uniq);
-      if (out_unique)
-        std::copy(uniq.begin(), uniq.end(), out_unique + unique_ptr[b]);
+      std::copy(uniq.begin(), uniq.end(), out_unique + unique_ptr[b]);
+    }
+  }
+}
+
+void gs_unique_relabel_cpu(const int64_t* seeds, const int64_t* seeds_ptr,
+                           int64_t num_seeds, const int64_t* rows,
+                           const int64_t* rows_ptr, int64_t num_rows_keys,
+                           int64_t num_batches, const int64_t* edge_col,
+                           int64_t* out_row, int64_t* out_col) {
+#pragma omp parallel
+  {
+    std::unordered_map<int64_t, int64_t> rank;
+    std::vector<int64_t> uniq;
+#pragma omp for schedule(dynamic, 1)
+    for (int64_t b = 0; b < num_batches; ++b) {
+      int64_t s_lo, s_hi, r_lo, r_hi;
+      batch_bounds(seeds_ptr, num_seeds, num_batches, b, &s_lo, &s_hi);
+      batch_bounds(rows_ptr, num_rows_keys, num_batches, b, &r_lo, &r_hi);
+      unique_batch(seeds, s_lo, s_hi, rows, r_lo, r_hi, &rank, &uniq);
       for (int64_t e = r_lo; e < r_hi; ++e) {
         if (out_row) out_row[e] = rank[rows[e]];
         if (out_col) out_col[e] = rank[seeds[edge_col[e]]];
       }
     }
+  }
+}
+
+// -------------------------------------------------------------------------
+// Format conversion, src/cuda/format_transform.cu.
+//  CSC -> COO (:24-46): col[e] = UpperBound(indptr, e) - 1.
+//  COO -> CSC (:109-142), after a sort by column:
+//    indptr[c + 1] = UpperBound(sorted_cols, c)  <=>  indptr[c] = #entries < c.
+void gs_csc2coo_cpu(const int64_t* indptr, int64_t num_cols, int64_t nnz,
+                    int64_t* out_col) {
+  for (int64_t c = 0; c < num_cols; ++c)
+    for (int64_t e = indptr[c]; e < indptr[c + 1] && e < nnz; ++e) out_col[e] = c;
+}
+
+void gs_sorted_to_indptr_cpu(const int64_t* sorted_ids, int64_t nnz,
+                             int64_t num_cols, int64_t* out_indptr) {
+  for (int64_t c = 0; c <= num_cols; ++c)
+    out_indptr[c] = std::lower_bound(sorted_ids, sorted_ids + nnz, c) - sorted_ids;
+}
+
+// -------------------------------------------------------------------------
+// Super-batch bookkeeping.
+//  decode: mask = id / size, orig = id - mask * size
+//    (src/cuda/batch/encoding_decoding.cu:99-113).
+//  split indptr: out[offset[b] + b + j] = indptr[offset[b] + j] - indptr[offset[b]]
+//    for j in [0, offset[b+1] - offset[b]]  (src/cuda/batch/batch_split.cu:53-72).
+void gs_decode_batch_ids_cpu(const int64_t* encoded, int64_t n, int64_t stride,
+                             int64_t* out_orig, int64_t* out_batch) {
+  for (int64_t i = 0; i < n; ++i) {
+    int64_t b = encoded[i] / stride;
+    if (out_batch) out_batch[i] = b;
+    if (out_orig) out_orig[i] = encoded[i] - b * stride;
+  }
+}
+
+void gs_split_indptr_cpu(const int64_t* indptr, const int64_t* offset,
+                         int64_t num_batches, int64_t /*out_len*/, int64_t* out) {
+  for (int64_t b = 0; b < num_batches; ++b) {
+    int64_t lo = offset[b], hi = offset[b + 1];
+    for (int64_t j = 0; j <= hi - lo; ++j)
+      out[lo - offset[0] + b + j] = indptr[lo + j] - indptr[lo];
   }
 }
 

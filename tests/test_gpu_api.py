@@ -1,0 +1,146 @@
+"""The drop-in API (gs.Matrix / gs.BatchMatrix over gs_classes.Graph) against
+the CPU oracle: the samplers below are the reference's example functions
+(examples/graphsage/graphsage.py:7-28) run unchanged on `gsampler_amd`."""
+import numpy as np
+import pytest
+import torch
+
+import gsampler_amd as gs
+from gsampler_amd.utils import batched_seeds, rmat_csc
+from oracle import binding as orc
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def graphsage_sampler(A, seeds, fanouts):
+    input_node = seeds
+    ret = []
+    for K in fanouts:
+        subA = A[:, seeds]
+        sampleA = subA.individual_sampling(K, None, False)
+        seeds = sampleA.all_nodes()
+        ret.append(sampleA.to_dgl_block())
+    output_node = seeds
+    return input_node, output_node, ret
+
+
+def batch_graphsage_sampler(A, seeds, seeds_ptr, fanouts):
+    ret = []
+    for k in fanouts:
+        subA = A[:, seeds::seeds_ptr]
+        sampleA = subA.individual_sampling(k, None, False)
+        seeds, seeds_ptr = sampleA.all_nodes()
+        ret.append(sampleA.to_dgl_block())
+    return ret
+
+
+@pytest.fixture(scope="module")
+def graph():
+    indptr, indices = rmat_csc(20000, 400000, seed=1)
+    m = gs.Matrix()
+    m.load_graph("CSC", [indptr.to(DEV), indices.to(DEV)])
+    return m, indptr.numpy(), indices.numpy()
+
+
+def oracle_layers(indptr, indices, seeds, ptr, fanouts, first_call):
+    out = []
+    for layer, fanout in enumerate(fanouts):
+        s, c, rows, sel = orc.sample_uniform(indptr, indices, seeds, fanout, False, 0, 7777,
+                                             first_call + layer)
+        eptr = s[ptr] if ptr is not None else None
+        uniq, uptr, r, cc = orc.unique_relabel(seeds, rows, ptr, eptr, c)
+        out.append((uniq, uptr, r, cc, sel))
+        seeds, ptr = uniq, (uptr if ptr is not None else None)
+    return out
+
+
+def test_load_graph_shape(graph):
+    m, indptr, indices = graph
+    assert m.num_cols() == 20000 and m.num_rows() == int(indices.max()) + 1
+    assert m.num_edges() == indices.size
+    assert torch.equal(m.csc[0].cpu(), torch.from_numpy(indptr))
+
+
+def test_matrix_graphsage_matches_oracle(graph):
+    m, indptr, indices = graph
+    seeds = torch.randperm(20000, generator=torch.Generator().manual_seed(3))[:256]
+    gs.manual_seed(7777)
+    inp, outp, blocks = graphsage_sampler(m, seeds.to(DEV), [25, 10])
+    want = oracle_layers(indptr, indices, seeds.numpy(), None, [25, 10], 0)
+    assert torch.equal(inp.cpu(), seeds)
+    for blk, (uniq, uptr, r, c, sel) in zip(blocks, want):
+        assert np.array_equal(blk.srcdata["_ID"].cpu().numpy(), uniq)
+        assert np.array_equal(blk.row.cpu().numpy(), r)
+        assert np.array_equal(blk.col.cpu().numpy(), c)
+        assert blk.num_src == uniq.size
+    assert np.array_equal(outp.cpu().numpy(), want[-1][0])
+    assert blocks[0].num_dst == 256 and blocks[1].num_dst == want[0][0].size
+    # distinct seeds lead the frontier
+    assert np.array_equal(want[0][0][:256], seeds.numpy())
+
+
+def test_fused_operator_equals_slice_then_sample(graph):
+    """_CAPI_SlicingSampling (what the JIT emits) picks the same edges as
+    _CAPI_Slicing + _CAPI_Sampling with the same call id."""
+    m, indptr, indices = graph
+    seeds = torch.arange(0, 3000, 7, device=DEV)
+    gs.manual_seed(11)
+    sub, _ = m._graph._CAPI_Slicing(seeds, 1, gs._CSC, gs._CSC | gs._COO)
+    a, a_idx = sub._CAPI_Sampling(1, 10, False, gs._CSC, gs._CSC | gs._COO)
+    gs.manual_seed(11)
+    b, b_idx = m._graph._CAPI_SlicingSampling(1, seeds, 10, False, gs._CSC, gs._CSC | gs._COO)
+    assert torch.equal(a._CAPI_GetCSCIndptr(), b._CAPI_GetCSCIndptr())
+    assert torch.equal(a._CAPI_GetCSCIndices(), b._CAPI_GetCSCIndices())
+    assert torch.equal(a._CAPI_GetCOOCols(), b._CAPI_GetCOOCols())
+    # the fused operator's edge index addresses the parent matrix directly
+    assert torch.equal(m.csc[1][b_idx], b._CAPI_GetCSCIndices())
+
+
+def test_batch_matrix_graphsage_matches_oracle(graph):
+    m, indptr, indices = graph
+    seeds, ptr = batched_seeds(20000, 8, 128, seed=5)
+    bm = gs.BatchMatrix()
+    bm.load_from_matrix(m, False)
+    gs.manual_seed(7777)
+    blocks_per_layer = batch_graphsage_sampler(bm, seeds.to(DEV), ptr.to(DEV), [15, 10, 5])
+    want = oracle_layers(indptr, indices, seeds.numpy(), ptr.numpy(), [15, 10, 5], 0)
+    o_ptr = ptr.numpy()
+    for blocks, (uniq, uptr, r, c, sel) in zip(blocks_per_layer, want):
+        assert len(blocks) == 8
+        s_counts = np.diff(o_ptr)
+        for b, blk in enumerate(blocks):
+            assert np.array_equal(blk.srcdata["_ID"].cpu().numpy(), uniq[uptr[b]:uptr[b + 1]])
+            assert blk.num_dst == s_counts[b] and blk.num_src == uptr[b + 1] - uptr[b]
+        got_r = torch.cat([blk.row for blk in blocks]).cpu().numpy()
+        got_c = torch.cat([blk.col for blk in blocks]).cpu().numpy()
+        assert np.array_equal(got_r, r) and np.array_equal(got_c, c)
+        o_ptr = uptr
+
+
+def test_coo_and_csr_views_round_trip(graph):
+    m, indptr, indices = graph
+    sub = m[:, torch.arange(0, 500, device=DEV)]
+    row, col, _ = sub.coo
+    ci, cx, _ = sub.csc
+    ri, rx, r_eids = sub.csr
+    import scipy.sparse as sp
+    a = sp.csc_matrix((np.ones(cx.numel()), cx.cpu().numpy(), ci.cpu().numpy()),
+                      shape=(sub.num_rows(), sub.num_cols()))
+    b = sp.csr_matrix((np.ones(rx.numel()), rx.cpu().numpy(), ri.cpu().numpy()),
+                      shape=(sub.num_rows(), sub.num_cols()))
+    assert (a != b).nnz == 0
+    # CSR e_ids map CSR order back to the COO / CSC edge order
+    assert torch.equal(col[r_eids], rx)
+
+
+def test_errors_are_exceptions_not_aborts(graph):
+    m, _, _ = graph
+    with pytest.raises(RuntimeError, match="GPU"):
+        m._graph._CAPI_Slicing(torch.arange(3), 1, gs._CSC, gs._COO)
+    with pytest.raises(RuntimeError, match="int64"):
+        m._graph._CAPI_Slicing(torch.arange(3, device=DEV, dtype=torch.int32), 1, gs._CSC, gs._COO)
+    with pytest.raises(RuntimeError, match="cannot produce"):
+        m._graph._CAPI_Slicing(torch.arange(3, device=DEV), 1, gs._CSC, gs._CSR)
+    with pytest.raises(RuntimeError, match="not implemented"):
+        m._graph._CAPI_Sampling(0, 3, False, gs._CSC, gs._COO)
