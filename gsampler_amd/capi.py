@@ -58,6 +58,14 @@ SIGNATURES = {
     "gs_sorted_to_indptr": (_int, [_p, _i64, _i64, _p, _p]),
     "gs_decode_batch_ids": (_int, [_p, _i64, _i64, _p, _p, _p]),
     "gs_split_indptr": (_int, [_p, _p, _i64, _i64, _p, _p]),
+    "gs_sddmm": (_int, [_int, _p, _p, _i64, _i64, _p, _int, _int, _p, _p, _p, _int, _int,
+                        _i64, _i64, _i64, _i64, _p, _p, _p]),
+    "gs_fused_u_op_v": (_int, [_int, _p, _p, _i64, _i64, _int, _int, _p, _p, _p, _p, _p,
+                               _p, _i64, _i64, _i64, _i64, _p, _p, _p]),
+    "gs_spmm": (_int, [_int, _p, _p, _i64, _i64, _p, _int, _int, _p, _p, _p, _p, _p, _int,
+                       _i64, _i64, _i64, _p, _p, _p]),
+    "gs_e_square_sum": (_int, [_int, _p, _p, _i64, _i64, _p, _p, _p, _int, _i64, _p]),
+    "gs_e_div_u_sum": (_int, [_int, _p, _p, _i64, _i64, _p, _p, _p, _p, _int, _i64, _p]),
 }
 
 _lib = None
@@ -287,4 +295,106 @@ def split_indptr(indptr: torch.Tensor, offset: torch.Tensor) -> torch.Tensor:
     out = torch.empty(total, dtype=torch.int64, device=indptr.device)
     check(lib().gs_split_indptr(_ptr(indptr), _ptr(offset), nb, total, _ptr(out),
                                 _stream()))
+    return out
+
+
+# ------------------------------------------------------ edge-wise operators
+OPS = {"add": 0, "sub": 1, "mul": 2, "div": 3, "copy_lhs": 4, "copy_rhs": 5, "dot": 6}
+REDUCERS = {"sum": 0, "max": 1, "min": 2}
+FMT_COO, FMT_COMPRESSED = 1, 2
+
+
+def _view(view):
+    """("coo", row, col) or ("csc", indptr, indices) -> ABI structure arguments."""
+    kind, a, b = view
+    a, b = _i64t(a, "a"), _i64t(b, "b")
+    if kind == "coo":
+        return FMT_COO, a, b, 0, a.numel()
+    return FMT_COMPRESSED, a, b, a.numel() - 1, b.numel()
+
+
+def _feat(t):
+    if t is None:
+        return None, 0
+    t = t.contiguous()
+    return t, (1 if t.dim() == 1 else int(t[0].numel()) if t.shape[0] > 0 else 1)
+
+
+def _fptr(t):
+    return None if t is None or t.numel() == 0 else t.data_ptr()
+
+
+def sddmm(view, op, lhs, rhs, lhs_target, rhs_target, edge_map=None):
+    """Same-shape (or scalar) features, no broadcasting; dot reduces the last dim."""
+    fmt, a, b, nmaj, nnz = _view(view)
+    lhs, llen = _feat(lhs)
+    rhs, rlen = _feat(rhs)
+    ref = lhs if lhs is not None else rhs
+    flen = llen if lhs is not None else rlen
+    red = flen if op == "dot" else 1
+    out_len = flen // red
+    shape = (nnz,) if ref.dim() == 1 else (nnz, out_len)
+    out = torch.zeros(shape, dtype=ref.dtype, device=ref.device)
+    dtype = 0 if ref.dtype == torch.float32 else 1
+    check(lib().gs_sddmm(fmt, _ptr(a), _ptr(b), nmaj, nnz, _ptr(edge_map), OPS[op], dtype,
+                         _fptr(lhs), _fptr(rhs), _fptr(out), lhs_target, rhs_target,
+                         llen, rlen, out_len, red, None, None, _stream()))
+    return out
+
+
+def fused_u_op_v(view, op, lhs1, rhs1, lhs2, rhs2):
+    fmt, a, b, nmaj, nnz = _view(view)
+    lhs1, llen = _feat(lhs1)
+    rhs1, rlen = _feat(rhs1)
+    lhs2, _ = _feat(lhs2)
+    rhs2, _ = _feat(rhs2)
+    shape = (nnz,) if lhs1.dim() == 1 else (nnz, llen)
+    out1 = torch.zeros(shape, dtype=lhs1.dtype, device=lhs1.device)
+    out2 = torch.zeros_like(out1)
+    dtype = 0 if lhs1.dtype == torch.float32 else 1
+    check(lib().gs_fused_u_op_v(fmt, _ptr(a), _ptr(b), nmaj, nnz, OPS[op], dtype,
+                                _fptr(lhs1), _fptr(rhs1), _fptr(out1), _fptr(lhs2),
+                                _fptr(rhs2), _fptr(out2), llen, rlen, llen, 1, None, None,
+                                _stream()))
+    return out1, out2
+
+
+def spmm(view, op, reduce, ufeat, efeat, u_target, n_out, edge_map=None, want_arg=False):
+    fmt, a, b, nmaj, nnz = _view(view)
+    ufeat, ulen = _feat(ufeat)
+    efeat, elen = _feat(efeat)
+    ref = ufeat if (ufeat is not None and op != "copy_rhs") else efeat
+    flen = ulen if ref is ufeat else elen
+    shape = (n_out,) if ref.dim() == 1 else (n_out, flen)
+    out = torch.zeros(shape, dtype=torch.float32, device=ref.device)
+    arg_u = arg_e = None
+    if want_arg:
+        arg_u = torch.zeros(shape, dtype=torch.int64, device=ref.device)
+        arg_e = torch.zeros(shape, dtype=torch.int64, device=ref.device)
+    check(lib().gs_spmm(fmt, _ptr(a), _ptr(b), nmaj, nnz, _ptr(edge_map), OPS[op],
+                        REDUCERS[reduce], _fptr(ufeat), _fptr(efeat), _fptr(out),
+                        _ptr(arg_u), _ptr(arg_e), u_target, ulen, elen, flen, None, None,
+                        _stream()))
+    return (out, arg_u, arg_e) if want_arg else out
+
+
+def e_square_sum(view, efeat, u_target, n_out, edge_map=None):
+    fmt, a, b, nmaj, nnz = _view(view)
+    efeat, elen = _feat(efeat)
+    shape = (n_out,) if efeat.dim() == 1 else (n_out, elen)
+    out = torch.zeros(shape, dtype=torch.float32, device=efeat.device)
+    check(lib().gs_e_square_sum(fmt, _ptr(a), _ptr(b), nmaj, nnz, _ptr(edge_map),
+                                _fptr(efeat), _fptr(out), u_target, elen, _stream()))
+    return out
+
+
+def e_div_u_sum(view, ufeat, efeat, u_target, n_out, edge_map=None):
+    fmt, a, b, nmaj, nnz = _view(view)
+    ufeat, ulen = _feat(ufeat)
+    efeat, elen = _feat(efeat)
+    shape = (n_out,) if efeat.dim() == 1 else (n_out, elen)
+    out = torch.zeros(shape, dtype=torch.float32, device=efeat.device)
+    check(lib().gs_e_div_u_sum(fmt, _ptr(a), _ptr(b), nmaj, nnz, _ptr(edge_map),
+                               _fptr(ufeat), _fptr(efeat), _fptr(out), u_target, elen,
+                               _stream()))
     return out

@@ -1,0 +1,447 @@
+// edgeops.hip -- edge-wise compute operators of layer-wise samplers:
+// generalized SDDMM (a value per edge from its endpoints), generalized SpMM
+// (reduce edge values onto rows or columns) and their fusions (sum of squares,
+// sum of e / u, two u-op-v products in one sweep).
+//
+// Endpoint convention (same as the reference, src/cuda/sddmm.cu:37-38,134-135):
+// on COO  src = row[e], dst = col[e]; on a compressed matrix src = indices[e]
+// and dst = the segment of indptr that holds e.  Targets: 0 = src ("u"),
+// 1 = edge, 2 = dst ("v").  All kernels are memory bound; features are scalar
+// in every sampler that uses them, so the fast paths are the feature-length-1
+// ones and the general-length paths favour simplicity.
+#include "common.h"
+
+namespace gs {
+
+enum { kOpAdd = 0, kOpSub, kOpMul, kOpDiv, kOpCopyLhs, kOpCopyRhs, kOpDot };
+enum { kReduceSum = 0, kReduceMax, kReduceMin };
+
+template <typename T>
+__device__ __forceinline__ T apply_op(int op, const T* l, const T* r,
+                                      int64_t reduce_size) {
+  switch (op) {
+    case kOpAdd: return l[0] + r[0];
+    case kOpSub: return l[0] - r[0];
+    case kOpMul: return l[0] * r[0];
+    case kOpDiv: return l[0] / r[0];
+    case kOpCopyLhs: return l[0];
+    case kOpCopyRhs: return r[0];
+    default: {
+      T acc = 0;
+      for (int64_t k = 0; k < reduce_size; ++k) acc += l[k] * r[k];
+      return acc;
+    }
+  }
+}
+
+__device__ __forceinline__ int64_t pick(int target, int64_t src, int64_t eid,
+                                        int64_t dst) {
+  return target == 0 ? src : (target == 1 ? eid : dst);
+}
+
+struct EdgeView {
+  int compressed;      // 1: (indptr, indices), 0: (row, col)
+  const int64_t* a;    // row | indptr
+  const int64_t* b;    // col | indices
+  int64_t num_major;   // segments of indptr
+  const int64_t* edge_map;
+  __device__ __forceinline__ void endpoints(int64_t e, int64_t* src,
+                                            int64_t* dst, int64_t* eid) const {
+    if (compressed) {
+      *src = b[e];
+      *dst = segment_of(a, num_major, e);
+    } else {
+      *src = a[e];
+      *dst = b[e];
+    }
+    *eid = edge_map ? edge_map[e] : e;
+  }
+};
+
+// ------------------------------------------------------------------ SDDMM
+template <typename T>
+__global__ __launch_bounds__(kBlock) void sddmm_kernel(
+    EdgeView g, int64_t nnz, int op, const T* __restrict__ lhs,
+    const T* __restrict__ rhs, T* __restrict__ out, int lhs_target,
+    int rhs_target, int64_t lhs_len, int64_t rhs_len, int64_t out_len,
+    int64_t reduce_size, const int64_t* __restrict__ lhs_off,
+    const int64_t* __restrict__ rhs_off) {
+  const int64_t idx = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (idx >= nnz * out_len) return;
+  const int64_t e = idx / out_len, f = idx - e * out_len;
+  int64_t src, dst, eid;
+  g.endpoints(e, &src, &dst, &eid);
+  const int64_t lf = lhs_off ? lhs_off[f] : f, rf = rhs_off ? rhs_off[f] : f;
+  const T* l = op == kOpCopyRhs
+                   ? nullptr
+                   : lhs + pick(lhs_target, src, eid, dst) * lhs_len + lf * reduce_size;
+  const T* r = op == kOpCopyLhs
+                   ? nullptr
+                   : rhs + pick(rhs_target, src, eid, dst) * rhs_len + rf * reduce_size;
+  out[eid * out_len + f] = apply_op<T>(op, l, r, reduce_size);
+}
+
+// Two SDDMMs (u op v) that share one edge sweep.
+template <typename T>
+__global__ __launch_bounds__(kBlock) void fused_u_op_v_kernel(
+    EdgeView g, int64_t nnz, int op, const T* __restrict__ lhs1,
+    const T* __restrict__ rhs1, T* __restrict__ out1,
+    const T* __restrict__ lhs2, const T* __restrict__ rhs2,
+    T* __restrict__ out2, int64_t lhs_len, int64_t rhs_len, int64_t out_len,
+    int64_t reduce_size, const int64_t* __restrict__ lhs_off,
+    const int64_t* __restrict__ rhs_off) {
+  const int64_t idx = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (idx >= nnz * out_len) return;
+  const int64_t e = idx / out_len, f = idx - e * out_len;
+  int64_t src, dst, eid;
+  g.endpoints(e, &src, &dst, &eid);
+  const int64_t lf = (lhs_off ? lhs_off[f] : f) * reduce_size;
+  const int64_t rf = (rhs_off ? rhs_off[f] : f) * reduce_size;
+  out1[eid * out_len + f] = apply_op<T>(op, lhs1 + src * lhs_len + lf,
+                                        rhs1 + dst * rhs_len + rf, reduce_size);
+  out2[eid * out_len + f] = apply_op<T>(op, lhs2 + src * lhs_len + lf,
+                                        rhs2 + dst * rhs_len + rf, reduce_size);
+}
+
+// ------------------------------------------------------------------- SpMM
+// Value an edge contributes: kind 0 = op(u, e), 1 = e * e, 2 = e / u.
+template <typename T>
+__device__ __forceinline__ T edge_value(int kind, int op, const T* u, const T* e) {
+  if (kind == 1) return e[0] * e[0];
+  if (kind == 2) return e[0] / u[0];
+  return apply_op<T>(op, u, e, 1);
+}
+
+__device__ __forceinline__ void atomic_reduce(float* addr, float v, int reduce) {
+  if (reduce == kReduceSum) {
+    unsafeAtomicAdd(addr, v);
+    return;
+  }
+  unsigned int* p = (unsigned int*)addr;
+  unsigned int old = *p;
+  for (;;) {
+    float cur = __uint_as_float(old);
+    bool better = reduce == kReduceMax ? v > cur : v < cur;
+    if (!better) return;
+    unsigned int prev = atomicCAS(p, old, __float_as_uint(v));
+    if (prev == old) return;
+    old = prev;
+  }
+}
+
+// Coordinate form: one thread per (edge, feature), atomics onto the output.
+__global__ __launch_bounds__(kBlock) void spmm_coo_kernel(
+    const int64_t* __restrict__ row, const int64_t* __restrict__ col,
+    const int64_t* __restrict__ edge_map, int64_t nnz, int kind, int op,
+    int reduce, const float* __restrict__ ufeat, const float* __restrict__ efeat,
+    float* out, int u_target, int64_t ufeat_len, int64_t efeat_len,
+    int64_t out_len, const int64_t* __restrict__ u_off,
+    const int64_t* __restrict__ e_off) {
+  const int64_t idx = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (idx >= nnz * out_len) return;
+  const int64_t e = idx / out_len, f = idx - e * out_len;
+  const int64_t src = u_target == 0 ? row[e] : col[e];
+  const int64_t dst = u_target == 0 ? col[e] : row[e];
+  const int64_t eid = edge_map ? edge_map[e] : e;
+  const float* u = ufeat ? ufeat + src * ufeat_len + (u_off ? u_off[f] : f) : nullptr;
+  const float* ev = efeat ? efeat + eid * efeat_len + (e_off ? e_off[f] : f) : nullptr;
+  atomic_reduce(out + dst * out_len + f, edge_value<float>(kind, op, u, ev), reduce);
+}
+
+// Second pass of arg-max / arg-min in coordinate form: the edge whose value
+// equals the reduced output records its source and edge id.
+__global__ __launch_bounds__(kBlock) void spmm_coo_arg_kernel(
+    const int64_t* __restrict__ row, const int64_t* __restrict__ col,
+    const int64_t* __restrict__ edge_map, int64_t nnz, int op,
+    const float* __restrict__ ufeat, const float* __restrict__ efeat,
+    const float* __restrict__ out, int64_t* arg_u, int64_t* arg_e, int u_target,
+    int64_t ufeat_len, int64_t efeat_len, int64_t out_len,
+    const int64_t* __restrict__ u_off, const int64_t* __restrict__ e_off) {
+  const int64_t idx = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (idx >= nnz * out_len) return;
+  const int64_t e = idx / out_len, f = idx - e * out_len;
+  const int64_t src = u_target == 0 ? row[e] : col[e];
+  const int64_t dst = u_target == 0 ? col[e] : row[e];
+  const int64_t eid = edge_map ? edge_map[e] : e;
+  const float* u = ufeat ? ufeat + src * ufeat_len + (u_off ? u_off[f] : f) : nullptr;
+  const float* ev = efeat ? efeat + eid * efeat_len + (e_off ? e_off[f] : f) : nullptr;
+  if (edge_value<float>(0, op, u, ev) == out[dst * out_len + f]) {
+    if (arg_u) arg_u[dst * out_len + f] = src;
+    if (arg_e) arg_e[dst * out_len + f] = eid;
+  }
+}
+
+// Compressed form, scalar features: a group of G lanes per segment strides over
+// its edges and reduces with shuffles -- no atomics, hubs spread over a wave.
+template <int G>
+__global__ __launch_bounds__(kBlock) void spmm_csc_scalar_kernel(
+    const int64_t* __restrict__ indptr, const int64_t* __restrict__ indices,
+    const int64_t* __restrict__ edge_map, int64_t num_major, int kind, int op,
+    int reduce, const float* __restrict__ ufeat, const float* __restrict__ efeat,
+    float* __restrict__ out, int64_t* __restrict__ arg_u,
+    int64_t* __restrict__ arg_e) {
+  const int lane = threadIdx.x & (G - 1);
+  const int64_t c = ((int64_t)blockIdx.x * kBlock + threadIdx.x) / G;
+  if (c >= num_major) return;
+  const int64_t lo = indptr[c], hi = indptr[c + 1];
+  // reduction starts from 0: outputs are zero-initialised accumulators
+  float acc = 0.f;
+  int64_t best_u = 0, best_e = 0;
+  for (int64_t i = lo + lane; i < hi; i += G) {
+    const int64_t eid = edge_map ? edge_map[i] : i;
+    const int64_t cid = indices[i];
+    const float v = edge_value<float>(kind, op, ufeat ? ufeat + cid : nullptr,
+                                      efeat ? efeat + eid : nullptr);
+    if (reduce == kReduceSum) {
+      acc += v;
+    } else if (reduce == kReduceMax ? v > acc : v < acc) {
+      acc = v;
+      best_u = cid;
+      best_e = eid;
+    }
+  }
+#pragma unroll
+  for (int d = G / 2; d > 0; d >>= 1) {
+    const float o = __shfl_down(acc, d, G);
+    const int64_t ou = __shfl_down(best_u, d, G);
+    const int64_t oe = __shfl_down(best_e, d, G);
+    if (reduce == kReduceSum) {
+      acc += o;
+    } else if (reduce == kReduceMax ? o > acc : o < acc) {
+      acc = o;
+      best_u = ou;
+      best_e = oe;
+    }
+  }
+  if (lane == 0) {
+    out[c] += acc;
+    if (reduce != kReduceSum) {
+      if (arg_u) arg_u[c] = best_u;
+      if (arg_e) arg_e[c] = best_e;
+    }
+  }
+}
+
+// Compressed form, general feature length: one thread per (segment, feature).
+__global__ __launch_bounds__(kBlock) void spmm_csc_kernel(
+    const int64_t* __restrict__ indptr, const int64_t* __restrict__ indices,
+    const int64_t* __restrict__ edge_map, int64_t num_major, int kind, int op,
+    int reduce, const float* __restrict__ ufeat, const float* __restrict__ efeat,
+    float* __restrict__ out, int64_t* __restrict__ arg_u,
+    int64_t* __restrict__ arg_e, int64_t ufeat_len, int64_t efeat_len,
+    int64_t out_len, const int64_t* __restrict__ u_off,
+    const int64_t* __restrict__ e_off) {
+  const int64_t idx = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (idx >= num_major * out_len) return;
+  const int64_t c = idx / out_len, f = idx - c * out_len;
+  const int64_t uf = u_off ? u_off[f] : f, ef = e_off ? e_off[f] : f;
+  float acc = 0.f;
+  int64_t best_u = 0, best_e = 0;
+  for (int64_t i = indptr[c]; i < indptr[c + 1]; ++i) {
+    const int64_t eid = edge_map ? edge_map[i] : i;
+    const int64_t cid = indices[i];
+    const float v =
+        edge_value<float>(kind, op, ufeat ? ufeat + cid * ufeat_len + uf : nullptr,
+                          efeat ? efeat + eid * efeat_len + ef : nullptr);
+    if (reduce == kReduceSum) {
+      acc += v;
+    } else if (reduce == kReduceMax ? v > acc : v < acc) {
+      acc = v;
+      best_u = cid;
+      best_e = eid;
+    }
+  }
+  out[idx] += acc;
+  if (reduce != kReduceSum) {
+    if (arg_u) arg_u[idx] = best_u;
+    if (arg_e) arg_e[idx] = best_e;
+  }
+}
+
+static int check_view(int format, const int64_t* a, const int64_t* b,
+                      int64_t num_major, int64_t nnz, const char* who) {
+  GS_REQUIRE(format == GS_FMT_COO || format == GS_FMT_COMPRESSED,
+             "%s: unknown format %d", who, format);
+  GS_REQUIRE(nnz >= 0 && num_major >= 0, "%s: negative size", who);
+  GS_REQUIRE(nnz == 0 || (a && b), "%s: null structure pointer", who);
+  return GS_OK;
+}
+
+static int spmm_launch(int format, const int64_t* a, const int64_t* b,
+                       int64_t num_major, int64_t nnz, const int64_t* edge_map,
+                       int kind, int op, int reduce, const float* ufeat,
+                       const float* efeat, float* out, int64_t* arg_u,
+                       int64_t* arg_e, int u_target, int64_t ufeat_len,
+                       int64_t efeat_len, int64_t out_len, const int64_t* u_off,
+                       const int64_t* e_off, hipStream_t s) {
+  if (nnz == 0 || out_len == 0) return GS_OK;
+  if (format == GS_FMT_COO) {
+    const int64_t total = nnz * out_len;
+    GS_LAUNCH("spmm_coo", s,
+              spmm_coo_kernel<<<dim3((unsigned)ceil_div(total, kBlock)),
+                                dim3(kBlock), 0, s>>>(
+                  a, b, edge_map, nnz, kind, op, reduce, ufeat, efeat, out,
+                  u_target, ufeat_len, efeat_len, out_len, u_off, e_off));
+    if (reduce != kReduceSum && (arg_u || arg_e))
+      GS_LAUNCH("spmm_coo_arg", s,
+                spmm_coo_arg_kernel<<<dim3((unsigned)ceil_div(total, kBlock)),
+                                      dim3(kBlock), 0, s>>>(
+                    a, b, edge_map, nnz, op, ufeat, efeat, out, arg_u, arg_e,
+                    u_target, ufeat_len, efeat_len, out_len, u_off, e_off));
+    return GS_OK;
+  }
+  const bool scalar = out_len == 1 && (ufeat == nullptr || ufeat_len == 1) &&
+                      (efeat == nullptr || efeat_len == 1);
+  if (scalar) {
+    const int64_t avg = nnz / (num_major > 0 ? num_major : 1);
+#define GS_SPMM_SCALAR(G)                                                      \
+  GS_LAUNCH("spmm_csc_scalar", s,                                              \
+            spmm_csc_scalar_kernel<G><<<dim3((unsigned)ceil_div(num_major * G, kBlock)), \
+                                        dim3(kBlock), 0, s>>>(                 \
+                a, b, edge_map, num_major, kind, op, reduce, ufeat, efeat, out, \
+                arg_u, arg_e))
+    if (avg <= 8)
+      GS_SPMM_SCALAR(4);
+    else if (avg <= 64)
+      GS_SPMM_SCALAR(16);
+    else
+      GS_SPMM_SCALAR(64);
+#undef GS_SPMM_SCALAR
+    return GS_OK;
+  }
+  GS_LAUNCH("spmm_csc", s,
+            spmm_csc_kernel<<<dim3((unsigned)ceil_div(num_major * out_len, kBlock)),
+                              dim3(kBlock), 0, s>>>(
+                a, b, edge_map, num_major, kind, op, reduce, ufeat, efeat, out,
+                arg_u, arg_e, ufeat_len, efeat_len, out_len, u_off, e_off));
+  return GS_OK;
+}
+
+}  // namespace gs
+
+extern "C" {
+
+int gs_sddmm(int format, const int64_t* a, const int64_t* b, int64_t num_major,
+             int64_t nnz, const int64_t* edge_map, int op, int dtype,
+             const void* lhs, const void* rhs, void* out, int lhs_target,
+             int rhs_target, int64_t lhs_len, int64_t rhs_len, int64_t out_len,
+             int64_t reduce_size, const int64_t* lhs_off, const int64_t* rhs_off,
+             gs_stream_t stream) {
+  using namespace gs;
+  int rc = check_view(format, a, b, num_major, nnz, "sddmm");
+  if (rc != GS_OK) return rc;
+  GS_REQUIRE(op >= kOpAdd && op <= kOpDot, "sddmm: unknown operator %d", op);
+  GS_REQUIRE(dtype == GS_F32 || dtype == GS_F64, "sddmm: unknown dtype %d", dtype);
+  GS_REQUIRE(lhs_target >= 0 && lhs_target <= 2 && rhs_target >= 0 && rhs_target <= 2,
+             "sddmm: targets must be 0 (u), 1 (e) or 2 (v)");
+  GS_REQUIRE(out_len >= 0 && reduce_size >= 1, "sddmm: bad feature sizes");
+  if (nnz == 0 || out_len == 0) return GS_OK;
+  GS_REQUIRE(out && (lhs || op == kOpCopyRhs) && (rhs || op == kOpCopyLhs),
+             "sddmm: null operand");
+  hipStream_t s = as_stream(stream);
+  const EdgeView g{format == GS_FMT_COMPRESSED, a, b, num_major, edge_map};
+  const unsigned blocks = (unsigned)ceil_div(nnz * out_len, kBlock);
+  if (dtype == GS_F32)
+    GS_LAUNCH("sddmm", s,
+              sddmm_kernel<float><<<dim3(blocks), dim3(kBlock), 0, s>>>(
+                  g, nnz, op, (const float*)lhs, (const float*)rhs, (float*)out,
+                  lhs_target, rhs_target, lhs_len, rhs_len, out_len, reduce_size,
+                  lhs_off, rhs_off));
+  else
+    GS_LAUNCH("sddmm", s,
+              sddmm_kernel<double><<<dim3(blocks), dim3(kBlock), 0, s>>>(
+                  g, nnz, op, (const double*)lhs, (const double*)rhs,
+                  (double*)out, lhs_target, rhs_target, lhs_len, rhs_len, out_len,
+                  reduce_size, lhs_off, rhs_off));
+  return GS_OK;
+}
+
+int gs_fused_u_op_v(int format, const int64_t* a, const int64_t* b,
+                    int64_t num_major, int64_t nnz, int op, int dtype,
+                    const void* lhs1, const void* rhs1, void* out1,
+                    const void* lhs2, const void* rhs2, void* out2,
+                    int64_t lhs_len, int64_t rhs_len, int64_t out_len,
+                    int64_t reduce_size, const int64_t* lhs_off,
+                    const int64_t* rhs_off, gs_stream_t stream) {
+  using namespace gs;
+  int rc = check_view(format, a, b, num_major, nnz, "fused_u_op_v");
+  if (rc != GS_OK) return rc;
+  GS_REQUIRE((op >= kOpAdd && op <= kOpDiv) || op == kOpDot,
+             "fused_u_op_v: operator %d needs both operands", op);
+  GS_REQUIRE(dtype == GS_F32 || dtype == GS_F64, "fused_u_op_v: unknown dtype %d", dtype);
+  if (nnz == 0 || out_len == 0) return GS_OK;
+  GS_REQUIRE(lhs1 && rhs1 && out1 && lhs2 && rhs2 && out2, "fused_u_op_v: null operand");
+  hipStream_t s = as_stream(stream);
+  const EdgeView g{format == GS_FMT_COMPRESSED, a, b, num_major, nullptr};
+  const unsigned blocks = (unsigned)ceil_div(nnz * out_len, kBlock);
+  if (dtype == GS_F32)
+    GS_LAUNCH("fused_u_op_v", s,
+              fused_u_op_v_kernel<float><<<dim3(blocks), dim3(kBlock), 0, s>>>(
+                  g, nnz, op, (const float*)lhs1, (const float*)rhs1,
+                  (float*)out1, (const float*)lhs2, (const float*)rhs2,
+                  (float*)out2, lhs_len, rhs_len, out_len, reduce_size, lhs_off,
+                  rhs_off));
+  else
+    GS_LAUNCH("fused_u_op_v", s,
+              fused_u_op_v_kernel<double><<<dim3(blocks), dim3(kBlock), 0, s>>>(
+                  g, nnz, op, (const double*)lhs1, (const double*)rhs1,
+                  (double*)out1, (const double*)lhs2, (const double*)rhs2,
+                  (double*)out2, lhs_len, rhs_len, out_len, reduce_size, lhs_off,
+                  rhs_off));
+  return GS_OK;
+}
+
+int gs_spmm(int format, const int64_t* a, const int64_t* b, int64_t num_major,
+            int64_t nnz, const int64_t* edge_map, int op, int reduce,
+            const float* ufeat, const float* efeat, float* out, int64_t* arg_u,
+            int64_t* arg_e, int u_target, int64_t ufeat_len, int64_t efeat_len,
+            int64_t out_len, const int64_t* u_off, const int64_t* e_off,
+            gs_stream_t stream) {
+  using namespace gs;
+  int rc = check_view(format, a, b, num_major, nnz, "spmm");
+  if (rc != GS_OK) return rc;
+  GS_REQUIRE((op >= kOpAdd && op <= kOpCopyRhs), "spmm: unknown operator %d", op);
+  GS_REQUIRE(reduce >= kReduceSum && reduce <= kReduceMin, "spmm: unknown reducer %d", reduce);
+  GS_REQUIRE(u_target == 0 || u_target == 2, "spmm: u_target must be 0 or 2");
+  if (nnz == 0 || out_len == 0) return GS_OK;
+  GS_REQUIRE(out && (ufeat || op == kOpCopyRhs) && (efeat || op == kOpCopyLhs),
+             "spmm: null operand");
+  return spmm_launch(format, a, b, num_major, nnz, edge_map, 0, op, reduce,
+                     op == kOpCopyRhs ? nullptr : ufeat,
+                     op == kOpCopyLhs ? nullptr : efeat, out, arg_u, arg_e,
+                     u_target, ufeat_len, efeat_len, out_len, u_off, e_off,
+                     as_stream(stream));
+}
+
+int gs_e_square_sum(int format, const int64_t* a, const int64_t* b,
+                    int64_t num_major, int64_t nnz, const int64_t* edge_map,
+                    const float* efeat, float* out, int u_target,
+                    int64_t feat_len, gs_stream_t stream) {
+  using namespace gs;
+  int rc = check_view(format, a, b, num_major, nnz, "e_square_sum");
+  if (rc != GS_OK) return rc;
+  GS_REQUIRE(u_target == 0 || u_target == 2, "e_square_sum: u_target must be 0 or 2");
+  if (nnz == 0 || feat_len == 0) return GS_OK;
+  GS_REQUIRE(efeat && out, "e_square_sum: null operand");
+  return spmm_launch(format, a, b, num_major, nnz, edge_map, 1, kOpCopyRhs,
+                     kReduceSum, nullptr, efeat, out, nullptr, nullptr, u_target,
+                     0, feat_len, feat_len, nullptr, nullptr, as_stream(stream));
+}
+
+int gs_e_div_u_sum(int format, const int64_t* a, const int64_t* b,
+                   int64_t num_major, int64_t nnz, const int64_t* edge_map,
+                   const float* ufeat, const float* efeat, float* out,
+                   int u_target, int64_t feat_len, gs_stream_t stream) {
+  using namespace gs;
+  int rc = check_view(format, a, b, num_major, nnz, "e_div_u_sum");
+  if (rc != GS_OK) return rc;
+  GS_REQUIRE(u_target == 0 || u_target == 2, "e_div_u_sum: u_target must be 0 or 2");
+  if (nnz == 0 || feat_len == 0) return GS_OK;
+  GS_REQUIRE(ufeat && efeat && out, "e_div_u_sum: null operand");
+  return spmm_launch(format, a, b, num_major, nnz, edge_map, 2, kOpDiv,
+                     kReduceSum, ufeat, efeat, out, nullptr, nullptr, u_target,
+                     feat_len, feat_len, feat_len, nullptr, nullptr,
+                     as_stream(stream));
+}
+
+}  // extern "C"

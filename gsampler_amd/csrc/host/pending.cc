@@ -25,30 +25,6 @@ torch::Tensor Graph::Node2Vec(torch::Tensor, int64_t, double, double) {
   GS_PENDING("Node2Vec");
 }
 void Graph::SortCSCIndices() { GS_PENDING("SortCSCIndices"); }
-void Graph::SDDMM(const std::string&, torch::Tensor, torch::Tensor, torch::Tensor,
-                  int64_t, int64_t, int64_t) {
-  GS_PENDING("SDDMM");
-}
-void Graph::SpMM(const std::string&, const std::string&, torch::Tensor,
-                 torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor,
-                 int64_t, int64_t) {
-  GS_PENDING("SpMM");
-}
-void Graph::FusedUOPV(const std::string&, torch::Tensor, torch::Tensor,
-                      torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor,
-                      int64_t) {
-  GS_PENDING("FusedUOPV");
-}
-void Graph::FusedESquareSum(const std::string&, const std::string&, torch::Tensor,
-                            torch::Tensor, torch::Tensor, torch::Tensor,
-                            torch::Tensor, int64_t, int64_t) {
-  GS_PENDING("FusedESquareSum");
-}
-void Graph::FusedEDivUSum(const std::string&, const std::string&, torch::Tensor,
-                          torch::Tensor, torch::Tensor, torch::Tensor,
-                          torch::Tensor, int64_t, int64_t) {
-  GS_PENDING("FusedEDivUSum");
-}
 GraphAndIndex Graph::BatchColRowSlcing(torch::Tensor, torch::Tensor, torch::Tensor,
                                        torch::Tensor) {
   GS_PENDING("BatchColRowSlcing");

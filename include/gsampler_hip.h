@@ -42,6 +42,28 @@ extern "C" {
 #define GS_ALGO_RESERVOIR 1 /* the reference's Algorithm R in max-form */
 #define GS_ALGO_FLOYD 2     /* Floyd's subset sampling, O(fanout) per column */
 
+/* Sparse structure handed to the edge-wise operators. */
+#define GS_FMT_COO 1        /* a = row[nnz], b = col[nnz] */
+#define GS_FMT_COMPRESSED 2 /* a = indptr[num_major + 1], b = indices[nnz] */
+
+/* Binary operators, reducers, operand targets and value types of the
+ * edge-wise operators (names follow src/cuda/macro.h:7-33 of the reference). */
+#define GS_OP_ADD 0
+#define GS_OP_SUB 1
+#define GS_OP_MUL 2
+#define GS_OP_DIV 3
+#define GS_OP_COPY_LHS 4
+#define GS_OP_COPY_RHS 5
+#define GS_OP_DOT 6
+#define GS_REDUCE_SUM 0
+#define GS_REDUCE_MAX 1
+#define GS_REDUCE_MIN 2
+#define GS_TARGET_U 0 /* source endpoint: row of a COO / indices of a compressed matrix */
+#define GS_TARGET_E 1 /* the edge itself */
+#define GS_TARGET_V 2 /* destination endpoint: column of a COO / owning segment */
+#define GS_F32 0
+#define GS_F64 1
+
 typedef void* gs_stream_t;
 
 /* Message of the last error raised on the calling thread ("" if none). */
@@ -197,6 +219,55 @@ int gs_decode_batch_ids(const int64_t* encoded, int64_t n, int64_t stride,
 int gs_split_indptr(const int64_t* indptr, const int64_t* offset,
                     int64_t num_batches, int64_t out_len, int64_t* out,
                     gs_stream_t stream);
+
+/* ------------------------------------------------------------------------
+ * Edge-wise compute operators.  Common arguments: (format, a, b, num_major,
+ * nnz) describe the structure; edge_map (nullable) maps an edge position to
+ * the row of the edge-feature arrays (the e_ids of a converted format).
+ * Feature arrays are row-major [n, len]; *_off (nullable) are broadcast offset
+ * tables of out_len entries as computed by CalcBcastOff (src/bcast.cc:24-76).
+ *
+ * gs_sddmm: out[eid] = lhs[t_l] op rhs[t_r]            SDDMMCOO / SDDMMCSC,
+ *   src/cuda/sddmm.cu:264-297.  fp32 or fp64.
+ * gs_fused_u_op_v: two u-op-v SDDMMs in one sweep       FUSED_COO/CSC_U_OP_V,
+ *   src/cuda/fusion/fused_coo_u_op_v.cu:109, fused_csc_u_op_v.cu:103.
+ * gs_spmm: out[dst] = reduce(out[dst], op(u[src], e[eid])), fp32.  Outputs
+ *   are accumulators: the caller zero-fills them (python/gs/ops/spmm.py:56).
+ *   COO: u_target 0 reduces onto columns, 2 onto rows (atomics).  Compressed:
+ *   reduces onto the segments of indptr (no atomics); u_target is ignored.
+ *   SpMMCOO / SpMMCSC, src/cuda/spmm.cu:274-348.
+ * gs_e_square_sum: out[dst] += sum e^2                  ESquareSumCSC/COO,
+ *   src/cuda/fusion/fused_csc_e_square_sum.cu:110, fused_coo_e_square_sum.cu:13.
+ * gs_e_div_u_sum: out[dst] += sum e / u[src]            EDivUSumCSC/COO,
+ *   src/cuda/fusion/fused_csc_e_div_u_sum.cu:103, fused_coo_e_div_u_sum.cu:88.
+ * ---------------------------------------------------------------------- */
+int gs_sddmm(int format, const int64_t* a, const int64_t* b, int64_t num_major,
+             int64_t nnz, const int64_t* edge_map, int op, int dtype,
+             const void* lhs, const void* rhs, void* out, int lhs_target,
+             int rhs_target, int64_t lhs_len, int64_t rhs_len, int64_t out_len,
+             int64_t reduce_size, const int64_t* lhs_off, const int64_t* rhs_off,
+             gs_stream_t stream);
+int gs_fused_u_op_v(int format, const int64_t* a, const int64_t* b,
+                    int64_t num_major, int64_t nnz, int op, int dtype,
+                    const void* lhs1, const void* rhs1, void* out1,
+                    const void* lhs2, const void* rhs2, void* out2,
+                    int64_t lhs_len, int64_t rhs_len, int64_t out_len,
+                    int64_t reduce_size, const int64_t* lhs_off,
+                    const int64_t* rhs_off, gs_stream_t stream);
+int gs_spmm(int format, const int64_t* a, const int64_t* b, int64_t num_major,
+            int64_t nnz, const int64_t* edge_map, int op, int reduce,
+            const float* ufeat, const float* efeat, float* out, int64_t* arg_u,
+            int64_t* arg_e, int u_target, int64_t ufeat_len, int64_t efeat_len,
+            int64_t out_len, const int64_t* u_off, const int64_t* e_off,
+            gs_stream_t stream);
+int gs_e_square_sum(int format, const int64_t* a, const int64_t* b,
+                    int64_t num_major, int64_t nnz, const int64_t* edge_map,
+                    const float* efeat, float* out, int u_target,
+                    int64_t feat_len, gs_stream_t stream);
+int gs_e_div_u_sum(int format, const int64_t* a, const int64_t* b,
+                   int64_t num_major, int64_t nnz, const int64_t* edge_map,
+                   const float* ufeat, const float* efeat, float* out,
+                   int u_target, int64_t feat_len, gs_stream_t stream);
 
 #ifdef __cplusplus
 }

@@ -191,3 +191,101 @@ def split_indptr(indptr, offset) -> np.ndarray:
     lib().gs_split_indptr_cpu(_p(indptr), _p(offset), C.c_int64(nb),
                               C.c_int64(total), _p(out))
     return out
+
+
+# ------------------------------------------------------ edge-wise operators
+OPS = {"add": 0, "sub": 1, "mul": 2, "div": 3, "copy_lhs": 4, "copy_rhs": 5, "dot": 6}
+REDUCERS = {"sum": 0, "max": 1, "min": 2}
+
+
+def _view(view):
+    kind, a, b = view
+    a, b = _i64(a), _i64(b)
+    if kind == "coo":
+        return 1, a, b, 0, a.size
+    return 2, a, b, a.size - 1, b.size
+
+
+def _feat(t):
+    if t is None:
+        return None, 0
+    t = np.ascontiguousarray(t)
+    return t, (1 if t.ndim == 1 else int(np.prod(t.shape[1:])))
+
+
+def _em(edge_map):
+    return None if edge_map is None else _i64(edge_map)
+
+
+def sddmm(view, op, lhs, rhs, lhs_target, rhs_target, edge_map=None):
+    fmt, a, b, nmaj, nnz = _view(view)
+    lhs, llen = _feat(lhs)
+    rhs, rlen = _feat(rhs)
+    ref = lhs if lhs is not None else rhs
+    flen = llen if lhs is not None else rlen
+    red = flen if op == "dot" else 1
+    out_len = flen // red
+    out = np.zeros((nnz,) if ref.ndim == 1 else (nnz, out_len), dtype=ref.dtype)
+    em = _em(edge_map)
+    lib().gs_sddmm_cpu(C.c_int(fmt), _p(a), _p(b), C.c_int64(nmaj), C.c_int64(nnz), _p(em),
+                       C.c_int(OPS[op]), C.c_int(0 if ref.dtype == np.float32 else 1),
+                       _p(lhs), _p(rhs), _p(out), C.c_int(lhs_target), C.c_int(rhs_target),
+                       C.c_int64(llen), C.c_int64(rlen), C.c_int64(out_len), C.c_int64(red),
+                       None, None)
+    return out
+
+
+def fused_u_op_v(view, op, lhs1, rhs1, lhs2, rhs2):
+    fmt, a, b, nmaj, nnz = _view(view)
+    lhs1, llen = _feat(lhs1)
+    rhs1, rlen = _feat(rhs1)
+    lhs2, _ = _feat(lhs2)
+    rhs2, _ = _feat(rhs2)
+    out1 = np.zeros((nnz,) if lhs1.ndim == 1 else (nnz, llen), dtype=lhs1.dtype)
+    out2 = np.zeros_like(out1)
+    lib().gs_fused_u_op_v_cpu(C.c_int(fmt), _p(a), _p(b), C.c_int64(nmaj), C.c_int64(nnz),
+                              C.c_int(OPS[op]), C.c_int(0 if lhs1.dtype == np.float32 else 1),
+                              _p(lhs1), _p(rhs1), _p(out1), _p(lhs2), _p(rhs2), _p(out2),
+                              C.c_int64(llen), C.c_int64(rlen), C.c_int64(llen), C.c_int64(1),
+                              None, None)
+    return out1, out2
+
+
+def spmm(view, op, reduce, ufeat, efeat, u_target, n_out, edge_map=None, want_arg=False):
+    fmt, a, b, nmaj, nnz = _view(view)
+    ufeat, ulen = _feat(ufeat)
+    efeat, elen = _feat(efeat)
+    ref = ufeat if (ufeat is not None and op != "copy_rhs") else efeat
+    flen = ulen if ref is ufeat else elen
+    shape = (n_out,) if ref.ndim == 1 else (n_out, flen)
+    out = np.zeros(shape, dtype=np.float32)
+    arg_u = np.zeros(shape, dtype=np.int64) if want_arg else None
+    arg_e = np.zeros(shape, dtype=np.int64) if want_arg else None
+    em = _em(edge_map)
+    lib().gs_spmm_cpu(C.c_int(fmt), _p(a), _p(b), C.c_int64(nmaj), C.c_int64(nnz), _p(em),
+                      C.c_int(OPS[op]), C.c_int(REDUCERS[reduce]), _p(ufeat), _p(efeat),
+                      _p(out), _p(arg_u), _p(arg_e), C.c_int(u_target), C.c_int64(ulen),
+                      C.c_int64(elen), C.c_int64(flen), None, None)
+    return (out, arg_u, arg_e) if want_arg else out
+
+
+def e_square_sum(view, efeat, u_target, n_out, edge_map=None):
+    fmt, a, b, nmaj, nnz = _view(view)
+    efeat, elen = _feat(efeat)
+    out = np.zeros((n_out,) if efeat.ndim == 1 else (n_out, elen), dtype=np.float32)
+    em = _em(edge_map)
+    lib().gs_e_square_sum_cpu(C.c_int(fmt), _p(a), _p(b), C.c_int64(nmaj), C.c_int64(nnz),
+                              _p(em), _p(efeat), _p(out), C.c_int(u_target), C.c_int64(elen))
+    return out
+
+
+def e_div_u_sum(view, ufeat, efeat, u_target, n_out, edge_map=None):
+    fmt, a, b, nmaj, nnz = _view(view)
+    ufeat, ulen = _feat(ufeat)
+    efeat, elen = _feat(efeat)
+    out = np.zeros((n_out,) if efeat.ndim == 1 else (n_out, elen), dtype=np.float32)
+    em = _em(edge_map)
+    lib().gs_e_div_u_sum_cpu(C.c_int(fmt), _p(a), _p(b), C.c_int64(nmaj), C.c_int64(nnz),
+                             _p(em), _p(ufeat), _p(efeat), _p(out), C.c_int(u_target),
+                             C.c_int64(elen))
+    return out

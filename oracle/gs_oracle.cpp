@@ -403,4 +403,194 @@ void gs_split_indptr_cpu(const int64_t* indptr, const int64_t* offset,
   }
 }
 
+// -------------------------------------------------------------------------
+// Edge-wise compute operators (DGL-derived in the reference).
+//  endpoints: COO src = row[e], dst = col[e] (src/cuda/sddmm.cu:37-38);
+//  compressed src = indices[e], dst = UpperBound(indptr, e) - 1 (:134-135);
+//  eid = edge_map ? edge_map[e] : e (:39,136).
+//  SDDMM  out[eid*len + f] = op(lhs[sel_l*lhs_len + off_l[f]*red], rhs[...])  (:40-57)
+//  SpMM   COO: out[dst] (+)= op(u[src], e[eid]) with src/dst swapped when
+//         u_target != 0 (src/cuda/spmm.cu:39-56); compressed: per segment
+//         accumulate from 0, then out += acc (:122-141).  Max / Min start from
+//         0 as well because the accumulator / output start at 0.
+//  e^2 sum (src/cuda/fusion/fused_csc_e_square_sum.cu:49-54), e/u sum
+//  (fused_csc_e_div_u_sum.cu:43: BinaryOp::Call(eoff, uoff)).
+}  // extern "C"
+
+namespace {
+template <typename T>
+T apply_op(int op, const T* l, const T* r, int64_t red) {
+  switch (op) {
+    case 0: return l[0] + r[0];
+    case 1: return l[0] - r[0];
+    case 2: return l[0] * r[0];
+    case 3: return l[0] / r[0];
+    case 4: return l[0];
+    case 5: return r[0];
+    default: {
+      T acc = 0;
+      for (int64_t k = 0; k < red; ++k) acc += l[k] * r[k];
+      return acc;
+    }
+  }
+}
+
+struct View {
+  int format;
+  const int64_t *a, *b;
+  int64_t num_major;
+  const int64_t* edge_map;
+  void endpoints(int64_t e, int64_t* src, int64_t* dst, int64_t* eid) const {
+    if (format == 2) {
+      *src = b[e];
+      *dst = (std::upper_bound(a, a + num_major + 1, e) - a) - 1;
+    } else {
+      *src = a[e];
+      *dst = b[e];
+    }
+    *eid = edge_map ? edge_map[e] : e;
+  }
+};
+
+template <typename T>
+void sddmm_impl(const View& g, int64_t nnz, int op, const T* lhs, const T* rhs,
+                T* out, int lt, int rt, int64_t lhs_len, int64_t rhs_len,
+                int64_t out_len, int64_t red, const int64_t* lo,
+                const int64_t* ro) {
+  for (int64_t e = 0; e < nnz; ++e) {
+    int64_t src, dst, eid;
+    g.endpoints(e, &src, &dst, &eid);
+    int64_t ls = lt == 0 ? src : (lt == 1 ? eid : dst);
+    int64_t rs = rt == 0 ? src : (rt == 1 ? eid : dst);
+    for (int64_t f = 0; f < out_len; ++f) {
+      const T* l = op == 5 ? nullptr : lhs + ls * lhs_len + (lo ? lo[f] : f) * red;
+      const T* r = op == 4 ? nullptr : rhs + rs * rhs_len + (ro ? ro[f] : f) * red;
+      out[eid * out_len + f] = apply_op<T>(op, l, r, red);
+    }
+  }
+}
+
+float edge_value(int kind, int op, const float* u, const float* e) {
+  if (kind == 1) return e[0] * e[0];
+  if (kind == 2) return e[0] / u[0];
+  return apply_op<float>(op, u, e, 1);
+}
+
+void spmm_impl(const View& g, int64_t nnz, int kind, int op, int reduce,
+               const float* ufeat, const float* efeat, float* out,
+               int64_t* arg_u, int64_t* arg_e, int u_target, int64_t ulen,
+               int64_t elen, int64_t out_len, const int64_t* uo,
+               const int64_t* eo) {
+  auto better = [&](float v, float cur) {
+    return reduce == 1 ? v > cur : v < cur;
+  };
+  if (g.format == 2) {
+    for (int64_t c = 0; c < g.num_major; ++c)
+      for (int64_t f = 0; f < out_len; ++f) {
+        float acc = 0.f;
+        int64_t bu = 0, be = 0;
+        for (int64_t i = g.a[c]; i < g.a[c + 1]; ++i) {
+          int64_t eid = g.edge_map ? g.edge_map[i] : i, cid = g.b[i];
+          float v = edge_value(kind, op,
+                               ufeat ? ufeat + cid * ulen + (uo ? uo[f] : f) : nullptr,
+                               efeat ? efeat + eid * elen + (eo ? eo[f] : f) : nullptr);
+          if (reduce == 0)
+            acc += v;
+          else if (better(v, acc)) {
+            acc = v;
+            bu = cid;
+            be = eid;
+          }
+        }
+        out[c * out_len + f] += acc;
+        if (reduce != 0) {
+          if (arg_u) arg_u[c * out_len + f] = bu;
+          if (arg_e) arg_e[c * out_len + f] = be;
+        }
+      }
+    return;
+  }
+  for (int64_t e = 0; e < nnz; ++e) {
+    int64_t src = u_target == 0 ? g.a[e] : g.b[e];
+    int64_t dst = u_target == 0 ? g.b[e] : g.a[e];
+    int64_t eid = g.edge_map ? g.edge_map[e] : e;
+    for (int64_t f = 0; f < out_len; ++f) {
+      float v = edge_value(kind, op,
+                           ufeat ? ufeat + src * ulen + (uo ? uo[f] : f) : nullptr,
+                           efeat ? efeat + eid * elen + (eo ? eo[f] : f) : nullptr);
+      float& o = out[dst * out_len + f];
+      if (reduce == 0)
+        o += v;
+      else if (better(v, o)) {
+        o = v;
+        if (arg_u) arg_u[dst * out_len + f] = src;
+        if (arg_e) arg_e[dst * out_len + f] = eid;
+      }
+    }
+  }
+}
+}  // namespace
+
+extern "C" {
+
+void gs_sddmm_cpu(int format, const int64_t* a, const int64_t* b,
+                  int64_t num_major, int64_t nnz, const int64_t* edge_map,
+                  int op, int dtype, const void* lhs, const void* rhs, void* out,
+                  int lhs_target, int rhs_target, int64_t lhs_len,
+                  int64_t rhs_len, int64_t out_len, int64_t reduce_size,
+                  const int64_t* lhs_off, const int64_t* rhs_off) {
+  View g{format, a, b, num_major, edge_map};
+  if (dtype == 0)
+    sddmm_impl<float>(g, nnz, op, (const float*)lhs, (const float*)rhs,
+                      (float*)out, lhs_target, rhs_target, lhs_len, rhs_len,
+                      out_len, reduce_size, lhs_off, rhs_off);
+  else
+    sddmm_impl<double>(g, nnz, op, (const double*)lhs, (const double*)rhs,
+                       (double*)out, lhs_target, rhs_target, lhs_len, rhs_len,
+                       out_len, reduce_size, lhs_off, rhs_off);
+}
+
+void gs_fused_u_op_v_cpu(int format, const int64_t* a, const int64_t* b,
+                         int64_t num_major, int64_t nnz, int op, int dtype,
+                         const void* lhs1, const void* rhs1, void* out1,
+                         const void* lhs2, const void* rhs2, void* out2,
+                         int64_t lhs_len, int64_t rhs_len, int64_t out_len,
+                         int64_t reduce_size, const int64_t* lhs_off,
+                         const int64_t* rhs_off) {
+  gs_sddmm_cpu(format, a, b, num_major, nnz, nullptr, op, dtype, lhs1, rhs1, out1,
+               0, 2, lhs_len, rhs_len, out_len, reduce_size, lhs_off, rhs_off);
+  gs_sddmm_cpu(format, a, b, num_major, nnz, nullptr, op, dtype, lhs2, rhs2, out2,
+               0, 2, lhs_len, rhs_len, out_len, reduce_size, lhs_off, rhs_off);
+}
+
+void gs_spmm_cpu(int format, const int64_t* a, const int64_t* b,
+                 int64_t num_major, int64_t nnz, const int64_t* edge_map, int op,
+                 int reduce, const float* ufeat, const float* efeat, float* out,
+                 int64_t* arg_u, int64_t* arg_e, int u_target, int64_t ufeat_len,
+                 int64_t efeat_len, int64_t out_len, const int64_t* u_off,
+                 const int64_t* e_off) {
+  View g{format, a, b, num_major, edge_map};
+  spmm_impl(g, nnz, 0, op, reduce, op == 5 ? nullptr : ufeat,
+            op == 4 ? nullptr : efeat, out, arg_u, arg_e, u_target, ufeat_len,
+            efeat_len, out_len, u_off, e_off);
+}
+
+void gs_e_square_sum_cpu(int format, const int64_t* a, const int64_t* b,
+                         int64_t num_major, int64_t nnz, const int64_t* edge_map,
+                         const float* efeat, float* out, int u_target,
+                         int64_t feat_len) {
+  View g{format, a, b, num_major, edge_map};
+  spmm_impl(g, nnz, 1, 5, 0, nullptr, efeat, out, nullptr, nullptr, u_target, 0,
+            feat_len, feat_len, nullptr, nullptr);
+}
+
+void gs_e_div_u_sum_cpu(int format, const int64_t* a, const int64_t* b,
+                        int64_t num_major, int64_t nnz, const int64_t* edge_map,
+                        const float* ufeat, const float* efeat, float* out,
+                        int u_target, int64_t feat_len) {
+  View g{format, a, b, num_major, edge_map};
+  spmm_impl(g, nnz, 2, 3, 0, ufeat, efeat, out, nullptr, nullptr, u_target,
+            feat_len, feat_len, feat_len, nullptr, nullptr);
+}
+
 }  // extern "C"
