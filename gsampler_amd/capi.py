@@ -66,6 +66,9 @@ SIGNATURES = {
                        _i64, _i64, _i64, _p, _p, _p]),
     "gs_e_square_sum": (_int, [_int, _p, _p, _i64, _i64, _p, _p, _p, _int, _i64, _p]),
     "gs_e_div_u_sum": (_int, [_int, _p, _p, _i64, _i64, _p, _p, _p, _p, _int, _i64, _p]),
+    "gs_minor_slice_workspace_bytes": (_sz, [_i64, _i64]),
+    "gs_minor_slice_count": (_int, [_p, _i64, _p, _i64, _p, _i64, _p, _p, _p, _sz, _p]),
+    "gs_minor_slice_fill": (_int, [_p, _i64, _i64, _p, _i64, _p, _p, _p, _p, _p, _sz, _p]),
 }
 
 _lib = None
@@ -398,3 +401,34 @@ def e_div_u_sum(view, ufeat, efeat, u_target, n_out, edge_map=None):
                                _fptr(ufeat), _fptr(efeat), _fptr(out), u_target, elen,
                                _stream()))
     return out
+
+
+def minor_slice(ids, picked, indptr=None, edge_major=None, with_major=True):
+    """Keep edges whose id is in `picked`.
+    -> (out_indptr | None, out_major | None, out_minor, out_select)"""
+    ids, picked = _i64t(ids, "ids"), _i64t(picked, "picked")
+    dev = ids.device
+    nnz, npick = ids.numel(), picked.numel()
+    nmaj = 0
+    out_indptr = None
+    if indptr is not None:
+        indptr = _i64t(indptr, "indptr")
+        nmaj = indptr.numel() - 1
+        out_indptr = torch.empty(nmaj + 1, dtype=torch.int64, device=dev)
+    if edge_major is not None:
+        edge_major = _i64t(edge_major, "edge_major")
+    l = lib()
+    ws = _workspace(l.gs_minor_slice_workspace_bytes(nnz, npick), dev)
+    total = torch.empty(1, dtype=torch.int64, device=dev)
+    check(l.gs_minor_slice_count(_ptr(ids), nnz, _ptr(picked), npick, _ptr(indptr), nmaj,
+                                 _ptr(out_indptr), total.data_ptr(), ws.data_ptr(),
+                                 ws.numel(), _stream()))
+    kept = int(total.item())
+    out_minor = torch.empty(kept, dtype=torch.int64, device=dev)
+    out_select = torch.empty(kept, dtype=torch.int64, device=dev)
+    want_major = with_major and (indptr is not None or edge_major is not None)
+    out_major = torch.empty(kept, dtype=torch.int64, device=dev) if want_major else None
+    check(l.gs_minor_slice_fill(_ptr(ids), nnz, npick, _ptr(indptr), nmaj, _ptr(edge_major),
+                                _ptr(out_major), _ptr(out_minor), _ptr(out_select),
+                                ws.data_ptr(), ws.numel(), _stream()))
+    return out_indptr, out_major, out_minor, out_select

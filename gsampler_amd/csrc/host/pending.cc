@@ -9,12 +9,6 @@ namespace gs {
 #define GS_PENDING(what) \
   TORCH_CHECK(false, what, " is not implemented in this build of gsampler_amd")
 
-MajorResult minor_slice(const Compressed&, const torch::Tensor&, bool) {
-  GS_PENDING("slicing across the compressed axis");
-}
-GraphAndIndex Graph::slice_coo(const torch::Tensor&, int64_t, int64_t, int64_t) {
-  GS_PENDING("COO slicing");
-}
 GraphAndIndex Graph::SamplingProbs(int64_t, torch::Tensor, int64_t, bool, int64_t,
                                    int64_t) {
   GS_PENDING("weighted per-column sampling");

@@ -17,11 +17,11 @@
 //   pass 4  relabel  one lookup per edge row; columns come from the per-seed
 //                    rank array written in pass 3
 #include "common.h"
+#include "hashtable.h"
 #include "scan.h"
 
 namespace gs {
 
-constexpr uint64_t kEmptySlot = ~0ull;
 constexpr int kWordsPerBlock = kBlock / kWave;
 
 struct UniqueWs {
@@ -49,14 +49,6 @@ static UniqueWs carve_unique(void* ws, int64_t S, int64_t E, int64_t B) {
   w.scan_ws = c.take<char>(w.scan_ws_bytes);
   w.total = c.total();
   return w;
-}
-
-__device__ __forceinline__ uint32_t hash32(uint64_t key) {
-  return (uint32_t)((key * 0x9E3779B97F4A7C15ull) >> 32);
-}
-// slot index in [0, cap)
-__device__ __forceinline__ uint64_t home_slot(uint64_t key, uint64_t cap) {
-  return ((uint64_t)hash32(key) * cap) >> 32;
 }
 
 // Where a flat position lives: batch, position inside the batch, key.
@@ -101,14 +93,6 @@ __global__ void unique_flat_ptr_kernel(const int64_t* seeds_ptr, int64_t S,
   flat_ptr[b] = s + r;
 }
 
-__global__ __launch_bounds__(kBlock) void unique_clear_kernel(uint64_t* table,
-                                                              int64_t n,
-                                                              uint64_t value) {
-  int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
-  const int64_t stride = (int64_t)gridDim.x * kBlock;
-  for (; i < n; i += stride) table[i] = value;
-}
-
 __global__ __launch_bounds__(kBlock) void unique_insert_kernel(
     const int64_t* __restrict__ flat_ptr, int64_t B,
     const int64_t* __restrict__ seeds, const int64_t* __restrict__ seeds_ptr,
@@ -117,37 +101,15 @@ __global__ __launch_bounds__(kBlock) void unique_insert_kernel(
   const int64_t p = (int64_t)blockIdx.x * kBlock + threadIdx.x;
   if (p >= N) return;
   const FlatItem it = locate(p, flat_ptr, B, seeds, seeds_ptr, S, rows, rows_ptr);
-  const uint64_t mine = (it.key << 32) | (uint64_t)it.local;
-  uint64_t* tab = table + it.table_base;
-  uint64_t slot = home_slot(it.key, it.cap);
-  // cap = 2 * (keys of the batch), so an empty slot always turns up; the probe
-  // budget only guards against inconsistent pointer arrays.
-  for (uint64_t probes = 0; probes < it.cap; ++probes) {
-    uint64_t cur = tab[slot];
-    if (cur == kEmptySlot) {
-      cur = atomicCAS((unsigned long long*)(tab + slot),
-                      (unsigned long long)kEmptySlot, (unsigned long long)mine);
-      if (cur == kEmptySlot) return;
-    }
-    if ((cur >> 32) == it.key) {
-      // values only ever decrease, so a stale read can only cost an atomic
-      if (cur > mine)
-        atomicMin((unsigned long long*)(tab + slot), (unsigned long long)mine);
-      return;
-    }
-    if (++slot == it.cap) slot = 0;
-  }
+  table_insert_min(table + it.table_base, it.cap, it.key, (uint64_t)it.local);
 }
 
+// Keys looked up here were all inserted, so the slot always exists; slot 0
+// stands in if a caller passed inconsistent pointer arrays.
 __device__ __forceinline__ uint64_t find_slot(const uint64_t* tab, uint64_t cap,
                                               uint64_t key) {
-  uint64_t slot = home_slot(key, cap);
-  for (uint64_t probes = 0; probes < cap; ++probes) {
-    uint64_t cur = tab[slot];
-    if ((cur >> 32) == key) return slot;
-    if (++slot == cap) slot = 0;
-  }
-  return 0;  // unreachable for keys that were inserted
+  const uint64_t slot = table_find(tab, cap, key);
+  return slot < cap ? slot : 0;
 }
 
 __global__ __launch_bounds__(kBlock) void unique_flag_kernel(
@@ -300,7 +262,7 @@ int gs_unique_count(const int64_t* seeds, const int64_t* seeds_ptr,
   const int64_t N = S + E;
   if (N == 0) {
     GS_LAUNCH("unique_clear", s,
-              unique_clear_kernel<<<dim3((unsigned)ceil_div(B + 1, kBlock)),
+              table_fill_kernel<><<<dim3((unsigned)ceil_div(B + 1, kBlock)),
                                     dim3(kBlock), 0, s>>>((uint64_t*)unique_ptr,
                                                           B + 1, 0ull));
     return GS_OK;
@@ -314,7 +276,7 @@ int gs_unique_count(const int64_t* seeds, const int64_t* seeds_ptr,
     const int64_t slots = 2 * N;
     int64_t blocks = ceil_div(slots, kBlock * 8);
     GS_LAUNCH("unique_clear", s,
-              unique_clear_kernel<<<dim3((unsigned)blocks), dim3(kBlock), 0, s>>>(
+              table_fill_kernel<><<<dim3((unsigned)blocks), dim3(kBlock), 0, s>>>(
                   w.table, slots, kEmptySlot));
   }
   GS_LAUNCH("unique_insert", s,

@@ -189,6 +189,33 @@ int gs_unique_relabel(const int64_t* seeds, const int64_t* seeds_ptr,
                       size_t workspace_bytes, gs_stream_t stream);
 
 /* ------------------------------------------------------------------------
+ * Slicing across the compressed axis (row slicing of a CSC, A[picked, :]) and
+ * coordinate-form slicing: keep the edges whose id in `ids[nnz]` belongs to
+ * `picked[num_picked]`, relabel that id to its position in `picked` (smallest
+ * position for a repeated id), keep the edge order.
+ *  count: with indptr given writes out_indptr[num_major + 1] (all segments
+ *    kept, out_indptr[num_major] = number of kept edges); out_total (nullable,
+ *    device) receives the number of kept edges.
+ *  fill:  same ids / workspace; out_minor[kept] = position in `picked`,
+ *    out_select[kept] = edge position, out_major[kept] (nullable) =
+ *    edge_major[e] if given else the segment of indptr holding e.
+ * Ids must be < 2^32 - 1.  Stands in for OnIndicesSlicingCUDA
+ * (src/cuda/slicing.cu:296-307) and COORowSlicingCUDA (src/cuda/slicing.cu:374-377).
+ * ---------------------------------------------------------------------- */
+size_t gs_minor_slice_workspace_bytes(int64_t nnz, int64_t num_picked);
+int gs_minor_slice_count(const int64_t* ids, int64_t nnz, const int64_t* picked,
+                         int64_t num_picked, const int64_t* indptr,
+                         int64_t num_major, int64_t* out_indptr,
+                         int64_t* out_total, void* workspace,
+                         size_t workspace_bytes, gs_stream_t stream);
+int gs_minor_slice_fill(const int64_t* ids, int64_t nnz, int64_t num_picked,
+                        const int64_t* indptr, int64_t num_major,
+                        const int64_t* edge_major, int64_t* out_major,
+                        int64_t* out_minor, int64_t* out_select,
+                        void* workspace, size_t workspace_bytes,
+                        gs_stream_t stream);
+
+/* ------------------------------------------------------------------------
  * Format conversion.
  *  gs_csc2coo: out_col[e] = column that owns edge position e
  *    (CSC2COOCUDA, src/cuda/format_transform.cu:24-46).

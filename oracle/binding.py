@@ -289,3 +289,26 @@ def e_div_u_sum(view, ufeat, efeat, u_target, n_out, edge_map=None):
                              _p(em), _p(ufeat), _p(efeat), _p(out), C.c_int(u_target),
                              C.c_int64(elen))
     return out
+
+
+def minor_slice(ids, picked, indptr=None, edge_major=None, with_major=True):
+    ids, picked = _i64(ids), _i64(picked)
+    nmaj = 0
+    out_indptr = None
+    if indptr is not None:
+        indptr = _i64(indptr)
+        nmaj = indptr.size - 1
+        out_indptr = np.empty(nmaj + 1, dtype=np.int64)
+    if edge_major is not None:
+        edge_major = _i64(edge_major)
+    total = np.zeros(1, dtype=np.int64)
+    args = [_p(ids), C.c_int64(ids.size), _p(picked), C.c_int64(picked.size), _p(indptr),
+            C.c_int64(nmaj), _p(edge_major), _p(out_indptr), _p(total)]
+    lib().gs_minor_slice_cpu(*args, None, None, None)
+    kept = int(total[0])
+    out_minor = np.empty(kept, dtype=np.int64)
+    out_select = np.empty(kept, dtype=np.int64)
+    want_major = with_major and (indptr is not None or edge_major is not None)
+    out_major = np.empty(kept, dtype=np.int64) if want_major else None
+    lib().gs_minor_slice_cpu(*args, _p(out_major), _p(out_minor), _p(out_select))
+    return out_indptr, out_major, out_minor, out_select

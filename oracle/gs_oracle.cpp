@@ -594,3 +594,42 @@ void gs_e_div_u_sum_cpu(int format, const int64_t* a, const int64_t* b,
 }
 
 }  // extern "C"
+
+// -------------------------------------------------------------------------
+// Slicing across the compressed axis and COO slicing.
+//  src/cuda/slicing.cu:185-229 (_OnIndicesSlicinigQueryKernel): every edge whose
+//  row id is in the picked set is kept, its row becomes the value stored for it
+//  in the set's hash map, edge order is preserved, every column is kept
+//  (:283-293 compaction by nonzero(mask)).  src/cuda/slicing.cu:312-371: the
+//  coordinate form keeps (relabelled id, other id, position).
+//  The reference stores the position of whichever duplicate wrote last
+//  (:56 `vptr[pos] = value`, racy); this restatement keeps the smallest.
+extern "C" void gs_minor_slice_cpu(const int64_t* ids, int64_t nnz,
+                                   const int64_t* picked, int64_t num_picked,
+                                   const int64_t* indptr, int64_t num_major,
+                                   const int64_t* edge_major, int64_t* out_indptr,
+                                   int64_t* out_total, int64_t* out_major,
+                                   int64_t* out_minor, int64_t* out_select) {
+  std::unordered_map<int64_t, int64_t> where;
+  for (int64_t i = 0; i < num_picked; ++i) where.emplace(picked[i], i);
+  int64_t kept = 0, c = 0;
+  if (out_indptr) out_indptr[0] = 0;
+  for (int64_t e = 0; e < nnz; ++e) {
+    if (indptr)
+      while (c < num_major && indptr[c + 1] <= e) {
+        ++c;
+        if (out_indptr) out_indptr[c] = kept;
+      }
+    auto it = where.find(ids[e]);
+    if (it == where.end()) continue;
+    if (out_minor) {
+      out_minor[kept] = it->second;
+      out_select[kept] = e;
+      if (out_major) out_major[kept] = edge_major ? edge_major[e] : c;
+    }
+    ++kept;
+  }
+  if (out_indptr)
+    for (int64_t k = c + 1; k <= num_major; ++k) out_indptr[k] = kept;
+  if (out_total) *out_total = kept;
+}
