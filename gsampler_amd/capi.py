@@ -69,6 +69,14 @@ SIGNATURES = {
     "gs_minor_slice_workspace_bytes": (_sz, [_i64, _i64]),
     "gs_minor_slice_count": (_int, [_p, _i64, _p, _i64, _p, _i64, _p, _p, _p, _sz, _p]),
     "gs_minor_slice_fill": (_int, [_p, _i64, _i64, _p, _i64, _p, _p, _p, _p, _p, _sz, _p]),
+    "gs_csc_col_sample_weighted_fill": (_int, [_p, _i64, _p, _p, _p, _i64, _i64, _int, _u64,
+                                               _u64, _p, _p, _p, _p, _p, _p, _p]),
+    "gs_weighted_key_probe": (_int, [_u64, _u64, _u64, _u64, C.c_float, _u64, _p, _p]),
+    "gs_list_sample_uniform": (_int, [_i64, _i64, _int, _int, _u64, _u64, _p, _p]),
+    "gs_list_sample_workspace_bytes": (_sz, [_i64, _i64]),
+    "gs_list_sample_weighted_count": (_int, [_p, _i64, _i64, _i64, _int, _p, _p, _sz, _p]),
+    "gs_list_sample_weighted_fill": (_int, [_p, _p, _i64, _i64, _i64, _int, _u64, _u64, _p,
+                                            _i64, _p, _p, _sz, _p]),
 }
 
 _lib = None
@@ -432,3 +440,81 @@ def minor_slice(ids, picked, indptr=None, edge_major=None, with_major=True):
                                 _ptr(out_major), _ptr(out_minor), _ptr(out_select),
                                 ws.data_ptr(), ws.numel(), _stream()))
     return out_indptr, out_major, out_minor, out_select
+
+
+# --------------------------------------------------------- weighted sampling
+def weighted_key_probe(seed, call_id, pos, draw, w, r64):
+    """(-log2 of the unit draw r64, key of weight w) evaluated on the device."""
+    out = torch.zeros(2, dtype=torch.float64, device="cuda")
+    check(lib().gs_weighted_key_probe(seed, call_id, pos, draw, w, r64, out.data_ptr(),
+                                      _stream()))
+    return out.cpu().tolist()
+
+
+def sample_weighted(indptr, indices, probs, column_ids, fanout, replace=False, seed=7777,
+                    call_id=0, with_coo=True):
+    """Weighted per-column sampling -> (sub_indptr, coo_col | None, sub_indices, select)."""
+    indptr, indices = _i64t(indptr, "indptr"), _i64t(indices, "indices")
+    probs = probs.contiguous()
+    if probs.dtype != torch.float32:
+        raise GsError("probs must be float32")
+    num_cols = indptr.numel() - 1
+    dev = indptr.device
+    if column_ids is not None:
+        column_ids = _i64t(column_ids, "column_ids")
+        n = column_ids.numel()
+    else:
+        n = num_cols
+    sub_indptr = col_count(indptr, column_ids, fanout, replace, n)
+    nnz = int(sub_indptr[-1].item())
+    out_idx = torch.empty(nnz, dtype=torch.int64, device=dev)
+    out_sel = torch.empty(nnz, dtype=torch.int64, device=dev)
+    out_col = torch.empty(nnz, dtype=torch.int64, device=dev) if with_coo else None
+    cdf_off = scratch = None
+    if replace:
+        if column_ids is not None:
+            cdf_off = col_count(indptr, column_ids, -1, False)
+            scratch = torch.empty(int(cdf_off[-1].item()) + 1, dtype=torch.int64, device=dev)
+        else:
+            scratch = torch.empty(indices.numel() + 1, dtype=torch.int64, device=dev)
+    if nnz > 0:
+        check(lib().gs_csc_col_sample_weighted_fill(
+            _ptr(indptr), num_cols, _ptr(indices), probs.data_ptr(), _ptr(column_ids), n,
+            fanout, int(replace), seed, call_id, sub_indptr.data_ptr(), _ptr(cdf_off),
+            _ptr(scratch), _ptr(out_col), out_idx.data_ptr(), out_sel.data_ptr(), _stream()))
+    return sub_indptr, out_col, out_idx, out_sel
+
+
+def list_sample_uniform(n, num_picks, replace=False, algo=ALGO_AUTO, seed=7777, call_id=0,
+                        device="cuda"):
+    count = (num_picks if n > 0 else 0) if replace else min(n, num_picks)
+    out = torch.empty(count, dtype=torch.int64, device=device)
+    check(lib().gs_list_sample_uniform(n, num_picks, int(replace), algo, seed, call_id,
+                                       _ptr(out), _stream()))
+    return out
+
+
+def list_sample_weighted(probs, num_picks, replace=False, range_=None, seed=7777, call_id=0):
+    """-> (index, out_range)"""
+    probs = probs.contiguous()
+    if probs.dtype != torch.float32 or not probs.is_cuda:
+        raise GsError("probs must be a CUDA float32 tensor")
+    dev = probs.device
+    n = probs.numel()
+    nseg = 1
+    if range_ is not None:
+        range_ = _i64t(range_, "range")
+        nseg = range_.numel() - 1
+    l = lib()
+    ws = _workspace(l.gs_list_sample_workspace_bytes(n, nseg), dev)
+    out_range = torch.empty(nseg + 1, dtype=torch.int64, device=dev)
+    check(l.gs_list_sample_weighted_count(_ptr(range_), n, nseg, num_picks, int(replace),
+                                          out_range.data_ptr(), ws.data_ptr(), ws.numel(),
+                                          _stream()))
+    total = int(out_range[-1].item())
+    out = torch.empty(total, dtype=torch.int64, device=dev)
+    check(l.gs_list_sample_weighted_fill(_fptr(probs), _ptr(range_), n, nseg, num_picks,
+                                         int(replace), seed, call_id, out_range.data_ptr(),
+                                         total, _ptr(out), ws.data_ptr(), ws.numel(),
+                                         _stream()))
+    return out, out_range

@@ -9,10 +9,6 @@ namespace gs {
 #define GS_PENDING(what) \
   TORCH_CHECK(false, what, " is not implemented in this build of gsampler_amd")
 
-GraphAndIndex Graph::SamplingProbs(int64_t, torch::Tensor, int64_t, bool, int64_t,
-                                   int64_t) {
-  GS_PENDING("weighted per-column sampling");
-}
 GraphAndIndex Graph::Compact(int64_t) { GS_PENDING("Compact"); }
 torch::Tensor Graph::RandomWalk(torch::Tensor, int64_t) { GS_PENDING("RandomWalk"); }
 torch::Tensor Graph::Node2Vec(torch::Tensor, int64_t, double, double) {
@@ -23,18 +19,4 @@ GraphAndIndex Graph::BatchColRowSlcing(torch::Tensor, torch::Tensor, torch::Tens
                                        torch::Tensor) {
   GS_PENDING("BatchColRowSlcing");
 }
-torch::Tensor ListSampling(int64_t, int64_t, bool) { GS_PENDING("ListSampling"); }
-torch::Tensor ListSamplingProbs(torch::Tensor, int64_t, bool) {
-  GS_PENDING("ListSamplingProbs");
-}
-std::tuple<torch::Tensor, torch::Tensor> BatchListSamplingProbs(torch::Tensor,
-                                                                int64_t, bool,
-                                                                torch::Tensor) {
-  GS_PENDING("BatchListSamplingProbs");
-}
-std::tuple<torch::Tensor, torch::Tensor> BatchListSampling(int64_t, bool,
-                                                           torch::Tensor) {
-  GS_PENDING("BatchListSampling");
-}
-
 }  // namespace gs

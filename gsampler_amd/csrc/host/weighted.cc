@@ -1,0 +1,118 @@
+// weighted.cc -- weighted per-column sampling and the collective (list)
+// sampling operators.
+#include "abi_call.h"
+#include "graph.h"
+
+namespace gs {
+
+static uint64_t take_call_id() { return random_state().next_call++; }
+
+static torch::Tensor f32(const torch::Tensor& t, const char* name) {
+  TORCH_CHECK(t.defined() && t.is_cuda(), name, " must live on the GPU");
+  TORCH_CHECK(t.scalar_type() == torch::kFloat32, name, " must be float32 (got ",
+              t.scalar_type(), ")");
+  return t.contiguous();
+}
+
+GraphAndIndex Graph::SamplingProbs(int64_t axis, torch::Tensor edge_probs,
+                                   int64_t fanout, bool replace,
+                                   int64_t on_format, int64_t output_format) {
+  TORCH_CHECK((axis == 1 && on_format == kCSC) || (axis == 0 && on_format == kCSR),
+              "SamplingProbs: not implemented for axis ", axis, " on format ",
+              on_format);
+  const int64_t other = on_format == kCSC ? kCSR : kCSC;
+  TORCH_CHECK(output_format != other, "SamplingProbs: on_format ", on_format,
+              " cannot produce output_format ", output_format);
+  TORCH_CHECK(fanout >= 0, "fanout must be non-negative, got ", fanout);
+  const Compressed& m = compressed(on_format);
+  torch::Tensor probs = f32(edge_probs, "edge_probs");
+  TORCH_CHECK(probs.numel() == m.indices.numel(), "SamplingProbs: ", probs.numel(),
+              " probabilities for ", m.indices.numel(), " edges");
+  // probabilities follow the original edge order; bring them into this
+  // format's order (src/graph_ops.cc:138-142 of the reference)
+  if (m.e_ids.has_value()) probs = probs.index_select(0, m.e_ids.value());
+  const bool with_coo = output_format & kCOO;
+  const int64_t n = m.indptr.numel() - 1;
+  MajorResult r;
+  r.indptr = new_ids(n + 1, m.indptr);
+  torch::Tensor ws = new_workspace(gs_scan_workspace_bytes(n + 1), m.indptr);
+  GS_CALL(gs_csc_col_count(cptr(m.indptr), n, nullptr, n, fanout, replace ? 1 : 0,
+                           mptr(r.indptr), ws.data_ptr(), ws.numel(), cur_stream()));
+  const int64_t nnz = read_last(r.indptr);
+  r.minor_ids = new_ids(nnz, m.indptr);
+  r.select = new_ids(nnz, m.indptr);
+  if (with_coo) r.major_ids = new_ids(nnz, m.indptr);
+  torch::Tensor scratch;
+  if (replace) scratch = new_ids(m.indices.numel() + 1, m.indptr);
+  const RandomState& rs = random_state();
+  GS_CALL(gs_csc_col_sample_weighted_fill(
+      cptr(m.indptr), n, cptr(m.indices), probs.data_ptr<float>(), nullptr, n,
+      fanout, replace ? 1 : 0, rs.seed, take_call_id(), cptr(r.indptr), nullptr,
+      replace ? scratch.data_ptr() : nullptr,
+      with_coo ? mptr(r.major_ids) : nullptr, mptr(r.minor_ids), mptr(r.select),
+      cur_stream()));
+  GraphPtr g = derive(on_format, output_format, r, num_rows_, num_cols_);
+  return {g, edge_index(m.e_ids, r.select)};
+}
+
+// ------------------------------------------------------------ list sampling
+torch::Tensor ListSampling(int64_t num_items, int64_t num_picks, bool replace) {
+  TORCH_CHECK(num_items >= 0 && num_picks >= 0, "ListSampling: negative size");
+  const int64_t count = replace ? (num_items > 0 ? num_picks : 0)
+                                : std::min(num_items, num_picks);
+  torch::Tensor out = torch::empty(
+      {count}, torch::TensorOptions().dtype(torch::kInt64).device(torch::kCUDA));
+  const RandomState& rs = random_state();
+  GS_CALL(gs_list_sample_uniform(num_items, num_picks, replace ? 1 : 0,
+                                 (int)rs.algo, rs.seed, take_call_id(), mptr(out),
+                                 cur_stream()));
+  return out;
+}
+
+static std::tuple<torch::Tensor, torch::Tensor> list_weighted(
+    const torch::Tensor& probs_in, int64_t num_picks, bool replace,
+    const torch::Tensor& range) {
+  TORCH_CHECK(num_picks >= 0, "list sampling: negative number of picks");
+  torch::Tensor probs = f32(probs_in, "probs");
+  const int64_t n = probs.numel();
+  const int64_t nseg = range.defined() ? range.numel() - 1 : 1;
+  TORCH_CHECK(nseg >= 1, "list sampling: range needs at least two entries");
+  torch::Tensor ws = new_workspace(gs_list_sample_workspace_bytes(n, nseg), probs);
+  torch::Tensor out_range = new_ids(nseg + 1, probs);
+  GS_CALL(gs_list_sample_weighted_count(cptr(range), n, nseg, num_picks,
+                                        replace ? 1 : 0, mptr(out_range),
+                                        ws.data_ptr(), ws.numel(), cur_stream()));
+  const int64_t total = read_last(out_range);
+  torch::Tensor out = new_ids(total, probs);
+  const RandomState& rs = random_state();
+  GS_CALL(gs_list_sample_weighted_fill(
+      probs.data_ptr<float>(), cptr(range), n, nseg, num_picks, replace ? 1 : 0,
+      rs.seed, take_call_id(), cptr(out_range), total, mptr(out), ws.data_ptr(),
+      ws.numel(), cur_stream()));
+  return {out, out_range};
+}
+
+torch::Tensor ListSamplingProbs(torch::Tensor probs, int64_t num_picks,
+                                bool replace) {
+  return std::get<0>(list_weighted(probs, num_picks, replace, {}));
+}
+
+std::tuple<torch::Tensor, torch::Tensor> BatchListSamplingProbs(
+    torch::Tensor probs, int64_t num_picks, bool replace, torch::Tensor range) {
+  return list_weighted(probs, num_picks, replace, ids(range, "range"));
+}
+
+// Uniform batched selection = weighted selection with unit weights over the
+// items the range covers (src/tensor_ops.cc:21-28 of the reference, which
+// sizes the weights by the number of segments; the number of items is meant).
+std::tuple<torch::Tensor, torch::Tensor> BatchListSampling(int64_t num_picks,
+                                                           bool replace,
+                                                           torch::Tensor range) {
+  range = ids(range, "range");
+  const int64_t n = read_last(range);
+  torch::Tensor ones = torch::ones(
+      {n}, torch::TensorOptions().dtype(torch::kFloat32).device(range.device()));
+  return list_weighted(ones, num_picks, replace, range);
+}
+
+}  // namespace gs

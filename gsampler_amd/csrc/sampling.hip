@@ -40,7 +40,7 @@ __global__ __launch_bounds__(kBlock) void sample_uniform_kernel(
     for (int64_t j = lane; j < fanout; j += G) {
       int64_t p = in_start + (int64_t)philox_bounded(key, pos, (uint64_t)j,
                                                       (uint64_t)deg);
-      out_indices[out_start + j] = indices[p];
+      out_indices[out_start + j] = indices ? indices[p] : p;
       out_select[out_start + j] = p;
       if (out_coo_col) out_coo_col[out_start + j] = item;
     }
@@ -51,7 +51,7 @@ __global__ __launch_bounds__(kBlock) void sample_uniform_kernel(
     // the whole column, original order
     for (int64_t j = lane; j < deg; j += G) {
       int64_t p = in_start + j;
-      out_indices[out_start + j] = indices[p];
+      out_indices[out_start + j] = indices ? indices[p] : p;
       out_select[out_start + j] = p;
       if (out_coo_col) out_coo_col[out_start + j] = item;
     }
@@ -85,7 +85,7 @@ __global__ __launch_bounds__(kBlock) void sample_uniform_kernel(
     }
     if (active) {
       int64_t p = in_start + (dup ? j : t);
-      out_indices[out_start + lane] = indices[p];
+      out_indices[out_start + lane] = indices ? indices[p] : p;
       out_select[out_start + lane] = p;
       if (out_coo_col) out_coo_col[out_start + lane] = item;
     }
@@ -109,7 +109,7 @@ __global__ __launch_bounds__(kBlock) void sample_uniform_kernel(
   __builtin_amdgcn_wave_barrier();
   for (int64_t jj = lane; jj < fanout; jj += G) {
     int64_t p = in_start + load_coherent(out_select + out_start + jj);
-    out_indices[out_start + jj] = indices[p];
+    out_indices[out_start + jj] = indices ? indices[p] : p;
     out_select[out_start + jj] = p;
     if (out_coo_col) out_coo_col[out_start + jj] = item;
   }
@@ -152,7 +152,7 @@ extern "C" int gs_csc_col_sample_uniform_fill(
              "sample_uniform: Floyd sampling needs fanout <= 64, got %lld",
              (long long)fanout);
   if (num_items == 0 || fanout == 0) return GS_OK;
-  GS_REQUIRE(indptr && indices && sub_indptr && out_indices && out_select,
+  GS_REQUIRE(indptr && sub_indptr && out_indices && out_select,
              "sample_uniform: null pointer");
   GS_REQUIRE(column_ids != nullptr || num_items <= num_cols,
              "sample_uniform: %lld items but the matrix has %lld columns",
@@ -169,4 +169,92 @@ extern "C" int gs_csc_col_sample_uniform_fill(
   if (fanout <= 32) return launch_sample_uniform<32>(GS_SAMPLE_ARGS);
   return launch_sample_uniform<64>(GS_SAMPLE_ARGS);
 #undef GS_SAMPLE_ARGS
+}
+
+// ---------------------------------------------------------------------------
+// Uniform collective (list) sampling: K of the positions 0..n-1.  It is the
+// per-column sampler applied to one virtual column whose row ids are the
+// positions themselves (stream position 0), so it produces exactly what
+// gs_csc_col_sample_uniform_fill would for that column; the reservoir form is
+// spread over the whole grid because a list can be far longer than a column.
+namespace gs {
+
+__global__ __launch_bounds__(kBlock) void list_uniform_kernel(
+    int64_t n, int64_t num_picks, int mode, PhiloxKey key,
+    int64_t* __restrict__ out) {
+  // mode 0: with replacement; 1: identity (n <= picks); 2: reservoir slot init
+  const int64_t j = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (j >= num_picks) return;
+  out[j] = mode == 0 ? (int64_t)philox_bounded(key, 0, (uint64_t)j, (uint64_t)n) : j;
+}
+
+__global__ __launch_bounds__(kBlock) void list_reservoir_kernel(
+    int64_t n, int64_t num_picks, PhiloxKey key, int64_t* out) {
+  const int64_t idx = num_picks + (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (idx >= n) return;
+  const int64_t num = (int64_t)philox_bounded(key, 0, (uint64_t)idx, (uint64_t)idx + 1);
+  if (num < num_picks) atomicMax((long long*)(out + num), (long long)idx);
+}
+
+// One wavefront, one lane per slot (num_picks <= 64): the Floyd rule of
+// sample_uniform_kernel on the virtual column.
+__global__ void list_floyd_kernel(int64_t n, int num_picks, PhiloxKey key,
+                                  int64_t* __restrict__ out) {
+  const int lane = threadIdx.x;
+  const int K = num_picks;
+  const int64_t base = n - K;
+  const int64_t j = base + lane;
+  int64_t t = -1;
+  if (lane < K) t = (int64_t)philox_bounded(key, 0, (uint64_t)lane, (uint64_t)j + 1);
+  bool dup = false;
+  for (int m = 0; m < K; ++m) {
+    const int64_t tm = __shfl(t, m, kWave);
+    dup |= (m < lane) & (tm == t);
+  }
+  const int64_t mi = t - base;
+  for (int m = 0; m < K; ++m) {
+    const int dm = __shfl((int)dup, m, kWave);
+    if (mi == m && m < lane) dup |= (dm != 0);
+  }
+  if (lane < K) out[lane] = dup ? j : t;
+}
+
+}  // namespace gs
+
+extern "C" int gs_list_sample_uniform(int64_t n, int64_t num_picks, int replace,
+                                      int algo, uint64_t seed, uint64_t call_id,
+                                      int64_t* out_index, gs_stream_t stream) {
+  using namespace gs;
+  GS_REQUIRE(n >= 0 && num_picks >= 0, "list_sample_uniform: negative size");
+  GS_REQUIRE(algo == GS_ALGO_AUTO || algo == GS_ALGO_RESERVOIR || algo == GS_ALGO_FLOYD,
+             "list_sample_uniform: unknown algorithm %d", algo);
+  const int64_t count = replace ? (n > 0 ? num_picks : 0) : (n < num_picks ? n : num_picks);
+  if (count == 0) return GS_OK;
+  GS_REQUIRE(out_index, "list_sample_uniform: null output");
+  const PhiloxKey key = make_key(seed, call_id);
+  hipStream_t s = as_stream(stream);
+  const unsigned blocks = (unsigned)ceil_div(count, kBlock);
+  if (replace || n <= num_picks) {
+    GS_LAUNCH("list_uniform", s,
+              list_uniform_kernel<<<dim3(blocks), dim3(kBlock), 0, s>>>(
+                  n, count, replace ? 0 : 1, key, out_index));
+    return GS_OK;
+  }
+  if (algo == GS_ALGO_AUTO) algo = num_picks <= 64 ? GS_ALGO_FLOYD : GS_ALGO_RESERVOIR;
+  GS_REQUIRE(!(algo == GS_ALGO_FLOYD && num_picks > 64),
+             "list_sample_uniform: Floyd sampling needs num_picks <= 64");
+  if (algo == GS_ALGO_FLOYD) {
+    GS_LAUNCH("list_floyd", s,
+              list_floyd_kernel<<<dim3(1), dim3(kWave), 0, s>>>(n, (int)num_picks,
+                                                                key, out_index));
+    return GS_OK;
+  }
+  GS_LAUNCH("list_uniform", s,
+            list_uniform_kernel<<<dim3(blocks), dim3(kBlock), 0, s>>>(
+                n, num_picks, 2, key, out_index));
+  GS_LAUNCH("list_reservoir", s,
+            list_reservoir_kernel<<<dim3((unsigned)ceil_div(n - num_picks, kBlock)),
+                                    dim3(kBlock), 0, s>>>(n, num_picks, key,
+                                                          out_index));
+  return GS_OK;
 }

@@ -1,0 +1,509 @@
+// weighted.hip -- weighted sampling: per column (individual) and over a list
+// (collective / layer-wise), with and without replacement.
+//
+// Without replacement: Efraimidis-Spirakis in exponential-clock form.  Item i
+// gets key (-log2 u_i) / w_i, the K smallest keys win (same ranking as the K
+// largest u^(1/w)).  The key uses correctly rounded double operations only, so
+// the CPU check computes bit-identical keys; ties break to the smaller index.
+// With replacement: integer CDF (weights quantised against the exact maximum,
+// integer prefix sums are order-independent) and a binary search per pick.
+#include "common.h"
+#include "scan.h"
+
+#include <cstring>
+#include <rocprim/device/device_radix_sort.hpp>
+#include <rocprim/device/device_segmented_radix_sort.hpp>
+
+namespace gs {
+
+// ------------------------------------------------------------ key arithmetic
+__device__ __forceinline__ double neg_log2_unit(uint64_t r64) {
+  const uint64_t v = (r64 >> 12) + 1;  // [1, 2^52]: exact as a double
+  int e = 63 - __clzll((long long)v);
+  double m = ldexp((double)(long long)v, -e);  // [1, 2)
+  if (m > 0x1.6a09e667f3bcdp+0) {
+    m = __dmul_rn(m, 0.5);
+    e += 1;
+  }
+  const double s = __ddiv_rn(__dsub_rn(m, 1.0), __dadd_rn(m, 1.0));
+  const double s2 = __dmul_rn(s, s);
+  double p = 0x1.1964ec6fc9491p-3;
+  p = __fma_rn(p, s2, 0x1.3703c1f4d0ffep-3);
+  p = __fma_rn(p, s2, 0x1.5b9ac9b743f0dp-3);
+  p = __fma_rn(p, s2, 0x1.89f3b1694cffep-3);
+  p = __fma_rn(p, s2, 0x1.c68f568d31761p-3);
+  p = __fma_rn(p, s2, 0x1.0c9a84994022dp-2);
+  p = __fma_rn(p, s2, 0x1.484b13d7c02a9p-2);
+  p = __fma_rn(p, s2, 0x1.a61762a7adedap-2);
+  p = __fma_rn(p, s2, 0x1.2776c50ef9bfep-1);
+  p = __fma_rn(p, s2, 0x1.ec709dc3a03fep-1);
+  p = __fma_rn(p, s2, 0x1.71547652b82fep+1);
+  return __dsub_rn((double)(52 - e), __dmul_rn(s, p));
+}
+
+__device__ __forceinline__ double weighted_key(PhiloxKey key, uint64_t pos,
+                                               uint64_t draw, float w) {
+  if (!(w > 0.0f)) return __longlong_as_double(0x7ff0000000000000ll);  // +inf
+  const Words4 wd = philox(key, pos, draw);
+  const uint64_t r = ((uint64_t)wd.y << 32) | wd.x;
+  return __ddiv_rn(neg_log2_unit(r), (double)w);
+}
+
+__global__ void weighted_key_probe_kernel(PhiloxKey key, uint64_t pos,
+                                          uint64_t draw, float w, uint64_t r64,
+                                          double* out) {
+  out[0] = neg_log2_unit(r64);
+  out[1] = weighted_key(key, pos, draw, w);
+}
+
+__device__ __forceinline__ bool key_less(double ka, int64_t ia, double kb,
+                                         int64_t ib) {
+  return ka < kb || (ka == kb && ia < ib);
+}
+
+// -------------------------------------------- per column, without replacement
+// One wavefront per requested column.  Every lane keeps the K smallest keys of
+// the edges it visits (lane l sees offsets l, l + 64, ...) as a sorted list in
+// LDS, laid out [slot][thread] so that a wavefront touches consecutive banks.
+// The 64 sorted lists are then merged by K rounds of a wavefront arg-min.
+__global__ __launch_bounds__(kBlock) void sample_weighted_kernel(
+    const int64_t* __restrict__ indptr, int64_t num_cols,
+    const int64_t* __restrict__ indices, const float* __restrict__ probs,
+    const int64_t* __restrict__ column_ids, int64_t num_items, int fanout,
+    PhiloxKey key, const int64_t* __restrict__ sub_indptr,
+    int64_t* __restrict__ out_coo_col, int64_t* __restrict__ out_indices,
+    int64_t* __restrict__ out_select) {
+  extern __shared__ __align__(8) unsigned char smem[];
+  const int nthreads = blockDim.x;
+  double* lkey = (double*)smem;                               // [fanout][nthreads]
+  int* lidx = (int*)(smem + (size_t)fanout * nthreads * sizeof(double));
+  const int tid = threadIdx.x;
+  const int lane = lane_id();
+  const int64_t item = ((int64_t)blockIdx.x * nthreads + tid) / kWave;
+  if (item >= num_items) return;
+  const int64_t c = column_ids ? column_ids[item] : item;
+  int64_t in_start;
+  const int64_t deg = column_degree(indptr, num_cols, c, &in_start);
+  if (deg == 0) return;
+  const int64_t out_start = sub_indptr[item];
+  const int K = fanout;
+
+  if (deg <= K) {  // whole column, original order, zero weights included
+    for (int64_t j = lane; j < deg; j += kWave) {
+      const int64_t p = in_start + j;
+      out_indices[out_start + j] = indices ? indices[p] : p;
+      out_select[out_start + j] = p;
+      if (out_coo_col) out_coo_col[out_start + j] = item;
+    }
+    return;
+  }
+
+  int cnt = 0;
+  for (int64_t j = lane; j < deg; j += kWave) {
+    const double k = weighted_key(key, (uint64_t)item, (uint64_t)j, probs[in_start + j]);
+    // offsets grow along a lane, so an equal key never displaces a kept one
+    if (cnt == K && !(k < lkey[(K - 1) * nthreads + tid])) continue;
+    int s = cnt < K ? cnt : K - 1;
+    while (s > 0 && k < lkey[(s - 1) * nthreads + tid]) {
+      lkey[s * nthreads + tid] = lkey[(s - 1) * nthreads + tid];
+      lidx[s * nthreads + tid] = lidx[(s - 1) * nthreads + tid];
+      --s;
+    }
+    lkey[s * nthreads + tid] = k;
+    lidx[s * nthreads + tid] = (int)(j / kWave);  // j = lane + 64 * (stored value)
+    if (cnt < K) ++cnt;
+  }
+
+  int head = 0;
+  int64_t mine = -1;  // lane r keeps the winner of round r
+  for (int r = 0; r < K; ++r) {
+    double k = __longlong_as_double(0x7ff0000000000000ll);
+    int64_t off = INT64_MAX;
+    if (head < cnt) {
+      k = lkey[head * nthreads + tid];
+      off = (int64_t)lidx[head * nthreads + tid] * kWave + lane;
+    }
+    double bk = k;
+    int64_t bo = off;
+#pragma unroll
+    for (int d = kWave / 2; d > 0; d >>= 1) {
+      const double ok = __shfl_xor(bk, d, kWave);
+      const int64_t oo = __shfl_xor(bo, d, kWave);
+      if (key_less(ok, oo, bk, bo)) {
+        bk = ok;
+        bo = oo;
+      }
+    }
+    if (off == bo) ++head;  // offsets are unique, so exactly one lane advances
+    if (lane == r) mine = bo;
+  }
+  if (lane < K) {
+    const int64_t p = in_start + mine;
+    out_indices[out_start + lane] = indices ? indices[p] : p;
+    out_select[out_start + lane] = p;
+    if (out_coo_col) out_coo_col[out_start + lane] = item;
+  }
+}
+
+// ----------------------------------------------- per column, with replacement
+__device__ __forceinline__ uint64_t quantise(float w, double scale) {
+  return w > 0.0f ? (uint64_t)__dmul_rn((double)w, scale) : 0ull;
+}
+
+// First position in cdf[0, n) whose value exceeds t, clamped to n - 1.
+__device__ __forceinline__ int64_t cdf_search(const uint64_t* cdf, int64_t n,
+                                              uint64_t t) {
+  int64_t lo = 0, hi = n;
+  while (lo < hi) {
+    const int64_t mid = (lo + hi) >> 1;
+    if (cdf[mid] > t)
+      hi = mid;
+    else
+      lo = mid + 1;
+  }
+  return lo < n ? lo : n - 1;
+}
+
+// One wavefront per column: exact max of the weights, integer CDF into the
+// scratch slice of the column, then one binary search per output slot.
+__global__ __launch_bounds__(kBlock) void sample_weighted_replace_kernel(
+    const int64_t* __restrict__ indptr, int64_t num_cols,
+    const int64_t* __restrict__ indices, const float* __restrict__ probs,
+    const int64_t* __restrict__ column_ids, int64_t num_items, int64_t fanout,
+    PhiloxKey key, const int64_t* __restrict__ sub_indptr,
+    const int64_t* __restrict__ cdf_offsets, uint64_t* cdf_scratch,
+    int64_t* __restrict__ out_coo_col, int64_t* __restrict__ out_indices,
+    int64_t* __restrict__ out_select) {
+  const int lane = lane_id();
+  const int64_t item = ((int64_t)blockIdx.x * kBlock + threadIdx.x) / kWave;
+  if (item >= num_items) return;
+  const int64_t c = column_ids ? column_ids[item] : item;
+  int64_t in_start;
+  const int64_t deg = column_degree(indptr, num_cols, c, &in_start);
+  if (deg == 0) return;
+  const int64_t out_start = sub_indptr[item];
+  uint64_t* cdf = cdf_scratch + (cdf_offsets ? cdf_offsets[item] : in_start);
+
+  float wmax = 0.0f;
+  for (int64_t j = lane; j < deg; j += kWave) {
+    const float w = probs[in_start + j];
+    if (w > wmax) wmax = w;
+  }
+#pragma unroll
+  for (int d = kWave / 2; d > 0; d >>= 1) {
+    const float o = __shfl_xor(wmax, d, kWave);
+    if (o > wmax) wmax = o;
+  }
+  const double scale = wmax > 0.0f ? __ddiv_rn(2147483648.0, (double)wmax) : 0.0;
+  uint64_t carry = 0;
+  for (int64_t base = 0; base < deg; base += kWave) {
+    const int64_t j = base + lane;
+    uint64_t q = (j < deg && wmax > 0.0f) ? quantise(probs[in_start + j], scale) : 0ull;
+    q = wave_inclusive_sum(q);
+    if (j < deg) cdf[j] = carry + q;
+    carry += __shfl(q, kWave - 1, kWave);
+  }
+  const uint64_t total = carry;
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+  __builtin_amdgcn_wave_barrier();
+  for (int64_t j = lane; j < fanout; j += kWave) {
+    const uint64_t t = total > 0 ? philox_bounded(key, (uint64_t)item, (uint64_t)j, total) : 0ull;
+    // the scratch was written by other lanes of this wavefront: read past L1
+    int64_t lo = 0, hi = deg;
+    while (lo < hi) {
+      const int64_t mid = (lo + hi) >> 1;
+      const uint64_t v = __hip_atomic_load(cdf + mid, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if (v > t)
+        hi = mid;
+      else
+        lo = mid + 1;
+    }
+    const int64_t p = in_start + (lo < deg ? lo : deg - 1);
+    out_indices[out_start + j] = indices ? indices[p] : p;
+    out_select[out_start + j] = p;
+    if (out_coo_col) out_coo_col[out_start + j] = item;
+  }
+}
+
+// ------------------------------------------------------------ list sampling
+__global__ __launch_bounds__(kBlock) void list_keys_kernel(
+    const float* __restrict__ probs, int64_t n, PhiloxKey key,
+    uint64_t* __restrict__ keys, int64_t* __restrict__ iota) {
+  const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (i >= n) return;
+  // non-negative doubles (and +inf) order like their bit patterns
+  keys[i] = (uint64_t)__double_as_longlong(weighted_key(key, (uint64_t)i, 0, probs[i]));
+  iota[i] = i;
+}
+
+// Per segment: number of picks (replace: K for a non-empty segment; else
+// min(K, n_b)).  One extra thread writes the trailing 0 for the scan.
+__global__ void list_counts_kernel(const int64_t* __restrict__ range, int64_t n,
+                                   int64_t nseg, int64_t num_picks, int replace,
+                                   int64_t* __restrict__ counts) {
+  const int64_t b = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (b > nseg) return;
+  int64_t cnt = 0;
+  if (b < nseg) {
+    const int64_t nb = range ? range[b + 1] - range[b] : n;
+    cnt = replace ? (nb > 0 ? num_picks : 0) : (nb < num_picks ? nb : num_picks);
+  }
+  counts[b] = cnt;
+}
+
+// Copies the first out_range[b+1] - out_range[b] sorted values of every
+// segment; a segment that is taken whole keeps its original order.
+__global__ __launch_bounds__(kBlock) void list_take_kernel(
+    const int64_t* __restrict__ sorted_vals, const int64_t* __restrict__ range,
+    int64_t n, int64_t nseg, int64_t num_picks,
+    const int64_t* __restrict__ out_range, int64_t total,
+    int64_t* __restrict__ out_index) {
+  const int64_t o = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (o >= total) return;
+  const int64_t b = nseg == 1 ? 0 : segment_of(out_range, nseg, o);
+  const int64_t lo = range ? range[b] : 0;
+  const int64_t nb = (range ? range[b + 1] : n) - lo;
+  const int64_t k = o - out_range[b];
+  out_index[o] = nb <= num_picks ? lo + k : sorted_vals[lo + k];
+}
+
+// Integer CDF of a list segment by segment is a device-wide problem; segments
+// are handled one wavefront each (layer-wise samplers have few, long segments
+// at most a few hundred thousand items long).
+__global__ __launch_bounds__(kBlock) void list_replace_kernel(
+    const float* __restrict__ probs, const int64_t* __restrict__ range,
+    int64_t n, int64_t nseg, int64_t num_picks, PhiloxKey key,
+    const int64_t* __restrict__ out_range, uint64_t* cdf_scratch,
+    int64_t* __restrict__ out_index) {
+  const int lane = lane_id();
+  const int64_t b = ((int64_t)blockIdx.x * kBlock + threadIdx.x) / kWave;
+  if (b >= nseg) return;
+  const int64_t lo = range ? range[b] : 0, hi = range ? range[b + 1] : n;
+  const int64_t nb = hi - lo;
+  if (nb == 0) return;
+  uint64_t* cdf = cdf_scratch + lo;
+  float wmax = 0.0f;
+  for (int64_t j = lane; j < nb; j += kWave) {
+    const float w = probs[lo + j];
+    if (w > wmax) wmax = w;
+  }
+#pragma unroll
+  for (int d = kWave / 2; d > 0; d >>= 1) {
+    const float o = __shfl_xor(wmax, d, kWave);
+    if (o > wmax) wmax = o;
+  }
+  const double scale = wmax > 0.0f ? __ddiv_rn(2147483648.0, (double)wmax) : 0.0;
+  uint64_t carry = 0;
+  for (int64_t base = 0; base < nb; base += kWave) {
+    const int64_t j = base + lane;
+    uint64_t q = (j < nb && wmax > 0.0f) ? quantise(probs[lo + j], scale) : 0ull;
+    q = wave_inclusive_sum(q);
+    if (j < nb) cdf[j] = carry + q;
+    carry += __shfl(q, kWave - 1, kWave);
+  }
+  const uint64_t total = carry;
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+  __builtin_amdgcn_wave_barrier();
+  const int64_t out_start = out_range[b];
+  for (int64_t k = lane; k < num_picks; k += kWave) {
+    const uint64_t t = total > 0 ? philox_bounded(key, (uint64_t)b, (uint64_t)k, total) : 0ull;
+    int64_t l = 0, h = nb;
+    while (l < h) {
+      const int64_t mid = (l + h) >> 1;
+      const uint64_t v = __hip_atomic_load(cdf + mid, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if (v > t)
+        h = mid;
+      else
+        l = mid + 1;
+    }
+    out_index[out_start + k] = lo + (l < nb ? l : nb - 1);
+  }
+}
+
+struct ListWs {
+  uint64_t *keys_in, *keys_out;  // also the CDF scratch when sampling with replacement
+  int64_t *vals_in, *vals_out;
+  void* sort_ws;
+  size_t sort_ws_bytes;
+  void* scan_ws;
+  size_t scan_ws_bytes;
+  size_t total;
+};
+
+static size_t sort_temp_bytes(int64_t n, int64_t nseg) {
+  size_t flat = 0, seg = 0;
+  uint64_t* k = nullptr;
+  int64_t* v = nullptr;
+  (void)rocprim::radix_sort_pairs(nullptr, flat, k, k, v, v, (size_t)(n > 0 ? n : 1), 0, 64);
+  const int64_t* off = nullptr;
+  (void)rocprim::segmented_radix_sort_pairs(nullptr, seg, k, k, v, v, (size_t)(n > 0 ? n : 1),
+                                            (unsigned)(nseg > 0 ? nseg : 1), off, off, 0, 64);
+  return flat > seg ? flat : seg;
+}
+
+static ListWs carve_list(void* ws, int64_t n, int64_t nseg) {
+  Carver c(ws);
+  ListWs w;
+  const size_t m = (size_t)(n > 0 ? n : 1);
+  w.keys_in = c.take<uint64_t>(m);
+  w.keys_out = c.take<uint64_t>(m);
+  w.vals_in = c.take<int64_t>(m);
+  w.vals_out = c.take<int64_t>(m);
+  w.sort_ws_bytes = sort_temp_bytes(n, nseg);
+  w.sort_ws = c.take<char>(w.sort_ws_bytes);
+  w.scan_ws_bytes = scan_workspace_bytes(nseg + 1);
+  w.scan_ws = c.take<char>(w.scan_ws_bytes);
+  w.total = c.total();
+  return w;
+}
+
+}  // namespace gs
+
+extern "C" {
+
+int gs_weighted_key_probe(uint64_t seed, uint64_t call_id, uint64_t pos,
+                          uint64_t draw, float w, uint64_t r64, double* out2,
+                          gs_stream_t stream) {
+  using namespace gs;
+  GS_REQUIRE(out2, "weighted_key_probe: null output");
+  hipStream_t s = as_stream(stream);
+  GS_LAUNCH("weighted_key_probe", s,
+            weighted_key_probe_kernel<<<dim3(1), dim3(1), 0, s>>>(
+                make_key(seed, call_id), pos, draw, w, r64, out2));
+  return GS_OK;
+}
+
+int gs_csc_col_sample_weighted_fill(
+    const int64_t* indptr, int64_t num_cols, const int64_t* indices,
+    const float* probs, const int64_t* column_ids, int64_t num_items,
+    int64_t fanout, int replace, uint64_t seed, uint64_t call_id,
+    const int64_t* sub_indptr, const int64_t* cdf_offsets, void* cdf_scratch,
+    int64_t* out_coo_col, int64_t* out_indices, int64_t* out_select,
+    gs_stream_t stream) {
+  using namespace gs;
+  GS_REQUIRE(num_items >= 0 && num_cols >= 0, "sample_weighted: negative size");
+  GS_REQUIRE(fanout >= 0, "sample_weighted: negative fanout %lld", (long long)fanout);
+  if (num_items == 0 || fanout == 0) return GS_OK;
+  GS_REQUIRE(indptr && probs && sub_indptr && out_indices && out_select,
+             "sample_weighted: null pointer");
+  GS_REQUIRE(column_ids != nullptr || num_items <= num_cols,
+             "sample_weighted: %lld items but the matrix has %lld columns",
+             (long long)num_items, (long long)num_cols);
+  const PhiloxKey key = make_key(seed, call_id);
+  hipStream_t s = as_stream(stream);
+  if (replace) {
+    GS_REQUIRE(cdf_scratch, "sample_weighted: sampling with replacement needs the CDF scratch");
+    GS_REQUIRE(column_ids == nullptr || cdf_offsets != nullptr,
+               "sample_weighted: cdf_offsets are required with column_ids");
+    GS_LAUNCH("sample_weighted_replace", s,
+              sample_weighted_replace_kernel<<<dim3((unsigned)ceil_div(num_items * kWave, kBlock)),
+                                               dim3(kBlock), 0, s>>>(
+                  indptr, num_cols, indices, probs, column_ids, num_items, fanout,
+                  key, sub_indptr, cdf_offsets, (uint64_t*)cdf_scratch, out_coo_col,
+                  out_indices, out_select));
+    return GS_OK;
+  }
+  GS_REQUIRE(fanout <= 64,
+             "sample_weighted: fanout %lld > 64 is not supported without replacement",
+             (long long)fanout);
+  const int threads = fanout <= 32 ? kBlock : kBlock / 2;
+  const size_t lds = (size_t)fanout * threads * (sizeof(double) + sizeof(int));
+  static bool raised = false;
+  if (!raised) {
+    GS_HIP(hipFuncSetAttribute((const void*)sample_weighted_kernel,
+                               hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024));
+    raised = true;
+  }
+  const int64_t blocks = ceil_div(num_items * kWave, threads);
+  GS_LAUNCH("sample_weighted", s,
+            sample_weighted_kernel<<<dim3((unsigned)blocks), dim3(threads), lds, s>>>(
+                indptr, num_cols, indices, probs, column_ids, num_items,
+                (int)fanout, key, sub_indptr, out_coo_col, out_indices,
+                out_select));
+  return GS_OK;
+}
+
+size_t gs_list_sample_workspace_bytes(int64_t n, int64_t num_segments) {
+  if (n < 0 || num_segments < 1) return 0;
+  return gs::carve_list(nullptr, n, num_segments).total;
+}
+
+int gs_list_sample_weighted_count(const int64_t* range, int64_t n,
+                                  int64_t num_segments, int64_t num_picks,
+                                  int replace, int64_t* out_range,
+                                  void* workspace, size_t workspace_bytes,
+                                  gs_stream_t stream) {
+  using namespace gs;
+  GS_REQUIRE(n >= 0 && num_segments >= 1 && num_picks >= 0,
+             "list_sample_count: bad sizes");
+  GS_REQUIRE(range != nullptr || num_segments == 1,
+             "list_sample_count: %lld segments need a range array", (long long)num_segments);
+  GS_REQUIRE(out_range, "list_sample_count: null out_range");
+  ListWs w = carve_list(workspace, n, num_segments);
+  if (workspace == nullptr || workspace_bytes < w.total) {
+    set_error("list_sample workspace too small: %zu < %zu", workspace_bytes, w.total);
+    return GS_ERR_WORKSPACE;
+  }
+  hipStream_t s = as_stream(stream);
+  GS_LAUNCH("list_counts", s,
+            list_counts_kernel<<<dim3((unsigned)ceil_div(num_segments + 1, kBlock)),
+                                 dim3(kBlock), 0, s>>>(range, n, num_segments,
+                                                       num_picks, replace, out_range));
+  return exclusive_scan_i64(out_range, out_range, num_segments + 1, w.scan_ws,
+                            w.scan_ws_bytes, s);
+}
+
+int gs_list_sample_weighted_fill(const float* probs, const int64_t* range,
+                                 int64_t n, int64_t num_segments,
+                                 int64_t num_picks, int replace, uint64_t seed,
+                                 uint64_t call_id, const int64_t* out_range,
+                                 int64_t total_picks, int64_t* out_index,
+                                 void* workspace, size_t workspace_bytes,
+                                 gs_stream_t stream) {
+  using namespace gs;
+  GS_REQUIRE(n >= 0 && num_segments >= 1 && num_picks >= 0 && total_picks >= 0,
+             "list_sample_fill: bad sizes");
+  if (total_picks == 0 || n == 0) return GS_OK;
+  GS_REQUIRE(probs && out_range && out_index, "list_sample_fill: null pointer");
+  GS_REQUIRE(range != nullptr || num_segments == 1,
+             "list_sample_fill: %lld segments need a range array", (long long)num_segments);
+  ListWs w = carve_list(workspace, n, num_segments);
+  if (workspace == nullptr || workspace_bytes < w.total) {
+    set_error("list_sample workspace too small: %zu < %zu", workspace_bytes, w.total);
+    return GS_ERR_WORKSPACE;
+  }
+  const PhiloxKey key = make_key(seed, call_id);
+  hipStream_t s = as_stream(stream);
+  if (replace) {
+    GS_LAUNCH("list_replace", s,
+              list_replace_kernel<<<dim3((unsigned)ceil_div(num_segments * kWave, kBlock)),
+                                    dim3(kBlock), 0, s>>>(
+                  probs, range, n, num_segments, num_picks, key, out_range,
+                  w.keys_in, out_index));
+    return GS_OK;
+  }
+  GS_LAUNCH("list_keys", s,
+            list_keys_kernel<<<dim3((unsigned)ceil_div(n, kBlock)), dim3(kBlock), 0, s>>>(
+                probs, n, key, w.keys_in, w.vals_in));
+  size_t temp = w.sort_ws_bytes;
+  {
+    ProfScope ps("list_sort", s);
+    if (num_segments == 1) {
+      GS_HIP(rocprim::radix_sort_pairs(w.sort_ws, temp, w.keys_in, w.keys_out,
+                                       w.vals_in, w.vals_out, (size_t)n, 0, 64, s));
+    } else {
+      GS_HIP(rocprim::segmented_radix_sort_pairs(
+          w.sort_ws, temp, w.keys_in, w.keys_out, w.vals_in, w.vals_out,
+          (size_t)n, (unsigned)num_segments, range, range + 1, 0, 64, s));
+    }
+  }
+  GS_LAUNCH("list_take", s,
+            list_take_kernel<<<dim3((unsigned)ceil_div(total_picks, kBlock)),
+                               dim3(kBlock), 0, s>>>(w.vals_out, range, n,
+                                                     num_segments, num_picks,
+                                                     out_range, total_picks,
+                                                     out_index));
+  return GS_OK;
+}
+
+}  // extern "C"

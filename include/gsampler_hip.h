@@ -149,6 +149,67 @@ int gs_csc_col_sample_uniform_fill(const int64_t* indptr, int64_t num_cols,
                                    int64_t* out_select, gs_stream_t stream);
 
 /* ------------------------------------------------------------------------
+ * Weighted per-column sampling (fill phase; counts come from
+ * gs_csc_col_count).  probs[nnz] (fp32) is aligned with `indices`; indices may
+ * be NULL, meaning "the edge position itself".
+ *  without replacement (fanout <= 64): columns with degree <= fanout are copied
+ *    whole and in order (zero weights included); otherwise the fanout edges
+ *    with the smallest keys (-log2 u) / w, in ascending key order (ties: smaller
+ *    edge offset; w <= 0: key +inf).  Stream: pos = column position, draw =
+ *    edge offset.
+ *  with replacement: integer CDF per column in cdf_scratch (uint64 per edge;
+ *    column i uses cdf_scratch + cdf_offsets[i], or + indptr[column] when
+ *    column_ids == NULL and cdf_offsets == NULL), pick j uses draw j.
+ * Stands in for CSCColSamplingProbsCUDA (src/cuda/sampling_probs.cu:268-281).
+ * ---------------------------------------------------------------------- */
+int gs_csc_col_sample_weighted_fill(
+    const int64_t* indptr, int64_t num_cols, const int64_t* indices,
+    const float* probs, const int64_t* column_ids, int64_t num_items,
+    int64_t fanout, int replace, uint64_t seed, uint64_t call_id,
+    const int64_t* sub_indptr, const int64_t* cdf_offsets, void* cdf_scratch,
+    int64_t* out_coo_col, int64_t* out_indices, int64_t* out_select,
+    gs_stream_t stream);
+
+/* Evaluates the key arithmetic on the device: out2[0] = -log2((r64>>12)+1)/2^52),
+ * out2[1] = key of weight w at stream (seed, call_id, pos, draw).  Test hook. */
+int gs_weighted_key_probe(uint64_t seed, uint64_t call_id, uint64_t pos,
+                          uint64_t draw, float w, uint64_t r64, double* out2,
+                          gs_stream_t stream);
+
+/* ------------------------------------------------------------------------
+ * Collective (list / layer-wise) sampling: picks positions of a list.
+ *  gs_list_sample_uniform: K of n positions; n <= K without replacement gives
+ *    0..n-1.  out_index holds min(K, n) (K with replacement) entries.
+ *    ListSamplingCUDA, src/cuda/list_sampling.cu:70-73.
+ *  gs_list_sample_weighted_{count,fill}: probs[n] fp32, optional
+ *    range[num_segments + 1] (segments = mini-batches; NULL = one list).
+ *    count writes out_range[num_segments + 1] (picks before each segment, last
+ *    = total).  fill writes global positions: without replacement per segment
+ *    the min(K, n_b) smallest keys in ascending key order (a segment with
+ *    n_b <= K keeps its order); with replacement K picks through an integer
+ *    CDF (stream pos = segment, draw = pick).  ListSamplingProbsCUDA
+ *    (src/cuda/list_sampling_probs.cu:85-89), BatchListSamplingProbsCUDA
+ *    (src/cuda/batch/list_sampling_probs.cu:102-107; the reference rejects
+ *    replace there).
+ * ---------------------------------------------------------------------- */
+int gs_list_sample_uniform(int64_t n, int64_t num_picks, int replace, int algo,
+                           uint64_t seed, uint64_t call_id, int64_t* out_index,
+                           gs_stream_t stream);
+size_t gs_list_sample_workspace_bytes(int64_t n, int64_t num_segments);
+int gs_list_sample_weighted_count(const int64_t* range, int64_t n,
+                                  int64_t num_segments, int64_t num_picks,
+                                  int replace, int64_t* out_range,
+                                  void* workspace, size_t workspace_bytes,
+                                  gs_stream_t stream);
+int gs_list_sample_weighted_fill(const float* probs, const int64_t* range,
+                                 int64_t n, int64_t num_segments,
+                                 int64_t num_picks, int replace, uint64_t seed,
+                                 uint64_t call_id, const int64_t* out_range,
+                                 int64_t total_picks, int64_t* out_index,
+                                 void* workspace, size_t workspace_bytes,
+                                 gs_stream_t stream);
+
+/* ------------------------------------------------------------------------
  * Unique in first-occurrence order + relabel, for one batch or a super-batch.
  * For batch b the key sequence is
  *     seeds[seeds_ptr[b] : seeds_ptr[b+1]] ++ rows[rows_ptr[b] : rows_ptr[b+1]]

@@ -312,3 +312,68 @@ def minor_slice(ids, picked, indptr=None, edge_major=None, with_major=True):
     out_major = np.empty(kept, dtype=np.int64) if want_major else None
     lib().gs_minor_slice_cpu(*args, _p(out_major), _p(out_minor), _p(out_select))
     return out_indptr, out_major, out_minor, out_select
+
+
+# --------------------------------------------------------- weighted sampling
+def neg_log2_unit(r64) -> float:
+    f = lib().gs_neg_log2_unit_cpu
+    f.restype = C.c_double
+    return f(C.c_uint64(r64))
+
+
+def weighted_key(seed, call_id, pos, draw, w) -> float:
+    f = lib().gs_weighted_key_cpu
+    f.restype = C.c_double
+    return f(C.c_uint64(seed), C.c_uint64(call_id), C.c_uint64(pos), C.c_uint64(draw),
+             C.c_float(w))
+
+
+def sample_weighted(indptr, indices, probs, column_ids, fanout, replace=False, seed=7777,
+                    call_id=0, with_coo=True):
+    indptr, indices = _i64(indptr), _i64(indices)
+    probs = np.ascontiguousarray(probs, dtype=np.float32)
+    num_cols = indptr.size - 1
+    if column_ids is not None:
+        column_ids = _i64(column_ids)
+        n = column_ids.size
+    else:
+        n = num_cols
+    sub_indptr = col_count(indptr, column_ids, fanout, replace, n)
+    nnz = int(sub_indptr[-1])
+    out_idx = np.empty(nnz, dtype=np.int64)
+    out_sel = np.empty(nnz, dtype=np.int64)
+    out_col = np.empty(nnz, dtype=np.int64) if with_coo else None
+    lib().gs_csc_col_sample_weighted_fill_cpu(
+        _p(indptr), C.c_int64(num_cols), _p(indices), _p(probs), _p(column_ids),
+        C.c_int64(n), C.c_int64(fanout), C.c_int(int(replace)), C.c_uint64(seed),
+        C.c_uint64(call_id), _p(sub_indptr), _p(out_col), _p(out_idx), _p(out_sel))
+    return sub_indptr, out_col, out_idx, out_sel
+
+
+def list_sample_uniform(n, num_picks, replace=False, algo=0, seed=7777, call_id=0):
+    f = lib().gs_list_sample_uniform_cpu
+    f.restype = C.c_int64
+    args = [C.c_int64(n), C.c_int64(num_picks), C.c_int(int(replace)), C.c_int(algo),
+            C.c_uint64(seed), C.c_uint64(call_id)]
+    count = f(*args, None)
+    out = np.empty(count, dtype=np.int64)
+    f(*args, _p(out))
+    return out
+
+
+def list_sample_weighted(probs, num_picks, replace=False, range_=None, seed=7777, call_id=0):
+    """-> (index, out_range)"""
+    probs = np.ascontiguousarray(probs, dtype=np.float32)
+    f = lib().gs_list_sample_weighted_cpu
+    f.restype = C.c_int64
+    nseg = 1
+    if range_ is not None:
+        range_ = _i64(range_)
+        nseg = range_.size - 1
+    out_range = np.empty(nseg + 1, dtype=np.int64)
+    args = [_p(probs), C.c_int64(probs.size), C.c_int64(num_picks), C.c_int(int(replace)),
+            _p(range_), C.c_int64(nseg), C.c_uint64(seed), C.c_uint64(call_id)]
+    total = f(*args, None, _p(out_range))
+    out = np.empty(total, dtype=np.int64)
+    f(*args, _p(out), _p(out_range))
+    return out, out_range

@@ -246,7 +246,7 @@ void gs_csc_col_sample_uniform_fill_cpu(
       }
       for (int64_t j = 0; j < cnt; ++j) {
         int64_t p = in_start + slot[j];
-        out_indices[out_start + j] = indices[p];
+        out_indices[out_start + j] = indices ? indices[p] : p;
         out_select[out_start + j] = p;
         if (out_coo_col) out_coo_col[out_start + j] = i;
       }
@@ -632,4 +632,215 @@ extern "C" void gs_minor_slice_cpu(const int64_t* ids, int64_t nnz,
   if (out_indptr)
     for (int64_t k = c + 1; k <= num_major; ++k) out_indptr[k] = kept;
   if (out_total) *out_total = kept;
+}
+
+// -------------------------------------------------------------------------
+// Weighted sampling.
+//
+// Without replacement the reference uses Efraimidis-Spirakis keys u^(1/w) and
+// keeps the K largest (src/cuda/sampling_probs.cu:55-75 per column,
+// src/cuda/list_sampling_probs.cu:51-80 for lists: sort all keys descending,
+// first K in sorted order).  Ranking by u^(1/w) descending is ranking by
+// (-log2 u) / w ascending; that form is used here because it can be computed
+// with correctly rounded double operations only (+, -, *, /, fma), hence
+// identically on the CPU and the GPU:
+//   v = (r64 >> 12) + 1 in [1, 2^52],  u = v / 2^52,
+//   -log2 u = (52 - e) - log2(m),  v = m * 2^e,  m in (sqrt(1/2), sqrt(2)],
+//   log2(m) = s * P(s^2),  s = (m - 1) / (m + 1),  P = 11-term atanh series.
+// Items with w <= 0 (or NaN) get key +inf: they are taken last, in index order
+// (the list form of the reference gives them key -1, :63-66).  Ties break
+// towards the smaller index.  Output order is ascending key, which is the
+// reference's descending u^(1/w) order.
+//
+// With replacement the reference inverts a per-column fp32 CDF
+// (src/cuda/sampling_probs.cu:150-174, src/cuda/list_sampling_probs.cu:28-48).
+// A floating-point prefix sum depends on the summation order, so weights are
+// first quantised to integers q = floor(w * 2^31 / wmax) (exact max, one
+// rounded division, one rounded product per item); integer prefix sums are
+// order-independent.  pick = min(upper_bound(cdf, t), n - 1), t = bounded(total)
+// (t = 0 when every weight is <= 0, which selects the last item as the
+// reference's all-zero CDF does).
+namespace {
+
+const double kLogC[11] = {0x1.71547652b82fep+1, 0x1.ec709dc3a03fep-1,
+                          0x1.2776c50ef9bfep-1, 0x1.a61762a7adedap-2,
+                          0x1.484b13d7c02a9p-2, 0x1.0c9a84994022dp-2,
+                          0x1.c68f568d31761p-3, 0x1.89f3b1694cffep-3,
+                          0x1.5b9ac9b743f0dp-3, 0x1.3703c1f4d0ffep-3,
+                          0x1.1964ec6fc9491p-3};
+
+double neg_log2_unit(uint64_t r64) {
+  uint64_t v = (r64 >> 12) + 1;
+  int e = 63 - __builtin_clzll(v);
+  double m = std::ldexp((double)v, -e);
+  if (m > 0x1.6a09e667f3bcdp+0) {
+    m *= 0.5;
+    e += 1;
+  }
+  double s = (m - 1.0) / (m + 1.0);
+  double s2 = s * s;
+  double p = kLogC[10];
+  for (int k = 9; k >= 0; --k) p = std::fma(p, s2, kLogC[k]);
+  double log2m = s * p;
+  return (double)(52 - e) - log2m;
+}
+
+double weighted_key(const Stream& rng, uint64_t pos, uint64_t draw, float w) {
+  if (!(w > 0.0f)) return std::numeric_limits<double>::infinity();
+  return neg_log2_unit(rng.r64(pos, draw)) / (double)w;
+}
+
+struct KeyIdx {
+  double key;
+  int64_t idx;
+  bool operator<(const KeyIdx& o) const {
+    return key < o.key || (key == o.key && idx < o.idx);
+  }
+};
+
+// Integer CDF of n weights into cdf[n]; returns the total.
+uint64_t integer_cdf(const float* w, int64_t n, uint64_t* cdf) {
+  float wmax = 0.0f;
+  for (int64_t i = 0; i < n; ++i)
+    if (w[i] > wmax) wmax = w[i];
+  uint64_t acc = 0;
+  if (wmax > 0.0f) {
+    double scale = 2147483648.0 / (double)wmax;
+    for (int64_t i = 0; i < n; ++i) {
+      uint64_t q = w[i] > 0.0f ? (uint64_t)((double)w[i] * scale) : 0;
+      acc += q;
+      cdf[i] = acc;
+    }
+  } else {
+    for (int64_t i = 0; i < n; ++i) cdf[i] = 0;
+  }
+  return acc;
+}
+
+int64_t cdf_pick(const uint64_t* cdf, int64_t n, uint64_t total, const Stream& rng,
+                 uint64_t pos, uint64_t draw) {
+  uint64_t t = total > 0 ? rng.bounded(pos, draw, total) : 0;
+  int64_t item = std::upper_bound(cdf, cdf + n, t) - cdf;
+  return std::min(item, n - 1);
+}
+
+}  // namespace
+
+extern "C" {
+
+// Known-answer hooks for the key arithmetic.
+double gs_neg_log2_unit_cpu(uint64_t r64) { return neg_log2_unit(r64); }
+double gs_weighted_key_cpu(uint64_t seed, uint64_t call_id, uint64_t pos,
+                           uint64_t draw, float w) {
+  return weighted_key(Stream(seed, call_id), pos, draw, w);
+}
+
+// Weighted per-column sampling, src/cuda/sampling_probs.cu:25-188.  probs are
+// aligned with `indices`.  deg <= fanout (no replace): whole column in order,
+// zero-weight edges included (:94-106).
+void gs_csc_col_sample_weighted_fill_cpu(
+    const int64_t* indptr, int64_t num_cols, const int64_t* indices,
+    const float* probs, const int64_t* column_ids, int64_t num_items,
+    int64_t fanout, int replace, uint64_t seed, uint64_t call_id,
+    const int64_t* sub_indptr, int64_t* out_coo_col, int64_t* out_indices,
+    int64_t* out_select) {
+  Stream rng(seed, call_id);
+#pragma omp parallel
+  {
+    std::vector<KeyIdx> keys;
+    std::vector<uint64_t> cdf;
+#pragma omp for schedule(dynamic, 64)
+    for (int64_t i = 0; i < num_items; ++i) {
+      int64_t c = column_ids ? column_ids[i] : i;
+      int64_t deg = col_degree(indptr, num_cols, c);
+      if (deg == 0) continue;
+      int64_t in_start = indptr[c], out_start = sub_indptr[i];
+      int64_t cnt = sub_indptr[i + 1] - out_start;
+      auto emit = [&](int64_t j, int64_t off) {
+        out_indices[out_start + j] = indices ? indices[in_start + off] : in_start + off;
+        out_select[out_start + j] = in_start + off;
+        if (out_coo_col) out_coo_col[out_start + j] = i;
+      };
+      if (replace) {
+        cdf.resize((size_t)deg);
+        uint64_t total = integer_cdf(probs + in_start, deg, cdf.data());
+        for (int64_t j = 0; j < cnt; ++j)
+          emit(j, cdf_pick(cdf.data(), deg, total, rng, (uint64_t)i, (uint64_t)j));
+      } else if (deg <= fanout) {
+        for (int64_t j = 0; j < cnt; ++j) emit(j, j);
+      } else {
+        keys.resize((size_t)deg);
+        for (int64_t j = 0; j < deg; ++j)
+          keys[(size_t)j] = {weighted_key(rng, (uint64_t)i, (uint64_t)j, probs[in_start + j]), j};
+        std::partial_sort(keys.begin(), keys.begin() + fanout, keys.end());
+        for (int64_t j = 0; j < cnt; ++j) emit(j, keys[(size_t)j].idx);
+      }
+    }
+  }
+}
+
+// Collective (list) sampling, weighted.  range == NULL: one list of n items.
+// Otherwise range[num_segments + 1] delimits segments; per segment
+// min(K, n_b) picks; indices are global positions
+// (src/cuda/batch/list_sampling_probs.cu:30-100).  out_range[b] = picks before
+// segment b.  Returns the number of picks.  n <= K without replacement: all
+// items in order (src/cuda/list_sampling_probs.cu:16-19).
+int64_t gs_list_sample_weighted_cpu(const float* probs, int64_t n, int64_t num_picks,
+                                    int replace, const int64_t* range,
+                                    int64_t num_segments, uint64_t seed,
+                                    uint64_t call_id, int64_t* out_index,
+                                    int64_t* out_range) {
+  Stream rng(seed, call_id);
+  int64_t total_out = 0;
+  const int64_t nseg = range ? num_segments : 1;
+  std::vector<KeyIdx> keys;
+  std::vector<uint64_t> cdf;
+  for (int64_t b = 0; b < nseg; ++b) {
+    int64_t lo = range ? range[b] : 0, hi = range ? range[b + 1] : n;
+    int64_t nb = hi - lo;
+    if (out_range) out_range[b] = total_out;
+    if (replace) {
+      if (nb == 0) continue;
+      cdf.resize((size_t)nb);
+      uint64_t total = integer_cdf(probs + lo, nb, cdf.data());
+      for (int64_t k = 0; k < num_picks; ++k)
+        if (out_index)
+          out_index[total_out + k] =
+              lo + cdf_pick(cdf.data(), nb, total, rng, (uint64_t)b, (uint64_t)k);
+      total_out += num_picks;
+    } else if (nb <= num_picks) {
+      if (out_index)
+        for (int64_t k = 0; k < nb; ++k) out_index[total_out + k] = lo + k;
+      total_out += nb;
+    } else {
+      keys.resize((size_t)nb);
+      for (int64_t j = 0; j < nb; ++j)
+        keys[(size_t)j] = {weighted_key(rng, (uint64_t)(lo + j), 0, probs[lo + j]), lo + j};
+      std::stable_sort(keys.begin(), keys.end());
+      if (out_index)
+        for (int64_t k = 0; k < num_picks; ++k) out_index[total_out + k] = keys[(size_t)k].idx;
+      total_out += num_picks;
+    }
+  }
+  if (out_range) out_range[nseg] = total_out;
+  return total_out;
+}
+
+}  // extern "C"
+
+// Uniform collective sampling, src/cuda/list_sampling.cu:21-68: the per-column
+// sampler on one virtual column 0..n-1 (stream position 0).
+extern "C" int64_t gs_list_sample_uniform_cpu(int64_t n, int64_t num_picks,
+                                              int replace, int algo, uint64_t seed,
+                                              uint64_t call_id, int64_t* out_index) {
+  int64_t indptr[2] = {0, n};
+  int64_t sub[2];
+  gs_csc_col_count_cpu(indptr, 1, nullptr, 1, num_picks, replace, sub);
+  if (out_index && sub[1] > 0) {
+    std::vector<int64_t> sel((size_t)sub[1]);
+    gs_csc_col_sample_uniform_fill_cpu(indptr, 1, nullptr, nullptr, 1, num_picks,
+                                       replace, algo, seed, call_id, sub, nullptr,
+                                       out_index, sel.data());
+  }
+  return sub[1];
 }

@@ -1,0 +1,127 @@
+"""Weighted sampling on the GPU vs the oracle: bit-exact keys and picks."""
+import numpy as np
+import pytest
+import torch
+
+import gsampler_amd as gs
+from gsampler_amd import capi
+from oracle import binding as orc
+from tests.conftest import random_csc
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def T(a):
+    return None if a is None else torch.as_tensor(np.asarray(a, dtype=np.int64), device=DEV)
+
+
+def F(a):
+    return torch.as_tensor(np.asarray(a, dtype=np.float32), device=DEV)
+
+
+def same(got, want):
+    assert len(got) == len(want)
+    for g, w in zip(got, want):
+        if w is None:
+            assert g is None
+        else:
+            assert np.array_equal(g.cpu().numpy(), w)
+
+
+def test_key_arithmetic_is_bit_identical():
+    rng = np.random.default_rng(0)
+    cases = [0, 2**64 - 1, (2**51 - 1) << 12, 1 << 12, 2**63] + \
+        [int(x) for x in rng.integers(0, 2**64, size=300, dtype=np.uint64)]
+    for i, r in enumerate(cases):
+        w = float(np.float32(rng.random() * 3 + 1e-3))
+        e, k = capi.weighted_key_probe(7, 3, 1000 + i, i, w, r)
+        assert e == orc.neg_log2_unit(r)
+        assert k == orc.weighted_key(7, 3, 1000 + i, i, w)
+    assert np.isinf(capi.weighted_key_probe(7, 3, 1, 1, 0.0, 5)[1])
+    assert np.isinf(capi.weighted_key_probe(7, 3, 1, 1, -2.0, 5)[1])
+
+
+@pytest.mark.parametrize("fanout", [1, 5, 15, 32, 33, 64])
+def test_column_sampling_parity(fanout):
+    rng = np.random.default_rng(fanout)
+    indptr, indices = random_csc(rng, 3000, 10**6, 120, hub_deg=30000)
+    probs = rng.lognormal(0, 1, size=indices.size).astype(np.float32)
+    probs[rng.random(indices.size) < 0.05] = 0.0
+    cols = rng.integers(0, 3000, size=2000)
+    same(capi.sample_weighted(T(indptr), T(indices), F(probs), T(cols), fanout, call_id=2),
+         orc.sample_weighted(indptr, indices, probs, cols, fanout, call_id=2))
+    same(capi.sample_weighted(T(indptr), T(indices), F(probs), None, fanout),
+         orc.sample_weighted(indptr, indices, probs, None, fanout))
+
+
+@pytest.mark.parametrize("fanout", [3, 70])
+def test_column_sampling_with_replacement_parity(fanout):
+    rng = np.random.default_rng(fanout)
+    indptr, indices = random_csc(rng, 2000, 10**6, 80, hub_deg=9000)
+    probs = rng.random(indices.size).astype(np.float32)
+    probs[rng.random(indices.size) < 0.1] = 0.0
+    probs[indptr[5]:indptr[6]] = 0.0            # a column without positive weight
+    cols = rng.integers(0, 2000, size=1500)
+    same(capi.sample_weighted(T(indptr), T(indices), F(probs), T(cols), fanout, True),
+         orc.sample_weighted(indptr, indices, probs, cols, fanout, True))
+    same(capi.sample_weighted(T(indptr), T(indices), F(probs), None, fanout, True),
+         orc.sample_weighted(indptr, indices, probs, None, fanout, True))
+
+
+@pytest.mark.parametrize("n,k", [(10, 20), (1000, 64), (233000, 512), (5000, 5000)])
+def test_list_sampling_parity(n, k):
+    rng = np.random.default_rng(n)
+    probs = rng.random(n).astype(np.float32)
+    probs[rng.random(n) < 0.2] = 0.0
+    same(capi.list_sample_weighted(F(probs), k, call_id=4),
+         orc.list_sample_weighted(probs, k, call_id=4))
+    same(capi.list_sample_weighted(F(probs), k, replace=True, call_id=4),
+         orc.list_sample_weighted(probs, k, replace=True, call_id=4))
+    for replace in (False, True):
+        for algo in (0, 1):
+            got = capi.list_sample_uniform(n, k, replace, algo, call_id=9)
+            assert np.array_equal(got.cpu().numpy(),
+                                  orc.list_sample_uniform(n, k, replace, algo, call_id=9))
+
+
+def test_batched_list_sampling_parity():
+    rng = np.random.default_rng(5)
+    sizes = np.array([0, 700, 3, 20000, 0, 512, 513])
+    ranges = np.concatenate([[0], np.cumsum(sizes)])
+    probs = rng.random(ranges[-1]).astype(np.float32)
+    probs[rng.random(probs.size) < 0.3] = 0.0
+    same(capi.list_sample_weighted(F(probs), 512, range_=T(ranges)),
+         orc.list_sample_weighted(probs, 512, range_=ranges))
+    same(capi.list_sample_weighted(F(probs), 100, replace=True, range_=T(ranges)),
+         orc.list_sample_weighted(probs, 100, replace=True, range_=ranges))
+
+
+def test_operators_through_the_api():
+    rng = np.random.default_rng(6)
+    indptr, indices = random_csc(rng, 500, 400, 60)
+    indices[0] = 399
+    probs = rng.random(indices.size).astype(np.float32)
+    m = gs.Matrix()
+    m.load_graph("CSC", [T(indptr), T(indices)])
+    m.edata["w"] = F(probs)
+    gs.manual_seed(99)
+    s = m.individual_sampling(7, m.edata["w"], False)
+    want = orc.sample_weighted(indptr, indices, probs, None, 7, seed=99, call_id=0)
+    assert np.array_equal(s.csc[1].cpu().numpy(), want[2])
+    assert np.array_equal(s.edata["w"].cpu().numpy(), probs[want[3]])
+    p = rng.random(400).astype(np.float32)
+    sub, picked = m.collective_sampling(50, F(p), False)          # call id 1
+    want_idx, _ = orc.list_sample_weighted(p, 50, seed=99, call_id=1)
+    assert np.array_equal(picked.cpu().numpy(), want_idx)
+    assert sub.num_rows() == 50
+    u = torch.ops.gs_ops._CAPI_ListSampling(400, 30, False)          # call id 2
+    assert np.array_equal(u.cpu().numpy(), orc.list_sample_uniform(400, 30, seed=99, call_id=2))
+    ranges = np.array([0, 100, 400])
+    idx, ptr = torch.ops.gs_ops._CAPI_BatchListSamplingWithProbs(F(p), 20, False, T(ranges))
+    w_idx, w_ptr = orc.list_sample_weighted(p, 20, range_=ranges, seed=99, call_id=3)
+    assert np.array_equal(idx.cpu().numpy(), w_idx) and np.array_equal(ptr.cpu().numpy(), w_ptr)
+    idx, ptr = torch.ops.gs_ops._CAPI_BatchListSampling(20, False, T(ranges))
+    w_idx, w_ptr = orc.list_sample_weighted(np.ones(400, dtype=np.float32), 20, range_=ranges,
+                                            seed=99, call_id=4)
+    assert np.array_equal(idx.cpu().numpy(), w_idx)
