@@ -17,6 +17,20 @@
 namespace gs {
 
 // ------------------------------------------------------------ key arithmetic
+// x / y for finite normal y > 0 from fused multiply-adds only: a bit-trick
+// reciprocal estimate (12 % off at worst), six Newton steps, one residual
+// correction.  Hardware division is avoided because its last bit need not
+// agree between a GPU and a CPU; every operation here is a correctly rounded
+// IEEE operation, so the result is reproducible anywhere (it lies within an
+// ulp or two of the true quotient, which is all a sampling key needs).
+__device__ __forceinline__ double det_div(double x, double y) {
+  double r = __longlong_as_double(0x7FDE623822FC16E6ll - __double_as_longlong(y));
+#pragma unroll
+  for (int i = 0; i < 6; ++i) r = __fma_rn(r, __fma_rn(-y, r, 1.0), r);
+  const double q = __dmul_rn(x, r);
+  return __fma_rn(__fma_rn(-y, q, x), r, q);
+}
+
 __device__ __forceinline__ double neg_log2_unit(uint64_t r64) {
   const uint64_t v = (r64 >> 12) + 1;  // [1, 2^52]: exact as a double
   int e = 63 - __clzll((long long)v);
@@ -25,7 +39,7 @@ __device__ __forceinline__ double neg_log2_unit(uint64_t r64) {
     m = __dmul_rn(m, 0.5);
     e += 1;
   }
-  const double s = __ddiv_rn(__dsub_rn(m, 1.0), __dadd_rn(m, 1.0));
+  const double s = det_div(__dsub_rn(m, 1.0), __dadd_rn(m, 1.0));
   const double s2 = __dmul_rn(s, s);
   double p = 0x1.1964ec6fc9491p-3;
   p = __fma_rn(p, s2, 0x1.3703c1f4d0ffep-3);
@@ -46,7 +60,7 @@ __device__ __forceinline__ double weighted_key(PhiloxKey key, uint64_t pos,
   if (!(w > 0.0f)) return __longlong_as_double(0x7ff0000000000000ll);  // +inf
   const Words4 wd = philox(key, pos, draw);
   const uint64_t r = ((uint64_t)wd.y << 32) | wd.x;
-  return __ddiv_rn(neg_log2_unit(r), (double)w);
+  return det_div(neg_log2_unit(r), (double)w);
 }
 
 __global__ void weighted_key_probe_kernel(PhiloxKey key, uint64_t pos,
@@ -194,7 +208,7 @@ __global__ __launch_bounds__(kBlock) void sample_weighted_replace_kernel(
     const float o = __shfl_xor(wmax, d, kWave);
     if (o > wmax) wmax = o;
   }
-  const double scale = wmax > 0.0f ? __ddiv_rn(2147483648.0, (double)wmax) : 0.0;
+  const double scale = wmax > 0.0f ? det_div(2147483648.0, (double)wmax) : 0.0;
   uint64_t carry = 0;
   for (int64_t base = 0; base < deg; base += kWave) {
     const int64_t j = base + lane;
@@ -292,7 +306,7 @@ __global__ __launch_bounds__(kBlock) void list_replace_kernel(
     const float o = __shfl_xor(wmax, d, kWave);
     if (o > wmax) wmax = o;
   }
-  const double scale = wmax > 0.0f ? __ddiv_rn(2147483648.0, (double)wmax) : 0.0;
+  const double scale = wmax > 0.0f ? det_div(2147483648.0, (double)wmax) : 0.0;
   uint64_t carry = 0;
   for (int64_t base = 0; base < nb; base += kWave) {
     const int64_t j = base + lane;

@@ -642,8 +642,8 @@ extern "C" void gs_minor_slice_cpu(const int64_t* ids, int64_t nnz,
 // src/cuda/list_sampling_probs.cu:51-80 for lists: sort all keys descending,
 // first K in sorted order).  Ranking by u^(1/w) descending is ranking by
 // (-log2 u) / w ascending; that form is used here because it can be computed
-// with correctly rounded double operations only (+, -, *, /, fma), hence
-// identically on the CPU and the GPU:
+// with correctly rounded double operations only (+, -, *, fma; quotients by
+// det_div below), hence identically on the CPU and the GPU:
 //   v = (r64 >> 12) + 1 in [1, 2^52],  u = v / 2^52,
 //   -log2 u = (52 - e) - log2(m),  v = m * 2^e,  m in (sqrt(1/2), sqrt(2)],
 //   log2(m) = s * P(s^2),  s = (m - 1) / (m + 1),  P = 11-term atanh series.
@@ -655,8 +655,8 @@ extern "C" void gs_minor_slice_cpu(const int64_t* ids, int64_t nnz,
 // With replacement the reference inverts a per-column fp32 CDF
 // (src/cuda/sampling_probs.cu:150-174, src/cuda/list_sampling_probs.cu:28-48).
 // A floating-point prefix sum depends on the summation order, so weights are
-// first quantised to integers q = floor(w * 2^31 / wmax) (exact max, one
-// rounded division, one rounded product per item); integer prefix sums are
+// first quantised to integers q = floor(w * scale), scale = det_div(2^31, wmax)
+// (exact max, one rounded product per item); integer prefix sums are
 // order-independent.  pick = min(upper_bound(cdf, t), n - 1), t = bounded(total)
 // (t = 0 when every weight is <= 0, which selects the last item as the
 // reference's all-zero CDF does).
@@ -669,6 +669,21 @@ const double kLogC[11] = {0x1.71547652b82fep+1, 0x1.ec709dc3a03fep-1,
                           0x1.5b9ac9b743f0dp-3, 0x1.3703c1f4d0ffep-3,
                           0x1.1964ec6fc9491p-3};
 
+// x / y (y > 0, finite, normal) from fused multiply-adds only, so that the
+// quotient is the same on every IEEE machine: reciprocal estimate by integer
+// subtraction on the bit pattern, six Newton steps r += r * (1 - y r), then
+// q = x r corrected once by the residual x - y q.
+double det_div(double x, double y) {
+  int64_t yb;
+  std::memcpy(&yb, &y, 8);
+  int64_t rb = 0x7FDE623822FC16E6ll - yb;
+  double r;
+  std::memcpy(&r, &rb, 8);
+  for (int i = 0; i < 6; ++i) r = std::fma(r, std::fma(-y, r, 1.0), r);
+  double q = x * r;
+  return std::fma(std::fma(-y, q, x), r, q);
+}
+
 double neg_log2_unit(uint64_t r64) {
   uint64_t v = (r64 >> 12) + 1;
   int e = 63 - __builtin_clzll(v);
@@ -677,7 +692,7 @@ double neg_log2_unit(uint64_t r64) {
     m *= 0.5;
     e += 1;
   }
-  double s = (m - 1.0) / (m + 1.0);
+  double s = det_div(m - 1.0, m + 1.0);
   double s2 = s * s;
   double p = kLogC[10];
   for (int k = 9; k >= 0; --k) p = std::fma(p, s2, kLogC[k]);
@@ -687,7 +702,7 @@ double neg_log2_unit(uint64_t r64) {
 
 double weighted_key(const Stream& rng, uint64_t pos, uint64_t draw, float w) {
   if (!(w > 0.0f)) return std::numeric_limits<double>::infinity();
-  return neg_log2_unit(rng.r64(pos, draw)) / (double)w;
+  return det_div(neg_log2_unit(rng.r64(pos, draw)), (double)w);
 }
 
 struct KeyIdx {
@@ -705,7 +720,7 @@ uint64_t integer_cdf(const float* w, int64_t n, uint64_t* cdf) {
     if (w[i] > wmax) wmax = w[i];
   uint64_t acc = 0;
   if (wmax > 0.0f) {
-    double scale = 2147483648.0 / (double)wmax;
+    double scale = det_div(2147483648.0, (double)wmax);
     for (int64_t i = 0; i < n; ++i) {
       uint64_t q = w[i] > 0.0f ? (uint64_t)((double)w[i] * scale) : 0;
       acc += q;

@@ -30,7 +30,8 @@ def test_key_definition():
     w = 0.37
     words = orc.stream_words(5, 2, 11, 3)
     r64 = (int(words[1]) << 32) | int(words[0])
-    assert orc.weighted_key(5, 2, 11, 3, w) == orc.neg_log2_unit(r64) / float(np.float32(w))
+    assert orc.weighted_key(5, 2, 11, 3, w) == pytest.approx(
+        orc.neg_log2_unit(r64) / float(np.float32(w)), rel=1e-15)
     assert math.isinf(orc.weighted_key(5, 2, 11, 3, 0.0))
     assert math.isinf(orc.weighted_key(5, 2, 11, 3, -1.0))
     assert math.isinf(orc.weighted_key(5, 2, 11, 3, float("nan")))
