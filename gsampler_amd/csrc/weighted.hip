@@ -10,6 +10,10 @@
 #include "common.h"
 #include "scan.h"
 
+// The sampling keys must come out bit-identical to the CPU check: no implicit
+// fusing of a multiply into a neighbouring add anywhere in this file.
+#pragma clang fp contract(off)
+
 #include <cstring>
 #include <rocprim/device/device_radix_sort.hpp>
 #include <rocprim/device/device_segmented_radix_sort.hpp>
@@ -52,7 +56,7 @@ __device__ __forceinline__ double neg_log2_unit(uint64_t r64) {
   p = __fma_rn(p, s2, 0x1.2776c50ef9bfep-1);
   p = __fma_rn(p, s2, 0x1.ec709dc3a03fep-1);
   p = __fma_rn(p, s2, 0x1.71547652b82fep+1);
-  return __dsub_rn((double)(52 - e), __dmul_rn(s, p));
+  return __fma_rn(-s, p, (double)(52 - e));
 }
 
 __device__ __forceinline__ double weighted_key(PhiloxKey key, uint64_t pos,

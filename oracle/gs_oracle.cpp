@@ -696,8 +696,7 @@ double neg_log2_unit(uint64_t r64) {
   double s2 = s * s;
   double p = kLogC[10];
   for (int k = 9; k >= 0; --k) p = std::fma(p, s2, kLogC[k]);
-  double log2m = s * p;
-  return (double)(52 - e) - log2m;
+  return std::fma(-s, p, (double)(52 - e));  // (52 - e) - log2(m), one rounding
 }
 
 double weighted_key(const Stream& rng, uint64_t pos, uint64_t draw, float w) {
