@@ -77,6 +77,11 @@ SIGNATURES = {
     "gs_list_sample_weighted_count": (_int, [_p, _i64, _i64, _i64, _int, _p, _p, _sz, _p]),
     "gs_list_sample_weighted_fill": (_int, [_p, _p, _i64, _i64, _i64, _int, _u64, _u64, _p,
                                             _i64, _p, _p, _sz, _p]),
+    "gs_random_walk": (_int, [_p, _p, _i64, _p, _i64, _i64, _u64, _u64, _p, _p]),
+    "gs_node2vec": (_int, [_p, _p, _i64, _p, _i64, _i64, C.c_double, C.c_double, _u64, _u64,
+                           _p, _p]),
+    "gs_segment_sort_workspace_bytes": (_sz, [_i64, _i64]),
+    "gs_segment_sort_i64": (_int, [_p, _i64, _p, _p, _i64, _p, _sz, _p]),
 }
 
 _lib = None
@@ -518,3 +523,33 @@ def list_sample_weighted(probs, num_picks, replace=False, range_=None, seed=7777
                                          total, _ptr(out), ws.data_ptr(), ws.numel(),
                                          _stream()))
     return out, out_range
+
+
+# --------------------------------------------------------------------- walks
+def random_walk(indptr, indices, seeds, walk_length, seed=7777, call_id=0):
+    """-> int64 [walk_length + 1, num_seeds] (step-major)."""
+    indptr, indices, seeds = _i64t(indptr, "indptr"), _i64t(indices, "indices"), _i64t(seeds, "seeds")
+    n = seeds.numel()
+    out = torch.empty((walk_length + 1, n), dtype=torch.int64, device=indptr.device)
+    check(lib().gs_random_walk(_ptr(indptr), _ptr(indices), indptr.numel() - 1, _ptr(seeds), n,
+                               walk_length, seed, call_id, _ptr(out), _stream()))
+    return out
+
+
+def node2vec(indptr, indices, seeds, walk_length, p, q, seed=7777, call_id=0):
+    indptr, indices, seeds = _i64t(indptr, "indptr"), _i64t(indices, "indices"), _i64t(seeds, "seeds")
+    n = seeds.numel()
+    out = torch.empty((walk_length + 1, n), dtype=torch.int64, device=indptr.device)
+    check(lib().gs_node2vec(_ptr(indptr), _ptr(indices), indptr.numel() - 1, _ptr(seeds), n,
+                            walk_length, p, q, seed, call_id, _ptr(out), _stream()))
+    return out
+
+
+def segment_sort(indptr, keys):
+    indptr, keys = _i64t(indptr, "indptr"), _i64t(keys, "keys")
+    out = torch.empty_like(keys)
+    nseg = indptr.numel() - 1
+    ws = _workspace(lib().gs_segment_sort_workspace_bytes(keys.numel(), nseg), keys.device)
+    check(lib().gs_segment_sort_i64(_ptr(indptr), nseg, _ptr(keys), _ptr(out), keys.numel(),
+                                    ws.data_ptr(), ws.numel(), _stream()))
+    return out

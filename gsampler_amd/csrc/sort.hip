@@ -1,0 +1,47 @@
+// sort.hip -- per-segment key sort (row ids inside every column), the
+// prerequisite of node2vec's connectivity test.  The sort itself is rocPRIM's
+// segmented radix sort; this file only adapts it to the workspace convention.
+#include "common.h"
+
+#include <cstring>
+#include <rocprim/device/device_segmented_radix_sort.hpp>
+
+extern "C" {
+
+size_t gs_segment_sort_workspace_bytes(int64_t nnz, int64_t num_segments) {
+  if (nnz < 0 || num_segments < 0) return 0;
+  size_t bytes = 0;
+  const int64_t* k = nullptr;
+  int64_t* o = nullptr;
+  (void)rocprim::segmented_radix_sort_keys(nullptr, bytes, k, o, (size_t)(nnz > 0 ? nnz : 1),
+                                           (unsigned)(num_segments > 0 ? num_segments : 1),
+                                           k, k, 0, 64);
+  return gs::align_up(bytes, 256);
+}
+
+// keys_out[seg] = sorted(keys_in[seg]) for every segment of indptr; in and out
+// must not alias.  SortIndicesCUDA, src/cuda/sort_indices.cu:11-37.
+int gs_segment_sort_i64(const int64_t* indptr, int64_t num_segments,
+                        const int64_t* keys_in, int64_t* keys_out, int64_t nnz,
+                        void* workspace, size_t workspace_bytes,
+                        gs_stream_t stream) {
+  using namespace gs;
+  GS_REQUIRE(nnz >= 0 && num_segments >= 0, "segment_sort: negative size");
+  if (nnz == 0 || num_segments == 0) return GS_OK;
+  GS_REQUIRE(indptr && keys_in && keys_out, "segment_sort: null pointer");
+  GS_REQUIRE(keys_in != keys_out, "segment_sort: in-place sorting is not supported");
+  size_t need = gs_segment_sort_workspace_bytes(nnz, num_segments);
+  if (workspace == nullptr || workspace_bytes < need) {
+    set_error("segment_sort workspace too small: %zu < %zu", workspace_bytes, need);
+    return GS_ERR_WORKSPACE;
+  }
+  hipStream_t s = as_stream(stream);
+  size_t bytes = workspace_bytes;
+  ProfScope ps("segment_sort", s);
+  GS_HIP(rocprim::segmented_radix_sort_keys(workspace, bytes, keys_in, keys_out,
+                                            (size_t)nnz, (unsigned)num_segments,
+                                            indptr, indptr + 1, 0, 64, s));
+  return GS_OK;
+}
+
+}  // extern "C"

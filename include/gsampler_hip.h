@@ -291,6 +291,34 @@ int gs_sorted_to_indptr(const int64_t* sorted_ids, int64_t nnz, int64_t num_cols
                         int64_t* out_indptr, gs_stream_t stream);
 
 /* ------------------------------------------------------------------------
+ * Walks over CSC in-neighbours (a step moves from `curr` to one of the row ids
+ * stored in column `curr`).  out_traces has (walk_length + 1) * num_seeds
+ * entries in step-major order, out[step * num_seeds + walk]; step 0 is the
+ * seed; -1 from a dead end onwards.
+ *  gs_random_walk: uniform next hop.  FusedRandomWalkCUDA,
+ *    src/cuda/fusion/random_walk.cu:49-70.
+ *  gs_node2vec: second-order walk by rejection sampling with integer levels
+ *    (return weight p, neighbour-of-previous weight q, otherwise 1); needs row
+ *    ids sorted inside every column.  FusedNode2VecCUDA,
+ *    src/cuda/fusion/node2vec.cu:139-162.
+ *  gs_segment_sort_i64: sorts the ids of every segment (column).
+ *    SortIndicesCUDA, src/cuda/sort_indices.cu:11-37.
+ * ---------------------------------------------------------------------- */
+int gs_random_walk(const int64_t* indptr, const int64_t* indices, int64_t num_cols,
+                   const int64_t* seeds, int64_t num_seeds, int64_t walk_length,
+                   uint64_t seed, uint64_t call_id, int64_t* out_traces,
+                   gs_stream_t stream);
+int gs_node2vec(const int64_t* indptr, const int64_t* indices, int64_t num_cols,
+                const int64_t* seeds, int64_t num_seeds, int64_t walk_length,
+                double p, double q, uint64_t seed, uint64_t call_id,
+                int64_t* out_traces, gs_stream_t stream);
+size_t gs_segment_sort_workspace_bytes(int64_t nnz, int64_t num_segments);
+int gs_segment_sort_i64(const int64_t* indptr, int64_t num_segments,
+                        const int64_t* keys_in, int64_t* keys_out, int64_t nnz,
+                        void* workspace, size_t workspace_bytes,
+                        gs_stream_t stream);
+
+/* ------------------------------------------------------------------------
  * Super-batch bookkeeping.
  *  gs_decode_batch_ids: ids encoded as id + batch * stride -> out_batch =
  *    id / stride, out_orig = id - batch * stride (either output nullable).

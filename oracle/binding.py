@@ -377,3 +377,29 @@ def list_sample_weighted(probs, num_picks, replace=False, range_=None, seed=7777
     out = np.empty(total, dtype=np.int64)
     f(*args, _p(out), _p(out_range))
     return out, out_range
+
+
+# --------------------------------------------------------------------- walks
+def random_walk(indptr, indices, seeds, walk_length, seed=7777, call_id=0):
+    indptr, indices, seeds = _i64(indptr), _i64(indices), _i64(seeds)
+    out = np.empty((walk_length + 1, seeds.size), dtype=np.int64)
+    lib().gs_random_walk_cpu(_p(indptr), _p(indices), C.c_int64(indptr.size - 1), _p(seeds),
+                             C.c_int64(seeds.size), C.c_int64(walk_length), C.c_uint64(seed),
+                             C.c_uint64(call_id), _p(out))
+    return out
+
+
+def node2vec(indptr, indices, seeds, walk_length, p, q, seed=7777, call_id=0):
+    indptr, indices, seeds = _i64(indptr), _i64(indices), _i64(seeds)
+    out = np.empty((walk_length + 1, seeds.size), dtype=np.int64)
+    lib().gs_node2vec_cpu(_p(indptr), _p(indices), C.c_int64(indptr.size - 1), _p(seeds),
+                          C.c_int64(seeds.size), C.c_int64(walk_length), C.c_double(p),
+                          C.c_double(q), C.c_uint64(seed), C.c_uint64(call_id), _p(out))
+    return out
+
+
+def segment_sort(indptr, keys):
+    indptr, keys = _i64(indptr), _i64(keys)
+    out = np.empty_like(keys)
+    lib().gs_segment_sort_i64_cpu(_p(indptr), C.c_int64(indptr.size - 1), _p(keys), _p(out))
+    return out

@@ -858,3 +858,110 @@ extern "C" int64_t gs_list_sample_uniform_cpu(int64_t n, int64_t num_picks,
   }
   return sub[1];
 }
+
+// -------------------------------------------------------------------------
+// Walks.  Trace layout out[step * N + walk] (src/cuda/fusion/random_walk.cu:34).
+//  random walk (:30-46): curr == -1 or deg == 0 -> -1, else a uniform row id of
+//  column curr; stream pos = walk, draw = step.
+//  node2vec (src/cuda/fusion/node2vec.cu:90-135), per step with deg > 1, per
+//  attempt (stream draw = step << 32 | attempt, one Philox block: w2 -> u,
+//  w1:w0 -> candidate):
+//    y = (int)floor(u * max(p, q));  reject if y >= max(max(p, q), 1);
+//    candidate = uniform row id of column curr;
+//    accept if y < min(p, q, 1);
+//    else h = p if candidate == previous, q if candidate is a row id of column
+//    `previous` (sorted, binary search), 1 otherwise;  accept if y < h.
+//  deg == 1 takes the only neighbour.  The reference starts with previous =
+//  thread id (:89); here there is no previous node before the first step.  Its
+//  candidate index floor(u * deg) can reach deg when u == 1; bounded() cannot.
+//  After 2^16 attempts the last candidate is taken (never reached in practice;
+//  it bounds the loop).
+namespace {
+bool sorted_contains(const int64_t* ptr, int64_t n, int64_t target) {
+  return std::binary_search(ptr, ptr + n, target);
+}
+}  // namespace
+
+extern "C" {
+
+void gs_random_walk_cpu(const int64_t* indptr, const int64_t* indices,
+                        int64_t num_cols, const int64_t* seeds, int64_t num_seeds,
+                        int64_t walk_length, uint64_t seed, uint64_t call_id,
+                        int64_t* out) {
+  Stream rng(seed, call_id);
+#pragma omp parallel for schedule(static)
+  for (int64_t i = 0; i < num_seeds; ++i) {
+    int64_t curr = seeds[i];
+    out[i] = curr;
+    for (int64_t step = 1; step <= walk_length; ++step) {
+      int64_t pick = -1;
+      if (curr >= 0 && curr < num_cols) {
+        int64_t deg = indptr[curr + 1] - indptr[curr];
+        if (deg > 0)
+          pick = indices[indptr[curr] +
+                         (int64_t)rng.bounded((uint64_t)i, (uint64_t)step, (uint64_t)deg)];
+      }
+      curr = pick;
+      out[step * num_seeds + i] = pick;
+    }
+  }
+}
+
+void gs_node2vec_cpu(const int64_t* indptr, const int64_t* indices,
+                     int64_t num_cols, const int64_t* seeds, int64_t num_seeds,
+                     int64_t walk_length, double p, double q, uint64_t seed,
+                     uint64_t call_id, int64_t* out) {
+  Stream rng(seed, call_id);
+  const double max_scale = std::max(p, q);
+  const double reject_from = std::max(max_scale, 1.0);
+  const double accept_below = std::min(std::min(p, q), 1.0);
+#pragma omp parallel for schedule(dynamic, 256)
+  for (int64_t i = 0; i < num_seeds; ++i) {
+    int64_t curr = seeds[i], last = -1;
+    out[i] = curr;
+    for (int64_t step = 1; step <= walk_length; ++step) {
+      int64_t pick = -1;
+      if (curr >= 0 && curr < num_cols) {
+        int64_t start = indptr[curr], deg = indptr[curr + 1] - start;
+        if (deg == 1) {
+          pick = indices[start];
+        } else if (deg > 1) {
+          for (uint32_t attempt = 0;; ++attempt) {
+            U4 w = rng.words((uint64_t)i, ((uint64_t)step << 32) | attempt);
+            double u = (double)((w.v[2] >> 8) + 1u) * 0x1p-24;
+            int y = (int)std::floor(u * max_scale);
+            uint64_t r = ((uint64_t)w.v[1] << 32) | w.v[0];
+            int64_t cand =
+                indices[start + (int64_t)(((unsigned __int128)r * (uint64_t)deg) >> 64)];
+            pick = cand;
+            if (attempt + 1 >= (1u << 16)) break;
+            if ((double)y >= reject_from) continue;
+            if ((double)y < accept_below) break;
+            double h = 1.0;
+            if (cand == last)
+              h = p;
+            else if (last >= 0 && last < num_cols &&
+                     sorted_contains(indices + indptr[last],
+                                     indptr[last + 1] - indptr[last], cand))
+              h = q;
+            if ((double)y < h) break;
+          }
+        }
+      }
+      last = curr;
+      curr = pick;
+      out[step * num_seeds + i] = pick;
+    }
+  }
+}
+
+// Sort of the row ids inside every column, src/cuda/sort_indices.cu:11-37.
+void gs_segment_sort_i64_cpu(const int64_t* indptr, int64_t num_segments,
+                             const int64_t* keys_in, int64_t* keys_out) {
+  for (int64_t c = 0; c < num_segments; ++c) {
+    std::copy(keys_in + indptr[c], keys_in + indptr[c + 1], keys_out + indptr[c]);
+    std::sort(keys_out + indptr[c], keys_out + indptr[c + 1]);
+  }
+}
+
+}  // extern "C"
