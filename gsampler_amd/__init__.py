@@ -9,7 +9,8 @@ _library.load()
 
 import torch  # noqa: E402
 
-from . import capi, ops, utils  # noqa: E402,F401
+from . import capi, jit, ops, utils  # noqa: E402,F401
+from .jit import GSTracer, compile, gs_symbolic_trace  # noqa: E402,F401
 from .format import _COO, _CSC, _CSR  # noqa: E402,F401
 from .matrix_api import BatchMatrix, Matrix  # noqa: E402,F401
 

@@ -26,6 +26,7 @@ inline gs_stream_t cur_stream() {
 // (src/graph_ops.cc:28 "Not implemented warning"), this raises instead.
 inline torch::Tensor ids(const torch::Tensor& t, const char* name) {
   TORCH_CHECK(t.defined(), name, " is undefined");
+  if (t.numel() == 0 && t.scalar_type() == torch::kInt64) return t;  // "none"
   TORCH_CHECK(t.is_cuda(), name, " must live on the GPU (got ", t.device(), ")");
   TORCH_CHECK(t.scalar_type() == torch::kInt64, name, " must be int64 (got ",
               t.scalar_type(), ")");

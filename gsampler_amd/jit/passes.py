@@ -1,0 +1,312 @@
+"""Rewrite passes over the traced operator graph.
+
+Structural clean-up: common-subexpression elimination, dead-code elimination,
+hoisting of tensor constants.  Operator rewrites (observable in
+`compiled.gm.graph`, same set as the reference's python/gs/jit/optimize.py):
+
+  merge_relabel_and_all_nodes   _CAPI_GetValidNodes + _CAPI_GraphRelabel on one
+                                matrix            -> one _CAPI_GraphRelabel
+  fuse_slicing_and_sampling     _CAPI_Slicing -> _CAPI_Sampling on one axis
+                                                  -> _CAPI_SlicingSampling
+  batch_fuse_slicing_and_sampling  _CAPI_BatchColSlicing(encoding=False) ->
+                                _CAPI_BatchRowSampling
+                                                  -> _CAPI_BatchFusedSlicingSampling
+  fuse_square_and_sum           (e ** 2) summed by a copy_rhs / sum SpMM
+                                                  -> _CAPI_FusedESquareSum
+  merge_u_mul_v                 two u-op-v SDDMMs on one matrix
+                                                  -> _CAPI_FusedUOPV
+  select_formats                deterministic on_format / output_format choice
+"""
+import operator
+from typing import Dict, Iterable, List, Optional
+
+import torch.fx as fx
+
+from ..format import _COO, _CSC, _CSR
+
+# Operators that write into a caller-allocated tensor: they have no users in the
+# graph but must survive dead-code elimination.
+IN_PLACE_OPS = ("_CAPI_SDDMM", "_CAPI_SpMM", "_CAPI_FusedUOPV", "_CAPI_FusedESquareSum",
+                "_CAPI_FusedEDivUSum")
+
+
+def _input_nodes(node: fx.Node) -> Iterable[fx.Node]:
+    return node.all_input_nodes
+
+
+def _finish(gm: fx.GraphModule) -> fx.GraphModule:
+    gm.graph.lint()
+    gm.recompile()
+    return gm
+
+
+def dce(gm: fx.GraphModule) -> fx.GraphModule:
+    live = set()
+    for node in reversed(gm.graph.nodes):
+        if node.op in ("output", "placeholder") or node.target in IN_PLACE_OPS:
+            live.add(node)
+        if node in live:
+            live.update(_input_nodes(node))
+    for node in reversed(gm.graph.nodes):
+        if node not in live:
+            gm.graph.erase_node(node)
+    return _finish(gm)
+
+
+def cse(gm: fx.GraphModule) -> fx.GraphModule:
+    """Merges nodes with identical target and arguments.  Sampling operators are
+    left alone: two textually identical sampling calls draw different samples."""
+    seen: Dict[str, fx.Node] = {}
+    for node in list(gm.graph.nodes):
+        if node.op in ("placeholder", "output"):
+            continue
+        if isinstance(node.target, str) and "Sampling" in node.target:
+            continue
+        if node.target in IN_PLACE_OPS:
+            continue
+        key = f"{node.op}|{node.target}|{node.args}|{node.kwargs}"
+        if key in seen:
+            node.replace_all_uses_with(seen[key])
+            gm.graph.erase_node(node)
+        else:
+            seen[key] = node
+    return _finish(gm)
+
+
+def move_constant_to_top(gm: fx.GraphModule) -> fx.GraphModule:
+    first = next(iter(gm.graph.nodes))
+    constants = [n for n in gm.graph.nodes if n.op == "get_attr" and "constant" in n.name]
+    with gm.graph.inserting_before(first):
+        for node in constants:
+            if node is first:
+                continue
+            node.replace_all_uses_with(gm.graph.node_copy(node))
+            gm.graph.erase_node(node)
+    return _finish(gm)
+
+
+def _is_method(node: fx.Node, name: str) -> bool:
+    return node.op == "call_method" and node.target == name
+
+
+def _getitem_users(node: fx.Node, index: int) -> List[fx.Node]:
+    return [u for u in node.users
+            if u.op == "call_function" and u.target is operator.getitem and u.args[1] == index]
+
+
+def merge_relabel_and_all_nodes(gm: fx.GraphModule) -> fx.GraphModule:
+    """all_nodes() and to_dgl_block() of one matrix share a single relabel."""
+    gm = cse(gm)
+    by_graph: Dict[fx.Node, List[fx.Node]] = {}
+    for node in gm.graph.nodes:
+        if _is_method(node, "_CAPI_GetValidNodes") or _is_method(node, "_CAPI_GraphRelabel"):
+            by_graph.setdefault(node.args[0], []).append(node)
+    for group in by_graph.values():
+        relabels = [n for n in group if n.target == "_CAPI_GraphRelabel"]
+        valid = [n for n in group if n.target == "_CAPI_GetValidNodes"]
+        if not relabels or not valid:
+            continue
+        keep = relabels[0]
+        first = min(group, key=lambda n: list(gm.graph.nodes).index(n))
+        if first is not keep:
+            first.prepend(keep)  # the relabel must precede every former user
+        with gm.graph.inserting_after(keep):
+            frontier = gm.graph.call_function(operator.getitem, args=(keep, 0))
+        for v in valid:
+            if v.args[1:] == keep.args[1:]:
+                v.replace_all_uses_with(frontier)
+    return dce(gm)
+
+
+def fuse_slicing_and_sampling(gm: fx.GraphModule) -> fx.GraphModule:
+    """Slicing(seeds, axis, on, out) -> [0] -> Sampling(axis, K, replace, on, out)
+       => SlicingSampling(axis, seeds, K, replace, on, out).
+
+    Edge data gathered through the slice index and then through the sampling
+    index is re-gathered from the parent with the fused index, which addresses
+    the parent's edges directly."""
+    for sampling in list(gm.graph.nodes):
+        if not _is_method(sampling, "_CAPI_Sampling"):
+            continue
+        sliced_graph = sampling.args[0]
+        if not (sliced_graph.op == "call_function" and sliced_graph.target is operator.getitem
+                and sliced_graph.args[1] == 0):
+            continue
+        slicing = sliced_graph.args[0]
+        if not _is_method(slicing, "_CAPI_Slicing"):
+            continue
+        if sampling.args[1] != slicing.args[2]:      # same axis
+            continue
+        if len(sliced_graph.users) > 1:              # the slice itself is used
+            continue
+        slice_index = _getitem_users(slicing, 1)
+        sample_index = _getitem_users(sampling, 1)
+        # every tensor gathered with the slice index may only feed a gather with
+        # the sampling index
+        rewires = []
+        ok = True
+        for idx_node in slice_index:
+            for gathered in idx_node.users:
+                users = list(gathered.users)
+                if len(users) != 1 or not sample_index or sample_index[0] not in users[0].args:
+                    ok = False
+                rewires.append((gathered, users[0] if users else None))
+        if not ok:
+            continue
+        with gm.graph.inserting_before(slicing):
+            fused = gm.graph.call_method(
+                "_CAPI_SlicingSampling",
+                args=(slicing.args[0], slicing.args[2], slicing.args[1], sampling.args[2],
+                      sampling.args[3], sampling.args[4], sampling.args[5]))
+            fused_graph = gm.graph.call_function(operator.getitem, args=(fused, 0))
+            fused_index = gm.graph.call_function(operator.getitem, args=(fused, 1))
+        for g in _getitem_users(sampling, 0):
+            g.replace_all_uses_with(fused_graph)
+        for gathered, second in rewires:
+            with gm.graph.inserting_before(second):
+                direct = gm.graph.call_function(operator.getitem,
+                                                args=(gathered.args[0], fused_index))
+            second.replace_all_uses_with(direct)
+    return dce(gm)
+
+
+def batch_fuse_slicing_and_sampling(gm: fx.GraphModule) -> fx.GraphModule:
+    """BatchColSlicing(seeds, ptr, encoding=False) -> [0] -> BatchRowSampling(K, replace)
+       => BatchFusedSlicingSampling(seeds, ptr, K, replace)."""
+    for sampling in list(gm.graph.nodes):
+        if not _is_method(sampling, "_CAPI_BatchRowSampling"):
+            continue
+        sliced_graph = sampling.args[0]
+        if not (sliced_graph.op == "call_function" and sliced_graph.target is operator.getitem):
+            continue
+        slicing = sliced_graph.args[0]
+        if not _is_method(slicing, "_CAPI_BatchColSlicing"):
+            continue
+        if slicing.args[3] is not False or len(sliced_graph.users) > 1:
+            continue
+        # edge data gathered through the slice index cannot be re-routed here
+        if any(list(i.users) for i in _getitem_users(slicing, 1)):
+            continue
+        with gm.graph.inserting_before(slicing):
+            fused = gm.graph.call_method(
+                "_CAPI_BatchFusedSlicingSampling",
+                args=(slicing.args[0], slicing.args[1], slicing.args[2], sampling.args[1],
+                      sampling.args[2]))
+        sampling.replace_all_uses_with(fused)
+    return dce(gm)
+
+
+def fuse_square_and_sum(gm: fx.GraphModule) -> fx.GraphModule:
+    """SpMM("copy_rhs", "sum", _, e ** 2, ...) => FusedESquareSum(..., e, ...)."""
+    for spmm in list(gm.graph.nodes):
+        if not _is_method(spmm, "_CAPI_SpMM"):
+            continue
+        if spmm.args[1] != "copy_rhs" or spmm.args[2] != "sum":
+            continue
+        efeat = spmm.args[4]
+        if not (isinstance(efeat, fx.Node) and efeat.op == "call_function"
+                and efeat.target is operator.pow and efeat.args[1] == 2):
+            continue
+        new_args = list(spmm.args)
+        new_args[4] = efeat.args[0]
+        with gm.graph.inserting_before(spmm):
+            gm.graph.call_method("_CAPI_FusedESquareSum", args=tuple(new_args))
+        gm.graph.erase_node(spmm)
+    return dce(gm)
+
+
+def merge_u_mul_v(gm: fx.GraphModule) -> fx.GraphModule:
+    """Two SDDMMs with targets (u, v), the same operator, graph and format
+       => one FusedUOPV that sweeps the edges once."""
+    groups: Dict[str, List[fx.Node]] = {}
+    for node in gm.graph.nodes:
+        if _is_method(node, "_CAPI_SDDMM") and node.args[5] == 0 and node.args[6] == 2:
+            groups.setdefault(f"{node.args[0]}|{node.args[1]}|{node.args[7]}", []).append(node)
+    order = {n: i for i, n in enumerate(gm.graph.nodes)}
+    for pair in groups.values():
+        if len(pair) != 2:
+            continue
+        first, second = sorted(pair, key=order.get)
+        # The fused operator runs where the second product ran.  Readers of the
+        # first output that sit in between (its squeeze step) move behind it;
+        # that is only sound when their own users come later still.
+        early = [u for u in first.args[4].users
+                 if u is not first and order[u] < order[second]]
+        if any(order[uu] < order[second] for u in early for uu in u.users):
+            continue
+        for u in sorted(early, key=order.get, reverse=True):
+            second.append(u)
+        with gm.graph.inserting_before(second):
+            gm.graph.call_method(
+                "_CAPI_FusedUOPV",
+                args=(first.args[0], first.args[1], first.args[2], first.args[3], first.args[4],
+                      second.args[2], second.args[3], second.args[4], second.args[7]))
+        gm.graph.erase_node(first)
+        gm.graph.erase_node(second)
+    return dce(gm)
+
+
+# --------------------------------------------------------------- formats
+# operator -> (position of on_format, position of output_format or None); positions
+# count the operator object itself as argument 0 (python/gs/jit/module.py:21-31).
+FORMAT_ARGS = {
+    "_CAPI_Slicing": (3, 4),
+    "_CAPI_Sampling": (4, 5),
+    "_CAPI_SamplingProbs": (5, 6),
+    "_CAPI_SlicingSampling": (5, 6),
+    "_CAPI_SDDMM": (7, None),
+    "_CAPI_SpMM": (9, None),
+    "_CAPI_FusedUOPV": (8, None),
+    "_CAPI_FusedESquareSum": (9, None),
+    "_CAPI_FusedEDivUSum": (9, None),
+}
+
+
+def _preferred(node: fx.Node) -> List[int]:
+    """Formats an operator can run on, best first.  Slicing prefers the format
+    whose compressed axis is the sliced one (a gather), then the other
+    compressed format (a filter pass, no sort), then COO."""
+    t = node.target
+    if t == "_CAPI_Slicing":
+        return [_CSR, _CSC, _COO] if node.args[2] == 0 else [_CSC, _CSR, _COO]
+    if t in ("_CAPI_Sampling", "_CAPI_SlicingSampling"):
+        return [_CSR] if node.args[1] == 0 else [_CSC]
+    if t == "_CAPI_SamplingProbs":
+        return [_CSR] if node.args[1] == 0 else [_CSC]
+    if t in ("_CAPI_SpMM", "_CAPI_FusedESquareSum", "_CAPI_FusedEDivUSum"):
+        return [_CSR, _COO] if node.args[8] == 2 else [_CSC, _COO]
+    if t == "_CAPI_SDDMM":
+        return [_COO, _CSC, _CSR]
+    return [_COO, _CSC]
+
+
+def select_formats(gm: fx.GraphModule, input_formats: int = _CSC) -> fx.GraphModule:
+    """Deterministic format assignment: every operator runs on the best format
+    its input already holds (no conversion), and producers materialise that
+    format plus COO.  Input matrices hold `input_formats`; derived matrices hold
+    what their producer was told to emit.  (The reference times every plan on
+    the device and keeps the fastest, python/gs/jit/module.py:306-421.)"""
+    holds: Dict[fx.Node, int] = {}
+
+    def formats_of(graph_node: fx.Node) -> int:
+        if graph_node in holds:
+            return holds[graph_node]
+        if (graph_node.op == "call_function" and graph_node.target is operator.getitem
+                and graph_node.args[0] in holds):
+            return holds[graph_node.args[0]]
+        return input_formats
+
+    for node in gm.graph.nodes:
+        if node.op != "call_method" or node.target not in FORMAT_ARGS:
+            continue
+        on_pos, out_pos = FORMAT_ARGS[node.target]
+        available = formats_of(node.args[0])
+        choice: Optional[int] = next((f for f in _preferred(node) if f & available), None)
+        if choice is None:                      # a conversion is unavoidable
+            choice = _preferred(node)[0]
+        node.update_arg(on_pos, choice)
+        if out_pos is not None:
+            out = choice | _COO if choice != _COO else _COO
+            node.update_arg(out_pos, out)
+            holds[node] = out
+    return _finish(gm)

@@ -59,7 +59,7 @@ class Matrix:
     def null_tensor(self) -> torch.Tensor:
         global _NULL_TENSOR
         if _NULL_TENSOR is None:
-            _NULL_TENSOR = torch.empty(0, dtype=torch.int64, device="cuda")
+            _NULL_TENSOR = torch.empty(0, dtype=torch.int64)
         return _NULL_TENSOR
 
     def load_graph(self, format: str, format_tensors: List[torch.Tensor]) -> "Matrix":

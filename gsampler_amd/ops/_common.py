@@ -31,14 +31,22 @@ def pad_feature_dims(lhs: torch.Tensor, rhs: torch.Tensor):
     return lhs, rhs
 
 
+def rewrite_inverse_ops(op: str, rhs):
+    """sub -> add of the negated operand, div -> mul by the reciprocal (as the
+    reference's wrappers intend, python/gs/ops/sddmm.py:20-25).  Runs on plain
+    Python strings, so the operator name stays a constant in a traced graph."""
+    if op == "sub":
+        return "add", -rhs
+    if op == "div":
+        return "mul", 1.0 / rhs
+    return op, rhs
+
+
 def prepare_binary(op: str, lhs: Optional[torch.Tensor], rhs: Optional[torch.Tensor]):
-    """-> (op, lhs, rhs, feature_shape, squeeze, dtype, device)."""
+    """-> (lhs, rhs, feature_shape, squeeze, dtype, device) for an operator that
+    has already been through rewrite_inverse_ops."""
     if op not in ("copy_lhs", "copy_rhs"):
         lhs, rhs = pad_feature_dims(lhs, rhs)
-    if op == "sub":
-        op, rhs = "add", -rhs
-    elif op == "div":
-        op, rhs = "mul", 1.0 / rhs
     use_l, use_r = op != "copy_rhs", op != "copy_lhs"
     if use_l and use_r:
         if lhs.device != rhs.device:
@@ -55,4 +63,4 @@ def prepare_binary(op: str, lhs: Optional[torch.Tensor], rhs: Optional[torch.Ten
                                  tuple(rhs.shape[1:]) if use_r else (0,)) \
         if (use_l and use_r) else tuple(ref.shape[1:])
     squeeze = (exp_l or not use_l) and (exp_r or not use_r)
-    return op, lhs, rhs, feat, squeeze, ref.dtype, ref.device
+    return lhs, rhs, feat, squeeze, ref.dtype, ref.device

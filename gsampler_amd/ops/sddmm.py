@@ -7,7 +7,7 @@ from itertools import product
 import torch
 
 from ..format import _COO
-from ._common import TARGET, prepare_binary
+from ._common import TARGET, prepare_binary, rewrite_inverse_ops
 
 torch.fx.wrap("_before_sddmm")
 torch.fx.wrap("_after_sddmm")
@@ -16,9 +16,9 @@ __all__ = ["gsddmm", "copy_u", "copy_v"]
 
 
 def _before_sddmm(num_edges, op, lhs_data, rhs_data):
-    op2, lhs, rhs, feat, squeeze, dtype, device = prepare_binary(op, lhs_data, rhs_data)
+    lhs, rhs, feat, squeeze, dtype, device = prepare_binary(op, lhs_data, rhs_data)
     out = torch.zeros((num_edges,) + tuple(feat), dtype=dtype, device=device)
-    return op2, lhs, rhs, out, squeeze
+    return lhs, rhs, out, squeeze
 
 
 def _after_sddmm(out, squeeze):
@@ -27,8 +27,9 @@ def _after_sddmm(out, squeeze):
 
 def gsddmm(g, op, lhs_data, rhs_data, lhs_target="u", rhs_target="v", on_format=_COO):
     num_edges = g._graph._CAPI_GetNumEdges()
-    op2, lhs, rhs, out, squeeze = _before_sddmm(num_edges, op, lhs_data, rhs_data)
-    g._graph._CAPI_SDDMM(op2, lhs, rhs, out, TARGET[lhs_target], TARGET[rhs_target],
+    op, rhs_data = rewrite_inverse_ops(op, rhs_data)
+    lhs, rhs, out, squeeze = _before_sddmm(num_edges, op, lhs_data, rhs_data)
+    g._graph._CAPI_SDDMM(op, lhs, rhs, out, TARGET[lhs_target], TARGET[rhs_target],
                          on_format)
     return _after_sddmm(out, squeeze)
 

@@ -6,7 +6,7 @@ import sys
 import torch
 
 from ..format import _CSC
-from ._common import prepare_binary
+from ._common import prepare_binary, rewrite_inverse_ops
 
 torch.fx.wrap("_before_spmm")
 torch.fx.wrap("_after_spmm")
@@ -15,17 +15,17 @@ __all__ = ["gspmm"]
 
 
 def _before_spmm(num_rows, num_cols, op, reduce_op, lhs_data, rhs_data, lhs_target):
-    op2, u, e, feat, squeeze, dtype, device = prepare_binary(op, lhs_data, rhs_data)
+    u, e, feat, squeeze, dtype, device = prepare_binary(op, lhs_data, rhs_data)
     n_out = num_cols if lhs_target == 0 else num_rows
     shape = (n_out,) + tuple(feat)
     v = torch.zeros(shape, dtype=dtype, device=device)
     arg_u = arg_e = None
     if reduce_op in ("max", "min"):
-        if op2 != "copy_rhs":
+        if op != "copy_rhs":
             arg_u = torch.zeros(shape, dtype=torch.int64, device=device)
-        if op2 != "copy_lhs":
+        if op != "copy_lhs":
             arg_e = torch.zeros(shape, dtype=torch.int64, device=device)
-    return op2, u, e, v, arg_u, arg_e, squeeze
+    return v, arg_u, arg_e, squeeze
 
 
 def _after_spmm(v, squeeze):
@@ -35,9 +35,14 @@ def _after_spmm(v, squeeze):
 def gspmm(g, op, reduce_op, lhs_data, rhs_data, lhs_target, on_format):
     num_rows = g._graph._CAPI_GetNumRows()
     num_cols = g._graph._CAPI_GetNumCols()
-    op2, u, e, v, arg_u, arg_e, squeeze = _before_spmm(
+    op, rhs_data = rewrite_inverse_ops(op, rhs_data)
+    v, arg_u, arg_e, squeeze = _before_spmm(
         num_rows, num_cols, op, reduce_op, lhs_data, rhs_data, lhs_target)
-    g._graph._CAPI_SpMM(op2, reduce_op, u, e, v, arg_u, arg_e, lhs_target, on_format)
+    # the operands go in as given (scalar features stay 1-D): the operator
+    # treats [n] and [n, 1] alike, and the traced graph keeps a direct
+    # producer -> SpMM edge for the fusion passes to match
+    g._graph._CAPI_SpMM(op, reduce_op, lhs_data, rhs_data, v, arg_u, arg_e, lhs_target,
+                        on_format)
     return _after_spmm(v, squeeze)
 
 

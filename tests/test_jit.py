@@ -1,0 +1,218 @@
+"""gs.jit.compile: the rewrites are visible in the traced graph (no GPU needed
+to trace), and compiled samplers return what eager execution returns (GPU)."""
+import numpy as np
+import pytest
+import torch
+
+import gsampler_amd as gs
+
+
+def graphsage_sampler(A, seeds, fanouts):
+    input_node = seeds
+    ret = []
+    for K in fanouts:
+        subA = A[:, seeds]
+        sampleA = subA.individual_sampling(K, None, False)
+        seeds = sampleA.all_nodes()
+        ret.append(sampleA.to_dgl_block())
+    output_node = seeds
+    return input_node, output_node, ret
+
+
+def batch_graphsage_sampler(A, seeds, seeds_ptr, fanouts):
+    ret = []
+    for k in fanouts:
+        subA = A[:, seeds::seeds_ptr]
+        sampleA = subA.individual_sampling(k, None, False)
+        seeds, seeds_ptr = sampleA.all_nodes()
+        ret.append(sampleA.to_dgl_block())
+    return ret
+
+
+def ladies_sampler(A, seeds, fanouts):
+    # examples/ladies/ladies.py:7-21 of the reference
+    input_node = seeds
+    ret = []
+    for K in fanouts:
+        subA = A[:, seeds]
+        subA.edata["p"] = subA.edata["w"] ** 2
+        prob = subA.sum("p", axis=1)
+        sampleA, select_index = subA.collective_sampling(K, prob, False)
+        sampleA = sampleA.div("w", prob[select_index], axis=1)
+        out = sampleA.sum("w", axis=0)
+        sampleA = sampleA.div("w", out, axis=0)
+        seeds = sampleA.all_nodes()
+        ret.append(sampleA.to_dgl_block(prefetch_edata={"w"}))
+    output_node = seeds
+    return input_node, output_node, ret
+
+
+def pass_like_sampler(A, seeds, u1, v1, u2, v2):
+    subA = A[:, seeds]
+    a = gs.ops.u_mul_v(subA, u1, v1)
+    b = gs.ops.u_mul_v(subA, u2, v2)
+    return a + b
+
+
+def targets(gm):
+    return [n.target for n in gm.graph.nodes if n.op == "call_method"]
+
+
+def test_graphsage_rewrites():
+    m = gs.Matrix(gs.Graph(10, 10))
+    c = gs.jit.compile(func=graphsage_sampler, args=(m, torch.arange(3), [25, 10]))
+    t = targets(c.gm)
+    assert t.count("_CAPI_SlicingSampling") == 2          # slice + sample fused
+    assert "_CAPI_Slicing" not in t and "_CAPI_Sampling" not in t
+    assert t.count("_CAPI_GraphRelabel") == 2 and "_CAPI_GetValidNodes" not in t
+    fused = [n for n in c.gm.graph.nodes if n.target == "_CAPI_SlicingSampling"]
+    assert [n.args[3] for n in fused] == [25, 10]         # fanouts are constants
+    assert all(n.args[1] == 1 and n.args[5] == gs._CSC and n.args[6] == gs._CSC | gs._COO
+               for n in fused)
+
+
+def test_batch_graphsage_rewrites():
+    m = gs.Matrix(gs.Graph(10, 10))
+    bm = gs.BatchMatrix()
+    bm.load_from_matrix(m, False)
+    c = gs.jit.compile(func=batch_graphsage_sampler,
+                       args=(bm, torch.arange(4), torch.tensor([0, 2, 4]), [5, 5]),
+                       try_compact=False, format_select=False)
+    t = targets(c.gm)
+    assert t.count("_CAPI_BatchFusedSlicingSampling") == 2
+    assert "_CAPI_BatchColSlicing" not in t and "_CAPI_BatchRowSampling" not in t
+    # encoded batches are not fused (rows are renumbered between the two steps)
+    bm2 = gs.BatchMatrix()
+    bm2.load_from_matrix(m, True)
+    c2 = gs.jit.compile(func=batch_graphsage_sampler,
+                        args=(bm2, torch.arange(4), torch.tensor([0, 2, 4]), [5]))
+    assert "_CAPI_BatchColSlicing" in targets(c2.gm)
+
+
+def test_ladies_rewrites():
+    m = gs.Matrix(gs.Graph(10, 10))
+    m.edata["w"] = torch.rand(7)
+    c = gs.jit.compile(func=ladies_sampler, args=(m, torch.arange(3), [4, 4]))
+    t = targets(c.gm)
+    assert t.count("_CAPI_FusedESquareSum") == 2          # (w ** 2).sum fused
+    assert t.count("_CAPI_SpMM") == 2                     # the column sums stay
+    assert t.count("_CAPI_SDDMM") == 4
+    assert "_CAPI_GetValidNodes" not in t
+    # formats: the row slice runs on the CSC the column slice produced (no sort)
+    row_slices = [n for n in c.gm.graph.nodes
+                  if n.target == "_CAPI_Slicing" and n.args[2] == 0]
+    assert row_slices and all(n.args[3] == gs._CSC for n in row_slices)
+    # edge data is a run-time input, not a baked constant
+    assert not any(n.op == "get_attr" and "constant" in n.name and n.meta.get("val") is not None
+                   for n in c.gm.graph.nodes)
+    assert sum(n.op == "placeholder" for n in c.gm.graph.nodes) >= 3
+
+
+def test_two_u_mul_v_are_merged():
+    m = gs.Matrix(gs.Graph(10, 10))
+    u, v = torch.rand(10), torch.rand(3)
+    c = gs.jit.compile(func=pass_like_sampler, args=(m, torch.arange(3), u, v, u + 1, v + 1))
+    t = targets(c.gm)
+    assert t.count("_CAPI_FusedUOPV") == 1 and "_CAPI_SDDMM" not in t
+
+
+# ------------------------------------------------------------------- on the GPU
+DEV = "cuda:0"
+
+
+def _graph():
+    from gsampler_amd.utils import rmat_csc
+    indptr, indices = rmat_csc(5000, 150000, seed=1)
+    m = gs.Matrix()
+    m.load_graph("CSC", [indptr.to(DEV), indices.to(DEV)])
+    g = torch.Generator().manual_seed(0)
+    m.edata["w"] = (torch.rand(indices.numel(), generator=g) + 0.05).to(DEV)
+    return m
+
+
+def _blocks_equal(a, b):
+    assert torch.equal(a.row, b.row) and torch.equal(a.col, b.col)
+    assert (a.num_src, a.num_dst) == (b.num_src, b.num_dst)
+    assert torch.equal(a.srcdata["_ID"], b.srcdata["_ID"])
+    assert set(a.edata) == set(b.edata)
+    for k in a.edata:
+        assert torch.allclose(a.edata[k], b.edata[k], rtol=1e-5)
+
+
+@pytest.mark.gpu
+def test_compiled_graphsage_equals_eager():
+    m = _graph()
+    seeds = torch.randperm(5000, generator=torch.Generator().manual_seed(1))[:200].to(DEV)
+    c = gs.jit.compile(func=graphsage_sampler, args=(m, seeds, [10, 5]))
+    gs.manual_seed(3)
+    e_in, e_out, e_blocks = graphsage_sampler(m, seeds, [10, 5])
+    gs.manual_seed(3)
+    c_in, c_out, c_blocks = c(m, seeds, [10, 5])
+    assert torch.equal(e_in, c_in) and torch.equal(e_out, c_out)
+    for a, b in zip(e_blocks, c_blocks):
+        _blocks_equal(a, b)
+    # other seeds through the same compiled object
+    seeds2 = seeds.flip(0)[:100].contiguous()
+    gs.manual_seed(4)
+    want = graphsage_sampler(m, seeds2, [10, 5])
+    gs.manual_seed(4)
+    got = c(m, seeds2, [10, 5])
+    assert torch.equal(want[1], got[1])
+
+
+@pytest.mark.gpu
+def test_compiled_batch_graphsage_equals_eager():
+    from gsampler_amd.utils import batched_seeds
+    m = _graph()
+    bm = gs.BatchMatrix()
+    bm.load_from_matrix(m, False)
+    seeds, ptr = batched_seeds(5000, 4, 64, seed=2)
+    seeds, ptr = seeds.to(DEV), ptr.to(DEV)
+    c = gs.jit.compile(func=batch_graphsage_sampler, args=(bm, seeds, ptr, [10, 5]),
+                       try_compact=False, format_select=False)
+    gs.manual_seed(5)
+    eager = batch_graphsage_sampler(bm, seeds, ptr, [10, 5])
+    gs.manual_seed(5)
+    comp = c(bm, seeds, ptr, [10, 5])
+    for le, lc in zip(eager, comp):
+        assert len(le) == len(lc) == 4
+        for a, b in zip(le, lc):
+            _blocks_equal(a, b)
+
+
+@pytest.mark.gpu
+def test_ladies_eager_compiled_and_invariants():
+    m = _graph()
+    seeds = torch.randperm(5000, generator=torch.Generator().manual_seed(6))[:128].to(DEV)
+    c = gs.jit.compile(func=ladies_sampler, args=(m, seeds, [64, 64]))
+    gs.manual_seed(7)
+    e_in, e_out, e_blocks = ladies_sampler(m, seeds, [64, 64])
+    gs.manual_seed(7)
+    c_in, c_out, c_blocks = c(m, seeds, [64, 64])
+    assert torch.equal(e_out, c_out)
+    for a, b in zip(e_blocks, c_blocks):
+        _blocks_equal(a, b)
+    blk = e_blocks[0]
+    # at most K distinct source rows besides the seeds; weights normalised per column
+    assert blk.num_dst == 128 and blk.num_src <= 128 + 64
+    w = blk.edata["w"].double()
+    col_sum = torch.zeros(blk.num_dst, dtype=torch.float64, device=DEV).index_add_(0, blk.col, w)
+    has_edge = torch.zeros(blk.num_dst, dtype=torch.bool, device=DEV)
+    has_edge[blk.col] = True
+    assert torch.allclose(col_sum[has_edge], torch.ones_like(col_sum[has_edge]), atol=1e-4)
+    # every block edge is an edge of the graph
+    indptr, indices, _ = m.csc
+    src = blk.srcdata["_ID"][blk.row]
+    dst = seeds[blk.col]
+    for s, d in list(zip(src.tolist(), dst.tolist()))[:300]:
+        assert s in indices[indptr[d]:indptr[d + 1]].tolist()
+
+
+@pytest.mark.gpu
+def test_merged_u_mul_v_equals_eager():
+    m = _graph()
+    seeds = torch.arange(0, 900, 3, device=DEV)
+    u, v = torch.rand(m.num_rows(), device=DEV), torch.rand(seeds.numel(), device=DEV)
+    c = gs.jit.compile(func=pass_like_sampler, args=(m, seeds, u, v, u + 1, v + 1))
+    assert torch.allclose(c(m, seeds, u, v, u + 1, v + 1),
+                          pass_like_sampler(m, seeds, u, v, u + 1, v + 1))
