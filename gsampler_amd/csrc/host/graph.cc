@@ -361,10 +361,13 @@ Graph::GraphRelabel(torch::Tensor col_seeds, torch::Tensor row_ids) {
 torch::Tensor Graph::GetValidNodes(torch::Tensor col_seeds,
                                    torch::Tensor row_ids) {
   col_seeds = ids(col_seeds, "col_seeds");
-  // Row ids in CSC order equal the column-sorted COO rows, so both formats
-  // give the same first-occurrence order (src/graph.cc:593-608).
-  if (!csc_) CreateSparseFormat(kCOO);
-  const torch::Tensor& base = csc_ ? csc_->indices : coo_->row;
+  // The frontier order must be the one GraphRelabel produces, because the next
+  // layer's seeds (all_nodes) have to line up with this layer's block sources
+  // (to_dgl_block): both walk the COO rows.  (The reference reads csc.indices
+  // here when a CSC exists, src/graph.cc:593-608, which is another edge order
+  // whenever that CSC was built by sorting a row-sorted COO.)
+  CreateSparseFormat(kCOO);
+  const torch::Tensor& base = coo_->row;
   torch::Tensor rows = mapped_rows(base, row_ids);
   return frontier_for(col_seeds, rows, {}, {}).unique;
 }
