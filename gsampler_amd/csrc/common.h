@@ -64,6 +64,7 @@ constexpr int kWave = 64;
 constexpr int kBlock = 256;  // 4 waves; the default block for flat kernels
 
 inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
+__device__ __forceinline__ int64_t ceil_div_dev(int64_t a, int64_t b) { return (a + b - 1) / b; }
 inline size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
 
 // Carves aligned sub-buffers out of a caller-supplied workspace.

@@ -24,9 +24,11 @@ __device__ __forceinline__ uint64_t home_slot(uint64_t key, uint64_t cap) {
   return ((uint64_t)hash32(key) * cap) >> 32;
 }
 
-// Inserts (key, value), keeping the smallest value per key.  The probe budget
-// (cap) only guards against a table that is too small for its keys.
-__device__ __forceinline__ void table_insert_min(uint64_t* tab, uint64_t cap,
+// Inserts (key, value), keeping the smallest value per key.  Returns whether
+// this value was the smallest seen for the key at that moment (false means a
+// smaller one is already there, for good: values only ever decrease).  The
+// probe budget (cap) only guards against a table too small for its keys.
+__device__ __forceinline__ bool table_insert_min(uint64_t* tab, uint64_t cap,
                                                  uint64_t key, uint64_t value) {
   const uint64_t mine = (key << 32) | value;
   uint64_t slot = home_slot(key, cap);
@@ -35,16 +37,18 @@ __device__ __forceinline__ void table_insert_min(uint64_t* tab, uint64_t cap,
     if (cur == kEmptySlot) {
       cur = atomicCAS((unsigned long long*)(tab + slot),
                       (unsigned long long)kEmptySlot, (unsigned long long)mine);
-      if (cur == kEmptySlot) return;
+      if (cur == kEmptySlot) return true;
     }
     if ((cur >> 32) == key) {
-      // values only ever decrease, so a stale read can only cost an atomic
-      if (cur > mine)
-        atomicMin((unsigned long long*)(tab + slot), (unsigned long long)mine);
-      return;
+      // a stale read can only cost an atomic, never a wrong answer
+      if (cur < mine) return false;
+      const uint64_t old =
+          atomicMin((unsigned long long*)(tab + slot), (unsigned long long)mine);
+      return old >= mine;
     }
     if (++slot == cap) slot = 0;
   }
+  return true;
 }
 
 // Slot that holds `key`, or cap when the key is absent.

@@ -4,32 +4,84 @@
 // Keys of batch b are seeds_b ++ rows_b.  All batches are laid out back to
 // back in one "flat" key space of N = num_seeds + num_rows_keys positions;
 // flat_ptr[b] is where batch b starts.  Batch b owns the open-addressing table
-// slots [2 * flat_ptr[b], 2 * flat_ptr[b+1])  (load factor <= 1/2, linear
-// probing so that a probe sequence stays inside one 128-byte line most of the
-// time).  A slot is one 64-bit word  key << 32 | value  so that insertion with
-// "smallest position wins" is a single 64-bit atomicMin on the slot:
-//   pass 1  insert   value = position of the key inside its batch (min wins)
-//   pass 2  flag     key is a first occurrence  <=>  slot value == own position;
-//                    one ballot bit per key + one count per block
-//   scan of the block counts, unique_ptr from the flags
-//   pass 3  fill     first occurrences write out_unique and replace the slot
-//                    value by their batch-local rank
-//   pass 4  relabel  one lookup per edge row; columns come from the per-seed
-//                    rank array written in pass 3
+// slots of its own (two per key: load factor <= 1/2, linear probing so that a
+// probe run stays inside one 128-byte line most of the time).  A slot is one
+// 64-bit word  key << 32 | value  so that insertion with "smallest position
+// wins" is a single 64-bit atomicMin on the slot.  Every random table access
+// costs a 128-byte line from HBM, so the passes are arranged to touch the table
+// as rarely as possible:
+//   pass 1  insert   value = position of the key inside its batch (min wins);
+//                    a key that loses on arrival can never be a first
+//                    occurrence, so each key also leaves a "may be first" bit
+//   pass 2  flag     only "may be first" keys look the table up again:
+//                    first occurrence <=> slot value == own position;
+//                    one ballot bit per key + one count per tile
+//   scan of the tile counts, unique_ptr from the flags
+//   pass 3  fill     streaming, no table access: first occurrences write
+//                    out_unique and their batch-local rank into rank[position]
+//   pass 4  relabel  one lookup per edge row gives the first position of its
+//                    key, rank[] (a per-batch array that stays in L2) gives the
+//                    label; column labels are rank[] of the seed positions
 #include "common.h"
 #include "hashtable.h"
 #include "scan.h"
 
+#include <cstdlib>
+
 namespace gs {
 
 constexpr int kWordsPerBlock = kBlock / kWave;
+constexpr int kXcds = 8;  // accelerator dies of an MI355X, each with its own L2
+
+// Table slots per key in percent (GS_TABLE_PERCENT, default below) and whether
+// blocks are laid out per die (GS_XCD_REMAP).  Read once.
+struct UniqueTuning {
+  int64_t percent;
+  int remap;
+};
+static UniqueTuning tuning() {
+  static const UniqueTuning t = [] {
+    UniqueTuning r{200, 1};
+    if (const char* e = getenv("GS_TABLE_PERCENT")) r.percent = atoll(e);
+    if (const char* e = getenv("GS_XCD_REMAP")) r.remap = atoi(e);
+    if (r.percent < 110) r.percent = 110;
+    return r;
+  }();
+  return t;
+}
+
+// Slot range of a batch whose keys occupy flat positions [lo, hi): base and
+// capacity grow with the key count at `percent` slots per 100 keys; the + batch
+// term absorbs the rounding so that ranges never overlap.
+__host__ __device__ inline uint64_t table_base_of(int64_t lo, int64_t batch,
+                                                  int64_t percent) {
+  return (uint64_t)(lo * percent / 100 + batch);
+}
+__host__ __device__ inline uint64_t table_cap_of(int64_t n, int64_t percent) {
+  return (uint64_t)(n * percent / 100 + 1);
+}
+
+// Work-group index -> tile of the flat key space.  Consecutive work-groups go
+// to consecutive dies, so die x is given the x-th eighth of the tiles, in
+// order: at any moment each die walks one batch (its keys are contiguous in
+// the flat space) and that batch's table stays in the die's own L2 instead of
+// being pulled into all eight.
+__device__ __forceinline__ int64_t tile_of_block(int64_t num_tiles, int remap) {
+  if (!remap) return blockIdx.x;
+  const int64_t per = (num_tiles + kXcds - 1) / kXcds;
+  return (int64_t)(blockIdx.x % kXcds) * per + blockIdx.x / kXcds;
+}
+static int64_t grid_for_tiles(int64_t num_tiles, int remap) {
+  return remap ? ceil_div(num_tiles, kXcds) * kXcds : num_tiles;
+}
 
 struct UniqueWs {
   int64_t* flat_ptr;      // [B + 1]
-  uint64_t* table;        // [2 N]
-  uint64_t* flags;        // [nblocks * kWordsPerBlock]
-  int64_t* block_off;     // [nblocks + 1]
-  int64_t* seed_rank;     // [S]
+  uint64_t* table;        // [percent/100 * N + B + 2]
+  uint64_t* maybe;        // [tiles * kWordsPerBlock]  "may be first" bits
+  uint64_t* flags;        // [tiles * kWordsPerBlock]  first-occurrence bits
+  int64_t* block_off;     // [tiles + 1]
+  int32_t* rank;          // [N] batch-local rank of a first occurrence, else -1
   void* scan_ws;
   size_t scan_ws_bytes;
   size_t total;
@@ -41,10 +93,11 @@ static UniqueWs carve_unique(void* ws, int64_t S, int64_t E, int64_t B) {
   Carver c(ws);
   UniqueWs w;
   w.flat_ptr = c.take<int64_t>((size_t)B + 1);
-  w.table = c.take<uint64_t>((size_t)(2 * N + 2));
+  w.table = c.take<uint64_t>((size_t)(N * tuning().percent / 100 + B + 2));
+  w.maybe = c.take<uint64_t>((size_t)nblocks * kWordsPerBlock);
   w.flags = c.take<uint64_t>((size_t)nblocks * kWordsPerBlock);
   w.block_off = c.take<int64_t>((size_t)nblocks + 1);
-  w.seed_rank = c.take<int64_t>((size_t)(S > 0 ? S : 1));
+  w.rank = c.take<int32_t>((size_t)(N > 0 ? N : 1));
   w.scan_ws_bytes = scan_workspace_bytes(nblocks + 1);
   w.scan_ws = c.take<char>(w.scan_ws_bytes);
   w.total = c.total();
@@ -53,7 +106,7 @@ static UniqueWs carve_unique(void* ws, int64_t S, int64_t E, int64_t B) {
 
 // Where a flat position lives: batch, position inside the batch, key.
 struct FlatItem {
-  int64_t batch, local, seed_index;  // seed_index = -1 for row keys
+  int64_t batch, local;
   uint64_t key;
   uint64_t table_base, cap;
 };
@@ -62,7 +115,7 @@ __device__ __forceinline__ FlatItem locate(
     int64_t p, const int64_t* __restrict__ flat_ptr, int64_t B,
     const int64_t* __restrict__ seeds, const int64_t* __restrict__ seeds_ptr,
     int64_t S, const int64_t* __restrict__ rows,
-    const int64_t* __restrict__ rows_ptr) {
+    const int64_t* __restrict__ rows_ptr, int64_t percent) {
   FlatItem it;
   it.batch = B == 1 ? 0 : segment_of(flat_ptr, B, p);
   const int64_t fb = flat_ptr[it.batch];
@@ -71,15 +124,13 @@ __device__ __forceinline__ FlatItem locate(
   const int64_t s_hi = seeds_ptr ? seeds_ptr[it.batch + 1] : S;
   const int64_t ns = s_hi - s_lo;
   if (it.local < ns) {
-    it.seed_index = s_lo + it.local;
-    it.key = (uint64_t)seeds[it.seed_index];
+    it.key = (uint64_t)seeds[s_lo + it.local];
   } else {
     const int64_t r_lo = rows_ptr ? rows_ptr[it.batch] : 0;
-    it.seed_index = -1;
     it.key = (uint64_t)rows[r_lo + it.local - ns];
   }
-  it.table_base = 2 * (uint64_t)fb;
-  it.cap = 2 * (uint64_t)(flat_ptr[it.batch + 1] - fb);
+  it.table_base = table_base_of(fb, it.batch, percent);
+  it.cap = table_cap_of(flat_ptr[it.batch + 1] - fb, percent);
   return it;
 }
 
@@ -97,11 +148,21 @@ __global__ __launch_bounds__(kBlock) void unique_insert_kernel(
     const int64_t* __restrict__ flat_ptr, int64_t B,
     const int64_t* __restrict__ seeds, const int64_t* __restrict__ seeds_ptr,
     int64_t S, const int64_t* __restrict__ rows,
-    const int64_t* __restrict__ rows_ptr, int64_t N, uint64_t* table) {
-  const int64_t p = (int64_t)blockIdx.x * kBlock + threadIdx.x;
-  if (p >= N) return;
-  const FlatItem it = locate(p, flat_ptr, B, seeds, seeds_ptr, S, rows, rows_ptr);
-  table_insert_min(table + it.table_base, it.cap, it.key, (uint64_t)it.local);
+    const int64_t* __restrict__ rows_ptr, int64_t N, uint64_t* table,
+    uint64_t* __restrict__ maybe, int64_t percent, int remap) {
+  const int64_t num_tiles = ceil_div_dev(N, kBlock);
+  const int64_t tile = tile_of_block(num_tiles, remap);
+  if (tile >= num_tiles) return;  // uniform per work-group
+  const int64_t p = tile * kBlock + threadIdx.x;
+  bool may_be_first = false;
+  if (p < N) {
+    const FlatItem it =
+        locate(p, flat_ptr, B, seeds, seeds_ptr, S, rows, rows_ptr, percent);
+    may_be_first = table_insert_min(table + it.table_base, it.cap, it.key,
+                                    (uint64_t)it.local);
+  }
+  const uint64_t word = __ballot(may_be_first);
+  if (lane_id() == 0) maybe[tile * kWordsPerBlock + threadIdx.x / kWave] = word;
 }
 
 // Keys looked up here were all inserted, so the slot always exists; slot 0
@@ -117,22 +178,26 @@ __global__ __launch_bounds__(kBlock) void unique_flag_kernel(
     const int64_t* __restrict__ seeds, const int64_t* __restrict__ seeds_ptr,
     int64_t S, const int64_t* __restrict__ rows,
     const int64_t* __restrict__ rows_ptr, int64_t N,
-    const uint64_t* __restrict__ table, uint64_t* __restrict__ flags,
-    int64_t* __restrict__ block_count) {
+    const uint64_t* __restrict__ table, const uint64_t* __restrict__ maybe,
+    uint64_t* __restrict__ flags, int64_t* __restrict__ block_count,
+    int64_t percent, int remap) {
   __shared__ int wave_count[kWordsPerBlock];
-  const int64_t p = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  const int64_t num_tiles = ceil_div_dev(N, kBlock);
+  const int64_t tile = tile_of_block(num_tiles, remap);
+  if (tile >= num_tiles) return;  // uniform per work-group
+  const int64_t p = tile * kBlock + threadIdx.x;
+  const int wave = threadIdx.x / kWave;
   bool first = false;
-  if (p < N) {
+  if (p < N && ((maybe[tile * kWordsPerBlock + wave] >> lane_id()) & 1ull)) {
     const FlatItem it =
-        locate(p, flat_ptr, B, seeds, seeds_ptr, S, rows, rows_ptr);
+        locate(p, flat_ptr, B, seeds, seeds_ptr, S, rows, rows_ptr, percent);
     const uint64_t* tab = table + it.table_base;
     const uint64_t cur = tab[find_slot(tab, it.cap, it.key)];
     first = (uint32_t)cur == (uint32_t)it.local;
   }
   const uint64_t word = __ballot(first);
-  const int wave = threadIdx.x / kWave;
   if (lane_id() == 0) {
-    flags[(int64_t)blockIdx.x * kWordsPerBlock + wave] = word;
+    flags[tile * kWordsPerBlock + wave] = word;
     wave_count[wave] = __popcll(word);
   }
   __syncthreads();
@@ -140,8 +205,8 @@ __global__ __launch_bounds__(kBlock) void unique_flag_kernel(
     int total = 0;
 #pragma unroll
     for (int w = 0; w < kWordsPerBlock; ++w) total += wave_count[w];
-    block_count[blockIdx.x] = total;
-    if (blockIdx.x == gridDim.x - 1) block_count[gridDim.x] = 0;
+    block_count[tile] = total;
+    if (tile == num_tiles - 1) block_count[num_tiles] = 0;
   }
 }
 
@@ -169,52 +234,54 @@ __global__ void unique_ptr_kernel(const int64_t* __restrict__ flat_ptr,
   unique_ptr[b] = rank_before(flat_ptr[b], flags, block_off);
 }
 
+// Streaming: every position writes its rank (or -1); first occurrences also
+// write their key to the frontier.
 __global__ __launch_bounds__(kBlock) void unique_fill_kernel(
     const int64_t* __restrict__ flat_ptr, int64_t B,
     const int64_t* __restrict__ seeds, const int64_t* __restrict__ seeds_ptr,
     int64_t S, const int64_t* __restrict__ rows,
-    const int64_t* __restrict__ rows_ptr, int64_t N, uint64_t* table,
+    const int64_t* __restrict__ rows_ptr, int64_t N,
     const uint64_t* __restrict__ flags, const int64_t* __restrict__ block_off,
     const int64_t* __restrict__ unique_ptr, int64_t* __restrict__ out_unique,
-    int64_t* __restrict__ seed_rank) {
+    int32_t* __restrict__ rank, int64_t percent) {
   const int64_t p = (int64_t)blockIdx.x * kBlock + threadIdx.x;
   if (p >= N) return;
-  const FlatItem it = locate(p, flat_ptr, B, seeds, seeds_ptr, S, rows, rows_ptr);
-  const bool first = (flags[p / kWave] >> (p % kWave)) & 1ull;
-  if (first) {
+  int32_t r = -1;
+  if ((flags[p / kWave] >> (p % kWave)) & 1ull) {
+    const FlatItem it =
+        locate(p, flat_ptr, B, seeds, seeds_ptr, S, rows, rows_ptr, percent);
     const int64_t grank = rank_before(p, flags, block_off);
-    const int64_t lrank = grank - unique_ptr[it.batch];
     out_unique[grank] = (int64_t)it.key;
-    uint64_t* tab = table + it.table_base;
-    // Only the value half changes; concurrent probes compare the key half.
-    tab[find_slot(tab, it.cap, it.key)] = (it.key << 32) | (uint64_t)lrank;
-    if (it.seed_index >= 0) seed_rank[it.seed_index] = lrank;
-  } else if (it.seed_index >= 0) {
-    seed_rank[it.seed_index] = -1;  // repeated seed: resolved by lookup later
+    r = (int32_t)(grank - unique_ptr[it.batch]);
   }
+  rank[p] = r;
 }
 
 __global__ __launch_bounds__(kBlock) void unique_relabel_kernel(
     const int64_t* __restrict__ flat_ptr, int64_t B,
     const int64_t* __restrict__ seeds, const int64_t* __restrict__ rows,
     const int64_t* __restrict__ rows_ptr, int64_t E,
-    const uint64_t* __restrict__ table, const int64_t* __restrict__ seed_rank,
+    const uint64_t* __restrict__ table, const int32_t* __restrict__ rank,
     const int64_t* __restrict__ edge_col, int64_t* __restrict__ out_row,
-    int64_t* __restrict__ out_col) {
-  const int64_t e = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    int64_t* __restrict__ out_col, int64_t percent, int remap) {
+  const int64_t tile = tile_of_block(ceil_div_dev(E, kBlock), remap);
+  const int64_t e = tile * kBlock + threadIdx.x;
   if (e >= E) return;
   const int64_t b = (B == 1 || rows_ptr == nullptr) ? 0 : segment_of(rows_ptr, B, e);
   const int64_t fb = flat_ptr[b];
-  const uint64_t* tab = table + 2 * (uint64_t)fb;
-  const uint64_t cap = 2 * (uint64_t)(flat_ptr[b + 1] - fb);
-  if (out_row) {
-    const uint64_t key = (uint64_t)rows[e];
-    out_row[e] = (int64_t)(uint32_t)tab[find_slot(tab, cap, key)];
-  }
+  const uint64_t* tab = table + table_base_of(fb, b, percent);
+  const uint64_t cap = table_cap_of(flat_ptr[b + 1] - fb, percent);
+  // first position of a key inside the batch -> its rank
+  auto label_of = [&](uint64_t key) -> int64_t {
+    const uint32_t first_local = (uint32_t)tab[find_slot(tab, cap, key)];
+    return (int64_t)rank[fb + first_local];
+  };
+  if (out_row) out_row[e] = label_of((uint64_t)rows[e]);
   if (out_col) {
+    // seed c of batch b sits at flat position c + rows_ptr[b]
     const int64_t c = edge_col[e];
-    int64_t r = seed_rank[c];
-    if (r < 0) r = (int64_t)(uint32_t)tab[find_slot(tab, cap, (uint64_t)seeds[c])];
+    int64_t r = rank[c + (rows_ptr ? rows_ptr[b] : 0)];
+    if (r < 0) r = label_of((uint64_t)seeds[c]);  // a repeated seed
     out_col[e] = r;
   }
 }
@@ -259,6 +326,7 @@ int gs_unique_count(const int64_t* seeds, const int64_t* seeds_ptr,
     return GS_ERR_WORKSPACE;
   }
   hipStream_t s = as_stream(stream);
+  const UniqueTuning tn = tuning();
   const int64_t N = S + E;
   if (N == 0) {
     GS_LAUNCH("unique_clear", s,
@@ -273,19 +341,22 @@ int gs_unique_count(const int64_t* seeds, const int64_t* seeds_ptr,
                                      dim3(kBlock), 0, s>>>(seeds_ptr, S, rows_ptr,
                                                            E, B, w.flat_ptr));
   {
-    const int64_t slots = 2 * N;
+    const int64_t slots = N * tuning().percent / 100 + B + 2;
     int64_t blocks = ceil_div(slots, kBlock * 8);
     GS_LAUNCH("unique_clear", s,
               table_fill_kernel<><<<dim3((unsigned)blocks), dim3(kBlock), 0, s>>>(
                   w.table, slots, kEmptySlot));
   }
   GS_LAUNCH("unique_insert", s,
-            unique_insert_kernel<<<dim3((unsigned)nblocks), dim3(kBlock), 0, s>>>(
-                w.flat_ptr, B, seeds, seeds_ptr, S, rows, rows_ptr, N, w.table));
-  GS_LAUNCH("unique_flag", s,
-            unique_flag_kernel<<<dim3((unsigned)nblocks), dim3(kBlock), 0, s>>>(
+            unique_insert_kernel<<<dim3((unsigned)grid_for_tiles(nblocks, tn.remap)),
+                                   dim3(kBlock), 0, s>>>(
                 w.flat_ptr, B, seeds, seeds_ptr, S, rows, rows_ptr, N, w.table,
-                w.flags, w.block_off));
+                w.maybe, tn.percent, tn.remap));
+  GS_LAUNCH("unique_flag", s,
+            unique_flag_kernel<<<dim3((unsigned)grid_for_tiles(nblocks, tn.remap)),
+                                 dim3(kBlock), 0, s>>>(
+                w.flat_ptr, B, seeds, seeds_ptr, S, rows, rows_ptr, N, w.table,
+                w.maybe, w.flags, w.block_off, tn.percent, tn.remap));
   rc = exclusive_scan_i64(w.block_off, w.block_off, nblocks + 1, w.scan_ws,
                           w.scan_ws_bytes, s);
   if (rc != GS_OK) return rc;
@@ -316,11 +387,12 @@ int gs_unique_fill(const int64_t* seeds, const int64_t* seeds_ptr,
   if (N == 0) return GS_OK;
   GS_REQUIRE(out_unique, "unique_fill: null out_unique");
   hipStream_t s = as_stream(stream);
+  const UniqueTuning tn = tuning();
   const int64_t nblocks = ceil_div(N, kBlock);
   GS_LAUNCH("unique_fill", s,
             unique_fill_kernel<<<dim3((unsigned)nblocks), dim3(kBlock), 0, s>>>(
-                w.flat_ptr, B, seeds, seeds_ptr, S, rows, rows_ptr, N, w.table,
-                w.flags, w.block_off, unique_ptr, out_unique, w.seed_rank));
+                w.flat_ptr, B, seeds, seeds_ptr, S, rows, rows_ptr, N, w.flags,
+                w.block_off, unique_ptr, out_unique, w.rank, tn.percent));
   return GS_OK;
 }
 
@@ -342,12 +414,13 @@ int gs_unique_relabel(const int64_t* seeds, const int64_t* seeds_ptr,
     return GS_ERR_WORKSPACE;
   }
   hipStream_t s = as_stream(stream);
+  const UniqueTuning tn = tuning();
   if (E > 0 && (out_row || out_col)) {
     GS_LAUNCH("unique_relabel", s,
-              unique_relabel_kernel<<<dim3((unsigned)ceil_div(E, kBlock)),
+              unique_relabel_kernel<<<dim3((unsigned)grid_for_tiles(ceil_div(E, kBlock), tn.remap)),
                                       dim3(kBlock), 0, s>>>(
-                  w.flat_ptr, B, seeds, rows, rows_ptr, E, w.table, w.seed_rank,
-                  edge_col, out_row, out_col));
+                  w.flat_ptr, B, seeds, rows, rows_ptr, E, w.table, w.rank,
+                  edge_col, out_row, out_col, tn.percent, tn.remap));
   }
   return GS_OK;
 }
