@@ -59,6 +59,9 @@ def graphsage_step(be, indptr, indices, seeds, ptr, fanouts, seed, call_base):
     return sizes, last
 
 
+CALIBRATION_BYTES = 256 << 20
+
+
 def kernel_bytes(name, sizes):
     """Algorithmic bytes moved by all launches of `name` in one step: the
     compulsory reads and writes of the kernel's interface (hash-table, scratch
@@ -69,11 +72,12 @@ def kernel_bytes(name, sizes):
         total += {
             "sample_uniform": 32 * S + 32 * E,   # seeds, indptr pair, sub_indptr, gather, 3 outputs
             "col_count": 32 * S,                 # seeds, indptr pair, counts
-            "unique_insert": 8 * N,              # keys in
-            "unique_flag": 8 * N + N // 8,       # keys in, flag bits out
-            "unique_fill": 8 * N + 8 * U + 8 * S,  # keys in, frontier + seed ranks out
-            "unique_relabel": 32 * E,            # row key + column id in, row + col out
-            "unique_clear": 16 * N,              # table initialisation
+            "unique_hist": 8 * N,                # keys in
+            "unique_scatter": 16 * N,            # keys in, packed entries out
+            "unique_dedup": 12 * N,              # packed entries in, first positions out
+            "unique_flag": 4 * N + N // 8,       # first positions in, flag bits out
+            "unique_fill": N // 8 + 16 * U + 4 * N,  # flags + first keys in, frontier + ranks out
+            "unique_relabel": 40 * E,            # 2 first positions + 2 ranks + column id in, row + col out
         }.get(name, 0)
     return total
 
@@ -110,6 +114,12 @@ def main():
     torch.cuda.synchronize()
     t_build = time.time() - t0
     fanouts = wl["fanouts"]
+
+    # One plain streaming kernel of known size (reads 256 MiB, writes 256 MiB):
+    # the yardstick that hardware traffic counters of a profiled run are scaled by.
+    yard = torch.zeros(CALIBRATION_BYTES // 8, dtype=torch.int64, device=dev)
+    yard = torch.bitwise_xor(yard, 1)
+    del yard
 
     def step(i):
         return graphsage_step(capi, indptr, indices, seeds, ptr, fanouts, args.seed,
@@ -149,9 +159,14 @@ def main():
     kernels.sort(key=lambda k: -k["total_ms"])
     dom = kernels[0]
     traffic = None
-    tpath = os.path.join(ROOT, "profiles", f"traffic_{args.workload}.json")
+    # measured HBM bytes per launch (hardware counters of a profiled run of this
+    # same command, kept as text: kernel launches fetch write total)
+    tpath = os.path.join(ROOT, "profiles", f"graphsage_{args.workload}_hbm_traffic.txt")
     if os.path.exists(tpath):
-        traffic = json.load(open(tpath)).get(dom["kernel"])
+        for line in open(tpath):
+            f = line.split()
+            if len(f) == 5 and f[0] == dom["kernel"]:
+                traffic = int(f[4])
     roofline = dict(bound="hbm", kernel=dom["kernel"], achieved=round(dom["gbs"], 1),
                     peak=HBM_PEAK_GBS, unit="GB/s", frac=round(dom["gbs"] / HBM_PEAK_GBS, 4),
                     traffic=traffic, avg_launch_ms=round(dom["avg_ms"], 4),

@@ -3,25 +3,33 @@
 //
 // Keys of batch b are seeds_b ++ rows_b.  All batches are laid out back to
 // back in one "flat" key space of N = num_seeds + num_rows_keys positions;
-// flat_ptr[b] is where batch b starts.  Batch b owns the open-addressing table
-// slots of its own (two per key: load factor <= 1/2, linear probing so that a
-// probe run stays inside one 128-byte line most of the time).  A slot is one
-// 64-bit word  key << 32 | value  so that insertion with "smallest position
-// wins" is a single 64-bit atomicMin on the slot.  Every random table access
-// costs a 128-byte line from HBM, so the passes are arranged to touch the table
-// as rarely as possible:
-//   pass 1  insert   value = position of the key inside its batch (min wins);
-//                    a key that loses on arrival can never be a first
-//                    occurrence, so each key also leaves a "may be first" bit
-//   pass 2  flag     only "may be first" keys look the table up again:
-//                    first occurrence <=> slot value == own position;
-//                    one ballot bit per key + one count per tile
-//   scan of the tile counts, unique_ptr from the flags
-//   pass 3  fill     streaming, no table access: first occurrences write
-//                    out_unique and their batch-local rank into rank[position]
-//   pass 4  relabel  one lookup per edge row gives the first position of its
-//                    key, rank[] (a per-batch array that stays in L2) gives the
-//                    label; column labels are rank[] of the seed positions
+// flat_ptr[b] is where batch b starts.
+//
+// A hash table over all keys of a batch does not fit in a die's L2, and every
+// random access to it costs a whole line from HBM.  So the keys of a batch are
+// first partitioned by hash into buckets of about a thousand entries (streaming
+// reads and writes only), and each bucket is then deduplicated by one
+// work-group in an LDS table:
+//   prep     per-batch offsets (flat positions, tiles, buckets); zero counters
+//   hist     per tile of one batch: LDS histogram over the batch's buckets,
+//            one global atomic per non-empty bin
+//   scan     bucket counts -> bucket offsets (bucket ranges of a batch tile its
+//            range of the flat space exactly)
+//   scatter  per tile: reserve a run in every bucket, write  key << 32 | local
+//   dedup    per bucket: LDS table with "smallest position wins" (64-bit
+//            atomicMin on the packed entry), then every entry writes the first
+//            position of its key into first[position]
+//   flag     streaming: position is a first occurrence <=> first[p] == local(p);
+//            one ballot bit per key + one count per tile; scan; unique_ptr
+//   fill     streaming: first occurrences write out_unique and their
+//            batch-local rank into rank[position]
+//   relabel  label of a position = rank[first[position]]: two gathers inside
+//            the batch's own range, which a die's L2 holds
+// The result does not depend on the order in which entries land in a bucket, so
+// the atomics above leave it deterministic.  A bucket with more entries than the
+// LDS table is sure to hold (a hub that repeats thousands of times, a batch too
+// large for kMaxBuckets buckets) is deduplicated by the same work-group in a
+// table in global memory that is private to the bucket.
 #include "common.h"
 #include "hashtable.h"
 #include "scan.h"
@@ -33,180 +41,556 @@ namespace gs {
 constexpr int kWordsPerBlock = kBlock / kWave;
 constexpr int kXcds = 8;  // accelerator dies of an MI355X, each with its own L2
 
-// Table slots per key in percent (GS_TABLE_PERCENT, default below) and whether
-// blocks are laid out per die (GS_XCD_REMAP).  Read once.
+constexpr int kPartItems = 16;                    // keys per thread and tile
+constexpr int kPartTile = kBlock * kPartItems;    // keys per partition tile
+constexpr int kMaxBuckets = 2048;                 // buckets per batch (LDS bins)
+constexpr int kLdsSlots = 4096;                   // dedup table, 32 KB of LDS
+constexpr int kLdsMaxEntries = kLdsSlots * 3 / 4; // bucket sizes the LDS table takes
+
+// Average entries per bucket (GS_BUCKET_KEYS) and whether work-groups are laid
+// out per die (GS_XCD_REMAP).  Read once.
 struct UniqueTuning {
-  int64_t percent;
+  int64_t bucket_keys;
   int remap;
 };
 static UniqueTuning tuning() {
   static const UniqueTuning t = [] {
-    UniqueTuning r{200, 1};
-    if (const char* e = getenv("GS_TABLE_PERCENT")) r.percent = atoll(e);
+    UniqueTuning r{1024, 1};
+    if (const char* e = getenv("GS_BUCKET_KEYS")) r.bucket_keys = atoll(e);
     if (const char* e = getenv("GS_XCD_REMAP")) r.remap = atoi(e);
-    if (r.percent < 110) r.percent = 110;
+    if (r.bucket_keys < 64) r.bucket_keys = 64;
+    if (r.bucket_keys > kLdsMaxEntries) r.bucket_keys = kLdsMaxEntries;
     return r;
   }();
   return t;
 }
 
-// Slot range of a batch whose keys occupy flat positions [lo, hi): base and
-// capacity grow with the key count at `percent` slots per 100 keys; the + batch
-// term absorbs the rounding so that ranges never overlap.
-__host__ __device__ inline uint64_t table_base_of(int64_t lo, int64_t batch,
-                                                  int64_t percent) {
-  return (uint64_t)(lo * percent / 100 + batch);
-}
-__host__ __device__ inline uint64_t table_cap_of(int64_t n, int64_t percent) {
-  return (uint64_t)(n * percent / 100 + 1);
-}
-
-// Work-group index -> tile of the flat key space.  Consecutive work-groups go
-// to consecutive dies, so die x is given the x-th eighth of the tiles, in
-// order: at any moment each die walks one batch (its keys are contiguous in
-// the flat space) and that batch's table stays in the die's own L2 instead of
-// being pulled into all eight.
-__device__ __forceinline__ int64_t tile_of_block(int64_t num_tiles, int remap) {
+// Work-group index -> unit of work (tile or bucket).  Consecutive work-groups
+// go to consecutive dies, so die x is given the x-th eighth of the units, in
+// order: at any moment each die walks one batch, and what that batch touches
+// (its open bucket lines, its first[] and rank[] ranges) stays in the die's own
+// L2 instead of being pulled into all eight.
+__device__ __forceinline__ int64_t unit_of_block(int64_t num_units, int remap) {
   if (!remap) return blockIdx.x;
-  const int64_t per = (num_tiles + kXcds - 1) / kXcds;
+  const int64_t per = (num_units + kXcds - 1) / kXcds;
   return (int64_t)(blockIdx.x % kXcds) * per + blockIdx.x / kXcds;
 }
-static int64_t grid_for_tiles(int64_t num_tiles, int remap) {
-  return remap ? ceil_div(num_tiles, kXcds) * kXcds : num_tiles;
+static int64_t grid_for_units(int64_t num_units, int remap) {
+  return remap ? ceil_div(num_units, kXcds) * kXcds : num_units;
 }
 
 struct UniqueWs {
-  int64_t* flat_ptr;      // [B + 1]
-  uint64_t* table;        // [percent/100 * N + B + 2]
-  uint64_t* maybe;        // [tiles * kWordsPerBlock]  "may be first" bits
-  uint64_t* flags;        // [tiles * kWordsPerBlock]  first-occurrence bits
-  int64_t* block_off;     // [tiles + 1]
+  int64_t* flat_ptr;      // [B + 1] first flat position of a batch
+  int64_t* tile_ptr;      // [B + 1] first partition tile of a batch
+  int64_t* bucket_ptr;    // [B + 1] first bucket of a batch
+  int64_t* bucket_cnt;    // [max_buckets + 1] entries per bucket
+  int64_t* bucket_off;    // [max_buckets + 1] first entry of a bucket
+  uint64_t* packed;       // [N] key << 32 | local, grouped by bucket
+  uint32_t* first;        // [N] local position of the first occurrence
+  uint64_t* spill;        // [2 N + max_buckets + 1] tables of oversize buckets
+  uint64_t* flags;        // [blocks * kWordsPerBlock] first-occurrence bits
+  int64_t* block_off;     // [blocks + 1]
   int32_t* rank;          // [N] batch-local rank of a first occurrence, else -1
   void* scan_ws;
   size_t scan_ws_bytes;
+  int64_t max_tiles, max_buckets;
   size_t total;
 };
 
 static UniqueWs carve_unique(void* ws, int64_t S, int64_t E, int64_t B) {
   const int64_t N = S + E;
-  const int64_t nblocks = ceil_div(N > 0 ? N : 1, kBlock);
+  const int64_t n1 = N > 0 ? N : 1;
+  const int64_t nblocks = ceil_div(n1, kBlock);
   Carver c(ws);
   UniqueWs w;
+  // sum over batches of ceil(n_b / x) <= N / x + B
+  w.max_tiles = N / kPartTile + B;
+  w.max_buckets = N / tuning().bucket_keys + B;
   w.flat_ptr = c.take<int64_t>((size_t)B + 1);
-  w.table = c.take<uint64_t>((size_t)(N * tuning().percent / 100 + B + 2));
-  w.maybe = c.take<uint64_t>((size_t)nblocks * kWordsPerBlock);
+  w.tile_ptr = c.take<int64_t>((size_t)B + 1);
+  w.bucket_ptr = c.take<int64_t>((size_t)B + 1);
+  w.bucket_cnt = c.take<int64_t>((size_t)w.max_buckets + 1);
+  w.bucket_off = c.take<int64_t>((size_t)w.max_buckets + 1);
+  w.packed = c.take<uint64_t>((size_t)n1);
+  w.first = c.take<uint32_t>((size_t)n1);
+  w.spill = c.take<uint64_t>((size_t)(2 * n1 + w.max_buckets + 1));
   w.flags = c.take<uint64_t>((size_t)nblocks * kWordsPerBlock);
   w.block_off = c.take<int64_t>((size_t)nblocks + 1);
-  w.rank = c.take<int32_t>((size_t)(N > 0 ? N : 1));
+  w.rank = c.take<int32_t>((size_t)n1);
   w.scan_ws_bytes = scan_workspace_bytes(nblocks + 1);
   w.scan_ws = c.take<char>(w.scan_ws_bytes);
   w.total = c.total();
   return w;
 }
 
-// Where a flat position lives: batch, position inside the batch, key.
-struct FlatItem {
-  int64_t batch, local;
-  uint64_t key;
-  uint64_t table_base, cap;
+// The caller's view of the keys.
+struct Keys {
+  const int64_t* seeds;
+  const int64_t* seeds_ptr;  // null: one batch
+  int64_t S;
+  const int64_t* rows;
+  const int64_t* rows_ptr;   // null: one batch
+  int64_t E;
+  int64_t B;
 };
 
-__device__ __forceinline__ FlatItem locate(
-    int64_t p, const int64_t* __restrict__ flat_ptr, int64_t B,
-    const int64_t* __restrict__ seeds, const int64_t* __restrict__ seeds_ptr,
-    int64_t S, const int64_t* __restrict__ rows,
-    const int64_t* __restrict__ rows_ptr, int64_t percent) {
-  FlatItem it;
-  it.batch = B == 1 ? 0 : segment_of(flat_ptr, B, p);
-  const int64_t fb = flat_ptr[it.batch];
-  it.local = p - fb;
-  const int64_t s_lo = seeds_ptr ? seeds_ptr[it.batch] : 0;
-  const int64_t s_hi = seeds_ptr ? seeds_ptr[it.batch + 1] : S;
-  const int64_t ns = s_hi - s_lo;
-  if (it.local < ns) {
-    it.key = (uint64_t)seeds[s_lo + it.local];
-  } else {
-    const int64_t r_lo = rows_ptr ? rows_ptr[it.batch] : 0;
-    it.key = (uint64_t)rows[r_lo + it.local - ns];
+__device__ __forceinline__ int64_t seeds_lo(const Keys& k, int64_t b) {
+  return k.seeds_ptr ? k.seeds_ptr[b] : (b == 0 ? 0 : k.S);
+}
+__device__ __forceinline__ int64_t rows_lo(const Keys& k, int64_t b) {
+  return k.rows_ptr ? k.rows_ptr[b] : (b == 0 ? 0 : k.E);
+}
+
+// Key at position `local` of batch b (whose seeds are [s_lo, s_lo + ns)).
+__device__ __forceinline__ uint64_t key_at(const Keys& k, int64_t s_lo,
+                                           int64_t ns, int64_t r_lo,
+                                           int64_t local) {
+  return (uint64_t)(local < ns ? k.seeds[s_lo + local] : k.rows[r_lo + local - ns]);
+}
+
+// Bucket of a key among the `buckets` of its batch: the high bits of the hash.
+__device__ __forceinline__ uint32_t bucket_of(uint64_t key, uint32_t buckets) {
+  return (uint32_t)(((uint64_t)hash32(key) * buckets) >> 32);
+}
+// Home slot inside a bucket's table: bits the bucket choice did not use.
+__device__ __forceinline__ uint32_t slot_hash(uint64_t key) {
+  return (uint32_t)((key * 0xC2B2AE3D27D4EB4Full) >> 29);
+}
+
+// ---------------------------------------------------------------- prep
+// Block 0 walks the batches (B + 1 offsets each for flat positions, tiles and
+// buckets); every block zeroes its share of the bucket counters.
+__global__ __launch_bounds__(kBlock) void unique_prep_kernel(
+    Keys k, int64_t bucket_keys, int64_t* __restrict__ flat_ptr,
+    int64_t* __restrict__ tile_ptr, int64_t* __restrict__ bucket_ptr,
+    int64_t* __restrict__ bucket_cnt, int64_t max_buckets) {
+  for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i <= max_buckets;
+       i += (int64_t)gridDim.x * kBlock)
+    bucket_cnt[i] = 0;
+  if (blockIdx.x != 0) return;
+  __shared__ int64_t smem[kBlock / kWave + 1];
+  int64_t tile_carry = 0, bucket_carry = 0;
+  for (int64_t base = 0; base <= k.B; base += kBlock) {
+    const int64_t b = base + threadIdx.x;
+    int64_t tiles = 0, buckets = 0;
+    if (b <= k.B) {
+      const int64_t lo = seeds_lo(k, b) + rows_lo(k, b);
+      flat_ptr[b] = lo;
+      if (b < k.B) {
+        const int64_t n = seeds_lo(k, b + 1) + rows_lo(k, b + 1) - lo;
+        tiles = ceil_div_dev(n, kPartTile);
+        buckets = ceil_div_dev(n, bucket_keys);
+        if (buckets > kMaxBuckets) buckets = kMaxBuckets;
+      }
+    }
+    int64_t total;
+    const int64_t t_ex = block_exclusive_sum(tiles, smem, &total);
+    if (b <= k.B) tile_ptr[b] = tile_carry + t_ex;
+    tile_carry += total;
+    __syncthreads();
+    const int64_t b_ex = block_exclusive_sum(buckets, smem, &total);
+    if (b <= k.B) bucket_ptr[b] = bucket_carry + b_ex;
+    bucket_carry += total;
+    __syncthreads();
   }
-  it.table_base = table_base_of(fb, it.batch, percent);
-  it.cap = table_cap_of(flat_ptr[it.batch + 1] - fb, percent);
-  return it;
 }
 
-__global__ void unique_flat_ptr_kernel(const int64_t* seeds_ptr, int64_t S,
-                                       const int64_t* rows_ptr, int64_t E,
-                                       int64_t B, int64_t* flat_ptr) {
-  const int64_t b = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (b > B) return;
-  const int64_t s = seeds_ptr ? seeds_ptr[b] : (b == 0 ? 0 : S);
-  const int64_t r = rows_ptr ? rows_ptr[b] : (b == 0 ? 0 : E);
-  flat_ptr[b] = s + r;
+// One partition tile: which batch, which keys.
+struct TileInfo {
+  int64_t batch, fb, n, s_lo, ns, r_lo;
+  int64_t begin, end;    // local positions [begin, end)
+  int64_t first_bucket;
+  uint32_t buckets;
+};
+
+__device__ __forceinline__ bool tile_info(
+    const Keys& k, int64_t tile, const int64_t* __restrict__ flat_ptr,
+    const int64_t* __restrict__ tile_ptr, const int64_t* __restrict__ bucket_ptr,
+    TileInfo* t) {
+  if (tile >= tile_ptr[k.B]) return false;
+  const int64_t b = k.B == 1 ? 0 : segment_of(tile_ptr, k.B, tile);
+  t->batch = b;
+  t->fb = flat_ptr[b];
+  t->n = flat_ptr[b + 1] - t->fb;
+  t->s_lo = seeds_lo(k, b);
+  t->ns = seeds_lo(k, b + 1) - t->s_lo;
+  t->r_lo = rows_lo(k, b);
+  t->begin = (tile - tile_ptr[b]) * kPartTile;
+  t->end = t->begin + kPartTile < t->n ? t->begin + kPartTile : t->n;
+  t->first_bucket = bucket_ptr[b];
+  t->buckets = (uint32_t)(bucket_ptr[b + 1] - t->first_bucket);
+  return true;
 }
 
-__global__ __launch_bounds__(kBlock) void unique_insert_kernel(
-    const int64_t* __restrict__ flat_ptr, int64_t B,
-    const int64_t* __restrict__ seeds, const int64_t* __restrict__ seeds_ptr,
-    int64_t S, const int64_t* __restrict__ rows,
-    const int64_t* __restrict__ rows_ptr, int64_t N, uint64_t* table,
-    uint64_t* __restrict__ maybe, int64_t percent, int remap) {
-  const int64_t num_tiles = ceil_div_dev(N, kBlock);
-  const int64_t tile = tile_of_block(num_tiles, remap);
-  if (tile >= num_tiles) return;  // uniform per work-group
-  const int64_t p = tile * kBlock + threadIdx.x;
-  bool may_be_first = false;
-  if (p < N) {
-    const FlatItem it =
-        locate(p, flat_ptr, B, seeds, seeds_ptr, S, rows, rows_ptr, percent);
-    may_be_first = table_insert_min(table + it.table_base, it.cap, it.key,
-                                    (uint64_t)it.local);
+// ---------------------------------------------------------------- hist
+__global__ __launch_bounds__(kBlock) void unique_hist_kernel(
+    Keys k, const int64_t* __restrict__ flat_ptr,
+    const int64_t* __restrict__ tile_ptr, const int64_t* __restrict__ bucket_ptr,
+    int64_t* bucket_cnt, int64_t max_tiles, int remap) {
+  __shared__ uint32_t hist[kMaxBuckets];
+  TileInfo t;
+  if (!tile_info(k, unit_of_block(max_tiles, remap), flat_ptr, tile_ptr,
+                 bucket_ptr, &t))
+    return;  // uniform per work-group
+  if (t.buckets == 1) {  // nothing to choose
+    if (threadIdx.x == 0)
+      atomicAdd((unsigned long long*)&bucket_cnt[t.first_bucket],
+                (unsigned long long)(t.end - t.begin));
+    return;
   }
-  const uint64_t word = __ballot(may_be_first);
-  if (lane_id() == 0) maybe[tile * kWordsPerBlock + threadIdx.x / kWave] = word;
-}
-
-// Keys looked up here were all inserted, so the slot always exists; slot 0
-// stands in if a caller passed inconsistent pointer arrays.
-__device__ __forceinline__ uint64_t find_slot(const uint64_t* tab, uint64_t cap,
-                                              uint64_t key) {
-  const uint64_t slot = table_find(tab, cap, key);
-  return slot < cap ? slot : 0;
-}
-
-__global__ __launch_bounds__(kBlock) void unique_flag_kernel(
-    const int64_t* __restrict__ flat_ptr, int64_t B,
-    const int64_t* __restrict__ seeds, const int64_t* __restrict__ seeds_ptr,
-    int64_t S, const int64_t* __restrict__ rows,
-    const int64_t* __restrict__ rows_ptr, int64_t N,
-    const uint64_t* __restrict__ table, const uint64_t* __restrict__ maybe,
-    uint64_t* __restrict__ flags, int64_t* __restrict__ block_count,
-    int64_t percent, int remap) {
-  __shared__ int wave_count[kWordsPerBlock];
-  const int64_t num_tiles = ceil_div_dev(N, kBlock);
-  const int64_t tile = tile_of_block(num_tiles, remap);
-  if (tile >= num_tiles) return;  // uniform per work-group
-  const int64_t p = tile * kBlock + threadIdx.x;
-  const int wave = threadIdx.x / kWave;
-  bool first = false;
-  if (p < N && ((maybe[tile * kWordsPerBlock + wave] >> lane_id()) & 1ull)) {
-    const FlatItem it =
-        locate(p, flat_ptr, B, seeds, seeds_ptr, S, rows, rows_ptr, percent);
-    const uint64_t* tab = table + it.table_base;
-    const uint64_t cur = tab[find_slot(tab, it.cap, it.key)];
-    first = (uint32_t)cur == (uint32_t)it.local;
+  for (uint32_t i = threadIdx.x; i < t.buckets; i += kBlock) hist[i] = 0;
+  __syncthreads();
+  for (int64_t l = t.begin + threadIdx.x; l < t.end; l += kBlock)
+    atomicAdd(&hist[bucket_of(key_at(k, t.s_lo, t.ns, t.r_lo, l), t.buckets)], 1u);
+  __syncthreads();
+  for (uint32_t i = threadIdx.x; i < t.buckets; i += kBlock) {
+    const uint32_t c = hist[i];
+    if (c)
+      atomicAdd((unsigned long long*)&bucket_cnt[t.first_bucket + i],
+                (unsigned long long)c);
   }
-  const uint64_t word = __ballot(first);
-  if (lane_id() == 0) {
-    flags[tile * kWordsPerBlock + wave] = word;
-    wave_count[wave] = __popcll(word);
+}
+
+// Exclusive scan of the bucket counts by one work-group (there are about
+// N / 1024 of them).  off[total_buckets] = N closes the last bucket.
+__global__ __launch_bounds__(kBlock) void unique_bucket_scan_kernel(
+    const int64_t* __restrict__ bucket_ptr, int64_t B,
+    const int64_t* __restrict__ bucket_cnt, int64_t* __restrict__ bucket_off) {
+  __shared__ int64_t smem[kBlock / kWave + 1];
+  const int64_t n = bucket_ptr[B] + 1;
+  int64_t carry = 0;
+  constexpr int kPer = 8;
+  for (int64_t base = 0; base < n; base += kBlock * kPer) {
+    const int64_t i0 = base + (int64_t)threadIdx.x * kPer;
+    int64_t v[kPer], sum = 0;
+#pragma unroll
+    for (int j = 0; j < kPer; ++j) {
+      v[j] = i0 + j < n ? bucket_cnt[i0 + j] : 0;
+      sum += v[j];
+    }
+    int64_t total;
+    int64_t run = carry + block_exclusive_sum(sum, smem, &total);
+#pragma unroll
+    for (int j = 0; j < kPer; ++j) {
+      if (i0 + j < n) bucket_off[i0 + j] = run;
+      run += v[j];
+    }
+    carry += total;
+    __syncthreads();
+  }
+}
+
+// ---------------------------------------------------------------- scatter
+// bucket_cnt doubles as the reservation counter: a tile that brings c entries
+// to a bucket takes the c places below the counter's current value.  The tile
+// is first ordered by bucket in LDS so that every run leaves as one contiguous
+// write instead of one line per entry.
+__global__ __launch_bounds__(kBlock) void unique_scatter_kernel(
+    Keys k, const int64_t* __restrict__ flat_ptr,
+    const int64_t* __restrict__ tile_ptr, const int64_t* __restrict__ bucket_ptr,
+    int64_t* bucket_cnt, const int64_t* __restrict__ bucket_off,
+    uint64_t* __restrict__ packed, int64_t max_tiles, int remap) {
+  __shared__ uint32_t hist[kMaxBuckets];   // counts, then offsets inside the tile
+  __shared__ uint32_t run_at[kMaxBuckets]; // where the tile's run starts, relative to the batch
+  __shared__ uint64_t stage[kPartTile];
+  __shared__ uint32_t scan_smem[kBlock / kWave + 1];
+  TileInfo t;
+  if (!tile_info(k, unit_of_block(max_tiles, remap), flat_ptr, tile_ptr,
+                 bucket_ptr, &t))
+    return;  // uniform per work-group
+  uint64_t* out = packed + t.fb;
+  if (t.buckets == 1) {  // the bucket is the batch, in order
+    for (int64_t l = t.begin + threadIdx.x; l < t.end; l += kBlock)
+      out[l] = (key_at(k, t.s_lo, t.ns, t.r_lo, l) << 32) | (uint64_t)l;
+    return;
+  }
+  for (uint32_t i = threadIdx.x; i < t.buckets; i += kBlock) hist[i] = 0;
+  __syncthreads();
+  uint32_t key[kPartItems], place[kPartItems];
+#pragma unroll
+  for (int i = 0; i < kPartItems; ++i) {
+    const int64_t l = t.begin + i * kBlock + threadIdx.x;
+    key[i] = l < t.end ? (uint32_t)key_at(k, t.s_lo, t.ns, t.r_lo, l) : 0u;
+  }
+#pragma unroll
+  for (int i = 0; i < kPartItems; ++i)
+    if (t.begin + i * kBlock + threadIdx.x < t.end)
+      place[i] = atomicAdd(&hist[bucket_of(key[i], t.buckets)], 1u);
+  __syncthreads();
+  {
+    constexpr int kBins = kMaxBuckets / kBlock;
+    const uint32_t bin0 = threadIdx.x * kBins;
+    uint32_t c[kBins], sum = 0;
+#pragma unroll
+    for (int j = 0; j < kBins; ++j) {
+      c[j] = bin0 + j < t.buckets ? hist[bin0 + j] : 0u;
+      sum += c[j];
+    }
+    uint32_t total;
+    uint32_t run = block_exclusive_sum(sum, scan_smem, &total);
+#pragma unroll
+    for (int j = 0; j < kBins; ++j) {
+      if (bin0 + j < t.buckets) hist[bin0 + j] = run;
+      run += c[j];
+      if (c[j]) {
+        const int64_t g = t.first_bucket + bin0 + j;
+        const int64_t before = (int64_t)atomicAdd(
+            (unsigned long long*)&bucket_cnt[g],
+            (unsigned long long)(-(int64_t)c[j]));
+        run_at[bin0 + j] = (uint32_t)(bucket_off[g] - t.fb + before - c[j]);
+      }
+    }
   }
   __syncthreads();
-  if (threadIdx.x == 0) {
-    int total = 0;
 #pragma unroll
-    for (int w = 0; w < kWordsPerBlock; ++w) total += wave_count[w];
-    block_count[tile] = total;
-    if (tile == num_tiles - 1) block_count[num_tiles] = 0;
+  for (int i = 0; i < kPartItems; ++i) {
+    const int64_t l = t.begin + i * kBlock + threadIdx.x;
+    if (l < t.end)
+      stage[hist[bucket_of(key[i], t.buckets)] + place[i]] =
+          ((uint64_t)key[i] << 32) | (uint64_t)l;
+  }
+  __syncthreads();
+  const uint32_t count = (uint32_t)(t.end - t.begin);
+  for (uint32_t j = threadIdx.x; j < count; j += kBlock) {
+    const uint64_t e = stage[j];
+    const uint32_t bk = bucket_of(e >> 32, t.buckets);
+    out[run_at[bk] + (j - hist[bk])] = e;
+  }
+}
+
+// ---------------------------------------------------------------- dedup
+__device__ __forceinline__ void lds_insert_min(uint64_t* tab, uint32_t mask,
+                                               uint64_t entry) {
+  const uint64_t key = entry >> 32;
+  uint32_t slot = slot_hash(key) & mask;
+  for (;;) {
+    uint64_t cur = tab[slot];
+    if (cur == kEmptySlot) {
+      cur = atomicCAS((unsigned long long*)&tab[slot],
+                      (unsigned long long)kEmptySlot, (unsigned long long)entry);
+      if (cur == kEmptySlot) return;
+    }
+    if ((cur >> 32) == key) {
+      if (cur > entry)
+        atomicMin((unsigned long long*)&tab[slot], (unsigned long long)entry);
+      return;
+    }
+    slot = (slot + 1) & mask;
+  }
+}
+
+__device__ __forceinline__ uint32_t lds_first_of(const uint64_t* tab,
+                                                 uint32_t mask, uint64_t key) {
+  uint32_t slot = slot_hash(key) & mask;
+  for (;;) {
+    const uint64_t cur = tab[slot];
+    if ((cur >> 32) == key) return (uint32_t)cur;
+    slot = (slot + 1) & mask;
+  }
+}
+
+// Table in global memory, used by one work-group inside one kernel: loads must
+// not be served from the compute unit's own cache.
+__device__ __forceinline__ uint64_t load_l2(const uint64_t* p) {
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+__device__ __forceinline__ void spill_insert_min(uint64_t* tab, uint64_t cap,
+                                                 uint64_t entry) {
+  const uint64_t key = entry >> 32;
+  uint64_t slot = ((uint64_t)slot_hash(key) * cap) >> 32;
+  for (uint64_t probes = 0; probes < cap; ++probes) {
+    uint64_t cur = load_l2(tab + slot);
+    if (cur == kEmptySlot) {
+      cur = atomicCAS((unsigned long long*)(tab + slot),
+                      (unsigned long long)kEmptySlot, (unsigned long long)entry);
+      if (cur == kEmptySlot) return;
+    }
+    if ((cur >> 32) == key) {
+      if (cur > entry)
+        atomicMin((unsigned long long*)(tab + slot), (unsigned long long)entry);
+      return;
+    }
+    if (++slot == cap) slot = 0;
+  }
+}
+
+__device__ __forceinline__ uint32_t spill_first_of(const uint64_t* tab,
+                                                   uint64_t cap, uint64_t key) {
+  uint64_t slot = ((uint64_t)slot_hash(key) * cap) >> 32;
+  for (uint64_t probes = 0; probes < cap; ++probes) {
+    const uint64_t cur = load_l2(tab + slot);
+    if ((cur >> 32) == key) return (uint32_t)cur;
+    if (++slot == cap) slot = 0;
+  }
+  return 0;  // not reached: every key looked up was inserted
+}
+
+// Same as lds_insert_min for a bucket that may hold more distinct keys than the
+// table takes: counts the slots it claims and raises *overflow instead of
+// filling the table up.
+__device__ __forceinline__ void lds_insert_min_counted(uint64_t* tab,
+                                                       uint32_t mask,
+                                                       uint64_t entry,
+                                                       uint32_t* distinct,
+                                                       volatile uint32_t* overflow) {
+  const uint64_t key = entry >> 32;
+  uint32_t slot = slot_hash(key) & mask;
+  for (;;) {
+    uint64_t cur = tab[slot];
+    if (cur == kEmptySlot) {
+      cur = atomicCAS((unsigned long long*)&tab[slot],
+                      (unsigned long long)kEmptySlot, (unsigned long long)entry);
+      if (cur == kEmptySlot) {
+        if (atomicAdd(distinct, 1u) >= (uint32_t)kLdsMaxEntries) *overflow = 1u;
+        return;
+      }
+    }
+    if ((cur >> 32) == key) {
+      if (cur > entry)
+        atomicMin((unsigned long long*)&tab[slot], (unsigned long long)entry);
+      return;
+    }
+    slot = (slot + 1) & mask;
+  }
+}
+
+__global__ __launch_bounds__(kBlock) void unique_dedup_kernel(
+    const int64_t* __restrict__ flat_ptr, const int64_t* __restrict__ bucket_ptr,
+    int64_t B, const int64_t* __restrict__ bucket_off,
+    const uint64_t* __restrict__ packed, uint64_t* spill,
+    uint32_t* __restrict__ first, int64_t max_buckets, int remap) {
+  __shared__ uint64_t tab[kLdsSlots];
+  __shared__ uint32_t distinct;
+  __shared__ uint32_t overflow;
+  const int64_t g = unit_of_block(max_buckets, remap);
+  if (g >= bucket_ptr[B]) return;  // uniform per work-group
+  const int64_t lo = bucket_off[g], hi = bucket_off[g + 1];
+  const int64_t n = hi - lo;
+  if (n == 0) return;
+  const int64_t b = B == 1 ? 0 : segment_of(bucket_ptr, B, g);
+  uint32_t* first_b = first + flat_ptr[b];
+  // table of two slots per entry, a power of two, at most kLdsSlots
+  uint32_t slots = 256;
+  while (slots < kLdsSlots && (int64_t)slots < 2 * n) slots <<= 1;
+  const uint32_t mask = slots - 1;
+  for (uint32_t i = threadIdx.x; i < slots; i += kBlock) tab[i] = kEmptySlot;
+  if (threadIdx.x == 0) distinct = overflow = 0;
+  __syncthreads();
+  constexpr int kKeep = kLdsMaxEntries / kBlock;
+  if (n <= kLdsMaxEntries) {
+    // sure to fit; the thread's entries stay in registers between the phases
+    uint64_t mine[kKeep];
+#pragma unroll
+    for (int j = 0; j < kKeep; ++j) {
+      const int64_t i = lo + j * kBlock + threadIdx.x;
+      mine[j] = i < hi ? packed[i] : kEmptySlot;
+    }
+#pragma unroll
+    for (int j = 0; j < kKeep; ++j)
+      if (mine[j] != kEmptySlot) lds_insert_min(tab, mask, mine[j]);
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < kKeep; ++j)
+      if (mine[j] != kEmptySlot)
+        first_b[(uint32_t)mine[j]] = lds_first_of(tab, mask, mine[j] >> 32);
+    return;
+  }
+  // Many entries: fine for the LDS table while few of them are distinct (a hub
+  // that repeats thousands of times), so try, and count.
+  for (int64_t i = lo + threadIdx.x; i < hi; i += kBlock) {
+    if (*(volatile uint32_t*)&overflow) break;
+    lds_insert_min_counted(tab, mask, packed[i], &distinct, &overflow);
+  }
+  __syncthreads();
+  if (!overflow) {
+    for (int64_t i = lo + threadIdx.x; i < hi; i += kBlock) {
+      const uint64_t e = packed[i];
+      first_b[(uint32_t)e] = lds_first_of(tab, mask, e >> 32);
+    }
+    return;
+  }
+  // too many distinct keys: a private table in global memory, two slots per entry
+  uint64_t* gt = spill + 2 * lo + g;
+  const uint64_t cap = (uint64_t)(2 * n + 1);
+  for (uint64_t i = threadIdx.x; i < cap; i += kBlock) gt[i] = kEmptySlot;
+  __threadfence();
+  __syncthreads();
+  for (int64_t i = lo + threadIdx.x; i < hi; i += kBlock)
+    spill_insert_min(gt, cap, packed[i]);
+  __threadfence();
+  __syncthreads();
+  for (int64_t i = lo + threadIdx.x; i < hi; i += kBlock) {
+    const uint64_t e = packed[i];
+    first_b[(uint32_t)e] = spill_first_of(gt, cap, e >> 32);
+  }
+}
+
+// ---------------------------------------------------------------- flag
+// The streaming passes below work in chunks of kBlock consecutive positions,
+// one chunk per wave at a time, lane l taking positions l, l + 64, ...: four
+// coalesced rows whose ballots are the chunk's four flag words.
+
+// A value that is the same in every lane, moved to scalar registers so that
+// what is computed from it (the batch search) runs on the scalar unit.
+__device__ __forceinline__ int64_t wave_uniform(int64_t v) {
+  const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v);
+  const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)((uint64_t)v >> 32));
+  return (int64_t)(((uint64_t)hi << 32) | lo);
+}
+
+// Batches that the items [x0, x1] of an offsets array touch.
+struct BatchSpan {
+  int64_t lo, hi;
+};
+__device__ __forceinline__ BatchSpan batch_span(const int64_t* __restrict__ ptr,
+                                                int64_t B, int64_t x0, int64_t x1) {
+  BatchSpan s{0, 0};
+  if (B > 1) {
+    s.lo = segment_of(ptr, B, wave_uniform(x0));
+    s.hi = segment_of(ptr, B, wave_uniform(x1));
+  }
+  return s;
+}
+__device__ __forceinline__ int64_t batch_in_span(const int64_t* __restrict__ ptr,
+                                                 const BatchSpan& s, int64_t x) {
+  return s.lo == s.hi ? s.lo : s.lo + segment_of(ptr + s.lo, s.hi - s.lo + 1, x);
+}
+
+constexpr int kChunksPerWave = 4;
+
+__global__ __launch_bounds__(kBlock) void unique_flag_kernel(
+    const int64_t* __restrict__ flat_ptr, int64_t B, int64_t N,
+    const uint32_t* __restrict__ first, uint64_t* __restrict__ flags,
+    int64_t* __restrict__ block_count) {
+  const int64_t num_chunks = ceil_div_dev(N, kBlock);
+  const int64_t wave = (int64_t)blockIdx.x * kWordsPerBlock + threadIdx.x / kWave;
+  const int lane = lane_id();
+  for (int c = 0; c < kChunksPerWave; ++c) {
+    const int64_t chunk = wave * kChunksPerWave + c;
+    if (chunk >= num_chunks) return;
+    const int64_t p0 = chunk * kBlock;
+    const int64_t p_last = p0 + kBlock - 1 < N ? p0 + kBlock - 1 : N - 1;
+    const BatchSpan span = batch_span(flat_ptr, B, p0, p_last);
+    uint64_t word[kWordsPerBlock];
+#pragma unroll
+    for (int j = 0; j < kWordsPerBlock; ++j) {
+      const int64_t p = p0 + j * kWave + lane;
+      bool is_first = false;
+      if (p < N)
+        is_first = (int64_t)first[p] == p - flat_ptr[batch_in_span(flat_ptr, span, p)];
+      word[j] = __ballot(is_first);
+    }
+    if (lane == 0) {
+      int total = 0;
+#pragma unroll
+      for (int j = 0; j < kWordsPerBlock; ++j) {
+        flags[chunk * kWordsPerBlock + j] = word[j];
+        total += __popcll(word[j]);
+      }
+      block_count[chunk] = total;
+      if (chunk == num_chunks - 1) block_count[num_chunks] = 0;
+    }
   }
 }
 
@@ -234,55 +618,71 @@ __global__ void unique_ptr_kernel(const int64_t* __restrict__ flat_ptr,
   unique_ptr[b] = rank_before(flat_ptr[b], flags, block_off);
 }
 
+// ---------------------------------------------------------------- fill
 // Streaming: every position writes its rank (or -1); first occurrences also
 // write their key to the frontier.
 __global__ __launch_bounds__(kBlock) void unique_fill_kernel(
-    const int64_t* __restrict__ flat_ptr, int64_t B,
-    const int64_t* __restrict__ seeds, const int64_t* __restrict__ seeds_ptr,
-    int64_t S, const int64_t* __restrict__ rows,
-    const int64_t* __restrict__ rows_ptr, int64_t N,
+    Keys k, const int64_t* __restrict__ flat_ptr, int64_t N,
     const uint64_t* __restrict__ flags, const int64_t* __restrict__ block_off,
     const int64_t* __restrict__ unique_ptr, int64_t* __restrict__ out_unique,
-    int32_t* __restrict__ rank, int64_t percent) {
-  const int64_t p = (int64_t)blockIdx.x * kBlock + threadIdx.x;
-  if (p >= N) return;
-  int32_t r = -1;
-  if ((flags[p / kWave] >> (p % kWave)) & 1ull) {
-    const FlatItem it =
-        locate(p, flat_ptr, B, seeds, seeds_ptr, S, rows, rows_ptr, percent);
-    const int64_t grank = rank_before(p, flags, block_off);
-    out_unique[grank] = (int64_t)it.key;
-    r = (int32_t)(grank - unique_ptr[it.batch]);
+    int32_t* __restrict__ rank) {
+  const int64_t num_chunks = ceil_div_dev(N, kBlock);
+  const int64_t wave = (int64_t)blockIdx.x * kWordsPerBlock + threadIdx.x / kWave;
+  const int lane = lane_id();
+  for (int c = 0; c < kChunksPerWave; ++c) {
+    const int64_t chunk = wave_uniform(wave * kChunksPerWave + c);
+    if (chunk >= num_chunks) return;
+    const int64_t p0 = chunk * kBlock;
+    const int64_t p_last = p0 + kBlock - 1 < N ? p0 + kBlock - 1 : N - 1;
+    const BatchSpan span = batch_span(flat_ptr, k.B, p0, p_last);
+    int64_t before = block_off[chunk];
+#pragma unroll
+    for (int j = 0; j < kWordsPerBlock; ++j) {
+      const uint64_t word = flags[chunk * kWordsPerBlock + j];
+      const int64_t p = p0 + j * kWave + lane;
+      if (p < N) {
+        int32_t r = -1;
+        if ((word >> lane) & 1ull) {
+          const int64_t b = batch_in_span(flat_ptr, span, p);
+          const int64_t s_lo = seeds_lo(k, b);
+          const uint64_t key = key_at(k, s_lo, seeds_lo(k, b + 1) - s_lo,
+                                      rows_lo(k, b), p - flat_ptr[b]);
+          const int64_t grank = before + __popcll(word & ((1ull << lane) - 1));
+          out_unique[grank] = (int64_t)key;
+          r = (int32_t)(grank - unique_ptr[b]);
+        }
+        rank[p] = r;
+      }
+      before += __popcll(word);
+    }
   }
-  rank[p] = r;
 }
 
+// ---------------------------------------------------------------- relabel
+constexpr int kRelabelItems = 4;
+constexpr int kRelabelTile = kBlock * kRelabelItems;
+
 __global__ __launch_bounds__(kBlock) void unique_relabel_kernel(
-    const int64_t* __restrict__ flat_ptr, int64_t B,
-    const int64_t* __restrict__ seeds, const int64_t* __restrict__ rows,
-    const int64_t* __restrict__ rows_ptr, int64_t E,
-    const uint64_t* __restrict__ table, const int32_t* __restrict__ rank,
+    Keys k, const int64_t* __restrict__ flat_ptr,
+    const uint32_t* __restrict__ first, const int32_t* __restrict__ rank,
     const int64_t* __restrict__ edge_col, int64_t* __restrict__ out_row,
-    int64_t* __restrict__ out_col, int64_t percent, int remap) {
-  const int64_t tile = tile_of_block(ceil_div_dev(E, kBlock), remap);
-  const int64_t e = tile * kBlock + threadIdx.x;
-  if (e >= E) return;
-  const int64_t b = (B == 1 || rows_ptr == nullptr) ? 0 : segment_of(rows_ptr, B, e);
-  const int64_t fb = flat_ptr[b];
-  const uint64_t* tab = table + table_base_of(fb, b, percent);
-  const uint64_t cap = table_cap_of(flat_ptr[b + 1] - fb, percent);
-  // first position of a key inside the batch -> its rank
-  auto label_of = [&](uint64_t key) -> int64_t {
-    const uint32_t first_local = (uint32_t)tab[find_slot(tab, cap, key)];
-    return (int64_t)rank[fb + first_local];
-  };
-  if (out_row) out_row[e] = label_of((uint64_t)rows[e]);
-  if (out_col) {
+    int64_t* __restrict__ out_col, int remap) {
+  const int64_t e0 =
+      unit_of_block(ceil_div_dev(k.E, kRelabelTile), remap) * kRelabelTile;
+  if (e0 >= k.E) return;
+  const int64_t e_last = e0 + kRelabelTile - 1 < k.E ? e0 + kRelabelTile - 1 : k.E - 1;
+  const BatchSpan span = batch_span(k.rows_ptr, k.B, e0, e_last);
+#pragma unroll
+  for (int i = 0; i < kRelabelItems; ++i) {
+    const int64_t e = e0 + i * kBlock + threadIdx.x;
+    if (e >= k.E) break;
+    const int64_t b = k.B == 1 ? 0 : batch_in_span(k.rows_ptr, span, e);
+    const int64_t fb = flat_ptr[b];
+    // row key e of batch b sits at flat position
+    //   fb + (seeds of b) + (e - rows_ptr[b])  =  e + seeds_ptr[b + 1]
+    if (out_row) out_row[e] = rank[fb + first[e + seeds_lo(k, b + 1)]];
     // seed c of batch b sits at flat position c + rows_ptr[b]
-    const int64_t c = edge_col[e];
-    int64_t r = rank[c + (rows_ptr ? rows_ptr[b] : 0)];
-    if (r < 0) r = label_of((uint64_t)seeds[c]);  // a repeated seed
-    out_col[e] = r;
+    if (out_col) out_col[e] = rank[fb + first[edge_col[e] + rows_lo(k, b)]];
   }
 }
 
@@ -297,6 +697,15 @@ static int check_unique_args(const int64_t* seeds, const int64_t* seeds_ptr,
              "unique: seeds_ptr and rows_ptr must both be given or both be null");
   GS_REQUIRE(seeds_ptr != nullptr || B == 1,
              "unique: %lld batches need seeds_ptr / rows_ptr", (long long)B);
+  return GS_OK;
+}
+
+static int check_workspace(const UniqueWs& w, const void* workspace,
+                           size_t workspace_bytes) {
+  if (workspace == nullptr || workspace_bytes < w.total) {
+    set_error("unique workspace too small: %zu < %zu", workspace_bytes, w.total);
+    return GS_ERR_WORKSPACE;
+  }
   return GS_OK;
 }
 
@@ -321,42 +730,50 @@ int gs_unique_count(const int64_t* seeds, const int64_t* seeds_ptr,
   if (rc != GS_OK) return rc;
   GS_REQUIRE(unique_ptr, "unique_count: null unique_ptr");
   UniqueWs w = carve_unique(workspace, S, E, B);
-  if (workspace == nullptr || workspace_bytes < w.total) {
-    set_error("unique workspace too small: %zu < %zu", workspace_bytes, w.total);
-    return GS_ERR_WORKSPACE;
-  }
+  if ((rc = check_workspace(w, workspace, workspace_bytes)) != GS_OK) return rc;
   hipStream_t s = as_stream(stream);
   const UniqueTuning tn = tuning();
   const int64_t N = S + E;
   if (N == 0) {
-    GS_LAUNCH("unique_clear", s,
+    GS_LAUNCH("unique_prep", s,
               table_fill_kernel<><<<dim3((unsigned)ceil_div(B + 1, kBlock)),
                                     dim3(kBlock), 0, s>>>((uint64_t*)unique_ptr,
                                                           B + 1, 0ull));
     return GS_OK;
   }
+  const Keys k{seeds, seeds_ptr, S, rows, rows_ptr, E, B};
   const int64_t nblocks = ceil_div(N, kBlock);
-  GS_LAUNCH("unique_flat_ptr", s,
-            unique_flat_ptr_kernel<<<dim3((unsigned)ceil_div(B + 1, kBlock)),
-                                     dim3(kBlock), 0, s>>>(seeds_ptr, S, rows_ptr,
-                                                           E, B, w.flat_ptr));
   {
-    const int64_t slots = N * tuning().percent / 100 + B + 2;
-    int64_t blocks = ceil_div(slots, kBlock * 8);
-    GS_LAUNCH("unique_clear", s,
-              table_fill_kernel<><<<dim3((unsigned)blocks), dim3(kBlock), 0, s>>>(
-                  w.table, slots, kEmptySlot));
+    int64_t blocks = ceil_div(w.max_buckets + 1, kBlock * 4);
+    if (blocks > 1024) blocks = 1024;
+    GS_LAUNCH("unique_prep", s,
+              unique_prep_kernel<<<dim3((unsigned)blocks), dim3(kBlock), 0, s>>>(
+                  k, tn.bucket_keys, w.flat_ptr, w.tile_ptr, w.bucket_ptr,
+                  w.bucket_cnt, w.max_buckets));
   }
-  GS_LAUNCH("unique_insert", s,
-            unique_insert_kernel<<<dim3((unsigned)grid_for_tiles(nblocks, tn.remap)),
-                                   dim3(kBlock), 0, s>>>(
-                w.flat_ptr, B, seeds, seeds_ptr, S, rows, rows_ptr, N, w.table,
-                w.maybe, tn.percent, tn.remap));
+  const dim3 tile_grid((unsigned)grid_for_units(w.max_tiles, tn.remap));
+  GS_LAUNCH("unique_hist", s,
+            unique_hist_kernel<<<tile_grid, dim3(kBlock), 0, s>>>(
+                k, w.flat_ptr, w.tile_ptr, w.bucket_ptr, w.bucket_cnt,
+                w.max_tiles, tn.remap));
+  GS_LAUNCH("unique_bucket_scan", s,
+            unique_bucket_scan_kernel<<<dim3(1), dim3(kBlock), 0, s>>>(
+                w.bucket_ptr, B, w.bucket_cnt, w.bucket_off));
+  GS_LAUNCH("unique_scatter", s,
+            unique_scatter_kernel<<<tile_grid, dim3(kBlock), 0, s>>>(
+                k, w.flat_ptr, w.tile_ptr, w.bucket_ptr, w.bucket_cnt,
+                w.bucket_off, w.packed, w.max_tiles, tn.remap));
+  GS_LAUNCH("unique_dedup", s,
+            unique_dedup_kernel<<<dim3((unsigned)grid_for_units(w.max_buckets,
+                                                                tn.remap)),
+                                  dim3(kBlock), 0, s>>>(
+                w.flat_ptr, w.bucket_ptr, B, w.bucket_off, w.packed, w.spill,
+                w.first, w.max_buckets, tn.remap));
   GS_LAUNCH("unique_flag", s,
-            unique_flag_kernel<<<dim3((unsigned)grid_for_tiles(nblocks, tn.remap)),
+            unique_flag_kernel<<<dim3((unsigned)ceil_div(
+                                     nblocks, kWordsPerBlock * kChunksPerWave)),
                                  dim3(kBlock), 0, s>>>(
-                w.flat_ptr, B, seeds, seeds_ptr, S, rows, rows_ptr, N, w.table,
-                w.maybe, w.flags, w.block_off, tn.percent, tn.remap));
+                w.flat_ptr, B, N, w.first, w.flags, w.block_off));
   rc = exclusive_scan_i64(w.block_off, w.block_off, nblocks + 1, w.scan_ws,
                           w.scan_ws_bytes, s);
   if (rc != GS_OK) return rc;
@@ -379,20 +796,19 @@ int gs_unique_fill(const int64_t* seeds, const int64_t* seeds_ptr,
   if (rc != GS_OK) return rc;
   GS_REQUIRE(unique_ptr, "unique_fill: null unique_ptr");
   UniqueWs w = carve_unique(workspace, S, E, B);
-  if (workspace == nullptr || workspace_bytes < w.total) {
-    set_error("unique workspace too small: %zu < %zu", workspace_bytes, w.total);
-    return GS_ERR_WORKSPACE;
-  }
+  if ((rc = check_workspace(w, workspace, workspace_bytes)) != GS_OK) return rc;
   const int64_t N = S + E;
   if (N == 0) return GS_OK;
   GS_REQUIRE(out_unique, "unique_fill: null out_unique");
   hipStream_t s = as_stream(stream);
-  const UniqueTuning tn = tuning();
-  const int64_t nblocks = ceil_div(N, kBlock);
+  const Keys k{seeds, seeds_ptr, S, rows, rows_ptr, E, B};
   GS_LAUNCH("unique_fill", s,
-            unique_fill_kernel<<<dim3((unsigned)nblocks), dim3(kBlock), 0, s>>>(
-                w.flat_ptr, B, seeds, seeds_ptr, S, rows, rows_ptr, N, w.flags,
-                w.block_off, unique_ptr, out_unique, w.rank, tn.percent));
+            unique_fill_kernel<<<dim3((unsigned)ceil_div(
+                                     ceil_div(N, kBlock),
+                                     kWordsPerBlock * kChunksPerWave)),
+                                 dim3(kBlock), 0, s>>>(
+                k, w.flat_ptr, N, w.flags, w.block_off, unique_ptr, out_unique,
+                w.rank));
   return GS_OK;
 }
 
@@ -409,18 +825,17 @@ int gs_unique_relabel(const int64_t* seeds, const int64_t* seeds_ptr,
   GS_REQUIRE(out_col == nullptr || edge_col != nullptr,
              "unique_relabel: out_col needs edge_col");
   UniqueWs w = carve_unique(workspace, S, E, B);
-  if (workspace == nullptr || workspace_bytes < w.total) {
-    set_error("unique workspace too small: %zu < %zu", workspace_bytes, w.total);
-    return GS_ERR_WORKSPACE;
-  }
+  if ((rc = check_workspace(w, workspace, workspace_bytes)) != GS_OK) return rc;
   hipStream_t s = as_stream(stream);
   const UniqueTuning tn = tuning();
   if (E > 0 && (out_row || out_col)) {
+    const Keys k{seeds, seeds_ptr, S, rows, rows_ptr, E, B};
     GS_LAUNCH("unique_relabel", s,
-              unique_relabel_kernel<<<dim3((unsigned)grid_for_tiles(ceil_div(E, kBlock), tn.remap)),
+              unique_relabel_kernel<<<dim3((unsigned)grid_for_units(
+                                          ceil_div(E, kRelabelTile), tn.remap)),
                                       dim3(kBlock), 0, s>>>(
-                  w.flat_ptr, B, seeds, rows, rows_ptr, E, w.table, w.rank,
-                  edge_col, out_row, out_col, tn.percent, tn.remap));
+                  k, w.flat_ptr, w.first, w.rank, edge_col, out_row, out_col,
+                  tn.remap));
   }
   return GS_OK;
 }

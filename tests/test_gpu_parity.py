@@ -132,6 +132,52 @@ def test_unique_relabel_batched_parity(B, id_range):
                 orc.unique_relabel(seeds, rows, sp, rp, edge_col))
 
 
+def test_unique_relabel_hubs_and_ragged_batches():
+    """A few ids that repeat thousands of times (buckets far above the average
+    size), batches from empty to tens of thousands of keys."""
+    rng = np.random.default_rng(11)
+    r_sizes = np.array([0, 1, 40000, 3, 0, 25000, 9000, 2, 60000, 0, 500])
+    B = r_sizes.size
+    s_sizes = rng.integers(1, 50, size=B)
+    s_sizes[4] = 0                      # a batch with nothing at all
+    sp = np.concatenate([[0], np.cumsum(s_sizes)])
+    rp = np.concatenate([[0], np.cumsum(r_sizes)])
+    seeds = rng.integers(0, 10**6, size=sp[-1])
+    rows = rng.integers(0, 10**6, size=rp[-1])
+    hub = rng.random(rows.size) < 0.5
+    rows[hub] = rng.choice([7, 123456, 999999], size=int(hub.sum()))
+    edge_col = np.concatenate(
+        [rng.integers(sp[b], max(sp[b + 1], sp[b] + 1), size=r_sizes[b]) for b in range(B)]
+    ).astype(np.int64)
+    edge_col = np.minimum(edge_col, max(sp[-1] - 1, 0))
+    assert_same(capi.unique_relabel(T(seeds), T(rows), T(sp), T(rp), T(edge_col)),
+                orc.unique_relabel(seeds, rows, sp, rp, edge_col))
+
+
+def test_unique_relabel_many_tiny_batches():
+    rng = np.random.default_rng(12)
+    B = 3000
+    s_sizes = rng.integers(0, 3, size=B)
+    r_sizes = rng.integers(0, 6, size=B)
+    sp = np.concatenate([[0], np.cumsum(s_sizes)])
+    rp = np.concatenate([[0], np.cumsum(r_sizes)])
+    seeds = rng.integers(0, 20, size=sp[-1])
+    rows = rng.integers(0, 20, size=rp[-1])
+    assert_same(capi.unique_relabel(T(seeds), T(rows), T(sp), T(rp)),
+                orc.unique_relabel(seeds, rows, sp, rp))
+
+
+def test_unique_relabel_one_huge_batch():
+    """More keys in one batch than its buckets can take at the usual size: every
+    bucket is deduplicated in global memory."""
+    rng = np.random.default_rng(13)
+    seeds = rng.integers(0, 3 * 10**6, size=1000)
+    rows = rng.integers(0, 3 * 10**6, size=7 * 10**6)
+    edge_col = rng.integers(0, 1000, size=rows.size)
+    assert_same(capi.unique_relabel(T(seeds), T(rows), edge_col=T(edge_col)),
+                orc.unique_relabel(seeds, rows, edge_col=edge_col))
+
+
 def test_graphsage_layers_end_to_end():
     """Three fused slice+sample + unique/relabel layers on an R-MAT graph, super-batch
     of 8, compared with the oracle layer by layer."""
