@@ -10,7 +10,11 @@
 // first partitioned by hash into buckets of about a thousand entries (streaming
 // reads and writes only), and each bucket is then deduplicated by one
 // work-group in an LDS table:
-//   prep     per-batch offsets (flat positions, tiles, buckets); zero counters
+//   prep     per-batch record (where its keys, tiles and buckets start); zero
+//            the bucket counters
+//   units    batch of every tile, bucket and chunk of positions, so that a
+//            work-group finds its work with two dependent loads instead of a
+//            binary search
 //   hist     per tile of one batch: LDS histogram over the batch's buckets,
 //            one global atomic per non-empty bin
 //   scan     bucket counts -> bucket offsets (bucket ranges of a batch tile its
@@ -79,45 +83,70 @@ static int64_t grid_for_units(int64_t num_units, int remap) {
   return remap ? ceil_div(num_units, kXcds) * kXcds : num_units;
 }
 
+// What a work-group needs to know about a batch, in one aligned record.
+struct alignas(16) BatchInfo {
+  int64_t fb;        // first flat position
+  int64_t n;         // keys (seeds + rows)
+  int64_t s_lo, ns;  // its seeds: seeds[s_lo .. s_lo + ns)
+  int64_t r_lo;      // its rows start at rows[r_lo]
+  int64_t tile0;     // first partition tile
+  int64_t bucket0;   // first bucket
+  int64_t buckets;   // number of buckets
+};
+
+constexpr int kRelabelItems = 4;
+constexpr int kRelabelTile = kBlock * kRelabelItems;
+
 struct UniqueWs {
+  BatchInfo* batch;       // [B]
   int64_t* flat_ptr;      // [B + 1] first flat position of a batch
   int64_t* tile_ptr;      // [B + 1] first partition tile of a batch
   int64_t* bucket_ptr;    // [B + 1] first bucket of a batch
+  int32_t* tile_batch;    // [max_tiles] batch of a tile, -1 past the last one
+  int32_t* bucket_batch;  // [max_buckets] batch of a bucket, -1 past the last one
+  int32_t* chunk_batch;   // [chunks + 1] batch of the first position of a chunk
+  int32_t* etile_batch;   // [edge tiles + 1] batch of the first edge of a tile
   int64_t* bucket_cnt;    // [max_buckets + 1] entries per bucket
   int64_t* bucket_off;    // [max_buckets + 1] first entry of a bucket
   uint64_t* packed;       // [N] key << 32 | local, grouped by bucket
   uint32_t* first;        // [N] local position of the first occurrence
   uint64_t* spill;        // [2 N + max_buckets + 1] tables of oversize buckets
-  uint64_t* flags;        // [blocks * kWordsPerBlock] first-occurrence bits
-  int64_t* block_off;     // [blocks + 1]
+  uint64_t* flags;        // [chunks * kWordsPerBlock] first-occurrence bits
+  int64_t* block_off;     // [chunks + 1]
   int32_t* rank;          // [N] batch-local rank of a first occurrence, else -1
   void* scan_ws;
   size_t scan_ws_bytes;
-  int64_t max_tiles, max_buckets;
+  int64_t max_tiles, max_buckets, chunks, etiles;
   size_t total;
 };
 
 static UniqueWs carve_unique(void* ws, int64_t S, int64_t E, int64_t B) {
   const int64_t N = S + E;
   const int64_t n1 = N > 0 ? N : 1;
-  const int64_t nblocks = ceil_div(n1, kBlock);
   Carver c(ws);
   UniqueWs w;
   // sum over batches of ceil(n_b / x) <= N / x + B
   w.max_tiles = N / kPartTile + B;
   w.max_buckets = N / tuning().bucket_keys + B;
+  w.chunks = ceil_div(n1, kBlock);
+  w.etiles = ceil_div(E > 0 ? E : 1, kRelabelTile);
+  w.batch = c.take<BatchInfo>((size_t)B);
   w.flat_ptr = c.take<int64_t>((size_t)B + 1);
   w.tile_ptr = c.take<int64_t>((size_t)B + 1);
   w.bucket_ptr = c.take<int64_t>((size_t)B + 1);
+  w.tile_batch = c.take<int32_t>((size_t)w.max_tiles);
+  w.bucket_batch = c.take<int32_t>((size_t)w.max_buckets);
+  w.chunk_batch = c.take<int32_t>((size_t)w.chunks + 1);
+  w.etile_batch = c.take<int32_t>((size_t)w.etiles + 1);
   w.bucket_cnt = c.take<int64_t>((size_t)w.max_buckets + 1);
   w.bucket_off = c.take<int64_t>((size_t)w.max_buckets + 1);
   w.packed = c.take<uint64_t>((size_t)n1);
   w.first = c.take<uint32_t>((size_t)n1);
   w.spill = c.take<uint64_t>((size_t)(2 * n1 + w.max_buckets + 1));
-  w.flags = c.take<uint64_t>((size_t)nblocks * kWordsPerBlock);
-  w.block_off = c.take<int64_t>((size_t)nblocks + 1);
+  w.flags = c.take<uint64_t>((size_t)w.chunks * kWordsPerBlock);
+  w.block_off = c.take<int64_t>((size_t)w.chunks + 1);
   w.rank = c.take<int32_t>((size_t)n1);
-  w.scan_ws_bytes = scan_workspace_bytes(nblocks + 1);
+  w.scan_ws_bytes = scan_workspace_bytes(w.chunks + 1);
   w.scan_ws = c.take<char>(w.scan_ws_bytes);
   w.total = c.total();
   return w;
@@ -158,12 +187,13 @@ __device__ __forceinline__ uint32_t slot_hash(uint64_t key) {
 }
 
 // ---------------------------------------------------------------- prep
-// Block 0 walks the batches (B + 1 offsets each for flat positions, tiles and
-// buckets); every block zeroes its share of the bucket counters.
+// Block 0 walks the batches; every block zeroes its share of the bucket
+// counters.
 __global__ __launch_bounds__(kBlock) void unique_prep_kernel(
-    Keys k, int64_t bucket_keys, int64_t* __restrict__ flat_ptr,
-    int64_t* __restrict__ tile_ptr, int64_t* __restrict__ bucket_ptr,
-    int64_t* __restrict__ bucket_cnt, int64_t max_buckets) {
+    Keys k, int64_t bucket_keys, BatchInfo* __restrict__ batch,
+    int64_t* __restrict__ flat_ptr, int64_t* __restrict__ tile_ptr,
+    int64_t* __restrict__ bucket_ptr, int64_t* __restrict__ bucket_cnt,
+    int64_t max_buckets) {
   for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i <= max_buckets;
        i += (int64_t)gridDim.x * kBlock)
     bucket_cnt[i] = 0;
@@ -172,81 +202,129 @@ __global__ __launch_bounds__(kBlock) void unique_prep_kernel(
   int64_t tile_carry = 0, bucket_carry = 0;
   for (int64_t base = 0; base <= k.B; base += kBlock) {
     const int64_t b = base + threadIdx.x;
-    int64_t tiles = 0, buckets = 0;
+    BatchInfo info{};
+    int64_t tiles = 0;
     if (b <= k.B) {
-      const int64_t lo = seeds_lo(k, b) + rows_lo(k, b);
-      flat_ptr[b] = lo;
+      info.s_lo = seeds_lo(k, b);
+      info.r_lo = rows_lo(k, b);
+      info.fb = info.s_lo + info.r_lo;
+      flat_ptr[b] = info.fb;
       if (b < k.B) {
-        const int64_t n = seeds_lo(k, b + 1) + rows_lo(k, b + 1) - lo;
-        tiles = ceil_div_dev(n, kPartTile);
-        buckets = ceil_div_dev(n, bucket_keys);
-        if (buckets > kMaxBuckets) buckets = kMaxBuckets;
+        info.ns = seeds_lo(k, b + 1) - info.s_lo;
+        info.n = info.ns + rows_lo(k, b + 1) - info.r_lo;
+        tiles = ceil_div_dev(info.n, kPartTile);
+        info.buckets = ceil_div_dev(info.n, bucket_keys);
+        if (info.buckets > kMaxBuckets) info.buckets = kMaxBuckets;
       }
     }
     int64_t total;
-    const int64_t t_ex = block_exclusive_sum(tiles, smem, &total);
-    if (b <= k.B) tile_ptr[b] = tile_carry + t_ex;
+    info.tile0 = tile_carry + block_exclusive_sum(tiles, smem, &total);
     tile_carry += total;
     __syncthreads();
-    const int64_t b_ex = block_exclusive_sum(buckets, smem, &total);
-    if (b <= k.B) bucket_ptr[b] = bucket_carry + b_ex;
+    info.bucket0 = bucket_carry + block_exclusive_sum(info.buckets, smem, &total);
     bucket_carry += total;
     __syncthreads();
+    if (b <= k.B) {
+      tile_ptr[b] = info.tile0;
+      bucket_ptr[b] = info.bucket0;
+    }
+    if (b < k.B) batch[b] = info;
+  }
+}
+
+// ---------------------------------------------------------------- units
+// One search per tile, bucket, chunk of positions and tile of edges, all in
+// parallel here, instead of one at the start of every work-group later.
+__global__ __launch_bounds__(kBlock) void unique_units_kernel(
+    Keys k, int64_t N, const int64_t* __restrict__ flat_ptr,
+    const int64_t* __restrict__ tile_ptr, const int64_t* __restrict__ bucket_ptr,
+    int64_t max_tiles, int64_t max_buckets, int64_t chunks, int64_t etiles,
+    int32_t* __restrict__ tile_batch, int32_t* __restrict__ bucket_batch,
+    int32_t* __restrict__ chunk_batch, int32_t* __restrict__ etile_batch) {
+  int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  const int64_t B = k.B;
+  if (i < max_tiles) {
+    tile_batch[i] = i < tile_ptr[B] ? (int32_t)segment_of(tile_ptr, B, i) : -1;
+    return;
+  }
+  i -= max_tiles;
+  if (i < max_buckets) {
+    bucket_batch[i] = i < bucket_ptr[B] ? (int32_t)segment_of(bucket_ptr, B, i) : -1;
+    return;
+  }
+  i -= max_buckets;
+  if (i <= chunks) {
+    int64_t p = i * kBlock;
+    if (p > N - 1) p = N - 1;
+    chunk_batch[i] = (int32_t)segment_of(flat_ptr, B, p);
+    return;
+  }
+  i -= chunks + 1;
+  if (i <= etiles) {
+    int64_t e = i * kRelabelTile;
+    if (e > k.E - 1) e = k.E - 1;
+    etile_batch[i] =
+        (k.rows_ptr && k.E > 0) ? (int32_t)segment_of(k.rows_ptr, B, e) : 0;
   }
 }
 
 // One partition tile: which batch, which keys.
 struct TileInfo {
-  int64_t batch, fb, n, s_lo, ns, r_lo;
-  int64_t begin, end;    // local positions [begin, end)
-  int64_t first_bucket;
-  uint32_t buckets;
+  BatchInfo b;
+  int64_t begin, end;  // local positions [begin, end)
 };
 
-__device__ __forceinline__ bool tile_info(
-    const Keys& k, int64_t tile, const int64_t* __restrict__ flat_ptr,
-    const int64_t* __restrict__ tile_ptr, const int64_t* __restrict__ bucket_ptr,
-    TileInfo* t) {
-  if (tile >= tile_ptr[k.B]) return false;
-  const int64_t b = k.B == 1 ? 0 : segment_of(tile_ptr, k.B, tile);
-  t->batch = b;
-  t->fb = flat_ptr[b];
-  t->n = flat_ptr[b + 1] - t->fb;
-  t->s_lo = seeds_lo(k, b);
-  t->ns = seeds_lo(k, b + 1) - t->s_lo;
-  t->r_lo = rows_lo(k, b);
-  t->begin = (tile - tile_ptr[b]) * kPartTile;
-  t->end = t->begin + kPartTile < t->n ? t->begin + kPartTile : t->n;
-  t->first_bucket = bucket_ptr[b];
-  t->buckets = (uint32_t)(bucket_ptr[b + 1] - t->first_bucket);
+__device__ __forceinline__ bool tile_info(int64_t tile,
+                                          const int32_t* __restrict__ tile_batch,
+                                          const BatchInfo* __restrict__ batch,
+                                          TileInfo* t) {
+  const int32_t b = tile_batch[tile];
+  if (b < 0) return false;
+  t->b = batch[b];
+  t->begin = (tile - t->b.tile0) * kPartTile;
+  t->end = t->begin + kPartTile < t->b.n ? t->begin + kPartTile : t->b.n;
   return true;
+}
+
+__device__ __forceinline__ uint64_t key_at(const Keys& k, const BatchInfo& b,
+                                           int64_t local) {
+  return key_at(k, b.s_lo, b.ns, b.r_lo, local);
 }
 
 // ---------------------------------------------------------------- hist
 __global__ __launch_bounds__(kBlock) void unique_hist_kernel(
-    Keys k, const int64_t* __restrict__ flat_ptr,
-    const int64_t* __restrict__ tile_ptr, const int64_t* __restrict__ bucket_ptr,
-    int64_t* bucket_cnt, int64_t max_tiles, int remap) {
+    Keys k, const int32_t* __restrict__ tile_batch,
+    const BatchInfo* __restrict__ batch, int64_t* bucket_cnt, int64_t max_tiles,
+    int remap) {
   __shared__ uint32_t hist[kMaxBuckets];
+  const int64_t tile = unit_of_block(max_tiles, remap);
+  if (tile >= max_tiles) return;
   TileInfo t;
-  if (!tile_info(k, unit_of_block(max_tiles, remap), flat_ptr, tile_ptr,
-                 bucket_ptr, &t))
-    return;  // uniform per work-group
-  if (t.buckets == 1) {  // nothing to choose
+  if (!tile_info(tile, tile_batch, batch, &t)) return;  // uniform per work-group
+  const uint32_t buckets = (uint32_t)t.b.buckets;
+  if (buckets == 1) {  // nothing to choose
     if (threadIdx.x == 0)
-      atomicAdd((unsigned long long*)&bucket_cnt[t.first_bucket],
+      atomicAdd((unsigned long long*)&bucket_cnt[t.b.bucket0],
                 (unsigned long long)(t.end - t.begin));
     return;
   }
-  for (uint32_t i = threadIdx.x; i < t.buckets; i += kBlock) hist[i] = 0;
+  uint32_t key[kPartItems];
+#pragma unroll
+  for (int i = 0; i < kPartItems; ++i) {  // all loads in flight before any use
+    const int64_t l = t.begin + i * kBlock + threadIdx.x;
+    key[i] = l < t.end ? (uint32_t)key_at(k, t.b, l) : 0u;
+  }
+  for (uint32_t i = threadIdx.x; i < buckets; i += kBlock) hist[i] = 0;
   __syncthreads();
-  for (int64_t l = t.begin + threadIdx.x; l < t.end; l += kBlock)
-    atomicAdd(&hist[bucket_of(key_at(k, t.s_lo, t.ns, t.r_lo, l), t.buckets)], 1u);
+#pragma unroll
+  for (int i = 0; i < kPartItems; ++i)
+    if (t.begin + i * kBlock + threadIdx.x < t.end)
+      atomicAdd(&hist[bucket_of(key[i], buckets)], 1u);
   __syncthreads();
-  for (uint32_t i = threadIdx.x; i < t.buckets; i += kBlock) {
+  for (uint32_t i = threadIdx.x; i < buckets; i += kBlock) {
     const uint32_t c = hist[i];
     if (c)
-      atomicAdd((unsigned long long*)&bucket_cnt[t.first_bucket + i],
+      atomicAdd((unsigned long long*)&bucket_cnt[t.b.bucket0 + i],
                 (unsigned long long)c);
   }
 }
@@ -286,59 +364,65 @@ __global__ __launch_bounds__(kBlock) void unique_bucket_scan_kernel(
 // is first ordered by bucket in LDS so that every run leaves as one contiguous
 // write instead of one line per entry.
 __global__ __launch_bounds__(kBlock) void unique_scatter_kernel(
-    Keys k, const int64_t* __restrict__ flat_ptr,
-    const int64_t* __restrict__ tile_ptr, const int64_t* __restrict__ bucket_ptr,
-    int64_t* bucket_cnt, const int64_t* __restrict__ bucket_off,
-    uint64_t* __restrict__ packed, int64_t max_tiles, int remap) {
+    Keys k, const int32_t* __restrict__ tile_batch,
+    const BatchInfo* __restrict__ batch, int64_t* bucket_cnt,
+    const int64_t* __restrict__ bucket_off, uint64_t* __restrict__ packed,
+    int64_t max_tiles, int remap) {
   __shared__ uint32_t hist[kMaxBuckets];   // counts, then offsets inside the tile
   __shared__ uint32_t run_at[kMaxBuckets]; // where the tile's run starts, relative to the batch
   __shared__ uint64_t stage[kPartTile];
   __shared__ uint32_t scan_smem[kBlock / kWave + 1];
+  const int64_t tile = unit_of_block(max_tiles, remap);
+  if (tile >= max_tiles) return;
   TileInfo t;
-  if (!tile_info(k, unit_of_block(max_tiles, remap), flat_ptr, tile_ptr,
-                 bucket_ptr, &t))
-    return;  // uniform per work-group
-  uint64_t* out = packed + t.fb;
-  if (t.buckets == 1) {  // the bucket is the batch, in order
+  if (!tile_info(tile, tile_batch, batch, &t)) return;  // uniform per work-group
+  const uint32_t buckets = (uint32_t)t.b.buckets;
+  uint64_t* out = packed + t.b.fb;
+  if (buckets == 1) {  // the bucket is the batch, in order
     for (int64_t l = t.begin + threadIdx.x; l < t.end; l += kBlock)
-      out[l] = (key_at(k, t.s_lo, t.ns, t.r_lo, l) << 32) | (uint64_t)l;
+      out[l] = (key_at(k, t.b, l) << 32) | (uint64_t)l;
     return;
   }
-  for (uint32_t i = threadIdx.x; i < t.buckets; i += kBlock) hist[i] = 0;
+  for (uint32_t i = threadIdx.x; i < buckets; i += kBlock) hist[i] = 0;
   __syncthreads();
   uint32_t key[kPartItems], place[kPartItems];
 #pragma unroll
   for (int i = 0; i < kPartItems; ++i) {
     const int64_t l = t.begin + i * kBlock + threadIdx.x;
-    key[i] = l < t.end ? (uint32_t)key_at(k, t.s_lo, t.ns, t.r_lo, l) : 0u;
+    key[i] = l < t.end ? (uint32_t)key_at(k, t.b, l) : 0u;
   }
 #pragma unroll
   for (int i = 0; i < kPartItems; ++i)
     if (t.begin + i * kBlock + threadIdx.x < t.end)
-      place[i] = atomicAdd(&hist[bucket_of(key[i], t.buckets)], 1u);
+      place[i] = atomicAdd(&hist[bucket_of(key[i], buckets)], 1u);
   __syncthreads();
+  const uint32_t count = (uint32_t)(t.end - t.begin);
   {
     constexpr int kBins = kMaxBuckets / kBlock;
     const uint32_t bin0 = threadIdx.x * kBins;
     uint32_t c[kBins], sum = 0;
 #pragma unroll
     for (int j = 0; j < kBins; ++j) {
-      c[j] = bin0 + j < t.buckets ? hist[bin0 + j] : 0u;
+      c[j] = bin0 + j < buckets ? hist[bin0 + j] : 0u;
       sum += c[j];
     }
     uint32_t total;
     uint32_t run = block_exclusive_sum(sum, scan_smem, &total);
 #pragma unroll
     for (int j = 0; j < kBins; ++j) {
-      if (bin0 + j < t.buckets) hist[bin0 + j] = run;
+      if (bin0 + j < buckets) hist[bin0 + j] = run;
       run += c[j];
-      if (c[j]) {
-        const int64_t g = t.first_bucket + bin0 + j;
-        const int64_t before = (int64_t)atomicAdd(
-            (unsigned long long*)&bucket_cnt[g],
-            (unsigned long long)(-(int64_t)c[j]));
-        run_at[bin0 + j] = (uint32_t)(bucket_off[g] - t.fb + before - c[j]);
-      }
+    }
+  }
+  __syncthreads();
+  // one bin per thread and round: the reservations of a round are in flight together
+  for (uint32_t bin = threadIdx.x; bin < buckets; bin += kBlock) {
+    const uint32_t c = (bin + 1 < buckets ? hist[bin + 1] : count) - hist[bin];
+    if (c) {
+      const int64_t g = t.b.bucket0 + bin;
+      const int64_t before = (int64_t)atomicAdd(
+          (unsigned long long*)&bucket_cnt[g], (unsigned long long)(-(int64_t)c));
+      run_at[bin] = (uint32_t)(bucket_off[g] - t.b.fb + before - c);
     }
   }
   __syncthreads();
@@ -346,14 +430,13 @@ __global__ __launch_bounds__(kBlock) void unique_scatter_kernel(
   for (int i = 0; i < kPartItems; ++i) {
     const int64_t l = t.begin + i * kBlock + threadIdx.x;
     if (l < t.end)
-      stage[hist[bucket_of(key[i], t.buckets)] + place[i]] =
+      stage[hist[bucket_of(key[i], buckets)] + place[i]] =
           ((uint64_t)key[i] << 32) | (uint64_t)l;
   }
   __syncthreads();
-  const uint32_t count = (uint32_t)(t.end - t.begin);
   for (uint32_t j = threadIdx.x; j < count; j += kBlock) {
     const uint64_t e = stage[j];
-    const uint32_t bk = bucket_of(e >> 32, t.buckets);
+    const uint32_t bk = bucket_of(e >> 32, buckets);
     out[run_at[bk] + (j - hist[bk])] = e;
   }
 }
@@ -456,20 +539,21 @@ __device__ __forceinline__ void lds_insert_min_counted(uint64_t* tab,
 }
 
 __global__ __launch_bounds__(kBlock) void unique_dedup_kernel(
-    const int64_t* __restrict__ flat_ptr, const int64_t* __restrict__ bucket_ptr,
-    int64_t B, const int64_t* __restrict__ bucket_off,
-    const uint64_t* __restrict__ packed, uint64_t* spill,
-    uint32_t* __restrict__ first, int64_t max_buckets, int remap) {
+    const int32_t* __restrict__ bucket_batch, const BatchInfo* __restrict__ batch,
+    const int64_t* __restrict__ bucket_off, const uint64_t* __restrict__ packed,
+    uint64_t* spill, uint32_t* __restrict__ first, int64_t max_buckets,
+    int remap) {
   __shared__ uint64_t tab[kLdsSlots];
   __shared__ uint32_t distinct;
   __shared__ uint32_t overflow;
   const int64_t g = unit_of_block(max_buckets, remap);
-  if (g >= bucket_ptr[B]) return;  // uniform per work-group
+  if (g >= max_buckets) return;
+  const int32_t b = bucket_batch[g];
+  if (b < 0) return;  // uniform per work-group
   const int64_t lo = bucket_off[g], hi = bucket_off[g + 1];
   const int64_t n = hi - lo;
   if (n == 0) return;
-  const int64_t b = B == 1 ? 0 : segment_of(bucket_ptr, B, g);
-  uint32_t* first_b = first + flat_ptr[b];
+  uint32_t* first_b = first + batch[b].fb;
   // table of two slots per entry, a power of two, at most kLdsSlots
   uint32_t slots = 256;
   while (slots < kLdsSlots && (int64_t)slots < 2 * n) slots <<= 1;
@@ -539,18 +623,14 @@ __device__ __forceinline__ int64_t wave_uniform(int64_t v) {
   return (int64_t)(((uint64_t)hi << 32) | lo);
 }
 
-// Batches that the items [x0, x1] of an offsets array touch.
+// Batches that a chunk of consecutive items may touch: from the batch of its
+// first item to the batch of the next chunk's first item.
 struct BatchSpan {
   int64_t lo, hi;
 };
-__device__ __forceinline__ BatchSpan batch_span(const int64_t* __restrict__ ptr,
-                                                int64_t B, int64_t x0, int64_t x1) {
-  BatchSpan s{0, 0};
-  if (B > 1) {
-    s.lo = segment_of(ptr, B, wave_uniform(x0));
-    s.hi = segment_of(ptr, B, wave_uniform(x1));
-  }
-  return s;
+__device__ __forceinline__ BatchSpan batch_span(
+    const int32_t* __restrict__ unit_batch, int64_t unit) {
+  return BatchSpan{unit_batch[unit], unit_batch[unit + 1]};
 }
 __device__ __forceinline__ int64_t batch_in_span(const int64_t* __restrict__ ptr,
                                                  const BatchSpan& s, int64_t x) {
@@ -560,25 +640,30 @@ __device__ __forceinline__ int64_t batch_in_span(const int64_t* __restrict__ ptr
 constexpr int kChunksPerWave = 4;
 
 __global__ __launch_bounds__(kBlock) void unique_flag_kernel(
-    const int64_t* __restrict__ flat_ptr, int64_t B, int64_t N,
-    const uint32_t* __restrict__ first, uint64_t* __restrict__ flags,
+    const int64_t* __restrict__ flat_ptr, const int32_t* __restrict__ chunk_batch,
+    int64_t N, const uint32_t* __restrict__ first, uint64_t* __restrict__ flags,
     int64_t* __restrict__ block_count) {
   const int64_t num_chunks = ceil_div_dev(N, kBlock);
   const int64_t wave = (int64_t)blockIdx.x * kWordsPerBlock + threadIdx.x / kWave;
   const int lane = lane_id();
   for (int c = 0; c < kChunksPerWave; ++c) {
-    const int64_t chunk = wave * kChunksPerWave + c;
+    const int64_t chunk = wave_uniform(wave * kChunksPerWave + c);
     if (chunk >= num_chunks) return;
     const int64_t p0 = chunk * kBlock;
-    const int64_t p_last = p0 + kBlock - 1 < N ? p0 + kBlock - 1 : N - 1;
-    const BatchSpan span = batch_span(flat_ptr, B, p0, p_last);
+    const BatchSpan span = batch_span(chunk_batch, chunk);
+    uint32_t f[kWordsPerBlock];
+#pragma unroll
+    for (int j = 0; j < kWordsPerBlock; ++j) {
+      const int64_t p = p0 + j * kWave + lane;
+      f[j] = p < N ? first[p] : 0u;
+    }
     uint64_t word[kWordsPerBlock];
 #pragma unroll
     for (int j = 0; j < kWordsPerBlock; ++j) {
       const int64_t p = p0 + j * kWave + lane;
       bool is_first = false;
       if (p < N)
-        is_first = (int64_t)first[p] == p - flat_ptr[batch_in_span(flat_ptr, span, p)];
+        is_first = (int64_t)f[j] == p - flat_ptr[batch_in_span(flat_ptr, span, p)];
       word[j] = __ballot(is_first);
     }
     if (lane == 0) {
@@ -622,10 +707,11 @@ __global__ void unique_ptr_kernel(const int64_t* __restrict__ flat_ptr,
 // Streaming: every position writes its rank (or -1); first occurrences also
 // write their key to the frontier.
 __global__ __launch_bounds__(kBlock) void unique_fill_kernel(
-    Keys k, const int64_t* __restrict__ flat_ptr, int64_t N,
-    const uint64_t* __restrict__ flags, const int64_t* __restrict__ block_off,
-    const int64_t* __restrict__ unique_ptr, int64_t* __restrict__ out_unique,
-    int32_t* __restrict__ rank) {
+    Keys k, const int64_t* __restrict__ flat_ptr,
+    const int32_t* __restrict__ chunk_batch, const BatchInfo* __restrict__ batch,
+    int64_t N, const uint64_t* __restrict__ flags,
+    const int64_t* __restrict__ block_off, const int64_t* __restrict__ unique_ptr,
+    int64_t* __restrict__ out_unique, int32_t* __restrict__ rank) {
   const int64_t num_chunks = ceil_div_dev(N, kBlock);
   const int64_t wave = (int64_t)blockIdx.x * kWordsPerBlock + threadIdx.x / kWave;
   const int lane = lane_id();
@@ -633,56 +719,69 @@ __global__ __launch_bounds__(kBlock) void unique_fill_kernel(
     const int64_t chunk = wave_uniform(wave * kChunksPerWave + c);
     if (chunk >= num_chunks) return;
     const int64_t p0 = chunk * kBlock;
-    const int64_t p_last = p0 + kBlock - 1 < N ? p0 + kBlock - 1 : N - 1;
-    const BatchSpan span = batch_span(flat_ptr, k.B, p0, p_last);
+    const BatchSpan span = batch_span(chunk_batch, chunk);
     int64_t before = block_off[chunk];
+    uint64_t word[kWordsPerBlock];
+#pragma unroll
+    for (int j = 0; j < kWordsPerBlock; ++j)
+      word[j] = flags[chunk * kWordsPerBlock + j];
+    BatchInfo info = batch[span.lo];
+    int64_t rank0 = unique_ptr[span.lo];
 #pragma unroll
     for (int j = 0; j < kWordsPerBlock; ++j) {
-      const uint64_t word = flags[chunk * kWordsPerBlock + j];
       const int64_t p = p0 + j * kWave + lane;
       if (p < N) {
         int32_t r = -1;
-        if ((word >> lane) & 1ull) {
-          const int64_t b = batch_in_span(flat_ptr, span, p);
-          const int64_t s_lo = seeds_lo(k, b);
-          const uint64_t key = key_at(k, s_lo, seeds_lo(k, b + 1) - s_lo,
-                                      rows_lo(k, b), p - flat_ptr[b]);
-          const int64_t grank = before + __popcll(word & ((1ull << lane) - 1));
+        if ((word[j] >> lane) & 1ull) {
+          if (span.lo != span.hi) {  // the chunk straddles batches
+            const int64_t b = batch_in_span(flat_ptr, span, p);
+            info = batch[b];
+            rank0 = unique_ptr[b];
+          }
+          const uint64_t key = key_at(k, info, p - info.fb);
+          const int64_t grank = before + __popcll(word[j] & ((1ull << lane) - 1));
           out_unique[grank] = (int64_t)key;
-          r = (int32_t)(grank - unique_ptr[b]);
+          r = (int32_t)(grank - rank0);
         }
         rank[p] = r;
       }
-      before += __popcll(word);
+      before += __popcll(word[j]);
     }
   }
 }
 
 // ---------------------------------------------------------------- relabel
-constexpr int kRelabelItems = 4;
-constexpr int kRelabelTile = kBlock * kRelabelItems;
-
 __global__ __launch_bounds__(kBlock) void unique_relabel_kernel(
-    Keys k, const int64_t* __restrict__ flat_ptr,
-    const uint32_t* __restrict__ first, const int32_t* __restrict__ rank,
-    const int64_t* __restrict__ edge_col, int64_t* __restrict__ out_row,
-    int64_t* __restrict__ out_col, int remap) {
-  const int64_t e0 =
-      unit_of_block(ceil_div_dev(k.E, kRelabelTile), remap) * kRelabelTile;
-  if (e0 >= k.E) return;
-  const int64_t e_last = e0 + kRelabelTile - 1 < k.E ? e0 + kRelabelTile - 1 : k.E - 1;
-  const BatchSpan span = batch_span(k.rows_ptr, k.B, e0, e_last);
+    Keys k, const int32_t* __restrict__ etile_batch,
+    const BatchInfo* __restrict__ batch, const uint32_t* __restrict__ first,
+    const int32_t* __restrict__ rank, const int64_t* __restrict__ edge_col,
+    int64_t* __restrict__ out_row, int64_t* __restrict__ out_col, int remap) {
+  const int64_t num_tiles = ceil_div_dev(k.E, kRelabelTile);
+  const int64_t tile = unit_of_block(num_tiles, remap);
+  if (tile >= num_tiles) return;
+  const int64_t e0 = tile * kRelabelTile;
+  const BatchSpan span = batch_span(etile_batch, tile);
+  int64_t col[kRelabelItems];
+  uint32_t row_first[kRelabelItems];
+  BatchInfo info = batch[span.lo];
 #pragma unroll
   for (int i = 0; i < kRelabelItems; ++i) {
     const int64_t e = e0 + i * kBlock + threadIdx.x;
     if (e >= k.E) break;
-    const int64_t b = k.B == 1 ? 0 : batch_in_span(k.rows_ptr, span, e);
-    const int64_t fb = flat_ptr[b];
+    if (span.lo != span.hi) info = batch[batch_in_span(k.rows_ptr, span, e)];
     // row key e of batch b sits at flat position
     //   fb + (seeds of b) + (e - rows_ptr[b])  =  e + seeds_ptr[b + 1]
-    if (out_row) out_row[e] = rank[fb + first[e + seeds_lo(k, b + 1)]];
+    if (out_row) row_first[i] = first[e + info.s_lo + info.ns];
+    if (out_col) col[i] = edge_col[e];
+  }
+#pragma unroll
+  for (int i = 0; i < kRelabelItems; ++i) {
+    const int64_t e = e0 + i * kBlock + threadIdx.x;
+    if (e >= k.E) break;
+    if (span.lo != span.hi) info = batch[batch_in_span(k.rows_ptr, span, e)];
+    if (out_row) out_row[e] = rank[info.fb + row_first[i]];
     // seed c of batch b sits at flat position c + rows_ptr[b]
-    if (out_col) out_col[e] = rank[fb + first[edge_col[e] + rows_lo(k, b)]];
+    if (out_col) out_col[e] = rank[info.fb + first[col[i] + info.r_lo]];
   }
 }
 
@@ -742,38 +841,44 @@ int gs_unique_count(const int64_t* seeds, const int64_t* seeds_ptr,
     return GS_OK;
   }
   const Keys k{seeds, seeds_ptr, S, rows, rows_ptr, E, B};
-  const int64_t nblocks = ceil_div(N, kBlock);
+  const int64_t nblocks = w.chunks;
   {
     int64_t blocks = ceil_div(w.max_buckets + 1, kBlock * 4);
     if (blocks > 1024) blocks = 1024;
     GS_LAUNCH("unique_prep", s,
               unique_prep_kernel<<<dim3((unsigned)blocks), dim3(kBlock), 0, s>>>(
-                  k, tn.bucket_keys, w.flat_ptr, w.tile_ptr, w.bucket_ptr,
-                  w.bucket_cnt, w.max_buckets));
+                  k, tn.bucket_keys, w.batch, w.flat_ptr, w.tile_ptr,
+                  w.bucket_ptr, w.bucket_cnt, w.max_buckets));
+    const int64_t units = w.max_tiles + w.max_buckets + w.chunks + 1 + w.etiles + 1;
+    GS_LAUNCH("unique_units", s,
+              unique_units_kernel<<<dim3((unsigned)ceil_div(units, kBlock)),
+                                    dim3(kBlock), 0, s>>>(
+                  k, N, w.flat_ptr, w.tile_ptr, w.bucket_ptr, w.max_tiles,
+                  w.max_buckets, w.chunks, w.etiles, w.tile_batch,
+                  w.bucket_batch, w.chunk_batch, w.etile_batch));
   }
   const dim3 tile_grid((unsigned)grid_for_units(w.max_tiles, tn.remap));
   GS_LAUNCH("unique_hist", s,
             unique_hist_kernel<<<tile_grid, dim3(kBlock), 0, s>>>(
-                k, w.flat_ptr, w.tile_ptr, w.bucket_ptr, w.bucket_cnt,
-                w.max_tiles, tn.remap));
+                k, w.tile_batch, w.batch, w.bucket_cnt, w.max_tiles, tn.remap));
   GS_LAUNCH("unique_bucket_scan", s,
             unique_bucket_scan_kernel<<<dim3(1), dim3(kBlock), 0, s>>>(
                 w.bucket_ptr, B, w.bucket_cnt, w.bucket_off));
   GS_LAUNCH("unique_scatter", s,
             unique_scatter_kernel<<<tile_grid, dim3(kBlock), 0, s>>>(
-                k, w.flat_ptr, w.tile_ptr, w.bucket_ptr, w.bucket_cnt,
-                w.bucket_off, w.packed, w.max_tiles, tn.remap));
+                k, w.tile_batch, w.batch, w.bucket_cnt, w.bucket_off, w.packed,
+                w.max_tiles, tn.remap));
   GS_LAUNCH("unique_dedup", s,
             unique_dedup_kernel<<<dim3((unsigned)grid_for_units(w.max_buckets,
                                                                 tn.remap)),
                                   dim3(kBlock), 0, s>>>(
-                w.flat_ptr, w.bucket_ptr, B, w.bucket_off, w.packed, w.spill,
+                w.bucket_batch, w.batch, w.bucket_off, w.packed, w.spill,
                 w.first, w.max_buckets, tn.remap));
   GS_LAUNCH("unique_flag", s,
             unique_flag_kernel<<<dim3((unsigned)ceil_div(
                                      nblocks, kWordsPerBlock * kChunksPerWave)),
                                  dim3(kBlock), 0, s>>>(
-                w.flat_ptr, B, N, w.first, w.flags, w.block_off));
+                w.flat_ptr, w.chunk_batch, N, w.first, w.flags, w.block_off));
   rc = exclusive_scan_i64(w.block_off, w.block_off, nblocks + 1, w.scan_ws,
                           w.scan_ws_bytes, s);
   if (rc != GS_OK) return rc;
@@ -807,8 +912,8 @@ int gs_unique_fill(const int64_t* seeds, const int64_t* seeds_ptr,
                                      ceil_div(N, kBlock),
                                      kWordsPerBlock * kChunksPerWave)),
                                  dim3(kBlock), 0, s>>>(
-                k, w.flat_ptr, N, w.flags, w.block_off, unique_ptr, out_unique,
-                w.rank));
+                k, w.flat_ptr, w.chunk_batch, w.batch, N, w.flags, w.block_off,
+                unique_ptr, out_unique, w.rank));
   return GS_OK;
 }
 
@@ -834,8 +939,8 @@ int gs_unique_relabel(const int64_t* seeds, const int64_t* seeds_ptr,
               unique_relabel_kernel<<<dim3((unsigned)grid_for_units(
                                           ceil_div(E, kRelabelTile), tn.remap)),
                                       dim3(kBlock), 0, s>>>(
-                  k, w.flat_ptr, w.first, w.rank, edge_col, out_row, out_col,
-                  tn.remap));
+                  k, w.etile_batch, w.batch, w.first, w.rank, edge_col, out_row,
+                  out_col, tn.remap));
   }
   return GS_OK;
 }
