@@ -141,9 +141,9 @@ __device__ __forceinline__ T wave_inclusive_sum(T v) {
   return v;
 }
 
-// Exclusive block scan for blocks of kBlock threads.  `total` receives the
-// block sum in every thread.  smem must hold kBlock / kWave + 1 elements.
-template <typename T>
+// Exclusive block scan for blocks of kThreads threads.  `total` receives the
+// block sum in every thread.  smem must hold kThreads / kWave + 1 elements.
+template <typename T, int kThreads = kBlock>
 __device__ __forceinline__ T block_exclusive_sum(T v, T* smem, T* total) {
   const int wave = threadIdx.x / kWave;
   T inc = wave_inclusive_sum(v);
@@ -151,7 +151,7 @@ __device__ __forceinline__ T block_exclusive_sum(T v, T* smem, T* total) {
   __syncthreads();
   T base = 0, sum = 0;
 #pragma unroll
-  for (int w = 0; w < kBlock / kWave; ++w) {
+  for (int w = 0; w < kThreads / kWave; ++w) {
     T s = smem[w];
     if (w < wave) base += s;
     sum += s;

@@ -131,6 +131,10 @@ __global__ __launch_bounds__(kBlock) void scan_spine_kernel(int64_t* tile_sums,
   }
 }
 
+// Tile t adds the sums of the tiles before it: already scanned by
+// scan_spine_kernel (kSpineDone), or summed here by the tile itself
+// (kSpineDone == false, for spines short enough that a launch costs more).
+template <bool kSpineDone>
 __global__ __launch_bounds__(kBlock) void scan_down_kernel(
     const int64_t* in, int64_t* out, int64_t n,
     const int64_t* __restrict__ tile_sums) {
@@ -144,8 +148,18 @@ __global__ __launch_bounds__(kBlock) void scan_down_kernel(
     v[k] = i < n ? in[i] : 0;
     s += v[k];
   }
+  int64_t before = 0;
+  if (kSpineDone) {
+    before = tile_sums[blockIdx.x];
+  } else {
+    int64_t part = 0;
+    for (int64_t t = threadIdx.x; t < (int64_t)blockIdx.x; t += kBlock)
+      part += tile_sums[t];
+    int64_t ignored = block_exclusive_sum(part, smem, &before);
+    (void)ignored;
+  }
   int64_t total;
-  int64_t ex = block_exclusive_sum(s, smem, &total) + tile_sums[blockIdx.x];
+  int64_t ex = block_exclusive_sum(s, smem, &total) + before;
 #pragma unroll
   for (int k = 0; k < kScanItems; ++k) {
     int64_t i = base + k;
@@ -153,6 +167,8 @@ __global__ __launch_bounds__(kBlock) void scan_down_kernel(
     ex += v[k];
   }
 }
+
+constexpr int64_t kShortSpine = 4096;  // tiles
 
 size_t scan_workspace_bytes(int64_t n) {
   int64_t tiles = n > 0 ? ceil_div(n, kScanTile) : 1;
@@ -169,15 +185,27 @@ int exclusive_scan_i64(const int64_t* in, int64_t* out, int64_t n, void* ws,
   }
   int64_t* tile_sums = (int64_t*)ws;
   const int64_t tiles = ceil_div(n, kScanTile);
+  if (tiles == 1) {  // nothing before the only tile
+    GS_LAUNCH("scan_down", stream,
+              scan_down_kernel<false><<<dim3(1), dim3(kBlock), 0, stream>>>(
+                  in, out, n, tile_sums));
+    return GS_OK;
+  }
   GS_LAUNCH("scan_tile_sums", stream,
             scan_tile_sums_kernel<<<dim3((unsigned)tiles), dim3(kBlock), 0,
                                     stream>>>(in, n, tile_sums));
+  if (tiles <= kShortSpine) {
+    GS_LAUNCH("scan_down", stream,
+              scan_down_kernel<false><<<dim3((unsigned)tiles), dim3(kBlock), 0,
+                                        stream>>>(in, out, n, tile_sums));
+    return GS_OK;
+  }
   GS_LAUNCH("scan_spine", stream,
             scan_spine_kernel<<<dim3(1), dim3(kBlock), 0, stream>>>(tile_sums,
                                                                     tiles));
   GS_LAUNCH("scan_down", stream,
-            scan_down_kernel<<<dim3((unsigned)tiles), dim3(kBlock), 0, stream>>>(
-                in, out, n, tile_sums));
+            scan_down_kernel<true><<<dim3((unsigned)tiles), dim3(kBlock), 0,
+                                      stream>>>(in, out, n, tile_sums));
   return GS_OK;
 }
 

@@ -7,7 +7,7 @@
 //
 // A hash table over all keys of a batch does not fit in a die's L2, and every
 // random access to it costs a whole line from HBM.  So the keys of a batch are
-// first partitioned by hash into buckets of about a thousand entries (streaming
+// first partitioned by hash into buckets of about 1500 entries (streaming
 // reads and writes only), and each bucket is then deduplicated by one
 // work-group in an LDS table:
 //   prep     per-batch record (where its keys, tiles and buckets start); zero
@@ -51,15 +51,19 @@ constexpr int kMaxBuckets = 2048;                 // buckets per batch (LDS bins
 constexpr int kLdsSlots = 4096;                   // dedup table, 32 KB of LDS
 constexpr int kLdsMaxEntries = kLdsSlots * 3 / 4; // bucket sizes the LDS table takes
 
-// Average entries per bucket (GS_BUCKET_KEYS) and whether work-groups are laid
-// out per die (GS_XCD_REMAP).  Read once.
+// Average entries per bucket (GS_BUCKET_KEYS), threads of a dedup work-group
+// (GS_DEDUP_THREADS: 256 or 512) and whether work-groups are laid out per die
+// (GS_XCD_REMAP).  The defaults are the best of a sweep on 21M keys in 64
+// batches; the variables exist for such sweeps.  Read once.
 struct UniqueTuning {
   int64_t bucket_keys;
   int remap;
+  int dedup_threads;
 };
 static UniqueTuning tuning() {
   static const UniqueTuning t = [] {
-    UniqueTuning r{1024, 1};
+    UniqueTuning r{1536, 1, 512};
+    if (const char* e = getenv("GS_DEDUP_THREADS")) r.dedup_threads = atoi(e);
     if (const char* e = getenv("GS_BUCKET_KEYS")) r.bucket_keys = atoll(e);
     if (const char* e = getenv("GS_XCD_REMAP")) r.remap = atoi(e);
     if (r.bucket_keys < 64) r.bucket_keys = 64;
@@ -330,15 +334,16 @@ __global__ __launch_bounds__(kBlock) void unique_hist_kernel(
 }
 
 // Exclusive scan of the bucket counts by one work-group (there are about
-// N / 1024 of them).  off[total_buckets] = N closes the last bucket.
-__global__ __launch_bounds__(kBlock) void unique_bucket_scan_kernel(
+// N / 1500 of them).  off[total_buckets] = N closes the last bucket.
+constexpr int kBucketScanThreads = 1024;
+__global__ __launch_bounds__(kBucketScanThreads) void unique_bucket_scan_kernel(
     const int64_t* __restrict__ bucket_ptr, int64_t B,
     const int64_t* __restrict__ bucket_cnt, int64_t* __restrict__ bucket_off) {
-  __shared__ int64_t smem[kBlock / kWave + 1];
+  __shared__ int64_t smem[kBucketScanThreads / kWave + 1];
   const int64_t n = bucket_ptr[B] + 1;
   int64_t carry = 0;
   constexpr int kPer = 8;
-  for (int64_t base = 0; base < n; base += kBlock * kPer) {
+  for (int64_t base = 0; base < n; base += kBucketScanThreads * kPer) {
     const int64_t i0 = base + (int64_t)threadIdx.x * kPer;
     int64_t v[kPer], sum = 0;
 #pragma unroll
@@ -347,14 +352,14 @@ __global__ __launch_bounds__(kBlock) void unique_bucket_scan_kernel(
       sum += v[j];
     }
     int64_t total;
-    int64_t run = carry + block_exclusive_sum(sum, smem, &total);
+    int64_t run = carry + block_exclusive_sum<int64_t, kBucketScanThreads>(
+                              sum, smem, &total);
 #pragma unroll
     for (int j = 0; j < kPer; ++j) {
       if (i0 + j < n) bucket_off[i0 + j] = run;
       run += v[j];
     }
     carry += total;
-    __syncthreads();
   }
 }
 
@@ -538,7 +543,8 @@ __device__ __forceinline__ void lds_insert_min_counted(uint64_t* tab,
   }
 }
 
-__global__ __launch_bounds__(kBlock) void unique_dedup_kernel(
+template <int kThreads>
+__global__ __launch_bounds__(kThreads) void unique_dedup_kernel(
     const int32_t* __restrict__ bucket_batch, const BatchInfo* __restrict__ batch,
     const int64_t* __restrict__ bucket_off, const uint64_t* __restrict__ packed,
     uint64_t* spill, uint32_t* __restrict__ first, int64_t max_buckets,
@@ -558,16 +564,16 @@ __global__ __launch_bounds__(kBlock) void unique_dedup_kernel(
   uint32_t slots = 256;
   while (slots < kLdsSlots && (int64_t)slots < 2 * n) slots <<= 1;
   const uint32_t mask = slots - 1;
-  for (uint32_t i = threadIdx.x; i < slots; i += kBlock) tab[i] = kEmptySlot;
+  for (uint32_t i = threadIdx.x; i < slots; i += kThreads) tab[i] = kEmptySlot;
   if (threadIdx.x == 0) distinct = overflow = 0;
   __syncthreads();
-  constexpr int kKeep = kLdsMaxEntries / kBlock;
+  constexpr int kKeep = kLdsMaxEntries / kThreads;
   if (n <= kLdsMaxEntries) {
     // sure to fit; the thread's entries stay in registers between the phases
     uint64_t mine[kKeep];
 #pragma unroll
     for (int j = 0; j < kKeep; ++j) {
-      const int64_t i = lo + j * kBlock + threadIdx.x;
+      const int64_t i = lo + j * kThreads + threadIdx.x;
       mine[j] = i < hi ? packed[i] : kEmptySlot;
     }
 #pragma unroll
@@ -582,13 +588,13 @@ __global__ __launch_bounds__(kBlock) void unique_dedup_kernel(
   }
   // Many entries: fine for the LDS table while few of them are distinct (a hub
   // that repeats thousands of times), so try, and count.
-  for (int64_t i = lo + threadIdx.x; i < hi; i += kBlock) {
+  for (int64_t i = lo + threadIdx.x; i < hi; i += kThreads) {
     if (*(volatile uint32_t*)&overflow) break;
     lds_insert_min_counted(tab, mask, packed[i], &distinct, &overflow);
   }
   __syncthreads();
   if (!overflow) {
-    for (int64_t i = lo + threadIdx.x; i < hi; i += kBlock) {
+    for (int64_t i = lo + threadIdx.x; i < hi; i += kThreads) {
       const uint64_t e = packed[i];
       first_b[(uint32_t)e] = lds_first_of(tab, mask, e >> 32);
     }
@@ -597,14 +603,14 @@ __global__ __launch_bounds__(kBlock) void unique_dedup_kernel(
   // too many distinct keys: a private table in global memory, two slots per entry
   uint64_t* gt = spill + 2 * lo + g;
   const uint64_t cap = (uint64_t)(2 * n + 1);
-  for (uint64_t i = threadIdx.x; i < cap; i += kBlock) gt[i] = kEmptySlot;
+  for (uint64_t i = threadIdx.x; i < cap; i += kThreads) gt[i] = kEmptySlot;
   __threadfence();
   __syncthreads();
-  for (int64_t i = lo + threadIdx.x; i < hi; i += kBlock)
+  for (int64_t i = lo + threadIdx.x; i < hi; i += kThreads)
     spill_insert_min(gt, cap, packed[i]);
   __threadfence();
   __syncthreads();
-  for (int64_t i = lo + threadIdx.x; i < hi; i += kBlock) {
+  for (int64_t i = lo + threadIdx.x; i < hi; i += kThreads) {
     const uint64_t e = packed[i];
     first_b[(uint32_t)e] = spill_first_of(gt, cap, e >> 32);
   }
@@ -862,18 +868,25 @@ int gs_unique_count(const int64_t* seeds, const int64_t* seeds_ptr,
             unique_hist_kernel<<<tile_grid, dim3(kBlock), 0, s>>>(
                 k, w.tile_batch, w.batch, w.bucket_cnt, w.max_tiles, tn.remap));
   GS_LAUNCH("unique_bucket_scan", s,
-            unique_bucket_scan_kernel<<<dim3(1), dim3(kBlock), 0, s>>>(
+            unique_bucket_scan_kernel<<<dim3(1), dim3(kBucketScanThreads), 0, s>>>(
                 w.bucket_ptr, B, w.bucket_cnt, w.bucket_off));
   GS_LAUNCH("unique_scatter", s,
             unique_scatter_kernel<<<tile_grid, dim3(kBlock), 0, s>>>(
                 k, w.tile_batch, w.batch, w.bucket_cnt, w.bucket_off, w.packed,
                 w.max_tiles, tn.remap));
   GS_LAUNCH("unique_dedup", s,
-            unique_dedup_kernel<<<dim3((unsigned)grid_for_units(w.max_buckets,
-                                                                tn.remap)),
-                                  dim3(kBlock), 0, s>>>(
-                w.bucket_batch, w.batch, w.bucket_off, w.packed, w.spill,
-                w.first, w.max_buckets, tn.remap));
+            if (tn.dedup_threads == 512)
+              unique_dedup_kernel<512><<<dim3((unsigned)grid_for_units(
+                                             w.max_buckets, tn.remap)),
+                                         dim3(512), 0, s>>>(
+                  w.bucket_batch, w.batch, w.bucket_off, w.packed, w.spill,
+                  w.first, w.max_buckets, tn.remap);
+            else
+              unique_dedup_kernel<256><<<dim3((unsigned)grid_for_units(
+                                             w.max_buckets, tn.remap)),
+                                         dim3(256), 0, s>>>(
+                  w.bucket_batch, w.batch, w.bucket_off, w.packed, w.spill,
+                  w.first, w.max_buckets, tn.remap));
   GS_LAUNCH("unique_flag", s,
             unique_flag_kernel<<<dim3((unsigned)ceil_div(
                                      nblocks, kWordsPerBlock * kChunksPerWave)),

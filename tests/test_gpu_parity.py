@@ -29,7 +29,7 @@ def assert_same(got, want):
             assert np.array_equal(N(g), w)
 
 
-@pytest.mark.parametrize("n", [0, 1, 255, 256, 2049, 1 << 20, (1 << 22) + 3])
+@pytest.mark.parametrize("n", [0, 1, 255, 256, 2048, 2049, 1 << 20, (1 << 22) + 3, (1 << 23) + 4099])
 def test_scan(n):
     rng = np.random.default_rng(n)
     x = rng.integers(0, 1000, size=n)
