@@ -41,3 +41,12 @@ def random_csc(rng, num_cols, num_rows, max_deg, empty_frac=0.2, hub_deg=0):
 @pytest.fixture
 def rng():
     return np.random.default_rng(12345)
+
+
+def golden() -> dict:
+    """Known answers of the reference's own tests (tests/golden/)."""
+    import json
+    import os
+    path = os.path.join(os.path.dirname(__file__), "golden", "reference_known_answers.json")
+    with open(path) as f:
+        return json.load(f)

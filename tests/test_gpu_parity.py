@@ -198,3 +198,18 @@ def test_graphsage_layers_end_to_end():
         assert_same(gu, ou)
         g_seeds, g_ptr = gu[0], gu[1]
         seeds, ptr = ou[0], ou[1]
+
+
+def test_format_and_batch_helpers_parity():
+    rng = np.random.default_rng(21)
+    indptr, indices = random_csc(rng, 3000, 5000, 40, hub_deg=20000)
+    assert np.array_equal(N(capi.csc2coo(T(indptr))), orc.csc2coo(indptr))
+    assert capi.csc2coo(T(np.zeros(5, dtype=np.int64))).numel() == 0
+    ids = np.sort(rng.integers(0, 777, size=100000))
+    assert np.array_equal(N(capi.sorted_to_indptr(T(ids), 777)), orc.sorted_to_indptr(ids, 777))
+    enc = rng.integers(0, 1000, size=5000) + rng.integers(0, 64, size=5000) * 1000
+    for g, o in zip(capi.decode_batch_ids(T(enc), 1000), orc.decode_batch_ids(enc, 1000)):
+        assert np.array_equal(N(g), o)
+    offset = np.array([0, 100, 100, 1500, 3000])
+    assert np.array_equal(N(capi.split_indptr(T(indptr), T(offset))),
+                          orc.split_indptr(indptr, offset))

@@ -2,17 +2,17 @@
 import numpy as np
 
 from oracle import binding as orc
-from tests.conftest import random_csc
+from tests.conftest import golden, random_csc
 
 
 def test_reference_rowwise_slicing_known_answer():
     # tests/test_rowwise_slicing.cc:7-24 : CSR-style slicing of id 5 keeps 2 edges;
     # the reference asserts the kept *column* ids are [10, 11] -- the segments
     # that hold the two edges whose id is 5.
-    indptr = np.concatenate([np.zeros(10, dtype=np.int64), np.arange(3) * 2])
-    indices = np.tile(np.arange(5, 7), 2)
-    out_indptr, major, minor, select = orc.minor_slice(indices, [5], indptr=indptr)
-    assert major.tolist() == [10, 11]
+    fx = golden()["rowwise_slicing"]
+    indptr, indices = np.array(fx["indptr"]), np.array(fx["indices"])
+    out_indptr, major, minor, select = orc.minor_slice(indices, fx["row_ids"], indptr=indptr)
+    assert major.tolist() == fx["kept_major_ids"]
     assert minor.tolist() == [0, 0] and select.tolist() == [0, 2]
     assert out_indptr.tolist() == [0] * 11 + [1, 2]
 

@@ -6,14 +6,11 @@ import numpy as np
 
 from oracle import binding as orc
 
-KAT = [
-    ((0, 0, 0, 0), (0, 0),
-     (0x6627e8d5, 0xe169c58d, 0xbc57ac4c, 0x9b00dbd8)),
-    ((0xffffffff,) * 4, (0xffffffff,) * 2,
-     (0x408f276d, 0x41c83b0e, 0xa20bc7c6, 0x6d5451fd)),
-    ((0x243f6a88, 0x85a308d3, 0x13198a2e, 0x03707344), (0xa4093822, 0x299f31d0),
-     (0xd16cfe09, 0x94fdcceb, 0x5001e420, 0x24126ea1)),
-]
+from tests.conftest import golden
+
+KAT = [(tuple(int(w, 16) for w in v["ctr"]), tuple(int(w, 16) for w in v["key"]),
+        tuple(int(w, 16) for w in v["out"]))
+       for v in golden()["philox4x32_10_kat"]["vectors"]]
 
 
 def test_philox_known_answers():

@@ -5,16 +5,16 @@ import pytest
 
 from oracle import binding as orc
 from tests import numpy_ref as ref
-from tests.conftest import random_csc
+from tests.conftest import golden, random_csc
 
 
 def test_reference_colwise_slicing_known_answer():
     # tests/test_colwise_slicing.cc:7-21 of the reference
-    indptr = np.arange(21) * 5
-    indices = np.arange(100)
-    sub_indptr, coo_col, sub_indices, sel = orc.col_slice(indptr, indices, [0, 1, 2])
-    assert np.array_equal(sub_indptr, np.arange(4) * 5)
-    assert np.array_equal(sub_indices, np.arange(15))
+    fx = golden()["colwise_slicing"]
+    indptr, indices = np.array(fx["indptr"]), np.array(fx["indices"])
+    sub_indptr, coo_col, sub_indices, sel = orc.col_slice(indptr, indices, fx["column_ids"])
+    assert np.array_equal(sub_indptr, fx["sub_indptr"])
+    assert np.array_equal(sub_indices, fx["sub_indices"])
     assert np.array_equal(sel, np.arange(15))
     assert np.array_equal(coo_col, np.repeat(np.arange(3), 5))
 

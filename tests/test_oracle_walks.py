@@ -4,11 +4,12 @@ import numpy as np
 from scipy import stats
 
 from oracle import binding as orc
-from tests.conftest import random_csc
+from tests.conftest import golden, random_csc
 
 # tests/test_random_walk.cc:27-60 and tests/test_node2vec.cc:27-60
-DAG_INDPTR = np.array([0, 0, 1, 2, 3, 5])
-DAG_INDICES = np.array([0, 1, 1, 2, 3])
+DAG = golden()["walk_dag"]
+DAG_INDPTR = np.array(DAG["indptr"])
+DAG_INDICES = np.array(DAG["indices"])
 
 
 def _edge_exists(src, dst):
