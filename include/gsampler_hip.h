@@ -135,7 +135,9 @@ int gs_csc_col_slice_fill(const int64_t* indptr, int64_t num_cols,
  * Uniform per-column sampling (fill phase), optionally fused with the column
  * slice (column_ids != NULL).  sub_indptr comes from gs_csc_col_count with
  * the same fanout / replace.  Columns with degree <= fanout are copied in
- * their original order (no replace).  `algo` is one of GS_ALGO_*.
+ * their original order (no replace).  `algo` is one of GS_ALGO_*.  `indices`
+ * may be NULL, meaning "the edge position itself" (out_indices then repeats
+ * out_select).
  * Stands in for CSCColSamplingCUDA (src/cuda/sampling.cu:161-172) and
  * FusedCSCColSlicingSamplingCUDA (src/cuda/fusion/slice_sampling.cu:164-177).
  * ---------------------------------------------------------------------- */
@@ -215,11 +217,11 @@ int gs_list_sample_weighted_fill(const float* probs, const int64_t* range,
  *     seeds[seeds_ptr[b] : seeds_ptr[b+1]] ++ rows[rows_ptr[b] : rows_ptr[b+1]]
  * (seeds_ptr == rows_ptr == NULL means a single batch holding everything).
  *
- * count: builds the per-batch hash tables inside the workspace and writes
- *   unique_ptr[num_batches + 1] (number of unique keys before each batch;
- *   the last element is the total U).
+ * count: finds the first occurrence of every key (state kept inside the
+ *   workspace) and writes unique_ptr[num_batches + 1] (number of unique keys
+ *   before each batch; the last element is the total U).
  * fill:  same arguments + the same workspace, untouched in between; writes
- *   out_unique[U] and turns the tables into key -> batch-local rank maps.
+ *   out_unique[U] and the rank of every first occurrence into the workspace.
  * relabel: after fill, same workspace; out_row[num_rows_keys] = batch-local
  *   rank of every row key (nullable); out_col[num_rows_keys] = batch-local rank
  *   of seeds[edge_col[e]] (nullable; edge_col holds positions into `seeds`).
