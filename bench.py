@@ -36,6 +36,13 @@ WORKLOADS = {
     "c1": dict(nodes=100_000, edges=2_000_000, gen="rmat", batches=1,
                batch_size=1024, fanouts=[25, 10],
                desc="GraphSAGE 2-layer uniform [25,10], 1024 seeds, R-MAT 100K nodes / 2M edges"),
+    "c3": dict(kind="ladies", nodes=233_000, edges=115_000_000, gen="chung_lu", seeds=512,
+               fanouts=[512, 512],
+               desc="LADIES 2 layers, 512 seeds, K=512 per layer, Chung-Lu power-law 233K nodes / "
+                    "115M edges, fp32 edge weights U(0,1], through Matrix / gs.jit.compile"),
+    "c4": dict(kind="node2vec", nodes=2_450_000, edges=124_000_000, gen="chung_lu",
+               walks=1_000_000, length=80, p=2.0, q=0.5,
+               desc="node2vec, 1M walks x 80 steps, p=2.0 q=0.5, C2's graph with sorted columns"),
     "tiny": dict(nodes=50_000, edges=1_000_000, gen="chung_lu", batches=8,
                  batch_size=256, fanouts=[15, 10, 5],
                  desc="1/50-scale twin of c2 (smoke runs)"),
@@ -82,6 +89,160 @@ def kernel_bytes(name, sizes):
     return total
 
 
+def _kernel_table(capi, bytes_of):
+    """Per-kernel totals of the library's event timers -> sorted list of dicts."""
+    kernels = []
+    for name, (calls, ms) in capi.profile_totals().items():
+        nbytes = bytes_of(name)
+        kernels.append(dict(kernel=name, launches=calls, avg_ms=round(ms / max(calls, 1), 4),
+                            total_ms=round(ms, 4), algorithmic_bytes=nbytes,
+                            gbs=round(nbytes / (ms * 1e-3) / 1e9, 1) if ms > 0 else 0.0))
+    kernels.sort(key=lambda k: -k["total_ms"])
+    return kernels
+
+
+def _roofline(dom):
+    return dict(bound="hbm", kernel=dom["kernel"], achieved=dom["gbs"], peak=HBM_PEAK_GBS,
+                unit="GB/s", frac=round(dom["gbs"] / HBM_PEAK_GBS, 4), traffic=None,
+                avg_launch_ms=dom["avg_ms"], launches=dom["launches"])
+
+
+def run_node2vec(args, wl, capi, dev):
+    """Second-order walks over C2's graph.  A step = one launch of all walks."""
+    import torch
+    from gsampler_amd.utils import chung_lu_csc
+    t0 = time.time()
+    indptr, indices = chung_lu_csc(wl["nodes"], wl["edges"], seed=1, device=dev)
+    indices = capi.segment_sort(indptr, indices)          # node2vec needs sorted columns
+    g = torch.Generator(device=dev)
+    g.manual_seed(3)
+    seeds = torch.randint(0, wl["nodes"], (wl["walks"],), generator=g, device=dev)
+    torch.cuda.synchronize()
+    t_build = time.time() - t0
+    L = wl["length"]
+
+    def step(i):
+        return capi.node2vec(indptr, indices, seeds, L, wl["p"], wl["q"], args.seed, i)
+
+    for i in range(args.warmup):
+        step(i)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        trace = step(args.warmup + i)
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    hops = int((trace[1:] >= 0).sum().item())             # hops taken in the last step
+    capi.profile_reset()
+    capi.profile_enable(True)
+    for i in range(args.steps):
+        step(args.warmup + i)
+    torch.cuda.synchronize()
+    # per hop: indptr pair 16 B + one candidate row id 8 B + trace write 8 B (retries of the
+    # rejection loop and the connectivity searches come on top and are not counted)
+    kernels = _kernel_table(capi, lambda name: 32 * hops * args.steps if name == "node2vec" else 0)
+    capi.profile_enable(False)
+    cpu = None
+    if args.cpu_seconds > 0:
+        from oracle import binding as orc
+        h_indptr, h_indices = indptr.cpu().numpy(), indices.cpu().numpy()
+        n = 20_000
+        h_seeds = seeds[:n].cpu().numpy()
+        orc.node2vec(h_indptr, h_indices, h_seeds[:1000], L, wl["p"], wl["q"], args.seed, 0)
+        t_cpu, h_cpu, runs = 0.0, 0, 0
+        while t_cpu < args.cpu_seconds and runs < 1000:
+            t = time.perf_counter()
+            tr = orc.node2vec(h_indptr, h_indices, h_seeds, L, wl["p"], wl["q"], args.seed, runs)
+            t_cpu += time.perf_counter() - t
+            h_cpu += int((tr[1:] >= 0).sum())
+            runs += 1
+        cpu = dict(value=round(h_cpu / t_cpu, 1), unit="hops/s", cores=orc.num_threads(),
+                   kind="port", sample=f"{runs} runs of the first {n} walks ({L} steps each) in "
+                                       f"{t_cpu:.1f} s, OpenMP oracle", host_cpus=os.cpu_count())
+    value = hops * args.steps / elapsed
+    return {
+        "metric": "walk_hops_per_sec", "value": round(value, 1), "unit": "hops/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(elapsed / args.steps * 1e3, 3), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "int64", "data": "synthetic",
+        "config": {"workload": f"{args.workload}: {wl['desc']}", "walks": wl["walks"],
+                   "walk_length": L, "p": wl["p"], "q": wl["q"], "hops_per_step": hops},
+        "roofline": _roofline(kernels[0]), "cpu_baseline": cpu,
+        "gpu_over_cpu": round(value / cpu["value"], 1) if cpu else None,
+        "kernels": kernels, "graph_build_s": round(t_build, 1),
+    }
+
+
+def ladies_sampler(A, seeds, fanouts):
+    """The layer-wise sampler of the reference's examples/ladies/ladies.py:7-21."""
+    ret = []
+    for K in fanouts:
+        subA = A[:, seeds]
+        subA.edata["p"] = subA.edata["w"] ** 2
+        prob = subA.sum("p", axis=1)
+        sampleA, select_index = subA.collective_sampling(K, prob, False)
+        sampleA = sampleA.div("w", prob[select_index], axis=1)
+        out = sampleA.sum("w", axis=0)
+        sampleA = sampleA.div("w", out, axis=0)
+        seeds = sampleA.all_nodes()
+        ret.append(sampleA.to_dgl_block(prefetch_edata={"w"}))
+    return seeds, ret
+
+
+def run_ladies(args, wl, capi, dev):
+    """LADIES through the Python Matrix API and the torch custom class (the
+    whole drop-in stack), compiled with gs.jit.compile.  A step = one 2-layer sample."""
+    import torch
+    import gsampler_amd as gs
+    from gsampler_amd.utils import chung_lu_csc
+    t0 = time.time()
+    indptr, indices = chung_lu_csc(wl["nodes"], wl["edges"], seed=1, device=dev)
+    g = torch.Generator(device=dev)
+    g.manual_seed(4)
+    w = 1.0 - torch.rand(indices.numel(), generator=g, device=dev, dtype=torch.float32)
+    A = gs.Matrix()
+    A.load_graph("CSC", [indptr, indices])
+    A.edata["w"] = w
+    seeds = torch.randperm(wl["nodes"], generator=g, device=dev)[:wl["seeds"]]
+    fanouts = wl["fanouts"]
+    compiled = gs.jit.compile(ladies_sampler, (A, seeds, fanouts))
+    torch.cuda.synchronize()
+    t_build = time.time() - t0
+
+    def step():
+        _, blocks = compiled(A, seeds, fanouts)
+        return blocks
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    edges = 0
+    for _ in range(args.steps):
+        blocks = step()
+        edges += sum(int(b.num_edges()) for b in blocks)
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    capi.profile_reset()
+    capi.profile_enable(True)
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    kernels = _kernel_table(capi, lambda name: 0)
+    capi.profile_enable(False)
+    sliced = [int(b.num_edges()) for b in blocks]
+    return {
+        "metric": "sampled_edges_per_sec", "value": round(edges / elapsed, 1), "unit": "edges/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(elapsed / args.steps * 1e3, 3), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": f"{args.workload}: {wl['desc']}", "fanouts": fanouts,
+                   "seeds": wl["seeds"], "block_edges_last_step": sliced},
+        "roofline": _roofline(kernels[0]), "cpu_baseline": None, "gpu_over_cpu": None,
+        "kernels": kernels, "graph_build_s": round(t_build, 1),
+    }
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -106,6 +267,10 @@ def main():
     capi.lib()  # fail loudly when the kernel library is missing
     dev = torch.device("cuda:0")
     wl = WORKLOADS[args.workload]
+    if wl.get("kind") == "node2vec":
+        return print(json.dumps(run_node2vec(args, wl, capi, dev)))
+    if wl.get("kind") == "ladies":
+        return print(json.dumps(run_ladies(args, wl, capi, dev)))
 
     t0 = time.time()
     gen = chung_lu_csc if wl["gen"] == "chung_lu" else rmat_csc

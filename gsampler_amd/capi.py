@@ -62,10 +62,13 @@ SIGNATURES = {
                         _i64, _i64, _i64, _i64, _p, _p, _p]),
     "gs_fused_u_op_v": (_int, [_int, _p, _p, _i64, _i64, _int, _int, _p, _p, _p, _p, _p,
                                _p, _i64, _i64, _i64, _i64, _p, _p, _p]),
+    "gs_spmm_workspace_bytes": (_sz, [_int, _i64, _i64]),
     "gs_spmm": (_int, [_int, _p, _p, _i64, _i64, _p, _int, _int, _p, _p, _p, _p, _p, _int,
-                       _i64, _i64, _i64, _p, _p, _p]),
-    "gs_e_square_sum": (_int, [_int, _p, _p, _i64, _i64, _p, _p, _p, _int, _i64, _p]),
-    "gs_e_div_u_sum": (_int, [_int, _p, _p, _i64, _i64, _p, _p, _p, _p, _int, _i64, _p]),
+                       _i64, _i64, _i64, _p, _p, _i64, _p, _sz, _p]),
+    "gs_e_square_sum": (_int, [_int, _p, _p, _i64, _i64, _p, _p, _p, _int, _i64, _i64, _p,
+                               _sz, _p]),
+    "gs_e_div_u_sum": (_int, [_int, _p, _p, _i64, _i64, _p, _p, _p, _p, _int, _i64, _i64,
+                              _p, _sz, _p]),
     "gs_minor_slice_workspace_bytes": (_sz, [_i64, _i64]),
     "gs_minor_slice_count": (_int, [_p, _i64, _p, _i64, _p, _i64, _p, _p, _p, _sz, _p]),
     "gs_minor_slice_fill": (_int, [_p, _i64, _i64, _p, _i64, _p, _p, _p, _p, _p, _sz, _p]),
@@ -375,6 +378,10 @@ def fused_u_op_v(view, op, lhs1, rhs1, lhs2, rhs2):
     return out1, out2
 
 
+def _spmm_workspace(fmt, nnz, n_out, device):
+    return _workspace(lib().gs_spmm_workspace_bytes(fmt, nnz, n_out), device)
+
+
 def spmm(view, op, reduce, ufeat, efeat, u_target, n_out, edge_map=None, want_arg=False):
     fmt, a, b, nmaj, nnz = _view(view)
     ufeat, ulen = _feat(ufeat)
@@ -387,10 +394,11 @@ def spmm(view, op, reduce, ufeat, efeat, u_target, n_out, edge_map=None, want_ar
     if want_arg:
         arg_u = torch.zeros(shape, dtype=torch.int64, device=ref.device)
         arg_e = torch.zeros(shape, dtype=torch.int64, device=ref.device)
+    ws = _spmm_workspace(fmt, nnz, n_out, out.device)
     check(lib().gs_spmm(fmt, _ptr(a), _ptr(b), nmaj, nnz, _ptr(edge_map), OPS[op],
                         REDUCERS[reduce], _fptr(ufeat), _fptr(efeat), _fptr(out),
                         _ptr(arg_u), _ptr(arg_e), u_target, ulen, elen, flen, None, None,
-                        _stream()))
+                        n_out, ws.data_ptr(), ws.numel(), _stream()))
     return (out, arg_u, arg_e) if want_arg else out
 
 
@@ -399,8 +407,10 @@ def e_square_sum(view, efeat, u_target, n_out, edge_map=None):
     efeat, elen = _feat(efeat)
     shape = (n_out,) if efeat.dim() == 1 else (n_out, elen)
     out = torch.zeros(shape, dtype=torch.float32, device=efeat.device)
+    ws = _spmm_workspace(fmt, nnz, n_out, out.device)
     check(lib().gs_e_square_sum(fmt, _ptr(a), _ptr(b), nmaj, nnz, _ptr(edge_map),
-                                _fptr(efeat), _fptr(out), u_target, elen, _stream()))
+                                _fptr(efeat), _fptr(out), u_target, elen, n_out,
+                                ws.data_ptr(), ws.numel(), _stream()))
     return out
 
 
@@ -410,9 +420,10 @@ def e_div_u_sum(view, ufeat, efeat, u_target, n_out, edge_map=None):
     efeat, elen = _feat(efeat)
     shape = (n_out,) if efeat.dim() == 1 else (n_out, elen)
     out = torch.zeros(shape, dtype=torch.float32, device=efeat.device)
+    ws = _spmm_workspace(fmt, nnz, n_out, out.device)
     check(lib().gs_e_div_u_sum(fmt, _ptr(a), _ptr(b), nmaj, nnz, _ptr(edge_map),
                                _fptr(ufeat), _fptr(efeat), _fptr(out), u_target, elen,
-                               _stream()))
+                               n_out, ws.data_ptr(), ws.numel(), _stream()))
     return out
 
 

@@ -130,6 +130,13 @@ __device__ __forceinline__ uint64_t philox_bounded(PhiloxKey key, uint64_t pos,
 // ------------------------------------------------------------- wave helpers
 __device__ __forceinline__ int lane_id() { return (int)__lane_id(); }
 
+// The first active lane's value, in every lane.
+__device__ __forceinline__ int64_t wave_uniform_first(int64_t v) {
+  const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v);
+  const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)((uint64_t)v >> 32));
+  return (int64_t)(((uint64_t)hi << 32) | lo);
+}
+
 // Inclusive scan across the 64 lanes of a wavefront.
 template <typename T>
 __device__ __forceinline__ T wave_inclusive_sum(T v) {

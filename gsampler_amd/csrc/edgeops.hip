@@ -258,6 +258,172 @@ __global__ __launch_bounds__(kBlock) void spmm_csc_kernel(
   }
 }
 
+// ------------------------------------------------- load-balanced scalar sums
+// The sums of layer-wise samplers run over slices of power-law graphs: one
+// column (or row) can hold a large share of all edges.  Both kernels below are
+// edge-parallel, combine inside LDS what a tile of edges adds to the same
+// output, and send one atomic per (tile, output) to memory.
+constexpr int kSumItems = 8;
+constexpr int kSumTile = kBlock * kSumItems;
+constexpr int kSumSegs = 2048;   // segments one tile can accumulate in LDS
+constexpr int kCooSlots = 4096;  // combining table of the coordinate kernel
+constexpr int kDies = 8;         // accelerator dies of an MI355X, one L2 each
+constexpr int64_t kPrivateMinEdges = 1 << 20;
+
+// out[i] += sum of the per-die copies; the copies were zero-filled before.
+__global__ __launch_bounds__(kBlock) void spmm_fold_kernel(
+    const float* __restrict__ copies, int64_t n, float* __restrict__ out) {
+  const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (i >= n) return;
+  float acc = 0.f;
+#pragma unroll
+  for (int d = 0; d < kDies; ++d) acc += copies[d * n + i];
+  if (acc != 0.f) out[i] += acc;
+}
+
+__global__ __launch_bounds__(kBlock) void spmm_zero_kernel(float* p, int64_t n) {
+  for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n;
+       i += (int64_t)gridDim.x * kBlock)
+    p[i] = 0.f;
+}
+
+// Per-die copies pay off when there are many edges per output row.
+static size_t private_bytes(int format, int64_t nnz, int64_t num_out) {
+  if (format != GS_FMT_COO || nnz < kPrivateMinEdges || num_out <= 0 ||
+      num_out > nnz / 4)
+    return 0;
+  return (size_t)kDies * (size_t)num_out * sizeof(float);
+}
+
+// Sum of v over the wavefront if every lane is active and targets the same
+// output (then *uniform is set and lane 0 should add the result).
+__device__ __forceinline__ float wave_sum_if_uniform(float v, int64_t target,
+                                                     bool active, bool* uniform) {
+  const int64_t t0 = wave_uniform_first(target);
+  *uniform = __all(active && target == t0);
+  if (!*uniform) return v;
+#pragma unroll
+  for (int d = kWave / 2; d > 0; d >>= 1) v += __shfl_down(v, d, kWave);
+  return v;
+}
+
+// Compressed form: tile of consecutive edges; the segments it touches are
+// consecutive, so LDS accumulators are indexed directly.
+__global__ __launch_bounds__(kBlock) void spmm_csc_sum_kernel(
+    const int64_t* __restrict__ indptr, const int64_t* __restrict__ indices,
+    const int64_t* __restrict__ edge_map, int64_t num_major, int64_t nnz,
+    int kind, int op, const float* __restrict__ ufeat,
+    const float* __restrict__ efeat, float* out) {
+  __shared__ float acc[kSumSegs];
+  __shared__ int64_t bounds[kSumSegs + 1];
+  const int64_t tile0 = (int64_t)blockIdx.x * kSumTile;
+  const int64_t tile_end = tile0 + kSumTile < nnz ? tile0 + kSumTile : nnz;
+  const int64_t c0 = segment_of(indptr, num_major, tile0);
+  const int64_t c1 = segment_of(indptr, num_major, tile_end - 1);
+  const int64_t nseg = c1 - c0 + 1;
+  const bool in_lds = nseg <= kSumSegs;
+  if (in_lds) {
+    for (int64_t j = threadIdx.x; j <= nseg; j += kBlock) {
+      bounds[j] = indptr[c0 + j];
+      if (j < nseg) acc[j] = 0.f;
+    }
+    __syncthreads();
+  }
+  float val[kSumItems];
+#pragma unroll
+  for (int i = 0; i < kSumItems; ++i) {  // loads first: in flight together
+    const int64_t e = tile0 + i * kBlock + threadIdx.x;
+    val[i] = 0.f;
+    if (e < tile_end) {
+      const int64_t eid = edge_map ? edge_map[e] : e;
+      val[i] = edge_value<float>(kind, op, ufeat ? ufeat + indices[e] : nullptr,
+                                 efeat ? efeat + eid : nullptr);
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < kSumItems; ++i) {
+    const int64_t e = tile0 + i * kBlock + threadIdx.x;
+    const bool active = e < tile_end;
+    int64_t seg = 0;
+    if (active)
+      seg = in_lds ? segment_of(bounds, nseg, e) : segment_of(indptr + c0, nseg, e);
+    bool uniform;
+    const float total = wave_sum_if_uniform(val[i], seg, active, &uniform);
+    if (uniform) {
+      if (lane_id() == 0) {
+        if (in_lds) atomicAdd(&acc[seg], total);
+        else unsafeAtomicAdd(out + c0 + seg, total);
+      }
+    } else if (active) {
+      if (in_lds) atomicAdd(&acc[seg], val[i]);
+      else unsafeAtomicAdd(out + c0 + seg, val[i]);
+    }
+  }
+  if (!in_lds) return;
+  __syncthreads();
+  for (int64_t j = threadIdx.x; j < nseg; j += kBlock)
+    if (acc[j] != 0.f) unsafeAtomicAdd(out + c0 + j, acc[j]);
+}
+
+// Coordinate form: outputs arrive in any order, so the tile combines them in
+// a small LDS hash table; an edge that finds no slot within a few probes adds
+// to memory directly.
+__global__ __launch_bounds__(kBlock) void spmm_coo_sum_kernel(
+    const int64_t* __restrict__ row, const int64_t* __restrict__ col,
+    const int64_t* __restrict__ edge_map, int64_t nnz, int kind, int op,
+    const float* __restrict__ ufeat, const float* __restrict__ efeat, float* out,
+    int u_target, int64_t copy_stride) {
+  __shared__ long long keys[kCooSlots];
+  __shared__ float vals[kCooSlots];
+  for (int j = threadIdx.x; j < kCooSlots; j += kBlock) {
+    keys[j] = -1;
+    vals[j] = 0.f;
+  }
+  __syncthreads();
+  // consecutive work-groups run on consecutive dies: with copy_stride > 0 every
+  // die adds to a copy of its own
+  out += (int64_t)(blockIdx.x % kDies) * copy_stride;
+  const int64_t tile0 = (int64_t)blockIdx.x * kSumTile;
+  const int64_t* dst_ids = u_target == 0 ? col : row;
+  const int64_t* src_ids = u_target == 0 ? row : col;
+  // all loads of the tile first, so that they are in flight together
+  int64_t dst[kSumItems];
+  float val[kSumItems];
+#pragma unroll
+  for (int i = 0; i < kSumItems; ++i) {
+    const int64_t e = tile0 + i * kBlock + threadIdx.x;
+    dst[i] = -1;
+    val[i] = 0.f;
+    if (e < nnz) {
+      dst[i] = dst_ids[e];
+      const int64_t eid = edge_map ? edge_map[e] : e;
+      val[i] = edge_value<float>(kind, op, ufeat ? ufeat + src_ids[e] : nullptr,
+                                 efeat ? efeat + eid : nullptr);
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < kSumItems; ++i) {
+    if (dst[i] < 0) continue;
+    uint32_t slot =
+        (uint32_t)(((uint64_t)dst[i] * 0x9E3779B97F4A7C15ull) >> 40) & (kCooSlots - 1);
+    bool placed = false;
+    for (int probe = 0; probe < 8 && !placed; ++probe) {
+      long long k = keys[slot];
+      if (k == -1) k = (long long)atomicCAS((unsigned long long*)&keys[slot],
+                                            ~0ull, (unsigned long long)dst[i]);
+      if (k == -1 || k == (long long)dst[i]) {
+        atomicAdd(&vals[slot], val[i]);
+        placed = true;
+      }
+      slot = (slot + 1) & (kCooSlots - 1);
+    }
+    if (!placed) unsafeAtomicAdd(out + dst[i], val[i]);
+  }
+  __syncthreads();
+  for (int j = threadIdx.x; j < kCooSlots; j += kBlock)
+    if (keys[j] != -1) unsafeAtomicAdd(out + keys[j], vals[j]);
+}
+
 static int check_view(int format, const int64_t* a, const int64_t* b,
                       int64_t num_major, int64_t nnz, const char* who) {
   GS_REQUIRE(format == GS_FMT_COO || format == GS_FMT_COMPRESSED,
@@ -273,8 +439,43 @@ static int spmm_launch(int format, const int64_t* a, const int64_t* b,
                        const float* efeat, float* out, int64_t* arg_u,
                        int64_t* arg_e, int u_target, int64_t ufeat_len,
                        int64_t efeat_len, int64_t out_len, const int64_t* u_off,
-                       const int64_t* e_off, hipStream_t s) {
+                       const int64_t* e_off, int64_t num_out, void* workspace,
+                       size_t workspace_bytes, hipStream_t s) {
   if (nnz == 0 || out_len == 0) return GS_OK;
+  const bool scalar = out_len == 1 && (ufeat == nullptr || ufeat_len == 1) &&
+                      (efeat == nullptr || efeat_len == 1);
+  if (scalar && reduce == kReduceSum) {
+    const dim3 grid((unsigned)ceil_div(nnz, kSumTile));
+    if (format == GS_FMT_COO) {
+      const size_t need = private_bytes(format, nnz, num_out);
+      if (need > 0 && workspace != nullptr && workspace_bytes >= need) {
+        float* copies = (float*)workspace;
+        const int64_t total = (int64_t)kDies * num_out;
+        int64_t zb = ceil_div(total, kBlock * 4);
+        if (zb > 4096) zb = 4096;
+        GS_LAUNCH("spmm_zero", s,
+                  spmm_zero_kernel<<<dim3((unsigned)zb), dim3(kBlock), 0, s>>>(
+                      copies, total));
+        GS_LAUNCH("spmm_coo_sum", s,
+                  spmm_coo_sum_kernel<<<grid, dim3(kBlock), 0, s>>>(
+                      a, b, edge_map, nnz, kind, op, ufeat, efeat, copies,
+                      u_target, num_out));
+        GS_LAUNCH("spmm_fold", s,
+                  spmm_fold_kernel<<<dim3((unsigned)ceil_div(num_out, kBlock)),
+                                     dim3(kBlock), 0, s>>>(copies, num_out, out));
+        return GS_OK;
+      }
+      GS_LAUNCH("spmm_coo_sum", s,
+                spmm_coo_sum_kernel<<<grid, dim3(kBlock), 0, s>>>(
+                    a, b, edge_map, nnz, kind, op, ufeat, efeat, out, u_target,
+                    (int64_t)0));
+    } else {
+      GS_LAUNCH("spmm_csc_sum", s,
+                spmm_csc_sum_kernel<<<grid, dim3(kBlock), 0, s>>>(
+                    a, b, edge_map, num_major, nnz, kind, op, ufeat, efeat, out));
+    }
+    return GS_OK;
+  }
   if (format == GS_FMT_COO) {
     const int64_t total = nnz * out_len;
     GS_LAUNCH("spmm_coo", s,
@@ -290,8 +491,6 @@ static int spmm_launch(int format, const int64_t* a, const int64_t* b,
                     u_target, ufeat_len, efeat_len, out_len, u_off, e_off));
     return GS_OK;
   }
-  const bool scalar = out_len == 1 && (ufeat == nullptr || ufeat_len == 1) &&
-                      (efeat == nullptr || efeat_len == 1);
   if (scalar) {
     const int64_t avg = nnz / (num_major > 0 ? num_major : 1);
 #define GS_SPMM_SCALAR(G)                                                      \
@@ -391,11 +590,16 @@ int gs_fused_u_op_v(int format, const int64_t* a, const int64_t* b,
   return GS_OK;
 }
 
+size_t gs_spmm_workspace_bytes(int format, int64_t nnz, int64_t num_out) {
+  return gs::private_bytes(format, nnz, num_out);
+}
+
 int gs_spmm(int format, const int64_t* a, const int64_t* b, int64_t num_major,
             int64_t nnz, const int64_t* edge_map, int op, int reduce,
             const float* ufeat, const float* efeat, float* out, int64_t* arg_u,
             int64_t* arg_e, int u_target, int64_t ufeat_len, int64_t efeat_len,
             int64_t out_len, const int64_t* u_off, const int64_t* e_off,
+            int64_t num_out, void* workspace, size_t workspace_bytes,
             gs_stream_t stream) {
   using namespace gs;
   int rc = check_view(format, a, b, num_major, nnz, "spmm");
@@ -410,13 +614,14 @@ int gs_spmm(int format, const int64_t* a, const int64_t* b, int64_t num_major,
                      op == kOpCopyRhs ? nullptr : ufeat,
                      op == kOpCopyLhs ? nullptr : efeat, out, arg_u, arg_e,
                      u_target, ufeat_len, efeat_len, out_len, u_off, e_off,
-                     as_stream(stream));
+                     num_out, workspace, workspace_bytes, as_stream(stream));
 }
 
 int gs_e_square_sum(int format, const int64_t* a, const int64_t* b,
                     int64_t num_major, int64_t nnz, const int64_t* edge_map,
                     const float* efeat, float* out, int u_target,
-                    int64_t feat_len, gs_stream_t stream) {
+                    int64_t feat_len, int64_t num_out, void* workspace,
+                    size_t workspace_bytes, gs_stream_t stream) {
   using namespace gs;
   int rc = check_view(format, a, b, num_major, nnz, "e_square_sum");
   if (rc != GS_OK) return rc;
@@ -425,13 +630,15 @@ int gs_e_square_sum(int format, const int64_t* a, const int64_t* b,
   GS_REQUIRE(efeat && out, "e_square_sum: null operand");
   return spmm_launch(format, a, b, num_major, nnz, edge_map, 1, kOpCopyRhs,
                      kReduceSum, nullptr, efeat, out, nullptr, nullptr, u_target,
-                     0, feat_len, feat_len, nullptr, nullptr, as_stream(stream));
+                     0, feat_len, feat_len, nullptr, nullptr, num_out, workspace,
+                     workspace_bytes, as_stream(stream));
 }
 
 int gs_e_div_u_sum(int format, const int64_t* a, const int64_t* b,
                    int64_t num_major, int64_t nnz, const int64_t* edge_map,
                    const float* ufeat, const float* efeat, float* out,
-                   int u_target, int64_t feat_len, gs_stream_t stream) {
+                   int u_target, int64_t feat_len, int64_t num_out,
+                   void* workspace, size_t workspace_bytes, gs_stream_t stream) {
   using namespace gs;
   int rc = check_view(format, a, b, num_major, nnz, "e_div_u_sum");
   if (rc != GS_OK) return rc;
@@ -440,8 +647,8 @@ int gs_e_div_u_sum(int format, const int64_t* a, const int64_t* b,
   GS_REQUIRE(ufeat && efeat && out, "e_div_u_sum: null operand");
   return spmm_launch(format, a, b, num_major, nnz, edge_map, 2, kOpDiv,
                      kReduceSum, ufeat, efeat, out, nullptr, nullptr, u_target,
-                     feat_len, feat_len, feat_len, nullptr, nullptr,
-                     as_stream(stream));
+                     feat_len, feat_len, feat_len, nullptr, nullptr, num_out,
+                     workspace, workspace_bytes, as_stream(stream));
 }
 
 }  // extern "C"

@@ -184,6 +184,13 @@ static StructureArgs reduce_structure(Graph& g, const Coordinate* coo,
   return structure_of(*csx);
 }
 
+// Scratch for the per-die accumulators of a coordinate-form sum (1 byte when
+// the reduction does not use them).
+static torch::Tensor reduce_workspace(const StructureArgs& s,
+                                      const torch::Tensor& out) {
+  return new_workspace(gs_spmm_workspace_bytes(s.format, s.nnz, out.size(0)), out);
+}
+
 void Graph::SpMM(const std::string& op, const std::string& reduce,
                  torch::Tensor ufeat, torch::Tensor efeat, torch::Tensor out,
                  torch::Tensor argu, torch::Tensor arge, int64_t u_target,
@@ -201,13 +208,15 @@ void Graph::SpMM(const std::string& op, const std::string& reduce,
   const StructureArgs s = reduce_structure(
       *this, coo_.get(), on_format == kCOO ? nullptr : &compressed(on_format),
       on_format, u_target, "SpMM");
+  torch::Tensor ws = reduce_workspace(s, out);
   GS_CALL(gs_spmm(s.format, s.a, s.b, s.num_major, s.nnz, s.edge_map,
                   op_code(op), reduce_code(reduce), (const float*)fptr(ufeat),
                   (const float*)fptr(efeat), (float*)out.data_ptr(),
                   argu.defined() ? mptr(argu) : nullptr,
                   arge.defined() ? mptr(arge) : nullptr, (int)u_target,
                   bc.lhs_len, bc.rhs_len, bc.out_len, cptr(bc.lhs_off),
-                  cptr(bc.rhs_off), cur_stream()));
+                  cptr(bc.rhs_off), out.size(0), ws.data_ptr(), (size_t)ws.numel(),
+                  cur_stream()));
 }
 
 void Graph::FusedESquareSum(const std::string& op, const std::string& reduce,
@@ -227,9 +236,11 @@ void Graph::FusedESquareSum(const std::string& op, const std::string& reduce,
   const StructureArgs s = reduce_structure(
       *this, coo_.get(), on_format == kCOO ? nullptr : &compressed(on_format),
       on_format, u_target, "FusedESquareSum");
+  torch::Tensor ws = reduce_workspace(s, out);
   GS_CALL(gs_e_square_sum(s.format, s.a, s.b, s.num_major, s.nnz, s.edge_map,
                           (const float*)fptr(efeat), (float*)out.data_ptr(),
-                          (int)u_target, len, cur_stream()));
+                          (int)u_target, len, out.size(0), ws.data_ptr(),
+                          (size_t)ws.numel(), cur_stream()));
 }
 
 void Graph::FusedEDivUSum(const std::string& op, const std::string& reduce,
@@ -251,10 +262,11 @@ void Graph::FusedEDivUSum(const std::string& op, const std::string& reduce,
   const StructureArgs s = reduce_structure(
       *this, coo_.get(), on_format == kCOO ? nullptr : &compressed(on_format),
       on_format, u_target, "FusedEDivUSum");
+  torch::Tensor ws = reduce_workspace(s, out);
   GS_CALL(gs_e_div_u_sum(s.format, s.a, s.b, s.num_major, s.nnz, s.edge_map,
                          (const float*)fptr(ufeat), (const float*)fptr(efeat),
-                         (float*)out.data_ptr(), (int)u_target, len,
-                         cur_stream()));
+                         (float*)out.data_ptr(), (int)u_target, len, out.size(0),
+                         ws.data_ptr(), (size_t)ws.numel(), cur_stream()));
 }
 
 }  // namespace gs

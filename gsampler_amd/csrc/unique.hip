@@ -587,16 +587,37 @@ __global__ __launch_bounds__(kThreads) void unique_dedup_kernel(
     return;
   }
   // Many entries: fine for the LDS table while few of them are distinct (a hub
-  // that repeats thousands of times), so try, and count.
-  for (int64_t i = lo + threadIdx.x; i < hi; i += kThreads) {
-    if (*(volatile uint32_t*)&overflow) break;
-    lds_insert_min_counted(tab, mask, packed[i], &distinct, &overflow);
+  // that repeats thousands of times), so try, and count.  Entries are read
+  // kDeep at a time per thread so that a long bucket streams at memory speed;
+  // the overflow flag is read before every insert, which bounds the slots
+  // claimed after it rises to one per thread.
+  constexpr int kDeep = 8;
+  volatile uint32_t* over = &overflow;
+  for (int64_t base = lo; base < hi && !*over; base += (int64_t)kThreads * kDeep) {
+    uint64_t e[kDeep];
+#pragma unroll
+    for (int j = 0; j < kDeep; ++j) {
+      const int64_t i = base + j * kThreads + threadIdx.x;
+      e[j] = i < hi ? packed[i] : kEmptySlot;
+    }
+#pragma unroll
+    for (int j = 0; j < kDeep; ++j)
+      if (e[j] != kEmptySlot && !*over)
+        lds_insert_min_counted(tab, mask, e[j], &distinct, over);
   }
   __syncthreads();
   if (!overflow) {
-    for (int64_t i = lo + threadIdx.x; i < hi; i += kThreads) {
-      const uint64_t e = packed[i];
-      first_b[(uint32_t)e] = lds_first_of(tab, mask, e >> 32);
+    for (int64_t base = lo; base < hi; base += (int64_t)kThreads * kDeep) {
+      uint64_t e[kDeep];
+#pragma unroll
+      for (int j = 0; j < kDeep; ++j) {
+        const int64_t i = base + j * kThreads + threadIdx.x;
+        e[j] = i < hi ? packed[i] : kEmptySlot;
+      }
+#pragma unroll
+      for (int j = 0; j < kDeep; ++j)
+        if (e[j] != kEmptySlot)
+          first_b[(uint32_t)e[j]] = lds_first_of(tab, mask, e[j] >> 32);
     }
     return;
   }
@@ -624,9 +645,7 @@ __global__ __launch_bounds__(kThreads) void unique_dedup_kernel(
 // A value that is the same in every lane, moved to scalar registers so that
 // what is computed from it (the batch search) runs on the scalar unit.
 __device__ __forceinline__ int64_t wave_uniform(int64_t v) {
-  const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v);
-  const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)((uint64_t)v >> 32));
-  return (int64_t)(((uint64_t)hi << 32) | lo);
+  return wave_uniform_first(v);
 }
 
 // Batches that a chunk of consecutive items may touch: from the batch of its
@@ -770,11 +789,17 @@ __global__ __launch_bounds__(kBlock) void unique_relabel_kernel(
   int64_t col[kRelabelItems];
   uint32_t row_first[kRelabelItems];
   BatchInfo info = batch[span.lo];
+  // Seeds of a batch are distinct <=> its last seed is a first occurrence of
+  // rank ns - 1; the label of seed c is then its place among the seeds.
+  const bool one_batch = span.lo == span.hi;
+  bool seeds_distinct = false;
+  if (one_batch && out_col && info.ns > 0)
+    seeds_distinct = rank[info.fb + info.ns - 1] == (int32_t)(info.ns - 1);
 #pragma unroll
   for (int i = 0; i < kRelabelItems; ++i) {
     const int64_t e = e0 + i * kBlock + threadIdx.x;
     if (e >= k.E) break;
-    if (span.lo != span.hi) info = batch[batch_in_span(k.rows_ptr, span, e)];
+    if (!one_batch) info = batch[batch_in_span(k.rows_ptr, span, e)];
     // row key e of batch b sits at flat position
     //   fb + (seeds of b) + (e - rows_ptr[b])  =  e + seeds_ptr[b + 1]
     if (out_row) row_first[i] = first[e + info.s_lo + info.ns];
@@ -784,10 +809,12 @@ __global__ __launch_bounds__(kBlock) void unique_relabel_kernel(
   for (int i = 0; i < kRelabelItems; ++i) {
     const int64_t e = e0 + i * kBlock + threadIdx.x;
     if (e >= k.E) break;
-    if (span.lo != span.hi) info = batch[batch_in_span(k.rows_ptr, span, e)];
+    if (!one_batch) info = batch[batch_in_span(k.rows_ptr, span, e)];
     if (out_row) out_row[e] = rank[info.fb + row_first[i]];
     // seed c of batch b sits at flat position c + rows_ptr[b]
-    if (out_col) out_col[e] = rank[info.fb + first[col[i] + info.r_lo]];
+    if (out_col)
+      out_col[e] = seeds_distinct ? col[i] - info.s_lo
+                                  : rank[info.fb + first[col[i] + info.r_lo]];
   }
 }
 

@@ -89,7 +89,11 @@ __global__ __launch_bounds__(kBlock) void node2vec_kernel(
           double h = 1.0;
           if (cand == last) {
             h = p;
-          } else if (last >= 0 && last < num_cols) {
+          } else if (((double)y < q) != ((double)y < 1.0) && last >= 0 &&
+                     last < num_cols) {
+            // the verdict differs between a neighbour of the previous node
+            // (h = q) and any other node (h = 1) only for levels between q and
+            // 1; everywhere else the adjacency search would change nothing
             const int64_t ls = indptr[last];
             if (sorted_contains(indices + ls, indptr[last + 1] - ls, cand)) h = q;
           }

@@ -352,7 +352,11 @@ int gs_split_indptr(const int64_t* indptr, const int64_t* offset,
  * gs_spmm: out[dst] = reduce(out[dst], op(u[src], e[eid])), fp32.  Outputs
  *   are accumulators: the caller zero-fills them (python/gs/ops/spmm.py:56).
  *   COO: u_target 0 reduces onto columns, 2 onto rows (atomics).  Compressed:
- *   reduces onto the segments of indptr (no atomics); u_target is ignored.
+ *   reduces onto the segments of indptr; u_target is ignored.  num_out is the
+ *   number of output rows.  workspace is optional (NULL / 0 is always valid):
+ *   with gs_spmm_workspace_bytes(format, nnz, num_out) bytes a scalar COO sum
+ *   accumulates per accelerator die and folds the copies at the end, which
+ *   keeps its atomics inside one L2 each.
  *   SpMMCOO / SpMMCSC, src/cuda/spmm.cu:274-348.
  * gs_e_square_sum: out[dst] += sum e^2                  ESquareSumCSC/COO,
  *   src/cuda/fusion/fused_csc_e_square_sum.cu:110, fused_coo_e_square_sum.cu:13.
@@ -372,20 +376,24 @@ int gs_fused_u_op_v(int format, const int64_t* a, const int64_t* b,
                     int64_t lhs_len, int64_t rhs_len, int64_t out_len,
                     int64_t reduce_size, const int64_t* lhs_off,
                     const int64_t* rhs_off, gs_stream_t stream);
+size_t gs_spmm_workspace_bytes(int format, int64_t nnz, int64_t num_out);
 int gs_spmm(int format, const int64_t* a, const int64_t* b, int64_t num_major,
             int64_t nnz, const int64_t* edge_map, int op, int reduce,
             const float* ufeat, const float* efeat, float* out, int64_t* arg_u,
             int64_t* arg_e, int u_target, int64_t ufeat_len, int64_t efeat_len,
             int64_t out_len, const int64_t* u_off, const int64_t* e_off,
+            int64_t num_out, void* workspace, size_t workspace_bytes,
             gs_stream_t stream);
 int gs_e_square_sum(int format, const int64_t* a, const int64_t* b,
                     int64_t num_major, int64_t nnz, const int64_t* edge_map,
                     const float* efeat, float* out, int u_target,
-                    int64_t feat_len, gs_stream_t stream);
+                    int64_t feat_len, int64_t num_out, void* workspace,
+                    size_t workspace_bytes, gs_stream_t stream);
 int gs_e_div_u_sum(int format, const int64_t* a, const int64_t* b,
                    int64_t num_major, int64_t nnz, const int64_t* edge_map,
                    const float* ufeat, const float* efeat, float* out,
-                   int u_target, int64_t feat_len, gs_stream_t stream);
+                   int u_target, int64_t feat_len, int64_t num_out,
+                   void* workspace, size_t workspace_bytes, gs_stream_t stream);
 
 #ifdef __cplusplus
 }

@@ -93,6 +93,44 @@ def test_spmm_and_fusions_parity(g, fmt):
     close(o1, w1); close(o2, w2)
 
 
+@pytest.mark.parametrize("shape", ["hubs", "tiny_segments"])
+def test_scalar_sums_on_skewed_matrices(shape):
+    """The load-balanced sum kernels: a few segments that hold most of the edges
+    (and rows that most edges point to), and thousands of segments with zero or
+    one edge.  Sums of up to 10^6 fp32 terms are compared with a float64 sum at
+    1e-4 relative (the order of additions is not fixed)."""
+    rng = np.random.default_rng(31)
+    if shape == "hubs":
+        deg = np.full(40, 50)
+        deg[[3, 17]] = [1200000, 400000]     # > 2^20 edges: per-die accumulators
+        R = 3000
+        w = 1.0 / np.arange(1, R + 1) ** 1.2
+        indices = rng.choice(R, size=int(deg.sum()), p=w / w.sum())
+    else:
+        deg = rng.integers(0, 2, size=9000)
+        R = 500
+        indices = rng.integers(0, R, size=int(deg.sum()))
+    C = deg.size
+    indptr = np.concatenate([[0], np.cumsum(deg)])
+    col = np.repeat(np.arange(C), deg)
+    e = rng.random(indices.size, dtype=np.float32) + 0.1
+    u = rng.random(R, dtype=np.float32) + 0.5
+    e64 = e.astype(np.float64)
+    onto_cols = np.bincount(col, weights=e64, minlength=C)
+    onto_rows = np.bincount(indices, weights=e64, minlength=R)
+    sq_rows = np.bincount(indices, weights=e64 * e64, minlength=R)
+    div_cols = np.bincount(col, weights=e64 / u[indices], minlength=C)
+    coo, csc = ("coo", T(indices), T(col)), ("csc", T(indptr), T(indices))
+    for view in (coo, csc):
+        close(capi.spmm(view, "copy_rhs", "sum", None, T(e), 0, C), onto_cols.astype(np.float32), 1e-4)
+        close(capi.e_div_u_sum(view, T(u), T(e), 0, C), div_cols.astype(np.float32), 1e-4)
+    close(capi.spmm(coo, "copy_rhs", "sum", None, T(e), 2, R), onto_rows.astype(np.float32), 1e-4)
+    close(capi.e_square_sum(coo, T(e), 2, R), sq_rows.astype(np.float32), 1e-4)
+    # and the oracle agrees with the float64 sums as well
+    assert np.allclose(orc.spmm(("csc", indptr, indices), "copy_rhs", "sum", None, e, 0, C),
+                       onto_cols, rtol=1e-3)
+
+
 def test_matrix_sum_div_and_ops_wrappers(g):
     rng, indptr, indices, col = g
     m = gs.Matrix()
