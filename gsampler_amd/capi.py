@@ -136,6 +136,34 @@ def _workspace(nbytes: int, device) -> torch.Tensor:
     return torch.empty(max(int(nbytes), 1), dtype=torch.uint8, device=device)
 
 
+class _Count:
+    """A count on its way from the device to the host: the 8-byte copy is queued
+    on the current stream at once, the host waits only when it needs the value.
+    Kernels launched in between (into buffers sized by an upper bound) keep the
+    GPU busy meanwhile."""
+    _slots = None
+    _next = 0
+
+    def __init__(self, prefix: torch.Tensor):
+        cls = _Count
+        if cls._slots is None:
+            cls._slots = torch.empty(64, dtype=torch.int64).pin_memory()
+        self._slot = cls._slots[cls._next % 64: cls._next % 64 + 1]
+        cls._next += 1
+        self._slot.copy_(prefix[-1:], non_blocking=True)
+        self._event = torch.cuda.Event()
+        self._event.record()
+
+    def get(self) -> int:
+        self._event.synchronize()
+        return int(self._slot[0])
+
+
+# Outputs are sized by an upper bound (and trimmed afterwards) only up to this
+# many elements; beyond it the count is awaited first.
+_BOUND_LIMIT = 1 << 26
+
+
 # -------------------------------------------------------------- profiling
 def profile_enable(on: bool) -> None:
     lib().gs_profile_enable(int(on))
@@ -227,17 +255,20 @@ def sample_uniform(indptr, indices, column_ids, fanout, replace=False,
     else:
         n = num_cols
     sub_indptr = col_count(indptr, column_ids, fanout, replace, n)
-    nnz = int(sub_indptr[-1].item())
+    count = _Count(sub_indptr)
+    bound = n * fanout                       # no column yields more than fanout edges
+    size = bound if bound <= _BOUND_LIMIT else count.get()
     dev = indptr.device
-    out_idx = torch.empty(nnz, dtype=torch.int64, device=dev)
-    out_sel = torch.empty(nnz, dtype=torch.int64, device=dev)
-    out_col = torch.empty(nnz, dtype=torch.int64, device=dev) if with_coo else None
-    if nnz > 0:
+    out_idx = torch.empty(size, dtype=torch.int64, device=dev)
+    out_sel = torch.empty(size, dtype=torch.int64, device=dev)
+    out_col = torch.empty(size, dtype=torch.int64, device=dev) if with_coo else None
+    if size > 0:
         check(lib().gs_csc_col_sample_uniform_fill(
             _ptr(indptr), num_cols, _ptr(indices), _ptr(column_ids), n, fanout,
             int(replace), algo, seed, call_id, sub_indptr.data_ptr(),
             _ptr(out_col), out_idx.data_ptr(), out_sel.data_ptr(), _stream()))
-    return sub_indptr, out_col, out_idx, out_sel
+    nnz = count.get()
+    return (sub_indptr, out_col[:nnz] if with_coo else None, out_idx[:nnz], out_sel[:nnz])
 
 
 def unique_relabel(seeds, rows, seeds_ptr=None, rows_ptr=None, edge_col=None,
@@ -262,8 +293,9 @@ def unique_relabel(seeds, rows, seeds_ptr=None, rows_ptr=None, edge_col=None,
     check(l.gs_unique_count(_ptr(seeds), sp, S, _ptr(rows), rp, E, B,
                             unique_ptr.data_ptr(), ws.data_ptr(), ws.numel(),
                             _stream()))
-    U = int(unique_ptr[-1].item())
-    unique = torch.empty(U, dtype=torch.int64, device=dev)
+    count = _Count(unique_ptr)
+    size = S + E if S + E <= _BOUND_LIMIT else count.get()   # U <= S + E
+    unique = torch.empty(size, dtype=torch.int64, device=dev)
     want_col = want_col and edge_col is not None
     out_row = torch.empty(E, dtype=torch.int64, device=dev) if want_row else None
     out_col = torch.empty(E, dtype=torch.int64, device=dev) if want_col else None
@@ -276,7 +308,7 @@ def unique_relabel(seeds, rows, seeds_ptr=None, rows_ptr=None, edge_col=None,
         check(l.gs_unique_relabel(_ptr(seeds), sp, S, _ptr(rows), rp, E, B,
                                   _ptr(edge_col), _ptr(out_row), _ptr(out_col),
                                   ws.data_ptr(), ws.numel(), _stream()))
-    return unique, unique_ptr, out_row, out_col
+    return unique[:count.get()], unique_ptr, out_row, out_col
 
 
 def csc2coo(indptr: torch.Tensor, nnz: Optional[int] = None) -> torch.Tensor:

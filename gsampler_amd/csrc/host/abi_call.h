@@ -5,6 +5,7 @@
 #define GS_HOST_ABI_CALL_H_
 
 #include <c10/hip/HIPStream.h>
+#include <hip/hip_runtime_api.h>
 #include <torch/torch.h>
 
 #include "../../../include/gsampler_hip.h"
@@ -53,6 +54,64 @@ inline torch::Tensor new_workspace(size_t bytes, const torch::Tensor& like) {
 inline int64_t read_last(const torch::Tensor& prefix) {
   return prefix[prefix.numel() - 1].item<int64_t>();
 }
+
+// The same value without stalling the GPU: the copy into pinned host memory is
+// queued on the current stream at once, get() waits for it.  Work launched in
+// between (into buffers sized by an upper bound) keeps the GPU busy while the
+// value travels.  Slots come from a small per-thread ring of pinned words that
+// lives until the process ends; a slot is reused after kSlots later reads.
+class AsyncCount {
+ public:
+  AsyncCount() = default;
+  explicit AsyncCount(const torch::Tensor& prefix) {
+    Ring& r = ring();
+    slot_ = r.next++ % kSlots;
+    hipStream_t s = (hipStream_t)cur_stream();
+    const int64_t* src = prefix.data_ptr<int64_t>() + prefix.numel() - 1;
+    check(hipMemcpyAsync(r.words + slot_, src, sizeof(int64_t),
+                         hipMemcpyDeviceToHost, s));
+    check(hipEventRecord(r.events[slot_], s));
+    pending_ = true;
+  }
+  int64_t get() {
+    TORCH_CHECK(slot_ >= 0, "AsyncCount: nothing was requested");
+    Ring& r = ring();
+    if (pending_) {
+      check(hipEventSynchronize(r.events[slot_]));
+      value_ = r.words[slot_];
+      pending_ = false;
+    }
+    return value_;
+  }
+
+ private:
+  static constexpr int kSlots = 64;
+  struct Ring {
+    int64_t* words = nullptr;
+    hipEvent_t events[kSlots];
+    unsigned next = 0;
+  };
+  static void check(hipError_t e) {
+    TORCH_CHECK(e == hipSuccess, "HIP error: ", hipGetErrorString(e));
+  }
+  static Ring& ring() {
+    static thread_local Ring* r = [] {
+      Ring* x = new Ring();
+      check(hipHostMalloc((void**)&x->words, kSlots * sizeof(int64_t), hipHostMallocDefault));
+      for (int i = 0; i < kSlots; ++i)
+        check(hipEventCreateWithFlags(&x->events[i], hipEventDisableTiming));
+      return x;
+    }();
+    return *r;
+  }
+  int slot_ = -1;
+  bool pending_ = false;
+  int64_t value_ = 0;
+};
+
+// Outputs are sized by an upper bound (and trimmed afterwards) only up to this
+// many elements; beyond it the count is awaited first.
+constexpr int64_t kBoundLimit = int64_t(1) << 26;
 
 }  // namespace gs
 

@@ -174,7 +174,7 @@ Graph::BatchGraphRelabel(torch::Tensor col_seeds, torch::Tensor row_ids) {
                             mptr(out_row), mptr(out_col),
                             f.workspace.data_ptr(), f.workspace.numel(),
                             cur_stream()));
-  return {f.unique, f.unique_ptr, out_row, out_col, coo_->e_ids, edge_bptr_};
+  return {f.frontier(), f.unique_ptr, out_row, out_col, coo_->e_ids, edge_bptr_};
 }
 
 std::tuple<torch::Tensor, torch::Tensor> Graph::BatchGetValidNodes(
@@ -187,7 +187,7 @@ std::tuple<torch::Tensor, torch::Tensor> Graph::BatchGetValidNodes(
   col_seeds = ids(col_seeds, "col_seeds");
   torch::Tensor rows = batch_rows_for_relabel(row_ids);
   Frontier& f = frontier_for(col_seeds, rows, col_bptr_, edge_bptr_);
-  return {f.unique, f.unique_ptr};
+  return {f.frontier(), f.unique_ptr};
 }
 
 // ------------------------------------------------------------ free operators

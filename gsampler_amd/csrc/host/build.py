@@ -47,6 +47,7 @@ def main() -> None:
     out = os.path.join(LIB_DIR, "libgs.so")
     cmd = ["g++", "-shared", "-o", out, *objs, f"-L{torch_lib}", "-ltorch", "-ltorch_cpu",
            "-lc10", "-lc10_hip", "-ltorch_hip", f"-L{LIB_DIR}", "-lgsampler_hip",
+           "-L/opt/rocm/lib", "-lamdhip64",
            "-Wl,-rpath,$ORIGIN", f"-Wl,-rpath,{torch_lib}"]
     print("+ link", out, flush=True)
     subprocess.check_call(cmd)

@@ -172,10 +172,14 @@ MajorResult major_sample_uniform(const Compressed& m,
                            fused ? cptr(picked) : nullptr, n, fanout,
                            replace ? 1 : 0, mptr(r.indptr), ws.data_ptr(),
                            ws.numel(), cur_stream()));
-  const int64_t nnz = read_last(r.indptr);
-  r.minor_ids = new_ids(nnz, m.indptr);
-  r.select = new_ids(nnz, m.indptr);
-  if (with_coo) r.major_ids = new_ids(nnz, m.indptr);
+  // No column yields more than fanout edges: size the outputs by that bound,
+  // launch, and trim when the count has arrived.
+  AsyncCount count(r.indptr);
+  const int64_t bound = n * fanout;
+  const int64_t size = bound <= kBoundLimit ? bound : count.get();
+  r.minor_ids = new_ids(size, m.indptr);
+  r.select = new_ids(size, m.indptr);
+  if (with_coo) r.major_ids = new_ids(size, m.indptr);
   const RandomState& rs = random_state();
   GS_CALL(gs_csc_col_sample_uniform_fill(
       cptr(m.indptr), num_major, cptr(m.indices),
@@ -183,6 +187,10 @@ MajorResult major_sample_uniform(const Compressed& m,
       rs.seed, next_call_id(), cptr(r.indptr),
       with_coo ? mptr(r.major_ids) : nullptr, mptr(r.minor_ids), mptr(r.select),
       cur_stream()));
+  const int64_t nnz = count.get();
+  r.minor_ids = r.minor_ids.narrow(0, 0, nnz);
+  r.select = r.select.narrow(0, 0, nnz);
+  if (with_coo) r.major_ids = r.major_ids.narrow(0, 0, nnz);
   return r;
 }
 
@@ -313,11 +321,12 @@ Graph::Frontier& Graph::frontier_for(const torch::Tensor& seeds,
                           cptr(rows_ptr), E, B, mptr(f->unique_ptr),
                           f->workspace.data_ptr(), f->workspace.numel(),
                           cur_stream()));
-  const int64_t U = read_last(f->unique_ptr);
-  f->unique = new_ids(U, rows);
+  f->count = AsyncCount(f->unique_ptr);
+  // at most S + E unique keys
+  f->unique_buffer = new_ids(S + E <= kBoundLimit ? S + E : f->count.get(), rows);
   GS_CALL(gs_unique_fill(cptr(seeds), cptr(seeds_ptr), S, cptr(rows),
                          cptr(rows_ptr), E, B, cptr(f->unique_ptr),
-                         mptr(f->unique), f->workspace.data_ptr(),
+                         mptr(f->unique_buffer), f->workspace.data_ptr(),
                          f->workspace.numel(), cur_stream()));
   frontier_ = std::move(f);
   return *frontier_;
@@ -355,7 +364,7 @@ Graph::GraphRelabel(torch::Tensor col_seeds, torch::Tensor row_ids) {
                             mptr(out_row), mptr(out_col),
                             f.workspace.data_ptr(), f.workspace.numel(),
                             cur_stream()));
-  return {f.unique, out_row, out_col, coo_->e_ids};
+  return {f.frontier(), out_row, out_col, coo_->e_ids};
 }
 
 torch::Tensor Graph::GetValidNodes(torch::Tensor col_seeds,
@@ -369,7 +378,7 @@ torch::Tensor Graph::GetValidNodes(torch::Tensor col_seeds,
   CreateSparseFormat(kCOO);
   const torch::Tensor& base = coo_->row;
   torch::Tensor rows = mapped_rows(base, row_ids);
-  return frontier_for(col_seeds, rows, {}, {}).unique;
+  return frontier_for(col_seeds, rows, {}, {}).frontier();
 }
 
 }  // namespace gs

@@ -9,6 +9,8 @@
 #include <torch/custom_class.h>
 #include <torch/script.h>
 
+#include "abi_call.h"
+
 #include <memory>
 #include <string>
 #include <tuple>
@@ -166,10 +168,21 @@ class Graph : public torch::CustomClassHolder {
   struct Frontier {
     torch::Tensor seeds, rows, seeds_ptr, rows_ptr;  // the keys it was built from
     int64_t seeds_version = -1, rows_version = -1;
-    torch::Tensor workspace, unique, unique_ptr;
+    torch::Tensor workspace, unique_ptr;
     int64_t num_batches = 0;
+    // The unique keys: filled into a buffer sized by the upper bound, trimmed
+    // once the count has arrived (frontier() waits for it).
+    torch::Tensor unique_buffer;
+    AsyncCount count;
+    const torch::Tensor& frontier() {
+      if (!unique_.defined()) unique_ = unique_buffer.narrow(0, 0, count.get());
+      return unique_;
+    }
     bool matches(const torch::Tensor& s, const torch::Tensor& r,
                  const torch::Tensor& sp, const torch::Tensor& rp) const;
+
+   private:
+    torch::Tensor unique_;
   };
   Frontier& frontier_for(const torch::Tensor& seeds, const torch::Tensor& rows,
                          const torch::Tensor& seeds_ptr,
