@@ -43,20 +43,30 @@ WORKLOADS = {
     "c4": dict(kind="node2vec", nodes=2_450_000, edges=124_000_000, gen="chung_lu",
                walks=1_000_000, length=80, p=2.0, q=0.5,
                desc="node2vec, 1M walks x 80 steps, p=2.0 q=0.5, C2's graph with sorted columns"),
+    "c5s": dict(nodes=2_450_000, edges=124_000_000, gen="chung_lu", batches=64,
+                batch_size=1024, fanouts=[15, 10, 5], weighted=True,
+                desc="weighted GraphSAGE [15,10,5] (fp32 edge weights LogNormal(0,1)), 64 batches x "
+                     "1024 seeds, on c2's graph: a 1/13-scale stand-in for the 1.6B-edge weighted "
+                     "configuration"),
     "tiny": dict(nodes=50_000, edges=1_000_000, gen="chung_lu", batches=8,
                  batch_size=256, fanouts=[15, 10, 5],
                  desc="1/50-scale twin of c2 (smoke runs)"),
 }
 
 
-def graphsage_step(be, indptr, indices, seeds, ptr, fanouts, seed, call_base):
+def graphsage_step(be, indptr, indices, seeds, ptr, fanouts, seed, call_base, probs=None):
     """The pipeline, written once for both back ends (`be` is gsampler_amd.capi
-    on torch CUDA tensors or oracle.binding on numpy arrays).
+    on torch CUDA tensors or oracle.binding on numpy arrays).  With `probs`
+    (fp32 per edge) neighbours are drawn by weight instead of uniformly.
     Returns per-layer (S, E, U) and the last layer's outputs."""
     sizes, last = [], None
     for layer, fanout in enumerate(fanouts):
-        sub_indptr, coo_col, rows, sel = be.sample_uniform(
-            indptr, indices, seeds, fanout, False, 0, seed, call_base + layer)
+        if probs is None:
+            sub_indptr, coo_col, rows, sel = be.sample_uniform(
+                indptr, indices, seeds, fanout, False, 0, seed, call_base + layer)
+        else:
+            sub_indptr, coo_col, rows, sel = be.sample_weighted(
+                indptr, indices, probs, seeds, fanout, False, seed, call_base + layer)
         edge_ptr = sub_indptr[ptr]
         uniq, uniq_ptr, out_row, out_col = be.unique_relabel(
             seeds, rows, ptr, edge_ptr, coo_col)
@@ -78,6 +88,7 @@ def kernel_bytes(name, sizes):
         N = S + E
         total += {
             "sample_uniform": 32 * S + 32 * E,   # seeds, indptr pair, sub_indptr, gather, 3 outputs
+            "sample_weighted": 32 * S + 32 * E,  # the same, plus 4 bytes per edge of every column (not known here)
             "col_count": 32 * S,                 # seeds, indptr pair, counts
             "unique_hist": 8 * N,                # keys in
             "unique_scatter": 16 * N,            # keys in, packed entries out
@@ -279,6 +290,11 @@ def main():
     torch.cuda.synchronize()
     t_build = time.time() - t0
     fanouts = wl["fanouts"]
+    probs = None
+    if wl.get("weighted"):
+        g = torch.Generator(device=dev)
+        g.manual_seed(5)
+        probs = torch.randn(indices.numel(), generator=g, device=dev).exp_().float()
 
     # One plain streaming kernel of known size (reads 256 MiB, writes 256 MiB):
     # the yardstick that hardware traffic counters of a profiled run are scaled by.
@@ -288,7 +304,7 @@ def main():
 
     def step(i):
         return graphsage_step(capi, indptr, indices, seeds, ptr, fanouts, args.seed,
-                              i * len(fanouts))
+                              i * len(fanouts), probs)
 
     for i in range(args.warmup):
         step(i)
@@ -344,11 +360,12 @@ def main():
         from oracle import binding as orc
         h_indptr, h_indices = indptr.cpu().numpy(), indices.cpu().numpy()
         h_seeds, h_ptr = seeds.cpu().numpy(), ptr.cpu().numpy()
+        h_probs = probs.cpu().numpy() if probs is not None else None
 
         def cpu_run(call_base):
             t = time.perf_counter()
             sz, _ = graphsage_step(orc, h_indptr, h_indices, h_seeds, h_ptr, fanouts,
-                                   args.seed, call_base)
+                                   args.seed, call_base, h_probs)
             return time.perf_counter() - t, sum(E for _, E, _ in sz)
 
         cpu_run(0)  # warm-up (page in the graph, spin up the thread pool)
