@@ -45,7 +45,7 @@ WORKLOADS = {
                desc="node2vec, 1M walks x 80 steps, p=2.0 q=0.5, C2's graph with sorted columns"),
     "c5s": dict(nodes=2_450_000, edges=124_000_000, gen="chung_lu", batches=64,
                 batch_size=1024, fanouts=[15, 10, 5], weighted=True,
-                desc="weighted GraphSAGE [15,10,5] (fp32 edge weights LogNormal(0,1)), 64 batches x "
+                desc="weighted GraphSAGE [15,10,5] (fp32 edge weights LogNormal(0,1), persistent CDF), 64 batches x "
                      "1024 seeds, on c2's graph: a 1/13-scale stand-in for the 1.6B-edge weighted "
                      "configuration"),
     "tiny": dict(nodes=50_000, edges=1_000_000, gen="chung_lu", batches=8,
@@ -54,10 +54,12 @@ WORKLOADS = {
 }
 
 
-def graphsage_step(be, indptr, indices, seeds, ptr, fanouts, seed, call_base, probs=None):
+def graphsage_step(be, indptr, indices, seeds, ptr, fanouts, seed, call_base, probs=None,
+                   cdf=None):
     """The pipeline, written once for both back ends (`be` is gsampler_amd.capi
     on torch CUDA tensors or oracle.binding on numpy arrays).  With `probs`
-    (fp32 per edge) neighbours are drawn by weight instead of uniformly.
+    (fp32 per edge) neighbours are drawn by weight instead of uniformly, through
+    the matrix's persistent CDF when `cdf` is given.
     Returns per-layer (S, E, U) and the last layer's outputs."""
     sizes, last = [], None
     for layer, fanout in enumerate(fanouts):
@@ -66,7 +68,8 @@ def graphsage_step(be, indptr, indices, seeds, ptr, fanouts, seed, call_base, pr
                 indptr, indices, seeds, fanout, False, 0, seed, call_base + layer)
         else:
             sub_indptr, coo_col, rows, sel = be.sample_weighted(
-                indptr, indices, probs, seeds, fanout, False, seed, call_base + layer)
+                indptr, indices, probs, seeds, fanout, False, seed, call_base + layer,
+                cdf=cdf)
         edge_ptr = sub_indptr[ptr]
         uniq, uniq_ptr, out_row, out_col = be.unique_relabel(
             seeds, rows, ptr, edge_ptr, coo_col)
@@ -88,7 +91,7 @@ def kernel_bytes(name, sizes):
         N = S + E
         total += {
             "sample_uniform": 32 * S + 32 * E,   # seeds, indptr pair, sub_indptr, gather, 3 outputs
-            "sample_weighted": 32 * S + 32 * E,  # the same, plus 4 bytes per edge of every column (not known here)
+            "sample_weighted_cdf": 32 * S + 32 * E,  # the same interface as the uniform sampler
             "col_count": 32 * S,                 # seeds, indptr pair, counts
             "unique_hist": 8 * N,                # keys in
             "unique_scatter": 16 * N,            # keys in, packed entries out
@@ -290,11 +293,17 @@ def main():
     torch.cuda.synchronize()
     t_build = time.time() - t0
     fanouts = wl["fanouts"]
-    probs = None
+    probs = cdf = None
+    t_cdf = 0.0
     if wl.get("weighted"):
         g = torch.Generator(device=dev)
         g.manual_seed(5)
         probs = torch.randn(indices.numel(), generator=g, device=dev).exp_().float()
+        torch.cuda.synchronize()
+        t0 = time.time()
+        cdf = capi.weight_cdf(indptr, probs)      # once per (graph, weights)
+        torch.cuda.synchronize()
+        t_cdf = time.time() - t0
 
     # One plain streaming kernel of known size (reads 256 MiB, writes 256 MiB):
     # the yardstick that hardware traffic counters of a profiled run are scaled by.
@@ -304,7 +313,7 @@ def main():
 
     def step(i):
         return graphsage_step(capi, indptr, indices, seeds, ptr, fanouts, args.seed,
-                              i * len(fanouts), probs)
+                              i * len(fanouts), probs, cdf)
 
     for i in range(args.warmup):
         step(i)
@@ -361,11 +370,12 @@ def main():
         h_indptr, h_indices = indptr.cpu().numpy(), indices.cpu().numpy()
         h_seeds, h_ptr = seeds.cpu().numpy(), ptr.cpu().numpy()
         h_probs = probs.cpu().numpy() if probs is not None else None
+        h_cdf = cdf.cpu().numpy() if cdf is not None else None
 
         def cpu_run(call_base):
             t = time.perf_counter()
             sz, _ = graphsage_step(orc, h_indptr, h_indices, h_seeds, h_ptr, fanouts,
-                                   args.seed, call_base, h_probs)
+                                   args.seed, call_base, h_probs, h_cdf)
             return time.perf_counter() - t, sum(E for _, E, _ in sz)
 
         cpu_run(0)  # warm-up (page in the graph, spin up the thread pool)
@@ -400,6 +410,8 @@ def main():
                     for kk in kernels],
         "graph_build_s": round(t_build, 1),
     }
+    if cdf is not None:
+        out["weight_cdf_build_ms"] = round(t_cdf * 1e3, 2)
     print(json.dumps(out))
 
 

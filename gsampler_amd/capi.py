@@ -72,7 +72,9 @@ SIGNATURES = {
     "gs_minor_slice_workspace_bytes": (_sz, [_i64, _i64]),
     "gs_minor_slice_count": (_int, [_p, _i64, _p, _i64, _p, _i64, _p, _p, _p, _sz, _p]),
     "gs_minor_slice_fill": (_int, [_p, _i64, _i64, _p, _i64, _p, _p, _p, _p, _p, _sz, _p]),
-    "gs_csc_col_sample_weighted_fill": (_int, [_p, _i64, _p, _p, _p, _i64, _i64, _int, _u64,
+    "gs_weight_cdf_workspace_bytes": (_sz, [_i64, _i64]),
+    "gs_weight_cdf_build": (_int, [_p, _i64, _p, _i64, _p, _p, _sz, _p]),
+    "gs_csc_col_sample_weighted_fill": (_int, [_p, _i64, _p, _p, _p, _p, _i64, _i64, _int, _u64,
                                                _u64, _p, _p, _p, _p, _p, _p, _p]),
     "gs_weighted_key_probe": (_int, [_u64, _u64, _u64, _u64, C.c_float, _u64, _p, _p]),
     "gs_list_sample_uniform": (_int, [_i64, _i64, _int, _int, _u64, _u64, _p, _p]),
@@ -499,10 +501,29 @@ def weighted_key_probe(seed, call_id, pos, draw, w, r64):
     return out.cpu().tolist()
 
 
+def weight_cdf(indptr, probs):
+    """Persistent integer CDF of the edge weights of a matrix (int64[nnz + 1])."""
+    indptr = _i64t(indptr, "indptr")
+    probs = probs.contiguous()
+    if probs.dtype != torch.float32:
+        raise GsError("probs must be float32")
+    nnz, num_cols = probs.numel(), indptr.numel() - 1
+    cdf = torch.empty(nnz + 1, dtype=torch.int64, device=indptr.device)
+    ws = _workspace(lib().gs_weight_cdf_workspace_bytes(num_cols, nnz), indptr.device)
+    check(lib().gs_weight_cdf_build(_ptr(indptr), num_cols, probs.data_ptr(), nnz,
+                                    cdf.data_ptr(), ws.data_ptr(), ws.numel(), _stream()))
+    return cdf
+
+
 def sample_weighted(indptr, indices, probs, column_ids, fanout, replace=False, seed=7777,
-                    call_id=0, with_coo=True):
-    """Weighted per-column sampling -> (sub_indptr, coo_col | None, sub_indices, select)."""
+                    call_id=0, with_coo=True, cdf=None):
+    """Weighted per-column sampling -> (sub_indptr, coo_col | None, sub_indices, select).
+    With `cdf` (from weight_cdf) draws are searches in the CDF instead of passes
+    over the weights."""
     indptr, indices = _i64t(indptr, "indptr"), _i64t(indices, "indices")
+    if cdf is not None:
+        return _sample_weighted_cdf(indptr, indices, _i64t(cdf, "cdf"), column_ids, fanout,
+                                    replace, seed, call_id, with_coo)
     probs = probs.contiguous()
     if probs.dtype != torch.float32:
         raise GsError("probs must be float32")
@@ -527,10 +548,35 @@ def sample_weighted(indptr, indices, probs, column_ids, fanout, replace=False, s
             scratch = torch.empty(indices.numel() + 1, dtype=torch.int64, device=dev)
     if nnz > 0:
         check(lib().gs_csc_col_sample_weighted_fill(
-            _ptr(indptr), num_cols, _ptr(indices), probs.data_ptr(), _ptr(column_ids), n,
-            fanout, int(replace), seed, call_id, sub_indptr.data_ptr(), _ptr(cdf_off),
+            _ptr(indptr), num_cols, _ptr(indices), probs.data_ptr(), None, _ptr(column_ids),
+            n, fanout, int(replace), seed, call_id, sub_indptr.data_ptr(), _ptr(cdf_off),
             _ptr(scratch), _ptr(out_col), out_idx.data_ptr(), out_sel.data_ptr(), _stream()))
     return sub_indptr, out_col, out_idx, out_sel
+
+
+def _sample_weighted_cdf(indptr, indices, cdf, column_ids, fanout, replace, seed, call_id,
+                         with_coo):
+    num_cols = indptr.numel() - 1
+    dev = indptr.device
+    if column_ids is not None:
+        column_ids = _i64t(column_ids, "column_ids")
+        n = column_ids.numel()
+    else:
+        n = num_cols
+    sub_indptr = col_count(indptr, column_ids, fanout, replace, n)
+    count = _Count(sub_indptr)
+    bound = n * fanout
+    size = bound if bound <= _BOUND_LIMIT else count.get()
+    out_idx = torch.empty(size, dtype=torch.int64, device=dev)
+    out_sel = torch.empty(size, dtype=torch.int64, device=dev)
+    out_col = torch.empty(size, dtype=torch.int64, device=dev) if with_coo else None
+    if size > 0:
+        check(lib().gs_csc_col_sample_weighted_fill(
+            _ptr(indptr), num_cols, _ptr(indices), None, cdf.data_ptr(), _ptr(column_ids), n,
+            fanout, int(replace), seed, call_id, sub_indptr.data_ptr(), None, None,
+            _ptr(out_col), out_idx.data_ptr(), out_sel.data_ptr(), _stream()))
+    nnz = count.get()
+    return (sub_indptr, out_col[:nnz] if with_coo else None, out_idx[:nnz], out_sel[:nnz])
 
 
 def list_sample_uniform(n, num_picks, replace=False, algo=ALGO_AUTO, seed=7777, call_id=0,

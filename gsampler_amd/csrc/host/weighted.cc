@@ -46,8 +46,9 @@ GraphAndIndex Graph::SamplingProbs(int64_t axis, torch::Tensor edge_probs,
   if (replace) scratch = new_ids(m.indices.numel() + 1, m.indptr);
   const RandomState& rs = random_state();
   GS_CALL(gs_csc_col_sample_weighted_fill(
-      cptr(m.indptr), n, cptr(m.indices), probs.data_ptr<float>(), nullptr, n,
-      fanout, replace ? 1 : 0, rs.seed, take_call_id(), cptr(r.indptr), nullptr,
+      cptr(m.indptr), n, cptr(m.indices), probs.data_ptr<float>(), nullptr,
+      nullptr, n, fanout, replace ? 1 : 0, rs.seed, take_call_id(), cptr(r.indptr),
+      nullptr,
       replace ? scratch.data_ptr() : nullptr,
       with_coo ? mptr(r.major_ids) : nullptr, mptr(r.minor_ids), mptr(r.select),
       cur_stream()));

@@ -14,6 +14,7 @@
 // fusing of a multiply into a neighbouring add anywhere in this file.
 #pragma clang fp contract(off)
 
+#include <cstdlib>
 #include <cstring>
 #include <rocprim/device/device_radix_sort.hpp>
 #include <rocprim/device/device_segmented_radix_sort.hpp>
@@ -243,6 +244,365 @@ __global__ __launch_bounds__(kBlock) void sample_weighted_replace_kernel(
   }
 }
 
+// ------------------------------------------- persistent integer CDF of a matrix
+// cdf[e] = sum of the quantised weights of all edges before e (over the whole
+// matrix, columns back to back), cdf[nnz] = grand total.  Weights of a column
+// are quantised against the column's exact maximum to 31 bits, so the prefix
+// sums are integers and do not depend on the order of additions.  Column c
+// owns [cdf[indptr[c]], cdf[indptr[c + 1]]).  Built once per (matrix, weights),
+// it turns a weighted draw into a search over O(log deg) entries instead of a
+// pass over the column.
+__global__ __launch_bounds__(kBlock) void cdf_colmax_kernel(
+    const int64_t* __restrict__ indptr, int64_t num_cols,
+    const float* __restrict__ probs, int64_t nnz, unsigned int* colmax_bits) {
+  const int64_t e = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  const bool active = e < nnz;
+  int64_t c = -1;
+  float w = 0.0f;
+  if (active) {
+    c = segment_of(indptr, num_cols, e);
+    w = probs[e];
+  }
+  // positive floats order like their bit patterns
+  const int64_t c0 = wave_uniform_first(c);
+  if (__all(active && c == c0)) {
+#pragma unroll
+    for (int d = kWave / 2; d > 0; d >>= 1) {
+      const float o = __shfl_xor(w, d, kWave);
+      if (o > w) w = o;
+    }
+    if (lane_id() == 0 && w > 0.0f) atomicMax(colmax_bits + c, __float_as_uint(w));
+  } else if (active && w > 0.0f) {
+    atomicMax(colmax_bits + c, __float_as_uint(w));
+  }
+}
+
+__global__ __launch_bounds__(kBlock) void cdf_quantise_kernel(
+    const int64_t* __restrict__ indptr, int64_t num_cols,
+    const float* __restrict__ probs, int64_t nnz,
+    const unsigned int* __restrict__ colmax_bits, int64_t* __restrict__ cdf) {
+  const int64_t e = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (e > nnz) return;
+  uint64_t q = 0;
+  if (e < nnz) {
+    const float wmax = __uint_as_float(colmax_bits[segment_of(indptr, num_cols, e)]);
+    if (wmax > 0.0f) q = quantise(probs[e], det_div(2147483648.0, (double)wmax));
+  }
+  cdf[e] = (int64_t)q;  // cdf[nnz] = 0 closes the exclusive scan
+}
+
+__global__ __launch_bounds__(kBlock) void cdf_zero_kernel(unsigned int* p, int64_t n) {
+  const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (i < n) p[i] = 0u;
+}
+
+// Search state of one draw: the item of the column whose interval holds x is
+// the last j in [0, deg) with a[j] <= x, for a[0] <= x < a[deg] (a = the
+// column's slice of the CDF).  Prefix sums of weights are close to a straight
+// line, so guesses interpolate; every other step (mode 1) or every step after
+// kInterpolations guesses (mode 2) is a plain bisection, which bounds the worst
+// case for any weights; mode 0 only bisects.
+constexpr int kInterpolations = 8;
+struct CdfSearch {
+  const int64_t* a;
+  int64_t lo, hi, a_lo, a_hi, x;
+  int guesses;
+  bool flip;
+  __device__ __forceinline__ void begin(const int64_t* col, int64_t deg, int64_t first,
+                                        int64_t last, int64_t point) {
+    a = col;
+    lo = 0;
+    hi = deg;
+    a_lo = first;
+    a_hi = last;
+    x = point;
+    guesses = 0;
+    flip = true;
+  }
+  __device__ __forceinline__ bool done() const { return hi - lo <= 1; }
+  __device__ __forceinline__ int64_t probe_at(int mode) {
+    bool interpolate = false;
+    if (hi - lo > 8) {
+      if (mode == 1) interpolate = flip;
+      if (mode == 2) interpolate = guesses < kInterpolations;
+    }
+    flip = !flip;
+    if (!interpolate) return (lo + hi) >> 1;
+    ++guesses;
+    const double frac = (double)(x - a_lo) / (double)(a_hi - a_lo);
+    int64_t mid = lo + (int64_t)(frac * (double)(hi - lo));
+    if (mid <= lo) mid = lo + 1;
+    if (mid >= hi) mid = hi - 1;
+    return mid;
+  }
+  __device__ __forceinline__ void narrow(int64_t mid, int64_t v) {
+    if (v <= x) {
+      lo = mid;
+      a_lo = v;
+    } else {
+      hi = mid;
+      a_hi = v;
+    }
+  }
+};
+
+__device__ __forceinline__ int64_t cdf_locate(const int64_t* __restrict__ a,
+                                              int64_t deg, int64_t x, int mode) {
+  CdfSearch s;
+  s.begin(a, deg, a[0], a[deg], x);
+  while (!s.done()) {
+    const int64_t mid = s.probe_at(mode);
+    s.narrow(mid, a[mid]);
+  }
+  return s.lo;
+}
+
+constexpr int kMaxCdfFanout = 64;
+
+// Independent draws a column may spend before the rare sequential phase.
+__host__ __device__ constexpr int cdf_free_draws(int fanout) { return 2 * fanout + 8; }
+
+// A group of G lanes (G >= fanout without replacement) takes U consecutive
+// columns and walks them through every stage together.  A wavefront advances
+// at the pace of its slowest search (up to 22 dependent probes in a hub column
+// of a power-law graph), which is what bounds this kernel; more columns per
+// group only add to that maximum (U = 2 and 4 measured 30 % and 100 % slower
+// than U = 1 on a 124M-edge graph), so U = 1 is the default.
+// Without replacement: successive weighted sampling, in the form "draw with
+// replacement and skip what was drawn before" -- draws 0, 1, 2, ... are
+// independent points of the whole mass, so a round of G of them is searched by
+// the G lanes at once; the items enter the output in draw order until fanout
+// distinct ones are there.  A column whose mass sits on a few items could
+// repeat for ever, so after cdf_free_draws(fanout) draws the group finishes in step:
+// every further draw takes a point of the mass that is left and maps it past
+// the intervals already taken (kept sorted), which never repeats; when the
+// positive mass runs out, zero-weight items follow in index order.
+// With replacement: one independent point per output slot.
+// Streams: pos = column position, draw = draw index as above.
+template <int G, int U>
+__global__ __launch_bounds__(kBlock) void sample_weighted_cdf_kernel(
+    const int64_t* __restrict__ indptr, int64_t num_cols,
+    const int64_t* __restrict__ indices, const int64_t* __restrict__ cdf,
+    const int64_t* __restrict__ column_ids, int64_t num_items, int fanout,
+    int replace, PhiloxKey key, const int64_t* __restrict__ sub_indptr,
+    int64_t* __restrict__ out_coo_col, int64_t* __restrict__ out_indices,
+    int64_t* __restrict__ out_select, int mode) {
+  const int lane = threadIdx.x & (G - 1);
+  const int64_t item0 = (((int64_t)blockIdx.x * kBlock + threadIdx.x) / G) * U;
+  if (item0 >= num_items) return;  // whole groups leave together
+  int64_t in_start[U], deg[U], out_start[U], base[U];
+  uint64_t total[U];
+  {
+    int64_t c[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int64_t item = item0 + u;
+      c[u] = item < num_items ? (column_ids ? column_ids[item] : item) : -1;
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) deg[u] = column_degree(indptr, num_cols, c[u], &in_start[u]);
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      out_start[u] = deg[u] > 0 ? sub_indptr[item0 + u] : 0;
+      base[u] = deg[u] > 0 ? cdf[in_start[u]] : 0;
+      total[u] = deg[u] > 0 ? (uint64_t)(cdf[in_start[u] + deg[u]] - base[u]) : 0;
+    }
+  }
+  auto emit = [&](int u, int64_t slot, int64_t off) {
+    const int64_t p = in_start[u] + off;
+    out_indices[out_start[u] + slot] = indices ? indices[p] : p;
+    out_select[out_start[u] + slot] = p;
+    if (out_coo_col) out_coo_col[out_start[u] + slot] = item0 + u;
+  };
+  // U searches in lockstep: all probes of a step are issued before any is used
+  auto locate_all = [&](const bool (&want)[U], const uint64_t (&point)[U], int64_t (&off)[U]) {
+    CdfSearch st[U];
+    bool open = false;
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      off[u] = -1;
+      if (want[u]) {
+        st[u].begin(cdf + in_start[u], deg[u], base[u], base[u] + (int64_t)total[u],
+                    base[u] + (int64_t)point[u]);
+        open |= !st[u].done();
+      }
+    }
+    while (open) {
+      int64_t mid[U], v[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) mid[u] = (want[u] && !st[u].done()) ? st[u].probe_at(mode) : -1;
+#pragma unroll
+      for (int u = 0; u < U; ++u) v[u] = mid[u] >= 0 ? st[u].a[mid[u]] : 0;
+      open = false;
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        if (mid[u] >= 0) st[u].narrow(mid[u], v[u]);
+        open |= want[u] && !st[u].done();
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+      if (want[u]) off[u] = st[u].lo;
+  };
+
+  if (replace) {
+    for (int j0 = 0; j0 < fanout; j0 += G) {
+      const int j = j0 + lane;
+      bool want[U];
+      uint64_t point[U];
+      int64_t off[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        want[u] = j < fanout && deg[u] > 0 && total[u] > 0;
+        point[u] = want[u] ? philox_bounded(key, (uint64_t)(item0 + u), (uint64_t)j, total[u]) : 0;
+      }
+      locate_all(want, point, off);
+#pragma unroll
+      for (int u = 0; u < U; ++u)
+        if (j < fanout && deg[u] > 0)
+          emit(u, j, want[u] ? off[u] : deg[u] - 1);  // no positive weight: the last item
+    }
+    return;
+  }
+
+  const int K = fanout;
+  const int free_draws = cdf_free_draws(K);
+  // this group's lanes inside the wavefront's ballot word
+  const uint64_t group_bits =
+      (G == kWave ? ~0ull : ((1ull << G) - 1)) << (lane_id() & ~(G - 1));
+  int count[U];      // items accepted so far (the same in every lane of the group)
+  int64_t mine[U];   // lane s holds the item of output slot s
+  bool sampling[U];  // columns that need draws at all
+  bool any_open = false;
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+    count[u] = 0;
+    mine[u] = -1;
+    sampling[u] = deg[u] > K && total[u] > 0;
+    any_open |= sampling[u];
+  }
+  for (int first = 0; first < free_draws && any_open; first += G) {
+    const int j = first + lane;
+    bool want[U];
+    uint64_t point[U];
+    int64_t drawn[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      want[u] = sampling[u] && count[u] < K && j < free_draws;
+      point[u] = want[u] ? philox_bounded(key, (uint64_t)(item0 + u), (uint64_t)j, total[u]) : 0;
+    }
+    locate_all(want, point, drawn);
+    any_open = false;
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      if (!(sampling[u] && count[u] < K)) continue;  // the same in every lane of the group
+      for (int m = 0; m < G; ++m) {  // in draw order
+        const int64_t cand = __shfl(drawn[u], m, G);
+        if (cand < 0 || count[u] >= K) continue;
+        const bool seen = (__ballot(lane < count[u] && mine[u] == cand) & group_bits) != 0;
+        if (!seen) {
+          if (lane == count[u]) mine[u] = cand;
+          ++count[u];
+        }
+      }
+      any_open |= count[u] < K;
+    }
+  }
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+    if (deg[u] == 0) continue;
+    if (deg[u] <= K) {  // whole column, original order, zero weights included
+      for (int64_t j = lane; j < deg[u]; j += G) emit(u, j, j);
+      continue;
+    }
+    if (lane < count[u]) emit(u, lane, mine[u]);
+    if (count[u] == K) continue;
+    // The rare rest: every lane of the group walks it in step (the shuffles
+    // below need the whole group), lane 0 writes.  Collect what was taken,
+    // sorted by position in the CDF.
+    const int64_t* a = cdf + in_start[u];
+    uint64_t start[kMaxCdfFanout];
+    uint32_t len[kMaxCdfFanout];
+    uint64_t removed = 0;
+    for (int s2 = 0; s2 < count[u]; ++s2) {
+      const int64_t off = __shfl(mine[u], s2, G);
+      const uint64_t st = (uint64_t)(a[off] - base[u]);
+      int at = s2;
+      for (; at > 0 && start[at - 1] > st; --at) {
+        start[at] = start[at - 1];
+        len[at] = len[at - 1];
+      }
+      start[at] = st;
+      len[at] = (uint32_t)(a[off + 1] - a[off]);
+      removed += len[at];
+    }
+    int taken = count[u];
+    for (int d = 0; taken < K && removed < total[u]; ++d, ++taken) {
+      uint64_t r = philox_bounded(key, (uint64_t)(item0 + u), (uint64_t)(free_draws + d),
+                                  total[u] - removed);
+      int at = 0;  // where the new interval goes
+      for (; at < taken && r >= start[at]; ++at) r += len[at];
+      const int64_t off = cdf_locate(a, deg[u], base[u] + (int64_t)r, mode);
+      if (lane == 0) emit(u, taken, off);
+      for (int m = taken; m > at; --m) {
+        start[m] = start[m - 1];
+        len[m] = len[m - 1];
+      }
+      start[at] = (uint64_t)(a[off] - base[u]);
+      len[at] = (uint32_t)(a[off + 1] - a[off]);
+      removed += len[at];
+    }
+    // fewer than fanout items have positive weight: zero-weight items in order
+    for (int64_t off = 0; taken < K && off < deg[u]; ++off)
+      if (a[off + 1] == a[off]) {
+        if (lane == 0) emit(u, taken, off);
+        ++taken;
+      }
+  }
+}
+
+// Columns per group and search mode of the CDF sampler (GS_WCDF_ILP: 1, 2, 4;
+// GS_WCDF_SEARCH: 0 bisection, 1 alternating, 2 interpolation first).  Read once.
+struct CdfTuning {
+  int ilp, mode;
+};
+static CdfTuning cdf_tuning() {
+  static const CdfTuning t = [] {
+    CdfTuning r{1, 2};
+    if (const char* e = getenv("GS_WCDF_ILP")) r.ilp = atoi(e);
+    if (const char* e = getenv("GS_WCDF_SEARCH")) r.mode = atoi(e);
+    r.ilp = r.ilp >= 4 ? 4 : (r.ilp >= 2 ? 2 : 1);
+    if (r.mode < 0 || r.mode > 2) r.mode = 1;
+    return r;
+  }();
+  return t;
+}
+
+template <int G>
+static int launch_weighted_cdf(const int64_t* indptr, int64_t num_cols,
+                               const int64_t* indices, const int64_t* cdf,
+                               const int64_t* column_ids, int64_t num_items,
+                               int fanout, int replace, PhiloxKey key,
+                               const int64_t* sub_indptr, int64_t* out_coo_col,
+                               int64_t* out_indices, int64_t* out_select,
+                               hipStream_t s) {
+  const CdfTuning t = cdf_tuning();
+  const int64_t blocks = ceil_div(ceil_div(num_items, t.ilp) * G, kBlock);
+#define GS_CDF_LAUNCH(UU)                                                          \
+  GS_LAUNCH("sample_weighted_cdf", s,                                              \
+            sample_weighted_cdf_kernel<G, UU><<<dim3((unsigned)blocks), dim3(kBlock), 0, s>>>( \
+                indptr, num_cols, indices, cdf, column_ids, num_items, fanout,     \
+                replace, key, sub_indptr, out_coo_col, out_indices, out_select, t.mode))
+  if (t.ilp == 4)
+    GS_CDF_LAUNCH(4);
+  else if (t.ilp == 2)
+    GS_CDF_LAUNCH(2);
+  else
+    GS_CDF_LAUNCH(1);
+#undef GS_CDF_LAUNCH
+  return GS_OK;
+}
+
 // ------------------------------------------------------------ list sampling
 __global__ __launch_bounds__(kBlock) void list_keys_kernel(
     const float* __restrict__ probs, int64_t n, PhiloxKey key,
@@ -391,9 +751,46 @@ int gs_weighted_key_probe(uint64_t seed, uint64_t call_id, uint64_t pos,
   return GS_OK;
 }
 
+size_t gs_weight_cdf_workspace_bytes(int64_t num_cols, int64_t nnz) {
+  if (num_cols < 0 || nnz < 0) return 0;
+  return gs::align_up((size_t)(num_cols > 0 ? num_cols : 1) * sizeof(unsigned int), 256) +
+         gs::scan_workspace_bytes(nnz + 1);
+}
+
+int gs_weight_cdf_build(const int64_t* indptr, int64_t num_cols, const float* probs,
+                        int64_t nnz, int64_t* cdf, void* workspace,
+                        size_t workspace_bytes, gs_stream_t stream) {
+  using namespace gs;
+  GS_REQUIRE(num_cols >= 0 && nnz >= 0, "weight_cdf_build: negative size");
+  GS_REQUIRE(cdf && (nnz == 0 || (indptr && probs)), "weight_cdf_build: null pointer");
+  const size_t need = gs_weight_cdf_workspace_bytes(num_cols, nnz);
+  if (workspace == nullptr || workspace_bytes < need) {
+    set_error("weight_cdf_build workspace too small: %zu < %zu", workspace_bytes, need);
+    return GS_ERR_WORKSPACE;
+  }
+  hipStream_t s = as_stream(stream);
+  unsigned int* colmax = (unsigned int*)workspace;
+  const size_t colmax_bytes =
+      align_up((size_t)(num_cols > 0 ? num_cols : 1) * sizeof(unsigned int), 256);
+  void* scan_ws = (char*)workspace + colmax_bytes;
+  if (num_cols > 0)
+    GS_LAUNCH("cdf_zero", s,
+              cdf_zero_kernel<<<dim3((unsigned)ceil_div(num_cols, kBlock)), dim3(kBlock),
+                                0, s>>>(colmax, num_cols));
+  if (nnz > 0)
+    GS_LAUNCH("cdf_colmax", s,
+              cdf_colmax_kernel<<<dim3((unsigned)ceil_div(nnz, kBlock)), dim3(kBlock), 0,
+                                  s>>>(indptr, num_cols, probs, nnz, colmax));
+  GS_LAUNCH("cdf_quantise", s,
+            cdf_quantise_kernel<<<dim3((unsigned)ceil_div(nnz + 1, kBlock)), dim3(kBlock),
+                                  0, s>>>(indptr, num_cols, probs, nnz, colmax, cdf));
+  return exclusive_scan_i64(cdf, cdf, nnz + 1, scan_ws, workspace_bytes - colmax_bytes, s);
+}
+
 int gs_csc_col_sample_weighted_fill(
     const int64_t* indptr, int64_t num_cols, const int64_t* indices,
-    const float* probs, const int64_t* column_ids, int64_t num_items,
+    const float* probs, const int64_t* cdf, const int64_t* column_ids,
+    int64_t num_items,
     int64_t fanout, int replace, uint64_t seed, uint64_t call_id,
     const int64_t* sub_indptr, const int64_t* cdf_offsets, void* cdf_scratch,
     int64_t* out_coo_col, int64_t* out_indices, int64_t* out_select,
@@ -402,13 +799,28 @@ int gs_csc_col_sample_weighted_fill(
   GS_REQUIRE(num_items >= 0 && num_cols >= 0, "sample_weighted: negative size");
   GS_REQUIRE(fanout >= 0, "sample_weighted: negative fanout %lld", (long long)fanout);
   if (num_items == 0 || fanout == 0) return GS_OK;
-  GS_REQUIRE(indptr && probs && sub_indptr && out_indices && out_select,
+  GS_REQUIRE(indptr && (probs || cdf) && sub_indptr && out_indices && out_select,
              "sample_weighted: null pointer");
   GS_REQUIRE(column_ids != nullptr || num_items <= num_cols,
              "sample_weighted: %lld items but the matrix has %lld columns",
              (long long)num_items, (long long)num_cols);
   const PhiloxKey key = make_key(seed, call_id);
   hipStream_t s = as_stream(stream);
+  if (cdf != nullptr) {
+    GS_REQUIRE(replace || fanout <= kMaxCdfFanout,
+               "sample_weighted: fanout %lld > %d is not supported without replacement",
+               (long long)fanout, kMaxCdfFanout);
+    GS_REQUIRE(fanout <= INT32_MAX, "sample_weighted: fanout too large");
+#define GS_CDF_ARGS                                                              \
+  indptr, num_cols, indices, cdf, column_ids, num_items, (int)fanout, replace, key, \
+      sub_indptr, out_coo_col, out_indices, out_select, s
+    if (fanout <= 8) return launch_weighted_cdf<8>(GS_CDF_ARGS);
+    if (fanout <= 16) return launch_weighted_cdf<16>(GS_CDF_ARGS);
+    if (fanout <= 32) return launch_weighted_cdf<32>(GS_CDF_ARGS);
+    return launch_weighted_cdf<64>(GS_CDF_ARGS);
+#undef GS_CDF_ARGS
+    return GS_OK;
+  }
   if (replace) {
     GS_REQUIRE(cdf_scratch, "sample_weighted: sampling with replacement needs the CDF scratch");
     GS_REQUIRE(column_ids == nullptr || cdf_offsets != nullptr,

@@ -162,11 +162,32 @@ int gs_csc_col_sample_uniform_fill(const int64_t* indptr, int64_t num_cols,
  *  with replacement: integer CDF per column in cdf_scratch (uint64 per edge;
  *    column i uses cdf_scratch + cdf_offsets[i], or + indptr[column] when
  *    column_ids == NULL and cdf_offsets == NULL), pick j uses draw j.
+ *  cdf != NULL (from gs_weight_cdf_build for the same indptr / probs; probs
+ *    may then be NULL, cdf_offsets / cdf_scratch are not used): every draw is
+ *    a search in the column's slice of the CDF, O(fanout * log deg) per
+ *    column instead of a pass over its weights.  Without replacement
+ *    (fanout <= 64) this is successive weighted sampling: draws 0 ..
+ *    2*fanout+7 are independent points of the whole mass and an edge already
+ *    drawn is skipped; if that leaves slots open, further draws take points of
+ *    the mass that is left.  The same distribution as the smallest-keys rule
+ *    above, other picks; output in draw order; when fewer than fanout edges
+ *    have positive (quantised) weight, zero-weight edges follow in index
+ *    order.  Stream: pos = column position, draw = draw index.
  * Stands in for CSCColSamplingProbsCUDA (src/cuda/sampling_probs.cu:268-281).
  * ---------------------------------------------------------------------- */
+/* Persistent integer CDF of a matrix's edge weights, the input of the fast
+ * weighted sampler below: cdf[nnz + 1], cdf[e] = sum of the quantised weights of
+ * the edges before e (all columns back to back; a column's weights are
+ * quantised to 31 bits against the column's maximum, w <= 0 counts as 0).
+ * Build it once per (matrix, weights); it costs one pass over the edges. */
+size_t gs_weight_cdf_workspace_bytes(int64_t num_cols, int64_t nnz);
+int gs_weight_cdf_build(const int64_t* indptr, int64_t num_cols,
+                        const float* probs, int64_t nnz, int64_t* cdf,
+                        void* workspace, size_t workspace_bytes,
+                        gs_stream_t stream);
 int gs_csc_col_sample_weighted_fill(
     const int64_t* indptr, int64_t num_cols, const int64_t* indices,
-    const float* probs, const int64_t* column_ids, int64_t num_items,
+    const float* probs, const int64_t* cdf, const int64_t* column_ids, int64_t num_items,
     int64_t fanout, int replace, uint64_t seed, uint64_t call_id,
     const int64_t* sub_indptr, const int64_t* cdf_offsets, void* cdf_scratch,
     int64_t* out_coo_col, int64_t* out_indices, int64_t* out_select,

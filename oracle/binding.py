@@ -328,9 +328,33 @@ def weighted_key(seed, call_id, pos, draw, w) -> float:
              C.c_float(w))
 
 
+def weight_cdf(indptr, probs) -> np.ndarray:
+    indptr = _i64(indptr)
+    probs = np.ascontiguousarray(probs, dtype=np.float32)
+    cdf = np.empty(probs.size + 1, dtype=np.int64)
+    lib().gs_weight_cdf_build_cpu(_p(indptr), C.c_int64(indptr.size - 1), _p(probs),
+                                  C.c_int64(probs.size), _p(cdf))
+    return cdf
+
+
 def sample_weighted(indptr, indices, probs, column_ids, fanout, replace=False, seed=7777,
-                    call_id=0, with_coo=True):
+                    call_id=0, with_coo=True, cdf=None):
     indptr, indices = _i64(indptr), _i64(indices)
+    if cdf is not None:
+        cdf = _i64(cdf)
+        num_cols = indptr.size - 1
+        if column_ids is not None:
+            column_ids = _i64(column_ids)
+        n = column_ids.size if column_ids is not None else num_cols
+        sub_indptr = col_count(indptr, column_ids, fanout, replace, n)
+        nnz = int(sub_indptr[-1])
+        out_idx, out_sel = np.empty(nnz, dtype=np.int64), np.empty(nnz, dtype=np.int64)
+        out_col = np.empty(nnz, dtype=np.int64) if with_coo else None
+        lib().gs_csc_col_sample_weighted_cdf_fill_cpu(
+            _p(indptr), C.c_int64(num_cols), _p(indices), _p(cdf), _p(column_ids),
+            C.c_int64(n), C.c_int64(fanout), C.c_int(int(replace)), C.c_uint64(seed),
+            C.c_uint64(call_id), _p(sub_indptr), _p(out_col), _p(out_idx), _p(out_sel))
+        return sub_indptr, out_col, out_idx, out_sel
     probs = np.ascontiguousarray(probs, dtype=np.float32)
     num_cols = indptr.size - 1
     if column_ids is not None:

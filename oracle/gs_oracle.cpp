@@ -965,3 +965,114 @@ void gs_segment_sort_i64_cpu(const int64_t* indptr, int64_t num_segments,
 }
 
 }  // extern "C"
+
+// -------------------------------------------------------------------------
+// Weighted sampling through a persistent integer CDF (no counterpart in the
+// reference, whose A-Res kernel reads every weight of a column on every call;
+// the distribution is the same: successive weighted sampling without
+// replacement, which is what A-Res produces).
+//  cdf[e] = sum of the quantised weights of all edges before e over the whole
+//  matrix; a column's weights are quantised to 31 bits against the column's
+//  maximum exactly as integer_cdf() does.
+//  Without replacement, deg > fanout: draws 0 .. 2*fanout+7 are independent
+//  uniform points of the whole mass; an item already drawn is skipped (drawing
+//  with replacement and discarding repeats is successive sampling).  If that
+//  does not give fanout items, draw 2*fanout+8+d takes r uniform in the mass
+//  left, walks the intervals already taken in ascending order
+//  (r >= start ? r += len) and picks the item whose interval holds r.  Output
+//  in draw order; when the positive mass runs out, zero-weight items follow in
+//  index order.
+//  With replacement: slot j picks the item holding a uniform point of the
+//  total; a column without positive weights gives its last item.
+//  Streams: pos = column position, draw = slot.
+extern "C" void gs_weight_cdf_build_cpu(const int64_t* indptr, int64_t num_cols,
+                                        const float* probs, int64_t nnz,
+                                        int64_t* cdf) {
+  std::vector<uint64_t> q((size_t)nnz, 0);
+#pragma omp parallel for schedule(dynamic, 256)
+  for (int64_t c = 0; c < num_cols; ++c) {
+    float wmax = 0.0f;
+    for (int64_t e = indptr[c]; e < indptr[c + 1]; ++e)
+      if (probs[e] > wmax) wmax = probs[e];
+    if (wmax <= 0.0f) continue;
+    const double scale = det_div(2147483648.0, (double)wmax);
+    for (int64_t e = indptr[c]; e < indptr[c + 1]; ++e)
+      q[(size_t)e] = probs[e] > 0.0f ? (uint64_t)((double)probs[e] * scale) : 0;
+  }
+  int64_t acc = 0;
+  for (int64_t e = 0; e < nnz; ++e) {
+    cdf[e] = acc;
+    acc += (int64_t)q[(size_t)e];
+  }
+  cdf[nnz] = acc;
+}
+
+extern "C" void gs_csc_col_sample_weighted_cdf_fill_cpu(
+    const int64_t* indptr, int64_t num_cols, const int64_t* indices,
+    const int64_t* cdf, const int64_t* column_ids, int64_t num_items,
+    int64_t fanout, int replace, uint64_t seed, uint64_t call_id,
+    const int64_t* sub_indptr, int64_t* out_coo_col, int64_t* out_indices,
+    int64_t* out_select) {
+  Stream rng(seed, call_id);
+#pragma omp parallel for schedule(dynamic, 64)
+  for (int64_t i = 0; i < num_items; ++i) {
+    const int64_t c = column_ids ? column_ids[i] : i;
+    const int64_t deg = col_degree(indptr, num_cols, c);
+    if (deg == 0) continue;
+    const int64_t in_start = indptr[c], out_start = sub_indptr[i];
+    auto emit = [&](int64_t j, int64_t off) {
+      out_indices[out_start + j] = indices ? indices[in_start + off] : in_start + off;
+      out_select[out_start + j] = in_start + off;
+      if (out_coo_col) out_coo_col[out_start + j] = i;
+    };
+    const int64_t* a = cdf + in_start;
+    const uint64_t total = (uint64_t)(a[deg] - a[0]);
+    // item whose interval [a[j], a[j+1]) holds the absolute point x
+    auto locate = [&](uint64_t rel) {
+      const int64_t x = a[0] + (int64_t)rel;
+      return (int64_t)(std::upper_bound(a, a + deg + 1, x) - a) - 1;
+    };
+    if (replace) {
+      for (int64_t j = 0; j < fanout; ++j)
+        emit(j, total > 0 ? locate(rng.bounded((uint64_t)i, (uint64_t)j, total)) : deg - 1);
+      continue;
+    }
+    if (deg <= fanout) {
+      for (int64_t j = 0; j < deg; ++j) emit(j, j);
+      continue;
+    }
+    // draws 0 .. free-1 are independent points of the whole mass; repeats are
+    // skipped ("with replacement, discarding what was drawn before")
+    const int64_t free_draws = 2 * fanout + 8;
+    std::vector<int64_t> accepted;
+    if (total > 0)
+      for (int64_t j = 0; j < free_draws && (int64_t)accepted.size() < fanout; ++j) {
+        const int64_t off = locate(rng.bounded((uint64_t)i, (uint64_t)j, total));
+        if (std::find(accepted.begin(), accepted.end(), off) == accepted.end())
+          accepted.push_back(off);
+      }
+    int64_t taken = (int64_t)accepted.size();
+    for (int64_t j = 0; j < taken; ++j) emit(j, accepted[(size_t)j]);
+    // the rare rest: points of the mass that is left, mapped past what was taken
+    std::vector<std::pair<uint64_t, uint64_t>> taken_iv;  // (start, len), ascending
+    uint64_t removed = 0;
+    for (int64_t off : accepted) {
+      taken_iv.push_back({(uint64_t)(a[off] - a[0]), (uint64_t)(a[off + 1] - a[off])});
+      removed += taken_iv.back().second;
+    }
+    std::sort(taken_iv.begin(), taken_iv.end());
+    for (int64_t d = 0; taken < fanout && removed < total; ++d, ++taken) {
+      uint64_t r = rng.bounded((uint64_t)i, (uint64_t)(free_draws + d), total - removed);
+      size_t at = 0;
+      for (; at < taken_iv.size() && r >= taken_iv[at].first; ++at) r += taken_iv[at].second;
+      const int64_t off = locate(r);
+      emit(taken, off);
+      const uint64_t len = (uint64_t)(a[off + 1] - a[off]);
+      taken_iv.insert(taken_iv.begin() + (std::ptrdiff_t)at,
+                      {(uint64_t)(a[off] - a[0]), len});
+      removed += len;
+    }
+    for (int64_t off = 0; taken < fanout && off < deg; ++off)
+      if (a[off + 1] == a[off]) emit(taken++, off);
+  }
+}

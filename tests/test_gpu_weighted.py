@@ -69,6 +69,45 @@ def test_column_sampling_with_replacement_parity(fanout):
          orc.sample_weighted(indptr, indices, probs, None, fanout, True))
 
 
+def _weighted_case(seed, cols=3000, hub=30000):
+    rng = np.random.default_rng(seed)
+    indptr, indices = random_csc(rng, cols, 10**6, 120, hub_deg=hub)
+    probs = rng.lognormal(0, 1, size=indices.size).astype(np.float32)
+    probs[rng.random(indices.size) < 0.05] = 0.0
+    probs[indptr[7]:indptr[8]] = 0.0             # a column without positive weight
+    lo = indptr[11]                              # a column with a single positive weight
+    probs[lo:indptr[12]] = 0.0
+    if indptr[12] > lo:
+        probs[lo] = 2.0
+    for c in (20, 21, 22, 23):                   # nearly all mass on one or two items
+        if indptr[c + 1] - indptr[c] > 2:
+            probs[indptr[c]] = 1e7
+            probs[indptr[c] + 2] = 3e6
+    return rng, indptr, indices, probs
+
+
+def test_weight_cdf_is_bit_identical():
+    rng, indptr, indices, probs = _weighted_case(1)
+    assert np.array_equal(capi.weight_cdf(T(indptr), F(probs)).cpu().numpy(),
+                          orc.weight_cdf(indptr, probs))
+    empty = capi.weight_cdf(T(np.zeros(4)), F(np.zeros(0)))
+    assert empty.cpu().tolist() == [0]
+
+
+@pytest.mark.parametrize("fanout", [1, 5, 15, 64])
+@pytest.mark.parametrize("replace", [False, True])
+def test_cdf_column_sampling_parity(fanout, replace):
+    rng, indptr, indices, probs = _weighted_case(fanout)
+    cdf = orc.weight_cdf(indptr, probs)
+    g_cdf = capi.weight_cdf(T(indptr), F(probs))
+    cols = np.concatenate([rng.integers(0, 3000, size=2000), [7, 11, 7, 20, 21, 22, 23, 20]])
+    same(capi.sample_weighted(T(indptr), T(indices), None, T(cols), fanout, replace, call_id=4,
+                              cdf=g_cdf),
+         orc.sample_weighted(indptr, indices, None, cols, fanout, replace, call_id=4, cdf=cdf))
+    same(capi.sample_weighted(T(indptr), T(indices), None, None, fanout, replace, cdf=g_cdf),
+         orc.sample_weighted(indptr, indices, None, None, fanout, replace, cdf=cdf))
+
+
 @pytest.mark.parametrize("n,k", [(10, 20), (1000, 64), (233000, 512), (5000, 5000)])
 def test_list_sampling_parity(n, k):
     rng = np.random.default_rng(n)

@@ -148,3 +148,90 @@ def test_uniform_list_sampling():
     for t in range(6000):
         counts[orc.list_sample_uniform(12, 4, call_id=t)] += 1
     assert stats.chisquare(counts).pvalue > 0.001
+
+
+# ------------------------------------------------ sampling through a persistent CDF
+def test_weight_cdf_is_a_quantised_prefix_sum():
+    rng = np.random.default_rng(3)
+    deg = np.array([5, 0, 300, 1, 4, 0, 7])
+    indptr = np.concatenate([[0], np.cumsum(deg)])
+    w = rng.lognormal(size=int(deg.sum())).astype(np.float32)
+    w[indptr[4]:indptr[5]] = [0.0, -1.0, 0.0, 0.0]      # a column without positive weights
+    w[indptr[6] + 2] = 0.0
+    cdf = orc.weight_cdf(indptr, w)
+    q = np.diff(cdf)
+    assert cdf[0] == 0 and np.all(q >= 0)
+    for c in range(deg.size):
+        lo, hi = indptr[c], indptr[c + 1]
+        wc, qc = w[lo:hi].astype(np.float64), q[lo:hi]
+        if hi == lo:
+            continue
+        if wc.max() <= 0:
+            assert np.all(qc == 0)
+            continue
+        # the maximum maps to 2^31 (give or take a unit), everything else in proportion
+        assert abs(int(qc[wc.argmax()]) - 2**31) <= 1
+        assert np.all(qc[wc <= 0] == 0)
+        want = np.where(wc > 0, wc / wc.max() * 2**31, 0)
+        assert np.all(np.abs(qc - want) <= 1.0 + want * 2**-40)
+
+
+@pytest.mark.parametrize("w,k", [([3, 1, 2, 2, 1], 2), ([5, 1, 0, 1, 2, 1], 3), ([1, 1, 1, 1], 3),
+                                 ([1000, 1, 2, 3, 2], 3)])   # mass on one item: the sequential phase
+def test_cdf_column_sampling_is_successive_weighted_sampling(w, k):
+    """Ordered k-tuples drawn through the CDF against the exact law of successive
+    weighted sampling without replacement (zero weights have probability 0)."""
+    n = 40000
+    indptr = np.array([0, len(w)]); indices = np.arange(len(w)) + 100
+    probs = np.array(w, dtype=np.float32)
+    cdf = orc.weight_cdf(indptr, probs)
+    s, c, rows, sel = orc.sample_weighted(indptr, indices, None, np.zeros(n, dtype=np.int64), k,
+                                          cdf=cdf)
+    assert np.array_equal(rows, indices[sel]) and np.array_equal(s, np.arange(n + 1) * k)
+    want = {t: p for t, p in _successive_probs(w, k).items() if p > 0}
+    counts = {}
+    for row in sel.reshape(n, k):
+        counts[tuple(row.tolist())] = counts.get(tuple(row.tolist()), 0) + 1
+    assert set(counts) <= set(want)
+    obs = np.array([counts.get(t, 0) for t in want])
+    exp = np.array([want[t] for t in want]) * n
+    assert stats.chisquare(obs, exp).pvalue > 0.01
+
+
+def test_cdf_sampling_structural_rules():
+    indptr = np.array([0, 6, 6, 9, 14]); indices = np.arange(14)
+    probs = np.array([0, 5, 0, 0, 0, 0,   1, 1, 1,   0, 0, 0, 0, 0], dtype=np.float32)
+    cdf = orc.weight_cdf(indptr, probs)
+    s, c, rows, sel = orc.sample_weighted(indptr, indices, None, None, 3, cdf=cdf)
+    assert s.tolist() == [0, 3, 3, 6, 9]
+    assert sel[:3].tolist() == [1, 0, 2]          # the only positive item, then zeros in order
+    assert sel[3:6].tolist() == [6, 7, 8]         # deg <= K: the column in order
+    assert sel[6:].tolist() == [9, 10, 11]        # no positive weight at all
+    assert c.tolist() == [0, 0, 0, 2, 2, 2, 3, 3, 3]
+    # with replacement: proportional to the weights; a column of zeros gives its last item
+    probs = np.array([1, 3, 0, 4,   0, 0], dtype=np.float32)
+    indptr = np.array([0, 4, 6])
+    cdf = orc.weight_cdf(indptr, probs)
+    n = 20000
+    s, c, rows, sel = orc.sample_weighted(indptr, np.arange(6), None,
+                                          np.zeros(n, dtype=np.int64), 2, replace=True, cdf=cdf)
+    cnt = np.bincount(sel, minlength=4)
+    assert cnt[2] == 0
+    assert stats.chisquare(cnt[[0, 1, 3]], 2 * n * np.array([1, 3, 4]) / 8).pvalue > 0.01
+    s, c, rows, sel = orc.sample_weighted(indptr, np.arange(6), None, np.array([1]), 3,
+                                          replace=True, cdf=cdf)
+    assert sel.tolist() == [5, 5, 5]
+
+
+def test_cdf_sampling_agrees_with_key_sampling_in_distribution():
+    """Inclusion frequencies of both weighted samplers on one skewed column."""
+    rng = np.random.default_rng(9)
+    deg, k, n = 40, 5, 20000
+    w = rng.lognormal(sigma=1.5, size=deg).astype(np.float32)
+    indptr = np.array([0, deg]); indices = np.arange(deg)
+    cols = np.zeros(n, dtype=np.int64)
+    a = orc.sample_weighted(indptr, indices, w, cols, k)[3]
+    b = orc.sample_weighted(indptr, indices, None, cols, k, cdf=orc.weight_cdf(indptr, w))[3]
+    ca, cb = np.bincount(a, minlength=deg), np.bincount(b, minlength=deg)
+    keep = (ca + cb) >= 20
+    assert stats.chi2_contingency(np.stack([ca[keep], cb[keep]]))[1] > 0.01
