@@ -88,6 +88,14 @@ class Graph : public torch::CustomClassHolder {
   GraphAndIndex SamplingProbs(int64_t axis, torch::Tensor edge_probs,
                               int64_t fanout, bool replace, int64_t on_format,
                               int64_t output_format);
+  // Not in the reference: column slice + weighted sampling in one step, on the
+  // weights of this (unsliced) matrix.  What gs.jit.compile turns
+  // Slicing -> SamplingProbs into; draws go through a persistent CDF of the
+  // weights that is built on first use and kept while the same tensor comes in.
+  GraphAndIndex FusedSlicingSamplingProbs(int64_t axis, torch::Tensor seeds,
+                                          torch::Tensor edge_probs, int64_t fanout,
+                                          bool replace, int64_t on_format,
+                                          int64_t output_format);
   GraphAndIndex FusedSlicingSampling(int64_t axis, torch::Tensor seeds,
                                      int64_t fanout, bool replace,
                                      int64_t on_format, int64_t output_format);
@@ -153,6 +161,10 @@ class Graph : public torch::CustomClassHolder {
   GraphAndIndex BatchRowSampling(int64_t fanout, bool replace);
   GraphAndIndex BatchRowSamplingProbs(int64_t fanout, bool replace,
                                       torch::Tensor edge_probs);
+  GraphAndIndex BatchFusedSlicingSamplingProbs(torch::Tensor seeds,
+                                               torch::Tensor col_bptr,
+                                               torch::Tensor edge_probs,
+                                               int64_t fanout, bool replace);
   GraphAndIndex BatchFusedSlicingSampling(torch::Tensor seeds,
                                           torch::Tensor col_bptr,
                                           int64_t fanout, bool replace);
@@ -189,6 +201,10 @@ class Graph : public torch::CustomClassHolder {
                          const torch::Tensor& rows_ptr);
 
   const Compressed& compressed(int64_t format);
+  // CDF of edge_probs in the edge order of `format` (cached per weights tensor).
+  torch::Tensor weight_cdf_for(const torch::Tensor& edge_probs, int64_t format);
+  torch::Tensor cdf_, cdf_probs_;
+  int64_t cdf_version_ = -1, cdf_format_ = 0;
   torch::Tensor mapped_rows(const torch::Tensor& base, const torch::Tensor& row_ids);
   GraphAndIndex slice_coo(const torch::Tensor& seeds, int64_t axis,
                           int64_t new_rows, int64_t new_cols);

@@ -59,6 +59,7 @@ TORCH_LIBRARY(gs_classes, m) {
       .def("_CAPI_GraphRelabel", &Graph::GraphRelabel)
       .def("_CAPI_GetValidNodes", &Graph::GetValidNodes)
       .def("_CAPI_SlicingSampling", &Graph::FusedSlicingSampling)
+      .def("_CAPI_SlicingSamplingProbs", &Graph::FusedSlicingSamplingProbs)
       .def("_CAPI_FusedUOPV", &Graph::FusedUOPV)
       .def("_CAPI_FusedESquareSum", &Graph::FusedESquareSum)
       .def("_CAPI_FusedEDivUSum", &Graph::FusedEDivUSum)
@@ -70,6 +71,7 @@ TORCH_LIBRARY(gs_classes, m) {
       .def("_CAPI_BatchRowSamplingProbs", &Graph::BatchRowSamplingProbs)
       .def("_CAPI_BatchGraphRelabel", &Graph::BatchGraphRelabel)
       .def("_CAPI_BatchFusedSlicingSampling", &Graph::BatchFusedSlicingSampling)
+      .def("_CAPI_BatchFusedSlicingSamplingProbs", &Graph::BatchFusedSlicingSamplingProbs)
       .def("_CAPI_GetEdgeBptr", &Graph::GetEdgeBptr)
       .def("_CAPI_GetColBptr", &Graph::GetColBptr)
       .def("_CAPI_GetRowBptr", &Graph::GetRowBptr)

@@ -56,6 +56,89 @@ GraphAndIndex Graph::SamplingProbs(int64_t axis, torch::Tensor edge_probs,
   return {g, edge_index(m.e_ids, r.select)};
 }
 
+// ----------------------------------------- fused slice + weighted sampling
+torch::Tensor Graph::weight_cdf_for(const torch::Tensor& edge_probs, int64_t format) {
+  if (cdf_.defined() && cdf_format_ == format && cdf_probs_.is_same(edge_probs) &&
+      cdf_version_ == (int64_t)edge_probs._version())
+    return cdf_;
+  const Compressed& m = compressed(format);
+  torch::Tensor probs = f32(edge_probs, "edge_probs");
+  TORCH_CHECK(probs.numel() == m.indices.numel(), "weighted sampling: ", probs.numel(),
+              " probabilities for ", m.indices.numel(), " edges");
+  if (m.e_ids.has_value()) probs = probs.index_select(0, m.e_ids.value());
+  const int64_t n = m.indptr.numel() - 1, nnz = m.indices.numel();
+  torch::Tensor cdf = new_ids(nnz + 1, m.indptr);
+  torch::Tensor ws = new_workspace(gs_weight_cdf_workspace_bytes(n, nnz), m.indptr);
+  GS_CALL(gs_weight_cdf_build(cptr(m.indptr), n, probs.data_ptr<float>(), nnz,
+                              mptr(cdf), ws.data_ptr(), ws.numel(), cur_stream()));
+  cdf_ = cdf;
+  cdf_probs_ = edge_probs;
+  cdf_version_ = edge_probs._version();
+  cdf_format_ = format;
+  return cdf_;
+}
+
+GraphAndIndex Graph::FusedSlicingSamplingProbs(int64_t axis, torch::Tensor seeds,
+                                               torch::Tensor edge_probs,
+                                               int64_t fanout, bool replace,
+                                               int64_t on_format,
+                                               int64_t output_format) {
+  TORCH_CHECK((axis == 1 && on_format == kCSC) || (axis == 0 && on_format == kCSR),
+              "FusedSlicingSamplingProbs: not implemented for axis ", axis,
+              " on format ", on_format);
+  const int64_t other = on_format == kCSC ? kCSR : kCSC;
+  TORCH_CHECK(output_format != other, "FusedSlicingSamplingProbs: on_format ", on_format,
+              " cannot produce output_format ", output_format);
+  TORCH_CHECK(fanout >= 0, "fanout must be non-negative, got ", fanout);
+  TORCH_CHECK(replace || fanout <= 64,
+              "FusedSlicingSamplingProbs: fanout above 64 needs replace=True");
+  seeds = ids(seeds, "seeds");
+  const Compressed& m = compressed(on_format);
+  torch::Tensor cdf = weight_cdf_for(edge_probs, on_format);
+  const bool with_coo = output_format & kCOO;
+  const int64_t num_major = m.indptr.numel() - 1, n = seeds.numel();
+  MajorResult r;
+  r.indptr = new_ids(n + 1, m.indptr);
+  torch::Tensor ws = new_workspace(gs_scan_workspace_bytes(n + 1), m.indptr);
+  GS_CALL(gs_csc_col_count(cptr(m.indptr), num_major, cptr(seeds), n, fanout,
+                           replace ? 1 : 0, mptr(r.indptr), ws.data_ptr(), ws.numel(),
+                           cur_stream()));
+  AsyncCount count(r.indptr);
+  const int64_t bound = n * fanout;
+  const int64_t size = bound <= kBoundLimit ? bound : count.get();
+  r.minor_ids = new_ids(size, m.indptr);
+  r.select = new_ids(size, m.indptr);
+  if (with_coo) r.major_ids = new_ids(size, m.indptr);
+  const RandomState& rs = random_state();
+  GS_CALL(gs_csc_col_sample_weighted_fill(
+      cptr(m.indptr), num_major, cptr(m.indices), nullptr, cptr(cdf), cptr(seeds), n,
+      fanout, replace ? 1 : 0, rs.seed, take_call_id(), cptr(r.indptr), nullptr, nullptr,
+      with_coo ? mptr(r.major_ids) : nullptr, mptr(r.minor_ids), mptr(r.select),
+      cur_stream()));
+  const int64_t nnz = count.get();
+  r.minor_ids = r.minor_ids.narrow(0, 0, nnz);
+  r.select = r.select.narrow(0, 0, nnz);
+  if (with_coo) r.major_ids = r.major_ids.narrow(0, 0, nnz);
+  const int64_t new_rows = axis == 0 ? n : num_rows_;
+  const int64_t new_cols = axis == 0 ? num_cols_ : n;
+  GraphPtr g = derive(on_format, output_format, r, new_rows, new_cols);
+  return {g, edge_index(m.e_ids, r.select)};
+}
+
+GraphAndIndex Graph::BatchFusedSlicingSamplingProbs(torch::Tensor seeds,
+                                                    torch::Tensor col_bptr,
+                                                    torch::Tensor edge_probs,
+                                                    int64_t fanout, bool replace) {
+  col_bptr = ids(col_bptr, "col_bptr");
+  auto ret = FusedSlicingSamplingProbs(1, seeds, edge_probs, fanout, replace, kCSC,
+                                       kCSC | kCOO);
+  Graph& g = *std::get<0>(ret);
+  g.col_bptr_ = col_bptr;
+  g.orig_col_ids_ = ids(seeds, "seeds");
+  g.edge_bptr_ = g.csc_->indptr.index_select(0, col_bptr);
+  return ret;
+}
+
 // ------------------------------------------------------------ list sampling
 torch::Tensor ListSampling(int64_t num_items, int64_t num_picks, bool replace) {
   TORCH_CHECK(num_items >= 0 && num_picks >= 0, "ListSampling: negative size");

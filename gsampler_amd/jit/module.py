@@ -94,9 +94,11 @@ class compile:  # noqa: N801 -- the reference's public name
         gm = passes.move_constant_to_top(gm)
         gm = passes.merge_relabel_and_all_nodes(gm)
         gm = passes.fuse_slicing_and_sampling(gm)
+        gm = passes.fuse_slicing_and_weighted_sampling(gm)
         gm = passes.fuse_square_and_sum(gm)
         gm = passes.merge_u_mul_v(gm)
         gm = passes.batch_fuse_slicing_and_sampling(gm)
+        gm = passes.batch_fuse_slicing_and_weighted_sampling(gm)
         gm = passes.dce(gm)
         if self._format_select and not self.use_batchmatrix:
             gm = passes.select_formats(gm)

@@ -170,6 +170,86 @@ def fuse_slicing_and_sampling(gm: fx.GraphModule) -> fx.GraphModule:
     return dce(gm)
 
 
+def _fuse_weighted(gm: fx.GraphModule, slice_name: str, sample_name: str,
+                   probs_arg: int, compatible, make_fused) -> fx.GraphModule:
+    """Shared by the two passes below.  The weights of the sampling call must be
+    a gather of some edge tensor through the slice index; the fused operator
+    takes that edge tensor itself (the parent's weights), and every edge tensor
+    that went through the slice index and then through the sampling index is
+    re-gathered from the parent with the fused index."""
+    for sampling in list(gm.graph.nodes):
+        if not _is_method(sampling, sample_name):
+            continue
+        sliced_graph = sampling.args[0]
+        if not (sliced_graph.op == "call_function" and sliced_graph.target is operator.getitem
+                and sliced_graph.args[1] == 0 and len(sliced_graph.users) == 1):
+            continue
+        slicing = sliced_graph.args[0]
+        if not _is_method(slicing, slice_name) or not compatible(slicing, sampling):
+            continue
+        slice_index = _getitem_users(slicing, 1)
+        sample_index = _getitem_users(sampling, 1)
+        probs = sampling.args[probs_arg]
+        if not (isinstance(probs, fx.Node) and probs.op == "call_function"
+                and len(probs.args) == 2 and probs.args[1] in slice_index):
+            continue
+        rewires, ok = [], True
+        for idx_node in slice_index:
+            for gathered in idx_node.users:
+                for user in list(gathered.users):
+                    if user is sampling:
+                        continue
+                    if not (sample_index and sample_index[0] in user.args):
+                        ok = False
+                    rewires.append((gathered, user))
+        if not ok:
+            continue
+        with gm.graph.inserting_before(slicing):
+            fused = make_fused(gm.graph, slicing, sampling, probs.args[0])
+            fused_graph = gm.graph.call_function(operator.getitem, args=(fused, 0))
+            fused_index = gm.graph.call_function(operator.getitem, args=(fused, 1))
+        for g in _getitem_users(sampling, 0):
+            g.replace_all_uses_with(fused_graph)
+        for gathered, second in rewires:
+            with gm.graph.inserting_before(second):
+                direct = gm.graph.call_function(operator.getitem,
+                                                args=(gathered.args[0], fused_index))
+            second.replace_all_uses_with(direct)
+    return dce(gm)
+
+
+def fuse_slicing_and_weighted_sampling(gm: fx.GraphModule) -> fx.GraphModule:
+    """Slicing(seeds, axis, on, out) -> [0] -> SamplingProbs(axis, w[slice index], K, ...)
+       => SlicingSamplingProbs(axis, seeds, w, K, replace, on, out): the slice is
+    never materialised and the draws go through the parent's weight CDF."""
+    def compatible(slicing, sampling):          # same axis, same format
+        return sampling.args[1] == slicing.args[2] and sampling.args[5] == slicing.args[3]
+
+    def make(graph, slicing, sampling, weights):
+        return graph.call_method(
+            "_CAPI_SlicingSamplingProbs",
+            args=(slicing.args[0], slicing.args[2], slicing.args[1], weights, sampling.args[3],
+                  sampling.args[4], sampling.args[5], sampling.args[6]))
+
+    return _fuse_weighted(gm, "_CAPI_Slicing", "_CAPI_SamplingProbs", 2, compatible, make)
+
+
+def batch_fuse_slicing_and_weighted_sampling(gm: fx.GraphModule) -> fx.GraphModule:
+    """BatchColSlicing(seeds, ptr, encoding=False) -> [0] -> BatchRowSamplingProbs(K, replace,
+    w[slice index]) => BatchFusedSlicingSamplingProbs(seeds, ptr, w, K, replace)."""
+    def compatible(slicing, sampling):          # encoded rows cannot be fused
+        return slicing.args[3] is False
+
+    def make(graph, slicing, sampling, weights):
+        return graph.call_method(
+            "_CAPI_BatchFusedSlicingSamplingProbs",
+            args=(slicing.args[0], slicing.args[1], slicing.args[2], weights, sampling.args[1],
+                  sampling.args[2]))
+
+    return _fuse_weighted(gm, "_CAPI_BatchColSlicing", "_CAPI_BatchRowSamplingProbs", 3,
+                          compatible, make)
+
+
 def batch_fuse_slicing_and_sampling(gm: fx.GraphModule) -> fx.GraphModule:
     """BatchColSlicing(seeds, ptr, encoding=False) -> [0] -> BatchRowSampling(K, replace)
        => BatchFusedSlicingSampling(seeds, ptr, K, replace)."""
@@ -254,6 +334,7 @@ FORMAT_ARGS = {
     "_CAPI_Sampling": (4, 5),
     "_CAPI_SamplingProbs": (5, 6),
     "_CAPI_SlicingSampling": (5, 6),
+    "_CAPI_SlicingSamplingProbs": (6, 7),
     "_CAPI_SDDMM": (7, None),
     "_CAPI_SpMM": (9, None),
     "_CAPI_FusedUOPV": (8, None),
@@ -271,7 +352,7 @@ def _preferred(node: fx.Node) -> List[int]:
         return [_CSR, _CSC, _COO] if node.args[2] == 0 else [_CSC, _CSR, _COO]
     if t in ("_CAPI_Sampling", "_CAPI_SlicingSampling"):
         return [_CSR] if node.args[1] == 0 else [_CSC]
-    if t == "_CAPI_SamplingProbs":
+    if t in ("_CAPI_SamplingProbs", "_CAPI_SlicingSamplingProbs"):
         return [_CSR] if node.args[1] == 0 else [_CSC]
     if t in ("_CAPI_SpMM", "_CAPI_FusedESquareSum", "_CAPI_FusedEDivUSum"):
         return [_CSR, _COO] if node.args[8] == 2 else [_CSC, _COO]

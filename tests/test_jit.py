@@ -29,6 +29,26 @@ def batch_graphsage_sampler(A, seeds, seeds_ptr, fanouts):
     return ret
 
 
+def weighted_graphsage_sampler(A, seeds, fanouts):
+    ret = []
+    for K in fanouts:
+        subA = A[:, seeds]
+        sampleA = subA.individual_sampling(K, subA.edata["w"], False)
+        seeds = sampleA.all_nodes()
+        ret.append(sampleA.to_dgl_block(prefetch_edata={"w"}))
+    return seeds, ret
+
+
+def batch_weighted_graphsage_sampler(A, seeds, seeds_ptr, fanouts):
+    ret = []
+    for k in fanouts:
+        subA = A[:, seeds::seeds_ptr]
+        sampleA = subA.individual_sampling(k, subA.edata["w"], False)
+        seeds, seeds_ptr = sampleA.all_nodes()
+        ret.append(sampleA.to_dgl_block())
+    return ret
+
+
 def ladies_sampler(A, seeds, fanouts):
     # examples/ladies/ladies.py:7-21 of the reference
     input_node = seeds
@@ -87,6 +107,30 @@ def test_batch_graphsage_rewrites():
     c2 = gs.jit.compile(func=batch_graphsage_sampler,
                         args=(bm2, torch.arange(4), torch.tensor([0, 2, 4]), [5]))
     assert "_CAPI_BatchColSlicing" in targets(c2.gm)
+
+
+def test_weighted_graphsage_rewrites():
+    m = gs.Matrix(gs.Graph(10, 10))
+    m.edata["w"] = torch.ones(5)
+    c = gs.jit.compile(func=weighted_graphsage_sampler, args=(m, torch.arange(3), [15, 10]))
+    t = targets(c.gm)
+    # slice + weighted sample fused: the slice is never materialised
+    assert t.count("_CAPI_SlicingSamplingProbs") == 2
+    assert "_CAPI_Slicing" not in t and "_CAPI_SamplingProbs" not in t
+    fused = [n for n in c.gm.graph.nodes if n.target == "_CAPI_SlicingSamplingProbs"]
+    assert [n.args[4] for n in fused] == [15, 10]
+    assert all(n.args[1] == 1 and n.args[6] == gs._CSC and n.args[7] == gs._CSC | gs._COO
+               for n in fused)
+    # both layers draw by the weights of the *input* matrix (its placeholder)
+    assert fused[0].args[3] is fused[1].args[3] and fused[0].args[3].op == "placeholder"
+    bm = gs.BatchMatrix()
+    bm.load_from_matrix(m, False)
+    cb = gs.jit.compile(func=batch_weighted_graphsage_sampler,
+                        args=(bm, torch.arange(4), torch.tensor([0, 2, 4]), [5, 5]),
+                        try_compact=False, format_select=False)
+    tb = targets(cb.gm)
+    assert tb.count("_CAPI_BatchFusedSlicingSamplingProbs") == 2
+    assert "_CAPI_BatchColSlicing" not in tb and "_CAPI_BatchRowSamplingProbs" not in tb
 
 
 def test_ladies_rewrites():
@@ -231,3 +275,42 @@ def test_merged_u_mul_v_equals_eager():
     c = gs.jit.compile(func=pass_like_sampler, args=(m, seeds, u, v, u + 1, v + 1))
     assert torch.allclose(c(m, seeds, u, v, u + 1, v + 1),
                           pass_like_sampler(m, seeds, u, v, u + 1, v + 1))
+
+
+@pytest.mark.gpu
+def test_compiled_weighted_graphsage_matches_the_cdf_oracle():
+    """The fused weighted operator draws through the weight CDF of the input
+    matrix: bit-exact against the oracle's CDF sampler with the same seed and
+    call ids; the eager path (slice, then key-based sampling) obeys the same
+    invariants on the same seeds."""
+    from oracle import binding as orc
+    m = _graph()
+    indptr, indices = m.csc[0].cpu().numpy(), m.csc[1].cpu().numpy()
+    w = m.edata["w"].cpu().numpy()
+    seeds = torch.randperm(5000, generator=torch.Generator().manual_seed(8))[:300].to(DEV)
+    c = gs.jit.compile(func=weighted_graphsage_sampler, args=(m, seeds, [10, 5]))
+    gs.manual_seed(21)
+    _, blocks = c(m, seeds, [10, 5])
+    cdf = orc.weight_cdf(indptr, w)
+    s = seeds.cpu().numpy()
+    for layer, (K, blk) in enumerate(zip([10, 5], blocks)):
+        sub_indptr, col, rows, sel = orc.sample_weighted(indptr, indices, None, s, K, False,
+                                                         seed=21, call_id=layer, cdf=cdf)
+        uniq, _, r, cc = orc.unique_relabel(s, rows, edge_col=col)
+        assert np.array_equal(blk.row.cpu().numpy(), r)
+        assert np.array_equal(blk.col.cpu().numpy(), cc)
+        assert np.array_equal(blk.srcdata["_ID"].cpu().numpy(), uniq)
+        assert np.array_equal(blk.edata["w"].cpu().numpy(), w[sel])
+        s = uniq
+    # eager: another algorithm, the same rules
+    gs.manual_seed(21)
+    _, eager = weighted_graphsage_sampler(m, seeds, [10, 5])
+    deg = np.diff(indptr)
+    s = seeds.cpu().numpy()
+    blk = eager[0]
+    counts = np.bincount(blk.col.cpu().numpy(), minlength=s.size)
+    assert np.array_equal(counts, np.minimum(deg[s], 10))
+    src = blk.srcdata["_ID"].cpu().numpy()[blk.row.cpu().numpy()]
+    dst = s[blk.col.cpu().numpy()]
+    edges = set(zip(np.repeat(np.arange(5000), deg).tolist(), indices.tolist()))
+    assert all((int(d), int(u)) in edges for d, u in zip(dst, src))
