@@ -103,6 +103,51 @@ def kernel_bytes(name, sizes):
     return total
 
 
+def batch_graphsage_sampler(A, seeds, seeds_ptr, fanouts):
+    """The super-batched sampler of the reference's examples/graphsage/graphsage_e2e.py."""
+    ret = []
+    for k in fanouts:
+        subA = A[:, seeds::seeds_ptr]
+        sampleA = subA.individual_sampling(k, None, False)
+        seeds, seeds_ptr = sampleA.all_nodes()
+        ret.append(sampleA.to_dgl_block())
+    return ret
+
+
+def batch_weighted_graphsage_sampler(A, seeds, seeds_ptr, fanouts):
+    ret = []
+    for k in fanouts:
+        subA = A[:, seeds::seeds_ptr]
+        sampleA = subA.individual_sampling(k, subA.edata["w"], False)
+        seeds, seeds_ptr = sampleA.all_nodes()
+        ret.append(sampleA.to_dgl_block())
+    return ret
+
+
+def api_step_factory(indptr, indices, seeds, ptr, fanouts, probs):
+    """step(i) -> (sizes, None) through BatchMatrix, gs.jit.compile and libgs.so."""
+    import gsampler_amd as gs
+    m = gs.Matrix()
+    m.load_graph("CSC", [indptr, indices])
+    func = batch_graphsage_sampler
+    if probs is not None:
+        m.edata["w"] = probs
+        func = batch_weighted_graphsage_sampler
+    bm = gs.BatchMatrix()
+    bm.load_from_matrix(m, False)
+    compiled = gs.jit.compile(func=func, args=(bm, seeds, ptr, fanouts), try_compact=False,
+                              format_select=False)
+
+    def step(i):
+        layers = compiled(bm, seeds, ptr, fanouts)
+        sizes = []
+        for blocks in layers:
+            sizes.append((sum(b.num_dst for b in blocks), sum(b.num_edges() for b in blocks),
+                          sum(b.num_src for b in blocks)))
+        return sizes, None
+    return step
+
+
 def _kernel_table(capi, bytes_of):
     """Per-kernel totals of the library's event timers -> sorted list of dicts."""
     kernels = []
@@ -266,6 +311,10 @@ def main():
     ap.add_argument("--cpu-seconds", type=float, default=15.0,
                     help="target CPU time of the oracle baseline (0 = skip)")
     ap.add_argument("--seed", type=int, default=7777)
+    ap.add_argument("--path", default="abi", choices=["abi", "api"],
+                    help="abi: the C ABI through ctypes (default); api: the same GraphSAGE "
+                         "workload through BatchMatrix + gs.jit.compile and the torch "
+                         "custom class, per-batch blocks included")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build drives exactly one GPU (the super-batch is the unit "
@@ -314,6 +363,9 @@ def main():
     def step(i):
         return graphsage_step(capi, indptr, indices, seeds, ptr, fanouts, args.seed,
                               i * len(fanouts), probs, cdf)
+
+    if args.path == "api":
+        step = api_step_factory(indptr, indices, seeds, ptr, fanouts, probs)
 
     for i in range(args.warmup):
         step(i)
@@ -395,7 +447,7 @@ def main():
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 3), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "int64", "data": "synthetic",
-        "config": {"workload": f"{args.workload}: {wl['desc']}",
+        "config": {"workload": f"{args.workload}: {wl['desc']}", "path": args.path,
                    "fanouts": fanouts, "batches_per_launch": wl["batches"],
                    "seeds_per_batch": wl["batch_size"], "sampler_seed": args.seed,
                    "layer_sizes_S_E_U": sizes},

@@ -8,6 +8,8 @@
 #include <hip/hip_runtime_api.h>
 #include <torch/torch.h>
 
+#include <vector>
+
 #include "../../../include/gsampler_hip.h"
 
 namespace gs {
@@ -107,6 +109,78 @@ class AsyncCount {
   int slot_ = -1;
   bool pending_ = false;
   int64_t value_ = 0;
+};
+
+// Host copies of small offset arrays (batch pointers).  Splitting results per
+// batch needs them on the host; a blocking copy at that point waits for
+// everything queued on the stream.  Producers therefore announce an array as
+// soon as its kernel is queued (prefetch): the copy into pinned memory travels
+// while later kernels run, and values() only waits for that copy.  The last few
+// arrays are remembered, keyed by tensor identity + version; an entry keeps its
+// tensor alive, which is what makes that key safe.  Pinned blocks are reused
+// and live until the process ends.
+class OffsetMirror {
+ public:
+  static void prefetch(const torch::Tensor& offsets) { (void)entry_for(offsets); }
+  static const std::vector<int64_t>& values(const torch::Tensor& offsets) {
+    Entry& e = entry_for(offsets);
+    if (e.pending) {
+      check(hipEventSynchronize(e.event));
+      e.host.assign(e.pinned, e.pinned + e.count);
+      e.pending = false;
+    }
+    return e.host;
+  }
+
+ private:
+  struct Entry {
+    torch::Tensor tensor;
+    int64_t version = -1;
+    int64_t* pinned = nullptr;
+    size_t capacity = 0, count = 0;
+    hipEvent_t event = nullptr;
+    bool pending = false;
+    std::vector<int64_t> host;
+  };
+  static constexpr size_t kEntries = 8;
+  static void check(hipError_t e) {
+    TORCH_CHECK(e == hipSuccess, "HIP error: ", hipGetErrorString(e));
+  }
+  static Entry& entry_for(const torch::Tensor& offsets) {
+    static thread_local std::vector<Entry> ring(kEntries);
+    static thread_local size_t next = 0;
+    TORCH_CHECK(offsets.defined() && offsets.scalar_type() == torch::kInt64,
+                "batch offsets must be an int64 tensor");
+    for (Entry& e : ring)
+      if (e.tensor.defined() && e.tensor.is_same(offsets) &&
+          e.version == (int64_t)offsets._version())
+        return e;
+    Entry& e = ring[next++ % kEntries];
+    if (e.pending) check(hipEventSynchronize(e.event));  // its copy must not land later
+    e.tensor = offsets;
+    e.version = offsets._version();
+    e.count = (size_t)offsets.numel();
+    e.pending = false;
+    if (!offsets.is_cuda()) {
+      torch::Tensor c = offsets.contiguous();
+      e.host.assign(c.data_ptr<int64_t>(), c.data_ptr<int64_t>() + e.count);
+      return e;
+    }
+    if (e.capacity < e.count) {
+      if (e.pinned) check(hipHostFree(e.pinned));
+      e.capacity = e.count < 1024 ? 1024 : e.count;
+      check(hipHostMalloc((void**)&e.pinned, e.capacity * sizeof(int64_t), hipHostMallocDefault));
+    }
+    if (!e.event) check(hipEventCreateWithFlags(&e.event, hipEventDisableTiming));
+    torch::Tensor c = offsets.contiguous();
+    hipStream_t s = (hipStream_t)cur_stream();
+    if (e.count > 0)
+      check(hipMemcpyAsync(e.pinned, c.data_ptr<int64_t>(), e.count * sizeof(int64_t),
+                           hipMemcpyDeviceToHost, s));
+    check(hipEventRecord(e.event, s));
+    e.pending = true;
+    return e;
+  }
 };
 
 // Outputs are sized by an upper bound (and trimmed afterwards) only up to this

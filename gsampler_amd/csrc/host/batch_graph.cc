@@ -46,12 +46,17 @@ std::tuple<torch::Tensor, torch::Tensor> Graph::BatchGetCOOEids() {
   return {torch::Tensor(), torch::Tensor()};
 }
 
+static const std::vector<int64_t>& host_offsets(const torch::Tensor& offset) {
+  if (offset.scalar_type() != torch::kInt64)
+    return OffsetMirror::values(offset.to(torch::kInt64));
+  return OffsetMirror::values(offset);
+}
+
 std::vector<int64_t> Graph::BatchGetColCounts() {
   TORCH_CHECK(col_bptr_.defined() && col_bptr_.numel() > 0,
               "BatchGetColCounts: no column batch pointer set");
-  torch::Tensor host = col_bptr_.to(torch::kCPU);
-  const int64_t* p = host.data_ptr<int64_t>();
-  std::vector<int64_t> counts((size_t)host.numel() - 1);
+  const std::vector<int64_t>& p = host_offsets(col_bptr_);
+  std::vector<int64_t> counts(p.size() - 1);
   for (size_t i = 0; i < counts.size(); ++i) counts[i] = p[i + 1] - p[i];
   return counts;
 }
@@ -135,6 +140,7 @@ GraphAndIndex Graph::BatchFusedSlicingSampling(torch::Tensor seeds,
   g.col_bptr_ = col_bptr;
   g.orig_col_ids_ = ids(seeds, "seeds");
   g.edge_bptr_ = g.csc_->indptr.index_select(0, col_bptr);
+  OffsetMirror::prefetch(g.edge_bptr_);  // per-batch splits will ask for it
   return ret;
 }
 
@@ -193,10 +199,9 @@ std::tuple<torch::Tensor, torch::Tensor> Graph::BatchGetValidNodes(
 // ------------------------------------------------------------ free operators
 std::vector<torch::Tensor> SplitByOffset(torch::Tensor data,
                                          torch::Tensor offset) {
-  torch::Tensor host = offset.to(torch::kCPU).to(torch::kInt64).contiguous();
-  const int64_t* p = host.data_ptr<int64_t>();
+  const std::vector<int64_t>& p = host_offsets(offset);
   std::vector<int64_t> sizes;
-  for (int64_t i = 0; i + 1 < host.numel(); ++i) sizes.push_back(p[i + 1] - p[i]);
+  for (size_t i = 0; i + 1 < p.size(); ++i) sizes.push_back(p[i + 1] - p[i]);
   return torch::split_with_sizes(data, sizes);
 }
 
@@ -208,8 +213,7 @@ std::vector<torch::Tensor> SplitIndptrByOffset(torch::Tensor indptr,
   indptr = ids(indptr, "indptr");
   offset = ids(offset, "offset");
   const int64_t B = offset.numel() - 1;
-  torch::Tensor host = offset.to(torch::kCPU);
-  const int64_t* p = host.data_ptr<int64_t>();
+  const std::vector<int64_t>& p = host_offsets(offset);
   std::vector<int64_t> sizes;
   int64_t total = 0;
   for (int64_t i = 0; i < B; ++i) {

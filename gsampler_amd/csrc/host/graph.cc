@@ -322,6 +322,7 @@ Graph::Frontier& Graph::frontier_for(const torch::Tensor& seeds,
                           f->workspace.data_ptr(), f->workspace.numel(),
                           cur_stream()));
   f->count = AsyncCount(f->unique_ptr);
+  if (B > 1) OffsetMirror::prefetch(f->unique_ptr);  // per-batch splits will ask for it
   // at most S + E unique keys
   f->unique_buffer = new_ids(S + E <= kBoundLimit ? S + E : f->count.get(), rows);
   GS_CALL(gs_unique_fill(cptr(seeds), cptr(seeds_ptr), S, cptr(rows),

@@ -136,6 +136,7 @@ GraphAndIndex Graph::BatchFusedSlicingSamplingProbs(torch::Tensor seeds,
   g.col_bptr_ = col_bptr;
   g.orig_col_ids_ = ids(seeds, "seeds");
   g.edge_bptr_ = g.csc_->indptr.index_select(0, col_bptr);
+  OffsetMirror::prefetch(g.edge_bptr_);
   return ret;
 }
 

@@ -102,6 +102,7 @@ class compile:  # noqa: N801 -- the reference's public name
         gm = passes.dce(gm)
         if self._format_select and not self.use_batchmatrix:
             gm = passes.select_formats(gm)
+        gm = passes.sink_block_construction(gm)
         return gm
 
     # -------------------------------------------------------------------- run

@@ -326,6 +326,35 @@ def merge_u_mul_v(gm: fx.GraphModule) -> fx.GraphModule:
     return dce(gm)
 
 
+def sink_block_construction(gm: fx.GraphModule) -> fx.GraphModule:
+    """Splitting results per batch and building blocks is host work (and, for the
+    splits, a blocking read of the offsets).  Done where the sampler wrote it,
+    it holds back the launches of the next layer; nothing on the device depends
+    on it, so it moves to the end of the graph, in its original order."""
+    host_functions = {"batch_gen_block", "create_block_from_coo", "create_block_from_csc",
+                      "assign_block", "_CAPI_BatchSplitByOffset",
+                      "_CAPI_BatchIndptrSplitByOffset"}
+
+    def is_host_work(n: fx.Node) -> bool:
+        if n.op == "call_method":
+            return n.target == "_CAPI_BatchGetColCounts"
+        if n.op != "call_function":
+            return False
+        name = getattr(n.target, "__name__", None) or str(n.target)
+        return name.split(".")[-1] in host_functions
+
+    output = next(n for n in gm.graph.nodes if n.op == "output")
+    moving = set()
+    for n in gm.graph.nodes:            # topological order: users come later
+        if n.op == "output":
+            continue
+        if is_host_work(n) or any(a in moving for a in n.all_input_nodes):
+            moving.add(n)
+    for n in [n for n in gm.graph.nodes if n in moving]:
+        output.prepend(n)
+    return _finish(gm)
+
+
 # --------------------------------------------------------------- formats
 # operator -> (position of on_format, position of output_format or None); positions
 # count the operator object itself as argument 0 (python/gs/jit/module.py:21-31).
