@@ -2,30 +2,48 @@
 // minor id (row id of a CSC, or any id array of a COO) belongs to a picked set
 // and relabel that id to its position in the set.
 //
-//   count: hash the picked ids (smallest position wins for repeated ids), flag
-//          every edge, exclusive-scan the flags; out_indptr[c] =
-//          prefix[indptr[c]] needs no per-column pass.
-//   fill : kept edge e goes to position prefix[e], edge order preserved.
+//   count: hash the picked ids (smallest position wins for repeated ids); a
+//          wave tests 256 consecutive edges as four coalesced rows whose
+//          ballots are the chunk's flag words and counts the kept ones; scan
+//          of the chunk counts; out_indptr[c] = kept edges before indptr[c].
+//   fill : kept edge e goes to its rank (chunk offset + popcounts), edge order
+//          preserved; the small table is looked up again instead of storing a
+//          value per edge.
 #include "common.h"
 #include "hashtable.h"
 #include "scan.h"
 
 namespace gs {
 
+constexpr int kMemberWords = kBlock / kWave;  // flag words per chunk of kBlock edges
+constexpr int kMemberChunksPerWave = 8;
+constexpr int kMemberLdsSlots = 4096;  // tables up to this size are staged in LDS (32 KB)
+
 struct MemberWs {
-  uint64_t* table;  // [2 * num_picked + 2]
-  int64_t* prefix;  // [nnz + 1]
+  uint64_t* table;     // [member_table_slots(num_picked)]
+  uint64_t* flags;     // [chunks * kMemberWords]
+  int64_t* chunk_off;  // [chunks + 1]
   void* scan_ws;
   size_t scan_ws_bytes;
+  int64_t chunks;
   size_t total;
 };
+
+// Slots of the table: four per picked id while that still fits in LDS (fewer
+// probes for the ids that are not there, which are most), else two.
+static uint64_t member_table_slots(int64_t num_picked) {
+  const uint64_t roomy = (uint64_t)(4 * num_picked + 2);
+  return roomy <= (uint64_t)kMemberLdsSlots ? roomy : (uint64_t)(2 * num_picked + 2);
+}
 
 static MemberWs carve_member(void* ws, int64_t nnz, int64_t num_picked) {
   Carver c(ws);
   MemberWs w;
-  w.table = c.take<uint64_t>((size_t)(2 * num_picked + 2));
-  w.prefix = c.take<int64_t>((size_t)nnz + 1);
-  w.scan_ws_bytes = scan_workspace_bytes(nnz + 1);
+  w.chunks = ceil_div(nnz > 0 ? nnz : 1, kBlock);
+  w.table = c.take<uint64_t>((size_t)member_table_slots(num_picked));
+  w.flags = c.take<uint64_t>((size_t)w.chunks * kMemberWords);
+  w.chunk_off = c.take<int64_t>((size_t)w.chunks + 1);
+  w.scan_ws_bytes = scan_workspace_bytes(w.chunks + 1);
   w.scan_ws = c.take<char>(w.scan_ws_bytes);
   w.total = c.total();
   return w;
@@ -40,46 +58,170 @@ __global__ __launch_bounds__(kBlock) void member_insert_kernel(
   table_insert_min(table, cap, key, (uint64_t)i);
 }
 
+// A small table (the picked set of a layer-wise sampler is a few hundred ids)
+// is copied into LDS once per work-group: 64 lanes probing 64 different slots
+// cost the vector cache a tag look-up each, the LDS a few cycles in all.
+template <bool kInLds>
+__device__ __forceinline__ const uint64_t* stage_table(const uint64_t* __restrict__ table,
+                                                       uint64_t cap, uint64_t* lds) {
+  if (!kInLds) return table;
+  for (uint64_t i = threadIdx.x; i < cap; i += kBlock) lds[i] = table[i];
+  __syncthreads();
+  return lds;
+}
+
+// N look-ups in step: the probes of a round are issued together, so a lane
+// waits for the longest of its N probe runs instead of their sum.  slot[j] is
+// where key[j] was found, cap if it is absent.
+template <int N>
+__device__ __forceinline__ void table_find_many(const uint64_t* tab, uint64_t cap,
+                                                const uint64_t (&key)[N],
+                                                uint64_t (&slot)[N]) {
+  bool open[N];
+  bool any = false;
+#pragma unroll
+  for (int j = 0; j < N; ++j) {
+    open[j] = key[j] <= kMaxPackedKey;
+    slot[j] = open[j] ? home_slot(key[j], cap) : cap;
+    any |= open[j];
+  }
+  for (uint64_t probes = 0; any && probes < cap; ++probes) {
+    uint64_t cur[N];
+#pragma unroll
+    for (int j = 0; j < N; ++j) cur[j] = open[j] ? tab[slot[j]] : 0;
+    any = false;
+#pragma unroll
+    for (int j = 0; j < N; ++j) {
+      if (!open[j]) continue;
+      if ((cur[j] >> 32) == key[j]) {
+        open[j] = false;
+      } else if (cur[j] == kEmptySlot) {
+        open[j] = false;
+        slot[j] = cap;
+      } else if (++slot[j] == cap) {
+        slot[j] = 0;
+      }
+      any |= open[j];
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < N; ++j)
+    if (open[j]) slot[j] = cap;  // probe budget spent: a table too small for its keys
+}
+
+template <bool kInLds>
 __global__ __launch_bounds__(kBlock) void member_flag_kernel(
     const int64_t* __restrict__ ids, int64_t nnz,
-    const uint64_t* __restrict__ table, uint64_t cap,
-    int64_t* __restrict__ flags) {
-  const int64_t e = (int64_t)blockIdx.x * kBlock + threadIdx.x;
-  if (e > nnz) return;
-  int64_t f = 0;
-  if (e < nnz) {
-    const uint64_t key = (uint64_t)ids[e];
-    f = (key <= kMaxPackedKey && table_find(table, cap, key) < cap) ? 1 : 0;
+    const uint64_t* __restrict__ global_table, uint64_t cap,
+    uint64_t* __restrict__ flags, int64_t* __restrict__ chunk_count) {
+  __shared__ uint64_t lds_table[kInLds ? kMemberLdsSlots : 1];
+  const uint64_t* table = stage_table<kInLds>(global_table, cap, lds_table);
+  const int64_t num_chunks = ceil_div_dev(nnz, kBlock);
+  const int64_t wave = (int64_t)blockIdx.x * kMemberWords + threadIdx.x / kWave;
+  const int lane = lane_id();
+  for (int c = 0; c < kMemberChunksPerWave; ++c) {
+    const int64_t chunk = wave * kMemberChunksPerWave + c;
+    if (chunk >= num_chunks) return;
+    const int64_t e0 = chunk * kBlock;
+    uint64_t key[kMemberWords];
+#pragma unroll
+    for (int j = 0; j < kMemberWords; ++j) {
+      const int64_t e = e0 + j * kWave + lane;
+      key[j] = e < nnz ? (uint64_t)ids[e] : ~0ull;
+    }
+    uint64_t slot[kMemberWords], word[kMemberWords];
+    table_find_many<kMemberWords>(table, cap, key, slot);
+#pragma unroll
+    for (int j = 0; j < kMemberWords; ++j) word[j] = __ballot(slot[j] < cap);
+    if (lane == 0) {
+      int total = 0;
+#pragma unroll
+      for (int j = 0; j < kMemberWords; ++j) {
+        flags[chunk * kMemberWords + j] = word[j];
+        total += __popcll(word[j]);
+      }
+      chunk_count[chunk] = total;
+      if (chunk == num_chunks - 1) chunk_count[num_chunks] = 0;
+    }
   }
-  flags[e] = f;  // flags[nnz] = 0 so that the scan leaves the total there
+}
+
+// Kept edges at positions < e.
+__device__ __forceinline__ int64_t member_rank_before(
+    int64_t e, const uint64_t* __restrict__ flags,
+    const int64_t* __restrict__ chunk_off) {
+  const int64_t chunk = e / kBlock;
+  int64_t r = chunk_off[chunk];
+  const int in_chunk = (int)(e - chunk * kBlock);
+  const int full = in_chunk / kWave, rem = in_chunk % kWave;
+  for (int w = 0; w < full; ++w) r += __popcll(flags[chunk * kMemberWords + w]);
+  if (rem) r += __popcll(flags[chunk * kMemberWords + full] & ((1ull << rem) - 1));
+  return r;
 }
 
 __global__ __launch_bounds__(kBlock) void member_indptr_kernel(
     const int64_t* __restrict__ indptr, int64_t num_major,
-    const int64_t* __restrict__ prefix, int64_t nnz,
-    int64_t* __restrict__ out_indptr, int64_t* __restrict__ out_total) {
+    const uint64_t* __restrict__ flags, const int64_t* __restrict__ chunk_off,
+    int64_t nnz, int64_t* __restrict__ out_indptr, int64_t* __restrict__ out_total) {
   const int64_t c = (int64_t)blockIdx.x * kBlock + threadIdx.x;
-  if (c == 0 && out_total) *out_total = prefix[nnz];
+  const int64_t num_chunks = ceil_div_dev(nnz, kBlock);
+  if (c == 0 && out_total) *out_total = nnz > 0 ? chunk_off[num_chunks] : 0;
   if (indptr == nullptr || c > num_major) return;
-  out_indptr[c] = prefix[indptr[c]];
+  const int64_t e = indptr[c];
+  out_indptr[c] = nnz == 0 ? 0
+                  : (e >= nnz ? chunk_off[num_chunks] : member_rank_before(e, flags, chunk_off));
 }
 
+template <bool kInLds>
 __global__ __launch_bounds__(kBlock) void member_fill_kernel(
     const int64_t* __restrict__ ids, int64_t nnz,
-    const uint64_t* __restrict__ table, uint64_t cap,
-    const int64_t* __restrict__ prefix, const int64_t* __restrict__ indptr,
-    int64_t num_major, const int64_t* __restrict__ edge_major,
-    int64_t* __restrict__ out_major, int64_t* __restrict__ out_minor,
-    int64_t* __restrict__ out_select) {
-  const int64_t e = (int64_t)blockIdx.x * kBlock + threadIdx.x;
-  if (e >= nnz) return;
-  const int64_t pos = prefix[e];
-  if (prefix[e + 1] == pos) return;
-  const uint64_t key = (uint64_t)ids[e];
-  out_minor[pos] = (int64_t)(uint32_t)table[table_find(table, cap, key)];
-  out_select[pos] = e;
-  if (out_major)
-    out_major[pos] = edge_major ? edge_major[e] : segment_of(indptr, num_major, e);
+    const uint64_t* __restrict__ global_table, uint64_t cap,
+    const uint64_t* __restrict__ flags, const int64_t* __restrict__ chunk_off,
+    const int64_t* __restrict__ indptr, int64_t num_major,
+    const int64_t* __restrict__ edge_major, int64_t* __restrict__ out_major,
+    int64_t* __restrict__ out_minor, int64_t* __restrict__ out_select) {
+  __shared__ uint64_t lds_table[kInLds ? kMemberLdsSlots : 1];
+  const uint64_t* table = stage_table<kInLds>(global_table, cap, lds_table);
+  const int64_t num_chunks = ceil_div_dev(nnz, kBlock);
+  const int64_t wave = (int64_t)blockIdx.x * kMemberWords + threadIdx.x / kWave;
+  const int lane = lane_id();
+  for (int c = 0; c < kMemberChunksPerWave; ++c) {
+    const int64_t chunk = wave * kMemberChunksPerWave + c;
+    if (chunk >= num_chunks) return;
+    const int64_t e0 = chunk * kBlock;
+    const int64_t e_last = e0 + kBlock - 1 < nnz ? e0 + kBlock - 1 : nnz - 1;
+    // segments the chunk touches (for out_major without edge_major): mostly one
+    int64_t seg_lo = 0, seg_hi = 0;
+    if (out_major && !edge_major) {
+      seg_lo = segment_of(indptr, num_major, wave_uniform_first(e0));
+      seg_hi = segment_of(indptr, num_major, wave_uniform_first(e_last));
+    }
+    int64_t before = chunk_off[chunk];
+    uint64_t word[kMemberWords], key[kMemberWords], slot[kMemberWords];
+#pragma unroll
+    for (int j = 0; j < kMemberWords; ++j) {
+      word[j] = flags[chunk * kMemberWords + j];
+      const int64_t e = e0 + j * kWave + lane;
+      key[j] = ((word[j] >> lane) & 1ull) ? (uint64_t)ids[e] : ~0ull;
+    }
+    table_find_many<kMemberWords>(table, cap, key, slot);
+#pragma unroll
+    for (int j = 0; j < kMemberWords; ++j) {
+      const int64_t e = e0 + j * kWave + lane;
+      if ((word[j] >> lane) & 1ull) {
+        const int64_t pos = before + __popcll(word[j] & ((1ull << lane) - 1));
+        out_minor[pos] = (int64_t)(uint32_t)table[slot[j] < cap ? slot[j] : 0];
+        out_select[pos] = e;
+        if (out_major)
+          out_major[pos] =
+              edge_major ? edge_major[e]
+                         : (seg_lo == seg_hi
+                                ? seg_lo
+                                : seg_lo + segment_of(indptr + seg_lo, seg_hi - seg_lo + 1, e));
+      }
+      before += __popcll(word[j]);
+    }
+  }
 }
 
 }  // namespace gs
@@ -112,7 +254,7 @@ int gs_minor_slice_count(const int64_t* ids, int64_t nnz, const int64_t* picked,
     return GS_ERR_WORKSPACE;
   }
   hipStream_t s = as_stream(stream);
-  const uint64_t cap = (uint64_t)(2 * num_picked + 2);
+  const uint64_t cap = member_table_slots(num_picked);
   GS_LAUNCH("member_clear", s,
             table_fill_kernel<><<<dim3((unsigned)ceil_div((int64_t)cap, kBlock * 4)),
                                   dim3(kBlock), 0, s>>>(w.table, (int64_t)cap,
@@ -122,18 +264,25 @@ int gs_minor_slice_count(const int64_t* ids, int64_t nnz, const int64_t* picked,
               member_insert_kernel<<<dim3((unsigned)ceil_div(num_picked, kBlock)),
                                      dim3(kBlock), 0, s>>>(picked, num_picked,
                                                            w.table, cap));
-  GS_LAUNCH("member_flag", s,
-            member_flag_kernel<<<dim3((unsigned)ceil_div(nnz + 1, kBlock)),
-                                 dim3(kBlock), 0, s>>>(ids, nnz, w.table, cap,
-                                                       w.prefix));
-  int rc = exclusive_scan_i64(w.prefix, w.prefix, nnz + 1, w.scan_ws,
-                              w.scan_ws_bytes, s);
-  if (rc != GS_OK) return rc;
+  if (nnz > 0) {
+    const int64_t blocks = ceil_div(w.chunks, kMemberWords * kMemberChunksPerWave);
+    if (cap <= (uint64_t)kMemberLdsSlots)
+      GS_LAUNCH("member_flag", s,
+                member_flag_kernel<true><<<dim3((unsigned)blocks), dim3(kBlock), 0, s>>>(
+                    ids, nnz, w.table, cap, w.flags, w.chunk_off));
+    else
+      GS_LAUNCH("member_flag", s,
+                member_flag_kernel<false><<<dim3((unsigned)blocks), dim3(kBlock), 0, s>>>(
+                    ids, nnz, w.table, cap, w.flags, w.chunk_off));
+    int rc = exclusive_scan_i64(w.chunk_off, w.chunk_off, w.chunks + 1, w.scan_ws,
+                                w.scan_ws_bytes, s);
+    if (rc != GS_OK) return rc;
+  }
   const int64_t n = indptr ? num_major + 1 : 1;
   GS_LAUNCH("member_indptr", s,
             member_indptr_kernel<<<dim3((unsigned)ceil_div(n, kBlock)),
-                                   dim3(kBlock), 0, s>>>(indptr, num_major,
-                                                         w.prefix, nnz,
+                                   dim3(kBlock), 0, s>>>(indptr, num_major, w.flags,
+                                                         w.chunk_off, nnz,
                                                          out_indptr, out_total));
   return GS_OK;
 }
@@ -157,12 +306,18 @@ int gs_minor_slice_fill(const int64_t* ids, int64_t nnz, int64_t num_picked,
     return GS_ERR_WORKSPACE;
   }
   hipStream_t s = as_stream(stream);
-  const uint64_t cap = (uint64_t)(2 * num_picked + 2);
-  GS_LAUNCH("member_fill", s,
-            member_fill_kernel<<<dim3((unsigned)ceil_div(nnz, kBlock)),
-                                 dim3(kBlock), 0, s>>>(
-                ids, nnz, w.table, cap, w.prefix, indptr, num_major, edge_major,
-                out_major, out_minor, out_select));
+  const uint64_t cap = member_table_slots(num_picked);
+  const dim3 grid((unsigned)ceil_div(w.chunks, kMemberWords * kMemberChunksPerWave));
+  if (cap <= (uint64_t)kMemberLdsSlots)
+    GS_LAUNCH("member_fill", s,
+              member_fill_kernel<true><<<grid, dim3(kBlock), 0, s>>>(
+                  ids, nnz, w.table, cap, w.flags, w.chunk_off, indptr, num_major,
+                  edge_major, out_major, out_minor, out_select));
+  else
+    GS_LAUNCH("member_fill", s,
+              member_fill_kernel<false><<<grid, dim3(kBlock), 0, s>>>(
+                  ids, nnz, w.table, cap, w.flags, w.chunk_off, indptr, num_major,
+                  edge_major, out_major, out_minor, out_select));
   return GS_OK;
 }
 
