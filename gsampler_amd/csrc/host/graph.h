@@ -187,7 +187,11 @@ class Graph : public torch::CustomClassHolder {
     torch::Tensor unique_buffer;
     AsyncCount count;
     const torch::Tensor& frontier() {
-      if (!unique_.defined()) unique_ = unique_buffer.narrow(0, 0, count.get());
+      if (!unique_.defined()) {
+        const int64_t total = count.get();
+        TORCH_CHECK(total >= 0, "unique / relabel: ids must lie in [0, 2^32 - 2]");
+        unique_ = unique_buffer.narrow(0, 0, total);
+      }
       return unique_;
     }
     bool matches(const torch::Tensor& s, const torch::Tensor& r,

@@ -111,6 +111,7 @@ struct UniqueWs {
   int32_t* chunk_batch;   // [chunks + 1] batch of the first position of a chunk
   int32_t* etile_batch;   // [edge tiles + 1] batch of the first edge of a tile
   int64_t* bucket_cnt;    // [max_buckets + 1] entries per bucket
+  int* bad_key;           // [1] set when a key does not fit the packed entry
   int64_t* bucket_off;    // [max_buckets + 1] first entry of a bucket
   uint64_t* packed;       // [N] key << 32 | local, grouped by bucket
   uint32_t* first;        // [N] local position of the first occurrence
@@ -143,6 +144,7 @@ static UniqueWs carve_unique(void* ws, int64_t S, int64_t E, int64_t B) {
   w.chunk_batch = c.take<int32_t>((size_t)w.chunks + 1);
   w.etile_batch = c.take<int32_t>((size_t)w.etiles + 1);
   w.bucket_cnt = c.take<int64_t>((size_t)w.max_buckets + 1);
+  w.bad_key = c.take<int>(1);
   w.bucket_off = c.take<int64_t>((size_t)w.max_buckets + 1);
   w.packed = c.take<uint64_t>((size_t)n1);
   w.first = c.take<uint32_t>((size_t)n1);
@@ -197,11 +199,12 @@ __global__ __launch_bounds__(kBlock) void unique_prep_kernel(
     Keys k, int64_t bucket_keys, BatchInfo* __restrict__ batch,
     int64_t* __restrict__ flat_ptr, int64_t* __restrict__ tile_ptr,
     int64_t* __restrict__ bucket_ptr, int64_t* __restrict__ bucket_cnt,
-    int64_t max_buckets) {
+    int64_t max_buckets, int* __restrict__ bad_key) {
   for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i <= max_buckets;
        i += (int64_t)gridDim.x * kBlock)
     bucket_cnt[i] = 0;
   if (blockIdx.x != 0) return;
+  if (threadIdx.x == 0) *bad_key = 0;
   __shared__ int64_t smem[kBlock / kWave + 1];
   int64_t tile_carry = 0, bucket_carry = 0;
   for (int64_t base = 0; base <= k.B; base += kBlock) {
@@ -299,25 +302,27 @@ __device__ __forceinline__ uint64_t key_at(const Keys& k, const BatchInfo& b,
 __global__ __launch_bounds__(kBlock) void unique_hist_kernel(
     Keys k, const int32_t* __restrict__ tile_batch,
     const BatchInfo* __restrict__ batch, int64_t* bucket_cnt, int64_t max_tiles,
-    int remap) {
+    int remap, int* bad_key) {
   __shared__ uint32_t hist[kMaxBuckets];
   const int64_t tile = unit_of_block(max_tiles, remap);
   if (tile >= max_tiles) return;
   TileInfo t;
   if (!tile_info(tile, tile_batch, batch, &t)) return;  // uniform per work-group
   const uint32_t buckets = (uint32_t)t.b.buckets;
-  if (buckets == 1) {  // nothing to choose
-    if (threadIdx.x == 0)
-      atomicAdd((unsigned long long*)&bucket_cnt[t.b.bucket0],
-                (unsigned long long)(t.end - t.begin));
-    return;
-  }
+  if (buckets == 1 && threadIdx.x == 0)
+    atomicAdd((unsigned long long*)&bucket_cnt[t.b.bucket0],
+              (unsigned long long)(t.end - t.begin));
   uint32_t key[kPartItems];
+  bool bad = false;
 #pragma unroll
   for (int i = 0; i < kPartItems; ++i) {  // all loads in flight before any use
     const int64_t l = t.begin + i * kBlock + threadIdx.x;
-    key[i] = l < t.end ? (uint32_t)key_at(k, t.b, l) : 0u;
+    const uint64_t full = l < t.end ? key_at(k, t.b, l) : 0ull;
+    bad |= full > kMaxPackedKey;  // negative ids land here too
+    key[i] = (uint32_t)full;
   }
+  if (bad) *bad_key = 1;  // every writer stores the same value
+  if (buckets == 1) return;  // nothing to choose
   for (uint32_t i = threadIdx.x; i < buckets; i += kBlock) hist[i] = 0;
   __syncthreads();
 #pragma unroll
@@ -719,13 +724,16 @@ __device__ __forceinline__ int64_t rank_before(
   return r;
 }
 
+// unique_ptr[B] = -1 tells the caller that some key did not fit the packed
+// entry (an id above 2^32 - 2 or a negative one): nothing else is valid then.
 __global__ void unique_ptr_kernel(const int64_t* __restrict__ flat_ptr,
                                   int64_t B, const uint64_t* __restrict__ flags,
                                   const int64_t* __restrict__ block_off,
+                                  const int* __restrict__ bad_key,
                                   int64_t* __restrict__ unique_ptr) {
   const int64_t b = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (b > B) return;
-  unique_ptr[b] = rank_before(flat_ptr[b], flags, block_off);
+  unique_ptr[b] = (b == B && *bad_key) ? -1 : rank_before(flat_ptr[b], flags, block_off);
 }
 
 // ---------------------------------------------------------------- fill
@@ -881,7 +889,7 @@ int gs_unique_count(const int64_t* seeds, const int64_t* seeds_ptr,
     GS_LAUNCH("unique_prep", s,
               unique_prep_kernel<<<dim3((unsigned)blocks), dim3(kBlock), 0, s>>>(
                   k, tn.bucket_keys, w.batch, w.flat_ptr, w.tile_ptr,
-                  w.bucket_ptr, w.bucket_cnt, w.max_buckets));
+                  w.bucket_ptr, w.bucket_cnt, w.max_buckets, w.bad_key));
     const int64_t units = w.max_tiles + w.max_buckets + w.chunks + 1 + w.etiles + 1;
     GS_LAUNCH("unique_units", s,
               unique_units_kernel<<<dim3((unsigned)ceil_div(units, kBlock)),
@@ -893,7 +901,8 @@ int gs_unique_count(const int64_t* seeds, const int64_t* seeds_ptr,
   const dim3 tile_grid((unsigned)grid_for_units(w.max_tiles, tn.remap));
   GS_LAUNCH("unique_hist", s,
             unique_hist_kernel<<<tile_grid, dim3(kBlock), 0, s>>>(
-                k, w.tile_batch, w.batch, w.bucket_cnt, w.max_tiles, tn.remap));
+                k, w.tile_batch, w.batch, w.bucket_cnt, w.max_tiles, tn.remap,
+                w.bad_key));
   GS_LAUNCH("unique_bucket_scan", s,
             unique_bucket_scan_kernel<<<dim3(1), dim3(kBucketScanThreads), 0, s>>>(
                 w.bucket_ptr, B, w.bucket_cnt, w.bucket_off));
@@ -925,7 +934,8 @@ int gs_unique_count(const int64_t* seeds, const int64_t* seeds_ptr,
   GS_LAUNCH("unique_ptr", s,
             unique_ptr_kernel<<<dim3((unsigned)ceil_div(B + 1, kBlock)),
                                 dim3(kBlock), 0, s>>>(w.flat_ptr, B, w.flags,
-                                                      w.block_off, unique_ptr));
+                                                      w.block_off, w.bad_key,
+                                                      unique_ptr));
   return GS_OK;
 }
 

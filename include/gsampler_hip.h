@@ -247,7 +247,8 @@ int gs_list_sample_weighted_fill(const float* probs, const int64_t* range,
  *   rank of every row key (nullable); out_col[num_rows_keys] = batch-local rank
  *   of seeds[edge_col[e]] (nullable; edge_col holds positions into `seeds`).
  *   May be called any number of times while the workspace is kept.
- * Keys must lie in [0, 2^32 - 2] and one batch may hold at most 2^32 - 2 keys.
+ * Keys must lie in [0, 2^32 - 2] and one batch may hold at most 2^32 - 2 keys;
+ * count reports a key outside that range as unique_ptr[num_batches] = -1.
  * Stands in for TensorUniqueCUDA / TensorRelabelCUDA
  * (src/cuda/unique_reindex.cu:174-199) and BatchCOORelabelCUDA
  * (src/cuda/batch/batch_relabel.cu:480-498).

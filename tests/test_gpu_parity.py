@@ -213,3 +213,14 @@ def test_format_and_batch_helpers_parity():
     offset = np.array([0, 100, 100, 1500, 3000])
     assert np.array_equal(N(capi.split_indptr(T(indptr), T(offset))),
                           orc.split_indptr(indptr, offset))
+
+
+def test_unique_rejects_ids_that_do_not_fit():
+    seeds = np.array([1, 2, 3])
+    for bad in (2**32 - 1, 2**40, -5):
+        rows = np.array([5, bad, 7])
+        with pytest.raises(capi.GsError):
+            capi.unique_relabel(T(seeds), T(rows))
+    # the largest admissible id still works afterwards
+    assert_same(capi.unique_relabel(T(seeds), T(np.array([2**32 - 2, 5]))),
+                orc.unique_relabel(seeds, np.array([2**32 - 2, 5])))
