@@ -248,6 +248,29 @@ def ladies_sampler(A, seeds, fanouts):
     return seeds, ret
 
 
+def ladies_step_oracle(orc, indptr, indices, w, seeds, fanouts, num_rows, call_base):
+    """The same two LADIES layers on the CPU: the oracle's operators chained by hand
+    (column slice, e^2 row sums, weighted collective pick, row slice, the two
+    normalisations, relabel).  Returns the number of block edges."""
+    import numpy as np
+    edges = 0
+    for layer, K in enumerate(fanouts):
+        sub_indptr, coo_col, rows, sel = orc.col_slice(indptr, indices, seeds)
+        w_sub = w[sel]
+        prob = orc.e_square_sum(("coo", rows, coo_col), w_sub, 2, num_rows)
+        selected, _ = orc.list_sample_weighted(prob, K, call_id=call_base + layer)
+        out_indptr, major, minor, select = orc.minor_slice(rows, selected, indptr=sub_indptr)
+        w2 = orc.sddmm(("csc", out_indptr, minor), "div", w_sub[select], prob[selected], 1, 0)
+        col_sum = orc.spmm(("csc", out_indptr, minor), "copy_rhs", "sum", None, w2, 0,
+                           seeds.size)
+        w3 = orc.sddmm(("csc", out_indptr, minor), "div", w2, col_sum, 1, 2)
+        uniq, _, _, _ = orc.unique_relabel(seeds, selected[minor], edge_col=major)
+        edges += int(minor.size)
+        seeds = uniq
+        del w3
+    return edges
+
+
 def run_ladies(args, wl, capi, dev):
     """LADIES through the Python Matrix API and the torch custom class (the
     whole drop-in stack), compiled with gs.jit.compile.  A step = one 2-layer sample."""
@@ -290,14 +313,31 @@ def run_ladies(args, wl, capi, dev):
     kernels = _kernel_table(capi, lambda name: 0)
     capi.profile_enable(False)
     sliced = [int(b.num_edges()) for b in blocks]
+    cpu = None
+    if args.cpu_seconds > 0:
+        from oracle import binding as orc
+        h = [t.cpu().numpy() for t in (indptr, indices, w, seeds)]
+        ladies_step_oracle(orc, *h, fanouts, A.num_rows(), 0)          # warm-up
+        t_cpu, e_cpu, runs = 0.0, 0, 0
+        while t_cpu < args.cpu_seconds and runs < 1000:
+            t = time.perf_counter()
+            e_cpu += ladies_step_oracle(orc, *h, fanouts, A.num_rows(), 2 * (runs + 1))
+            t_cpu += time.perf_counter() - t
+            runs += 1
+        cpu = dict(value=round(e_cpu / t_cpu, 1), unit="edges/s", cores=orc.num_threads(),
+                   kind="port", sample=f"{runs} two-layer samples on the same graph and seeds in "
+                                       f"{t_cpu:.1f} s, OpenMP oracle operators chained by hand",
+                   host_cpus=os.cpu_count())
+    value = edges / elapsed
     return {
-        "metric": "sampled_edges_per_sec", "value": round(edges / elapsed, 1), "unit": "edges/s",
+        "metric": "sampled_edges_per_sec", "value": round(value, 1), "unit": "edges/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(elapsed / args.steps * 1e3, 3), "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": f"{args.workload}: {wl['desc']}", "fanouts": fanouts,
                    "seeds": wl["seeds"], "block_edges_last_step": sliced},
-        "roofline": _roofline(kernels[0]), "cpu_baseline": None, "gpu_over_cpu": None,
+        "roofline": _roofline(kernels[0]), "cpu_baseline": cpu,
+        "gpu_over_cpu": round(value / cpu["value"], 1) if cpu else None,
         "kernels": kernels, "graph_build_s": round(t_build, 1),
     }
 

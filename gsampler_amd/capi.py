@@ -58,6 +58,7 @@ SIGNATURES = {
     "gs_sorted_to_indptr": (_int, [_p, _i64, _i64, _p, _p]),
     "gs_decode_batch_ids": (_int, [_p, _i64, _i64, _p, _p, _p]),
     "gs_split_indptr": (_int, [_p, _p, _i64, _i64, _p, _p]),
+    "gs_first_position": (_int, [_p, _i64, _i64, _p, _p]),
     "gs_sddmm": (_int, [_int, _p, _p, _i64, _i64, _p, _int, _int, _p, _p, _p, _int, _int,
                         _i64, _i64, _i64, _i64, _p, _p, _p]),
     "gs_fused_u_op_v": (_int, [_int, _p, _p, _i64, _i64, _int, _int, _p, _p, _p, _p, _p,
@@ -331,6 +332,14 @@ def sorted_to_indptr(sorted_ids: torch.Tensor, num_cols: int) -> torch.Tensor:
     out = torch.empty(num_cols + 1, dtype=torch.int64, device=sorted_ids.device)
     check(lib().gs_sorted_to_indptr(_ptr(sorted_ids), sorted_ids.numel(), num_cols,
                                     out.data_ptr(), _stream()))
+    return out
+
+
+def first_position(ids: torch.Tensor, num_ids: int) -> torch.Tensor:
+    """first[r] = smallest e with ids[e] == r, INT64_MAX when r does not occur."""
+    ids = _i64t(ids, "ids")
+    out = torch.empty(num_ids, dtype=torch.int64, device=ids.device)
+    check(lib().gs_first_position(_ptr(ids), ids.numel(), num_ids, _ptr(out), _stream()))
     return out
 
 

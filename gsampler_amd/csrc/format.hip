@@ -31,6 +31,66 @@ __global__ __launch_bounds__(kBlock) void sorted_to_indptr_kernel(
 
 }  // namespace gs
 
+namespace gs {
+
+// first[r] = smallest e with ids[e] == r (INT64_MAX for an id that does not
+// occur), for ids in a small dense range [0, num_ids).  Atomics from all dies
+// on a few hundred addresses would queue up at the memory side, so a
+// work-group first takes the minimum over its tile of edges in LDS and then
+// sends one atomic per id it met -- and only if the value in memory is not
+// already smaller, which it is for every tile but the first few.
+constexpr int kFirstLdsIds = 4096;
+constexpr int kFirstTile = kBlock * 32;
+
+__global__ __launch_bounds__(kBlock) void first_position_lds_kernel(
+    const int64_t* __restrict__ ids, int64_t n, int64_t num_ids, long long* first) {
+  __shared__ long long tile_min[kFirstLdsIds];
+  for (int i = threadIdx.x; i < num_ids; i += kBlock) tile_min[i] = INT64_MAX;
+  __syncthreads();
+  const int64_t e0 = (int64_t)blockIdx.x * kFirstTile;
+  const int64_t e1 = e0 + kFirstTile < n ? e0 + kFirstTile : n;
+  for (int64_t base = e0; base < e1; base += kBlock * 8) {
+    int64_t r[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int64_t e = base + j * kBlock + threadIdx.x;
+      r[j] = e < e1 ? ids[e] : -1;
+    }
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int64_t e = base + j * kBlock + threadIdx.x;
+      if (r[j] >= 0 && r[j] < num_ids && tile_min[r[j]] > e)
+        atomicMin(&tile_min[r[j]], (long long)e);
+    }
+  }
+  __syncthreads();
+  for (int i = threadIdx.x; i < num_ids; i += kBlock) {
+    const long long m = tile_min[i];
+    if (m != INT64_MAX &&
+        __hip_atomic_load(first + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) > m)
+      atomicMin(first + i, m);
+  }
+}
+
+// The same for a range of ids too large for LDS: one atomic per edge unless a
+// smaller position is already there.
+__global__ __launch_bounds__(kBlock) void first_position_kernel(
+    const int64_t* __restrict__ ids, int64_t n, int64_t num_ids, long long* first) {
+  const int64_t e = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (e >= n) return;
+  const int64_t r = ids[e];
+  if (r < 0 || r >= num_ids) return;
+  if (__hip_atomic_load(first + r, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) > e)
+    atomicMin(first + r, (long long)e);
+}
+
+__global__ __launch_bounds__(kBlock) void fill_i64_kernel(int64_t* p, int64_t n, int64_t v) {
+  const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (i < n) p[i] = v;
+}
+
+}  // namespace gs
+
 extern "C" {
 
 int gs_csc2coo(const int64_t* indptr, int64_t num_cols, int64_t nnz,
@@ -58,6 +118,28 @@ int gs_sorted_to_indptr(const int64_t* sorted_ids, int64_t nnz, int64_t num_cols
             sorted_to_indptr_kernel<<<dim3((unsigned)ceil_div(num_cols + 1, kBlock)),
                                       dim3(kBlock), 0, s>>>(sorted_ids, nnz,
                                                             num_cols, out_indptr));
+  return GS_OK;
+}
+
+int gs_first_position(const int64_t* ids, int64_t n, int64_t num_ids,
+                      int64_t* out_first, gs_stream_t stream) {
+  using namespace gs;
+  GS_REQUIRE(n >= 0 && num_ids >= 0, "first_position: negative size");
+  if (num_ids == 0) return GS_OK;
+  GS_REQUIRE(out_first && (n == 0 || ids), "first_position: null pointer");
+  hipStream_t s = as_stream(stream);
+  GS_LAUNCH("first_position_init", s,
+            fill_i64_kernel<<<dim3((unsigned)ceil_div(num_ids, kBlock)), dim3(kBlock), 0,
+                              s>>>(out_first, num_ids, INT64_MAX));
+  if (n > 0 && num_ids <= kFirstLdsIds)
+    GS_LAUNCH("first_position", s,
+              first_position_lds_kernel<<<dim3((unsigned)ceil_div(n, kFirstTile)),
+                                          dim3(kBlock), 0, s>>>(ids, n, num_ids,
+                                                                (long long*)out_first));
+  else if (n > 0)
+    GS_LAUNCH("first_position", s,
+              first_position_kernel<<<dim3((unsigned)ceil_div(n, kBlock)), dim3(kBlock), 0,
+                                      s>>>(ids, n, num_ids, (long long*)out_first));
   return GS_OK;
 }
 

@@ -3,6 +3,8 @@
 // workspaces through torch, and calls the C ABI on the current HIP stream.
 #include "graph.h"
 
+#include <limits>
+
 #include "abi_call.h"
 
 namespace gs {
@@ -350,6 +352,58 @@ torch::Tensor Graph::mapped_rows(const torch::Tensor& base,
   return mapped_out_;
 }
 
+// Worth it when the edges outnumber the listed ids by far (a layer-wise
+// sampler keeps a few hundred rows and millions of edges between them).
+bool Graph::use_list_labels(const torch::Tensor& col_seeds,
+                            const torch::Tensor& row_ids) const {
+  const int64_t R = row_ids.numel(), S = col_seeds.numel();
+  return R > 0 && coo_ && coo_->row.numel() >= 8 * (R + S);
+}
+
+// The frontier is the unique of seeds ++ row_ids[coo.row] in first-occurrence
+// order.  Every edge of local row l carries the same key row_ids[l], so the
+// listed ids, ordered by the first edge that uses them, give the same frontier
+// as the edges themselves; ids that no edge uses are replaced by a key that is
+// already there.  One pass over the edges (first position per local row)
+// replaces hashing every edge.
+Graph::ListLabels& Graph::list_labels_for(const torch::Tensor& col_seeds,
+                                          const torch::Tensor& row_ids) {
+  const torch::Tensor& base = coo_->row;
+  if (list_labels_ && list_labels_->base.is_same(base) &&
+      list_labels_->row_ids.is_same(row_ids) && list_labels_->seeds.is_same(col_seeds) &&
+      list_labels_->row_ids_version == (int64_t)row_ids._version() &&
+      list_labels_->seeds_version == (int64_t)col_seeds._version())
+    return *list_labels_;
+  auto out = std::make_unique<ListLabels>();
+  out->base = base;
+  out->row_ids = row_ids;
+  out->seeds = col_seeds;
+  out->row_ids_version = row_ids._version();
+  out->seeds_version = col_seeds._version();
+  torch::Tensor table = ids(row_ids, "row_ids");
+  const int64_t R = table.numel(), S = col_seeds.numel(), E = base.numel();
+  torch::Tensor first = new_ids(R, base);
+  GS_CALL(gs_first_position(cptr(base), E, R, mptr(first), cur_stream()));
+  auto sorted = torch::sort(first);  // R values: which listed id is met first
+  const torch::Tensor& when = std::get<0>(sorted);
+  const torch::Tensor& order = std::get<1>(sorted);
+  torch::Tensor keys = table.index_select(0, order);
+  // E > 0, so the earliest listed id is used by some edge
+  keys = torch::where(when != std::numeric_limits<int64_t>::max(), keys, keys.select(0, 0));
+  torch::Tensor rows = torch::cat({keys, col_seeds});  // the seeds again: their labels
+  Frontier& f = frontier_for(col_seeds, rows, {}, {});
+  torch::Tensor labels = new_ids(R + S, base);
+  GS_CALL(gs_unique_relabel(cptr(col_seeds), nullptr, S, cptr(rows), nullptr, R + S, 1,
+                            nullptr, mptr(labels), nullptr, f.workspace.data_ptr(),
+                            f.workspace.numel(), cur_stream()));
+  out->label_by_local = new_ids(R, base);
+  out->label_by_local.index_copy_(0, order, labels.narrow(0, 0, R));
+  out->seed_label = labels.narrow(0, R, S);
+  out->frontier = f.frontier();
+  list_labels_ = std::move(out);
+  return *list_labels_;
+}
+
 std::tuple<torch::Tensor, torch::Tensor, torch::Tensor,
            c10::optional<torch::Tensor>>
 Graph::GraphRelabel(torch::Tensor col_seeds, torch::Tensor row_ids) {
@@ -357,6 +411,11 @@ Graph::GraphRelabel(torch::Tensor col_seeds, torch::Tensor row_ids) {
   col_seeds = ids(col_seeds, "col_seeds");
   TORCH_CHECK(col_seeds.numel() > 0 || coo_->col.numel() == 0,
               "GraphRelabel: the matrix has edges but col_seeds is empty");
+  if (use_list_labels(col_seeds, row_ids)) {
+    ListLabels& l = list_labels_for(col_seeds, row_ids);
+    return {l.frontier, l.label_by_local.index_select(0, coo_->row),
+            l.seed_label.index_select(0, coo_->col), coo_->e_ids};
+  }
   torch::Tensor rows = mapped_rows(coo_->row, row_ids);
   Frontier& f = frontier_for(col_seeds, rows, {}, {});
   const int64_t E = rows.numel();
@@ -378,6 +437,7 @@ torch::Tensor Graph::GetValidNodes(torch::Tensor col_seeds,
   // here when a CSC exists, src/graph.cc:593-608, which is another edge order
   // whenever that CSC was built by sorting a row-sorted COO.)
   CreateSparseFormat(kCOO);
+  if (use_list_labels(col_seeds, row_ids)) return list_labels_for(col_seeds, row_ids).frontier;
   const torch::Tensor& base = coo_->row;
   torch::Tensor rows = mapped_rows(base, row_ids);
   return frontier_for(col_seeds, rows, {}, {}).frontier();

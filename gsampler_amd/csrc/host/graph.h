@@ -227,6 +227,17 @@ class Graph : public torch::CustomClassHolder {
   int64_t row_encoding_size_ = 0;
   std::unique_ptr<Frontier> frontier_;
   torch::Tensor mapped_out_, mapped_from_, mapped_by_;
+  // Relabel of a matrix whose rows are positions in a short list of ids
+  // (row slicing leaves it that way): label of every list entry and of every
+  // seed, computed from the list instead of from every edge.
+  struct ListLabels {
+    torch::Tensor base, row_ids, seeds;
+    int64_t row_ids_version = -1, seeds_version = -1;
+    torch::Tensor frontier, label_by_local, seed_label;
+  };
+  std::unique_ptr<ListLabels> list_labels_;
+  bool use_list_labels(const torch::Tensor& col_seeds, const torch::Tensor& row_ids) const;
+  ListLabels& list_labels_for(const torch::Tensor& col_seeds, const torch::Tensor& row_ids);
 };
 
 // Operators along the compressed axis (graph.cc) and across it (slicing.cc).

@@ -274,6 +274,17 @@ int gs_unique_relabel(const int64_t* seeds, const int64_t* seeds_ptr,
                       size_t workspace_bytes, gs_stream_t stream);
 
 /* ------------------------------------------------------------------------
+ * out_first[r] = smallest position e with ids[e] == r, INT64_MAX when r does
+ * not occur, for ids of a small dense range [0, num_ids) (ids outside it are
+ * ignored).  The relabel step of a row-sliced matrix uses it: its rows are
+ * positions in the list of picked rows, so first occurrences can be found per
+ * picked row instead of per edge (no counterpart in the reference, which
+ * hashes every edge, src/cuda/unique_reindex.cu:81-151).
+ * ---------------------------------------------------------------------- */
+int gs_first_position(const int64_t* ids, int64_t n, int64_t num_ids,
+                      int64_t* out_first, gs_stream_t stream);
+
+/* ------------------------------------------------------------------------
  * Slicing across the compressed axis (row slicing of a CSC, A[picked, :]) and
  * coordinate-form slicing: keep the edges whose id in `ids[nnz]` belongs to
  * `picked[num_picked]`, relabel that id to its position in `picked` (smallest

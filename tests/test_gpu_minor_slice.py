@@ -85,3 +85,38 @@ def test_matrix_row_and_column_slicing_with_edata():
     mask = np.isin(indices, rows)
     assert np.array_equal(sel.cpu().numpy(), np.nonzero(mask)[0])
     assert np.array_equal(subc._CAPI_GetCOOCols().cpu().numpy(), col[mask])
+
+
+@pytest.mark.parametrize("num_rows_picked,max_deg", [(6, 400), (40, 12)])
+def test_relabel_of_a_row_sliced_matrix(num_rows_picked, max_deg):
+    """After row slicing the rows of a matrix are positions in the list of picked
+    rows.  With few picked rows and many edges the relabel works on that list
+    (first edge per picked row) instead of hashing every edge; with more picked
+    rows it hashes the edges.  Both must give the unique of
+    seeds ++ picked[coo.row] in first-occurrence order, and the same labels."""
+    rng = np.random.default_rng(num_rows_picked)
+    indptr, indices = random_csc(rng, 60, 50, max_deg, empty_frac=0.0)
+    indices[indices == 49] = 48   # row 49 has no edge
+    m = gs.Matrix()
+    m.load_graph("CSC", [T(indptr), T(indices)])
+    cols = rng.permutation(60)[:12]
+    picked = rng.permutation(50)[:num_rows_picked]
+    if num_rows_picked == 6:
+        picked[2] = 49            # a picked row without any edge
+    sub = m[T(picked), T(cols)]
+    row, col, _ = sub.coo
+    assert (row.numel() >= 8 * (num_rows_picked + 12)) == (num_rows_picked == 6)
+    seeds = T(cols)
+    uniq, out_row, out_col, _ = sub._graph._CAPI_GraphRelabel(seeds, T(picked))
+    keys = picked[row.cpu().numpy()]
+    want = orc.unique_relabel(cols, keys, edge_col=col.cpu().numpy())
+    assert np.array_equal(uniq.cpu().numpy(), want[0])
+    assert np.array_equal(out_row.cpu().numpy(), want[2])
+    assert np.array_equal(out_col.cpu().numpy(), want[3])
+    assert np.array_equal(sub.all_nodes().cpu().numpy(), want[0])
+    # first_position itself
+    first = capi.first_position(row, num_rows_picked).cpu().numpy()
+    r = row.cpu().numpy()
+    for l in range(num_rows_picked):
+        hits = np.nonzero(r == l)[0]
+        assert first[l] == (hits[0] if hits.size else np.iinfo(np.int64).max)

@@ -224,3 +224,19 @@ def test_unique_rejects_ids_that_do_not_fit():
     # the largest admissible id still works afterwards
     assert_same(capi.unique_relabel(T(seeds), T(np.array([2**32 - 2, 5]))),
                 orc.unique_relabel(seeds, np.array([2**32 - 2, 5])))
+
+
+@pytest.mark.parametrize("num_ids", [1, 300, 4096, 5000])
+def test_first_position(num_ids):
+    rng = np.random.default_rng(num_ids)
+    ids = rng.integers(0, num_ids + 3, size=200000)          # a few ids outside the range
+    ids[rng.random(ids.size) < 0.3] = 0                      # one hot id
+    if num_ids > 10:
+        ids[ids == 7] = 8                                    # an id that never occurs
+    got = capi.first_position(T(ids), num_ids).cpu().numpy()
+    want = np.full(num_ids, np.iinfo(np.int64).max)
+    inside = ids < num_ids
+    np.minimum.at(want, ids[inside], np.nonzero(inside)[0])
+    assert np.array_equal(got, want)
+    empty = capi.first_position(T(np.empty(0, dtype=np.int64)), 4).cpu().tolist()
+    assert empty == [np.iinfo(np.int64).max] * 4
