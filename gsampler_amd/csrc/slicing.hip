@@ -28,26 +28,51 @@ __global__ __launch_bounds__(kBlock) void col_count_kernel(
 }
 
 // Edge-parallel slice: thread e owns output edge e, finds its column by binary
-// search in sub_indptr (L2-resident) and copies one row id.  Load balance is
+// search in sub_indptr (L2-resident; skipped when its whole tile lies in one
+// column) and copies one row id.  Load balance is
 // independent of the degree distribution; reads within a column and all
 // writes are coalesced.
+constexpr int kSliceItems = 4;
+constexpr int kSliceTile = kBlock * kSliceItems;
+
 __global__ __launch_bounds__(kBlock) void col_slice_fill_kernel(
     const int64_t* __restrict__ indptr, const int64_t* __restrict__ indices, const int64_t* __restrict__ column_ids,
     int64_t num_items, const int64_t* __restrict__ sub_indptr, int64_t nnz,
     const int64_t* __restrict__ batch_ptr, int64_t num_batches,
     int64_t encode_stride, int64_t* __restrict__ out_coo_col,
     int64_t* __restrict__ out_indices, int64_t* __restrict__ out_select) {
-  const int64_t e = (int64_t)blockIdx.x * kBlock + threadIdx.x;
-  if (e >= nnz) return;
-  const int64_t item = segment_of(sub_indptr, num_items, e);
-  const int64_t c = column_ids ? column_ids[item] : item;
-  const int64_t in_pos = indptr[c] + (e - sub_indptr[item]);
-  int64_t row = indices[in_pos];
-  if (batch_ptr != nullptr && encode_stride > 0)
-    row += segment_of(batch_ptr, num_batches, item) * encode_stride;
-  out_indices[e] = row;
-  out_select[e] = in_pos;
-  if (out_coo_col) out_coo_col[e] = item;
+  const int64_t e0 = (int64_t)blockIdx.x * kSliceTile;
+  if (e0 >= nnz) return;
+  const int64_t e_last = e0 + kSliceTile - 1 < nnz ? e0 + kSliceTile - 1 : nnz - 1;
+  // columns that the tile touches: one search per work-group (on the scalar
+  // unit) instead of one per edge; a long column covers whole tiles
+  const int64_t item_lo = segment_of(sub_indptr, num_items, wave_uniform_first(e0));
+  const int64_t item_hi = segment_of(sub_indptr, num_items, wave_uniform_first(e_last));
+  int64_t item[kSliceItems], in_pos[kSliceItems], row[kSliceItems];
+#pragma unroll
+  for (int j = 0; j < kSliceItems; ++j) {
+    const int64_t e = e0 + j * kBlock + threadIdx.x;
+    item[j] = -1;
+    if (e >= nnz) continue;
+    item[j] = item_lo == item_hi
+                  ? item_lo
+                  : item_lo + segment_of(sub_indptr + item_lo, item_hi - item_lo + 1, e);
+    const int64_t c = column_ids ? column_ids[item[j]] : item[j];
+    in_pos[j] = indptr[c] + (e - sub_indptr[item[j]]);
+  }
+#pragma unroll
+  for (int j = 0; j < kSliceItems; ++j)
+    if (item[j] >= 0) row[j] = indices[in_pos[j]];
+#pragma unroll
+  for (int j = 0; j < kSliceItems; ++j) {
+    if (item[j] < 0) continue;
+    const int64_t e = e0 + j * kBlock + threadIdx.x;
+    if (batch_ptr != nullptr && encode_stride > 0)
+      row[j] += segment_of(batch_ptr, num_batches, item[j]) * encode_stride;
+    out_indices[e] = row[j];
+    out_select[e] = in_pos[j];
+    if (out_coo_col) out_coo_col[e] = item[j];
+  }
 }
 
 }  // namespace gs
@@ -93,7 +118,7 @@ int gs_csc_col_slice_fill(const int64_t* indptr, int64_t num_cols,
   (void)num_cols;  // ids were validated by the count phase
   hipStream_t s = as_stream(stream);
   GS_LAUNCH("col_slice_fill", s,
-            col_slice_fill_kernel<<<dim3((unsigned)ceil_div(nnz, kBlock)),
+            col_slice_fill_kernel<<<dim3((unsigned)ceil_div(nnz, kSliceTile)),
                                     dim3(kBlock), 0, s>>>(
                 indptr, indices, column_ids, num_items, sub_indptr, nnz,
                 batch_ptr, num_batches, encode_stride, out_coo_col, out_indices,
