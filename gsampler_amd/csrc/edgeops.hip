@@ -10,6 +10,7 @@
 // in every sampler that uses them, so the fast paths are the feature-length-1
 // ones and the general-length paths favour simplicity.
 #include "common.h"
+#include "scan.h"
 
 namespace gs {
 
@@ -424,6 +425,231 @@ __global__ __launch_bounds__(kBlock) void spmm_coo_sum_kernel(
     if (keys[j] != -1) unsafeAtomicAdd(out + keys[j], vals[j]);
 }
 
+// ------------------------------------------- coordinate sums by row ranges
+// Atomic adds to device memory are executed next to the memory, at a rate far
+// below what the edges stream at, and a tile of a large slice rarely adds
+// twice to the same row.  Large coordinate-form sums therefore go through a
+// counting sort by row range instead: (1) every tile of edges counts its edges
+// per range of kRangeRows rows, (2) a scan over the (range, tile) counts gives
+// every tile a private place in every range, (3) the tile writes
+// (row within range, value) pairs there, (4) a work-group sums a slice of one
+// range in LDS and stores its kRangeRows partial sums, (5) the partial sums of
+// a range are folded into the output.  Every pass streams; none uses an atomic
+// on device memory.  The floor of pass 4 is the rate of fp32 adds in LDS
+// (about a quarter of the integer rate), not memory.
+constexpr int kRangeShift = 13;
+constexpr int kRangeRows = 1 << kRangeShift;  // 32 KB of LDS accumulators
+constexpr int kMaxRanges = 1024;
+constexpr int kPartThreads = 512;
+constexpr int kPartItems = 8;
+constexpr int kPartTile = kPartThreads * kPartItems;
+constexpr int kSliceEntries = 32768;  // (row, value) pairs one work-group sums
+constexpr int kSliceItems = 8;
+
+struct RowRangePlan {
+  int64_t ranges = 0, tiles = 0, max_units = 0;
+  size_t off_offsets = 0, off_scan = 0, scan_bytes = 0, off_entries = 0,
+         off_unit_start = 0, off_partial = 0, total = 0;
+};
+
+static bool row_range_enabled() {
+  static const bool on = [] {
+    const char* v = getenv("GS_SPMM_PARTITION");
+    return v == nullptr || atoi(v) != 0;
+  }();
+  return on;
+}
+
+// Worth it when the slice is large and rows repeat; empty plan otherwise.
+static RowRangePlan row_range_plan(int format, int64_t nnz, int64_t num_out) {
+  RowRangePlan p;
+  if (!row_range_enabled() || format != GS_FMT_COO || nnz < kPrivateMinEdges ||
+      nnz >= ((int64_t)1 << 31) || num_out <= 0 || num_out > nnz / 4 ||
+      ceil_div(num_out, kRangeRows) > kMaxRanges)
+    return p;
+  p.ranges = ceil_div(num_out, kRangeRows);
+  p.tiles = ceil_div(nnz, kPartTile);
+  p.max_units = nnz / kSliceEntries + p.ranges;
+  auto take = [&p](size_t bytes) {
+    const size_t at = p.total;
+    p.total += (bytes + 255) / 256 * 256;
+    return at;
+  };
+  const int64_t cells = p.ranges * p.tiles + 1;
+  p.off_offsets = take((size_t)cells * sizeof(int64_t));
+  p.scan_bytes = scan_workspace_bytes(cells);
+  p.off_scan = take(p.scan_bytes);
+  p.off_entries = take((size_t)nnz * sizeof(uint2));
+  p.off_unit_start = take((size_t)(p.ranges + 1) * sizeof(int64_t));
+  p.off_partial = take((size_t)p.max_units * kRangeRows * sizeof(float));
+  return p;
+}
+
+// counts[range * tiles + tile] = edges of the tile whose target lies in range
+__global__ __launch_bounds__(kPartThreads) void rowsum_hist_kernel(
+    const int64_t* __restrict__ dst_ids, int64_t nnz, int64_t num_out, int ranges,
+    int64_t tiles, int64_t* __restrict__ counts) {
+  __shared__ int hist[kMaxRanges];
+  for (int j = threadIdx.x; j < ranges; j += kPartThreads) hist[j] = 0;
+  __syncthreads();
+  const int64_t tile0 = (int64_t)blockIdx.x * kPartTile;
+  int64_t dst[kPartItems];
+#pragma unroll
+  for (int i = 0; i < kPartItems; ++i) {
+    const int64_t e = tile0 + i * kPartThreads + threadIdx.x;
+    dst[i] = e < nnz ? dst_ids[e] : -1;
+  }
+#pragma unroll
+  for (int i = 0; i < kPartItems; ++i)
+    if (dst[i] >= 0 && dst[i] < num_out) atomicAdd(&hist[dst[i] >> kRangeShift], 1);
+  __syncthreads();
+  for (int j = threadIdx.x; j < ranges; j += kPartThreads)
+    counts[(int64_t)j * tiles + blockIdx.x] = hist[j];
+  if (blockIdx.x == 0 && threadIdx.x == 0) counts[(int64_t)ranges * tiles] = 0;
+}
+
+// A tile is kept small (4096 edges) so that several work-groups share a
+// compute unit and the loads of one overlap the stores of another; what a tile
+// sends to one range is a contiguous run, filled within a few microseconds, so
+// the 8-byte stores merge into whole lines in L2.  A pair keeps its range above
+// the row bits (the accumulate pass masks it off).
+__global__ __launch_bounds__(kPartThreads) void rowsum_scatter_kernel(
+    const int64_t* __restrict__ dst_ids, const int64_t* __restrict__ src_ids,
+    const int64_t* __restrict__ edge_map, int64_t nnz, int64_t num_out, int kind,
+    int op, const float* __restrict__ ufeat, const float* __restrict__ efeat,
+    int ranges, int64_t tiles, const int64_t* __restrict__ offsets,
+    uint2* __restrict__ entries) {
+  __shared__ unsigned cursor[kMaxRanges];  // next free place of the tile per range
+  for (int j = threadIdx.x; j < ranges; j += kPartThreads)
+    cursor[j] = (unsigned)offsets[(int64_t)j * tiles + blockIdx.x];
+  __syncthreads();
+  const int64_t tile0 = (int64_t)blockIdx.x * kPartTile;
+  int64_t dst[kPartItems];
+  float val[kPartItems];
+#pragma unroll
+  for (int i = 0; i < kPartItems; ++i) {
+    const int64_t e = tile0 + i * kPartThreads + threadIdx.x;
+    dst[i] = -1;
+    val[i] = 0.f;
+    if (e < nnz) {
+      dst[i] = dst_ids[e];
+      const int64_t eid = edge_map ? edge_map[e] : e;
+      val[i] = edge_value<float>(kind, op, ufeat ? ufeat + src_ids[e] : nullptr,
+                                 efeat ? efeat + eid : nullptr);
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < kPartItems; ++i) {
+    if (dst[i] < 0 || dst[i] >= num_out) continue;
+    const unsigned pos = atomicAdd(&cursor[dst[i] >> kRangeShift], 1u);
+    entries[pos] = make_uint2((unsigned)dst[i], __float_as_uint(val[i]));
+  }
+}
+
+// unit_start[r] = first work unit (slice of kSliceEntries pairs) of range r
+__global__ __launch_bounds__(kMaxRanges) void rowsum_units_kernel(
+    const int64_t* __restrict__ offsets, int ranges, int64_t tiles,
+    int64_t* __restrict__ unit_start) {
+  __shared__ int64_t smem[kMaxRanges / kWave + 1];
+  const int r = threadIdx.x;
+  int64_t units = 0;
+  if (r < ranges) {
+    const int64_t n = offsets[(int64_t)(r + 1) * tiles] - offsets[(int64_t)r * tiles];
+    units = ceil_div_dev(n, (int64_t)kSliceEntries);
+  }
+  int64_t total;
+  const int64_t before = block_exclusive_sum<int64_t, kMaxRanges>(units, smem, &total);
+  if (r < ranges) unit_start[r] = before;
+  if (r == 0) unit_start[ranges] = total;
+}
+
+__global__ __launch_bounds__(kPartThreads) void rowsum_accumulate_kernel(
+    const uint2* __restrict__ entries, const int64_t* __restrict__ offsets,
+    const int64_t* __restrict__ unit_start, int ranges, int64_t tiles,
+    float* __restrict__ partial) {
+  __shared__ float acc[kRangeRows];
+  const int64_t u = blockIdx.x;
+  if (u >= unit_start[ranges]) return;
+  const int64_t r = segment_of(unit_start, ranges, u);
+  const int64_t range_end = offsets[(r + 1) * tiles];
+  const int64_t begin = offsets[r * tiles] + (u - unit_start[r]) * kSliceEntries;
+  const int64_t end = begin + kSliceEntries < range_end ? begin + kSliceEntries : range_end;
+  for (int j = threadIdx.x; j < kRangeRows; j += kPartThreads) acc[j] = 0.f;
+  __syncthreads();
+  for (int64_t base = begin; base < end; base += kPartThreads * kSliceItems) {
+    uint2 item[kSliceItems];
+#pragma unroll
+    for (int i = 0; i < kSliceItems; ++i) {
+      const int64_t p = base + i * kPartThreads + threadIdx.x;
+      item[i] = p < end ? entries[p] : make_uint2(~0u, 0u);
+    }
+#pragma unroll
+    for (int i = 0; i < kSliceItems; ++i)
+      if (item[i].x != ~0u)
+        atomicAdd(&acc[item[i].x & (kRangeRows - 1)], __uint_as_float(item[i].y));
+  }
+  __syncthreads();
+  float* mine = partial + u * kRangeRows;
+  for (int j = threadIdx.x; j < kRangeRows; j += kPartThreads) mine[j] = acc[j];
+}
+
+__global__ __launch_bounds__(kBlock) void rowsum_fold_kernel(
+    const float* __restrict__ partial, const int64_t* __restrict__ unit_start,
+    int64_t num_out, float* __restrict__ out) {
+  const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (i >= num_out) return;
+  const int64_t r = i >> kRangeShift;  // uniform over the work-group
+  const int64_t u0 = unit_start[r], u1 = unit_start[r + 1];
+  const float* p = partial + (i & (kRangeRows - 1));
+  float acc = 0.f;
+  int64_t u = u0;
+  for (; u + 8 <= u1; u += 8) {  // eight loads in flight
+    float v[8];
+#pragma unroll
+    for (int k = 0; k < 8; ++k) v[k] = p[(u + k) * kRangeRows];
+#pragma unroll
+    for (int k = 0; k < 8; ++k) acc += v[k];
+  }
+  for (; u < u1; ++u) acc += p[u * kRangeRows];
+  if (acc != 0.f) out[i] += acc;
+}
+
+static int row_range_sum(const RowRangePlan& p, const int64_t* dst_ids,
+                         const int64_t* src_ids, const int64_t* edge_map,
+                         int64_t nnz, int64_t num_out, int kind, int op,
+                         const float* ufeat, const float* efeat, float* out,
+                         void* workspace, hipStream_t s) {
+  char* ws = (char*)workspace;
+  int64_t* offsets = (int64_t*)(ws + p.off_offsets);
+  uint2* entries = (uint2*)(ws + p.off_entries);
+  int64_t* unit_start = (int64_t*)(ws + p.off_unit_start);
+  float* partial = (float*)(ws + p.off_partial);
+  const int ranges = (int)p.ranges;
+  const dim3 tiles_grid((unsigned)p.tiles);
+  GS_LAUNCH("rowsum_hist", s,
+            rowsum_hist_kernel<<<tiles_grid, dim3(kPartThreads), 0, s>>>(
+                dst_ids, nnz, num_out, ranges, p.tiles, offsets));
+  int rc = exclusive_scan_i64(offsets, offsets, p.ranges * p.tiles + 1,
+                              ws + p.off_scan, p.scan_bytes, s);
+  if (rc != GS_OK) return rc;
+  GS_LAUNCH("rowsum_scatter", s,
+            rowsum_scatter_kernel<<<tiles_grid, dim3(kPartThreads), 0, s>>>(
+                dst_ids, src_ids, edge_map, nnz, num_out, kind, op, ufeat, efeat,
+                ranges, p.tiles, offsets, entries));
+  GS_LAUNCH("rowsum_units", s,
+            rowsum_units_kernel<<<dim3(1), dim3(kMaxRanges), 0, s>>>(
+                offsets, ranges, p.tiles, unit_start));
+  GS_LAUNCH("rowsum_accumulate", s,
+            rowsum_accumulate_kernel<<<dim3((unsigned)p.max_units),
+                                       dim3(kPartThreads), 0, s>>>(
+                entries, offsets, unit_start, ranges, p.tiles, partial));
+  GS_LAUNCH("rowsum_fold", s,
+            rowsum_fold_kernel<<<dim3((unsigned)ceil_div(num_out, kBlock)),
+                                 dim3(kBlock), 0, s>>>(partial, unit_start,
+                                                       num_out, out));
+  return GS_OK;
+}
+
 static int check_view(int format, const int64_t* a, const int64_t* b,
                       int64_t num_major, int64_t nnz, const char* who) {
   GS_REQUIRE(format == GS_FMT_COO || format == GS_FMT_COMPRESSED,
@@ -447,6 +673,11 @@ static int spmm_launch(int format, const int64_t* a, const int64_t* b,
   if (scalar && reduce == kReduceSum) {
     const dim3 grid((unsigned)ceil_div(nnz, kSumTile));
     if (format == GS_FMT_COO) {
+      const RowRangePlan plan = row_range_plan(format, nnz, num_out);
+      if (plan.total > 0 && workspace != nullptr && workspace_bytes >= plan.total)
+        return row_range_sum(plan, u_target == 0 ? b : a, u_target == 0 ? a : b,
+                             edge_map, nnz, num_out, kind, op, ufeat, efeat, out,
+                             workspace, s);
       const size_t need = private_bytes(format, nnz, num_out);
       if (need > 0 && workspace != nullptr && workspace_bytes >= need) {
         float* copies = (float*)workspace;
@@ -591,6 +822,8 @@ int gs_fused_u_op_v(int format, const int64_t* a, const int64_t* b,
 }
 
 size_t gs_spmm_workspace_bytes(int format, int64_t nnz, int64_t num_out) {
+  const gs::RowRangePlan plan = gs::row_range_plan(format, nnz, num_out);
+  if (plan.total > 0) return plan.total;
   return gs::private_bytes(format, nnz, num_out);
 }
 

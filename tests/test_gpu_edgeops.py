@@ -93,7 +93,7 @@ def test_spmm_and_fusions_parity(g, fmt):
     close(o1, w1); close(o2, w2)
 
 
-@pytest.mark.parametrize("shape", ["hubs", "tiny_segments"])
+@pytest.mark.parametrize("shape", ["hubs", "row_ranges", "tiny_segments"])
 def test_scalar_sums_on_skewed_matrices(shape):
     """The load-balanced sum kernels: a few segments that hold most of the edges
     (and rows that most edges point to), and thousands of segments with zero or
@@ -106,6 +106,14 @@ def test_scalar_sums_on_skewed_matrices(shape):
         R = 3000
         w = 1.0 / np.arange(1, R + 1) ** 1.2
         indices = rng.choice(R, size=int(deg.sum()), p=w / w.sum())
+    elif shape == "row_ranges":
+        # several ranges of 8192 rows: one holds a hub row (many slices of one
+        # range), one is empty, the last one is partial
+        deg = np.full(300, 5000)
+        R = 30000
+        indices = rng.integers(0, R, size=int(deg.sum()))
+        indices[(indices >= 8192) & (indices < 16384)] += 8192
+        indices[rng.random(indices.size) < 0.4] = 20001
     else:
         deg = rng.integers(0, 2, size=9000)
         R = 500
