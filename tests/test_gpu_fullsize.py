@@ -1,0 +1,151 @@
+"""The headline workload at its full size (2.45 M nodes, 124 M edges, 64 x 1024
+seeds, fan-outs 15/10/5) through the C ABI: size-independent properties checked
+on the device for every layer, and the whole step compared bit for bit with the
+CPU restatement (which finishes a step of this size in well under a second).
+The weighted variant (persistent weight CDF) and node2vec on the same graph are
+covered the same way."""
+import numpy as np
+import pytest
+import torch
+
+from gsampler_amd import capi
+from oracle import binding as orc
+
+pytestmark = pytest.mark.gpu
+
+NODES, EDGES = 2_450_000, 124_000_000
+FANOUTS = [15, 10, 5]
+
+
+@pytest.fixture(scope="module")
+def graph():
+    from gsampler_amd.utils import batched_seeds, chung_lu_csc
+    dev = torch.device("cuda:0")
+    indptr, indices = chung_lu_csc(NODES, EDGES, seed=1, device=dev)
+    seeds, ptr = batched_seeds(NODES, 64, 1024, seed=2, device=dev)
+    return indptr, indices, seeds, ptr
+
+
+def batch_of(ptr, n):
+    """Batch index of every position 0..n-1 for an offsets array."""
+    return torch.searchsorted(ptr, torch.arange(n, device=ptr.device), right=True) - 1
+
+
+def check_sampled_layer(indptr, indices, seeds, fanout, out):
+    sub_indptr, coo_col, rows, sel = out
+    deg = indptr[seeds + 1] - indptr[seeds]
+    assert torch.equal(sub_indptr[1:] - sub_indptr[:-1], deg.clamp(max=fanout))
+    assert int(sub_indptr[0]) == 0 and int(sub_indptr[-1]) == rows.numel()
+    assert bool((coo_col[1:] >= coo_col[:-1]).all())               # column-sorted
+    col = seeds[coo_col]
+    assert bool(((sel >= indptr[col]) & (sel < indptr[col + 1])).all())   # an edge of that column
+    assert torch.equal(rows, indices[sel])
+    # no edge twice within one requested column
+    pair = coo_col * EDGES + sel
+    assert torch.unique(pair).numel() == pair.numel()
+
+
+def check_relabelled_layer(seeds, ptr, rows, edge_ptr, coo_col, out):
+    uniq, uniq_ptr, out_row, out_col = out
+    B = ptr.numel() - 1
+    assert int(uniq_ptr[0]) == 0 and int(uniq_ptr[-1]) == uniq.numel()
+    assert bool((uniq_ptr[1:] >= uniq_ptr[:-1]).all())
+    ub = batch_of(uniq_ptr, uniq.numel())
+    # a batch's frontier holds every id once ...
+    assert torch.unique(ub * NODES + uniq).numel() == uniq.numel()
+    # ... starts with its seeds (the seeds of this workload are distinct per batch) ...
+    sb = batch_of(ptr, seeds.numel())
+    local = torch.arange(seeds.numel(), device=seeds.device) - ptr[sb]
+    assert torch.equal(uniq[uniq_ptr[sb] + local], seeds)
+    # ... and is exactly the set of ids of seeds ++ rows
+    eb = batch_of(edge_ptr, rows.numel())
+    keys = torch.cat([sb * NODES + seeds, eb * NODES + rows])
+    assert torch.unique(keys).numel() == uniq.numel()
+    # relabelling round-trips
+    assert torch.equal(uniq[uniq_ptr[eb] + out_row], rows)
+    assert torch.equal(uniq[uniq_ptr[eb] + out_col], seeds[coo_col])
+    assert B == 64
+
+
+def same(gpu, cpu):
+    for g, c in zip(gpu, cpu):
+        assert np.array_equal(g.cpu().numpy(), c)
+
+
+def test_graphsage_step_properties_and_oracle(graph):
+    indptr, indices, seeds, ptr = graph
+    h_indptr, h_indices = indptr.cpu().numpy(), indices.cpu().numpy()
+    h_seeds, h_ptr = seeds.cpu().numpy(), ptr.cpu().numpy()
+    total = 0
+    for layer, fanout in enumerate(FANOUTS):
+        out = capi.sample_uniform(indptr, indices, seeds, fanout, False, 0, 7777, layer)
+        check_sampled_layer(indptr, indices, seeds, fanout, out)
+        want = orc.sample_uniform(h_indptr, h_indices, h_seeds, fanout, False, 0, 7777, layer)
+        same(out, want)
+        sub_indptr, coo_col, rows, _ = out
+        edge_ptr = sub_indptr[ptr]
+        rel = capi.unique_relabel(seeds, rows, ptr, edge_ptr, coo_col)
+        check_relabelled_layer(seeds, ptr, rows, edge_ptr, coo_col, rel)
+        want_rel = orc.unique_relabel(h_seeds, want[2], h_ptr, want[0][h_ptr], want[1])
+        same(rel, want_rel)
+        total += rows.numel()
+        seeds, ptr = rel[0], rel[1]
+        h_seeds, h_ptr = want_rel[0], want_rel[1]
+    assert total > 20_000_000          # the step really is the full-size one
+
+
+def test_weighted_step_with_persistent_cdf(graph):
+    indptr, indices, seeds, ptr = graph
+    g = torch.Generator(device=indices.device)
+    g.manual_seed(5)
+    probs = torch.randn(indices.numel(), generator=g, device=indices.device).exp_().float()
+    cdf = capi.weight_cdf(indptr, probs)
+    h_indptr, h_indices, h_probs = indptr.cpu().numpy(), indices.cpu().numpy(), probs.cpu().numpy()
+    h_cdf = orc.weight_cdf(h_indptr, h_probs)
+    assert np.array_equal(cdf.cpu().numpy(), h_cdf)
+    out = capi.sample_weighted(indptr, indices, probs, seeds, 15, False, 7777, 0, cdf=cdf)
+    check_sampled_layer(indptr, indices, seeds, 15, out)
+    want = orc.sample_weighted(h_indptr, h_indices, h_probs, seeds.cpu().numpy(), 15, False,
+                               7777, 0, cdf=h_cdf)
+    same(out, want)
+    # a second, larger layer: the frontier of the first
+    edge_ptr = out[0][ptr]
+    rel = capi.unique_relabel(seeds, out[2], ptr, edge_ptr, out[1])
+    out2 = capi.sample_weighted(indptr, indices, probs, rel[0], 10, False, 7777, 1, cdf=cdf)
+    check_sampled_layer(indptr, indices, rel[0], 10, out2)
+    want2 = orc.sample_weighted(h_indptr, h_indices, h_probs, rel[0].cpu().numpy(), 10, False,
+                                7777, 1, cdf=h_cdf)
+    same(out2, want2)
+
+
+def test_node2vec_walks(graph):
+    indptr, indices, _, _ = graph
+    indices = capi.segment_sort(indptr, indices)
+    g = torch.Generator(device=indices.device)
+    g.manual_seed(3)
+    walks, length = 200_000, 80
+    start = torch.randint(0, NODES, (walks,), generator=g, device=indices.device)
+    trace = capi.node2vec(indptr, indices, start, length, 2.0, 0.5, 7777, 0)
+    assert trace.shape == (length + 1, walks) and torch.equal(trace[0], start)
+    # every hop follows an edge of the matrix (columns hold in-neighbours); a
+    # walk that stopped stays at -1
+    for step in (1, 2, 40, 80):
+        prev, cur = trace[step - 1], trace[step]
+        alive = cur >= 0
+        assert bool((prev[alive] >= 0).all())
+        p, c = prev[alive], cur[alive]
+        lo, hi = indptr[p], indptr[p + 1]
+        # columns are sorted: lower bound of c inside [lo, hi), all walks at once
+        left, right = lo.clone(), hi.clone()
+        for _ in range(24):                       # degrees stay below 2^24
+            active = left < right
+            mid = (left + right) // 2
+            less = indices[mid.clamp(max=EDGES - 1)] < c
+            left = torch.where(active & less, mid + 1, left)
+            right = torch.where(active & ~less, mid, right)
+        assert bool(((left < hi) & (indices[left.clamp(max=EDGES - 1)] == c)).all())
+        dead = ~alive
+        assert bool((trace[step:, dead] == -1).all())
+    want = orc.node2vec(indptr.cpu().numpy(), indices.cpu().numpy(), start.cpu().numpy(),
+                        length, 2.0, 0.5, 7777, 0)
+    assert np.array_equal(trace.cpu().numpy(), want)
