@@ -48,6 +48,10 @@ WORKLOADS = {
                 desc="weighted GraphSAGE [15,10,5] (fp32 edge weights LogNormal(0,1), persistent CDF), 64 batches x "
                      "1024 seeds, on c2's graph: a 1/13-scale stand-in for the 1.6B-edge weighted "
                      "configuration"),
+    "gather": dict(kind="gather", nodes=2_450_000, edges=124_000_000, gen="chung_lu", batches=64,
+                   batch_size=1024, fanouts=[15, 10, 5], feat=128,
+                   desc="feature fetch for the input nodes of one c2 step: fp32 features "
+                        "[2.45M, 128] gathered by the layer-3 frontier of 64 mini-batches"),
     "tiny": dict(nodes=50_000, edges=1_000_000, gen="chung_lu", batches=8,
                  batch_size=256, fanouts=[15, 10, 5],
                  desc="1/50-scale twin of c2 (smoke runs)"),
@@ -232,6 +236,83 @@ def run_node2vec(args, wl, capi, dev):
     }
 
 
+def run_gather(args, wl, capi, dev):
+    """The fetch that follows sampling in a training loop: features[input_nodes]
+    for the frontier of the last layer of one c2 step.  A step = one gather."""
+    import numpy as np
+    import torch
+    from gsampler_amd.utils import batched_seeds, chung_lu_csc
+    t0 = time.time()
+    indptr, indices = chung_lu_csc(wl["nodes"], wl["edges"], seed=1, device=dev)
+    seeds, ptr = batched_seeds(wl["nodes"], wl["batches"], wl["batch_size"], seed=2, device=dev)
+    _, last = graphsage_step(capi, indptr, indices, seeds, ptr, wl["fanouts"], args.seed, 0)
+    ids = last[0].clone()
+    del indptr, indices, last
+    F = wl["feat"]
+    g = torch.Generator(device=dev)
+    g.manual_seed(11)
+    table = torch.rand((wl["nodes"], F), generator=g, device=dev)
+    torch.cuda.synchronize()
+    t_build = time.time() - t0
+    n = ids.numel()
+    step_bytes = 8 * n + 2 * n * F * 4       # ids + every row read once and written once
+
+    for _ in range(args.warmup):
+        capi.gather_rows(table, ids)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        out = capi.gather_rows(table, ids)
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    check = bool(torch.equal(out[::997], table[ids[::997]]))
+    del out
+    capi.profile_reset()
+    capi.profile_enable(True)
+    for _ in range(args.steps):
+        capi.gather_rows(table, ids)
+    torch.cuda.synchronize()
+    kernels = _kernel_table(capi, lambda name: step_bytes * args.steps if name == "gather_rows" else 0)
+    capi.profile_enable(False)
+    # torch's own indexing on the same inputs, for scale
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        ref = table[ids]
+    torch.cuda.synchronize()
+    torch_ms = (time.perf_counter() - t0) / args.steps * 1e3
+    del ref
+    cpu = None
+    if args.cpu_seconds > 0:
+        from oracle import binding as orc
+        m = min(n, 2_000_000)
+        h_table, h_ids = table.cpu().numpy(), ids[:m].cpu().numpy()
+        orc.gather_rows(h_table, h_ids[:1000])
+        t_cpu, rows, runs = 0.0, 0, 0
+        while t_cpu < args.cpu_seconds and runs < 1000:
+            t = time.perf_counter()
+            orc.gather_rows(h_table, h_ids)
+            t_cpu += time.perf_counter() - t
+            rows += m
+            runs += 1
+        cpu = dict(value=round(rows / t_cpu, 1), unit="rows/s", cores=orc.num_threads(),
+                   kind="port", sample=f"{runs} gathers of the first {m} ids in {t_cpu:.1f} s, "
+                                       f"OpenMP oracle", host_cpus=os.cpu_count())
+    value = n * args.steps / elapsed
+    return {
+        "metric": "gathered_rows_per_sec", "value": round(value, 1), "unit": "rows/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(elapsed / args.steps * 1e3, 3), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": f"{args.workload}: {wl['desc']}", "rows_per_step": n,
+                   "row_bytes": F * 4, "spot_check_against_torch_indexing": check,
+                   "torch_indexing_ms": round(torch_ms, 3)},
+        "roofline": _roofline(kernels[0]), "cpu_baseline": cpu,
+        "gpu_over_cpu": round(value / cpu["value"], 1) if cpu else None,
+        "kernels": kernels, "graph_build_s": round(t_build, 1),
+    }
+
+
 def ladies_sampler(A, seeds, fanouts):
     """The layer-wise sampler of the reference's examples/ladies/ladies.py:7-21."""
     ret = []
@@ -372,6 +453,8 @@ def main():
     wl = WORKLOADS[args.workload]
     if wl.get("kind") == "node2vec":
         return print(json.dumps(run_node2vec(args, wl, capi, dev)))
+    if wl.get("kind") == "gather":
+        return print(json.dumps(run_gather(args, wl, capi, dev)))
     if wl.get("kind") == "ladies":
         return print(json.dumps(run_ladies(args, wl, capi, dev)))
 

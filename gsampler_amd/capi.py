@@ -59,6 +59,7 @@ SIGNATURES = {
     "gs_decode_batch_ids": (_int, [_p, _i64, _i64, _p, _p, _p]),
     "gs_split_indptr": (_int, [_p, _p, _i64, _i64, _p, _p]),
     "gs_first_position": (_int, [_p, _i64, _i64, _p, _p]),
+    "gs_gather_rows": (_int, [_p, _i64, _i64, _p, _i64, _p, _p, _p]),
     "gs_sddmm": (_int, [_int, _p, _p, _i64, _i64, _p, _int, _int, _p, _p, _p, _int, _int,
                         _i64, _i64, _i64, _i64, _p, _p, _p]),
     "gs_fused_u_op_v": (_int, [_int, _p, _p, _i64, _i64, _int, _int, _p, _p, _p, _p, _p,
@@ -341,6 +342,28 @@ def first_position(ids: torch.Tensor, num_ids: int) -> torch.Tensor:
     out = torch.empty(num_ids, dtype=torch.int64, device=ids.device)
     check(lib().gs_first_position(_ptr(ids), ids.numel(), num_ids, _ptr(out), _stream()))
     return out
+
+
+def gather_rows(table: torch.Tensor, ids: torch.Tensor, count_bad: bool = False):
+    """out[i] = table[ids[i]] along the first axis, for any dtype and row shape.
+    `table` is a CUDA tensor or a pinned CPU tensor (read in place over the host
+    link); the result lives on the device of `ids`.  Ids outside the table give
+    zero rows; with `count_bad` the pair (out, number of such ids) is returned."""
+    ids = _i64t(ids, "ids")
+    if not (table.is_cuda or table.is_pinned()):
+        raise GsError("gather_rows: table must be a CUDA tensor or a pinned CPU tensor")
+    if table.dim() < 1:
+        raise GsError("gather_rows: table needs at least one axis")
+    table = table.contiguous()
+    out = torch.empty((ids.numel(),) + tuple(table.shape[1:]), dtype=table.dtype,
+                      device=ids.device)
+    rows, row_bytes = table.shape[0], table.element_size()
+    for extent in table.shape[1:]:
+        row_bytes *= extent
+    bad = torch.empty(1, dtype=torch.int64, device=ids.device) if count_bad else None
+    check(lib().gs_gather_rows(table.data_ptr() if table.numel() else None, rows, row_bytes,
+                               _ptr(ids), ids.numel(), _ptr(out), _ptr(bad), _stream()))
+    return (out, int(bad.item())) if count_bad else out
 
 
 def decode_batch_ids(encoded: torch.Tensor, stride: int):

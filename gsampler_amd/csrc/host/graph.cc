@@ -221,10 +221,34 @@ GraphPtr Graph::derive(int64_t on_format, int64_t output_format,
   return g;
 }
 
+// out[i] = table[ids[i]] along the first axis.  The table may be a pinned host
+// tensor, which the kernel reads in place (IndexSelectCPUFromGPU,
+// src/cuda/index_select_uvm.cu:22-50, and dgl's gather_pinned_tensor_rows that
+// python/gs/matrix_api/matrix.py:19-23 calls for pinned edge data).
+torch::Tensor GatherRows(torch::Tensor table, torch::Tensor ids) {
+  TORCH_CHECK(table.dim() >= 1, "GatherRows: the table needs at least one axis");
+  TORCH_CHECK(table.is_cuda() || table.is_pinned(),
+              "GatherRows: the table must be on the GPU or in pinned host memory");
+  TORCH_CHECK(ids.is_cuda() && ids.scalar_type() == torch::kInt64 && ids.dim() == 1,
+              "GatherRows: ids must be a 1-D int64 GPU tensor");
+  table = table.contiguous();
+  ids = ids.contiguous();
+  std::vector<int64_t> shape = table.sizes().vec();
+  shape[0] = ids.numel();
+  torch::Tensor out = torch::empty(shape, table.options().device(ids.device()).pinned_memory(false));
+  int64_t row_bytes = (int64_t)table.element_size();
+  for (size_t d = 1; d < shape.size(); ++d) row_bytes *= shape[d];
+  GS_CALL(gs_gather_rows(table.numel() ? table.data_ptr() : nullptr, table.size(0),
+                         row_bytes, cptr(ids), ids.numel(),
+                         out.numel() ? out.data_ptr() : nullptr, nullptr, cur_stream()));
+  return out;
+}
+
 torch::Tensor Graph::edge_index(const c10::optional<torch::Tensor>& parent_eids,
                                 const torch::Tensor& select) {
-  return parent_eids.has_value() ? parent_eids.value().index_select(0, select)
-                                 : select;
+  if (!parent_eids.has_value()) return select;
+  if (parent_eids.value().is_pinned()) return GatherRows(parent_eids.value(), select);
+  return parent_eids.value().index_select(0, select);
 }
 
 static void check_out_format(int64_t on_format, int64_t output_format,

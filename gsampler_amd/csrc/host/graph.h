@@ -250,6 +250,7 @@ MajorResult minor_slice(const Compressed& m, const torch::Tensor& picked,
                         bool with_coo);
 
 // ---- free operators (gs_ops)
+torch::Tensor GatherRows(torch::Tensor table, torch::Tensor ids);
 torch::Tensor ListSampling(int64_t num_items, int64_t num_picks, bool replace);
 torch::Tensor ListSamplingProbs(torch::Tensor probs, int64_t num_picks,
                                 bool replace);

@@ -99,6 +99,7 @@ TORCH_LIBRARY(gs_ops, m) {
   m.def("_CAPI_BatchListSampling", &gs::BatchListSampling);
   m.def("_CAPI_BatchSplitByOffset", &gs::SplitByOffset);
   m.def("_CAPI_BatchIndptrSplitByOffset", &gs::SplitIndptrByOffset);
+  m.def("_CAPI_GatherRows", &gs::GatherRows);
   m.def("_CAPI_SetRandomSeed", &gs::set_random_seed);
   m.def("_CAPI_GetRandomState", &gs::get_random_state);
   m.def("_CAPI_SetNextCallId", &gs::set_next_call_id);

@@ -12,6 +12,7 @@ from torch.fx import Proxy
 from ..format import _COO, _CSC, _CSR
 from ..ops import gsddmm, gspmm
 from ..utils.block import Block, create_block_from_coo, create_block_from_csc  # noqa: F401
+from ..utils.gather import gather_pinned_tensor_rows
 
 torch.fx.wrap("create_block_from_coo")
 torch.fx.wrap("create_block_from_csc")
@@ -21,6 +22,10 @@ torch.fx.wrap("data_index")
 
 
 def data_index(data: torch.Tensor, index: torch.Tensor) -> torch.Tensor:
+    """data[index]; pinned host data is gathered in place by the GPU
+    (python/gs/matrix_api/matrix.py:19-23 of the reference)."""
+    if data.is_pinned():
+        return gather_pinned_tensor_rows(data, index)
     return data[index]
 
 

@@ -285,6 +285,23 @@ int gs_first_position(const int64_t* ids, int64_t n, int64_t num_ids,
                       int64_t* out_first, gs_stream_t stream);
 
 /* ------------------------------------------------------------------------
+ * Row gather: out[i, :] = table[ids[i], :] for rows of `row_bytes` bytes of any
+ * element type (node features of the sampled frontier, labels, edge data
+ * behind an edge index).  `table` is device memory or pinned host memory that
+ * the device can address; `ids` and `out` are device memory.  Replaces
+ * IndexSelectCPUFromGPU (src/cuda/index_select_uvm.cu:9-50, pinned e_ids) and
+ * the dgl.utils.gather_pinned_tensor_rows / data[index] calls of the callers
+ * (python/gs/matrix_api/matrix.py:19-23,
+ * examples/graphsage/graphsage_e2e.py:113-118).  An id outside [0, num_rows)
+ * yields a row of zero bytes (the reference asserts on the device,
+ * index_select_uvm.cu:16); when `bad_count` is not NULL it receives the number
+ * of such ids.
+ * ---------------------------------------------------------------------- */
+int gs_gather_rows(const void* table, int64_t num_rows, int64_t row_bytes,
+                   const int64_t* ids, int64_t n, void* out, int64_t* bad_count,
+                   gs_stream_t stream);
+
+/* ------------------------------------------------------------------------
  * Slicing across the compressed axis (row slicing of a CSC, A[picked, :]) and
  * coordinate-form slicing: keep the edges whose id in `ids[nnz]` belongs to
  * `picked[num_picked]`, relabel that id to its position in `picked` (smallest

@@ -427,3 +427,17 @@ def segment_sort(indptr, keys):
     out = np.empty_like(keys)
     lib().gs_segment_sort_i64_cpu(_p(indptr), C.c_int64(indptr.size - 1), _p(keys), _p(out))
     return out
+
+
+def gather_rows(table, ids):
+    """out[i] = table[ids[i]] along the first axis (any dtype, any row shape);
+    returns (out, number of ids outside the table, whose rows are zero)."""
+    table = np.ascontiguousarray(table)
+    ids = _i64(ids)
+    out = np.empty((ids.size,) + table.shape[1:], dtype=table.dtype)
+    row_bytes = int(table.dtype.itemsize * np.prod(table.shape[1:], dtype=np.int64))
+    bad = C.c_int64(0)
+    lib().gs_gather_rows_cpu(table.ctypes.data_as(C.c_void_p), C.c_int64(table.shape[0]),
+                             C.c_int64(row_bytes), _p(ids), C.c_int64(ids.size),
+                             out.ctypes.data_as(C.c_void_p), C.byref(bad))
+    return out, bad.value

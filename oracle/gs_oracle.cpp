@@ -1076,3 +1076,26 @@ extern "C" void gs_csc_col_sample_weighted_cdf_fill_cpu(
       if (a[off + 1] == a[off]) emit(taken++, off);
   }
 }
+
+// -------------------------------------------------------------------------
+// Row gather, out[i, :] = table[ids[i], :] over rows of row_bytes bytes:
+// IndexSelectSingleKernel of src/cuda/index_select_uvm.cu:9-19 generalised
+// from scalars to rows (what dgl.utils.gather_pinned_tensor_rows does for
+// python/gs/matrix_api/matrix.py:19-23).  An id outside [0, num_rows) gives a
+// row of zero bytes and is counted.
+extern "C" void gs_gather_rows_cpu(const void* table, int64_t num_rows,
+                                   int64_t row_bytes, const int64_t* ids, int64_t n,
+                                   void* out, int64_t* bad_count) {
+  int64_t bad = 0;
+#pragma omp parallel for schedule(static) reduction(+ : bad)
+  for (int64_t i = 0; i < n; ++i) {
+    char* dst = (char*)out + i * row_bytes;
+    if (ids[i] >= 0 && ids[i] < num_rows)
+      std::memcpy(dst, (const char*)table + ids[i] * row_bytes, (size_t)row_bytes);
+    else {
+      std::memset(dst, 0, (size_t)row_bytes);
+      ++bad;
+    }
+  }
+  if (bad_count) *bad_count = bad;
+}
