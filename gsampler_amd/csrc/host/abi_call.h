@@ -4,6 +4,7 @@
 #ifndef GS_HOST_ABI_CALL_H_
 #define GS_HOST_ABI_CALL_H_
 
+#include <c10/hip/HIPFunctions.h>
 #include <c10/hip/HIPStream.h>
 #include <hip/hip_runtime_api.h>
 #include <torch/torch.h>
@@ -43,13 +44,35 @@ inline int64_t* mptr(torch::Tensor& t) {
   return (t.defined() && t.numel() > 0) ? t.data_ptr<int64_t>() : nullptr;
 }
 
+// Structure arrays of a loaded matrix may also sit in pinned host memory, which
+// the kernels read in place over the host link (the reference's UVA mode:
+// examples/graphsage/graphsage_e2e.py:62-66 pins indptr / indices before
+// load_graph).  Everything an operator produces lives on the GPU.
+inline torch::Tensor graph_ids(const torch::Tensor& t, const char* name) {
+  TORCH_CHECK(t.defined(), name, " is undefined");
+  TORCH_CHECK(t.is_cuda() || t.is_pinned(), name,
+              " must live on the GPU or in pinned host memory (got ", t.device(), ")");
+  TORCH_CHECK(t.scalar_type() == torch::kInt64, name, " must be int64 (got ",
+              t.scalar_type(), ")");
+  return t.contiguous();
+}
+
+// Options of a fresh output: on the device of `like`, or on the current GPU
+// when `like` is a pinned host tensor.
+inline torch::TensorOptions device_options(const torch::Tensor& like) {
+  if (like.is_cuda()) return like.options();
+  return like.options()
+      .device(c10::Device(c10::kCUDA, c10::hip::current_device()))
+      .pinned_memory(false);
+}
+
 inline torch::Tensor new_ids(int64_t n, const torch::Tensor& like) {
-  return torch::empty({n}, like.options().dtype(torch::kInt64));
+  return torch::empty({n}, device_options(like).dtype(torch::kInt64));
 }
 
 inline torch::Tensor new_workspace(size_t bytes, const torch::Tensor& like) {
   return torch::empty({(int64_t)(bytes > 0 ? bytes : 1)},
-                      like.options().dtype(torch::kUInt8));
+                      device_options(like).dtype(torch::kUInt8));
 }
 
 // Last element of a device prefix array (one blocking 8-byte copy).

@@ -19,8 +19,8 @@ static uint64_t next_call_id() { return random_state().next_call++; }
 // ------------------------------------------------------------------ loading
 void Graph::LoadCSC(torch::Tensor indptr, torch::Tensor indices) {
   auto m = std::make_shared<Compressed>();
-  m->indptr = ids(indptr, "indptr");
-  m->indices = ids(indices, "indices");
+  m->indptr = graph_ids(indptr, "indptr");
+  m->indices = graph_ids(indices, "indices");
   TORCH_CHECK(m->indptr.numel() == num_cols_ + 1, "LoadCSC: indptr has ",
               indptr.numel(), " entries for ", num_cols_, " columns");
   csc_ = m;
@@ -29,8 +29,8 @@ void Graph::LoadCSC(torch::Tensor indptr, torch::Tensor indices) {
 
 void Graph::LoadCSR(torch::Tensor indptr, torch::Tensor indices) {
   auto m = std::make_shared<Compressed>();
-  m->indptr = ids(indptr, "indptr");
-  m->indices = ids(indices, "indices");
+  m->indptr = graph_ids(indptr, "indptr");
+  m->indices = graph_ids(indices, "indices");
   TORCH_CHECK(m->indptr.numel() == num_rows_ + 1, "LoadCSR: indptr has ",
               indptr.numel(), " entries for ", num_rows_, " rows");
   csr_ = m;
@@ -40,8 +40,8 @@ void Graph::LoadCSR(torch::Tensor indptr, torch::Tensor indices) {
 void Graph::LoadCOO(torch::Tensor row, torch::Tensor col, bool row_sorted,
                     bool col_sorted) {
   auto m = std::make_shared<Coordinate>();
-  m->row = ids(row, "row");
-  m->col = ids(col, "col");
+  m->row = graph_ids(row, "row");
+  m->col = graph_ids(col, "col");
   TORCH_CHECK(row.numel() == col.numel(), "LoadCOO: row and col differ in length");
   m->row_sorted = row_sorted;
   m->col_sorted = col_sorted;
@@ -98,6 +98,13 @@ static std::shared_ptr<Coordinate> expand(const Compressed& m, bool is_csc) {
 
 void Graph::CreateSparseFormat(int64_t format) {
   TORCH_CHECK(csc_ || csr_ || coo_, "the graph holds no sparse format yet");
+  const bool have = (format == kCOO && coo_) || (format == kCSC && csc_) ||
+                    (format == kCSR && csr_);
+  if (!have) {
+    const torch::Tensor& any = csc_ ? csc_->indices : csr_ ? csr_->indices : coo_->row;
+    TORCH_CHECK(any.is_cuda(), "a matrix in pinned host memory is not converted to "
+                "another sparse format: load the format the operator runs on");
+  }
   if (format == kCOO) {
     if (coo_) return;
     coo_ = csc_ ? expand(*csc_, true) : expand(*csr_, false);
