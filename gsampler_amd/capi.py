@@ -60,6 +60,8 @@ SIGNATURES = {
     "gs_split_indptr": (_int, [_p, _p, _i64, _i64, _p, _p]),
     "gs_first_position": (_int, [_p, _i64, _i64, _p, _p]),
     "gs_gather_rows": (_int, [_p, _i64, _i64, _p, _i64, _p, _p, _p]),
+    "gs_coo_sort_workspace_bytes": (_sz, [_i64, _i64]),
+    "gs_coo_sort": (_int, [_p, _i64, _i64, _p, _p, _p, _sz, _p]),
     "gs_sddmm": (_int, [_int, _p, _p, _i64, _i64, _p, _int, _int, _p, _p, _p, _int, _int,
                         _i64, _i64, _i64, _i64, _p, _p, _p]),
     "gs_fused_u_op_v": (_int, [_int, _p, _p, _i64, _i64, _int, _int, _p, _p, _p, _p, _p,
@@ -342,6 +344,24 @@ def first_position(ids: torch.Tensor, num_ids: int) -> torch.Tensor:
     out = torch.empty(num_ids, dtype=torch.int64, device=ids.device)
     check(lib().gs_first_position(_ptr(ids), ids.numel(), num_ids, _ptr(out), _stream()))
     return out
+
+
+def coo_sort(major: torch.Tensor, num_major: int):
+    """Stable sort of edge positions by their id on the axis to compress:
+    (sorted ids, positions)."""
+    major = _i64t(major, "major")
+    n = major.numel()
+    out, perm = torch.empty_like(major), torch.empty_like(major)
+    ws = _workspace(lib().gs_coo_sort_workspace_bytes(n, num_major), major.device)
+    check(lib().gs_coo_sort(_ptr(major), n, num_major, _ptr(out), _ptr(perm), ws.data_ptr(),
+                            ws.numel(), _stream()))
+    return out, perm
+
+
+def coo_to_csc(row: torch.Tensor, col: torch.Tensor, num_cols: int):
+    """(indptr, row ids in column order, edge positions in column order)."""
+    sorted_col, perm = coo_sort(col, num_cols)
+    return sorted_to_indptr(sorted_col, num_cols), gather_rows(_i64t(row, "row"), perm), perm
 
 
 def gather_rows(table: torch.Tensor, ids: torch.Tensor, count_bad: bool = False):

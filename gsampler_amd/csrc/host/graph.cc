@@ -73,11 +73,14 @@ static std::shared_ptr<Compressed> compress(const Coordinate& coo, bool by_col,
     out->indices = minor;
     out->e_ids = coo.e_ids;
   } else {
-    torch::Tensor perm = torch::argsort(major, /*stable=*/true, /*dim=*/0);
-    sorted_major = major.index_select(0, perm);
-    out->indices = minor.index_select(0, perm);
-    out->e_ids = coo.e_ids.has_value() ? coo.e_ids.value().index_select(0, perm)
-                                       : perm;
+    const int64_t nnz = major.numel();
+    torch::Tensor perm = new_ids(nnz, major);
+    sorted_major = new_ids(nnz, major);
+    torch::Tensor ws = new_workspace(gs_coo_sort_workspace_bytes(nnz, num_major), major);
+    GS_CALL(gs_coo_sort(cptr(major), nnz, num_major, mptr(sorted_major), mptr(perm),
+                        ws.data_ptr(), (size_t)ws.numel(), cur_stream()));
+    out->indices = GatherRows(minor, perm);
+    out->e_ids = coo.e_ids.has_value() ? GatherRows(coo.e_ids.value(), perm) : perm;
   }
   out->indptr = new_ids(num_major + 1, major);
   GS_CALL(gs_sorted_to_indptr(cptr(sorted_major), sorted_major.numel(),

@@ -1,10 +1,14 @@
 // sort.hip -- per-segment key sort (row ids inside every column), the
-// prerequisite of node2vec's connectivity test.  The sort itself is rocPRIM's
-// segmented radix sort; this file only adapts it to the workspace convention.
+// prerequisite of node2vec's connectivity test, and the stable sort of edges by
+// column (or row) id that turns an edge list into a compressed format.  The
+// sorts themselves are rocPRIM's radix sorts; this file adapts them to the
+// workspace convention and limits the sorted bits to what the ids need.
 #include "common.h"
 
 #include <cstring>
+#include <rocprim/device/device_radix_sort.hpp>
 #include <rocprim/device/device_segmented_radix_sort.hpp>
+#include <rocprim/iterator/counting_iterator.hpp>
 
 extern "C" {
 
@@ -41,6 +45,50 @@ int gs_segment_sort_i64(const int64_t* indptr, int64_t num_segments,
   GS_HIP(rocprim::segmented_radix_sort_keys(workspace, bytes, keys_in, keys_out,
                                             (size_t)nnz, (unsigned)num_segments,
                                             indptr, indptr + 1, 0, 64, s));
+  return GS_OK;
+}
+
+
+static int id_bits(int64_t num_ids) {
+  int bits = 1;
+  while (bits < 63 && ((int64_t)1 << bits) < num_ids) ++bits;
+  return bits;
+}
+
+size_t gs_coo_sort_workspace_bytes(int64_t nnz, int64_t num_major) {
+  if (nnz < 0) return 0;
+  size_t bytes = 0;
+  const int64_t* k = nullptr;
+  int64_t* o = nullptr;
+  (void)rocprim::radix_sort_pairs(nullptr, bytes, k, o, rocprim::counting_iterator<int64_t>(0), o,
+                                  (size_t)(nnz > 0 ? nnz : 1), 0u, (unsigned)id_bits(num_major));
+  return gs::align_up(bytes, 256);
+}
+
+// Stable sort of the edge positions 0..nnz-1 by major[position]: sorted_major
+// receives the ids in order, perm the positions.  Only the low bits that ids
+// below num_major can have are sorted (COOSort, src/cuda/format_transform.cu:
+// 65-84, does the same through cub): three 8-bit passes instead of eight for a
+// few million columns.  Ids must lie in [0, num_major).
+int gs_coo_sort(const int64_t* major, int64_t nnz, int64_t num_major,
+                int64_t* sorted_major, int64_t* perm, void* workspace,
+                size_t workspace_bytes, gs_stream_t stream) {
+  using namespace gs;
+  GS_REQUIRE(nnz >= 0 && num_major >= 0, "coo_sort: negative size");
+  if (nnz == 0) return GS_OK;
+  GS_REQUIRE(major && sorted_major && perm, "coo_sort: null pointer");
+  GS_REQUIRE(major != sorted_major, "coo_sort: in-place sorting is not supported");
+  size_t need = gs_coo_sort_workspace_bytes(nnz, num_major);
+  if (workspace == nullptr || workspace_bytes < need) {
+    set_error("coo_sort workspace too small: %zu < %zu", workspace_bytes, need);
+    return GS_ERR_WORKSPACE;
+  }
+  hipStream_t s = as_stream(stream);
+  size_t bytes = workspace_bytes;
+  ProfScope ps("coo_sort", s);
+  GS_HIP(rocprim::radix_sort_pairs(workspace, bytes, major, sorted_major,
+                                   rocprim::counting_iterator<int64_t>(0), perm, (size_t)nnz,
+                                   0u, (unsigned)id_bits(num_major), s));
   return GS_OK;
 }
 

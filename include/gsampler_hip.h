@@ -285,6 +285,19 @@ int gs_first_position(const int64_t* ids, int64_t n, int64_t num_ids,
                       int64_t* out_first, gs_stream_t stream);
 
 /* ------------------------------------------------------------------------
+ * Edge list -> compressed format, first half: stable sort of the edge
+ * positions by their id on the axis to compress (`major`, ids in
+ * [0, num_major)).  sorted_major receives the ids in order, perm the positions
+ * (the e_ids of the new format); gs_sorted_to_indptr and two gathers by perm
+ * finish the conversion.  COOSort / COO2CSCCUDA,
+ * src/cuda/format_transform.cu:65-84,121-142.
+ * ---------------------------------------------------------------------- */
+size_t gs_coo_sort_workspace_bytes(int64_t nnz, int64_t num_major);
+int gs_coo_sort(const int64_t* major, int64_t nnz, int64_t num_major,
+                int64_t* sorted_major, int64_t* perm, void* workspace,
+                size_t workspace_bytes, gs_stream_t stream);
+
+/* ------------------------------------------------------------------------
  * Row gather: out[i, :] = table[ids[i], :] for rows of `row_bytes` bytes of any
  * element type (node features of the sampled frontier, labels, edge data
  * behind an edge index).  `table` is device memory or pinned host memory that

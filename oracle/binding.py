@@ -441,3 +441,16 @@ def gather_rows(table, ids):
                              C.c_int64(row_bytes), _p(ids), C.c_int64(ids.size),
                              out.ctypes.data_as(C.c_void_p), C.byref(bad))
     return out, bad.value
+
+
+def coo_sort(major):
+    major = _i64(major)
+    out, perm = np.empty_like(major), np.empty_like(major)
+    lib().gs_coo_sort_cpu(_p(major), C.c_int64(major.size), _p(out), _p(perm))
+    return out, perm
+
+
+def coo_to_csc(row, col, num_cols):
+    """(indptr, row ids in column order, edge positions in column order)."""
+    sorted_col, perm = coo_sort(col)
+    return sorted_to_indptr(sorted_col, num_cols), _i64(row)[perm], perm

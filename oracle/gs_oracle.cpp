@@ -1099,3 +1099,13 @@ extern "C" void gs_gather_rows_cpu(const void* table, int64_t num_rows,
   }
   if (bad_count) *bad_count = bad;
 }
+
+// Stable sort of edge positions by their id on the axis to compress (the
+// first half of COO2CSCCUDA, src/cuda/format_transform.cu:65-84,121-142).
+extern "C" void gs_coo_sort_cpu(const int64_t* major, int64_t nnz, int64_t* sorted_major,
+                                int64_t* perm) {
+  for (int64_t e = 0; e < nnz; ++e) perm[e] = e;
+  std::stable_sort(perm, perm + nnz,
+                   [major](int64_t a, int64_t b) { return major[a] < major[b]; });
+  for (int64_t e = 0; e < nnz; ++e) sorted_major[e] = major[perm[e]];
+}

@@ -240,3 +240,14 @@ def test_first_position(num_ids):
     assert np.array_equal(got, want)
     empty = capi.first_position(T(np.empty(0, dtype=np.int64)), 4).cpu().tolist()
     assert empty == [np.iinfo(np.int64).max] * 4
+
+
+@pytest.mark.parametrize("num_cols,nnz", [(1, 50), (300, 20000), (70000, 300000), (5, 0)])
+def test_coo_to_csc_parity(num_cols, nnz):
+    """Edge list -> CSC: stable sort over the id bits, indptr, gathers."""
+    rng = np.random.default_rng(num_cols)
+    col = rng.integers(0, num_cols, size=nnz)
+    row = rng.integers(0, 1000, size=nnz)
+    want = orc.coo_to_csc(row, col, num_cols)
+    got = capi.coo_to_csc(T(row), T(col), num_cols)
+    assert_same(got, want)

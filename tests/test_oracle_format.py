@@ -69,3 +69,18 @@ def test_split_indptr_rebases_every_batch():
     want = np.concatenate([indptr[a:b + 1] - indptr[a] for a, b in zip(offset[:-1], offset[1:])])
     assert np.array_equal(out, want)
     assert out.tolist() == [0, 2, 5, 0, 0, 0, 4, 7, 0, 0, 8]
+
+
+def test_coo_sort_is_a_stable_argsort_and_builds_the_csc():
+    rng = np.random.default_rng(11)
+    C, E = 300, 20000
+    col = rng.integers(0, C, size=E)
+    row = rng.integers(0, 500, size=E)
+    sorted_col, perm = orc.coo_sort(col)
+    want = np.argsort(col, kind="stable")
+    assert np.array_equal(perm, want) and np.array_equal(sorted_col, col[want])
+    indptr, indices, eids = orc.coo_to_csc(row, col, C)
+    assert np.array_equal(np.diff(indptr), np.bincount(col, minlength=C))
+    for c in (0, 17, C - 1):                              # column contents in edge order
+        assert np.array_equal(indices[indptr[c]:indptr[c + 1]], row[col == c])
+    assert np.array_equal(eids, want)
