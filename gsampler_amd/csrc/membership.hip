@@ -17,6 +17,7 @@ namespace gs {
 
 constexpr int kMemberWords = kBlock / kWave;  // flag words per chunk of kBlock edges
 constexpr int kMemberChunksPerWave = 8;
+constexpr int kMemberThreads = 1024;  // 16 waves share one staged table: 32 Ki edges per 32 KB copied
 constexpr int kMemberLdsSlots = 4096;  // tables up to this size are staged in LDS (32 KB)
 
 struct MemberWs {
@@ -49,88 +50,148 @@ static MemberWs carve_member(void* ws, int64_t nnz, int64_t num_picked) {
   return w;
 }
 
+// The look-ups run once per edge, so they are kept to 32-bit arithmetic: an
+// admissible id fits 32 bits, the home slot is one multiply and one
+// multiply-high, and a probe compares the upper half of a packed slot.
+constexpr uint32_t kNoKey = 0xFFFFFFFFu;  // upper half of the empty slot; no admissible id
+
+__device__ __forceinline__ uint32_t member_home(uint32_t key, uint32_t cap) {
+  return __umulhi(key * 0x9E3779B1u, cap);
+}
+
+// 32-bit form of an id, kNoKey for one that no picked id can equal
+__device__ __forceinline__ uint32_t member_key(uint64_t id) {
+  return id <= kMaxPackedKey ? (uint32_t)id : kNoKey;
+}
+
 __global__ __launch_bounds__(kBlock) void member_insert_kernel(
-    const int64_t* __restrict__ picked, int64_t n, uint64_t* table, uint64_t cap) {
+    const int64_t* __restrict__ picked, int64_t n, uint64_t* table, uint32_t cap) {
   const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
   if (i >= n) return;
-  const uint64_t key = (uint64_t)picked[i];
-  if (key > kMaxPackedKey) return;  // cannot equal any admissible id
-  table_insert_min(table, cap, key, (uint64_t)i);
+  const uint32_t key = member_key((uint64_t)picked[i]);
+  if (key == kNoKey) return;  // cannot equal any admissible id
+  const uint64_t mine = ((uint64_t)key << 32) | (uint64_t)i;
+  uint32_t slot = member_home(key, cap);
+  for (uint32_t probes = 0; probes < cap; ++probes) {  // the table has free slots: ends early
+    uint64_t cur = table[slot];
+    if (cur == kEmptySlot) {
+      cur = atomicCAS((unsigned long long*)(table + slot), (unsigned long long)kEmptySlot,
+                      (unsigned long long)mine);
+      if (cur == kEmptySlot) return;
+    }
+    if ((uint32_t)(cur >> 32) == key) {  // a repeated id keeps its smallest position
+      atomicMin((unsigned long long*)(table + slot), (unsigned long long)mine);
+      return;
+    }
+    if (++slot == cap) slot = 0;
+  }
 }
 
 // A small table (the picked set of a layer-wise sampler is a few hundred ids)
-// is copied into LDS once per work-group: 64 lanes probing 64 different slots
-// cost the vector cache a tag look-up each, the LDS a few cycles in all.
-template <bool kInLds>
-__device__ __forceinline__ const uint64_t* stage_table(const uint64_t* __restrict__ table,
-                                                       uint64_t cap, uint64_t* lds) {
-  if (!kInLds) return table;
-  for (uint64_t i = threadIdx.x; i < cap; i += kBlock) lds[i] = table[i];
-  __syncthreads();
-  return lds;
-}
+// is copied into LDS once per work-group, keys and positions apart: 64 lanes
+// probing 64 different slots cost the vector cache a tag look-up each, the LDS
+// a few cycles in all.
+template <bool kInLds, bool kWithValues>
+struct MemberTable {
+  const uint64_t* slots;
+  const uint32_t* keys;
+  const uint32_t* values;
+  uint32_t cap;
 
-// N look-ups in step: the probes of a round are issued together, so a lane
-// waits for the longest of its N probe runs instead of their sum.  slot[j] is
-// where key[j] was found, cap if it is absent.
-template <int N>
-__device__ __forceinline__ void table_find_many(const uint64_t* tab, uint64_t cap,
-                                                const uint64_t (&key)[N],
-                                                uint64_t (&slot)[N]) {
-  bool open[N];
-  bool any = false;
-#pragma unroll
-  for (int j = 0; j < N; ++j) {
-    open[j] = key[j] <= kMaxPackedKey;
-    slot[j] = open[j] ? home_slot(key[j], cap) : cap;
-    any |= open[j];
+  __device__ __forceinline__ void stage(const uint64_t* __restrict__ table, uint32_t capacity,
+                                        uint32_t* lds_keys, uint32_t* lds_values) {
+    slots = table;
+    keys = lds_keys;
+    values = lds_values;
+    cap = capacity;
+    if (!kInLds) return;
+    for (uint32_t i = threadIdx.x; i < capacity; i += blockDim.x) {
+      const uint64_t t = table[i];
+      lds_keys[i] = (uint32_t)(t >> 32);
+      if (kWithValues) lds_values[i] = (uint32_t)t;
+    }
+    __syncthreads();
   }
-  for (uint64_t probes = 0; any && probes < cap; ++probes) {
-    uint64_t cur[N];
-#pragma unroll
-    for (int j = 0; j < N; ++j) cur[j] = open[j] ? tab[slot[j]] : 0;
-    any = false;
+  __device__ __forceinline__ uint32_t key_at(uint32_t slot) const {
+    return kInLds ? keys[slot] : (uint32_t)(slots[slot] >> 32);
+  }
+  __device__ __forceinline__ uint32_t value_at(uint32_t slot) const {
+    return kInLds ? values[slot] : (uint32_t)slots[slot];
+  }
+
+  // N look-ups in step: the probes of a round are issued together, so a lane
+  // waits for the longest of its N probe runs instead of their sum.  slot[j]
+  // is where key[j] sits, cap when it is absent (or kNoKey).
+  template <int N>
+  __device__ __forceinline__ void find_many(const uint32_t (&key)[N], uint32_t (&slot)[N]) const {
+    uint32_t open = 0;  // bit j: key j is still probing
 #pragma unroll
     for (int j = 0; j < N; ++j) {
-      if (!open[j]) continue;
-      if ((cur[j] >> 32) == key[j]) {
-        open[j] = false;
-      } else if (cur[j] == kEmptySlot) {
-        open[j] = false;
-        slot[j] = cap;
-      } else if (++slot[j] == cap) {
-        slot[j] = 0;
+      slot[j] = cap;
+      if (key[j] != kNoKey) {
+        slot[j] = member_home(key[j], cap);
+        open |= 1u << j;
       }
-      any |= open[j];
     }
-  }
+    for (uint32_t probes = 0; open != 0 && probes < cap; ++probes) {
+      uint32_t cur[N];
 #pragma unroll
-  for (int j = 0; j < N; ++j)
-    if (open[j]) slot[j] = cap;  // probe budget spent: a table too small for its keys
-}
+      for (int j = 0; j < N; ++j) cur[j] = (open >> j) & 1u ? key_at(slot[j]) : 0u;
+#pragma unroll
+      for (int j = 0; j < N; ++j) {
+        if (!((open >> j) & 1u)) continue;
+        if (cur[j] == key[j]) {
+          open &= ~(1u << j);
+        } else if (cur[j] == kNoKey) {
+          open &= ~(1u << j);
+          slot[j] = cap;
+        } else if (++slot[j] == cap) {
+          slot[j] = 0;
+        }
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < N; ++j)
+      if ((open >> j) & 1u) slot[j] = cap;  // probe budget spent: cannot happen with free slots
+  }
+};
 
 template <bool kInLds>
-__global__ __launch_bounds__(kBlock) void member_flag_kernel(
+__global__ __launch_bounds__(kMemberThreads) void member_flag_kernel(
     const int64_t* __restrict__ ids, int64_t nnz,
-    const uint64_t* __restrict__ global_table, uint64_t cap,
+    const uint64_t* __restrict__ global_table, uint32_t cap,
     uint64_t* __restrict__ flags, int64_t* __restrict__ chunk_count) {
-  __shared__ uint64_t lds_table[kInLds ? kMemberLdsSlots : 1];
-  const uint64_t* table = stage_table<kInLds>(global_table, cap, lds_table);
+  __shared__ uint32_t lds_keys[kInLds ? kMemberLdsSlots : 1];
+  MemberTable<kInLds, false> table;
+  table.stage(global_table, cap, lds_keys, nullptr);
   const int64_t num_chunks = ceil_div_dev(nnz, kBlock);
-  const int64_t wave = (int64_t)blockIdx.x * kMemberWords + threadIdx.x / kWave;
+  const int64_t wave = (int64_t)blockIdx.x * (kMemberThreads / kWave) + threadIdx.x / kWave;
   const int lane = lane_id();
-  for (int c = 0; c < kMemberChunksPerWave; ++c) {
-    const int64_t chunk = wave * kMemberChunksPerWave + c;
-    if (chunk >= num_chunks) return;
-    const int64_t e0 = chunk * kBlock;
-    uint64_t key[kMemberWords];
+  // the ids of the next chunk are requested before the look-ups of this one
+  uint32_t next_key[kMemberWords];
+  const int64_t first_chunk = wave * kMemberChunksPerWave;
+  if (first_chunk >= num_chunks) return;
 #pragma unroll
-    for (int j = 0; j < kMemberWords; ++j) {
-      const int64_t e = e0 + j * kWave + lane;
-      key[j] = e < nnz ? (uint64_t)ids[e] : ~0ull;
+  for (int j = 0; j < kMemberWords; ++j) {
+    const int64_t e = first_chunk * kBlock + j * kWave + lane;
+    next_key[j] = e < nnz ? member_key((uint64_t)ids[e]) : kNoKey;
+  }
+  for (int c = 0; c < kMemberChunksPerWave; ++c) {
+    const int64_t chunk = first_chunk + c;
+    if (chunk >= num_chunks) return;
+    uint32_t key[kMemberWords];
+#pragma unroll
+    for (int j = 0; j < kMemberWords; ++j) key[j] = next_key[j];
+    if (c + 1 < kMemberChunksPerWave && chunk + 1 < num_chunks) {
+#pragma unroll
+      for (int j = 0; j < kMemberWords; ++j) {
+        const int64_t e = (chunk + 1) * kBlock + j * kWave + lane;
+        next_key[j] = e < nnz ? member_key((uint64_t)ids[e]) : kNoKey;
+      }
     }
-    uint64_t slot[kMemberWords], word[kMemberWords];
-    table_find_many<kMemberWords>(table, cap, key, slot);
+    uint32_t slot[kMemberWords];
+    uint64_t word[kMemberWords];
+    table.find_many(key, slot);
 #pragma unroll
     for (int j = 0; j < kMemberWords; ++j) word[j] = __ballot(slot[j] < cap);
     if (lane == 0) {
@@ -173,20 +234,37 @@ __global__ __launch_bounds__(kBlock) void member_indptr_kernel(
 }
 
 template <bool kInLds>
-__global__ __launch_bounds__(kBlock) void member_fill_kernel(
+__global__ __launch_bounds__(kMemberThreads) void member_fill_kernel(
     const int64_t* __restrict__ ids, int64_t nnz,
-    const uint64_t* __restrict__ global_table, uint64_t cap,
+    const uint64_t* __restrict__ global_table, uint32_t cap,
     const uint64_t* __restrict__ flags, const int64_t* __restrict__ chunk_off,
     const int64_t* __restrict__ indptr, int64_t num_major,
     const int64_t* __restrict__ edge_major, int64_t* __restrict__ out_major,
     int64_t* __restrict__ out_minor, int64_t* __restrict__ out_select) {
-  __shared__ uint64_t lds_table[kInLds ? kMemberLdsSlots : 1];
-  const uint64_t* table = stage_table<kInLds>(global_table, cap, lds_table);
+  __shared__ uint32_t lds_keys[kInLds ? kMemberLdsSlots : 1];
+  __shared__ uint32_t lds_values[kInLds ? kMemberLdsSlots : 1];
+  MemberTable<kInLds, true> table;
+  table.stage(global_table, cap, lds_keys, lds_values);
   const int64_t num_chunks = ceil_div_dev(nnz, kBlock);
-  const int64_t wave = (int64_t)blockIdx.x * kMemberWords + threadIdx.x / kWave;
+  const int64_t wave = (int64_t)blockIdx.x * (kMemberThreads / kWave) + threadIdx.x / kWave;
   const int lane = lane_id();
+  const int64_t first_chunk = wave * kMemberChunksPerWave;
+  if (first_chunk >= num_chunks) return;
+  // flag words and kept ids of the next chunk are requested ahead
+  uint64_t next_word[kMemberWords];
+  uint32_t next_key[kMemberWords];
+  auto request = [&](int64_t chunk) {
+#pragma unroll
+    for (int j = 0; j < kMemberWords; ++j) next_word[j] = flags[chunk * kMemberWords + j];
+#pragma unroll
+    for (int j = 0; j < kMemberWords; ++j) {
+      const int64_t e = chunk * kBlock + j * kWave + lane;
+      next_key[j] = ((next_word[j] >> lane) & 1ull) ? member_key((uint64_t)ids[e]) : kNoKey;
+    }
+  };
+  request(first_chunk);
   for (int c = 0; c < kMemberChunksPerWave; ++c) {
-    const int64_t chunk = wave * kMemberChunksPerWave + c;
+    const int64_t chunk = first_chunk + c;
     if (chunk >= num_chunks) return;
     const int64_t e0 = chunk * kBlock;
     const int64_t e_last = e0 + kBlock - 1 < nnz ? e0 + kBlock - 1 : nnz - 1;
@@ -197,20 +275,21 @@ __global__ __launch_bounds__(kBlock) void member_fill_kernel(
       seg_hi = segment_of(indptr, num_major, wave_uniform_first(e_last));
     }
     int64_t before = chunk_off[chunk];
-    uint64_t word[kMemberWords], key[kMemberWords], slot[kMemberWords];
+    uint64_t word[kMemberWords];
+    uint32_t key[kMemberWords], slot[kMemberWords];
 #pragma unroll
     for (int j = 0; j < kMemberWords; ++j) {
-      word[j] = flags[chunk * kMemberWords + j];
-      const int64_t e = e0 + j * kWave + lane;
-      key[j] = ((word[j] >> lane) & 1ull) ? (uint64_t)ids[e] : ~0ull;
+      word[j] = next_word[j];
+      key[j] = next_key[j];
     }
-    table_find_many<kMemberWords>(table, cap, key, slot);
+    if (c + 1 < kMemberChunksPerWave && chunk + 1 < num_chunks) request(chunk + 1);
+    table.find_many(key, slot);
 #pragma unroll
     for (int j = 0; j < kMemberWords; ++j) {
       const int64_t e = e0 + j * kWave + lane;
       if ((word[j] >> lane) & 1ull) {
         const int64_t pos = before + __popcll(word[j] & ((1ull << lane) - 1));
-        out_minor[pos] = (int64_t)(uint32_t)table[slot[j] < cap ? slot[j] : 0];
+        out_minor[pos] = (int64_t)table.value_at(slot[j] < cap ? slot[j] : 0);
         out_select[pos] = e;
         if (out_major)
           out_major[pos] =
@@ -254,7 +333,7 @@ int gs_minor_slice_count(const int64_t* ids, int64_t nnz, const int64_t* picked,
     return GS_ERR_WORKSPACE;
   }
   hipStream_t s = as_stream(stream);
-  const uint64_t cap = member_table_slots(num_picked);
+  const uint32_t cap = (uint32_t)member_table_slots(num_picked);
   GS_LAUNCH("member_clear", s,
             table_fill_kernel<><<<dim3((unsigned)ceil_div((int64_t)cap, kBlock * 4)),
                                   dim3(kBlock), 0, s>>>(w.table, (int64_t)cap,
@@ -265,14 +344,14 @@ int gs_minor_slice_count(const int64_t* ids, int64_t nnz, const int64_t* picked,
                                      dim3(kBlock), 0, s>>>(picked, num_picked,
                                                            w.table, cap));
   if (nnz > 0) {
-    const int64_t blocks = ceil_div(w.chunks, kMemberWords * kMemberChunksPerWave);
+    const int64_t blocks = ceil_div(w.chunks, (kMemberThreads / kWave) * kMemberChunksPerWave);
     if (cap <= (uint64_t)kMemberLdsSlots)
       GS_LAUNCH("member_flag", s,
-                member_flag_kernel<true><<<dim3((unsigned)blocks), dim3(kBlock), 0, s>>>(
+                member_flag_kernel<true><<<dim3((unsigned)blocks), dim3(kMemberThreads), 0, s>>>(
                     ids, nnz, w.table, cap, w.flags, w.chunk_off));
     else
       GS_LAUNCH("member_flag", s,
-                member_flag_kernel<false><<<dim3((unsigned)blocks), dim3(kBlock), 0, s>>>(
+                member_flag_kernel<false><<<dim3((unsigned)blocks), dim3(kMemberThreads), 0, s>>>(
                     ids, nnz, w.table, cap, w.flags, w.chunk_off));
     int rc = exclusive_scan_i64(w.chunk_off, w.chunk_off, w.chunks + 1, w.scan_ws,
                                 w.scan_ws_bytes, s);
@@ -306,16 +385,16 @@ int gs_minor_slice_fill(const int64_t* ids, int64_t nnz, int64_t num_picked,
     return GS_ERR_WORKSPACE;
   }
   hipStream_t s = as_stream(stream);
-  const uint64_t cap = member_table_slots(num_picked);
-  const dim3 grid((unsigned)ceil_div(w.chunks, kMemberWords * kMemberChunksPerWave));
+  const uint32_t cap = (uint32_t)member_table_slots(num_picked);
+  const dim3 grid((unsigned)ceil_div(w.chunks, (kMemberThreads / kWave) * kMemberChunksPerWave));
   if (cap <= (uint64_t)kMemberLdsSlots)
     GS_LAUNCH("member_fill", s,
-              member_fill_kernel<true><<<grid, dim3(kBlock), 0, s>>>(
+              member_fill_kernel<true><<<grid, dim3(kMemberThreads), 0, s>>>(
                   ids, nnz, w.table, cap, w.flags, w.chunk_off, indptr, num_major,
                   edge_major, out_major, out_minor, out_select));
   else
     GS_LAUNCH("member_fill", s,
-              member_fill_kernel<false><<<grid, dim3(kBlock), 0, s>>>(
+              member_fill_kernel<false><<<grid, dim3(kMemberThreads), 0, s>>>(
                   ids, nnz, w.table, cap, w.flags, w.chunk_off, indptr, num_major,
                   edge_major, out_major, out_minor, out_select));
   return GS_OK;
