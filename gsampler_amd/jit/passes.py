@@ -53,6 +53,14 @@ def dce(gm: fx.GraphModule) -> fx.GraphModule:
     return _finish(gm)
 
 
+def _draws_random_numbers(node: fx.Node) -> bool:
+    """Sampling and walk operators, whether methods of the graph class
+    (call_method, target is the name) or free operators of gs_ops
+    (call_function, target is the operator object)."""
+    name = node.target if isinstance(node.target, str) else str(node.target)
+    return any(word in name for word in ("Sampling", "RandomWalk", "Node2Vec"))
+
+
 def cse(gm: fx.GraphModule) -> fx.GraphModule:
     """Merges nodes with identical target and arguments.  Sampling operators are
     left alone: two textually identical sampling calls draw different samples."""
@@ -60,7 +68,7 @@ def cse(gm: fx.GraphModule) -> fx.GraphModule:
     for node in list(gm.graph.nodes):
         if node.op in ("placeholder", "output"):
             continue
-        if isinstance(node.target, str) and "Sampling" in node.target:
+        if _draws_random_numbers(node):
             continue
         if node.target in IN_PLACE_OPS:
             continue

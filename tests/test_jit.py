@@ -152,6 +152,32 @@ def test_ladies_rewrites():
     assert sum(n.op == "placeholder" for n in c.gm.graph.nodes) >= 3
 
 
+def fastgcn_like_sampler(A, seeds, fanouts):
+    ret = []
+    for K in fanouts:
+        subA = A[:, seeds]
+        sampleA, _ = subA.collective_sampling(K, subA.row_ndata["deg"], False)
+        seeds = sampleA.all_nodes()
+        ret.append(sampleA.to_dgl_block())
+    return seeds, ret
+
+
+def walks_twice(A, seeds):
+    return A.random_walk(seeds, 3), A.random_walk(seeds, 3)
+
+
+def test_identical_sampling_calls_are_not_merged():
+    """Every layer of FastGCN samples the same list of row weights: the calls
+    look alike but each draws its own sample (free operators and walks too)."""
+    m = gs.Matrix(gs.Graph(10, 10))
+    m.row_ndata["deg"] = torch.rand(10)
+    c = gs.jit.compile(func=fastgcn_like_sampler, args=(m, torch.arange(3), [4, 4]))
+    names = [str(n.target) for n in c.gm.graph.nodes if n.op == "call_function"]
+    assert sum("ListSamplingWithProbs" in n for n in names) == 2
+    c = gs.jit.compile(func=walks_twice, args=(m, torch.arange(3)))
+    assert targets(c.gm).count("_CAPI_RandomWalk") == 2
+
+
 def test_two_u_mul_v_are_merged():
     m = gs.Matrix(gs.Graph(10, 10))
     u, v = torch.rand(10), torch.rand(3)
