@@ -82,7 +82,11 @@ class BatchMatrix(Matrix):
                     raise NotImplementedError("encoded slicing of an already row-sliced BatchMatrix")
                 row_ids, _ = graph._CAPI_BatchGetRows()
                 out.row_ndata["_ID"] = row_ids
-            row_pick, col_pick = None, cols
+            # Encoded slicing renumbers the rows (one run of compact ids per
+            # batch), so other per-row data follows them.  The reference keeps
+            # the old arrays there (python/gs/matrix_api/batch_matrix.py:140-141),
+            # which a later row slice then indexes with compact ids.
+            row_pick, col_pick = (row_ids if self.encoding else None), cols
         else:
             raise NotImplementedError("BatchMatrix indices must be `ids::ptr` slices")
 

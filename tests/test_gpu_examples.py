@@ -263,3 +263,55 @@ def test_kgcn(world):
     assert bool((adj[rows, torch.repeat_interleave(seeds, deg)] > 0).all())
     for a, b in zip(e_layers, c_layers):
         assert all(torch.equal(x, y) for x, y in zip(a.csc[:2], b.csc[:2]))
+
+
+# ------------------------------------------------------------ batched LADIES
+def batch_ladies_sampler(A, fanouts, seeds, seeds_ptr):
+    blocks = []
+    for K in fanouts:
+        sub = A[:, seeds::seeds_ptr]
+        sub.edata["p"] = sub.edata["w"] ** 2
+        prob = sub.sum("p", axis=1)
+        _, probs_ptr = sub.all_rows()
+        picked, index = sub.collective_sampling(K, prob, probs_ptr, False)
+        picked = picked.div("w", prob[index], axis=1)
+        picked = picked.div("w", picked.sum("w", axis=0), axis=0)
+        seeds, seeds_ptr = picked.all_nodes()
+        blocks.append(picked.to_dgl_block(prefetch_edata={"w"}))
+    return blocks
+
+
+def test_batch_ladies(world):
+    m, _, adj = world
+    bm = gs.BatchMatrix()
+    bm.load_from_matrix(m)
+    parts = [torch.arange(s, N, 97, device=DEV) for s in (0, 11, 50)]
+    seeds = torch.cat(parts)
+    ptr = torch.tensor([0] + list(torch.cumsum(torch.tensor([p.numel() for p in parts]), 0)),
+                       device=DEV)
+    K = 64
+    gs.manual_seed(11)
+    eager = batch_ladies_sampler(bm, [K, K], seeds, ptr)
+    assert gs.random_state() == (11, 2)
+    compiled = gs.jit.compile(func=batch_ladies_sampler, args=(bm, [K, K], seeds, ptr))
+    gs.manual_seed(11)
+    jit = compiled(bm, [K, K], seeds, ptr)
+    assert gs.random_state() == (11, 2)
+    for layers in (eager, jit):
+        assert len(layers) == 2 and all(len(per_batch) == 3 for per_batch in layers)
+        dst = parts
+        for per_batch in layers:
+            nxt = []
+            for block, ids in zip(per_batch, dst):
+                edges_exist(block, ids, adj)
+                assert block.num_dst == ids.numel()
+                assert torch.equal(block.srcdata["_ID"][: ids.numel()], ids)
+                assert torch.unique(block.srcdata["_ID"][block.row]).numel() <= K
+                # weights are normalised per destination node
+                sums = torch.zeros(ids.numel(), device=DEV).index_add_(0, block.col, block.edata["w"])
+                has = torch.bincount(block.col, minlength=ids.numel()) > 0
+                assert torch.allclose(sums[has], torch.ones_like(sums[has]), rtol=1e-4)
+                nxt.append(block.srcdata["_ID"])
+            dst = nxt
+    for a, b, ids in zip(eager[0], jit[0], parts):     # first layer: the same picks
+        same_edge_sets(a, b, ids)
