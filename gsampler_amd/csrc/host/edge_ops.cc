@@ -95,6 +95,22 @@ torch::Tensor feat(const torch::Tensor& t, const char* name) {
   return t.contiguous();
 }
 
+// An operand indexed by row ids, edge ids or column ids must have a row for
+// every one of them: a shorter tensor would be read out of bounds on the GPU
+// (the reference does not check, src/graph.cc:320-379).
+void need_rows(const torch::Tensor& t, int64_t rows, const char* who, const char* name) {
+  if (!t.defined()) return;
+  TORCH_CHECK(t.dim() >= 1 && t.size(0) >= rows, who, ": ", name, " has ",
+              t.dim() >= 1 ? t.size(0) : 0, " rows, the matrix needs ", rows);
+}
+
+void same_dtype(const torch::Tensor& t, const torch::Tensor& out, const char* who,
+                const char* name) {
+  if (!t.defined()) return;
+  TORCH_CHECK(t.scalar_type() == out.scalar_type(), who, ": ", name, " is ",
+              t.scalar_type(), " but out is ", out.scalar_type());
+}
+
 int dtype_code(const torch::Tensor& t) {
   if (t.scalar_type() == torch::kFloat32) return GS_F32;
   if (t.scalar_type() == torch::kFloat64) return GS_F64;
@@ -135,7 +151,17 @@ void Graph::SDDMM(const std::string& op, torch::Tensor lhs, torch::Tensor rhs,
   rhs = feat(rhs, "rhs");
   TORCH_CHECK(out.defined() && out.is_cuda() && out.is_contiguous(),
               "SDDMM: out must be a contiguous GPU tensor");
+  const int64_t per_target[3] = {num_rows_, num_edges_, num_cols_};
+  TORCH_CHECK(lhs_target >= 0 && lhs_target <= 2 && rhs_target >= 0 && rhs_target <= 2,
+              "SDDMM: targets must be 0 (u), 1 (e) or 2 (v)");
+  if (op != "copy_rhs") need_rows(lhs, per_target[lhs_target], "SDDMM", "lhs");
+  if (op != "copy_lhs") need_rows(rhs, per_target[rhs_target], "SDDMM", "rhs");
+  need_rows(out, num_edges_, "SDDMM", "out");
+  same_dtype(lhs, out, "SDDMM", "lhs");
+  same_dtype(rhs, out, "SDDMM", "rhs");
   const Broadcast bc = make_broadcast(op, lhs, rhs, out);
+  TORCH_CHECK(out.numel() >= num_edges_ * bc.out_len, "SDDMM: out holds ", out.numel(),
+              " values, ", num_edges_ * bc.out_len, " are written");
   if (on_format == kCSR) {  // rows are the compressed axis: swap u and v
     lhs_target = lhs_target == 1 ? 1 : 2 - lhs_target;
     rhs_target = rhs_target == 1 ? 1 : 2 - rhs_target;
@@ -159,7 +185,19 @@ void Graph::FusedUOPV(const std::string& op, torch::Tensor lhs1,
   lhs2 = feat(lhs2, "lhs2"), rhs2 = feat(rhs2, "rhs2");
   TORCH_CHECK(lhs1.sizes() == lhs2.sizes() && rhs1.sizes() == rhs2.sizes(),
               "FusedUOPV: the two operand pairs must have equal shapes");
+  TORCH_CHECK(out1.defined() && out2.defined() && out1.is_cuda() && out2.is_cuda() &&
+                  out1.is_contiguous() && out2.is_contiguous() &&
+                  out1.scalar_type() == out2.scalar_type(),
+              "FusedUOPV: outputs must be contiguous GPU tensors of one type");
+  need_rows(lhs1, num_rows_, "FusedUOPV", "lhs");
+  need_rows(rhs1, num_cols_, "FusedUOPV", "rhs");
+  same_dtype(lhs1, out1, "FusedUOPV", "lhs1");
+  same_dtype(rhs1, out1, "FusedUOPV", "rhs1");
+  same_dtype(lhs2, out1, "FusedUOPV", "lhs2");
+  same_dtype(rhs2, out1, "FusedUOPV", "rhs2");
   const Broadcast bc = make_broadcast(op, lhs1, rhs1, out1);
+  TORCH_CHECK(out1.numel() >= num_edges_ * bc.out_len && out2.numel() >= num_edges_ * bc.out_len,
+              "FusedUOPV: outputs are too small for ", num_edges_, " edges");
   const StructureArgs s = on_format == kCOO ? structure_of(*coo_)
                                             : structure_of(compressed(kCSC));
   GS_CALL(gs_fused_u_op_v(s.format, s.a, s.b, s.num_major, s.nnz, op_code(op),
@@ -191,6 +229,22 @@ static torch::Tensor reduce_workspace(const StructureArgs& s,
   return new_workspace(gs_spmm_workspace_bytes(s.format, s.nnz, out.size(0)), out);
 }
 
+// Shapes and types of a reduction's operands: u features per source node,
+// e features per edge, one output row per target node, all float32.
+void Graph::check_reduce_operands(const std::string& op, const torch::Tensor& ufeat,
+                                  const torch::Tensor& efeat, const torch::Tensor& out,
+                                  int64_t u_target, const char* who) const {
+  TORCH_CHECK(u_target == 0 || u_target == 2, who, ": invalid u_target ", u_target);
+  TORCH_CHECK(out.defined() && out.is_cuda() && out.is_contiguous() && out.dim() >= 1 &&
+                  out.scalar_type() == torch::kFloat32,
+              who, ": out must be a contiguous float32 GPU tensor");
+  if (op != "copy_rhs") need_rows(ufeat, u_target == 0 ? num_rows_ : num_cols_, who, "ufeat");
+  if (op != "copy_lhs") need_rows(efeat, num_edges_, who, "efeat");
+  need_rows(out, u_target == 0 ? num_cols_ : num_rows_, who, "out");
+  same_dtype(ufeat, out, who, "ufeat");
+  same_dtype(efeat, out, who, "efeat");
+}
+
 void Graph::SpMM(const std::string& op, const std::string& reduce,
                  torch::Tensor ufeat, torch::Tensor efeat, torch::Tensor out,
                  torch::Tensor argu, torch::Tensor arge, int64_t u_target,
@@ -204,7 +258,14 @@ void Graph::SpMM(const std::string& op, const std::string& reduce,
   TORCH_CHECK(out.defined() && out.is_cuda() && out.is_contiguous() &&
                   out.scalar_type() == torch::kFloat32,
               "SpMM: out must be a contiguous float32 GPU tensor");
+  check_reduce_operands(op, ufeat, efeat, out, u_target, "SpMM");
   const Broadcast bc = make_broadcast(op, ufeat, efeat, out);
+  TORCH_CHECK(out.numel() >= out.size(0) * bc.out_len, "SpMM: out is too small");
+  for (const torch::Tensor* arg : {&argu, &arge})
+    TORCH_CHECK(!arg->defined() || arg->numel() == 0 ||
+                    (arg->is_cuda() && arg->scalar_type() == torch::kInt64 &&
+                     arg->numel() >= out.size(0) * bc.out_len),
+                "SpMM: arg tensors must be int64 GPU tensors as large as out");
   const StructureArgs s = reduce_structure(
       *this, coo_.get(), on_format == kCOO ? nullptr : &compressed(on_format),
       on_format, u_target, "SpMM");
@@ -231,8 +292,10 @@ void Graph::FusedESquareSum(const std::string& op, const std::string& reduce,
   TORCH_CHECK(efeat.scalar_type() == torch::kFloat32 &&
                   out.scalar_type() == torch::kFloat32,
               "FusedESquareSum needs float32 tensors");
+  check_reduce_operands("copy_rhs", torch::Tensor(), efeat, out, u_target, "FusedESquareSum");
   int64_t len = 1;
   for (int64_t i = 1; i < efeat.dim(); ++i) len *= efeat.size(i);
+  TORCH_CHECK(out.numel() >= out.size(0) * len, "FusedESquareSum: out is too small");
   const StructureArgs s = reduce_structure(
       *this, coo_.get(), on_format == kCOO ? nullptr : &compressed(on_format),
       on_format, u_target, "FusedESquareSum");
@@ -257,8 +320,12 @@ void Graph::FusedEDivUSum(const std::string& op, const std::string& reduce,
                   ufeat.scalar_type() == torch::kFloat32 &&
                   out.scalar_type() == torch::kFloat32,
               "FusedEDivUSum needs float32 tensors");
+  check_reduce_operands("div", ufeat, efeat, out, u_target, "FusedEDivUSum");
   int64_t len = 1;
   for (int64_t i = 1; i < efeat.dim(); ++i) len *= efeat.size(i);
+  TORCH_CHECK(ufeat.numel() / std::max<int64_t>(ufeat.size(0), 1) == len,
+              "FusedEDivUSum: ufeat and efeat must have the same feature length");
+  TORCH_CHECK(out.numel() >= out.size(0) * len, "FusedEDivUSum: out is too small");
   const StructureArgs s = reduce_structure(
       *this, coo_.get(), on_format == kCOO ? nullptr : &compressed(on_format),
       on_format, u_target, "FusedEDivUSum");

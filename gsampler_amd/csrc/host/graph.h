@@ -207,6 +207,9 @@ class Graph : public torch::CustomClassHolder {
   const Compressed& compressed(int64_t format);
   // CDF of edge_probs in the edge order of `format` (cached per weights tensor).
   torch::Tensor weight_cdf_for(const torch::Tensor& edge_probs, int64_t format);
+  void check_reduce_operands(const std::string& op, const torch::Tensor& ufeat,
+                             const torch::Tensor& efeat, const torch::Tensor& out,
+                             int64_t u_target, const char* who) const;
   torch::Tensor cdf_, cdf_probs_;
   int64_t cdf_version_ = -1, cdf_format_ = 0;
   torch::Tensor mapped_rows(const torch::Tensor& base, const torch::Tensor& row_ids);

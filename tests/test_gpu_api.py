@@ -144,3 +144,40 @@ def test_errors_are_exceptions_not_aborts(graph):
         m._graph._CAPI_Slicing(torch.arange(3, device=DEV), 1, gs._CSC, gs._CSR)
     with pytest.raises(RuntimeError, match="not implemented"):
         m._graph._CAPI_Sampling(0, 3, False, gs._CSC, gs._COO)
+
+
+def test_edge_operators_reject_operands_that_would_be_read_out_of_bounds(graph):
+    """Feature tensors shorter than the axis they are indexed by, outputs that
+    are too small and mixed element types raise before any kernel runs."""
+    m, _, _ = graph
+    sub = m[:, torch.arange(0, 300, device=DEV)]
+    g = sub._graph
+    R, C, E = g._CAPI_GetNumRows(), g._CAPI_GetNumCols(), g._CAPI_GetNumEdges()
+    f = lambda n, dtype=torch.float32: torch.ones(n, device=DEV, dtype=dtype)
+    out_e, out_c = f(E), torch.zeros(C, device=DEV)
+    with pytest.raises(RuntimeError, match="lhs has"):
+        g._CAPI_SDDMM("mul", f(R - 1), f(C), out_e, 0, 2, gs._COO)
+    with pytest.raises(RuntimeError, match="rhs has"):
+        g._CAPI_SDDMM("mul", f(R), f(C - 1), out_e, 0, 2, gs._CSC)
+    with pytest.raises(RuntimeError, match="out has"):
+        g._CAPI_SDDMM("mul", f(R), f(C), f(E - 1), 0, 2, gs._COO)
+    with pytest.raises(RuntimeError, match="but out is"):
+        g._CAPI_SDDMM("mul", f(R, torch.float64), f(C), out_e, 0, 2, gs._COO)
+    with pytest.raises(RuntimeError, match="targets"):
+        g._CAPI_SDDMM("mul", f(R), f(C), out_e, 0, 3, gs._COO)
+    with pytest.raises(RuntimeError, match="efeat has"):
+        g._CAPI_SpMM("copy_rhs", "sum", None, f(E - 1), out_c, None, None, 0, gs._CSC)
+    with pytest.raises(RuntimeError, match="ufeat has"):
+        g._CAPI_SpMM("mul", "sum", f(R - 1), f(E), out_c, None, None, 0, gs._CSC)
+    with pytest.raises(RuntimeError, match="out has"):
+        g._CAPI_SpMM("copy_rhs", "sum", None, f(E), out_c[:-1].contiguous(), None, None, 0, gs._CSC)
+    with pytest.raises(RuntimeError, match="efeat has"):
+        g._CAPI_FusedESquareSum("copy_rhs", "sum", None, f(E - 1), out_c, None, None, 0, gs._CSC)
+    with pytest.raises(RuntimeError, match="ufeat has"):
+        g._CAPI_FusedEDivUSum("div", "sum", f(R - 1), f(E), out_c, None, None, 0, gs._CSC)
+    with pytest.raises(RuntimeError, match="lhs has"):
+        g._CAPI_FusedUOPV("mul", f(R - 1), f(C), f(E), f(R - 1), f(C), f(E), gs._COO)
+    # and the well-formed calls still work
+    g._CAPI_SDDMM("mul", f(R), f(C), out_e, 0, 2, gs._COO)
+    g._CAPI_SpMM("copy_rhs", "sum", None, f(E), out_c, None, None, 0, gs._CSC)
+    assert float(out_c.sum()) == pytest.approx(E)
