@@ -17,12 +17,37 @@ RandomState& random_state() {
 static uint64_t next_call_id() { return random_state().next_call++; }
 
 // ------------------------------------------------------------------ loading
+// A loaded matrix is checked once (a few reductions and one read-back): every
+// kernel afterwards trusts offsets and ids, and a malformed array would send
+// its loads out of bounds.  The reference loads without looking
+// (src/graph.h:19-37).
+static void check_ids_below(const torch::Tensor& ids, int64_t bound, const char* who,
+                            const char* name) {
+  if (ids.numel() == 0) return;
+  const int64_t lo = ids.min().item<int64_t>(), hi = ids.max().item<int64_t>();
+  TORCH_CHECK(lo >= 0 && hi < bound, who, ": ", name, " must lie in [0, ", bound,
+              "), found ", lo, " .. ", hi);
+}
+
+static void check_compressed(const torch::Tensor& indptr, const torch::Tensor& indices,
+                             int64_t num_minor, const char* who) {
+  const int64_t first = indptr[0].item<int64_t>();
+  const int64_t last = indptr[indptr.numel() - 1].item<int64_t>();
+  TORCH_CHECK(first == 0 && last == indices.numel(), who, ": indptr must run from 0 to ",
+              indices.numel(), " (the number of indices), found ", first, " .. ", last);
+  if (indptr.numel() > 1)
+    TORCH_CHECK(indptr.slice(0, 1).ge(indptr.slice(0, 0, indptr.numel() - 1)).all().item<bool>(),
+                who, ": indptr must not decrease");
+  check_ids_below(indices, num_minor, who, "indices");
+}
+
 void Graph::LoadCSC(torch::Tensor indptr, torch::Tensor indices) {
   auto m = std::make_shared<Compressed>();
   m->indptr = graph_ids(indptr, "indptr");
   m->indices = graph_ids(indices, "indices");
   TORCH_CHECK(m->indptr.numel() == num_cols_ + 1, "LoadCSC: indptr has ",
               indptr.numel(), " entries for ", num_cols_, " columns");
+  check_compressed(m->indptr, m->indices, num_rows_, "LoadCSC");
   csc_ = m;
   num_edges_ = indices.numel();
 }
@@ -33,6 +58,7 @@ void Graph::LoadCSR(torch::Tensor indptr, torch::Tensor indices) {
   m->indices = graph_ids(indices, "indices");
   TORCH_CHECK(m->indptr.numel() == num_rows_ + 1, "LoadCSR: indptr has ",
               indptr.numel(), " entries for ", num_rows_, " rows");
+  check_compressed(m->indptr, m->indices, num_cols_, "LoadCSR");
   csr_ = m;
   num_edges_ = indices.numel();
 }
@@ -43,6 +69,8 @@ void Graph::LoadCOO(torch::Tensor row, torch::Tensor col, bool row_sorted,
   m->row = graph_ids(row, "row");
   m->col = graph_ids(col, "col");
   TORCH_CHECK(row.numel() == col.numel(), "LoadCOO: row and col differ in length");
+  check_ids_below(m->row, num_rows_, "LoadCOO", "row ids");
+  check_ids_below(m->col, num_cols_, "LoadCOO", "column ids");
   m->row_sorted = row_sorted;
   m->col_sorted = col_sorted;
   coo_ = m;

@@ -181,3 +181,23 @@ def test_edge_operators_reject_operands_that_would_be_read_out_of_bounds(graph):
     g._CAPI_SDDMM("mul", f(R), f(C), out_e, 0, 2, gs._COO)
     g._CAPI_SpMM("copy_rhs", "sum", None, f(E), out_c, None, None, 0, gs._CSC)
     assert float(out_c.sum()) == pytest.approx(E)
+
+
+def test_malformed_matrices_are_refused_at_load():
+    ok_ptr = torch.tensor([0, 2, 2, 5], device=DEV)
+    ok_idx = torch.tensor([0, 3, 1, 2, 3], device=DEV)
+    gs.Graph(4, 3)._CAPI_LoadCSC(ok_ptr, ok_idx)
+    with pytest.raises(RuntimeError, match="entries for"):
+        gs.Graph(4, 4)._CAPI_LoadCSC(ok_ptr, ok_idx)
+    with pytest.raises(RuntimeError, match="must run from 0"):
+        gs.Graph(4, 3)._CAPI_LoadCSC(torch.tensor([0, 2, 2, 6], device=DEV), ok_idx)
+    with pytest.raises(RuntimeError, match="must not decrease"):
+        gs.Graph(4, 3)._CAPI_LoadCSC(torch.tensor([0, 3, 2, 5], device=DEV), ok_idx)
+    with pytest.raises(RuntimeError, match="indices must lie"):
+        gs.Graph(3, 3)._CAPI_LoadCSC(ok_ptr, ok_idx)
+    with pytest.raises(RuntimeError, match="indices must lie"):
+        gs.Graph(4, 3)._CAPI_LoadCSR(torch.tensor([0, 2, 2, 4, 5], device=DEV), ok_idx)
+    with pytest.raises(RuntimeError, match="column ids"):
+        gs.Graph(4, 3)._CAPI_LoadCOO(ok_idx, torch.tensor([0, 0, 2, 2, 3], device=DEV), False, False)
+    with pytest.raises(RuntimeError, match="row ids"):
+        gs.Graph(4, 3)._CAPI_LoadCOO(ok_idx - 1, torch.tensor([0, 0, 2, 2, 2], device=DEV), False, False)
