@@ -206,6 +206,60 @@ class OffsetMirror {
   }
 };
 
+// Batch pointer arrays (int64[B + 1] offsets into a concatenation) reach the
+// kernels unchecked, so one that a caller supplies is looked at on the host
+// first: it must start at 0, never decrease and end at the length it splits.
+// Arrays that this library's own operators produced are remembered and skip
+// the check (and the device read-back it costs); a caller's array is read back
+// once and then found in the mirror while it stays unchanged.
+class BatchOffsets {
+ public:
+  static void trust(const torch::Tensor& offsets) {
+    if (!offsets.defined()) return;
+    Known& k = ring()[next()++ % kEntries];
+    k.impl = offsets.unsafeGetTensorImpl();
+    k.data = offsets.numel() ? offsets.data_ptr() : nullptr;
+    k.version = (int64_t)offsets._version();
+    k.numel = offsets.numel();
+  }
+  static void check(const torch::Tensor& offsets, int64_t total, const char* who) {
+    TORCH_CHECK(offsets.defined() && offsets.scalar_type() == torch::kInt64 &&
+                    offsets.dim() == 1 && offsets.numel() >= 2,
+                who, ": batch offsets must be an int64 vector with at least two entries");
+    if (trusted(offsets)) return;
+    const std::vector<int64_t>& p = OffsetMirror::values(offsets);
+    bool ok = p.front() == 0 && p.back() == total;
+    for (size_t i = 1; ok && i < p.size(); ++i) ok = p[i] >= p[i - 1];
+    TORCH_CHECK(ok, who, ": batch offsets must start at 0, never decrease and end at ",
+                total, " (found ", p.front(), " .. ", p.back(), ")");
+    trust(offsets);
+  }
+
+ private:
+  struct Known {
+    const void* impl = nullptr;
+    const void* data = nullptr;
+    int64_t version = -1, numel = -1;
+  };
+  static constexpr size_t kEntries = 32;
+  static std::vector<Known>& ring() {
+    static thread_local std::vector<Known> r(kEntries);
+    return r;
+  }
+  static size_t& next() {
+    static thread_local size_t n = 0;
+    return n;
+  }
+  static bool trusted(const torch::Tensor& t) {
+    const void* data = t.numel() ? t.data_ptr() : nullptr;
+    for (const Known& k : ring())
+      if (k.impl == t.unsafeGetTensorImpl() && k.data == data &&
+          k.version == (int64_t)t._version() && k.numel == t.numel())
+        return true;
+    return false;
+  }
+};
+
 // Outputs are sized by an upper bound (and trimmed afterwards) only up to this
 // many elements; beyond it the count is awaited first.
 constexpr int64_t kBoundLimit = int64_t(1) << 26;

@@ -15,8 +15,10 @@ void Graph::copy_batch_state_to(Graph& g, bool with_rows) {
     g.orig_row_ids_ = orig_row_ids_;
   }
   g.row_encoding_size_ = row_encoding_size_;
-  if (g.csc_ && col_bptr_.defined())
+  if (g.csc_ && col_bptr_.defined()) {
     g.edge_bptr_ = g.csc_->indptr.index_select(0, col_bptr_);
+    BatchOffsets::trust(g.edge_bptr_);
+  }
 }
 
 std::tuple<torch::Tensor, torch::Tensor> Graph::BatchGetCSCIndptr() {
@@ -82,6 +84,7 @@ GraphAndIndex Graph::BatchColSlicing(torch::Tensor seeds, torch::Tensor col_bptr
   col_bptr = ids(col_bptr, "col_bptr");
   const int64_t B = col_bptr.numel() - 1;
   TORCH_CHECK(B >= 1, "BatchColSlicing: col_bptr needs at least two entries");
+  BatchOffsets::check(col_bptr, seeds.numel(), "BatchColSlicing");
   const Compressed& m = compressed(kCSC);
   const int64_t stride = num_rows_;
   MajorResult r = major_slice(m, seeds, true, col_bptr, encoding ? stride : 0);
@@ -92,12 +95,14 @@ GraphAndIndex Graph::BatchColSlicing(torch::Tensor seeds, torch::Tensor col_bptr
                                 /*return_inverse=*/true, /*return_counts=*/false);
     r.minor_ids = std::get<1>(uniq);
     std::tie(row_bptr, orig_rows) = batch_offsets(std::get<0>(uniq), B, stride);
+    BatchOffsets::trust(row_bptr);
   }
   const int64_t new_rows = encoding ? orig_rows.numel() : num_rows_ * B;
   GraphPtr g = derive(kCSC, kCSC | kCOO, r, new_rows, seeds.numel());
   g->col_bptr_ = col_bptr;
   g->orig_col_ids_ = seeds;
   g->edge_bptr_ = r.indptr.index_select(0, col_bptr);
+  BatchOffsets::trust(g->edge_bptr_);
   if (encoding) {
     g->row_bptr_ = row_bptr;
     g->orig_row_ids_ = orig_rows;
@@ -108,6 +113,7 @@ GraphAndIndex Graph::BatchColSlicing(torch::Tensor seeds, torch::Tensor col_bptr
 
 GraphAndIndex Graph::BatchRowSlicing(torch::Tensor row_ids,
                                      torch::Tensor row_bptr) {
+  BatchOffsets::check(ids(row_bptr, "row_bptr"), row_ids.numel(), "BatchRowSlicing");
   auto ret = Slicing(row_ids, 0, kCSC, kCSC | kCOO);
   Graph& g = *std::get<0>(ret);
   copy_batch_state_to(g, false);
@@ -135,11 +141,13 @@ GraphAndIndex Graph::BatchFusedSlicingSampling(torch::Tensor seeds,
                                                torch::Tensor col_bptr,
                                                int64_t fanout, bool replace) {
   col_bptr = ids(col_bptr, "col_bptr");
+  BatchOffsets::check(col_bptr, seeds.numel(), "BatchFusedSlicingSampling");
   auto ret = FusedSlicingSampling(1, seeds, fanout, replace, kCSC, kCSC | kCOO);
   Graph& g = *std::get<0>(ret);
   g.col_bptr_ = col_bptr;
   g.orig_col_ids_ = ids(seeds, "seeds");
   g.edge_bptr_ = g.csc_->indptr.index_select(0, col_bptr);
+  BatchOffsets::trust(g.edge_bptr_);
   OffsetMirror::prefetch(g.edge_bptr_);  // per-batch splits will ask for it
   return ret;
 }

@@ -386,6 +386,7 @@ Graph::Frontier& Graph::frontier_for(const torch::Tensor& seeds,
                           f->workspace.data_ptr(), f->workspace.numel(),
                           cur_stream()));
   f->count = AsyncCount(f->unique_ptr);
+  BatchOffsets::trust(f->unique_ptr);
   if (B > 1) OffsetMirror::prefetch(f->unique_ptr);  // per-batch splits will ask for it
   // at most S + E unique keys
   f->unique_buffer =

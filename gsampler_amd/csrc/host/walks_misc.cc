@@ -113,6 +113,8 @@ GraphAndIndex Graph::BatchColRowSlcing(torch::Tensor col, torch::Tensor col_bptr
   row_bptr = ids(row_bptr, "row_bptr");
   TORCH_CHECK(col_bptr.numel() == row_bptr.numel() && col_bptr.numel() >= 2,
               "BatchColRowSlcing: column and row batch pointers must have the same length");
+  BatchOffsets::check(col_bptr, col.numel(), "BatchColRowSlicing");
+  BatchOffsets::check(row_bptr, row.numel(), "BatchColRowSlicing");
   const Compressed& m = compressed(kCSC);
   const int64_t stride = num_rows_;
   // batched column slice with rows encoded as id + batch * num_rows ...
@@ -135,6 +137,7 @@ GraphAndIndex Graph::BatchColRowSlcing(torch::Tensor col, torch::Tensor col_bptr
   g->orig_col_ids_ = col;
   g->orig_row_ids_ = row;
   g->edge_bptr_ = kept.indptr.index_select(0, col_bptr);
+  BatchOffsets::trust(g->edge_bptr_);
   torch::Tensor select = sliced.select.index_select(0, kept.select);
   return {g, edge_index(m.e_ids, select)};
 }

@@ -130,12 +130,14 @@ GraphAndIndex Graph::BatchFusedSlicingSamplingProbs(torch::Tensor seeds,
                                                     torch::Tensor edge_probs,
                                                     int64_t fanout, bool replace) {
   col_bptr = ids(col_bptr, "col_bptr");
+  BatchOffsets::check(col_bptr, seeds.numel(), "BatchFusedSlicingSamplingProbs");
   auto ret = FusedSlicingSamplingProbs(1, seeds, edge_probs, fanout, replace, kCSC,
                                        kCSC | kCOO);
   Graph& g = *std::get<0>(ret);
   g.col_bptr_ = col_bptr;
   g.orig_col_ids_ = ids(seeds, "seeds");
   g.edge_bptr_ = g.csc_->indptr.index_select(0, col_bptr);
+  BatchOffsets::trust(g.edge_bptr_);
   OffsetMirror::prefetch(g.edge_bptr_);
   return ret;
 }
@@ -162,11 +164,13 @@ static std::tuple<torch::Tensor, torch::Tensor> list_weighted(
   const int64_t n = probs.numel();
   const int64_t nseg = range.defined() ? range.numel() - 1 : 1;
   TORCH_CHECK(nseg >= 1, "list sampling: range needs at least two entries");
+  if (range.defined()) BatchOffsets::check(range, n, "list sampling");
   torch::Tensor ws = new_workspace(gs_list_sample_workspace_bytes(n, nseg), probs);
   torch::Tensor out_range = new_ids(nseg + 1, probs);
   GS_CALL(gs_list_sample_weighted_count(cptr(range), n, nseg, num_picks,
                                         replace ? 1 : 0, mptr(out_range),
                                         ws.data_ptr(), ws.numel(), cur_stream()));
+  BatchOffsets::trust(out_range);
   const int64_t total = read_last(out_range);
   torch::Tensor out = new_ids(total, probs);
   const RandomState& rs = random_state();

@@ -201,3 +201,28 @@ def test_malformed_matrices_are_refused_at_load():
         gs.Graph(4, 3)._CAPI_LoadCOO(ok_idx, torch.tensor([0, 0, 2, 2, 3], device=DEV), False, False)
     with pytest.raises(RuntimeError, match="row ids"):
         gs.Graph(4, 3)._CAPI_LoadCOO(ok_idx - 1, torch.tensor([0, 0, 2, 2, 2], device=DEV), False, False)
+
+
+def test_batch_offsets_from_the_caller_are_checked(graph):
+    m, _, _ = graph
+    g = m._graph
+    seeds = torch.arange(0, 600, device=DEV)
+    good = torch.tensor([0, 200, 200, 600], device=DEV)
+    g._CAPI_BatchFusedSlicingSampling(seeds, good, 5, False)
+    for bad in ([0, 200, 700], [0, 300, 200, 600], [1, 200, 600], [0, 200, 500]):
+        ptr = torch.tensor(bad, device=DEV)
+        with pytest.raises(RuntimeError, match="batch offsets"):
+            g._CAPI_BatchFusedSlicingSampling(seeds, ptr, 5, False)
+        with pytest.raises(RuntimeError, match="batch offsets"):
+            g._CAPI_BatchColSlicing(seeds, ptr, True)
+        with pytest.raises(RuntimeError, match="batch offsets"):
+            torch.ops.gs_ops._CAPI_BatchListSamplingWithProbs(
+                torch.ones(600, device=DEV), 4, False, ptr)
+    with pytest.raises(RuntimeError, match="batch offsets"):
+        g._CAPI_BatchColRowSlcing(seeds, good, seeds, torch.tensor([0, 100, 200, 601], device=DEV))
+    # an array changed in place after it was accepted is looked at again
+    ptr = good.clone()
+    g._CAPI_BatchFusedSlicingSampling(seeds, ptr, 5, False)
+    ptr[3] = 900
+    with pytest.raises(RuntimeError, match="batch offsets"):
+        g._CAPI_BatchFusedSlicingSampling(seeds, ptr, 5, False)
