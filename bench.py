@@ -48,6 +48,11 @@ WORKLOADS = {
                 desc="weighted GraphSAGE [15,10,5] (fp32 edge weights LogNormal(0,1), persistent CDF), 64 batches x "
                      "1024 seeds, on c2's graph: a 1/13-scale stand-in for the 1.6B-edge weighted "
                      "configuration"),
+    "c5": dict(nodes=111_000_000, edges=1_600_000_000, gen="chung_lu", batches=128,
+               batch_size=1024, fanouts=[15, 10, 5], weighted=True,
+               desc="large-graph weighted GraphSAGE [15,10,5] (fp32 edge weights LogNormal(0,1), "
+                    "persistent CDF), 128 batches x 1024 seeds, Chung-Lu power-law (exp 2.1) "
+                    "111M nodes / 1.6B edges, CSC int64, all resident in HBM"),
     "gather": dict(kind="gather", nodes=2_450_000, edges=124_000_000, gen="chung_lu", batches=64,
                    batch_size=1024, fanouts=[15, 10, 5], feat=128,
                    desc="feature fetch for the input nodes of one c2 step: fp32 features "

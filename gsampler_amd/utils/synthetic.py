@@ -23,6 +23,10 @@ def coo_to_csc(row: torch.Tensor, col: torch.Tensor, num_nodes: int,
                sort_rows: bool = False) -> Tuple[torch.Tensor, torch.Tensor]:
     """(indptr[num_nodes + 1], indices[E]); rows inside a column are sorted
     when sort_rows is set (what node2vec's connectivity test needs)."""
+    if row.is_cuda and not sort_rows:
+        from .. import capi  # the library's own edge-list ingest (stable sort by column)
+        indptr, indices, _ = capi.coo_to_csc(row, col, num_nodes)
+        return indptr, indices
     if sort_rows:
         order = torch.argsort(col * num_nodes + row)
     else:

@@ -149,3 +149,51 @@ def test_node2vec_walks(graph):
     want = orc.node2vec(indptr.cpu().numpy(), indices.cpu().numpy(), start.cpu().numpy(),
                         length, 2.0, 0.5, 7777, 0)
     assert np.array_equal(trace.cpu().numpy(), want)
+
+
+def test_largest_configuration_weighted_layers():
+    """111 M nodes, 1.6 B edges (13 GB of int64 indices, positions beyond 2^30,
+    a CDF whose prefix sums pass 2^61): edge-list ingest, CDF build and two
+    weighted layers of 128 x 1024 seeds, checked through properties on the
+    device."""
+    from gsampler_amd.utils import batched_seeds, chung_lu_csc
+    dev = torch.device("cuda:0")
+    nodes, edges = 111_000_000, 1_600_000_000
+    indptr, indices = chung_lu_csc(nodes, edges, seed=1, device=dev)
+    assert int(indptr[-1]) == edges and indices.numel() == edges
+    assert bool((indptr[1:] >= indptr[:-1]).all())
+    assert int(indices.min()) >= 0 and int(indices.max()) < nodes
+    g = torch.Generator(device=dev)
+    g.manual_seed(5)
+    probs = torch.empty(edges, device=dev).normal_(generator=g).exp_()
+    cdf = capi.weight_cdf(indptr, probs)
+    assert bool((cdf[1:] >= cdf[:-1]).all()) and int(cdf[0]) == 0
+    # a column's largest weight quantises to 2^31 (spot check on some columns)
+    for c in (0, 1, 77, 1_000_000, nodes - 1):
+        lo, hi = int(indptr[c]), int(indptr[c + 1])
+        if hi > lo:
+            steps = cdf[lo + 1:hi + 1] - cdf[lo:hi]
+            assert int(steps.max()) == 2 ** 31
+            assert int(torch.argmax(steps)) == int(torch.argmax(probs[lo:hi]))
+    seeds, ptr = batched_seeds(nodes, 128, 1024, seed=2, device=dev)
+
+    def check(seeds, fanout, out):
+        sub_indptr, coo_col, rows, sel = out
+        deg = indptr[seeds + 1] - indptr[seeds]
+        assert torch.equal(sub_indptr[1:] - sub_indptr[:-1], deg.clamp(max=fanout))
+        col = seeds[coo_col]
+        assert bool(((sel >= indptr[col]) & (sel < indptr[col + 1])).all())
+        assert torch.equal(rows, indices[sel])
+        assert torch.unique(coo_col * edges + sel).numel() == sel.numel()
+        # positive weights only, unless the column has fewer than fanout of them
+        zero = probs[sel] <= 0
+        assert int(zero.sum()) == 0
+
+    out = capi.sample_weighted(indptr, indices, probs, seeds, 15, False, 7777, 0, cdf=cdf)
+    check(seeds, 15, out)
+    rel = capi.unique_relabel(seeds, out[2], ptr, out[0][ptr], out[1])
+    assert torch.equal(rel[0][rel[1][:-1].unsqueeze(1) + torch.arange(1024, device=dev)].flatten(),
+                       seeds)
+    out2 = capi.sample_weighted(indptr, indices, probs, rel[0], 10, False, 7777, 1, cdf=cdf)
+    check(rel[0], 10, out2)
+    assert out2[2].numel() > 4_000_000
