@@ -129,7 +129,10 @@ def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
 
 
 def _stream() -> int:
-    return torch.cuda.current_stream().cuda_stream
+    """Raw handle of torch's current stream on the current device (the direct
+    binding: torch.cuda.current_stream() spends microseconds in Python per call,
+    which a step of a few dozen launches notices)."""
+    return torch._C._cuda_getCurrentRawStream(torch._C._cuda_getDevice())
 
 
 def _i64t(t: torch.Tensor, name: str) -> torch.Tensor:
