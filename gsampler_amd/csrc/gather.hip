@@ -52,6 +52,37 @@ __global__ __launch_bounds__(kBlock) void gather_rows_kernel(
   }
 }
 
+// Rows of a single vector (edge data, labels, id arrays): consecutive lanes take
+// consecutive output positions, kGatherRows of them per thread a block apart,
+// so that stores and the id loads are coalesced.
+template <typename V>
+__global__ __launch_bounds__(kBlock) void gather_scalar_kernel(
+    const V* __restrict__ table, int64_t num_rows, const int64_t* __restrict__ ids,
+    int64_t n, V* __restrict__ out, unsigned long long* bad_count) {
+  const int64_t base = (int64_t)blockIdx.x * (kBlock * kGatherRows) + threadIdx.x;
+  int64_t id[kGatherRows];
+#pragma unroll
+  for (int u = 0; u < kGatherRows; ++u) {
+    const int64_t i = base + u * kBlock;
+    id[u] = i < n ? ids[i] : 0;
+  }
+  V v[kGatherRows];
+#pragma unroll
+  for (int u = 0; u < kGatherRows; ++u) {
+    const bool ok = id[u] >= 0 && id[u] < num_rows;
+    v[u] = V(0);
+    if (ok)
+      v[u] = table[id[u]];
+    else if (base + u * kBlock < n && bad_count != nullptr)
+      atomicAdd(bad_count, 1ull);
+  }
+#pragma unroll
+  for (int u = 0; u < kGatherRows; ++u) {
+    const int64_t i = base + u * kBlock;
+    if (i < n) __builtin_nontemporal_store(v[u], out + i);
+  }
+}
+
 __global__ void gather_clear_kernel(unsigned long long* bad_count) { *bad_count = 0; }
 
 template <typename V>
@@ -59,6 +90,15 @@ static int gather_launch(const void* table, int64_t num_rows, int64_t row_bytes,
                          const int64_t* ids, int64_t n, void* out,
                          unsigned long long* bad_count, hipStream_t s) {
   const int64_t vpr = row_bytes / (int64_t)sizeof(V);
+  if (vpr == 1) {
+    const int64_t blocks = ceil_div(n, (int64_t)kBlock * kGatherRows);
+    GS_REQUIRE(blocks < ((int64_t)1 << 31), "gather_rows: %lld rows need too many work-groups",
+               (long long)n);
+    GS_LAUNCH("gather_rows", s,
+              gather_scalar_kernel<V><<<dim3((unsigned)blocks), dim3(kBlock), 0, s>>>(
+                  (const V*)table, num_rows, ids, n, (V*)out, bad_count));
+    return GS_OK;
+  }
   int lanes = 1;
   while (lanes < kWave && lanes < vpr) lanes *= 2;
   const int64_t groups = ceil_div(n, (int64_t)kGatherRows);

@@ -12,7 +12,7 @@ from torch.fx import Proxy
 from ..format import _COO, _CSC, _CSR
 from ..ops import gsddmm, gspmm
 from ..utils.block import Block, create_block_from_coo, create_block_from_csc  # noqa: F401
-from ..utils.gather import gather_pinned_tensor_rows
+from ..utils.gather import gather_pinned_tensor_rows, gather_rows
 
 torch.fx.wrap("create_block_from_coo")
 torch.fx.wrap("create_block_from_csc")
@@ -26,6 +26,9 @@ def data_index(data: torch.Tensor, index: torch.Tensor) -> torch.Tensor:
     (python/gs/matrix_api/matrix.py:19-23 of the reference)."""
     if data.is_pinned():
         return gather_pinned_tensor_rows(data, index)
+    if (data.is_cuda and index.is_cuda and index.dtype == torch.int64 and index.dim() == 1
+            and data.dim() >= 1 and data.is_contiguous()):
+        return gather_rows(data, index)      # edge indices come from the operators: in range
     return data[index]
 
 
