@@ -226,3 +226,31 @@ def test_batch_offsets_from_the_caller_are_checked(graph):
     ptr[3] = 900
     with pytest.raises(RuntimeError, match="batch offsets"):
         g._CAPI_BatchFusedSlicingSampling(seeds, ptr, 5, False)
+
+
+def test_operators_follow_the_current_stream(graph):
+    """Everything is launched on torch's current stream (counts travel on it
+    too): a step issued on a side stream of default priority gives the same
+    result as on the default stream, without any device-wide synchronisation in
+    between."""
+    from gsampler_amd import capi
+    m, indptr, indices = graph
+    g_indptr, g_indices = torch.tensor(indptr, device=DEV), torch.tensor(indices, device=DEV)
+    seeds = torch.arange(0, 20000, 7, device=DEV)
+
+    def step():
+        gs.manual_seed(21)
+        sub = m[:, seeds].individual_sampling(10, None, False)
+        block = sub.to_dgl_block()
+        raw = capi.sample_uniform(g_indptr, g_indices, seeds, 10, False, 0, 7777, 3)
+        return sub.all_nodes(), block.row, block.col, raw[2]
+
+    want = step()
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        got = step()
+    side.synchronize()
+    for a, b in zip(got, want):
+        assert torch.equal(a, b)
