@@ -210,6 +210,7 @@ class Graph : public torch::CustomClassHolder {
   void check_reduce_operands(const std::string& op, const torch::Tensor& ufeat,
                              const torch::Tensor& efeat, const torch::Tensor& out,
                              int64_t u_target, const char* who) const;
+  bool csc_sorted_ = false;  // row ids known to be sorted inside every column
   torch::Tensor cdf_, cdf_probs_;
   int64_t cdf_version_ = -1, cdf_format_ = 0;
   torch::Tensor mapped_rows(const torch::Tensor& base, const torch::Tensor& row_ids);

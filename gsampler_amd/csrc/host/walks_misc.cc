@@ -29,6 +29,22 @@ torch::Tensor Graph::Node2Vec(torch::Tensor seeds, int64_t walk_length, double p
   TORCH_CHECK(csc_ != nullptr, "Node2Vec needs the CSC format");
   TORCH_CHECK(walk_length >= 0, "walk_length must be non-negative");
   TORCH_CHECK(p > 0 && q > 0, "Node2Vec: p and q must be positive");
+  // The connectivity test bisects the previous node's column: row ids must be
+  // sorted inside every column.  Looked at once per matrix (one pass over the
+  // edges); the reference walks on unsorted columns without noticing.
+  if (!csc_sorted_) {
+    const torch::Tensor& idx = csc_->indices;
+    const int64_t nnz = idx.numel();
+    if (nnz > 1) {
+      torch::Tensor drop = idx.slice(0, 1).lt(idx.slice(0, 0, nnz - 1));
+      torch::Tensor ends = csc_->indptr.slice(0, 1, num_cols_) - 1;  // last edge of a column
+      ends = ends.masked_select(ends.ge(0).logical_and(ends.lt(nnz - 1)));
+      drop.index_fill_(0, ends.to(drop.device()), false);
+      TORCH_CHECK(!drop.any().item<bool>(),
+                  "Node2Vec needs row ids sorted inside every column: call SortCSCIndices first");
+    }
+    csc_sorted_ = true;
+  }
   seeds = ids(seeds, "seeds");
   const int64_t n = seeds.numel();
   torch::Tensor out = new_ids(n * (walk_length + 1), seeds);
@@ -50,6 +66,7 @@ void Graph::SortCSCIndices() {
                               mptr(sorted), nnz, ws.data_ptr(), ws.numel(),
                               cur_stream()));
   csc_->indices = sorted;
+  csc_sorted_ = true;
   coo_ = nullptr;  // derived formats followed the old edge order
   csr_ = nullptr;
 }

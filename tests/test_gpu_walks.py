@@ -61,6 +61,8 @@ def test_sort_csc_indices_and_matrix_walks(graph):
                           orc.segment_sort(indptr, indices))
     m = gs.Matrix()
     m.load_graph("CSC", [T(indptr), T(indices)])
+    with pytest.raises(RuntimeError, match="SortCSCIndices"):
+        m.node2vec(T(rng.integers(0, 2000, size=5)), 3, 2.0, 0.5)     # unsorted columns
     m._graph._CAPI_SortCSCIndices()
     srt = orc.segment_sort(indptr, indices)
     assert np.array_equal(m.csc[1].cpu().numpy(), srt)
