@@ -90,7 +90,8 @@ class AsyncCount {
   AsyncCount() = default;
   explicit AsyncCount(const torch::Tensor& prefix) {
     Ring& r = ring();
-    slot_ = r.next++ % kSlots;
+    ticket_ = r.next++;
+    slot_ = (int)(ticket_ % kSlots);
     hipStream_t s = (hipStream_t)cur_stream();
     const int64_t* src = prefix.data_ptr<int64_t>() + prefix.numel() - 1;
     check(hipMemcpyAsync(r.words + slot_, src, sizeof(int64_t),
@@ -102,6 +103,9 @@ class AsyncCount {
     TORCH_CHECK(slot_ >= 0, "AsyncCount: nothing was requested");
     Ring& r = ring();
     if (pending_) {
+      // every operator reads its counts before it returns; one left waiting
+      // while kSlots later requests went by would read another request's word
+      TORCH_CHECK(r.next - ticket_ <= (unsigned)kSlots, "AsyncCount: the slot was reused");
       check(hipEventSynchronize(r.events[slot_]));
       value_ = r.words[slot_];
       pending_ = false;
@@ -130,6 +134,7 @@ class AsyncCount {
     return *r;
   }
   int slot_ = -1;
+  unsigned ticket_ = 0;
   bool pending_ = false;
   int64_t value_ = 0;
 };
