@@ -222,10 +222,8 @@ class BatchOffsets {
   static void trust(const torch::Tensor& offsets) {
     if (!offsets.defined()) return;
     Known& k = ring()[next()++ % kEntries];
-    k.impl = offsets.unsafeGetTensorImpl();
-    k.data = offsets.numel() ? offsets.data_ptr() : nullptr;
+    k.tensor = offsets;  // kept alive: neither its address nor its memory can be handed out again
     k.version = (int64_t)offsets._version();
-    k.numel = offsets.numel();
   }
   static void check(const torch::Tensor& offsets, int64_t total, const char* who) {
     TORCH_CHECK(offsets.defined() && offsets.scalar_type() == torch::kInt64 &&
@@ -242,9 +240,8 @@ class BatchOffsets {
 
  private:
   struct Known {
-    const void* impl = nullptr;
-    const void* data = nullptr;
-    int64_t version = -1, numel = -1;
+    torch::Tensor tensor;
+    int64_t version = -1;
   };
   static constexpr size_t kEntries = 32;
   static std::vector<Known>& ring() {
@@ -256,10 +253,8 @@ class BatchOffsets {
     return n;
   }
   static bool trusted(const torch::Tensor& t) {
-    const void* data = t.numel() ? t.data_ptr() : nullptr;
     for (const Known& k : ring())
-      if (k.impl == t.unsafeGetTensorImpl() && k.data == data &&
-          k.version == (int64_t)t._version() && k.numel == t.numel())
+      if (k.tensor.defined() && k.tensor.is_same(t) && k.version == (int64_t)t._version())
         return true;
     return false;
   }
