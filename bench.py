@@ -541,6 +541,12 @@ def main():
                     peak=HBM_PEAK_GBS, unit="GB/s", frac=round(dom["gbs"] / HBM_PEAK_GBS, 4),
                     traffic=traffic, avg_launch_ms=round(dom["avg_ms"], 4),
                     launches=dom["launches"])
+    if traffic and dom["avg_ms"] > 0:
+        # what the memory system actually moved per launch (every request of this
+        # part's L2 to memory is a 128-byte line) over the same duration
+        moved = traffic / (dom["avg_ms"] * 1e-3) / 1e9
+        roofline["traffic_gbs"] = round(moved, 1)
+        roofline["traffic_frac"] = round(moved / HBM_PEAK_GBS, 4)
     pipeline_bytes = sum(40 * S + 56 * E + 8 * U for S, E, U in sizes)
 
     # ---- CPU baseline: the oracle on the first few batches of the same super-batch
