@@ -315,3 +315,39 @@ def test_batch_ladies(world):
             dst = nxt
     for a, b, ids in zip(eager[0], jit[0], parts):     # first layer: the same picks
         same_edge_sets(a, b, ids)
+
+
+def test_compiled_with_compaction_describes_the_same_blocks(world):
+    """must_compact renumbers the rows of every slice densely (the variant the
+    reference's compiler may pick by timing): same edges, same data."""
+    m, feats, adj = world
+    seeds = torch.arange(4, N, 29, device=DEV)
+
+    def ladies(A, seeds, fanouts):
+        blocks = []
+        for K in fanouts:
+            sub = A[:, seeds]
+            sub.edata["p"] = sub.edata["w"] ** 2
+            prob = sub.sum("p", axis=1)
+            picked, index = sub.collective_sampling(K, prob, False)
+            picked = picked.div("w", prob[index], axis=1)
+            picked = picked.div("w", picked.sum("w", axis=0), axis=0)
+            seeds = picked.all_nodes()
+            blocks.append(picked.to_dgl_block(prefetch_edata={"w"}))
+        return seeds, blocks
+
+    plain = gs.jit.compile(func=ladies, args=(m, seeds, [200, 200]))
+    dense = gs.jit.compile(func=ladies, args=(m, seeds, [200, 200]), must_compact=True)
+    gs.manual_seed(8)
+    p_nodes, p_blocks = plain(m, seeds, [200, 200])
+    gs.manual_seed(8)
+    d_nodes, d_blocks = dense(m, seeds, [200, 200])
+    for blocks in (p_blocks, d_blocks):
+        edges_exist(blocks[0], seeds, adj)
+        edges_exist(blocks[1], blocks[0].srcdata["_ID"], adj)
+        for b in blocks:
+            sums = torch.zeros(b.num_dst, device=DEV).index_add_(0, b.col, b.edata["w"])
+            has = torch.bincount(b.col, minlength=b.num_dst) > 0
+            assert torch.allclose(sums[has], torch.ones_like(sums[has]), rtol=1e-4)
+            assert torch.unique(b.srcdata["_ID"][b.row]).numel() <= 200
+    assert p_blocks[0].num_dst == d_blocks[0].num_dst == seeds.numel()
