@@ -6,9 +6,11 @@
 //          wave tests 256 consecutive edges as four coalesced rows whose
 //          ballots are the chunk's flag words and counts the kept ones; scan
 //          of the chunk counts; out_indptr[c] = kept edges before indptr[c].
+//          The count pass also leaves, per chunk, the new ids (positions in
+//          the picked set) of the chunk's kept edges in edge order.
 //   fill : kept edge e goes to its rank (chunk offset + popcounts), edge order
-//          preserved; the small table is looked up again instead of storing a
-//          value per edge.
+//          preserved; its new id comes from the chunk's staged run, so the fill
+//          pass reads neither the ids nor the table again.
 #include "common.h"
 #include "hashtable.h"
 #include "scan.h"
@@ -23,6 +25,7 @@ constexpr int kMemberLdsSlots = 4096;  // tables up to this size are staged in L
 struct MemberWs {
   uint64_t* table;     // [member_table_slots(num_picked)]
   uint64_t* flags;     // [chunks * kMemberWords]
+  uint32_t* staged;    // [chunks * kBlock]: per chunk, the new ids of its kept edges, in order
   int64_t* chunk_off;  // [chunks + 1]
   void* scan_ws;
   size_t scan_ws_bytes;
@@ -43,6 +46,7 @@ static MemberWs carve_member(void* ws, int64_t nnz, int64_t num_picked) {
   w.chunks = ceil_div(nnz > 0 ? nnz : 1, kBlock);
   w.table = c.take<uint64_t>((size_t)member_table_slots(num_picked));
   w.flags = c.take<uint64_t>((size_t)w.chunks * kMemberWords);
+  w.staged = c.take<uint32_t>((size_t)w.chunks * kBlock);
   w.chunk_off = c.take<int64_t>((size_t)w.chunks + 1);
   w.scan_ws_bytes = scan_workspace_bytes(w.chunks + 1);
   w.scan_ws = c.take<char>(w.scan_ws_bytes);
@@ -160,10 +164,12 @@ template <bool kInLds>
 __global__ __launch_bounds__(kMemberThreads) void member_flag_kernel(
     const int64_t* __restrict__ ids, int64_t nnz,
     const uint64_t* __restrict__ global_table, uint32_t cap,
-    uint64_t* __restrict__ flags, int64_t* __restrict__ chunk_count) {
+    uint64_t* __restrict__ flags, int64_t* __restrict__ chunk_count,
+    uint32_t* __restrict__ staged) {
   __shared__ uint32_t lds_keys[kInLds ? kMemberLdsSlots : 1];
-  MemberTable<kInLds, false> table;
-  table.stage(global_table, cap, lds_keys, nullptr);
+  __shared__ uint32_t lds_values[kInLds ? kMemberLdsSlots : 1];
+  MemberTable<kInLds, true> table;
+  table.stage(global_table, cap, lds_keys, lds_values);
   const int64_t num_chunks = ceil_div_dev(nnz, kBlock);
   const int64_t wave = (int64_t)blockIdx.x * (kMemberThreads / kWave) + threadIdx.x / kWave;
   const int lane = lane_id();
@@ -194,6 +200,16 @@ __global__ __launch_bounds__(kMemberThreads) void member_flag_kernel(
     table.find_many(key, slot);
 #pragma unroll
     for (int j = 0; j < kMemberWords; ++j) word[j] = __ballot(slot[j] < cap);
+    {
+      int before = 0;  // kept edges of the chunk in front of this row of 64
+#pragma unroll
+      for (int j = 0; j < kMemberWords; ++j) {
+        if (slot[j] < cap)
+          staged[chunk * kBlock + before + __popcll(word[j] & ((1ull << lane) - 1))] =
+              table.value_at(slot[j]);
+        before += __popcll(word[j]);
+      }
+    }
     if (lane == 0) {
       int total = 0;
 #pragma unroll
@@ -233,63 +249,55 @@ __global__ __launch_bounds__(kBlock) void member_indptr_kernel(
                   : (e >= nnz ? chunk_off[num_chunks] : member_rank_before(e, flags, chunk_off));
 }
 
-template <bool kInLds>
+// Segment of position x given a segment `from` at or before it: a few steps
+// forward, then a search in what is left (a chunk can cross many empty columns).
+__device__ __forceinline__ int64_t segment_from(const int64_t* __restrict__ ptr, int64_t n,
+                                                int64_t from, int64_t x) {
+  int64_t s = from;
+  for (int step = 0; step < 3; ++step) {
+    if (s + 1 >= n || ptr[s + 1] > x) return s;
+    ++s;
+  }
+  return s + segment_of(ptr + s, n - s, x);
+}
+
 __global__ __launch_bounds__(kMemberThreads) void member_fill_kernel(
-    const int64_t* __restrict__ ids, int64_t nnz,
-    const uint64_t* __restrict__ global_table, uint32_t cap,
-    const uint64_t* __restrict__ flags, const int64_t* __restrict__ chunk_off,
-    const int64_t* __restrict__ indptr, int64_t num_major,
-    const int64_t* __restrict__ edge_major, int64_t* __restrict__ out_major,
-    int64_t* __restrict__ out_minor, int64_t* __restrict__ out_select) {
-  __shared__ uint32_t lds_keys[kInLds ? kMemberLdsSlots : 1];
-  __shared__ uint32_t lds_values[kInLds ? kMemberLdsSlots : 1];
-  MemberTable<kInLds, true> table;
-  table.stage(global_table, cap, lds_keys, lds_values);
+    int64_t nnz, const uint64_t* __restrict__ flags, const int64_t* __restrict__ chunk_off,
+    const uint32_t* __restrict__ staged, const int64_t* __restrict__ indptr,
+    int64_t num_major, const int64_t* __restrict__ edge_major,
+    int64_t* __restrict__ out_major, int64_t* __restrict__ out_minor,
+    int64_t* __restrict__ out_select) {
   const int64_t num_chunks = ceil_div_dev(nnz, kBlock);
   const int64_t wave = (int64_t)blockIdx.x * (kMemberThreads / kWave) + threadIdx.x / kWave;
   const int lane = lane_id();
   const int64_t first_chunk = wave * kMemberChunksPerWave;
-  if (first_chunk >= num_chunks) return;
-  // flag words and kept ids of the next chunk are requested ahead
-  uint64_t next_word[kMemberWords];
-  uint32_t next_key[kMemberWords];
-  auto request = [&](int64_t chunk) {
-#pragma unroll
-    for (int j = 0; j < kMemberWords; ++j) next_word[j] = flags[chunk * kMemberWords + j];
-#pragma unroll
-    for (int j = 0; j < kMemberWords; ++j) {
-      const int64_t e = chunk * kBlock + j * kWave + lane;
-      next_key[j] = ((next_word[j] >> lane) & 1ull) ? member_key((uint64_t)ids[e]) : kNoKey;
-    }
-  };
-  request(first_chunk);
+  int64_t seg_cursor = 0;
   for (int c = 0; c < kMemberChunksPerWave; ++c) {
     const int64_t chunk = first_chunk + c;
     if (chunk >= num_chunks) return;
     const int64_t e0 = chunk * kBlock;
     const int64_t e_last = e0 + kBlock - 1 < nnz ? e0 + kBlock - 1 : nnz - 1;
-    // segments the chunk touches (for out_major without edge_major): mostly one
+    uint64_t word[kMemberWords];
+#pragma unroll
+    for (int j = 0; j < kMemberWords; ++j) word[j] = flags[chunk * kMemberWords + j];
+    const int64_t out0 = chunk_off[chunk];
+    // segments the chunk touches (for out_major without edge_major): mostly the
+    // one the previous chunk ended in, so the search starts from there
     int64_t seg_lo = 0, seg_hi = 0;
     if (out_major && !edge_major) {
-      seg_lo = segment_of(indptr, num_major, wave_uniform_first(e0));
-      seg_hi = segment_of(indptr, num_major, wave_uniform_first(e_last));
+      seg_lo = c == 0 ? segment_of(indptr, num_major, wave_uniform_first(e0))
+                      : segment_from(indptr, num_major, seg_cursor, wave_uniform_first(e0));
+      seg_hi = segment_from(indptr, num_major, seg_lo, wave_uniform_first(e_last));
+      seg_cursor = seg_hi;
     }
-    int64_t before = chunk_off[chunk];
-    uint64_t word[kMemberWords];
-    uint32_t key[kMemberWords], slot[kMemberWords];
-#pragma unroll
-    for (int j = 0; j < kMemberWords; ++j) {
-      word[j] = next_word[j];
-      key[j] = next_key[j];
-    }
-    if (c + 1 < kMemberChunksPerWave && chunk + 1 < num_chunks) request(chunk + 1);
-    table.find_many(key, slot);
+    int before = 0;
 #pragma unroll
     for (int j = 0; j < kMemberWords; ++j) {
       const int64_t e = e0 + j * kWave + lane;
       if ((word[j] >> lane) & 1ull) {
-        const int64_t pos = before + __popcll(word[j] & ((1ull << lane) - 1));
-        out_minor[pos] = (int64_t)table.value_at(slot[j] < cap ? slot[j] : 0);
+        const int in_chunk = before + __popcll(word[j] & ((1ull << lane) - 1));
+        const int64_t pos = out0 + in_chunk;
+        out_minor[pos] = (int64_t)staged[chunk * kBlock + in_chunk];
         out_select[pos] = e;
         if (out_major)
           out_major[pos] =
@@ -348,11 +356,11 @@ int gs_minor_slice_count(const int64_t* ids, int64_t nnz, const int64_t* picked,
     if (cap <= (uint64_t)kMemberLdsSlots)
       GS_LAUNCH("member_flag", s,
                 member_flag_kernel<true><<<dim3((unsigned)blocks), dim3(kMemberThreads), 0, s>>>(
-                    ids, nnz, w.table, cap, w.flags, w.chunk_off));
+                    ids, nnz, w.table, cap, w.flags, w.chunk_off, w.staged));
     else
       GS_LAUNCH("member_flag", s,
                 member_flag_kernel<false><<<dim3((unsigned)blocks), dim3(kMemberThreads), 0, s>>>(
-                    ids, nnz, w.table, cap, w.flags, w.chunk_off));
+                    ids, nnz, w.table, cap, w.flags, w.chunk_off, w.staged));
     int rc = exclusive_scan_i64(w.chunk_off, w.chunk_off, w.chunks + 1, w.scan_ws,
                                 w.scan_ws_bytes, s);
     if (rc != GS_OK) return rc;
@@ -385,18 +393,11 @@ int gs_minor_slice_fill(const int64_t* ids, int64_t nnz, int64_t num_picked,
     return GS_ERR_WORKSPACE;
   }
   hipStream_t s = as_stream(stream);
-  const uint32_t cap = (uint32_t)member_table_slots(num_picked);
   const dim3 grid((unsigned)ceil_div(w.chunks, (kMemberThreads / kWave) * kMemberChunksPerWave));
-  if (cap <= (uint64_t)kMemberLdsSlots)
-    GS_LAUNCH("member_fill", s,
-              member_fill_kernel<true><<<grid, dim3(kMemberThreads), 0, s>>>(
-                  ids, nnz, w.table, cap, w.flags, w.chunk_off, indptr, num_major,
-                  edge_major, out_major, out_minor, out_select));
-  else
-    GS_LAUNCH("member_fill", s,
-              member_fill_kernel<false><<<grid, dim3(kMemberThreads), 0, s>>>(
-                  ids, nnz, w.table, cap, w.flags, w.chunk_off, indptr, num_major,
-                  edge_major, out_major, out_minor, out_select));
+  GS_LAUNCH("member_fill", s,
+            member_fill_kernel<<<grid, dim3(kMemberThreads), 0, s>>>(
+                nnz, w.flags, w.chunk_off, w.staged, indptr, num_major, edge_major,
+                out_major, out_minor, out_select));
   return GS_OK;
 }
 
