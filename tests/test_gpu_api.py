@@ -254,3 +254,40 @@ def test_operators_follow_the_current_stream(graph):
     side.synchronize()
     for a, b in zip(got, want):
         assert torch.equal(a, b)
+
+
+def test_super_batch_with_an_empty_batch(graph):
+    """A mini-batch without seeds travels through the super-batched sampler as
+    an empty block; its neighbours are unaffected."""
+    m, _, _ = graph
+    bm = gs.BatchMatrix()
+    bm.load_from_matrix(m, False)
+    first = torch.arange(0, 20000, 101, device=DEV)
+    third = torch.arange(7, 20000, 131, device=DEV)
+    seeds = torch.cat([first, third])
+    ptr = torch.tensor([0, first.numel(), first.numel(), seeds.numel()], device=DEV)
+
+    def sampler(A, seeds, seeds_ptr, fanouts):
+        out = []
+        for k in fanouts:
+            sub = A[:, seeds::seeds_ptr].individual_sampling(k, None, False)
+            seeds, seeds_ptr = sub.all_nodes()
+            out.append(sub.to_dgl_block())
+        return out
+
+    gs.manual_seed(2)
+    eager = sampler(bm, seeds, ptr, [6, 3])
+    compiled = gs.jit.compile(func=sampler, args=(bm, seeds, ptr, [6, 3]))
+    gs.manual_seed(2)
+    jit = compiled(bm, seeds, ptr, [6, 3])
+    for layers in (eager, jit):
+        assert [len(per_batch) for per_batch in layers] == [3, 3]
+        for per_batch in layers:
+            empty = per_batch[1]
+            assert empty.num_edges() == 0 and empty.num_src == 0 and empty.num_dst == 0
+        assert torch.equal(layers[0][0].srcdata["_ID"][: first.numel()], first)
+        assert torch.equal(layers[0][2].srcdata["_ID"][: third.numel()], third)
+    for a, b in zip(eager, jit):
+        for x, y in zip(a, b):
+            assert torch.equal(x.row, y.row) and torch.equal(x.col, y.col)
+            assert torch.equal(x.srcdata["_ID"], y.srcdata["_ID"])
