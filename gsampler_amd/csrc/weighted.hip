@@ -359,27 +359,23 @@ __device__ __forceinline__ int64_t cdf_locate(const int64_t* __restrict__ a,
 
 constexpr int kMaxCdfFanout = 64;
 
-// Independent draws a column may spend before the rare sequential phase.
-__host__ __device__ constexpr int cdf_free_draws(int fanout) { return 2 * fanout + 8; }
-
-// A group of G lanes (G >= fanout without replacement) takes U consecutive
-// columns and walks them through every stage together.  A wavefront advances
-// at the pace of its slowest search (up to 22 dependent probes in a hub column
-// of a power-law graph), which is what bounds this kernel; more columns per
-// group only add to that maximum (U = 2 and 4 measured 30 % and 100 % slower
-// than U = 1 on a 124M-edge graph), so U = 1 is the default.
-// Without replacement: successive weighted sampling, in the form "draw with
-// replacement and skip what was drawn before" -- draws 0, 1, 2, ... are
-// independent points of the whole mass, so a round of G of them is searched by
-// the G lanes at once; the items enter the output in draw order until fanout
-// distinct ones are there.  A column whose mass sits on a few items could
-// repeat for ever, so after cdf_free_draws(fanout) draws the group finishes in step:
-// every further draw takes a point of the mass that is left and maps it past
-// the intervals already taken (kept sorted), which never repeats; when the
-// positive mass runs out, zero-weight items follow in index order.
-// With replacement: one independent point per output slot.
-// Streams: pos = column position, draw = draw index as above.
-template <int G, int U>
+// One lane per requested column.
+// Without replacement: successive weighted sampling.  Draw j takes a uniform
+// point r of the mass that is still there and maps it past the intervals of the
+// items already taken (x = r + the lengths of all taken intervals that start at
+// or before x, found by iterating from x = r), so no draw repeats an item and
+// a column costs exactly fanout searches whatever its weights look like; when
+// the positive mass runs out, zero-weight items follow in index order.
+// An earlier version let a group of lanes search independent points of the
+// whole mass at once and skipped repeats: columns whose degree or effective
+// number of items is close to the fan-out then need several rounds, every round
+// costs the whole wavefront a Philox block and a search per lane, and the
+// bookkeeping of repeats alone was half of the kernel's time.
+// With replacement: one independent point of the whole mass per output slot.
+// Streams: pos = column position, draw = output slot.
+// The taken intervals live in registers: every access runs over all KMAX slots
+// with a predicate instead of indexing.
+template <int KMAX>
 __global__ __launch_bounds__(kBlock) void sample_weighted_cdf_kernel(
     const int64_t* __restrict__ indptr, int64_t num_cols,
     const int64_t* __restrict__ indices, const int64_t* __restrict__ cdf,
@@ -387,198 +383,84 @@ __global__ __launch_bounds__(kBlock) void sample_weighted_cdf_kernel(
     int replace, PhiloxKey key, const int64_t* __restrict__ sub_indptr,
     int64_t* __restrict__ out_coo_col, int64_t* __restrict__ out_indices,
     int64_t* __restrict__ out_select, int mode) {
-  const int lane = threadIdx.x & (G - 1);
-  const int64_t item0 = (((int64_t)blockIdx.x * kBlock + threadIdx.x) / G) * U;
-  if (item0 >= num_items) return;  // whole groups leave together
-  int64_t in_start[U], deg[U], out_start[U], base[U];
-  uint64_t total[U];
-  {
-    int64_t c[U];
-#pragma unroll
-    for (int u = 0; u < U; ++u) {
-      const int64_t item = item0 + u;
-      c[u] = item < num_items ? (column_ids ? column_ids[item] : item) : -1;
-    }
-#pragma unroll
-    for (int u = 0; u < U; ++u) deg[u] = column_degree(indptr, num_cols, c[u], &in_start[u]);
-#pragma unroll
-    for (int u = 0; u < U; ++u) {
-      out_start[u] = deg[u] > 0 ? sub_indptr[item0 + u] : 0;
-      base[u] = deg[u] > 0 ? cdf[in_start[u]] : 0;
-      total[u] = deg[u] > 0 ? (uint64_t)(cdf[in_start[u] + deg[u]] - base[u]) : 0;
-    }
-  }
-  auto emit = [&](int u, int64_t slot, int64_t off) {
-    const int64_t p = in_start[u] + off;
-    out_indices[out_start[u] + slot] = indices ? indices[p] : p;
-    out_select[out_start[u] + slot] = p;
-    if (out_coo_col) out_coo_col[out_start[u] + slot] = item0 + u;
+  const int64_t item = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (item >= num_items) return;
+  const int64_t c = column_ids ? column_ids[item] : item;
+  int64_t in_start;
+  const int64_t deg = column_degree(indptr, num_cols, c, &in_start);
+  if (deg == 0) return;
+  const int64_t out_start = sub_indptr[item];
+  const int64_t* a = cdf + in_start;
+  const int64_t base = a[0];
+  const uint64_t total = (uint64_t)(a[deg] - base);
+  auto emit = [&](int64_t slot, int64_t off) {
+    const int64_t p = in_start + off;
+    out_indices[out_start + slot] = indices ? indices[p] : p;
+    out_select[out_start + slot] = p;
+    if (out_coo_col) out_coo_col[out_start + slot] = item;
   };
-  // U searches in lockstep: all probes of a step are issued before any is used
-  auto locate_all = [&](const bool (&want)[U], const uint64_t (&point)[U], int64_t (&off)[U]) {
-    CdfSearch st[U];
-    bool open = false;
-#pragma unroll
-    for (int u = 0; u < U; ++u) {
-      off[u] = -1;
-      if (want[u]) {
-        st[u].begin(cdf + in_start[u], deg[u], base[u], base[u] + (int64_t)total[u],
-                    base[u] + (int64_t)point[u]);
-        open |= !st[u].done();
-      }
-    }
-    while (open) {
-      int64_t mid[U], v[U];
-#pragma unroll
-      for (int u = 0; u < U; ++u) mid[u] = (want[u] && !st[u].done()) ? st[u].probe_at(mode) : -1;
-#pragma unroll
-      for (int u = 0; u < U; ++u) v[u] = mid[u] >= 0 ? st[u].a[mid[u]] : 0;
-      open = false;
-#pragma unroll
-      for (int u = 0; u < U; ++u) {
-        if (mid[u] >= 0) st[u].narrow(mid[u], v[u]);
-        open |= want[u] && !st[u].done();
-      }
-    }
-#pragma unroll
-    for (int u = 0; u < U; ++u)
-      if (want[u]) off[u] = st[u].lo;
-  };
-
   if (replace) {
-    for (int j0 = 0; j0 < fanout; j0 += G) {
-      const int j = j0 + lane;
-      bool want[U];
-      uint64_t point[U];
-      int64_t off[U];
-#pragma unroll
-      for (int u = 0; u < U; ++u) {
-        want[u] = j < fanout && deg[u] > 0 && total[u] > 0;
-        point[u] = want[u] ? philox_bounded(key, (uint64_t)(item0 + u), (uint64_t)j, total[u]) : 0;
-      }
-      locate_all(want, point, off);
-#pragma unroll
-      for (int u = 0; u < U; ++u)
-        if (j < fanout && deg[u] > 0)
-          emit(u, j, want[u] ? off[u] : deg[u] - 1);  // no positive weight: the last item
+    for (int j = 0; j < fanout; ++j) {
+      int64_t off = deg - 1;  // no positive weight: the last item
+      if (total > 0)
+        off = cdf_locate(a, deg,
+                         base + (int64_t)philox_bounded(key, (uint64_t)item, (uint64_t)j, total),
+                         mode);
+      emit(j, off);
     }
     return;
   }
-
-  const int K = fanout;
-  const int free_draws = cdf_free_draws(K);
-  // this group's lanes inside the wavefront's ballot word
-  const uint64_t group_bits =
-      (G == kWave ? ~0ull : ((1ull << G) - 1)) << (lane_id() & ~(G - 1));
-  int count[U];      // items accepted so far (the same in every lane of the group)
-  int64_t mine[U];   // lane s holds the item of output slot s
-  bool sampling[U];  // columns that need draws at all
-  bool any_open = false;
-#pragma unroll
-  for (int u = 0; u < U; ++u) {
-    count[u] = 0;
-    mine[u] = -1;
-    sampling[u] = deg[u] > K && total[u] > 0;
-    any_open |= sampling[u];
+  if (deg <= fanout) {  // whole column, original order, zero weights included
+    for (int64_t j = 0; j < deg; ++j) emit(j, j);
+    return;
   }
-  for (int first = 0; first < free_draws && any_open; first += G) {
-    const int j = first + lane;
-    bool want[U];
-    uint64_t point[U];
-    int64_t drawn[U];
+  uint64_t start[KMAX];
+  uint32_t len[KMAX];
 #pragma unroll
-    for (int u = 0; u < U; ++u) {
-      want[u] = sampling[u] && count[u] < K && j < free_draws;
-      point[u] = want[u] ? philox_bounded(key, (uint64_t)(item0 + u), (uint64_t)j, total[u]) : 0;
-    }
-    locate_all(want, point, drawn);
-    any_open = false;
-#pragma unroll
-    for (int u = 0; u < U; ++u) {
-      if (!(sampling[u] && count[u] < K)) continue;  // the same in every lane of the group
-      for (int m = 0; m < G; ++m) {  // in draw order
-        const int64_t cand = __shfl(drawn[u], m, G);
-        if (cand < 0 || count[u] >= K) continue;
-        const bool seen = (__ballot(lane < count[u] && mine[u] == cand) & group_bits) != 0;
-        if (!seen) {
-          if (lane == count[u]) mine[u] = cand;
-          ++count[u];
-        }
-      }
-      any_open |= count[u] < K;
-    }
+  for (int i = 0; i < KMAX; ++i) {
+    start[i] = ~0ull;  // never at or before a point
+    len[i] = 0;
   }
+  uint64_t removed = 0;
+  int taken = 0;
+  for (; taken < fanout && removed < total; ++taken) {
+    const uint64_t r = philox_bounded(key, (uint64_t)item, (uint64_t)taken, total - removed);
+    uint64_t x = r;
+    for (int round = 0; round <= taken; ++round) {
+      uint64_t skipped = 0;
 #pragma unroll
-  for (int u = 0; u < U; ++u) {
-    if (deg[u] == 0) continue;
-    if (deg[u] <= K) {  // whole column, original order, zero weights included
-      for (int64_t j = lane; j < deg[u]; j += G) emit(u, j, j);
-      continue;
+      for (int i = 0; i < KMAX; ++i) skipped += start[i] <= x ? len[i] : 0u;
+      if (r + skipped == x) break;
+      x = r + skipped;
     }
-    if (lane < count[u]) emit(u, lane, mine[u]);
-    if (count[u] == K) continue;
-    // The rare rest: every lane of the group walks it in step (the shuffles
-    // below need the whole group), lane 0 writes.  Collect what was taken,
-    // sorted by position in the CDF.
-    const int64_t* a = cdf + in_start[u];
-    uint64_t start[kMaxCdfFanout];
-    uint32_t len[kMaxCdfFanout];
-    uint64_t removed = 0;
-    for (int s2 = 0; s2 < count[u]; ++s2) {
-      const int64_t off = __shfl(mine[u], s2, G);
-      const uint64_t st = (uint64_t)(a[off] - base[u]);
-      int at = s2;
-      for (; at > 0 && start[at - 1] > st; --at) {
-        start[at] = start[at - 1];
-        len[at] = len[at - 1];
+    const int64_t off = cdf_locate(a, deg, base + (int64_t)x, mode);
+    emit(taken, off);
+    const int64_t lo = a[off], hi = a[off + 1];
+#pragma unroll
+    for (int i = 0; i < KMAX; ++i)
+      if (i == taken) {
+        start[i] = (uint64_t)(lo - base);
+        len[i] = (uint32_t)(hi - lo);
       }
-      start[at] = st;
-      len[at] = (uint32_t)(a[off + 1] - a[off]);
-      removed += len[at];
-    }
-    int taken = count[u];
-    for (int d = 0; taken < K && removed < total[u]; ++d, ++taken) {
-      uint64_t r = philox_bounded(key, (uint64_t)(item0 + u), (uint64_t)(free_draws + d),
-                                  total[u] - removed);
-      int at = 0;  // where the new interval goes
-      for (; at < taken && r >= start[at]; ++at) r += len[at];
-      const int64_t off = cdf_locate(a, deg[u], base[u] + (int64_t)r, mode);
-      if (lane == 0) emit(u, taken, off);
-      for (int m = taken; m > at; --m) {
-        start[m] = start[m - 1];
-        len[m] = len[m - 1];
-      }
-      start[at] = (uint64_t)(a[off] - base[u]);
-      len[at] = (uint32_t)(a[off + 1] - a[off]);
-      removed += len[at];
-    }
-    // fewer than fanout items have positive weight: zero-weight items in order
-    for (int64_t off = 0; taken < K && off < deg[u]; ++off)
-      if (a[off + 1] == a[off]) {
-        if (lane == 0) emit(u, taken, off);
-        ++taken;
-      }
+    removed += (uint64_t)(hi - lo);
   }
+  // fewer than fanout items have positive weight: zero-weight items in order
+  for (int64_t off = 0; taken < fanout && off < deg; ++off)
+    if (a[off + 1] == a[off]) emit(taken++, off);
 }
 
-// Columns per group and search mode of the CDF sampler (GS_WCDF_ILP: 1, 2, 4;
-// GS_WCDF_SEARCH: 0 bisection, 1 alternating, 2 interpolation first).  Read once.
-struct CdfTuning {
-  int ilp, mode;
-};
-static CdfTuning cdf_tuning() {
-  static const CdfTuning t = [] {
-    CdfTuning r{1, 2};
-    if (const char* e = getenv("GS_WCDF_ILP")) r.ilp = atoi(e);
-    if (const char* e = getenv("GS_WCDF_SEARCH")) r.mode = atoi(e);
-    r.ilp = r.ilp >= 4 ? 4 : (r.ilp >= 2 ? 2 : 1);
-    if (r.mode < 0 || r.mode > 2) r.mode = 1;
-    return r;
+// Search mode of the CDF sampler (GS_WCDF_SEARCH: 0 bisection, 1 alternating,
+// 2 interpolation first).  Read once.
+static int cdf_search_mode() {
+  static const int mode = [] {
+    int m = 2;
+    if (const char* e = getenv("GS_WCDF_SEARCH")) m = atoi(e);
+    return m < 0 || m > 2 ? 1 : m;
   }();
-  return t;
+  return mode;
 }
 
-template <int G>
+template <int KMAX>
 static int launch_weighted_cdf(const int64_t* indptr, int64_t num_cols,
                                const int64_t* indices, const int64_t* cdf,
                                const int64_t* column_ids, int64_t num_items,
@@ -586,20 +468,11 @@ static int launch_weighted_cdf(const int64_t* indptr, int64_t num_cols,
                                const int64_t* sub_indptr, int64_t* out_coo_col,
                                int64_t* out_indices, int64_t* out_select,
                                hipStream_t s) {
-  const CdfTuning t = cdf_tuning();
-  const int64_t blocks = ceil_div(ceil_div(num_items, t.ilp) * G, kBlock);
-#define GS_CDF_LAUNCH(UU)                                                          \
-  GS_LAUNCH("sample_weighted_cdf", s,                                              \
-            sample_weighted_cdf_kernel<G, UU><<<dim3((unsigned)blocks), dim3(kBlock), 0, s>>>( \
-                indptr, num_cols, indices, cdf, column_ids, num_items, fanout,     \
-                replace, key, sub_indptr, out_coo_col, out_indices, out_select, t.mode))
-  if (t.ilp == 4)
-    GS_CDF_LAUNCH(4);
-  else if (t.ilp == 2)
-    GS_CDF_LAUNCH(2);
-  else
-    GS_CDF_LAUNCH(1);
-#undef GS_CDF_LAUNCH
+  GS_LAUNCH("sample_weighted_cdf", s,
+            sample_weighted_cdf_kernel<KMAX><<<dim3((unsigned)ceil_div(num_items, kBlock)),
+                                               dim3(kBlock), 0, s>>>(
+                indptr, num_cols, indices, cdf, column_ids, num_items, fanout, replace,
+                key, sub_indptr, out_coo_col, out_indices, out_select, cdf_search_mode()));
   return GS_OK;
 }
 
@@ -789,8 +662,8 @@ int gs_weight_cdf_build(const int64_t* indptr, int64_t num_cols, const float* pr
 
 int gs_csc_col_sample_weighted_fill(
     const int64_t* indptr, int64_t num_cols, const int64_t* indices,
-    const float* probs, const int64_t* cdf, const int64_t* column_ids,
-    int64_t num_items,
+    const float* probs, const int64_t* cdf,
+    const int64_t* column_ids, int64_t num_items,
     int64_t fanout, int replace, uint64_t seed, uint64_t call_id,
     const int64_t* sub_indptr, const int64_t* cdf_offsets, void* cdf_scratch,
     int64_t* out_coo_col, int64_t* out_indices, int64_t* out_select,
@@ -812,8 +685,8 @@ int gs_csc_col_sample_weighted_fill(
                (long long)fanout, kMaxCdfFanout);
     GS_REQUIRE(fanout <= INT32_MAX, "sample_weighted: fanout too large");
 #define GS_CDF_ARGS                                                              \
-  indptr, num_cols, indices, cdf, column_ids, num_items, (int)fanout, replace, key, \
-      sub_indptr, out_coo_col, out_indices, out_select, s
+  indptr, num_cols, indices, cdf, column_ids, num_items, (int)fanout, replace, \
+      key, sub_indptr, out_coo_col, out_indices, out_select, s
     if (fanout <= 8) return launch_weighted_cdf<8>(GS_CDF_ARGS);
     if (fanout <= 16) return launch_weighted_cdf<16>(GS_CDF_ARGS);
     if (fanout <= 32) return launch_weighted_cdf<32>(GS_CDF_ARGS);

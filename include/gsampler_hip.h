@@ -166,13 +166,13 @@ int gs_csc_col_sample_uniform_fill(const int64_t* indptr, int64_t num_cols,
  *    may then be NULL, cdf_offsets / cdf_scratch are not used): every draw is
  *    a search in the column's slice of the CDF, O(fanout * log deg) per
  *    column instead of a pass over its weights.  Without replacement
- *    (fanout <= 64) this is successive weighted sampling: draws 0 ..
- *    2*fanout+7 are independent points of the whole mass and an edge already
- *    drawn is skipped; if that leaves slots open, further draws take points of
- *    the mass that is left.  The same distribution as the smallest-keys rule
- *    above, other picks; output in draw order; when fewer than fanout edges
- *    have positive (quantised) weight, zero-weight edges follow in index
- *    order.  Stream: pos = column position, draw = draw index.
+ *    (fanout <= 64) this is successive weighted sampling: draw j takes a
+ *    uniform point of the mass that is left and maps it past the intervals of
+ *    the edges already taken, so a column costs exactly fanout searches.  The
+ *    same distribution as the smallest-keys rule above, other picks; output in
+ *    draw order; when fewer than fanout edges have positive (quantised)
+ *    weight, zero-weight edges follow in index order.  Stream: pos = column
+ *    position, draw = output slot.
  * Stands in for CSCColSamplingProbsCUDA (src/cuda/sampling_probs.cu:268-281).
  * ---------------------------------------------------------------------- */
 /* Persistent integer CDF of a matrix's edge weights, the input of the fast

@@ -974,14 +974,11 @@ void gs_segment_sort_i64_cpu(const int64_t* indptr, int64_t num_segments,
 //  cdf[e] = sum of the quantised weights of all edges before e over the whole
 //  matrix; a column's weights are quantised to 31 bits against the column's
 //  maximum exactly as integer_cdf() does.
-//  Without replacement, deg > fanout: draws 0 .. 2*fanout+7 are independent
-//  uniform points of the whole mass; an item already drawn is skipped (drawing
-//  with replacement and discarding repeats is successive sampling).  If that
-//  does not give fanout items, draw 2*fanout+8+d takes r uniform in the mass
-//  left, walks the intervals already taken in ascending order
-//  (r >= start ? r += len) and picks the item whose interval holds r.  Output
-//  in draw order; when the positive mass runs out, zero-weight items follow in
-//  index order.
+//  Without replacement, deg > fanout: draw d = 0, 1, ... takes r uniform in the
+//  mass that is left, walks the intervals already taken in ascending order
+//  (r >= start ? r += len) and picks the item whose interval holds r -- the
+//  textbook form of successive sampling.  Output in draw order; when the
+//  positive mass runs out, zero-weight items follow in index order.
 //  With replacement: slot j picks the item holding a uniform point of the
 //  total; a column without positive weights gives its last item.
 //  Streams: pos = column position, draw = slot.
@@ -1041,28 +1038,14 @@ extern "C" void gs_csc_col_sample_weighted_cdf_fill_cpu(
       for (int64_t j = 0; j < deg; ++j) emit(j, j);
       continue;
     }
-    // draws 0 .. free-1 are independent points of the whole mass; repeats are
-    // skipped ("with replacement, discarding what was drawn before")
-    const int64_t free_draws = 2 * fanout + 8;
-    std::vector<int64_t> accepted;
-    if (total > 0)
-      for (int64_t j = 0; j < free_draws && (int64_t)accepted.size() < fanout; ++j) {
-        const int64_t off = locate(rng.bounded((uint64_t)i, (uint64_t)j, total));
-        if (std::find(accepted.begin(), accepted.end(), off) == accepted.end())
-          accepted.push_back(off);
-      }
-    int64_t taken = (int64_t)accepted.size();
-    for (int64_t j = 0; j < taken; ++j) emit(j, accepted[(size_t)j]);
-    // the rare rest: points of the mass that is left, mapped past what was taken
+    // Draw d takes a uniform point r of the mass that is left, walks the
+    // intervals already taken in ascending order (r >= start ? r += len) and
+    // picks the item whose interval holds r: no draw repeats an item.
     std::vector<std::pair<uint64_t, uint64_t>> taken_iv;  // (start, len), ascending
     uint64_t removed = 0;
-    for (int64_t off : accepted) {
-      taken_iv.push_back({(uint64_t)(a[off] - a[0]), (uint64_t)(a[off + 1] - a[off])});
-      removed += taken_iv.back().second;
-    }
-    std::sort(taken_iv.begin(), taken_iv.end());
-    for (int64_t d = 0; taken < fanout && removed < total; ++d, ++taken) {
-      uint64_t r = rng.bounded((uint64_t)i, (uint64_t)(free_draws + d), total - removed);
+    int64_t taken = 0;
+    for (; taken < fanout && removed < total; ++taken) {
+      uint64_t r = rng.bounded((uint64_t)i, (uint64_t)taken, total - removed);
       size_t at = 0;
       for (; at < taken_iv.size() && r >= taken_iv[at].first; ++at) r += taken_iv[at].second;
       const int64_t off = locate(r);
