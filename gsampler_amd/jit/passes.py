@@ -13,6 +13,9 @@ hoisting of tensor constants.  Operator rewrites (observable in
                                                   -> _CAPI_BatchFusedSlicingSampling
   fuse_square_and_sum           (e ** 2) summed by a copy_rhs / sum SpMM
                                                   -> _CAPI_FusedESquareSum
+  fuse_div_and_sum              e / u[endpoint] summed onto the other endpoint,
+                                quotient not used otherwise
+                                                  -> _CAPI_FusedEDivUSum
   merge_u_mul_v                 two u-op-v SDDMMs on one matrix
                                                   -> _CAPI_FusedUOPV
   select_formats                deterministic on_format / output_format choice
@@ -300,6 +303,72 @@ def fuse_square_and_sum(gm: fx.GraphModule) -> fx.GraphModule:
         with gm.graph.inserting_before(spmm):
             gm.graph.call_method("_CAPI_FusedESquareSum", args=tuple(new_args))
         gm.graph.erase_node(spmm)
+    return dce(gm)
+
+
+def _is_wrapped(node, name: str) -> bool:
+    return (isinstance(node, fx.Node) and node.op == "call_function"
+            and getattr(node.target, "__name__", "") == name)
+
+
+def fuse_div_and_sum(gm: fx.GraphModule) -> fx.GraphModule:
+    """q = e / u[t] (an SDDMM with targets (e, t), written as a product with
+    the reciprocal by the operator wrappers), then SpMM("copy_rhs", "sum", _, q)
+    onto the other endpoint, q read by nothing else
+        => FusedEDivUSum("div", "sum", u, e, ...): the quotient is never stored.
+    The reference names this pass and leaves it empty
+    (python/gs/jit/optimize.py:372-374)."""
+    from ..ops.fused_op import _before_e_div_u_sum
+    for spmm in list(gm.graph.nodes):
+        if not _is_method(spmm, "_CAPI_SpMM"):
+            continue
+        if spmm.args[1] != "copy_rhs" or spmm.args[2] != "sum":
+            continue
+        quotient, u_target = spmm.args[4], spmm.args[8]
+        v_item = spmm.args[5]
+        if not (_is_wrapped(quotient, "_after_sddmm") and isinstance(v_item, fx.Node)
+                and v_item.target is operator.getitem
+                and _is_wrapped(v_item.args[0], "_before_spmm")):
+            continue
+        before_spmm = v_item.args[0]
+        if set(quotient.users) != {spmm, before_spmm}:
+            continue                      # the quotient itself is wanted as well
+        out_item = quotient.args[0]
+        if not (isinstance(out_item, fx.Node) and out_item.target is operator.getitem
+                and _is_wrapped(out_item.args[0], "_before_sddmm")):
+            continue
+        before_sddmm = out_item.args[0]
+        writers = [n for n in out_item.users if _is_method(n, "_CAPI_SDDMM")]
+        if len(writers) != 1 or set(out_item.users) != {writers[0], quotient}:
+            continue
+        sddmm = writers[0]
+        if not (sddmm.args[0] is spmm.args[0] and sddmm.args[4] is out_item
+                and sddmm.args[5] == 1 and sddmm.args[6] == u_target and u_target in (0, 2)):
+            continue
+        op, e, rhs = before_sddmm.args[1], before_sddmm.args[2], before_sddmm.args[3]
+        if op == "div":
+            u = rhs
+        elif (op == "mul" and isinstance(rhs, fx.Node) and rhs.op == "call_function"
+              and rhs.target is operator.truediv and rhs.args[0] == 1.0):
+            u = rhs.args[1]
+        else:
+            continue
+        # the accumulator's users: the SpMM and the step that squeezes the result
+        finish = [n for n in v_item.users if _is_wrapped(n, "_after_spmm")]
+        if len(finish) != 1 or set(v_item.users) != {spmm, finish[0]}:
+            continue
+        with gm.graph.inserting_before(spmm):
+            parts = gm.graph.call_function(
+                _before_e_div_u_sum,
+                args=(before_spmm.args[0], before_spmm.args[1], e, u, u_target))
+            u2, e2, v, squeeze = (gm.graph.call_function(operator.getitem, args=(parts, i))
+                                  for i in range(4))
+            gm.graph.call_method("_CAPI_FusedEDivUSum",
+                                 args=(spmm.args[0], "div", "sum", u2, e2, v, None, None,
+                                       u_target, spmm.args[9]))
+        finish[0].args = (v, squeeze)
+        gm.graph.erase_node(spmm)
+        gm.graph.erase_node(sddmm)
     return dce(gm)
 
 

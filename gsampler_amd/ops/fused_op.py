@@ -10,7 +10,28 @@ import torch
 from ..format import _COO, _CSC, _CSR
 from ._common import infer_broadcast_shape
 
+torch.fx.wrap("_before_e_div_u_sum")
+
 __all__ = ["fused_u_mul_v", "e_square_sum", "e_div_u_sum"]
+
+
+def _before_e_div_u_sum(num_rows, num_cols, e, u, u_target):
+    """Operands of _CAPI_FusedEDivUSum for the compiled rewrite of
+    `div` followed by `sum`: both with the broadcast feature shape the two
+    separate operators would have produced, and the zero-filled accumulator."""
+    if u.device != e.device:
+        raise ValueError(f"operand devices differ: {u.device} and {e.device}")
+    if u.dtype != e.dtype:
+        raise ValueError(f"operand dtypes differ: {u.dtype} and {e.dtype}")
+    squeeze = e.dim() == 1 and u.dim() == 1
+    e2 = e.unsqueeze(-1) if e.dim() == 1 else e
+    u2 = u.unsqueeze(-1) if u.dim() == 1 else u
+    feat = infer_broadcast_shape("div", tuple(e2.shape[1:]), tuple(u2.shape[1:]))
+    e2 = e2.expand((e2.shape[0],) + feat).contiguous()
+    u2 = u2.expand((u2.shape[0],) + feat).contiguous()
+    n_out = num_cols if u_target == 0 else num_rows
+    v = torch.zeros((n_out,) + feat, dtype=e.dtype, device=e.device)
+    return u2, e2, v, squeeze
 
 
 def fused_u_mul_v(m, lhs1, rhs1, lhs2, rhs2, on_format=_COO):

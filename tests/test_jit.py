@@ -186,6 +186,33 @@ def test_two_u_mul_v_are_merged():
     assert t.count("_CAPI_FusedUOPV") == 1 and "_CAPI_SDDMM" not in t
 
 
+def div_then_sum_sampler(A, seeds, col_scale):
+    sub = A[:, seeds]
+    return sub.div("w", col_scale, axis=0).sum("w", axis=1)
+
+
+def div_then_sum_keeping_the_quotient(A, seeds, col_scale):
+    q = A[:, seeds].div("w", col_scale, axis=0)
+    return q.sum("w", axis=1), q.edata["w"]
+
+
+def div_then_sum_on_the_same_axis(A, seeds, col_scale):
+    return A[:, seeds].div("w", col_scale, axis=0).sum("w", axis=0)
+
+
+def test_div_then_sum_is_fused_when_only_the_sum_is_wanted():
+    m = gs.Matrix(gs.Graph(10, 10))
+    m.edata["w"] = torch.rand(7)
+    args = (m, torch.arange(3), torch.rand(3))
+    t = targets(gs.jit.compile(func=div_then_sum_sampler, args=args).gm)
+    assert t.count("_CAPI_FusedEDivUSum") == 1
+    assert "_CAPI_SDDMM" not in t and "_CAPI_SpMM" not in t
+    for kept in (div_then_sum_keeping_the_quotient, div_then_sum_on_the_same_axis):
+        t = targets(gs.jit.compile(func=kept, args=args).gm)
+        assert "_CAPI_FusedEDivUSum" not in t
+        assert t.count("_CAPI_SDDMM") == 1 and t.count("_CAPI_SpMM") == 1
+
+
 # ------------------------------------------------------------------- on the GPU
 DEV = "cuda:0"
 
@@ -301,6 +328,28 @@ def test_merged_u_mul_v_equals_eager():
     c = gs.jit.compile(func=pass_like_sampler, args=(m, seeds, u, v, u + 1, v + 1))
     assert torch.allclose(c(m, seeds, u, v, u + 1, v + 1),
                           pass_like_sampler(m, seeds, u, v, u + 1, v + 1))
+
+
+@pytest.mark.gpu
+def test_fused_div_then_sum_equals_eager():
+    m = _graph()
+    seeds = torch.arange(0, 900, 3, device=DEV)
+    scale = torch.rand(seeds.numel(), device=DEV) + 0.5
+    want = div_then_sum_sampler(m, seeds, scale)
+    c = gs.jit.compile(func=div_then_sum_sampler, args=(m, seeds, scale))
+    assert "_CAPI_FusedEDivUSum" in targets(c.gm)
+    got = c(m, seeds, scale)
+    assert got.shape == want.shape
+    # eager multiplies by the reciprocal, the fused operator divides, and the row
+    # sums accumulate in another order: 1e-5 relative
+    torch.testing.assert_close(got, want, rtol=1e-5, atol=1e-6)
+    # against float64 arithmetic on the host
+    sub = m[:, seeds]
+    row, col = (t.cpu().numpy() for t in sub.coo[:2])
+    w = sub.edata["w"].double().cpu().numpy()
+    exact = np.zeros(sub._graph._CAPI_GetNumRows())
+    np.add.at(exact, row, w / scale.double().cpu().numpy()[col])
+    assert np.allclose(got.cpu().numpy(), exact, rtol=1e-5, atol=1e-6)
 
 
 @pytest.mark.gpu
