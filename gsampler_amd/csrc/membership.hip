@@ -333,8 +333,10 @@ int gs_minor_slice_count(const int64_t* ids, int64_t nnz, const int64_t* picked,
   GS_REQUIRE((indptr == nullptr) == (out_indptr == nullptr),
              "minor_slice_count: indptr and out_indptr go together");
   GS_REQUIRE(out_indptr || out_total, "minor_slice_count: nothing to write");
-  GS_REQUIRE(num_picked <= (int64_t)kMaxPackedKey,
-             "minor_slice_count: too many picked ids");
+  // positions among the picked ids are 32-bit values and the table (two slots
+  // per id) is addressed with 32-bit arithmetic
+  GS_REQUIRE(num_picked < (int64_t(1) << 30),
+             "minor_slice_count: at most 2^30 - 1 picked ids, got %lld", (long long)num_picked);
   MemberWs w = carve_member(workspace, nnz, num_picked);
   if (workspace == nullptr || workspace_bytes < w.total) {
     set_error("minor_slice workspace too small: %zu < %zu", workspace_bytes, w.total);

@@ -831,6 +831,9 @@ static int check_unique_args(const int64_t* seeds, const int64_t* seeds_ptr,
                              const int64_t* rows_ptr, int64_t E, int64_t B) {
   GS_REQUIRE(S >= 0 && E >= 0, "unique: negative size");
   GS_REQUIRE(B >= 1, "unique: num_batches must be >= 1, got %lld", (long long)B);
+  // positions and ranks inside a batch are kept as 32-bit values
+  GS_REQUIRE(S + E < (int64_t(1) << 31),
+             "unique: at most 2^31 - 1 keys per call, got %lld", (long long)(S + E));
   GS_REQUIRE(S == 0 || seeds, "unique: null seeds");
   GS_REQUIRE(E == 0 || rows, "unique: null rows");
   GS_REQUIRE((seeds_ptr == nullptr) == (rows_ptr == nullptr),
