@@ -108,6 +108,20 @@ def test_cdf_column_sampling_parity(fanout, replace):
          orc.sample_weighted(indptr, indices, None, None, fanout, replace, cdf=cdf))
 
 
+def test_cdf_sampling_with_replacement_beyond_the_register_budget():
+    # fanouts above 64 are written pick by pick instead of being held in registers
+    rng, indptr, indices, probs = _weighted_case(3)
+    cdf = orc.weight_cdf(indptr, probs)
+    g_cdf = capi.weight_cdf(T(indptr), F(probs))
+    cols = rng.integers(0, 3000, size=500)
+    for fanout in (65, 100):
+        same(capi.sample_weighted(T(indptr), T(indices), None, T(cols), fanout, True, call_id=2,
+                                  cdf=g_cdf),
+             orc.sample_weighted(indptr, indices, None, cols, fanout, True, call_id=2, cdf=cdf))
+    with pytest.raises(capi.GsError):
+        capi.sample_weighted(T(indptr), T(indices), None, T(cols), 65, False, cdf=g_cdf)
+
+
 @pytest.mark.parametrize("n,k", [(10, 20), (1000, 64), (233000, 512), (5000, 5000)])
 def test_list_sampling_parity(n, k):
     rng = np.random.default_rng(n)
