@@ -171,7 +171,20 @@ static std::tuple<torch::Tensor, torch::Tensor> list_weighted(
                                         replace ? 1 : 0, mptr(out_range),
                                         ws.data_ptr(), ws.numel(), cur_stream()));
   BatchOffsets::trust(out_range);
-  const int64_t total = read_last(out_range);
+  // The number of picks follows from the sizes alone, so it is worked out here
+  // instead of being read back from the device (which would wait for all the
+  // work queued so far): the segment sizes of a range are already on the host,
+  // where its check left them.
+  auto picks_of = [&](int64_t size) {
+    return replace ? (size > 0 ? num_picks : 0) : std::min(size, num_picks);
+  };
+  int64_t total = 0;
+  if (range.defined()) {
+    const std::vector<int64_t>& p = OffsetMirror::values(range);
+    for (size_t b = 0; b + 1 < p.size(); ++b) total += picks_of(p[b + 1] - p[b]);
+  } else {
+    total = picks_of(n);
+  }
   torch::Tensor out = new_ids(total, probs);
   const RandomState& rs = random_state();
   GS_CALL(gs_list_sample_weighted_fill(

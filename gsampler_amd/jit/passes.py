@@ -287,6 +287,11 @@ def batch_fuse_slicing_and_sampling(gm: fx.GraphModule) -> fx.GraphModule:
     return dce(gm)
 
 
+def _is_wrapped(node, name: str) -> bool:
+    return (isinstance(node, fx.Node) and node.op == "call_function"
+            and getattr(node.target, "__name__", "") == name)
+
+
 def fuse_square_and_sum(gm: fx.GraphModule) -> fx.GraphModule:
     """SpMM("copy_rhs", "sum", _, e ** 2, ...) => FusedESquareSum(..., e, ...)."""
     for spmm in list(gm.graph.nodes):
@@ -303,17 +308,17 @@ def fuse_square_and_sum(gm: fx.GraphModule) -> fx.GraphModule:
         with gm.graph.inserting_before(spmm):
             gm.graph.call_method("_CAPI_FusedESquareSum", args=tuple(new_args))
         gm.graph.erase_node(spmm)
+        # the step that shapes the accumulator only looks at shape and dtype:
+        # give it the plain weights, so that the square is dead and goes away
+        for user in list(efeat.users):
+            if _is_wrapped(user, "_before_spmm"):
+                user.replace_input_with(efeat, efeat.args[0])
     return dce(gm)
 
 
-def _is_wrapped(node, name: str) -> bool:
-    return (isinstance(node, fx.Node) and node.op == "call_function"
-            and getattr(node.target, "__name__", "") == name)
-
-
 def fuse_div_and_sum(gm: fx.GraphModule) -> fx.GraphModule:
-    """q = e / u[t] (an SDDMM with targets (e, t), written as a product with
-    the reciprocal by the operator wrappers), then SpMM("copy_rhs", "sum", _, q)
+    """q = e / u[t] (an SDDMM with targets (e, t) and operator "div", or "mul"
+    with 1.0 / u as its operand), then SpMM("copy_rhs", "sum", _, q)
     onto the other endpoint, q read by nothing else
         => FusedEDivUSum("div", "sum", u, e, ...): the quotient is never stored.
     The reference names this pass and leaves it empty

@@ -1,6 +1,5 @@
 """Operand preparation shared by the SDDMM / SpMM wrappers: broadcasting
-rules, the sub -> add(-x) and div -> mul(1/x) rewrites, scalar-feature
-unsqueezing.  Same observable behaviour as the reference's
+rules, scalar-feature unsqueezing.  Same observable behaviour as the reference's
 python/gs/ops/sddmm.py:16-100 and spmm.py:13-107."""
 from typing import Optional, Tuple
 
@@ -31,20 +30,8 @@ def pad_feature_dims(lhs: torch.Tensor, rhs: torch.Tensor):
     return lhs, rhs
 
 
-def rewrite_inverse_ops(op: str, rhs):
-    """sub -> add of the negated operand, div -> mul by the reciprocal (as the
-    reference's wrappers intend, python/gs/ops/sddmm.py:20-25).  Runs on plain
-    Python strings, so the operator name stays a constant in a traced graph."""
-    if op == "sub":
-        return "add", -rhs
-    if op == "div":
-        return "mul", 1.0 / rhs
-    return op, rhs
-
-
 def prepare_binary(op: str, lhs: Optional[torch.Tensor], rhs: Optional[torch.Tensor]):
-    """-> (lhs, rhs, feature_shape, squeeze, dtype, device) for an operator that
-    has already been through rewrite_inverse_ops."""
+    """-> (lhs, rhs, feature_shape, squeeze, dtype, device)."""
     if op not in ("copy_lhs", "copy_rhs"):
         lhs, rhs = pad_feature_dims(lhs, rhs)
     use_l, use_r = op != "copy_rhs", op != "copy_lhs"

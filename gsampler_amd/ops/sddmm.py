@@ -7,7 +7,7 @@ from itertools import product
 import torch
 
 from ..format import _COO
-from ._common import TARGET, prepare_binary, rewrite_inverse_ops
+from ._common import TARGET, prepare_binary
 
 torch.fx.wrap("_before_sddmm")
 torch.fx.wrap("_after_sddmm")
@@ -17,7 +17,8 @@ __all__ = ["gsddmm", "copy_u", "copy_v"]
 
 def _before_sddmm(num_edges, op, lhs_data, rhs_data):
     lhs, rhs, feat, squeeze, dtype, device = prepare_binary(op, lhs_data, rhs_data)
-    out = torch.zeros((num_edges,) + tuple(feat), dtype=dtype, device=device)
+    # every element is written by the operator: no need to clear it first
+    out = torch.empty((num_edges,) + tuple(feat), dtype=dtype, device=device)
     return lhs, rhs, out, squeeze
 
 
@@ -27,7 +28,10 @@ def _after_sddmm(out, squeeze):
 
 def gsddmm(g, op, lhs_data, rhs_data, lhs_target="u", rhs_target="v", on_format=_COO):
     num_edges = g._graph._CAPI_GetNumEdges()
-    op, rhs_data = rewrite_inverse_ops(op, rhs_data)
+    # sub and div go to the operator as they are (the reference's wrapper turns
+    # them into add / mul of the negated / reciprocal operand first,
+    # python/gs/ops/sddmm.py:20-25: two more passes over the operand and one
+    # more rounding)
     lhs, rhs, out, squeeze = _before_sddmm(num_edges, op, lhs_data, rhs_data)
     g._graph._CAPI_SDDMM(op, lhs, rhs, out, TARGET[lhs_target], TARGET[rhs_target],
                          on_format)

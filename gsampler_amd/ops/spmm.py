@@ -6,7 +6,7 @@ import sys
 import torch
 
 from ..format import _CSC
-from ._common import prepare_binary, rewrite_inverse_ops
+from ._common import prepare_binary
 
 torch.fx.wrap("_before_spmm")
 torch.fx.wrap("_after_spmm")
@@ -35,7 +35,6 @@ def _after_spmm(v, squeeze):
 def gspmm(g, op, reduce_op, lhs_data, rhs_data, lhs_target, on_format):
     num_rows = g._graph._CAPI_GetNumRows()
     num_cols = g._graph._CAPI_GetNumCols()
-    op, rhs_data = rewrite_inverse_ops(op, rhs_data)
     v, arg_u, arg_e, squeeze = _before_spmm(
         num_rows, num_cols, op, reduce_op, lhs_data, rhs_data, lhs_target)
     # the operands go in as given (scalar features stay 1-D): the operator
