@@ -197,3 +197,78 @@ def test_largest_configuration_weighted_layers():
     out2 = capi.sample_weighted(indptr, indices, probs, rel[0], 10, False, 7777, 1, cdf=cdf)
     check(rel[0], 10, out2)
     assert out2[2].numel() > 4_000_000
+
+
+# ------------------------------------------------------------------ LADIES
+def _ladies(A, seeds, fanouts):
+    """examples/ladies/ladies.py:7-21 of the reference."""
+    ret = []
+    for K in fanouts:
+        subA = A[:, seeds]
+        subA.edata["p"] = subA.edata["w"] ** 2
+        prob = subA.sum("p", axis=1)
+        sampleA, select_index = subA.collective_sampling(K, prob, False)
+        sampleA = sampleA.div("w", prob[select_index], axis=1)
+        out = sampleA.sum("w", axis=0)
+        sampleA = sampleA.div("w", out, axis=0)
+        seeds = sampleA.all_nodes()
+        ret.append(sampleA.to_dgl_block(prefetch_edata={"w"}))
+    return seeds, ret
+
+
+def test_ladies_layers_at_full_size_against_the_operator_chain_on_the_cpu():
+    """The layer-wise configuration (233 K nodes, 115 M edges, 512 seeds, 512
+    nodes per layer) through Matrix + gs.jit.compile against the CPU operators
+    chained by hand.  Weights are 0.5 or 1 (the hub rows of this multigraph
+    collect more than a million edges of the sliced columns), so the row sums of
+    their squares are exact in float32 in any order of summation and both sides pick
+    the same 512 nodes; the normalised weights are held to 1e-5 relative of the
+    same chain in float64."""
+    import gsampler_amd as gs
+    from gsampler_amd.utils import chung_lu_csc
+    dev = torch.device("cuda:0")
+    nodes, edges, K = 233_000, 115_000_000, 512
+    indptr, indices = chung_lu_csc(nodes, edges, seed=1, device=dev)
+    g = torch.Generator(device=dev)
+    g.manual_seed(4)
+    w = torch.randint(1, 3, (indices.numel(),), generator=g, device=dev).float() / 2.0
+    seeds = torch.randperm(nodes, generator=g, device=dev)[:512]
+    A = gs.Matrix()
+    A.load_graph("CSC", [indptr, indices])
+    A.edata["w"] = w
+    compiled = gs.jit.compile(_ladies, (A, seeds, [K, K]))
+    gs.manual_seed(99)
+    frontier, blocks = compiled(A, seeds, [K, K])
+
+    h_indptr, h_indices, h_w = indptr.cpu().numpy(), indices.cpu().numpy(), w.cpu().numpy()
+    h_seeds = seeds.cpu().numpy()
+    for layer, blk in enumerate(blocks):
+        sub_indptr, coo_col, rows, sel = orc.col_slice(h_indptr, h_indices, h_seeds)
+        w_sub = h_w[sel]
+        prob = orc.e_square_sum(("coo", rows, coo_col), w_sub, 2, nodes)
+        exact = np.zeros(nodes)
+        np.add.at(exact, rows, w_sub.astype(np.float64) ** 2)
+        assert np.array_equal(prob, exact.astype(np.float32))        # the sums are exact
+        picked, _ = orc.list_sample_weighted(prob, K, seed=99, call_id=layer)
+        out_indptr, major, minor, select = orc.minor_slice(rows, picked, indptr=sub_indptr)
+        uniq, _, out_row, out_col = orc.unique_relabel(h_seeds, picked[minor], edge_col=major)
+        assert blk.num_dst_nodes() == h_seeds.size and blk.num_src_nodes() == uniq.size
+        assert np.array_equal(blk.srcdata["_ID"].cpu().numpy(), uniq)
+        assert np.array_equal(blk.row.cpu().numpy(), out_row)
+        assert np.array_equal(blk.col.cpu().numpy(), out_col)
+        # Values: a column of these blocks sums ten thousand and more quotients
+        # (a sequential float32 sum of that length, which is what the CPU
+        # operators do, is itself off by more than 1e-4), so the yardstick is
+        # the same chain in float64.
+        q = w_sub[select].astype(np.float64) / prob[picked].astype(np.float64)[minor]
+        col64 = np.zeros(h_seeds.size)
+        np.add.at(col64, major, q)
+        truth = q / col64[major]
+        assert np.allclose(blk.edata["w"].double().cpu().numpy(), truth, rtol=1e-5, atol=0)
+        # the weights of every column of a block sum to one
+        sums = np.zeros(h_seeds.size)
+        np.add.at(sums, out_col, blk.edata["w"].double().cpu().numpy())
+        assert np.allclose(sums[np.bincount(out_col, minlength=h_seeds.size) > 0], 1.0, atol=1e-4)
+        h_seeds = uniq
+    assert np.array_equal(frontier.cpu().numpy(), h_seeds)
+    assert blocks[1].num_edges() > 1_000_000          # the second layer really is a large one
