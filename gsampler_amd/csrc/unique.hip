@@ -377,7 +377,7 @@ __global__ __launch_bounds__(kBlock) void unique_scatter_kernel(
     Keys k, const int32_t* __restrict__ tile_batch,
     const BatchInfo* __restrict__ batch, int64_t* bucket_cnt,
     const int64_t* __restrict__ bucket_off, uint64_t* __restrict__ packed,
-    int64_t max_tiles, int remap) {
+    uint32_t* __restrict__ first, int64_t max_tiles, int remap) {
   __shared__ uint32_t hist[kMaxBuckets];   // counts, then offsets inside the tile
   __shared__ uint32_t run_at[kMaxBuckets]; // where the tile's run starts, relative to the batch
   __shared__ uint64_t stage[kPartTile];
@@ -389,8 +389,10 @@ __global__ __launch_bounds__(kBlock) void unique_scatter_kernel(
   const uint32_t buckets = (uint32_t)t.b.buckets;
   uint64_t* out = packed + t.b.fb;
   if (buckets == 1) {  // the bucket is the batch, in order
-    for (int64_t l = t.begin + threadIdx.x; l < t.end; l += kBlock)
+    for (int64_t l = t.begin + threadIdx.x; l < t.end; l += kBlock) {
       out[l] = (key_at(k, t.b, l) << 32) | (uint64_t)l;
+      first[t.b.fb + l] = (uint32_t)l;
+    }
     return;
   }
   for (uint32_t i = threadIdx.x; i < buckets; i += kBlock) hist[i] = 0;
@@ -400,6 +402,9 @@ __global__ __launch_bounds__(kBlock) void unique_scatter_kernel(
   for (int i = 0; i < kPartItems; ++i) {
     const int64_t l = t.begin + i * kBlock + threadIdx.x;
     key[i] = l < t.end ? (uint32_t)key_at(k, t.b, l) : 0u;
+    // every position starts as its own first occurrence; the dedup pass only
+    // writes the positions that are not (half as many scattered stores)
+    if (l < t.end) first[t.b.fb + l] = (uint32_t)l;
   }
 #pragma unroll
   for (int i = 0; i < kPartItems; ++i)
@@ -587,8 +592,10 @@ __global__ __launch_bounds__(kThreads) void unique_dedup_kernel(
     __syncthreads();
 #pragma unroll
     for (int j = 0; j < kKeep; ++j)
-      if (mine[j] != kEmptySlot)
-        first_b[(uint32_t)mine[j]] = lds_first_of(tab, mask, mine[j] >> 32);
+      if (mine[j] != kEmptySlot) {
+        const uint32_t f = lds_first_of(tab, mask, mine[j] >> 32);
+        if (f != (uint32_t)mine[j]) first_b[(uint32_t)mine[j]] = f;
+      }
     return;
   }
   // Many entries: fine for the LDS table while few of them are distinct (a hub
@@ -621,8 +628,10 @@ __global__ __launch_bounds__(kThreads) void unique_dedup_kernel(
       }
 #pragma unroll
       for (int j = 0; j < kDeep; ++j)
-        if (e[j] != kEmptySlot)
-          first_b[(uint32_t)e[j]] = lds_first_of(tab, mask, e[j] >> 32);
+        if (e[j] != kEmptySlot) {
+          const uint32_t f = lds_first_of(tab, mask, e[j] >> 32);
+          if (f != (uint32_t)e[j]) first_b[(uint32_t)e[j]] = f;
+        }
     }
     return;
   }
@@ -638,7 +647,8 @@ __global__ __launch_bounds__(kThreads) void unique_dedup_kernel(
   __syncthreads();
   for (int64_t i = lo + threadIdx.x; i < hi; i += kThreads) {
     const uint64_t e = packed[i];
-    first_b[(uint32_t)e] = spill_first_of(gt, cap, e >> 32);
+    const uint32_t f = spill_first_of(gt, cap, e >> 32);
+    if (f != (uint32_t)e) first_b[(uint32_t)e] = f;
   }
 }
 
@@ -911,7 +921,7 @@ int gs_unique_count(const int64_t* seeds, const int64_t* seeds_ptr,
                 w.bucket_ptr, B, w.bucket_cnt, w.bucket_off));
   GS_LAUNCH("unique_scatter", s,
             unique_scatter_kernel<<<tile_grid, dim3(kBlock), 0, s>>>(
-                k, w.tile_batch, w.batch, w.bucket_cnt, w.bucket_off, w.packed,
+                k, w.tile_batch, w.batch, w.bucket_cnt, w.bucket_off, w.packed, w.first,
                 w.max_tiles, tn.remap));
   GS_LAUNCH("unique_dedup", s,
             if (tn.dedup_threads == 512)
