@@ -11,7 +11,7 @@ import torch
 
 from ..format import _COO
 from ..ops import gsddmm, gspmm
-from ..utils.block import Block, create_block_from_coo
+from ..utils.block import Block
 from .matrix import Matrix, data_index
 
 torch.fx.wrap("batch_gen_block")
@@ -28,13 +28,13 @@ def batch_gen_block(frontier_list, coo_row_list, coo_col_list, coo_eids, coo_ptr
     for key, value in edata.items():
         edata_list[key] = split(value, coo_ptr)
     blocks = []
-    for i, frontier in enumerate(frontier_list):
-        block = create_block_from_coo(coo_row_list[i], coo_col_list[i], frontier.numel(),
-                                      col_counts[i])
+    for frontier, row, col, num_dst in zip(frontier_list, coo_row_list, coo_col_list, col_counts):
+        block = Block(row, col, frontier.shape[0], num_dst)
         block.srcdata["_ID"] = frontier
-        for key, parts in edata_list.items():
-            block.edata[key] = parts[i]
         blocks.append(block)
+    for key, parts in edata_list.items():
+        for block, part in zip(blocks, parts):
+            block.edata[key] = part
     return blocks
 
 

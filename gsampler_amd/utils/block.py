@@ -14,9 +14,15 @@ import torch
 
 
 class Block:
+    # A super-batched sampler builds hundreds of these per step: fixed slots
+    # and a plain constructor keep that loop short.
+    __slots__ = ("row", "col", "num_src", "num_dst", "srcdata", "dstdata", "edata")
+
     def __init__(self, row: torch.Tensor, col: torch.Tensor, num_src: int, num_dst: int):
-        self.row, self.col = row, col
-        self.num_src, self.num_dst = int(num_src), int(num_dst)
+        self.row = row
+        self.col = col
+        self.num_src = num_src if type(num_src) is int else int(num_src)
+        self.num_dst = num_dst if type(num_dst) is int else int(num_dst)
         self.srcdata: Dict[str, torch.Tensor] = {}
         self.dstdata: Dict[str, torch.Tensor] = {}
         self.edata: Dict[str, torch.Tensor] = {}
