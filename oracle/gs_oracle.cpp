@@ -488,6 +488,7 @@ void spmm_impl(const View& g, int64_t nnz, int kind, int op, int reduce,
     for (int64_t c = 0; c < g.num_major; ++c)
       for (int64_t f = 0; f < out_len; ++f) {
         float acc = 0.f;
+        double sum = 0.0;
         int64_t bu = 0, be = 0;
         for (int64_t i = g.a[c]; i < g.a[c + 1]; ++i) {
           int64_t eid = g.edge_map ? g.edge_map[i] : i, cid = g.b[i];
@@ -495,13 +496,14 @@ void spmm_impl(const View& g, int64_t nnz, int kind, int op, int reduce,
                                ufeat ? ufeat + cid * ulen + (uo ? uo[f] : f) : nullptr,
                                efeat ? efeat + eid * elen + (eo ? eo[f] : f) : nullptr);
           if (reduce == 0)
-            acc += v;
+            sum += (double)v;
           else if (better(v, acc)) {
             acc = v;
             bu = cid;
             be = eid;
           }
         }
+        if (reduce == 0) acc = (float)sum;
         out[c * out_len + f] += acc;
         if (reduce != 0) {
           if (arg_u) arg_u[c * out_len + f] = bu;
@@ -509,6 +511,18 @@ void spmm_impl(const View& g, int64_t nnz, int kind, int op, int reduce,
         }
       }
     return;
+  }
+  // Sums are taken in double and rounded once (per-edge values stay float32,
+  // as on the device): the reference adds with float atomics in whatever order
+  // the hardware takes them, so no float32 sum is "the" result, and a yardstick
+  // that carries a rounding error of its own per term would only blur the
+  // comparison for long rows.
+  std::vector<double> sums;
+  if (reduce == 0) {
+    int64_t n_out = 0;
+    for (int64_t e = 0; e < nnz; ++e)
+      n_out = std::max(n_out, (u_target == 0 ? g.b[e] : g.a[e]) + 1);
+    sums.assign((size_t)(n_out * out_len), 0.0);
   }
   for (int64_t e = 0; e < nnz; ++e) {
     int64_t src = u_target == 0 ? g.a[e] : g.b[e];
@@ -520,7 +534,7 @@ void spmm_impl(const View& g, int64_t nnz, int kind, int op, int reduce,
                            efeat ? efeat + eid * elen + (eo ? eo[f] : f) : nullptr);
       float& o = out[dst * out_len + f];
       if (reduce == 0)
-        o += v;
+        sums[(size_t)(dst * out_len + f)] += (double)v;
       else if (better(v, o)) {
         o = v;
         if (arg_u) arg_u[dst * out_len + f] = src;
@@ -528,6 +542,7 @@ void spmm_impl(const View& g, int64_t nnz, int kind, int op, int reduce,
       }
     }
   }
+  for (size_t i = 0; i < sums.size(); ++i) out[i] += (float)sums[i];
 }
 }  // namespace
 
