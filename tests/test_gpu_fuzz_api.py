@@ -2,7 +2,10 @@
 repeated and empty id lists, sums, quotients, per-column and collective
 sampling, the block hand-off) on random multigraphs loaded as edge list, CSC or
 CSR, checked after every step against a dense float64 model.  Weights are
-multiples of 1/8, so sums are exact in any order."""
+multiples of 1/8, so sums are exact in any order.
+The super-batched API the same way: random mini-batches (some empty) through
+BatchMatrix column slicing, per-column sampling, all_nodes and the per-batch
+blocks, one or two layers, checked batch by batch against the matrix."""
 import numpy as np
 import pytest
 import torch
@@ -116,3 +119,74 @@ def case(seed):
 def test_random_operator_sequences(block):
     for seed in range(block * 100, block * 100 + 100):
         case(seed)
+
+
+# ------------------------------------------------------------ super-batches
+def batch_case(seed):
+    rng = np.random.default_rng(seed)
+    N = int(rng.integers(2, 500))
+    E = int(rng.integers(1, 6000))
+    row = rng.integers(0, N, size=E); col = rng.integers(0, N, size=E)
+    row[-1], col[-1] = N - 1, N - 1
+    w = (rng.integers(1, 9, size=E) / 8.0).astype(np.float32)
+    order = np.argsort(col, kind="stable")
+    indptr = np.concatenate([[0], np.cumsum(np.bincount(col, minlength=N))])
+    m = gs.Matrix()
+    m.load_graph("CSC", [torch.tensor(indptr, device=DEV), torch.tensor(row[order], device=DEV)])
+    m.edata["w"] = torch.tensor(w[order], device=DEV)
+    count = np.zeros((N, N), dtype=np.int64); np.add.at(count, (row, col), 1)
+    deg = count.sum(axis=0)
+    encoding = bool(rng.integers(0, 2))
+    bm = gs.BatchMatrix(); bm.load_from_matrix(m, encoding)
+    B = int(rng.integers(1, 9))
+    sizes = [int(rng.integers(0, 40)) if rng.random() > 0.15 else 0 for _ in range(B)]
+    distinct = True          # seeds of a mini-batch are distinct (duplicates share one label)
+    seeds_l = [rng.permutation(N)[:min(s, N)] if distinct else rng.integers(0, N, size=s) for s in sizes]
+    ptr = np.concatenate([[0], np.cumsum([len(s) for s in seeds_l])]).astype(np.int64)
+    seeds = np.concatenate(seeds_l).astype(np.int64) if ptr[-1] else np.zeros(0, np.int64)
+    g_seeds, g_ptr = torch.tensor(seeds, device=DEV), torch.tensor(ptr, device=DEV)
+    layers = int(rng.integers(1, 3))
+    gs.manual_seed(seed)
+    for layer in range(layers):
+        k = int(rng.integers(1, 7))
+        sub = bm[:, g_seeds::g_ptr]
+        smp = sub.individual_sampling(k, None, False)
+        nodes, nodes_ptr = smp.all_nodes()
+        blocks = smp.to_dgl_block()
+        assert len(blocks) == B, "blocks"
+        nodes, nodes_ptr = nodes.cpu().numpy(), nodes_ptr.cpu().numpy()
+        assert nodes_ptr[0] == 0 and nodes_ptr[-1] == nodes.size
+        new_seeds = []
+        for b, blk in enumerate(blocks):
+            sb = seeds[ptr[b]:ptr[b + 1]]
+            fr = blk.srcdata["_ID"].cpu().numpy()
+            assert np.array_equal(fr, nodes[nodes_ptr[b]:nodes_ptr[b + 1]]), ("frontier", seed, b)
+            assert blk.num_dst == sb.size and blk.num_src == fr.size
+            r, c = blk.row.cpu().numpy(), blk.col.cpu().numpy()
+            src, dst_pos = fr[r], c
+            assert np.all((dst_pos >= 0) & (dst_pos < max(sb.size, 1))) or r.size == 0
+            dst = sb[dst_pos] if r.size else dst_pos
+            # counts per requested column (position), edges exist, no more copies than the matrix has
+            per_col = np.bincount(dst_pos, minlength=sb.size) if r.size else np.zeros(sb.size, int)
+            assert np.array_equal(per_col, np.minimum(deg[sb], k)), ("count", seed, b)
+            got = {}
+            for s_, p_ in zip(src.tolist(), dst_pos.tolist()):
+                got[(s_, p_)] = got.get((s_, p_), 0) + 1
+            for (s_, p_), n_ in got.items():
+                assert n_ <= count[s_, sb[p_]], ("edge", seed, b)
+            # frontier: unique of seeds ++ sources in first-occurrence order
+            keys = np.concatenate([sb, src])
+            # block edge order is the sampled edge order of this batch, so first occurrences follow it
+            _, first = np.unique(keys, return_index=True)
+            assert np.array_equal(fr, keys[np.sort(first)]), ("order", seed, b)
+            new_seeds.append(fr)
+        seeds_l = new_seeds
+        ptr = np.concatenate([[0], np.cumsum([len(s) for s in seeds_l])]).astype(np.int64)
+        seeds = np.concatenate(seeds_l).astype(np.int64) if ptr[-1] else np.zeros(0, np.int64)
+        g_seeds, g_ptr = torch.tensor(seeds, device=DEV), torch.tensor(ptr, device=DEV)
+
+
+@pytest.mark.parametrize("block", range(3))
+def test_random_super_batches(block):
+    for seed in range(block * 100, block * 100 + 100):
+        batch_case(seed)
