@@ -40,6 +40,10 @@ WORKLOADS = {
                fanouts=[512, 512],
                desc="LADIES 2 layers, 512 seeds, K=512 per layer, Chung-Lu power-law 233K nodes / "
                     "115M edges, fp32 edge weights U(0,1], through Matrix / gs.jit.compile"),
+    "ops": dict(kind="ops", nodes=2_450_000, edges=124_000_000, gen="chung_lu", batches=64,
+                batch_size=1024, fanouts=[15, 10, 5],
+                desc="every operator of the path on its own: C2's graph, the frontiers and edge "
+                     "lists of one GraphSAGE step as inputs, LogNormal weights"),
     "c4": dict(kind="node2vec", nodes=2_450_000, edges=124_000_000, gen="chung_lu",
                walks=1_000_000, length=80, p=2.0, q=0.5,
                desc="node2vec, 1M walks x 80 steps, p=2.0 q=0.5, C2's graph with sorted columns"),
@@ -181,7 +185,7 @@ def run_node2vec(args, wl, capi, dev):
     from gsampler_amd.utils import chung_lu_csc
     t0 = time.time()
     indptr, indices = chung_lu_csc(wl["nodes"], wl["edges"], seed=1, device=dev)
-    indices = capi.segment_sort(indptr, indices)          # node2vec needs sorted columns
+    indices = capi.segment_sort(indptr, indices, wl["nodes"])   # node2vec needs sorted columns
     g = torch.Generator(device=dev)
     g.manual_seed(3)
     seeds = torch.randint(0, wl["nodes"], (wl["walks"],), generator=g, device=dev)
@@ -357,6 +361,120 @@ def ladies_step_oracle(orc, indptr, indices, w, seeds, fanouts, num_rows, call_b
     return edges
 
 
+def run_ops(args, wl, capi, dev):
+    """Every operator of the path timed on its own.  Device time = the sum of
+    the operator's kernels by the library's event timers (a count pass and a
+    fill pass belong to one operator); bytes = the operator's compulsory
+    reads and writes.  Inputs: C2's graph and what one GraphSAGE step makes of
+    it (layer-2 frontier: ~0.6 M columns; layer-3 frontier: ~3.5 M columns and
+    17 M sampled edges)."""
+    import torch
+    from gsampler_amd.utils import batched_seeds, chung_lu_csc
+    t0 = time.time()
+    indptr, indices = chung_lu_csc(wl["nodes"], wl["edges"], seed=1, device=dev)
+    N, nnz = wl["nodes"], int(indices.numel())
+    seeds, ptr = batched_seeds(N, wl["batches"], wl["batch_size"], seed=2, device=dev)
+    g = torch.Generator(device=dev)
+    g.manual_seed(5)
+    probs = torch.randn(nnz, generator=g, device=dev).exp_().float()
+    cdf = capi.weight_cdf(indptr, probs)
+    # frontiers of a step
+    s1 = capi.sample_uniform(indptr, indices, seeds, 15, False, 0, args.seed, 0)
+    r1 = capi.unique_relabel(seeds, s1[2], ptr, s1[0][ptr], s1[1])
+    s2 = capi.sample_uniform(indptr, indices, r1[0], 10, False, 0, args.seed, 1)
+    r2 = capi.unique_relabel(r1[0], s2[2], r1[1], s2[0][r1[1]], s2[1])
+    f2, f3, f3_ptr = r1[0][:131072].contiguous(), r2[0], r2[1]   # f2: the first two mini-batches' worth
+    s3 = capi.sample_uniform(indptr, indices, f3, 5, False, 0, args.seed, 2)
+    e3_ptr = s3[0][f3_ptr]
+    S2, S3, E3 = int(f2.numel()), int(f3.numel()), int(s3[2].numel())
+    torch.cuda.synchronize()
+    t_build = time.time() - t0
+    rows = []
+
+    def measure(name, ref, fn, nbytes, note):
+        out = fn()                       # warm-up; the result sizes the byte count if needed
+        if callable(nbytes):
+            nbytes = nbytes(out)
+        del out
+        torch.cuda.synchronize()
+        capi.profile_reset()
+        capi.profile_enable(True)
+        t = time.perf_counter()
+        for _ in range(args.steps):
+            fn()
+        torch.cuda.synchronize()
+        wall = (time.perf_counter() - t) / args.steps * 1e3
+        capi.profile_enable(False)
+        dev_ms = sum(ms for _, ms in capi.profile_totals().values()) / args.steps
+        gbs = nbytes / (dev_ms * 1e-3) / 1e9 if dev_ms > 0 else 0.0
+        rows.append(dict(operator=name, reference=ref, device_ms=round(dev_ms, 4),
+                         wall_ms=round(wall, 4), algorithmic_mb=round(nbytes / 1e6, 1),
+                         gbs=round(gbs, 1), frac_of_hbm_peak=round(gbs / HBM_PEAK_GBS, 4),
+                         input=note))
+
+    # column slice of the layer-2 frontier
+    measure("column slice", "OnIndptrSlicingCUDA", lambda: capi.col_slice(indptr, indices, f2),
+            lambda o: 24 * S2 + 32 * int(o[2].numel()), f"{S2} columns")
+    sl = capi.col_slice(indptr, indices, f2)
+    sl_nnz = int(sl[2].numel())
+    # row slice of that slice by 512 picked rows per ... here: 65 536 picked ids
+    picked = torch.randperm(N, generator=g, device=dev)[:65536]
+    measure("row slice", "OnIndicesSlicingCUDA", lambda: capi.minor_slice(sl[2], picked, indptr=sl[0]),
+            lambda o: 8 * 65536 + 8 * sl_nnz + 32 * int(o[2].numel()),
+            f"{sl_nnz} edges against 65536 picked rows")
+    e_w = probs[sl[3]]
+    coo_view = ("coo", sl[2], sl[1])
+    csc_view = ("csc", sl[0], sl[2])
+    measure("e^2 row sums (edge list)", "ESquareSumCOO",
+            lambda: capi.e_square_sum(coo_view, e_w, 2, N), 12 * sl_nnz + 4 * N, f"{sl_nnz} edges onto {N} rows")
+    measure("column sums (compressed)", "SpMMCSC",
+            lambda: capi.spmm(csc_view, "copy_rhs", "sum", None, e_w, 0, S2), 4 * sl_nnz + 12 * S2,
+            f"{sl_nnz} edges onto {S2} columns")
+    col_sum = capi.spmm(csc_view, "copy_rhs", "sum", None, e_w, 0, S2)
+    measure("edge / column value", "SDDMMCOO", lambda: capi.sddmm(coo_view, "div", e_w, col_sum, 1, 2),
+            24 * sl_nnz, f"{sl_nnz} edges")
+    measure("edges' columns from offsets", "CSC2COOCUDA", lambda: capi.csc2coo(sl[0], sl_nnz),
+            8 * S2 + 8 * sl_nnz, f"{sl_nnz} edges")
+    del sl, e_w, col_sum, coo_view, csc_view
+    # samplers on the layer-3 frontier
+    measure("uniform slice + sample, K=5", "FusedCSCColSlicingSamplingCUDA",
+            lambda: capi.sample_uniform(indptr, indices, f3, 5, False, 0, args.seed, 2),
+            32 * S3 + 32 * E3, f"{S3} columns")
+    measure("weighted slice + sample, K=5 (CDF)", "CSCColSamplingProbsCUDA",
+            lambda: capi.sample_weighted(indptr, indices, probs, f3, 5, False, args.seed, 2, cdf=cdf),
+            32 * S3 + 32 * E3, f"{S3} columns")
+    measure("unique + relabel, 64 batches", "BatchCOORelabelCUDA",
+            lambda: capi.unique_relabel(f3, s3[2], f3_ptr, e3_ptr, s3[1]),
+            lambda o: 8 * S3 + 24 * E3 + 8 * int(o[0].numel()), f"{S3} + {E3} keys")
+    node_w = torch.rand(N, generator=g, device=dev)
+    measure("collective pick of 512", "ListSamplingProbsCUDA",
+            lambda: capi.list_sample_weighted(node_w, 512, False, None, args.seed, 3), 4 * N + 8 * 512,
+            f"{N} weights")
+    walkers = torch.randint(0, N, (1_000_000,), generator=g, device=dev)
+    measure("random walk, 80 steps", "FusedRandomWalkCUDA",
+            lambda: capi.random_walk(indptr, indices, walkers, 80, args.seed, 4),
+            lambda o: 32 * int((o[1:] >= 0).sum()), "1 M walks")
+    measure("per-column sort", "SortIndicesCUDA", lambda: capi.segment_sort(indptr, indices, N), 16 * nnz,
+            f"{nnz} edges in {N} columns")
+    coo_col = capi.csc2coo(indptr, nnz)
+    measure("edge list -> compressed", "COO2CSCCUDA", lambda: capi.coo_to_csc(indices, coo_col, N),
+            8 * nnz * 2 + 8 * nnz * 2 + 8 * N, f"{nnz} edges")
+    measure("weight CDF build", "(none)", lambda: capi.weight_cdf(indptr, probs), 12 * nnz, f"{nnz} edges")
+    rows.sort(key=lambda r: -r["device_ms"])
+    dom = rows[0]
+    return {
+        "metric": "operators_measured", "value": len(rows), "unit": "operators", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(sum(r["device_ms"] for r in rows), 3), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "int64", "data": "synthetic",
+        "config": {"workload": f"{args.workload}: {wl['desc']}"},
+        "roofline": dict(bound="hbm", kernel=dom["operator"], achieved=dom["gbs"],
+                         peak=HBM_PEAK_GBS, unit="GB/s", frac=dom["frac_of_hbm_peak"],
+                         traffic=None, avg_launch_ms=dom["device_ms"], launches=args.steps),
+        "cpu_baseline": None, "operators": rows, "graph_build_s": round(t_build, 1),
+    }
+
+
 def run_ladies(args, wl, capi, dev):
     """LADIES through the Python Matrix API and the torch custom class (the
     whole drop-in stack), compiled with gs.jit.compile.  A step = one 2-layer sample."""
@@ -462,6 +580,8 @@ def main():
         return print(json.dumps(run_gather(args, wl, capi, dev)))
     if wl.get("kind") == "ladies":
         return print(json.dumps(run_ladies(args, wl, capi, dev)))
+    if wl.get("kind") == "ops":
+        return print(json.dumps(run_ops(args, wl, capi, dev)))
 
     t0 = time.time()
     gen = chung_lu_csc if wl["gen"] == "chung_lu" else rmat_csc

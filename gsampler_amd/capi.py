@@ -89,8 +89,8 @@ SIGNATURES = {
     "gs_random_walk": (_int, [_p, _p, _i64, _p, _i64, _i64, _u64, _u64, _p, _p]),
     "gs_node2vec": (_int, [_p, _p, _i64, _p, _i64, _i64, C.c_double, C.c_double, _u64, _u64,
                            _p, _p]),
-    "gs_segment_sort_workspace_bytes": (_sz, [_i64, _i64]),
-    "gs_segment_sort_i64": (_int, [_p, _i64, _p, _p, _i64, _p, _sz, _p]),
+    "gs_segment_sort_workspace_bytes": (_sz, [_i64, _i64, _i64]),
+    "gs_segment_sort_i64": (_int, [_p, _i64, _p, _p, _i64, _i64, _p, _sz, _p]),
 }
 
 _lib = None
@@ -699,11 +699,14 @@ def node2vec(indptr, indices, seeds, walk_length, p, q, seed=7777, call_id=0):
     return out
 
 
-def segment_sort(indptr, keys):
+def segment_sort(indptr, keys, key_bound=0):
+    """Keys sorted inside every segment.  `key_bound` (every key in [0, key_bound),
+    e.g. the number of rows) selects the much faster packed sort; 0 = not known."""
     indptr, keys = _i64t(indptr, "indptr"), _i64t(keys, "keys")
     out = torch.empty_like(keys)
     nseg = indptr.numel() - 1
-    ws = _workspace(lib().gs_segment_sort_workspace_bytes(keys.numel(), nseg), keys.device)
+    ws = _workspace(lib().gs_segment_sort_workspace_bytes(keys.numel(), nseg, key_bound),
+                    keys.device)
     check(lib().gs_segment_sort_i64(_ptr(indptr), nseg, _ptr(keys), _ptr(out), keys.numel(),
-                                    ws.data_ptr(), ws.numel(), _stream()))
+                                    key_bound, ws.data_ptr(), ws.numel(), _stream()))
     return out

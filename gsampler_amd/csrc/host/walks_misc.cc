@@ -60,10 +60,11 @@ void Graph::SortCSCIndices() {
   TORCH_CHECK(!csc_->e_ids.has_value(), "SortCSCIndices: the CSC format carries e_ids");
   const int64_t nnz = csc_->indices.numel();
   torch::Tensor sorted = new_ids(nnz, csc_->indices);
-  torch::Tensor ws = new_workspace(gs_segment_sort_workspace_bytes(nnz, num_cols_),
+  // row ids lie in [0, num_rows): the loaders check that
+  torch::Tensor ws = new_workspace(gs_segment_sort_workspace_bytes(nnz, num_cols_, num_rows_),
                                    csc_->indices);
   GS_CALL(gs_segment_sort_i64(cptr(csc_->indptr), num_cols_, cptr(csc_->indices),
-                              mptr(sorted), nnz, ws.data_ptr(), ws.numel(),
+                              mptr(sorted), nnz, num_rows_, ws.data_ptr(), ws.numel(),
                               cur_stream()));
   csc_->indices = sorted;
   csc_sorted_ = true;

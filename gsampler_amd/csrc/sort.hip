@@ -10,44 +10,7 @@
 #include <rocprim/device/device_segmented_radix_sort.hpp>
 #include <rocprim/iterator/counting_iterator.hpp>
 
-extern "C" {
-
-size_t gs_segment_sort_workspace_bytes(int64_t nnz, int64_t num_segments) {
-  if (nnz < 0 || num_segments < 0) return 0;
-  size_t bytes = 0;
-  const int64_t* k = nullptr;
-  int64_t* o = nullptr;
-  (void)rocprim::segmented_radix_sort_keys(nullptr, bytes, k, o, (size_t)(nnz > 0 ? nnz : 1),
-                                           (unsigned)(num_segments > 0 ? num_segments : 1),
-                                           k, k, 0, 64);
-  return gs::align_up(bytes, 256);
-}
-
-// keys_out[seg] = sorted(keys_in[seg]) for every segment of indptr; in and out
-// must not alias.  SortIndicesCUDA, src/cuda/sort_indices.cu:11-37.
-int gs_segment_sort_i64(const int64_t* indptr, int64_t num_segments,
-                        const int64_t* keys_in, int64_t* keys_out, int64_t nnz,
-                        void* workspace, size_t workspace_bytes,
-                        gs_stream_t stream) {
-  using namespace gs;
-  GS_REQUIRE(nnz >= 0 && num_segments >= 0, "segment_sort: negative size");
-  if (nnz == 0 || num_segments == 0) return GS_OK;
-  GS_REQUIRE(indptr && keys_in && keys_out, "segment_sort: null pointer");
-  GS_REQUIRE(keys_in != keys_out, "segment_sort: in-place sorting is not supported");
-  size_t need = gs_segment_sort_workspace_bytes(nnz, num_segments);
-  if (workspace == nullptr || workspace_bytes < need) {
-    set_error("segment_sort workspace too small: %zu < %zu", workspace_bytes, need);
-    return GS_ERR_WORKSPACE;
-  }
-  hipStream_t s = as_stream(stream);
-  size_t bytes = workspace_bytes;
-  ProfScope ps("segment_sort", s);
-  GS_HIP(rocprim::segmented_radix_sort_keys(workspace, bytes, keys_in, keys_out,
-                                            (size_t)nnz, (unsigned)num_segments,
-                                            indptr, indptr + 1, 0, 64, s));
-  return GS_OK;
-}
-
+namespace gs {
 
 static int id_bits(int64_t num_ids) {
   int bits = 1;
@@ -55,13 +18,124 @@ static int id_bits(int64_t num_ids) {
   return bits;
 }
 
+// Segment and key in one word: (segment << key_bits) | key.  A plain radix sort
+// of these words over the bits they use sorts every segment, because the input
+// is already grouped by segment; it moves every key a fixed number of times
+// whatever the segment sizes are, where a segmented sort of millions of short
+// segments and a few hubs spends its time on scheduling them.
+__global__ __launch_bounds__(kBlock) void pack_segment_keys_kernel(
+    const int64_t* __restrict__ indptr, int64_t num_segments,
+    const int64_t* __restrict__ keys, int64_t nnz, int key_bits,
+    uint64_t* __restrict__ packed) {
+  const int64_t e = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (e >= nnz) return;
+  const uint64_t seg = (uint64_t)segment_of(indptr, num_segments, e);
+  packed[e] = (seg << key_bits) | (uint64_t)keys[e];
+}
+
+__global__ __launch_bounds__(kBlock) void unpack_segment_keys_kernel(
+    int64_t* __restrict__ keys, int64_t nnz, int key_bits) {
+  const int64_t e = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (e >= nnz) return;
+  keys[e] = (int64_t)((uint64_t)keys[e] & (((uint64_t)1 << key_bits) - 1));
+}
+
+// Bits of the packed word, or 0 when segment and key do not fit one word (or
+// the key range is not known): then the segmented sort over all 64 bits runs.
+static int packed_bits(int64_t num_segments, int64_t key_bound, int* key_bits) {
+  if (key_bound <= 0) return 0;
+  *key_bits = id_bits(key_bound);
+  const int total = *key_bits + id_bits(num_segments);
+  return total <= 64 ? total : 0;
+}
+
+static size_t segmented_temp_bytes(int64_t nnz, int64_t num_segments) {
+  size_t bytes = 0;
+  const int64_t* k = nullptr;
+  int64_t* o = nullptr;
+  (void)rocprim::segmented_radix_sort_keys(nullptr, bytes, k, o, (size_t)(nnz > 0 ? nnz : 1),
+                                           (unsigned)(num_segments > 0 ? num_segments : 1),
+                                           k, k, 0, 64);
+  return align_up(bytes, 256);
+}
+
+static size_t packed_temp_bytes(int64_t nnz, int bits) {
+  size_t bytes = 0;
+  const uint64_t* k = nullptr;
+  uint64_t* o = nullptr;
+  (void)rocprim::radix_sort_keys(nullptr, bytes, k, o, (size_t)(nnz > 0 ? nnz : 1), 0u,
+                                 (unsigned)bits);
+  return align_up(bytes, 256);
+}
+
+}  // namespace gs
+
+extern "C" {
+
+size_t gs_segment_sort_workspace_bytes(int64_t nnz, int64_t num_segments, int64_t key_bound) {
+  using namespace gs;
+  if (nnz < 0 || num_segments < 0) return 0;
+  int key_bits = 0;
+  const int bits = packed_bits(num_segments, key_bound, &key_bits);
+  if (bits == 0) return segmented_temp_bytes(nnz, num_segments);
+  return align_up((size_t)(nnz > 0 ? nnz : 1) * sizeof(uint64_t), 256) + packed_temp_bytes(nnz, bits);
+}
+
+// keys_out[seg] = sorted(keys_in[seg]) for every segment of indptr; in and out
+// must not alias.  key_bound: every key lies in [0, key_bound) (the number of
+// rows, for the row ids of a column); 0 = not known.
+// SortIndicesCUDA, src/cuda/sort_indices.cu:11-37.
+int gs_segment_sort_i64(const int64_t* indptr, int64_t num_segments,
+                        const int64_t* keys_in, int64_t* keys_out, int64_t nnz,
+                        int64_t key_bound, void* workspace, size_t workspace_bytes,
+                        gs_stream_t stream) {
+  using namespace gs;
+  GS_REQUIRE(nnz >= 0 && num_segments >= 0, "segment_sort: negative size");
+  if (nnz == 0 || num_segments == 0) return GS_OK;
+  GS_REQUIRE(indptr && keys_in && keys_out, "segment_sort: null pointer");
+  GS_REQUIRE(keys_in != keys_out, "segment_sort: in-place sorting is not supported");
+  size_t need = gs_segment_sort_workspace_bytes(nnz, num_segments, key_bound);
+  if (workspace == nullptr || workspace_bytes < need) {
+    set_error("segment_sort workspace too small: %zu < %zu", workspace_bytes, need);
+    return GS_ERR_WORKSPACE;
+  }
+  hipStream_t s = as_stream(stream);
+  int key_bits = 0;
+  const int bits = packed_bits(num_segments, key_bound, &key_bits);
+  if (bits == 0) {
+    size_t bytes = workspace_bytes;
+    ProfScope ps("segment_sort", s);
+    GS_HIP(rocprim::segmented_radix_sort_keys(workspace, bytes, keys_in, keys_out,
+                                              (size_t)nnz, (unsigned)num_segments,
+                                              indptr, indptr + 1, 0, 64, s));
+    return GS_OK;
+  }
+  uint64_t* packed = (uint64_t*)workspace;
+  const size_t packed_bytes = align_up((size_t)nnz * sizeof(uint64_t), 256);
+  void* temp = (char*)workspace + packed_bytes;
+  size_t temp_bytes = workspace_bytes - packed_bytes;
+  const dim3 grid((unsigned)ceil_div(nnz, kBlock));
+  GS_LAUNCH("segment_sort_pack", s,
+            pack_segment_keys_kernel<<<grid, dim3(kBlock), 0, s>>>(indptr, num_segments, keys_in,
+                                                                  nnz, key_bits, packed));
+  {
+    ProfScope ps("segment_sort", s);
+    GS_HIP(rocprim::radix_sort_keys(temp, temp_bytes, packed, (uint64_t*)keys_out, (size_t)nnz,
+                                    0u, (unsigned)bits, s));
+  }
+  GS_LAUNCH("segment_sort_unpack", s,
+            unpack_segment_keys_kernel<<<grid, dim3(kBlock), 0, s>>>(keys_out, nnz, key_bits));
+  return GS_OK;
+}
+
+
 size_t gs_coo_sort_workspace_bytes(int64_t nnz, int64_t num_major) {
   if (nnz < 0) return 0;
   size_t bytes = 0;
   const int64_t* k = nullptr;
   int64_t* o = nullptr;
   (void)rocprim::radix_sort_pairs(nullptr, bytes, k, o, rocprim::counting_iterator<int64_t>(0), o,
-                                  (size_t)(nnz > 0 ? nnz : 1), 0u, (unsigned)id_bits(num_major));
+                                  (size_t)(nnz > 0 ? nnz : 1), 0u, (unsigned)gs::id_bits(num_major));
   return gs::align_up(bytes, 256);
 }
 

@@ -366,7 +366,10 @@ int gs_sorted_to_indptr(const int64_t* sorted_ids, int64_t nnz, int64_t num_cols
  *    (return weight p, neighbour-of-previous weight q, otherwise 1); needs row
  *    ids sorted inside every column.  FusedNode2VecCUDA,
  *    src/cuda/fusion/node2vec.cu:139-162.
- *  gs_segment_sort_i64: sorts the ids of every segment (column).
+ *  gs_segment_sort_i64: sorts the ids of every segment (column).  key_bound:
+ *    every key lies in [0, key_bound) (0 = not known).  With it, segment and
+ *    key are sorted as one word over the bits they use; without it (or when
+ *    the two do not fit 64 bits) a segmented sort over all 64 bits runs.
  *    SortIndicesCUDA, src/cuda/sort_indices.cu:11-37.
  * ---------------------------------------------------------------------- */
 int gs_random_walk(const int64_t* indptr, const int64_t* indices, int64_t num_cols,
@@ -377,10 +380,11 @@ int gs_node2vec(const int64_t* indptr, const int64_t* indices, int64_t num_cols,
                 const int64_t* seeds, int64_t num_seeds, int64_t walk_length,
                 double p, double q, uint64_t seed, uint64_t call_id,
                 int64_t* out_traces, gs_stream_t stream);
-size_t gs_segment_sort_workspace_bytes(int64_t nnz, int64_t num_segments);
+size_t gs_segment_sort_workspace_bytes(int64_t nnz, int64_t num_segments,
+                                       int64_t key_bound);
 int gs_segment_sort_i64(const int64_t* indptr, int64_t num_segments,
                         const int64_t* keys_in, int64_t* keys_out, int64_t nnz,
-                        void* workspace, size_t workspace_bytes,
+                        int64_t key_bound, void* workspace, size_t workspace_bytes,
                         gs_stream_t stream);
 
 /* ------------------------------------------------------------------------

@@ -120,7 +120,7 @@ def test_weighted_step_with_persistent_cdf(graph):
 
 def test_node2vec_walks(graph):
     indptr, indices, _, _ = graph
-    indices = capi.segment_sort(indptr, indices)
+    indices = capi.segment_sort(indptr, indices, NODES)
     g = torch.Generator(device=indices.device)
     g.manual_seed(3)
     walks, length = 200_000, 80

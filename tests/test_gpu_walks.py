@@ -57,8 +57,18 @@ def test_sort_csc_indices_and_matrix_walks(graph):
     rng = np.random.default_rng(2)
     indptr, indices = random_csc(rng, 2000, 2000, 50, hub_deg=7000)
     indices[0] = 1999
-    assert np.array_equal(capi.segment_sort(T(indptr), T(indices)).cpu().numpy(),
-                          orc.segment_sort(indptr, indices))
+    want = orc.segment_sort(indptr, indices)
+    # without a key range: segmented sort over all bits; with one: column and
+    # row id sorted as one word (2000 and 2^40 rows: 22 and 51 bits; 2^60: back
+    # to the segmented sort, the word would not fit)
+    for bound in (0, 2000, 1 << 40, 1 << 60):
+        assert np.array_equal(capi.segment_sort(T(indptr), T(indices), bound).cpu().numpy(), want)
+    big = indices.copy()
+    big[::3] += (1 << 39)                                   # ids that need the wide key range
+    assert np.array_equal(capi.segment_sort(T(indptr), T(big), 1 << 40).cpu().numpy(),
+                          orc.segment_sort(indptr, big))
+    empty = capi.segment_sort(T(np.zeros(5)), T(np.zeros(0)), 10)
+    assert empty.numel() == 0
     m = gs.Matrix()
     m.load_graph("CSC", [T(indptr), T(indices)])
     with pytest.raises(RuntimeError, match="SortCSCIndices"):
