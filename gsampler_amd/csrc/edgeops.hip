@@ -309,7 +309,12 @@ __device__ __forceinline__ float wave_sum_if_uniform(float v, int64_t target,
 }
 
 // Compressed form: tile of consecutive edges; the segments it touches are
-// consecutive, so LDS accumulators are indexed directly.
+// consecutive, so LDS accumulators are indexed directly.  A work-group takes
+// kCscRounds tiles in a row: the look-up of the columns it covers (two
+// dependent chains of loads over indptr) is paid once per 8192 edges.
+constexpr int kCscRounds = 4;
+constexpr int kCscTile = kSumTile * kCscRounds;
+
 __global__ __launch_bounds__(kBlock) void spmm_csc_sum_kernel(
     const int64_t* __restrict__ indptr, const int64_t* __restrict__ indices,
     const int64_t* __restrict__ edge_map, int64_t num_major, int64_t nnz,
@@ -317,10 +322,31 @@ __global__ __launch_bounds__(kBlock) void spmm_csc_sum_kernel(
     const float* __restrict__ efeat, float* out) {
   __shared__ float acc[kSumSegs];
   __shared__ int64_t bounds[kSumSegs + 1];
-  const int64_t tile0 = (int64_t)blockIdx.x * kSumTile;
-  const int64_t tile_end = tile0 + kSumTile < nnz ? tile0 + kSumTile : nnz;
-  const int64_t c0 = segment_of(indptr, num_major, tile0);
-  const int64_t c1 = segment_of(indptr, num_major, tile_end - 1);
+  const int64_t tile0 = (int64_t)blockIdx.x * kCscTile;
+  const int64_t tile_end = tile0 + kCscTile < nnz ? tile0 + kCscTile : nnz;
+  auto load_round = [&](int64_t base, float (&val)[kSumItems]) {
+#pragma unroll
+    for (int i = 0; i < kSumItems; ++i) {
+      const int64_t e = base + i * kBlock + threadIdx.x;
+      val[i] = 0.f;
+      if (e < tile_end) {
+        const int64_t eid = edge_map ? edge_map[e] : e;
+        val[i] = edge_value<float>(kind, op, ufeat ? ufeat + indices[e] : nullptr,
+                                   efeat ? efeat + eid : nullptr);
+      }
+    }
+  };
+  // the first round's values before anything else: their loads are in flight
+  // while the columns are looked up
+  float val[kSumItems];
+  load_round(tile0, val);
+  // both look-ups on the scalar unit; a long column covers the whole tile, and
+  // then the second one is a single comparison
+  const int64_t c0 = segment_of(indptr, num_major, wave_uniform_first(tile0));
+  const int64_t last = wave_uniform_first(tile_end - 1);
+  const int64_t c1 = indptr[c0 + 1] > last
+                         ? c0
+                         : c0 + segment_of(indptr + c0, num_major - c0, last);
   const int64_t nseg = c1 - c0 + 1;
   const bool in_lds = nseg <= kSumSegs;
   if (in_lds) {
@@ -330,34 +356,48 @@ __global__ __launch_bounds__(kBlock) void spmm_csc_sum_kernel(
     }
     __syncthreads();
   }
-  float val[kSumItems];
+  for (int r = 0; r < kCscRounds; ++r) {
+    const int64_t base = tile0 + (int64_t)r * kSumTile;
+    if (base >= tile_end) break;
+    if (r > 0) load_round(base, val);
+    // a round that lies inside one column (any column of 2048 edges or more
+    // has such rounds): the lanes add their values up first, and the
+    // wavefront sends one sum
+    const int64_t round_last = base + kSumTile - 1 < tile_end - 1 ? base + kSumTile - 1
+                                                                : tile_end - 1;
+    const int64_t s_first = in_lds ? segment_of(bounds, nseg, wave_uniform_first(base))
+                                   : segment_of(indptr + c0, nseg, wave_uniform_first(base));
+    const int64_t s_next = in_lds ? bounds[s_first + 1] : indptr[c0 + s_first + 1];
+    if (s_next > round_last) {
+      float mine = 0.f;
 #pragma unroll
-  for (int i = 0; i < kSumItems; ++i) {  // loads first: in flight together
-    const int64_t e = tile0 + i * kBlock + threadIdx.x;
-    val[i] = 0.f;
-    if (e < tile_end) {
-      const int64_t eid = edge_map ? edge_map[e] : e;
-      val[i] = edge_value<float>(kind, op, ufeat ? ufeat + indices[e] : nullptr,
-                                 efeat ? efeat + eid : nullptr);
-    }
-  }
+      for (int i = 0; i < kSumItems; ++i) mine += val[i];   // inactive slots hold 0
 #pragma unroll
-  for (int i = 0; i < kSumItems; ++i) {
-    const int64_t e = tile0 + i * kBlock + threadIdx.x;
-    const bool active = e < tile_end;
-    int64_t seg = 0;
-    if (active)
-      seg = in_lds ? segment_of(bounds, nseg, e) : segment_of(indptr + c0, nseg, e);
-    bool uniform;
-    const float total = wave_sum_if_uniform(val[i], seg, active, &uniform);
-    if (uniform) {
+      for (int d = kWave / 2; d > 0; d >>= 1) mine += __shfl_down(mine, d, kWave);
       if (lane_id() == 0) {
-        if (in_lds) atomicAdd(&acc[seg], total);
-        else unsafeAtomicAdd(out + c0 + seg, total);
+        if (in_lds) atomicAdd(&acc[s_first], mine);
+        else unsafeAtomicAdd(out + c0 + s_first, mine);
       }
-    } else if (active) {
-      if (in_lds) atomicAdd(&acc[seg], val[i]);
-      else unsafeAtomicAdd(out + c0 + seg, val[i]);
+      continue;
+    }
+#pragma unroll
+    for (int i = 0; i < kSumItems; ++i) {
+      const int64_t e = base + i * kBlock + threadIdx.x;
+      const bool active = e < tile_end;
+      int64_t seg = 0;
+      if (active)
+        seg = in_lds ? segment_of(bounds, nseg, e) : segment_of(indptr + c0, nseg, e);
+      bool uniform;
+      const float total = wave_sum_if_uniform(val[i], seg, active, &uniform);
+      if (uniform) {
+        if (lane_id() == 0) {
+          if (in_lds) atomicAdd(&acc[seg], total);
+          else unsafeAtomicAdd(out + c0 + seg, total);
+        }
+      } else if (active) {
+        if (in_lds) atomicAdd(&acc[seg], val[i]);
+        else unsafeAtomicAdd(out + c0 + seg, val[i]);
+      }
     }
   }
   if (!in_lds) return;
@@ -702,7 +742,8 @@ static int spmm_launch(int format, const int64_t* a, const int64_t* b,
                     (int64_t)0));
     } else {
       GS_LAUNCH("spmm_csc_sum", s,
-                spmm_csc_sum_kernel<<<grid, dim3(kBlock), 0, s>>>(
+                spmm_csc_sum_kernel<<<dim3((unsigned)ceil_div(nnz, kCscTile)), dim3(kBlock), 0,
+                                      s>>>(
                     a, b, edge_map, num_major, nnz, kind, op, ufeat, efeat, out));
     }
     return GS_OK;

@@ -4,12 +4,27 @@
 namespace gs {
 
 // Column id of every edge: the segment of indptr that holds the edge position.
+// A work-group takes a tile of consecutive edges, finds the columns of its
+// first and last edge once (on the scalar unit) and searches every edge only
+// among the columns in between; a long column covers whole tiles, which then
+// search nothing at all.
+constexpr int kCooItems = 8;
+constexpr int kCooTile = kBlock * kCooItems;
+
 __global__ __launch_bounds__(kBlock) void csc2coo_kernel(
     const int64_t* __restrict__ indptr, int64_t num_cols, int64_t nnz,
     int64_t* __restrict__ out_col) {
-  const int64_t e = (int64_t)blockIdx.x * kBlock + threadIdx.x;
-  if (e >= nnz) return;
-  out_col[e] = segment_of(indptr, num_cols, e);
+  const int64_t e0 = (int64_t)blockIdx.x * kCooTile;
+  if (e0 >= nnz) return;
+  const int64_t e_last = e0 + kCooTile - 1 < nnz ? e0 + kCooTile - 1 : nnz - 1;
+  const int64_t lo = segment_of(indptr, num_cols, wave_uniform_first(e0));
+  const int64_t hi = segment_of(indptr, num_cols, wave_uniform_first(e_last));
+#pragma unroll
+  for (int j = 0; j < kCooItems; ++j) {
+    const int64_t e = e0 + j * kBlock + threadIdx.x;
+    if (e >= nnz) break;
+    out_col[e] = lo == hi ? lo : lo + segment_of(indptr + lo, hi - lo + 1, e);
+  }
 }
 
 // indptr[c] = number of entries of the sorted column array that are < c.
@@ -102,7 +117,7 @@ int gs_csc2coo(const int64_t* indptr, int64_t num_cols, int64_t nnz,
   GS_REQUIRE(num_cols > 0, "csc2coo: %lld edges but no columns", (long long)nnz);
   hipStream_t s = as_stream(stream);
   GS_LAUNCH("csc2coo", s,
-            csc2coo_kernel<<<dim3((unsigned)ceil_div(nnz, kBlock)), dim3(kBlock),
+            csc2coo_kernel<<<dim3((unsigned)ceil_div(nnz, kCooTile)), dim3(kBlock),
                              0, s>>>(indptr, num_cols, nnz, out_col));
   return GS_OK;
 }

@@ -252,28 +252,58 @@ __global__ __launch_bounds__(kBlock) void sample_weighted_replace_kernel(
 // owns [cdf[indptr[c]], cdf[indptr[c + 1]]).  Built once per (matrix, weights),
 // it turns a weighted draw into a search over O(log deg) entries instead of a
 // pass over the column.
+// Both passes take tiles of consecutive edges and look the tile's first and
+// last column up once, on the scalar unit; an edge then searches only among
+// the columns of its tile instead of all of them.
+constexpr int kCdfItems = 8;
+constexpr int kCdfTile = kBlock * kCdfItems;
+
+struct ColumnSpan {
+  int64_t lo, hi;
+  __device__ __forceinline__ int64_t column_of(const int64_t* __restrict__ indptr,
+                                               int64_t e) const {
+    return lo == hi ? lo : lo + segment_of(indptr + lo, hi - lo + 1, e);
+  }
+};
+__device__ __forceinline__ ColumnSpan column_span(const int64_t* __restrict__ indptr,
+                                                  int64_t num_cols, int64_t e0, int64_t e_last) {
+  ColumnSpan s;
+  s.lo = segment_of(indptr, num_cols, wave_uniform_first(e0));
+  s.hi = segment_of(indptr, num_cols, wave_uniform_first(e_last));
+  return s;
+}
+
 __global__ __launch_bounds__(kBlock) void cdf_colmax_kernel(
     const int64_t* __restrict__ indptr, int64_t num_cols,
     const float* __restrict__ probs, int64_t nnz, unsigned int* colmax_bits) {
-  const int64_t e = (int64_t)blockIdx.x * kBlock + threadIdx.x;
-  const bool active = e < nnz;
-  int64_t c = -1;
-  float w = 0.0f;
-  if (active) {
-    c = segment_of(indptr, num_cols, e);
-    w = probs[e];
-  }
-  // positive floats order like their bit patterns
-  const int64_t c0 = wave_uniform_first(c);
-  if (__all(active && c == c0)) {
+  const int64_t e0 = (int64_t)blockIdx.x * kCdfTile;
+  if (e0 >= nnz) return;
+  const int64_t e_last = e0 + kCdfTile - 1 < nnz ? e0 + kCdfTile - 1 : nnz - 1;
+  float w[kCdfItems];
 #pragma unroll
-    for (int d = kWave / 2; d > 0; d >>= 1) {
-      const float o = __shfl_xor(w, d, kWave);
-      if (o > w) w = o;
+  for (int j = 0; j < kCdfItems; ++j) {
+    const int64_t e = e0 + j * kBlock + threadIdx.x;
+    w[j] = e <= e_last ? probs[e] : 0.0f;
+  }
+  const ColumnSpan span = column_span(indptr, num_cols, e0, e_last);
+#pragma unroll
+  for (int j = 0; j < kCdfItems; ++j) {
+    const int64_t e = e0 + j * kBlock + threadIdx.x;
+    const bool active = e <= e_last;
+    const int64_t c = active ? span.column_of(indptr, e) : -1;
+    float m = w[j];
+    // positive floats order like their bit patterns
+    const int64_t c0 = wave_uniform_first(c);
+    if (__all(active && c == c0)) {
+#pragma unroll
+      for (int d = kWave / 2; d > 0; d >>= 1) {
+        const float o = __shfl_xor(m, d, kWave);
+        if (o > m) m = o;
+      }
+      if (lane_id() == 0 && m > 0.0f) atomicMax(colmax_bits + c, __float_as_uint(m));
+    } else if (active && m > 0.0f) {
+      atomicMax(colmax_bits + c, __float_as_uint(m));
     }
-    if (lane_id() == 0 && w > 0.0f) atomicMax(colmax_bits + c, __float_as_uint(w));
-  } else if (active && w > 0.0f) {
-    atomicMax(colmax_bits + c, __float_as_uint(w));
   }
 }
 
@@ -281,14 +311,24 @@ __global__ __launch_bounds__(kBlock) void cdf_quantise_kernel(
     const int64_t* __restrict__ indptr, int64_t num_cols,
     const float* __restrict__ probs, int64_t nnz,
     const unsigned int* __restrict__ colmax_bits, int64_t* __restrict__ cdf) {
-  const int64_t e = (int64_t)blockIdx.x * kBlock + threadIdx.x;
-  if (e > nnz) return;
-  uint64_t q = 0;
-  if (e < nnz) {
-    const float wmax = __uint_as_float(colmax_bits[segment_of(indptr, num_cols, e)]);
-    if (wmax > 0.0f) q = quantise(probs[e], det_div(2147483648.0, (double)wmax));
+  const int64_t e0 = (int64_t)blockIdx.x * kCdfTile;
+  if (e0 > nnz) return;
+  if (e0 == nnz) {  // cdf[nnz] = 0 closes the exclusive scan
+    if (threadIdx.x == 0) cdf[nnz] = 0;
+    return;
   }
-  cdf[e] = (int64_t)q;  // cdf[nnz] = 0 closes the exclusive scan
+  const int64_t e_last = e0 + kCdfTile - 1 < nnz ? e0 + kCdfTile - 1 : nnz - 1;
+  const ColumnSpan span = column_span(indptr, num_cols, e0, e_last);
+#pragma unroll
+  for (int j = 0; j < kCdfItems; ++j) {
+    const int64_t e = e0 + j * kBlock + threadIdx.x;
+    if (e > e_last) break;
+    uint64_t q = 0;
+    const float wmax = __uint_as_float(colmax_bits[span.column_of(indptr, e)]);
+    if (wmax > 0.0f) q = quantise(probs[e], det_div(2147483648.0, (double)wmax));
+    cdf[e] = (int64_t)q;
+  }
+  if (e_last == nnz - 1 && threadIdx.x == 0) cdf[nnz] = 0;
 }
 
 __global__ __launch_bounds__(kBlock) void cdf_zero_kernel(unsigned int* p, int64_t n) {
@@ -687,10 +727,10 @@ int gs_weight_cdf_build(const int64_t* indptr, int64_t num_cols, const float* pr
                                 0, s>>>(colmax, num_cols));
   if (nnz > 0)
     GS_LAUNCH("cdf_colmax", s,
-              cdf_colmax_kernel<<<dim3((unsigned)ceil_div(nnz, kBlock)), dim3(kBlock), 0,
+              cdf_colmax_kernel<<<dim3((unsigned)ceil_div(nnz, kCdfTile)), dim3(kBlock), 0,
                                   s>>>(indptr, num_cols, probs, nnz, colmax));
   GS_LAUNCH("cdf_quantise", s,
-            cdf_quantise_kernel<<<dim3((unsigned)ceil_div(nnz + 1, kBlock)), dim3(kBlock),
+            cdf_quantise_kernel<<<dim3((unsigned)ceil_div(nnz + 1, kCdfTile)), dim3(kBlock),
                                   0, s>>>(indptr, num_cols, probs, nnz, colmax, cdf));
   return exclusive_scan_i64(cdf, cdf, nnz + 1, scan_ws, workspace_bytes - colmax_bytes, s);
 }
