@@ -273,9 +273,16 @@ __device__ __forceinline__ ColumnSpan column_span(const int64_t* __restrict__ in
   return s;
 }
 
+// Column maxima: the tile's maxima are first taken in LDS (integer atomics on
+// the bit patterns: positive floats order like their bits), then every column
+// the tile touches sends one atomic to memory.  With one atomic per edge the
+// pass ran at the rate of the memory-side atomic units.
+constexpr int kCdfSegs = 4096;
+
 __global__ __launch_bounds__(kBlock) void cdf_colmax_kernel(
     const int64_t* __restrict__ indptr, int64_t num_cols,
     const float* __restrict__ probs, int64_t nnz, unsigned int* colmax_bits) {
+  __shared__ unsigned int tile_max[kCdfSegs];
   const int64_t e0 = (int64_t)blockIdx.x * kCdfTile;
   if (e0 >= nnz) return;
   const int64_t e_last = e0 + kCdfTile - 1 < nnz ? e0 + kCdfTile - 1 : nnz - 1;
@@ -286,25 +293,24 @@ __global__ __launch_bounds__(kBlock) void cdf_colmax_kernel(
     w[j] = e <= e_last ? probs[e] : 0.0f;
   }
   const ColumnSpan span = column_span(indptr, num_cols, e0, e_last);
+  const int64_t nseg = span.hi - span.lo + 1;
+  const bool in_lds = nseg <= kCdfSegs;
+  if (in_lds) {
+    for (int64_t j = threadIdx.x; j < nseg; j += kBlock) tile_max[j] = 0u;
+    __syncthreads();
+  }
 #pragma unroll
   for (int j = 0; j < kCdfItems; ++j) {
     const int64_t e = e0 + j * kBlock + threadIdx.x;
-    const bool active = e <= e_last;
-    const int64_t c = active ? span.column_of(indptr, e) : -1;
-    float m = w[j];
-    // positive floats order like their bit patterns
-    const int64_t c0 = wave_uniform_first(c);
-    if (__all(active && c == c0)) {
-#pragma unroll
-      for (int d = kWave / 2; d > 0; d >>= 1) {
-        const float o = __shfl_xor(m, d, kWave);
-        if (o > m) m = o;
-      }
-      if (lane_id() == 0 && m > 0.0f) atomicMax(colmax_bits + c, __float_as_uint(m));
-    } else if (active && m > 0.0f) {
-      atomicMax(colmax_bits + c, __float_as_uint(m));
-    }
+    if (e > e_last || !(w[j] > 0.0f)) continue;
+    const int64_t c = span.column_of(indptr, e);
+    if (in_lds) atomicMax(&tile_max[c - span.lo], __float_as_uint(w[j]));
+    else atomicMax(colmax_bits + c, __float_as_uint(w[j]));
   }
+  if (!in_lds) return;
+  __syncthreads();
+  for (int64_t j = threadIdx.x; j < nseg; j += kBlock)
+    if (tile_max[j] != 0u) atomicMax(colmax_bits + span.lo + j, tile_max[j]);
 }
 
 __global__ __launch_bounds__(kBlock) void cdf_quantise_kernel(
