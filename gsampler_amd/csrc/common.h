@@ -183,6 +183,25 @@ __device__ __forceinline__ int64_t segment_of(const int64_t* ptr, int64_t n,
   return lo;
 }
 
+// Segments that a tile of consecutive positions [p0, p_last] touches.  The two
+// look-ups run once per wavefront on the scalar unit (p0 and p_last are the
+// same in every lane); a position of the tile is then searched only among the
+// segments in between, and not at all when one segment covers the tile.
+struct SegmentSpan {
+  int64_t lo, hi;
+  __device__ __forceinline__ int64_t segment_at(const int64_t* __restrict__ ptr,
+                                                int64_t p) const {
+    return lo == hi ? lo : lo + segment_of(ptr + lo, hi - lo + 1, p);
+  }
+};
+__device__ __forceinline__ SegmentSpan segment_span(const int64_t* __restrict__ ptr, int64_t n,
+                                                    int64_t p0, int64_t p_last) {
+  SegmentSpan s;
+  s.lo = segment_of(ptr, n, wave_uniform_first(p0));
+  s.hi = segment_of(ptr, n, wave_uniform_first(p_last));
+  return s;
+}
+
 __device__ __forceinline__ int64_t column_degree(const int64_t* indptr,
                                                  int64_t num_cols, int64_t c,
                                                  int64_t* in_start) {

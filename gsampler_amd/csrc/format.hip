@@ -3,11 +3,8 @@
 
 namespace gs {
 
-// Column id of every edge: the segment of indptr that holds the edge position.
-// A work-group takes a tile of consecutive edges, finds the columns of its
-// first and last edge once (on the scalar unit) and searches every edge only
-// among the columns in between; a long column covers whole tiles, which then
-// search nothing at all.
+// Column id of every edge: the segment of indptr that holds the edge position,
+// looked up per tile of consecutive edges.
 constexpr int kCooItems = 8;
 constexpr int kCooTile = kBlock * kCooItems;
 
@@ -17,13 +14,12 @@ __global__ __launch_bounds__(kBlock) void csc2coo_kernel(
   const int64_t e0 = (int64_t)blockIdx.x * kCooTile;
   if (e0 >= nnz) return;
   const int64_t e_last = e0 + kCooTile - 1 < nnz ? e0 + kCooTile - 1 : nnz - 1;
-  const int64_t lo = segment_of(indptr, num_cols, wave_uniform_first(e0));
-  const int64_t hi = segment_of(indptr, num_cols, wave_uniform_first(e_last));
+  const SegmentSpan span = segment_span(indptr, num_cols, e0, e_last);
 #pragma unroll
   for (int j = 0; j < kCooItems; ++j) {
     const int64_t e = e0 + j * kBlock + threadIdx.x;
     if (e >= nnz) break;
-    out_col[e] = lo == hi ? lo : lo + segment_of(indptr + lo, hi - lo + 1, e);
+    out_col[e] = span.segment_at(indptr, e);
   }
 }
 

@@ -46,17 +46,14 @@ __global__ __launch_bounds__(kBlock) void col_slice_fill_kernel(
   const int64_t e_last = e0 + kSliceTile - 1 < nnz ? e0 + kSliceTile - 1 : nnz - 1;
   // columns that the tile touches: one search per work-group (on the scalar
   // unit) instead of one per edge; a long column covers whole tiles
-  const int64_t item_lo = segment_of(sub_indptr, num_items, wave_uniform_first(e0));
-  const int64_t item_hi = segment_of(sub_indptr, num_items, wave_uniform_first(e_last));
+  const SegmentSpan span = segment_span(sub_indptr, num_items, e0, e_last);
   int64_t item[kSliceItems], in_pos[kSliceItems], row[kSliceItems];
 #pragma unroll
   for (int j = 0; j < kSliceItems; ++j) {
     const int64_t e = e0 + j * kBlock + threadIdx.x;
     item[j] = -1;
     if (e >= nnz) continue;
-    item[j] = item_lo == item_hi
-                  ? item_lo
-                  : item_lo + segment_of(sub_indptr + item_lo, item_hi - item_lo + 1, e);
+    item[j] = span.segment_at(sub_indptr, e);
     const int64_t c = column_ids ? column_ids[item[j]] : item[j];
     in_pos[j] = indptr[c] + (e - sub_indptr[item[j]]);
   }

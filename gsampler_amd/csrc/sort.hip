@@ -23,14 +23,23 @@ static int id_bits(int64_t num_ids) {
 // is already grouped by segment; it moves every key a fixed number of times
 // whatever the segment sizes are, where a segmented sort of millions of short
 // segments and a few hubs spends its time on scheduling them.
+constexpr int kPackItems = 8;
+constexpr int kPackTile = kBlock * kPackItems;
+
 __global__ __launch_bounds__(kBlock) void pack_segment_keys_kernel(
     const int64_t* __restrict__ indptr, int64_t num_segments,
     const int64_t* __restrict__ keys, int64_t nnz, int key_bits,
     uint64_t* __restrict__ packed) {
-  const int64_t e = (int64_t)blockIdx.x * kBlock + threadIdx.x;
-  if (e >= nnz) return;
-  const uint64_t seg = (uint64_t)segment_of(indptr, num_segments, e);
-  packed[e] = (seg << key_bits) | (uint64_t)keys[e];
+  const int64_t e0 = (int64_t)blockIdx.x * kPackTile;
+  if (e0 >= nnz) return;
+  const int64_t e_last = e0 + kPackTile - 1 < nnz ? e0 + kPackTile - 1 : nnz - 1;
+  const SegmentSpan span = segment_span(indptr, num_segments, e0, e_last);
+#pragma unroll
+  for (int j = 0; j < kPackItems; ++j) {
+    const int64_t e = e0 + j * kBlock + threadIdx.x;
+    if (e > e_last) break;
+    packed[e] = ((uint64_t)span.segment_at(indptr, e) << key_bits) | (uint64_t)keys[e];
+  }
 }
 
 __global__ __launch_bounds__(kBlock) void unpack_segment_keys_kernel(
@@ -116,8 +125,8 @@ int gs_segment_sort_i64(const int64_t* indptr, int64_t num_segments,
   size_t temp_bytes = workspace_bytes - packed_bytes;
   const dim3 grid((unsigned)ceil_div(nnz, kBlock));
   GS_LAUNCH("segment_sort_pack", s,
-            pack_segment_keys_kernel<<<grid, dim3(kBlock), 0, s>>>(indptr, num_segments, keys_in,
-                                                                  nnz, key_bits, packed));
+            pack_segment_keys_kernel<<<dim3((unsigned)ceil_div(nnz, kPackTile)), dim3(kBlock), 0,
+                                       s>>>(indptr, num_segments, keys_in, nnz, key_bits, packed));
   {
     ProfScope ps("segment_sort", s);
     GS_HIP(rocprim::radix_sort_keys(temp, temp_bytes, packed, (uint64_t*)keys_out, (size_t)nnz,

@@ -258,21 +258,6 @@ __global__ __launch_bounds__(kBlock) void sample_weighted_replace_kernel(
 constexpr int kCdfItems = 8;
 constexpr int kCdfTile = kBlock * kCdfItems;
 
-struct ColumnSpan {
-  int64_t lo, hi;
-  __device__ __forceinline__ int64_t column_of(const int64_t* __restrict__ indptr,
-                                               int64_t e) const {
-    return lo == hi ? lo : lo + segment_of(indptr + lo, hi - lo + 1, e);
-  }
-};
-__device__ __forceinline__ ColumnSpan column_span(const int64_t* __restrict__ indptr,
-                                                  int64_t num_cols, int64_t e0, int64_t e_last) {
-  ColumnSpan s;
-  s.lo = segment_of(indptr, num_cols, wave_uniform_first(e0));
-  s.hi = segment_of(indptr, num_cols, wave_uniform_first(e_last));
-  return s;
-}
-
 // Column maxima: the tile's maxima are first taken in LDS (integer atomics on
 // the bit patterns: positive floats order like their bits), then every column
 // the tile touches sends one atomic to memory.  With one atomic per edge the
@@ -292,7 +277,7 @@ __global__ __launch_bounds__(kBlock) void cdf_colmax_kernel(
     const int64_t e = e0 + j * kBlock + threadIdx.x;
     w[j] = e <= e_last ? probs[e] : 0.0f;
   }
-  const ColumnSpan span = column_span(indptr, num_cols, e0, e_last);
+  const SegmentSpan span = segment_span(indptr, num_cols, e0, e_last);
   const int64_t nseg = span.hi - span.lo + 1;
   const bool in_lds = nseg <= kCdfSegs;
   if (in_lds) {
@@ -303,7 +288,7 @@ __global__ __launch_bounds__(kBlock) void cdf_colmax_kernel(
   for (int j = 0; j < kCdfItems; ++j) {
     const int64_t e = e0 + j * kBlock + threadIdx.x;
     if (e > e_last || !(w[j] > 0.0f)) continue;
-    const int64_t c = span.column_of(indptr, e);
+    const int64_t c = span.segment_at(indptr, e);
     if (in_lds) atomicMax(&tile_max[c - span.lo], __float_as_uint(w[j]));
     else atomicMax(colmax_bits + c, __float_as_uint(w[j]));
   }
@@ -324,13 +309,13 @@ __global__ __launch_bounds__(kBlock) void cdf_quantise_kernel(
     return;
   }
   const int64_t e_last = e0 + kCdfTile - 1 < nnz ? e0 + kCdfTile - 1 : nnz - 1;
-  const ColumnSpan span = column_span(indptr, num_cols, e0, e_last);
+  const SegmentSpan span = segment_span(indptr, num_cols, e0, e_last);
 #pragma unroll
   for (int j = 0; j < kCdfItems; ++j) {
     const int64_t e = e0 + j * kBlock + threadIdx.x;
     if (e > e_last) break;
     uint64_t q = 0;
-    const float wmax = __uint_as_float(colmax_bits[span.column_of(indptr, e)]);
+    const float wmax = __uint_as_float(colmax_bits[span.segment_at(indptr, e)]);
     if (wmax > 0.0f) q = quantise(probs[e], det_div(2147483648.0, (double)wmax));
     cdf[e] = (int64_t)q;
   }
