@@ -431,8 +431,12 @@ def run_ops(args, wl, capi, dev):
             lambda: capi.spmm(csc_view, "copy_rhs", "sum", None, e_w, 0, S2), 4 * sl_nnz + 12 * S2,
             f"{sl_nnz} edges onto {S2} columns")
     col_sum = capi.spmm(csc_view, "copy_rhs", "sum", None, e_w, 0, S2)
-    measure("edge / column value", "SDDMMCOO", lambda: capi.sddmm(coo_view, "div", e_w, col_sum, 1, 2),
+    measure("edge / column value (edge list)", "SDDMMCOO",
+            lambda: capi.sddmm(coo_view, "div", e_w, col_sum, 1, 2),
             24 * sl_nnz, f"{sl_nnz} edges")
+    measure("edge / column value (compressed)", "SDDMMCSC",
+            lambda: capi.sddmm(csc_view, "div", e_w, col_sum, 1, 2), 16 * sl_nnz + 16 * S2,
+            f"{sl_nnz} edges")
     measure("edges' columns from offsets", "CSC2COOCUDA", lambda: capi.csc2coo(sl[0], sl_nnz),
             8 * S2 + 8 * sl_nnz, f"{sl_nnz} edges")
     del sl, e_w, col_sum, coo_view, csc_view

@@ -46,11 +46,17 @@ struct EdgeView {
   const int64_t* b;    // col | indices
   int64_t num_major;   // segments of indptr
   const int64_t* edge_map;
-  __device__ __forceinline__ void endpoints(int64_t e, int64_t* src,
+  // Segments that the edges [e_first, e_last] of one work-group touch
+  // (compressed form only): looked up once, on the scalar unit.
+  __device__ __forceinline__ SegmentSpan span(int64_t e_first, int64_t e_last) const {
+    if (!compressed) return SegmentSpan{0, 0};
+    return segment_span(a, num_major, e_first, e_last);
+  }
+  __device__ __forceinline__ void endpoints(const SegmentSpan& sp, int64_t e, int64_t* src,
                                             int64_t* dst, int64_t* eid) const {
     if (compressed) {
       *src = b[e];
-      *dst = segment_of(a, num_major, e);
+      *dst = sp.segment_at(a, e);
     } else {
       *src = a[e];
       *dst = b[e];
@@ -58,6 +64,20 @@ struct EdgeView {
     *eid = edge_map ? edge_map[e] : e;
   }
 };
+
+// A work-group handles kEdgeTile consecutive elements of an [nnz, out_len]
+// output, kEdgeItems per thread, so that the look-up of the segments its edges
+// touch is paid once per 2048 elements.
+constexpr int kEdgeItems = 8;
+constexpr int kEdgeTile = kBlock * kEdgeItems;
+
+__device__ __forceinline__ SegmentSpan block_edge_span(const EdgeView& g, int64_t nnz,
+                                                       int64_t out_len) {
+  const int64_t idx0 = (int64_t)blockIdx.x * kEdgeTile;
+  int64_t idx_last = idx0 + kEdgeTile - 1;
+  if (idx_last > nnz * out_len - 1) idx_last = nnz * out_len - 1;
+  return g.span(idx0 / out_len, idx_last / out_len);
+}
 
 // ------------------------------------------------------------------ SDDMM
 template <typename T>
@@ -67,19 +87,25 @@ __global__ __launch_bounds__(kBlock) void sddmm_kernel(
     int rhs_target, int64_t lhs_len, int64_t rhs_len, int64_t out_len,
     int64_t reduce_size, const int64_t* __restrict__ lhs_off,
     const int64_t* __restrict__ rhs_off) {
-  const int64_t idx = (int64_t)blockIdx.x * kBlock + threadIdx.x;
-  if (idx >= nnz * out_len) return;
-  const int64_t e = idx / out_len, f = idx - e * out_len;
-  int64_t src, dst, eid;
-  g.endpoints(e, &src, &dst, &eid);
-  const int64_t lf = lhs_off ? lhs_off[f] : f, rf = rhs_off ? rhs_off[f] : f;
-  const T* l = op == kOpCopyRhs
-                   ? nullptr
-                   : lhs + pick(lhs_target, src, eid, dst) * lhs_len + lf * reduce_size;
-  const T* r = op == kOpCopyLhs
-                   ? nullptr
-                   : rhs + pick(rhs_target, src, eid, dst) * rhs_len + rf * reduce_size;
-  out[eid * out_len + f] = apply_op<T>(op, l, r, reduce_size);
+  const int64_t idx0 = (int64_t)blockIdx.x * kEdgeTile;
+  if (idx0 >= nnz * out_len) return;
+  const SegmentSpan sp = block_edge_span(g, nnz, out_len);
+#pragma unroll
+  for (int j = 0; j < kEdgeItems; ++j) {
+    const int64_t idx = idx0 + j * kBlock + threadIdx.x;
+    if (idx >= nnz * out_len) break;
+    const int64_t e = idx / out_len, f = idx - e * out_len;
+    int64_t src, dst, eid;
+    g.endpoints(sp, e, &src, &dst, &eid);
+    const int64_t lf = lhs_off ? lhs_off[f] : f, rf = rhs_off ? rhs_off[f] : f;
+    const T* l = op == kOpCopyRhs
+                     ? nullptr
+                     : lhs + pick(lhs_target, src, eid, dst) * lhs_len + lf * reduce_size;
+    const T* r = op == kOpCopyLhs
+                     ? nullptr
+                     : rhs + pick(rhs_target, src, eid, dst) * rhs_len + rf * reduce_size;
+    out[eid * out_len + f] = apply_op<T>(op, l, r, reduce_size);
+  }
 }
 
 // Two SDDMMs (u op v) that share one edge sweep.
@@ -91,17 +117,23 @@ __global__ __launch_bounds__(kBlock) void fused_u_op_v_kernel(
     T* __restrict__ out2, int64_t lhs_len, int64_t rhs_len, int64_t out_len,
     int64_t reduce_size, const int64_t* __restrict__ lhs_off,
     const int64_t* __restrict__ rhs_off) {
-  const int64_t idx = (int64_t)blockIdx.x * kBlock + threadIdx.x;
-  if (idx >= nnz * out_len) return;
-  const int64_t e = idx / out_len, f = idx - e * out_len;
-  int64_t src, dst, eid;
-  g.endpoints(e, &src, &dst, &eid);
-  const int64_t lf = (lhs_off ? lhs_off[f] : f) * reduce_size;
-  const int64_t rf = (rhs_off ? rhs_off[f] : f) * reduce_size;
-  out1[eid * out_len + f] = apply_op<T>(op, lhs1 + src * lhs_len + lf,
-                                        rhs1 + dst * rhs_len + rf, reduce_size);
-  out2[eid * out_len + f] = apply_op<T>(op, lhs2 + src * lhs_len + lf,
-                                        rhs2 + dst * rhs_len + rf, reduce_size);
+  const int64_t idx0 = (int64_t)blockIdx.x * kEdgeTile;
+  if (idx0 >= nnz * out_len) return;
+  const SegmentSpan sp = block_edge_span(g, nnz, out_len);
+#pragma unroll
+  for (int j = 0; j < kEdgeItems; ++j) {
+    const int64_t idx = idx0 + j * kBlock + threadIdx.x;
+    if (idx >= nnz * out_len) break;
+    const int64_t e = idx / out_len, f = idx - e * out_len;
+    int64_t src, dst, eid;
+    g.endpoints(sp, e, &src, &dst, &eid);
+    const int64_t lf = (lhs_off ? lhs_off[f] : f) * reduce_size;
+    const int64_t rf = (rhs_off ? rhs_off[f] : f) * reduce_size;
+    out1[eid * out_len + f] = apply_op<T>(op, lhs1 + src * lhs_len + lf,
+                                          rhs1 + dst * rhs_len + rf, reduce_size);
+    out2[eid * out_len + f] = apply_op<T>(op, lhs2 + src * lhs_len + lf,
+                                          rhs2 + dst * rhs_len + rf, reduce_size);
+  }
 }
 
 // ------------------------------------------------------------------- SpMM
@@ -811,7 +843,7 @@ int gs_sddmm(int format, const int64_t* a, const int64_t* b, int64_t num_major,
              "sddmm: null operand");
   hipStream_t s = as_stream(stream);
   const EdgeView g{format == GS_FMT_COMPRESSED, a, b, num_major, edge_map};
-  const unsigned blocks = (unsigned)ceil_div(nnz * out_len, kBlock);
+  const unsigned blocks = (unsigned)ceil_div(nnz * out_len, kEdgeTile);
   if (dtype == GS_F32)
     GS_LAUNCH("sddmm", s,
               sddmm_kernel<float><<<dim3(blocks), dim3(kBlock), 0, s>>>(
@@ -844,7 +876,7 @@ int gs_fused_u_op_v(int format, const int64_t* a, const int64_t* b,
   GS_REQUIRE(lhs1 && rhs1 && out1 && lhs2 && rhs2 && out2, "fused_u_op_v: null operand");
   hipStream_t s = as_stream(stream);
   const EdgeView g{format == GS_FMT_COMPRESSED, a, b, num_major, nullptr};
-  const unsigned blocks = (unsigned)ceil_div(nnz * out_len, kBlock);
+  const unsigned blocks = (unsigned)ceil_div(nnz * out_len, kEdgeTile);
   if (dtype == GS_F32)
     GS_LAUNCH("fused_u_op_v", s,
               fused_u_op_v_kernel<float><<<dim3(blocks), dim3(kBlock), 0, s>>>(
