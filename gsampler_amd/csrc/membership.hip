@@ -33,11 +33,15 @@ struct MemberWs {
   size_t total;
 };
 
-// Slots of the table: four per picked id while that still fits in LDS (fewer
-// probes for the ids that are not there, which are most), else two.
+// Slots of the table: four per picked id (fewer probes for the ids that are
+// not there, which are most: 1.4 instead of 2.5 on average) while the table
+// fits in LDS or stays a small part of a die's L2, else two.
+constexpr int64_t kMemberRoomyIds = 65536;   // 4 slots * 8 B * 65536 = 2 MB
 static uint64_t member_table_slots(int64_t num_picked) {
-  const uint64_t roomy = (uint64_t)(4 * num_picked + 2);
-  return roomy <= (uint64_t)kMemberLdsSlots ? roomy : (uint64_t)(2 * num_picked + 2);
+  const uint64_t roomy = (uint64_t)(4 * num_picked + 2), tight = (uint64_t)(2 * num_picked + 2);
+  if (roomy <= (uint64_t)kMemberLdsSlots) return roomy;   // in LDS, roomy
+  if (tight <= (uint64_t)kMemberLdsSlots) return tight;   // still in LDS
+  return num_picked <= kMemberRoomyIds ? roomy : tight;   // in L2
 }
 
 static MemberWs carve_member(void* ws, int64_t nnz, int64_t num_picked) {
