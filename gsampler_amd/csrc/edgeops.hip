@@ -65,33 +65,34 @@ struct EdgeView {
   }
 };
 
-// A work-group handles kEdgeTile consecutive elements of an [nnz, out_len]
-// output, kEdgeItems per thread, so that the look-up of the segments its edges
-// touch is paid once per 2048 elements.
+// A work-group handles kBlock * ITEMS consecutive elements of an
+// [nnz, out_len] output.  On a compressed form ITEMS = kEdgeItems, so that the
+// look-up of the segments its edges touch is paid once per 2048 elements; an
+// edge list needs no look-up and runs with one element per thread.
 constexpr int kEdgeItems = 8;
-constexpr int kEdgeTile = kBlock * kEdgeItems;
 
+template <int ITEMS>
 __device__ __forceinline__ SegmentSpan block_edge_span(const EdgeView& g, int64_t nnz,
                                                        int64_t out_len) {
-  const int64_t idx0 = (int64_t)blockIdx.x * kEdgeTile;
-  int64_t idx_last = idx0 + kEdgeTile - 1;
+  const int64_t idx0 = (int64_t)blockIdx.x * (kBlock * ITEMS);
+  int64_t idx_last = idx0 + kBlock * ITEMS - 1;
   if (idx_last > nnz * out_len - 1) idx_last = nnz * out_len - 1;
   return g.span(idx0 / out_len, idx_last / out_len);
 }
 
 // ------------------------------------------------------------------ SDDMM
-template <typename T>
+template <typename T, int ITEMS>
 __global__ __launch_bounds__(kBlock) void sddmm_kernel(
     EdgeView g, int64_t nnz, int op, const T* __restrict__ lhs,
     const T* __restrict__ rhs, T* __restrict__ out, int lhs_target,
     int rhs_target, int64_t lhs_len, int64_t rhs_len, int64_t out_len,
     int64_t reduce_size, const int64_t* __restrict__ lhs_off,
     const int64_t* __restrict__ rhs_off) {
-  const int64_t idx0 = (int64_t)blockIdx.x * kEdgeTile;
+  const int64_t idx0 = (int64_t)blockIdx.x * (kBlock * ITEMS);
   if (idx0 >= nnz * out_len) return;
-  const SegmentSpan sp = block_edge_span(g, nnz, out_len);
+  const SegmentSpan sp = block_edge_span<ITEMS>(g, nnz, out_len);
 #pragma unroll
-  for (int j = 0; j < kEdgeItems; ++j) {
+  for (int j = 0; j < ITEMS; ++j) {
     const int64_t idx = idx0 + j * kBlock + threadIdx.x;
     if (idx >= nnz * out_len) break;
     const int64_t e = idx / out_len, f = idx - e * out_len;
@@ -109,7 +110,7 @@ __global__ __launch_bounds__(kBlock) void sddmm_kernel(
 }
 
 // Two SDDMMs (u op v) that share one edge sweep.
-template <typename T>
+template <typename T, int ITEMS>
 __global__ __launch_bounds__(kBlock) void fused_u_op_v_kernel(
     EdgeView g, int64_t nnz, int op, const T* __restrict__ lhs1,
     const T* __restrict__ rhs1, T* __restrict__ out1,
@@ -117,11 +118,11 @@ __global__ __launch_bounds__(kBlock) void fused_u_op_v_kernel(
     T* __restrict__ out2, int64_t lhs_len, int64_t rhs_len, int64_t out_len,
     int64_t reduce_size, const int64_t* __restrict__ lhs_off,
     const int64_t* __restrict__ rhs_off) {
-  const int64_t idx0 = (int64_t)blockIdx.x * kEdgeTile;
+  const int64_t idx0 = (int64_t)blockIdx.x * (kBlock * ITEMS);
   if (idx0 >= nnz * out_len) return;
-  const SegmentSpan sp = block_edge_span(g, nnz, out_len);
+  const SegmentSpan sp = block_edge_span<ITEMS>(g, nnz, out_len);
 #pragma unroll
-  for (int j = 0; j < kEdgeItems; ++j) {
+  for (int j = 0; j < ITEMS; ++j) {
     const int64_t idx = idx0 + j * kBlock + threadIdx.x;
     if (idx >= nnz * out_len) break;
     const int64_t e = idx / out_len, f = idx - e * out_len;
@@ -341,21 +342,22 @@ __device__ __forceinline__ float wave_sum_if_uniform(float v, int64_t target,
 }
 
 // Compressed form: tile of consecutive edges; the segments it touches are
-// consecutive, so LDS accumulators are indexed directly.  A work-group takes
-// kCscRounds tiles in a row: the look-up of the columns it covers (two
-// dependent chains of loads over indptr) is paid once per 8192 edges.
+// consecutive, so LDS accumulators are indexed directly.  On large inputs a
+// work-group takes kCscRounds tiles in a row: the look-up of the columns it
+// covers (two dependent chains of loads over indptr) is then paid once per
+// 8192 edges.
 constexpr int kCscRounds = 4;
-constexpr int kCscTile = kSumTile * kCscRounds;
 
 __global__ __launch_bounds__(kBlock) void spmm_csc_sum_kernel(
     const int64_t* __restrict__ indptr, const int64_t* __restrict__ indices,
     const int64_t* __restrict__ edge_map, int64_t num_major, int64_t nnz,
     int kind, int op, const float* __restrict__ ufeat,
-    const float* __restrict__ efeat, float* out) {
+    const float* __restrict__ efeat, float* out, int rounds) {
   __shared__ float acc[kSumSegs];
   __shared__ int64_t bounds[kSumSegs + 1];
-  const int64_t tile0 = (int64_t)blockIdx.x * kCscTile;
-  const int64_t tile_end = tile0 + kCscTile < nnz ? tile0 + kCscTile : nnz;
+  const int64_t tile_len = (int64_t)kSumTile * rounds;
+  const int64_t tile0 = (int64_t)blockIdx.x * tile_len;
+  const int64_t tile_end = tile0 + tile_len < nnz ? tile0 + tile_len : nnz;
   auto load_round = [&](int64_t base, float (&val)[kSumItems]) {
 #pragma unroll
     for (int i = 0; i < kSumItems; ++i) {
@@ -388,7 +390,7 @@ __global__ __launch_bounds__(kBlock) void spmm_csc_sum_kernel(
     }
     __syncthreads();
   }
-  for (int r = 0; r < kCscRounds; ++r) {
+  for (int r = 0; r < rounds; ++r) {
     const int64_t base = tile0 + (int64_t)r * kSumTile;
     if (base >= tile_end) break;
     if (r > 0) load_round(base, val);
@@ -776,10 +778,12 @@ static int spmm_launch(int format, const int64_t* a, const int64_t* b,
                     a, b, edge_map, nnz, kind, op, ufeat, efeat, out, u_target,
                     (int64_t)0));
     } else {
+      // four tiles per work-group once there are work-groups to spare
+      const int rounds = nnz >= ((int64_t)kSumTile * kCscRounds) * 8192 ? kCscRounds : 1;
       GS_LAUNCH("spmm_csc_sum", s,
-                spmm_csc_sum_kernel<<<dim3((unsigned)ceil_div(nnz, kCscTile)), dim3(kBlock), 0,
-                                      s>>>(
-                    a, b, edge_map, num_major, nnz, kind, op, ufeat, efeat, out));
+                spmm_csc_sum_kernel<<<dim3((unsigned)ceil_div(nnz, (int64_t)kSumTile * rounds)),
+                                      dim3(kBlock), 0, s>>>(
+                    a, b, edge_map, num_major, nnz, kind, op, ufeat, efeat, out, rounds));
     }
     return GS_OK;
   }
@@ -846,19 +850,20 @@ int gs_sddmm(int format, const int64_t* a, const int64_t* b, int64_t num_major,
              "sddmm: null operand");
   hipStream_t s = as_stream(stream);
   const EdgeView g{format == GS_FMT_COMPRESSED, a, b, num_major, edge_map};
-  const unsigned blocks = (unsigned)ceil_div(nnz * out_len, kEdgeTile);
-  if (dtype == GS_F32)
-    GS_LAUNCH("sddmm", s,
-              sddmm_kernel<float><<<dim3(blocks), dim3(kBlock), 0, s>>>(
-                  g, nnz, op, (const float*)lhs, (const float*)rhs, (float*)out,
-                  lhs_target, rhs_target, lhs_len, rhs_len, out_len, reduce_size,
-                  lhs_off, rhs_off));
-  else
-    GS_LAUNCH("sddmm", s,
-              sddmm_kernel<double><<<dim3(blocks), dim3(kBlock), 0, s>>>(
-                  g, nnz, op, (const double*)lhs, (const double*)rhs,
-                  (double*)out, lhs_target, rhs_target, lhs_len, rhs_len, out_len,
-                  reduce_size, lhs_off, rhs_off));
+#define GS_SDDMM_LAUNCH(T, ITEMS)                                                         \
+  GS_LAUNCH("sddmm", s,                                                                   \
+            (sddmm_kernel<T, ITEMS>)<<<dim3((unsigned)ceil_div(nnz * out_len, kBlock * ITEMS)), \
+                                     dim3(kBlock), 0, s>>>(                               \
+                g, nnz, op, (const T*)lhs, (const T*)rhs, (T*)out, lhs_target, rhs_target, \
+                lhs_len, rhs_len, out_len, reduce_size, lhs_off, rhs_off))
+  if (g.compressed) {
+    if (dtype == GS_F32) GS_SDDMM_LAUNCH(float, kEdgeItems);
+    else GS_SDDMM_LAUNCH(double, kEdgeItems);
+  } else {
+    if (dtype == GS_F32) GS_SDDMM_LAUNCH(float, 1);
+    else GS_SDDMM_LAUNCH(double, 1);
+  }
+#undef GS_SDDMM_LAUNCH
   return GS_OK;
 }
 
@@ -879,21 +884,22 @@ int gs_fused_u_op_v(int format, const int64_t* a, const int64_t* b,
   GS_REQUIRE(lhs1 && rhs1 && out1 && lhs2 && rhs2 && out2, "fused_u_op_v: null operand");
   hipStream_t s = as_stream(stream);
   const EdgeView g{format == GS_FMT_COMPRESSED, a, b, num_major, nullptr};
-  const unsigned blocks = (unsigned)ceil_div(nnz * out_len, kEdgeTile);
-  if (dtype == GS_F32)
-    GS_LAUNCH("fused_u_op_v", s,
-              fused_u_op_v_kernel<float><<<dim3(blocks), dim3(kBlock), 0, s>>>(
-                  g, nnz, op, (const float*)lhs1, (const float*)rhs1,
-                  (float*)out1, (const float*)lhs2, (const float*)rhs2,
-                  (float*)out2, lhs_len, rhs_len, out_len, reduce_size, lhs_off,
-                  rhs_off));
-  else
-    GS_LAUNCH("fused_u_op_v", s,
-              fused_u_op_v_kernel<double><<<dim3(blocks), dim3(kBlock), 0, s>>>(
-                  g, nnz, op, (const double*)lhs1, (const double*)rhs1,
-                  (double*)out1, (const double*)lhs2, (const double*)rhs2,
-                  (double*)out2, lhs_len, rhs_len, out_len, reduce_size, lhs_off,
-                  rhs_off));
+#define GS_UOPV_LAUNCH(T, ITEMS)                                                          \
+  GS_LAUNCH("fused_u_op_v", s,                                                            \
+            (fused_u_op_v_kernel<T, ITEMS>)<<<dim3((unsigned)ceil_div(nnz * out_len,      \
+                                                                      kBlock * ITEMS)),   \
+                                            dim3(kBlock), 0, s>>>(                        \
+                g, nnz, op, (const T*)lhs1, (const T*)rhs1, (T*)out1, (const T*)lhs2,     \
+                (const T*)rhs2, (T*)out2, lhs_len, rhs_len, out_len, reduce_size, lhs_off, \
+                rhs_off))
+  if (g.compressed) {
+    if (dtype == GS_F32) GS_UOPV_LAUNCH(float, kEdgeItems);
+    else GS_UOPV_LAUNCH(double, kEdgeItems);
+  } else {
+    if (dtype == GS_F32) GS_UOPV_LAUNCH(float, 1);
+    else GS_UOPV_LAUNCH(double, 1);
+  }
+#undef GS_UOPV_LAUNCH
   return GS_OK;
 }
 
