@@ -670,25 +670,31 @@ __global__ __launch_bounds__(kPartThreads) void rowsum_accumulate_kernel(
   for (int j = threadIdx.x; j < kRangeRows; j += kPartThreads) mine[j] = (float)acc[j];
 }
 
+// out[row] += the row's partial sums over all slices of its range.  Ranges
+// differ a lot in how many slices they have (the rows of hubs sit in one range
+// and draw half of the edges), so the slices of a range are dealt out over
+// gridDim.y work-groups per block of rows, which add their shares atomically.
+constexpr int kFoldSplit = 8;
+
 __global__ __launch_bounds__(kBlock) void rowsum_fold_kernel(
     const float* __restrict__ partial, const int64_t* __restrict__ unit_start,
     int64_t num_out, float* __restrict__ out) {
   const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
   if (i >= num_out) return;
   const int64_t r = i >> kRangeShift;  // uniform over the work-group
-  const int64_t u0 = unit_start[r], u1 = unit_start[r + 1];
+  const int64_t u1 = unit_start[r + 1], step = gridDim.y;
   const float* p = partial + (i & (kRangeRows - 1));
   float acc = 0.f;
-  int64_t u = u0;
-  for (; u + 8 <= u1; u += 8) {  // eight loads in flight
+  int64_t u = unit_start[r] + blockIdx.y;
+  for (; u + 7 * step < u1; u += 8 * step) {  // eight loads in flight
     float v[8];
 #pragma unroll
-    for (int k = 0; k < 8; ++k) v[k] = p[(u + k) * kRangeRows];
+    for (int k = 0; k < 8; ++k) v[k] = p[(u + k * step) * kRangeRows];
 #pragma unroll
     for (int k = 0; k < 8; ++k) acc += v[k];
   }
-  for (; u < u1; ++u) acc += p[u * kRangeRows];
-  if (acc != 0.f) out[i] += acc;
+  for (; u < u1; u += step) acc += p[u * kRangeRows];
+  if (acc != 0.f) unsafeAtomicAdd(out + i, acc);
 }
 
 static int row_range_sum(const RowRangePlan& p, const int64_t* dst_ids,
@@ -721,7 +727,7 @@ static int row_range_sum(const RowRangePlan& p, const int64_t* dst_ids,
                                        dim3(kPartThreads), 0, s>>>(
                 entries, offsets, unit_start, ranges, p.tiles, partial));
   GS_LAUNCH("rowsum_fold", s,
-            rowsum_fold_kernel<<<dim3((unsigned)ceil_div(num_out, kBlock)),
+            rowsum_fold_kernel<<<dim3((unsigned)ceil_div(num_out, kBlock), kFoldSplit),
                                  dim3(kBlock), 0, s>>>(partial, unit_start,
                                                        num_out, out));
   return GS_OK;
