@@ -44,6 +44,7 @@ SIGNATURES = {
     "gs_scan_workspace_bytes": (_sz, [_i64]),
     "gs_exclusive_scan_i64": (_int, [_p, _p, _i64, _p, _sz, _p]),
     "gs_csc_col_count": (_int, [_p, _i64, _p, _i64, _i64, _int, _p, _p, _sz, _p]),
+    "gs_csc_col_count_static": (_int, [_p, _i64, _p, _i64, _i64, _int, _p, _p]),
     "gs_csc_col_slice_fill": (_int, [_p, _i64, _p, _p, _i64, _p, _i64, _p, _i64,
                                      _i64, _p, _p, _p, _p]),
     "gs_csc_col_sample_uniform_fill": (_int, [_p, _i64, _p, _p, _i64, _i64, _int,

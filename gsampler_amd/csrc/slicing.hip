@@ -2,7 +2,36 @@
 #include "common.h"
 #include "scan.h"
 
+#include <mutex>
+
 namespace gs {
+
+// Scan scratch of gs_csc_col_count_static: one tile sum per kScanTile counts,
+// held by every device the library runs on until the process ends.
+constexpr int64_t kStaticScanTiles = 65536;  // 512 KiB
+constexpr int64_t kStaticCountMaxItems = kStaticScanTiles * kScanTile - 1;
+static __device__ __align__(256) int64_t scratch[kStaticScanTiles];
+
+// Device address of `scratch` on the current device.  The array's name is only
+// a host-side handle; every device has its own copy at its own address, looked
+// up once per device.
+constexpr int kMaxDevices = 64;
+static int static_scratch(int64_t** out) {
+  static std::mutex mutex;
+  static int64_t* ptr[kMaxDevices] = {};
+  int dev = -1;
+  GS_HIP(hipGetDevice(&dev));
+  GS_REQUIRE(dev >= 0 && dev < kMaxDevices, "col_count_static: device %d not supported", dev);
+  std::lock_guard<std::mutex> lock(mutex);
+  if (ptr[dev] == nullptr) {
+    void* p = nullptr;
+    GS_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+    GS_REQUIRE(p != nullptr, "col_count_static: no device address for the scratch array");
+    ptr[dev] = (int64_t*)p;
+  }
+  *out = ptr[dev];
+  return GS_OK;
+}
 
 // One thread per requested column: writes its output count; the scan that
 // follows turns the counts into sub_indptr in place.
@@ -95,6 +124,24 @@ int gs_csc_col_count(const int64_t* indptr, int64_t num_cols,
                                        fanout, replace, sub_indptr));
   return exclusive_scan_i64(sub_indptr, sub_indptr, n, workspace,
                             workspace_bytes, s);
+}
+
+int gs_csc_col_count_static(const int64_t* indptr, int64_t num_cols,
+                            const int64_t* column_ids, int64_t num_items,
+                            int64_t fanout, int replace, int64_t* sub_indptr,
+                            gs_stream_t stream) {
+  using namespace gs;
+  GS_REQUIRE(num_items >= 0 && num_cols >= 0, "col_count_static: negative size");
+  GS_REQUIRE(num_items <= kStaticCountMaxItems,
+             "col_count_static: %lld items exceed the fixed scratch (at most %lld); "
+             "use gs_csc_col_count with a workspace",
+             (long long)num_items, (long long)kStaticCountMaxItems);
+  int64_t* ws = nullptr;
+  const int rc = static_scratch(&ws);
+  if (rc != GS_OK) return rc;
+  return gs_csc_col_count(indptr, num_cols, column_ids, num_items, fanout, replace,
+                          sub_indptr, ws, (size_t)kStaticScanTiles * sizeof(int64_t),
+                          stream);
 }
 
 int gs_csc_col_slice_fill(const int64_t* indptr, int64_t num_cols,

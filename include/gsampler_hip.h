@@ -111,6 +111,23 @@ int gs_csc_col_count(const int64_t* indptr, int64_t num_cols,
                      gs_stream_t stream);
 
 /* ------------------------------------------------------------------------
+ * gs_csc_col_count for callers that cannot allocate device memory (code under
+ * HIP graph capture, serving loops, harnesses that forbid hipMalloc): the same
+ * result with the scan scratch in a fixed 512 KiB array inside the library
+ * instead of a workspace, and no allocating call of any kind.  It has no
+ * counterpart in the reference, whose scans allocate through the torch caching
+ * allocator (src/cuda/utils.h:18-28).  At most 134 217 727 items; more is
+ * rejected with GS_ERR_INVALID.  All calls on one GPU share that array: calls
+ * that overlap in time on one GPU (different streams) race and must be
+ * serialised by the caller.  The first call on a device looks up the array's
+ * address (no allocation, but not capturable): make it before a capture.
+ * ---------------------------------------------------------------------- */
+int gs_csc_col_count_static(const int64_t* indptr, int64_t num_cols,
+                            const int64_t* column_ids, int64_t num_items,
+                            int64_t fanout, int replace, int64_t* sub_indptr,
+                            gs_stream_t stream);
+
+/* ------------------------------------------------------------------------
  * Column slicing A[:, column_ids] (fill phase).
  *   nnz = sub_indptr[num_items], as read back by the caller.
  *   out_coo_col   (nullable) : local column id of every output edge.
