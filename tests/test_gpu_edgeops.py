@@ -53,7 +53,7 @@ def test_sddmm_parity(g, fmt):
     assert np.array_equal(capi.sddmm(gv, "copy_lhs", T(u), None, 0, 2).cpu().numpy(),
                           orc.sddmm(ov, "copy_lhs", u, None, 0, 2))
     U, V = rng.random((500, 6), dtype=np.float32), rng.random((700, 6), dtype=np.float32)
-    close(capi.sddmm(gv, "dot", T(U), T(V), 0, 2), orc.sddmm(ov, "dot", U, V, 0, 2), 1e-4)
+    close(capi.sddmm(gv, "dot", T(U), T(V), 0, 2), orc.sddmm(ov, "dot", U, V, 0, 2))
     close(capi.sddmm(gv, "mul", T(U), T(V), 0, 2), orc.sddmm(ov, "mul", U, V, 0, 2))
     perm = rng.permutation(E)
     e64 = rng.random(E)
@@ -98,7 +98,7 @@ def test_scalar_sums_on_skewed_matrices(shape):
     """The load-balanced sum kernels: a few segments that hold most of the edges
     (and rows that most edges point to), and thousands of segments with zero or
     one edge.  Sums of up to 10^6 fp32 terms are compared with a float64 sum at
-    1e-4 relative (the order of additions is not fixed)."""
+    1e-5 relative (the order of additions is not fixed)."""
     rng = np.random.default_rng(31)
     if shape == "hubs":
         deg = np.full(40, 50)
@@ -130,13 +130,13 @@ def test_scalar_sums_on_skewed_matrices(shape):
     div_cols = np.bincount(col, weights=e64 / u[indices], minlength=C)
     coo, csc = ("coo", T(indices), T(col)), ("csc", T(indptr), T(indices))
     for view in (coo, csc):
-        close(capi.spmm(view, "copy_rhs", "sum", None, T(e), 0, C), onto_cols.astype(np.float32), 1e-4)
-        close(capi.e_div_u_sum(view, T(u), T(e), 0, C), div_cols.astype(np.float32), 1e-4)
-    close(capi.spmm(coo, "copy_rhs", "sum", None, T(e), 2, R), onto_rows.astype(np.float32), 1e-4)
-    close(capi.e_square_sum(coo, T(e), 2, R), sq_rows.astype(np.float32), 1e-4)
+        close(capi.spmm(view, "copy_rhs", "sum", None, T(e), 0, C), onto_cols.astype(np.float32))
+        close(capi.e_div_u_sum(view, T(u), T(e), 0, C), div_cols.astype(np.float32))
+    close(capi.spmm(coo, "copy_rhs", "sum", None, T(e), 2, R), onto_rows.astype(np.float32))
+    close(capi.e_square_sum(coo, T(e), 2, R), sq_rows.astype(np.float32))
     # and the oracle agrees with the float64 sums as well
     assert np.allclose(orc.spmm(("csc", indptr, indices), "copy_rhs", "sum", None, e, 0, C),
-                       onto_cols, rtol=1e-3)
+                       onto_cols, rtol=1e-5)
 
 
 def test_matrix_sum_div_and_ops_wrappers(g):

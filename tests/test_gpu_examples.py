@@ -46,7 +46,7 @@ def same_blocks(a, b):
         assert torch.equal(x.srcdata["_ID"], y.srcdata["_ID"])
         assert set(x.edata) == set(y.edata)
         for k in x.edata:
-            assert torch.allclose(x.edata[k], y.edata[k], rtol=1e-4, atol=1e-6)
+            assert torch.allclose(x.edata[k], y.edata[k], rtol=1e-5, atol=1e-7)
 
 
 def both_ways(func, args, sampling_calls):
@@ -133,7 +133,7 @@ def test_asgcn(world):
         asgcn_sampler, (m, seeds, [300, 300], feats, W), sampling_calls=2)
     same_edge_sets(e_blocks[0], c_blocks[0], seeds)
     assert torch.allclose(torch.sort(e_blocks[0].edata["w"])[0], torch.sort(c_blocks[0].edata["w"])[0],
-                          rtol=1e-4)
+                          rtol=1e-5)
     for nodes, blocks in ((e_nodes, e_blocks), (c_nodes, c_blocks)):
         edges_exist(blocks[0], seeds, adj)
         edges_exist(blocks[1], blocks[0].srcdata["_ID"], adj)
@@ -310,7 +310,7 @@ def test_batch_ladies(world):
                 # weights are normalised per destination node
                 sums = torch.zeros(ids.numel(), device=DEV).index_add_(0, block.col, block.edata["w"])
                 has = torch.bincount(block.col, minlength=ids.numel()) > 0
-                assert torch.allclose(sums[has], torch.ones_like(sums[has]), rtol=1e-4)
+                assert torch.allclose(sums[has], torch.ones_like(sums[has]), rtol=1e-5)
                 nxt.append(block.srcdata["_ID"])
             dst = nxt
     for a, b, ids in zip(eager[0], jit[0], parts):     # first layer: the same picks
@@ -348,6 +348,6 @@ def test_compiled_with_compaction_describes_the_same_blocks(world):
         for b in blocks:
             sums = torch.zeros(b.num_dst, device=DEV).index_add_(0, b.col, b.edata["w"])
             has = torch.bincount(b.col, minlength=b.num_dst) > 0
-            assert torch.allclose(sums[has], torch.ones_like(sums[has]), rtol=1e-4)
+            assert torch.allclose(sums[has], torch.ones_like(sums[has]), rtol=1e-5)
             assert torch.unique(b.srcdata["_ID"][b.row]).numel() <= 200
     assert p_blocks[0].num_dst == d_blocks[0].num_dst == seeds.numel()
