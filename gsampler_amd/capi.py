@@ -311,7 +311,7 @@ def unique_relabel(seeds, rows, seeds_ptr=None, rows_ptr=None, edge_col=None,
                             unique_ptr.data_ptr(), ws.data_ptr(), ws.numel(),
                             _stream()))
     count = _Count(unique_ptr)
-    size = S + E if S + E <= _BOUND_LIMIT else max(count.get(), 0)   # U <= S + E
+    size = S + E if S + E <= _BOUND_LIMIT else count.get()   # U <= S + E
     unique = torch.empty(size, dtype=torch.int64, device=dev)
     want_col = want_col and edge_col is not None
     out_row = torch.empty(E, dtype=torch.int64, device=dev) if want_row else None
@@ -326,8 +326,6 @@ def unique_relabel(seeds, rows, seeds_ptr=None, rows_ptr=None, edge_col=None,
                                   _ptr(edge_col), _ptr(out_row), _ptr(out_col),
                                   ws.data_ptr(), ws.numel(), _stream()))
     total = count.get()
-    if total < 0:
-        raise GsError("unique: ids must lie in [0, 2^32 - 2]")
     return unique[:total], unique_ptr, out_row, out_col
 
 

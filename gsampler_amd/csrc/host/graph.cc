@@ -390,7 +390,7 @@ Graph::Frontier& Graph::frontier_for(const torch::Tensor& seeds,
   if (B > 1) OffsetMirror::prefetch(f->unique_ptr);  // per-batch splits will ask for it
   // at most S + E unique keys
   f->unique_buffer =
-      new_ids(S + E <= kBoundLimit ? S + E : std::max<int64_t>(f->count.get(), 0), rows);
+      new_ids(S + E <= kBoundLimit ? S + E : f->count.get(), rows);
   GS_CALL(gs_unique_fill(cptr(seeds), cptr(seeds_ptr), S, cptr(rows),
                          cptr(rows_ptr), E, B, cptr(f->unique_ptr),
                          mptr(f->unique_buffer), f->workspace.data_ptr(),

@@ -189,7 +189,6 @@ class Graph : public torch::CustomClassHolder {
     const torch::Tensor& frontier() {
       if (!unique_.defined()) {
         const int64_t total = count.get();
-        TORCH_CHECK(total >= 0, "unique / relabel: ids must lie in [0, 2^32 - 2]");
         unique_ = unique_buffer.narrow(0, 0, total);
       }
       return unique_;

@@ -11,6 +11,13 @@
 //   fill : kept edge e goes to its rank (chunk offset + popcounts), edge order
 //          preserved; its new id comes from the chunk's staged run, so the fill
 //          pass reads neither the ids nor the table again.
+//
+// A table slot is  low 32 bits of the id << 32 | position in the picked set.
+// While every picked id is below 2^32 - 1 those bits are the id, and an edge
+// whose id is larger cannot match.  When a picked id is larger (an id of a very
+// large graph, an id encoded as id + batch * num_rows) the insert pass raises a
+// flag, and every match of the 32-bit halves is then confirmed against the
+// picked id itself.
 #include "common.h"
 #include "hashtable.h"
 #include "scan.h"
@@ -27,6 +34,7 @@ struct MemberWs {
   uint64_t* flags;     // [chunks * kMemberWords]
   uint32_t* staged;    // [chunks * kBlock]: per chunk, the new ids of its kept edges, in order
   int64_t* chunk_off;  // [chunks + 1]
+  int* wide;           // [1] set when a picked id does not fit the upper half of a slot
   void* scan_ws;
   size_t scan_ws_bytes;
   int64_t chunks;
@@ -52,6 +60,7 @@ static MemberWs carve_member(void* ws, int64_t nnz, int64_t num_picked) {
   w.flags = c.take<uint64_t>((size_t)w.chunks * kMemberWords);
   w.staged = c.take<uint32_t>((size_t)w.chunks * kBlock);
   w.chunk_off = c.take<int64_t>((size_t)w.chunks + 1);
+  w.wide = c.take<int>(1);
   w.scan_ws_bytes = scan_workspace_bytes(w.chunks + 1);
   w.scan_ws = c.take<char>(w.scan_ws_bytes);
   w.total = c.total();
@@ -67,17 +76,28 @@ __device__ __forceinline__ uint32_t member_home(uint32_t key, uint32_t cap) {
   return __umulhi(key * 0x9E3779B1u, cap);
 }
 
-// 32-bit form of an id, kNoKey for one that no picked id can equal
+// 32-bit form of an id when every picked id fits 32 bits: kNoKey for one that
+// no picked id can equal
 __device__ __forceinline__ uint32_t member_key(uint64_t id) {
   return id <= kMaxPackedKey ? (uint32_t)id : kNoKey;
 }
+// 32-bit tag of any id: its low half, kept clear of kNoKey
+__device__ __forceinline__ uint32_t member_tag(uint64_t id) {
+  const uint32_t t = (uint32_t)id;
+  return t == kNoKey ? kNoKey - 1 : t;
+}
 
+// *wide must be 0 before the launch.  Two picked ids with the same tag are the
+// same id unless one of them is wide, so matches are always confirmed here (the
+// picked set is small next to the edges).
 __global__ __launch_bounds__(kBlock) void member_insert_kernel(
-    const int64_t* __restrict__ picked, int64_t n, uint64_t* table, uint32_t cap) {
+    const int64_t* __restrict__ picked, int64_t n, uint64_t* table, uint32_t cap,
+    int* __restrict__ wide) {
   const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
   if (i >= n) return;
-  const uint32_t key = member_key((uint64_t)picked[i]);
-  if (key == kNoKey) return;  // cannot equal any admissible id
+  const uint64_t id = (uint64_t)picked[i];
+  if (id > kMaxPackedKey) *wide = 1;  // every writer stores the same value
+  const uint32_t key = member_tag(id);
   const uint64_t mine = ((uint64_t)key << 32) | (uint64_t)i;
   uint32_t slot = member_home(key, cap);
   for (uint32_t probes = 0; probes < cap; ++probes) {  // the table has free slots: ends early
@@ -87,12 +107,22 @@ __global__ __launch_bounds__(kBlock) void member_insert_kernel(
                       (unsigned long long)mine);
       if (cur == kEmptySlot) return;
     }
-    if ((uint32_t)(cur >> 32) == key) {  // a repeated id keeps its smallest position
+    // a slot only ever holds positions of one id; a repeated id keeps its smallest
+    if ((uint32_t)(cur >> 32) == key && (uint64_t)picked[(uint32_t)cur] == id) {
       atomicMin((unsigned long long*)(table + slot), (unsigned long long)mine);
       return;
     }
     if (++slot == cap) slot = 0;
   }
+}
+
+// Empties the table and lowers the wide-id flag.
+__global__ __launch_bounds__(kBlock) void member_clear_kernel(uint64_t* table, int64_t n,
+                                                              int* __restrict__ wide) {
+  int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (i == 0) *wide = 0;
+  const int64_t stride = (int64_t)gridDim.x * kBlock;
+  for (; i < n; i += stride) table[i] = kEmptySlot;
 }
 
 // A small table (the picked set of a layer-wise sampler is a few hundred ids)
@@ -162,18 +192,35 @@ struct MemberTable {
     for (int j = 0; j < N; ++j)
       if ((open >> j) & 1u) slot[j] = cap;  // probe budget spent: cannot happen with free slots
   }
+
+  // One look-up whose tag matches are confirmed against the picked ids (the
+  // path of picked sets with ids of 2^32 - 1 and above).
+  __device__ __forceinline__ uint32_t find_confirmed(uint64_t id,
+                                                     const int64_t* __restrict__ picked) const {
+    const uint32_t tag = member_tag(id);
+    uint32_t slot = member_home(tag, cap);
+    for (uint32_t probes = 0; probes < cap; ++probes) {
+      const uint32_t cur = key_at(slot);
+      if (cur == kNoKey) return cap;
+      if (cur == tag && (uint64_t)picked[value_at(slot)] == id) return slot;
+      if (++slot == cap) slot = 0;
+    }
+    return cap;
+  }
 };
 
 template <bool kInLds>
 __global__ __launch_bounds__(kMemberThreads) void member_flag_kernel(
     const int64_t* __restrict__ ids, int64_t nnz,
     const uint64_t* __restrict__ global_table, uint32_t cap,
+    const int64_t* __restrict__ picked, const int* __restrict__ wide_flag,
     uint64_t* __restrict__ flags, int64_t* __restrict__ chunk_count,
     uint32_t* __restrict__ staged) {
   __shared__ uint32_t lds_keys[kInLds ? kMemberLdsSlots : 1];
   __shared__ uint32_t lds_values[kInLds ? kMemberLdsSlots : 1];
   MemberTable<kInLds, true> table;
   table.stage(global_table, cap, lds_keys, lds_values);
+  const bool wide = *wide_flag != 0;  // the same for every thread of the launch
   const int64_t num_chunks = ceil_div_dev(nnz, kBlock);
   const int64_t wave = (int64_t)blockIdx.x * (kMemberThreads / kWave) + threadIdx.x / kWave;
   const int lane = lane_id();
@@ -201,7 +248,15 @@ __global__ __launch_bounds__(kMemberThreads) void member_flag_kernel(
     }
     uint32_t slot[kMemberWords];
     uint64_t word[kMemberWords];
-    table.find_many(key, slot);
+    if (!wide) {
+      table.find_many(key, slot);
+    } else {
+#pragma unroll
+      for (int j = 0; j < kMemberWords; ++j) {
+        const int64_t e = chunk * kBlock + j * kWave + lane;
+        slot[j] = e < nnz ? table.find_confirmed((uint64_t)ids[e], picked) : cap;
+      }
+    }
 #pragma unroll
     for (int j = 0; j < kMemberWords; ++j) word[j] = __ballot(slot[j] < cap);
     {
@@ -349,24 +404,23 @@ int gs_minor_slice_count(const int64_t* ids, int64_t nnz, const int64_t* picked,
   hipStream_t s = as_stream(stream);
   const uint32_t cap = (uint32_t)member_table_slots(num_picked);
   GS_LAUNCH("member_clear", s,
-            table_fill_kernel<><<<dim3((unsigned)ceil_div((int64_t)cap, kBlock * 4)),
-                                  dim3(kBlock), 0, s>>>(w.table, (int64_t)cap,
-                                                        kEmptySlot));
+            member_clear_kernel<<<dim3((unsigned)ceil_div((int64_t)cap, kBlock * 4)),
+                                  dim3(kBlock), 0, s>>>(w.table, (int64_t)cap, w.wide));
   if (num_picked > 0)
     GS_LAUNCH("member_insert", s,
               member_insert_kernel<<<dim3((unsigned)ceil_div(num_picked, kBlock)),
                                      dim3(kBlock), 0, s>>>(picked, num_picked,
-                                                           w.table, cap));
+                                                           w.table, cap, w.wide));
   if (nnz > 0) {
     const int64_t blocks = ceil_div(w.chunks, (kMemberThreads / kWave) * kMemberChunksPerWave);
     if (cap <= (uint64_t)kMemberLdsSlots)
       GS_LAUNCH("member_flag", s,
                 member_flag_kernel<true><<<dim3((unsigned)blocks), dim3(kMemberThreads), 0, s>>>(
-                    ids, nnz, w.table, cap, w.flags, w.chunk_off, w.staged));
+                    ids, nnz, w.table, cap, picked, w.wide, w.flags, w.chunk_off, w.staged));
     else
       GS_LAUNCH("member_flag", s,
                 member_flag_kernel<false><<<dim3((unsigned)blocks), dim3(kMemberThreads), 0, s>>>(
-                    ids, nnz, w.table, cap, w.flags, w.chunk_off, w.staged));
+                    ids, nnz, w.table, cap, picked, w.wide, w.flags, w.chunk_off, w.staged));
     int rc = exclusive_scan_i64(w.chunk_off, w.chunk_off, w.chunks + 1, w.scan_ws,
                                 w.scan_ws_bytes, s);
     if (rc != GS_OK) return rc;

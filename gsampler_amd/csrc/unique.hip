@@ -34,6 +34,13 @@
 // LDS table is sure to hold (a hub that repeats thousands of times, a batch too
 // large for kMaxBuckets buckets) is deduplicated by the same work-group in a
 // table in global memory that is private to the bucket.
+//
+// A packed entry is  low 32 bits of the key << 32 | position.  While every key
+// of a call is below 2^32 - 1 those bits are the key.  The partition pass notes
+// when one is not (an id of a very large graph, an id encoded as
+// id + batch * num_rows): the upper half is then only a fingerprint, and the
+// dedup pass confirms every fingerprint match by comparing the two keys
+// themselves, read back through their positions.
 #include "common.h"
 #include "hashtable.h"
 #include "scan.h"
@@ -111,7 +118,7 @@ struct UniqueWs {
   int32_t* chunk_batch;   // [chunks + 1] batch of the first position of a chunk
   int32_t* etile_batch;   // [edge tiles + 1] batch of the first edge of a tile
   int64_t* bucket_cnt;    // [max_buckets + 1] entries per bucket
-  int* bad_key;           // [1] set when a key does not fit the packed entry
+  int* wide_keys;         // [1] set when some key does not fit the upper half of an entry
   int64_t* bucket_off;    // [max_buckets + 1] first entry of a bucket
   uint64_t* packed;       // [N] key << 32 | local, grouped by bucket
   uint32_t* first;        // [N] local position of the first occurrence
@@ -144,7 +151,7 @@ static UniqueWs carve_unique(void* ws, int64_t S, int64_t E, int64_t B) {
   w.chunk_batch = c.take<int32_t>((size_t)w.chunks + 1);
   w.etile_batch = c.take<int32_t>((size_t)w.etiles + 1);
   w.bucket_cnt = c.take<int64_t>((size_t)w.max_buckets + 1);
-  w.bad_key = c.take<int>(1);
+  w.wide_keys = c.take<int>(1);
   w.bucket_off = c.take<int64_t>((size_t)w.max_buckets + 1);
   w.packed = c.take<uint64_t>((size_t)n1);
   w.first = c.take<uint32_t>((size_t)n1);
@@ -199,12 +206,12 @@ __global__ __launch_bounds__(kBlock) void unique_prep_kernel(
     Keys k, int64_t bucket_keys, BatchInfo* __restrict__ batch,
     int64_t* __restrict__ flat_ptr, int64_t* __restrict__ tile_ptr,
     int64_t* __restrict__ bucket_ptr, int64_t* __restrict__ bucket_cnt,
-    int64_t max_buckets, int* __restrict__ bad_key) {
+    int64_t max_buckets, int* __restrict__ wide_keys) {
   for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i <= max_buckets;
        i += (int64_t)gridDim.x * kBlock)
     bucket_cnt[i] = 0;
   if (blockIdx.x != 0) return;
-  if (threadIdx.x == 0) *bad_key = 0;
+  if (threadIdx.x == 0) *wide_keys = 0;
   __shared__ int64_t smem[kBlock / kWave + 1];
   int64_t tile_carry = 0, bucket_carry = 0;
   for (int64_t base = 0; base <= k.B; base += kBlock) {
@@ -298,11 +305,18 @@ __device__ __forceinline__ uint64_t key_at(const Keys& k, const BatchInfo& b,
   return key_at(k, b.s_lo, b.ns, b.r_lo, local);
 }
 
+// Upper half of a packed entry: the low 32 bits of the key, kept clear of the
+// pattern of the empty slot (for keys below 2^32 - 1 this is the key itself).
+__device__ __forceinline__ uint32_t key_tag(uint64_t key) {
+  const uint32_t t = (uint32_t)key;
+  return t == 0xFFFFFFFFu ? 0xFFFFFFFEu : t;
+}
+
 // ---------------------------------------------------------------- hist
 __global__ __launch_bounds__(kBlock) void unique_hist_kernel(
     Keys k, const int32_t* __restrict__ tile_batch,
     const BatchInfo* __restrict__ batch, int64_t* bucket_cnt, int64_t max_tiles,
-    int remap, int* bad_key) {
+    int remap, int* wide_keys) {
   __shared__ uint32_t hist[kMaxBuckets];
   const int64_t tile = unit_of_block(max_tiles, remap);
   if (tile >= max_tiles) return;
@@ -313,15 +327,15 @@ __global__ __launch_bounds__(kBlock) void unique_hist_kernel(
     atomicAdd((unsigned long long*)&bucket_cnt[t.b.bucket0],
               (unsigned long long)(t.end - t.begin));
   uint32_t key[kPartItems];
-  bool bad = false;
+  bool wide = false;
 #pragma unroll
   for (int i = 0; i < kPartItems; ++i) {  // all loads in flight before any use
     const int64_t l = t.begin + i * kBlock + threadIdx.x;
     const uint64_t full = l < t.end ? key_at(k, t.b, l) : 0ull;
-    bad |= full > kMaxPackedKey;  // negative ids land here too
-    key[i] = (uint32_t)full;
+    wide |= full > kMaxPackedKey;  // negative ids land here too
+    key[i] = key_tag(full);
   }
-  if (bad) *bad_key = 1;  // every writer stores the same value
+  if (wide) *wide_keys = 1;  // every writer stores the same value
   if (buckets == 1) return;  // nothing to choose
   for (uint32_t i = threadIdx.x; i < buckets; i += kBlock) hist[i] = 0;
   __syncthreads();
@@ -390,7 +404,7 @@ __global__ __launch_bounds__(kBlock) void unique_scatter_kernel(
   uint64_t* out = packed + t.b.fb;
   if (buckets == 1) {  // the bucket is the batch, in order
     for (int64_t l = t.begin + threadIdx.x; l < t.end; l += kBlock) {
-      out[l] = (key_at(k, t.b, l) << 32) | (uint64_t)l;
+      out[l] = ((uint64_t)key_tag(key_at(k, t.b, l)) << 32) | (uint64_t)l;
       first[t.b.fb + l] = (uint32_t)l;
     }
     return;
@@ -401,7 +415,7 @@ __global__ __launch_bounds__(kBlock) void unique_scatter_kernel(
 #pragma unroll
   for (int i = 0; i < kPartItems; ++i) {
     const int64_t l = t.begin + i * kBlock + threadIdx.x;
-    key[i] = l < t.end ? (uint32_t)key_at(k, t.b, l) : 0u;
+    key[i] = l < t.end ? key_tag(key_at(k, t.b, l)) : 0u;
     // every position starts as its own first occurrence; the dedup pass only
     // writes the positions that are not (half as many scattered stores)
     if (l < t.end) first[t.b.fb + l] = (uint32_t)l;
@@ -457,10 +471,23 @@ __global__ __launch_bounds__(kBlock) void unique_scatter_kernel(
 }
 
 // ---------------------------------------------------------------- dedup
+// Whether two entries with the same upper half stand for the same key: always
+// when every key of the call fits that half; otherwise the keys themselves are
+// read back through the entries' positions and compared.
+struct SameKey {
+  const Keys* k;
+  const BatchInfo* b;
+  bool wide;
+  __device__ __forceinline__ bool operator()(uint64_t a, uint64_t c) const {
+    if (!wide) return true;
+    return key_at(*k, *b, (int64_t)(uint32_t)a) == key_at(*k, *b, (int64_t)(uint32_t)c);
+  }
+};
+
 __device__ __forceinline__ void lds_insert_min(uint64_t* tab, uint32_t mask,
-                                               uint64_t entry) {
-  const uint64_t key = entry >> 32;
-  uint32_t slot = slot_hash(key) & mask;
+                                               uint64_t entry, const SameKey& same) {
+  const uint64_t tag = entry >> 32;
+  uint32_t slot = slot_hash(tag) & mask;
   for (;;) {
     uint64_t cur = tab[slot];
     if (cur == kEmptySlot) {
@@ -468,7 +495,8 @@ __device__ __forceinline__ void lds_insert_min(uint64_t* tab, uint32_t mask,
                       (unsigned long long)kEmptySlot, (unsigned long long)entry);
       if (cur == kEmptySlot) return;
     }
-    if ((cur >> 32) == key) {
+    // a slot only ever holds positions of one key, so a stale read is as good
+    if ((cur >> 32) == tag && same(cur, entry)) {
       if (cur > entry)
         atomicMin((unsigned long long*)&tab[slot], (unsigned long long)entry);
       return;
@@ -478,11 +506,14 @@ __device__ __forceinline__ void lds_insert_min(uint64_t* tab, uint32_t mask,
 }
 
 __device__ __forceinline__ uint32_t lds_first_of(const uint64_t* tab,
-                                                 uint32_t mask, uint64_t key) {
-  uint32_t slot = slot_hash(key) & mask;
+                                                 uint32_t mask, uint64_t entry,
+                                                 const SameKey& same) {
+  const uint64_t tag = entry >> 32;
+  uint32_t slot = slot_hash(tag) & mask;
   for (;;) {
     const uint64_t cur = tab[slot];
-    if ((cur >> 32) == key) return (uint32_t)cur;
+    if (cur == kEmptySlot) return (uint32_t)entry;  // not reached: every entry was inserted
+    if ((cur >> 32) == tag && same(cur, entry)) return (uint32_t)cur;
     slot = (slot + 1) & mask;
   }
 }
@@ -494,9 +525,9 @@ __device__ __forceinline__ uint64_t load_l2(const uint64_t* p) {
 }
 
 __device__ __forceinline__ void spill_insert_min(uint64_t* tab, uint64_t cap,
-                                                 uint64_t entry) {
-  const uint64_t key = entry >> 32;
-  uint64_t slot = ((uint64_t)slot_hash(key) * cap) >> 32;
+                                                 uint64_t entry, const SameKey& same) {
+  const uint64_t tag = entry >> 32;
+  uint64_t slot = ((uint64_t)slot_hash(tag) * cap) >> 32;
   for (uint64_t probes = 0; probes < cap; ++probes) {
     uint64_t cur = load_l2(tab + slot);
     if (cur == kEmptySlot) {
@@ -504,7 +535,7 @@ __device__ __forceinline__ void spill_insert_min(uint64_t* tab, uint64_t cap,
                       (unsigned long long)kEmptySlot, (unsigned long long)entry);
       if (cur == kEmptySlot) return;
     }
-    if ((cur >> 32) == key) {
+    if ((cur >> 32) == tag && same(cur, entry)) {
       if (cur > entry)
         atomicMin((unsigned long long*)(tab + slot), (unsigned long long)entry);
       return;
@@ -514,14 +545,17 @@ __device__ __forceinline__ void spill_insert_min(uint64_t* tab, uint64_t cap,
 }
 
 __device__ __forceinline__ uint32_t spill_first_of(const uint64_t* tab,
-                                                   uint64_t cap, uint64_t key) {
-  uint64_t slot = ((uint64_t)slot_hash(key) * cap) >> 32;
+                                                   uint64_t cap, uint64_t entry,
+                                                   const SameKey& same) {
+  const uint64_t tag = entry >> 32;
+  uint64_t slot = ((uint64_t)slot_hash(tag) * cap) >> 32;
   for (uint64_t probes = 0; probes < cap; ++probes) {
     const uint64_t cur = load_l2(tab + slot);
-    if ((cur >> 32) == key) return (uint32_t)cur;
+    if (cur == kEmptySlot) break;
+    if ((cur >> 32) == tag && same(cur, entry)) return (uint32_t)cur;
     if (++slot == cap) slot = 0;
   }
-  return 0;  // not reached: every key looked up was inserted
+  return (uint32_t)entry;  // not reached: every entry looked up was inserted
 }
 
 // Same as lds_insert_min for a bucket that may hold more distinct keys than the
@@ -530,10 +564,11 @@ __device__ __forceinline__ uint32_t spill_first_of(const uint64_t* tab,
 __device__ __forceinline__ void lds_insert_min_counted(uint64_t* tab,
                                                        uint32_t mask,
                                                        uint64_t entry,
+                                                       const SameKey& same,
                                                        uint32_t* distinct,
                                                        volatile uint32_t* overflow) {
-  const uint64_t key = entry >> 32;
-  uint32_t slot = slot_hash(key) & mask;
+  const uint64_t tag = entry >> 32;
+  uint32_t slot = slot_hash(tag) & mask;
   for (;;) {
     uint64_t cur = tab[slot];
     if (cur == kEmptySlot) {
@@ -544,7 +579,7 @@ __device__ __forceinline__ void lds_insert_min_counted(uint64_t* tab,
         return;
       }
     }
-    if ((cur >> 32) == key) {
+    if ((cur >> 32) == tag && same(cur, entry)) {
       if (cur > entry)
         atomicMin((unsigned long long*)&tab[slot], (unsigned long long)entry);
       return;
@@ -555,6 +590,7 @@ __device__ __forceinline__ void lds_insert_min_counted(uint64_t* tab,
 
 template <int kThreads>
 __global__ __launch_bounds__(kThreads) void unique_dedup_kernel(
+    Keys k, const int* __restrict__ wide_keys,
     const int32_t* __restrict__ bucket_batch, const BatchInfo* __restrict__ batch,
     const int64_t* __restrict__ bucket_off, const uint64_t* __restrict__ packed,
     uint64_t* spill, uint32_t* __restrict__ first, int64_t max_buckets,
@@ -569,7 +605,9 @@ __global__ __launch_bounds__(kThreads) void unique_dedup_kernel(
   const int64_t lo = bucket_off[g], hi = bucket_off[g + 1];
   const int64_t n = hi - lo;
   if (n == 0) return;
-  uint32_t* first_b = first + batch[b].fb;
+  const BatchInfo info = batch[b];
+  const SameKey same{&k, &info, *wide_keys != 0};
+  uint32_t* first_b = first + info.fb;
   // table of two slots per entry, a power of two, at most kLdsSlots
   uint32_t slots = 256;
   while (slots < kLdsSlots && (int64_t)slots < 2 * n) slots <<= 1;
@@ -588,12 +626,12 @@ __global__ __launch_bounds__(kThreads) void unique_dedup_kernel(
     }
 #pragma unroll
     for (int j = 0; j < kKeep; ++j)
-      if (mine[j] != kEmptySlot) lds_insert_min(tab, mask, mine[j]);
+      if (mine[j] != kEmptySlot) lds_insert_min(tab, mask, mine[j], same);
     __syncthreads();
 #pragma unroll
     for (int j = 0; j < kKeep; ++j)
       if (mine[j] != kEmptySlot) {
-        const uint32_t f = lds_first_of(tab, mask, mine[j] >> 32);
+        const uint32_t f = lds_first_of(tab, mask, mine[j], same);
         if (f != (uint32_t)mine[j]) first_b[(uint32_t)mine[j]] = f;
       }
     return;
@@ -615,7 +653,7 @@ __global__ __launch_bounds__(kThreads) void unique_dedup_kernel(
 #pragma unroll
     for (int j = 0; j < kDeep; ++j)
       if (e[j] != kEmptySlot && !*over)
-        lds_insert_min_counted(tab, mask, e[j], &distinct, over);
+        lds_insert_min_counted(tab, mask, e[j], same, &distinct, over);
   }
   __syncthreads();
   if (!overflow) {
@@ -629,7 +667,7 @@ __global__ __launch_bounds__(kThreads) void unique_dedup_kernel(
 #pragma unroll
       for (int j = 0; j < kDeep; ++j)
         if (e[j] != kEmptySlot) {
-          const uint32_t f = lds_first_of(tab, mask, e[j] >> 32);
+          const uint32_t f = lds_first_of(tab, mask, e[j], same);
           if (f != (uint32_t)e[j]) first_b[(uint32_t)e[j]] = f;
         }
     }
@@ -642,12 +680,12 @@ __global__ __launch_bounds__(kThreads) void unique_dedup_kernel(
   __threadfence();
   __syncthreads();
   for (int64_t i = lo + threadIdx.x; i < hi; i += kThreads)
-    spill_insert_min(gt, cap, packed[i]);
+    spill_insert_min(gt, cap, packed[i], same);
   __threadfence();
   __syncthreads();
   for (int64_t i = lo + threadIdx.x; i < hi; i += kThreads) {
     const uint64_t e = packed[i];
-    const uint32_t f = spill_first_of(gt, cap, e >> 32);
+    const uint32_t f = spill_first_of(gt, cap, e, same);
     if (f != (uint32_t)e) first_b[(uint32_t)e] = f;
   }
 }
@@ -734,16 +772,13 @@ __device__ __forceinline__ int64_t rank_before(
   return r;
 }
 
-// unique_ptr[B] = -1 tells the caller that some key did not fit the packed
-// entry (an id above 2^32 - 2 or a negative one): nothing else is valid then.
 __global__ void unique_ptr_kernel(const int64_t* __restrict__ flat_ptr,
                                   int64_t B, const uint64_t* __restrict__ flags,
                                   const int64_t* __restrict__ block_off,
-                                  const int* __restrict__ bad_key,
                                   int64_t* __restrict__ unique_ptr) {
   const int64_t b = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (b > B) return;
-  unique_ptr[b] = (b == B && *bad_key) ? -1 : rank_before(flat_ptr[b], flags, block_off);
+  unique_ptr[b] = rank_before(flat_ptr[b], flags, block_off);
 }
 
 // ---------------------------------------------------------------- fill
@@ -902,7 +937,7 @@ int gs_unique_count(const int64_t* seeds, const int64_t* seeds_ptr,
     GS_LAUNCH("unique_prep", s,
               unique_prep_kernel<<<dim3((unsigned)blocks), dim3(kBlock), 0, s>>>(
                   k, tn.bucket_keys, w.batch, w.flat_ptr, w.tile_ptr,
-                  w.bucket_ptr, w.bucket_cnt, w.max_buckets, w.bad_key));
+                  w.bucket_ptr, w.bucket_cnt, w.max_buckets, w.wide_keys));
     const int64_t units = w.max_tiles + w.max_buckets + w.chunks + 1 + w.etiles + 1;
     GS_LAUNCH("unique_units", s,
               unique_units_kernel<<<dim3((unsigned)ceil_div(units, kBlock)),
@@ -915,7 +950,7 @@ int gs_unique_count(const int64_t* seeds, const int64_t* seeds_ptr,
   GS_LAUNCH("unique_hist", s,
             unique_hist_kernel<<<tile_grid, dim3(kBlock), 0, s>>>(
                 k, w.tile_batch, w.batch, w.bucket_cnt, w.max_tiles, tn.remap,
-                w.bad_key));
+                w.wide_keys));
   GS_LAUNCH("unique_bucket_scan", s,
             unique_bucket_scan_kernel<<<dim3(1), dim3(kBucketScanThreads), 0, s>>>(
                 w.bucket_ptr, B, w.bucket_cnt, w.bucket_off));
@@ -928,13 +963,13 @@ int gs_unique_count(const int64_t* seeds, const int64_t* seeds_ptr,
               unique_dedup_kernel<512><<<dim3((unsigned)grid_for_units(
                                              w.max_buckets, tn.remap)),
                                          dim3(512), 0, s>>>(
-                  w.bucket_batch, w.batch, w.bucket_off, w.packed, w.spill,
+                  k, w.wide_keys, w.bucket_batch, w.batch, w.bucket_off, w.packed, w.spill,
                   w.first, w.max_buckets, tn.remap);
             else
               unique_dedup_kernel<256><<<dim3((unsigned)grid_for_units(
                                              w.max_buckets, tn.remap)),
                                          dim3(256), 0, s>>>(
-                  w.bucket_batch, w.batch, w.bucket_off, w.packed, w.spill,
+                  k, w.wide_keys, w.bucket_batch, w.batch, w.bucket_off, w.packed, w.spill,
                   w.first, w.max_buckets, tn.remap));
   GS_LAUNCH("unique_flag", s,
             unique_flag_kernel<<<dim3((unsigned)ceil_div(
@@ -947,8 +982,7 @@ int gs_unique_count(const int64_t* seeds, const int64_t* seeds_ptr,
   GS_LAUNCH("unique_ptr", s,
             unique_ptr_kernel<<<dim3((unsigned)ceil_div(B + 1, kBlock)),
                                 dim3(kBlock), 0, s>>>(w.flat_ptr, B, w.flags,
-                                                      w.block_off, w.bad_key,
-                                                      unique_ptr));
+                                                      w.block_off, unique_ptr));
   return GS_OK;
 }
 

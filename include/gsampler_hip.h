@@ -264,8 +264,12 @@ int gs_list_sample_weighted_fill(const float* probs, const int64_t* range,
  *   rank of every row key (nullable); out_col[num_rows_keys] = batch-local rank
  *   of seeds[edge_col[e]] (nullable; edge_col holds positions into `seeds`).
  *   May be called any number of times while the workspace is kept.
- * Keys must lie in [0, 2^32 - 2] and one batch may hold at most 2^32 - 2 keys;
- * count reports a key outside that range as unique_ptr[num_batches] = -1.
+ * Keys are any int64 values; one call takes at most 2^31 - 1 keys.  While all
+ * keys of a call lie in [0, 2^32 - 2] a packed table entry holds the key itself;
+ * when one does not (ids of a very large graph, ids encoded as id + batch *
+ * num_rows, src/cuda/batch/slicing.cu:25-27), the kernels notice during the
+ * partition pass and confirm every match of the 32-bit halves against the keys
+ * themselves: same result, a few extra reads per repeated key.
  * Stands in for TensorUniqueCUDA / TensorRelabelCUDA
  * (src/cuda/unique_reindex.cu:174-199) and BatchCOORelabelCUDA
  * (src/cuda/batch/batch_relabel.cu:480-498).
@@ -342,7 +346,9 @@ int gs_gather_rows(const void* table, int64_t num_rows, int64_t row_bytes,
  *  fill:  same ids / workspace; out_minor[kept] = position in `picked`,
  *    out_select[kept] = edge position, out_major[kept] (nullable) =
  *    edge_major[e] if given else the segment of indptr holding e.
- * Ids must be < 2^32 - 1.  Stands in for OnIndicesSlicingCUDA
+ * Ids are any int64 values (picked ids of 2^32 - 1 and above switch the
+ * look-ups to confirming every match against the picked id, as in the unique
+ * pass); at most 2^30 - 1 picked ids.  Stands in for OnIndicesSlicingCUDA
  * (src/cuda/slicing.cu:296-307) and COORowSlicingCUDA (src/cuda/slicing.cu:374-377).
  * ---------------------------------------------------------------------- */
 size_t gs_minor_slice_workspace_bytes(int64_t nnz, int64_t num_picked);

@@ -39,6 +39,41 @@ def test_minor_slice_parity(npick):
          orc.minor_slice(indices, picked, indptr=indptr, with_major=False))
 
 
+@pytest.mark.parametrize("npick", [3, 700, 5000])
+def test_minor_slice_with_ids_beyond_32_bits(npick):
+    """Picked ids of 2^32 - 1 and above: ids that agree in their low 32 bits must
+    not be taken for each other, repeated picked ids keep their smallest
+    position, and a narrow picked set still ignores wide edge ids."""
+    rng = np.random.default_rng(npick)
+    indptr, _ = random_csc(rng, 2000, 10, 60, hub_deg=30000)
+    nnz = int(indptr[-1])
+    low = rng.integers(0, 3000, size=nnz)
+    low[rng.random(nnz) < 0.01] = 2**32 - 1
+    ids = low + rng.integers(0, 4, size=nnz) * 2**32          # four ids per low half
+    ids[:7] = [-3, 2**40, 2**32 - 1, 2**32 - 2, 2**63 - 1, 0, 2**32]
+    col = np.repeat(np.arange(2000), np.diff(indptr))
+    picked = rng.choice(ids, size=npick)
+    picked[: min(npick, 3)] = [2**40, 2**32 - 1, -3][: min(npick, 3)]
+    if npick > 10:
+        picked[5] = picked[9]                                  # a repeated picked id
+        picked[7] = 2**50 + 11                                 # one that no edge carries
+    got = capi.minor_slice(T(ids), T(picked), indptr=T(indptr))
+    same(got, orc.minor_slice(ids, picked, indptr=indptr))
+    same(capi.minor_slice(T(ids), T(picked), edge_major=T(col)),
+         orc.minor_slice(ids, picked, edge_major=col))
+    # closed form: kept edges and their positions in the picked list
+    first = {}
+    for i, v in enumerate(picked.tolist()):
+        first.setdefault(v, i)
+    keep = np.array([v in first for v in ids.tolist()])
+    assert np.array_equal(got[3].cpu().numpy(), np.nonzero(keep)[0])
+    assert np.array_equal(got[2].cpu().numpy(), np.array([first[v] for v in ids[keep].tolist()]))
+    # a narrow picked set against the same wide edge ids
+    narrow = rng.integers(0, 3000, size=50)
+    same(capi.minor_slice(T(ids), T(narrow), indptr=T(indptr)),
+         orc.minor_slice(ids, narrow, indptr=indptr))
+
+
 def test_reference_rowwise_slicing_through_the_api():
     # tests/test_rowwise_slicing.cc:7-24
     indptr = torch.cat([torch.zeros(10, dtype=torch.int64), torch.arange(3) * 2]).to(DEV)
@@ -120,3 +155,41 @@ def test_relabel_of_a_row_sliced_matrix(num_rows_picked, max_deg):
     for l in range(num_rows_picked):
         hits = np.nonzero(r == l)[0]
         assert first[l] == (hits[0] if hits.size else np.iinfo(np.int64).max)
+
+
+def test_batched_column_and_row_slice_whose_encoded_ids_pass_32_bits():
+    """_CAPI_BatchColRowSlcing encodes a row of batch b as id + b * num_rows
+    (src/cuda/batch/slicing.cu:25-27).  With 2^30 + 5 rows and 8 batches the
+    encoded ids reach 2^33: every batch must still keep exactly the edges of its
+    columns whose row it picked, relabelled to positions in `row`."""
+    rng = np.random.default_rng(8)
+    num_rows, num_cols, B = 2**30 + 5, 300, 8
+    deg = rng.integers(0, 40, size=num_cols)
+    indptr = np.concatenate([[0], np.cumsum(deg)])
+    pool = np.concatenate([rng.integers(0, num_rows, size=400), [num_rows - 1, 0, 2**30]])
+    indices = rng.choice(pool, size=int(indptr[-1]))
+    g = gs.Graph(num_rows, num_cols)
+    g._CAPI_LoadCSC(T(indptr), T(indices))
+    cols = np.concatenate([rng.permutation(num_cols)[:30] for _ in range(B)])
+    col_bptr = np.arange(B + 1) * 30
+    rows = np.concatenate([rng.choice(pool, size=120, replace=False) for _ in range(B)])
+    row_bptr = np.arange(B + 1) * 120
+    sub, edge_index = g._CAPI_BatchColRowSlcing(T(cols), T(col_bptr), T(rows), T(row_bptr))
+    got_indptr = sub._CAPI_GetCSCIndptr().cpu().numpy()
+    got_rows = sub._CAPI_GetCSCIndices().cpu().numpy()
+    got_sel = edge_index.cpu().numpy()
+    want_rows, want_sel, want_cnt = [], [], []
+    for b in range(B):
+        where = {int(v): row_bptr[b] + i for i, v in enumerate(rows[row_bptr[b]:row_bptr[b + 1]])}
+        for c in cols[col_bptr[b]:col_bptr[b + 1]]:
+            n = 0
+            for e in range(indptr[c], indptr[c + 1]):
+                if int(indices[e]) in where:
+                    want_rows.append(where[int(indices[e])])
+                    want_sel.append(e)
+                    n += 1
+            want_cnt.append(n)
+    assert len(want_sel) > 500 and max(want_rows) >= 7 * 120       # the later batches kept theirs
+    assert np.array_equal(got_indptr, np.concatenate([[0], np.cumsum(want_cnt)]))
+    assert np.array_equal(got_rows, np.array(want_rows))
+    assert np.array_equal(got_sel, np.array(want_sel))

@@ -215,15 +215,52 @@ def test_format_and_batch_helpers_parity():
                           orc.split_indptr(indptr, offset))
 
 
-def test_unique_rejects_ids_that_do_not_fit():
-    seeds = np.array([1, 2, 3])
-    for bad in (2**32 - 1, 2**40, -5):
-        rows = np.array([5, bad, 7])
-        with pytest.raises(capi.GsError):
-            capi.unique_relabel(T(seeds), T(rows))
-    # the largest admissible id still works afterwards
-    assert_same(capi.unique_relabel(T(seeds), T(np.array([2**32 - 2, 5]))),
-                orc.unique_relabel(seeds, np.array([2**32 - 2, 5])))
+@pytest.mark.parametrize("B", [1, 5])
+@pytest.mark.parametrize("shape", ["mixed", "tag_collisions", "hubs"])
+def test_unique_relabel_with_ids_beyond_32_bits(B, shape):
+    """Ids of 2^32 - 1 and above (up to 2^40, and negative ones) go through the
+    same kernels; the packed entries then carry only a 32-bit tag and every tag
+    match is confirmed against the keys themselves.  `tag_collisions`: many
+    distinct ids that agree in their low 32 bits (and repeat), so that equal tags
+    meet in one table; `hubs`: two wide ids that repeat tens of thousands of
+    times (buckets beyond the LDS table's sure size)."""
+    rng = np.random.default_rng(B + len(shape))
+    n_s, n_r = 400 * B, 60000 * B
+    if shape == "mixed":
+        pool = np.concatenate([rng.integers(0, 1000, size=300),
+                               rng.integers(2**32 - 3, 2**32 + 3, size=50),
+                               rng.integers(2**32, 2**40, size=3000),
+                               np.array([2**40, -5, -1, 2**32 - 1, 2**63 - 1])])
+    elif shape == "tag_collisions":
+        low = rng.integers(0, 40, size=4000)
+        low[:10] = 2**32 - 1                       # the tag that has to be moved
+        pool = low + rng.integers(0, 50, size=4000) * 2**32
+    else:
+        pool = np.concatenate([rng.integers(2**33, 2**34, size=20000),
+                               np.full(30000, 2**35 + 7), np.full(30000, 2**35 + 7 + 2**32)])
+    seeds = rng.choice(pool, size=n_s)
+    rows = rng.choice(pool, size=n_r)
+    sp = rp = None
+    if B > 1:
+        sp = np.arange(B + 1) * 400
+        cuts = np.sort(rng.integers(0, n_r, size=B - 1))
+        rp = np.concatenate([[0], cuts, [n_r]])
+        edge_col = np.concatenate([rng.integers(sp[b], sp[b + 1], size=rp[b + 1] - rp[b])
+                                   for b in range(B)]).astype(np.int64)
+    else:
+        edge_col = rng.integers(0, n_s, size=n_r)
+    got = capi.unique_relabel(T(seeds), T(rows), T(sp) if B > 1 else None,
+                              T(rp) if B > 1 else None, T(edge_col))
+    want = orc.unique_relabel(seeds, rows, sp, rp, edge_col)
+    assert_same(got, want)
+    # independent closed form for one batch: first occurrences in order
+    if B == 1:
+        keys = np.concatenate([seeds, rows])
+        _, idx = np.unique(keys, return_index=True)
+        assert np.array_equal(N(got[0]), keys[np.sort(idx)])
+    # narrow ids still work afterwards (the flag is per call)
+    small = rng.integers(0, 500, size=5000)
+    assert_same(capi.unique_relabel(T(small[:50]), T(small)), orc.unique_relabel(small[:50], small))
 
 
 @pytest.mark.parametrize("num_ids", [1, 300, 4096, 5000])
