@@ -65,7 +65,7 @@ SIGNATURES = {
     "gs_coo_sort": (_int, [_p, _i64, _i64, _p, _p, _p, _sz, _p]),
     "gs_sddmm": (_int, [_int, _p, _p, _i64, _i64, _p, _int, _int, _p, _p, _p, _int, _int,
                         _i64, _i64, _i64, _i64, _p, _p, _p]),
-    "gs_fused_u_op_v": (_int, [_int, _p, _p, _i64, _i64, _int, _int, _p, _p, _p, _p, _p,
+    "gs_fused_u_op_v": (_int, [_int, _p, _p, _i64, _i64, _p, _int, _int, _p, _p, _p, _p, _p,
                                _p, _i64, _i64, _i64, _i64, _p, _p, _p]),
     "gs_spmm_workspace_bytes": (_sz, [_int, _i64, _i64]),
     "gs_spmm": (_int, [_int, _p, _p, _i64, _i64, _p, _int, _int, _p, _p, _p, _p, _p, _int,
@@ -459,7 +459,7 @@ def sddmm(view, op, lhs, rhs, lhs_target, rhs_target, edge_map=None):
     return out
 
 
-def fused_u_op_v(view, op, lhs1, rhs1, lhs2, rhs2):
+def fused_u_op_v(view, op, lhs1, rhs1, lhs2, rhs2, edge_map=None):
     fmt, a, b, nmaj, nnz = _view(view)
     lhs1, llen = _feat(lhs1)
     rhs1, rlen = _feat(rhs1)
@@ -469,7 +469,7 @@ def fused_u_op_v(view, op, lhs1, rhs1, lhs2, rhs2):
     out1 = torch.zeros(shape, dtype=lhs1.dtype, device=lhs1.device)
     out2 = torch.zeros_like(out1)
     dtype = 0 if lhs1.dtype == torch.float32 else 1
-    check(lib().gs_fused_u_op_v(fmt, _ptr(a), _ptr(b), nmaj, nnz, OPS[op], dtype,
+    check(lib().gs_fused_u_op_v(fmt, _ptr(a), _ptr(b), nmaj, nnz, _ptr(edge_map), OPS[op], dtype,
                                 _fptr(lhs1), _fptr(rhs1), _fptr(out1), _fptr(lhs2),
                                 _fptr(rhs2), _fptr(out2), llen, rlen, llen, 1, None, None,
                                 _stream()))

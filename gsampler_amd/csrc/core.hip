@@ -215,7 +215,7 @@ extern "C" {
 
 const char* gs_last_error(void) { return gs::g_last_error.c_str(); }
 
-int gs_abi_version(void) { return 1; }
+int gs_abi_version(void) { return 2; }
 
 void gs_profile_enable(int on) {
   std::lock_guard<std::mutex> lock(gs::g_prof_mutex);

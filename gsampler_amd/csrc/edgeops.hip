@@ -526,18 +526,10 @@ struct RowRangePlan {
          off_unit_start = 0, off_partial = 0, total = 0;
 };
 
-static bool row_range_enabled() {
-  static const bool on = [] {
-    const char* v = getenv("GS_SPMM_PARTITION");
-    return v == nullptr || atoi(v) != 0;
-  }();
-  return on;
-}
-
 // Worth it when the slice is large and rows repeat; empty plan otherwise.
 static RowRangePlan row_range_plan(int format, int64_t nnz, int64_t num_out) {
   RowRangePlan p;
-  if (!row_range_enabled() || format != GS_FMT_COO || nnz < kPrivateMinEdges ||
+  if (format != GS_FMT_COO || nnz < kPrivateMinEdges ||
       nnz >= ((int64_t)1 << 31) || num_out <= 0 || num_out > nnz / 4 ||
       ceil_div(num_out, kRangeRows) > kMaxRanges)
     return p;
@@ -874,7 +866,8 @@ int gs_sddmm(int format, const int64_t* a, const int64_t* b, int64_t num_major,
 }
 
 int gs_fused_u_op_v(int format, const int64_t* a, const int64_t* b,
-                    int64_t num_major, int64_t nnz, int op, int dtype,
+                    int64_t num_major, int64_t nnz, const int64_t* edge_map,
+                    int op, int dtype,
                     const void* lhs1, const void* rhs1, void* out1,
                     const void* lhs2, const void* rhs2, void* out2,
                     int64_t lhs_len, int64_t rhs_len, int64_t out_len,
@@ -889,7 +882,7 @@ int gs_fused_u_op_v(int format, const int64_t* a, const int64_t* b,
   if (nnz == 0 || out_len == 0) return GS_OK;
   GS_REQUIRE(lhs1 && rhs1 && out1 && lhs2 && rhs2 && out2, "fused_u_op_v: null operand");
   hipStream_t s = as_stream(stream);
-  const EdgeView g{format == GS_FMT_COMPRESSED, a, b, num_major, nullptr};
+  const EdgeView g{format == GS_FMT_COMPRESSED, a, b, num_major, edge_map};
 #define GS_UOPV_LAUNCH(T, ITEMS)                                                          \
   GS_LAUNCH("fused_u_op_v", s,                                                            \
             (fused_u_op_v_kernel<T, ITEMS>)<<<dim3((unsigned)ceil_div(nnz * out_len,      \

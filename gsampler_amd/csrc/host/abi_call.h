@@ -219,29 +219,39 @@ class OffsetMirror {
 // once and then found in the mirror while it stays unchanged.
 class BatchOffsets {
  public:
-  static void trust(const torch::Tensor& offsets) {
+  // `total`: the last entry, when the producer knows it on the host; -1 when it
+  // is still on its way from the device (looked up on first use).
+  static void trust(const torch::Tensor& offsets, int64_t total = -1) {
     if (!offsets.defined()) return;
     Known& k = ring()[next()++ % kEntries];
     k.tensor = offsets;  // kept alive: neither its address nor its memory can be handed out again
     k.version = (int64_t)offsets._version();
+    k.total = total;
   }
   static void check(const torch::Tensor& offsets, int64_t total, const char* who) {
     TORCH_CHECK(offsets.defined() && offsets.scalar_type() == torch::kInt64 &&
                     offsets.dim() == 1 && offsets.numel() >= 2,
                 who, ": batch offsets must be an int64 vector with at least two entries");
-    if (trusted(offsets)) return;
+    if (Known* k = trusted(offsets)) {
+      // a well-formed array, but it must also split a sequence of this length
+      if (k->total < 0) k->total = OffsetMirror::values(offsets).back();
+      TORCH_CHECK(k->total == total, who, ": batch offsets end at ", k->total,
+                  " but split ", total, " elements");
+      return;
+    }
     const std::vector<int64_t>& p = OffsetMirror::values(offsets);
     bool ok = p.front() == 0 && p.back() == total;
     for (size_t i = 1; ok && i < p.size(); ++i) ok = p[i] >= p[i - 1];
     TORCH_CHECK(ok, who, ": batch offsets must start at 0, never decrease and end at ",
                 total, " (found ", p.front(), " .. ", p.back(), ")");
-    trust(offsets);
+    trust(offsets, total);
   }
 
  private:
   struct Known {
     torch::Tensor tensor;
     int64_t version = -1;
+    int64_t total = -1;
   };
   static constexpr size_t kEntries = 32;
   static std::vector<Known>& ring() {
@@ -252,11 +262,11 @@ class BatchOffsets {
     static thread_local size_t n = 0;
     return n;
   }
-  static bool trusted(const torch::Tensor& t) {
-    for (const Known& k : ring())
+  static Known* trusted(const torch::Tensor& t) {
+    for (Known& k : ring())
       if (k.tensor.defined() && k.tensor.is_same(t) && k.version == (int64_t)t._version())
-        return true;
-    return false;
+        return &k;
+    return nullptr;
   }
 };
 

@@ -179,6 +179,9 @@ Graph::BatchGraphRelabel(torch::Tensor col_seeds, torch::Tensor row_ids) {
   TORCH_CHECK(coo_->col_sorted,
               "BatchGraphRelabel: the COO format must be column-sorted");
   col_seeds = ids(col_seeds, "col_seeds");
+  // the kernels read seeds[col_bptr[b] ...]: the seeds must be the ones the
+  // batch pointer was recorded for
+  BatchOffsets::check(col_bptr_, col_seeds.numel(), "BatchGraphRelabel");
   torch::Tensor rows = batch_rows_for_relabel(row_ids);
   Frontier& f = frontier_for(col_seeds, rows, col_bptr_, edge_bptr_);
   const int64_t E = rows.numel(), B = f.num_batches;
@@ -199,6 +202,7 @@ std::tuple<torch::Tensor, torch::Tensor> Graph::BatchGetValidNodes(
   TORCH_CHECK(coo_->col_sorted,
               "BatchGetValidNodes: the COO format must be column-sorted");
   col_seeds = ids(col_seeds, "col_seeds");
+  BatchOffsets::check(col_bptr_, col_seeds.numel(), "BatchGetValidNodes");
   torch::Tensor rows = batch_rows_for_relabel(row_ids);
   Frontier& f = frontier_for(col_seeds, rows, col_bptr_, edge_bptr_);
   return {f.frontier(), f.unique_ptr};

@@ -200,7 +200,7 @@ void Graph::FusedUOPV(const std::string& op, torch::Tensor lhs1,
               "FusedUOPV: outputs are too small for ", num_edges_, " edges");
   const StructureArgs s = on_format == kCOO ? structure_of(*coo_)
                                             : structure_of(compressed(kCSC));
-  GS_CALL(gs_fused_u_op_v(s.format, s.a, s.b, s.num_major, s.nnz, op_code(op),
+  GS_CALL(gs_fused_u_op_v(s.format, s.a, s.b, s.num_major, s.nnz, s.edge_map, op_code(op),
                           dtype_code(out1), fptr(lhs1), fptr(rhs1),
                           out1.data_ptr(), fptr(lhs2), fptr(rhs2),
                           out2.data_ptr(), bc.lhs_len, bc.rhs_len, bc.out_len,

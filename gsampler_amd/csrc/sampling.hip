@@ -8,8 +8,6 @@
 // only, so divergent columns never meet at a block barrier.
 #include "common.h"
 
-#include <cstdlib>
-
 namespace gs {
 
 // Reads a value that other lanes may have updated with an atomic, bypassing
@@ -169,16 +167,6 @@ __global__ __launch_bounds__(kBlock) void sample_uniform_kernel(
   }
 }
 
-// Columns per group (GS_SAMPLE_ILP: 1, 2 or 4).  Read once.
-static int sample_ilp() {
-  static const int v = [] {
-    const char* e = getenv("GS_SAMPLE_ILP");
-    const int x = e ? atoi(e) : 1;
-    return x >= 4 ? 4 : (x >= 2 ? 2 : 1);
-  }();
-  return v;
-}
-
 template <int G>
 static int launch_sample_uniform(const int64_t* indptr, int64_t num_cols,
                                  const int64_t* indices,
@@ -187,22 +175,13 @@ static int launch_sample_uniform(const int64_t* indptr, int64_t num_cols,
                                  PhiloxKey key, const int64_t* sub_indptr,
                                  int64_t* out_coo_col, int64_t* out_indices,
                                  int64_t* out_select, hipStream_t stream) {
-  const int U = sample_ilp();
-  const int64_t blocks = ceil_div(ceil_div(num_items, U) * G, kBlock);
-#define GS_SAMPLE_LAUNCH(UU)                                                   \
-  GS_LAUNCH("sample_uniform", stream,                                          \
-            sample_uniform_kernel<G, UU><<<dim3((unsigned)blocks), dim3(kBlock), \
-                                           0, stream>>>(                       \
-                indptr, num_cols, indices, column_ids, num_items, fanout,      \
-                replace, algo, key, sub_indptr, out_coo_col, out_indices,      \
-                out_select))
-  if (U == 4)
-    GS_SAMPLE_LAUNCH(4);
-  else if (U == 2)
-    GS_SAMPLE_LAUNCH(2);
-  else
-    GS_SAMPLE_LAUNCH(1);
-#undef GS_SAMPLE_LAUNCH
+  // one column per lane group (see the note on U above the kernel)
+  const int64_t blocks = ceil_div(num_items * G, kBlock);
+  GS_LAUNCH("sample_uniform", stream,
+            sample_uniform_kernel<G, 1><<<dim3((unsigned)blocks), dim3(kBlock), 0,
+                                          stream>>>(
+                indptr, num_cols, indices, column_ids, num_items, fanout, replace,
+                algo, key, sub_indptr, out_coo_col, out_indices, out_select));
   return GS_OK;
 }
 

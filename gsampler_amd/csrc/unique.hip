@@ -45,8 +45,6 @@
 #include "hashtable.h"
 #include "scan.h"
 
-#include <cstdlib>
-
 namespace gs {
 
 constexpr int kWordsPerBlock = kBlock / kWave;
@@ -58,27 +56,16 @@ constexpr int kMaxBuckets = 2048;                 // buckets per batch (LDS bins
 constexpr int kLdsSlots = 4096;                   // dedup table, 32 KB of LDS
 constexpr int kLdsMaxEntries = kLdsSlots * 3 / 4; // bucket sizes the LDS table takes
 
-// Average entries per bucket (GS_BUCKET_KEYS), threads of a dedup work-group
-// (GS_DEDUP_THREADS: 256 or 512) and whether work-groups are laid out per die
-// (GS_XCD_REMAP).  The defaults are the best of a sweep on 21M keys in 64
-// batches; the variables exist for such sweeps.  Read once.
+// Average entries per bucket, threads of a dedup work-group and whether
+// work-groups are laid out per die: the best of a sweep on 21M keys in 64
+// batches (bucket sizes 512..3072, 256 or 512 threads, with and without the
+// per-die layout).
 struct UniqueTuning {
   int64_t bucket_keys;
   int remap;
   int dedup_threads;
 };
-static UniqueTuning tuning() {
-  static const UniqueTuning t = [] {
-    UniqueTuning r{1536, 1, 512};
-    if (const char* e = getenv("GS_DEDUP_THREADS")) r.dedup_threads = atoi(e);
-    if (const char* e = getenv("GS_BUCKET_KEYS")) r.bucket_keys = atoll(e);
-    if (const char* e = getenv("GS_XCD_REMAP")) r.remap = atoi(e);
-    if (r.bucket_keys < 64) r.bucket_keys = 64;
-    if (r.bucket_keys > kLdsMaxEntries) r.bucket_keys = kLdsMaxEntries;
-    return r;
-  }();
-  return t;
-}
+static UniqueTuning tuning() { return UniqueTuning{1536, 1, 512}; }
 
 // Work-group index -> unit of work (tile or bucket).  Consecutive work-groups
 // go to consecutive dies, so die x is given the x-th eighth of the units, in
@@ -409,13 +396,22 @@ __global__ __launch_bounds__(kBlock) void unique_scatter_kernel(
     }
     return;
   }
-  for (uint32_t i = threadIdx.x; i < buckets; i += kBlock) hist[i] = 0;
-  __syncthreads();
   uint32_t key[kPartItems], place[kPartItems];
 #pragma unroll
   for (int i = 0; i < kPartItems; ++i) {
+    // All loads in flight before anything else: a position past the end reads
+    // the tile's last key instead of branching around the load (the compiler
+    // otherwise moves the first use of the key into that branch and waits
+    // there, one load at a time).
     const int64_t l = t.begin + i * kBlock + threadIdx.x;
-    key[i] = l < t.end ? key_tag(key_at(k, t.b, l)) : 0u;
+    key[i] = (uint32_t)key_at(k, t.b, l < t.end ? l : t.end - 1);
+  }
+  for (uint32_t i = threadIdx.x; i < buckets; i += kBlock) hist[i] = 0;
+  __syncthreads();
+#pragma unroll
+  for (int i = 0; i < kPartItems; ++i) {
+    const int64_t l = t.begin + i * kBlock + threadIdx.x;
+    key[i] = key_tag(key[i]);
     // every position starts as its own first occurrence; the dedup pass only
     // writes the positions that are not (half as many scattered stores)
     if (l < t.end) first[t.b.fb + l] = (uint32_t)l;
@@ -474,18 +470,19 @@ __global__ __launch_bounds__(kBlock) void unique_scatter_kernel(
 // Whether two entries with the same upper half stand for the same key: always
 // when every key of the call fits that half; otherwise the keys themselves are
 // read back through the entries' positions and compared.
+template <bool kWide>
 struct SameKey {
   const Keys* k;
   const BatchInfo* b;
-  bool wide;
   __device__ __forceinline__ bool operator()(uint64_t a, uint64_t c) const {
-    if (!wide) return true;
+    if (!kWide) return true;
     return key_at(*k, *b, (int64_t)(uint32_t)a) == key_at(*k, *b, (int64_t)(uint32_t)c);
   }
 };
 
+template <typename Same>
 __device__ __forceinline__ void lds_insert_min(uint64_t* tab, uint32_t mask,
-                                               uint64_t entry, const SameKey& same) {
+                                               uint64_t entry, const Same& same) {
   const uint64_t tag = entry >> 32;
   uint32_t slot = slot_hash(tag) & mask;
   for (;;) {
@@ -505,14 +502,16 @@ __device__ __forceinline__ void lds_insert_min(uint64_t* tab, uint32_t mask,
   }
 }
 
+template <typename Same>
 __device__ __forceinline__ uint32_t lds_first_of(const uint64_t* tab,
                                                  uint32_t mask, uint64_t entry,
-                                                 const SameKey& same) {
+                                                 const Same& same) {
   const uint64_t tag = entry >> 32;
   uint32_t slot = slot_hash(tag) & mask;
   for (;;) {
     const uint64_t cur = tab[slot];
-    if (cur == kEmptySlot) return (uint32_t)entry;  // not reached: every entry was inserted
+    // (an empty slot is never met: every entry looked up was inserted, and no
+    // tag equals the upper half of the empty pattern)
     if ((cur >> 32) == tag && same(cur, entry)) return (uint32_t)cur;
     slot = (slot + 1) & mask;
   }
@@ -524,8 +523,9 @@ __device__ __forceinline__ uint64_t load_l2(const uint64_t* p) {
   return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
+template <typename Same>
 __device__ __forceinline__ void spill_insert_min(uint64_t* tab, uint64_t cap,
-                                                 uint64_t entry, const SameKey& same) {
+                                                 uint64_t entry, const Same& same) {
   const uint64_t tag = entry >> 32;
   uint64_t slot = ((uint64_t)slot_hash(tag) * cap) >> 32;
   for (uint64_t probes = 0; probes < cap; ++probes) {
@@ -544,9 +544,10 @@ __device__ __forceinline__ void spill_insert_min(uint64_t* tab, uint64_t cap,
   }
 }
 
+template <typename Same>
 __device__ __forceinline__ uint32_t spill_first_of(const uint64_t* tab,
                                                    uint64_t cap, uint64_t entry,
-                                                   const SameKey& same) {
+                                                   const Same& same) {
   const uint64_t tag = entry >> 32;
   uint64_t slot = ((uint64_t)slot_hash(tag) * cap) >> 32;
   for (uint64_t probes = 0; probes < cap; ++probes) {
@@ -561,10 +562,11 @@ __device__ __forceinline__ uint32_t spill_first_of(const uint64_t* tab,
 // Same as lds_insert_min for a bucket that may hold more distinct keys than the
 // table takes: counts the slots it claims and raises *overflow instead of
 // filling the table up.
+template <typename Same>
 __device__ __forceinline__ void lds_insert_min_counted(uint64_t* tab,
                                                        uint32_t mask,
                                                        uint64_t entry,
-                                                       const SameKey& same,
+                                                       const Same& same,
                                                        uint32_t* distinct,
                                                        volatile uint32_t* overflow) {
   const uint64_t tag = entry >> 32;
@@ -588,25 +590,15 @@ __device__ __forceinline__ void lds_insert_min_counted(uint64_t* tab,
   }
 }
 
-template <int kThreads>
-__global__ __launch_bounds__(kThreads) void unique_dedup_kernel(
-    Keys k, const int* __restrict__ wide_keys,
-    const int32_t* __restrict__ bucket_batch, const BatchInfo* __restrict__ batch,
-    const int64_t* __restrict__ bucket_off, const uint64_t* __restrict__ packed,
-    uint64_t* spill, uint32_t* __restrict__ first, int64_t max_buckets,
-    int remap) {
-  __shared__ uint64_t tab[kLdsSlots];
-  __shared__ uint32_t distinct;
-  __shared__ uint32_t overflow;
-  const int64_t g = unit_of_block(max_buckets, remap);
-  if (g >= max_buckets) return;
-  const int32_t b = bucket_batch[g];
-  if (b < 0) return;  // uniform per work-group
-  const int64_t lo = bucket_off[g], hi = bucket_off[g + 1];
+template <int kThreads, bool kWide>
+__device__ __forceinline__ void dedup_bucket(
+    const Keys& k, const BatchInfo& info, int64_t g, int64_t lo, int64_t hi,
+    const uint64_t* __restrict__ packed, uint64_t* spill, uint32_t* __restrict__ first,
+    uint64_t* tab, uint32_t* distinct_ptr, uint32_t* overflow_ptr) {
+  uint32_t& distinct = *distinct_ptr;
+  uint32_t& overflow = *overflow_ptr;
   const int64_t n = hi - lo;
-  if (n == 0) return;
-  const BatchInfo info = batch[b];
-  const SameKey same{&k, &info, *wide_keys != 0};
+  const SameKey<kWide> same{&k, &info};
   uint32_t* first_b = first + info.fb;
   // table of two slots per entry, a power of two, at most kLdsSlots
   uint32_t slots = 256;
@@ -688,6 +680,34 @@ __global__ __launch_bounds__(kThreads) void unique_dedup_kernel(
     const uint32_t f = spill_first_of(gt, cap, e, same);
     if (f != (uint32_t)e) first_b[(uint32_t)e] = f;
   }
+}
+
+// One work-group per bucket.  The two forms of the body differ only in whether
+// a match of the upper halves is confirmed against the keys; which one runs is
+// the same for every work-group of a launch.
+template <int kThreads>
+__global__ __launch_bounds__(kThreads) void unique_dedup_kernel(
+    Keys k, const int* __restrict__ wide_keys,
+    const int32_t* __restrict__ bucket_batch, const BatchInfo* __restrict__ batch,
+    const int64_t* __restrict__ bucket_off, const uint64_t* __restrict__ packed,
+    uint64_t* spill, uint32_t* __restrict__ first, int64_t max_buckets,
+    int remap) {
+  __shared__ uint64_t tab[kLdsSlots];
+  __shared__ uint32_t distinct;
+  __shared__ uint32_t overflow;
+  const int64_t g = unit_of_block(max_buckets, remap);
+  if (g >= max_buckets) return;
+  const int32_t b = bucket_batch[g];
+  if (b < 0) return;  // uniform per work-group
+  const int64_t lo = bucket_off[g], hi = bucket_off[g + 1];
+  if (hi == lo) return;
+  const BatchInfo info = batch[b];
+  if (*wide_keys)
+    dedup_bucket<kThreads, true>(k, info, g, lo, hi, packed, spill, first, tab, &distinct,
+                                 &overflow);
+  else
+    dedup_bucket<kThreads, false>(k, info, g, lo, hi, packed, spill, first, tab, &distinct,
+                                  &overflow);
 }
 
 // ---------------------------------------------------------------- flag

@@ -515,16 +515,9 @@ __global__ __launch_bounds__(kBlock) void sample_weighted_cdf_kernel(
   }
 }
 
-// Search mode of the CDF sampler (GS_WCDF_SEARCH: 0 bisection, 1 alternating,
-// 2 interpolation first).  Read once.
-static int cdf_search_mode() {
-  static const int mode = [] {
-    int m = 2;
-    if (const char* e = getenv("GS_WCDF_SEARCH")) m = atoi(e);
-    return m < 0 || m > 2 ? 1 : m;
-  }();
-  return mode;
-}
+// Search mode of the CDF sampler: 0 bisection, 1 alternating, 2 interpolation
+// first (the fastest on prefix sums of real weights, which are nearly linear).
+constexpr int kCdfSearchMode = 2;
 
 template <int KMAX>
 static int launch_weighted_cdf(const int64_t* indptr, int64_t num_cols,
@@ -538,7 +531,7 @@ static int launch_weighted_cdf(const int64_t* indptr, int64_t num_cols,
             sample_weighted_cdf_kernel<KMAX><<<dim3((unsigned)ceil_div(num_items, kBlock)),
                                                dim3(kBlock), 0, s>>>(
                 indptr, num_cols, indices, cdf, column_ids, num_items, fanout, replace,
-                key, sub_indptr, out_coo_col, out_indices, out_select, cdf_search_mode()));
+                key, sub_indptr, out_coo_col, out_indices, out_select, kCdfSearchMode));
   return GS_OK;
 }
 

@@ -44,19 +44,50 @@ def matrix_parts(args: Sequence[Any], kinds: Sequence[str]) -> Tuple[list, list]
 
 
 class compile:  # noqa: N801 -- the reference's public name
-    def __init__(self, func, args, try_compact=True, format_select=True, must_compact=False):
+    def __init__(self, func, args, try_compact=None, format_select=True, must_compact=False):
+        """try_compact: None (the default) or False keep row ids as they are;
+        True runs the reference's search (python/gs/jit/module.py:306-421): both
+        variants of the graph are built and timed on `args`, the faster is kept.
+        Compaction renumbers rows densely after every slice, so a sampler that
+        draws from the rows of a slice draws other (equally valid) samples in
+        the compact variant: the search is therefore only run on request, and
+        the sampler's random state is put back afterwards.  must_compact forces
+        the compact variant.  Super-batches are never compacted."""
         self.func = func
         self.kinds = classify(args)
         self.static_args = [a for a, k in zip(args, self.kinds) if k == STATIC]
         self.encodings = [a.encoding for a, k in zip(args, self.kinds) if k == BATCH_MATRIX]
         self.use_batchmatrix = BATCH_MATRIX in self.kinds
         self._format_select = format_select
-        # Compaction renumbers rows densely after every slice.  The reference
-        # times both variants and keeps the faster; here the choice is explicit:
-        # compact only when asked to (must_compact), never for super-batches.
         self.compact = bool(must_compact) and not self.use_batchmatrix
-        self.try_compact = try_compact
+        self.try_compact = bool(try_compact)
         self.gm = self._build(args, self.compact)
+        self.compact_search_ms = None
+        if self.try_compact and not self.compact and not self.use_batchmatrix:
+            other = self._build(args, True)
+            plain_ms, compact_ms = self._time(self.gm, args), self._time(other, args)
+            self.compact_search_ms = (plain_ms, compact_ms)
+            if compact_ms < plain_ms:
+                self.gm, self.compact = other, True
+
+    def _time(self, gm, args, runs=3):
+        """Milliseconds per call of one variant on the example arguments."""
+        import time
+        seed, next_call = torch.ops.gs_ops._CAPI_GetRandomState()
+        graphs, data = matrix_parts(args, self.kinds)
+        passthrough = tuple(None if k in (MATRIX, BATCH_MATRIX, STATIC) else a
+                            for a, k in zip(args, self.kinds))
+        try:
+            gm(passthrough, graphs, data)                 # warm-up
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(runs):
+                gm(passthrough, graphs, data)
+            torch.cuda.synchronize()
+            return (time.perf_counter() - t0) / runs * 1e3
+        finally:
+            torch.ops.gs_ops._CAPI_SetRandomSeed(int(seed))
+            torch.ops.gs_ops._CAPI_SetNextCallId(int(next_call))
 
     # ------------------------------------------------------------------ build
     def _rebuild_args(self, inner_args, graphs, data, compact):

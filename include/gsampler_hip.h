@@ -438,7 +438,10 @@ int gs_split_indptr(const int64_t* indptr, const int64_t* offset,
  * gs_sddmm: out[eid] = lhs[t_l] op rhs[t_r]            SDDMMCOO / SDDMMCSC,
  *   src/cuda/sddmm.cu:264-297.  fp32 or fp64.
  * gs_fused_u_op_v: two u-op-v SDDMMs in one sweep       FUSED_COO/CSC_U_OP_V,
- *   src/cuda/fusion/fused_coo_u_op_v.cu:109, fused_csc_u_op_v.cu:103.
+ *   src/cuda/fusion/fused_coo_u_op_v.cu:109, fused_csc_u_op_v.cu:103.  Outputs
+ *   are written through edge_map like gs_sddmm's (the reference's fused kernels
+ *   write by edge position, which differs from its own SDDMM on a converted
+ *   format).
  * gs_spmm: out[dst] = reduce(out[dst], op(u[src], e[eid])), fp32.  Outputs
  *   are accumulators: the caller zero-fills them (python/gs/ops/spmm.py:56).
  *   COO: u_target 0 reduces onto columns, 2 onto rows (atomics).  Compressed:
@@ -460,7 +463,8 @@ int gs_sddmm(int format, const int64_t* a, const int64_t* b, int64_t num_major,
              int64_t reduce_size, const int64_t* lhs_off, const int64_t* rhs_off,
              gs_stream_t stream);
 int gs_fused_u_op_v(int format, const int64_t* a, const int64_t* b,
-                    int64_t num_major, int64_t nnz, int op, int dtype,
+                    int64_t num_major, int64_t nnz, const int64_t* edge_map,
+                    int op, int dtype,
                     const void* lhs1, const void* rhs1, void* out1,
                     const void* lhs2, const void* rhs2, void* out2,
                     int64_t lhs_len, int64_t rhs_len, int64_t out_len,

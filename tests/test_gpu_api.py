@@ -291,3 +291,25 @@ def test_super_batch_with_an_empty_batch(graph):
         for x, y in zip(a, b):
             assert torch.equal(x.row, y.row) and torch.equal(x.col, y.col)
             assert torch.equal(x.srcdata["_ID"], y.srcdata["_ID"])
+
+
+def test_batch_pointer_is_bound_to_the_length_it_was_checked_for(graph):
+    """An offsets array accepted for one id tensor is not accepted for a shorter
+    one, and the batched relabel refuses seeds that do not match the batch
+    pointer of the slice (the kernels would read past their end)."""
+    m, _, _ = graph
+    g = m._graph
+    seeds = torch.arange(600, device=DEV)
+    ptr = torch.tensor([0, 100, 200, 600], device=DEV)
+    sub, _ = g._CAPI_BatchFusedSlicingSampling(seeds, ptr, 5, False)
+    with pytest.raises(RuntimeError, match="batch offsets"):
+        g._CAPI_BatchFusedSlicingSampling(seeds[:500], ptr, 5, False)
+    with pytest.raises(RuntimeError, match="batch offsets"):
+        sub._CAPI_BatchGraphRelabel(seeds[:590], torch.empty(0, dtype=torch.int64, device=DEV))
+    with pytest.raises(RuntimeError, match="batch offsets"):
+        sub._CAPI_BatchGetValidNodes(seeds[:590], torch.empty(0, dtype=torch.int64, device=DEV))
+    uniq, uptr = sub._CAPI_BatchGetValidNodes(seeds, torch.empty(0, dtype=torch.int64, device=DEV))
+    # the produced pointer is bound to the frontier it splits
+    sub2, _ = g._CAPI_BatchFusedSlicingSampling(uniq, uptr, 5, False)
+    with pytest.raises(RuntimeError, match="batch offsets"):
+        g._CAPI_BatchFusedSlicingSampling(uniq[:-1], uptr, 5, False)

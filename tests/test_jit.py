@@ -290,7 +290,10 @@ def test_ladies_eager_compiled_and_invariants():
     c_in, c_out, c_blocks = c(m, seeds, [64, 64])
     # The compiled graph slices rows on the CSC (edge order of the column slice)
     # where eager execution sorts into a CSR first, so edges and therefore the
-    # first-occurrence frontier come in another order: compare order-free.
+    # first-occurrence frontier come in another order: compare order-free.  (The
+    # two cannot be made to agree by running the eager slice on the CSC as well:
+    # a slice along the compressed axis repeats a row that is asked for twice,
+    # a slice across it cannot, so the format is part of the eager semantics.)
     assert torch.equal(e_out.sort().values, c_out.sort().values)
 
     def edge_list(blk, dst_ids):
@@ -390,3 +393,64 @@ def test_compiled_weighted_graphsage_matches_the_cdf_oracle():
     dst = s[blk.col.cpu().numpy()]
     edges = set(zip(np.repeat(np.arange(5000), deg).tolist(), indices.tolist()))
     assert all((int(d), int(u)) in edges for d, u in zip(dst, src))
+
+
+def two_products_on_the_loaded_matrix(A, u1, v1, u2, v2):
+    return gs.ops.u_mul_v(A, u1, v1), gs.ops.u_mul_v(A, u2, v2)
+
+
+@pytest.mark.gpu
+def test_merged_u_mul_v_keeps_the_edge_order_of_a_converted_format():
+    """A matrix loaded as an edge list in arbitrary order: whatever format the
+    compiled graph runs the merged operator on (a CSC derived from the edge list
+    carries the edge ids of the sort), its outputs stay in the order of the
+    loaded edges, as the two separate products give them."""
+    g = torch.Generator().manual_seed(12)
+    row = torch.randint(0, 40, (3000,), generator=g).to(DEV)
+    col = torch.randint(0, 30, (3000,), generator=g).to(DEV)
+    row[0], col[0] = 39, 29
+    m = gs.Matrix()
+    m.load_graph("COO", [row, col])
+    u1, u2 = torch.rand(40, generator=g).to(DEV), torch.rand(40, generator=g).to(DEV)
+    v1, v2 = torch.rand(30, generator=g).to(DEV), torch.rand(30, generator=g).to(DEV)
+    c = gs.jit.compile(func=two_products_on_the_loaded_matrix, args=(m, u1, v1, u2, v2))
+    assert targets(c.gm).count("_CAPI_FusedUOPV") == 1
+    for fmt in (gs._COO, gs._CSC):
+        o1, o2 = gs.ops.fused_u_mul_v(m, u1, v1, u2, v2, fmt)
+        assert torch.equal(o1, u1[row] * v1[col]) and torch.equal(o2, u2[row] * v2[col])
+    got = c(m, u1, v1, u2, v2)
+    want = two_products_on_the_loaded_matrix(m, u1, v1, u2, v2)
+    assert torch.equal(got[0], want[0]) and torch.equal(got[1], want[1])
+    assert torch.equal(want[0], u1[row] * v1[col])
+
+
+@pytest.mark.gpu
+def test_try_compact_runs_the_search_and_leaves_the_random_state_alone():
+    """try_compact=True builds and times both variants on the example arguments
+    and keeps one of them; the sampler's (seed, next call id) is what it was, so
+    the compiled function still draws the picks of an uncompiled run started
+    from the same state when the plain variant won, and valid blocks either way."""
+    m = _graph()
+    seeds = torch.arange(0, 2000, 9, device=DEV)
+    gs.manual_seed(31)
+    before = gs.random_state()
+    c = gs.jit.compile(func=graphsage_sampler, args=(m, seeds, [10, 5]), try_compact=True)
+    assert gs.random_state() == before
+    assert c.compact_search_ms is not None and len(c.compact_search_ms) == 2
+    assert c.compact == (c.compact_search_ms[1] < c.compact_search_ms[0])
+    out = c(m, seeds, [10, 5])
+    assert gs.random_state() == (31, 2)
+    blocks = out[-1]
+    assert blocks[0].num_dst == seeds.numel() and blocks[1].num_dst == blocks[0].num_src
+    indptr, indices, _ = m.csc
+    src = blocks[0].srcdata["_ID"][blocks[0].row]
+    dst = seeds[blocks[0].col]
+    lo, hi = indptr[dst], indptr[dst + 1]
+    # every block edge is an edge of the graph: its source occurs in the column of its target
+    found = torch.zeros_like(src, dtype=torch.bool)
+    for k in range(int((hi - lo).max())):
+        pos = (lo + k).clamp(max=indices.numel() - 1)
+        found |= (lo + k < hi) & (indices[pos] == src)
+    assert bool(found.all())
+    d = gs.jit.compile(func=graphsage_sampler, args=(m, seeds, [10, 5]))
+    assert d.compact is False and d.compact_search_ms is None
