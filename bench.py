@@ -153,11 +153,12 @@ def api_step_factory(indptr, indices, seeds, ptr, fanouts, probs):
 
     def step(i):
         layers = compiled(bm, seeds, ptr, fanouts)
+        # every layer is a BlockList: its blocks are views of the layer's arrays
         sizes = []
         for blocks in layers:
-            sizes.append((sum(b.num_dst for b in blocks), sum(b.num_edges() for b in blocks),
-                          sum(b.num_src for b in blocks)))
-        return sizes, None
+            src, dst, edges = blocks.totals()
+            sizes.append((dst, edges, src))
+        return sizes, layers
     return step
 
 
@@ -559,6 +560,8 @@ def main():
     ap.add_argument("--cpu-seconds", type=float, default=15.0,
                     help="target CPU time of the oracle baseline (0 = skip)")
     ap.add_argument("--seed", type=int, default=7777)
+    ap.add_argument("--no-api", action="store_true",
+                    help="skip the second timing of the same workload through the Python API")
     ap.add_argument("--path", default="abi", choices=["abi", "api"],
                     help="abi: the C ABI through ctypes (default); api: the same GraphSAGE "
                          "workload through BatchMatrix + gs.jit.compile and the torch "
@@ -673,6 +676,35 @@ def main():
         roofline["traffic_frac"] = round(moved / HBM_PEAK_GBS, 4)
     pipeline_bytes = sum(40 * S + 56 * E + 8 * U for S, E, U in sizes)
 
+    # ---- the same workload through the drop-in stack: BatchMatrix + gs.jit.compile +
+    # the torch operator class (libgs.so), every layer handed out as per-batch blocks
+    api = None
+    if args.path == "abi" and not args.no_api:
+        api_step = api_step_factory(indptr, indices, seeds, ptr, fanouts, probs)
+        for i in range(args.warmup):
+            api_step(i)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        api_edges = 0
+        for i in range(args.steps):
+            api_sizes, _ = api_step(args.warmup + i)
+            api_edges += sum(E for _, E, _ in api_sizes)
+        torch.cuda.synchronize()
+        api_elapsed = time.perf_counter() - t0
+        # ... and with a Block object made for every mini-batch of every layer
+        t0 = time.perf_counter()
+        made = 0
+        for i in range(args.steps):
+            _, layers = api_step(args.warmup + i)
+            made += sum(len(blocks.materialize()) for blocks in layers)
+        torch.cuda.synchronize()
+        api_made = time.perf_counter() - t0
+        api = dict(ms_per_step=round(api_elapsed / args.steps * 1e3, 3),
+                   value=round(api_edges / api_elapsed, 1),
+                   ms_per_step_blocks_materialised=round(api_made / args.steps * 1e3, 3),
+                   blocks_per_step=made // max(args.steps, 1),
+                   layer_sizes_match=bool(api_sizes == sizes))
+
     # ---- CPU baseline: the oracle on the first few batches of the same super-batch
     cpu = None
     if args.cpu_seconds > 0:
@@ -716,6 +748,9 @@ def main():
         "roofline": roofline,
         "cpu_baseline": cpu,
         "gpu_over_cpu": round(edges_per_s / cpu["value"], 1) if cpu else None,
+        "api_ms_per_step": api["ms_per_step"] if api else None,
+        "api_value": api["value"] if api else None,
+        "api": api,
         "kernels": [{k: (round(v, 4) if isinstance(v, float) else v) for k, v in kk.items()}
                     for kk in kernels],
         "graph_build_s": round(t_build, 1),

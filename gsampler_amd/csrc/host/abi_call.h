@@ -170,7 +170,10 @@ class OffsetMirror {
     bool pending = false;
     std::vector<int64_t> host;
   };
-  static constexpr size_t kEntries = 8;
+  // Deep enough that an entry is reused several sampler steps after its copy was
+  // queued (a step of a three-layer super-batched sampler announces about ten
+  // arrays): reusing one whose copy is still pending would stall the host.
+  static constexpr size_t kEntries = 64;
   static void check(hipError_t e) {
     TORCH_CHECK(e == hipSuccess, "HIP error: ", hipGetErrorString(e));
   }

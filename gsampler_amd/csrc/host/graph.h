@@ -52,6 +52,46 @@ struct RandomState {
 };
 RandomState& random_state();
 
+// Views of one mini-batch block: (row, col, indptr by destination -- absent for
+// a mini-batch whose seeds repeat --, source ids, edge ids if the matrix carries
+// any, number of source nodes, number of destination nodes).
+using BlockViews = std::tuple<torch::Tensor, torch::Tensor, c10::optional<torch::Tensor>,
+                              torch::Tensor, c10::optional<torch::Tensor>, int64_t, int64_t>;
+
+// All blocks of one layer of a super-batched sampler (see blocks.cc).  The
+// tensors are the layer's concatenated arrays; a block is a set of views.  The
+// per-batch offsets reach the host on first use (they are already on their way
+// when the object is handed out).
+class BlockBatch : public torch::CustomClassHolder {
+ public:
+  torch::Tensor frontier, frontier_ptr, row, col, coo_ptr, col_bptr, col_seeds, indptr;
+  c10::optional<torch::Tensor> e_ids;
+  int64_t num_batches = 0, num_dst_total = 0;
+
+  int64_t Size() { return num_batches; }
+  // (source nodes, destination nodes, edges) over all blocks; no device read
+  std::vector<int64_t> Totals();
+  // host copies of (frontier_ptr, col_bptr, coo_ptr)
+  std::tuple<std::vector<int64_t>, std::vector<int64_t>, std::vector<int64_t>> Offsets();
+  BlockViews Block(int64_t b);
+  std::vector<BlockViews> Blocks();
+  int64_t NumSrcOf(int64_t b);
+  torch::Tensor Frontier() { return frontier; }
+  torch::Tensor FrontierPtr() { return frontier_ptr; }
+  torch::Tensor Row() { return row; }
+  torch::Tensor Col() { return col; }
+  torch::Tensor Indptr() { return indptr; }
+  torch::Tensor EdgePtr() { return coo_ptr; }
+  torch::Tensor ColPtr() { return col_bptr; }
+  c10::optional<torch::Tensor> EdgeIds() { return e_ids; }
+
+ private:
+  void fetch();
+  bool have_host_ = false;
+  std::vector<int64_t> f_off_, e_off_, c_off_;
+  std::vector<uint8_t> grouped_;  // per batch: edges grouped by destination in offset order
+};
+
 class Graph;
 using GraphPtr = c10::intrusive_ptr<Graph>;
 using GraphAndIndex = std::tuple<GraphPtr, torch::Tensor>;
@@ -173,6 +213,9 @@ class Graph : public torch::CustomClassHolder {
   BatchGraphRelabel(torch::Tensor col_seeds, torch::Tensor row_ids);
   std::tuple<torch::Tensor, torch::Tensor> BatchGetValidNodes(
       torch::Tensor col_seeds, torch::Tensor row_ids);
+  // Not in the reference: relabel + all mini-batch blocks of the layer (edge
+  // list and compressed form) in one call; see blocks.cc.
+  c10::intrusive_ptr<BlockBatch> BatchBlocks(torch::Tensor col_seeds, torch::Tensor row_ids);
 
  private:
   // Unique/relabel state shared by all_nodes() and to_dgl_block(): the

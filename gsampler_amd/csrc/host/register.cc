@@ -28,9 +28,25 @@ static int64_t abi_version() { return gs_abi_version(); }
 
 }  // namespace gs
 
+using gs::BlockBatch;
 using gs::Graph;
 
 TORCH_LIBRARY(gs_classes, m) {
+  m.class_<BlockBatch>("BlockBatch")
+      .def("size", &BlockBatch::Size)
+      .def("totals", &BlockBatch::Totals)
+      .def("offsets", &BlockBatch::Offsets)
+      .def("block", &BlockBatch::Block)
+      .def("blocks", &BlockBatch::Blocks)
+      .def("num_src_of", &BlockBatch::NumSrcOf)
+      .def("frontier", &BlockBatch::Frontier)
+      .def("frontier_ptr", &BlockBatch::FrontierPtr)
+      .def("row", &BlockBatch::Row)
+      .def("col", &BlockBatch::Col)
+      .def("indptr", &BlockBatch::Indptr)
+      .def("edge_ptr", &BlockBatch::EdgePtr)
+      .def("col_ptr", &BlockBatch::ColPtr)
+      .def("edge_ids", &BlockBatch::EdgeIds);
   m.class_<Graph>("Graph")
       .def(torch::init<int64_t, int64_t>())
       .def("_CAPI_LoadCSC", &Graph::LoadCSC)
@@ -89,7 +105,8 @@ TORCH_LIBRARY(gs_classes, m) {
       .def("_CAPI_BatchGetCOOCols", &Graph::BatchGetCOOCols)
       .def("_CAPI_BatchGetCOOEids", &Graph::BatchGetCOOEids)
       .def("_CAPI_BatchGetColCounts", &Graph::BatchGetColCounts)
-      .def("_CAPI_BatchGetValidNodes", &Graph::BatchGetValidNodes);
+      .def("_CAPI_BatchGetValidNodes", &Graph::BatchGetValidNodes)
+      .def("_CAPI_BatchBlocks", &Graph::BatchBlocks);
 }
 
 TORCH_LIBRARY(gs_ops, m) {

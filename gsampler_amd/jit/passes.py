@@ -5,7 +5,9 @@ hoisting of tensor constants.  Operator rewrites (observable in
 `compiled.gm.graph`, same set as the reference's python/gs/jit/optimize.py):
 
   merge_relabel_and_all_nodes   _CAPI_GetValidNodes + _CAPI_GraphRelabel on one
-                                matrix            -> one _CAPI_GraphRelabel
+                                matrix            -> one _CAPI_GraphRelabel;
+                                _CAPI_BatchGetValidNodes + _CAPI_BatchBlocks
+                                                  -> the block batch's frontier
   fuse_slicing_and_sampling     _CAPI_Slicing -> _CAPI_Sampling on one axis
                                                   -> _CAPI_SlicingSampling
   batch_fuse_slicing_and_sampling  _CAPI_BatchColSlicing(encoding=False) ->
@@ -126,7 +128,39 @@ def merge_relabel_and_all_nodes(gm: fx.GraphModule) -> fx.GraphModule:
         for v in valid:
             if v.args[1:] == keep.args[1:]:
                 v.replace_all_uses_with(frontier)
-    return dce(gm)
+    return dce(_merge_batch_blocks_and_all_nodes(gm))
+
+
+def _merge_batch_blocks_and_all_nodes(gm: fx.GraphModule) -> fx.GraphModule:
+    """The super-batched twin: all_nodes() reads the frontier and its batch
+    pointer off the layer's block batch, which is built first.  The relabel is
+    then queued before the host waits for the size of the frontier, so the
+    device has work while that number travels."""
+    by_graph: Dict[fx.Node, List[fx.Node]] = {}
+    for node in gm.graph.nodes:
+        if _is_method(node, "_CAPI_BatchGetValidNodes") or _is_method(node, "_CAPI_BatchBlocks"):
+            by_graph.setdefault(node.args[0], []).append(node)
+    order = {n: i for i, n in enumerate(gm.graph.nodes)}
+    for group in by_graph.values():
+        builders = [n for n in group if n.target == "_CAPI_BatchBlocks"]
+        valid = [n for n in group if n.target == "_CAPI_BatchGetValidNodes"]
+        if not builders or not valid:
+            continue
+        keep = builders[0]
+        first = min(group, key=lambda n: order[n])
+        if first is not keep:
+            first.prepend(keep)
+        with gm.graph.inserting_after(keep):
+            ptr = gm.graph.call_method("frontier_ptr", args=(keep,))
+            frontier = gm.graph.call_method("frontier", args=(keep,))
+        for v in valid:
+            if v.args[1:] != keep.args[1:]:
+                continue
+            for user in list(v.users):
+                if (user.op == "call_function" and user.target is operator.getitem
+                        and user.args[1] in (0, 1)):
+                    user.replace_all_uses_with(frontier if user.args[1] == 0 else ptr)
+    return gm
 
 
 def fuse_slicing_and_sampling(gm: fx.GraphModule) -> fx.GraphModule:
@@ -413,7 +447,7 @@ def sink_block_construction(gm: fx.GraphModule) -> fx.GraphModule:
     splits, a blocking read of the offsets).  Done where the sampler wrote it,
     it holds back the launches of the next layer; nothing on the device depends
     on it, so it moves to the end of the graph, in its original order."""
-    host_functions = {"batch_gen_block", "create_block_from_coo", "create_block_from_csc",
+    host_functions = {"batch_gen_block", "batch_block_list", "create_block_from_coo", "create_block_from_csc",
                       "assign_block", "_CAPI_BatchSplitByOffset",
                       "_CAPI_BatchIndptrSplitByOffset"}
 

@@ -11,11 +11,17 @@ import torch
 
 from ..format import _COO
 from ..ops import gsddmm, gspmm
-from ..utils.block import Block
+from ..utils.block import Block, BlockList
 from .matrix import Matrix, data_index
 
 torch.fx.wrap("batch_gen_block")
+torch.fx.wrap("batch_block_list")
 torch.fx.wrap("data_index")
+
+
+def batch_block_list(batch, edata: Dict[str, torch.Tensor]) -> BlockList:
+    """The layer's blocks around the operator library's BlockBatch."""
+    return BlockList(batch, edata)
 
 
 def batch_gen_block(frontier_list, coo_row_list, coo_col_list, coo_eids, coo_ptr,
@@ -143,19 +149,18 @@ class BatchMatrix(Matrix):
         return out
 
     # ------------------------------------------------------------ finalize
-    def to_dgl_block(self, prefetch_edata=()) -> List[Block]:
-        (frontiers, frontiers_ptr, coo_row, coo_col, coo_eids,
-         coo_ptr) = self._graph._CAPI_BatchGraphRelabel(
+    def to_dgl_block(self, prefetch_edata=()) -> BlockList:
+        """One block per mini-batch.  The reference relabels, splits three arrays
+        per batch and builds the blocks in a Python loop
+        (python/gs/matrix_api/batch_matrix.py:232-248, batch_gen_block above);
+        here one operator call relabels the super-batch and lays out every
+        block's edge list and compressed form, and the returned sequence makes a
+        Block object when it is asked for."""
+        batch = self._graph._CAPI_BatchBlocks(
             self.col_ndata.get("_ID", self.null_tensor),
             self.row_ndata.get("_ID", self.null_tensor))
-        split = torch.ops.gs_ops._CAPI_BatchSplitByOffset
-        frontier_list = split(frontiers, frontiers_ptr)
-        coo_row_list = split(coo_row, coo_ptr)
-        coo_col_list = split(coo_col, coo_ptr)
-        col_counts = self._graph._CAPI_BatchGetColCounts()
         edata = {key: self.edata[key] for key in prefetch_edata}
-        return batch_gen_block(frontier_list, coo_row_list, coo_col_list, coo_eids, coo_ptr,
-                               edata, col_counts)
+        return batch_block_list(batch, edata)
 
     def all_nodes(self):
         return self._graph._CAPI_BatchGetValidNodes(

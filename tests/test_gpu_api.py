@@ -313,3 +313,66 @@ def test_batch_pointer_is_bound_to_the_length_it_was_checked_for(graph):
     sub2, _ = g._CAPI_BatchFusedSlicingSampling(uniq, uptr, 5, False)
     with pytest.raises(RuntimeError, match="batch offsets"):
         g._CAPI_BatchFusedSlicingSampling(uniq[:-1], uptr, 5, False)
+
+
+def test_block_batch_emits_edge_list_and_compressed_form(graph):
+    """to_dgl_block of a super-batch: one operator call lays out every block; the
+    compressed form by destination of each block equals SciPy's conversion of the
+    block's edge list, the blocks equal the per-batch split of the relabelled
+    super-batch, and per-edge data travels with the edges."""
+    import scipy.sparse as sp
+    m, indptr, indices = graph
+    seeds, ptr = batched_seeds(20000, 6, 100, seed=9)
+    seeds[150:200] = seeds[100:150]                 # repeated seeds inside batch 1
+    ptr = torch.tensor([0, 100, 250, 250, 400, 401, 600])      # an empty batch, a batch of one
+    w = torch.rand(indices.size, device=DEV)
+    m2 = gs.Matrix(m._graph, {}, {}, {"w": w})
+    bm = gs.BatchMatrix()
+    bm.load_from_matrix(m2, False)
+    gs.manual_seed(3)
+    sub = bm[:, seeds.to(DEV)::ptr.to(DEV)].individual_sampling(7, None, False)
+    blocks = sub.to_dgl_block(prefetch_edata={"w"})
+    frontier, fptr, row, col, eids, eptr = sub._graph._CAPI_BatchGraphRelabel(
+        seeds.to(DEV), torch.empty(0, dtype=torch.int64))
+    assert len(blocks) == 6 and blocks.totals() == (frontier.numel(), 600, row.numel())
+    fptr, eptr = fptr.tolist(), eptr.tolist()
+    whole_w = sub.edata["w"]
+    listed = list(blocks)
+    assert listed[2].num_edges() == 0 and listed[2].num_dst == 0 and listed[2].num_src == 0
+    assert blocks[-1] is listed[5] and blocks[1:3] == listed[1:3]
+    for b, blk in enumerate(listed):
+        lo, hi = eptr[b], eptr[b + 1]
+        assert torch.equal(blk.row, row[lo:hi]) and torch.equal(blk.col, col[lo:hi])
+        assert torch.equal(blk.srcdata["_ID"], frontier[fptr[b]:fptr[b + 1]])
+        assert torch.equal(blk.edata["w"], whole_w[lo:hi])
+        assert blk.num_dst == int(ptr[b + 1] - ptr[b]) and blk.num_src == fptr[b + 1] - fptr[b]
+        b_indptr, b_indices, _ = blk.csc()
+        assert b_indptr.numel() == blk.num_dst + 1 and int(b_indptr[0]) == 0
+        ones = np.ones(blk.num_edges())
+        from_coo = sp.coo_matrix((ones, (blk.row.cpu().numpy(), blk.col.cpu().numpy())),
+                                 shape=(max(blk.num_src, 1), max(blk.num_dst, 1))).tocsc()
+        direct = sp.csc_matrix((ones, b_indices.cpu().numpy(),
+                                np.concatenate([b_indptr.cpu().numpy(),
+                                                [] if blk.num_dst else [0]]).astype(np.int64)),
+                               shape=(max(blk.num_src, 1), max(blk.num_dst, 1)))
+        assert (from_coo != direct).nnz == 0        # parallel edges add up on both sides
+        # and entry by entry: offsets are the running count of edges per destination,
+        # the indices are the edges' sources in their (destination-grouped) order
+        counts = np.bincount(blk.col.cpu().numpy(), minlength=blk.num_dst)
+        assert np.array_equal(b_indptr.cpu().numpy(), np.concatenate([[0], np.cumsum(counts)]))
+        if b == 1:
+            # repeated seeds share the label of their first occurrence: the offsets
+            # by seed position do not describe this block, so none are handed out
+            # and the compressed form is derived from the edge list
+            assert blk.indptr is None and counts[100:150].sum() == 0
+        else:
+            assert blk.indptr is not None and torch.equal(b_indices, blk.row)
+            assert bool((blk.col[1:] >= blk.col[:-1]).all())
+    # a block asked for on its own, before anything else was materialised
+    again = sub.to_dgl_block()
+    one = again[3]
+    assert torch.equal(one.row, listed[3].row) and "w" not in one.edata
+    # a block built from an edge list alone derives its compressed form
+    loose = gs.utils.block.Block(listed[0].row, listed[0].col, listed[0].num_src, listed[0].num_dst)
+    li, lx, _ = loose.csc()
+    assert torch.equal(li, listed[0].csc()[0]) and torch.equal(lx, listed[0].csc()[1])
