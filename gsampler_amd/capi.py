@@ -41,6 +41,7 @@ SIGNATURES = {
     "gs_profile_count": (_int, []),
     "gs_profile_get": (_int, [_int, C.c_char_p, _sz, C.POINTER(C.c_longlong),
                               C.POINTER(C.c_double)]),
+    "gs_copy_i64": (_int, [_p, _i64, _p, _p]),
     "gs_scan_workspace_bytes": (_sz, [_i64]),
     "gs_exclusive_scan_i64": (_int, [_p, _p, _i64, _p, _sz, _p]),
     "gs_csc_col_count": (_int, [_p, _i64, _p, _i64, _i64, _int, _p, _p, _sz, _p]),
@@ -59,6 +60,7 @@ SIGNATURES = {
     "gs_sorted_to_indptr": (_int, [_p, _i64, _i64, _p, _p]),
     "gs_decode_batch_ids": (_int, [_p, _i64, _i64, _p, _p, _p]),
     "gs_split_indptr": (_int, [_p, _p, _i64, _i64, _p, _p]),
+    "gs_batch_seeds_distinct": (_int, [_p, _p, _p, _p, _i64, _p, _p]),
     "gs_first_position": (_int, [_p, _i64, _i64, _p, _p]),
     "gs_gather_rows": (_int, [_p, _i64, _i64, _p, _i64, _p, _p, _p]),
     "gs_coo_sort_workspace_bytes": (_sz, [_i64, _i64]),
@@ -160,7 +162,9 @@ class _Count:
             cls._slots = torch.empty(64, dtype=torch.int64).pin_memory()
         self._slot = cls._slots[cls._next % 64: cls._next % 64 + 1]
         cls._next += 1
-        self._slot.copy_(prefix[-1:], non_blocking=True)
+        # a one-element copy kernel into the pinned word, in stream order
+        check(lib().gs_copy_i64(prefix.data_ptr() + 8 * (prefix.numel() - 1), 1,
+                                self._slot.data_ptr(), _stream()))
         self._event = torch.cuda.Event()
         self._event.record()
         self._ticket = cls._next

@@ -209,9 +209,28 @@ int exclusive_scan_i64(const int64_t* in, int64_t* out, int64_t n, void* ws,
   return GS_OK;
 }
 
+// n values from one array to another; the destination may be pinned host memory.
+__global__ __launch_bounds__(kBlock) void copy_i64_kernel(const int64_t* __restrict__ src,
+                                                          int64_t n, int64_t* __restrict__ dst) {
+  const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (i < n) dst[i] = src[i];
+}
+
 }  // namespace gs
 
 extern "C" {
+
+int gs_copy_i64(const int64_t* src, int64_t n, int64_t* dst, gs_stream_t stream) {
+  using namespace gs;
+  GS_REQUIRE(n >= 0, "copy_i64: negative length %lld", (long long)n);
+  if (n == 0) return GS_OK;
+  GS_REQUIRE(src && dst, "copy_i64: null pointer");
+  hipStream_t s = as_stream(stream);
+  GS_LAUNCH("copy_i64", s,
+            copy_i64_kernel<<<dim3((unsigned)ceil_div(n, kBlock)), dim3(kBlock), 0, s>>>(src, n,
+                                                                                          dst));
+  return GS_OK;
+}
 
 const char* gs_last_error(void) { return gs::g_last_error.c_str(); }
 

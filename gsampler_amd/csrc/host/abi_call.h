@@ -94,8 +94,7 @@ class AsyncCount {
     slot_ = (int)(ticket_ % kSlots);
     hipStream_t s = (hipStream_t)cur_stream();
     const int64_t* src = prefix.data_ptr<int64_t>() + prefix.numel() - 1;
-    check(hipMemcpyAsync(r.words + slot_, src, sizeof(int64_t),
-                         hipMemcpyDeviceToHost, s));
+    GS_CALL(gs_copy_i64(src, 1, r.words + slot_, (gs_stream_t)s));
     check(hipEventRecord(r.events[slot_], s));
     pending_ = true;
   }
@@ -206,12 +205,54 @@ class OffsetMirror {
     torch::Tensor c = offsets.contiguous();
     hipStream_t s = (hipStream_t)cur_stream();
     if (e.count > 0)
-      check(hipMemcpyAsync(e.pinned, c.data_ptr<int64_t>(), e.count * sizeof(int64_t),
-                           hipMemcpyDeviceToHost, s));
+      GS_CALL(gs_copy_i64(c.data_ptr<int64_t>(), (int64_t)e.count, e.pinned, (gs_stream_t)s));
     check(hipEventRecord(e.event, s));
     e.pending = true;
     return e;
   }
+};
+
+// The number of edges a sampling operator produced.  A plain operator copies the
+// last entry of its prefix array to the host (AsyncCount).  A super-batched
+// operator needs the per-batch edge pointer prefix[col_bptr] on the host anyway
+// (its last entry is the same total), so it announces col_bptr through hint()
+// before the call: the sampler then gathers the edge pointer at once, sends that
+// one array to the host and leaves it in the hint.  One copy instead of two;
+// a copy to the host costs the device about as much as a small kernel.
+class EdgeCount {
+ public:
+  struct Hint {
+    torch::Tensor col_bptr;   // set by the caller
+    torch::Tensor edge_bptr;  // left by the sampler
+  };
+  static Hint& hint() {
+    static thread_local Hint h;
+    return h;
+  }
+  struct HintScope {
+    explicit HintScope(const torch::Tensor& col_bptr) {
+      hint().col_bptr = col_bptr;
+      hint().edge_bptr = torch::Tensor();
+    }
+    ~HintScope() { hint() = Hint(); }
+  };
+  explicit EdgeCount(const torch::Tensor& prefix) {
+    Hint& h = hint();
+    if (h.col_bptr.defined()) {
+      edge_bptr_ = prefix.index_select(0, h.col_bptr);
+      OffsetMirror::prefetch(edge_bptr_);
+      h.edge_bptr = edge_bptr_;
+    } else {
+      count_ = AsyncCount(prefix);
+    }
+  }
+  int64_t get() {
+    return edge_bptr_.defined() ? OffsetMirror::values(edge_bptr_).back() : count_.get();
+  }
+
+ private:
+  torch::Tensor edge_bptr_;
+  AsyncCount count_;
 };
 
 // Batch pointer arrays (int64[B + 1] offsets into a concatenation) reach the

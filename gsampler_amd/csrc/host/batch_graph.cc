@@ -142,13 +142,14 @@ GraphAndIndex Graph::BatchFusedSlicingSampling(torch::Tensor seeds,
                                                int64_t fanout, bool replace) {
   col_bptr = ids(col_bptr, "col_bptr");
   BatchOffsets::check(col_bptr, seeds.numel(), "BatchFusedSlicingSampling");
+  EdgeCount::HintScope batch(col_bptr);  // the sampler leaves the edge pointer here
   auto ret = FusedSlicingSampling(1, seeds, fanout, replace, kCSC, kCSC | kCOO);
   Graph& g = *std::get<0>(ret);
   g.col_bptr_ = col_bptr;
   g.orig_col_ids_ = ids(seeds, "seeds");
-  g.edge_bptr_ = g.csc_->indptr.index_select(0, col_bptr);
-  BatchOffsets::trust(g.edge_bptr_);
-  OffsetMirror::prefetch(g.edge_bptr_);  // per-batch splits will ask for it
+  g.edge_bptr_ = EdgeCount::hint().edge_bptr;
+  if (!g.edge_bptr_.defined()) g.edge_bptr_ = g.csc_->indptr.index_select(0, col_bptr);
+  BatchOffsets::trust(g.edge_bptr_, g.num_edges_);
   return ret;
 }
 
@@ -170,9 +171,12 @@ torch::Tensor Graph::batch_rows_for_relabel(const torch::Tensor& row_ids) {
   return mapped_out_;
 }
 
-std::tuple<torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor,
-           c10::optional<torch::Tensor>, torch::Tensor>
-Graph::BatchGraphRelabel(torch::Tensor col_seeds, torch::Tensor row_ids) {
+// Queues unique (count + fill) and relabel for the super-batch; nothing here
+// waits for the device.  The frontier's size is still on its way when this
+// returns: f.frontier() waits for it.
+Graph::Frontier& Graph::batch_relabel_launch(torch::Tensor& col_seeds,
+                                             const torch::Tensor& row_ids,
+                                             torch::Tensor* out_row, torch::Tensor* out_col) {
   TORCH_CHECK(edge_bptr_.defined() && edge_bptr_.numel() > 0,
               "BatchGraphRelabel: the graph has no edge batch pointer");
   CreateSparseFormat(kCOO);
@@ -185,12 +189,21 @@ Graph::BatchGraphRelabel(torch::Tensor col_seeds, torch::Tensor row_ids) {
   torch::Tensor rows = batch_rows_for_relabel(row_ids);
   Frontier& f = frontier_for(col_seeds, rows, col_bptr_, edge_bptr_);
   const int64_t E = rows.numel(), B = f.num_batches;
-  torch::Tensor out_row = new_ids(E, rows), out_col = new_ids(E, rows);
+  *out_row = new_ids(E, rows);
+  *out_col = new_ids(E, rows);
   GS_CALL(gs_unique_relabel(cptr(col_seeds), cptr(col_bptr_), col_seeds.numel(),
                             cptr(rows), cptr(edge_bptr_), E, B, cptr(coo_->col),
-                            mptr(out_row), mptr(out_col),
+                            mptr(*out_row), mptr(*out_col),
                             f.workspace.data_ptr(), f.workspace.numel(),
                             cur_stream()));
+  return f;
+}
+
+std::tuple<torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor,
+           c10::optional<torch::Tensor>, torch::Tensor>
+Graph::BatchGraphRelabel(torch::Tensor col_seeds, torch::Tensor row_ids) {
+  torch::Tensor out_row, out_col;
+  Frontier& f = batch_relabel_launch(col_seeds, row_ids, &out_row, &out_col);
   return {f.frontier(), f.unique_ptr, out_row, out_col, coo_->e_ids, edge_bptr_};
 }
 

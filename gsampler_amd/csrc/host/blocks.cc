@@ -22,6 +22,18 @@ int64_t BlockBatch::NumSrcOf(int64_t b) {
 
 void BlockBatch::fetch() {
   if (have_host_) return;
+  // Offsets by destination of every block: the columns of the sampled matrix
+  // are the destinations, so its indptr, cut at the batch boundaries and
+  // rebased, is the blocks' indptr (the relabelled edges keep their order).
+  // Two small launches, made when the first block is asked for rather than in
+  // the sampler's launch sequence.
+  const int64_t total = sampled_indptr.numel() - 1 + num_batches;
+  indptr = new_ids(total, sampled_indptr);
+  GS_CALL(gs_split_indptr(cptr(sampled_indptr), cptr(col_bptr), num_batches, total, mptr(indptr),
+                          cur_stream()));
+  distinct = new_ids(num_batches, sampled_indptr);
+  GS_CALL(gs_batch_seeds_distinct(cptr(frontier), cptr(frontier_ptr), cptr(col_seeds),
+                                  cptr(col_bptr), num_batches, mptr(distinct), cur_stream()));
   f_off_ = OffsetMirror::values(frontier_ptr);
   e_off_ = OffsetMirror::values(coo_ptr);
   c_off_ = OffsetMirror::values(col_bptr);
@@ -29,25 +41,11 @@ void BlockBatch::fetch() {
   // a mini-batch are distinct the label of a seed is its position, and the
   // block's edges are grouped by destination in the order of the offsets; a
   // repeated seed shares the label of its first occurrence, and the offsets by
-  // position no longer describe the block.  A batch's seeds are distinct exactly
-  // when its last seed sits at the place ns - 1 of the batch's frontier: one
-  // small gather per layer, on first use.
+  // position no longer describe the block.
   grouped_.assign((size_t)num_batches, 1);
-  if (num_batches > 0 && col_seeds.numel() > 0) {
-    torch::Tensor ns = col_bptr.narrow(0, 1, num_batches) - col_bptr.narrow(0, 0, num_batches);
-    torch::Tensor nu =
-        frontier_ptr.narrow(0, 1, num_batches) - frontier_ptr.narrow(0, 0, num_batches);
-    torch::Tensor has = (ns > 0) & (nu >= ns);
-    torch::Tensor at_f = (frontier_ptr.narrow(0, 0, num_batches) + ns - 1)
-                             .clamp(0, std::max<int64_t>(frontier.numel() - 1, 0));
-    torch::Tensor at_s =
-        (col_bptr.narrow(0, 1, num_batches) - 1).clamp(0, col_seeds.numel() - 1);
-    torch::Tensor ok = (ns == 0);
-    if (frontier.numel() > 0)
-      ok = ok | (has & (frontier.index_select(0, at_f) == col_seeds.index_select(0, at_s)));
-    torch::Tensor host = ok.to(torch::kCPU).to(torch::kUInt8).contiguous();
-    for (int64_t b = 0; b < num_batches; ++b)
-      grouped_[(size_t)b] = host.data_ptr<uint8_t>()[b];
+  if (distinct.defined()) {
+    const std::vector<int64_t>& d = OffsetMirror::values(distinct);
+    for (int64_t b = 0; b < num_batches; ++b) grouped_[(size_t)b] = d[(size_t)b] != 0;
   }
   have_host_ = true;
 }
@@ -78,44 +76,61 @@ BlockViews BlockBatch::Block(int64_t b) {
           nf, nc};
 }
 
-std::vector<BlockViews> BlockBatch::Blocks() {
-  std::vector<BlockViews> out;
-  out.reserve((size_t)num_batches);
-  for (int64_t b = 0; b < num_batches; ++b) out.push_back(Block(b));
-  return out;
+// All blocks at once, one list per field (the per-batch splits are made by
+// torch's split, which is far cheaper than a view at a time).
+BlockParts BlockBatch::Blocks() {
+  fetch();
+  auto sizes = [](const std::vector<int64_t>& off) {
+    std::vector<int64_t> s(off.size() - 1);
+    for (size_t i = 0; i + 1 < off.size(); ++i) s[i] = off[i + 1] - off[i];
+    return s;
+  };
+  const std::vector<int64_t> ne = sizes(e_off_), nf = sizes(f_off_), nc = sizes(c_off_);
+  std::vector<torch::Tensor> rows = torch::split_with_sizes(row, ne);
+  std::vector<torch::Tensor> cols = torch::split_with_sizes(col, ne);
+  std::vector<torch::Tensor> fronts = torch::split_with_sizes(frontier, nf);
+  std::vector<c10::optional<torch::Tensor>> eids((size_t)num_batches), offs((size_t)num_batches);
+  if (e_ids.has_value()) {
+    std::vector<torch::Tensor> parts = torch::split_with_sizes(e_ids.value(), ne);
+    for (size_t i = 0; i < parts.size(); ++i) eids[i] = parts[i];
+  }
+  std::vector<int64_t> with_end(nc);
+  for (int64_t& n : with_end) n += 1;  // a block's offsets have one entry more than it has columns
+  std::vector<torch::Tensor> pieces = torch::split_with_sizes(indptr, with_end);
+  for (size_t i = 0; i < pieces.size(); ++i)
+    if (grouped_[i]) offs[i] = pieces[i];
+  return {rows, cols, offs, fronts, eids, nf, nc};
 }
 
+// Everything is queued before the host waits for the size of the frontier (the
+// last statement): the device works through the relabel while that number
+// travels, and the caller's next launches follow at once.
 c10::intrusive_ptr<BlockBatch> Graph::BatchBlocks(torch::Tensor col_seeds,
                                                   torch::Tensor row_ids) {
-  auto rel = BatchGraphRelabel(col_seeds, row_ids);  // queues count, fill and relabel
+  TORCH_CHECK(col_bptr_.defined() && col_bptr_.numel() >= 2,
+              "BatchBlocks: the graph has no column batch pointer");
   auto out = c10::make_intrusive<BlockBatch>();
-  out->frontier = std::get<0>(rel);
-  out->frontier_ptr = std::get<1>(rel);
-  out->row = std::get<2>(rel);
-  out->col = std::get<3>(rel);
-  out->e_ids = std::get<4>(rel);
-  out->coo_ptr = std::get<5>(rel);
-  out->col_bptr = col_bptr_;
-  out->col_seeds = ids(col_seeds, "col_seeds");
   out->num_batches = col_bptr_.numel() - 1;
-  out->num_dst_total = col_seeds.numel();
-  // Offsets by destination of every block: the columns of the sampled matrix
-  // are the destinations, so its indptr, cut at the batch boundaries and
-  // rebased, is the blocks' indptr (the relabelled edges keep their order).
-  torch::Tensor indptr;
+  CreateSparseFormat(kCOO);
   if (csc_) {
-    indptr = csc_->indptr;
+    out->sampled_indptr = csc_->indptr;
   } else {
-    indptr = new_ids(num_cols_ + 1, coo_->col);  // the edge list is column-sorted
-    GS_CALL(gs_sorted_to_indptr(cptr(coo_->col), coo_->col.numel(), num_cols_, mptr(indptr),
-                                cur_stream()));
+    TORCH_CHECK(coo_->col_sorted, "BatchBlocks: the COO format must be column-sorted");
+    out->sampled_indptr = new_ids(num_cols_ + 1, coo_->col);
+    GS_CALL(gs_sorted_to_indptr(cptr(coo_->col), coo_->col.numel(), num_cols_,
+                                mptr(out->sampled_indptr), cur_stream()));
   }
-  const int64_t total = num_cols_ + out->num_batches;
-  out->indptr = new_ids(total, indptr);
-  GS_CALL(gs_split_indptr(cptr(indptr), cptr(col_bptr_), out->num_batches, total,
-                          mptr(out->indptr), cur_stream()));
-  OffsetMirror::prefetch(col_bptr_);
-  OffsetMirror::prefetch(out->coo_ptr);
+  Frontier& f = batch_relabel_launch(col_seeds, row_ids, &out->row, &out->col);
+  out->col_seeds = col_seeds;
+  out->num_dst_total = col_seeds.numel();
+  out->frontier_ptr = f.unique_ptr;
+  out->e_ids = coo_->e_ids;
+  out->coo_ptr = edge_bptr_;
+  out->col_bptr = col_bptr_;
+  // (the pointer arrays are on their way to the host or there already: the
+  // sampler sent the edge pointer, the unique pass the frontier pointer, and the
+  // column pointer is the caller's or the previous layer's frontier pointer)
+  out->frontier = f.frontier();  // waits for the number of unique ids
   return out;
 }
 

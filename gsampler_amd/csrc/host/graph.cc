@@ -214,7 +214,7 @@ MajorResult major_sample_uniform(const Compressed& m,
                            ws.numel(), cur_stream()));
   // No column yields more than fanout edges: size the outputs by that bound,
   // launch, and trim when the count has arrived.
-  AsyncCount count(r.indptr);
+  EdgeCount count(r.indptr);
   const int64_t bound = n * fanout;
   const int64_t size = bound <= kBoundLimit ? bound : count.get();
   r.minor_ids = new_ids(size, m.indptr);
@@ -385,12 +385,13 @@ Graph::Frontier& Graph::frontier_for(const torch::Tensor& seeds,
                           cptr(rows_ptr), E, B, mptr(f->unique_ptr),
                           f->workspace.data_ptr(), f->workspace.numel(),
                           cur_stream()));
-  f->count = AsyncCount(f->unique_ptr);
+  // The whole pointer array goes to the host in one copy: its last entry is the
+  // size of the frontier, the rest is what per-batch splits ask for later.
+  OffsetMirror::prefetch(f->unique_ptr);
   BatchOffsets::trust(f->unique_ptr);
-  if (B > 1) OffsetMirror::prefetch(f->unique_ptr);  // per-batch splits will ask for it
   // at most S + E unique keys
   f->unique_buffer =
-      new_ids(S + E <= kBoundLimit ? S + E : f->count.get(), rows);
+      new_ids(S + E <= kBoundLimit ? S + E : f->total(), rows);
   GS_CALL(gs_unique_fill(cptr(seeds), cptr(seeds_ptr), S, cptr(rows),
                          cptr(rows_ptr), E, B, cptr(f->unique_ptr),
                          mptr(f->unique_buffer), f->workspace.data_ptr(),

@@ -58,13 +58,22 @@ RandomState& random_state();
 using BlockViews = std::tuple<torch::Tensor, torch::Tensor, c10::optional<torch::Tensor>,
                               torch::Tensor, c10::optional<torch::Tensor>, int64_t, int64_t>;
 
+// The same for every block of a layer, one list per field.
+using BlockParts =
+    std::tuple<std::vector<torch::Tensor>, std::vector<torch::Tensor>,
+               std::vector<c10::optional<torch::Tensor>>, std::vector<torch::Tensor>,
+               std::vector<c10::optional<torch::Tensor>>, std::vector<int64_t>,
+               std::vector<int64_t>>;
+
 // All blocks of one layer of a super-batched sampler (see blocks.cc).  The
 // tensors are the layer's concatenated arrays; a block is a set of views.  The
 // per-batch offsets reach the host on first use (they are already on their way
 // when the object is handed out).
 class BlockBatch : public torch::CustomClassHolder {
  public:
-  torch::Tensor frontier, frontier_ptr, row, col, coo_ptr, col_bptr, col_seeds, indptr;
+  torch::Tensor frontier, frontier_ptr, row, col, coo_ptr, col_bptr, col_seeds;
+  torch::Tensor sampled_indptr;    // offsets of the sampled matrix over all its columns
+  torch::Tensor indptr, distinct;  // per-block offsets and per-batch flags, made on first use
   c10::optional<torch::Tensor> e_ids;
   int64_t num_batches = 0, num_dst_total = 0;
 
@@ -74,13 +83,16 @@ class BlockBatch : public torch::CustomClassHolder {
   // host copies of (frontier_ptr, col_bptr, coo_ptr)
   std::tuple<std::vector<int64_t>, std::vector<int64_t>, std::vector<int64_t>> Offsets();
   BlockViews Block(int64_t b);
-  std::vector<BlockViews> Blocks();
+  BlockParts Blocks();
   int64_t NumSrcOf(int64_t b);
   torch::Tensor Frontier() { return frontier; }
   torch::Tensor FrontierPtr() { return frontier_ptr; }
   torch::Tensor Row() { return row; }
   torch::Tensor Col() { return col; }
-  torch::Tensor Indptr() { return indptr; }
+  torch::Tensor Indptr() {
+    fetch();
+    return indptr;
+  }
   torch::Tensor EdgePtr() { return coo_ptr; }
   torch::Tensor ColPtr() { return col_bptr; }
   c10::optional<torch::Tensor> EdgeIds() { return e_ids; }
@@ -228,12 +240,9 @@ class Graph : public torch::CustomClassHolder {
     // The unique keys: filled into a buffer sized by the upper bound, trimmed
     // once the count has arrived (frontier() waits for it).
     torch::Tensor unique_buffer;
-    AsyncCount count;
+    int64_t total() { return OffsetMirror::values(unique_ptr).back(); }
     const torch::Tensor& frontier() {
-      if (!unique_.defined()) {
-        const int64_t total = count.get();
-        unique_ = unique_buffer.narrow(0, 0, total);
-      }
+      if (!unique_.defined()) unique_ = unique_buffer.narrow(0, 0, total());
       return unique_;
     }
     bool matches(const torch::Tensor& s, const torch::Tensor& r,
@@ -245,6 +254,8 @@ class Graph : public torch::CustomClassHolder {
   Frontier& frontier_for(const torch::Tensor& seeds, const torch::Tensor& rows,
                          const torch::Tensor& seeds_ptr,
                          const torch::Tensor& rows_ptr);
+  Frontier& batch_relabel_launch(torch::Tensor& col_seeds, const torch::Tensor& row_ids,
+                                 torch::Tensor* out_row, torch::Tensor* out_col);
 
   const Compressed& compressed(int64_t format);
   // CDF of edge_probs in the edge order of `format` (cached per weights tensor).

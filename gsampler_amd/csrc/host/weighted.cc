@@ -103,7 +103,7 @@ GraphAndIndex Graph::FusedSlicingSamplingProbs(int64_t axis, torch::Tensor seeds
   GS_CALL(gs_csc_col_count(cptr(m.indptr), num_major, cptr(seeds), n, fanout,
                            replace ? 1 : 0, mptr(r.indptr), ws.data_ptr(), ws.numel(),
                            cur_stream()));
-  AsyncCount count(r.indptr);
+  EdgeCount count(r.indptr);
   const int64_t bound = n * fanout;
   const int64_t size = bound <= kBoundLimit ? bound : count.get();
   r.minor_ids = new_ids(size, m.indptr);
@@ -131,14 +131,15 @@ GraphAndIndex Graph::BatchFusedSlicingSamplingProbs(torch::Tensor seeds,
                                                     int64_t fanout, bool replace) {
   col_bptr = ids(col_bptr, "col_bptr");
   BatchOffsets::check(col_bptr, seeds.numel(), "BatchFusedSlicingSamplingProbs");
+  EdgeCount::HintScope batch(col_bptr);  // the sampler leaves the edge pointer here
   auto ret = FusedSlicingSamplingProbs(1, seeds, edge_probs, fanout, replace, kCSC,
                                        kCSC | kCOO);
   Graph& g = *std::get<0>(ret);
   g.col_bptr_ = col_bptr;
   g.orig_col_ids_ = ids(seeds, "seeds");
-  g.edge_bptr_ = g.csc_->indptr.index_select(0, col_bptr);
-  BatchOffsets::trust(g.edge_bptr_);
-  OffsetMirror::prefetch(g.edge_bptr_);
+  g.edge_bptr_ = EdgeCount::hint().edge_bptr;
+  if (!g.edge_bptr_.defined()) g.edge_bptr_ = g.csc_->indptr.index_select(0, col_bptr);
+  BatchOffsets::trust(g.edge_bptr_, g.num_edges_);
   return ret;
 }
 

@@ -139,7 +139,7 @@ class BlockList(Sequence):
 
     def materialize(self) -> List[Block]:
         if self._blocks is None or any(b is None for b in self._blocks):
-            views = self._batch.blocks()
+            views = list(zip(*self._batch.blocks()))
             have = self._blocks or [None] * len(views)
             self._blocks = [b if b is not None else self._wrap(i, v)
                             for i, (b, v) in enumerate(zip(have, views))]

@@ -84,6 +84,16 @@ int gs_profile_get(int index, char* name, size_t name_bytes, long long* calls,
                    double* total_ms);
 
 /* ------------------------------------------------------------------------
+ * dst[0..n) = src[0..n).  dst may be pinned host memory that the device can
+ * address: counts and batch pointer arrays that the host needs (to size the next
+ * launch, to split results per batch) are sent this way, by a kernel in stream
+ * order whose completion an event marks, instead of a memcpy call per array
+ * (the reference reads them with blocking copies, e.g.
+ * src/cuda/slicing.cu:146, src/cuda/batch/batch_split.cu:107-119).
+ * ---------------------------------------------------------------------- */
+int gs_copy_i64(const int64_t* src, int64_t n, int64_t* dst, gs_stream_t stream);
+
+/* ------------------------------------------------------------------------
  * Exclusive prefix sum of n int64 values, in place allowed (in == out).
  * Stands in for cub_exclusiveSum, src/cuda/utils.h:18-28.
  * ---------------------------------------------------------------------- */
@@ -427,6 +437,17 @@ int gs_decode_batch_ids(const int64_t* encoded, int64_t n, int64_t stride,
 int gs_split_indptr(const int64_t* indptr, const int64_t* offset,
                     int64_t num_batches, int64_t out_len, int64_t* out,
                     gs_stream_t stream);
+/* out_distinct[b] = 1 when the seeds of batch b are pairwise different, else 0,
+ * read off the batch's frontier (unique keys in first-occurrence order, seeds
+ * first, as gs_unique_fill writes it).  Tells whether the relabelled edges of a
+ * batch are grouped by destination in seed order, i.e. whether the batch's
+ * piece of gs_split_indptr is the block's compressed form.  No counterpart in
+ * the reference, which hands DGL an edge list only
+ * (python/gs/utils/to_dgl_block.py:19-23). */
+int gs_batch_seeds_distinct(const int64_t* frontier, const int64_t* frontier_ptr,
+                            const int64_t* seeds, const int64_t* seeds_ptr,
+                            int64_t num_batches, int64_t* out_distinct,
+                            gs_stream_t stream);
 
 /* ------------------------------------------------------------------------
  * Edge-wise compute operators.  Common arguments: (format, a, b, num_major,

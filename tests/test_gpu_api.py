@@ -360,11 +360,15 @@ def test_block_batch_emits_edge_list_and_compressed_form(graph):
         # the indices are the edges' sources in their (destination-grouped) order
         counts = np.bincount(blk.col.cpu().numpy(), minlength=blk.num_dst)
         assert np.array_equal(b_indptr.cpu().numpy(), np.concatenate([[0], np.cumsum(counts)]))
-        if b == 1:
+        mine = seeds[int(ptr[b]):int(ptr[b + 1])]
+        distinct = torch.unique(mine).numel() == mine.numel()
+        assert (b == 1) <= (not distinct)
+        if not distinct:
             # repeated seeds share the label of their first occurrence: the offsets
             # by seed position do not describe this block, so none are handed out
             # and the compressed form is derived from the edge list
-            assert blk.indptr is None and counts[100:150].sum() == 0
+            assert blk.indptr is None
+            assert counts[torch.unique(mine).numel():].sum() == 0
         else:
             assert blk.indptr is not None and torch.equal(b_indices, blk.row)
             assert bool((blk.col[1:] >= blk.col[:-1]).all())
