@@ -615,8 +615,14 @@ def main():
     yard = torch.bitwise_xor(yard, 1)
     del yard
 
+    # the int32 copy of the row ids that a loaded matrix keeps for the uniform sampler
+    # (the operator class makes the same copy on its first sampling call)
+    pick_ids = indices
+    if probs is None and wl["nodes"] < 2 ** 31 and indices.numel() >= 1 << 20:
+        pick_ids = indices.to(torch.int32)
+
     def step(i):
-        return graphsage_step(capi, indptr, indices, seeds, ptr, fanouts, args.seed,
+        return graphsage_step(capi, indptr, pick_ids, seeds, ptr, fanouts, args.seed,
                               i * len(fanouts), probs, cdf)
 
     if args.path == "api":

@@ -51,6 +51,9 @@ SIGNATURES = {
     "gs_csc_col_sample_uniform_fill": (_int, [_p, _i64, _p, _p, _i64, _i64, _int,
                                               _int, _u64, _u64, _p, _p, _p, _p,
                                               _p]),
+    "gs_csc_col_sample_uniform_fill_i32": (_int, [_p, _i64, _p, _p, _i64, _i64, _int,
+                                                  _int, _u64, _u64, _p, _p, _p, _p,
+                                                  _p]),
     "gs_unique_workspace_bytes": (_sz, [_i64, _i64, _i64]),
     "gs_unique_count": (_int, [_p, _p, _i64, _p, _p, _i64, _i64, _p, _p, _sz, _p]),
     "gs_unique_fill": (_int, [_p, _p, _i64, _p, _p, _i64, _i64, _p, _p, _p, _sz, _p]),
@@ -266,9 +269,16 @@ def sample_uniform(indptr, indices, column_ids, fanout, replace=False,
                    algo=ALGO_AUTO, seed=7777, call_id=0, with_coo=True):
     """Uniform per-column sampling, fused with the slice when column_ids is given.
 
+    `indices` may be the matrix's int32 copy of the row ids (same outputs).
+
     -> (sub_indptr, coo_col | None, sub_indices, select_index)
     """
-    indptr, indices = _i64t(indptr, "indptr"), _i64t(indices, "indices")
+    indptr = _i64t(indptr, "indptr")
+    fill = lib().gs_csc_col_sample_uniform_fill
+    if indices.dtype == torch.int32 and indices.is_cuda:
+        indices, fill = indices.contiguous(), lib().gs_csc_col_sample_uniform_fill_i32
+    else:
+        indices = _i64t(indices, "indices")
     num_cols = indptr.numel() - 1
     if column_ids is not None:
         column_ids = _i64t(column_ids, "column_ids")
@@ -284,7 +294,7 @@ def sample_uniform(indptr, indices, column_ids, fanout, replace=False,
     out_sel = torch.empty(size, dtype=torch.int64, device=dev)
     out_col = torch.empty(size, dtype=torch.int64, device=dev) if with_coo else None
     if size > 0:
-        check(lib().gs_csc_col_sample_uniform_fill(
+        check(fill(
             _ptr(indptr), num_cols, _ptr(indices), _ptr(column_ids), n, fanout,
             int(replace), algo, seed, call_id, sub_indptr.data_ptr(),
             _ptr(out_col), out_idx.data_ptr(), out_sel.data_ptr(), _stream()))

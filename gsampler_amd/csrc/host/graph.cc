@@ -48,6 +48,7 @@ void Graph::LoadCSC(torch::Tensor indptr, torch::Tensor indices) {
   TORCH_CHECK(m->indptr.numel() == num_cols_ + 1, "LoadCSC: indptr has ",
               indptr.numel(), " entries for ", num_cols_, " columns");
   check_compressed(m->indptr, m->indices, num_rows_, "LoadCSC");
+  m->num_minor = num_rows_;
   csc_ = m;
   num_edges_ = indices.numel();
 }
@@ -59,6 +60,7 @@ void Graph::LoadCSR(torch::Tensor indptr, torch::Tensor indices) {
   TORCH_CHECK(m->indptr.numel() == num_rows_ + 1, "LoadCSR: indptr has ",
               indptr.numel(), " entries for ", num_rows_, " rows");
   check_compressed(m->indptr, m->indices, num_cols_, "LoadCSR");
+  m->num_minor = num_cols_;
   csr_ = m;
   num_edges_ = indices.numel();
 }
@@ -143,10 +145,12 @@ void Graph::CreateSparseFormat(int64_t format) {
     if (csc_) return;
     if (!coo_) coo_ = expand(*csr_, false);
     csc_ = compress(*coo_, true, num_cols_);
+    csc_->num_minor = num_rows_;
   } else if (format == kCSR) {
     if (csr_) return;
     if (!coo_) coo_ = expand(*csc_, true);
     csr_ = compress(*coo_, false, num_rows_);
+    csr_->num_minor = num_cols_;
   } else {
     TORCH_CHECK(false, "unsupported sparse format ", format);
   }
@@ -196,6 +200,16 @@ MajorResult major_slice(const Compressed& m, const torch::Tensor& picked,
   return r;
 }
 
+// The int32 copy pays from a few megabytes of ids on (below that the int64
+// array stays in cache anyway); undefined when the matrix does not qualify.
+const torch::Tensor& Compressed::narrow_indices() const {
+  constexpr int64_t kMinEdges = int64_t(1) << 20;
+  if (!indices32.defined() && num_minor >= 0 && num_minor < (int64_t(1) << 31) &&
+      indices.is_cuda() && indices.numel() >= kMinEdges)
+    indices32 = indices.to(torch::kInt32);
+  return indices32;
+}
+
 // picked undefined: sample every column of the matrix itself.
 MajorResult major_sample_uniform(const Compressed& m,
                                         const torch::Tensor& picked,
@@ -221,12 +235,22 @@ MajorResult major_sample_uniform(const Compressed& m,
   r.select = new_ids(size, m.indptr);
   if (with_coo) r.major_ids = new_ids(size, m.indptr);
   const RandomState& rs = random_state();
-  GS_CALL(gs_csc_col_sample_uniform_fill(
-      cptr(m.indptr), num_major, cptr(m.indices),
-      fused ? cptr(picked) : nullptr, n, fanout, replace ? 1 : 0, (int)rs.algo,
-      rs.seed, next_call_id(), cptr(r.indptr),
-      with_coo ? mptr(r.major_ids) : nullptr, mptr(r.minor_ids), mptr(r.select),
-      cur_stream()));
+  const torch::Tensor& narrow = m.narrow_indices();
+  if (narrow.defined()) {
+    GS_CALL(gs_csc_col_sample_uniform_fill_i32(
+        cptr(m.indptr), num_major, narrow.data_ptr<int32_t>(),
+        fused ? cptr(picked) : nullptr, n, fanout, replace ? 1 : 0, (int)rs.algo,
+        rs.seed, next_call_id(), cptr(r.indptr),
+        with_coo ? mptr(r.major_ids) : nullptr, mptr(r.minor_ids), mptr(r.select),
+        cur_stream()));
+  } else {
+    GS_CALL(gs_csc_col_sample_uniform_fill(
+        cptr(m.indptr), num_major, cptr(m.indices),
+        fused ? cptr(picked) : nullptr, n, fanout, replace ? 1 : 0, (int)rs.algo,
+        rs.seed, next_call_id(), cptr(r.indptr),
+        with_coo ? mptr(r.major_ids) : nullptr, mptr(r.minor_ids), mptr(r.select),
+        cur_stream()));
+  }
   const int64_t nnz = count.get();
   r.minor_ids = r.minor_ids.narrow(0, 0, nnz);
   r.select = r.select.narrow(0, 0, nnz);

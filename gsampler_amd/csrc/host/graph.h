@@ -26,6 +26,14 @@ constexpr int64_t kCOO = 1, kCSC = 2, kCSR = 4;
 struct Compressed {
   torch::Tensor indptr, indices;
   c10::optional<torch::Tensor> e_ids;
+  // Exclusive bound of the ids in `indices` when it is known (a loaded or
+  // converted matrix), else -1.
+  int64_t num_minor = -1;
+  // int32 copy of `indices` for the uniform sampler (half the bytes behind
+  // every random pick); made on the first sampling call of a matrix in device
+  // memory whose ids fit.
+  mutable torch::Tensor indices32;
+  const torch::Tensor& narrow_indices() const;
 };
 
 struct Coordinate {

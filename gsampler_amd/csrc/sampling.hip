@@ -18,10 +18,10 @@ __device__ __forceinline__ int64_t load_coherent(const int64_t* p) {
 
 // One column by a group of G lanes, any fanout: slots are strided over the
 // lanes.  The path of the reservoir algorithm and of fanouts above 64.
-template <int G>
+template <int G, typename IdxT>
 __device__ __forceinline__ void sample_column_generic(
     int lane, int64_t item, int64_t in_start, int64_t deg, int64_t out_start,
-    const int64_t* __restrict__ indices, int64_t fanout, int replace,
+    const IdxT* __restrict__ indices, int64_t fanout, int replace,
     PhiloxKey key, int64_t* __restrict__ out_coo_col,
     int64_t* __restrict__ out_indices, int64_t* __restrict__ out_select) {
   const uint64_t pos = (uint64_t)item;
@@ -30,7 +30,7 @@ __device__ __forceinline__ void sample_column_generic(
     for (int64_t j = lane; j < fanout; j += G) {
       int64_t p = in_start + (int64_t)philox_bounded(key, pos, (uint64_t)j,
                                                       (uint64_t)deg);
-      out_indices[out_start + j] = indices ? indices[p] : p;
+      out_indices[out_start + j] = indices ? (int64_t)indices[p] : p;
       out_select[out_start + j] = p;
       if (out_coo_col) out_coo_col[out_start + j] = item;
     }
@@ -40,7 +40,7 @@ __device__ __forceinline__ void sample_column_generic(
     // the whole column, original order
     for (int64_t j = lane; j < deg; j += G) {
       int64_t p = in_start + j;
-      out_indices[out_start + j] = indices ? indices[p] : p;
+      out_indices[out_start + j] = indices ? (int64_t)indices[p] : p;
       out_select[out_start + j] = p;
       if (out_coo_col) out_coo_col[out_start + j] = item;
     }
@@ -63,7 +63,7 @@ __device__ __forceinline__ void sample_column_generic(
   __builtin_amdgcn_wave_barrier();
   for (int64_t jj = lane; jj < fanout; jj += G) {
     int64_t p = in_start + load_coherent(out_select + out_start + jj);
-    out_indices[out_start + jj] = indices ? indices[p] : p;
+    out_indices[out_start + jj] = indices ? (int64_t)indices[p] : p;
     out_select[out_start + jj] = p;
     if (out_coo_col) out_coo_col[out_start + jj] = item;
   }
@@ -104,10 +104,10 @@ __device__ __forceinline__ int64_t floyd_slot(int lane, int K, int64_t deg,
 // flight instead of 64 / G.  On a 124M-edge power-law graph U = 2 and U = 4
 // measured 3 % and 20 % slower than U = 1: at full occupancy the kernel is
 // bound by the sectors its random gathers pull in, not by their latency.
-template <int G, int U>
+template <int G, int U, typename IdxT>
 __global__ __launch_bounds__(kBlock) void sample_uniform_kernel(
     const int64_t* __restrict__ indptr, int64_t num_cols,
-    const int64_t* __restrict__ indices, const int64_t* __restrict__ column_ids,
+    const IdxT* __restrict__ indices, const int64_t* __restrict__ column_ids,
     int64_t num_items, int64_t fanout, int replace, int algo, PhiloxKey key,
     const int64_t* __restrict__ sub_indptr, int64_t* __restrict__ out_coo_col,
     int64_t* __restrict__ out_indices, int64_t* __restrict__ out_select) {
@@ -138,7 +138,7 @@ __global__ __launch_bounds__(kBlock) void sample_uniform_kernel(
     const int64_t item = item0 + u;
     if (!slot_per_lane ||
         (!replace && deg[u] > fanout && algo != GS_ALGO_FLOYD)) {
-      sample_column_generic<G>(lane, item, in_start[u], deg[u], out_start[u],
+      sample_column_generic<G, IdxT>(lane, item, in_start[u], deg[u], out_start[u],
                                indices, fanout, replace, key, out_coo_col,
                                out_indices, out_select);
     } else if (replace) {
@@ -157,7 +157,7 @@ __global__ __launch_bounds__(kBlock) void sample_uniform_kernel(
   int64_t v[U];
 #pragma unroll
   for (int u = 0; u < U; ++u)
-    v[u] = (p[u] >= 0 && indices) ? indices[p[u]] : p[u];
+    v[u] = (p[u] >= 0 && indices) ? (int64_t)indices[p[u]] : p[u];
 #pragma unroll
   for (int u = 0; u < U; ++u) {
     if (p[u] < 0) continue;
@@ -167,9 +167,9 @@ __global__ __launch_bounds__(kBlock) void sample_uniform_kernel(
   }
 }
 
-template <int G>
+template <int G, typename IdxT>
 static int launch_sample_uniform(const int64_t* indptr, int64_t num_cols,
-                                 const int64_t* indices,
+                                 const IdxT* indices,
                                  const int64_t* column_ids, int64_t num_items,
                                  int64_t fanout, int replace, int algo,
                                  PhiloxKey key, const int64_t* sub_indptr,
@@ -178,8 +178,8 @@ static int launch_sample_uniform(const int64_t* indptr, int64_t num_cols,
   // one column per lane group (see the note on U above the kernel)
   const int64_t blocks = ceil_div(num_items * G, kBlock);
   GS_LAUNCH("sample_uniform", stream,
-            sample_uniform_kernel<G, 1><<<dim3((unsigned)blocks), dim3(kBlock), 0,
-                                          stream>>>(
+            (sample_uniform_kernel<G, 1, IdxT>)<<<dim3((unsigned)blocks), dim3(kBlock), 0,
+                                                stream>>>(
                 indptr, num_cols, indices, column_ids, num_items, fanout, replace,
                 algo, key, sub_indptr, out_coo_col, out_indices, out_select));
   return GS_OK;
@@ -187,13 +187,13 @@ static int launch_sample_uniform(const int64_t* indptr, int64_t num_cols,
 
 }  // namespace gs
 
-extern "C" int gs_csc_col_sample_uniform_fill(
-    const int64_t* indptr, int64_t num_cols, const int64_t* indices,
-    const int64_t* column_ids, int64_t num_items, int64_t fanout, int replace,
-    int algo, uint64_t seed, uint64_t call_id, const int64_t* sub_indptr,
-    int64_t* out_coo_col, int64_t* out_indices, int64_t* out_select,
-    gs_stream_t stream) {
-  using namespace gs;
+namespace gs {
+template <typename IdxT>
+static int sample_uniform_fill(const int64_t* indptr, int64_t num_cols, const IdxT* indices,
+                               const int64_t* column_ids, int64_t num_items, int64_t fanout,
+                               int replace, int algo, uint64_t seed, uint64_t call_id,
+                               const int64_t* sub_indptr, int64_t* out_coo_col,
+                               int64_t* out_indices, int64_t* out_select, gs_stream_t stream) {
   GS_REQUIRE(num_items >= 0 && num_cols >= 0, "sample_uniform: negative size");
   GS_REQUIRE(fanout >= 0, "sample_uniform: negative fanout %lld",
              (long long)fanout);
@@ -216,11 +216,35 @@ extern "C" int gs_csc_col_sample_uniform_fill(
 #define GS_SAMPLE_ARGS                                                    \
   indptr, num_cols, indices, column_ids, num_items, fanout, replace, algo, \
       key, sub_indptr, out_coo_col, out_indices, out_select, s
-  if (fanout <= 8) return launch_sample_uniform<8>(GS_SAMPLE_ARGS);
-  if (fanout <= 16) return launch_sample_uniform<16>(GS_SAMPLE_ARGS);
-  if (fanout <= 32) return launch_sample_uniform<32>(GS_SAMPLE_ARGS);
-  return launch_sample_uniform<64>(GS_SAMPLE_ARGS);
+  if (fanout <= 8) return launch_sample_uniform<8, IdxT>(GS_SAMPLE_ARGS);
+  if (fanout <= 16) return launch_sample_uniform<16, IdxT>(GS_SAMPLE_ARGS);
+  if (fanout <= 32) return launch_sample_uniform<32, IdxT>(GS_SAMPLE_ARGS);
+  return launch_sample_uniform<64, IdxT>(GS_SAMPLE_ARGS);
 #undef GS_SAMPLE_ARGS
+}
+}  // namespace gs
+
+extern "C" int gs_csc_col_sample_uniform_fill(
+    const int64_t* indptr, int64_t num_cols, const int64_t* indices,
+    const int64_t* column_ids, int64_t num_items, int64_t fanout, int replace,
+    int algo, uint64_t seed, uint64_t call_id, const int64_t* sub_indptr,
+    int64_t* out_coo_col, int64_t* out_indices, int64_t* out_select,
+    gs_stream_t stream) {
+  return gs::sample_uniform_fill<int64_t>(indptr, num_cols, indices, column_ids, num_items,
+                                          fanout, replace, algo, seed, call_id, sub_indptr,
+                                          out_coo_col, out_indices, out_select, stream);
+}
+
+extern "C" int gs_csc_col_sample_uniform_fill_i32(
+    const int64_t* indptr, int64_t num_cols, const int32_t* indices32,
+    const int64_t* column_ids, int64_t num_items, int64_t fanout, int replace,
+    int algo, uint64_t seed, uint64_t call_id, const int64_t* sub_indptr,
+    int64_t* out_coo_col, int64_t* out_indices, int64_t* out_select,
+    gs_stream_t stream) {
+  GS_REQUIRE(indices32 != nullptr, "sample_uniform_i32: null indices");
+  return gs::sample_uniform_fill<int32_t>(indptr, num_cols, indices32, column_ids, num_items,
+                                          fanout, replace, algo, seed, call_id, sub_indptr,
+                                          out_coo_col, out_indices, out_select, stream);
 }
 
 // ---------------------------------------------------------------------------

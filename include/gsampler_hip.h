@@ -177,6 +177,21 @@ int gs_csc_col_sample_uniform_fill(const int64_t* indptr, int64_t num_cols,
                                    int64_t* out_coo_col, int64_t* out_indices,
                                    int64_t* out_select, gs_stream_t stream);
 
+/* The same with the row ids read from a 32-bit copy of `indices`
+ * (indices32[e] == indices[e] for every edge, all ids < 2^31): identical
+ * outputs (int64), half the bytes behind every random pick.  A matrix whose
+ * row count allows it keeps such a copy beside the int64 array. */
+int gs_csc_col_sample_uniform_fill_i32(const int64_t* indptr, int64_t num_cols,
+                                       const int32_t* indices32,
+                                       const int64_t* column_ids,
+                                       int64_t num_items, int64_t fanout,
+                                       int replace, int algo, uint64_t seed,
+                                       uint64_t call_id,
+                                       const int64_t* sub_indptr,
+                                       int64_t* out_coo_col,
+                                       int64_t* out_indices,
+                                       int64_t* out_select, gs_stream_t stream);
+
 /* ------------------------------------------------------------------------
  * Weighted per-column sampling (fill phase; counts come from
  * gs_csc_col_count).  probs[nnz] (fp32) is aligned with `indices`; indices may

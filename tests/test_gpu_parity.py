@@ -70,12 +70,13 @@ def test_sample_uniform_parity(algo, fanout):
     rng = np.random.default_rng(fanout)
     indptr, indices = random_csc(rng, 5000, 10**6, 90, hub_deg=20000)
     cols = rng.integers(0, 5000, size=4097)
+    narrow = T(indices).to(torch.int32)      # the int32 copy of the row ids: same outputs
     for call_id in (0, 3):
-        assert_same(
-            capi.sample_uniform(T(indptr), T(indices), T(cols), fanout, False, algo,
-                                seed=7777, call_id=call_id),
-            orc.sample_uniform(indptr, indices, cols, fanout, False, algo,
-                               seed=7777, call_id=call_id))
+        want = orc.sample_uniform(indptr, indices, cols, fanout, False, algo,
+                                  seed=7777, call_id=call_id)
+        for ids in (T(indices), narrow):
+            assert_same(capi.sample_uniform(T(indptr), ids, T(cols), fanout, False, algo,
+                                            seed=7777, call_id=call_id), want)
 
 
 @pytest.mark.parametrize("fanout", [3, 20, 100])
@@ -84,6 +85,8 @@ def test_sample_replace_and_unfused_parity(fanout):
     indptr, indices = random_csc(rng, 2000, 10**6, 50, hub_deg=3000)
     cols = rng.integers(0, 2000, size=1500)
     assert_same(capi.sample_uniform(T(indptr), T(indices), T(cols), fanout, True),
+                orc.sample_uniform(indptr, indices, cols, fanout, True))
+    assert_same(capi.sample_uniform(T(indptr), T(indices).to(torch.int32), T(cols), fanout, True),
                 orc.sample_uniform(indptr, indices, cols, fanout, True))
     # column_ids = None: sample the matrix's own columns (un-fused Sampling)
     for replace in (False, True):
