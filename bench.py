@@ -109,9 +109,9 @@ def kernel_bytes(name, sizes):
             "unique_hist": 8 * N,                # keys in
             "unique_scatter": 16 * N,            # keys in, packed entries out
             "unique_dedup": 12 * N,              # packed entries in, first positions out
-            "unique_flag": 4 * N + N // 8,       # first positions in, flag bits out
-            "unique_fill": N // 8 + 16 * U + 4 * N,  # flags + first keys in, frontier + ranks out
-            "unique_relabel": 40 * E,            # 2 first positions + 2 ranks + column id in, row + col out
+            "unique_flag": 4 * N + N // 4,       # first positions in, rank words out
+            "unique_fill": N // 4 + 16 * U,      # rank words + first keys in, frontier out
+            "unique_relabel": 28 * E,            # first position + column id in, row + col out
         }.get(name, 0)
     return total
 

@@ -44,7 +44,7 @@ SIGNATURES = {
     "gs_copy_i64": (_int, [_p, _i64, _p, _p]),
     "gs_scan_workspace_bytes": (_sz, [_i64]),
     "gs_exclusive_scan_i64": (_int, [_p, _p, _i64, _p, _sz, _p]),
-    "gs_csc_col_count": (_int, [_p, _i64, _p, _i64, _i64, _int, _p, _p, _sz, _p]),
+    "gs_csc_col_count": (_int, [_p, _i64, _p, _i64, _i64, _int, _p, _p, _p, _sz, _p]),
     "gs_csc_col_count_static": (_int, [_p, _i64, _p, _i64, _i64, _int, _p, _p]),
     "gs_csc_col_slice_fill": (_int, [_p, _i64, _p, _p, _i64, _p, _i64, _p, _i64,
                                      _i64, _p, _p, _p, _p]),
@@ -55,7 +55,7 @@ SIGNATURES = {
                                                   _int, _u64, _u64, _p, _p, _p, _p,
                                                   _p]),
     "gs_unique_workspace_bytes": (_sz, [_i64, _i64, _i64]),
-    "gs_unique_count": (_int, [_p, _p, _i64, _p, _p, _i64, _i64, _p, _p, _sz, _p]),
+    "gs_unique_count": (_int, [_p, _p, _i64, _p, _p, _i64, _i64, _p, _p, _p, _sz, _p]),
     "gs_unique_fill": (_int, [_p, _p, _i64, _p, _p, _i64, _i64, _p, _p, _p, _sz, _p]),
     "gs_unique_relabel": (_int, [_p, _p, _i64, _p, _p, _i64, _i64, _p, _p, _p, _p,
                                  _sz, _p]),
@@ -152,34 +152,60 @@ def _workspace(nbytes: int, device) -> torch.Tensor:
 
 
 class _Count:
-    """A count on its way from the device to the host: the 8-byte copy is queued
-    on the current stream at once, the host waits only when it needs the value.
-    Kernels launched in between (into buffers sized by an upper bound) keep the
-    GPU busy meanwhile."""
+    """A count on its way from the device to the host.  The kernel that produces
+    it stores it into a word of pinned host memory as well (the `mirror` argument
+    of the count entry points), so the host only waits for an event recorded
+    behind that kernel, and only when it needs the value.  Kernels launched in
+    between (into buffers sized by an upper bound) keep the GPU busy meanwhile.
+
+        c = _Count(); entry_point(..., c.mirror(), ...); c.arm(); ...; c.get()
+
+    A mirror of `words` entries (a whole offsets array) delivers its last one."""
     _slots = None
     _next = 0
+    _RING = 64
+    _WIDTH = 4096          # words per slot: offset arrays up to this many entries
 
-    def __init__(self, prefix: torch.Tensor):
+    def __init__(self, words: int = 1):
         cls = _Count
+        if words > cls._WIDTH:
+            raise GsError(f"a mirrored offsets array holds at most {cls._WIDTH} entries")
         if cls._slots is None:
-            cls._slots = torch.empty(64, dtype=torch.int64).pin_memory()
-        self._slot = cls._slots[cls._next % 64: cls._next % 64 + 1]
+            cls._slots = torch.empty((cls._RING, cls._WIDTH), dtype=torch.int64).pin_memory()
+        self._slot = cls._slots[cls._next % cls._RING]
+        self._words = words
         cls._next += 1
-        # a one-element copy kernel into the pinned word, in stream order
-        check(lib().gs_copy_i64(prefix.data_ptr() + 8 * (prefix.numel() - 1), 1,
-                                self._slot.data_ptr(), _stream()))
+        self._ticket = cls._next
+        self._event = None
+        self._value = None
+
+    def mirror(self) -> int:
+        return self._slot.data_ptr()
+
+    def arm(self) -> "_Count":
         self._event = torch.cuda.Event()
         self._event.record()
-        self._ticket = cls._next
-        self._value = None
+        return self
 
     def get(self) -> int:
         if self._value is None:
             # helpers read their counts before they return; the ring is 64 deep
-            if _Count._next - self._ticket >= 64:
+            if _Count._next - self._ticket >= _Count._RING:
                 raise GsError("a pending count was overwritten by later requests")
             self._event.synchronize()
-            self._value = int(self._slot[0])
+            self._value = int(self._slot[self._words - 1])
+        return self._value
+
+
+class _Fetched:
+    """The last entry of a device array, read with a blocking copy on first use."""
+
+    def __init__(self, prefix: torch.Tensor):
+        self._prefix, self._value = prefix, None
+
+    def get(self) -> int:
+        if self._value is None:
+            self._value = int(self._prefix[-1].item())
         return self._value
 
 
@@ -222,8 +248,9 @@ def exclusive_scan(x: torch.Tensor) -> torch.Tensor:
 
 def col_count(indptr: torch.Tensor, column_ids: Optional[torch.Tensor],
               fanout: int, replace: bool,
-              num_items: Optional[int] = None) -> torch.Tensor:
-    """sub_indptr[num_items + 1] for slicing (fanout < 0) or sampling."""
+              num_items: Optional[int] = None, count: Optional[_Count] = None) -> torch.Tensor:
+    """sub_indptr[num_items + 1] for slicing (fanout < 0) or sampling.  With
+    `count` the edge total is also on its way to the host when this returns."""
     indptr = _i64t(indptr, "indptr")
     num_cols = indptr.numel() - 1
     if column_ids is not None:
@@ -235,8 +262,10 @@ def col_count(indptr: torch.Tensor, column_ids: Optional[torch.Tensor],
     ws = _workspace(lib().gs_scan_workspace_bytes(num_items + 1), indptr.device)
     check(lib().gs_csc_col_count(_ptr(indptr), num_cols, _ptr(column_ids),
                                  num_items, fanout, int(replace),
-                                 sub_indptr.data_ptr(), ws.data_ptr(), ws.numel(),
-                                 _stream()))
+                                 sub_indptr.data_ptr(), count.mirror() if count else None,
+                                 ws.data_ptr(), ws.numel(), _stream()))
+    if count:
+        count.arm()
     return sub_indptr
 
 
@@ -285,8 +314,8 @@ def sample_uniform(indptr, indices, column_ids, fanout, replace=False,
         n = column_ids.numel()
     else:
         n = num_cols
-    sub_indptr = col_count(indptr, column_ids, fanout, replace, n)
-    count = _Count(sub_indptr)
+    count = _Count()
+    sub_indptr = col_count(indptr, column_ids, fanout, replace, n, count)
     bound = n * fanout                       # no column yields more than fanout edges
     size = bound if bound <= _BOUND_LIMIT else count.get()
     dev = indptr.device
@@ -321,10 +350,11 @@ def unique_relabel(seeds, rows, seeds_ptr=None, rows_ptr=None, edge_col=None,
     unique_ptr = torch.empty(B + 1, dtype=torch.int64, device=dev)
     sp = seeds_ptr.data_ptr() if seeds_ptr is not None else None
     rp = rows_ptr.data_ptr() if rows_ptr is not None else None
+    count = _Count(B + 1) if B + 1 <= _Count._WIDTH else None
     check(l.gs_unique_count(_ptr(seeds), sp, S, _ptr(rows), rp, E, B,
-                            unique_ptr.data_ptr(), ws.data_ptr(), ws.numel(),
-                            _stream()))
-    count = _Count(unique_ptr)
+                            unique_ptr.data_ptr(), count.mirror() if count else None,
+                            ws.data_ptr(), ws.numel(), _stream()))
+    count = count.arm() if count else _Fetched(unique_ptr)
     size = S + E if S + E <= _BOUND_LIMIT else count.get()   # U <= S + E
     unique = torch.empty(size, dtype=torch.int64, device=dev)
     want_col = want_col and edge_col is not None
@@ -641,8 +671,8 @@ def _sample_weighted_cdf(indptr, indices, cdf, column_ids, fanout, replace, seed
         n = column_ids.numel()
     else:
         n = num_cols
-    sub_indptr = col_count(indptr, column_ids, fanout, replace, n)
-    count = _Count(sub_indptr)
+    count = _Count()
+    sub_indptr = col_count(indptr, column_ids, fanout, replace, n, count)
     bound = n * fanout
     size = bound if bound <= _BOUND_LIMIT else count.get()
     out_idx = torch.empty(size, dtype=torch.int64, device=dev)

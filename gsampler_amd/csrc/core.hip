@@ -137,7 +137,7 @@ __global__ __launch_bounds__(kBlock) void scan_spine_kernel(int64_t* tile_sums,
 template <bool kSpineDone>
 __global__ __launch_bounds__(kBlock) void scan_down_kernel(
     const int64_t* in, int64_t* out, int64_t n,
-    const int64_t* __restrict__ tile_sums) {
+    const int64_t* __restrict__ tile_sums, int64_t* last_mirror) {
   __shared__ int64_t smem[kBlock / kWave + 1];
   const int64_t base = (int64_t)blockIdx.x * kScanTile + threadIdx.x * kScanItems;
   int64_t v[kScanItems];
@@ -164,6 +164,7 @@ __global__ __launch_bounds__(kBlock) void scan_down_kernel(
   for (int k = 0; k < kScanItems; ++k) {
     int64_t i = base + k;
     if (i < n) out[i] = ex;
+    if (i == n - 1 && last_mirror) *last_mirror = ex;
     ex += v[k];
   }
 }
@@ -176,7 +177,8 @@ size_t scan_workspace_bytes(int64_t n) {
 }
 
 int exclusive_scan_i64(const int64_t* in, int64_t* out, int64_t n, void* ws,
-                       size_t ws_bytes, hipStream_t stream) {
+                       size_t ws_bytes, hipStream_t stream, bool sums_ready,
+                       int64_t* last_mirror) {
   if (n <= 0) return GS_OK;
   if (ws_bytes < scan_workspace_bytes(n) || ws == nullptr) {
     set_error("scan workspace too small: %zu < %zu", ws_bytes,
@@ -188,16 +190,17 @@ int exclusive_scan_i64(const int64_t* in, int64_t* out, int64_t n, void* ws,
   if (tiles == 1) {  // nothing before the only tile
     GS_LAUNCH("scan_down", stream,
               scan_down_kernel<false><<<dim3(1), dim3(kBlock), 0, stream>>>(
-                  in, out, n, tile_sums));
+                  in, out, n, tile_sums, last_mirror));
     return GS_OK;
   }
-  GS_LAUNCH("scan_tile_sums", stream,
-            scan_tile_sums_kernel<<<dim3((unsigned)tiles), dim3(kBlock), 0,
-                                    stream>>>(in, n, tile_sums));
+  if (!sums_ready)
+    GS_LAUNCH("scan_tile_sums", stream,
+              scan_tile_sums_kernel<<<dim3((unsigned)tiles), dim3(kBlock), 0,
+                                      stream>>>(in, n, tile_sums));
   if (tiles <= kShortSpine) {
     GS_LAUNCH("scan_down", stream,
               scan_down_kernel<false><<<dim3((unsigned)tiles), dim3(kBlock), 0,
-                                        stream>>>(in, out, n, tile_sums));
+                                        stream>>>(in, out, n, tile_sums, last_mirror));
     return GS_OK;
   }
   GS_LAUNCH("scan_spine", stream,
@@ -205,7 +208,7 @@ int exclusive_scan_i64(const int64_t* in, int64_t* out, int64_t n, void* ws,
                                                                     tiles));
   GS_LAUNCH("scan_down", stream,
             scan_down_kernel<true><<<dim3((unsigned)tiles), dim3(kBlock), 0,
-                                      stream>>>(in, out, n, tile_sums));
+                                      stream>>>(in, out, n, tile_sums, last_mirror));
   return GS_OK;
 }
 
@@ -234,7 +237,7 @@ int gs_copy_i64(const int64_t* src, int64_t n, int64_t* dst, gs_stream_t stream)
 
 const char* gs_last_error(void) { return gs::g_last_error.c_str(); }
 
-int gs_abi_version(void) { return 2; }
+int gs_abi_version(void) { return 3; }
 
 void gs_profile_enable(int on) {
   std::lock_guard<std::mutex> lock(gs::g_prof_mutex);

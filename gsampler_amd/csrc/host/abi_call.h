@@ -98,6 +98,20 @@ class AsyncCount {
     check(hipEventRecord(r.events[slot_], s));
     pending_ = true;
   }
+  // For a kernel that stores the value to the host itself: hand it mirror(),
+  // then arm() once it is queued.
+  static AsyncCount mirrored() {
+    AsyncCount c;
+    Ring& r = ring();
+    c.ticket_ = r.next++;
+    c.slot_ = (int)(c.ticket_ % kSlots);
+    return c;
+  }
+  int64_t* mirror() const { return ring().words + slot_; }
+  void arm() {
+    check(hipEventRecord(ring().events[slot_], (hipStream_t)cur_stream()));
+    pending_ = true;
+  }
   int64_t get() {
     TORCH_CHECK(slot_ >= 0, "AsyncCount: nothing was requested");
     Ring& r = ring();
@@ -149,6 +163,17 @@ class AsyncCount {
 class OffsetMirror {
  public:
   static void prefetch(const torch::Tensor& offsets) { (void)entry_for(offsets); }
+  // For a kernel that stores the array to the host itself: the pinned block it
+  // should write to (as many entries as `offsets` has), and arm() once that
+  // kernel is queued.
+  static int64_t* reserve(const torch::Tensor& offsets) {
+    return entry_for(offsets, /*copy=*/false).pinned;
+  }
+  static void arm(const torch::Tensor& offsets) {
+    Entry& e = entry_for(offsets, false);
+    check(hipEventRecord(e.event, (hipStream_t)cur_stream()));
+    e.pending = true;
+  }
   static const std::vector<int64_t>& values(const torch::Tensor& offsets) {
     Entry& e = entry_for(offsets);
     if (e.pending) {
@@ -176,7 +201,7 @@ class OffsetMirror {
   static void check(hipError_t e) {
     TORCH_CHECK(e == hipSuccess, "HIP error: ", hipGetErrorString(e));
   }
-  static Entry& entry_for(const torch::Tensor& offsets) {
+  static Entry& entry_for(const torch::Tensor& offsets, bool copy = true) {
     static thread_local std::vector<Entry> ring(kEntries);
     static thread_local size_t next = 0;
     TORCH_CHECK(offsets.defined() && offsets.scalar_type() == torch::kInt64,
@@ -191,7 +216,7 @@ class OffsetMirror {
     e.version = offsets._version();
     e.count = (size_t)offsets.numel();
     e.pending = false;
-    if (!offsets.is_cuda()) {
+    if (!offsets.is_cuda() && copy) {
       torch::Tensor c = offsets.contiguous();
       e.host.assign(c.data_ptr<int64_t>(), c.data_ptr<int64_t>() + e.count);
       return e;
@@ -202,6 +227,7 @@ class OffsetMirror {
       check(hipHostMalloc((void**)&e.pinned, e.capacity * sizeof(int64_t), hipHostMallocDefault));
     }
     if (!e.event) check(hipEventCreateWithFlags(&e.event, hipEventDisableTiming));
+    if (!copy) return e;
     torch::Tensor c = offsets.contiguous();
     hipStream_t s = (hipStream_t)cur_stream();
     if (e.count > 0)
@@ -236,14 +262,21 @@ class EdgeCount {
     }
     ~HintScope() { hint() = Hint(); }
   };
-  explicit EdgeCount(const torch::Tensor& prefix) {
+  // Before the count pass: what to give it as total_mirror (null when the
+  // per-batch edge pointer is sent instead).
+  EdgeCount() {
+    if (!hint().col_bptr.defined()) count_ = AsyncCount::mirrored();
+  }
+  int64_t* mirror() const { return hint().col_bptr.defined() ? nullptr : count_.mirror(); }
+  // After the count pass is queued.
+  void arm(const torch::Tensor& prefix) {
     Hint& h = hint();
     if (h.col_bptr.defined()) {
       edge_bptr_ = prefix.index_select(0, h.col_bptr);
       OffsetMirror::prefetch(edge_bptr_);
       h.edge_bptr = edge_bptr_;
     } else {
-      count_ = AsyncCount(prefix);
+      count_.arm();
     }
   }
   int64_t get() {

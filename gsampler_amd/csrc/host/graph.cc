@@ -185,7 +185,7 @@ MajorResult major_slice(const Compressed& m, const torch::Tensor& picked,
   r.indptr = new_ids(n + 1, m.indptr);
   torch::Tensor ws = new_workspace(gs_scan_workspace_bytes(n + 1), m.indptr);
   GS_CALL(gs_csc_col_count(cptr(m.indptr), num_major, cptr(picked), n, -1, 0,
-                           mptr(r.indptr), ws.data_ptr(), ws.numel(),
+                           mptr(r.indptr), nullptr, ws.data_ptr(), ws.numel(),
                            cur_stream()));
   const int64_t nnz = read_last(r.indptr);
   r.minor_ids = new_ids(nnz, m.indptr);
@@ -222,13 +222,14 @@ MajorResult major_sample_uniform(const Compressed& m,
   MajorResult r;
   r.indptr = new_ids(n + 1, m.indptr);
   torch::Tensor ws = new_workspace(gs_scan_workspace_bytes(n + 1), m.indptr);
-  GS_CALL(gs_csc_col_count(cptr(m.indptr), num_major,
-                           fused ? cptr(picked) : nullptr, n, fanout,
-                           replace ? 1 : 0, mptr(r.indptr), ws.data_ptr(),
-                           ws.numel(), cur_stream()));
   // No column yields more than fanout edges: size the outputs by that bound,
   // launch, and trim when the count has arrived.
-  EdgeCount count(r.indptr);
+  EdgeCount count;
+  GS_CALL(gs_csc_col_count(cptr(m.indptr), num_major,
+                           fused ? cptr(picked) : nullptr, n, fanout,
+                           replace ? 1 : 0, mptr(r.indptr), count.mirror(),
+                           ws.data_ptr(), ws.numel(), cur_stream()));
+  count.arm(r.indptr);
   const int64_t bound = n * fanout;
   const int64_t size = bound <= kBoundLimit ? bound : count.get();
   r.minor_ids = new_ids(size, m.indptr);
@@ -405,13 +406,15 @@ Graph::Frontier& Graph::frontier_for(const torch::Tensor& seeds,
   const int64_t S = seeds.numel(), E = rows.numel();
   f->workspace = new_workspace(gs_unique_workspace_bytes(S, E, B), rows);
   f->unique_ptr = new_ids(B + 1, rows);
+  // The whole pointer array goes to the host as well, written there by the kernel
+  // that computes it: its last entry is the size of the frontier, the rest is
+  // what per-batch splits ask for later.
+  int64_t* mirror = OffsetMirror::reserve(f->unique_ptr);
   GS_CALL(gs_unique_count(cptr(seeds), cptr(seeds_ptr), S, cptr(rows),
-                          cptr(rows_ptr), E, B, mptr(f->unique_ptr),
+                          cptr(rows_ptr), E, B, mptr(f->unique_ptr), mirror,
                           f->workspace.data_ptr(), f->workspace.numel(),
                           cur_stream()));
-  // The whole pointer array goes to the host in one copy: its last entry is the
-  // size of the frontier, the rest is what per-batch splits ask for later.
-  OffsetMirror::prefetch(f->unique_ptr);
+  OffsetMirror::arm(f->unique_ptr);
   BatchOffsets::trust(f->unique_ptr);
   // at most S + E unique keys
   f->unique_buffer =

@@ -37,7 +37,8 @@ GraphAndIndex Graph::SamplingProbs(int64_t axis, torch::Tensor edge_probs,
   r.indptr = new_ids(n + 1, m.indptr);
   torch::Tensor ws = new_workspace(gs_scan_workspace_bytes(n + 1), m.indptr);
   GS_CALL(gs_csc_col_count(cptr(m.indptr), n, nullptr, n, fanout, replace ? 1 : 0,
-                           mptr(r.indptr), ws.data_ptr(), ws.numel(), cur_stream()));
+                           mptr(r.indptr), nullptr, ws.data_ptr(), ws.numel(),
+                           cur_stream()));
   const int64_t nnz = read_last(r.indptr);
   r.minor_ids = new_ids(nnz, m.indptr);
   r.select = new_ids(nnz, m.indptr);
@@ -100,10 +101,11 @@ GraphAndIndex Graph::FusedSlicingSamplingProbs(int64_t axis, torch::Tensor seeds
   MajorResult r;
   r.indptr = new_ids(n + 1, m.indptr);
   torch::Tensor ws = new_workspace(gs_scan_workspace_bytes(n + 1), m.indptr);
+  EdgeCount count;
   GS_CALL(gs_csc_col_count(cptr(m.indptr), num_major, cptr(seeds), n, fanout,
-                           replace ? 1 : 0, mptr(r.indptr), ws.data_ptr(), ws.numel(),
-                           cur_stream()));
-  EdgeCount count(r.indptr);
+                           replace ? 1 : 0, mptr(r.indptr), count.mirror(), ws.data_ptr(),
+                           ws.numel(), cur_stream()));
+  count.arm(r.indptr);
   const int64_t bound = n * fanout;
   const int64_t size = bound <= kBoundLimit ? bound : count.get();
   r.minor_ids = new_ids(size, m.indptr);

@@ -33,27 +33,44 @@ static int static_scratch(int64_t** out) {
   return GS_OK;
 }
 
-// One thread per requested column: writes its output count; the scan that
-// follows turns the counts into sub_indptr in place.
-__global__ __launch_bounds__(kBlock) void col_count_kernel(
+// One work-group of kCountThreads threads per tile of the scan that follows
+// (kScanTile consecutive columns): writes the output counts and the tile's sum,
+// so that the scan only has its down sweep left to turn the counts into
+// sub_indptr in place.
+constexpr int kCountThreads = 1024;
+constexpr int kCountItems = kScanTile / kCountThreads;
+__global__ __launch_bounds__(kCountThreads) void col_count_kernel(
     const int64_t* __restrict__ indptr, int64_t num_cols,
     const int64_t* __restrict__ column_ids, int64_t num_items, int64_t fanout,
-    int replace, int64_t* __restrict__ counts) {
-  const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
-  if (i > num_items) return;
-  int64_t cnt = 0;
-  if (i < num_items) {
-    int64_t c = column_ids ? column_ids[i] : i;
-    int64_t in_start;
-    int64_t deg = column_degree(indptr, num_cols, c, &in_start);
-    if (fanout < 0)
-      cnt = deg;
-    else if (replace)
-      cnt = deg == 0 ? 0 : fanout;
-    else
-      cnt = deg < fanout ? deg : fanout;
+    int replace, int64_t* __restrict__ counts, int64_t* __restrict__ tile_sums) {
+  __shared__ int64_t smem[kCountThreads / kWave + 1];
+  const int64_t base = (int64_t)blockIdx.x * kScanTile + threadIdx.x;
+  int64_t cnt[kCountItems], sum = 0;
+#pragma unroll
+  for (int k = 0; k < kCountItems; ++k) {
+    const int64_t i = base + k * kCountThreads;
+    cnt[k] = 0;
+    if (i < num_items) {
+      int64_t in_start;
+      const int64_t deg =
+          column_degree(indptr, num_cols, column_ids ? column_ids[i] : i, &in_start);
+      if (fanout < 0)
+        cnt[k] = deg;
+      else if (replace)
+        cnt[k] = deg == 0 ? 0 : fanout;
+      else
+        cnt[k] = deg < fanout ? deg : fanout;
+    }
+    sum += cnt[k];
   }
-  counts[i] = cnt;  // counts[num_items] = 0 so the scan leaves the total there
+#pragma unroll
+  for (int k = 0; k < kCountItems; ++k) {
+    const int64_t i = base + k * kCountThreads;
+    if (i <= num_items) counts[i] = cnt[k];  // counts[num_items] = 0: the scan leaves the total there
+  }
+  int64_t total;
+  block_exclusive_sum<int64_t, kCountThreads>(sum, smem, &total);
+  if (threadIdx.x == 0) tile_sums[blockIdx.x] = total;
 }
 
 // Edge-parallel slice: thread e owns output edge e, finds its column by binary
@@ -108,8 +125,8 @@ extern "C" {
 int gs_csc_col_count(const int64_t* indptr, int64_t num_cols,
                      const int64_t* column_ids, int64_t num_items,
                      int64_t fanout, int replace, int64_t* sub_indptr,
-                     void* workspace, size_t workspace_bytes,
-                     gs_stream_t stream) {
+                     int64_t* total_mirror, void* workspace,
+                     size_t workspace_bytes, gs_stream_t stream) {
   using namespace gs;
   GS_REQUIRE(num_items >= 0 && num_cols >= 0, "col_count: negative size");
   GS_REQUIRE(indptr && sub_indptr, "col_count: null pointer");
@@ -118,12 +135,18 @@ int gs_csc_col_count(const int64_t* indptr, int64_t num_cols,
              (long long)num_items, (long long)num_cols);
   hipStream_t s = as_stream(stream);
   const int64_t n = num_items + 1;
+  if (workspace == nullptr || workspace_bytes < scan_workspace_bytes(n)) {
+    set_error("col_count: workspace too small: %zu < %zu", workspace_bytes,
+              scan_workspace_bytes(n));
+    return GS_ERR_WORKSPACE;
+  }
   GS_LAUNCH("col_count", s,
-            col_count_kernel<<<dim3((unsigned)ceil_div(n, kBlock)), dim3(kBlock),
+            col_count_kernel<<<dim3((unsigned)ceil_div(n, kScanTile)), dim3(kCountThreads),
                                0, s>>>(indptr, num_cols, column_ids, num_items,
-                                       fanout, replace, sub_indptr));
+                                       fanout, replace, sub_indptr,
+                                       (int64_t*)workspace));
   return exclusive_scan_i64(sub_indptr, sub_indptr, n, workspace,
-                            workspace_bytes, s);
+                            workspace_bytes, s, /*sums_ready=*/true, total_mirror);
 }
 
 int gs_csc_col_count_static(const int64_t* indptr, int64_t num_cols,
@@ -140,8 +163,8 @@ int gs_csc_col_count_static(const int64_t* indptr, int64_t num_cols,
   const int rc = static_scratch(&ws);
   if (rc != GS_OK) return rc;
   return gs_csc_col_count(indptr, num_cols, column_ids, num_items, fanout, replace,
-                          sub_indptr, ws, (size_t)kStaticScanTiles * sizeof(int64_t),
-                          stream);
+                          sub_indptr, nullptr, ws,
+                          (size_t)kStaticScanTiles * sizeof(int64_t), stream);
 }
 
 int gs_csc_col_slice_fill(const int64_t* indptr, int64_t num_cols,

@@ -10,25 +10,28 @@
 // first partitioned by hash into buckets of about 1500 entries (streaming
 // reads and writes only), and each bucket is then deduplicated by one
 // work-group in an LDS table:
-//   prep     per-batch record (where its keys, tiles and buckets start); zero
-//            the bucket counters
-//   units    batch of every tile, bucket and chunk of positions, so that a
-//            work-group finds its work with two dependent loads instead of a
-//            binary search
+//   plan     per-batch record (where its keys, tiles and buckets start), the
+//            batch of every tile, bucket, group of positions and tile of edges
+//            (so that a work-group finds its work with two dependent loads
+//            instead of a binary search); zero the bucket counters
 //   hist     per tile of one batch: LDS histogram over the batch's buckets,
 //            one global atomic per non-empty bin
-//   scan     bucket counts -> bucket offsets (bucket ranges of a batch tile its
-//            range of the flat space exactly)
-//   scatter  per tile: reserve a run in every bucket, write  key << 32 | local
+//   scatter  per tile: bucket offsets of the batch (a scan of its bucket counts
+//            in LDS: the bucket ranges of a batch tile its range of the flat
+//            space exactly), reserve a run in every bucket, write
+//            key << 32 | local
 //   dedup    per bucket: LDS table with "smallest position wins" (64-bit
 //            atomicMin on the packed entry), then every entry writes the first
 //            position of its key into first[position]
-//   flag     streaming: position is a first occurrence <=> first[p] == local(p);
-//            one ballot bit per key + one count per tile; scan; unique_ptr
-//   fill     streaming: first occurrences write out_unique and their
-//            batch-local rank into rank[position]
-//   relabel  label of a position = rank[first[position]]: two gathers inside
-//            the batch's own range, which a die's L2 holds
+//   flag     streaming, one work-group per group of 4096 positions: position is
+//            a first occurrence <=> first[p] == local(p); per 64 positions one
+//            rank word (the ballot + the first occurrences of the group before
+//            it), per group one count
+//   offsets  one work-group: group counts -> group offsets; unique_ptr
+//   fill     streaming: first occurrences write out_unique
+//   relabel  label of a position = rank of its first occurrence = group offset
+//            + rank word of that position: two gathers in tables of N/4 bytes
+//            (80 KB per batch of 330 K keys), which a die's L2 holds
 // The result does not depend on the order in which entries land in a bucket, so
 // the atomics above leave it deterministic.  A bucket with more entries than the
 // LDS table is sure to hold (a hub that repeats thousands of times, a batch too
@@ -47,7 +50,6 @@
 
 namespace gs {
 
-constexpr int kWordsPerBlock = kBlock / kWave;
 constexpr int kXcds = 8;  // accelerator dies of an MI355X, each with its own L2
 
 constexpr int kPartItems = 16;                    // keys per thread and tile
@@ -95,6 +97,19 @@ struct alignas(16) BatchInfo {
 constexpr int kRelabelItems = 4;
 constexpr int kRelabelTile = kBlock * kRelabelItems;
 
+// First occurrences are counted per group of kGroup consecutive flat positions
+// (one work-group of the flag pass).  A rank word covers 64 positions: which of
+// them are first occurrences, and how many first occurrences the group has
+// before the word.
+constexpr int kGroupWords = 64;
+constexpr int kGroup = kGroupWords * kWave;
+constexpr int kWordsPerWave = kGroupWords / (kBlock / kWave);
+struct alignas(16) RankWord {
+  uint64_t bits;
+  uint32_t before;
+  uint32_t unused;
+};
+
 struct UniqueWs {
   BatchInfo* batch;       // [B]
   int64_t* flat_ptr;      // [B + 1] first flat position of a batch
@@ -102,20 +117,20 @@ struct UniqueWs {
   int64_t* bucket_ptr;    // [B + 1] first bucket of a batch
   int32_t* tile_batch;    // [max_tiles] batch of a tile, -1 past the last one
   int32_t* bucket_batch;  // [max_buckets] batch of a bucket, -1 past the last one
-  int32_t* chunk_batch;   // [chunks + 1] batch of the first position of a chunk
+  int32_t* group_batch;   // [groups + 1] batch of the first position of a group
   int32_t* etile_batch;   // [edge tiles + 1] batch of the first edge of a tile
   int64_t* bucket_cnt;    // [max_buckets + 1] entries per bucket
+  int64_t* bucket_cur;    // [max_buckets + 1] entries placed so far
   int* wide_keys;         // [1] set when some key does not fit the upper half of an entry
   int64_t* bucket_off;    // [max_buckets + 1] first entry of a bucket
   uint64_t* packed;       // [N] key << 32 | local, grouped by bucket
   uint32_t* first;        // [N] local position of the first occurrence
   uint64_t* spill;        // [2 N + max_buckets + 1] tables of oversize buckets
-  uint64_t* flags;        // [chunks * kWordsPerBlock] first-occurrence bits
-  int64_t* block_off;     // [chunks + 1]
-  int32_t* rank;          // [N] batch-local rank of a first occurrence, else -1
-  void* scan_ws;
-  size_t scan_ws_bytes;
-  int64_t max_tiles, max_buckets, chunks, etiles;
+  RankWord* words;        // [groups * kGroupWords]
+  int64_t* group_cnt;     // [groups] first occurrences per group
+  int64_t* group_off;     // [groups + 1] first occurrences before a group
+  int64_t* unique_ptr;    // [B + 1] copy of the caller's unique_ptr for the relabel pass
+  int64_t max_tiles, max_buckets, groups, etiles;
   size_t total;
 };
 
@@ -127,7 +142,7 @@ static UniqueWs carve_unique(void* ws, int64_t S, int64_t E, int64_t B) {
   // sum over batches of ceil(n_b / x) <= N / x + B
   w.max_tiles = N / kPartTile + B;
   w.max_buckets = N / tuning().bucket_keys + B;
-  w.chunks = ceil_div(n1, kBlock);
+  w.groups = ceil_div(n1, kGroup);
   w.etiles = ceil_div(E > 0 ? E : 1, kRelabelTile);
   w.batch = c.take<BatchInfo>((size_t)B);
   w.flat_ptr = c.take<int64_t>((size_t)B + 1);
@@ -135,19 +150,19 @@ static UniqueWs carve_unique(void* ws, int64_t S, int64_t E, int64_t B) {
   w.bucket_ptr = c.take<int64_t>((size_t)B + 1);
   w.tile_batch = c.take<int32_t>((size_t)w.max_tiles);
   w.bucket_batch = c.take<int32_t>((size_t)w.max_buckets);
-  w.chunk_batch = c.take<int32_t>((size_t)w.chunks + 1);
+  w.group_batch = c.take<int32_t>((size_t)w.groups + 1);
   w.etile_batch = c.take<int32_t>((size_t)w.etiles + 1);
   w.bucket_cnt = c.take<int64_t>((size_t)w.max_buckets + 1);
+  w.bucket_cur = c.take<int64_t>((size_t)w.max_buckets + 1);
   w.wide_keys = c.take<int>(1);
   w.bucket_off = c.take<int64_t>((size_t)w.max_buckets + 1);
   w.packed = c.take<uint64_t>((size_t)n1);
   w.first = c.take<uint32_t>((size_t)n1);
   w.spill = c.take<uint64_t>((size_t)(2 * n1 + w.max_buckets + 1));
-  w.flags = c.take<uint64_t>((size_t)w.chunks * kWordsPerBlock);
-  w.block_off = c.take<int64_t>((size_t)w.chunks + 1);
-  w.rank = c.take<int32_t>((size_t)n1);
-  w.scan_ws_bytes = scan_workspace_bytes(w.chunks + 1);
-  w.scan_ws = c.take<char>(w.scan_ws_bytes);
+  w.words = c.take<RankWord>((size_t)w.groups * kGroupWords);
+  w.group_cnt = c.take<int64_t>((size_t)w.groups);
+  w.group_off = c.take<int64_t>((size_t)w.groups + 1);
+  w.unique_ptr = c.take<int64_t>((size_t)B + 1);
   w.total = c.total();
   return w;
 }
@@ -186,20 +201,14 @@ __device__ __forceinline__ uint32_t slot_hash(uint64_t key) {
   return (uint32_t)((key * 0xC2B2AE3D27D4EB4Full) >> 29);
 }
 
-// ---------------------------------------------------------------- prep
-// Block 0 walks the batches; every block zeroes its share of the bucket
-// counters.
-__global__ __launch_bounds__(kBlock) void unique_prep_kernel(
-    Keys k, int64_t bucket_keys, BatchInfo* __restrict__ batch,
-    int64_t* __restrict__ flat_ptr, int64_t* __restrict__ tile_ptr,
-    int64_t* __restrict__ bucket_ptr, int64_t* __restrict__ bucket_cnt,
-    int64_t max_buckets, int* __restrict__ wide_keys) {
-  for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i <= max_buckets;
-       i += (int64_t)gridDim.x * kBlock)
-    bucket_cnt[i] = 0;
-  if (blockIdx.x != 0) return;
-  if (threadIdx.x == 0) *wide_keys = 0;
-  __shared__ int64_t smem[kBlock / kWave + 1];
+// ---------------------------------------------------------------- plan
+// The walk over the batches: where the keys, tiles and buckets of every batch
+// start.  Run by one whole work-group; the three offset arrays may live in LDS
+// or in global memory, `batch` (the records) may be null.
+__device__ __forceinline__ void walk_batches(const Keys& k, int64_t bucket_keys,
+                                             BatchInfo* batch, int64_t* flat_ptr,
+                                             int64_t* tile_ptr, int64_t* bucket_ptr,
+                                             int64_t* smem) {
   int64_t tile_carry = 0, bucket_carry = 0;
   for (int64_t base = 0; base <= k.B; base += kBlock) {
     const int64_t b = base + threadIdx.x;
@@ -229,44 +238,108 @@ __global__ __launch_bounds__(kBlock) void unique_prep_kernel(
       tile_ptr[b] = info.tile0;
       bucket_ptr[b] = info.bucket0;
     }
-    if (b < k.B) batch[b] = info;
+    if (batch && b < k.B) batch[b] = info;
   }
 }
 
-// ---------------------------------------------------------------- units
-// One search per tile, bucket, chunk of positions and tile of edges, all in
-// parallel here, instead of one at the start of every work-group later.
+// Unit i of the list (tiles, buckets, groups of positions, tiles of edges):
+// which batch it belongs to.  One search per unit here instead of one at the
+// start of every work-group later.
+struct UnitTables {
+  int64_t max_tiles, max_buckets, groups, etiles;
+  int32_t *tile_batch, *bucket_batch, *group_batch, *etile_batch;
+  __host__ __device__ int64_t units() const {
+    return max_tiles + max_buckets + groups + 1 + etiles + 1;
+  }
+};
+__device__ __forceinline__ void assign_unit(int64_t i, const Keys& k, int64_t N,
+                                            const int64_t* flat_ptr,
+                                            const int64_t* tile_ptr,
+                                            const int64_t* bucket_ptr,
+                                            const UnitTables& u) {
+  const int64_t B = k.B;
+  if (i < u.max_tiles) {
+    u.tile_batch[i] = i < tile_ptr[B] ? (int32_t)segment_of(tile_ptr, B, i) : -1;
+    return;
+  }
+  i -= u.max_tiles;
+  if (i < u.max_buckets) {
+    u.bucket_batch[i] = i < bucket_ptr[B] ? (int32_t)segment_of(bucket_ptr, B, i) : -1;
+    return;
+  }
+  i -= u.max_buckets;
+  if (i <= u.groups) {
+    int64_t p = i * kGroup;
+    if (p > N - 1) p = N - 1;
+    u.group_batch[i] = (int32_t)segment_of(flat_ptr, B, p);
+    return;
+  }
+  i -= u.groups + 1;
+  if (i <= u.etiles) {
+    int64_t e = i * kRelabelTile;
+    if (e > k.E - 1) e = k.E - 1;
+    u.etile_batch[i] =
+        (k.rows_ptr && k.E > 0) ? (int32_t)segment_of(k.rows_ptr, B, e) : 0;
+  }
+}
+
+__device__ __forceinline__ void zero_counters(int64_t* bucket_cnt, int64_t* bucket_cur,
+                                              int64_t max_buckets, int* wide_keys) {
+  for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i <= max_buckets;
+       i += (int64_t)gridDim.x * kBlock) {
+    bucket_cnt[i] = 0;
+    bucket_cur[i] = 0;
+  }
+  if (blockIdx.x == 0 && threadIdx.x == 0) *wide_keys = 0;
+}
+
+// Up to kPlanMaxBatches batches: every work-group walks the batches into LDS
+// (a few block scans) and then assigns its units from there; work-group 0 also
+// leaves the records and offset arrays in global memory.
+constexpr int kPlanMaxBatches = 1024;
+__global__ __launch_bounds__(kBlock) void unique_plan_kernel(
+    Keys k, int64_t N, int64_t bucket_keys, BatchInfo* __restrict__ batch,
+    int64_t* __restrict__ flat_ptr, int64_t* __restrict__ tile_ptr,
+    int64_t* __restrict__ bucket_ptr, int64_t* __restrict__ bucket_cnt,
+    int64_t* __restrict__ bucket_cur, int* __restrict__ wide_keys, UnitTables u) {
+  __shared__ int64_t l_flat[kPlanMaxBatches + 1];
+  __shared__ int64_t l_tile[kPlanMaxBatches + 1];
+  __shared__ int64_t l_bucket[kPlanMaxBatches + 1];
+  __shared__ int64_t smem[kBlock / kWave + 1];
+  zero_counters(bucket_cnt, bucket_cur, u.max_buckets, wide_keys);
+  walk_batches(k, bucket_keys, blockIdx.x == 0 ? batch : nullptr, l_flat, l_tile,
+               l_bucket, smem);
+  __syncthreads();
+  if (blockIdx.x == 0)
+    for (int64_t b = threadIdx.x; b <= k.B; b += kBlock) {
+      flat_ptr[b] = l_flat[b];
+      tile_ptr[b] = l_tile[b];
+      bucket_ptr[b] = l_bucket[b];
+    }
+  const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (i < u.units()) assign_unit(i, k, N, l_flat, l_tile, l_bucket, u);
+}
+
+// More batches than that: the walk by one work-group into global memory ...
+__global__ __launch_bounds__(kBlock) void unique_prep_kernel(
+    Keys k, int64_t bucket_keys, BatchInfo* __restrict__ batch,
+    int64_t* __restrict__ flat_ptr, int64_t* __restrict__ tile_ptr,
+    int64_t* __restrict__ bucket_ptr, int64_t* __restrict__ bucket_cnt,
+    int64_t* __restrict__ bucket_cur, int64_t max_buckets,
+    int* __restrict__ wide_keys) {
+  __shared__ int64_t smem[kBlock / kWave + 1];
+  zero_counters(bucket_cnt, bucket_cur, max_buckets, wide_keys);
+  if (blockIdx.x != 0) return;
+  walk_batches(k, bucket_keys, batch, flat_ptr, tile_ptr, bucket_ptr, smem);
+}
+
+// ... and the units from there in a launch of their own.
 __global__ __launch_bounds__(kBlock) void unique_units_kernel(
     Keys k, int64_t N, const int64_t* __restrict__ flat_ptr,
     const int64_t* __restrict__ tile_ptr, const int64_t* __restrict__ bucket_ptr,
-    int64_t max_tiles, int64_t max_buckets, int64_t chunks, int64_t etiles,
-    int32_t* __restrict__ tile_batch, int32_t* __restrict__ bucket_batch,
-    int32_t* __restrict__ chunk_batch, int32_t* __restrict__ etile_batch) {
-  int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
-  const int64_t B = k.B;
-  if (i < max_tiles) {
-    tile_batch[i] = i < tile_ptr[B] ? (int32_t)segment_of(tile_ptr, B, i) : -1;
-    return;
-  }
-  i -= max_tiles;
-  if (i < max_buckets) {
-    bucket_batch[i] = i < bucket_ptr[B] ? (int32_t)segment_of(bucket_ptr, B, i) : -1;
-    return;
-  }
-  i -= max_buckets;
-  if (i <= chunks) {
-    int64_t p = i * kBlock;
-    if (p > N - 1) p = N - 1;
-    chunk_batch[i] = (int32_t)segment_of(flat_ptr, B, p);
-    return;
-  }
-  i -= chunks + 1;
-  if (i <= etiles) {
-    int64_t e = i * kRelabelTile;
-    if (e > k.E - 1) e = k.E - 1;
-    etile_batch[i] =
-        (k.rows_ptr && k.E > 0) ? (int32_t)segment_of(k.rows_ptr, B, e) : 0;
-  }
+    UnitTables u) {
+  const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (i < u.units()) assign_unit(i, k, N, flat_ptr, tile_ptr, bucket_ptr, u);
 }
 
 // One partition tile: which batch, which keys.
@@ -339,48 +412,22 @@ __global__ __launch_bounds__(kBlock) void unique_hist_kernel(
   }
 }
 
-// Exclusive scan of the bucket counts by one work-group (there are about
-// N / 1500 of them).  off[total_buckets] = N closes the last bucket.
-constexpr int kBucketScanThreads = 1024;
-__global__ __launch_bounds__(kBucketScanThreads) void unique_bucket_scan_kernel(
-    const int64_t* __restrict__ bucket_ptr, int64_t B,
-    const int64_t* __restrict__ bucket_cnt, int64_t* __restrict__ bucket_off) {
-  __shared__ int64_t smem[kBucketScanThreads / kWave + 1];
-  const int64_t n = bucket_ptr[B] + 1;
-  int64_t carry = 0;
-  constexpr int kPer = 8;
-  for (int64_t base = 0; base < n; base += kBucketScanThreads * kPer) {
-    const int64_t i0 = base + (int64_t)threadIdx.x * kPer;
-    int64_t v[kPer], sum = 0;
-#pragma unroll
-    for (int j = 0; j < kPer; ++j) {
-      v[j] = i0 + j < n ? bucket_cnt[i0 + j] : 0;
-      sum += v[j];
-    }
-    int64_t total;
-    int64_t run = carry + block_exclusive_sum<int64_t, kBucketScanThreads>(
-                              sum, smem, &total);
-#pragma unroll
-    for (int j = 0; j < kPer; ++j) {
-      if (i0 + j < n) bucket_off[i0 + j] = run;
-      run += v[j];
-    }
-    carry += total;
-  }
-}
-
 // ---------------------------------------------------------------- scatter
-// bucket_cnt doubles as the reservation counter: a tile that brings c entries
-// to a bucket takes the c places below the counter's current value.  The tile
-// is first ordered by bucket in LDS so that every run leaves as one contiguous
-// write instead of one line per entry.
+// The buckets of a batch tile its range of the flat space in bucket order, so
+// every work-group gets the bucket offsets of its batch from a scan of the
+// batch's bucket counts in LDS (at most kMaxBuckets of them; the first tile of
+// a batch also leaves them in bucket_off for the dedup pass).  A tile that
+// brings c entries to a bucket takes the next c places at the bucket's cursor.
+// The tile is first ordered by bucket in LDS so that every run leaves as one
+// contiguous write instead of one line per entry.
 __global__ __launch_bounds__(kBlock) void unique_scatter_kernel(
     Keys k, const int32_t* __restrict__ tile_batch,
-    const BatchInfo* __restrict__ batch, int64_t* bucket_cnt,
-    const int64_t* __restrict__ bucket_off, uint64_t* __restrict__ packed,
-    uint32_t* __restrict__ first, int64_t max_tiles, int remap) {
+    const BatchInfo* __restrict__ batch, const int64_t* __restrict__ bucket_cnt,
+    int64_t* bucket_cur, int64_t* __restrict__ bucket_off,
+    uint64_t* __restrict__ packed, uint32_t* __restrict__ first, int64_t max_tiles,
+    int remap) {
   __shared__ uint32_t hist[kMaxBuckets];   // counts, then offsets inside the tile
-  __shared__ uint32_t run_at[kMaxBuckets]; // where the tile's run starts, relative to the batch
+  __shared__ uint32_t run_at[kMaxBuckets]; // first entry of the bucket, then of the tile's run in it, relative to the batch
   __shared__ uint64_t stage[kPartTile];
   __shared__ uint32_t scan_smem[kBlock / kWave + 1];
   const int64_t tile = unit_of_block(max_tiles, remap);
@@ -389,7 +436,9 @@ __global__ __launch_bounds__(kBlock) void unique_scatter_kernel(
   if (!tile_info(tile, tile_batch, batch, &t)) return;  // uniform per work-group
   const uint32_t buckets = (uint32_t)t.b.buckets;
   uint64_t* out = packed + t.b.fb;
+  const bool first_tile = tile == t.b.tile0;
   if (buckets == 1) {  // the bucket is the batch, in order
+    if (first_tile && threadIdx.x == 0) bucket_off[t.b.bucket0] = t.b.fb;
     for (int64_t l = t.begin + threadIdx.x; l < t.end; l += kBlock) {
       out[l] = ((uint64_t)key_tag(key_at(k, t.b, l)) << 32) | (uint64_t)l;
       first[t.b.fb + l] = (uint32_t)l;
@@ -406,7 +455,27 @@ __global__ __launch_bounds__(kBlock) void unique_scatter_kernel(
     const int64_t l = t.begin + i * kBlock + threadIdx.x;
     key[i] = (uint32_t)key_at(k, t.b, l < t.end ? l : t.end - 1);
   }
-  for (uint32_t i = threadIdx.x; i < buckets; i += kBlock) hist[i] = 0;
+  constexpr int kBins = kMaxBuckets / kBlock;
+  {
+    const uint32_t bin0 = threadIdx.x * kBins;
+    uint32_t c[kBins], sum = 0;
+#pragma unroll
+    for (int j = 0; j < kBins; ++j) {
+      c[j] = bin0 + j < buckets ? (uint32_t)bucket_cnt[t.b.bucket0 + bin0 + j] : 0u;
+      sum += c[j];
+    }
+    uint32_t total;
+    uint32_t run = block_exclusive_sum(sum, scan_smem, &total);
+#pragma unroll
+    for (int j = 0; j < kBins; ++j) {
+      if (bin0 + j < buckets) {
+        run_at[bin0 + j] = run;
+        hist[bin0 + j] = 0;
+        if (first_tile) bucket_off[t.b.bucket0 + bin0 + j] = t.b.fb + run;
+      }
+      run += c[j];
+    }
+  }
   __syncthreads();
 #pragma unroll
   for (int i = 0; i < kPartItems; ++i) {
@@ -423,7 +492,6 @@ __global__ __launch_bounds__(kBlock) void unique_scatter_kernel(
   __syncthreads();
   const uint32_t count = (uint32_t)(t.end - t.begin);
   {
-    constexpr int kBins = kMaxBuckets / kBlock;
     const uint32_t bin0 = threadIdx.x * kBins;
     uint32_t c[kBins], sum = 0;
 #pragma unroll
@@ -443,12 +511,9 @@ __global__ __launch_bounds__(kBlock) void unique_scatter_kernel(
   // one bin per thread and round: the reservations of a round are in flight together
   for (uint32_t bin = threadIdx.x; bin < buckets; bin += kBlock) {
     const uint32_t c = (bin + 1 < buckets ? hist[bin + 1] : count) - hist[bin];
-    if (c) {
-      const int64_t g = t.b.bucket0 + bin;
-      const int64_t before = (int64_t)atomicAdd(
-          (unsigned long long*)&bucket_cnt[g], (unsigned long long)(-(int64_t)c));
-      run_at[bin] = (uint32_t)(bucket_off[g] - t.b.fb + before - c);
-    }
+    if (c)
+      run_at[bin] += (uint32_t)atomicAdd((unsigned long long*)&bucket_cur[t.b.bucket0 + bin],
+                                         (unsigned long long)c);
   }
   __syncthreads();
 #pragma unroll
@@ -689,9 +754,9 @@ template <int kThreads>
 __global__ __launch_bounds__(kThreads) void unique_dedup_kernel(
     Keys k, const int* __restrict__ wide_keys,
     const int32_t* __restrict__ bucket_batch, const BatchInfo* __restrict__ batch,
-    const int64_t* __restrict__ bucket_off, const uint64_t* __restrict__ packed,
-    uint64_t* spill, uint32_t* __restrict__ first, int64_t max_buckets,
-    int remap) {
+    const int64_t* __restrict__ bucket_cnt, const int64_t* __restrict__ bucket_off,
+    const uint64_t* __restrict__ packed, uint64_t* spill, uint32_t* __restrict__ first,
+    int64_t max_buckets, int remap) {
   __shared__ uint64_t tab[kLdsSlots];
   __shared__ uint32_t distinct;
   __shared__ uint32_t overflow;
@@ -699,7 +764,7 @@ __global__ __launch_bounds__(kThreads) void unique_dedup_kernel(
   if (g >= max_buckets) return;
   const int32_t b = bucket_batch[g];
   if (b < 0) return;  // uniform per work-group
-  const int64_t lo = bucket_off[g], hi = bucket_off[g + 1];
+  const int64_t lo = bucket_off[g], hi = lo + bucket_cnt[g];
   if (hi == lo) return;
   const BatchInfo info = batch[b];
   if (*wide_keys)
@@ -711,18 +776,14 @@ __global__ __launch_bounds__(kThreads) void unique_dedup_kernel(
 }
 
 // ---------------------------------------------------------------- flag
-// The streaming passes below work in chunks of kBlock consecutive positions,
-// one chunk per wave at a time, lane l taking positions l, l + 64, ...: four
-// coalesced rows whose ballots are the chunk's four flag words.
-
 // A value that is the same in every lane, moved to scalar registers so that
 // what is computed from it (the batch search) runs on the scalar unit.
 __device__ __forceinline__ int64_t wave_uniform(int64_t v) {
   return wave_uniform_first(v);
 }
 
-// Batches that a chunk of consecutive items may touch: from the batch of its
-// first item to the batch of the next chunk's first item.
+// Batches that a run of consecutive items may touch: from the batch of its
+// first item to the batch of the next run's first item.
 struct BatchSpan {
   int64_t lo, hi;
 };
@@ -735,116 +796,154 @@ __device__ __forceinline__ int64_t batch_in_span(const int64_t* __restrict__ ptr
   return s.lo == s.hi ? s.lo : s.lo + segment_of(ptr + s.lo, s.hi - s.lo + 1, x);
 }
 
-constexpr int kChunksPerWave = 4;
-
+// One work-group per group of kGroup positions; a wave takes kWordsPerWave
+// consecutive words, lane l the positions l, l + 64, ...: coalesced rows whose
+// ballots are the words.
 __global__ __launch_bounds__(kBlock) void unique_flag_kernel(
-    const int64_t* __restrict__ flat_ptr, const int32_t* __restrict__ chunk_batch,
-    int64_t N, const uint32_t* __restrict__ first, uint64_t* __restrict__ flags,
-    int64_t* __restrict__ block_count) {
-  const int64_t num_chunks = ceil_div_dev(N, kBlock);
-  const int64_t wave = (int64_t)blockIdx.x * kWordsPerBlock + threadIdx.x / kWave;
-  const int lane = lane_id();
-  for (int c = 0; c < kChunksPerWave; ++c) {
-    const int64_t chunk = wave_uniform(wave * kChunksPerWave + c);
-    if (chunk >= num_chunks) return;
-    const int64_t p0 = chunk * kBlock;
-    const BatchSpan span = batch_span(chunk_batch, chunk);
-    uint32_t f[kWordsPerBlock];
+    const int64_t* __restrict__ flat_ptr, const int32_t* __restrict__ group_batch,
+    int64_t N, const uint32_t* __restrict__ first, RankWord* __restrict__ words,
+    int64_t* __restrict__ group_cnt) {
+  __shared__ uint32_t wave_total[kBlock / kWave];
+  const int64_t group = blockIdx.x;
+  const int wave = threadIdx.x / kWave, lane = lane_id();
+  const int64_t word0 = group * kGroupWords + wave * kWordsPerWave;
+  const int64_t p0 = word0 * kWave;
+  const BatchSpan span = batch_span(group_batch, group);
+  const int64_t fb_lo = flat_ptr[span.lo];
+  uint32_t f[kWordsPerWave];
 #pragma unroll
-    for (int j = 0; j < kWordsPerBlock; ++j) {
-      const int64_t p = p0 + j * kWave + lane;
-      f[j] = p < N ? first[p] : 0u;
-    }
-    uint64_t word[kWordsPerBlock];
+  for (int j = 0; j < kWordsPerWave; ++j) {
+    const int64_t p = p0 + j * kWave + lane;
+    f[j] = p < N ? first[p] : 0u;
+  }
+  uint64_t my_bits = 0;
+  uint32_t my_before = 0, total = 0;
 #pragma unroll
-    for (int j = 0; j < kWordsPerBlock; ++j) {
-      const int64_t p = p0 + j * kWave + lane;
-      bool is_first = false;
-      if (p < N)
-        is_first = (int64_t)f[j] == p - flat_ptr[batch_in_span(flat_ptr, span, p)];
-      word[j] = __ballot(is_first);
+  for (int j = 0; j < kWordsPerWave; ++j) {
+    const int64_t p = p0 + j * kWave + lane;
+    bool is_first = false;
+    if (p < N) {
+      const int64_t fb =
+          span.lo == span.hi ? fb_lo : flat_ptr[batch_in_span(flat_ptr, span, p)];
+      is_first = (int64_t)f[j] == p - fb;
     }
-    if (lane == 0) {
-      int total = 0;
+    const uint64_t bits = __ballot(is_first);
+    if (lane == j) {
+      my_bits = bits;
+      my_before = total;
+    }
+    total += (uint32_t)__popcll(bits);
+  }
+  if (lane == 0) wave_total[wave] = total;
+  __syncthreads();
+  uint32_t base = 0, all = 0;
 #pragma unroll
-      for (int j = 0; j < kWordsPerBlock; ++j) {
-        flags[chunk * kWordsPerBlock + j] = word[j];
-        total += __popcll(word[j]);
-      }
-      block_count[chunk] = total;
-      if (chunk == num_chunks - 1) block_count[num_chunks] = 0;
+  for (int w = 0; w < kBlock / kWave; ++w) {
+    const uint32_t t = wave_total[w];
+    if (w < wave) base += t;
+    all += t;
+  }
+  if (lane < kWordsPerWave && (word0 + lane) * kWave < N)
+    words[word0 + lane] = RankWord{my_bits, base + my_before, 0u};
+  if (threadIdx.x == 0) group_cnt[group] = (int64_t)all;
+}
+
+// Number of first occurrences at flat positions < p, for p < N.
+__device__ __forceinline__ int64_t rank_of(int64_t p, const RankWord* __restrict__ words,
+                                           const int64_t* __restrict__ group_off) {
+  const RankWord w = words[p / kWave];
+  const int bit = (int)(p % kWave);
+  return group_off[p / kGroup] + w.before +
+         __popcll(w.bits & ((1ull << bit) - 1ull));
+}
+
+// ---------------------------------------------------------------- offsets
+// One work-group: group counts -> group offsets (group_off[groups] = number of
+// unique keys), then where the unique keys of every batch start.  The offsets
+// also go to unique_ptr_mirror when that is given (pinned host memory, so that
+// the host has them without a copy of its own).
+constexpr int kOffsetsThreads = 1024;
+__global__ __launch_bounds__(kOffsetsThreads) void unique_offsets_kernel(
+    const int64_t* __restrict__ flat_ptr, int64_t B, int64_t N, int64_t groups,
+    const int64_t* __restrict__ group_cnt, int64_t* group_off,
+    const RankWord* __restrict__ words, int64_t* __restrict__ unique_ptr,
+    int64_t* __restrict__ unique_ptr_ws, int64_t* unique_ptr_mirror) {
+  __shared__ int64_t smem[kOffsetsThreads / kWave + 1];
+  int64_t carry = 0;
+  constexpr int kPer = 8;
+  for (int64_t base = 0; base < groups; base += kOffsetsThreads * kPer) {
+    const int64_t i0 = base + (int64_t)threadIdx.x * kPer;
+    int64_t v[kPer], sum = 0;
+#pragma unroll
+    for (int j = 0; j < kPer; ++j) {
+      v[j] = i0 + j < groups ? group_cnt[i0 + j] : 0;
+      sum += v[j];
     }
+    int64_t total;
+    int64_t run = carry + block_exclusive_sum<int64_t, kOffsetsThreads>(sum, smem, &total);
+#pragma unroll
+    for (int j = 0; j < kPer; ++j) {
+      if (i0 + j < groups) group_off[i0 + j] = run;
+      run += v[j];
+    }
+    carry += total;
+  }
+  if (threadIdx.x == 0) group_off[groups] = carry;
+  __threadfence();
+  __syncthreads();
+  for (int64_t b = threadIdx.x; b <= B; b += kOffsetsThreads) {
+    const int64_t p = flat_ptr[b];
+    int64_t r = carry;
+    if (p < N) {
+      const RankWord w = words[p / kWave];
+      // written above by other threads of this work-group: read past the
+      // compute unit's own cache
+      const int64_t off = __hip_atomic_load(group_off + p / kGroup, __ATOMIC_RELAXED,
+                                            __HIP_MEMORY_SCOPE_AGENT);
+      r = off + w.before + __popcll(w.bits & ((1ull << (int)(p % kWave)) - 1ull));
+    }
+    unique_ptr[b] = r;
+    unique_ptr_ws[b] = r;
+    if (unique_ptr_mirror) unique_ptr_mirror[b] = r;
   }
 }
 
-// Number of first occurrences at flat positions < p.
-__device__ __forceinline__ int64_t rank_before(
-    int64_t p, const uint64_t* __restrict__ flags,
-    const int64_t* __restrict__ block_off) {
-  const int64_t blk = p / kBlock;
-  int64_t r = block_off[blk];
-  const int in_blk = (int)(p - blk * kBlock);
-  const int full = in_blk / kWave, rem = in_blk % kWave;
-  for (int w = 0; w < full; ++w)
-    r += __popcll(flags[blk * kWordsPerBlock + w]);
-  if (rem)
-    r += __popcll(flags[blk * kWordsPerBlock + full] & ((1ull << rem) - 1));
-  return r;
-}
-
-__global__ void unique_ptr_kernel(const int64_t* __restrict__ flat_ptr,
-                                  int64_t B, const uint64_t* __restrict__ flags,
-                                  const int64_t* __restrict__ block_off,
-                                  int64_t* __restrict__ unique_ptr) {
-  const int64_t b = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (b > B) return;
-  unique_ptr[b] = rank_before(flat_ptr[b], flags, block_off);
-}
-
 // ---------------------------------------------------------------- fill
-// Streaming: every position writes its rank (or -1); first occurrences also
-// write their key to the frontier.
+// Streaming: first occurrences write their key to the frontier.  A wave reads
+// the keys of its kWordsPerWave rows of 64 positions in one go (whole rows:
+// about half of the positions are first occurrences, so every line is needed
+// anyway) and then stores the flagged ones.
 __global__ __launch_bounds__(kBlock) void unique_fill_kernel(
     Keys k, const int64_t* __restrict__ flat_ptr,
-    const int32_t* __restrict__ chunk_batch, const BatchInfo* __restrict__ batch,
-    int64_t N, const uint64_t* __restrict__ flags,
-    const int64_t* __restrict__ block_off, const int64_t* __restrict__ unique_ptr,
-    int64_t* __restrict__ out_unique, int32_t* __restrict__ rank) {
-  const int64_t num_chunks = ceil_div_dev(N, kBlock);
-  const int64_t wave = (int64_t)blockIdx.x * kWordsPerBlock + threadIdx.x / kWave;
-  const int lane = lane_id();
-  for (int c = 0; c < kChunksPerWave; ++c) {
-    const int64_t chunk = wave_uniform(wave * kChunksPerWave + c);
-    if (chunk >= num_chunks) return;
-    const int64_t p0 = chunk * kBlock;
-    const BatchSpan span = batch_span(chunk_batch, chunk);
-    int64_t before = block_off[chunk];
-    uint64_t word[kWordsPerBlock];
+    const int32_t* __restrict__ group_batch, const BatchInfo* __restrict__ batch,
+    int64_t N, const RankWord* __restrict__ words,
+    const int64_t* __restrict__ group_off, int64_t* __restrict__ out_unique) {
+  const int64_t group = blockIdx.x;
+  const int wave = threadIdx.x / kWave, lane = lane_id();
+  const int64_t word0 = group * kGroupWords + wave * kWordsPerWave;
+  if (wave_uniform(word0 * kWave) >= N) return;
+  const BatchSpan span = batch_span(group_batch, group);
+  const bool one_batch = span.lo == span.hi;
+  BatchInfo info = batch[span.lo];
+  RankWord mine{0ull, 0u, 0u};  // lane j holds word j of this wave
+  if (lane < kWordsPerWave && (word0 + lane) * kWave < N) mine = words[word0 + lane];
+  int64_t* out = out_unique + group_off[group];
+  uint64_t key[kWordsPerWave];
 #pragma unroll
-    for (int j = 0; j < kWordsPerBlock; ++j)
-      word[j] = flags[chunk * kWordsPerBlock + j];
-    BatchInfo info = batch[span.lo];
-    int64_t rank0 = unique_ptr[span.lo];
-#pragma unroll
-    for (int j = 0; j < kWordsPerBlock; ++j) {
-      const int64_t p = p0 + j * kWave + lane;
-      if (p < N) {
-        int32_t r = -1;
-        if ((word[j] >> lane) & 1ull) {
-          if (span.lo != span.hi) {  // the chunk straddles batches
-            const int64_t b = batch_in_span(flat_ptr, span, p);
-            info = batch[b];
-            rank0 = unique_ptr[b];
-          }
-          const uint64_t key = key_at(k, info, p - info.fb);
-          const int64_t grank = before + __popcll(word[j] & ((1ull << lane) - 1));
-          out_unique[grank] = (int64_t)key;
-          r = (int32_t)(grank - rank0);
-        }
-        rank[p] = r;
-      }
-      before += __popcll(word[j]);
+  for (int j = 0; j < kWordsPerWave; ++j) {
+    const int64_t p = (word0 + j) * kWave + lane;
+    key[j] = 0;
+    if (p < N) {
+      if (!one_batch) info = batch[batch_in_span(flat_ptr, span, p)];
+      key[j] = key_at(k, info, p - info.fb);
     }
+  }
+#pragma unroll
+  for (int j = 0; j < kWordsPerWave; ++j) {
+    const uint64_t bits = __shfl((unsigned long long)mine.bits, j, kWave);
+    const uint32_t before = __shfl(mine.before, j, kWave);
+    if ((bits >> lane) & 1ull)
+      out[before + __popcll(bits & ((1ull << lane) - 1ull))] = (int64_t)key[j];
   }
 }
 
@@ -852,7 +951,8 @@ __global__ __launch_bounds__(kBlock) void unique_fill_kernel(
 __global__ __launch_bounds__(kBlock) void unique_relabel_kernel(
     Keys k, const int32_t* __restrict__ etile_batch,
     const BatchInfo* __restrict__ batch, const uint32_t* __restrict__ first,
-    const int32_t* __restrict__ rank, const int64_t* __restrict__ edge_col,
+    const RankWord* __restrict__ words, const int64_t* __restrict__ group_off,
+    const int64_t* __restrict__ unique_ptr, const int64_t* __restrict__ edge_col,
     int64_t* __restrict__ out_row, int64_t* __restrict__ out_col, int remap) {
   const int64_t num_tiles = ceil_div_dev(k.E, kRelabelTile);
   const int64_t tile = unit_of_block(num_tiles, remap);
@@ -862,12 +962,16 @@ __global__ __launch_bounds__(kBlock) void unique_relabel_kernel(
   int64_t col[kRelabelItems];
   uint32_t row_first[kRelabelItems];
   BatchInfo info = batch[span.lo];
+  int64_t rank0 = unique_ptr[span.lo];
   // Seeds of a batch are distinct <=> its last seed is a first occurrence of
   // rank ns - 1; the label of seed c is then its place among the seeds.
   const bool one_batch = span.lo == span.hi;
   bool seeds_distinct = false;
-  if (one_batch && out_col && info.ns > 0)
-    seeds_distinct = rank[info.fb + info.ns - 1] == (int32_t)(info.ns - 1);
+  if (one_batch && out_col && info.ns > 0) {
+    const int64_t q = info.fb + info.ns - 1;
+    seeds_distinct = ((words[q / kWave].bits >> (int)(q % kWave)) & 1ull) &&
+                     rank_of(q, words, group_off) - rank0 == info.ns - 1;
+  }
 #pragma unroll
   for (int i = 0; i < kRelabelItems; ++i) {
     const int64_t e = e0 + i * kBlock + threadIdx.x;
@@ -882,13 +986,27 @@ __global__ __launch_bounds__(kBlock) void unique_relabel_kernel(
   for (int i = 0; i < kRelabelItems; ++i) {
     const int64_t e = e0 + i * kBlock + threadIdx.x;
     if (e >= k.E) break;
-    if (!one_batch) info = batch[batch_in_span(k.rows_ptr, span, e)];
-    if (out_row) out_row[e] = rank[info.fb + row_first[i]];
+    if (!one_batch) {
+      const int64_t b = batch_in_span(k.rows_ptr, span, e);
+      info = batch[b];
+      rank0 = unique_ptr[b];
+    }
+    if (out_row) out_row[e] = rank_of(info.fb + row_first[i], words, group_off) - rank0;
     // seed c of batch b sits at flat position c + rows_ptr[b]
     if (out_col)
-      out_col[e] = seeds_distinct ? col[i] - info.s_lo
-                                  : rank[info.fb + first[col[i] + info.r_lo]];
+      out_col[e] = seeds_distinct
+                       ? col[i] - info.s_lo
+                       : rank_of(info.fb + first[col[i] + info.r_lo], words, group_off) - rank0;
   }
+}
+
+// No keys at all: every batch is empty.
+__global__ __launch_bounds__(kBlock) void unique_empty_kernel(
+    int64_t* __restrict__ unique_ptr, int64_t* unique_ptr_mirror, int64_t n) {
+  const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (i >= n) return;
+  unique_ptr[i] = 0;
+  if (unique_ptr_mirror) unique_ptr_mirror[i] = 0;
 }
 
 static int check_unique_args(const int64_t* seeds, const int64_t* seeds_ptr,
@@ -930,7 +1048,8 @@ size_t gs_unique_workspace_bytes(int64_t num_seeds, int64_t num_rows_keys,
 int gs_unique_count(const int64_t* seeds, const int64_t* seeds_ptr,
                     int64_t num_seeds, const int64_t* rows,
                     const int64_t* rows_ptr, int64_t num_rows_keys,
-                    int64_t num_batches, int64_t* unique_ptr, void* workspace,
+                    int64_t num_batches, int64_t* unique_ptr,
+                    int64_t* unique_ptr_mirror, void* workspace,
                     size_t workspace_bytes, gs_stream_t stream) {
   using namespace gs;
   const int64_t S = num_seeds, E = num_rows_keys, B = num_batches;
@@ -943,66 +1062,61 @@ int gs_unique_count(const int64_t* seeds, const int64_t* seeds_ptr,
   const UniqueTuning tn = tuning();
   const int64_t N = S + E;
   if (N == 0) {
-    GS_LAUNCH("unique_prep", s,
-              table_fill_kernel<><<<dim3((unsigned)ceil_div(B + 1, kBlock)),
-                                    dim3(kBlock), 0, s>>>((uint64_t*)unique_ptr,
-                                                          B + 1, 0ull));
+    GS_LAUNCH("unique_plan", s,
+              unique_empty_kernel<<<dim3((unsigned)ceil_div(B + 1, kBlock)),
+                                    dim3(kBlock), 0, s>>>(unique_ptr,
+                                                          unique_ptr_mirror, B + 1));
     return GS_OK;
   }
   const Keys k{seeds, seeds_ptr, S, rows, rows_ptr, E, B};
-  const int64_t nblocks = w.chunks;
-  {
+  const UnitTables units{w.max_tiles, w.max_buckets, w.groups,      w.etiles,
+                         w.tile_batch, w.bucket_batch, w.group_batch, w.etile_batch};
+  const dim3 unit_grid((unsigned)ceil_div(units.units(), kBlock));
+  if (B <= kPlanMaxBatches) {
+    GS_LAUNCH("unique_plan", s,
+              unique_plan_kernel<<<unit_grid, dim3(kBlock), 0, s>>>(
+                  k, N, tn.bucket_keys, w.batch, w.flat_ptr, w.tile_ptr, w.bucket_ptr,
+                  w.bucket_cnt, w.bucket_cur, w.wide_keys, units));
+  } else {
     int64_t blocks = ceil_div(w.max_buckets + 1, kBlock * 4);
     if (blocks > 1024) blocks = 1024;
-    GS_LAUNCH("unique_prep", s,
+    GS_LAUNCH("unique_plan", s,
               unique_prep_kernel<<<dim3((unsigned)blocks), dim3(kBlock), 0, s>>>(
                   k, tn.bucket_keys, w.batch, w.flat_ptr, w.tile_ptr,
-                  w.bucket_ptr, w.bucket_cnt, w.max_buckets, w.wide_keys));
-    const int64_t units = w.max_tiles + w.max_buckets + w.chunks + 1 + w.etiles + 1;
+                  w.bucket_ptr, w.bucket_cnt, w.bucket_cur, w.max_buckets, w.wide_keys));
     GS_LAUNCH("unique_units", s,
-              unique_units_kernel<<<dim3((unsigned)ceil_div(units, kBlock)),
-                                    dim3(kBlock), 0, s>>>(
-                  k, N, w.flat_ptr, w.tile_ptr, w.bucket_ptr, w.max_tiles,
-                  w.max_buckets, w.chunks, w.etiles, w.tile_batch,
-                  w.bucket_batch, w.chunk_batch, w.etile_batch));
+              unique_units_kernel<<<unit_grid, dim3(kBlock), 0, s>>>(
+                  k, N, w.flat_ptr, w.tile_ptr, w.bucket_ptr, units));
   }
   const dim3 tile_grid((unsigned)grid_for_units(w.max_tiles, tn.remap));
   GS_LAUNCH("unique_hist", s,
             unique_hist_kernel<<<tile_grid, dim3(kBlock), 0, s>>>(
                 k, w.tile_batch, w.batch, w.bucket_cnt, w.max_tiles, tn.remap,
                 w.wide_keys));
-  GS_LAUNCH("unique_bucket_scan", s,
-            unique_bucket_scan_kernel<<<dim3(1), dim3(kBucketScanThreads), 0, s>>>(
-                w.bucket_ptr, B, w.bucket_cnt, w.bucket_off));
   GS_LAUNCH("unique_scatter", s,
             unique_scatter_kernel<<<tile_grid, dim3(kBlock), 0, s>>>(
-                k, w.tile_batch, w.batch, w.bucket_cnt, w.bucket_off, w.packed, w.first,
-                w.max_tiles, tn.remap));
+                k, w.tile_batch, w.batch, w.bucket_cnt, w.bucket_cur, w.bucket_off,
+                w.packed, w.first, w.max_tiles, tn.remap));
   GS_LAUNCH("unique_dedup", s,
             if (tn.dedup_threads == 512)
               unique_dedup_kernel<512><<<dim3((unsigned)grid_for_units(
                                              w.max_buckets, tn.remap)),
                                          dim3(512), 0, s>>>(
-                  k, w.wide_keys, w.bucket_batch, w.batch, w.bucket_off, w.packed, w.spill,
-                  w.first, w.max_buckets, tn.remap);
+                  k, w.wide_keys, w.bucket_batch, w.batch, w.bucket_cnt, w.bucket_off,
+                  w.packed, w.spill, w.first, w.max_buckets, tn.remap);
             else
               unique_dedup_kernel<256><<<dim3((unsigned)grid_for_units(
                                              w.max_buckets, tn.remap)),
                                          dim3(256), 0, s>>>(
-                  k, w.wide_keys, w.bucket_batch, w.batch, w.bucket_off, w.packed, w.spill,
-                  w.first, w.max_buckets, tn.remap));
+                  k, w.wide_keys, w.bucket_batch, w.batch, w.bucket_cnt, w.bucket_off,
+                  w.packed, w.spill, w.first, w.max_buckets, tn.remap));
   GS_LAUNCH("unique_flag", s,
-            unique_flag_kernel<<<dim3((unsigned)ceil_div(
-                                     nblocks, kWordsPerBlock * kChunksPerWave)),
-                                 dim3(kBlock), 0, s>>>(
-                w.flat_ptr, w.chunk_batch, N, w.first, w.flags, w.block_off));
-  rc = exclusive_scan_i64(w.block_off, w.block_off, nblocks + 1, w.scan_ws,
-                          w.scan_ws_bytes, s);
-  if (rc != GS_OK) return rc;
-  GS_LAUNCH("unique_ptr", s,
-            unique_ptr_kernel<<<dim3((unsigned)ceil_div(B + 1, kBlock)),
-                                dim3(kBlock), 0, s>>>(w.flat_ptr, B, w.flags,
-                                                      w.block_off, unique_ptr));
+            unique_flag_kernel<<<dim3((unsigned)w.groups), dim3(kBlock), 0, s>>>(
+                w.flat_ptr, w.group_batch, N, w.first, w.words, w.group_cnt));
+  GS_LAUNCH("unique_offsets", s,
+            unique_offsets_kernel<<<dim3(1), dim3(kOffsetsThreads), 0, s>>>(
+                w.flat_ptr, B, N, w.groups, w.group_cnt, w.group_off, w.words,
+                unique_ptr, w.unique_ptr, unique_ptr_mirror));
   return GS_OK;
 }
 
@@ -1025,12 +1139,9 @@ int gs_unique_fill(const int64_t* seeds, const int64_t* seeds_ptr,
   hipStream_t s = as_stream(stream);
   const Keys k{seeds, seeds_ptr, S, rows, rows_ptr, E, B};
   GS_LAUNCH("unique_fill", s,
-            unique_fill_kernel<<<dim3((unsigned)ceil_div(
-                                     ceil_div(N, kBlock),
-                                     kWordsPerBlock * kChunksPerWave)),
-                                 dim3(kBlock), 0, s>>>(
-                k, w.flat_ptr, w.chunk_batch, w.batch, N, w.flags, w.block_off,
-                unique_ptr, out_unique, w.rank));
+            unique_fill_kernel<<<dim3((unsigned)w.groups), dim3(kBlock), 0, s>>>(
+                k, w.flat_ptr, w.group_batch, w.batch, N, w.words, w.group_off,
+                out_unique));
   return GS_OK;
 }
 
@@ -1056,8 +1167,8 @@ int gs_unique_relabel(const int64_t* seeds, const int64_t* seeds_ptr,
               unique_relabel_kernel<<<dim3((unsigned)grid_for_units(
                                           ceil_div(E, kRelabelTile), tn.remap)),
                                       dim3(kBlock), 0, s>>>(
-                  k, w.etile_batch, w.batch, w.first, w.rank, edge_col, out_row,
-                  out_col, tn.remap));
+                  k, w.etile_batch, w.batch, w.first, w.words, w.group_off,
+                  w.unique_ptr, edge_col, out_row, out_col, tn.remap));
   }
   return GS_OK;
 }

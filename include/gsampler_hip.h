@@ -108,7 +108,10 @@ int gs_exclusive_scan_i64(const int64_t* in, int64_t* out, int64_t n,
  *   fanout < 0         : whole column (slicing).
  *   replace            : count = degree == 0 ? 0 : fanout, else min(degree, fanout).
  * Column ids outside [0, num_cols) count as empty columns.
- * Writes sub_indptr[num_items + 1]; sub_indptr[num_items] is the edge total.
+ * Writes sub_indptr[num_items + 1]; sub_indptr[num_items] is the edge total,
+ * which the kernel that produces it also stores to *total_mirror when that is
+ * given (a word of pinned host memory: the host then has the total as soon as
+ * the stream reaches that point, without a copy of its own).
  * Stands in for the degree lambda + scan of
  *   src/cuda/slicing.cu:133-141, src/cuda/sampling.cu:112-124,
  *   src/cuda/fusion/slice_sampling.cu:111-124, src/cuda/sampling_probs.cu:201-216.
@@ -117,8 +120,8 @@ int gs_exclusive_scan_i64(const int64_t* in, int64_t* out, int64_t n,
 int gs_csc_col_count(const int64_t* indptr, int64_t num_cols,
                      const int64_t* column_ids, int64_t num_items,
                      int64_t fanout, int replace, int64_t* sub_indptr,
-                     void* workspace, size_t workspace_bytes,
-                     gs_stream_t stream);
+                     int64_t* total_mirror, void* workspace,
+                     size_t workspace_bytes, gs_stream_t stream);
 
 /* ------------------------------------------------------------------------
  * gs_csc_col_count for callers that cannot allocate device memory (code under
@@ -282,10 +285,12 @@ int gs_list_sample_weighted_fill(const float* probs, const int64_t* range,
  *
  * count: finds the first occurrence of every key (state kept inside the
  *   workspace) and writes unique_ptr[num_batches + 1] (number of unique keys
- *   before each batch; the last element is the total U).
+ *   before each batch; the last element is the total U), and the same values
+ *   to unique_ptr_mirror[num_batches + 1] when that is given (pinned host
+ *   memory: the host then has the offsets without a copy of its own).
  * fill:  same arguments + the same workspace, untouched in between; writes
- *   out_unique[U] and the rank of every first occurrence into the workspace.
- * relabel: after fill, same workspace; out_row[num_rows_keys] = batch-local
+ *   out_unique[U].
+ * relabel: after count, same workspace; out_row[num_rows_keys] = batch-local
  *   rank of every row key (nullable); out_col[num_rows_keys] = batch-local rank
  *   of seeds[edge_col[e]] (nullable; edge_col holds positions into `seeds`).
  *   May be called any number of times while the workspace is kept.
@@ -304,7 +309,8 @@ size_t gs_unique_workspace_bytes(int64_t num_seeds, int64_t num_rows_keys,
 int gs_unique_count(const int64_t* seeds, const int64_t* seeds_ptr,
                     int64_t num_seeds, const int64_t* rows,
                     const int64_t* rows_ptr, int64_t num_rows_keys,
-                    int64_t num_batches, int64_t* unique_ptr, void* workspace,
+                    int64_t num_batches, int64_t* unique_ptr,
+                    int64_t* unique_ptr_mirror, void* workspace,
                     size_t workspace_bytes, gs_stream_t stream);
 int gs_unique_fill(const int64_t* seeds, const int64_t* seeds_ptr,
                    int64_t num_seeds, const int64_t* rows,

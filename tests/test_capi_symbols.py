@@ -44,5 +44,5 @@ def test_argument_errors_are_reported_without_a_gpu():
     rc = l.gs_csc_col_sample_uniform_fill(None, 0, None, None, 0, 100, 0, 2, 0, 0,
                                           None, None, None, None, None)
     assert rc == 1 and b"Floyd" in l.gs_last_error()
-    rc = l.gs_unique_count(None, None, 0, None, None, 0, 0, None, None, 0, None)
+    rc = l.gs_unique_count(None, None, 0, None, None, 0, 0, None, None, None, 0, None)
     assert rc == 1
