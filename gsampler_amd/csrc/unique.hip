@@ -58,16 +58,14 @@ constexpr int kMaxBuckets = 2048;                 // buckets per batch (LDS bins
 constexpr int kLdsSlots = 4096;                   // dedup table, 32 KB of LDS
 constexpr int kLdsMaxEntries = kLdsSlots * 3 / 4; // bucket sizes the LDS table takes
 
-// Average entries per bucket, threads of a dedup work-group and whether
-// work-groups are laid out per die: the best of a sweep on 21M keys in 64
-// batches (bucket sizes 512..3072, 256 or 512 threads, with and without the
-// per-die layout).
+// Average entries per bucket and whether work-groups are laid out per die: the
+// best of a sweep on 21M keys in 64 batches (bucket sizes 512..3072, with and
+// without the per-die layout).
 struct UniqueTuning {
   int64_t bucket_keys;
   int remap;
-  int dedup_threads;
 };
-static UniqueTuning tuning() { return UniqueTuning{1536, 1, 512}; }
+static UniqueTuning tuning() { return UniqueTuning{1536, 1}; }
 
 // Work-group index -> unit of work (tile or bucket).  Consecutive work-groups
 // go to consecutive dies, so die x is given the x-th eighth of the units, in
@@ -508,20 +506,32 @@ __global__ __launch_bounds__(kBlock) void unique_scatter_kernel(
     }
   }
   __syncthreads();
-  // one bin per thread and round: the reservations of a round are in flight together
-  for (uint32_t bin = threadIdx.x; bin < buckets; bin += kBlock) {
-    const uint32_t c = (bin + 1 < buckets ? hist[bin + 1] : count) - hist[bin];
-    if (c)
-      run_at[bin] += (uint32_t)atomicAdd((unsigned long long*)&bucket_cur[t.b.bucket0 + bin],
-                                         (unsigned long long)c);
+  // One bin per thread and round; all reservations are sent off before the tile
+  // is ordered in LDS, and their answers (a trip to the L2 and back) are only
+  // looked at after that.
+  uint32_t taken[kBins];
+#pragma unroll
+  for (int r = 0; r < kBins; ++r) {
+    const uint32_t bin = threadIdx.x + r * kBlock;
+    taken[r] = 0;
+    if (bin < buckets) {
+      const uint32_t c = (bin + 1 < buckets ? hist[bin + 1] : count) - hist[bin];
+      if (c)
+        taken[r] = (uint32_t)atomicAdd((unsigned long long*)&bucket_cur[t.b.bucket0 + bin],
+                                       (unsigned long long)c);
+    }
   }
-  __syncthreads();
 #pragma unroll
   for (int i = 0; i < kPartItems; ++i) {
     const int64_t l = t.begin + i * kBlock + threadIdx.x;
     if (l < t.end)
       stage[hist[bucket_of(key[i], buckets)] + place[i]] =
           ((uint64_t)key[i] << 32) | (uint64_t)l;
+  }
+#pragma unroll
+  for (int r = 0; r < kBins; ++r) {
+    const uint32_t bin = threadIdx.x + r * kBlock;
+    if (bin < buckets) run_at[bin] += taken[r];
   }
   __syncthreads();
   for (uint32_t j = threadIdx.x; j < count; j += kBlock) {
@@ -747,9 +757,16 @@ __device__ __forceinline__ void dedup_bucket(
   }
 }
 
-// One work-group per bucket.  The two forms of the body differ only in whether
-// a match of the upper halves is confirmed against the keys; which one runs is
-// the same for every work-group of a launch.
+// One work-group per bucket.  A bucket that is sure to fit the LDS table, in a
+// call whose keys all fit the upper half of an entry (nearly every bucket of
+// nearly every call), takes the short path below: the pass is bound by the
+// instructions of its probe loops, not by LDS or memory, so the table is split
+// into 32-bit keys and 32-bit positions (32-bit compares and atomics, a 32-bit
+// multiplicative hash), and an entry remembers the slot its key landed in, so
+// that reading the first position back is one load and no second probe.
+// Everything else (oversize buckets, wide keys) goes through dedup_bucket.
+constexpr uint32_t kNoTag = 0xFFFFFFFFu;  // never a tag, see key_tag
+
 template <int kThreads>
 __global__ __launch_bounds__(kThreads) void unique_dedup_kernel(
     Keys k, const int* __restrict__ wide_keys,
@@ -762,17 +779,65 @@ __global__ __launch_bounds__(kThreads) void unique_dedup_kernel(
   __shared__ uint32_t overflow;
   const int64_t g = unit_of_block(max_buckets, remap);
   if (g >= max_buckets) return;
+  // Everything the bucket needs to know is asked for at once, and its entries
+  // right behind (two round trips to memory, not one per early exit): an unused
+  // bucket has count 0, and entries are only read below that count.
   const int32_t b = bucket_batch[g];
-  if (b < 0) return;  // uniform per work-group
-  const int64_t lo = bucket_off[g], hi = lo + bucket_cnt[g];
-  if (hi == lo) return;
+  const int64_t lo = bucket_off[g], n = bucket_cnt[g];
+  const bool wide = *wide_keys != 0;
+  constexpr int kKeep = kLdsMaxEntries / kThreads;
+  uint64_t mine[kKeep];
+  const bool small = n <= kLdsMaxEntries;
+#pragma unroll
+  for (int j = 0; j < kKeep; ++j) {
+    const int64_t i = j * kThreads + threadIdx.x;
+    mine[j] = small && i < n ? packed[lo + i] : kEmptySlot;
+  }
+  if (b < 0 || n == 0) return;  // uniform per work-group
   const BatchInfo info = batch[b];
-  if (*wide_keys)
-    dedup_bucket<kThreads, true>(k, info, g, lo, hi, packed, spill, first, tab, &distinct,
+  if (wide) {
+    dedup_bucket<kThreads, true>(k, info, g, lo, lo + n, packed, spill, first, tab, &distinct,
                                  &overflow);
-  else
-    dedup_bucket<kThreads, false>(k, info, g, lo, hi, packed, spill, first, tab, &distinct,
-                                  &overflow);
+    return;
+  }
+  if (!small) {
+    dedup_bucket<kThreads, false>(k, info, g, lo, lo + n, packed, spill, first, tab,
+                                  &distinct, &overflow);
+    return;
+  }
+  uint32_t* tags = (uint32_t*)tab;          // [slots]
+  uint32_t* mins = tags + kLdsSlots;        // [slots]
+  uint32_t shift = 24;  // 32 - log2(slots): 256 slots to start with
+  while (shift > 20 && (int64_t)(1u << (32 - shift)) < 2 * n) --shift;
+  const uint32_t slots = 1u << (32 - shift), mask = slots - 1;
+  for (uint32_t i = threadIdx.x; i < slots; i += kThreads) {
+    tags[i] = kNoTag;
+    mins[i] = 0xFFFFFFFFu;
+  }
+  __syncthreads();
+  uint32_t at[kKeep];
+#pragma unroll
+  for (int j = 0; j < kKeep; ++j) {
+    if (mine[j] == kEmptySlot) continue;
+    const uint32_t tag = (uint32_t)(mine[j] >> 32), pos = (uint32_t)mine[j];
+    uint32_t slot = (tag * 0x85EBCA6Bu) >> shift;  // a multiplier unrelated to the one that chose the bucket
+    for (;;) {
+      uint32_t cur = tags[slot];
+      if (cur == kNoTag) cur = atomicCAS(&tags[slot], kNoTag, tag);
+      if (cur == kNoTag || cur == tag) break;
+      slot = (slot + 1) & mask;
+    }
+    at[j] = slot;
+    if (mins[slot] > pos) atomicMin(&mins[slot], pos);
+  }
+  __syncthreads();
+  uint32_t* first_b = first + info.fb;
+#pragma unroll
+  for (int j = 0; j < kKeep; ++j) {
+    if (mine[j] == kEmptySlot) continue;
+    const uint32_t f = mins[at[j]];
+    if (f != (uint32_t)mine[j]) first_b[(uint32_t)mine[j]] = f;
+  }
 }
 
 // ---------------------------------------------------------------- flag
@@ -1098,18 +1163,10 @@ int gs_unique_count(const int64_t* seeds, const int64_t* seeds_ptr,
                 k, w.tile_batch, w.batch, w.bucket_cnt, w.bucket_cur, w.bucket_off,
                 w.packed, w.first, w.max_tiles, tn.remap));
   GS_LAUNCH("unique_dedup", s,
-            if (tn.dedup_threads == 512)
-              unique_dedup_kernel<512><<<dim3((unsigned)grid_for_units(
-                                             w.max_buckets, tn.remap)),
-                                         dim3(512), 0, s>>>(
-                  k, w.wide_keys, w.bucket_batch, w.batch, w.bucket_cnt, w.bucket_off,
-                  w.packed, w.spill, w.first, w.max_buckets, tn.remap);
-            else
-              unique_dedup_kernel<256><<<dim3((unsigned)grid_for_units(
-                                             w.max_buckets, tn.remap)),
-                                         dim3(256), 0, s>>>(
-                  k, w.wide_keys, w.bucket_batch, w.batch, w.bucket_cnt, w.bucket_off,
-                  w.packed, w.spill, w.first, w.max_buckets, tn.remap));
+            unique_dedup_kernel<512><<<dim3((unsigned)grid_for_units(w.max_buckets, tn.remap)),
+                                       dim3(512), 0, s>>>(
+                k, w.wide_keys, w.bucket_batch, w.batch, w.bucket_cnt, w.bucket_off, w.packed,
+                w.spill, w.first, w.max_buckets, tn.remap));
   GS_LAUNCH("unique_flag", s,
             unique_flag_kernel<<<dim3((unsigned)w.groups), dim3(kBlock), 0, s>>>(
                 w.flat_ptr, w.group_batch, N, w.first, w.words, w.group_cnt));
