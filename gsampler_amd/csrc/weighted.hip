@@ -630,6 +630,346 @@ __global__ __launch_bounds__(kBlock) void list_replace_kernel(
   }
 }
 
+// Zeroes n 32-bit words (a kernel rather than a memset so that callers may
+// capture the launches in a HIP graph).
+__global__ __launch_bounds__(kBlock) void table_fill_kernel32(uint32_t* __restrict__ words,
+                                                              int64_t n) {
+  int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  const int64_t stride = (int64_t)gridDim.x * kBlock;
+  for (; i < n; i += stride) words[i] = 0u;
+}
+
+// ---------------------------------------------- the K smallest keys by selection
+// Without replacement the pick is "the K smallest keys, in ascending order, ties
+// to the smaller index".  Sorting all n keys for that costs sixteen launches of
+// a radix sort; for K up to kSelMaxPicks the kernels below select instead:
+//   keys     key of every item (kept), histogram of its top 12 bits (the
+//            exponent of a non-negative double) per segment
+//   refine   the bin that holds the K-th smallest key follows from that
+//            histogram (every work-group scans it for itself: 4096 bins); items
+//            of that bin are counted by their next 12 bits
+//   emit     the same again one level down; items below the K-th item's
+//            (bin, sub-bin) cell are certain picks and go to the segment's pick
+//            list, items inside the cell to its candidate list
+//   finish   one work-group per segment: picks + the smallest candidates are
+//            ordered by (key, index) in LDS and written out
+// The cell of the K-th item holds a handful of items unless keys repeat (items
+// of weight zero all have the key +inf); a cell too large for LDS is narrowed
+// by a byte-wise radix selection over its remaining key bits and indices first.
+constexpr int kSelBins = 4096;
+constexpr int kSelTile = 4096;  // shortest average segment the selection takes on
+constexpr int64_t kSelMaxPicks = 2048;
+constexpr int kFinishThreads = 1024;
+constexpr int kFinishSlots = 4096;
+constexpr int kFinishSplit = 16;  // work-groups that share the ordering of one segment's picks
+
+__host__ __device__ inline bool list_can_select(int64_t n, int64_t nseg) {
+  return n < (int64_t(1) << 31) && (nseg == 1 || n / nseg >= kSelTile);
+}
+
+__device__ __forceinline__ uint32_t sel_digit1(uint64_t k) { return (uint32_t)(k >> 52); }
+__device__ __forceinline__ uint32_t sel_digit2(uint64_t k) {
+  return (uint32_t)(k >> 40) & (kSelBins - 1);
+}
+
+// The bin of a kSelBins-bin histogram that holds the want-th smallest item
+// (1-based, want <= number of items), and the number of items in the bins
+// below it.  Called by the whole work-group; the result is the same in every
+// thread.
+__device__ __forceinline__ void find_bin(const uint32_t* __restrict__ hist, uint32_t want,
+                                         uint32_t* smem, uint32_t* found, uint32_t* bin,
+                                         uint32_t* below) {
+  constexpr int kPer = kSelBins / kBlock;
+  uint32_t c[kPer], sum = 0;
+#pragma unroll
+  for (int j = 0; j < kPer; ++j) {
+    c[j] = hist[threadIdx.x * kPer + j];
+    sum += c[j];
+  }
+  uint32_t total;
+  uint32_t run = block_exclusive_sum(sum, smem, &total);
+  const uint32_t target = want - 1;
+  if (target >= run && target < run + sum) {
+#pragma unroll
+    for (int j = 0; j < kPer; ++j) {
+      if (target >= run && target < run + c[j]) {
+        found[0] = threadIdx.x * kPer + j;
+        found[1] = run;
+      }
+      run += c[j];
+    }
+  }
+  __syncthreads();
+  *bin = found[0];
+  *below = found[1];
+  __syncthreads();
+}
+
+struct SelSegment {
+  int64_t lo, hi;
+};
+__device__ __forceinline__ SelSegment sel_segment(const int64_t* __restrict__ range, int64_t n,
+                                                  int64_t seg) {
+  return range ? SelSegment{range[seg], range[seg + 1]} : SelSegment{0, n};
+}
+__device__ __forceinline__ SegmentSpan sel_span(const int64_t* __restrict__ range, int64_t nseg,
+                                                int64_t i0, int64_t i_last) {
+  return range ? segment_span(range, nseg, i0, i_last) : SegmentSpan{0, 0};
+}
+
+template <int kSelItems>
+__global__ __launch_bounds__(kBlock) void list_keys_hist_kernel(
+    const float* __restrict__ probs, const int64_t* __restrict__ range, int64_t n,
+    int64_t nseg, PhiloxKey key, uint64_t* __restrict__ keys, uint32_t* hist1) {
+  __shared__ uint32_t lh[kSelBins];
+  const int64_t i0 = (int64_t)blockIdx.x * (kBlock * kSelItems);
+  const int64_t i_last = i0 + (kBlock * kSelItems) - 1 < n ? i0 + (kBlock * kSelItems) - 1 : n - 1;
+  const SegmentSpan span = sel_span(range, nseg, i0, i_last);
+  for (int b = threadIdx.x; b < kSelBins; b += kBlock) lh[b] = 0;
+  __syncthreads();
+#pragma unroll 4
+  for (int j = 0; j < kSelItems; ++j) {
+    const int64_t i = i0 + j * kBlock + threadIdx.x;
+    if (i >= n) break;
+    // non-negative doubles (and +inf) order like their bit patterns
+    const uint64_t k =
+        (uint64_t)__double_as_longlong(weighted_key(key, (uint64_t)i, 0, probs[i]));
+    keys[i] = k;
+    const int64_t seg = span.segment_at(range, i);
+    if (seg == span.lo)
+      atomicAdd(&lh[sel_digit1(k)], 1u);
+    else
+      atomicAdd(&hist1[seg * kSelBins + sel_digit1(k)], 1u);
+  }
+  __syncthreads();
+  for (int b = threadIdx.x; b < kSelBins; b += kBlock)
+    if (lh[b]) atomicAdd(&hist1[span.lo * kSelBins + b], lh[b]);
+}
+
+template <int kSelItems>
+__global__ __launch_bounds__(kBlock) void list_refine_kernel(
+    const int64_t* __restrict__ range, int64_t n, int64_t nseg, int64_t num_picks,
+    const uint64_t* __restrict__ keys, const uint32_t* __restrict__ hist1, uint32_t* hist2) {
+  __shared__ uint32_t lh[kSelBins];
+  __shared__ uint32_t smem[kBlock / kWave + 1];
+  __shared__ uint32_t found[2];
+  const int64_t i0 = (int64_t)blockIdx.x * (kBlock * kSelItems);
+  const int64_t i_last = i0 + (kBlock * kSelItems) - 1 < n ? i0 + (kBlock * kSelItems) - 1 : n - 1;
+  const SegmentSpan span = sel_span(range, nseg, i0, i_last);
+  for (int64_t seg = span.lo; seg <= span.hi; ++seg) {  // the same in every thread
+    const SelSegment sg = sel_segment(range, n, seg);
+    if (sg.hi - sg.lo <= num_picks) continue;  // taken whole
+    uint32_t b1, below1;
+    find_bin(hist1 + seg * kSelBins, (uint32_t)num_picks, smem, found, &b1, &below1);
+    for (int b = threadIdx.x; b < kSelBins; b += kBlock) lh[b] = 0;
+    __syncthreads();
+#pragma unroll 4
+    for (int j = 0; j < kSelItems; ++j) {
+      const int64_t i = i0 + j * kBlock + threadIdx.x;
+      if (i >= sg.lo && i < sg.hi && i <= i_last) {
+        const uint64_t k = keys[i];
+        if (sel_digit1(k) == b1) atomicAdd(&lh[sel_digit2(k)], 1u);
+      }
+    }
+    __syncthreads();
+    for (int b = threadIdx.x; b < kSelBins; b += kBlock)
+      if (lh[b]) atomicAdd(&hist2[seg * kSelBins + b], lh[b]);
+    __syncthreads();
+  }
+}
+
+template <int kSelItems>
+__global__ __launch_bounds__(kBlock) void list_emit_kernel(
+    const int64_t* __restrict__ range, int64_t n, int64_t nseg, int64_t num_picks,
+    const uint64_t* __restrict__ keys, const uint32_t* __restrict__ hist1,
+    const uint32_t* __restrict__ hist2, uint32_t* counts, uint64_t* __restrict__ win_key,
+    int64_t* __restrict__ win_idx, uint64_t* __restrict__ cand_key,
+    int64_t* __restrict__ cand_idx) {
+  __shared__ uint32_t smem[kBlock / kWave + 1];
+  __shared__ uint32_t found[2];
+  __shared__ uint32_t bases[2];
+  const int64_t i0 = (int64_t)blockIdx.x * (kBlock * kSelItems);
+  const int64_t i_last = i0 + (kBlock * kSelItems) - 1 < n ? i0 + (kBlock * kSelItems) - 1 : n - 1;
+  const SegmentSpan span = sel_span(range, nseg, i0, i_last);
+  for (int64_t seg = span.lo; seg <= span.hi; ++seg) {  // the same in every thread
+    const SelSegment sg = sel_segment(range, n, seg);
+    if (sg.hi - sg.lo <= num_picks) continue;
+    uint32_t b1, below1, b2, below2;
+    find_bin(hist1 + seg * kSelBins, (uint32_t)num_picks, smem, found, &b1, &below1);
+    find_bin(hist2 + seg * kSelBins, (uint32_t)num_picks - below1, smem, found, &b2, &below2);
+    uint64_t k[kSelItems];
+    uint32_t is_win = 0, is_cand = 0;  // one bit per item of this thread
+#pragma unroll
+    for (int j = 0; j < kSelItems; ++j) {
+      const int64_t i = i0 + j * kBlock + threadIdx.x;
+      k[j] = 0;
+      if (i >= sg.lo && i < sg.hi && i <= i_last) {
+        k[j] = keys[i];
+        const uint32_t d1 = sel_digit1(k[j]), d2 = sel_digit2(k[j]);
+        if (d1 < b1 || (d1 == b1 && d2 < b2))
+          is_win |= 1u << j;
+        else if (d1 == b1 && d2 == b2)
+          is_cand |= 1u << j;
+      }
+    }
+    uint32_t wins, cands;
+    uint32_t w_at = block_exclusive_sum((uint32_t)__popc(is_win), smem, &wins);
+    uint32_t c_at = block_exclusive_sum((uint32_t)__popc(is_cand), smem, &cands);
+    if (threadIdx.x == 0) {
+      bases[0] = wins ? atomicAdd(&counts[2 * seg], wins) : 0u;
+      bases[1] = cands ? atomicAdd(&counts[2 * seg + 1], cands) : 0u;
+    }
+    __syncthreads();
+    w_at += bases[0];
+    c_at += bases[1];
+#pragma unroll
+    for (int j = 0; j < kSelItems; ++j) {
+      const int64_t i = i0 + j * kBlock + threadIdx.x;
+      if ((is_win >> j) & 1u) {
+        if (w_at < (uint32_t)kSelMaxPicks) {  // always: fewer than num_picks items lie below the cell
+          win_key[seg * kSelMaxPicks + w_at] = k[j];
+          win_idx[seg * kSelMaxPicks + w_at] = i;
+        }
+        ++w_at;
+      } else if ((is_cand >> j) & 1u) {
+        if ((int64_t)c_at < sg.hi - sg.lo) {
+          cand_key[sg.lo + c_at] = k[j];
+          cand_idx[sg.lo + c_at] = i;
+        }
+        ++c_at;
+      }
+    }
+    __syncthreads();
+  }
+}
+
+// (key, index) as one number: the low 40 bits of the key (the upper 24 are the
+// same for all candidates of a cell) above the 32-bit index.
+__device__ __forceinline__ unsigned __int128 sel_composite(uint64_t k, int64_t i) {
+  return ((unsigned __int128)(k & ((1ull << 40) - 1)) << 32) | (unsigned __int128)(uint32_t)i;
+}
+
+__global__ __launch_bounds__(kFinishThreads) void list_finish_kernel(
+    const int64_t* __restrict__ range, int64_t n, int64_t num_picks,
+    const uint32_t* __restrict__ counts, const uint64_t* __restrict__ win_key,
+    const int64_t* __restrict__ win_idx, const uint64_t* __restrict__ cand_key,
+    const int64_t* __restrict__ cand_idx, const int64_t* __restrict__ out_range,
+    int64_t* __restrict__ out_index) {
+  __shared__ uint64_t sk[kFinishSlots];
+  __shared__ int64_t si[kFinishSlots];
+  __shared__ uint32_t hist[256];
+  __shared__ uint32_t chosen[2];
+  __shared__ uint32_t appended;
+  const int64_t seg = blockIdx.x;
+  const SelSegment sg = sel_segment(range, n, seg);
+  const int64_t nb = sg.hi - sg.lo, out0 = out_range[seg];
+  if (nb <= num_picks) {  // taken whole, in the original order
+    if (blockIdx.y == 0)
+      for (int64_t k = threadIdx.x; k < nb; k += kFinishThreads) out_index[out0 + k] = sg.lo + k;
+    return;
+  }
+  const uint32_t W = counts[2 * seg], M = counts[2 * seg + 1];
+  const uint64_t* ck = cand_key + sg.lo;
+  const int64_t* ci = cand_idx + sg.lo;
+  for (uint32_t t = threadIdx.x; t < W; t += kFinishThreads) {
+    sk[t] = win_key[seg * kSelMaxPicks + t];
+    si[t] = win_idx[seg * kSelMaxPicks + t];
+  }
+  uint32_t total = W + M;
+  if (total <= (uint32_t)kFinishSlots) {
+    for (uint32_t t = threadIdx.x; t < M; t += kFinishThreads) {
+      sk[W + t] = ck[t];
+      si[W + t] = ci[t];
+    }
+  } else {
+    // the `want` smallest of the M candidates: fix the composite of the last
+    // of them byte by byte, most significant first
+    uint32_t want = (uint32_t)num_picks - W;
+    unsigned __int128 fixed = 0;
+    for (int d = 0; d < 9; ++d) {
+      const int shift = 8 * (8 - d);
+      for (int b = threadIdx.x; b < 256; b += kFinishThreads) hist[b] = 0;
+      __syncthreads();
+      for (uint32_t t = threadIdx.x; t < M; t += kFinishThreads) {
+        const unsigned __int128 c = sel_composite(ck[t], ci[t]);
+        if ((c >> (shift + 8)) == (fixed >> (shift + 8)))
+          atomicAdd(&hist[(uint32_t)(c >> shift) & 255u], 1u);
+      }
+      __syncthreads();
+      if (threadIdx.x == 0) {
+        uint32_t run = 0, b = 0;
+        for (; b < 255 && run + hist[b] < want; ++b) run += hist[b];
+        chosen[0] = b;
+        chosen[1] = run;
+      }
+      __syncthreads();
+      fixed |= (unsigned __int128)chosen[0] << shift;
+      want -= chosen[1];
+      __syncthreads();
+    }
+    if (threadIdx.x == 0) appended = 0;
+    __syncthreads();
+    for (uint32_t t = threadIdx.x; t < M; t += kFinishThreads) {
+      const uint64_t k = ck[t];
+      const int64_t i = ci[t];
+      if (sel_composite(k, i) <= fixed) {
+        const uint32_t at = W + atomicAdd(&appended, 1u);
+        sk[at] = k;
+        si[at] = i;
+      }
+    }
+    total = (uint32_t)num_picks;
+  }
+  __syncthreads();
+  // Order by (key, index): the rank of an item is the number of smaller ones.
+  // The work is dealt out as (item, part of the others) pairs so that all
+  // threads have some whatever the number of items; a thread reads eight keys
+  // ahead (every lane of a wave reads the same ones: a broadcast), partial
+  // ranks meet in LDS.
+  // The kFinishSplit work-groups of a segment all hold all items and each ranks
+  // its share of them (by index, so that the split does not depend on the order
+  // the lists were filled in): the comparisons (the square of the number of
+  // items) are more than one compute unit should do alone.
+  __shared__ uint32_t rank_of_item[kFinishSlots];
+  __shared__ uint16_t my_items[kFinishSlots];
+  if (threadIdx.x == 0) appended = 0;
+  for (uint32_t t = threadIdx.x; t < total; t += kFinishThreads) rank_of_item[t] = 0;
+  __syncthreads();
+  for (uint32_t t = threadIdx.x; t < total; t += kFinishThreads)
+    if ((uint32_t)si[t] % kFinishSplit == blockIdx.y) my_items[atomicAdd(&appended, 1u)] = (uint16_t)t;
+  __syncthreads();
+  const uint32_t mine = appended;
+  uint32_t parts = kFinishThreads / (mine ? mine : 1);
+  if (parts < 1) parts = 1;
+  if (parts > 8) parts = 8;
+  const uint32_t per = (total + parts - 1) / parts;
+  for (uint32_t w = threadIdx.x; w < mine * parts; w += kFinishThreads) {
+    const uint32_t t = my_items[w % mine], part = w / mine;
+    const uint64_t k = sk[t];
+    const int64_t i = si[t];
+    const uint32_t o_end = (part + 1) * per < total ? (part + 1) * per : total;
+    uint32_t smaller = 0;
+    for (uint32_t o = part * per; o < o_end; o += 8) {
+      uint64_t ko[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) ko[u] = o + u < o_end ? sk[o + u] : ~0ull;
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        if (ko[u] < k)
+          ++smaller;
+        else if (ko[u] == k && o + u < o_end && si[o + u] < i)
+          ++smaller;
+      }
+    }
+    atomicAdd(&rank_of_item[t], smaller);
+  }
+  __syncthreads();
+  for (uint32_t m = threadIdx.x; m < mine; m += kFinishThreads) {
+    const uint32_t t = my_items[m], r = rank_of_item[t];
+    if (r < (uint32_t)num_picks) out_index[out0 + r] = si[t];
+  }
+}
+
 struct ListWs {
   uint64_t *keys_in, *keys_out;  // also the CDF scratch when sampling with replacement
   int64_t *vals_in, *vals_out;
@@ -637,6 +977,12 @@ struct ListWs {
   size_t sort_ws_bytes;
   void* scan_ws;
   size_t scan_ws_bytes;
+  // selection (list_can_select): histograms, then counters, in one block
+  uint32_t* sel_block;
+  size_t sel_words;
+  uint32_t *hist1, *hist2, *counts;
+  uint64_t* win_key;
+  int64_t* win_idx;
   size_t total;
 };
 
@@ -663,6 +1009,14 @@ static ListWs carve_list(void* ws, int64_t n, int64_t nseg) {
   w.sort_ws = c.take<char>(w.sort_ws_bytes);
   w.scan_ws_bytes = scan_workspace_bytes(nseg + 1);
   w.scan_ws = c.take<char>(w.scan_ws_bytes);
+  const size_t segs = list_can_select(n, nseg) ? (size_t)nseg : 0;
+  w.sel_words = segs * (2 * kSelBins + 2);
+  w.sel_block = c.take<uint32_t>(w.sel_words);
+  w.hist1 = w.sel_block;
+  w.hist2 = w.hist1 ? w.hist1 + segs * kSelBins : nullptr;
+  w.counts = w.hist2 ? w.hist2 + segs * kSelBins : nullptr;
+  w.win_key = c.take<uint64_t>(segs * (size_t)kSelMaxPicks);
+  w.win_idx = c.take<int64_t>(segs * (size_t)kSelMaxPicks);
   w.total = c.total();
   return w;
 }
@@ -842,6 +1196,31 @@ int gs_list_sample_weighted_fill(const float* probs, const int64_t* range,
                                     dim3(kBlock), 0, s>>>(
                   probs, range, n, num_segments, num_picks, key, out_range,
                   w.keys_in, out_index));
+    return GS_OK;
+  }
+  if (num_picks >= 1 && num_picks <= kSelMaxPicks && list_can_select(n, num_segments)) {
+    // few items per thread while that still fills the device, else sixteen (fewer
+    // work-groups meet at the same histogram bins)
+    const bool deep = n >= (int64_t(1) << 21);
+    const dim3 tiles((unsigned)ceil_div(n, kBlock * (deep ? 16 : 4)));
+    GS_LAUNCH("list_zero", s,
+              table_fill_kernel32<<<dim3((unsigned)ceil_div((int64_t)w.sel_words, kBlock * 8)),
+                                    dim3(kBlock), 0, s>>>(w.sel_block, (int64_t)w.sel_words));
+#define GS_SEL_LAUNCH(name, kernel, ...)                                              \
+  GS_LAUNCH(name, s,                                                                  \
+            if (deep) kernel<16><<<tiles, dim3(kBlock), 0, s>>>(__VA_ARGS__);         \
+            else kernel<4><<<tiles, dim3(kBlock), 0, s>>>(__VA_ARGS__))
+    GS_SEL_LAUNCH("list_keys", list_keys_hist_kernel, probs, range, n, num_segments, key,
+                  w.keys_in, w.hist1);
+    GS_SEL_LAUNCH("list_refine", list_refine_kernel, range, n, num_segments, num_picks,
+                  w.keys_in, w.hist1, w.hist2);
+    GS_SEL_LAUNCH("list_emit", list_emit_kernel, range, n, num_segments, num_picks, w.keys_in,
+                  w.hist1, w.hist2, w.counts, w.win_key, w.win_idx, w.keys_out, w.vals_out);
+#undef GS_SEL_LAUNCH
+    GS_LAUNCH("list_finish", s,
+              list_finish_kernel<<<dim3((unsigned)num_segments, kFinishSplit), dim3(kFinishThreads), 0, s>>>(
+                  range, n, num_picks, w.counts, w.win_key, w.win_idx, w.keys_out, w.vals_out,
+                  out_range, out_index));
     return GS_OK;
   }
   GS_LAUNCH("list_keys", s,

@@ -150,6 +150,47 @@ def test_batched_list_sampling_parity():
          orc.list_sample_weighted(probs, 100, replace=True, range_=ranges))
 
 
+@pytest.mark.parametrize("case", ["few_positive", "all_zero", "repeated_weights", "one_heavy",
+                                  "k_limits"])
+def test_list_selection_cases(case):
+    """The K smallest keys by selection (up to 2048 picks): cells of equal keys far larger
+    than the pick count, weights that repeat, one dominant weight, pick counts at and
+    around the limit of the selection path."""
+    rng = np.random.default_rng(len(case))
+    n = 300_000
+    probs = rng.random(n).astype(np.float32)
+    ks = [512]
+    if case == "few_positive":        # fewer positive weights than picks: the rest by index
+        probs[rng.permutation(n)[300:]] = 0.0
+    elif case == "all_zero":
+        probs[:] = 0.0
+    elif case == "repeated_weights":  # many equal weights (keys still differ: other draws)
+        probs = rng.choice(np.array([0.25, 0.5, 1.0], dtype=np.float32), size=n)
+    elif case == "one_heavy":
+        probs *= 1e-6
+        probs[12345] = 1e6
+    else:
+        ks = [1, 2047, 2048, 2049]
+    for k in ks:
+        same(capi.list_sample_weighted(F(probs), k, call_id=2),
+             orc.list_sample_weighted(probs, k, call_id=2))
+
+
+def test_batched_list_selection_parity():
+    """Segments long enough for the selection path, ragged, one of them empty, one taken
+    whole, one with fewer positive weights than picks."""
+    rng = np.random.default_rng(8)
+    sizes = np.array([60000, 0, 300, 4097, 150000, 33000])
+    ranges = np.concatenate([[0], np.cumsum(sizes)])
+    probs = rng.random(ranges[-1]).astype(np.float32)
+    probs[rng.random(probs.size) < 0.3] = 0.0
+    probs[ranges[5]:ranges[6]] = 0.0
+    probs[ranges[5] + 100:ranges[5] + 200] = 0.5
+    for k in (64, 512):
+        same(capi.list_sample_weighted(F(probs), k, range_=T(ranges), call_id=3),
+             orc.list_sample_weighted(probs, k, range_=ranges, call_id=3))
+
+
 def test_operators_through_the_api():
     rng = np.random.default_rng(6)
     indptr, indices = random_csc(rng, 500, 400, 60)
