@@ -661,25 +661,32 @@ def main():
                             gbs=(nbytes / (ms * 1e-3) / 1e9) if ms > 0 else 0.0))
     kernels.sort(key=lambda k: -k["total_ms"])
     dom = kernels[0]
-    traffic = None
-    # measured HBM bytes per launch (hardware counters of a profiled run of this
-    # same command, kept as text: kernel launches fetch write total)
-    tpath = os.path.join(ROOT, "profiles", f"graphsage_{args.workload}_hbm_traffic.txt")
+    # Bytes that the L2s exchanged with the memory fabric per launch (rocprofv3 FETCH_SIZE +
+    # WRITE_SIZE; reads served by the Infinity Cache are included, the counters cannot tell
+    # them from HBM accesses).  Not measured in this run: transcribed from the committed
+    # counter summary of this same command, which names the commit it was taken at.
+    traffic, traffic_source = None, None
+    tname = f"graphsage_{args.workload}_hbm_traffic.txt"
+    tpath = os.path.join(ROOT, "profiles", tname)
     if os.path.exists(tpath):
+        commit = None
         for line in open(tpath):
             f = line.split()
+            if line.startswith("# commit:") and len(f) >= 3:
+                commit = f[2]
             if len(f) == 5 and f[0] == dom["kernel"]:
                 traffic = int(f[4])
+        traffic_source = {"file": f"profiles/{tname}", "commit": commit,
+                          "kind": "transcribed, not measured in this run"}
     roofline = dict(bound="hbm", kernel=dom["kernel"], achieved=round(dom["gbs"], 1),
                     peak=HBM_PEAK_GBS, unit="GB/s", frac=round(dom["gbs"] / HBM_PEAK_GBS, 4),
                     traffic=traffic, avg_launch_ms=round(dom["avg_ms"], 4),
                     launches=dom["launches"])
     if traffic and dom["avg_ms"] > 0:
-        # what the memory system actually moved per launch (every request of this
-        # part's L2 to memory is a 128-byte line) over the same duration
-        moved = traffic / (dom["avg_ms"] * 1e-3) / 1e9
-        roofline["traffic_gbs"] = round(moved, 1)
-        roofline["traffic_frac"] = round(moved / HBM_PEAK_GBS, 4)
+        roofline["traffic_source"] = traffic_source
+        # the same bytes over this run's launch duration: the rate at the L2-fabric
+        # boundary, not an HBM rate
+        roofline["fabric_traffic_gbs"] = round(traffic / (dom["avg_ms"] * 1e-3) / 1e9, 1)
     pipeline_bytes = sum(40 * S + 56 * E + 8 * U for S, E, U in sizes)
 
     # ---- the same workload through the drop-in stack: BatchMatrix + gs.jit.compile +
