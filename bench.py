@@ -442,8 +442,9 @@ def run_ops(args, wl, capi, dev):
             8 * S2 + 8 * sl_nnz, f"{sl_nnz} edges")
     del sl, e_w, col_sum, coo_view, csc_view
     # samplers on the layer-3 frontier
+    idx32 = indices.to(torch.int32)      # the copy a loaded matrix keeps for this sampler
     measure("uniform slice + sample, K=5", "FusedCSCColSlicingSamplingCUDA",
-            lambda: capi.sample_uniform(indptr, indices, f3, 5, False, 0, args.seed, 2),
+            lambda: capi.sample_uniform(indptr, idx32, f3, 5, False, 0, args.seed, 2),
             32 * S3 + 32 * E3, f"{S3} columns")
     measure("weighted slice + sample, K=5 (CDF)", "CSCColSamplingProbsCUDA",
             lambda: capi.sample_weighted(indptr, indices, probs, f3, 5, False, args.seed, 2, cdf=cdf),
