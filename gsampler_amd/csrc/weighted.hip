@@ -922,14 +922,14 @@ __global__ __launch_bounds__(kFinishThreads) void list_finish_kernel(
   }
   __syncthreads();
   // Order by (key, index): the rank of an item is the number of smaller ones.
-  // The work is dealt out as (item, part of the others) pairs so that all
-  // threads have some whatever the number of items; a thread reads eight keys
-  // ahead (every lane of a wave reads the same ones: a broadcast), partial
-  // ranks meet in LDS.
   // The kFinishSplit work-groups of a segment all hold all items and each ranks
-  // its share of them (by index, so that the split does not depend on the order
-  // the lists were filled in): the comparisons (the square of the number of
-  // items) are more than one compute unit should do alone.
+  // its share of them (shares go by index, so that they do not depend on the
+  // order the lists were filled in): the comparisons (the square of the number
+  // of items) are more than one compute unit should do alone.  Inside a
+  // work-group the work is dealt out as (item, part of the others) pairs so
+  // that all threads have some whatever the number of items; a thread reads
+  // eight keys ahead (every lane of a wave reads the same ones: a broadcast),
+  // partial ranks meet in LDS.
   __shared__ uint32_t rank_of_item[kFinishSlots];
   __shared__ uint16_t my_items[kFinishSlots];
   if (threadIdx.x == 0) appended = 0;
