@@ -204,9 +204,13 @@ MajorResult major_slice(const Compressed& m, const torch::Tensor& picked,
 // array stays in cache anyway); undefined when the matrix does not qualify.
 const torch::Tensor& Compressed::narrow_indices() const {
   constexpr int64_t kMinEdges = int64_t(1) << 20;
+  const int64_t version = (int64_t)indices._version();
+  if (indices32.defined() && indices32_version != version) indices32 = torch::Tensor();  // edited in place
   if (!indices32.defined() && num_minor >= 0 && num_minor < (int64_t(1) << 31) &&
-      indices.is_cuda() && indices.numel() >= kMinEdges)
+      indices.is_cuda() && indices.numel() >= kMinEdges) {
     indices32 = indices.to(torch::kInt32);
+    indices32_version = version;
+  }
   return indices32;
 }
 

@@ -33,6 +33,7 @@ struct Compressed {
   // every random pick); made on the first sampling call of a matrix in device
   // memory whose ids fit.
   mutable torch::Tensor indices32;
+  mutable int64_t indices32_version = -1;  // version of `indices` the copy was made from
   const torch::Tensor& narrow_indices() const;
 };
 
