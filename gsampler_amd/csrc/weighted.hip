@@ -651,8 +651,9 @@ __global__ __launch_bounds__(kBlock) void table_fill_kernel32(uint32_t* __restri
 //   emit     the same again one level down; items below the K-th item's
 //            (bin, sub-bin) cell are certain picks and go to the segment's pick
 //            list, items inside the cell to its candidate list
-//   finish   one work-group per segment: picks + the smallest candidates are
-//            ordered by (key, index) in LDS and written out
+//   finish   picks + the smallest candidates of a segment are ordered by
+//            (key, index) in LDS and written out (sixteen work-groups per
+//            segment share the comparisons)
 // The cell of the K-th item holds a handful of items unless keys repeat (items
 // of weight zero all have the key +inf); a cell too large for LDS is narrowed
 // by a byte-wise radix selection over its remaining key bits and indices first.

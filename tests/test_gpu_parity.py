@@ -157,9 +157,11 @@ def test_unique_relabel_hubs_and_ragged_batches():
                 orc.unique_relabel(seeds, rows, sp, rp, edge_col))
 
 
-def test_unique_relabel_many_tiny_batches():
+@pytest.mark.parametrize("B", [1023, 1024, 1025, 3000])
+def test_unique_relabel_many_tiny_batches(B):
+    """Around 1024 batches the batch walk moves from every work-group's LDS to a launch
+    of its own."""
     rng = np.random.default_rng(12)
-    B = 3000
     s_sizes = rng.integers(0, 3, size=B)
     r_sizes = rng.integers(0, 6, size=B)
     sp = np.concatenate([[0], np.cumsum(s_sizes)])
