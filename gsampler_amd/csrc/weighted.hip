@@ -869,7 +869,12 @@ __global__ __launch_bounds__(kFinishThreads) void list_finish_kernel(
       for (int64_t k = threadIdx.x; k < nb; k += kFinishThreads) out_index[out0 + k] = sg.lo + k;
     return;
   }
-  const uint32_t W = counts[2 * seg], M = counts[2 * seg + 1];
+  // (fewer than num_picks picks lie below the cell and no list is longer than its
+  // segment; the bounds are restated here because LDS indices follow from them)
+  uint32_t W = counts[2 * seg], M = counts[2 * seg + 1];
+  if (W > (uint32_t)kSelMaxPicks) W = (uint32_t)kSelMaxPicks;
+  if (W > (uint32_t)num_picks) W = (uint32_t)num_picks;
+  if ((int64_t)M > nb) M = (uint32_t)nb;
   const uint64_t* ck = cand_key + sg.lo;
   const int64_t* ci = cand_idx + sg.lo;
   for (uint32_t t = threadIdx.x; t < W; t += kFinishThreads) {
@@ -915,8 +920,10 @@ __global__ __launch_bounds__(kFinishThreads) void list_finish_kernel(
       const int64_t i = ci[t];
       if (sel_composite(k, i) <= fixed) {
         const uint32_t at = W + atomicAdd(&appended, 1u);
-        sk[at] = k;
-        si[at] = i;
+        if (at < (uint32_t)kFinishSlots) {
+          sk[at] = k;
+          si[at] = i;
+        }
       }
     }
     total = (uint32_t)num_picks;
