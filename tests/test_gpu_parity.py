@@ -293,3 +293,42 @@ def test_coo_to_csc_parity(num_cols, nnz):
     want = orc.coo_to_csc(row, col, num_cols)
     got = capi.coo_to_csc(T(row), T(col), num_cols)
     assert_same(got, want)
+
+
+def test_count_mirrors_in_pinned_host_memory():
+    """The optional mirror arguments of the two count entry points: the kernel that
+    computes the edge total / the per-batch offsets stores them to pinned host memory
+    as well; with NULL nothing else changes."""
+    rng = np.random.default_rng(21)
+    indptr, indices = random_csc(rng, 4000, 10**5, 40, hub_deg=9000)
+    cols = rng.integers(0, 4000, size=7000)
+    l = capi.lib()
+    d_indptr, d_cols = T(indptr), T(cols)
+    n = cols.size
+    ws = torch.empty(l.gs_scan_workspace_bytes(n + 1), dtype=torch.uint8, device=DEV)
+    mirror = torch.full((4,), -7, dtype=torch.int64).pin_memory()
+    outs = []
+    for use_mirror in (True, False):
+        sub = torch.empty(n + 1, dtype=torch.int64, device=DEV)
+        capi.check(l.gs_csc_col_count(d_indptr.data_ptr(), indptr.size - 1, d_cols.data_ptr(), n, 5, 0,
+                                      sub.data_ptr(), mirror.data_ptr() if use_mirror else None,
+                                      ws.data_ptr(), ws.numel(), None))
+        torch.cuda.synchronize()
+        outs.append(sub.cpu().numpy())
+    assert np.array_equal(outs[0], outs[1])
+    assert int(mirror[0]) == outs[0][-1] and mirror[1:].tolist() == [-7, -7, -7]
+    want = orc.col_count(indptr, cols, 5, False)
+    assert np.array_equal(outs[0], want)
+
+    seeds, rows, sp, rp, _ = _batched_case(rng, 9, 50, 400, 300)
+    B = sp.size - 1
+    d = [T(x) for x in (seeds, rows, sp, rp)]
+    uws = torch.empty(l.gs_unique_workspace_bytes(seeds.size, rows.size, B), dtype=torch.uint8, device=DEV)
+    host = torch.full((B + 3,), -7, dtype=torch.int64).pin_memory()
+    uptr = torch.empty(B + 1, dtype=torch.int64, device=DEV)
+    capi.check(l.gs_unique_count(d[0].data_ptr(), d[2].data_ptr(), seeds.size, d[1].data_ptr(),
+                                 d[3].data_ptr(), rows.size, B, uptr.data_ptr(), host.data_ptr(),
+                                 uws.data_ptr(), uws.numel(), None))
+    torch.cuda.synchronize()
+    assert host[:B + 1].tolist() == uptr.cpu().tolist() and host[B + 1:].tolist() == [-7, -7]
+    assert np.array_equal(uptr.cpu().numpy(), orc.unique_relabel(seeds, rows, sp, rp)[1])
