@@ -167,6 +167,66 @@ __global__ __launch_bounds__(kBlock) void sample_uniform_kernel(
   }
 }
 
+// The same columns with the lanes packed: a column takes exactly `fanout` lanes
+// (one per output slot), so a wavefront holds 64 / fanout columns -- twelve at
+// fanout 5 where power-of-two groups hold eight, six instead of four at fanout
+// 10.  The kernel is bound by the instructions it issues (a Philox call per
+// slot, the group exchanges of Floyd's rule, three stores), not by the lines
+// behind its picks, and every idle lane of a group is issue bandwidth lost.
+// Covers what gives every slot a lane of its own: sampling with replacement,
+// whole columns, Floyd's rule; picks and outputs are those of
+// sample_uniform_kernel (the same draws: position = column, draw = slot).
+__device__ __forceinline__ int64_t floyd_slot_packed(int lane, int gbase, int K, int64_t deg,
+                                                     PhiloxKey key, uint64_t pos) {
+  const int64_t base = deg - K;
+  const int64_t j = base + lane;
+  const int64_t t = (int64_t)philox_bounded(key, pos, (uint64_t)lane, (uint64_t)j + 1);
+  bool dup = false;
+  for (int m = 0; m < K; ++m) {
+    const int64_t tm = __shfl(t, gbase + m, kWave);
+    dup |= (m < lane) & (tm == t);
+  }
+  const int64_t mi = t - base;  // slot whose j equals my t, if in [0, lane)
+  for (int m = 0; m < K; ++m) {
+    const int dm = __shfl((int)dup, gbase + m, kWave);
+    if (mi == m && m < lane) dup |= (dm != 0);
+  }
+  return dup ? j : t;
+}
+
+template <typename IdxT>
+__global__ __launch_bounds__(kBlock) void sample_uniform_packed_kernel(
+    const int64_t* __restrict__ indptr, int64_t num_cols,
+    const IdxT* __restrict__ indices, const int64_t* __restrict__ column_ids,
+    int64_t num_items, int fanout, int cols_per_wave, int replace, PhiloxKey key,
+    const int64_t* __restrict__ sub_indptr, int64_t* __restrict__ out_coo_col,
+    int64_t* __restrict__ out_indices, int64_t* __restrict__ out_select) {
+  const int wave_lane = threadIdx.x & (kWave - 1);
+  const int group = wave_lane / fanout;
+  const int lane = wave_lane - group * fanout;
+  const int64_t wave = ((int64_t)blockIdx.x * kBlock + threadIdx.x) / kWave;
+  const int64_t item = wave * cols_per_wave + group;
+  if (group >= cols_per_wave || item >= num_items) return;  // whole groups leave together
+  const int64_t c = column_ids ? column_ids[item] : item;
+  int64_t in_start;
+  const int64_t deg = column_degree(indptr, num_cols, c, &in_start);
+  if (deg == 0) return;
+  const int64_t out_start = sub_indptr[item];
+  int64_t p = -1;
+  if (replace) {
+    p = in_start + (int64_t)philox_bounded(key, (uint64_t)item, (uint64_t)lane, (uint64_t)deg);
+  } else if (deg <= fanout) {
+    if (lane < deg) p = in_start + lane;  // whole column, in order
+  } else {
+    p = in_start + floyd_slot_packed(lane, group * fanout, fanout, deg, key, (uint64_t)item);
+  }
+  if (p < 0) return;
+  const int64_t v = indices ? (int64_t)indices[p] : p;
+  out_indices[out_start + lane] = v;
+  out_select[out_start + lane] = p;
+  if (out_coo_col) out_coo_col[out_start + lane] = item;
+}
+
 template <int G, typename IdxT>
 static int launch_sample_uniform(const int64_t* indptr, int64_t num_cols,
                                  const IdxT* indices,
@@ -213,6 +273,16 @@ static int sample_uniform_fill(const int64_t* indptr, int64_t num_cols, const Id
     algo = fanout <= 64 ? GS_ALGO_FLOYD : GS_ALGO_RESERVOIR;
   const PhiloxKey key = make_key(seed, call_id);
   hipStream_t s = as_stream(stream);
+  if (fanout <= kWave && (replace || algo == GS_ALGO_FLOYD)) {
+    const int cols_per_wave = kWave / (int)fanout;
+    const int64_t waves = ceil_div(num_items, cols_per_wave);
+    GS_LAUNCH("sample_uniform", s,
+              sample_uniform_packed_kernel<IdxT><<<dim3((unsigned)ceil_div(waves * kWave, kBlock)),
+                                                   dim3(kBlock), 0, s>>>(
+                  indptr, num_cols, indices, column_ids, num_items, (int)fanout, cols_per_wave,
+                  replace, key, sub_indptr, out_coo_col, out_indices, out_select));
+    return GS_OK;
+  }
 #define GS_SAMPLE_ARGS                                                    \
   indptr, num_cols, indices, column_ids, num_items, fanout, replace, algo, \
       key, sub_indptr, out_coo_col, out_indices, out_select, s
