@@ -68,24 +68,31 @@ WORKLOADS = {
 
 
 def graphsage_step(be, indptr, indices, seeds, ptr, fanouts, seed, call_base, probs=None,
-                   cdf=None):
+                   cdf=None, by_pointer=False):
     """The pipeline, written once for both back ends (`be` is gsampler_amd.capi
     on torch CUDA tensors or oracle.binding on numpy arrays).  With `probs`
     (fp32 per edge) neighbours are drawn by weight instead of uniformly, through
-    the matrix's persistent CDF when `cdf` is given.
+    the matrix's persistent CDF when `cdf` is given.  `by_pointer`: the relabel
+    pass takes the column of an edge from the sampled matrix's column pointer,
+    and the sampler does not write a column per edge (same outputs).
     Returns per-layer (S, E, U) and the last layer's outputs."""
     sizes, last = [], None
     for layer, fanout in enumerate(fanouts):
         if probs is None:
             sub_indptr, coo_col, rows, sel = be.sample_uniform(
-                indptr, indices, seeds, fanout, False, 0, seed, call_base + layer)
+                indptr, indices, seeds, fanout, False, 0, seed, call_base + layer,
+                with_coo=not by_pointer)
         else:
             sub_indptr, coo_col, rows, sel = be.sample_weighted(
                 indptr, indices, probs, seeds, fanout, False, seed, call_base + layer,
-                cdf=cdf)
+                with_coo=not by_pointer, cdf=cdf)
         edge_ptr = sub_indptr[ptr]
-        uniq, uniq_ptr, out_row, out_col = be.unique_relabel(
-            seeds, rows, ptr, edge_ptr, coo_col)
+        if by_pointer:
+            uniq, uniq_ptr, out_row, out_col = be.unique_relabel(
+                seeds, rows, ptr, edge_ptr, col_indptr=sub_indptr)
+        else:
+            uniq, uniq_ptr, out_row, out_col = be.unique_relabel(
+                seeds, rows, ptr, edge_ptr, coo_col)
         sizes.append((int(seeds.shape[0]), int(rows.shape[0]), int(uniq.shape[0])))
         last = (uniq, uniq_ptr, out_row, out_col, sel)
         seeds, ptr = uniq, uniq_ptr
@@ -103,7 +110,10 @@ def kernel_bytes(name, sizes):
     for S, E, U in sizes:
         N = S + E
         total += {
-            "sample_uniform": 32 * S + 32 * E,   # seeds, indptr pair, sub_indptr, gather, 3 outputs
+            # the operator's interface: seeds, indptr pair, sub_indptr, gather, and row id,
+            # edge position and column of every edge (the column is delivered as the
+            # column pointer when the caller relabels by pointer: sampler_bytes_moved)
+            "sample_uniform": 32 * S + 32 * E,
             "sample_weighted_cdf": 32 * S + 32 * E,  # the same interface as the uniform sampler
             "col_count": 32 * S,                 # seeds, indptr pair, counts
             "unique_hist": 8 * N,                # keys in
@@ -111,9 +121,16 @@ def kernel_bytes(name, sizes):
             "unique_dedup": 12 * N,              # packed entries in, first positions out
             "unique_flag": 4 * N + N // 4,       # first positions in, rank words out
             "unique_fill": N // 4 + 16 * U,      # rank words + first keys in, frontier out
-            "unique_relabel": 28 * E,            # first position + column id in, row + col out
+            "unique_relabel": 20 * E + 8 * S,    # first position + column pointer in, row + col out
         }.get(name, 0)
     return total
+
+
+def sampler_bytes_moved(sizes):
+    """What the sampler launches of one step read and write when no column per edge is
+    stored (the relabel pass reads the column pointer instead): 8 bytes per edge less than
+    the operator's interface of kernel_bytes."""
+    return sum(32 * S + 24 * E for S, E, _ in sizes)
 
 
 def batch_graphsage_sampler(A, seeds, seeds_ptr, fanouts):
@@ -624,7 +641,7 @@ def main():
 
     def step(i):
         return graphsage_step(capi, indptr, pick_ids, seeds, ptr, fanouts, args.seed,
-                              i * len(fanouts), probs, cdf)
+                              i * len(fanouts), probs, cdf, by_pointer=True)
 
     if args.path == "api":
         step = api_step_factory(indptr, indices, seeds, ptr, fanouts, probs)
@@ -683,6 +700,13 @@ def main():
                     peak=HBM_PEAK_GBS, unit="GB/s", frac=round(dom["gbs"] / HBM_PEAK_GBS, 4),
                     traffic=traffic, avg_launch_ms=round(dom["avg_ms"], 4),
                     launches=dom["launches"])
+    if dom["kernel"] in ("sample_uniform", "sample_weighted_cdf") and dom["total_ms"] > 0:
+        # without the column per edge that this path does not store
+        moved = sum(sampler_bytes_moved(s) for s in prof_sizes)
+        roofline["achieved_without_edge_columns"] = round(
+            moved / (dom["total_ms"] * 1e-3) / 1e9, 1)
+        roofline["frac_without_edge_columns"] = round(
+            roofline["achieved_without_edge_columns"] / HBM_PEAK_GBS, 4)
     if traffic and dom["avg_ms"] > 0:
         roofline["traffic_source"] = traffic_source
         # the same bytes over this run's launch duration: the rate at the L2-fabric

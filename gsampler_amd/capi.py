@@ -57,7 +57,7 @@ SIGNATURES = {
     "gs_unique_workspace_bytes": (_sz, [_i64, _i64, _i64]),
     "gs_unique_count": (_int, [_p, _p, _i64, _p, _p, _i64, _i64, _p, _p, _p, _sz, _p]),
     "gs_unique_fill": (_int, [_p, _p, _i64, _p, _p, _i64, _i64, _p, _p, _p, _sz, _p]),
-    "gs_unique_relabel": (_int, [_p, _p, _i64, _p, _p, _i64, _i64, _p, _p, _p, _p,
+    "gs_unique_relabel": (_int, [_p, _p, _i64, _p, _p, _i64, _i64, _p, _p, _p, _p, _p,
                                  _sz, _p]),
     "gs_csc2coo": (_int, [_p, _i64, _i64, _p, _p]),
     "gs_sorted_to_indptr": (_int, [_p, _i64, _i64, _p, _p]),
@@ -332,8 +332,11 @@ def sample_uniform(indptr, indices, column_ids, fanout, replace=False,
 
 
 def unique_relabel(seeds, rows, seeds_ptr=None, rows_ptr=None, edge_col=None,
-                   want_row=True, want_col=True):
+                   want_row=True, want_col=True, col_indptr=None):
     """First-occurrence unique of seeds_b ++ rows_b per batch, plus relabel.
+
+    The column of an edge comes from `edge_col` (a position into `seeds` per
+    edge) or, for edges grouped by column, from `col_indptr` (len(seeds) + 1).
 
     -> (unique, unique_ptr, out_row | None, out_col | None)
     """
@@ -357,18 +360,25 @@ def unique_relabel(seeds, rows, seeds_ptr=None, rows_ptr=None, edge_col=None,
     count = count.arm() if count else _Fetched(unique_ptr)
     size = S + E if S + E <= _BOUND_LIMIT else count.get()   # U <= S + E
     unique = torch.empty(size, dtype=torch.int64, device=dev)
-    want_col = want_col and edge_col is not None
+    want_col = want_col and (edge_col is not None or col_indptr is not None)
     out_row = torch.empty(E, dtype=torch.int64, device=dev) if want_row else None
     out_col = torch.empty(E, dtype=torch.int64, device=dev) if want_col else None
     if edge_col is not None:
         edge_col = _i64t(edge_col, "edge_col")
+    if col_indptr is not None:
+        if edge_col is not None:
+            raise ValueError("unique_relabel: give edge_col or col_indptr, not both")
+        col_indptr = _i64t(col_indptr, "col_indptr")
+        if col_indptr.numel() != S + 1:
+            raise ValueError(f"unique_relabel: col_indptr has {col_indptr.numel()} entries "
+                             f"for {S} seeds")
     check(l.gs_unique_fill(_ptr(seeds), sp, S, _ptr(rows), rp, E, B,
                            unique_ptr.data_ptr(), _ptr(unique), ws.data_ptr(),
                            ws.numel(), _stream()))
     if want_row or want_col:
         check(l.gs_unique_relabel(_ptr(seeds), sp, S, _ptr(rows), rp, E, B,
-                                  _ptr(edge_col), _ptr(out_row), _ptr(out_col),
-                                  ws.data_ptr(), ws.numel(), _stream()))
+                                  _ptr(edge_col), _ptr(col_indptr), _ptr(out_row),
+                                  _ptr(out_col), ws.data_ptr(), ws.numel(), _stream()))
     total = count.get()
     return unique[:total], unique_ptr, out_row, out_col
 

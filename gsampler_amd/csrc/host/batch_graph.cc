@@ -143,7 +143,9 @@ GraphAndIndex Graph::BatchFusedSlicingSampling(torch::Tensor seeds,
   col_bptr = ids(col_bptr, "col_bptr");
   BatchOffsets::check(col_bptr, seeds.numel(), "BatchFusedSlicingSampling");
   EdgeCount::HintScope batch(col_bptr);  // the sampler leaves the edge pointer here
-  auto ret = FusedSlicingSampling(1, seeds, fanout, replace, kCSC, kCSC | kCOO);
+  // compressed by column only: the relabel pass reads the column pointer, and
+  // the coordinate form is expanded from it if somebody asks
+  auto ret = FusedSlicingSampling(1, seeds, fanout, replace, kCSC, kCSC);
   Graph& g = *std::get<0>(ret);
   g.col_bptr_ = col_bptr;
   g.orig_col_ids_ = ids(seeds, "seeds");
@@ -153,19 +155,29 @@ GraphAndIndex Graph::BatchFusedSlicingSampling(torch::Tensor seeds,
   return ret;
 }
 
+// A compressed-by-column matrix whose coordinate form nobody has asked for
+// hands over its column pointer; the coordinate form is then not built at all.
+Graph::ColumnOrderedEdges Graph::column_ordered_edges(const char* who) {
+  if (csc_ && !coo_) return {csc_->indices, {}, csc_->indptr, csc_->e_ids};
+  CreateSparseFormat(kCOO);
+  TORCH_CHECK(coo_->col_sorted, who, ": the COO format must be column-sorted");
+  return {coo_->row, coo_->col, {}, coo_->e_ids};
+}
+
 // Global row ids of every edge as the relabel pass needs them: rows of an
 // encoded (compacted) batch graph are decoded back through row_ids.
-torch::Tensor Graph::batch_rows_for_relabel(const torch::Tensor& row_ids) {
-  if (row_ids.numel() == 0) return coo_->row;
-  if (!(mapped_out_.defined() && mapped_from_.is_same(coo_->row) &&
+torch::Tensor Graph::batch_rows_for_relabel(const torch::Tensor& edge_rows,
+                                            const torch::Tensor& row_ids) {
+  if (row_ids.numel() == 0) return edge_rows;
+  if (!(mapped_out_.defined() && mapped_from_.is_same(edge_rows) &&
         mapped_by_.is_same(row_ids))) {
-    torch::Tensor enc = ids(row_ids, "row_ids").index_select(0, coo_->row);
+    torch::Tensor enc = ids(row_ids, "row_ids").index_select(0, edge_rows);
     const int64_t B = edge_bptr_.numel() - 1;
     torch::Tensor orig = enc;
     if (row_encoding_size_ > 0)
       orig = std::get<1>(batch_offsets(enc, B, row_encoding_size_));
     mapped_out_ = orig;
-    mapped_from_ = coo_->row;
+    mapped_from_ = edge_rows;
     mapped_by_ = row_ids;
   }
   return mapped_out_;
@@ -176,26 +188,32 @@ torch::Tensor Graph::batch_rows_for_relabel(const torch::Tensor& row_ids) {
 // returns: f.frontier() waits for it.
 Graph::Frontier& Graph::batch_relabel_launch(torch::Tensor& col_seeds,
                                              const torch::Tensor& row_ids,
-                                             torch::Tensor* out_row, torch::Tensor* out_col) {
+                                             torch::Tensor* out_row, torch::Tensor* out_col,
+                                             c10::optional<torch::Tensor>* e_ids) {
   TORCH_CHECK(edge_bptr_.defined() && edge_bptr_.numel() > 0,
               "BatchGraphRelabel: the graph has no edge batch pointer");
-  CreateSparseFormat(kCOO);
-  TORCH_CHECK(coo_->col_sorted,
-              "BatchGraphRelabel: the COO format must be column-sorted");
+  ColumnOrderedEdges edges = column_ordered_edges("BatchGraphRelabel");
   col_seeds = ids(col_seeds, "col_seeds");
   // the kernels read seeds[col_bptr[b] ...]: the seeds must be the ones the
   // batch pointer was recorded for
   BatchOffsets::check(col_bptr_, col_seeds.numel(), "BatchGraphRelabel");
-  torch::Tensor rows = batch_rows_for_relabel(row_ids);
+  if (edges.col_indptr.defined())
+    TORCH_CHECK(edges.col_indptr.numel() == col_seeds.numel() + 1,
+                "BatchGraphRelabel: ", col_seeds.numel(), " seeds for a matrix of ",
+                edges.col_indptr.numel() - 1, " columns");
+  torch::Tensor rows = batch_rows_for_relabel(edges.row, row_ids);
   Frontier& f = frontier_for(col_seeds, rows, col_bptr_, edge_bptr_);
   const int64_t E = rows.numel(), B = f.num_batches;
   *out_row = new_ids(E, rows);
   *out_col = new_ids(E, rows);
   GS_CALL(gs_unique_relabel(cptr(col_seeds), cptr(col_bptr_), col_seeds.numel(),
-                            cptr(rows), cptr(edge_bptr_), E, B, cptr(coo_->col),
+                            cptr(rows), cptr(edge_bptr_), E, B,
+                            edges.col.defined() ? cptr(edges.col) : nullptr,
+                            edges.col_indptr.defined() ? cptr(edges.col_indptr) : nullptr,
                             mptr(*out_row), mptr(*out_col),
                             f.workspace.data_ptr(), f.workspace.numel(),
                             cur_stream()));
+  if (e_ids) *e_ids = edges.e_ids;
   return f;
 }
 
@@ -203,20 +221,19 @@ std::tuple<torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor,
            c10::optional<torch::Tensor>, torch::Tensor>
 Graph::BatchGraphRelabel(torch::Tensor col_seeds, torch::Tensor row_ids) {
   torch::Tensor out_row, out_col;
-  Frontier& f = batch_relabel_launch(col_seeds, row_ids, &out_row, &out_col);
-  return {f.frontier(), f.unique_ptr, out_row, out_col, coo_->e_ids, edge_bptr_};
+  c10::optional<torch::Tensor> e_ids;
+  Frontier& f = batch_relabel_launch(col_seeds, row_ids, &out_row, &out_col, &e_ids);
+  return {f.frontier(), f.unique_ptr, out_row, out_col, e_ids, edge_bptr_};
 }
 
 std::tuple<torch::Tensor, torch::Tensor> Graph::BatchGetValidNodes(
     torch::Tensor col_seeds, torch::Tensor row_ids) {
   TORCH_CHECK(edge_bptr_.defined() && edge_bptr_.numel() > 0,
               "BatchGetValidNodes: the graph has no edge batch pointer");
-  CreateSparseFormat(kCOO);
-  TORCH_CHECK(coo_->col_sorted,
-              "BatchGetValidNodes: the COO format must be column-sorted");
+  ColumnOrderedEdges edges = column_ordered_edges("BatchGetValidNodes");
   col_seeds = ids(col_seeds, "col_seeds");
   BatchOffsets::check(col_bptr_, col_seeds.numel(), "BatchGetValidNodes");
-  torch::Tensor rows = batch_rows_for_relabel(row_ids);
+  torch::Tensor rows = batch_rows_for_relabel(edges.row, row_ids);
   Frontier& f = frontier_for(col_seeds, rows, col_bptr_, edge_bptr_);
   return {f.frontier(), f.unique_ptr};
 }

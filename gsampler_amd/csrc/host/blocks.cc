@@ -111,20 +111,19 @@ c10::intrusive_ptr<BlockBatch> Graph::BatchBlocks(torch::Tensor col_seeds,
               "BatchBlocks: the graph has no column batch pointer");
   auto out = c10::make_intrusive<BlockBatch>();
   out->num_batches = col_bptr_.numel() - 1;
-  CreateSparseFormat(kCOO);
   if (csc_) {
     out->sampled_indptr = csc_->indptr;
   } else {
+    CreateSparseFormat(kCOO);
     TORCH_CHECK(coo_->col_sorted, "BatchBlocks: the COO format must be column-sorted");
     out->sampled_indptr = new_ids(num_cols_ + 1, coo_->col);
     GS_CALL(gs_sorted_to_indptr(cptr(coo_->col), coo_->col.numel(), num_cols_,
                                 mptr(out->sampled_indptr), cur_stream()));
   }
-  Frontier& f = batch_relabel_launch(col_seeds, row_ids, &out->row, &out->col);
+  Frontier& f = batch_relabel_launch(col_seeds, row_ids, &out->row, &out->col, &out->e_ids);
   out->col_seeds = col_seeds;
   out->num_dst_total = col_seeds.numel();
   out->frontier_ptr = f.unique_ptr;
-  out->e_ids = coo_->e_ids;
   out->coo_ptr = edge_bptr_;
   out->col_bptr = col_bptr_;
   // (the pointer arrays are on their way to the host or there already: the

@@ -489,7 +489,7 @@ Graph::ListLabels& Graph::list_labels_for(const torch::Tensor& col_seeds,
   Frontier& f = frontier_for(col_seeds, rows, {}, {});
   torch::Tensor labels = new_ids(R + S, base);
   GS_CALL(gs_unique_relabel(cptr(col_seeds), nullptr, S, cptr(rows), nullptr, R + S, 1,
-                            nullptr, mptr(labels), nullptr, f.workspace.data_ptr(),
+                            nullptr, nullptr, mptr(labels), nullptr, f.workspace.data_ptr(),
                             f.workspace.numel(), cur_stream()));
   out->label_by_local = new_ids(R, base);
   out->label_by_local.index_copy_(0, order, labels.narrow(0, 0, R));
@@ -516,7 +516,7 @@ Graph::GraphRelabel(torch::Tensor col_seeds, torch::Tensor row_ids) {
   const int64_t E = rows.numel();
   torch::Tensor out_row = new_ids(E, rows), out_col = new_ids(E, rows);
   GS_CALL(gs_unique_relabel(cptr(col_seeds), nullptr, col_seeds.numel(),
-                            cptr(rows), nullptr, E, 1, cptr(coo_->col),
+                            cptr(rows), nullptr, E, 1, cptr(coo_->col), nullptr,
                             mptr(out_row), mptr(out_col),
                             f.workspace.data_ptr(), f.workspace.numel(),
                             cur_stream()));

@@ -264,7 +264,8 @@ class Graph : public torch::CustomClassHolder {
                          const torch::Tensor& seeds_ptr,
                          const torch::Tensor& rows_ptr);
   Frontier& batch_relabel_launch(torch::Tensor& col_seeds, const torch::Tensor& row_ids,
-                                 torch::Tensor* out_row, torch::Tensor* out_col);
+                                 torch::Tensor* out_row, torch::Tensor* out_col,
+                                 c10::optional<torch::Tensor>* e_ids);
 
   const Compressed& compressed(int64_t format);
   // CDF of edge_probs in the edge order of `format` (cached per weights tensor).
@@ -283,7 +284,17 @@ class Graph : public torch::CustomClassHolder {
   torch::Tensor edge_index(const c10::optional<torch::Tensor>& parent_eids,
                            const torch::Tensor& select);
   void copy_batch_state_to(Graph& g, bool with_rows);
-  torch::Tensor batch_rows_for_relabel(const torch::Tensor& row_ids);
+  // The edges in column order, for the relabel pass: their row ids and either
+  // the column of every edge or the column pointer that implies it.
+  struct ColumnOrderedEdges {
+    torch::Tensor row;
+    torch::Tensor col;         // undefined when col_indptr is given
+    torch::Tensor col_indptr;  // undefined when col is given
+    c10::optional<torch::Tensor> e_ids;
+  };
+  ColumnOrderedEdges column_ordered_edges(const char* who);
+  torch::Tensor batch_rows_for_relabel(const torch::Tensor& edge_rows,
+                                       const torch::Tensor& row_ids);
 
   int64_t num_rows_ = 0, num_cols_ = 0, num_edges_ = 0;
   std::shared_ptr<Compressed> csc_, csr_;

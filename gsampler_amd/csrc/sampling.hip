@@ -1,10 +1,12 @@
 // sampling.hip -- uniform per-column sampling, optionally fused with the
 // column slice (the GraphSAGE kernel).
 //
-// Work mapping: a group of G lanes (G a power of two <= 64, a slice of one
-// wavefront) owns one requested column; a wavefront therefore keeps 64 / G
-// independent columns -- and their dependent seed -> indptr -> indices load
-// chains -- in flight at once.  Group-level exchange uses wavefront shuffles
+// Work mapping: a slice of one wavefront owns one requested column, so that a
+// wavefront keeps several independent columns -- and their dependent seed ->
+// indptr -> indices load chains -- in flight at once.  With one lane per
+// output slot (fanout <= 64, Floyd's rule or sampling with replacement) the
+// slice is exactly `fanout` lanes; otherwise it is a power-of-two group that
+// strides over the slots.  Exchange inside a slice uses wavefront shuffles
 // only, so divergent columns never meet at a block barrier.
 #include "common.h"
 
@@ -69,113 +71,14 @@ __device__ __forceinline__ void sample_column_generic(
   }
 }
 
-// Floyd's subset sampling, one lane per output slot (fanout <= G).  Slot i
-// draws t_i in [0, j_i], j_i = deg - fanout + i, and keeps t_i unless an
-// earlier slot already holds it, in which case it keeps j_i.  "Already held"
-// <=> some earlier slot drew the same t, or t_i equals the j_m of an earlier
-// slot m that fell back to j_m; m is then unique (m = t_i - (deg - fanout)),
-// so the fall-back flags form a chain that is settled by visiting slots in
-// increasing order.  Returns the slot's offset inside the column.
-template <int G>
-__device__ __forceinline__ int64_t floyd_slot(int lane, int K, int64_t deg,
-                                              PhiloxKey key, uint64_t pos) {
-  const int64_t base = deg - K;
-  const int64_t j = base + lane;
-  int64_t t = -1;
-  if (lane < K)
-    t = (int64_t)philox_bounded(key, pos, (uint64_t)lane, (uint64_t)j + 1);
-  bool dup = false;
-  for (int m = 0; m < K; ++m) {
-    int64_t tm = __shfl(t, m, G);
-    dup |= (m < lane) & (tm == t);
-  }
-  const int64_t mi = t - base;  // slot whose j equals my t, if in [0, lane)
-  for (int m = 0; m < K; ++m) {
-    int dm = __shfl((int)dup, m, G);
-    if (mi == m && m < lane) dup |= (dm != 0);
-  }
-  return dup ? j : t;
-}
-
-// A group of G lanes takes U consecutive columns.  With fanout <= G every
-// output slot has a lane of its own, and the U columns go through the stages
-// together: all column ids, then all indptr pairs, then all picks, then all
-// gathers, so that a wavefront keeps U * 64 / G dependent load chains in
-// flight instead of 64 / G.  On a 124M-edge power-law graph U = 2 and U = 4
-// measured 3 % and 20 % slower than U = 1: at full occupancy the kernel is
-// bound by the sectors its random gathers pull in, not by their latency.
-template <int G, int U, typename IdxT>
-__global__ __launch_bounds__(kBlock) void sample_uniform_kernel(
-    const int64_t* __restrict__ indptr, int64_t num_cols,
-    const IdxT* __restrict__ indices, const int64_t* __restrict__ column_ids,
-    int64_t num_items, int64_t fanout, int replace, int algo, PhiloxKey key,
-    const int64_t* __restrict__ sub_indptr, int64_t* __restrict__ out_coo_col,
-    int64_t* __restrict__ out_indices, int64_t* __restrict__ out_select) {
-  const int lane = threadIdx.x & (G - 1);
-  const int64_t item0 =
-      (((int64_t)blockIdx.x * kBlock + threadIdx.x) / G) * U;
-  if (item0 >= num_items) return;  // whole groups leave together
-
-  int64_t c[U], in_start[U], deg[U], out_start[U];
-#pragma unroll
-  for (int u = 0; u < U; ++u) {
-    const int64_t item = item0 + u;
-    c[u] = item < num_items ? (column_ids ? column_ids[item] : item) : -1;
-  }
-#pragma unroll
-  for (int u = 0; u < U; ++u)
-    deg[u] = column_degree(indptr, num_cols, c[u], &in_start[u]);
-#pragma unroll
-  for (int u = 0; u < U; ++u)
-    out_start[u] = deg[u] > 0 ? sub_indptr[item0 + u] : 0;
-
-  const bool slot_per_lane = fanout <= G;
-  int64_t p[U];
-#pragma unroll
-  for (int u = 0; u < U; ++u) {
-    p[u] = -1;  // no slot for this lane
-    if (deg[u] == 0) continue;
-    const int64_t item = item0 + u;
-    if (!slot_per_lane ||
-        (!replace && deg[u] > fanout && algo != GS_ALGO_FLOYD)) {
-      sample_column_generic<G, IdxT>(lane, item, in_start[u], deg[u], out_start[u],
-                               indices, fanout, replace, key, out_coo_col,
-                               out_indices, out_select);
-    } else if (replace) {
-      if (lane < fanout)
-        p[u] = in_start[u] + (int64_t)philox_bounded(key, (uint64_t)item,
-                                                     (uint64_t)lane,
-                                                     (uint64_t)deg[u]);
-    } else if (deg[u] <= fanout) {
-      if (lane < deg[u]) p[u] = in_start[u] + lane;  // whole column, in order
-    } else {
-      const int64_t off =
-          floyd_slot<G>(lane, (int)fanout, deg[u], key, (uint64_t)item);
-      if (lane < fanout) p[u] = in_start[u] + off;
-    }
-  }
-  int64_t v[U];
-#pragma unroll
-  for (int u = 0; u < U; ++u)
-    v[u] = (p[u] >= 0 && indices) ? (int64_t)indices[p[u]] : p[u];
-#pragma unroll
-  for (int u = 0; u < U; ++u) {
-    if (p[u] < 0) continue;
-    out_indices[out_start[u] + lane] = v[u];
-    out_select[out_start[u] + lane] = p[u];
-    if (out_coo_col) out_coo_col[out_start[u] + lane] = item0 + u;
-  }
-}
-
-// The same columns with the lanes packed: a column takes exactly `fanout` lanes
-// (one per output slot), so a wavefront holds 64 / fanout columns -- twelve at
-// fanout 5 where power-of-two groups hold eight, six instead of four at fanout
-// 10.  The kernel is bound by the instructions it issues (a Philox call per
-// slot, the group exchanges of Floyd's rule, three stores), not by the lines
-// behind its picks, and every idle lane of a group is issue bandwidth lost.
-// Covers what gives every slot a lane of its own: sampling with replacement,
-// whole columns, Floyd's rule; picks and outputs are those of
-// sample_uniform_kernel (the same draws: position = column, draw = slot).
+// Floyd's subset sampling, one lane per output slot: slot i of a column is lane
+// gbase + i of the wavefront (K <= 64 slots).  Slot i draws t_i in [0, j_i],
+// j_i = deg - K + i, and keeps t_i unless an earlier slot already holds it, in
+// which case it keeps j_i.  "Already held" <=> some earlier slot drew the same
+// t, or t_i equals the j_m of an earlier slot m that fell back to j_m; m is
+// then unique (m = t_i - (deg - K)), so the fall-back flags form a chain that
+// is settled by visiting slots in increasing order.  Returns the slot's offset
+// inside the column.
 __device__ __forceinline__ int64_t floyd_slot_packed(int lane, int gbase, int K, int64_t deg,
                                                      PhiloxKey key, uint64_t pos) {
   const int64_t base = deg - K;
@@ -194,6 +97,12 @@ __device__ __forceinline__ int64_t floyd_slot_packed(int lane, int gbase, int K,
   return dup ? j : t;
 }
 
+// One lane per output slot, a column on exactly `fanout` consecutive lanes: a
+// wavefront holds 64 / fanout columns (twelve at fanout 5, where power-of-two
+// groups would hold eight).  Lanes past the last whole slice idle.  On a
+// 124M-edge power-law graph the kernel moves about 6 TB/s through the memory
+// fabric, nearly all of it the 128-byte lines behind 4- or 8-byte picks;
+// giving a slice several columns to pipeline measured 3 % to 20 % slower.
 template <typename IdxT>
 __global__ __launch_bounds__(kBlock) void sample_uniform_packed_kernel(
     const int64_t* __restrict__ indptr, int64_t num_cols,
@@ -204,7 +113,10 @@ __global__ __launch_bounds__(kBlock) void sample_uniform_packed_kernel(
   const int wave_lane = threadIdx.x & (kWave - 1);
   const int group = wave_lane / fanout;
   const int lane = wave_lane - group * fanout;
-  const int64_t wave = ((int64_t)blockIdx.x * kBlock + threadIdx.x) / kWave;
+  // die x (work-groups x, x + 8, ...) takes the x-th eighth of the columns in order
+  const int64_t per_die = gridDim.x / 8;
+  const int64_t block = (int64_t)(blockIdx.x % 8) * per_die + blockIdx.x / 8;
+  const int64_t wave = (block * kBlock + threadIdx.x) / kWave;
   const int64_t item = wave * cols_per_wave + group;
   if (group >= cols_per_wave || item >= num_items) return;  // whole groups leave together
   const int64_t c = column_ids ? column_ids[item] : item;
@@ -227,21 +139,39 @@ __global__ __launch_bounds__(kBlock) void sample_uniform_packed_kernel(
   if (out_coo_col) out_coo_col[out_start + lane] = item;
 }
 
+// Any fanout, any algorithm: a group of G lanes (a power of two) owns a column
+// and strides over its slots.  The path of the reservoir algorithm and of
+// fanouts above 64.
 template <int G, typename IdxT>
-static int launch_sample_uniform(const int64_t* indptr, int64_t num_cols,
-                                 const IdxT* indices,
-                                 const int64_t* column_ids, int64_t num_items,
-                                 int64_t fanout, int replace, int algo,
-                                 PhiloxKey key, const int64_t* sub_indptr,
-                                 int64_t* out_coo_col, int64_t* out_indices,
-                                 int64_t* out_select, hipStream_t stream) {
-  // one column per lane group (see the note on U above the kernel)
+__global__ __launch_bounds__(kBlock) void sample_uniform_strided_kernel(
+    const int64_t* __restrict__ indptr, int64_t num_cols,
+    const IdxT* __restrict__ indices, const int64_t* __restrict__ column_ids,
+    int64_t num_items, int64_t fanout, int replace, PhiloxKey key,
+    const int64_t* __restrict__ sub_indptr, int64_t* __restrict__ out_coo_col,
+    int64_t* __restrict__ out_indices, int64_t* __restrict__ out_select) {
+  const int lane = threadIdx.x & (G - 1);
+  const int64_t item = ((int64_t)blockIdx.x * kBlock + threadIdx.x) / G;
+  if (item >= num_items) return;  // whole groups leave together
+  const int64_t c = column_ids ? column_ids[item] : item;
+  int64_t in_start;
+  const int64_t deg = column_degree(indptr, num_cols, c, &in_start);
+  if (deg == 0) return;
+  sample_column_generic<G, IdxT>(lane, item, in_start, deg, sub_indptr[item], indices, fanout,
+                                 replace, key, out_coo_col, out_indices, out_select);
+}
+
+template <int G, typename IdxT>
+static int launch_sample_strided(const int64_t* indptr, int64_t num_cols, const IdxT* indices,
+                                 const int64_t* column_ids, int64_t num_items, int64_t fanout,
+                                 int replace, PhiloxKey key, const int64_t* sub_indptr,
+                                 int64_t* out_coo_col, int64_t* out_indices, int64_t* out_select,
+                                 hipStream_t stream) {
   const int64_t blocks = ceil_div(num_items * G, kBlock);
   GS_LAUNCH("sample_uniform", stream,
-            (sample_uniform_kernel<G, 1, IdxT>)<<<dim3((unsigned)blocks), dim3(kBlock), 0,
-                                                stream>>>(
-                indptr, num_cols, indices, column_ids, num_items, fanout, replace,
-                algo, key, sub_indptr, out_coo_col, out_indices, out_select));
+            (sample_uniform_strided_kernel<G, IdxT>)<<<dim3((unsigned)blocks), dim3(kBlock), 0,
+                                                      stream>>>(
+                indptr, num_cols, indices, column_ids, num_items, fanout, replace, key,
+                sub_indptr, out_coo_col, out_indices, out_select));
   return GS_OK;
 }
 
@@ -277,19 +207,19 @@ static int sample_uniform_fill(const int64_t* indptr, int64_t num_cols, const Id
     const int cols_per_wave = kWave / (int)fanout;
     const int64_t waves = ceil_div(num_items, cols_per_wave);
     GS_LAUNCH("sample_uniform", s,
-              sample_uniform_packed_kernel<IdxT><<<dim3((unsigned)ceil_div(waves * kWave, kBlock)),
+              sample_uniform_packed_kernel<IdxT><<<dim3((unsigned)(ceil_div(ceil_div(waves * kWave, kBlock), 8) * 8)),
                                                    dim3(kBlock), 0, s>>>(
                   indptr, num_cols, indices, column_ids, num_items, (int)fanout, cols_per_wave,
                   replace, key, sub_indptr, out_coo_col, out_indices, out_select));
     return GS_OK;
   }
-#define GS_SAMPLE_ARGS                                                    \
-  indptr, num_cols, indices, column_ids, num_items, fanout, replace, algo, \
-      key, sub_indptr, out_coo_col, out_indices, out_select, s
-  if (fanout <= 8) return launch_sample_uniform<8, IdxT>(GS_SAMPLE_ARGS);
-  if (fanout <= 16) return launch_sample_uniform<16, IdxT>(GS_SAMPLE_ARGS);
-  if (fanout <= 32) return launch_sample_uniform<32, IdxT>(GS_SAMPLE_ARGS);
-  return launch_sample_uniform<64, IdxT>(GS_SAMPLE_ARGS);
+#define GS_SAMPLE_ARGS                                                          \
+  indptr, num_cols, indices, column_ids, num_items, fanout, replace, key, sub_indptr, \
+      out_coo_col, out_indices, out_select, s
+  if (fanout <= 8) return launch_sample_strided<8, IdxT>(GS_SAMPLE_ARGS);
+  if (fanout <= 16) return launch_sample_strided<16, IdxT>(GS_SAMPLE_ARGS);
+  if (fanout <= 32) return launch_sample_strided<32, IdxT>(GS_SAMPLE_ARGS);
+  return launch_sample_strided<64, IdxT>(GS_SAMPLE_ARGS);
 #undef GS_SAMPLE_ARGS
 }
 }  // namespace gs

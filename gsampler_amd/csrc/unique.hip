@@ -1013,18 +1013,100 @@ __global__ __launch_bounds__(kBlock) void unique_fill_kernel(
 }
 
 // ---------------------------------------------------------------- relabel
+// The largest c in [0, n) with ptr[c] <= x, for nondecreasing ptr with
+// ptr[0] <= x; found by one wavefront, 64 probes a round.
+__device__ __forceinline__ int64_t wave_last_at_most(const int64_t* __restrict__ ptr, int64_t n,
+                                                     int64_t x) {
+  int64_t lo = 0, hi = n;  // ptr[lo] <= x; hi == n or ptr[hi] > x
+  while (hi - lo > 1) {
+    const int64_t step = (hi - lo + kWave - 1) / kWave;
+    const int64_t c = lo + (int64_t)(lane_id() + 1) * step;
+    const bool ok = c < hi && ptr[c] <= x;
+    const int hits = __popcll(__ballot(ok));  // ok is monotone over the lanes
+    const int64_t next_hi = lo + (int64_t)(hits + 1) * step;
+    lo += (int64_t)hits * step;
+    if (next_hi < hi) hi = next_hi;
+  }
+  return lo;
+}
+
+// The column of every edge of a tile from the column pointer: edge e belongs
+// to the last column c with col_indptr[c] <= e.  Two wavefronts find the
+// columns of the tile's first and last edge among [col_begin, col_end), the
+// columns of the tile's batches; every column that starts inside
+// the tile marks its first edge with its number (of several empty columns at
+// one edge the last, the owner, wins), and a running maximum over the tile
+// carries the marks forward.  Leaves column - c_lo in head[] and returns c_lo.
+__device__ __forceinline__ int64_t tile_columns(const int64_t* __restrict__ col_indptr,
+                                                int64_t col_begin, int64_t col_end, int64_t e0,
+                                                int64_t e1, int32_t* head, int64_t* ends,
+                                                int32_t* wave_max) {
+  static_assert(kRelabelItems % 4 == 0, "a thread scans whole int4s of head[]");
+  constexpr int kQuads = kRelabelItems / 4;
+  const int wave = threadIdx.x / kWave;
+  int4* quads = reinterpret_cast<int4*>(head) + threadIdx.x * kQuads;
+#pragma unroll
+  for (int q = 0; q < kQuads; ++q) quads[q] = make_int4(0, 0, 0, 0);
+  if (wave < 2) {
+    const int64_t c = wave_last_at_most(col_indptr + col_begin, col_end - col_begin,
+                                        wave == 0 ? e0 : e1 - 1);
+    if (lane_id() == 0) ends[wave] = col_begin + c;
+  }
+  __syncthreads();
+  const int64_t c_lo = ends[0], c_hi = ends[1];
+  for (int64_t c = c_lo + 1 + threadIdx.x; c <= c_hi; c += kBlock) {
+    const int64_t off = col_indptr[c] - e0;
+    if (off > 0 && off < kRelabelTile) atomicMax(&head[off], (int32_t)(c - c_lo));
+  }
+  __syncthreads();
+  int4 m[kQuads];
+  int32_t run = 0;  // running maximum over this thread's chunk, then over the lanes' chunks
+#pragma unroll
+  for (int q = 0; q < kQuads; ++q) {
+    m[q] = quads[q];
+    m[q].x = max(m[q].x, run);
+    m[q].y = max(m[q].y, m[q].x);
+    m[q].z = max(m[q].z, m[q].y);
+    m[q].w = max(m[q].w, m[q].z);
+    run = m[q].w;
+  }
+#pragma unroll
+  for (int d = 1; d < kWave; d <<= 1) {
+    const int32_t o = __shfl_up(run, d, kWave);
+    if (lane_id() >= d) run = max(run, o);
+  }
+  if (lane_id() == kWave - 1) wave_max[wave] = run;
+  int32_t before = __shfl_up(run, 1, kWave);
+  if (lane_id() == 0) before = 0;
+  __syncthreads();
+  for (int w = 0; w < wave; ++w) before = max(before, wave_max[w]);
+#pragma unroll
+  for (int q = 0; q < kQuads; ++q)
+    quads[q] = make_int4(max(m[q].x, before), max(m[q].y, before), max(m[q].z, before),
+                         max(m[q].w, before));
+  __syncthreads();
+  return c_lo;
+}
+
+// kByIndptr: the edges are grouped by column and col_indptr (k.S + 1 entries)
+// says where each column's edges start; edge_col is not read.
+template <bool kByIndptr>
 __global__ __launch_bounds__(kBlock) void unique_relabel_kernel(
     Keys k, const int32_t* __restrict__ etile_batch,
     const BatchInfo* __restrict__ batch, const uint32_t* __restrict__ first,
     const RankWord* __restrict__ words, const int64_t* __restrict__ group_off,
     const int64_t* __restrict__ unique_ptr, const int64_t* __restrict__ edge_col,
-    int64_t* __restrict__ out_row, int64_t* __restrict__ out_col, int remap) {
+    const int64_t* __restrict__ col_indptr, int64_t* __restrict__ out_row,
+    int64_t* __restrict__ out_col, int remap) {
   const int64_t num_tiles = ceil_div_dev(k.E, kRelabelTile);
   const int64_t tile = unit_of_block(num_tiles, remap);
   if (tile >= num_tiles) return;
   const int64_t e0 = tile * kRelabelTile;
   const BatchSpan span = batch_span(etile_batch, tile);
   int64_t col[kRelabelItems];
+  __shared__ __align__(16) int32_t head[kByIndptr ? kRelabelTile : 4];
+  __shared__ int64_t ends[2];
+  __shared__ int32_t wave_max[kBlock / kWave];
   uint32_t row_first[kRelabelItems];
   BatchInfo info = batch[span.lo];
   int64_t rank0 = unique_ptr[span.lo];
@@ -1045,7 +1127,16 @@ __global__ __launch_bounds__(kBlock) void unique_relabel_kernel(
     // row key e of batch b sits at flat position
     //   fb + (seeds of b) + (e - rows_ptr[b])  =  e + seeds_ptr[b + 1]
     if (out_row) row_first[i] = first[e + info.s_lo + info.ns];
-    if (out_col) col[i] = edge_col[e];
+    if (out_col && !kByIndptr) col[i] = edge_col[e];
+  }
+  if (kByIndptr && out_col) {
+    // (after the loads above have been issued: they travel during the search)
+    const int64_t e1 = e0 + kRelabelTile < k.E ? e0 + kRelabelTile : k.E;
+    const BatchInfo last = batch[span.hi];
+    const int64_t c_lo = tile_columns(col_indptr, batch[span.lo].s_lo, last.s_lo + last.ns, e0,
+                                      e1, head, ends, wave_max);
+#pragma unroll
+    for (int i = 0; i < kRelabelItems; ++i) col[i] = c_lo + head[i * kBlock + threadIdx.x];
   }
 #pragma unroll
   for (int i = 0; i < kRelabelItems; ++i) {
@@ -1206,26 +1297,34 @@ int gs_unique_relabel(const int64_t* seeds, const int64_t* seeds_ptr,
                       int64_t num_seeds, const int64_t* rows,
                       const int64_t* rows_ptr, int64_t num_rows_keys,
                       int64_t num_batches, const int64_t* edge_col,
-                      int64_t* out_row, int64_t* out_col, void* workspace,
-                      size_t workspace_bytes, gs_stream_t stream) {
+                      const int64_t* col_indptr, int64_t* out_row, int64_t* out_col,
+                      void* workspace, size_t workspace_bytes, gs_stream_t stream) {
   using namespace gs;
   const int64_t S = num_seeds, E = num_rows_keys, B = num_batches;
   int rc = check_unique_args(seeds, seeds_ptr, S, rows, rows_ptr, E, B);
   if (rc != GS_OK) return rc;
-  GS_REQUIRE(out_col == nullptr || edge_col != nullptr,
-             "unique_relabel: out_col needs edge_col");
+  GS_REQUIRE(out_col == nullptr || E == 0 || (edge_col != nullptr) != (col_indptr != nullptr),
+             "unique_relabel: out_col needs edge_col or col_indptr (one of them)");
+  GS_REQUIRE(col_indptr == nullptr || E == 0 || S > 0,
+             "unique_relabel: %lld edges grouped by column but no seeds", (long long)E);
   UniqueWs w = carve_unique(workspace, S, E, B);
   if ((rc = check_workspace(w, workspace, workspace_bytes)) != GS_OK) return rc;
   hipStream_t s = as_stream(stream);
   const UniqueTuning tn = tuning();
   if (E > 0 && (out_row || out_col)) {
     const Keys k{seeds, seeds_ptr, S, rows, rows_ptr, E, B};
-    GS_LAUNCH("unique_relabel", s,
-              unique_relabel_kernel<<<dim3((unsigned)grid_for_units(
-                                          ceil_div(E, kRelabelTile), tn.remap)),
-                                      dim3(kBlock), 0, s>>>(
-                  k, w.etile_batch, w.batch, w.first, w.words, w.group_off,
-                  w.unique_ptr, edge_col, out_row, out_col, tn.remap));
+    const dim3 grid((unsigned)grid_for_units(ceil_div(E, kRelabelTile), tn.remap));
+    if (out_col && col_indptr) {
+      GS_LAUNCH("unique_relabel", s,
+                unique_relabel_kernel<true><<<grid, dim3(kBlock), 0, s>>>(
+                    k, w.etile_batch, w.batch, w.first, w.words, w.group_off, w.unique_ptr,
+                    nullptr, col_indptr, out_row, out_col, tn.remap));
+    } else {
+      GS_LAUNCH("unique_relabel", s,
+                unique_relabel_kernel<false><<<grid, dim3(kBlock), 0, s>>>(
+                    k, w.etile_batch, w.batch, w.first, w.words, w.group_off, w.unique_ptr,
+                    edge_col, nullptr, out_row, out_col, tn.remap));
+    }
   }
   return GS_OK;
 }

@@ -292,8 +292,14 @@ int gs_list_sample_weighted_fill(const float* probs, const int64_t* range,
  *   out_unique[U].
  * relabel: after count, same workspace; out_row[num_rows_keys] = batch-local
  *   rank of every row key (nullable); out_col[num_rows_keys] = batch-local rank
- *   of seeds[edge_col[e]] (nullable; edge_col holds positions into `seeds`).
- *   May be called any number of times while the workspace is kept.
+ *   of seeds[c(e)] (nullable), c(e) being the position into `seeds` of edge e's
+ *   column: edge_col[e], or -- for edges grouped by column, as a compressed
+ *   matrix holds them -- the column c with col_indptr[c] <= e < col_indptr[c + 1]
+ *   (col_indptr[num_seeds + 1], col_indptr[0] = 0; the coordinate form of such
+ *   a matrix then need not exist: the reference expands it first,
+ *   src/cuda/batch/batch_relabel.cu:480-498 takes coo_col).  Give one of the
+ *   two, the other NULL.  May be called any number of times while the
+ *   workspace is kept.
  * Keys are any int64 values; one call takes at most 2^31 - 1 keys.  While all
  * keys of a call lie in [0, 2^32 - 2] a packed table entry holds the key itself;
  * when one does not (ids of a very large graph, ids encoded as id + batch *
@@ -322,8 +328,8 @@ int gs_unique_relabel(const int64_t* seeds, const int64_t* seeds_ptr,
                       int64_t num_seeds, const int64_t* rows,
                       const int64_t* rows_ptr, int64_t num_rows_keys,
                       int64_t num_batches, const int64_t* edge_col,
-                      int64_t* out_row, int64_t* out_col, void* workspace,
-                      size_t workspace_bytes, gs_stream_t stream);
+                      const int64_t* col_indptr, int64_t* out_row, int64_t* out_col,
+                      void* workspace, size_t workspace_bytes, gs_stream_t stream);
 
 /* ------------------------------------------------------------------------
  * out_first[r] = smallest position e with ids[e] == r, INT64_MAX when r does

@@ -157,6 +157,63 @@ def test_unique_relabel_hubs_and_ragged_batches():
                 orc.unique_relabel(seeds, rows, sp, rp, edge_col))
 
 
+def _grouped_case(rng, counts, B, id_range):
+    """Edges grouped by seed position: counts[c] edges for seed c, B batches of seeds."""
+    S = counts.size
+    col_indptr = np.concatenate([[0], np.cumsum(counts)]).astype(np.int64)
+    cuts = np.sort(rng.integers(0, S + 1, size=B - 1)) if B > 1 else np.empty(0, np.int64)
+    sp = np.concatenate([[0], cuts, [S]]).astype(np.int64)
+    rp = col_indptr[sp]
+    seeds = rng.permutation(id_range)[:S] if id_range >= S else rng.integers(0, id_range, size=S)
+    rows = rng.integers(0, id_range, size=int(col_indptr[-1]))
+    edge_col = np.repeat(np.arange(S, dtype=np.int64), counts)
+    return seeds.astype(np.int64), rows, sp, rp, edge_col, col_indptr
+
+
+@pytest.mark.parametrize("shape", ["ragged", "fives", "gaps", "giant", "exact_tiles", "one_edge",
+                                   "repeated_seeds"])
+@pytest.mark.parametrize("B", [1, 7, 64])
+def test_unique_relabel_by_column_pointer(shape, B):
+    """The column of an edge read off the column pointer of a matrix compressed by
+    column gives the labels that an explicit column per edge gives."""
+    rng = np.random.default_rng(sum(shape.encode()) * 100 + B)
+    id_range = 10**5
+    if shape == "ragged":
+        counts = rng.integers(0, 11, size=5000)
+    elif shape == "fives":
+        counts = np.full(6000, 5)
+    elif shape == "gaps":      # long runs of empty columns, also at both ends and across tiles
+        counts = np.zeros(20000, dtype=np.int64)
+        counts[[4000, 4001, 9000, 15000, 15002]] = [3000, 1, 2047, 1, 5000]
+    elif shape == "giant":     # one column over many tiles
+        counts = rng.integers(0, 4, size=3000)
+        counts[1500] = 50000
+    elif shape == "exact_tiles":
+        counts = np.full(1024, 4)
+    elif shape == "one_edge":
+        counts = np.zeros(300, dtype=np.int64)
+        counts[299] = 1
+    else:                      # seeds that repeat: labels go through the first occurrence
+        counts = rng.integers(0, 6, size=4000)
+        id_range = 500
+    seeds, rows, sp, rp, edge_col, col_indptr = _grouped_case(rng, counts, B, id_range)
+    bp = (T(sp), T(rp)) if B > 1 else (None, None)
+    got = capi.unique_relabel(T(seeds), T(rows), *bp, col_indptr=T(col_indptr))
+    assert_same(got, orc.unique_relabel(seeds, rows, sp if B > 1 else None,
+                                        rp if B > 1 else None, edge_col))
+    other = capi.unique_relabel(T(seeds), T(rows), *bp, edge_col=T(edge_col))
+    assert_same(got, tuple(None if x is None else N(x) for x in other))
+
+
+def test_unique_relabel_column_arguments_are_checked():
+    seeds, rows = T(np.arange(4)), T(np.arange(8))
+    with pytest.raises(ValueError, match="not both"):
+        capi.unique_relabel(seeds, rows, edge_col=T(np.zeros(8, np.int64)),
+                            col_indptr=T(np.array([0, 2, 4, 6, 8])))
+    with pytest.raises(ValueError, match="entries"):
+        capi.unique_relabel(seeds, rows, col_indptr=T(np.array([0, 8])))
+
+
 @pytest.mark.parametrize("B", [1023, 1024, 1025, 3000])
 def test_unique_relabel_many_tiny_batches(B):
     """Around 1024 batches the batch walk moves from every work-group's LDS to a launch
