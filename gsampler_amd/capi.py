@@ -65,6 +65,7 @@ SIGNATURES = {
     "gs_split_indptr": (_int, [_p, _p, _i64, _i64, _p, _p]),
     "gs_batch_seeds_distinct": (_int, [_p, _p, _p, _p, _i64, _p, _p]),
     "gs_first_position": (_int, [_p, _i64, _i64, _p, _p]),
+    "gs_list_labels": (_int, [_p, _i64, _p, _p, _i64, _p, _p, _p, _p, _p, _p]),
     "gs_gather_rows": (_int, [_p, _i64, _i64, _p, _i64, _p, _p, _p]),
     "gs_coo_sort_workspace_bytes": (_sz, [_i64, _i64]),
     "gs_coo_sort": (_int, [_p, _i64, _i64, _p, _p, _p, _sz, _p]),
@@ -407,6 +408,33 @@ def first_position(ids: torch.Tensor, num_ids: int) -> torch.Tensor:
     out = torch.empty(num_ids, dtype=torch.int64, device=ids.device)
     check(lib().gs_first_position(_ptr(ids), ids.numel(), num_ids, _ptr(out), _stream()))
     return out
+
+
+LIST_LABELS_MAX_KEYS = 2048
+
+
+def list_labels(seeds, list_ids, first_pos):
+    """Frontier and labels of a matrix whose rows are positions in `list_ids`:
+    the unique of seeds ++ list_ids[row[e]] in first-occurrence order, given the
+    first edge of every listed id (first_position).
+
+    -> (frontier, list_label, seed_label)
+    """
+    seeds, list_ids = _i64t(seeds, "seeds"), _i64t(list_ids, "list_ids")
+    first_pos = _i64t(first_pos, "first_pos")
+    S, R = seeds.numel(), list_ids.numel()
+    if first_pos.numel() != R:
+        raise ValueError(f"list_labels: {first_pos.numel()} first positions for {R} ids")
+    dev = list_ids.device
+    frontier = torch.empty(S + R, dtype=torch.int64, device=dev)
+    list_label = torch.empty(R, dtype=torch.int64, device=dev)
+    seed_label = torch.empty(S, dtype=torch.int64, device=dev)
+    count = _Count()
+    check(lib().gs_list_labels(_ptr(seeds), S, _ptr(list_ids), _ptr(first_pos), R,
+                               _ptr(frontier), None, count.mirror(), _ptr(list_label),
+                               _ptr(seed_label), _stream()))
+    count.arm()
+    return frontier[:count.get()], list_label, seed_label
 
 
 def coo_sort(major: torch.Tensor, num_major: int):

@@ -479,6 +479,20 @@ Graph::ListLabels& Graph::list_labels_for(const torch::Tensor& col_seeds,
   const int64_t R = table.numel(), S = col_seeds.numel(), E = base.numel();
   torch::Tensor first = new_ids(R, base);
   GS_CALL(gs_first_position(cptr(base), E, R, mptr(first), cur_stream()));
+  if (R + S <= GS_LIST_LABELS_MAX_KEYS) {
+    // few enough keys for one work-group: frontier and labels in one launch
+    torch::Tensor frontier = new_ids(R + S, base);
+    out->label_by_local = new_ids(R, base);
+    out->seed_label = new_ids(S, base);
+    AsyncCount count = AsyncCount::mirrored();
+    GS_CALL(gs_list_labels(cptr(col_seeds), S, cptr(table), cptr(first), R, mptr(frontier),
+                           nullptr, count.mirror(), mptr(out->label_by_local),
+                           mptr(out->seed_label), cur_stream()));
+    count.arm();
+    out->frontier = frontier.narrow(0, 0, count.get());
+    list_labels_ = std::move(out);
+    return *list_labels_;
+  }
   auto sorted = torch::sort(first);  // R values: which listed id is met first
   const torch::Tensor& when = std::get<0>(sorted);
   const torch::Tensor& order = std::get<1>(sorted);

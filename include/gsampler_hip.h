@@ -343,6 +343,29 @@ int gs_first_position(const int64_t* ids, int64_t n, int64_t num_ids,
                       int64_t* out_first, gs_stream_t stream);
 
 /* ------------------------------------------------------------------------
+ * Frontier and labels for such a matrix in one launch.  Every edge of local
+ * row l carries the key list_ids[l], so the unique of
+ *     seeds ++ list_ids[row[e]] (e = 0, 1, ...)
+ * in first-occurrence order -- what TensorUniqueCUDA / TensorRelabelCUDA
+ * (src/cuda/unique_reindex.cu:174-199) compute over all edges -- is the unique
+ * of seeds ++ (the listed ids in the order of first_pos, as gs_first_position
+ * gives it; ids with first_pos == INT64_MAX are used by no edge and left out).
+ *   out_frontier[num_seeds + num_ids]  the first out_count[0] entries are written
+ *   out_count, out_count_mirror        nullable; device memory / pinned host memory
+ *   out_list_label[num_ids]            label of list_ids[l] (0 for an unused id);
+ *                                      the label of edge e's row is out_list_label[row[e]]
+ *   out_seed_label[num_seeds]          label of seeds[c] (repeated seeds share one)
+ * One work-group, all in LDS: num_seeds + num_ids <= GS_LIST_LABELS_MAX_KEYS,
+ * more is refused with GS_ERR_INVALID (use gs_unique_count / gs_unique_relabel).
+ * ---------------------------------------------------------------------- */
+#define GS_LIST_LABELS_MAX_KEYS 2048
+int gs_list_labels(const int64_t* seeds, int64_t num_seeds, const int64_t* list_ids,
+                   const int64_t* first_pos, int64_t num_ids, int64_t* out_frontier,
+                   int64_t* out_count, int64_t* out_count_mirror,
+                   int64_t* out_list_label, int64_t* out_seed_label,
+                   gs_stream_t stream);
+
+/* ------------------------------------------------------------------------
  * Edge list -> compressed format, first half: stable sort of the edge
  * positions by their id on the axis to compress (`major`, ids in
  * [0, num_major)).  sorted_major receives the ids in order, perm the positions
