@@ -107,6 +107,7 @@ class AsyncCount {
     c.slot_ = (int)(c.ticket_ % kSlots);
     return c;
   }
+  bool requested() const { return slot_ >= 0; }
   int64_t* mirror() const { return ring().words + slot_; }
   void arm() {
     check(hipEventRecord(ring().events[slot_], (hipStream_t)cur_stream()));

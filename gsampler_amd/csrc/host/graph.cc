@@ -489,7 +489,8 @@ Graph::ListLabels& Graph::list_labels_for(const torch::Tensor& col_seeds,
                            nullptr, count.mirror(), mptr(out->label_by_local),
                            mptr(out->seed_label), cur_stream()));
     count.arm();
-    out->frontier = frontier.narrow(0, 0, count.get());
+    out->frontier_bound = frontier;
+    out->frontier_count = count;
     list_labels_ = std::move(out);
     return *list_labels_;
   }
@@ -508,7 +509,7 @@ Graph::ListLabels& Graph::list_labels_for(const torch::Tensor& col_seeds,
   out->label_by_local = new_ids(R, base);
   out->label_by_local.index_copy_(0, order, labels.narrow(0, 0, R));
   out->seed_label = labels.narrow(0, R, S);
-  out->frontier = f.frontier();
+  out->frontier_bound = f.frontier();
   list_labels_ = std::move(out);
   return *list_labels_;
 }
@@ -522,8 +523,10 @@ Graph::GraphRelabel(torch::Tensor col_seeds, torch::Tensor row_ids) {
               "GraphRelabel: the matrix has edges but col_seeds is empty");
   if (use_list_labels(col_seeds, row_ids)) {
     ListLabels& l = list_labels_for(col_seeds, row_ids);
-    return {l.frontier, l.label_by_local.index_select(0, coo_->row),
-            l.seed_label.index_select(0, coo_->col), coo_->e_ids};
+    // the gathers are queued before the host waits for the size of the frontier
+    torch::Tensor out_row = l.label_by_local.index_select(0, coo_->row);
+    torch::Tensor out_col = l.seed_label.index_select(0, coo_->col);
+    return {l.frontier(), out_row, out_col, coo_->e_ids};
   }
   torch::Tensor rows = mapped_rows(coo_->row, row_ids);
   Frontier& f = frontier_for(col_seeds, rows, {}, {});
@@ -546,7 +549,7 @@ torch::Tensor Graph::GetValidNodes(torch::Tensor col_seeds,
   // here when a CSC exists, src/graph.cc:593-608, which is another edge order
   // whenever that CSC was built by sorting a row-sorted COO.)
   CreateSparseFormat(kCOO);
-  if (use_list_labels(col_seeds, row_ids)) return list_labels_for(col_seeds, row_ids).frontier;
+  if (use_list_labels(col_seeds, row_ids)) return list_labels_for(col_seeds, row_ids).frontier();
   const torch::Tensor& base = coo_->row;
   torch::Tensor rows = mapped_rows(base, row_ids);
   return frontier_for(col_seeds, rows, {}, {}).frontier();

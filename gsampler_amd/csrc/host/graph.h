@@ -310,7 +310,20 @@ class Graph : public torch::CustomClassHolder {
   struct ListLabels {
     torch::Tensor base, row_ids, seeds;
     int64_t row_ids_version = -1, seeds_version = -1;
-    torch::Tensor frontier, label_by_local, seed_label;
+    torch::Tensor label_by_local, seed_label;
+    // The unique keys sit at the front of a buffer sized by the bound; how many
+    // there are may still be on its way from the device.
+    torch::Tensor frontier_bound;
+    AsyncCount frontier_count;
+    bool counted = false;
+    const torch::Tensor& frontier() {
+      if (!counted) {
+        if (frontier_count.requested())
+          frontier_bound = frontier_bound.narrow(0, 0, frontier_count.get());
+        counted = true;
+      }
+      return frontier_bound;
+    }
   };
   std::unique_ptr<ListLabels> list_labels_;
   bool use_list_labels(const torch::Tensor& col_seeds, const torch::Tensor& row_ids) const;

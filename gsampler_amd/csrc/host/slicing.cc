@@ -18,21 +18,29 @@ MinorKept keep_members(const torch::Tensor& ids_per_edge, const torch::Tensor& p
   const int64_t num_major = indptr.defined() ? indptr.numel() - 1 : 0;
   MinorKept r;
   torch::Tensor ws = new_workspace(gs_minor_slice_workspace_bytes(nnz, np), ids_per_edge);
-  torch::Tensor total = new_ids(1, ids_per_edge);
   if (indptr.defined()) r.indptr = new_ids(num_major + 1, ids_per_edge);
+  // the number of kept edges goes straight to pinned host memory; the fill pass
+  // is queued into buffers sized by the bound (every edge kept) and runs while
+  // the number travels
+  AsyncCount kept = AsyncCount::mirrored();
   GS_CALL(gs_minor_slice_count(cptr(ids_per_edge), nnz, cptr(picked), np,
                                cptr(indptr), num_major,
                                indptr.defined() ? mptr(r.indptr) : nullptr,
-                               mptr(total), ws.data_ptr(), ws.numel(),
+                               kept.mirror(), ws.data_ptr(), ws.numel(),
                                cur_stream()));
-  const int64_t kept = total.item<int64_t>();
-  r.minor = new_ids(kept, ids_per_edge);
-  r.select = new_ids(kept, ids_per_edge);
-  if (want_major) r.major = new_ids(kept, ids_per_edge);
+  kept.arm();
+  const int64_t size = nnz <= kBoundLimit ? nnz : kept.get();
+  r.minor = new_ids(size, ids_per_edge);
+  r.select = new_ids(size, ids_per_edge);
+  if (want_major) r.major = new_ids(size, ids_per_edge);
   GS_CALL(gs_minor_slice_fill(cptr(ids_per_edge), nnz, np, cptr(indptr), num_major,
                               cptr(edge_major), want_major ? mptr(r.major) : nullptr,
                               mptr(r.minor), mptr(r.select), ws.data_ptr(),
                               ws.numel(), cur_stream()));
+  const int64_t n = kept.get();
+  r.minor = r.minor.narrow(0, 0, n);
+  r.select = r.select.narrow(0, 0, n);
+  if (want_major) r.major = r.major.narrow(0, 0, n);
   return r;
 }
 }  // namespace
