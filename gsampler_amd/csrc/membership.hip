@@ -26,8 +26,12 @@ namespace gs {
 
 constexpr int kMemberWords = kBlock / kWave;  // flag words per chunk of kBlock edges
 constexpr int kMemberChunksPerWave = 8;
+constexpr int kMemberAhead = 4;  // chunks of a wave whose loads are in flight together
+static_assert(kMemberChunksPerWave % kMemberAhead == 0 && kMemberChunksPerWave * kMemberWords <= kWave,
+              "a wave's flag words fit one word per lane");
 constexpr int kMemberThreads = 1024;  // 16 waves share one staged table: 32 Ki edges per 32 KB copied
 constexpr int kMemberLdsSlots = 4096;  // tables up to this size are staged in LDS (32 KB)
+constexpr int64_t kMemberSmallEdges = int64_t(1) << 23;  // below: work-groups of kBlock threads
 
 struct MemberWs {
   uint64_t* table;     // [member_table_slots(num_picked)]
@@ -209,8 +213,10 @@ struct MemberTable {
   }
 };
 
-template <bool kInLds>
-__global__ __launch_bounds__(kMemberThreads) void member_flag_kernel(
+// kThreads: work-group size.  A large one shares a staged table among more
+// edges; a small one spreads a short edge list over all compute units.
+template <bool kInLds, int kThreads>
+__global__ __launch_bounds__(kThreads) void member_flag_kernel(
     const int64_t* __restrict__ ids, int64_t nnz,
     const uint64_t* __restrict__ global_table, uint32_t cap,
     const int64_t* __restrict__ picked, const int* __restrict__ wide_flag,
@@ -222,62 +228,60 @@ __global__ __launch_bounds__(kMemberThreads) void member_flag_kernel(
   table.stage(global_table, cap, lds_keys, lds_values);
   const bool wide = *wide_flag != 0;  // the same for every thread of the launch
   const int64_t num_chunks = ceil_div_dev(nnz, kBlock);
-  const int64_t wave = (int64_t)blockIdx.x * (kMemberThreads / kWave) + threadIdx.x / kWave;
+  const int64_t wave = (int64_t)blockIdx.x * (kThreads / kWave) + threadIdx.x / kWave;
   const int lane = lane_id();
-  // the ids of the next chunk are requested before the look-ups of this one
-  uint32_t next_key[kMemberWords];
+  // The ids of kMemberAhead chunks are requested together, before anything is
+  // stored: a store between a load and its use makes the wait for the load
+  // (loads and stores count down one in-order counter) a wait for everything.
   const int64_t first_chunk = wave * kMemberChunksPerWave;
-  if (first_chunk >= num_chunks) return;
+  for (int part = 0; part < kMemberChunksPerWave / kMemberAhead; ++part) {
+    const int64_t chunk0 = first_chunk + part * kMemberAhead;
+    if (chunk0 >= num_chunks) return;
+    uint32_t keys[kMemberAhead][kMemberWords];
 #pragma unroll
-  for (int j = 0; j < kMemberWords; ++j) {
-    const int64_t e = first_chunk * kBlock + j * kWave + lane;
-    next_key[j] = e < nnz ? member_key((uint64_t)ids[e]) : kNoKey;
-  }
-  for (int c = 0; c < kMemberChunksPerWave; ++c) {
-    const int64_t chunk = first_chunk + c;
-    if (chunk >= num_chunks) return;
-    uint32_t key[kMemberWords];
-#pragma unroll
-    for (int j = 0; j < kMemberWords; ++j) key[j] = next_key[j];
-    if (c + 1 < kMemberChunksPerWave && chunk + 1 < num_chunks) {
+    for (int c = 0; c < kMemberAhead; ++c)
 #pragma unroll
       for (int j = 0; j < kMemberWords; ++j) {
-        const int64_t e = (chunk + 1) * kBlock + j * kWave + lane;
-        next_key[j] = e < nnz ? member_key((uint64_t)ids[e]) : kNoKey;
+        const int64_t e = (chunk0 + c) * kBlock + j * kWave + lane;
+        keys[c][j] = e < nnz ? member_key((uint64_t)ids[e]) : kNoKey;
       }
-    }
-    uint32_t slot[kMemberWords];
-    uint64_t word[kMemberWords];
-    if (!wide) {
-      table.find_many(key, slot);
-    } else {
 #pragma unroll
-      for (int j = 0; j < kMemberWords; ++j) {
-        const int64_t e = chunk * kBlock + j * kWave + lane;
-        slot[j] = e < nnz ? table.find_confirmed((uint64_t)ids[e], picked) : cap;
+    for (int c = 0; c < kMemberAhead; ++c) {
+      const int64_t chunk = chunk0 + c;
+      if (chunk >= num_chunks) return;
+      uint32_t slot[kMemberWords];
+      uint64_t word[kMemberWords];
+      if (!wide) {
+        table.find_many(keys[c], slot);
+      } else {
+#pragma unroll
+        for (int j = 0; j < kMemberWords; ++j) {
+          const int64_t e = chunk * kBlock + j * kWave + lane;
+          slot[j] = e < nnz ? table.find_confirmed((uint64_t)ids[e], picked) : cap;
+        }
       }
-    }
 #pragma unroll
-    for (int j = 0; j < kMemberWords; ++j) word[j] = __ballot(slot[j] < cap);
-    {
-      int before = 0;  // kept edges of the chunk in front of this row of 64
+      for (int j = 0; j < kMemberWords; ++j) word[j] = __ballot(slot[j] < cap);
+      {
+        int before = 0;  // kept edges of the chunk in front of this row of 64
 #pragma unroll
-      for (int j = 0; j < kMemberWords; ++j) {
-        if (slot[j] < cap)
-          staged[chunk * kBlock + before + __popcll(word[j] & ((1ull << lane) - 1))] =
-              table.value_at(slot[j]);
-        before += __popcll(word[j]);
+        for (int j = 0; j < kMemberWords; ++j) {
+          if (slot[j] < cap)
+            staged[chunk * kBlock + before + __popcll(word[j] & ((1ull << lane) - 1))] =
+                table.value_at(slot[j]);
+          before += __popcll(word[j]);
+        }
       }
-    }
-    if (lane == 0) {
-      int total = 0;
+      if (lane == 0) {
+        int total = 0;
 #pragma unroll
-      for (int j = 0; j < kMemberWords; ++j) {
-        flags[chunk * kMemberWords + j] = word[j];
-        total += __popcll(word[j]);
+        for (int j = 0; j < kMemberWords; ++j) {
+          flags[chunk * kMemberWords + j] = word[j];
+          total += __popcll(word[j]);
+        }
+        chunk_count[chunk] = total;
+        if (chunk == num_chunks - 1) chunk_count[num_chunks] = 0;
       }
-      chunk_count[chunk] = total;
-      if (chunk == num_chunks - 1) chunk_count[num_chunks] = 0;
     }
   }
 }
@@ -308,64 +312,84 @@ __global__ __launch_bounds__(kBlock) void member_indptr_kernel(
                   : (e >= nnz ? chunk_off[num_chunks] : member_rank_before(e, flags, chunk_off));
 }
 
-// Segment of position x given a segment `from` at or before it: a few steps
-// forward, then a search in what is left (a chunk can cross many empty columns).
-__device__ __forceinline__ int64_t segment_from(const int64_t* __restrict__ ptr, int64_t n,
-                                                int64_t from, int64_t x) {
-  int64_t s = from;
-  for (int step = 0; step < 3; ++step) {
-    if (s + 1 >= n || ptr[s + 1] > x) return s;
-    ++s;
-  }
-  return s + segment_of(ptr + s, n - s, x);
-}
-
-__global__ __launch_bounds__(kMemberThreads) void member_fill_kernel(
+// A wave writes the kept edges of kMemberChunksPerWave consecutive chunks.  What
+// it needs to know about them arrives in one round trip (lane l holds flag word
+// l of the wave's chunks, the first lanes also a chunk offset each); the columns
+// of the wave's first and last edge take a wavefront search each (one column
+// covers the whole span unless columns are short); then the staged ids of all
+// chunks of a part are requested together, and only then anything is stored.
+// kEdgeMajor: the id on the other axis comes from edge_major (an edge list)
+// instead of the compressed pointer.
+template <bool kEdgeMajor>
+__global__ __launch_bounds__(kBlock) void member_fill_kernel(
     int64_t nnz, const uint64_t* __restrict__ flags, const int64_t* __restrict__ chunk_off,
     const uint32_t* __restrict__ staged, const int64_t* __restrict__ indptr,
     int64_t num_major, const int64_t* __restrict__ edge_major,
     int64_t* __restrict__ out_major, int64_t* __restrict__ out_minor,
     int64_t* __restrict__ out_select) {
   const int64_t num_chunks = ceil_div_dev(nnz, kBlock);
-  const int64_t wave = (int64_t)blockIdx.x * (kMemberThreads / kWave) + threadIdx.x / kWave;
+  const int64_t wave = (int64_t)blockIdx.x * (kBlock / kWave) + threadIdx.x / kWave;
   const int lane = lane_id();
   const int64_t first_chunk = wave * kMemberChunksPerWave;
-  int64_t seg_cursor = 0;
-  for (int c = 0; c < kMemberChunksPerWave; ++c) {
-    const int64_t chunk = first_chunk + c;
-    if (chunk >= num_chunks) return;
-    const int64_t e0 = chunk * kBlock;
-    const int64_t e_last = e0 + kBlock - 1 < nnz ? e0 + kBlock - 1 : nnz - 1;
-    uint64_t word[kMemberWords];
+  if (first_chunk >= num_chunks) return;
+  const int64_t my_word = first_chunk * kMemberWords + lane;
+  const uint64_t lane_word =
+      lane < kMemberChunksPerWave * kMemberWords && my_word < num_chunks * kMemberWords
+          ? flags[my_word]
+          : 0ull;
+  const int64_t lane_off =
+      lane < kMemberChunksPerWave && first_chunk + lane < num_chunks ? chunk_off[first_chunk + lane]
+                                                                    : 0;
+  const int64_t e_first = first_chunk * kBlock;
+  const int64_t e_end =
+      (first_chunk + kMemberChunksPerWave) * kBlock < nnz ? (first_chunk + kMemberChunksPerWave) * kBlock
+                                                          : nnz;
+  SegmentSpan span{0, 0};
+  if (out_major && !kEdgeMajor) {
+    span.lo = wave_segment_of(indptr, num_major, e_first);
+    span.hi = span.lo + wave_segment_of(indptr + span.lo, num_major - span.lo, e_end - 1);
+  }
 #pragma unroll
-    for (int j = 0; j < kMemberWords; ++j) word[j] = flags[chunk * kMemberWords + j];
-    const int64_t out0 = chunk_off[chunk];
-    // segments the chunk touches (for out_major without edge_major): mostly the
-    // one the previous chunk ended in, so the search starts from there
-    int64_t seg_lo = 0, seg_hi = 0;
-    if (out_major && !edge_major) {
-      seg_lo = c == 0 ? segment_of(indptr, num_major, wave_uniform_first(e0))
-                      : segment_from(indptr, num_major, seg_cursor, wave_uniform_first(e0));
-      seg_hi = segment_from(indptr, num_major, seg_lo, wave_uniform_first(e_last));
-      seg_cursor = seg_hi;
-    }
-    int before = 0;
+  for (int part = 0; part < kMemberChunksPerWave / kMemberAhead; ++part) {
+    const int c0 = part * kMemberAhead;
+    if (first_chunk + c0 >= num_chunks) return;
+    uint32_t minor[kMemberAhead][kMemberWords];
+    int64_t major[kMemberAhead][kMemberWords];
 #pragma unroll
-    for (int j = 0; j < kMemberWords; ++j) {
-      const int64_t e = e0 + j * kWave + lane;
-      if ((word[j] >> lane) & 1ull) {
-        const int in_chunk = before + __popcll(word[j] & ((1ull << lane) - 1));
-        const int64_t pos = out0 + in_chunk;
-        out_minor[pos] = (int64_t)staged[chunk * kBlock + in_chunk];
-        out_select[pos] = e;
-        if (out_major)
-          out_major[pos] =
-              edge_major ? edge_major[e]
-                         : (seg_lo == seg_hi
-                                ? seg_lo
-                                : seg_lo + segment_of(indptr + seg_lo, seg_hi - seg_lo + 1, e));
+    for (int c = 0; c < kMemberAhead; ++c) {
+      int before = 0;
+#pragma unroll
+      for (int j = 0; j < kMemberWords; ++j) {
+        const uint64_t word =
+            __shfl((unsigned long long)lane_word, (c0 + c) * kMemberWords + j, kWave);
+        const int64_t e = (first_chunk + c0 + c) * kBlock + j * kWave + lane;
+        minor[c][j] = 0;
+        major[c][j] = 0;
+        if ((word >> lane) & 1ull) {
+          minor[c][j] = staged[(first_chunk + c0 + c) * kBlock + before +
+                               __popcll(word & ((1ull << lane) - 1))];
+          if (kEdgeMajor) major[c][j] = edge_major[e];
+        }
+        before += __popcll(word);
       }
-      before += __popcll(word[j]);
+    }
+#pragma unroll
+    for (int c = 0; c < kMemberAhead; ++c) {
+      const int64_t out0 = __shfl((long long)lane_off, c0 + c, kWave);
+      int before = 0;
+#pragma unroll
+      for (int j = 0; j < kMemberWords; ++j) {
+        const uint64_t word =
+            __shfl((unsigned long long)lane_word, (c0 + c) * kMemberWords + j, kWave);
+        const int64_t e = (first_chunk + c0 + c) * kBlock + j * kWave + lane;
+        if ((word >> lane) & 1ull) {
+          const int64_t pos = out0 + before + __popcll(word & ((1ull << lane) - 1));
+          out_minor[pos] = (int64_t)minor[c][j];
+          out_select[pos] = e;
+          if (out_major) out_major[pos] = kEdgeMajor ? major[c][j] : span.segment_at(indptr, e);
+        }
+        before += __popcll(word);
+      }
     }
   }
 }
@@ -412,15 +436,19 @@ int gs_minor_slice_count(const int64_t* ids, int64_t nnz, const int64_t* picked,
                                      dim3(kBlock), 0, s>>>(picked, num_picked,
                                                            w.table, cap, w.wide));
   if (nnz > 0) {
-    const int64_t blocks = ceil_div(w.chunks, (kMemberThreads / kWave) * kMemberChunksPerWave);
-    if (cap <= (uint64_t)kMemberLdsSlots)
-      GS_LAUNCH("member_flag", s,
-                member_flag_kernel<true><<<dim3((unsigned)blocks), dim3(kMemberThreads), 0, s>>>(
-                    ids, nnz, w.table, cap, picked, w.wide, w.flags, w.chunk_off, w.staged));
-    else
-      GS_LAUNCH("member_flag", s,
-                member_flag_kernel<false><<<dim3((unsigned)blocks), dim3(kMemberThreads), 0, s>>>(
-                    ids, nnz, w.table, cap, picked, w.wide, w.flags, w.chunk_off, w.staged));
+    const bool in_lds = cap <= (uint64_t)kMemberLdsSlots;
+    const bool small = nnz < kMemberSmallEdges;
+    const int threads = small ? kBlock : kMemberThreads;
+    const dim3 grid((unsigned)ceil_div(w.chunks, (threads / kWave) * kMemberChunksPerWave));
+#define GS_MEMBER_FLAG(LDS, THREADS)                                                          \
+  GS_LAUNCH("member_flag", s,                                                                 \
+            (member_flag_kernel<LDS, THREADS>)<<<grid, dim3(THREADS), 0, s>>>(                \
+                ids, nnz, w.table, cap, picked, w.wide, w.flags, w.chunk_off, w.staged))
+    if (in_lds && small) GS_MEMBER_FLAG(true, kBlock);
+    else if (in_lds) GS_MEMBER_FLAG(true, kMemberThreads);
+    else if (small) GS_MEMBER_FLAG(false, kBlock);
+    else GS_MEMBER_FLAG(false, kMemberThreads);
+#undef GS_MEMBER_FLAG
     int rc = exclusive_scan_i64(w.chunk_off, w.chunk_off, w.chunks + 1, w.scan_ws,
                                 w.scan_ws_bytes, s);
     if (rc != GS_OK) return rc;
@@ -453,11 +481,17 @@ int gs_minor_slice_fill(const int64_t* ids, int64_t nnz, int64_t num_picked,
     return GS_ERR_WORKSPACE;
   }
   hipStream_t s = as_stream(stream);
-  const dim3 grid((unsigned)ceil_div(w.chunks, (kMemberThreads / kWave) * kMemberChunksPerWave));
-  GS_LAUNCH("member_fill", s,
-            member_fill_kernel<<<grid, dim3(kMemberThreads), 0, s>>>(
-                nnz, w.flags, w.chunk_off, w.staged, indptr, num_major, edge_major,
-                out_major, out_minor, out_select));
+  const dim3 grid((unsigned)ceil_div(w.chunks, (kBlock / kWave) * kMemberChunksPerWave));
+  if (edge_major)
+    GS_LAUNCH("member_fill", s,
+              member_fill_kernel<true><<<grid, dim3(kBlock), 0, s>>>(
+                  nnz, w.flags, w.chunk_off, w.staged, indptr, num_major, edge_major,
+                  out_major, out_minor, out_select));
+  else
+    GS_LAUNCH("member_fill", s,
+              member_fill_kernel<false><<<grid, dim3(kBlock), 0, s>>>(
+                  nnz, w.flags, w.chunk_off, w.staged, indptr, num_major, edge_major,
+                  out_major, out_minor, out_select));
   return GS_OK;
 }
 

@@ -1013,23 +1013,6 @@ __global__ __launch_bounds__(kBlock) void unique_fill_kernel(
 }
 
 // ---------------------------------------------------------------- relabel
-// The largest c in [0, n) with ptr[c] <= x, for nondecreasing ptr with
-// ptr[0] <= x; found by one wavefront, 64 probes a round.
-__device__ __forceinline__ int64_t wave_last_at_most(const int64_t* __restrict__ ptr, int64_t n,
-                                                     int64_t x) {
-  int64_t lo = 0, hi = n;  // ptr[lo] <= x; hi == n or ptr[hi] > x
-  while (hi - lo > 1) {
-    const int64_t step = (hi - lo + kWave - 1) / kWave;
-    const int64_t c = lo + (int64_t)(lane_id() + 1) * step;
-    const bool ok = c < hi && ptr[c] <= x;
-    const int hits = __popcll(__ballot(ok));  // ok is monotone over the lanes
-    const int64_t next_hi = lo + (int64_t)(hits + 1) * step;
-    lo += (int64_t)hits * step;
-    if (next_hi < hi) hi = next_hi;
-  }
-  return lo;
-}
-
 // The column of every edge of a tile from the column pointer: edge e belongs
 // to the last column c with col_indptr[c] <= e.  Two wavefronts find the
 // columns of the tile's first and last edge among [col_begin, col_end), the
@@ -1048,7 +1031,7 @@ __device__ __forceinline__ int64_t tile_columns(const int64_t* __restrict__ col_
 #pragma unroll
   for (int q = 0; q < kQuads; ++q) quads[q] = make_int4(0, 0, 0, 0);
   if (wave < 2) {
-    const int64_t c = wave_last_at_most(col_indptr + col_begin, col_end - col_begin,
+    const int64_t c = wave_segment_of(col_indptr + col_begin, col_end - col_begin,
                                         wave == 0 ? e0 : e1 - 1);
     if (lane_id() == 0) ends[wave] = col_begin + c;
   }
