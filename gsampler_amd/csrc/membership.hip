@@ -213,6 +213,84 @@ struct MemberTable {
   }
 };
 
+// The same small table, rebuilt in LDS as buckets of four keys: a look-up reads
+// one bucket (16 bytes, one instruction) and compares four keys, and goes on to
+// the next bucket only from a full one.  With at most two keys per bucket on
+// average nearly every look-up ends at its first bucket, where the linear table
+// makes a wave repeat its probe loop until the longest of its 256 probe runs
+// has ended -- the pass is bound by the instructions it issues.  For picked
+// sets whose ids all fit 32 bits (a match of the key is then a match of the id).
+constexpr int kMemberBuckets = kMemberLdsSlots / 4;
+struct BucketTable {
+  const uint4* keys;       // [kMemberBuckets] filled from .x on; kNoKey = free
+  const uint32_t* values;  // [kMemberLdsSlots] position in the picked set, by slot
+
+  __device__ __forceinline__ static uint32_t home(uint32_t key) {
+    return __umulhi(key * 0x9E3779B1u, (uint32_t)kMemberBuckets);
+  }
+
+  // fill: a counter per bucket, only used here
+  __device__ __forceinline__ void stage(const uint64_t* __restrict__ table, uint32_t capacity,
+                                        uint32_t* lds_keys, uint32_t* lds_values,
+                                        uint32_t* fill) {
+    keys = reinterpret_cast<const uint4*>(lds_keys);
+    values = lds_values;
+    for (uint32_t i = threadIdx.x; i < (uint32_t)kMemberLdsSlots; i += blockDim.x)
+      lds_keys[i] = kNoKey;
+    for (uint32_t i = threadIdx.x; i < (uint32_t)kMemberBuckets; i += blockDim.x) fill[i] = 0;
+    __syncthreads();
+    for (uint32_t i = threadIdx.x; i < capacity; i += blockDim.x) {
+      const uint64_t t = table[i];
+      if (t == kEmptySlot) continue;
+      const uint32_t key = (uint32_t)(t >> 32);
+      uint32_t b = home(key);
+      for (int tries = 0; tries < kMemberBuckets; ++tries) {  // fewer keys than slots: ends early
+        const uint32_t at = atomicAdd(&fill[b], 1u);
+        if (at < 4u) {
+          lds_keys[b * 4 + at] = key;
+          lds_values[b * 4 + at] = (uint32_t)t;
+          break;
+        }
+        b = (b + 1) & (kMemberBuckets - 1);
+      }
+    }
+    __syncthreads();
+  }
+
+  // N look-ups in step; slot[j] is where key[j] sits, kMemberLdsSlots when it
+  // is absent (or kNoKey).
+  template <int N>
+  __device__ __forceinline__ void find_many(const uint32_t (&key)[N], uint32_t (&slot)[N]) const {
+    uint32_t b[N];
+    uint32_t open = 0;  // bit j: key j goes on to the next bucket
+#pragma unroll
+    for (int j = 0; j < N; ++j) {
+      slot[j] = kMemberLdsSlots;
+      b[j] = home(key[j]);
+      if (key[j] != kNoKey) open |= 1u << j;
+    }
+    for (int rounds = 0; open != 0 && rounds < kMemberBuckets; ++rounds) {
+      uint4 k[N];
+#pragma unroll
+      for (int j = 0; j < N; ++j) k[j] = keys[b[j]];
+#pragma unroll
+      for (int j = 0; j < N; ++j) {
+        if (!((open >> j) & 1u)) continue;
+        const int hit = k[j].x == key[j] ? 0 : k[j].y == key[j] ? 1 : k[j].z == key[j] ? 2
+                        : k[j].w == key[j] ? 3 : -1;
+        if (hit >= 0) {
+          slot[j] = b[j] * 4 + hit;
+          open &= ~(1u << j);
+        } else if (k[j].w == kNoKey) {
+          open &= ~(1u << j);  // a bucket with room would hold the key
+        } else {
+          b[j] = (b[j] + 1) & (kMemberBuckets - 1);
+        }
+      }
+    }
+  }
+};
+
 // kThreads: work-group size.  A large one shares a staged table among more
 // edges; a small one spreads a short edge list over all compute units.
 template <bool kInLds, int kThreads>
@@ -222,11 +300,19 @@ __global__ __launch_bounds__(kThreads) void member_flag_kernel(
     const int64_t* __restrict__ picked, const int* __restrict__ wide_flag,
     uint64_t* __restrict__ flags, int64_t* __restrict__ chunk_count,
     uint32_t* __restrict__ staged) {
-  __shared__ uint32_t lds_keys[kInLds ? kMemberLdsSlots : 1];
+  __shared__ __align__(16) uint32_t lds_keys[kInLds ? kMemberLdsSlots : 1];
   __shared__ uint32_t lds_values[kInLds ? kMemberLdsSlots : 1];
-  MemberTable<kInLds, true> table;
-  table.stage(global_table, cap, lds_keys, lds_values);
+  __shared__ uint32_t lds_fill[kInLds ? kMemberBuckets : 1];
   const bool wide = *wide_flag != 0;  // the same for every thread of the launch
+  const bool bucketed = kInLds && !wide;
+  MemberTable<kInLds, true> table;
+  BucketTable buckets;
+  if (bucketed) {
+    buckets.stage(global_table, cap, lds_keys, lds_values, lds_fill);
+  } else {
+    table.stage(global_table, cap, lds_keys, lds_values);
+  }
+  const uint32_t absent = bucketed ? (uint32_t)kMemberLdsSlots : cap;
   const int64_t num_chunks = ceil_div_dev(nnz, kBlock);
   const int64_t wave = (int64_t)blockIdx.x * (kThreads / kWave) + threadIdx.x / kWave;
   const int lane = lane_id();
@@ -251,7 +337,9 @@ __global__ __launch_bounds__(kThreads) void member_flag_kernel(
       if (chunk >= num_chunks) return;
       uint32_t slot[kMemberWords];
       uint64_t word[kMemberWords];
-      if (!wide) {
+      if (bucketed) {
+        buckets.find_many(keys[c], slot);
+      } else if (!wide) {
         table.find_many(keys[c], slot);
       } else {
 #pragma unroll
@@ -261,14 +349,14 @@ __global__ __launch_bounds__(kThreads) void member_flag_kernel(
         }
       }
 #pragma unroll
-      for (int j = 0; j < kMemberWords; ++j) word[j] = __ballot(slot[j] < cap);
+      for (int j = 0; j < kMemberWords; ++j) word[j] = __ballot(slot[j] < absent);
       {
         int before = 0;  // kept edges of the chunk in front of this row of 64
 #pragma unroll
         for (int j = 0; j < kMemberWords; ++j) {
-          if (slot[j] < cap)
+          if (slot[j] < absent)
             staged[chunk * kBlock + before + __popcll(word[j] & ((1ull << lane) - 1))] =
-                table.value_at(slot[j]);
+                bucketed ? buckets.values[slot[j]] : table.value_at(slot[j]);
           before += __popcll(word[j]);
         }
       }
