@@ -356,6 +356,40 @@ def ladies_sampler(A, seeds, fanouts):
     return seeds, ret
 
 
+def ladies_layer_sizes(A, seeds, fanouts):
+    """(columns sliced, edges of the column slice, edges kept by the row slice) per layer of
+    one eager run of ladies_sampler: what the byte counts of a step are taken from."""
+    sizes = []
+    for K in fanouts:
+        subA = A[:, seeds]
+        subA.edata["p"] = subA.edata["w"] ** 2
+        prob = subA.sum("p", axis=1)
+        sampleA, _ = subA.collective_sampling(K, prob, False)
+        sizes.append((int(seeds.numel()), int(subA.num_edges()), int(sampleA.num_edges())))
+        seeds = sampleA.all_nodes()
+    return sizes
+
+
+def ladies_kernel_bytes(name, sizes, num_rows):
+    """Algorithmic bytes of all launches of `name` in one LADIES step (interface reads
+    and writes; tables, scratch and re-reads excluded)."""
+    total = 0
+    for S, nnz, kept in sizes:
+        total += {
+            "col_slice_fill": 24 * S + 32 * nnz,          # seeds, indptr pair, row id in; 3 outputs
+            "gather_rows": 16 * nnz + 16 * kept,          # edge data of both slices: index + value in, value out
+            "member_flag": 8 * nnz,                       # row id of every edge
+            "member_fill": 4 * kept + 24 * kept,          # staged ids in; row, column, position out
+            "rowsum_hist": 8 * nnz, "rowsum_scatter": 12 * nnz + 8 * nnz,
+            "rowsum_accumulate": 8 * nnz + 4 * num_rows,
+            "spmm_coo_sum": 12 * nnz + 4 * num_rows,
+            "spmm_csc_sum": 4 * kept + 4 * S,
+            "sddmm": 2 * 20 * kept,                       # two quotients: value, id and operand in, value out
+            "first_position": 8 * kept,
+        }.get(name, 0)
+    return total
+
+
 def ladies_step_oracle(orc, indptr, indices, w, seeds, fanouts, num_rows, call_base):
     """The same two LADIES layers on the CPU: the oracle's operators chained by hand
     (column slice, e^2 row sums, weighted collective pick, row slice, the two
@@ -537,8 +571,16 @@ def run_ladies(args, wl, capi, dev):
     for _ in range(args.steps):
         step()
     torch.cuda.synchronize()
-    kernels = _kernel_table(capi, lambda name: 0)
+    totals_seen = capi.profile_totals()
     capi.profile_enable(False)
+    layer_sizes = ladies_layer_sizes(A, seeds, fanouts)
+    kernels = []
+    for name, (calls, ms) in totals_seen.items():
+        nbytes = ladies_kernel_bytes(name, layer_sizes, A.num_rows()) * args.steps
+        kernels.append(dict(kernel=name, launches=calls, avg_ms=round(ms / max(calls, 1), 4),
+                            total_ms=round(ms, 4), algorithmic_bytes=nbytes,
+                            gbs=round(nbytes / (ms * 1e-3) / 1e9, 1) if ms > 0 else 0.0))
+    kernels.sort(key=lambda k: -k["total_ms"])
     sliced = [int(b.num_edges()) for b in blocks]
     cpu = None
     if args.cpu_seconds > 0:
@@ -562,7 +604,8 @@ def run_ladies(args, wl, capi, dev):
         "ms_per_step": round(elapsed / args.steps * 1e3, 3), "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": f"{args.workload}: {wl['desc']}", "fanouts": fanouts,
-                   "seeds": wl["seeds"], "block_edges_last_step": sliced},
+                   "seeds": wl["seeds"], "block_edges_last_step": sliced,
+                   "layer_sizes_cols_sliced_kept": layer_sizes},
         "roofline": _roofline(kernels[0]), "cpu_baseline": cpu,
         "gpu_over_cpu": round(value / cpu["value"], 1) if cpu else None,
         "kernels": kernels, "graph_build_s": round(t_build, 1),
