@@ -157,6 +157,29 @@ def test_relabel_of_a_row_sliced_matrix(num_rows_picked, max_deg):
         assert first[l] == (hits[0] if hits.size else np.iinfo(np.int64).max)
 
 
+@pytest.mark.parametrize("num_rows_picked,num_cols_picked", [(1500, 800), (1200, 848), (1300, 700)])
+def test_relabel_of_a_row_sliced_matrix_with_a_long_list(num_rows_picked, num_cols_picked):
+    """Around the 2048 keys that one work-group relabels from the picked list
+    (more: sort + the general unique path; exactly that many and fewer: one
+    launch), with repeated seeds among the columns."""
+    rng = np.random.default_rng(num_rows_picked)
+    indptr, indices = random_csc(rng, 3000, 4000, 160, empty_frac=0.05)
+    m = gs.Matrix()
+    m.load_graph("CSC", [T(indptr), T(indices)])
+    cols = rng.integers(0, 3000, size=num_cols_picked)          # repeats allowed
+    picked = rng.permutation(4000)[:num_rows_picked]
+    sub = m[T(picked), T(cols)]
+    row, col, _ = sub.coo
+    assert row.numel() >= 8 * (num_rows_picked + num_cols_picked)   # the list path is taken
+    uniq, out_row, out_col, _ = sub._graph._CAPI_GraphRelabel(T(cols), T(picked))
+    keys = picked[row.cpu().numpy()]
+    want = orc.unique_relabel(cols, keys, edge_col=col.cpu().numpy())
+    assert np.array_equal(uniq.cpu().numpy(), want[0])
+    assert np.array_equal(out_row.cpu().numpy(), want[2])
+    assert np.array_equal(out_col.cpu().numpy(), want[3])
+    assert np.array_equal(sub.all_nodes().cpu().numpy(), want[0])
+
+
 def test_batched_column_and_row_slice_whose_encoded_ids_pass_32_bits():
     """_CAPI_BatchColRowSlcing encodes a row of batch b as id + b * num_rows
     (src/cuda/batch/slicing.cu:25-27).  With 2^30 + 5 rows and 8 batches the
