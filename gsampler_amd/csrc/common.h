@@ -35,6 +35,9 @@ int hip_fail(hipError_t e, const char* what, const char* file, int line);
 
 inline hipStream_t as_stream(gs_stream_t s) { return (hipStream_t)s; }
 
+// Compute units of the current device (256 on the part this is written for).
+int num_compute_units();
+
 // Optional per-kernel timing (gs_profile_*): while enabled, every launch that
 // sits inside a ProfScope is bracketed by two HIP events on its own stream.
 bool profile_enabled();

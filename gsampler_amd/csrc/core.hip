@@ -171,6 +171,19 @@ __global__ __launch_bounds__(kBlock) void scan_down_kernel(
 
 constexpr int64_t kShortSpine = 4096;  // tiles
 
+int num_compute_units() {
+  static int cached[64] = {0};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+  if (cached[dev] == 0) {
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
+      n = 256;
+    cached[dev] = n;
+  }
+  return cached[dev];
+}
+
 size_t scan_workspace_bytes(int64_t n) {
   int64_t tiles = n > 0 ? ceil_div(n, kScanTile) : 1;
   return align_up((size_t)tiles * sizeof(int64_t), 256);

@@ -33,12 +33,32 @@ constexpr int kMemberThreads = 1024;  // 16 waves share one staged table: 32 Ki 
 constexpr int kMemberLdsSlots = 4096;  // tables up to this size are staged in LDS (32 KB)
 constexpr int64_t kMemberSmallEdges = int64_t(1) << 23;  // below: work-groups of kBlock threads
 
+// A table too large for LDS is looked up in L2, one request per probe, and the
+// flag pass then runs at the rate of those requests.  Most edges are not kept
+// (a slice picks a small part of the rows), so a filter that does fit LDS sends
+// them away first: a word of 32 bits per id group, three bits per picked id
+// (a blocked Bloom filter; with up to eight ids per word about one absent id in
+// twenty passes).  Only ids that pass go on to the table.
+constexpr int kFilterWords = 16384;            // 64 KB of LDS
+constexpr int kFilterGroupsPerCu = 2;          // work-groups of 1024 threads that fit a compute unit
+constexpr int64_t kFilterMaxIds = 8 * kFilterWords;  // beyond: too many bits set to be worth a look
+
+__device__ __forceinline__ uint32_t filter_word(uint32_t key) {
+  return (key * 0x9E3779B1u) >> 18;  // top 14 bits: [0, kFilterWords)
+}
+__device__ __forceinline__ uint32_t filter_bits(uint32_t key) {
+  const uint32_t h = key * 0x85EBCA6Bu;
+  return (1u << (h >> 27)) | (1u << ((h >> 22) & 31u)) | (1u << ((h >> 17) & 31u));
+}
+static_assert(kFilterWords == 1 << 14, "filter_word keeps 14 bits");
+
 struct MemberWs {
   uint64_t* table;     // [member_table_slots(num_picked)]
   uint64_t* flags;     // [chunks * kMemberWords]
   uint32_t* staged;    // [chunks * kBlock]: per chunk, the new ids of its kept edges, in order
   int64_t* chunk_off;  // [chunks + 1]
   int* wide;           // [1] set when a picked id does not fit the upper half of a slot
+  uint32_t* filter;    // [kFilterWords] which ids may be in the table (for tables kept in L2)
   void* scan_ws;
   size_t scan_ws_bytes;
   int64_t chunks;
@@ -65,6 +85,7 @@ static MemberWs carve_member(void* ws, int64_t nnz, int64_t num_picked) {
   w.staged = c.take<uint32_t>((size_t)w.chunks * kBlock);
   w.chunk_off = c.take<int64_t>((size_t)w.chunks + 1);
   w.wide = c.take<int>(1);
+  w.filter = c.take<uint32_t>((size_t)kFilterWords);
   w.scan_ws_bytes = scan_workspace_bytes(w.chunks + 1);
   w.scan_ws = c.take<char>(w.scan_ws_bytes);
   w.total = c.total();
@@ -96,12 +117,13 @@ __device__ __forceinline__ uint32_t member_tag(uint64_t id) {
 // picked set is small next to the edges).
 __global__ __launch_bounds__(kBlock) void member_insert_kernel(
     const int64_t* __restrict__ picked, int64_t n, uint64_t* table, uint32_t cap,
-    int* __restrict__ wide) {
+    int* __restrict__ wide, uint32_t* filter) {
   const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
   if (i >= n) return;
   const uint64_t id = (uint64_t)picked[i];
   if (id > kMaxPackedKey) *wide = 1;  // every writer stores the same value
   const uint32_t key = member_tag(id);
+  if (filter) atomicOr(filter + filter_word(key), filter_bits(key));
   const uint64_t mine = ((uint64_t)key << 32) | (uint64_t)i;
   uint32_t slot = member_home(key, cap);
   for (uint32_t probes = 0; probes < cap; ++probes) {  // the table has free slots: ends early
@@ -122,10 +144,13 @@ __global__ __launch_bounds__(kBlock) void member_insert_kernel(
 
 // Empties the table and lowers the wide-id flag.
 __global__ __launch_bounds__(kBlock) void member_clear_kernel(uint64_t* table, int64_t n,
-                                                              int* __restrict__ wide) {
+                                                              int* __restrict__ wide,
+                                                              uint32_t* filter) {
   int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
   if (i == 0) *wide = 0;
   const int64_t stride = (int64_t)gridDim.x * kBlock;
+  if (filter)
+    for (int64_t j = i; j < kFilterWords; j += stride) filter[j] = 0u;
   for (; i < n; i += stride) table[i] = kEmptySlot;
 }
 
@@ -299,12 +324,18 @@ __global__ __launch_bounds__(kThreads) void member_flag_kernel(
     const uint64_t* __restrict__ global_table, uint32_t cap,
     const int64_t* __restrict__ picked, const int* __restrict__ wide_flag,
     uint64_t* __restrict__ flags, int64_t* __restrict__ chunk_count,
-    uint32_t* __restrict__ staged) {
+    uint32_t* __restrict__ staged, const uint32_t* __restrict__ filter) {
   __shared__ __align__(16) uint32_t lds_keys[kInLds ? kMemberLdsSlots : 1];
   __shared__ uint32_t lds_values[kInLds ? kMemberLdsSlots : 1];
   __shared__ uint32_t lds_fill[kInLds ? kMemberBuckets : 1];
+  __shared__ uint32_t lds_filter[kInLds ? 1 : kFilterWords];
   const bool wide = *wide_flag != 0;  // the same for every thread of the launch
   const bool bucketed = kInLds && !wide;
+  const bool filtered = !kInLds && !wide && filter != nullptr;
+  if (filtered) {
+    for (int i = threadIdx.x; i < kFilterWords; i += kThreads) lds_filter[i] = filter[i];
+    __syncthreads();
+  }
   MemberTable<kInLds, true> table;
   BucketTable buckets;
   if (bucketed) {
@@ -314,15 +345,19 @@ __global__ __launch_bounds__(kThreads) void member_flag_kernel(
   }
   const uint32_t absent = bucketed ? (uint32_t)kMemberLdsSlots : cap;
   const int64_t num_chunks = ceil_div_dev(nnz, kBlock);
-  const int64_t wave = (int64_t)blockIdx.x * (kThreads / kWave) + threadIdx.x / kWave;
   const int lane = lane_id();
+  // A wave takes runs of kMemberChunksPerWave chunks, the work-groups of the
+  // launch striding over the runs (a launch with fewer work-groups than runs
+  // stages its tables once per work-group, not once per run).
   // The ids of kMemberAhead chunks are requested together, before anything is
   // stored: a store between a load and its use makes the wait for the load
   // (loads and stores count down one in-order counter) a wait for everything.
-  const int64_t first_chunk = wave * kMemberChunksPerWave;
+  const int64_t num_runs = ceil_div_dev(num_chunks, kMemberChunksPerWave);
+  for (int64_t run = (int64_t)blockIdx.x * (kThreads / kWave) + threadIdx.x / kWave;
+       run < num_runs; run += (int64_t)gridDim.x * (kThreads / kWave))
   for (int part = 0; part < kMemberChunksPerWave / kMemberAhead; ++part) {
-    const int64_t chunk0 = first_chunk + part * kMemberAhead;
-    if (chunk0 >= num_chunks) return;
+    const int64_t chunk0 = run * kMemberChunksPerWave + part * kMemberAhead;
+    if (chunk0 >= num_chunks) break;
     uint32_t keys[kMemberAhead][kMemberWords];
 #pragma unroll
     for (int c = 0; c < kMemberAhead; ++c)
@@ -331,16 +366,41 @@ __global__ __launch_bounds__(kThreads) void member_flag_kernel(
         const int64_t e = (chunk0 + c) * kBlock + j * kWave + lane;
         keys[c][j] = e < nnz ? member_key((uint64_t)ids[e]) : kNoKey;
       }
+    if (filtered) {
+#pragma unroll
+      for (int c = 0; c < kMemberAhead; ++c)
+#pragma unroll
+        for (int j = 0; j < kMemberWords; ++j) {
+          const uint32_t bits = filter_bits(keys[c][j]);
+          if ((lds_filter[filter_word(keys[c][j])] & bits) != bits) keys[c][j] = kNoKey;
+        }
+    }
+    // a table in L2 answers after a round trip: the few look-ups that the filter
+    // lets through go through their probe rounds together for all chunks of the part
+    uint32_t all_slots[kMemberAhead * kMemberWords];
+    if (filtered) {
+      uint32_t all_keys[kMemberAhead * kMemberWords];
+#pragma unroll
+      for (int c = 0; c < kMemberAhead; ++c)
+#pragma unroll
+        for (int j = 0; j < kMemberWords; ++j) all_keys[c * kMemberWords + j] = keys[c][j];
+      table.find_many(all_keys, all_slots);
+    }
 #pragma unroll
     for (int c = 0; c < kMemberAhead; ++c) {
       const int64_t chunk = chunk0 + c;
-      if (chunk >= num_chunks) return;
+      if (chunk >= num_chunks) break;
       uint32_t slot[kMemberWords];
       uint64_t word[kMemberWords];
       if (bucketed) {
         buckets.find_many(keys[c], slot);
       } else if (!wide) {
-        table.find_many(keys[c], slot);
+        if (!filtered) {
+          table.find_many(keys[c], slot);
+        } else {
+#pragma unroll
+          for (int j = 0; j < kMemberWords; ++j) slot[j] = all_slots[c * kMemberWords + j];
+        }
       } else {
 #pragma unroll
         for (int j = 0; j < kMemberWords; ++j) {
@@ -515,23 +575,29 @@ int gs_minor_slice_count(const int64_t* ids, int64_t nnz, const int64_t* picked,
   }
   hipStream_t s = as_stream(stream);
   const uint32_t cap = (uint32_t)member_table_slots(num_picked);
+  const bool in_lds = cap <= (uint64_t)kMemberLdsSlots;
+  uint32_t* filter = !in_lds && num_picked <= kFilterMaxIds ? w.filter : nullptr;
   GS_LAUNCH("member_clear", s,
             member_clear_kernel<<<dim3((unsigned)ceil_div((int64_t)cap, kBlock * 4)),
-                                  dim3(kBlock), 0, s>>>(w.table, (int64_t)cap, w.wide));
+                                  dim3(kBlock), 0, s>>>(w.table, (int64_t)cap, w.wide, filter));
   if (num_picked > 0)
     GS_LAUNCH("member_insert", s,
               member_insert_kernel<<<dim3((unsigned)ceil_div(num_picked, kBlock)),
                                      dim3(kBlock), 0, s>>>(picked, num_picked,
-                                                           w.table, cap, w.wide));
+                                                           w.table, cap, w.wide, filter));
   if (nnz > 0) {
-    const bool in_lds = cap <= (uint64_t)kMemberLdsSlots;
     const bool small = nnz < kMemberSmallEdges;
     const int threads = small ? kBlock : kMemberThreads;
-    const dim3 grid((unsigned)ceil_div(w.chunks, (threads / kWave) * kMemberChunksPerWave));
+    int64_t blocks = ceil_div(w.chunks, (threads / kWave) * kMemberChunksPerWave);
+    // a work-group that stages the 64 KB filter does so once and strides over its runs
+    const int64_t resident = (int64_t)(kFilterGroupsPerCu * kMemberThreads / threads) * num_compute_units();
+    if (filter && blocks > resident) blocks = resident;
+    const dim3 grid((unsigned)blocks);
 #define GS_MEMBER_FLAG(LDS, THREADS)                                                          \
   GS_LAUNCH("member_flag", s,                                                                 \
             (member_flag_kernel<LDS, THREADS>)<<<grid, dim3(THREADS), 0, s>>>(                \
-                ids, nnz, w.table, cap, picked, w.wide, w.flags, w.chunk_off, w.staged))
+                ids, nnz, w.table, cap, picked, w.wide, w.flags, w.chunk_off, w.staged,       \
+                filter))
     if (in_lds && small) GS_MEMBER_FLAG(true, kBlock);
     else if (in_lds) GS_MEMBER_FLAG(true, kMemberThreads);
     else if (small) GS_MEMBER_FLAG(false, kBlock);

@@ -39,6 +39,18 @@ def test_minor_slice_parity(npick):
          orc.minor_slice(indices, picked, indptr=indptr, with_major=False))
 
 
+@pytest.mark.parametrize("npick", [20000, 140000])
+def test_minor_slice_with_a_table_outside_lds(npick):
+    """Picked sets whose table lives in L2: behind the filter that is kept in LDS
+    (up to 131 072 ids) and without it; 19 M edges, so that work-groups stride
+    over several runs of chunks."""
+    rng = np.random.default_rng(npick)
+    indptr, indices = random_csc(rng, 20000, 400000, 2400, hub_deg=60000)
+    picked = rng.integers(0, 410000, size=npick)  # repeats and absent ids
+    same(capi.minor_slice(T(indices), T(picked), indptr=T(indptr)),
+         orc.minor_slice(indices, picked, indptr=indptr))
+
+
 @pytest.mark.parametrize("npick", [3, 700, 5000])
 def test_minor_slice_with_ids_beyond_32_bits(npick):
     """Picked ids of 2^32 - 1 and above: ids that agree in their low 32 bits must
