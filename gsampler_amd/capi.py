@@ -65,6 +65,7 @@ SIGNATURES = {
     "gs_split_indptr": (_int, [_p, _p, _i64, _i64, _p, _p]),
     "gs_batch_seeds_distinct": (_int, [_p, _p, _p, _p, _i64, _p, _p]),
     "gs_first_position": (_int, [_p, _i64, _i64, _p, _p]),
+    "gs_csc_col_slice_values": (_int, [_p, _p, _i64, _p, _i64, _p, _i64, _p, _p]),
     "gs_list_labels": (_int, [_p, _i64, _p, _p, _i64, _p, _p, _p, _p, _p, _p]),
     "gs_gather_rows": (_int, [_p, _i64, _i64, _p, _i64, _p, _p, _p]),
     "gs_coo_sort_workspace_bytes": (_sz, [_i64, _i64]),
@@ -293,6 +294,22 @@ def col_slice(indptr, indices, column_ids, with_coo=True, batch_ptr=None,
                                       _ptr(out_col), _ptr(out_idx), _ptr(out_sel),
                                       _stream()))
     return sub_indptr, out_col, out_idx, out_sel
+
+
+def col_slice_values(indptr, column_ids, sub_indptr, values):
+    """Per-edge values (4- or 8-byte elements) of A[:, column_ids], from the parent's
+    `values` and the slice's `sub_indptr`."""
+    indptr, sub_indptr = _i64t(indptr, "indptr"), _i64t(sub_indptr, "sub_indptr")
+    if column_ids is not None:
+        column_ids = _i64t(column_ids, "column_ids")
+    values = values.contiguous()
+    n = sub_indptr.numel() - 1
+    nnz = int(sub_indptr[-1].item())
+    out = torch.empty(nnz, dtype=values.dtype, device=values.device)
+    check(lib().gs_csc_col_slice_values(_ptr(indptr), _ptr(column_ids), n, _ptr(sub_indptr), nnz,
+                                        values.data_ptr(), values.element_size(),
+                                        out.data_ptr(), _stream()))
+    return out
 
 
 def sample_uniform(indptr, indices, column_ids, fanout, replace=False,

@@ -292,8 +292,51 @@ GraphPtr Graph::derive(int64_t on_format, int64_t output_format,
 // tensor, which the kernel reads in place (IndexSelectCPUFromGPU,
 // src/cuda/index_select_uvm.cu:22-50, and dgl's gather_pinned_tensor_rows that
 // python/gs/matrix_api/matrix.py:19-23 calls for pinned edge data).
+// The edge index that the latest slice along a compressed axis returned, with
+// where its edges come from.  A slice copies runs of the parent's edges, so
+// scalar edge data of the slice (data[edge_index], which the Python layer asks
+// for right after slicing) can be copied by column ranges of the parent's
+// array without reading the 8-byte positions back.  Recognised by the identity
+// and version of the index tensor; one entry per thread, replaced by the next
+// slice.
+struct SliceRuns {
+  torch::Tensor select, parent_indptr, picked, sub_indptr;
+  int64_t version = -1, parent_edges = 0;
+  static SliceRuns& last() {
+    static thread_local SliceRuns s;
+    return s;
+  }
+  static void remember(const torch::Tensor& select, const torch::Tensor& parent_indptr,
+                       const torch::Tensor& picked, const torch::Tensor& sub_indptr,
+                       int64_t parent_edges) {
+    SliceRuns& s = last();
+    s.parent_edges = parent_edges;
+    s.select = select;
+    s.parent_indptr = parent_indptr;
+    s.picked = picked;
+    s.sub_indptr = sub_indptr;
+    s.version = (int64_t)select._version();
+  }
+  bool covers(const torch::Tensor& ids) const {
+    return select.defined() && ids.is_same(select) && (int64_t)ids._version() == version;
+  }
+};
+
 torch::Tensor GatherRows(torch::Tensor table, torch::Tensor ids) {
   TORCH_CHECK(table.dim() >= 1, "GatherRows: the table needs at least one axis");
+  {
+    const SliceRuns& runs = SliceRuns::last();
+    if (runs.covers(ids) && table.is_cuda() && table.dim() == 1 && table.is_contiguous() &&
+        (table.element_size() == 4 || table.element_size() == 8) &&
+        table.numel() >= runs.parent_edges) {
+      torch::Tensor out = torch::empty({ids.numel()}, table.options());
+      GS_CALL(gs_csc_col_slice_values(cptr(runs.parent_indptr), cptr(runs.picked),
+                                      runs.picked.numel(), cptr(runs.sub_indptr), ids.numel(),
+                                      table.data_ptr(), (int64_t)table.element_size(),
+                                      out.data_ptr(), cur_stream()));
+      return out;
+    }
+  }
   TORCH_CHECK(table.is_cuda() || table.is_pinned(),
               "GatherRows: the table must be on the GPU or in pinned host memory");
   TORCH_CHECK(ids.is_cuda() && ids.scalar_type() == torch::kInt64 && ids.dim() == 1,
@@ -343,6 +386,7 @@ GraphAndIndex Graph::Slicing(torch::Tensor seeds, int64_t axis,
   MajorResult r = along_major ? major_slice(m, seeds, with_coo, {}, 0)
                               : minor_slice(m, seeds, with_coo);
   GraphPtr g = derive(on_format, output_format, r, new_rows, new_cols);
+  if (along_major && !m.e_ids.has_value()) SliceRuns::remember(r.select, m.indptr, seeds, r.indptr, m.indices.numel());
   return {g, edge_index(m.e_ids, r.select)};
 }
 

@@ -115,11 +115,9 @@ __device__ __forceinline__ uint32_t member_tag(uint64_t id) {
 // *wide must be 0 before the launch.  Two picked ids with the same tag are the
 // same id unless one of them is wide, so matches are always confirmed here (the
 // picked set is small next to the edges).
-__global__ __launch_bounds__(kBlock) void member_insert_kernel(
-    const int64_t* __restrict__ picked, int64_t n, uint64_t* table, uint32_t cap,
-    int* __restrict__ wide, uint32_t* filter) {
-  const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
-  if (i >= n) return;
+__device__ __forceinline__ void member_insert_one(const int64_t* __restrict__ picked, int64_t i,
+                                                  uint64_t* table, uint32_t cap,
+                                                  int* __restrict__ wide, uint32_t* filter) {
   const uint64_t id = (uint64_t)picked[i];
   if (id > kMaxPackedKey) *wide = 1;  // every writer stores the same value
   const uint32_t key = member_tag(id);
@@ -127,7 +125,7 @@ __global__ __launch_bounds__(kBlock) void member_insert_kernel(
   const uint64_t mine = ((uint64_t)key << 32) | (uint64_t)i;
   uint32_t slot = member_home(key, cap);
   for (uint32_t probes = 0; probes < cap; ++probes) {  // the table has free slots: ends early
-    uint64_t cur = table[slot];
+    uint64_t cur = __hip_atomic_load(table + slot, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     if (cur == kEmptySlot) {
       cur = atomicCAS((unsigned long long*)(table + slot), (unsigned long long)kEmptySlot,
                       (unsigned long long)mine);
@@ -140,6 +138,29 @@ __global__ __launch_bounds__(kBlock) void member_insert_kernel(
     }
     if (++slot == cap) slot = 0;
   }
+}
+
+__global__ __launch_bounds__(kBlock) void member_insert_kernel(
+    const int64_t* __restrict__ picked, int64_t n, uint64_t* table, uint32_t cap,
+    int* __restrict__ wide, uint32_t* filter) {
+  const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (i >= n) return;
+  member_insert_one(picked, i, table, cap, wide, filter);
+}
+
+// Both in one work-group, for a table small enough (the picked set of a
+// layer-wise sampler): clear, barrier, insert.
+constexpr int kMemberSetupThreads = 1024;
+__global__ __launch_bounds__(kMemberSetupThreads) void member_setup_kernel(
+    const int64_t* __restrict__ picked, int64_t n, uint64_t* table, uint32_t cap,
+    int* __restrict__ wide) {
+  for (uint32_t i = threadIdx.x; i < cap; i += kMemberSetupThreads) table[i] = kEmptySlot;
+  if (threadIdx.x == 0) *wide = 0;
+  // the table is read and written below by other threads of this work-group
+  __threadfence_block();
+  __syncthreads();
+  for (int64_t i = threadIdx.x; i < n; i += kMemberSetupThreads)
+    member_insert_one(picked, i, table, cap, wide, nullptr);
 }
 
 // Empties the table and lowers the wide-id flag.
@@ -463,8 +484,8 @@ __global__ __launch_bounds__(kBlock) void member_indptr_kernel(
 // A wave writes the kept edges of kMemberChunksPerWave consecutive chunks.  What
 // it needs to know about them arrives in one round trip (lane l holds flag word
 // l of the wave's chunks, the first lanes also a chunk offset each); the columns
-// of the wave's first and last edge take a wavefront search each (one column
-// covers the whole span unless columns are short); then the staged ids of all
+// of the wave's first and last edge take a search each on the scalar unit (one
+// column covers the whole span unless columns are short); then the staged ids of all
 // chunks of a part are requested together, and only then anything is stored.
 // kEdgeMajor: the id on the other axis comes from edge_major (an edge list)
 // instead of the compressed pointer.
@@ -493,10 +514,7 @@ __global__ __launch_bounds__(kBlock) void member_fill_kernel(
       (first_chunk + kMemberChunksPerWave) * kBlock < nnz ? (first_chunk + kMemberChunksPerWave) * kBlock
                                                           : nnz;
   SegmentSpan span{0, 0};
-  if (out_major && !kEdgeMajor) {
-    span.lo = wave_segment_of(indptr, num_major, e_first);
-    span.hi = span.lo + wave_segment_of(indptr + span.lo, num_major - span.lo, e_end - 1);
-  }
+  if (out_major && !kEdgeMajor) span = segment_span(indptr, num_major, e_first, e_end - 1);
 #pragma unroll
   for (int part = 0; part < kMemberChunksPerWave / kMemberAhead; ++part) {
     const int c0 = part * kMemberAhead;
@@ -577,14 +595,19 @@ int gs_minor_slice_count(const int64_t* ids, int64_t nnz, const int64_t* picked,
   const uint32_t cap = (uint32_t)member_table_slots(num_picked);
   const bool in_lds = cap <= (uint64_t)kMemberLdsSlots;
   uint32_t* filter = !in_lds && num_picked <= kFilterMaxIds ? w.filter : nullptr;
-  GS_LAUNCH("member_clear", s,
-            member_clear_kernel<<<dim3((unsigned)ceil_div((int64_t)cap, kBlock * 4)),
-                                  dim3(kBlock), 0, s>>>(w.table, (int64_t)cap, w.wide, filter));
-  if (num_picked > 0)
+  if (in_lds) {
+    GS_LAUNCH("member_insert", s,
+              member_setup_kernel<<<dim3(1), dim3(kMemberSetupThreads), 0, s>>>(
+                  picked, num_picked, w.table, cap, w.wide));
+  } else {
+    GS_LAUNCH("member_clear", s,
+              member_clear_kernel<<<dim3((unsigned)ceil_div((int64_t)cap, kBlock * 4)),
+                                    dim3(kBlock), 0, s>>>(w.table, (int64_t)cap, w.wide, filter));
     GS_LAUNCH("member_insert", s,
               member_insert_kernel<<<dim3((unsigned)ceil_div(num_picked, kBlock)),
                                      dim3(kBlock), 0, s>>>(picked, num_picked,
                                                            w.table, cap, w.wide, filter));
+  }
   if (nnz > 0) {
     const bool small = nnz < kMemberSmallEdges;
     const int threads = small ? kBlock : kMemberThreads;

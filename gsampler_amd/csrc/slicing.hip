@@ -118,9 +118,81 @@ __global__ __launch_bounds__(kBlock) void col_slice_fill_kernel(
   }
 }
 
+// Per-edge values of the slice: out[sub_indptr[i] + k] = values[indptr[c_i] + k].
+// The edges of a sliced column are a run of the parent's edges, so the values
+// come straight from the parent's array; the edge positions the slice kernel
+// wrote (8 bytes per edge) are not read back.
+// (Four bytes in and out per edge: a work-group takes sixteen edges per thread
+// so that the look-ups at its head are paid once per 4096 edges.)
+constexpr int kValueItems = 16;
+constexpr int kValueTile = kBlock * kValueItems;
+template <typename T>
+__global__ __launch_bounds__(kBlock) void col_slice_values_kernel(
+    const int64_t* __restrict__ indptr, const int64_t* __restrict__ column_ids, int64_t num_items,
+    const int64_t* __restrict__ sub_indptr, int64_t nnz, const T* __restrict__ values,
+    T* __restrict__ out) {
+  const int64_t e0 = (int64_t)blockIdx.x * kValueTile;
+  if (e0 >= nnz) return;
+  const int64_t e_last = e0 + kValueTile - 1 < nnz ? e0 + kValueTile - 1 : nnz - 1;
+  const SegmentSpan span = segment_span(sub_indptr, num_items, e0, e_last);
+  // one column covers the tile (columns of a slice worth copying are long): its
+  // offset is the same for every edge
+  int64_t shift = 0;
+  if (span.lo == span.hi) {
+    const int64_t c = column_ids ? column_ids[span.lo] : span.lo;
+    shift = indptr[c] - sub_indptr[span.lo];
+  }
+  int64_t src[kValueItems];
+#pragma unroll
+  for (int j = 0; j < kValueItems; ++j) {
+    const int64_t e = e0 + j * kBlock + threadIdx.x;
+    src[j] = -1;
+    if (e >= nnz) continue;
+    if (span.lo == span.hi) {
+      src[j] = e + shift;
+    } else {
+      const int64_t item = span.segment_at(sub_indptr, e);
+      const int64_t c = column_ids ? column_ids[item] : item;
+      src[j] = indptr[c] + (e - sub_indptr[item]);
+    }
+  }
+  T v[kValueItems];
+#pragma unroll
+  for (int j = 0; j < kValueItems; ++j)
+    if (src[j] >= 0) v[j] = values[src[j]];
+#pragma unroll
+  for (int j = 0; j < kValueItems; ++j)
+    if (src[j] >= 0) out[e0 + j * kBlock + threadIdx.x] = v[j];
+}
+
 }  // namespace gs
 
 extern "C" {
+
+int gs_csc_col_slice_values(const int64_t* indptr, const int64_t* column_ids, int64_t num_items,
+                            const int64_t* sub_indptr, int64_t nnz, const void* values,
+                            int64_t value_bytes, void* out_values, gs_stream_t stream) {
+  using namespace gs;
+  GS_REQUIRE(num_items >= 0 && nnz >= 0, "col_slice_values: negative size");
+  GS_REQUIRE(value_bytes == 4 || value_bytes == 8,
+             "col_slice_values: values of 4 or 8 bytes, got %lld (gather by edge position instead)",
+             (long long)value_bytes);
+  if (nnz == 0 || num_items == 0) return GS_OK;
+  GS_REQUIRE(indptr && sub_indptr && values && out_values, "col_slice_values: null pointer");
+  hipStream_t s = as_stream(stream);
+  const dim3 grid((unsigned)ceil_div(nnz, kValueTile));
+  if (value_bytes == 4)
+    GS_LAUNCH("col_slice_values", s,
+              col_slice_values_kernel<uint32_t><<<grid, dim3(kBlock), 0, s>>>(
+                  indptr, column_ids, num_items, sub_indptr, nnz, (const uint32_t*)values,
+                  (uint32_t*)out_values));
+  else
+    GS_LAUNCH("col_slice_values", s,
+              col_slice_values_kernel<uint64_t><<<grid, dim3(kBlock), 0, s>>>(
+                  indptr, column_ids, num_items, sub_indptr, nnz, (const uint64_t*)values,
+                  (uint64_t*)out_values));
+  return GS_OK;
+}
 
 int gs_csc_col_count(const int64_t* indptr, int64_t num_cols,
                      const int64_t* column_ids, int64_t num_items,

@@ -561,6 +561,23 @@ __global__ void list_counts_kernel(const int64_t* __restrict__ range, int64_t n,
   counts[b] = cnt;
 }
 
+// The same for at most kBlock - 1 segments, with the running sum: one launch
+// instead of counts + scan.
+__global__ __launch_bounds__(kBlock) void list_offsets_kernel(
+    const int64_t* __restrict__ range, int64_t n, int64_t nseg, int64_t num_picks, int replace,
+    int64_t* __restrict__ out_range) {
+  __shared__ int64_t smem[kBlock / kWave + 1];
+  const int64_t b = threadIdx.x;
+  int64_t cnt = 0;
+  if (b < nseg) {
+    const int64_t nb = range ? range[b + 1] - range[b] : n;
+    cnt = replace ? (nb > 0 ? num_picks : 0) : (nb < num_picks ? nb : num_picks);
+  }
+  int64_t total;
+  const int64_t before = block_exclusive_sum(cnt, smem, &total);
+  if (b <= nseg) out_range[b] = before;
+}
+
 // Copies the first out_range[b+1] - out_range[b] sorted values of every
 // segment; a segment that is taken whole keeps its original order.
 __global__ __launch_bounds__(kBlock) void list_take_kernel(
@@ -1169,6 +1186,12 @@ int gs_list_sample_weighted_count(const int64_t* range, int64_t n,
     return GS_ERR_WORKSPACE;
   }
   hipStream_t s = as_stream(stream);
+  if (num_segments < kBlock) {
+    GS_LAUNCH("list_counts", s,
+              list_offsets_kernel<<<dim3(1), dim3(kBlock), 0, s>>>(range, n, num_segments,
+                                                                   num_picks, replace, out_range));
+    return GS_OK;
+  }
   GS_LAUNCH("list_counts", s,
             list_counts_kernel<<<dim3((unsigned)ceil_div(num_segments + 1, kBlock)),
                                  dim3(kBlock), 0, s>>>(range, n, num_segments,

@@ -161,6 +161,17 @@ int gs_csc_col_slice_fill(const int64_t* indptr, int64_t num_cols,
                           int64_t* out_indices, int64_t* out_select,
                           gs_stream_t stream);
 
+/* Edge data of a column slice: out_values[sub_indptr[i] + k] = values[indptr[c_i] + k]
+ * for values of 4 or 8 bytes aligned with the parent's edges (c_i = column_ids[i],
+ * or i when column_ids is NULL).  The same result as gathering values by the
+ * edge positions that gs_csc_col_slice_fill wrote (data_index(edata, edge_index),
+ * python/gs/matrix_api/matrix.py:19-23 behind the slice of :103) without reading
+ * those positions back. */
+int gs_csc_col_slice_values(const int64_t* indptr, const int64_t* column_ids,
+                            int64_t num_items, const int64_t* sub_indptr, int64_t nnz,
+                            const void* values, int64_t value_bytes, void* out_values,
+                            gs_stream_t stream);
+
 /* ------------------------------------------------------------------------
  * Uniform per-column sampling (fill phase), optionally fused with the column
  * slice (column_ids != NULL).  sub_indptr comes from gs_csc_col_count with
