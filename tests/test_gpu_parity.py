@@ -97,6 +97,28 @@ def test_sample_replace_and_unfused_parity(fanout):
                 orc.sample_uniform(indptr, indices, cols, 100, False))
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.int64, torch.float64, torch.int32])
+def test_col_slice_values_equal_a_gather_by_the_edge_positions(dtype):
+    """Edge data of A[:, cols] copied by column runs of the parent's array is what
+    indexing the data with the slice's edge positions gives (the positions are the
+    oracle-checked output of the column slice)."""
+    rng = np.random.default_rng(3)
+    indptr, indices = random_csc(rng, 4000, 3000, 60, hub_deg=30000)
+    nnz = int(indptr[-1])
+    data = torch.as_tensor(rng.integers(0, 1 << 20, size=nnz), device=DEV).to(dtype)
+    for cols in (rng.integers(0, 4000, size=700), np.arange(4000), np.empty(0, dtype=np.int64),
+                 np.full(5, int(np.argmax(np.diff(indptr))))):      # repeats of the hub column
+        sub_indptr, _, _, sel = capi.col_slice(T(indptr), T(indices), T(cols))
+        want = orc.col_slice(indptr, indices, cols)
+        assert np.array_equal(N(sel), want[3])
+        got = capi.col_slice_values(T(indptr), T(cols), sub_indptr, data)
+        assert torch.equal(got, data[sel])
+    whole = capi.col_slice_values(T(indptr), None, T(indptr), data)   # every column, in order
+    assert torch.equal(whole, data)
+    with pytest.raises(capi.GsError, match="4 or 8 bytes"):
+        capi.col_slice_values(T(indptr), None, T(indptr), data.to(torch.float16))
+
+
 def _batched_case(rng, B, max_seeds, max_rows, id_range):
     s_sizes = rng.integers(1, max_seeds, size=B)
     r_sizes = rng.integers(0, max_rows, size=B)
