@@ -302,6 +302,7 @@ GraphPtr Graph::derive(int64_t on_format, int64_t output_format,
 struct SliceRuns {
   torch::Tensor select, parent_indptr, picked, sub_indptr;
   int64_t version = -1, parent_edges = 0;
+  int64_t source_versions[3] = {-1, -1, -1};  // of parent_indptr, picked, sub_indptr
   static SliceRuns& last() {
     static thread_local SliceRuns s;
     return s;
@@ -316,9 +317,16 @@ struct SliceRuns {
     s.picked = picked;
     s.sub_indptr = sub_indptr;
     s.version = (int64_t)select._version();
+    s.source_versions[0] = (int64_t)parent_indptr._version();
+    s.source_versions[1] = (int64_t)picked._version();
+    s.source_versions[2] = (int64_t)sub_indptr._version();
   }
+  // the index is the one remembered and nothing was written to since
   bool covers(const torch::Tensor& ids) const {
-    return select.defined() && ids.is_same(select) && (int64_t)ids._version() == version;
+    return select.defined() && ids.is_same(select) && (int64_t)ids._version() == version &&
+           (int64_t)parent_indptr._version() == source_versions[0] &&
+           (int64_t)picked._version() == source_versions[1] &&
+           (int64_t)sub_indptr._version() == source_versions[2];
   }
 };
 

@@ -134,6 +134,37 @@ def test_matrix_row_and_column_slicing_with_edata():
     assert np.array_equal(subc._CAPI_GetCOOCols().cpu().numpy(), col[mask])
 
 
+def test_column_slice_carries_edge_data_of_any_shape():
+    """Edge data of A[:, cols]: scalar data goes by column runs of the parent's
+    array, anything else through the edge index; both are data[edge positions]."""
+    rng = np.random.default_rng(9)
+    indptr, indices = random_csc(rng, 500, 300, 40, hub_deg=5000)
+    nnz = indices.size
+    m = gs.Matrix()
+    m.load_graph("CSC", [T(indptr), T(indices)])
+    data = {"f32": torch.as_tensor(rng.random(nnz, dtype=np.float32), device=DEV),
+            "f64": torch.as_tensor(rng.random(nnz), device=DEV),
+            "i64": T(rng.integers(0, 10**12, size=nnz)),
+            "f16": torch.as_tensor(rng.random(nnz, dtype=np.float32), device=DEV).half(),
+            "wide": torch.as_tensor(rng.random((nnz, 3), dtype=np.float32), device=DEV),
+            "strided": torch.as_tensor(rng.random((nnz, 2), dtype=np.float32), device=DEV)[:, 0]}
+    for key, value in data.items():
+        m.edata[key] = value
+    for cols in (rng.integers(0, 500, size=90), np.arange(500)):
+        sub = m[:, T(cols)]
+        want = orc.col_slice(indptr, indices, cols)
+        sel = torch.as_tensor(want[3], device=DEV)
+        assert np.array_equal(sub.csc[1].cpu().numpy(), want[2])
+        for key, value in data.items():
+            assert torch.equal(sub.edata[key], value[sel]), key
+    # a second slice in between does not confuse the first one's edge index
+    g = m._graph
+    a, sel_a = g._CAPI_Slicing(T(np.arange(10)), 1, gs._CSC, gs._CSC)
+    b, sel_b = g._CAPI_Slicing(T(np.arange(20, 60)), 1, gs._CSC, gs._CSC)
+    for sel in (sel_a, sel_b):
+        assert torch.equal(torch.ops.gs_ops._CAPI_GatherRows(data["f32"], sel), data["f32"][sel])
+
+
 @pytest.mark.parametrize("num_rows_picked,max_deg", [(6, 400), (40, 12)])
 def test_relabel_of_a_row_sliced_matrix(num_rows_picked, max_deg):
     """After row slicing the rows of a matrix are positions in the list of picked
