@@ -1013,6 +1013,25 @@ __global__ __launch_bounds__(kBlock) void unique_fill_kernel(
 }
 
 // ---------------------------------------------------------------- relabel
+// The largest c in [0, n) with ptr[c] <= x (ptr nondecreasing, ptr[0] <= x) when
+// a good guess is at hand: the wavefront looks at the 64 entries around the
+// guess first, one round trip, and searches the rest only when the answer is
+// not among them.  Columns of a sampled matrix hold about the same number of
+// edges, so the column of an edge is close to its share of the batch's columns.
+__device__ __forceinline__ int64_t wave_segment_near(const int64_t* __restrict__ ptr, int64_t n,
+                                                     int64_t x, int64_t guess) {
+  int64_t w0 = guess - kWave / 2;
+  if (w0 > n - kWave) w0 = n - kWave;
+  if (w0 < 0) w0 = 0;
+  const int64_t c = w0 + lane_id();
+  const bool ok = c < n && ptr[c] <= x;
+  const int hits = __popcll(__ballot(ok));  // ok is monotone over the lanes
+  if (hits == 0) return wave_segment_of(ptr, w0, x);  // before the window (w0 > 0 here)
+  if (hits == kWave && w0 + kWave < n)
+    return w0 + kWave - 1 + wave_segment_of(ptr + w0 + kWave - 1, n - (w0 + kWave - 1), x);
+  return w0 + hits - 1;
+}
+
 // The column of every edge of a tile from the column pointer: edge e belongs
 // to the last column c with col_indptr[c] <= e.  Two wavefronts find the
 // columns of the tile's first and last edge among [col_begin, col_end), the
@@ -1022,7 +1041,8 @@ __global__ __launch_bounds__(kBlock) void unique_fill_kernel(
 // carries the marks forward.  Leaves column - c_lo in head[] and returns c_lo.
 __device__ __forceinline__ int64_t tile_columns(const int64_t* __restrict__ col_indptr,
                                                 int64_t col_begin, int64_t col_end, int64_t e0,
-                                                int64_t e1, int32_t* head, int64_t* ends,
+                                                int64_t e1, int64_t guess_lo, int64_t guess_hi,
+                                                int32_t* head, int64_t* ends,
                                                 int32_t* wave_max) {
   static_assert(kRelabelItems % 4 == 0, "a thread scans whole int4s of head[]");
   constexpr int kQuads = kRelabelItems / 4;
@@ -1031,8 +1051,9 @@ __device__ __forceinline__ int64_t tile_columns(const int64_t* __restrict__ col_
 #pragma unroll
   for (int q = 0; q < kQuads; ++q) quads[q] = make_int4(0, 0, 0, 0);
   if (wave < 2) {
-    const int64_t c = wave_segment_of(col_indptr + col_begin, col_end - col_begin,
-                                        wave == 0 ? e0 : e1 - 1);
+    const int64_t c = wave_segment_near(col_indptr + col_begin, col_end - col_begin,
+                                        wave == 0 ? e0 : e1 - 1,
+                                        (wave == 0 ? guess_lo : guess_hi) - col_begin);
     if (lane_id() == 0) ends[wave] = col_begin + c;
   }
   __syncthreads();
@@ -1115,9 +1136,15 @@ __global__ __launch_bounds__(kBlock) void unique_relabel_kernel(
   if (kByIndptr && out_col) {
     // (after the loads above have been issued: they travel during the search)
     const int64_t e1 = e0 + kRelabelTile < k.E ? e0 + kRelabelTile : k.E;
-    const BatchInfo last = batch[span.hi];
-    const int64_t c_lo = tile_columns(col_indptr, batch[span.lo].s_lo, last.s_lo + last.ns, e0,
-                                      e1, head, ends, wave_max);
+    const BatchInfo head_b = batch[span.lo], last = batch[span.hi];
+    // an edge's share of its batch's edges, taken of the batch's columns
+    auto guess = [](const BatchInfo& b, int64_t e) {
+      const int64_t edges = b.n - b.ns;
+      return b.s_lo + (edges > 0 ? (int64_t)((double)(e - b.r_lo) / (double)edges * (double)b.ns) : 0);
+    };
+    const int64_t c_lo = tile_columns(col_indptr, head_b.s_lo, last.s_lo + last.ns, e0, e1,
+                                      guess(head_b, e0), guess(last, e1 - 1), head, ends,
+                                      wave_max);
 #pragma unroll
     for (int i = 0; i < kRelabelItems; ++i) col[i] = c_lo + head[i * kBlock + threadIdx.x];
   }
