@@ -205,11 +205,14 @@ MajorResult major_slice(const Compressed& m, const torch::Tensor& picked,
 const torch::Tensor& Compressed::narrow_indices() const {
   constexpr int64_t kMinEdges = int64_t(1) << 20;
   const int64_t version = (int64_t)indices._version();
-  if (indices32.defined() && indices32_version != version) indices32 = torch::Tensor();  // edited in place
+  if (indices32.defined() &&
+      (indices32_version != version || indices32_source != indices.data_ptr()))
+    indices32 = torch::Tensor();  // edited in place, or another array
   if (!indices32.defined() && num_minor >= 0 && num_minor < (int64_t(1) << 31) &&
       indices.is_cuda() && indices.numel() >= kMinEdges) {
     indices32 = indices.to(torch::kInt32);
     indices32_version = version;
+    indices32_source = indices.data_ptr();
   }
   return indices32;
 }

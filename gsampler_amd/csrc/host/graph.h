@@ -34,7 +34,12 @@ struct Compressed {
   // memory whose ids fit.
   mutable torch::Tensor indices32;
   mutable int64_t indices32_version = -1;  // version of `indices` the copy was made from
+  mutable const void* indices32_source = nullptr;  // and its address
   const torch::Tensor& narrow_indices() const;
+  // Call after assigning another `indices` or `indptr` to a matrix that was used.
+  void forget_derived() {
+    indices32 = torch::Tensor();
+  }
 };
 
 struct Coordinate {

@@ -67,6 +67,7 @@ void Graph::SortCSCIndices() {
                               mptr(sorted), nnz, num_rows_, ws.data_ptr(), ws.numel(),
                               cur_stream()));
   csc_->indices = sorted;
+  csc_->forget_derived();
   csc_sorted_ = true;
   coo_ = nullptr;  // derived formats followed the old edge order
   csr_ = nullptr;
@@ -107,6 +108,7 @@ GraphAndIndex Graph::Compact(int64_t axis) {
     }
     auto m = std::make_shared<Compressed>(*other);
     m->indices = ids_local;
+    m->forget_derived();
     (axis == 0 ? csc : csr) = m;
   }
   TORCH_CHECK(kept.defined(), "Compact: the graph has no format with explicit ids on axis ",

@@ -140,3 +140,26 @@ def test_batch_col_row_slicing():
             assert got == want
             k += len(want)
     assert k == cx.size and sub.num_rows() == 160 and sub.num_cols() == 80
+
+
+def test_sampling_after_a_column_sort_reads_the_sorted_row_ids():
+    """From 2^20 edges on the uniform sampler reads an int32 copy of the row
+    ids; a sort of the columns replaces the array the copy was made from."""
+    n = 60000
+    indptr, indices = chung_lu_csc(n, 1300000, seed=9, sort_rows=False)
+    indptr, indices = indptr.numpy(), indices.numpy()
+    assert indices.size >= 1 << 20
+    m = gs.Matrix()
+    m.load_graph("CSC", [T(indptr), T(indices)])
+    seeds = np.random.default_rng(3).integers(0, n, size=3000)
+    gs.manual_seed(4)
+    CSC = 2
+    sub, _ = m._graph._CAPI_SlicingSampling(1, T(seeds), 5, False, CSC, CSC)   # fused: reads m's own arrays
+    want = orc.sample_uniform(indptr, indices, seeds, 5, False, 0, 4, 0)
+    assert np.array_equal(sub._CAPI_GetCSCIndices().cpu().numpy(), want[2])
+    m._graph._CAPI_SortCSCIndices()
+    srt = orc.segment_sort(indptr, indices)
+    assert not np.array_equal(srt, indices)
+    sub, _ = m._graph._CAPI_SlicingSampling(1, T(seeds), 5, False, CSC, CSC)
+    want = orc.sample_uniform(indptr, srt, seeds, 5, False, 0, 4, 1)
+    assert np.array_equal(sub._CAPI_GetCSCIndices().cpu().numpy(), want[2])
