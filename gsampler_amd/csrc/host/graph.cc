@@ -301,9 +301,12 @@ GraphPtr Graph::derive(int64_t on_format, int64_t output_format,
 // for right after slicing) can be copied by column ranges of the parent's
 // array without reading the 8-byte positions back.  Recognised by the identity
 // and version of the index tensor; one entry per thread, replaced by the next
-// slice.
+// slice.  The index itself (8 bytes per edge) is held weakly, so the entry does
+// not keep it alive after its users are gone; the three small arrays the copy
+// kernel reads are held.
 struct SliceRuns {
-  torch::Tensor select, parent_indptr, picked, sub_indptr;
+  c10::optional<c10::weak_intrusive_ptr<c10::TensorImpl>> select;
+  torch::Tensor parent_indptr, picked, sub_indptr;
   int64_t version = -1, parent_edges = 0;
   int64_t source_versions[3] = {-1, -1, -1};  // of parent_indptr, picked, sub_indptr
   static SliceRuns& last() {
@@ -315,7 +318,7 @@ struct SliceRuns {
                        int64_t parent_edges) {
     SliceRuns& s = last();
     s.parent_edges = parent_edges;
-    s.select = select;
+    s.select = c10::weak_intrusive_ptr<c10::TensorImpl>(select.getIntrusivePtr());
     s.parent_indptr = parent_indptr;
     s.picked = picked;
     s.sub_indptr = sub_indptr;
@@ -326,7 +329,11 @@ struct SliceRuns {
   }
   // the index is the one remembered and nothing was written to since
   bool covers(const torch::Tensor& ids) const {
-    return select.defined() && ids.is_same(select) && (int64_t)ids._version() == version &&
+    if (!select.has_value() || !ids.defined()) return false;
+    // a live target cannot have been replaced by another tensor at the same address
+    const c10::intrusive_ptr<c10::TensorImpl> held = select->lock();
+    return held && held.get() == ids.unsafeGetTensorImpl() &&
+           (int64_t)ids._version() == version &&
            (int64_t)parent_indptr._version() == source_versions[0] &&
            (int64_t)picked._version() == source_versions[1] &&
            (int64_t)sub_indptr._version() == source_versions[2];
