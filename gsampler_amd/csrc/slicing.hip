@@ -142,6 +142,26 @@ __global__ __launch_bounds__(kBlock) void col_slice_values_kernel(
     const int64_t c = column_ids ? column_ids[span.lo] : span.lo;
     shift = indptr[c] - sub_indptr[span.lo];
   }
+  if (span.lo == span.hi && e0 + kValueTile <= nnz && ((uintptr_t)out & 15) == 0) {
+    // a whole tile out of one column: 16 bytes per lane and instruction; the
+    // source run starts wherever the column does, so its vectors are only
+    // aligned to the value size (the loads are issued as such)
+    constexpr int kPer = 16 / (int)sizeof(T), kVecs = kValueItems / kPer;
+    struct Vec {
+      T v[kPer];
+    };
+    const T* from = values + e0 + shift;
+    T* to = out + e0;
+    Vec held[kVecs];
+#pragma unroll
+    for (int j = 0; j < kVecs; ++j)
+      __builtin_memcpy(&held[j], from + (j * kBlock + (int)threadIdx.x) * kPer, sizeof(Vec));
+#pragma unroll
+    for (int j = 0; j < kVecs; ++j)
+      __builtin_memcpy(__builtin_assume_aligned(to + (j * kBlock + (int)threadIdx.x) * kPer, 16),
+                       &held[j], sizeof(Vec));
+    return;
+  }
   int64_t src[kValueItems];
 #pragma unroll
   for (int j = 0; j < kValueItems; ++j) {
