@@ -93,6 +93,39 @@ __global__ __launch_bounds__(kBlock) void col_slice_fill_kernel(
   // columns that the tile touches: one search per work-group (on the scalar
   // unit) instead of one per edge; a long column covers whole tiles
   const SegmentSpan span = segment_span(sub_indptr, num_items, e0, e_last);
+  if (span.lo == span.hi && e0 + kSliceTile <= nnz &&
+      (((uintptr_t)out_indices | (uintptr_t)out_select | (uintptr_t)out_coo_col) & 15) == 0) {
+    // a whole tile out of one column: two edges (16 bytes) per lane and
+    // instruction; the source run is only aligned to 8 bytes
+    struct Pair {
+      int64_t v[2];
+    };
+    const int64_t col = span.lo;
+    const int64_t c = column_ids ? column_ids[col] : col;
+    const int64_t shift = indptr[c] - sub_indptr[col];
+    int64_t add = 0;
+    if (batch_ptr != nullptr && encode_stride > 0)
+      add = segment_of(batch_ptr, num_batches, col) * encode_stride;
+    constexpr int kVecs = kSliceItems / 2;
+    Pair rows[kVecs];
+#pragma unroll
+    for (int j = 0; j < kVecs; ++j)
+      __builtin_memcpy(&rows[j], indices + e0 + shift + (j * kBlock + (int)threadIdx.x) * 2,
+                       sizeof(Pair));
+#pragma unroll
+    for (int j = 0; j < kVecs; ++j) {
+      const int64_t e = e0 + (j * kBlock + (int)threadIdx.x) * 2;
+      const Pair r{{rows[j].v[0] + add, rows[j].v[1] + add}};
+      const Pair p{{e + shift, e + shift + 1}};
+      __builtin_memcpy(__builtin_assume_aligned(out_indices + e, 16), &r, sizeof(Pair));
+      __builtin_memcpy(__builtin_assume_aligned(out_select + e, 16), &p, sizeof(Pair));
+      if (out_coo_col) {
+        const Pair cc{{col, col}};
+        __builtin_memcpy(__builtin_assume_aligned(out_coo_col + e, 16), &cc, sizeof(Pair));
+      }
+    }
+    return;
+  }
   int64_t item[kSliceItems], in_pos[kSliceItems], row[kSliceItems];
 #pragma unroll
   for (int j = 0; j < kSliceItems; ++j) {
@@ -122,9 +155,10 @@ __global__ __launch_bounds__(kBlock) void col_slice_fill_kernel(
 // The edges of a sliced column are a run of the parent's edges, so the values
 // come straight from the parent's array; the edge positions the slice kernel
 // wrote (8 bytes per edge) are not read back.
-// (Four bytes in and out per edge: a work-group takes sixteen edges per thread
-// so that the look-ups at its head are paid once per 4096 edges.)
-constexpr int kValueItems = 16;
+// (Four bytes in and out per edge: a work-group takes eight edges per thread,
+// so the look-ups at its head are paid once per 2048 edges; four, sixteen and
+// thirty-two per thread all measured slower.)
+constexpr int kValueItems = 8;
 constexpr int kValueTile = kBlock * kValueItems;
 template <typename T>
 __global__ __launch_bounds__(kBlock) void col_slice_values_kernel(
