@@ -98,17 +98,16 @@ void profile_end(hipStream_t stream) {
 
 // ------------------------------------------------------------------ scan
 // Three launches: per-tile sums, a single-block scan of the tile sums, and a
-// per-tile down-sweep.  A tile is kBlock threads x kScanItems consecutive
-// values per thread, so global accesses stay coalesced per thread-vector.
+// per-tile down-sweep.  A tile is kScanTile consecutive values.
 
 __global__ __launch_bounds__(kBlock) void scan_tile_sums_kernel(
     const int64_t* __restrict__ in, int64_t n, int64_t* __restrict__ tile_sums) {
   __shared__ int64_t smem[kBlock / kWave + 1];
-  const int64_t base = (int64_t)blockIdx.x * kScanTile + threadIdx.x * kScanItems;
+  const int64_t base = (int64_t)blockIdx.x * kScanTile + threadIdx.x;
   int64_t s = 0;
 #pragma unroll
   for (int k = 0; k < kScanItems; ++k) {
-    int64_t i = base + k;
+    const int64_t i = base + k * kBlock;  // the order of an integer sum does not matter
     if (i < n) s += in[i];
   }
   int64_t total;
@@ -134,19 +133,33 @@ __global__ __launch_bounds__(kBlock) void scan_spine_kernel(int64_t* tile_sums,
 // Tile t adds the sums of the tiles before it: already scanned by
 // scan_spine_kernel (kSpineDone), or summed here by the tile itself
 // (kSpineDone == false, for spines short enough that a launch costs more).
+// Inside a tile every wavefront owns a contiguous quarter and walks it in
+// rounds of 128 values, two neighbouring values (16 bytes) per lane, so each
+// load and store of a wavefront covers one contiguous kilobyte; the running sum
+// travels from round to round in a register and the four wavefronts meet once.
+constexpr int kScanRounds = kScanItems / 2;
+static_assert(kScanItems % 2 == 0, "a lane takes pairs of values");
+
 template <bool kSpineDone>
 __global__ __launch_bounds__(kBlock) void scan_down_kernel(
     const int64_t* in, int64_t* out, int64_t n,
     const int64_t* __restrict__ tile_sums, int64_t* last_mirror) {
   __shared__ int64_t smem[kBlock / kWave + 1];
-  const int64_t base = (int64_t)blockIdx.x * kScanTile + threadIdx.x * kScanItems;
-  int64_t v[kScanItems];
-  int64_t s = 0;
+  __shared__ int64_t wave_total[kBlock / kWave];
+  struct Pair {
+    int64_t v[2];
+  };
+  const int lane = lane_id(), wave = threadIdx.x / kWave;
+  const int64_t wave0 = (int64_t)blockIdx.x * kScanTile + (int64_t)wave * (kScanTile / (kBlock / kWave));
+  Pair held[kScanRounds];
 #pragma unroll
-  for (int k = 0; k < kScanItems; ++k) {
-    int64_t i = base + k;
-    v[k] = i < n ? in[i] : 0;
-    s += v[k];
+  for (int r = 0; r < kScanRounds; ++r) {
+    const int64_t i = wave0 + r * (2 * kWave) + 2 * lane;
+    held[r] = Pair{{0, 0}};
+    if (i + 1 < n)
+      __builtin_memcpy(&held[r], in + i, sizeof(Pair));
+    else if (i < n)
+      held[r].v[0] = in[i];
   }
   int64_t before = 0;
   if (kSpineDone) {
@@ -158,14 +171,31 @@ __global__ __launch_bounds__(kBlock) void scan_down_kernel(
     int64_t ignored = block_exclusive_sum(part, smem, &before);
     (void)ignored;
   }
-  int64_t total;
-  int64_t ex = block_exclusive_sum(s, smem, &total) + before;
+  // exclusive sums inside the wavefront's quarter
+  int64_t ex[kScanRounds];
+  int64_t running = 0;
 #pragma unroll
-  for (int k = 0; k < kScanItems; ++k) {
-    int64_t i = base + k;
-    if (i < n) out[i] = ex;
-    if (i == n - 1 && last_mirror) *last_mirror = ex;
-    ex += v[k];
+  for (int r = 0; r < kScanRounds; ++r) {
+    const int64_t own = held[r].v[0] + held[r].v[1];
+    const int64_t incl = wave_inclusive_sum(own);
+    ex[r] = running + incl - own;
+    running += __shfl(incl, kWave - 1, kWave);
+  }
+  if (lane == 0) wave_total[wave] = running;
+  __syncthreads();
+  for (int w = 0; w < wave; ++w) before += wave_total[w];
+#pragma unroll
+  for (int r = 0; r < kScanRounds; ++r) {
+    const int64_t i = wave0 + r * (2 * kWave) + 2 * lane;
+    const Pair result{{before + ex[r], before + ex[r] + held[r].v[0]}};
+    if (i + 1 < n)
+      __builtin_memcpy(out + i, &result, sizeof(Pair));
+    else if (i < n)
+      out[i] = result.v[0];
+    if (last_mirror) {
+      if (i == n - 1) *last_mirror = result.v[0];
+      if (i + 1 == n - 1) *last_mirror = result.v[1];
+    }
   }
 }
 
