@@ -1123,9 +1123,14 @@ __global__ __launch_bounds__(kBlock) void unique_relabel_kernel(
     seeds_distinct = ((words[q / kWave].bits >> (int)(q % kWave)) & 1ull) &&
                      rank_of(q, words, group_off) - rank0 == info.ns - 1;
   }
+  // A lane takes pairs of neighbouring edges, so that its labels leave as
+  // 16-byte stores: item i is edge  e0 + (i / 2) * 2 * kBlock + 2 * lane + i % 2.
+  auto edge_of = [e0](int i) {
+    return e0 + (int64_t)(i >> 1) * (2 * kBlock) + 2 * (int)threadIdx.x + (i & 1);
+  };
 #pragma unroll
   for (int i = 0; i < kRelabelItems; ++i) {
-    const int64_t e = e0 + i * kBlock + threadIdx.x;
+    const int64_t e = edge_of(i);
     if (e >= k.E) break;
     if (!one_batch) info = batch[batch_in_span(k.rows_ptr, span, e)];
     // row key e of batch b sits at flat position
@@ -1146,23 +1151,44 @@ __global__ __launch_bounds__(kBlock) void unique_relabel_kernel(
                                       guess(head_b, e0), guess(last, e1 - 1), head, ends,
                                       wave_max);
 #pragma unroll
-    for (int i = 0; i < kRelabelItems; ++i) col[i] = c_lo + head[i * kBlock + threadIdx.x];
+    for (int i = 0; i < kRelabelItems; ++i) col[i] = c_lo + head[edge_of(i) - e0];
   }
+  struct Pair {
+    int64_t v[2];
+  };
+  const bool wide_stores = (((uintptr_t)out_row | (uintptr_t)out_col) & 15) == 0;
 #pragma unroll
-  for (int i = 0; i < kRelabelItems; ++i) {
-    const int64_t e = e0 + i * kBlock + threadIdx.x;
-    if (e >= k.E) break;
-    if (!one_batch) {
-      const int64_t b = batch_in_span(k.rows_ptr, span, e);
-      info = batch[b];
-      rank0 = unique_ptr[b];
+  for (int i = 0; i < kRelabelItems; i += 2) {
+    Pair row_label{{0, 0}}, col_label{{0, 0}};
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int64_t e = edge_of(i + j);
+      if (e >= k.E) break;
+      if (!one_batch) {
+        const int64_t b = batch_in_span(k.rows_ptr, span, e);
+        info = batch[b];
+        rank0 = unique_ptr[b];
+      }
+      if (out_row) row_label.v[j] = rank_of(info.fb + row_first[i + j], words, group_off) - rank0;
+      // seed c of batch b sits at flat position c + rows_ptr[b]
+      if (out_col)
+        col_label.v[j] =
+            seeds_distinct
+                ? col[i + j] - info.s_lo
+                : rank_of(info.fb + first[col[i + j] + info.r_lo], words, group_off) - rank0;
     }
-    if (out_row) out_row[e] = rank_of(info.fb + row_first[i], words, group_off) - rank0;
-    // seed c of batch b sits at flat position c + rows_ptr[b]
-    if (out_col)
-      out_col[e] = seeds_distinct
-                       ? col[i] - info.s_lo
-                       : rank_of(info.fb + first[col[i] + info.r_lo], words, group_off) - rank0;
+    const int64_t e = edge_of(i);
+    if (e + 1 < k.E && wide_stores) {
+      if (out_row) __builtin_memcpy(__builtin_assume_aligned(out_row + e, 16), &row_label, sizeof(Pair));
+      if (out_col) __builtin_memcpy(__builtin_assume_aligned(out_col + e, 16), &col_label, sizeof(Pair));
+    } else {
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+        if (e + j < k.E) {
+          if (out_row) out_row[e + j] = row_label.v[j];
+          if (out_col) out_col[e + j] = col_label.v[j];
+        }
+    }
   }
 }
 
