@@ -519,6 +519,9 @@ constexpr int kPartItems = 8;
 constexpr int kPartTile = kPartThreads * kPartItems;
 constexpr int kSliceEntries = 32768;  // (row, value) pairs one work-group sums
 constexpr int kSliceItems = 8;
+// The accumulators of a range take 64 KB of LDS, so two work-groups share a
+// compute unit: 1024 threads each keep all its wavefront slots busy.
+constexpr int kAccThreads = 1024;
 
 struct RowRangePlan {
   int64_t ranges = 0, tiles = 0, max_units = 0;
@@ -629,7 +632,7 @@ __global__ __launch_bounds__(kMaxRanges) void rowsum_units_kernel(
   if (r == 0) unit_start[ranges] = total;
 }
 
-__global__ __launch_bounds__(kPartThreads) void rowsum_accumulate_kernel(
+__global__ __launch_bounds__(kAccThreads) void rowsum_accumulate_kernel(
     const uint2* __restrict__ entries, const int64_t* __restrict__ offsets,
     const int64_t* __restrict__ unit_start, int ranges, int64_t tiles,
     float* __restrict__ partial) {
@@ -643,13 +646,13 @@ __global__ __launch_bounds__(kPartThreads) void rowsum_accumulate_kernel(
   const int64_t range_end = offsets[(r + 1) * tiles];
   const int64_t begin = offsets[r * tiles] + (u - unit_start[r]) * kSliceEntries;
   const int64_t end = begin + kSliceEntries < range_end ? begin + kSliceEntries : range_end;
-  for (int j = threadIdx.x; j < kRangeRows; j += kPartThreads) acc[j] = 0.0;
+  for (int j = threadIdx.x; j < kRangeRows; j += kAccThreads) acc[j] = 0.0;
   __syncthreads();
-  for (int64_t base = begin; base < end; base += kPartThreads * kSliceItems) {
+  for (int64_t base = begin; base < end; base += kAccThreads * kSliceItems) {
     uint2 item[kSliceItems];
 #pragma unroll
     for (int i = 0; i < kSliceItems; ++i) {
-      const int64_t p = base + i * kPartThreads + threadIdx.x;
+      const int64_t p = base + i * kAccThreads + threadIdx.x;
       item[i] = p < end ? entries[p] : make_uint2(~0u, 0u);
     }
 #pragma unroll
@@ -659,7 +662,7 @@ __global__ __launch_bounds__(kPartThreads) void rowsum_accumulate_kernel(
   }
   __syncthreads();
   float* mine = partial + u * kRangeRows;
-  for (int j = threadIdx.x; j < kRangeRows; j += kPartThreads) mine[j] = (float)acc[j];
+  for (int j = threadIdx.x; j < kRangeRows; j += kAccThreads) mine[j] = (float)acc[j];
 }
 
 // out[row] += the row's partial sums over all slices of its range.  Ranges
@@ -716,7 +719,7 @@ static int row_range_sum(const RowRangePlan& p, const int64_t* dst_ids,
                 offsets, ranges, p.tiles, unit_start));
   GS_LAUNCH("rowsum_accumulate", s,
             rowsum_accumulate_kernel<<<dim3((unsigned)p.max_units),
-                                       dim3(kPartThreads), 0, s>>>(
+                                       dim3(kAccThreads), 0, s>>>(
                 entries, offsets, unit_start, ranges, p.tiles, partial));
   GS_LAUNCH("rowsum_fold", s,
             rowsum_fold_kernel<<<dim3((unsigned)ceil_div(num_out, kBlock), kFoldSplit),
