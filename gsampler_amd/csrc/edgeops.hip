@@ -517,6 +517,7 @@ constexpr int kMaxRanges = 1024;
 constexpr int kPartThreads = 512;
 constexpr int kPartItems = 8;
 constexpr int kPartTile = kPartThreads * kPartItems;
+constexpr int kPartMaxRounds = 8;
 constexpr int kSliceEntries = 32768;  // (row, value) pairs one work-group sums
 constexpr int kSliceItems = 8;
 // The accumulators of a range take 64 KB of LDS, so two work-groups share a
@@ -525,6 +526,7 @@ constexpr int kAccThreads = 1024;
 
 struct RowRangePlan {
   int64_t ranges = 0, tiles = 0, max_units = 0;
+  int rounds = 1;  // sub-tiles of kPartTile edges one work-group of the partition passes takes
   size_t off_offsets = 0, off_scan = 0, scan_bytes = 0, off_entries = 0,
          off_unit_start = 0, off_partial = 0, total = 0;
 };
@@ -537,7 +539,12 @@ static RowRangePlan row_range_plan(int format, int64_t nnz, int64_t num_out) {
       ceil_div(num_out, kRangeRows) > kMaxRanges)
     return p;
   p.ranges = ceil_div(num_out, kRangeRows);
-  p.tiles = ceil_div(nnz, kPartTile);
+  // The (range, tile) table costs a strided 8-byte access per cell in both
+  // partition passes: once there are work-groups to spare a tile grows to up
+  // to eight sub-tiles, which shrinks the table by as much.
+  int64_t rounds = nnz / ((int64_t)kPartTile * 8192);
+  p.rounds = (int)(rounds < 1 ? 1 : rounds > kPartMaxRounds ? kPartMaxRounds : rounds);
+  p.tiles = ceil_div(nnz, (int64_t)kPartTile * p.rounds);
   p.max_units = nnz / kSliceEntries + p.ranges;
   auto take = [&p](size_t bytes) {
     const size_t at = p.total;
@@ -557,27 +564,30 @@ static RowRangePlan row_range_plan(int format, int64_t nnz, int64_t num_out) {
 // counts[range * tiles + tile] = edges of the tile whose target lies in range
 __global__ __launch_bounds__(kPartThreads) void rowsum_hist_kernel(
     const int64_t* __restrict__ dst_ids, int64_t nnz, int64_t num_out, int ranges,
-    int64_t tiles, int64_t* __restrict__ counts) {
+    int64_t tiles, int rounds, int64_t* __restrict__ counts) {
   __shared__ int hist[kMaxRanges];
   for (int j = threadIdx.x; j < ranges; j += kPartThreads) hist[j] = 0;
   __syncthreads();
-  const int64_t tile0 = (int64_t)blockIdx.x * kPartTile;
-  int64_t dst[kPartItems];
+  for (int r = 0; r < rounds; ++r) {
+    const int64_t tile0 = ((int64_t)blockIdx.x * rounds + r) * kPartTile;
+    if (tile0 >= nnz) break;
+    int64_t dst[kPartItems];
 #pragma unroll
-  for (int i = 0; i < kPartItems; ++i) {
-    const int64_t e = tile0 + i * kPartThreads + threadIdx.x;
-    dst[i] = e < nnz ? dst_ids[e] : -1;
+    for (int i = 0; i < kPartItems; ++i) {
+      const int64_t e = tile0 + i * kPartThreads + threadIdx.x;
+      dst[i] = e < nnz ? dst_ids[e] : -1;
+    }
+#pragma unroll
+    for (int i = 0; i < kPartItems; ++i)
+      if (dst[i] >= 0 && dst[i] < num_out) atomicAdd(&hist[dst[i] >> kRangeShift], 1);
   }
-#pragma unroll
-  for (int i = 0; i < kPartItems; ++i)
-    if (dst[i] >= 0 && dst[i] < num_out) atomicAdd(&hist[dst[i] >> kRangeShift], 1);
   __syncthreads();
   for (int j = threadIdx.x; j < ranges; j += kPartThreads)
     counts[(int64_t)j * tiles + blockIdx.x] = hist[j];
   if (blockIdx.x == 0 && threadIdx.x == 0) counts[(int64_t)ranges * tiles] = 0;
 }
 
-// A tile is kept small (4096 edges) so that several work-groups share a
+// A sub-tile is kept small (4096 edges) so that several work-groups share a
 // compute unit and the loads of one overlap the stores of another; what a tile
 // sends to one range is a contiguous run, filled within a few microseconds, so
 // the 8-byte stores merge into whole lines in L2.  A pair keeps its range above
@@ -586,32 +596,35 @@ __global__ __launch_bounds__(kPartThreads) void rowsum_scatter_kernel(
     const int64_t* __restrict__ dst_ids, const int64_t* __restrict__ src_ids,
     const int64_t* __restrict__ edge_map, int64_t nnz, int64_t num_out, int kind,
     int op, const float* __restrict__ ufeat, const float* __restrict__ efeat,
-    int ranges, int64_t tiles, const int64_t* __restrict__ offsets,
+    int ranges, int64_t tiles, int rounds, const int64_t* __restrict__ offsets,
     uint2* __restrict__ entries) {
   __shared__ unsigned cursor[kMaxRanges];  // next free place of the tile per range
   for (int j = threadIdx.x; j < ranges; j += kPartThreads)
     cursor[j] = (unsigned)offsets[(int64_t)j * tiles + blockIdx.x];
   __syncthreads();
-  const int64_t tile0 = (int64_t)blockIdx.x * kPartTile;
-  int64_t dst[kPartItems];
-  float val[kPartItems];
+  for (int r = 0; r < rounds; ++r) {
+    const int64_t tile0 = ((int64_t)blockIdx.x * rounds + r) * kPartTile;
+    if (tile0 >= nnz) break;
+    int64_t dst[kPartItems];
+    float val[kPartItems];
 #pragma unroll
-  for (int i = 0; i < kPartItems; ++i) {
-    const int64_t e = tile0 + i * kPartThreads + threadIdx.x;
-    dst[i] = -1;
-    val[i] = 0.f;
-    if (e < nnz) {
-      dst[i] = dst_ids[e];
-      const int64_t eid = edge_map ? edge_map[e] : e;
-      val[i] = edge_value<float>(kind, op, ufeat ? ufeat + src_ids[e] : nullptr,
-                                 efeat ? efeat + eid : nullptr);
+    for (int i = 0; i < kPartItems; ++i) {
+      const int64_t e = tile0 + i * kPartThreads + threadIdx.x;
+      dst[i] = -1;
+      val[i] = 0.f;
+      if (e < nnz) {
+        dst[i] = dst_ids[e];
+        const int64_t eid = edge_map ? edge_map[e] : e;
+        val[i] = edge_value<float>(kind, op, ufeat ? ufeat + src_ids[e] : nullptr,
+                                   efeat ? efeat + eid : nullptr);
+      }
     }
-  }
 #pragma unroll
-  for (int i = 0; i < kPartItems; ++i) {
-    if (dst[i] < 0 || dst[i] >= num_out) continue;
-    const unsigned pos = atomicAdd(&cursor[dst[i] >> kRangeShift], 1u);
-    entries[pos] = make_uint2((unsigned)dst[i], __float_as_uint(val[i]));
+    for (int i = 0; i < kPartItems; ++i) {
+      if (dst[i] < 0 || dst[i] >= num_out) continue;
+      const unsigned pos = atomicAdd(&cursor[dst[i] >> kRangeShift], 1u);
+      entries[pos] = make_uint2((unsigned)dst[i], __float_as_uint(val[i]));
+    }
   }
 }
 
@@ -706,14 +719,14 @@ static int row_range_sum(const RowRangePlan& p, const int64_t* dst_ids,
   const dim3 tiles_grid((unsigned)p.tiles);
   GS_LAUNCH("rowsum_hist", s,
             rowsum_hist_kernel<<<tiles_grid, dim3(kPartThreads), 0, s>>>(
-                dst_ids, nnz, num_out, ranges, p.tiles, offsets));
+                dst_ids, nnz, num_out, ranges, p.tiles, p.rounds, offsets));
   int rc = exclusive_scan_i64(offsets, offsets, p.ranges * p.tiles + 1,
                               ws + p.off_scan, p.scan_bytes, s);
   if (rc != GS_OK) return rc;
   GS_LAUNCH("rowsum_scatter", s,
             rowsum_scatter_kernel<<<tiles_grid, dim3(kPartThreads), 0, s>>>(
                 dst_ids, src_ids, edge_map, nnz, num_out, kind, op, ufeat, efeat,
-                ranges, p.tiles, offsets, entries));
+                ranges, p.tiles, p.rounds, offsets, entries));
   GS_LAUNCH("rowsum_units", s,
             rowsum_units_kernel<<<dim3(1), dim3(kMaxRanges), 0, s>>>(
                 offsets, ranges, p.tiles, unit_start));
