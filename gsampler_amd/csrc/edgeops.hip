@@ -358,15 +358,36 @@ __global__ __launch_bounds__(kBlock) void spmm_csc_sum_kernel(
   const int64_t tile_len = (int64_t)kSumTile * rounds;
   const int64_t tile0 = (int64_t)blockIdx.x * tile_len;
   const int64_t tile_end = tile0 + tile_len < nnz ? tile0 + tile_len : nnz;
+  // A lane takes quads of neighbouring edges: item i of a round is edge
+  //   base + (i / 4) * 4 * kBlock + 4 * lane + i % 4,
+  // so that values which come straight from the edge array arrive as 16-byte loads.
+  static_assert(kSumItems % 4 == 0, "a lane takes whole quads");
+  auto edge_of = [](int64_t base, int i) {
+    return base + (int64_t)(i >> 2) * (4 * kBlock) + 4 * (int)threadIdx.x + (i & 3);
+  };
+  const bool plain = edge_map == nullptr && ufeat == nullptr && efeat != nullptr;
   auto load_round = [&](int64_t base, float (&val)[kSumItems]) {
 #pragma unroll
-    for (int i = 0; i < kSumItems; ++i) {
-      const int64_t e = base + i * kBlock + threadIdx.x;
-      val[i] = 0.f;
-      if (e < tile_end) {
-        const int64_t eid = edge_map ? edge_map[e] : e;
-        val[i] = edge_value<float>(kind, op, ufeat ? ufeat + indices[e] : nullptr,
-                                   efeat ? efeat + eid : nullptr);
+    for (int q = 0; q < kSumItems / 4; ++q) {
+      const int64_t e = edge_of(base, 4 * q);
+      if (plain && e + 3 < tile_end) {
+        struct Quad {
+          float v[4];
+        } held;
+        __builtin_memcpy(&held, efeat + e, sizeof(Quad));
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          val[4 * q + j] = edge_value<float>(kind, op, nullptr, &held.v[j]);
+        continue;
+      }
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        val[4 * q + j] = 0.f;
+        if (e + j < tile_end) {
+          const int64_t eid = edge_map ? edge_map[e + j] : e + j;
+          val[4 * q + j] = edge_value<float>(kind, op, ufeat ? ufeat + indices[e + j] : nullptr,
+                                             efeat ? efeat + eid : nullptr);
+        }
       }
     }
   };
@@ -416,7 +437,7 @@ __global__ __launch_bounds__(kBlock) void spmm_csc_sum_kernel(
     }
 #pragma unroll
     for (int i = 0; i < kSumItems; ++i) {
-      const int64_t e = base + i * kBlock + threadIdx.x;
+      const int64_t e = edge_of(base, i);
       const bool active = e < tile_end;
       int64_t seg = 0;
       if (active)
