@@ -411,3 +411,36 @@ def test_count_mirrors_in_pinned_host_memory():
     torch.cuda.synchronize()
     assert host[:B + 1].tolist() == uptr.cpu().tolist() and host[B + 1:].tolist() == [-7, -7]
     assert np.array_equal(uptr.cpu().numpy(), orc.unique_relabel(seeds, rows, sp, rp)[1])
+
+
+def test_outputs_that_are_only_8_byte_aligned(monkeypatch):
+    """The kernels that store 16 bytes per lane fall back to narrower stores when an
+    output array does not allow it: every array the wrappers allocate here starts one
+    element past a 16-byte boundary."""
+    real_empty = torch.empty
+
+    def shifted(*size, **kw):
+        if len(size) == 1 and isinstance(size[0], int) and kw.get("dtype") in (torch.int64, torch.float32):
+            return real_empty(size[0] + 1, **kw)[1:]
+        return real_empty(*size, **kw)
+
+    monkeypatch.setattr(torch, "empty", shifted)
+    rng = np.random.default_rng(31)
+    indptr, indices = random_csc(rng, 3000, 10**5, 60, hub_deg=50000)
+    cols = rng.integers(0, 3000, size=2500)
+    got = capi.col_slice(T(indptr), T(indices), T(cols))
+    assert all(t.data_ptr() % 16 == 8 for t in got)
+    assert_same(got, orc.col_slice(indptr, indices, cols))
+    data = torch.as_tensor(rng.random(indices.size).astype(np.float32), device=DEV)
+    vals = capi.col_slice_values(T(indptr), T(cols), got[0], data)
+    assert vals.data_ptr() % 16 == 4 and torch.equal(vals, data[got[3]])
+    x = rng.integers(0, 50, size=100001)
+    assert np.array_equal(N(capi.exclusive_scan(T(x))), np.cumsum(x) - x)
+    counts = rng.integers(0, 11, size=5000)
+    counts[100] = 6000
+    seeds, rows, sp, rp, edge_col, col_indptr = _grouped_case(rng, counts, 7, 10**5)
+    want = orc.unique_relabel(seeds, rows, sp, rp, edge_col)
+    by_pointer = capi.unique_relabel(T(seeds), T(rows), T(sp), T(rp), col_indptr=T(col_indptr))
+    assert by_pointer[2].data_ptr() % 16 == 8 and by_pointer[3].data_ptr() % 16 == 8
+    assert_same(by_pointer, want)
+    assert_same(capi.unique_relabel(T(seeds), T(rows), T(sp), T(rp), edge_col=T(edge_col)), want)
