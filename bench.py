@@ -429,7 +429,7 @@ def run_ops(args, wl, capi, dev):
     g = torch.Generator(device=dev)
     g.manual_seed(5)
     probs = torch.randn(nnz, generator=g, device=dev).exp_().float()
-    cdf = capi.weight_cdf(indptr, probs)
+    cdf = capi.weight_cdf(indptr, probs, indices, N)
     # frontiers of a step
     s1 = capi.sample_uniform(indptr, indices, seeds, 15, False, 0, args.seed, 0)
     r1 = capi.unique_relabel(seeds, s1[2], ptr, s1[0][ptr], s1[1])
@@ -516,7 +516,8 @@ def run_ops(args, wl, capi, dev):
     coo_col = capi.csc2coo(indptr, nnz)
     measure("edge list -> compressed", "COO2CSCCUDA", lambda: capi.coo_to_csc(indices, coo_col, N),
             8 * nnz * 2 + 8 * nnz * 2 + 8 * N, f"{nnz} edges")
-    measure("weight CDF build", "(none)", lambda: capi.weight_cdf(indptr, probs), 12 * nnz, f"{nnz} edges")
+    measure("weight CDF build", "(none)", lambda: capi.weight_cdf(indptr, probs, indices, N),
+            12 * nnz + 8 * nnz, f"{nnz} edges")
     rows.sort(key=lambda r: -r["device_ms"])
     dom = rows[0]
     return {
@@ -666,7 +667,7 @@ def main():
         probs = torch.randn(indices.numel(), generator=g, device=dev).exp_().float()
         torch.cuda.synchronize()
         t0 = time.time()
-        cdf = capi.weight_cdf(indptr, probs)      # once per (graph, weights)
+        cdf = capi.weight_cdf(indptr, probs, indices, wl["nodes"])   # once per (graph, weights)
         torch.cuda.synchronize()
         t_cdf = time.time() - t0
 

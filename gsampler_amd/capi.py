@@ -85,7 +85,7 @@ SIGNATURES = {
     "gs_minor_slice_count": (_int, [_p, _i64, _p, _i64, _p, _i64, _p, _p, _p, _sz, _p]),
     "gs_minor_slice_fill": (_int, [_p, _i64, _i64, _p, _i64, _p, _p, _p, _p, _p, _sz, _p]),
     "gs_weight_cdf_workspace_bytes": (_sz, [_i64, _i64]),
-    "gs_weight_cdf_build": (_int, [_p, _i64, _p, _i64, _p, _p, _sz, _p]),
+    "gs_weight_cdf_build": (_int, [_p, _i64, _p, _i64, _p, _i64, _p, _p, _sz, _p]),
     "gs_csc_col_sample_weighted_fill": (_int, [_p, _i64, _p, _p, _p, _p, _i64, _i64, _int, _u64,
                                                _u64, _p, _p, _p, _p, _p, _p, _p]),
     "gs_weighted_key_probe": (_int, [_u64, _u64, _u64, _u64, C.c_float, _u64, _p, _p]),
@@ -664,17 +664,25 @@ def weighted_key_probe(seed, call_id, pos, draw, w, r64):
     return out.cpu().tolist()
 
 
-def weight_cdf(indptr, probs):
-    """Persistent integer CDF of the edge weights of a matrix (int64[nnz + 1])."""
+def weight_cdf(indptr, probs, indices=None, num_rows=None):
+    """Persistent packed CDF of the edge weights of a matrix (int64[nnz + 1]).
+    With `indices` the row id of every edge is packed beside its share of the
+    column's mass (ids below `num_rows`, default max id + 1), and the sampler
+    never reads `indices`."""
     indptr = _i64t(indptr, "indptr")
+    if indices is not None:
+        indices = _i64t(indices, "indices")
+        if num_rows is None:
+            num_rows = int(indices.max().item()) + 1 if indices.numel() else 0
     probs = probs.contiguous()
     if probs.dtype != torch.float32:
         raise GsError("probs must be float32")
     nnz, num_cols = probs.numel(), indptr.numel() - 1
     cdf = torch.empty(nnz + 1, dtype=torch.int64, device=indptr.device)
     ws = _workspace(lib().gs_weight_cdf_workspace_bytes(num_cols, nnz), indptr.device)
-    check(lib().gs_weight_cdf_build(_ptr(indptr), num_cols, probs.data_ptr(), nnz,
-                                    cdf.data_ptr(), ws.data_ptr(), ws.numel(), _stream()))
+    check(lib().gs_weight_cdf_build(_ptr(indptr), num_cols, _ptr(indices), num_rows or 0,
+                                    probs.data_ptr(), nnz, cdf.data_ptr(), ws.data_ptr(),
+                                    ws.numel(), _stream()))
     return cdf
 
 

@@ -70,8 +70,11 @@ torch::Tensor Graph::weight_cdf_for(const torch::Tensor& edge_probs, int64_t for
   const int64_t n = m.indptr.numel() - 1, nnz = m.indices.numel();
   torch::Tensor cdf = new_ids(nnz + 1, m.indptr);
   torch::Tensor ws = new_workspace(gs_weight_cdf_workspace_bytes(n, nnz), m.indptr);
-  GS_CALL(gs_weight_cdf_build(cptr(m.indptr), n, probs.data_ptr<float>(), nnz,
-                              mptr(cdf), ws.data_ptr(), ws.numel(), cur_stream()));
+  // the ids on the other axis ride in the CDF's entries
+  const int64_t num_minor = format == kCSC ? num_rows_ : num_cols_;
+  GS_CALL(gs_weight_cdf_build(cptr(m.indptr), n, cptr(m.indices), num_minor,
+                              probs.data_ptr<float>(), nnz, mptr(cdf), ws.data_ptr(),
+                              ws.numel(), cur_stream()));
   cdf_ = cdf;
   cdf_probs_ = edge_probs;
   cdf_version_ = edge_probs._version();

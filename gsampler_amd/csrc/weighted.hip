@@ -244,19 +244,30 @@ __global__ __launch_bounds__(kBlock) void sample_weighted_replace_kernel(
   }
 }
 
-// ------------------------------------------- persistent integer CDF of a matrix
-// cdf[e] = sum of the quantised weights of all edges before e (over the whole
-// matrix, columns back to back), cdf[nnz] = grand total.  Weights of a column
-// are quantised against the column's exact maximum to 31 bits, so the prefix
-// sums are integers and do not depend on the order of additions.  Column c
-// owns [cdf[indptr[c]], cdf[indptr[c + 1]]).  Built once per (matrix, weights),
-// it turns a weighted draw into a search over O(log deg) entries instead of a
-// pass over the column.
+// ------------------------------------------- persistent packed CDF of a matrix
+// One 64-bit entry per edge, built once per (matrix, weights):
+//   cdf[0]      = row_bits, the number of low bits of an entry that hold a row id
+//                 (0: no row ids packed, the sampler reads them from `indices`)
+//   cdf[e + 1]  = share(e) << row_bits | row id of edge e
+// share(e) is the part of its column's mass that lies at or before edge e, in
+// units of 2^-cb (cb = min(62, 64 - row_bits)): the weights of a column are
+// quantised to 31 bits against the column's exact maximum (integers, so their
+// prefix sums G do not depend on the order of additions), and
+//   share(e) = floor(G(e) * 2^cb / T)   for G(e) < T = the column's total,
+//   share(e) = 2^cb - 1                 from the last positive item on
+// (0 everywhere in a column without positive weights).  Item j of a column
+// owns [share(j - 1), share(j)); a draw is a search for the item whose interval
+// holds a point, over 8-byte entries, and the row id of the item arrives with
+// the entry that ends the search: a pick costs the lines of its search and
+// nothing else.  (Row ids and prefix sums in arrays of their own cost a random
+// 128-byte line per pick for the row id and two for the ends of the column's
+// slice of a global prefix sum.)
 // Both passes take tiles of consecutive edges and look the tile's first and
 // last column up once, on the scalar unit; an edge then searches only among
 // the columns of its tile instead of all of them.
 constexpr int kCdfItems = 8;
 constexpr int kCdfTile = kBlock * kCdfItems;
+constexpr int kCdfMaxRowBits = 32;
 
 // Column maxima: the tile's maxima are first taken in LDS (integer atomics on
 // the bit patterns: positive floats order like their bits), then every column
@@ -298,14 +309,16 @@ __global__ __launch_bounds__(kBlock) void cdf_colmax_kernel(
     if (tile_max[j] != 0u) atomicMax(colmax_bits + span.lo + j, tile_max[j]);
 }
 
+// prefix[e] = quantised weight of edge e (the device-wide scan that follows
+// turns it into the sum of all quantised weights before e); prefix[nnz] = 0.
 __global__ __launch_bounds__(kBlock) void cdf_quantise_kernel(
     const int64_t* __restrict__ indptr, int64_t num_cols,
     const float* __restrict__ probs, int64_t nnz,
-    const unsigned int* __restrict__ colmax_bits, int64_t* __restrict__ cdf) {
+    const unsigned int* __restrict__ colmax_bits, int64_t* __restrict__ prefix) {
   const int64_t e0 = (int64_t)blockIdx.x * kCdfTile;
   if (e0 > nnz) return;
-  if (e0 == nnz) {  // cdf[nnz] = 0 closes the exclusive scan
-    if (threadIdx.x == 0) cdf[nnz] = 0;
+  if (e0 == nnz) {  // prefix[nnz] = 0 closes the exclusive scan
+    if (threadIdx.x == 0) prefix[nnz] = 0;
     return;
   }
   const int64_t e_last = e0 + kCdfTile - 1 < nnz ? e0 + kCdfTile - 1 : nnz - 1;
@@ -317,9 +330,9 @@ __global__ __launch_bounds__(kBlock) void cdf_quantise_kernel(
     uint64_t q = 0;
     const float wmax = __uint_as_float(colmax_bits[span.segment_at(indptr, e)]);
     if (wmax > 0.0f) q = quantise(probs[e], det_div(2147483648.0, (double)wmax));
-    cdf[e] = (int64_t)q;
+    prefix[e] = (int64_t)q;
   }
-  if (e_last == nnz - 1 && threadIdx.x == 0) cdf[nnz] = 0;
+  if (e_last == nnz - 1 && threadIdx.x == 0) prefix[nnz] = 0;
 }
 
 __global__ __launch_bounds__(kBlock) void cdf_zero_kernel(unsigned int* p, int64_t n) {
@@ -327,25 +340,69 @@ __global__ __launch_bounds__(kBlock) void cdf_zero_kernel(unsigned int* p, int64
   if (i < n) p[i] = 0u;
 }
 
-// Search state of one draw: the item of the column whose interval holds x is
-// the last j in [0, deg) with a[j] <= x, for a[0] <= x < a[deg] (a = the
-// column's slice of the CDF).  Prefix sums of weights are close to a straight
-// line, so guesses interpolate; every other step (mode 1) or every step after
-// kInterpolations guesses (mode 2) is a plain bisection, which bounds the worst
-// case for any weights; mode 0 only bisects.
+// floor(a * 2^bits / t) for a < t < 2^63, by shift and subtract: exact integer
+// arithmetic, so the CPU check (a 128-bit division) agrees to the bit.
+__device__ __forceinline__ uint64_t scale_share(uint64_t a, uint64_t t, int bits) {
+  uint64_t rem = a, q = 0;
+  for (int i = 0; i < bits; ++i) {
+    rem <<= 1;
+    q <<= 1;
+    if (rem >= t) {
+      rem -= t;
+      q |= 1ull;
+    }
+  }
+  return q;
+}
+
+// prefix[] (global exclusive prefix sums of the quantised weights) -> entries.
+__global__ __launch_bounds__(kBlock) void cdf_pack_kernel(
+    const int64_t* __restrict__ indptr, int64_t num_cols,
+    const int64_t* __restrict__ indices, int64_t nnz,
+    const int64_t* __restrict__ prefix, int row_bits, uint64_t* __restrict__ cdf) {
+  const int64_t e0 = (int64_t)blockIdx.x * kCdfTile;
+  if (blockIdx.x == 0 && threadIdx.x == 0) cdf[0] = (uint64_t)row_bits;
+  if (e0 >= nnz) return;
+  const int64_t e_last = e0 + kCdfTile - 1 < nnz ? e0 + kCdfTile - 1 : nnz - 1;
+  const SegmentSpan span = segment_span(indptr, num_cols, e0, e_last);
+  const int cb = 64 - row_bits < 62 ? 64 - row_bits : 62;
+  const uint64_t full = (1ull << cb) - 1ull;
+  const uint64_t row_mask = row_bits ? (~0ull >> (64 - row_bits)) : 0ull;
+#pragma unroll
+  for (int j = 0; j < kCdfItems; ++j) {
+    const int64_t e = e0 + j * kBlock + threadIdx.x;
+    if (e > e_last) break;
+    const int64_t c = span.segment_at(indptr, e);
+    const uint64_t base = (uint64_t)prefix[indptr[c]];
+    const uint64_t t = (uint64_t)prefix[indptr[c + 1]] - base;
+    const uint64_t a = (uint64_t)prefix[e + 1] - base;
+    const uint64_t share = a == t ? (t ? full : 0ull) : scale_share(a, t, cb);
+    const uint64_t row = row_bits ? ((uint64_t)indices[e] & row_mask) : 0ull;
+    cdf[e + 1] = (share << row_bits) | row;
+  }
+}
+
+// Search state of one draw over a column's entries col[1 .. deg] (col[j] is the
+// entry of item j - 1, so its share is the point where item j starts): the
+// item whose interval holds x is the last j in [0, deg) with start(j) <= x, for
+// start(0) = 0 <= x < start(deg) = the column's mass.  Shares of weights are
+// close to a straight line, so guesses interpolate; every other step (mode 1)
+// or every step after kInterpolations guesses (mode 2) is a plain bisection,
+// which bounds the worst case for any weights; mode 0 only bisects.  The entry
+// that last lowered `hi` stays at hand: when the search ends it is the entry
+// of the item found, row id included.
 constexpr int kInterpolations = 8;
 struct CdfSearch {
-  const int64_t* a;
-  int64_t lo, hi, a_lo, a_hi, x;
+  int64_t lo, hi;
+  uint64_t a_lo, a_hi, x, e_hi;
   int guesses;
   bool flip;
-  __device__ __forceinline__ void begin(const int64_t* col, int64_t deg, int64_t first,
-                                        int64_t last, int64_t point) {
-    a = col;
+  __device__ __forceinline__ void begin(int64_t deg, uint64_t mass, uint64_t point) {
     lo = 0;
     hi = deg;
-    a_lo = first;
-    a_hi = last;
+    a_lo = 0;
+    a_hi = mass;
+    e_hi = 0;  // the column's last entry, which nobody has read yet
     x = point;
     guesses = 0;
     flip = true;
@@ -366,26 +423,30 @@ struct CdfSearch {
     if (mid >= hi) mid = hi - 1;
     return mid;
   }
-  __device__ __forceinline__ void narrow(int64_t mid, int64_t v) {
+  __device__ __forceinline__ void narrow(int64_t mid, uint64_t entry, int row_bits) {
+    const uint64_t v = entry >> row_bits;
     if (v <= x) {
       lo = mid;
       a_lo = v;
     } else {
       hi = mid;
       a_hi = v;
+      e_hi = entry;
     }
   }
 };
 
-__device__ __forceinline__ int64_t cdf_locate(const int64_t* __restrict__ a,
-                                              int64_t deg, int64_t x, int mode) {
-  CdfSearch s;
-  s.begin(a, deg, a[0], a[deg], x);
+// Leaves the item in s.lo and its interval in [s.a_lo, s.a_hi); its entry is in
+// s.e_hi unless the search ended at the column's last item without having
+// looked at it (s.hi == deg).  `mass` is what the column's shares add up to.
+__device__ __forceinline__ void cdf_locate(CdfSearch& s, const uint64_t* __restrict__ col,
+                                           int64_t deg, uint64_t mass, int row_bits,
+                                           uint64_t x, int mode) {
+  s.begin(deg, mass, x);
   while (!s.done()) {
     const int64_t mid = s.probe_at(mode);
-    s.narrow(mid, a[mid]);
+    s.narrow(mid, col[mid], row_bits);
   }
-  return s.lo;
 }
 
 constexpr int kMaxCdfFanout = 64;
@@ -409,102 +470,133 @@ constexpr int kMaxCdfFanout = 64;
 template <int KMAX>
 __global__ __launch_bounds__(kBlock) void sample_weighted_cdf_kernel(
     const int64_t* __restrict__ indptr, int64_t num_cols,
-    const int64_t* __restrict__ indices, const int64_t* __restrict__ cdf,
+    const int64_t* __restrict__ indices, const uint64_t* __restrict__ cdf,
     const int64_t* __restrict__ column_ids, int64_t num_items, int fanout,
     int replace, PhiloxKey key, const int64_t* __restrict__ sub_indptr,
     int64_t* __restrict__ out_coo_col, int64_t* __restrict__ out_indices,
     int64_t* __restrict__ out_select, int mode) {
   const int64_t item = (int64_t)blockIdx.x * kBlock + threadIdx.x;
   if (item >= num_items) return;
+  const int row_bits = (int)cdf[0];  // the same word for every lane: a scalar load
+  const uint64_t row_mask = row_bits ? (~0ull >> (64 - row_bits)) : 0ull;
   const int64_t c = column_ids ? column_ids[item] : item;
   int64_t in_start;
   const int64_t deg = column_degree(indptr, num_cols, c, &in_start);
   if (deg == 0) return;
   const int64_t out_start = sub_indptr[item];
-  const int64_t* a = cdf + in_start;
-  const int64_t base = a[0];
-  const uint64_t total = (uint64_t)(a[deg] - base);
-  auto emit = [&](int64_t slot, int64_t off) {
-    const int64_t p = in_start + off;
-    out_indices[out_start + slot] = indices ? indices[p] : p;
-    out_select[out_start + slot] = p;
-    if (out_coo_col) out_coo_col[out_start + slot] = item;
+  const uint64_t* col = cdf + in_start;  // col[j], 1 <= j <= deg: entry of item j - 1
+  // A column's shares add up to 2^cb - 1, or to 0 when it has no positive weight.
+  // Which of the two is in the column's last entry, one more random line that a
+  // column longer than the fan-out only reads when a search ends at its last item
+  // (in a column without mass the first search does: every share is 0).
+  const int cb = 64 - row_bits < 62 ? 64 - row_bits : 62;
+  const uint64_t full = (1ull << cb) - 1ull;
+  auto row_of = [&](int64_t off, uint64_t entry) -> int64_t {
+    if (row_bits) return (int64_t)(entry & row_mask);
+    return indices ? indices[in_start + off] : in_start + off;
   };
-  // The picks of a column wait in registers (their offsets: `held`) and leave
-  // together at the end: the row ids are then gathered side by side instead of
-  // one per search, and a lane's outputs reach each array back to back, so the
-  // wavefront fills whole lines where pick-by-pick stores leave partial lines
-  // to be evicted and reopened (measured on 3.5 M columns with fanout 5: 33 M
-  // write requests and 1.8 ms pick by pick, 1.2 ms held).  What does not fit
-  // the registers is written pick by pick: columns of 2^32 or more items (no
-  // graph seen so far has one, nothing forbids it) and fanouts above KMAX,
-  // which only occur with replacement.
+  // The picks of a column wait in registers (offset and row id) and leave
+  // together at the end, so that a lane's outputs reach each array back to
+  // back and the wavefront fills whole lines where pick-by-pick stores leave
+  // partial lines to be evicted and reopened (measured on 3.5 M columns with
+  // fanout 5: 33 M write requests and 1.8 ms pick by pick, 1.2 ms held).  What
+  // does not fit the registers is written pick by pick: columns of 2^32 or
+  // more items (no graph seen so far has one, nothing forbids it) and fanouts
+  // above KMAX, which only occur with replacement.
   const bool hold = deg <= 0xFFFFFFFFll && fanout <= KMAX;
-  uint32_t held[KMAX];
+  uint32_t held[KMAX], held_row[KMAX];
 #pragma unroll
-  for (int i = 0; i < KMAX; ++i) held[i] = 0;
+  for (int i = 0; i < KMAX; ++i) held[i] = held_row[i] = 0;
   int taken = 0;
-  auto pick = [&](int64_t off) {
-    if (!hold) emit(taken, off);
+  auto pick = [&](int64_t off, uint64_t entry) {
+    if (!hold) {
+      const int64_t p = in_start + off;
+      out_indices[out_start + taken] = row_of(off, entry);
+      out_select[out_start + taken] = p;
+      if (out_coo_col) out_coo_col[out_start + taken] = item;
+    }
 #pragma unroll
     for (int i = 0; i < KMAX; ++i)
-      if (i == taken) held[i] = (uint32_t)off;
+      if (i == taken) {
+        held[i] = (uint32_t)off;
+        held_row[i] = (uint32_t)(entry & row_mask);
+      }
     ++taken;
   };
+  CdfSearch s;
   if (replace) {
+    bool mass = true;
     for (int j = 0; j < fanout; ++j) {
-      int64_t off = deg - 1;  // no positive weight: the last item
-      if (total > 0)
-        off = cdf_locate(a, deg,
-                         base + (int64_t)philox_bounded(key, (uint64_t)item, (uint64_t)j, total),
-                         mode);
-      pick(off);
+      if (mass) {
+        cdf_locate(s, col, deg, full, row_bits,
+                   philox_bounded(key, (uint64_t)item, (uint64_t)j, full), mode);
+        if (s.hi == deg) {
+          s.e_hi = col[deg];
+          mass = (s.e_hi >> row_bits) != 0;
+        }
+      }
+      if (mass) pick(s.lo, s.e_hi);
+      else pick(deg - 1, s.e_hi);  // no positive weight: the last item
     }
   } else if (deg <= fanout) {  // whole column, original order, zero weights included
-    for (int64_t j = 0; j < deg; ++j) pick(j);
+    for (int64_t j = 0; j < deg; ++j) pick(j, col[j + 1]);
   } else {
-    uint64_t start[KMAX];
-    uint32_t len[KMAX];
+    uint64_t start[KMAX], len[KMAX];
 #pragma unroll
     for (int i = 0; i < KMAX; ++i) {
       start[i] = ~0ull;  // never at or before a point
       len[i] = 0;
     }
     uint64_t removed = 0;
-    while (taken < fanout && removed < total) {
+    while (taken < fanout && removed < full) {
       const uint64_t r =
-          philox_bounded(key, (uint64_t)item, (uint64_t)taken, total - removed);
+          philox_bounded(key, (uint64_t)item, (uint64_t)taken, full - removed);
       uint64_t x = r;
       for (int round = 0; round <= taken; ++round) {
         uint64_t skipped = 0;
 #pragma unroll
-        for (int i = 0; i < KMAX; ++i) skipped += start[i] <= x ? len[i] : 0u;
+        for (int i = 0; i < KMAX; ++i) skipped += start[i] <= x ? len[i] : 0ull;
         if (r + skipped == x) break;
         x = r + skipped;
       }
-      const int64_t off = cdf_locate(a, deg, base + (int64_t)x, mode);
-      const int64_t lo = a[off], hi = a[off + 1];
+      cdf_locate(s, col, deg, full, row_bits, x, mode);
+      if (s.hi == deg) {  // ended at the last item without having read its entry
+        s.e_hi = col[deg];
+        if ((s.e_hi >> row_bits) == 0) break;  // a column without mass
+      }
 #pragma unroll
       for (int i = 0; i < KMAX; ++i)
         if (i == taken) {
-          start[i] = (uint64_t)(lo - base);
-          len[i] = (uint32_t)(hi - lo);
+          start[i] = s.a_lo;
+          len[i] = s.a_hi - s.a_lo;
         }
-      removed += (uint64_t)(hi - lo);
-      pick(off);
+      removed += s.a_hi - s.a_lo;
+      pick(s.lo, s.e_hi);
     }
     // fewer than fanout items have positive weight: zero-weight items in order
-    for (int64_t off = 0; taken < fanout && off < deg; ++off)
-      if (a[off + 1] == a[off]) pick(off);
+    if (taken < fanout) {
+      uint64_t before = 0;
+      for (int64_t off = 0; taken < fanout && off < deg; ++off) {
+        const uint64_t entry = col[off + 1], here = entry >> row_bits;
+        if (here == before) pick(off, entry);
+        before = here;
+      }
+    }
   }
   if (!hold) return;
-  int64_t row[KMAX];
+  if (!row_bits) {
+    int64_t row[KMAX];
 #pragma unroll
-  for (int i = 0; i < KMAX; ++i)
-    if (i < taken) row[i] = indices ? indices[in_start + held[i]] : in_start + held[i];
+    for (int i = 0; i < KMAX; ++i)
+      if (i < taken) row[i] = indices ? indices[in_start + held[i]] : in_start + held[i];
 #pragma unroll
-  for (int i = 0; i < KMAX; ++i)
-    if (i < taken) out_indices[out_start + i] = row[i];
+    for (int i = 0; i < KMAX; ++i)
+      if (i < taken) out_indices[out_start + i] = row[i];
+  } else {
+#pragma unroll
+    for (int i = 0; i < KMAX; ++i)
+      if (i < taken) out_indices[out_start + i] = (int64_t)held_row[i];
+  }
 #pragma unroll
   for (int i = 0; i < KMAX; ++i)
     if (i < taken) out_select[out_start + i] = in_start + held[i];
@@ -530,8 +622,9 @@ static int launch_weighted_cdf(const int64_t* indptr, int64_t num_cols,
   GS_LAUNCH("sample_weighted_cdf", s,
             sample_weighted_cdf_kernel<KMAX><<<dim3((unsigned)ceil_div(num_items, kBlock)),
                                                dim3(kBlock), 0, s>>>(
-                indptr, num_cols, indices, cdf, column_ids, num_items, fanout, replace,
-                key, sub_indptr, out_coo_col, out_indices, out_select, kCdfSearchMode));
+                indptr, num_cols, indices, (const uint64_t*)cdf, column_ids, num_items,
+                fanout, replace, key, sub_indptr, out_coo_col, out_indices, out_select,
+                kCdfSearchMode));
   return GS_OK;
 }
 
@@ -1065,25 +1158,37 @@ int gs_weighted_key_probe(uint64_t seed, uint64_t call_id, uint64_t pos,
 size_t gs_weight_cdf_workspace_bytes(int64_t num_cols, int64_t nnz) {
   if (num_cols < 0 || nnz < 0) return 0;
   return gs::align_up((size_t)(num_cols > 0 ? num_cols : 1) * sizeof(unsigned int), 256) +
+         gs::align_up((size_t)(nnz + 1) * sizeof(int64_t), 256) +
          gs::scan_workspace_bytes(nnz + 1);
 }
 
-int gs_weight_cdf_build(const int64_t* indptr, int64_t num_cols, const float* probs,
-                        int64_t nnz, int64_t* cdf, void* workspace,
-                        size_t workspace_bytes, gs_stream_t stream) {
+int gs_weight_cdf_build(const int64_t* indptr, int64_t num_cols, const int64_t* indices,
+                        int64_t num_rows, const float* probs, int64_t nnz, int64_t* cdf,
+                        void* workspace, size_t workspace_bytes, gs_stream_t stream) {
   using namespace gs;
   GS_REQUIRE(num_cols >= 0 && nnz >= 0, "weight_cdf_build: negative size");
   GS_REQUIRE(cdf && (nnz == 0 || (indptr && probs)), "weight_cdf_build: null pointer");
+  GS_REQUIRE(indices == nullptr || num_rows >= 0, "weight_cdf_build: negative num_rows");
   const size_t need = gs_weight_cdf_workspace_bytes(num_cols, nnz);
   if (workspace == nullptr || workspace_bytes < need) {
     set_error("weight_cdf_build workspace too small: %zu < %zu", workspace_bytes, need);
     return GS_ERR_WORKSPACE;
   }
+  // bits that hold any row id below num_rows; ids too wide to share an entry
+  // with a useful share stay in `indices`
+  int row_bits = 0;
+  if (indices != nullptr) {
+    row_bits = 1;
+    while (row_bits < 63 && (int64_t(1) << row_bits) < num_rows) ++row_bits;
+    if (row_bits > kCdfMaxRowBits) row_bits = 0;
+  }
   hipStream_t s = as_stream(stream);
   unsigned int* colmax = (unsigned int*)workspace;
   const size_t colmax_bytes =
       align_up((size_t)(num_cols > 0 ? num_cols : 1) * sizeof(unsigned int), 256);
-  void* scan_ws = (char*)workspace + colmax_bytes;
+  int64_t* prefix = (int64_t*)((char*)workspace + colmax_bytes);
+  const size_t prefix_bytes = align_up((size_t)(nnz + 1) * sizeof(int64_t), 256);
+  void* scan_ws = (char*)prefix + prefix_bytes;
   if (num_cols > 0)
     GS_LAUNCH("cdf_zero", s,
               cdf_zero_kernel<<<dim3((unsigned)ceil_div(num_cols, kBlock)), dim3(kBlock),
@@ -1094,8 +1199,15 @@ int gs_weight_cdf_build(const int64_t* indptr, int64_t num_cols, const float* pr
                                   s>>>(indptr, num_cols, probs, nnz, colmax));
   GS_LAUNCH("cdf_quantise", s,
             cdf_quantise_kernel<<<dim3((unsigned)ceil_div(nnz + 1, kCdfTile)), dim3(kBlock),
-                                  0, s>>>(indptr, num_cols, probs, nnz, colmax, cdf));
-  return exclusive_scan_i64(cdf, cdf, nnz + 1, scan_ws, workspace_bytes - colmax_bytes, s);
+                                  0, s>>>(indptr, num_cols, probs, nnz, colmax, prefix));
+  const int rc = exclusive_scan_i64(prefix, prefix, nnz + 1, scan_ws,
+                                    workspace_bytes - colmax_bytes - prefix_bytes, s);
+  if (rc != GS_OK) return rc;
+  GS_LAUNCH("cdf_pack", s,
+            cdf_pack_kernel<<<dim3((unsigned)ceil_div(nnz > 0 ? nnz : 1, kCdfTile)),
+                              dim3(kBlock), 0, s>>>(indptr, num_cols, indices, nnz, prefix,
+                                                    row_bits, (uint64_t*)cdf));
+  return GS_OK;
 }
 
 int gs_csc_col_sample_weighted_fill(

@@ -62,12 +62,15 @@ class Block:
         import dgl
         from dgl.heterograph import DGLBlock
         if self.indptr is not None:
-            # python/gs/utils/to_dgl_block.py:5-16: the unit graph straight from the CSC
-            eids = self.edata.get("_ID")
+            # python/gs/utils/to_dgl_block.py:5-16: the unit graph straight from the CSC.
+            # The edge-id argument maps compressed positions to the block's own
+            # edge numbers (a permutation of 0..E-1); an empty tensor numbers the
+            # edges in compressed order, which is the order of row / col / edata.
+            # edata["_ID"] holds positions in the parent matrix and stays edge data.
             idx = dgl.heterograph_index.create_unitgraph_from_csr(
                 2, self.num_src, self.num_dst, self.indptr, self.row,
-                eids if eids is not None else torch.empty(0, dtype=torch.int64), ["coo", "csr", "csc"],
-                transpose=True)
+                torch.empty(0, dtype=torch.int64, device=self.row.device),
+                ["coo", "csr", "csc"], transpose=True)
         else:
             idx = dgl.heterograph_index.create_unitgraph_from_coo(
                 2, self.num_src, self.num_dst, self.row, self.col, formats=["coo", "csr", "csc"])

@@ -218,9 +218,10 @@ int gs_csc_col_sample_uniform_fill_i32(const int64_t* indptr, int64_t num_cols,
  *  with replacement: integer CDF per column in cdf_scratch (uint64 per edge;
  *    column i uses cdf_scratch + cdf_offsets[i], or + indptr[column] when
  *    column_ids == NULL and cdf_offsets == NULL), pick j uses draw j.
- *  cdf != NULL (from gs_weight_cdf_build for the same indptr / probs; probs
- *    may then be NULL, cdf_offsets / cdf_scratch are not used): every draw is
- *    a search in the column's slice of the CDF, O(fanout * log deg) per
+ *  cdf != NULL (from gs_weight_cdf_build for the same indptr / indices / probs;
+ *    probs may then be NULL, cdf_offsets / cdf_scratch are not used, and
+ *    `indices` is only read when the CDF holds no row ids): every draw is
+ *    a search in the column's entries of the CDF, O(fanout * log deg) per
  *    column instead of a pass over its weights.  Without replacement
  *    (fanout <= 64) this is successive weighted sampling: draw j takes a
  *    uniform point of the mass that is left and maps it past the intervals of
@@ -231,13 +232,25 @@ int gs_csc_col_sample_uniform_fill_i32(const int64_t* indptr, int64_t num_cols,
  *    position, draw = output slot.
  * Stands in for CSCColSamplingProbsCUDA (src/cuda/sampling_probs.cu:268-281).
  * ---------------------------------------------------------------------- */
-/* Persistent integer CDF of a matrix's edge weights, the input of the fast
- * weighted sampler below: cdf[nnz + 1], cdf[e] = sum of the quantised weights of
- * the edges before e (all columns back to back; a column's weights are
- * quantised to 31 bits against the column's maximum, w <= 0 counts as 0).
- * Build it once per (matrix, weights); it costs one pass over the edges. */
+/* Persistent packed CDF of a matrix's edge weights, the input of the fast
+ * weighted sampler below: cdf[nnz + 1] 64-bit words.
+ *   cdf[0]     = row_bits: how many low bits of an entry hold a row id (the
+ *                bits that ids below num_rows need; 0 when indices == NULL or
+ *                the ids need more than 32 bits: the sampler then reads the row
+ *                ids from `indices`)
+ *   cdf[e + 1] = share(e) << row_bits | indices[e]
+ * share(e) = the part of the column's mass at or before edge e in units of
+ * 2^-cb, cb = min(62, 64 - row_bits): floor(G(e) * 2^cb / T), with G the prefix
+ * sums inside the column of the weights quantised to 31 bits against the
+ * column's maximum (w <= 0 counts as 0) and T the column's total; 2^cb - 1 from
+ * the last positive edge on; 0 throughout a column without positive weights.
+ * Edge j of a column is drawn with probability (share(j) - share(j - 1)) /
+ * (2^cb - 1).  Build it once per (matrix, weights): four passes over the edges.
+ * No counterpart in the reference, whose sampler reads every weight of a
+ * column on every call (src/cuda/sampling_probs.cu:25-110). */
 size_t gs_weight_cdf_workspace_bytes(int64_t num_cols, int64_t nnz);
 int gs_weight_cdf_build(const int64_t* indptr, int64_t num_cols,
+                        const int64_t* indices, int64_t num_rows,
                         const float* probs, int64_t nnz, int64_t* cdf,
                         void* workspace, size_t workspace_bytes,
                         gs_stream_t stream);

@@ -328,11 +328,16 @@ def weighted_key(seed, call_id, pos, draw, w) -> float:
              C.c_float(w))
 
 
-def weight_cdf(indptr, probs) -> np.ndarray:
+def weight_cdf(indptr, probs, indices=None, num_rows=None) -> np.ndarray:
     indptr = _i64(indptr)
     probs = np.ascontiguousarray(probs, dtype=np.float32)
+    if indices is not None:
+        indices = _i64(indices)
+        if num_rows is None:
+            num_rows = int(indices.max()) + 1 if indices.size else 0
     cdf = np.empty(probs.size + 1, dtype=np.int64)
-    lib().gs_weight_cdf_build_cpu(_p(indptr), C.c_int64(indptr.size - 1), _p(probs),
+    lib().gs_weight_cdf_build_cpu(_p(indptr), C.c_int64(indptr.size - 1), _p(indices),
+                                  C.c_int64(num_rows or 0), _p(probs),
                                   C.c_int64(probs.size), _p(cdf))
     return cdf
 

@@ -982,13 +982,17 @@ void gs_segment_sort_i64_cpu(const int64_t* indptr, int64_t num_segments,
 }  // extern "C"
 
 // -------------------------------------------------------------------------
-// Weighted sampling through a persistent integer CDF (no counterpart in the
-// reference, whose A-Res kernel reads every weight of a column on every call;
-// the distribution is the same: successive weighted sampling without
-// replacement, which is what A-Res produces).
-//  cdf[e] = sum of the quantised weights of all edges before e over the whole
-//  matrix; a column's weights are quantised to 31 bits against the column's
-//  maximum exactly as integer_cdf() does.
+// Weighted sampling through a persistent CDF (no counterpart in the
+// reference, whose A-Res kernel reads every weight of a column on every call,
+// src/cuda/sampling_probs.cu:25-110; the distribution is the same: successive
+// weighted sampling without replacement, which is what A-Res produces).
+//  cdf[0] = row_bits, cdf[e + 1] = share(e) << row_bits | indices[e], where
+//  share(e) = floor(G(e) * 2^cb / T) for G(e) < T and 2^cb - 1 for G(e) = T > 0
+//  (0 when T = 0); G = inclusive prefix sums inside the column of the weights
+//  quantised to 31 bits against the column's maximum exactly as integer_cdf()
+//  does, T = the column's total, cb = min(62, 64 - row_bits); row_bits = the
+//  bits that ids below num_rows need, or 0 (no ids packed) when there are no
+//  indices or they need more than 32 bits.
 //  Without replacement, deg > fanout: draw d = 0, 1, ... takes r uniform in the
 //  mass that is left, walks the intervals already taken in ascending order
 //  (r >= start ? r += len) and picks the item whose interval holds r -- the
@@ -998,25 +1002,44 @@ void gs_segment_sort_i64_cpu(const int64_t* indptr, int64_t num_segments,
 //  total; a column without positive weights gives its last item.
 //  Streams: pos = column position, draw = slot.
 extern "C" void gs_weight_cdf_build_cpu(const int64_t* indptr, int64_t num_cols,
+                                        const int64_t* indices, int64_t num_rows,
                                         const float* probs, int64_t nnz,
                                         int64_t* cdf) {
-  std::vector<uint64_t> q((size_t)nnz, 0);
+  int row_bits = 0;
+  if (indices) {
+    row_bits = 1;
+    while (row_bits < 63 && (int64_t(1) << row_bits) < num_rows) ++row_bits;
+    if (row_bits > 32) row_bits = 0;
+  }
+  const int cb = std::min(62, 64 - row_bits);
+  const uint64_t full = (uint64_t(1) << cb) - 1;
+  uint64_t* out = (uint64_t*)cdf;
+  out[0] = (uint64_t)row_bits;
+  (void)nnz;
 #pragma omp parallel for schedule(dynamic, 256)
   for (int64_t c = 0; c < num_cols; ++c) {
+    const int64_t lo = indptr[c], hi = indptr[c + 1];
     float wmax = 0.0f;
-    for (int64_t e = indptr[c]; e < indptr[c + 1]; ++e)
+    for (int64_t e = lo; e < hi; ++e)
       if (probs[e] > wmax) wmax = probs[e];
-    if (wmax <= 0.0f) continue;
-    const double scale = det_div(2147483648.0, (double)wmax);
-    for (int64_t e = indptr[c]; e < indptr[c + 1]; ++e)
-      q[(size_t)e] = probs[e] > 0.0f ? (uint64_t)((double)probs[e] * scale) : 0;
+    const double scale = wmax > 0.0f ? det_div(2147483648.0, (double)wmax) : 0.0;
+    auto q = [&](int64_t e) -> uint64_t {
+      return wmax > 0.0f && probs[e] > 0.0f ? (uint64_t)((double)probs[e] * scale) : 0;
+    };
+    uint64_t total = 0;
+    for (int64_t e = lo; e < hi; ++e) total += q(e);
+    uint64_t g = 0;
+    for (int64_t e = lo; e < hi; ++e) {
+      g += q(e);
+      uint64_t share = 0;
+      if (total > 0)
+        share = g == total ? full
+                           : (uint64_t)(((unsigned __int128)g << cb) / (unsigned __int128)total);
+      const uint64_t row =
+          row_bits ? ((uint64_t)indices[e] & (~uint64_t(0) >> (64 - row_bits))) : 0;
+      out[e + 1] = (share << row_bits) | row;
+    }
   }
-  int64_t acc = 0;
-  for (int64_t e = 0; e < nnz; ++e) {
-    cdf[e] = acc;
-    acc += (int64_t)q[(size_t)e];
-  }
-  cdf[nnz] = acc;
 }
 
 extern "C" void gs_csc_col_sample_weighted_cdf_fill_cpu(
@@ -1026,23 +1049,31 @@ extern "C" void gs_csc_col_sample_weighted_cdf_fill_cpu(
     const int64_t* sub_indptr, int64_t* out_coo_col, int64_t* out_indices,
     int64_t* out_select) {
   Stream rng(seed, call_id);
+  const uint64_t* packed = (const uint64_t*)cdf;
+  const int row_bits = (int)packed[0];
+  const uint64_t row_mask = row_bits ? (~uint64_t(0) >> (64 - row_bits)) : 0;
 #pragma omp parallel for schedule(dynamic, 64)
   for (int64_t i = 0; i < num_items; ++i) {
     const int64_t c = column_ids ? column_ids[i] : i;
     const int64_t deg = col_degree(indptr, num_cols, c);
     if (deg == 0) continue;
     const int64_t in_start = indptr[c], out_start = sub_indptr[i];
+    const uint64_t* col = packed + 1 + in_start;  // entry of item j at col[j]
+    // start(j): the share at which item j begins, 0 <= j <= deg
+    std::vector<uint64_t> start((size_t)deg + 1, 0);
+    for (int64_t j = 0; j < deg; ++j) start[(size_t)j + 1] = col[j] >> row_bits;
     auto emit = [&](int64_t j, int64_t off) {
-      out_indices[out_start + j] = indices ? indices[in_start + off] : in_start + off;
+      int64_t row = in_start + off;
+      if (row_bits) row = (int64_t)(col[off] & row_mask);
+      else if (indices) row = indices[in_start + off];
+      out_indices[out_start + j] = row;
       out_select[out_start + j] = in_start + off;
       if (out_coo_col) out_coo_col[out_start + j] = i;
     };
-    const int64_t* a = cdf + in_start;
-    const uint64_t total = (uint64_t)(a[deg] - a[0]);
-    // item whose interval [a[j], a[j+1]) holds the absolute point x
-    auto locate = [&](uint64_t rel) {
-      const int64_t x = a[0] + (int64_t)rel;
-      return (int64_t)(std::upper_bound(a, a + deg + 1, x) - a) - 1;
+    const uint64_t total = start[(size_t)deg];
+    // item whose interval [start(j), start(j + 1)) holds the point x
+    auto locate = [&](uint64_t x) {
+      return (int64_t)(std::upper_bound(start.begin(), start.end(), x) - start.begin()) - 1;
     };
     if (replace) {
       for (int64_t j = 0; j < fanout; ++j)
@@ -1065,13 +1096,12 @@ extern "C" void gs_csc_col_sample_weighted_cdf_fill_cpu(
       for (; at < taken_iv.size() && r >= taken_iv[at].first; ++at) r += taken_iv[at].second;
       const int64_t off = locate(r);
       emit(taken, off);
-      const uint64_t len = (uint64_t)(a[off + 1] - a[off]);
-      taken_iv.insert(taken_iv.begin() + (std::ptrdiff_t)at,
-                      {(uint64_t)(a[off] - a[0]), len});
+      const uint64_t len = start[(size_t)off + 1] - start[(size_t)off];
+      taken_iv.insert(taken_iv.begin() + (std::ptrdiff_t)at, {start[(size_t)off], len});
       removed += len;
     }
     for (int64_t off = 0; taken < fanout && off < deg; ++off)
-      if (a[off + 1] == a[off]) emit(taken++, off);
+      if (start[(size_t)off + 1] == start[(size_t)off]) emit(taken++, off);
   }
 }
 

@@ -100,9 +100,10 @@ def test_weighted_step_with_persistent_cdf(graph):
     g = torch.Generator(device=indices.device)
     g.manual_seed(5)
     probs = torch.randn(indices.numel(), generator=g, device=indices.device).exp_().float()
-    cdf = capi.weight_cdf(indptr, probs)
+    nodes = indptr.numel() - 1
+    cdf = capi.weight_cdf(indptr, probs, indices, nodes)
     h_indptr, h_indices, h_probs = indptr.cpu().numpy(), indices.cpu().numpy(), probs.cpu().numpy()
-    h_cdf = orc.weight_cdf(h_indptr, h_probs)
+    h_cdf = orc.weight_cdf(h_indptr, h_probs, h_indices, nodes)
     assert np.array_equal(cdf.cpu().numpy(), h_cdf)
     out = capi.sample_weighted(indptr, indices, probs, seeds, 15, False, 7777, 0, cdf=cdf)
     check_sampled_layer(indptr, indices, seeds, 15, out)
@@ -168,14 +169,20 @@ def test_largest_configuration_weighted_layers():
     g = torch.Generator(device=dev)
     g.manual_seed(5)
     probs = torch.empty(edges, device=dev).normal_(generator=g).exp_()
-    cdf = capi.weight_cdf(indptr, probs)
-    assert bool((cdf[1:] >= cdf[:-1]).all()) and int(cdf[0]) == 0
-    # a column's largest weight quantises to 2^31 (spot check on some columns)
+    cdf = capi.weight_cdf(indptr, probs, indices, nodes)
+    row_bits = int(cdf[0])
+    assert row_bits == (nodes - 1).bit_length()
+    share_bits = min(62, 64 - row_bits)
+    # every entry carries its edge's row id ...
+    assert bool(((cdf[1:] & ((1 << row_bits) - 1)) == indices).all())
+    # ... and inside a column the shares rise to 2^share_bits - 1 (spot check on some columns;
+    # entries are unsigned 64-bit words, so shift as such)
     for c in (0, 1, 77, 1_000_000, nodes - 1):
         lo, hi = int(indptr[c]), int(indptr[c + 1])
         if hi > lo:
-            steps = cdf[lo + 1:hi + 1] - cdf[lo:hi]
-            assert int(steps.max()) == 2 ** 31
+            share = cdf[lo + 1:hi + 1].cpu().numpy().view(np.uint64) >> np.uint64(row_bits)
+            assert int(share[-1]) == (1 << share_bits) - 1
+            assert bool((share[1:] >= share[:-1]).all())
             assert int(torch.argmax(steps)) == int(torch.argmax(probs[lo:hi]))
     seeds, ptr = batched_seeds(nodes, 128, 1024, seed=2, device=dev)
 

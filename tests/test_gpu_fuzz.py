@@ -97,8 +97,9 @@ def test_random_case(seed):
         Kw = min(K, 64)
         same(capi.sample_weighted(g_indptr, g_indices, g_probs, T(ok_seeds), Kw, replace, 7777, call),
              orc.sample_weighted(indptr, indices, probs, ok_seeds, Kw, replace, 7777, call))
-        cdf = capi.weight_cdf(g_indptr, g_probs)
-        h_cdf = orc.weight_cdf(indptr, probs)
+        packed = bool(call % 2)           # row ids inside the CDF's entries, or not
+        cdf = capi.weight_cdf(g_indptr, g_probs, g_indices if packed else None)
+        h_cdf = orc.weight_cdf(indptr, probs, indices if packed else None)
         assert np.array_equal(cdf.cpu().numpy(), h_cdf)
         same(capi.sample_weighted(g_indptr, g_indices, None, T(ok_seeds), Kw, replace, 7777, call,
                                   cdf=cdf),

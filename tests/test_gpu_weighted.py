@@ -86,20 +86,40 @@ def _weighted_case(seed, cols=3000, hub=30000):
     return rng, indptr, indices, probs
 
 
-def test_weight_cdf_is_bit_identical():
+@pytest.mark.parametrize("num_rows", [None, 0, 2**22, 2**27, 2**32, 2**40])
+def test_weight_cdf_is_bit_identical(num_rows):
+    """None: no row ids packed; 0: the bits that the largest id needs; wider id spaces leave
+    fewer bits to the shares; ids beyond 32 bits are not packed."""
     rng, indptr, indices, probs = _weighted_case(1)
-    assert np.array_equal(capi.weight_cdf(T(indptr), F(probs)).cpu().numpy(),
-                          orc.weight_cdf(indptr, probs))
+    if num_rows is None:
+        g, h = capi.weight_cdf(T(indptr), F(probs)), orc.weight_cdf(indptr, probs)
+    else:
+        ids = indices if num_rows == 0 else rng.integers(0, num_rows, size=indices.size)
+        g = capi.weight_cdf(T(indptr), F(probs), T(ids), num_rows or None)
+        h = orc.weight_cdf(indptr, probs, ids, num_rows or None)
+    assert np.array_equal(g.cpu().numpy(), h)
     empty = capi.weight_cdf(T(np.zeros(4)), F(np.zeros(0)))
     assert empty.cpu().tolist() == [0]
 
 
+def test_weight_cdf_of_one_long_column():
+    """A column far longer than a tile: the shares of every tile refer to the same total."""
+    rng = np.random.default_rng(8)
+    deg = np.array([3, 300_000, 0, 5])
+    indptr = np.concatenate([[0], np.cumsum(deg)])
+    probs = rng.lognormal(size=int(deg.sum())).astype(np.float32)
+    ids = rng.integers(0, 2_450_000, size=probs.size)
+    assert np.array_equal(capi.weight_cdf(T(indptr), F(probs), T(ids), 2_450_000).cpu().numpy(),
+                          orc.weight_cdf(indptr, probs, ids, 2_450_000))
+
+
 @pytest.mark.parametrize("fanout", [1, 5, 15, 64])
 @pytest.mark.parametrize("replace", [False, True])
-def test_cdf_column_sampling_parity(fanout, replace):
+@pytest.mark.parametrize("packed_rows", [False, True])
+def test_cdf_column_sampling_parity(fanout, replace, packed_rows):
     rng, indptr, indices, probs = _weighted_case(fanout)
-    cdf = orc.weight_cdf(indptr, probs)
-    g_cdf = capi.weight_cdf(T(indptr), F(probs))
+    cdf = orc.weight_cdf(indptr, probs, indices if packed_rows else None)
+    g_cdf = capi.weight_cdf(T(indptr), F(probs), T(indices) if packed_rows else None)
     cols = np.concatenate([rng.integers(0, 3000, size=2000), [7, 11, 7, 20, 21, 22, 23, 20]])
     same(capi.sample_weighted(T(indptr), T(indices), None, T(cols), fanout, replace, call_id=4,
                               cdf=g_cdf),
@@ -111,8 +131,8 @@ def test_cdf_column_sampling_parity(fanout, replace):
 def test_cdf_sampling_with_replacement_beyond_the_register_budget():
     # fanouts above 64 are written pick by pick instead of being held in registers
     rng, indptr, indices, probs = _weighted_case(3)
-    cdf = orc.weight_cdf(indptr, probs)
-    g_cdf = capi.weight_cdf(T(indptr), F(probs))
+    cdf = orc.weight_cdf(indptr, probs, indices)
+    g_cdf = capi.weight_cdf(T(indptr), F(probs), T(indices))
     cols = rng.integers(0, 3000, size=500)
     for fanout in (65, 100):
         same(capi.sample_weighted(T(indptr), T(indices), None, T(cols), fanout, True, call_id=2,

@@ -370,7 +370,7 @@ def test_compiled_weighted_graphsage_matches_the_cdf_oracle():
     c = gs.jit.compile(func=weighted_graphsage_sampler, args=(m, seeds, [10, 5]))
     gs.manual_seed(21)
     _, blocks = c(m, seeds, [10, 5])
-    cdf = orc.weight_cdf(indptr, w)
+    cdf = orc.weight_cdf(indptr, w, indices, m.num_rows())   # the operator class packs the row ids
     s = seeds.cpu().numpy()
     for layer, (K, blk) in enumerate(zip([10, 5], blocks)):
         sub_indptr, col, rows, sel = orc.sample_weighted(indptr, indices, None, s, K, False,

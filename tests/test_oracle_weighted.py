@@ -151,40 +151,90 @@ def test_uniform_list_sampling():
 
 
 # ------------------------------------------------ sampling through a persistent CDF
-def test_weight_cdf_is_a_quantised_prefix_sum():
+def _unpack_cdf(cdf, indptr):
+    """(row_bits, share bits, per-edge share, per-edge row) of a packed CDF."""
+    words = cdf.view(np.uint64)
+    row_bits = int(words[0])
+    cb = min(62, 64 - row_bits)
+    entries = words[1:]
+    share = entries >> np.uint64(row_bits)
+    rows = entries & np.uint64((1 << row_bits) - 1) if row_bits else None
+    return row_bits, cb, share, rows
+
+
+@pytest.mark.parametrize("num_rows", [None, 1000, 2**22, 2**32, 2**33])
+def test_weight_cdf_holds_shares_of_the_column_mass_and_row_ids(num_rows):
+    """Entry e = share(e) << row_bits | row: shares are non-decreasing inside a column, end at
+    2^cb - 1, and an edge's piece is its weight's part of the column's weight (to the 31-bit
+    quantisation of the weights and one unit of the share); rows come back unchanged."""
     rng = np.random.default_rng(3)
-    deg = np.array([5, 0, 300, 1, 4, 0, 7])
+    deg = np.array([5, 0, 300, 1, 4, 0, 7, 70000])
     indptr = np.concatenate([[0], np.cumsum(deg)])
-    w = rng.lognormal(size=int(deg.sum())).astype(np.float32)
+    nnz = int(deg.sum())
+    w = rng.lognormal(size=nnz).astype(np.float32)
     w[indptr[4]:indptr[5]] = [0.0, -1.0, 0.0, 0.0]      # a column without positive weights
     w[indptr[6] + 2] = 0.0
-    cdf = orc.weight_cdf(indptr, w)
-    q = np.diff(cdf)
-    assert cdf[0] == 0 and np.all(q >= 0)
+    w[indptr[6] + 5:indptr[6] + 7] = 0.0                 # zeros after the last positive edge
+    indices = None
+    if num_rows is not None:
+        indices = rng.integers(0, num_rows, size=nnz)
+        indices[0] = num_rows - 1
+    cdf = orc.weight_cdf(indptr, w, indices, num_rows)
+    row_bits, cb, share, rows = _unpack_cdf(cdf, indptr)
+    if num_rows is None or num_rows > 2**32:
+        assert row_bits == 0 and cb == 62
+    else:
+        assert row_bits == max(1, int(num_rows - 1).bit_length()) and cb == min(62, 64 - row_bits)
+        assert np.array_equal(rows.astype(np.int64), indices)
+    full = (1 << cb) - 1
     for c in range(deg.size):
         lo, hi = indptr[c], indptr[c + 1]
-        wc, qc = w[lo:hi].astype(np.float64), q[lo:hi]
         if hi == lo:
             continue
+        wc = np.where(w[lo:hi] > 0, w[lo:hi], 0).astype(np.float64)
+        sc = [int(v) for v in share[lo:hi]]
         if wc.max() <= 0:
-            assert np.all(qc == 0)
+            assert all(v == 0 for v in sc)
             continue
-        # the maximum maps to 2^31 (give or take a unit), everything else in proportion
-        assert abs(int(qc[wc.argmax()]) - 2**31) <= 1
-        assert np.all(qc[wc <= 0] == 0)
-        want = np.where(wc > 0, wc / wc.max() * 2**31, 0)
-        assert np.all(np.abs(qc - want) <= 1.0 + want * 2**-40)
+        assert sc[-1] == full and all(b >= a for a, b in zip(sc, sc[1:]))
+        piece = np.diff(np.array([0] + sc, dtype=object)).astype(np.float64)
+        assert np.all(piece[wc == 0] == 0)
+        # from the last positive edge on the share is 2^cb - 1
+        last_pos = int(np.nonzero(wc)[0][-1])
+        assert all(v == full for v in sc[last_pos:])
+        want = wc / wc.sum() * 2.0**cb
+        # weights are cut to multiples of max / 2^31 first: relative error below deg / 2^31 on
+        # the total and one such unit on the edge itself
+        unit = wc.max() / 2**31 / wc.sum() * 2.0**cb
+        assert np.all(np.abs(piece - want) <= 2.0 + unit + want * (hi - lo) * 2.0**-30)
+
+
+def test_weight_cdf_shares_are_exact_integer_quotients():
+    """share = floor(G * 2^cb / T) recomputed with Python integers from the quantised weights
+    (weights that are powers of two times the maximum quantise exactly)."""
+    w = np.array([1, 0.5, 0.25, 1, 0.125, 0.5, 0, 1], dtype=np.float32)
+    indptr = np.array([0, 8])
+    for num_rows, idx in ((None, None), (5, np.array([4, 3, 2, 1, 0, 1, 2, 3]))):
+        cdf = orc.weight_cdf(indptr, w, idx, num_rows)
+        row_bits, cb, share, rows = _unpack_cdf(cdf, indptr)
+        q = [int(x * 2**31) for x in w.tolist()]
+        total, g, want = sum(q), 0, []
+        for x in q:
+            g += x
+            want.append((1 << cb) - 1 if g == total else (g << cb) // total)
+        assert [int(v) for v in share] == want
 
 
 @pytest.mark.parametrize("w,k", [([3, 1, 2, 2, 1], 2), ([5, 1, 0, 1, 2, 1], 3), ([1, 1, 1, 1], 3),
                                  ([1000, 1, 2, 3, 2], 3)])   # mass on one item: the sequential phase
-def test_cdf_column_sampling_is_successive_weighted_sampling(w, k):
+@pytest.mark.parametrize("packed_rows", [False, True])
+def test_cdf_column_sampling_is_successive_weighted_sampling(w, k, packed_rows):
     """Ordered k-tuples drawn through the CDF against the exact law of successive
     weighted sampling without replacement (zero weights have probability 0)."""
     n = 40000
     indptr = np.array([0, len(w)]); indices = np.arange(len(w)) + 100
     probs = np.array(w, dtype=np.float32)
-    cdf = orc.weight_cdf(indptr, probs)
+    cdf = orc.weight_cdf(indptr, probs, indices if packed_rows else None)
     s, c, rows, sel = orc.sample_weighted(indptr, indices, None, np.zeros(n, dtype=np.int64), k,
                                           cdf=cdf)
     assert np.array_equal(rows, indices[sel]) and np.array_equal(s, np.arange(n + 1) * k)
@@ -201,9 +251,9 @@ def test_cdf_column_sampling_is_successive_weighted_sampling(w, k):
 def test_cdf_sampling_structural_rules():
     indptr = np.array([0, 6, 6, 9, 14]); indices = np.arange(14)
     probs = np.array([0, 5, 0, 0, 0, 0,   1, 1, 1,   0, 0, 0, 0, 0], dtype=np.float32)
-    cdf = orc.weight_cdf(indptr, probs)
-    s, c, rows, sel = orc.sample_weighted(indptr, indices, None, None, 3, cdf=cdf)
-    assert s.tolist() == [0, 3, 3, 6, 9]
+    cdf = orc.weight_cdf(indptr, probs, indices + 7)
+    s, c, rows, sel = orc.sample_weighted(indptr, indices + 7, None, None, 3, cdf=cdf)
+    assert s.tolist() == [0, 3, 3, 6, 9] and np.array_equal(rows, sel + 7)
     assert sel[:3].tolist() == [1, 0, 2]          # the only positive item, then zeros in order
     assert sel[3:6].tolist() == [6, 7, 8]         # deg <= K: the column in order
     assert sel[6:].tolist() == [9, 10, 11]        # no positive weight at all
