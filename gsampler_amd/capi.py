@@ -84,6 +84,11 @@ SIGNATURES = {
     "gs_minor_slice_workspace_bytes": (_sz, [_i64, _i64]),
     "gs_minor_slice_count": (_int, [_p, _i64, _p, _i64, _p, _i64, _p, _p, _p, _sz, _p]),
     "gs_minor_slice_fill": (_int, [_p, _i64, _i64, _p, _i64, _p, _p, _p, _p, _p, _sz, _p]),
+    "gs_col_row_slice_count": (_int, [_p, _p, _p, _p, _i64, _p, _i64, _p, _i64, _p, _p, _p, _sz,
+                                      _p]),
+    "gs_col_row_slice_fill": (_int, [_p, _p, _p, _i64, _p, _i64, _i64, _p, _p, _p, _p, _sz, _p]),
+    "gs_sliced_e_square_sum_workspace_bytes": (_sz, [_i64, _i64]),
+    "gs_sliced_e_square_sum": (_int, [_p, _p, _p, _i64, _p, _i64, _p, _p, _p, _i64, _p, _sz, _p]),
     "gs_weight_cdf_workspace_bytes": (_sz, [_i64, _i64]),
     "gs_weight_cdf_build": (_int, [_p, _i64, _p, _i64, _p, _i64, _p, _p, _sz, _p]),
     "gs_csc_col_sample_weighted_fill": (_int, [_p, _i64, _p, _p, _p, _p, _i64, _i64, _int, _u64,
@@ -653,6 +658,62 @@ def minor_slice(ids, picked, indptr=None, edge_major=None, with_major=True):
                                 _ptr(out_major), _ptr(out_minor), _ptr(out_select),
                                 ws.data_ptr(), ws.numel(), _stream()))
     return out_indptr, out_major, out_minor, out_select
+
+
+def col_row_slice(indptr, indices, cols, rows, key_offset=None, with_major=True):
+    """A[rows, cols] read from the parent matrix, the column slice never written.
+    -> (out_indptr[len(cols) + 1], out_major | None = position of the edge's column in
+    `cols`, out_minor = position of its row in `rows`, out_select = its position in the
+    parent's `indices`).  `key_offset[len(cols)]` is added to the row ids of a column's
+    edges before they are looked up among `rows`."""
+    indptr, indices = _i64t(indptr, "indptr"), _i64t(indices, "indices")
+    cols, rows = _i64t(cols, "cols"), _i64t(rows, "rows")
+    if key_offset is not None:
+        key_offset = _i64t(key_offset, "key_offset")
+    dev = indptr.device
+    ncol, nrow = cols.numel(), rows.numel()
+    sub_indptr = col_count(indptr, cols, -1, False)
+    nnz = int(sub_indptr[-1].item())
+    l = lib()
+    ws = _workspace(l.gs_minor_slice_workspace_bytes(nnz, nrow), dev)
+    out_indptr = torch.empty(ncol + 1, dtype=torch.int64, device=dev)
+    total = torch.empty(1, dtype=torch.int64, device=dev)
+    check(l.gs_col_row_slice_count(_ptr(indptr), _ptr(indices), _ptr(cols), _ptr(key_offset),
+                                   ncol, sub_indptr.data_ptr(), nnz, _ptr(rows), nrow,
+                                   out_indptr.data_ptr(), total.data_ptr(), ws.data_ptr(),
+                                   ws.numel(), _stream()))
+    kept = int(total.item())
+    out_minor = torch.empty(kept, dtype=torch.int64, device=dev)
+    out_select = torch.empty(kept, dtype=torch.int64, device=dev)
+    out_major = torch.empty(kept, dtype=torch.int64, device=dev) if with_major else None
+    check(l.gs_col_row_slice_fill(_ptr(indptr), _ptr(indices), _ptr(cols), ncol,
+                                  sub_indptr.data_ptr(), nnz, nrow, _ptr(out_major),
+                                  _ptr(out_minor), _ptr(out_select), ws.data_ptr(), ws.numel(),
+                                  _stream()))
+    return out_indptr, out_major, out_minor, out_select
+
+
+def sliced_e_square_sum(indptr, indices, cols, efeat, num_out, use_workspace=True,
+                        edge_map=None):
+    """out[row] = sum of efeat^2 over the edges of A[:, cols], read from the parent
+    (edge p's value is efeat[edge_map[p]] when an edge map is given)."""
+    indptr, indices = _i64t(indptr, "indptr"), _i64t(indices, "indices")
+    cols = _i64t(cols, "cols")
+    efeat = efeat.contiguous()
+    if efeat.dtype != torch.float32:
+        raise GsError("efeat must be float32")
+    dev = indptr.device
+    sub_indptr = col_count(indptr, cols, -1, False)
+    nnz = int(sub_indptr[-1].item())
+    out = torch.zeros(num_out, dtype=torch.float32, device=dev)
+    l = lib()
+    ws = _workspace(l.gs_sliced_e_square_sum_workspace_bytes(nnz, num_out) if use_workspace
+                    else 0, dev)
+    check(l.gs_sliced_e_square_sum(_ptr(indptr), _ptr(indices), _ptr(cols), cols.numel(),
+                                   sub_indptr.data_ptr(), nnz, _ptr(edge_map), efeat.data_ptr(),
+                                   out.data_ptr(), num_out, ws.data_ptr() if ws.numel() else None,
+                                   ws.numel(), _stream()))
+    return out
 
 
 # --------------------------------------------------------- weighted sampling

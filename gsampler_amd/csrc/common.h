@@ -223,6 +223,114 @@ __device__ __forceinline__ SegmentSpan segment_span(const int64_t* __restrict__ 
   return s;
 }
 
+// A column slice that is not written out.  Edge v of the slice A[:, cols] is
+// edge  indptr[cols[c]] + (v - sub_indptr[c])  of the parent, where c is the
+// position with sub_indptr[c] <= v < sub_indptr[c + 1] (sub_indptr = the
+// exclusive scan of the picked columns' degrees).  key_offset[c], when given, is
+// added to the ids of column c's edges (ids of a super-batch are told apart as
+// id + batch * stride).  A view with sub_indptr == nullptr is no view: edge v is
+// edge v of the arrays at hand.
+struct SliceView {
+  const int64_t* sub_indptr;
+  const int64_t* cols;
+  const int64_t* indptr;
+  const int64_t* key_offset;
+  int64_t n;
+  __device__ __forceinline__ bool on() const { return sub_indptr != nullptr; }
+
+  // A run of consecutive slice edges [first, last], the same for every lane of
+  // the wavefront: the columns it touches are looked up once, on the scalar
+  // unit.  Columns worth slicing are long, so a run nearly always lies inside
+  // one column or across the border of two neighbours: an edge's place in the
+  // parent is then its number plus one of two distances, chosen by which side
+  // of the border it is on, and nothing is searched or loaded per edge.  A run
+  // over up to 64 columns keeps one column per lane (where it starts inside the
+  // run, its distance, its offset) and an edge finds its column by a search over
+  // the lanes with shuffles; only beyond that does an edge search the pointer.
+  struct Run {
+    SegmentSpan span;
+    int64_t first;            // first edge of the run
+    int64_t split;            // first edge of the second column (none: beyond every edge)
+    int64_t shift[2], offset[2];
+    int count;                // columns held by the lanes (0: none are)
+    int32_t lane_start;       // this lane's column: first edge, relative to `first`, not below 0
+    int64_t lane_shift, lane_offset;
+    // At most two neighbouring columns.  Callers branch on this once per run,
+    // around their whole loop over the run's edges, not per edge: a branch
+    // between a load and its use keeps the loads of an unrolled loop from being
+    // in flight together.
+    __device__ __forceinline__ bool near() const { return span.hi - span.lo <= 1; }
+    // for near() runs
+    __device__ __forceinline__ int64_t place(int64_t v) const {
+      return v + (v < split ? shift[0] : shift[1]);
+    }
+    __device__ __forceinline__ int64_t id_offset(int64_t v) const {
+      return v < split ? offset[0] : offset[1];
+    }
+    __device__ __forceinline__ int64_t column(int64_t v) const {
+      return v < split ? span.lo : span.hi;
+    }
+  };
+  // Every lane of the wavefront must call this, with the same arguments.
+  __device__ __forceinline__ Run run(int64_t first, int64_t last) const {
+    Run r;
+    // the column of the first edge by a search; the last edge is nearly always
+    // in the same column, which one more look at the pointer tells
+    const int64_t first_u = wave_uniform_first(first), last_u = wave_uniform_first(last);
+    r.first = first_u;
+    r.span.lo = segment_of(sub_indptr, n, first_u);
+    r.span.hi = r.span.lo;
+    if (sub_indptr[r.span.lo + 1] <= last_u)
+      r.span.hi = r.span.lo + segment_of(sub_indptr + r.span.lo, n - r.span.lo, last_u);
+    r.split = INT64_MAX;
+    r.shift[0] = r.shift[1] = r.offset[0] = r.offset[1] = 0;
+    r.count = 0;
+    r.lane_start = 0;
+    r.lane_shift = r.lane_offset = 0;
+    if (r.near()) {
+      r.shift[0] = indptr[cols[r.span.lo]] - sub_indptr[r.span.lo];
+      if (key_offset) r.offset[0] = key_offset[r.span.lo];
+      if (r.span.hi != r.span.lo) {
+        r.split = sub_indptr[r.span.hi];
+        r.shift[1] = indptr[cols[r.span.hi]] - r.split;
+        if (key_offset) r.offset[1] = key_offset[r.span.hi];
+      }
+    } else if (r.span.hi - r.span.lo < kWave) {
+      r.count = (int)(r.span.hi - r.span.lo) + 1;
+      const int64_t c = r.span.lo + (lane_id() < r.count ? lane_id() : r.count - 1);
+      const int64_t start = sub_indptr[c];
+      r.lane_start = start > first_u ? (int32_t)(start - first_u) : 0;
+      r.lane_shift = indptr[cols[c]] - start;
+      if (key_offset) r.lane_offset = key_offset[c];
+    }
+    return r;
+  }
+  // Position in the parent of edge v of a run that is not near(): *col = its
+  // column position, *offset = what to add to its id.  Every lane of the
+  // wavefront must call this together (it shuffles), with v inside the run.
+  __device__ __forceinline__ int64_t position(const Run& r, int64_t v, int64_t* col,
+                                              int64_t* offset) const {
+    if (r.count > 0) {  // the same in every lane
+      const int32_t x = (int32_t)(v - r.first);
+      int i = 0;  // the last column that starts at or before the edge
+#pragma unroll
+      for (int step = kWave / 2; step >= 1; step >>= 1) {
+        const int probe = i + step;
+        const int32_t s = __shfl(r.lane_start, probe < r.count ? probe : r.count - 1, kWave);
+        i = (probe < r.count && s <= x) ? probe : i;
+      }
+      *col = r.span.lo + i;
+      *offset = key_offset ? (int64_t)__shfl((long long)r.lane_offset, i, kWave) : 0;
+      return v + (int64_t)__shfl((long long)r.lane_shift, i, kWave);
+    }
+    const int64_t c = r.span.lo + segment_of(sub_indptr + r.span.lo, r.span.hi - r.span.lo + 1, v);
+    *col = c;
+    *offset = key_offset ? key_offset[c] : 0;
+    return indptr[cols[c]] + (v - sub_indptr[c]);
+  }
+};
+inline SliceView no_view() { return SliceView{nullptr, nullptr, nullptr, nullptr, 0}; }
+
 __device__ __forceinline__ int64_t column_degree(const int64_t* indptr,
                                                  int64_t num_cols, int64_t c,
                                                  int64_t* in_start) {

@@ -468,7 +468,7 @@ __global__ __launch_bounds__(kBlock) void spmm_coo_sum_kernel(
     const int64_t* __restrict__ row, const int64_t* __restrict__ col,
     const int64_t* __restrict__ edge_map, int64_t nnz, int kind, int op,
     const float* __restrict__ ufeat, const float* __restrict__ efeat, float* out,
-    int u_target, int64_t copy_stride) {
+    int u_target, int64_t copy_stride, SliceView view) {
   __shared__ long long keys[kCooSlots];
   __shared__ float vals[kCooSlots];
   for (int j = threadIdx.x; j < kCooSlots; j += kBlock) {
@@ -483,6 +483,12 @@ __global__ __launch_bounds__(kBlock) void spmm_coo_sum_kernel(
   const int64_t* dst_ids = u_target == 0 ? col : row;
   const int64_t* src_ids = u_target == 0 ? row : col;
   // all loads of the tile first, so that they are in flight together
+  // (with a view: the edges of a column slice that was never written, dst_ids
+  // and efeat being the parent's arrays)
+  SliceView::Run vrun{};
+  vrun.split = INT64_MAX;  // no view: every edge at distance 0
+  if (view.on() && tile0 < nnz)
+    vrun = view.run(tile0, (tile0 + kSumTile < nnz ? tile0 + kSumTile : nnz) - 1);
   int64_t dst[kSumItems];
   float val[kSumItems];
 #pragma unroll
@@ -490,11 +496,25 @@ __global__ __launch_bounds__(kBlock) void spmm_coo_sum_kernel(
     const int64_t e = tile0 + i * kBlock + threadIdx.x;
     dst[i] = -1;
     val[i] = 0.f;
-    if (e < nnz) {
-      dst[i] = dst_ids[e];
-      const int64_t eid = edge_map ? edge_map[e] : e;
-      val[i] = edge_value<float>(kind, op, ufeat ? ufeat + src_ids[e] : nullptr,
+    if (e < nnz && vrun.near()) {
+      const int64_t p = vrun.place(e);
+      dst[i] = dst_ids[p];
+      const int64_t eid = edge_map ? edge_map[p] : p;
+      val[i] = edge_value<float>(kind, op, ufeat ? ufeat + src_ids[p] : nullptr,
                                  efeat ? efeat + eid : nullptr);
+    }
+  }
+  if (!vrun.near()) {
+#pragma unroll
+    for (int i = 0; i < kSumItems; ++i) {
+      const int64_t e = tile0 + i * kBlock + threadIdx.x;
+      int64_t col, offset;  // (looked up by all lanes together, a lane past the end included)
+      const int64_t p = view.position(vrun, e < nnz ? e : nnz - 1, &col, &offset);
+      if (e < nnz) {
+        dst[i] = dst_ids[p];
+        val[i] = edge_value<float>(kind, op, ufeat ? ufeat + src_ids[p] : nullptr,
+                                   efeat ? efeat + (edge_map ? edge_map[p] : p) : nullptr);
+      }
     }
   }
 #pragma unroll
@@ -583,20 +603,44 @@ static RowRangePlan row_range_plan(int format, int64_t nnz, int64_t num_out) {
 }
 
 // counts[range * tiles + tile] = edges of the tile whose target lies in range
+// With a view the edges are those of a column slice that was never written:
+// dst_ids and efeat are then the parent's arrays (see SliceView).
+__device__ __forceinline__ SliceView::Run view_run(const SliceView& view, int64_t tile0,
+                                                   int64_t tile, int64_t nnz) {
+  if (!view.on()) {  // every edge at distance 0
+    SliceView::Run r{};
+    r.split = INT64_MAX;
+    return r;
+  }
+  const int64_t stop = tile0 + tile < nnz ? tile0 + tile : nnz;
+  return view.run(tile0, stop - 1);
+}
+
 __global__ __launch_bounds__(kPartThreads) void rowsum_hist_kernel(
     const int64_t* __restrict__ dst_ids, int64_t nnz, int64_t num_out, int ranges,
-    int64_t tiles, int rounds, int64_t* __restrict__ counts) {
+    int64_t tiles, int rounds, int64_t* __restrict__ counts, SliceView view) {
   __shared__ int hist[kMaxRanges];
   for (int j = threadIdx.x; j < ranges; j += kPartThreads) hist[j] = 0;
   __syncthreads();
   for (int r = 0; r < rounds; ++r) {
     const int64_t tile0 = ((int64_t)blockIdx.x * rounds + r) * kPartTile;
     if (tile0 >= nnz) break;
+    const SliceView::Run vrun = view_run(view, tile0, kPartTile, nnz);
     int64_t dst[kPartItems];
+    if (vrun.near()) {  // (no view: distance 0)
 #pragma unroll
-    for (int i = 0; i < kPartItems; ++i) {
-      const int64_t e = tile0 + i * kPartThreads + threadIdx.x;
-      dst[i] = e < nnz ? dst_ids[e] : -1;
+      for (int i = 0; i < kPartItems; ++i) {
+        const int64_t e = tile0 + i * kPartThreads + threadIdx.x;
+        dst[i] = e < nnz ? dst_ids[vrun.place(e)] : -1;
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < kPartItems; ++i) {
+        const int64_t e = tile0 + i * kPartThreads + threadIdx.x;
+        int64_t col, offset;  // (looked up by all lanes together, a lane past the end included)
+        const int64_t p = view.position(vrun, e < nnz ? e : nnz - 1, &col, &offset);
+        dst[i] = e < nnz ? dst_ids[p] : -1;
+      }
     }
 #pragma unroll
     for (int i = 0; i < kPartItems; ++i)
@@ -618,7 +662,7 @@ __global__ __launch_bounds__(kPartThreads) void rowsum_scatter_kernel(
     const int64_t* __restrict__ edge_map, int64_t nnz, int64_t num_out, int kind,
     int op, const float* __restrict__ ufeat, const float* __restrict__ efeat,
     int ranges, int64_t tiles, int rounds, const int64_t* __restrict__ offsets,
-    uint2* __restrict__ entries) {
+    uint2* __restrict__ entries, SliceView view) {
   __shared__ unsigned cursor[kMaxRanges];  // next free place of the tile per range
   for (int j = threadIdx.x; j < ranges; j += kPartThreads)
     cursor[j] = (unsigned)offsets[(int64_t)j * tiles + blockIdx.x];
@@ -626,18 +670,35 @@ __global__ __launch_bounds__(kPartThreads) void rowsum_scatter_kernel(
   for (int r = 0; r < rounds; ++r) {
     const int64_t tile0 = ((int64_t)blockIdx.x * rounds + r) * kPartTile;
     if (tile0 >= nnz) break;
+    const SliceView::Run vrun = view_run(view, tile0, kPartTile, nnz);
     int64_t dst[kPartItems];
     float val[kPartItems];
+    const bool shifted = vrun.near();  // the same in every lane (no view: distance 0)
 #pragma unroll
     for (int i = 0; i < kPartItems; ++i) {
       const int64_t e = tile0 + i * kPartThreads + threadIdx.x;
       dst[i] = -1;
       val[i] = 0.f;
-      if (e < nnz) {
-        dst[i] = dst_ids[e];
-        const int64_t eid = edge_map ? edge_map[e] : e;
-        val[i] = edge_value<float>(kind, op, ufeat ? ufeat + src_ids[e] : nullptr,
+      if (e < nnz && shifted) {
+        const int64_t p = vrun.place(e);
+        dst[i] = dst_ids[p];
+        const int64_t eid = edge_map ? edge_map[p] : p;
+        val[i] = edge_value<float>(kind, op, ufeat ? ufeat + src_ids[p] : nullptr,
                                    efeat ? efeat + eid : nullptr);
+      }
+    }
+    if (!shifted) {
+#pragma unroll
+      for (int i = 0; i < kPartItems; ++i) {
+        const int64_t e = tile0 + i * kPartThreads + threadIdx.x;
+        int64_t col, offset;  // (looked up by all lanes together, a lane past the end included)
+        const int64_t p = view.position(vrun, e < nnz ? e : nnz - 1, &col, &offset);
+        if (e < nnz) {
+          dst[i] = dst_ids[p];
+          const int64_t eid = edge_map ? edge_map[p] : p;
+          val[i] = edge_value<float>(kind, op, ufeat ? ufeat + src_ids[p] : nullptr,
+                                     efeat ? efeat + eid : nullptr);
+        }
       }
     }
 #pragma unroll
@@ -730,7 +791,7 @@ static int row_range_sum(const RowRangePlan& p, const int64_t* dst_ids,
                          const int64_t* src_ids, const int64_t* edge_map,
                          int64_t nnz, int64_t num_out, int kind, int op,
                          const float* ufeat, const float* efeat, float* out,
-                         void* workspace, hipStream_t s) {
+                         void* workspace, hipStream_t s, SliceView view = no_view()) {
   char* ws = (char*)workspace;
   int64_t* offsets = (int64_t*)(ws + p.off_offsets);
   uint2* entries = (uint2*)(ws + p.off_entries);
@@ -740,14 +801,14 @@ static int row_range_sum(const RowRangePlan& p, const int64_t* dst_ids,
   const dim3 tiles_grid((unsigned)p.tiles);
   GS_LAUNCH("rowsum_hist", s,
             rowsum_hist_kernel<<<tiles_grid, dim3(kPartThreads), 0, s>>>(
-                dst_ids, nnz, num_out, ranges, p.tiles, p.rounds, offsets));
+                dst_ids, nnz, num_out, ranges, p.tiles, p.rounds, offsets, view));
   int rc = exclusive_scan_i64(offsets, offsets, p.ranges * p.tiles + 1,
                               ws + p.off_scan, p.scan_bytes, s);
   if (rc != GS_OK) return rc;
   GS_LAUNCH("rowsum_scatter", s,
             rowsum_scatter_kernel<<<tiles_grid, dim3(kPartThreads), 0, s>>>(
                 dst_ids, src_ids, edge_map, nnz, num_out, kind, op, ufeat, efeat,
-                ranges, p.tiles, p.rounds, offsets, entries));
+                ranges, p.tiles, p.rounds, offsets, entries, view));
   GS_LAUNCH("rowsum_units", s,
             rowsum_units_kernel<<<dim3(1), dim3(kMaxRanges), 0, s>>>(
                 offsets, ranges, p.tiles, unit_start));
@@ -802,7 +863,7 @@ static int spmm_launch(int format, const int64_t* a, const int64_t* b,
         GS_LAUNCH("spmm_coo_sum", s,
                   spmm_coo_sum_kernel<<<grid, dim3(kBlock), 0, s>>>(
                       a, b, edge_map, nnz, kind, op, ufeat, efeat, copies,
-                      u_target, num_out));
+                      u_target, num_out, no_view()));
         GS_LAUNCH("spmm_fold", s,
                   spmm_fold_kernel<<<dim3((unsigned)ceil_div(num_out, kBlock)),
                                      dim3(kBlock), 0, s>>>(copies, num_out, out));
@@ -811,7 +872,7 @@ static int spmm_launch(int format, const int64_t* a, const int64_t* b,
       GS_LAUNCH("spmm_coo_sum", s,
                 spmm_coo_sum_kernel<<<grid, dim3(kBlock), 0, s>>>(
                     a, b, edge_map, nnz, kind, op, ufeat, efeat, out, u_target,
-                    (int64_t)0));
+                    (int64_t)0, no_view()));
     } else {
       // four tiles per work-group once there are work-groups to spare
       const int rounds = nnz >= ((int64_t)kSumTile * kCscRounds) * 8192 ? kCscRounds : 1;
@@ -983,6 +1044,39 @@ int gs_e_square_sum(int format, const int64_t* a, const int64_t* b,
                      kReduceSum, nullptr, efeat, out, nullptr, nullptr, u_target,
                      0, feat_len, feat_len, nullptr, nullptr, num_out, workspace,
                      workspace_bytes, as_stream(stream));
+}
+
+size_t gs_sliced_e_square_sum_workspace_bytes(int64_t slice_nnz, int64_t num_out) {
+  if (slice_nnz < 0 || num_out < 0) return 0;
+  return gs::row_range_plan(GS_FMT_COO, slice_nnz, num_out).total;
+}
+
+int gs_sliced_e_square_sum(const int64_t* indptr, const int64_t* indices, const int64_t* cols,
+                           int64_t num_cols_picked, const int64_t* sub_indptr,
+                           int64_t slice_nnz, const int64_t* edge_map, const float* efeat,
+                           float* out,
+                           int64_t num_out, void* workspace, size_t workspace_bytes,
+                           gs_stream_t stream) {
+  using namespace gs;
+  GS_REQUIRE(num_cols_picked >= 0 && slice_nnz >= 0 && num_out >= 0,
+             "sliced_e_square_sum: negative size");
+  if (slice_nnz == 0) return GS_OK;
+  GS_REQUIRE(indptr && indices && cols && sub_indptr && efeat && out,
+             "sliced_e_square_sum: null pointer");
+  hipStream_t s = as_stream(stream);
+  const SliceView view{sub_indptr, cols, indptr, nullptr, num_cols_picked};
+  const RowRangePlan plan = row_range_plan(GS_FMT_COO, slice_nnz, num_out);
+  if (plan.total > 0 && workspace != nullptr && workspace_bytes >= plan.total)
+    return row_range_sum(plan, indices, nullptr, edge_map, slice_nnz, num_out, 1, kOpCopyRhs,
+                         nullptr, efeat, out, workspace, s, view);
+  // short slices: combined per tile in LDS, one atomic per (tile, row present);
+  // ids outside [0, num_out) cannot occur for a slice of a checked matrix
+  GS_LAUNCH("spmm_coo_sum", s,
+            spmm_coo_sum_kernel<<<dim3((unsigned)ceil_div(slice_nnz, (int64_t)kSumTile)),
+                                  dim3(kBlock), 0, s>>>(indices, indices, edge_map, slice_nnz, 1,
+                                                        kOpCopyRhs, nullptr, efeat, out, 2,
+                                                        (int64_t)0, view));
+  return GS_OK;
 }
 
 int gs_e_div_u_sum(int format, const int64_t* a, const int64_t* b,

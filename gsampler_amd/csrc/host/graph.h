@@ -165,6 +165,13 @@ class Graph : public torch::CustomClassHolder {
   GraphAndIndex FusedSlicingSampling(int64_t axis, torch::Tensor seeds,
                                      int64_t fanout, bool replace,
                                      int64_t on_format, int64_t output_format);
+  // Not in the reference: operators that read the column slice A[:, cols]
+  // straight from this matrix instead of from a written slice (fused_slices.cc).
+  // out[row] += sum of efeat^2 over the edges of A[:, cols];
+  void SlicedESquareSum(torch::Tensor cols, torch::Tensor efeat, torch::Tensor out);
+  // A[rows, cols], the edge index addressing this matrix's edges.
+  GraphAndIndex ColRowSlicing(torch::Tensor cols, torch::Tensor rows, int64_t on_format,
+                              int64_t output_format);
   GraphAndIndex Compact(int64_t axis);
   torch::Tensor RandomWalk(torch::Tensor seeds, int64_t walk_length);
   torch::Tensor Node2Vec(torch::Tensor seeds, int64_t walk_length, double p,
@@ -273,6 +280,17 @@ class Graph : public torch::CustomClassHolder {
                                  c10::optional<torch::Tensor>* e_ids);
 
   const Compressed& compressed(int64_t format);
+  // Offsets and size of the column slice A[:, cols], kept for the next operator
+  // that is handed the same tensor of columns.
+  struct SliceOffsets {
+    torch::Tensor cols, sub_indptr;
+    int64_t version = -1, indptr_version = -1, nnz = 0;
+    MajorResult written;  // the slice itself, when an operator had to write it
+  };
+  std::unique_ptr<SliceOffsets> slice_offsets_;
+  const SliceOffsets& slice_offsets_for(const torch::Tensor& cols);
+  static bool read_in_place(int64_t slice_nnz, int64_t num_cols_picked);
+  const MajorResult& written_slice(const torch::Tensor& cols);
   // CDF of edge_probs in the edge order of `format` (cached per weights tensor).
   torch::Tensor weight_cdf_for(const torch::Tensor& edge_probs, int64_t format);
   void check_reduce_operands(const std::string& op, const torch::Tensor& ufeat,

@@ -79,6 +79,8 @@ TORCH_LIBRARY(gs_classes, m) {
       .def("_CAPI_FusedUOPV", &Graph::FusedUOPV)
       .def("_CAPI_FusedESquareSum", &Graph::FusedESquareSum)
       .def("_CAPI_FusedEDivUSum", &Graph::FusedEDivUSum)
+      .def("_CAPI_SlicedESquareSum", &Graph::SlicedESquareSum)
+      .def("_CAPI_ColRowSlicing", &Graph::ColRowSlicing)
       .def("_CAPI_SortCSCIndices", &Graph::SortCSCIndices)
       .def("_CAPI_BatchColSlicing", &Graph::BatchColSlicing)
       .def("_CAPI_BatchRowSlicing", &Graph::BatchRowSlicing)

@@ -122,44 +122,4 @@ GraphAndIndex Graph::Compact(int64_t axis) {
   return {g, kept};
 }
 
-// Per batch b: the columns col[col_bptr[b] : col_bptr[b+1]] restricted to the
-// rows row[row_bptr[b] : row_bptr[b+1]]; row ids become positions in `row`.
-// The returned edge index addresses the parent's edges.
-GraphAndIndex Graph::BatchColRowSlcing(torch::Tensor col, torch::Tensor col_bptr,
-                                       torch::Tensor row, torch::Tensor row_bptr) {
-  col = ids(col, "col");
-  row = ids(row, "row");
-  col_bptr = ids(col_bptr, "col_bptr");
-  row_bptr = ids(row_bptr, "row_bptr");
-  TORCH_CHECK(col_bptr.numel() == row_bptr.numel() && col_bptr.numel() >= 2,
-              "BatchColRowSlcing: column and row batch pointers must have the same length");
-  BatchOffsets::check(col_bptr, col.numel(), "BatchColRowSlicing");
-  BatchOffsets::check(row_bptr, row.numel(), "BatchColRowSlicing");
-  const Compressed& m = compressed(kCSC);
-  const int64_t stride = num_rows_;
-  // batched column slice with rows encoded as id + batch * num_rows ...
-  MajorResult sliced = major_slice(m, col, false, col_bptr, stride);
-  // ... tested against the picked rows encoded the same way
-  torch::Tensor row_batch = new_ids(row.numel(), row);
-  GS_CALL(gs_csc2coo(cptr(row_bptr), row_bptr.numel() - 1, row.numel(),
-                     mptr(row_batch), cur_stream()));
-  torch::Tensor picked = row + row_batch * stride;
-  Compressed tmp{sliced.indptr, sliced.minor_ids, c10::nullopt};
-  MajorResult kept = minor_slice(tmp, picked, false);
-  auto g = c10::make_intrusive<Graph>(row.numel(), col.numel());
-  auto csc = std::make_shared<Compressed>();
-  csc->indptr = kept.indptr;
-  csc->indices = kept.minor_ids;
-  g->csc_ = csc;
-  g->num_edges_ = kept.select.numel();
-  g->col_bptr_ = col_bptr;
-  g->row_bptr_ = row_bptr;
-  g->orig_col_ids_ = col;
-  g->orig_row_ids_ = row;
-  g->edge_bptr_ = kept.indptr.index_select(0, col_bptr);
-  BatchOffsets::trust(g->edge_bptr_);
-  torch::Tensor select = sliced.select.index_select(0, kept.select);
-  return {g, edge_index(m.e_ids, select)};
-}
-
 }  // namespace gs

@@ -345,7 +345,7 @@ __global__ __launch_bounds__(kThreads) void member_flag_kernel(
     const uint64_t* __restrict__ global_table, uint32_t cap,
     const int64_t* __restrict__ picked, const int* __restrict__ wide_flag,
     uint64_t* __restrict__ flags, int64_t* __restrict__ chunk_count,
-    uint32_t* __restrict__ staged, const uint32_t* __restrict__ filter) {
+    uint32_t* __restrict__ staged, const uint32_t* __restrict__ filter, SliceView view) {
   __shared__ __align__(16) uint32_t lds_keys[kInLds ? kMemberLdsSlots : 1];
   __shared__ uint32_t lds_values[kInLds ? kMemberLdsSlots : 1];
   __shared__ uint32_t lds_fill[kInLds ? kMemberBuckets : 1];
@@ -375,18 +375,51 @@ __global__ __launch_bounds__(kThreads) void member_flag_kernel(
   // (loads and stores count down one in-order counter) a wait for everything.
   const int64_t num_runs = ceil_div_dev(num_chunks, kMemberChunksPerWave);
   for (int64_t run = (int64_t)blockIdx.x * (kThreads / kWave) + threadIdx.x / kWave;
-       run < num_runs; run += (int64_t)gridDim.x * (kThreads / kWave))
+       run < num_runs; run += (int64_t)gridDim.x * (kThreads / kWave)) {
+  // With a view the edges are those of a column slice that was never written:
+  // the run's columns are looked up once, on the scalar unit, and an edge's id
+  // is read from the parent's array.
+  SliceView::Run vrun{};
+  vrun.split = INT64_MAX;  // no view: every edge at distance 0, offset 0
+  bool scattered = false;  // the same in every lane
+  if (view.on()) {
+    const int64_t e_first = run * kMemberChunksPerWave * kBlock;
+    const int64_t e_stop = e_first + kMemberChunksPerWave * kBlock;
+    vrun = view.run(e_first, (e_stop < nnz ? e_stop : nnz) - 1);
+    scattered = !vrun.near();
+  }
+  // id of edge e, or of the last edge for a lane past the end: on a scattered
+  // run the look-up shuffles, so all lanes go through it together
+  auto id_of = [&](int64_t e) -> uint64_t {
+    if (e >= nnz) e = nnz - 1;
+    if (!scattered) return (uint64_t)(ids[vrun.place(e)] + vrun.id_offset(e));
+    int64_t c, offset;
+    const int64_t p = view.position(vrun, e, &c, &offset);
+    return (uint64_t)(ids[p] + offset);
+  };
   for (int part = 0; part < kMemberChunksPerWave / kMemberAhead; ++part) {
     const int64_t chunk0 = run * kMemberChunksPerWave + part * kMemberAhead;
     if (chunk0 >= num_chunks) break;
     uint32_t keys[kMemberAhead][kMemberWords];
+    if (!scattered) {
 #pragma unroll
-    for (int c = 0; c < kMemberAhead; ++c)
+      for (int c = 0; c < kMemberAhead; ++c)
 #pragma unroll
-      for (int j = 0; j < kMemberWords; ++j) {
-        const int64_t e = (chunk0 + c) * kBlock + j * kWave + lane;
-        keys[c][j] = e < nnz ? member_key((uint64_t)ids[e]) : kNoKey;
-      }
+        for (int j = 0; j < kMemberWords; ++j) {
+          const int64_t e = (chunk0 + c) * kBlock + j * kWave + lane;
+          keys[c][j] =
+              e < nnz ? member_key((uint64_t)(ids[vrun.place(e)] + vrun.id_offset(e))) : kNoKey;
+        }
+    } else {
+#pragma unroll
+      for (int c = 0; c < kMemberAhead; ++c)
+#pragma unroll
+        for (int j = 0; j < kMemberWords; ++j) {
+          const int64_t e = (chunk0 + c) * kBlock + j * kWave + lane;
+          const uint64_t id = id_of(e);
+          keys[c][j] = e < nnz ? member_key(id) : kNoKey;
+        }
+    }
     if (filtered) {
 #pragma unroll
       for (int c = 0; c < kMemberAhead; ++c)
@@ -426,7 +459,8 @@ __global__ __launch_bounds__(kThreads) void member_flag_kernel(
 #pragma unroll
         for (int j = 0; j < kMemberWords; ++j) {
           const int64_t e = chunk * kBlock + j * kWave + lane;
-          slot[j] = e < nnz ? table.find_confirmed((uint64_t)ids[e], picked) : cap;
+          const uint64_t id = id_of(e);
+          slot[j] = e < nnz ? table.find_confirmed(id, picked) : cap;
         }
       }
 #pragma unroll
@@ -452,6 +486,7 @@ __global__ __launch_bounds__(kThreads) void member_flag_kernel(
         if (chunk == num_chunks - 1) chunk_count[num_chunks] = 0;
       }
     }
+  }
   }
 }
 
@@ -495,7 +530,7 @@ __global__ __launch_bounds__(kBlock) void member_fill_kernel(
     const uint32_t* __restrict__ staged, const int64_t* __restrict__ indptr,
     int64_t num_major, const int64_t* __restrict__ edge_major,
     int64_t* __restrict__ out_major, int64_t* __restrict__ out_minor,
-    int64_t* __restrict__ out_select) {
+    int64_t* __restrict__ out_select, SliceView view) {
   const int64_t num_chunks = ceil_div_dev(nnz, kBlock);
   const int64_t wave = (int64_t)blockIdx.x * (kBlock / kWave) + threadIdx.x / kWave;
   const int lane = lane_id();
@@ -514,7 +549,13 @@ __global__ __launch_bounds__(kBlock) void member_fill_kernel(
       (first_chunk + kMemberChunksPerWave) * kBlock < nnz ? (first_chunk + kMemberChunksPerWave) * kBlock
                                                           : nnz;
   SegmentSpan span{0, 0};
-  if (out_major && !kEdgeMajor) span = segment_span(indptr, num_major, e_first, e_end - 1);
+  SliceView::Run vrun{};
+  if (view.on()) {  // indptr is the view's column pointer: one look-up serves both
+    vrun = view.run(e_first, e_end - 1);
+    span = vrun.span;
+  } else if (out_major && !kEdgeMajor) {
+    span = segment_span(indptr, num_major, e_first, e_end - 1);
+  }
 #pragma unroll
   for (int part = 0; part < kMemberChunksPerWave / kMemberAhead; ++part) {
     const int c0 = part * kMemberAhead;
@@ -548,11 +589,29 @@ __global__ __launch_bounds__(kBlock) void member_fill_kernel(
         const uint64_t word =
             __shfl((unsigned long long)lane_word, (c0 + c) * kMemberWords + j, kWave);
         const int64_t e = (first_chunk + c0 + c) * kBlock + j * kWave + lane;
+        // with a view: the edge's place in the parent and its column in the slice
+        // (on a scattered run the look-up shuffles: all lanes take it, kept or not)
+        int64_t parent_pos = 0, slice_col = 0;
+        if (view.on()) {
+          const int64_t ec = e < nnz ? e : nnz - 1;
+          if (vrun.near()) {
+            parent_pos = vrun.place(ec);
+            slice_col = vrun.column(ec);
+          } else {
+            int64_t offset;
+            parent_pos = view.position(vrun, ec, &slice_col, &offset);
+          }
+        }
         if ((word >> lane) & 1ull) {
           const int64_t pos = out0 + before + __popcll(word & ((1ull << lane) - 1));
           out_minor[pos] = (int64_t)minor[c][j];
-          out_select[pos] = e;
-          if (out_major) out_major[pos] = kEdgeMajor ? major[c][j] : span.segment_at(indptr, e);
+          if (view.on()) {
+            out_select[pos] = parent_pos;
+            if (out_major) out_major[pos] = slice_col;
+          } else {
+            out_select[pos] = e;
+            if (out_major) out_major[pos] = kEdgeMajor ? major[c][j] : span.segment_at(indptr, e);
+          }
         }
         before += __popcll(word);
       }
@@ -569,11 +628,12 @@ size_t gs_minor_slice_workspace_bytes(int64_t nnz, int64_t num_picked) {
   return gs::carve_member(nullptr, nnz, num_picked).total;
 }
 
-int gs_minor_slice_count(const int64_t* ids, int64_t nnz, const int64_t* picked,
-                         int64_t num_picked, const int64_t* indptr,
-                         int64_t num_major, int64_t* out_indptr,
-                         int64_t* out_total, void* workspace,
-                         size_t workspace_bytes, gs_stream_t stream) {
+static int minor_slice_count_impl(const int64_t* ids, int64_t nnz, const int64_t* picked,
+                                  int64_t num_picked, const int64_t* indptr,
+                                  int64_t num_major, int64_t* out_indptr,
+                                  int64_t* out_total, void* workspace,
+                                  size_t workspace_bytes, gs_stream_t stream,
+                                  gs::SliceView view) {
   using namespace gs;
   GS_REQUIRE(nnz >= 0 && num_picked >= 0 && num_major >= 0,
              "minor_slice_count: negative size");
@@ -620,7 +680,7 @@ int gs_minor_slice_count(const int64_t* ids, int64_t nnz, const int64_t* picked,
   GS_LAUNCH("member_flag", s,                                                                 \
             (member_flag_kernel<LDS, THREADS>)<<<grid, dim3(THREADS), 0, s>>>(                \
                 ids, nnz, w.table, cap, picked, w.wide, w.flags, w.chunk_off, w.staged,       \
-                filter))
+                filter, view))
     if (in_lds && small) GS_MEMBER_FLAG(true, kBlock);
     else if (in_lds) GS_MEMBER_FLAG(true, kMemberThreads);
     else if (small) GS_MEMBER_FLAG(false, kBlock);
@@ -639,12 +699,12 @@ int gs_minor_slice_count(const int64_t* ids, int64_t nnz, const int64_t* picked,
   return GS_OK;
 }
 
-int gs_minor_slice_fill(const int64_t* ids, int64_t nnz, int64_t num_picked,
-                        const int64_t* indptr, int64_t num_major,
-                        const int64_t* edge_major, int64_t* out_major,
-                        int64_t* out_minor, int64_t* out_select,
-                        void* workspace, size_t workspace_bytes,
-                        gs_stream_t stream) {
+static int minor_slice_fill_impl(const int64_t* ids, int64_t nnz, int64_t num_picked,
+                                 const int64_t* indptr, int64_t num_major,
+                                 const int64_t* edge_major, int64_t* out_major,
+                                 int64_t* out_minor, int64_t* out_select,
+                                 void* workspace, size_t workspace_bytes,
+                                 gs_stream_t stream, gs::SliceView view) {
   using namespace gs;
   GS_REQUIRE(nnz >= 0 && num_picked >= 0 && num_major >= 0,
              "minor_slice_fill: negative size");
@@ -663,13 +723,73 @@ int gs_minor_slice_fill(const int64_t* ids, int64_t nnz, int64_t num_picked,
     GS_LAUNCH("member_fill", s,
               member_fill_kernel<true><<<grid, dim3(kBlock), 0, s>>>(
                   nnz, w.flags, w.chunk_off, w.staged, indptr, num_major, edge_major,
-                  out_major, out_minor, out_select));
+                  out_major, out_minor, out_select, view));
   else
     GS_LAUNCH("member_fill", s,
               member_fill_kernel<false><<<grid, dim3(kBlock), 0, s>>>(
                   nnz, w.flags, w.chunk_off, w.staged, indptr, num_major, edge_major,
-                  out_major, out_minor, out_select));
+                  out_major, out_minor, out_select, view));
   return GS_OK;
+}
+
+int gs_minor_slice_count(const int64_t* ids, int64_t nnz, const int64_t* picked,
+                         int64_t num_picked, const int64_t* indptr,
+                         int64_t num_major, int64_t* out_indptr,
+                         int64_t* out_total, void* workspace,
+                         size_t workspace_bytes, gs_stream_t stream) {
+  return minor_slice_count_impl(ids, nnz, picked, num_picked, indptr, num_major, out_indptr,
+                                out_total, workspace, workspace_bytes, stream, gs::no_view());
+}
+
+int gs_minor_slice_fill(const int64_t* ids, int64_t nnz, int64_t num_picked,
+                        const int64_t* indptr, int64_t num_major,
+                        const int64_t* edge_major, int64_t* out_major,
+                        int64_t* out_minor, int64_t* out_select,
+                        void* workspace, size_t workspace_bytes,
+                        gs_stream_t stream) {
+  return minor_slice_fill_impl(ids, nnz, num_picked, indptr, num_major, edge_major, out_major,
+                               out_minor, out_select, workspace, workspace_bytes, stream,
+                               gs::no_view());
+}
+
+static int check_slice_view(const int64_t* indptr, const int64_t* indices, const int64_t* cols,
+                            int64_t num_cols_picked, const int64_t* sub_indptr,
+                            int64_t slice_nnz, const char* who) {
+  using namespace gs;
+  GS_REQUIRE(num_cols_picked >= 0 && slice_nnz >= 0, "%s: negative size", who);
+  GS_REQUIRE(sub_indptr, "%s: null sub_indptr", who);
+  GS_REQUIRE(slice_nnz == 0 || (indptr && indices && cols && num_cols_picked > 0),
+             "%s: null pointer", who);
+  return GS_OK;
+}
+
+int gs_col_row_slice_count(const int64_t* indptr, const int64_t* indices, const int64_t* cols,
+                           const int64_t* key_offset, int64_t num_cols_picked,
+                           const int64_t* sub_indptr, int64_t slice_nnz,
+                           const int64_t* rows, int64_t num_rows_picked,
+                           int64_t* out_indptr, int64_t* out_total, void* workspace,
+                           size_t workspace_bytes, gs_stream_t stream) {
+  int rc = check_slice_view(indptr, indices, cols, num_cols_picked, sub_indptr, slice_nnz,
+                            "col_row_slice_count");
+  if (rc != GS_OK) return rc;
+  const gs::SliceView view{sub_indptr, cols, indptr, key_offset, num_cols_picked};
+  return minor_slice_count_impl(indices, slice_nnz, rows, num_rows_picked, sub_indptr,
+                                num_cols_picked, out_indptr, out_total, workspace,
+                                workspace_bytes, stream, view);
+}
+
+int gs_col_row_slice_fill(const int64_t* indptr, const int64_t* indices, const int64_t* cols,
+                          int64_t num_cols_picked, const int64_t* sub_indptr,
+                          int64_t slice_nnz, int64_t num_rows_picked, int64_t* out_major,
+                          int64_t* out_minor, int64_t* out_select, void* workspace,
+                          size_t workspace_bytes, gs_stream_t stream) {
+  int rc = check_slice_view(indptr, indices, cols, num_cols_picked, sub_indptr, slice_nnz,
+                            "col_row_slice_fill");
+  if (rc != GS_OK) return rc;
+  const gs::SliceView view{sub_indptr, cols, indptr, nullptr, num_cols_picked};
+  return minor_slice_fill_impl(indices, slice_nnz, num_rows_picked, sub_indptr,
+                               num_cols_picked, nullptr, out_major, out_minor, out_select,
+                               workspace, workspace_bytes, stream, view);
 }
 
 }  // extern "C"

@@ -128,6 +128,7 @@ class compile:  # noqa: N801 -- the reference's public name
         gm = passes.fuse_slicing_and_weighted_sampling(gm)
         gm = passes.fuse_square_and_sum(gm)
         gm = passes.fuse_div_and_sum(gm)
+        gm = passes.read_column_slice_in_place(gm)
         gm = passes.merge_u_mul_v(gm)
         gm = passes.batch_fuse_slicing_and_sampling(gm)
         gm = passes.batch_fuse_slicing_and_weighted_sampling(gm)

@@ -20,6 +20,11 @@ hoisting of tensor constants.  Operator rewrites (observable in
                                                   -> _CAPI_FusedEDivUSum
   merge_u_mul_v                 two u-op-v SDDMMs on one matrix
                                                   -> _CAPI_FusedUOPV
+  read_column_slice_in_place    a column slice that is only summed (squares
+                                onto rows) and row-sliced is never written:
+                                                  -> _CAPI_SlicedESquareSum,
+                                                     _CAPI_ColRowSlicing on the
+                                                     parent matrix
   select_formats                deterministic on_format / output_format choice
 """
 import operator
@@ -32,7 +37,7 @@ from ..format import _COO, _CSC, _CSR
 # Operators that write into a caller-allocated tensor: they have no users in the
 # graph but must survive dead-code elimination.
 IN_PLACE_OPS = ("_CAPI_SDDMM", "_CAPI_SpMM", "_CAPI_FusedUOPV", "_CAPI_FusedESquareSum",
-                "_CAPI_FusedEDivUSum")
+                "_CAPI_FusedEDivUSum", "_CAPI_SlicedESquareSum")
 
 
 def _input_nodes(node: fx.Node) -> Iterable[fx.Node]:
@@ -442,6 +447,89 @@ def merge_u_mul_v(gm: fx.GraphModule) -> fx.GraphModule:
     return dce(gm)
 
 
+def read_column_slice_in_place(gm: fx.GraphModule) -> fx.GraphModule:
+    """s = A._CAPI_Slicing(cols, axis=1, ...) whose matrix s[0] is only asked for its
+    shape, summed by _CAPI_FusedESquareSum(copy_rhs, sum, e = w[s[1]]) onto rows, and
+    row-sliced (s[0]._CAPI_Slicing(rows, axis=0, ...)), and whose edge index s[1] only
+    gathers edge data that feeds those operators
+        => A._CAPI_SlicedESquareSum(cols, w, out)
+           A._CAPI_ColRowSlicing(cols, rows, on, out)   (edge index into A's edges)
+    The slice -- row id, edge position and column of every edge, and every edge
+    tensor gathered through it -- is then dead and is not computed: a layer-wise
+    sampler slices a few hundred long columns, sums them onto rows, keeps a quarter
+    of the edges and never looks at the rest again (examples/ladies/ladies.py:7-21 of
+    the reference, which fuses neither step for a single matrix)."""
+    for slicing in list(gm.graph.nodes):
+        if not _is_method(slicing, "_CAPI_Slicing") or slicing.args[2] != 1:
+            continue
+        parent, cols = slicing.args[0], slicing.args[1]
+        sliced = _getitem_users(slicing, 0)
+        index = _getitem_users(slicing, 1)
+        if len(sliced) != 1 or len(index) > 1 or len(slicing.users) != len(sliced) + len(index):
+            continue
+        g = sliced[0]
+        gathered = list(index[0].users) if index else []
+        if not all(_is_wrapped(n, "data_index") and n.args[1] is index[0] for n in gathered):
+            continue
+        sums, row_slices, shapes, ok = [], [], [], True
+        for user in g.users:
+            if (_is_method(user, "_CAPI_FusedESquareSum") and user.args[0] is g
+                    and user.args[1] == "copy_rhs" and user.args[2] == "sum"
+                    and user.args[8] == 2 and user.args[4] in gathered):
+                sums.append(user)
+            elif (_is_method(user, "_CAPI_Slicing") and user.args[0] is g
+                  and user.args[2] == 0):
+                row_slices.append(user)
+            elif (_is_method(user, "_CAPI_GetNumRows") or _is_method(user, "_CAPI_GetNumCols")):
+                shapes.append(user)
+            else:
+                ok = False
+        if not ok or not row_slices:
+            continue
+        # what was gathered through the slice may only be summed, looked at for its
+        # shape, or gathered again through the index of one of the row slices
+        regather = []
+        row_indices = [i for rs in row_slices for i in _getitem_users(rs, 1)]
+        for w in gathered:
+            for user in w.users:
+                if user in sums and user.args[4] is w and list(user.all_input_nodes).count(w) == 1:
+                    continue
+                if _is_wrapped(user, "_before_spmm"):
+                    continue
+                if (_is_wrapped(user, "data_index") and user.args[0] is w
+                        and user.args[1] in row_indices):
+                    regather.append(user)
+                    continue
+                ok = False
+        if not ok:
+            continue
+        for node in shapes:
+            with gm.graph.inserting_before(node):
+                if node.target == "_CAPI_GetNumRows":      # a column slice keeps the rows
+                    fresh = gm.graph.call_method("_CAPI_GetNumRows", args=(parent,))
+                else:
+                    fresh = gm.graph.call_method("numel", args=(cols,))
+            node.replace_all_uses_with(fresh)
+        for node in sums:
+            w = node.args[4]
+            with gm.graph.inserting_before(node):
+                gm.graph.call_method("_CAPI_SlicedESquareSum",
+                                     args=(parent, cols, w.args[0], node.args[5]))
+            gm.graph.erase_node(node)
+        for w in gathered:
+            for user in list(w.users):
+                if _is_wrapped(user, "_before_spmm"):      # reads shape and dtype only
+                    user.replace_input_with(w, w.args[0])
+        for rs in row_slices:
+            with gm.graph.inserting_before(rs):
+                fused = gm.graph.call_method(
+                    "_CAPI_ColRowSlicing", args=(parent, cols, rs.args[1], _CSC, rs.args[4]))
+            rs.replace_all_uses_with(fused)
+        for node in regather:                              # the new index addresses the parent
+            node.replace_input_with(node.args[0], node.args[0].args[0])
+    return dce(gm)
+
+
 def sink_block_construction(gm: fx.GraphModule) -> fx.GraphModule:
     """Splitting results per batch and building blocks is host work (and, for the
     splits, a blocking read of the offsets).  Done where the sampler wrote it,
@@ -485,6 +573,7 @@ FORMAT_ARGS = {
     "_CAPI_FusedUOPV": (8, None),
     "_CAPI_FusedESquareSum": (9, None),
     "_CAPI_FusedEDivUSum": (9, None),
+    "_CAPI_ColRowSlicing": (3, 4),
 }
 
 
@@ -503,6 +592,8 @@ def _preferred(node: fx.Node) -> List[int]:
         return [_CSR, _COO] if node.args[8] == 2 else [_CSC, _COO]
     if t == "_CAPI_SDDMM":
         return [_COO, _CSC, _CSR]
+    if t == "_CAPI_ColRowSlicing":
+        return [_CSC]
     return [_COO, _CSC]
 
 

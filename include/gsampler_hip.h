@@ -449,6 +449,38 @@ int gs_minor_slice_fill(const int64_t* ids, int64_t nnz, int64_t num_picked,
                         gs_stream_t stream);
 
 /* ------------------------------------------------------------------------
+ * Column slice and row slice in one: A[rows, cols] read straight from the
+ * parent matrix, without writing the column slice A[:, cols] first.  Edge v of
+ * that slice (sub_indptr = exclusive scan of the picked columns' degrees, e.g.
+ * from gs_csc_col_count with fanout -1; slice_nnz = sub_indptr[num_cols_picked])
+ * is tested like an edge of gs_minor_slice_*: kept when its row id is in
+ * `rows`, relabelled to its position there, order kept.
+ *  count: out_indptr[num_cols_picked + 1] and out_total (nullable, device).
+ *    key_offset[num_cols_picked] (nullable) is added to the row ids of a column's
+ *    edges before the test: the picked sets of the mini-batches of a super-batch
+ *    are told apart as id + batch * stride on both sides.
+ *  fill: out_minor[kept] = position in `rows`, out_select[kept] = position of the
+ *    edge in the PARENT's indices, out_major[kept] (nullable) = position of its
+ *    column in `cols`.
+ * Workspace: gs_minor_slice_workspace_bytes(slice_nnz, num_rows_picked), the
+ * same buffer for both calls.  Stands in for CSCColRowSlicingCUDA and
+ * BatchCSCColRowSlicingCUDA (src/cuda/fusion/column_row_slicing.cu:213-217,
+ * 356-362; kernels :102-146, :220-264), whose select index addresses the
+ * intermediate slice instead of the parent.
+ * ---------------------------------------------------------------------- */
+int gs_col_row_slice_count(const int64_t* indptr, const int64_t* indices, const int64_t* cols,
+                           const int64_t* key_offset, int64_t num_cols_picked,
+                           const int64_t* sub_indptr, int64_t slice_nnz,
+                           const int64_t* rows, int64_t num_rows_picked,
+                           int64_t* out_indptr, int64_t* out_total, void* workspace,
+                           size_t workspace_bytes, gs_stream_t stream);
+int gs_col_row_slice_fill(const int64_t* indptr, const int64_t* indices, const int64_t* cols,
+                          int64_t num_cols_picked, const int64_t* sub_indptr,
+                          int64_t slice_nnz, int64_t num_rows_picked, int64_t* out_major,
+                          int64_t* out_minor, int64_t* out_select, void* workspace,
+                          size_t workspace_bytes, gs_stream_t stream);
+
+/* ------------------------------------------------------------------------
  * Format conversion.
  *  gs_csc2coo: out_col[e] = column that owns edge position e
  *    (CSC2COOCUDA, src/cuda/format_transform.cu:24-46).
@@ -578,6 +610,20 @@ int gs_e_square_sum(int format, const int64_t* a, const int64_t* b,
                     const float* efeat, float* out, int u_target,
                     int64_t feat_len, int64_t num_out, void* workspace,
                     size_t workspace_bytes, gs_stream_t stream);
+/* out[row] += sum of e^2 over the edges of A[:, cols], read from the parent
+ * matrix (the column slice is not written): cols / sub_indptr / slice_nnz as in
+ * gs_col_row_slice_count, the value of the parent's edge p is efeat[edge_map[p]]
+ * (efeat[p] when edge_map is NULL), out[num_out] an fp32 accumulator that the
+ * caller zero-fills.  The workspace is optional
+ * (NULL / 0 is valid, then every edge is an atomic add).  No counterpart in the
+ * reference, which writes the slice and then runs ESquareSumCOO over it
+ * (src/cuda/fusion/fused_coo_e_square_sum.cu:13-60). */
+size_t gs_sliced_e_square_sum_workspace_bytes(int64_t slice_nnz, int64_t num_out);
+int gs_sliced_e_square_sum(const int64_t* indptr, const int64_t* indices, const int64_t* cols,
+                           int64_t num_cols_picked, const int64_t* sub_indptr,
+                           int64_t slice_nnz, const int64_t* edge_map, const float* efeat,
+                           float* out, int64_t num_out, void* workspace,
+                           size_t workspace_bytes, gs_stream_t stream);
 int gs_e_div_u_sum(int format, const int64_t* a, const int64_t* b,
                    int64_t num_major, int64_t nnz, const int64_t* edge_map,
                    const float* ufeat, const float* efeat, float* out,

@@ -138,20 +138,55 @@ def test_ladies_rewrites():
     m.edata["w"] = torch.rand(7)
     c = gs.jit.compile(func=ladies_sampler, args=(m, torch.arange(3), [4, 4]))
     t = targets(c.gm)
-    assert t.count("_CAPI_FusedESquareSum") == 2          # (w ** 2).sum fused
+    # the column slice is only summed and row-sliced: it is read in place, never written
+    assert t.count("_CAPI_SlicedESquareSum") == 2 and t.count("_CAPI_ColRowSlicing") == 2
+    assert "_CAPI_Slicing" not in t and "_CAPI_FusedESquareSum" not in t
     import operator
     assert not any(n.target is operator.pow for n in c.gm.graph.nodes)   # the square itself is gone
     assert t.count("_CAPI_SpMM") == 2                     # the column sums stay
     assert t.count("_CAPI_SDDMM") == 4
     assert "_CAPI_GetValidNodes" not in t
-    # formats: the row slice runs on the CSC the column slice produced (no sort)
-    row_slices = [n for n in c.gm.graph.nodes
-                  if n.target == "_CAPI_Slicing" and n.args[2] == 0]
-    assert row_slices and all(n.args[3] == gs._CSC for n in row_slices)
+    fused = [n for n in c.gm.graph.nodes if n.target == "_CAPI_ColRowSlicing"]
+    for n in fused:
+        # on the parent matrix (a run-time input), on its CSC, giving CSC + COO
+        assert n.args[0].op == "call_function" and n.args[0].args[0].op == "placeholder"
+        assert n.args[3] == gs._CSC and n.args[4] == gs._CSC | gs._COO
+    # the weights of the kept edges are gathered from the parent's edge data with the
+    # fused operator's index; nothing is gathered through a slice index any more
+    gathers = [n for n in c.gm.graph.nodes
+               if getattr(n.target, "__name__", "") == "data_index"]
+    assert len(gathers) == 2 and all(g.args[0].op == "placeholder" for g in gathers)
     # edge data is a run-time input, not a baked constant
     assert not any(n.op == "get_attr" and "constant" in n.name and n.meta.get("val") is not None
                    for n in c.gm.graph.nodes)
     assert sum(n.op == "placeholder" for n in c.gm.graph.nodes) >= 3
+
+
+def test_column_slice_stays_when_something_else_reads_it():
+    """The rewrite must not fire when the slice, or edge data gathered through it, has a
+    reader it cannot serve from the parent matrix."""
+    def keeps_the_slice(A, seeds, K):
+        subA = A[:, seeds]
+        subA.edata["p"] = subA.edata["w"] ** 2
+        prob = subA.sum("p", axis=1)
+        sampleA, _ = subA.collective_sampling(K, prob, False)
+        return sampleA.all_nodes(), subA.edata["w"]          # the slice's weights escape
+
+    def sums_columns_too(A, seeds, K):
+        subA = A[:, seeds]
+        subA.edata["p"] = subA.edata["w"] ** 2
+        prob = subA.sum("p", axis=1)
+        extra = subA.sum("w", axis=0)                         # another reader of the slice
+        sampleA, _ = subA.collective_sampling(K, prob, False)
+        return sampleA.all_nodes(), extra
+
+    for func in (keeps_the_slice, sums_columns_too):
+        m = gs.Matrix(gs.Graph(10, 10))
+        m.edata["w"] = torch.rand(7)
+        c = gs.jit.compile(func=func, args=(m, torch.arange(3), 4))
+        t = targets(c.gm)
+        assert "_CAPI_ColRowSlicing" not in t and "_CAPI_SlicedESquareSum" not in t
+        assert t.count("_CAPI_Slicing") == 2
 
 
 def fastgcn_like_sampler(A, seeds, fanouts):
