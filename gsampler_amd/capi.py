@@ -87,6 +87,10 @@ SIGNATURES = {
     "gs_col_row_slice_count": (_int, [_p, _p, _p, _p, _i64, _p, _i64, _p, _i64, _p, _p, _p, _sz,
                                       _p]),
     "gs_col_row_slice_fill": (_int, [_p, _p, _p, _i64, _p, _i64, _i64, _p, _p, _p, _p, _sz, _p]),
+    "gs_probe_stream_copy": (_int, [_p, _p, _i64, _p]),
+    "gs_probe_line_gather": (_int, [_p, _i64, _i64, _u64, _int, _p, _p]),
+    "gs_probe_sample_uniform": (_int, [_p, _i64, _p, _p, _i64, _i64, _int, _i64, _u64, _u64, _p,
+                                       _p, _p, _p, _p]),
     "gs_sliced_e_square_sum_workspace_bytes": (_sz, [_i64, _i64]),
     "gs_sliced_e_square_sum": (_int, [_p, _p, _p, _i64, _p, _i64, _p, _p, _p, _i64, _p, _sz, _p]),
     "gs_weight_cdf_workspace_bytes": (_sz, [_i64, _i64]),
@@ -714,6 +718,32 @@ def sliced_e_square_sum(indptr, indices, cols, efeat, num_out, use_workspace=Tru
                                    out.data_ptr(), num_out, ws.data_ptr() if ws.numel() else None,
                                    ws.numel(), _stream()))
     return out
+
+
+# ------------------------------------------------------------------ yardsticks
+def probe_stream_copy(src, dst):
+    """dst = src by the library's own copy kernel (a streaming yardstick)."""
+    nbytes = src.numel() * src.element_size()
+    check(lib().gs_probe_stream_copy(src.data_ptr(), dst.data_ptr(), nbytes, _stream()))
+
+
+def probe_line_gather(table, num_picks, salt=0, ordered=False, out=None):
+    """Every lane reads 4 bytes of a 128-byte line of its own of `table`."""
+    if out is None:
+        out = torch.empty(num_picks // 4 + 1, dtype=torch.int32, device=table.device)
+    check(lib().gs_probe_line_gather(table.data_ptr(), table.numel() * table.element_size(),
+                                     num_picks, salt, int(ordered), out.data_ptr(), _stream()))
+    return out
+
+
+def probe_sample_uniform(indptr, indices32, column_ids, fanout, variant, sub_indptr, outs,
+                         probe_degree=0, seed=7777, call_id=0):
+    """One launch of the packed uniform sampler with parts switched off (see
+    gs_probe_sample_uniform); outs = (coo_col | None, rows, select) preallocated."""
+    check(lib().gs_probe_sample_uniform(
+        _ptr(indptr), indptr.numel() - 1, indices32.data_ptr(), _ptr(column_ids),
+        column_ids.numel(), fanout, variant, probe_degree, seed, call_id, _ptr(sub_indptr),
+        _ptr(outs[0]), outs[1].data_ptr(), outs[2].data_ptr(), _stream()))
 
 
 # --------------------------------------------------------- weighted sampling

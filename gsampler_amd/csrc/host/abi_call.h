@@ -7,6 +7,7 @@
 #include <c10/hip/HIPFunctions.h>
 #include <c10/hip/HIPStream.h>
 #include <hip/hip_runtime_api.h>
+#include <atomic>
 #include <torch/torch.h>
 
 #include <vector>
@@ -21,6 +22,27 @@ namespace gs {
     TORCH_CHECK(gs_rc__ == GS_OK, "gsampler_hip error ", gs_rc__, ": ",      \
                 gs_last_error());                                            \
   } while (0)
+
+// Everything the operators remember between calls (the int32 copy of a matrix's
+// ids, its weight CDF, offsets read back to the host, the frontier of the last
+// relabel, ...) is keyed by the identity and version counter of the tensors it
+// was made from.  A write that goes around torch (another extension, a raw
+// pointer, a replayed HIP graph) changes the memory without moving that counter:
+// whoever makes one calls invalidate_caches(), which ages everything at once.
+// Entries carry the epoch they were made in and are ignored in a later one.
+inline std::atomic<int64_t>& cache_epoch_counter() {
+  static std::atomic<int64_t> epoch{0};
+  return epoch;
+}
+inline int64_t cache_epoch() { return cache_epoch_counter().load(std::memory_order_relaxed); }
+inline void invalidate_caches() { cache_epoch_counter().fetch_add(1); }
+
+// Whether a loaded matrix may keep an int32 copy of its ids for the uniform
+// sampler (4 bytes per edge of device memory for half the bytes behind a pick).
+inline std::atomic<bool>& narrow_ids_allowed() {
+  static std::atomic<bool> on{true};
+  return on;
+}
 
 inline gs_stream_t cur_stream() {
   return (gs_stream_t)c10::hip::getCurrentHIPStream().stream();
@@ -188,7 +210,7 @@ class OffsetMirror {
  private:
   struct Entry {
     torch::Tensor tensor;
-    int64_t version = -1;
+    int64_t version = -1, epoch = -1;
     int64_t* pinned = nullptr;
     size_t capacity = 0, count = 0;
     hipEvent_t event = nullptr;
@@ -209,12 +231,13 @@ class OffsetMirror {
                 "batch offsets must be an int64 tensor");
     for (Entry& e : ring)
       if (e.tensor.defined() && e.tensor.is_same(offsets) &&
-          e.version == (int64_t)offsets._version())
+          e.version == (int64_t)offsets._version() && e.epoch == cache_epoch())
         return e;
     Entry& e = ring[next++ % kEntries];
     if (e.pending) check(hipEventSynchronize(e.event));  // its copy must not land later
     e.tensor = offsets;
     e.version = offsets._version();
+    e.epoch = cache_epoch();
     e.count = (size_t)offsets.numel();
     e.pending = false;
     if (!offsets.is_cuda() && copy) {
@@ -304,6 +327,7 @@ class BatchOffsets {
     Known& k = ring()[next()++ % kEntries];
     k.tensor = offsets;  // kept alive: neither its address nor its memory can be handed out again
     k.version = (int64_t)offsets._version();
+    k.epoch = cache_epoch();
     k.total = total;
   }
   static void check(const torch::Tensor& offsets, int64_t total, const char* who) {
@@ -328,7 +352,7 @@ class BatchOffsets {
  private:
   struct Known {
     torch::Tensor tensor;
-    int64_t version = -1;
+    int64_t version = -1, epoch = -1;
     int64_t total = -1;
   };
   static constexpr size_t kEntries = 32;
@@ -342,7 +366,8 @@ class BatchOffsets {
   }
   static Known* trusted(const torch::Tensor& t) {
     for (Known& k : ring())
-      if (k.tensor.defined() && k.tensor.is_same(t) && k.version == (int64_t)t._version())
+      if (k.tensor.defined() && k.tensor.is_same(t) && k.version == (int64_t)t._version() &&
+          k.epoch == cache_epoch())
         return &k;
     return nullptr;
   }

@@ -17,13 +17,15 @@ const Graph::SliceOffsets& Graph::slice_offsets_for(const torch::Tensor& cols) {
   const Compressed& m = compressed(kCSC);
   if (slice_offsets_ && slice_offsets_->cols.is_same(cols) &&
       slice_offsets_->version == (int64_t)cols._version() &&
-      slice_offsets_->indptr_version == (int64_t)m.indptr._version())
+      slice_offsets_->indptr_version == (int64_t)m.indptr._version() &&
+      slice_offsets_->epoch == cache_epoch())
     return *slice_offsets_;
   auto so = std::make_unique<SliceOffsets>();
   const int64_t num_major = m.indptr.numel() - 1, n = cols.numel();
   so->cols = cols;
   so->version = cols._version();
   so->indptr_version = m.indptr._version();
+  so->epoch = cache_epoch();
   so->sub_indptr = new_ids(n + 1, m.indptr);
   torch::Tensor ws = new_workspace(gs_scan_workspace_bytes(n + 1), m.indptr);
   AsyncCount count = AsyncCount::mirrored();
@@ -115,9 +117,9 @@ static MajorResult col_row_slice(const Compressed& m, const torch::Tensor& cols,
                                 with_coo ? mptr(r.major_ids) : nullptr, mptr(r.minor_ids),
                                 mptr(r.select), ws.data_ptr(), ws.numel(), cur_stream()));
   const int64_t k = kept.get();
-  r.minor_ids = r.minor_ids.narrow(0, 0, k);
-  r.select = r.select.narrow(0, 0, k);
-  if (with_coo) r.major_ids = r.major_ids.narrow(0, 0, k);
+  r.minor_ids = trim_to(r.minor_ids, k);
+  r.select = trim_to(r.select, k);
+  if (with_coo) r.major_ids = trim_to(r.major_ids, k);
   return r;
 }
 

@@ -7,6 +7,8 @@
 
 #include "abi_call.h"
 
+#include <mutex>
+
 namespace gs {
 
 RandomState& random_state() {
@@ -42,6 +44,7 @@ static void check_compressed(const torch::Tensor& indptr, const torch::Tensor& i
 }
 
 void Graph::LoadCSC(torch::Tensor indptr, torch::Tensor indices) {
+  invalidate_caches();  // whatever was derived from an earlier matrix of this object
   auto m = std::make_shared<Compressed>();
   m->indptr = graph_ids(indptr, "indptr");
   m->indices = graph_ids(indices, "indices");
@@ -54,6 +57,7 @@ void Graph::LoadCSC(torch::Tensor indptr, torch::Tensor indices) {
 }
 
 void Graph::LoadCSR(torch::Tensor indptr, torch::Tensor indices) {
+  invalidate_caches();  // whatever was derived from an earlier matrix of this object
   auto m = std::make_shared<Compressed>();
   m->indptr = graph_ids(indptr, "indptr");
   m->indices = graph_ids(indices, "indices");
@@ -67,6 +71,7 @@ void Graph::LoadCSR(torch::Tensor indptr, torch::Tensor indices) {
 
 void Graph::LoadCOO(torch::Tensor row, torch::Tensor col, bool row_sorted,
                     bool col_sorted) {
+  invalidate_caches();  // whatever was derived from an earlier matrix of this object
   auto m = std::make_shared<Coordinate>();
   m->row = graph_ids(row, "row");
   m->col = graph_ids(col, "col");
@@ -204,14 +209,20 @@ MajorResult major_slice(const Compressed& m, const torch::Tensor& picked,
 // array stays in cache anyway); undefined when the matrix does not qualify.
 const torch::Tensor& Compressed::narrow_indices() const {
   constexpr int64_t kMinEdges = int64_t(1) << 20;
+  // one matrix is shared by every handle derived from it and by every sampler
+  // thread: the copy is made (and dropped) under a lock
+  static std::mutex guard;
+  std::lock_guard<std::mutex> lock(guard);
   const int64_t version = (int64_t)indices._version();
   if (indices32.defined() &&
-      (indices32_version != version || indices32_source != indices.data_ptr()))
-    indices32 = torch::Tensor();  // edited in place, or another array
-  if (!indices32.defined() && num_minor >= 0 && num_minor < (int64_t(1) << 31) &&
-      indices.is_cuda() && indices.numel() >= kMinEdges) {
+      (indices32_version != version || indices32_source != indices.data_ptr() ||
+       indices32_epoch != cache_epoch() || !narrow_ids_allowed().load()))
+    indices32 = torch::Tensor();  // edited, another array, or switched off
+  if (!indices32.defined() && narrow_ids_allowed().load() && num_minor >= 0 &&
+      num_minor < (int64_t(1) << 31) && indices.is_cuda() && indices.numel() >= kMinEdges) {
     indices32 = indices.to(torch::kInt32);
     indices32_version = version;
+    indices32_epoch = cache_epoch();
     indices32_source = indices.data_ptr();
   }
   return indices32;
@@ -307,7 +318,7 @@ GraphPtr Graph::derive(int64_t on_format, int64_t output_format,
 struct SliceRuns {
   c10::optional<c10::weak_intrusive_ptr<c10::TensorImpl>> select;
   torch::Tensor parent_indptr, picked, sub_indptr;
-  int64_t version = -1, parent_edges = 0;
+  int64_t version = -1, parent_edges = 0, epoch = -1;
   int64_t source_versions[3] = {-1, -1, -1};  // of parent_indptr, picked, sub_indptr
   static SliceRuns& last() {
     static thread_local SliceRuns s;
@@ -323,6 +334,7 @@ struct SliceRuns {
     s.picked = picked;
     s.sub_indptr = sub_indptr;
     s.version = (int64_t)select._version();
+    s.epoch = cache_epoch();
     s.source_versions[0] = (int64_t)parent_indptr._version();
     s.source_versions[1] = (int64_t)picked._version();
     s.source_versions[2] = (int64_t)sub_indptr._version();
@@ -332,7 +344,7 @@ struct SliceRuns {
     if (!select.has_value() || !ids.defined()) return false;
     // a live target cannot have been replaced by another tensor at the same address
     const c10::intrusive_ptr<c10::TensorImpl> held = select->lock();
-    return held && held.get() == ids.unsafeGetTensorImpl() &&
+    return held && held.get() == ids.unsafeGetTensorImpl() && epoch == cache_epoch() &&
            (int64_t)ids._version() == version &&
            (int64_t)parent_indptr._version() == source_versions[0] &&
            (int64_t)picked._version() == source_versions[1] &&
@@ -448,7 +460,7 @@ bool Graph::Frontier::matches(const torch::Tensor& s, const torch::Tensor& r,
   };
   return same(seeds, s) && same(rows, r) && same(seeds_ptr, sp) &&
          same(rows_ptr, rp) && seeds_version == (int64_t)s._version() &&
-         rows_version == (int64_t)r._version();
+         rows_version == (int64_t)r._version() && epoch == cache_epoch();
 }
 
 // Unique (first-occurrence order) of seeds_b ++ rows_b per batch; the hash
@@ -466,6 +478,7 @@ Graph::Frontier& Graph::frontier_for(const torch::Tensor& seeds,
   f->rows_ptr = rows_ptr;
   f->seeds_version = seeds._version();
   f->rows_version = rows._version();
+  f->epoch = cache_epoch();
   const int64_t B = seeds_ptr.defined() ? seeds_ptr.numel() - 1 : 1;
   TORCH_CHECK(B >= 1, "unique: at least one batch is required");
   f->num_batches = B;
@@ -529,7 +542,8 @@ Graph::ListLabels& Graph::list_labels_for(const torch::Tensor& col_seeds,
   if (list_labels_ && list_labels_->base.is_same(base) &&
       list_labels_->row_ids.is_same(row_ids) && list_labels_->seeds.is_same(col_seeds) &&
       list_labels_->row_ids_version == (int64_t)row_ids._version() &&
-      list_labels_->seeds_version == (int64_t)col_seeds._version())
+      list_labels_->seeds_version == (int64_t)col_seeds._version() &&
+      list_labels_->epoch == cache_epoch())
     return *list_labels_;
   auto out = std::make_unique<ListLabels>();
   out->base = base;
@@ -537,6 +551,7 @@ Graph::ListLabels& Graph::list_labels_for(const torch::Tensor& col_seeds,
   out->seeds = col_seeds;
   out->row_ids_version = row_ids._version();
   out->seeds_version = col_seeds._version();
+  out->epoch = cache_epoch();
   torch::Tensor table = ids(row_ids, "row_ids");
   const int64_t R = table.numel(), S = col_seeds.numel(), E = base.numel();
   torch::Tensor first = new_ids(R, base);

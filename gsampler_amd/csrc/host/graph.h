@@ -34,6 +34,7 @@ struct Compressed {
   // memory whose ids fit.
   mutable torch::Tensor indices32;
   mutable int64_t indices32_version = -1;  // version of `indices` the copy was made from
+  mutable int64_t indices32_epoch = -1;    // and the cache epoch (invalidate_caches)
   mutable const void* indices32_source = nullptr;  // and its address
   const torch::Tensor& narrow_indices() const;
   // Call after assigning another `indices` or `indptr` to a matrix that was used.
@@ -255,7 +256,7 @@ class Graph : public torch::CustomClassHolder {
   // frontier is computed once, the relabel pass reuses the hash tables.
   struct Frontier {
     torch::Tensor seeds, rows, seeds_ptr, rows_ptr;  // the keys it was built from
-    int64_t seeds_version = -1, rows_version = -1;
+    int64_t seeds_version = -1, rows_version = -1, epoch = -1;
     torch::Tensor workspace, unique_ptr;
     int64_t num_batches = 0;
     // The unique keys: filled into a buffer sized by the upper bound, trimmed
@@ -284,7 +285,7 @@ class Graph : public torch::CustomClassHolder {
   // that is handed the same tensor of columns.
   struct SliceOffsets {
     torch::Tensor cols, sub_indptr;
-    int64_t version = -1, indptr_version = -1, nnz = 0;
+    int64_t version = -1, indptr_version = -1, epoch = -1, nnz = 0;
     MajorResult written;  // the slice itself, when an operator had to write it
   };
   std::unique_ptr<SliceOffsets> slice_offsets_;
@@ -298,7 +299,7 @@ class Graph : public torch::CustomClassHolder {
                              int64_t u_target, const char* who) const;
   bool csc_sorted_ = false;  // row ids known to be sorted inside every column
   torch::Tensor cdf_, cdf_probs_;
-  int64_t cdf_version_ = -1, cdf_format_ = 0;
+  int64_t cdf_version_ = -1, cdf_format_ = 0, cdf_epoch_ = -1;
   torch::Tensor mapped_rows(const torch::Tensor& base, const torch::Tensor& row_ids);
   GraphAndIndex slice_coo(const torch::Tensor& seeds, int64_t axis,
                           int64_t new_rows, int64_t new_cols);
@@ -332,7 +333,7 @@ class Graph : public torch::CustomClassHolder {
   // seed, computed from the list instead of from every edge.
   struct ListLabels {
     torch::Tensor base, row_ids, seeds;
-    int64_t row_ids_version = -1, seeds_version = -1;
+    int64_t row_ids_version = -1, seeds_version = -1, epoch = -1;
     torch::Tensor label_by_local, seed_label;
     // The unique keys sit at the front of a buffer sized by the bound; how many
     // there are may still be on its way from the device.
@@ -361,6 +362,9 @@ MajorResult major_sample_uniform(const Compressed& m, const torch::Tensor& picke
                                  int64_t fanout, bool replace, bool with_coo);
 MajorResult minor_slice(const Compressed& m, const torch::Tensor& picked,
                         bool with_coo);
+// First n entries of a buffer sized by an upper bound: a view, or a copy when
+// the view would pin a large buffer for a small result.
+torch::Tensor trim_to(const torch::Tensor& buffer, int64_t n);
 
 // ---- free operators (gs_ops)
 torch::Tensor GatherRows(torch::Tensor table, torch::Tensor ids);

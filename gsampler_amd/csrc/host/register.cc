@@ -25,6 +25,12 @@ static void set_sampling_algorithm(int64_t algo) {
   random_state().algo = algo;
 }
 static int64_t abi_version() { return gs_abi_version(); }
+// After a write to a graph or weight tensor that went around torch (a raw
+// pointer, another extension, a replayed HIP graph): forget everything derived
+// from tensor contents.
+static void invalidate_all_caches() { invalidate_caches(); }
+// Whether loaded matrices may keep an int32 copy of their ids (on by default).
+static void set_narrow_ids(bool on) { narrow_ids_allowed().store(on); }
 
 }  // namespace gs
 
@@ -124,4 +130,6 @@ TORCH_LIBRARY(gs_ops, m) {
   m.def("_CAPI_SetNextCallId", &gs::set_next_call_id);
   m.def("_CAPI_SetSamplingAlgorithm", &gs::set_sampling_algorithm);
   m.def("_CAPI_AbiVersion", &gs::abi_version);
+  m.def("_CAPI_InvalidateCaches", &gs::invalidate_all_caches);
+  m.def("_CAPI_SetNarrowIds", &gs::set_narrow_ids);
 }

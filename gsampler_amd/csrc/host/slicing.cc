@@ -5,6 +5,17 @@
 
 namespace gs {
 
+// The first n entries of a buffer that was sized by an upper bound.  A view
+// keeps the whole buffer alive for as long as the result lives: when the result
+// is a small part of a large buffer (a row slice that keeps one edge in a hundred
+// of a 60 M-edge matrix would pin three 480 MB buffers) it is copied out instead.
+torch::Tensor trim_to(const torch::Tensor& buffer, int64_t n) {
+  constexpr int64_t kLarge = int64_t(1) << 22;  // elements
+  torch::Tensor head = buffer.narrow(0, 0, n);
+  if (buffer.numel() > kLarge && n * 8 < buffer.numel()) return head.clone();
+  return head;
+}
+
 namespace {
 struct MinorKept {
   torch::Tensor indptr, major, minor, select;
@@ -38,9 +49,9 @@ MinorKept keep_members(const torch::Tensor& ids_per_edge, const torch::Tensor& p
                               mptr(r.minor), mptr(r.select), ws.data_ptr(),
                               ws.numel(), cur_stream()));
   const int64_t n = kept.get();
-  r.minor = r.minor.narrow(0, 0, n);
-  r.select = r.select.narrow(0, 0, n);
-  if (want_major) r.major = r.major.narrow(0, 0, n);
+  r.minor = trim_to(r.minor, n);
+  r.select = trim_to(r.select, n);
+  if (want_major) r.major = trim_to(r.major, n);
   return r;
 }
 }  // namespace

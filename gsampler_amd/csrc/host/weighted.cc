@@ -60,7 +60,7 @@ GraphAndIndex Graph::SamplingProbs(int64_t axis, torch::Tensor edge_probs,
 // ----------------------------------------- fused slice + weighted sampling
 torch::Tensor Graph::weight_cdf_for(const torch::Tensor& edge_probs, int64_t format) {
   if (cdf_.defined() && cdf_format_ == format && cdf_probs_.is_same(edge_probs) &&
-      cdf_version_ == (int64_t)edge_probs._version())
+      cdf_version_ == (int64_t)edge_probs._version() && cdf_epoch_ == cache_epoch())
     return cdf_;
   const Compressed& m = compressed(format);
   torch::Tensor probs = f32(edge_probs, "edge_probs");
@@ -78,6 +78,7 @@ torch::Tensor Graph::weight_cdf_for(const torch::Tensor& edge_probs, int64_t for
   cdf_ = cdf;
   cdf_probs_ = edge_probs;
   cdf_version_ = edge_probs._version();
+  cdf_epoch_ = cache_epoch();
   cdf_format_ = format;
   return cdf_;
 }

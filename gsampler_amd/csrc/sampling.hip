@@ -103,13 +103,22 @@ __device__ __forceinline__ int64_t floyd_slot_packed(int lane, int gbase, int K,
 // 124M-edge power-law graph the kernel moves about 6 TB/s through the memory
 // fabric, nearly all of it the 128-byte lines behind 4- or 8-byte picks;
 // giving a slice several columns to pipeline measured 3 % to 20 % slower.
-template <typename IdxT>
+// kProbe (0 in every operator) switches parts of the kernel off for the
+// measurement that prices them (gs_probe_sample_uniform): 1 a multiplicative hash
+// instead of Philox, 2 no exchange among a column's lanes (repeats are kept),
+// 4 no read of the column pointer (every column `probe_degree` long, starting at
+// id * probe_degree), 8 no read of the row ids, 16 only the row id is stored,
+// 32 nothing is stored.
+constexpr int kProbeHash = 1, kProbeNoExchange = 2, kProbeNoIndptr = 4, kProbeNoIndices = 8,
+              kProbeOneStore = 16, kProbeNoStore = 32;
+template <typename IdxT, int kProbe = 0>
 __global__ __launch_bounds__(kBlock) void sample_uniform_packed_kernel(
     const int64_t* __restrict__ indptr, int64_t num_cols,
     const IdxT* __restrict__ indices, const int64_t* __restrict__ column_ids,
     int64_t num_items, int fanout, int cols_per_wave, int replace, PhiloxKey key,
     const int64_t* __restrict__ sub_indptr, int64_t* __restrict__ out_coo_col,
-    int64_t* __restrict__ out_indices, int64_t* __restrict__ out_select) {
+    int64_t* __restrict__ out_indices, int64_t* __restrict__ out_select,
+    int64_t probe_degree = 0) {
   const int wave_lane = threadIdx.x & (kWave - 1);
   const int group = wave_lane / fanout;
   const int lane = wave_lane - group * fanout;
@@ -121,20 +130,58 @@ __global__ __launch_bounds__(kBlock) void sample_uniform_packed_kernel(
   if (group >= cols_per_wave || item >= num_items) return;  // whole groups leave together
   const int64_t c = column_ids ? column_ids[item] : item;
   int64_t in_start;
-  const int64_t deg = column_degree(indptr, num_cols, c, &in_start);
+  int64_t deg;
+  if (kProbe & kProbeNoIndptr) {
+    deg = probe_degree;
+    in_start = c * probe_degree;
+  } else {
+    deg = column_degree(indptr, num_cols, c, &in_start);
+  }
   if (deg == 0) return;
-  const int64_t out_start = sub_indptr[item];
+  const int64_t out_start = (kProbe & kProbeNoIndptr) ? item * fanout : sub_indptr[item];
   int64_t p = -1;
   if (replace) {
     p = in_start + (int64_t)philox_bounded(key, (uint64_t)item, (uint64_t)lane, (uint64_t)deg);
   } else if (deg <= fanout) {
     if (lane < deg) p = in_start + lane;  // whole column, in order
+  } else if (kProbe & (kProbeHash | kProbeNoExchange)) {
+    const int64_t j = deg - fanout + lane;
+    uint64_t r;
+    if (kProbe & kProbeHash) {
+      r = ((uint64_t)item * 64 + (uint64_t)lane + key.k0) * 0x9E3779B97F4A7C15ull;
+      r ^= r >> 31;
+      r = __umul64hi(r * 0xBF58476D1CE4E5B9ull, (uint64_t)j + 1);
+    } else {
+      r = philox_bounded(key, (uint64_t)item, (uint64_t)lane, (uint64_t)j + 1);
+    }
+    p = in_start + (int64_t)r;
+    if (!(kProbe & kProbeNoExchange)) {  // the exchange of floyd_slot_packed on these draws
+      const int gbase = group * fanout;
+      const int64_t t = (int64_t)r, base = deg - fanout;
+      bool dup = false;
+      for (int m = 0; m < fanout; ++m) {
+        const int64_t tm = __shfl(t, gbase + m, kWave);
+        dup |= (m < lane) & (tm == t);
+      }
+      const int64_t mi = t - base;
+      for (int m = 0; m < fanout; ++m) {
+        const int dm = __shfl((int)dup, gbase + m, kWave);
+        if (mi == m && m < lane) dup |= (dm != 0);
+      }
+      p = in_start + (dup ? j : t);
+    }
   } else {
     p = in_start + floyd_slot_packed(lane, group * fanout, fanout, deg, key, (uint64_t)item);
   }
   if (p < 0) return;
-  const int64_t v = indices ? (int64_t)indices[p] : p;
+  const int64_t v = (indices && !(kProbe & kProbeNoIndices)) ? (int64_t)indices[p] : p;
+  if (kProbe & kProbeNoStore) {
+    // keep the pick (and the row id behind it) live without a store that happens
+    if (v == -7777) out_indices[0] = p;  // ids are not negative; the compiler cannot know
+    return;
+  }
   out_indices[out_start + lane] = v;
+  if (kProbe & kProbeOneStore) return;
   out_select[out_start + lane] = p;
   if (out_coo_col) out_coo_col[out_start + lane] = item;
 }
@@ -245,6 +292,53 @@ extern "C" int gs_csc_col_sample_uniform_fill_i32(
   return gs::sample_uniform_fill<int32_t>(indptr, num_cols, indices32, column_ids, num_items,
                                           fanout, replace, algo, seed, call_id, sub_indptr,
                                           out_coo_col, out_indices, out_select, stream);
+}
+
+// One launch of the packed sampler with parts switched off (`variant` = a sum of
+// the kProbe* bits above); int32 row ids, fanout <= 64, without replacement.
+// With kProbeNoIndptr the columns are taken to be probe_degree long and the
+// outputs need num_items * fanout entries.  Measurement only: the picks of a
+// variant are not those of the operator.
+extern "C" int gs_probe_sample_uniform(
+    const int64_t* indptr, int64_t num_cols, const int32_t* indices32,
+    const int64_t* column_ids, int64_t num_items, int64_t fanout, int variant,
+    int64_t probe_degree, uint64_t seed, uint64_t call_id, const int64_t* sub_indptr,
+    int64_t* out_coo_col, int64_t* out_indices, int64_t* out_select, gs_stream_t stream) {
+  using namespace gs;
+  GS_REQUIRE(num_items > 0 && fanout >= 1 && fanout <= kWave, "probe_sample_uniform: bad size");
+  GS_REQUIRE(indptr && indices32 && column_ids && sub_indptr && out_indices && out_select,
+             "probe_sample_uniform: null pointer");
+  GS_REQUIRE(!(variant & kProbeNoIndptr) || probe_degree > fanout,
+             "probe_sample_uniform: probe_degree must exceed the fanout");
+  const PhiloxKey key = make_key(seed, call_id);
+  hipStream_t s = as_stream(stream);
+  const int cols_per_wave = kWave / (int)fanout;
+  const int64_t waves = ceil_div(num_items, cols_per_wave);
+  const dim3 grid((unsigned)(ceil_div(ceil_div(waves * kWave, kBlock), 8) * 8));
+#define GS_PROBE_CASE(V)                                                                      \
+  case V:                                                                                     \
+    GS_LAUNCH("probe_sample_uniform", s,                                                      \
+              (sample_uniform_packed_kernel<int32_t, V>)<<<grid, dim3(kBlock), 0, s>>>(       \
+                  indptr, num_cols, indices32, column_ids, num_items, (int)fanout,            \
+                  cols_per_wave, 0, key, sub_indptr, out_coo_col, out_indices, out_select,    \
+                  probe_degree));                                                             \
+    return GS_OK;
+  switch (variant) {
+    GS_PROBE_CASE(0)
+    GS_PROBE_CASE(kProbeHash)
+    GS_PROBE_CASE(kProbeNoExchange)
+    GS_PROBE_CASE(kProbeNoIndptr)
+    GS_PROBE_CASE(kProbeNoIndices)
+    GS_PROBE_CASE(kProbeNoIndices | kProbeOneStore)
+    GS_PROBE_CASE(kProbeOneStore)
+    GS_PROBE_CASE(kProbeNoStore)
+    GS_PROBE_CASE(kProbeNoIndices | kProbeNoStore)
+    default:
+      break;
+  }
+#undef GS_PROBE_CASE
+  set_error("probe_sample_uniform: variant %d is not built", variant);
+  return GS_ERR_INVALID;
 }
 
 // ---------------------------------------------------------------------------

@@ -152,19 +152,26 @@ def _merge_batch_blocks_and_all_nodes(gm: fx.GraphModule) -> fx.GraphModule:
         if not builders or not valid:
             continue
         keep = builders[0]
-        first = min(group, key=lambda n: order[n])
+        # only all_nodes() calls with the builder's own id tensors read its frontier
+        matching = [v for v in valid if v.args[1:] == keep.args[1:]]
+        if not matching:
+            continue
+        first = min(matching + [keep], key=lambda n: order[n])
         if first is not keep:
+            # the builder moves in front of its first reader, but never in front of
+            # one of its own arguments
+            if any(order[a] > order[first] for a in keep.all_input_nodes):
+                continue
             first.prepend(keep)
         with gm.graph.inserting_after(keep):
             ptr = gm.graph.call_method("frontier_ptr", args=(keep,))
             frontier = gm.graph.call_method("frontier", args=(keep,))
-        for v in valid:
-            if v.args[1:] != keep.args[1:]:
-                continue
+        for v in matching:
             for user in list(v.users):
                 if (user.op == "call_function" and user.target is operator.getitem
                         and user.args[1] in (0, 1)):
                     user.replace_all_uses_with(frontier if user.args[1] == 0 else ptr)
+    gm.graph.lint()
     return gm
 
 

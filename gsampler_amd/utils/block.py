@@ -141,12 +141,36 @@ class BlockList(Sequence):
         return block
 
     def materialize(self) -> List[Block]:
-        if self._blocks is None or any(b is None for b in self._blocks):
-            views = list(zip(*self._batch.blocks()))
-            have = self._blocks or [None] * len(views)
-            self._blocks = [b if b is not None else self._wrap(i, v)
-                            for i, (b, v) in enumerate(zip(have, views))]
-        return self._blocks
+        """Every block of the layer, from one call that cuts the layer's arrays into
+        per-batch views.  The objects are filled slot by slot (no constructor call,
+        no per-block conversions): a step hands out a few hundred of them."""
+        if self._blocks is not None and all(b is not None for b in self._blocks):
+            return self._blocks
+        rows, cols, indptrs, fronts, eids, num_src, num_dst = self._batch.blocks()
+        have = self._blocks or [None] * len(rows)
+        edata = self._edata
+        if edata and self._edge_offsets is None:
+            self._edge_offsets = self._batch.offsets()[2]
+        off = self._edge_offsets
+        new = Block.__new__
+        blocks = []
+        for i in range(len(rows)):
+            b = have[i]
+            if b is None:
+                b = new(Block)
+                b.row, b.col, b.indptr = rows[i], cols[i], indptrs[i]
+                b.num_src, b.num_dst = num_src[i], num_dst[i]
+                b.srcdata = {"_ID": fronts[i]}
+                b.dstdata = {}
+                e = eids[i]
+                b.edata = {} if e is None else {"_ID": e}
+                if edata:
+                    lo, hi = off[i], off[i + 1]
+                    for key, value in edata.items():
+                        b.edata[key] = value[lo:hi]
+            blocks.append(b)
+        self._blocks = blocks
+        return blocks
 
     def __getitem__(self, index):
         if isinstance(index, slice):

@@ -630,6 +630,31 @@ int gs_e_div_u_sum(int format, const int64_t* a, const int64_t* b,
                    int u_target, int64_t feat_len, int64_t num_out,
                    void* workspace, size_t workspace_bytes, gs_stream_t stream);
 
+/* ------------------------------------------------------------------------
+ * Yardsticks (measurement helpers, no counterpart in the reference; no
+ * operator calls them).
+ *  gs_probe_stream_copy: dst[0..bytes) = src[0..bytes), 16 bytes per lane.
+ *  gs_probe_line_gather: every lane reads 4 bytes from a 128-byte line of its
+ *    own of `table`, chosen by a hash of its number and `salt` (ordered != 0:
+ *    the same number of lines in address order); out needs num_picks / 4 + 1
+ *    32-bit words.  How many scattered lines per second the GPU delivers.
+ *  gs_probe_sample_uniform: one launch of the packed uniform sampler (int32
+ *    row ids, without replacement, fanout <= 64) with parts switched off;
+ *    variant is a sum of 1 (hash instead of Philox), 2 (no exchange among a
+ *    column's lanes), 4 (column pointer not read: every column probe_degree
+ *    long, outputs sized num_items * fanout), 8 (row ids not read), 16 (only
+ *    the row id stored), 32 (nothing stored).  Built: 0, 1, 2, 4, 8, 24, 16,
+ *    32, 40.
+ * ---------------------------------------------------------------------- */
+int gs_probe_stream_copy(const void* src, void* dst, int64_t bytes, gs_stream_t stream);
+int gs_probe_line_gather(const void* table, int64_t table_bytes, int64_t num_picks,
+                         uint64_t salt, int ordered, void* out, gs_stream_t stream);
+int gs_probe_sample_uniform(
+    const int64_t* indptr, int64_t num_cols, const int32_t* indices32,
+    const int64_t* column_ids, int64_t num_items, int64_t fanout, int variant,
+    int64_t probe_degree, uint64_t seed, uint64_t call_id, const int64_t* sub_indptr,
+    int64_t* out_coo_col, int64_t* out_indices, int64_t* out_select, gs_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

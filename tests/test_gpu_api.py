@@ -380,3 +380,60 @@ def test_block_batch_emits_edge_list_and_compressed_form(graph):
     loose = gs.utils.block.Block(listed[0].row, listed[0].col, listed[0].num_src, listed[0].num_dst)
     li, lx, _ = loose.csc()
     assert torch.equal(li, listed[0].csc()[0]) and torch.equal(lx, listed[0].csc()[1])
+
+
+def test_writes_that_go_around_torch_need_invalidate_caches():
+    """A matrix of a million edges or more keeps an int32 copy of its row ids for the uniform
+    sampler, keyed by the tensor's identity and version counter.  A write through a raw
+    pointer moves neither: the sampler goes on reading the copy until
+    _CAPI_InvalidateCaches() ages everything that was derived from tensor contents."""
+    from gsampler_amd import capi
+    nodes = 60_000
+    indptr, indices = rmat_csc(nodes, 1_500_000, seed=3)
+    indptr, indices = indptr.to(DEV), indices.to(DEV)
+    m = gs.Matrix()
+    m.load_graph("CSC", [indptr, indices])
+    seeds = torch.arange(0, 4000, device=DEV)
+
+    def sample():                                      # the fused operator reads the copy
+        gs.manual_seed(11)
+        sub, _ = m._graph._CAPI_SlicingSampling(1, seeds, 5, False, gs._CSC, gs._COO)
+        return sub._CAPI_GetCOORows().clone()
+
+    before = sample()
+    other = (indices + 1) % nodes                      # another graph on the same offsets
+    capi.probe_stream_copy(other, indices)             # raw pointers: no version bump
+    torch.cuda.synchronize()
+    assert torch.equal(indices, other)
+    stale = sample()
+    assert torch.equal(stale, before)                  # still the picks of the old ids
+    torch.ops.gs_ops._CAPI_InvalidateCaches()
+    fresh = sample()
+    assert torch.equal(fresh, (before + 1) % nodes)    # same positions, the new ids
+
+
+def test_the_int32_copy_of_the_ids_can_be_switched_off():
+    """Same picks with and without the copy; without it a matrix keeps no extra array."""
+    nodes = 60_000
+    indptr, indices = rmat_csc(nodes, 1_500_000, seed=4)
+    m = gs.Matrix()
+    m.load_graph("CSC", [indptr.to(DEV), indices.to(DEV)])
+    seeds = torch.arange(100, 3100, device=DEV)
+
+    def sample():
+        gs.manual_seed(5)
+        sub, _ = m._graph._CAPI_SlicingSampling(1, seeds, 7, False, gs._CSC, gs._COO)
+        return sub._CAPI_GetCOORows().clone()
+
+    with_copy = sample()
+    torch.cuda.synchronize()
+    base = torch.cuda.memory_allocated()
+    torch.ops.gs_ops._CAPI_SetNarrowIds(False)
+    try:
+        without = sample()
+        torch.cuda.synchronize()
+        assert torch.equal(with_copy, without)
+        # the 6 MB copy is gone (everything else the call allocated was released again)
+        assert torch.cuda.memory_allocated() <= base - 4 * 1_500_000 + (1 << 20)
+    finally:
+        torch.ops.gs_ops._CAPI_SetNarrowIds(True)

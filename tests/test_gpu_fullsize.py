@@ -120,24 +120,19 @@ def test_weighted_step_with_persistent_cdf(graph):
     same(out2, want2)
 
 
-def test_node2vec_walks(graph):
-    indptr, indices, _, _ = graph
-    indices = capi.segment_sort(indptr, indices, NODES)
-    g = torch.Generator(device=indices.device)
-    g.manual_seed(3)
-    walks, length = 200_000, 80
-    start = torch.randint(0, NODES, (walks,), generator=g, device=indices.device)
-    trace = capi.node2vec(indptr, indices, start, length, 2.0, 0.5, 7777, 0)
+def _check_walk_trace(indptr, indices, start, trace, length, steps):
+    """Properties of a walk trace that hold at any size: row 0 is the start nodes; every hop
+    follows an edge of the matrix (columns hold in-neighbours and are sorted); a walk that
+    stopped stays at -1."""
+    walks = start.numel()
     assert trace.shape == (length + 1, walks) and torch.equal(trace[0], start)
-    # every hop follows an edge of the matrix (columns hold in-neighbours); a
-    # walk that stopped stays at -1
-    for step in (1, 2, 40, 80):
+    for step in steps:
         prev, cur = trace[step - 1], trace[step]
         alive = cur >= 0
         assert bool((prev[alive] >= 0).all())
         p, c = prev[alive], cur[alive]
         lo, hi = indptr[p], indptr[p + 1]
-        # columns are sorted: lower bound of c inside [lo, hi), all walks at once
+        # lower bound of c inside [lo, hi), all walks at once
         left, right = lo.clone(), hi.clone()
         for _ in range(24):                       # degrees stay below 2^24
             active = left < right
@@ -148,9 +143,50 @@ def test_node2vec_walks(graph):
         assert bool(((left < hi) & (indices[left.clamp(max=EDGES - 1)] == c)).all())
         dead = ~alive
         assert bool((trace[step:, dead] == -1).all())
+        # a walk only stops at a node without in-neighbours
+        stopped = (prev >= 0) & dead
+        ps = prev[stopped]
+        assert bool((indptr[ps + 1] == indptr[ps]).all())
+
+
+def test_node2vec_walks(graph):
+    indptr, indices, _, _ = graph
+    indices = capi.segment_sort(indptr, indices, NODES)
+    g = torch.Generator(device=indices.device)
+    g.manual_seed(3)
+    walks, length = 200_000, 80
+    start = torch.randint(0, NODES, (walks,), generator=g, device=indices.device)
+    trace = capi.node2vec(indptr, indices, start, length, 2.0, 0.5, 7777, 0)
+    _check_walk_trace(indptr, indices, start, trace, length, (1, 2, 40, 80))
     want = orc.node2vec(indptr.cpu().numpy(), indices.cpu().numpy(), start.cpu().numpy(),
                         length, 2.0, 0.5, 7777, 0)
     assert np.array_equal(trace.cpu().numpy(), want)
+
+
+def test_node2vec_walks_at_the_configured_size(graph):
+    """1 M walks of 80 steps, p = 2, q = 0.5 (648 MB of trace), through the properties alone;
+    the first 20 000 walks also against the CPU walks bit for bit (a walk depends on its
+    position among the start nodes only, so a prefix of the launch is a launch of its own).
+    With p = 2 a step back to the previous node is accepted at both levels of the rejection
+    rule and any other neighbour at one of two: the share of steps that return is therefore
+    well above the share a first-order walk shows, which is checked as a sanity bound."""
+    indptr, indices, _, _ = graph
+    indices = capi.segment_sort(indptr, indices, NODES)
+    g = torch.Generator(device=indices.device)
+    g.manual_seed(3)
+    walks, length = 1_000_000, 80
+    start = torch.randint(0, NODES, (walks,), generator=g, device=indices.device)
+    trace = capi.node2vec(indptr, indices, start, length, 2.0, 0.5, 7777, 0)
+    _check_walk_trace(indptr, indices, start, trace, length, (1, 2, 3, 17, 40, 79, 80))
+    n = 20_000
+    want = orc.node2vec(indptr.cpu().numpy(), indices.cpu().numpy(), start[:n].cpu().numpy(),
+                        length, 2.0, 0.5, 7777, 0)
+    assert np.array_equal(trace[:, :n].cpu().numpy(), want)
+    first_order = capi.random_walk(indptr, indices, start, length, 7777, 1)
+    def returns(t):
+        back = (t[2:] == t[:-2]) & (t[2:] >= 0)
+        return float(back.sum()) / float((t[2:] >= 0).sum())
+    assert returns(trace) > 1.5 * returns(first_order)
 
 
 def test_largest_configuration_weighted_layers():
