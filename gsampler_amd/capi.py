@@ -84,15 +84,16 @@ SIGNATURES = {
     "gs_minor_slice_workspace_bytes": (_sz, [_i64, _i64]),
     "gs_minor_slice_count": (_int, [_p, _i64, _p, _i64, _p, _i64, _p, _p, _p, _sz, _p]),
     "gs_minor_slice_fill": (_int, [_p, _i64, _i64, _p, _i64, _p, _p, _p, _p, _p, _sz, _p]),
-    "gs_col_row_slice_count": (_int, [_p, _p, _p, _p, _i64, _p, _i64, _p, _i64, _p, _p, _p, _sz,
-                                      _p]),
+    "gs_col_row_slice_count": (_int, [_p, _p, _p, _p, _p, _i64, _p, _i64, _p, _i64, _p, _p, _p,
+                                      _sz, _p]),
     "gs_col_row_slice_fill": (_int, [_p, _p, _p, _i64, _p, _i64, _i64, _p, _p, _p, _p, _sz, _p]),
     "gs_probe_stream_copy": (_int, [_p, _p, _i64, _p]),
     "gs_probe_line_gather": (_int, [_p, _i64, _i64, _u64, _int, _p, _p]),
     "gs_probe_sample_uniform": (_int, [_p, _i64, _p, _p, _i64, _i64, _int, _i64, _u64, _u64, _p,
                                        _p, _p, _p, _p]),
     "gs_sliced_e_square_sum_workspace_bytes": (_sz, [_i64, _i64]),
-    "gs_sliced_e_square_sum": (_int, [_p, _p, _p, _i64, _p, _i64, _p, _p, _p, _i64, _p, _sz, _p]),
+    "gs_sliced_e_square_sum": (_int, [_p, _p, _p, _p, _i64, _p, _i64, _p, _p, _p, _i64, _p, _sz,
+                                      _p]),
     "gs_weight_cdf_workspace_bytes": (_sz, [_i64, _i64]),
     "gs_weight_cdf_build": (_int, [_p, _i64, _p, _i64, _p, _i64, _p, _p, _sz, _p]),
     "gs_csc_col_sample_weighted_fill": (_int, [_p, _i64, _p, _p, _p, _p, _i64, _i64, _int, _u64,
@@ -664,7 +665,8 @@ def minor_slice(ids, picked, indptr=None, edge_major=None, with_major=True):
     return out_indptr, out_major, out_minor, out_select
 
 
-def col_row_slice(indptr, indices, cols, rows, key_offset=None, with_major=True):
+def col_row_slice(indptr, indices, cols, rows, key_offset=None, with_major=True,
+                  indices32=None):
     """A[rows, cols] read from the parent matrix, the column slice never written.
     -> (out_indptr[len(cols) + 1], out_major | None = position of the edge's column in
     `cols`, out_minor = position of its row in `rows`, out_select = its position in the
@@ -682,7 +684,9 @@ def col_row_slice(indptr, indices, cols, rows, key_offset=None, with_major=True)
     ws = _workspace(l.gs_minor_slice_workspace_bytes(nnz, nrow), dev)
     out_indptr = torch.empty(ncol + 1, dtype=torch.int64, device=dev)
     total = torch.empty(1, dtype=torch.int64, device=dev)
-    check(l.gs_col_row_slice_count(_ptr(indptr), _ptr(indices), _ptr(cols), _ptr(key_offset),
+    check(l.gs_col_row_slice_count(_ptr(indptr), _ptr(indices),
+                                   indices32.data_ptr() if indices32 is not None else None,
+                                   _ptr(cols), _ptr(key_offset),
                                    ncol, sub_indptr.data_ptr(), nnz, _ptr(rows), nrow,
                                    out_indptr.data_ptr(), total.data_ptr(), ws.data_ptr(),
                                    ws.numel(), _stream()))
@@ -698,7 +702,7 @@ def col_row_slice(indptr, indices, cols, rows, key_offset=None, with_major=True)
 
 
 def sliced_e_square_sum(indptr, indices, cols, efeat, num_out, use_workspace=True,
-                        edge_map=None):
+                        edge_map=None, indices32=None):
     """out[row] = sum of efeat^2 over the edges of A[:, cols], read from the parent
     (edge p's value is efeat[edge_map[p]] when an edge map is given)."""
     indptr, indices = _i64t(indptr, "indptr"), _i64t(indices, "indices")
@@ -713,7 +717,9 @@ def sliced_e_square_sum(indptr, indices, cols, efeat, num_out, use_workspace=Tru
     l = lib()
     ws = _workspace(l.gs_sliced_e_square_sum_workspace_bytes(nnz, num_out) if use_workspace
                     else 0, dev)
-    check(l.gs_sliced_e_square_sum(_ptr(indptr), _ptr(indices), _ptr(cols), cols.numel(),
+    check(l.gs_sliced_e_square_sum(_ptr(indptr), _ptr(indices),
+                                   indices32.data_ptr() if indices32 is not None else None,
+                                   _ptr(cols), cols.numel(),
                                    sub_indptr.data_ptr(), nnz, _ptr(edge_map), efeat.data_ptr(),
                                    out.data_ptr(), num_out, ws.data_ptr() if ws.numel() else None,
                                    ws.numel(), _stream()))

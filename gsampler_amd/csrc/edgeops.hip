@@ -603,6 +603,22 @@ static RowRangePlan row_range_plan(int format, int64_t nnz, int64_t num_out) {
 }
 
 // counts[range * tiles + tile] = edges of the tile whose target lies in range
+// Lanes of the wavefront that hold the same value (of `bits` bits) as this one,
+// among the valid ones: one ballot per bit.  Many lanes of a wave meet at the
+// same few counters here (a tile's edges fall into a few dozen row ranges, and
+// the range that holds the hubs' rows draws most of them): the first lane of a
+// set of peers sends one atomic for all of them, where 64 single ones to the
+// same LDS word are taken one after another.  Every lane must call this.
+__device__ __forceinline__ uint64_t wave_peers(int value, int bits, bool valid) {
+  uint64_t peers = __ballot(valid);
+  for (int b = 0; b < bits; ++b) {
+    const bool bit = (value >> b) & 1;
+    const uint64_t m = __ballot(bit);
+    peers &= bit ? m : ~m;
+  }
+  return peers;
+}
+
 // With a view the edges are those of a column slice that was never written:
 // dst_ids and efeat are then the parent's arrays (see SliceView).
 __device__ __forceinline__ SliceView::Run view_run(const SliceView& view, int64_t tile0,
@@ -616,8 +632,9 @@ __device__ __forceinline__ SliceView::Run view_run(const SliceView& view, int64_
   return view.run(tile0, stop - 1);
 }
 
+template <typename IdT>
 __global__ __launch_bounds__(kPartThreads) void rowsum_hist_kernel(
-    const int64_t* __restrict__ dst_ids, int64_t nnz, int64_t num_out, int ranges,
+    const IdT* __restrict__ dst_ids, int64_t nnz, int64_t num_out, int ranges, int range_bits,
     int64_t tiles, int rounds, int64_t* __restrict__ counts, SliceView view) {
   __shared__ int hist[kMaxRanges];
   for (int j = threadIdx.x; j < ranges; j += kPartThreads) hist[j] = 0;
@@ -631,7 +648,7 @@ __global__ __launch_bounds__(kPartThreads) void rowsum_hist_kernel(
 #pragma unroll
       for (int i = 0; i < kPartItems; ++i) {
         const int64_t e = tile0 + i * kPartThreads + threadIdx.x;
-        dst[i] = e < nnz ? dst_ids[vrun.place(e)] : -1;
+        dst[i] = e < nnz ? (int64_t)dst_ids[vrun.place(e)] : -1;
       }
     } else {
 #pragma unroll
@@ -639,12 +656,17 @@ __global__ __launch_bounds__(kPartThreads) void rowsum_hist_kernel(
         const int64_t e = tile0 + i * kPartThreads + threadIdx.x;
         int64_t col, offset;  // (looked up by all lanes together, a lane past the end included)
         const int64_t p = view.position(vrun, e < nnz ? e : nnz - 1, &col, &offset);
-        dst[i] = e < nnz ? dst_ids[p] : -1;
+        dst[i] = e < nnz ? (int64_t)dst_ids[p] : -1;
       }
     }
 #pragma unroll
-    for (int i = 0; i < kPartItems; ++i)
-      if (dst[i] >= 0 && dst[i] < num_out) atomicAdd(&hist[dst[i] >> kRangeShift], 1);
+    for (int i = 0; i < kPartItems; ++i) {
+      const bool valid = dst[i] >= 0 && dst[i] < num_out;
+      const int range = valid ? (int)(dst[i] >> kRangeShift) : 0;
+      const uint64_t peers = wave_peers(range, range_bits, valid);
+      if (valid && (peers & ((1ull << lane_id()) - 1ull)) == 0)  // the first of its peers
+        atomicAdd(&hist[range], __popcll(peers));
+    }
   }
   __syncthreads();
   for (int j = threadIdx.x; j < ranges; j += kPartThreads)
@@ -657,12 +679,13 @@ __global__ __launch_bounds__(kPartThreads) void rowsum_hist_kernel(
 // sends to one range is a contiguous run, filled within a few microseconds, so
 // the 8-byte stores merge into whole lines in L2.  A pair keeps its range above
 // the row bits (the accumulate pass masks it off).
+template <typename IdT>
 __global__ __launch_bounds__(kPartThreads) void rowsum_scatter_kernel(
-    const int64_t* __restrict__ dst_ids, const int64_t* __restrict__ src_ids,
+    const IdT* __restrict__ dst_ids, const int64_t* __restrict__ src_ids,
     const int64_t* __restrict__ edge_map, int64_t nnz, int64_t num_out, int kind,
     int op, const float* __restrict__ ufeat, const float* __restrict__ efeat,
-    int ranges, int64_t tiles, int rounds, const int64_t* __restrict__ offsets,
-    uint2* __restrict__ entries, SliceView view) {
+    int ranges, int range_bits, int64_t tiles, int rounds,
+    const int64_t* __restrict__ offsets, uint2* __restrict__ entries, SliceView view) {
   __shared__ unsigned cursor[kMaxRanges];  // next free place of the tile per range
   for (int j = threadIdx.x; j < ranges; j += kPartThreads)
     cursor[j] = (unsigned)offsets[(int64_t)j * tiles + blockIdx.x];
@@ -681,7 +704,7 @@ __global__ __launch_bounds__(kPartThreads) void rowsum_scatter_kernel(
       val[i] = 0.f;
       if (e < nnz && shifted) {
         const int64_t p = vrun.place(e);
-        dst[i] = dst_ids[p];
+        dst[i] = (int64_t)dst_ids[p];
         const int64_t eid = edge_map ? edge_map[p] : p;
         val[i] = edge_value<float>(kind, op, ufeat ? ufeat + src_ids[p] : nullptr,
                                    efeat ? efeat + eid : nullptr);
@@ -694,7 +717,7 @@ __global__ __launch_bounds__(kPartThreads) void rowsum_scatter_kernel(
         int64_t col, offset;  // (looked up by all lanes together, a lane past the end included)
         const int64_t p = view.position(vrun, e < nnz ? e : nnz - 1, &col, &offset);
         if (e < nnz) {
-          dst[i] = dst_ids[p];
+          dst[i] = (int64_t)dst_ids[p];
           const int64_t eid = edge_map ? edge_map[p] : p;
           val[i] = edge_value<float>(kind, op, ufeat ? ufeat + src_ids[p] : nullptr,
                                      efeat ? efeat + eid : nullptr);
@@ -703,9 +726,16 @@ __global__ __launch_bounds__(kPartThreads) void rowsum_scatter_kernel(
     }
 #pragma unroll
     for (int i = 0; i < kPartItems; ++i) {
-      if (dst[i] < 0 || dst[i] >= num_out) continue;
-      const unsigned pos = atomicAdd(&cursor[dst[i] >> kRangeShift], 1u);
-      entries[pos] = make_uint2((unsigned)dst[i], __float_as_uint(val[i]));
+      const bool valid = dst[i] >= 0 && dst[i] < num_out;
+      const int range = valid ? (int)(dst[i] >> kRangeShift) : 0;
+      const uint64_t peers = wave_peers(range, range_bits, valid);
+      const uint64_t before = peers & ((1ull << lane_id()) - 1ull);
+      unsigned base = 0;
+      if (valid && before == 0) base = atomicAdd(&cursor[range], (unsigned)__popcll(peers));
+      // the first of the peers took places for all of them
+      base = __shfl(base, valid ? __ffsll((long long)peers) - 1 : lane_id(), kWave);
+      if (valid)
+        entries[base + __popcll(before)] = make_uint2((unsigned)dst[i], __float_as_uint(val[i]));
     }
   }
 }
@@ -787,7 +817,9 @@ __global__ __launch_bounds__(kBlock) void rowsum_fold_kernel(
   if (acc != 0.f) unsafeAtomicAdd(out + i, acc);
 }
 
-static int row_range_sum(const RowRangePlan& p, const int64_t* dst_ids,
+// dst_ids32: the same ids as dst_ids in 32 bits (a matrix's narrow copy), read
+// instead when given.
+static int row_range_sum(const RowRangePlan& p, const int64_t* dst_ids, const int32_t* dst_ids32,
                          const int64_t* src_ids, const int64_t* edge_map,
                          int64_t nnz, int64_t num_out, int kind, int op,
                          const float* ufeat, const float* efeat, float* out,
@@ -798,17 +830,30 @@ static int row_range_sum(const RowRangePlan& p, const int64_t* dst_ids,
   int64_t* unit_start = (int64_t*)(ws + p.off_unit_start);
   float* partial = (float*)(ws + p.off_partial);
   const int ranges = (int)p.ranges;
+  int range_bits = 0;
+  while ((1 << range_bits) < ranges) ++range_bits;
   const dim3 tiles_grid((unsigned)p.tiles);
-  GS_LAUNCH("rowsum_hist", s,
-            rowsum_hist_kernel<<<tiles_grid, dim3(kPartThreads), 0, s>>>(
-                dst_ids, nnz, num_out, ranges, p.tiles, p.rounds, offsets, view));
+  if (dst_ids32)
+    GS_LAUNCH("rowsum_hist", s,
+              rowsum_hist_kernel<int32_t><<<tiles_grid, dim3(kPartThreads), 0, s>>>(
+                  dst_ids32, nnz, num_out, ranges, range_bits, p.tiles, p.rounds, offsets, view));
+  else
+    GS_LAUNCH("rowsum_hist", s,
+              rowsum_hist_kernel<int64_t><<<tiles_grid, dim3(kPartThreads), 0, s>>>(
+                  dst_ids, nnz, num_out, ranges, range_bits, p.tiles, p.rounds, offsets, view));
   int rc = exclusive_scan_i64(offsets, offsets, p.ranges * p.tiles + 1,
                               ws + p.off_scan, p.scan_bytes, s);
   if (rc != GS_OK) return rc;
-  GS_LAUNCH("rowsum_scatter", s,
-            rowsum_scatter_kernel<<<tiles_grid, dim3(kPartThreads), 0, s>>>(
-                dst_ids, src_ids, edge_map, nnz, num_out, kind, op, ufeat, efeat,
-                ranges, p.tiles, p.rounds, offsets, entries, view));
+  if (dst_ids32)
+    GS_LAUNCH("rowsum_scatter", s,
+              rowsum_scatter_kernel<int32_t><<<tiles_grid, dim3(kPartThreads), 0, s>>>(
+                  dst_ids32, src_ids, edge_map, nnz, num_out, kind, op, ufeat, efeat,
+                  ranges, range_bits, p.tiles, p.rounds, offsets, entries, view));
+  else
+    GS_LAUNCH("rowsum_scatter", s,
+              rowsum_scatter_kernel<int64_t><<<tiles_grid, dim3(kPartThreads), 0, s>>>(
+                  dst_ids, src_ids, edge_map, nnz, num_out, kind, op, ufeat, efeat,
+                  ranges, range_bits, p.tiles, p.rounds, offsets, entries, view));
   GS_LAUNCH("rowsum_units", s,
             rowsum_units_kernel<<<dim3(1), dim3(kMaxRanges), 0, s>>>(
                 offsets, ranges, p.tiles, unit_start));
@@ -848,7 +893,7 @@ static int spmm_launch(int format, const int64_t* a, const int64_t* b,
     if (format == GS_FMT_COO) {
       const RowRangePlan plan = row_range_plan(format, nnz, num_out);
       if (plan.total > 0 && workspace != nullptr && workspace_bytes >= plan.total)
-        return row_range_sum(plan, u_target == 0 ? b : a, u_target == 0 ? a : b,
+        return row_range_sum(plan, u_target == 0 ? b : a, nullptr, u_target == 0 ? a : b,
                              edge_map, nnz, num_out, kind, op, ufeat, efeat, out,
                              workspace, s);
       const size_t need = private_bytes(format, nnz, num_out);
@@ -1051,7 +1096,8 @@ size_t gs_sliced_e_square_sum_workspace_bytes(int64_t slice_nnz, int64_t num_out
   return gs::row_range_plan(GS_FMT_COO, slice_nnz, num_out).total;
 }
 
-int gs_sliced_e_square_sum(const int64_t* indptr, const int64_t* indices, const int64_t* cols,
+int gs_sliced_e_square_sum(const int64_t* indptr, const int64_t* indices,
+                           const int32_t* indices32, const int64_t* cols,
                            int64_t num_cols_picked, const int64_t* sub_indptr,
                            int64_t slice_nnz, const int64_t* edge_map, const float* efeat,
                            float* out,
@@ -1067,8 +1113,8 @@ int gs_sliced_e_square_sum(const int64_t* indptr, const int64_t* indices, const 
   const SliceView view{sub_indptr, cols, indptr, nullptr, num_cols_picked};
   const RowRangePlan plan = row_range_plan(GS_FMT_COO, slice_nnz, num_out);
   if (plan.total > 0 && workspace != nullptr && workspace_bytes >= plan.total)
-    return row_range_sum(plan, indices, nullptr, edge_map, slice_nnz, num_out, 1, kOpCopyRhs,
-                         nullptr, efeat, out, workspace, s, view);
+    return row_range_sum(plan, indices, indices32, nullptr, edge_map, slice_nnz, num_out, 1,
+                         kOpCopyRhs, nullptr, efeat, out, workspace, s, view);
   // short slices: combined per tile in LDS, one atomic per (tile, row present);
   // ids outside [0, num_out) cannot occur for a slice of a checked matrix
   GS_LAUNCH("spmm_coo_sum", s,

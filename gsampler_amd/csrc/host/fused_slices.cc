@@ -84,7 +84,10 @@ void Graph::SlicedESquareSum(torch::Tensor cols, torch::Tensor efeat, torch::Ten
   torch::Tensor ws = new_workspace(gs_sliced_e_square_sum_workspace_bytes(so.nnz, num_rows_),
                                    m.indptr);
   const torch::Tensor e_ids = m.e_ids.has_value() ? m.e_ids.value() : torch::Tensor();
-  GS_CALL(gs_sliced_e_square_sum(cptr(m.indptr), cptr(m.indices), cptr(cols), cols.numel(),
+  const torch::Tensor& narrow = m.narrow_indices();  // half the bytes behind every id
+  GS_CALL(gs_sliced_e_square_sum(cptr(m.indptr), cptr(m.indices),
+                                 narrow.defined() ? narrow.data_ptr<int32_t>() : nullptr,
+                                 cptr(cols), cols.numel(),
                                  cptr(so.sub_indptr), so.nnz, cptr(e_ids),
                                  efeat.data_ptr<float>(), out.data_ptr<float>(), num_rows_,
                                  ws.data_ptr(), (size_t)ws.numel(), cur_stream()));
@@ -104,7 +107,10 @@ static MajorResult col_row_slice(const Compressed& m, const torch::Tensor& cols,
   // is queued into buffers sized by the bound (every edge kept) and runs while
   // the number travels
   AsyncCount kept = AsyncCount::mirrored();
-  GS_CALL(gs_col_row_slice_count(cptr(m.indptr), cptr(m.indices), cptr(cols), cptr(key_offset),
+  const torch::Tensor& narrow = m.narrow_indices();  // half the bytes behind every id
+  GS_CALL(gs_col_row_slice_count(cptr(m.indptr), cptr(m.indices),
+                                 narrow.defined() ? narrow.data_ptr<int32_t>() : nullptr,
+                                 cptr(cols), cptr(key_offset),
                                  n, cptr(sub_indptr), nnz, cptr(picked), np, mptr(r.indptr),
                                  kept.mirror(), ws.data_ptr(), ws.numel(), cur_stream()));
   kept.arm();

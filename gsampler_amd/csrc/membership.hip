@@ -339,9 +339,10 @@ struct BucketTable {
 
 // kThreads: work-group size.  A large one shares a staged table among more
 // edges; a small one spreads a short edge list over all compute units.
-template <bool kInLds, int kThreads>
+// IdT: int64_t, or int32_t when the ids are read from a matrix's narrow copy.
+template <bool kInLds, int kThreads, typename IdT>
 __global__ __launch_bounds__(kThreads) void member_flag_kernel(
-    const int64_t* __restrict__ ids, int64_t nnz,
+    const IdT* __restrict__ ids, int64_t nnz,
     const uint64_t* __restrict__ global_table, uint32_t cap,
     const int64_t* __restrict__ picked, const int* __restrict__ wide_flag,
     uint64_t* __restrict__ flags, int64_t* __restrict__ chunk_count,
@@ -392,10 +393,10 @@ __global__ __launch_bounds__(kThreads) void member_flag_kernel(
   // run the look-up shuffles, so all lanes go through it together
   auto id_of = [&](int64_t e) -> uint64_t {
     if (e >= nnz) e = nnz - 1;
-    if (!scattered) return (uint64_t)(ids[vrun.place(e)] + vrun.id_offset(e));
+    if (!scattered) return (uint64_t)((int64_t)ids[vrun.place(e)] + vrun.id_offset(e));
     int64_t c, offset;
     const int64_t p = view.position(vrun, e, &c, &offset);
-    return (uint64_t)(ids[p] + offset);
+    return (uint64_t)((int64_t)ids[p] + offset);
   };
   for (int part = 0; part < kMemberChunksPerWave / kMemberAhead; ++part) {
     const int64_t chunk0 = run * kMemberChunksPerWave + part * kMemberAhead;
@@ -408,7 +409,8 @@ __global__ __launch_bounds__(kThreads) void member_flag_kernel(
         for (int j = 0; j < kMemberWords; ++j) {
           const int64_t e = (chunk0 + c) * kBlock + j * kWave + lane;
           keys[c][j] =
-              e < nnz ? member_key((uint64_t)(ids[vrun.place(e)] + vrun.id_offset(e))) : kNoKey;
+              e < nnz ? member_key((uint64_t)((int64_t)ids[vrun.place(e)] + vrun.id_offset(e)))
+                      : kNoKey;
         }
     } else {
 #pragma unroll
@@ -628,7 +630,8 @@ size_t gs_minor_slice_workspace_bytes(int64_t nnz, int64_t num_picked) {
   return gs::carve_member(nullptr, nnz, num_picked).total;
 }
 
-static int minor_slice_count_impl(const int64_t* ids, int64_t nnz, const int64_t* picked,
+static int minor_slice_count_impl(const int64_t* ids, const int32_t* ids32, int64_t nnz,
+                                  const int64_t* picked,
                                   int64_t num_picked, const int64_t* indptr,
                                   int64_t num_major, int64_t* out_indptr,
                                   int64_t* out_total, void* workspace,
@@ -637,7 +640,7 @@ static int minor_slice_count_impl(const int64_t* ids, int64_t nnz, const int64_t
   using namespace gs;
   GS_REQUIRE(nnz >= 0 && num_picked >= 0 && num_major >= 0,
              "minor_slice_count: negative size");
-  GS_REQUIRE((nnz == 0 || ids) && (num_picked == 0 || picked),
+  GS_REQUIRE((nnz == 0 || ids || ids32) && (num_picked == 0 || picked),
              "minor_slice_count: null pointer");
   GS_REQUIRE((indptr == nullptr) == (out_indptr == nullptr),
              "minor_slice_count: indptr and out_indptr go together");
@@ -677,10 +680,18 @@ static int minor_slice_count_impl(const int64_t* ids, int64_t nnz, const int64_t
     if (filter && blocks > resident) blocks = resident;
     const dim3 grid((unsigned)blocks);
 #define GS_MEMBER_FLAG(LDS, THREADS)                                                          \
-  GS_LAUNCH("member_flag", s,                                                                 \
-            (member_flag_kernel<LDS, THREADS>)<<<grid, dim3(THREADS), 0, s>>>(                \
-                ids, nnz, w.table, cap, picked, w.wide, w.flags, w.chunk_off, w.staged,       \
-                filter, view))
+  do {                                                                                        \
+    if (ids32)                                                                                \
+      GS_LAUNCH("member_flag", s,                                                             \
+                (member_flag_kernel<LDS, THREADS, int32_t>)<<<grid, dim3(THREADS), 0, s>>>(   \
+                    ids32, nnz, w.table, cap, picked, w.wide, w.flags, w.chunk_off, w.staged, \
+                    filter, view));                                                           \
+    else                                                                                      \
+      GS_LAUNCH("member_flag", s,                                                             \
+                (member_flag_kernel<LDS, THREADS, int64_t>)<<<grid, dim3(THREADS), 0, s>>>(   \
+                    ids, nnz, w.table, cap, picked, w.wide, w.flags, w.chunk_off, w.staged,   \
+                    filter, view));                                                           \
+  } while (0)
     if (in_lds && small) GS_MEMBER_FLAG(true, kBlock);
     else if (in_lds) GS_MEMBER_FLAG(true, kMemberThreads);
     else if (small) GS_MEMBER_FLAG(false, kBlock);
@@ -737,8 +748,9 @@ int gs_minor_slice_count(const int64_t* ids, int64_t nnz, const int64_t* picked,
                          int64_t num_major, int64_t* out_indptr,
                          int64_t* out_total, void* workspace,
                          size_t workspace_bytes, gs_stream_t stream) {
-  return minor_slice_count_impl(ids, nnz, picked, num_picked, indptr, num_major, out_indptr,
-                                out_total, workspace, workspace_bytes, stream, gs::no_view());
+  return minor_slice_count_impl(ids, nullptr, nnz, picked, num_picked, indptr, num_major,
+                                out_indptr, out_total, workspace, workspace_bytes, stream,
+                                gs::no_view());
 }
 
 int gs_minor_slice_fill(const int64_t* ids, int64_t nnz, int64_t num_picked,
@@ -763,7 +775,8 @@ static int check_slice_view(const int64_t* indptr, const int64_t* indices, const
   return GS_OK;
 }
 
-int gs_col_row_slice_count(const int64_t* indptr, const int64_t* indices, const int64_t* cols,
+int gs_col_row_slice_count(const int64_t* indptr, const int64_t* indices,
+                           const int32_t* indices32, const int64_t* cols,
                            const int64_t* key_offset, int64_t num_cols_picked,
                            const int64_t* sub_indptr, int64_t slice_nnz,
                            const int64_t* rows, int64_t num_rows_picked,
@@ -773,7 +786,7 @@ int gs_col_row_slice_count(const int64_t* indptr, const int64_t* indices, const 
                             "col_row_slice_count");
   if (rc != GS_OK) return rc;
   const gs::SliceView view{sub_indptr, cols, indptr, key_offset, num_cols_picked};
-  return minor_slice_count_impl(indices, slice_nnz, rows, num_rows_picked, sub_indptr,
+  return minor_slice_count_impl(indices, indices32, slice_nnz, rows, num_rows_picked, sub_indptr,
                                 num_cols_picked, out_indptr, out_total, workspace,
                                 workspace_bytes, stream, view);
 }

@@ -459,6 +459,8 @@ int gs_minor_slice_fill(const int64_t* ids, int64_t nnz, int64_t num_picked,
  *    key_offset[num_cols_picked] (nullable) is added to the row ids of a column's
  *    edges before the test: the picked sets of the mini-batches of a super-batch
  *    are told apart as id + batch * stride on both sides.
+ *    indices32 (nullable): the same row ids as `indices` in 32 bits; read instead
+ *    of `indices` when given (half the bytes of the pass).
  *  fill: out_minor[kept] = position in `rows`, out_select[kept] = position of the
  *    edge in the PARENT's indices, out_major[kept] (nullable) = position of its
  *    column in `cols`.
@@ -468,7 +470,8 @@ int gs_minor_slice_fill(const int64_t* ids, int64_t nnz, int64_t num_picked,
  * 356-362; kernels :102-146, :220-264), whose select index addresses the
  * intermediate slice instead of the parent.
  * ---------------------------------------------------------------------- */
-int gs_col_row_slice_count(const int64_t* indptr, const int64_t* indices, const int64_t* cols,
+int gs_col_row_slice_count(const int64_t* indptr, const int64_t* indices,
+                           const int32_t* indices32, const int64_t* cols,
                            const int64_t* key_offset, int64_t num_cols_picked,
                            const int64_t* sub_indptr, int64_t slice_nnz,
                            const int64_t* rows, int64_t num_rows_picked,
@@ -612,14 +615,15 @@ int gs_e_square_sum(int format, const int64_t* a, const int64_t* b,
                     size_t workspace_bytes, gs_stream_t stream);
 /* out[row] += sum of e^2 over the edges of A[:, cols], read from the parent
  * matrix (the column slice is not written): cols / sub_indptr / slice_nnz as in
- * gs_col_row_slice_count, the value of the parent's edge p is efeat[edge_map[p]]
+ * gs_col_row_slice_count (indices32 likewise), the value of the parent's edge p is efeat[edge_map[p]]
  * (efeat[p] when edge_map is NULL), out[num_out] an fp32 accumulator that the
  * caller zero-fills.  The workspace is optional
  * (NULL / 0 is valid, then every edge is an atomic add).  No counterpart in the
  * reference, which writes the slice and then runs ESquareSumCOO over it
  * (src/cuda/fusion/fused_coo_e_square_sum.cu:13-60). */
 size_t gs_sliced_e_square_sum_workspace_bytes(int64_t slice_nnz, int64_t num_out);
-int gs_sliced_e_square_sum(const int64_t* indptr, const int64_t* indices, const int64_t* cols,
+int gs_sliced_e_square_sum(const int64_t* indptr, const int64_t* indices,
+                           const int32_t* indices32, const int64_t* cols,
                            int64_t num_cols_picked, const int64_t* sub_indptr,
                            int64_t slice_nnz, const int64_t* edge_map, const float* efeat,
                            float* out, int64_t num_out, void* workspace,

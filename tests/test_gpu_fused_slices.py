@@ -47,6 +47,9 @@ def test_col_row_slice_parity(ncol, nrow):
     rows = rng.integers(0, 5200, size=nrow)                 # repeats and absent ids
     want = chained_col_row_slice(indptr, indices, cols, rows)
     same(capi.col_row_slice(T(indptr), T(indices), T(cols), T(rows)), want)
+    # the row ids read from a 32-bit copy
+    same(capi.col_row_slice(T(indptr), T(indices), T(cols), T(rows),
+                            indices32=T(indices).to(torch.int32)), want)
     got = capi.col_row_slice(T(indptr), T(indices), T(cols), T(rows), with_major=False)
     assert got[1] is None
     same((got[0], got[2], got[3]), (want[0], want[2], want[3]))
@@ -80,8 +83,10 @@ def test_col_row_slice_with_per_column_key_offsets():
         key_offset = batch_of_col * stride
         picked = np.concatenate([rng.choice(3000, size=80, replace=False) + b * stride
                                  for b in range(4)])
-        same(capi.col_row_slice(T(indptr), T(indices), T(cols), T(picked), T(key_offset)),
-             chained_col_row_slice(indptr, indices, cols, picked, key_offset))
+        want = chained_col_row_slice(indptr, indices, cols, picked, key_offset)
+        same(capi.col_row_slice(T(indptr), T(indices), T(cols), T(picked), T(key_offset)), want)
+        same(capi.col_row_slice(T(indptr), T(indices), T(cols), T(picked), T(key_offset),
+                                indices32=T(indices).to(torch.int32)), want)
 
 
 @pytest.mark.parametrize("ncol,num_rows", [(0, 100), (3, 5000), (600, 5200), (512, 100_000)])
@@ -109,6 +114,11 @@ def test_sliced_e_square_sum_parity(ncol, num_rows, use_workspace):
                                    torch.as_tensor(w, device=DEV), num_rows,
                                    use_workspace=use_workspace).cpu().numpy()
     assert np.allclose(got, want, rtol=1e-5, atol=1e-30)
+    got32 = capi.sliced_e_square_sum(T(indptr), T(indices), T(cols),
+                                     torch.as_tensor(w, device=DEV), num_rows,
+                                     use_workspace=use_workspace,
+                                     indices32=T(indices).to(torch.int32)).cpu().numpy()
+    assert np.allclose(got32, want, rtol=1e-5, atol=1e-30)
     # and the CPU operator over the written slice agrees with the same sums
     cpu = orc.e_square_sum(("coo", sub_rows[ok], np.zeros(int(ok.sum()), dtype=np.int64)),
                            w[sel][ok], 2, num_rows)
