@@ -324,3 +324,73 @@ def test_ladies_layers_at_full_size_against_the_operator_chain_on_the_cpu():
         h_seeds = uniq
     assert np.array_equal(frontier.cpu().numpy(), h_seeds)
     assert blocks[1].num_edges() > 1_000_000          # the second layer really is a large one
+
+
+def _ladies_with_probabilities(A, seeds, fanouts):
+    """The same sampler, also handing out each layer's row probabilities and picked rows."""
+    ret, probs, picks = [], [], []
+    for K in fanouts:
+        subA = A[:, seeds]
+        subA.edata["p"] = subA.edata["w"] ** 2
+        prob = subA.sum("p", axis=1)
+        sampleA, select_index = subA.collective_sampling(K, prob, False)
+        sampleA = sampleA.div("w", prob[select_index], axis=1)
+        out = sampleA.sum("w", axis=0)
+        sampleA = sampleA.div("w", out, axis=0)
+        seeds = sampleA.all_nodes()
+        ret.append(sampleA.to_dgl_block(prefetch_edata={"w"}))
+        probs.append(prob)
+        picks.append(select_index)
+    return seeds, ret, probs, picks
+
+
+def test_ladies_layers_at_full_size_with_unit_interval_weights_through_the_compiled_sampler():
+    """The layer-wise configuration with its stated weights, U(0, 1], through Matrix +
+    gs.jit.compile (the column slice is read in place: no slice is written).  Sums of up to a
+    million squared weights depend on the order of addition in their last bits, so the GPU's row
+    probabilities are held to 1e-5 of float64 and then handed to the CPU pick: picked rows,
+    frontier and block structure are compared bit for bit, the normalised weights to 1e-5 of
+    the same chain in float64."""
+    import gsampler_amd as gs
+    from gsampler_amd.utils import chung_lu_csc
+    dev = torch.device("cuda:0")
+    nodes, edges, K = 233_000, 115_000_000, 512
+    indptr, indices = chung_lu_csc(nodes, edges, seed=1, device=dev)
+    g = torch.Generator(device=dev)
+    g.manual_seed(4)
+    w = 1.0 - torch.rand(edges, generator=g, device=dev, dtype=torch.float32)    # (0, 1]
+    seeds = torch.randperm(nodes, generator=g, device=dev)[:512]
+    A = gs.Matrix()
+    A.load_graph("CSC", [indptr, indices])
+    A.edata["w"] = w
+    compiled = gs.jit.compile(_ladies_with_probabilities, (A, seeds, [K, K]))
+    targets = [n.target for n in compiled.gm.graph.nodes if n.op == "call_method"]
+    assert targets.count("_CAPI_ColRowSlicing") == 2 and "_CAPI_Slicing" not in targets
+    gs.manual_seed(99)
+    frontier, blocks, probs, picks = compiled(A, seeds, [K, K])
+
+    h_indptr, h_indices, h_w = indptr.cpu().numpy(), indices.cpu().numpy(), w.cpu().numpy()
+    h_seeds = seeds.cpu().numpy()
+    for layer, blk in enumerate(blocks):
+        sub_indptr, coo_col, rows, sel = orc.col_slice(h_indptr, h_indices, h_seeds)
+        w_sub = h_w[sel]
+        exact = np.zeros(nodes)
+        np.add.at(exact, rows, w_sub.astype(np.float64) ** 2)
+        g_prob = probs[layer].cpu().numpy()
+        assert np.allclose(g_prob, exact, rtol=1e-5, atol=0)
+        picked, _ = orc.list_sample_weighted(g_prob, K, seed=99, call_id=layer)
+        assert np.array_equal(picks[layer].cpu().numpy(), picked)
+        out_indptr, major, minor, select = orc.minor_slice(rows, picked, indptr=sub_indptr)
+        uniq, _, out_row, out_col = orc.unique_relabel(h_seeds, picked[minor], edge_col=major)
+        assert blk.num_dst_nodes() == h_seeds.size and blk.num_src_nodes() == uniq.size
+        assert np.array_equal(blk.srcdata["_ID"].cpu().numpy(), uniq)
+        assert np.array_equal(blk.row.cpu().numpy(), out_row)
+        assert np.array_equal(blk.col.cpu().numpy(), out_col)
+        q = w_sub[select].astype(np.float64) / g_prob[picked].astype(np.float64)[minor]
+        col64 = np.zeros(h_seeds.size)
+        np.add.at(col64, major, q)
+        assert np.allclose(blk.edata["w"].double().cpu().numpy(), q / col64[major], rtol=1e-5,
+                           atol=0)
+        h_seeds = uniq
+    assert np.array_equal(frontier.cpu().numpy(), h_seeds)
+    assert blocks[1].num_edges() > 1_000_000
