@@ -121,7 +121,6 @@ def kernel_bytes(name, sizes):
             "sample_uniform": 32 * S + 32 * E,
             "sample_weighted_cdf": 32 * S + 32 * E,  # the same interface as the uniform sampler
             "col_count": 32 * S,                 # seeds, indptr pair, counts
-            "unique_hist": 8 * N,                # keys in
             "unique_scatter": 16 * N,            # keys in, packed entries out
             "unique_dedup": 12 * N,              # packed entries in, first positions out
             "unique_flag": 4 * N + N // 4,       # first positions in, rank words out

@@ -53,7 +53,9 @@ __device__ __forceinline__ void sample_column_generic(
   // largest idx that hit it.  The slots live in out_select until the final
   // gather.  Order-independent, so lanes take idx values strided by G.
   for (int64_t jj = lane; jj < fanout; jj += G) out_select[out_start + jj] = jj;
-  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+  // (the slots are shared among lanes of this wavefront only; a fence for the
+  // whole device would make the die write its L2 back)
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
   __builtin_amdgcn_wave_barrier();
   for (int64_t idx = fanout + lane; idx < deg; idx += G) {
     int64_t num = (int64_t)philox_bounded(key, pos, (uint64_t)idx,
@@ -61,7 +63,7 @@ __device__ __forceinline__ void sample_column_generic(
     if (num < fanout)
       atomicMax((long long*)(out_select + out_start + num), (long long)idx);
   }
-  __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "agent");
+  __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "workgroup");
   __builtin_amdgcn_wave_barrier();
   for (int64_t jj = lane; jj < fanout; jj += G) {
     int64_t p = in_start + load_coherent(out_select + out_start + jj);

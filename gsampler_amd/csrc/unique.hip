@@ -10,16 +10,19 @@
 // first partitioned by hash into buckets of about 1500 entries (streaming
 // reads and writes only), and each bucket is then deduplicated by one
 // work-group in an LDS table:
-//   plan     per-batch record (where its keys, tiles and buckets start), the
-//            batch of every tile, bucket, group of positions and tile of edges
-//            (so that a work-group finds its work with two dependent loads
-//            instead of a binary search); zero the bucket counters
-//   hist     per tile of one batch: LDS histogram over the batch's buckets,
-//            one global atomic per non-empty bin
-//   scatter  per tile: bucket offsets of the batch (a scan of its bucket counts
-//            in LDS: the bucket ranges of a batch tile its range of the flat
-//            space exactly), reserve a run in every bucket, write
-//            key << 32 | local
+//   plan     per-batch record (where its keys, tiles, buckets and bucket regions
+//            start), the batch of every tile, bucket, group of positions and
+//            tile of edges (so that a work-group finds its work with two
+//            dependent loads instead of a binary search); zero the counters
+//   scatter  per tile: order the tile by bucket in LDS, reserve a run in every
+//            bucket with one atomic on the bucket's cursor, write
+//            key << 32 | local.  A bucket owns a region of fixed capacity (as
+//            many entries as the batch has keys, at most kBucketCap, five times
+//            the average bucket), so where a run goes is known without
+//            counting the keys per bucket first: the keys are read once here,
+//            not twice.  What does not fit a region (a key that repeats more
+//            than kBucketCap times in one batch) goes to the batch's overflow
+//            list together with its bucket
 //   dedup    per bucket: LDS table with "smallest position wins" (64-bit
 //            atomicMin on the packed entry), then every entry writes the first
 //            position of its key into first[position]
@@ -36,7 +39,8 @@
 // the atomics above leave it deterministic.  A bucket with more entries than the
 // LDS table is sure to hold (a hub that repeats thousands of times, a batch too
 // large for kMaxBuckets buckets) is deduplicated by the same work-group in a
-// table in global memory that is private to the bucket.
+// table in global memory that is private to the bucket; a bucket whose region
+// ran over first collects its entries from the batch's overflow list.
 //
 // A packed entry is  low 32 bits of the key << 32 | position.  While every key
 // of a call is below 2^32 - 1 those bits are the key.  The partition pass notes
@@ -57,6 +61,8 @@ constexpr int kPartTile = kBlock * kPartItems;    // keys per partition tile
 constexpr int kMaxBuckets = 2048;                 // buckets per batch (LDS bins)
 constexpr int kLdsSlots = 4096;                   // dedup table, 32 KB of LDS
 constexpr int kLdsMaxEntries = kLdsSlots * 3 / 4; // bucket sizes the LDS table takes
+constexpr int64_t kBucketCap = 8192;              // entries a bucket's region holds at most
+static_assert(kBucketCap >= kLdsMaxEntries, "the short dedup path reads a bucket from its region alone");
 
 // Average entries per bucket and whether work-groups are laid out per die: the
 // best of a sweep on 21M keys in 64 batches (bucket sizes 512..3072, with and
@@ -90,6 +96,8 @@ struct alignas(16) BatchInfo {
   int64_t tile0;     // first partition tile
   int64_t bucket0;   // first bucket
   int64_t buckets;   // number of buckets
+  int64_t region0;   // first entry of its first bucket's region
+  int64_t cap;       // entries per bucket region: min(n, kBucketCap)
 };
 
 constexpr int kRelabelItems = 4;
@@ -113,22 +121,27 @@ struct UniqueWs {
   int64_t* flat_ptr;      // [B + 1] first flat position of a batch
   int64_t* tile_ptr;      // [B + 1] first partition tile of a batch
   int64_t* bucket_ptr;    // [B + 1] first bucket of a batch
+  int64_t* region_ptr;    // [B + 1] first region entry of a batch
   int32_t* tile_batch;    // [max_tiles] batch of a tile, -1 past the last one
   int32_t* bucket_batch;  // [max_buckets] batch of a bucket, -1 past the last one
+  int64_t* bucket_base;   // [max_buckets] first entry of a bucket's region
+  int32_t* bucket_cap;    // [max_buckets] capacity of a bucket's region
   int32_t* group_batch;   // [groups + 1] batch of the first position of a group
   int32_t* etile_batch;   // [edge tiles + 1] batch of the first edge of a tile
-  int64_t* bucket_cnt;    // [max_buckets + 1] entries per bucket
-  int64_t* bucket_cur;    // [max_buckets + 1] entries placed so far
+  int64_t* bucket_cur;    // [max_buckets + 1] entries sent to a bucket
+  int64_t* ovf_cur;       // [B + 1] entries on a batch's overflow list
+  unsigned long long* pool_cur;  // [1] entries handed out from the spill pool
   int* wide_keys;         // [1] set when some key does not fit the upper half of an entry
-  int64_t* bucket_off;    // [max_buckets + 1] first entry of a bucket
-  uint64_t* packed;       // [N] key << 32 | local, grouped by bucket
+  uint64_t* packed;       // [region_entries] key << 32 | local, one region per bucket
+  uint64_t* ovf_entry;    // [N] entries that found their region full, per batch at flat_ptr[b]
+  int32_t* ovf_bucket;    // [N] and their buckets
   uint32_t* first;        // [N] local position of the first occurrence
-  uint64_t* spill;        // [2 N + max_buckets + 1] tables of oversize buckets
+  uint64_t* spill;        // [3 N + max_buckets + 1] pool: tables of oversize buckets, collected overflow
   RankWord* words;        // [groups * kGroupWords]
   int64_t* group_cnt;     // [groups] first occurrences per group
   int64_t* group_off;     // [groups + 1] first occurrences before a group
   int64_t* unique_ptr;    // [B + 1] copy of the caller's unique_ptr for the relabel pass
-  int64_t max_tiles, max_buckets, groups, etiles;
+  int64_t max_tiles, max_buckets, groups, etiles, region_entries, pool_entries;
   size_t total;
 };
 
@@ -142,21 +155,32 @@ static UniqueWs carve_unique(void* ws, int64_t S, int64_t E, int64_t B) {
   w.max_buckets = N / tuning().bucket_keys + B;
   w.groups = ceil_div(n1, kGroup);
   w.etiles = ceil_div(E > 0 ? E : 1, kRelabelTile);
+  // A batch of n keys has ceil(n / bucket_keys) regions of min(n, kBucketCap)
+  // entries: at most n (kBucketCap / bucket_keys + 1) entries when n <= kBucketCap,
+  // at most n kBucketCap / bucket_keys + kBucketCap otherwise, and there are at
+  // most N / kBucketCap batches of the second kind.
+  w.region_entries = n1 * (kBucketCap / tuning().bucket_keys + 2) + kBucketCap;
+  w.pool_entries = 3 * n1 + w.max_buckets + 1;
   w.batch = c.take<BatchInfo>((size_t)B);
   w.flat_ptr = c.take<int64_t>((size_t)B + 1);
   w.tile_ptr = c.take<int64_t>((size_t)B + 1);
   w.bucket_ptr = c.take<int64_t>((size_t)B + 1);
+  w.region_ptr = c.take<int64_t>((size_t)B + 1);
   w.tile_batch = c.take<int32_t>((size_t)w.max_tiles);
   w.bucket_batch = c.take<int32_t>((size_t)w.max_buckets);
+  w.bucket_base = c.take<int64_t>((size_t)w.max_buckets);
+  w.bucket_cap = c.take<int32_t>((size_t)w.max_buckets);
   w.group_batch = c.take<int32_t>((size_t)w.groups + 1);
   w.etile_batch = c.take<int32_t>((size_t)w.etiles + 1);
-  w.bucket_cnt = c.take<int64_t>((size_t)w.max_buckets + 1);
   w.bucket_cur = c.take<int64_t>((size_t)w.max_buckets + 1);
+  w.ovf_cur = c.take<int64_t>((size_t)B + 1);
+  w.pool_cur = c.take<unsigned long long>(1);
   w.wide_keys = c.take<int>(1);
-  w.bucket_off = c.take<int64_t>((size_t)w.max_buckets + 1);
-  w.packed = c.take<uint64_t>((size_t)n1);
+  w.packed = c.take<uint64_t>((size_t)w.region_entries);
+  w.ovf_entry = c.take<uint64_t>((size_t)n1);
+  w.ovf_bucket = c.take<int32_t>((size_t)n1);
   w.first = c.take<uint32_t>((size_t)n1);
-  w.spill = c.take<uint64_t>((size_t)(2 * n1 + w.max_buckets + 1));
+  w.spill = c.take<uint64_t>((size_t)w.pool_entries);
   w.words = c.take<RankWord>((size_t)w.groups * kGroupWords);
   w.group_cnt = c.take<int64_t>((size_t)w.groups);
   w.group_off = c.take<int64_t>((size_t)w.groups + 1);
@@ -206,8 +230,8 @@ __device__ __forceinline__ uint32_t slot_hash(uint64_t key) {
 __device__ __forceinline__ void walk_batches(const Keys& k, int64_t bucket_keys,
                                              BatchInfo* batch, int64_t* flat_ptr,
                                              int64_t* tile_ptr, int64_t* bucket_ptr,
-                                             int64_t* smem) {
-  int64_t tile_carry = 0, bucket_carry = 0;
+                                             int64_t* region_ptr, int64_t* smem) {
+  int64_t tile_carry = 0, bucket_carry = 0, region_carry = 0;
   for (int64_t base = 0; base <= k.B; base += kBlock) {
     const int64_t b = base + threadIdx.x;
     BatchInfo info{};
@@ -223,6 +247,7 @@ __device__ __forceinline__ void walk_batches(const Keys& k, int64_t bucket_keys,
         tiles = ceil_div_dev(info.n, kPartTile);
         info.buckets = ceil_div_dev(info.n, bucket_keys);
         if (info.buckets > kMaxBuckets) info.buckets = kMaxBuckets;
+        info.cap = info.n < kBucketCap ? info.n : kBucketCap;
       }
     }
     int64_t total;
@@ -232,9 +257,13 @@ __device__ __forceinline__ void walk_batches(const Keys& k, int64_t bucket_keys,
     info.bucket0 = bucket_carry + block_exclusive_sum(info.buckets, smem, &total);
     bucket_carry += total;
     __syncthreads();
+    info.region0 = region_carry + block_exclusive_sum(info.buckets * info.cap, smem, &total);
+    region_carry += total;
+    __syncthreads();
     if (b <= k.B) {
       tile_ptr[b] = info.tile0;
       bucket_ptr[b] = info.bucket0;
+      region_ptr[b] = info.region0;
     }
     if (batch && b < k.B) batch[b] = info;
   }
@@ -246,6 +275,8 @@ __device__ __forceinline__ void walk_batches(const Keys& k, int64_t bucket_keys,
 struct UnitTables {
   int64_t max_tiles, max_buckets, groups, etiles;
   int32_t *tile_batch, *bucket_batch, *group_batch, *etile_batch;
+  int64_t* bucket_base;
+  int32_t* bucket_cap;
   __host__ __device__ int64_t units() const {
     return max_tiles + max_buckets + groups + 1 + etiles + 1;
   }
@@ -254,6 +285,7 @@ __device__ __forceinline__ void assign_unit(int64_t i, const Keys& k, int64_t N,
                                             const int64_t* flat_ptr,
                                             const int64_t* tile_ptr,
                                             const int64_t* bucket_ptr,
+                                            const int64_t* region_ptr,
                                             const UnitTables& u) {
   const int64_t B = k.B;
   if (i < u.max_tiles) {
@@ -262,7 +294,17 @@ __device__ __forceinline__ void assign_unit(int64_t i, const Keys& k, int64_t N,
   }
   i -= u.max_tiles;
   if (i < u.max_buckets) {
-    u.bucket_batch[i] = i < bucket_ptr[B] ? (int32_t)segment_of(bucket_ptr, B, i) : -1;
+    int32_t b = -1;
+    int64_t base = 0, cap = 0;
+    if (i < bucket_ptr[B]) {
+      b = (int32_t)segment_of(bucket_ptr, B, i);
+      const int64_t n = flat_ptr[b + 1] - flat_ptr[b];
+      cap = n < kBucketCap ? n : kBucketCap;
+      base = region_ptr[b] + (i - bucket_ptr[b]) * cap;
+    }
+    u.bucket_batch[i] = b;
+    u.bucket_base[i] = base;
+    u.bucket_cap[i] = (int32_t)cap;
     return;
   }
   i -= u.max_buckets;
@@ -281,14 +323,17 @@ __device__ __forceinline__ void assign_unit(int64_t i, const Keys& k, int64_t N,
   }
 }
 
-__device__ __forceinline__ void zero_counters(int64_t* bucket_cnt, int64_t* bucket_cur,
-                                              int64_t max_buckets, int* wide_keys) {
-  for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i <= max_buckets;
-       i += (int64_t)gridDim.x * kBlock) {
-    bucket_cnt[i] = 0;
-    bucket_cur[i] = 0;
+__device__ __forceinline__ void zero_counters(int64_t* bucket_cur, int64_t max_buckets,
+                                              int64_t* ovf_cur, int64_t num_batches,
+                                              unsigned long long* pool_cur, int* wide_keys) {
+  const int64_t i0 = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  const int64_t stride = (int64_t)gridDim.x * kBlock;
+  for (int64_t i = i0; i <= max_buckets; i += stride) bucket_cur[i] = 0;
+  for (int64_t i = i0; i <= num_batches; i += stride) ovf_cur[i] = 0;
+  if (blockIdx.x == 0 && threadIdx.x == 0) {
+    *wide_keys = 0;
+    *pool_cur = 0ull;
   }
-  if (blockIdx.x == 0 && threadIdx.x == 0) *wide_keys = 0;
 }
 
 // Up to kPlanMaxBatches batches: every work-group walks the batches into LDS
@@ -298,46 +343,49 @@ constexpr int kPlanMaxBatches = 1024;
 __global__ __launch_bounds__(kBlock) void unique_plan_kernel(
     Keys k, int64_t N, int64_t bucket_keys, BatchInfo* __restrict__ batch,
     int64_t* __restrict__ flat_ptr, int64_t* __restrict__ tile_ptr,
-    int64_t* __restrict__ bucket_ptr, int64_t* __restrict__ bucket_cnt,
-    int64_t* __restrict__ bucket_cur, int* __restrict__ wide_keys, UnitTables u) {
+    int64_t* __restrict__ bucket_ptr, int64_t* __restrict__ region_ptr,
+    int64_t* __restrict__ bucket_cur, int64_t* __restrict__ ovf_cur,
+    unsigned long long* __restrict__ pool_cur, int* __restrict__ wide_keys, UnitTables u) {
   __shared__ int64_t l_flat[kPlanMaxBatches + 1];
   __shared__ int64_t l_tile[kPlanMaxBatches + 1];
   __shared__ int64_t l_bucket[kPlanMaxBatches + 1];
+  __shared__ int64_t l_region[kPlanMaxBatches + 1];
   __shared__ int64_t smem[kBlock / kWave + 1];
-  zero_counters(bucket_cnt, bucket_cur, u.max_buckets, wide_keys);
+  zero_counters(bucket_cur, u.max_buckets, ovf_cur, k.B, pool_cur, wide_keys);
   walk_batches(k, bucket_keys, blockIdx.x == 0 ? batch : nullptr, l_flat, l_tile,
-               l_bucket, smem);
+               l_bucket, l_region, smem);
   __syncthreads();
   if (blockIdx.x == 0)
     for (int64_t b = threadIdx.x; b <= k.B; b += kBlock) {
       flat_ptr[b] = l_flat[b];
       tile_ptr[b] = l_tile[b];
       bucket_ptr[b] = l_bucket[b];
+      region_ptr[b] = l_region[b];
     }
   const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
-  if (i < u.units()) assign_unit(i, k, N, l_flat, l_tile, l_bucket, u);
+  if (i < u.units()) assign_unit(i, k, N, l_flat, l_tile, l_bucket, l_region, u);
 }
 
 // More batches than that: the walk by one work-group into global memory ...
 __global__ __launch_bounds__(kBlock) void unique_prep_kernel(
     Keys k, int64_t bucket_keys, BatchInfo* __restrict__ batch,
     int64_t* __restrict__ flat_ptr, int64_t* __restrict__ tile_ptr,
-    int64_t* __restrict__ bucket_ptr, int64_t* __restrict__ bucket_cnt,
-    int64_t* __restrict__ bucket_cur, int64_t max_buckets,
-    int* __restrict__ wide_keys) {
+    int64_t* __restrict__ bucket_ptr, int64_t* __restrict__ region_ptr,
+    int64_t* __restrict__ bucket_cur, int64_t max_buckets, int64_t* __restrict__ ovf_cur,
+    unsigned long long* __restrict__ pool_cur, int* __restrict__ wide_keys) {
   __shared__ int64_t smem[kBlock / kWave + 1];
-  zero_counters(bucket_cnt, bucket_cur, max_buckets, wide_keys);
+  zero_counters(bucket_cur, max_buckets, ovf_cur, k.B, pool_cur, wide_keys);
   if (blockIdx.x != 0) return;
-  walk_batches(k, bucket_keys, batch, flat_ptr, tile_ptr, bucket_ptr, smem);
+  walk_batches(k, bucket_keys, batch, flat_ptr, tile_ptr, bucket_ptr, region_ptr, smem);
 }
 
 // ... and the units from there in a launch of their own.
 __global__ __launch_bounds__(kBlock) void unique_units_kernel(
     Keys k, int64_t N, const int64_t* __restrict__ flat_ptr,
     const int64_t* __restrict__ tile_ptr, const int64_t* __restrict__ bucket_ptr,
-    UnitTables u) {
+    const int64_t* __restrict__ region_ptr, UnitTables u) {
   const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
-  if (i < u.units()) assign_unit(i, k, N, flat_ptr, tile_ptr, bucket_ptr, u);
+  if (i < u.units()) assign_unit(i, k, N, flat_ptr, tile_ptr, bucket_ptr, region_ptr, u);
 }
 
 // One partition tile: which batch, which keys.
@@ -370,54 +418,13 @@ __device__ __forceinline__ uint32_t key_tag(uint64_t key) {
   return t == 0xFFFFFFFFu ? 0xFFFFFFFEu : t;
 }
 
-// ---------------------------------------------------------------- hist
-__global__ __launch_bounds__(kBlock) void unique_hist_kernel(
-    Keys k, const int32_t* __restrict__ tile_batch,
-    const BatchInfo* __restrict__ batch, int64_t* bucket_cnt, int64_t max_tiles,
-    int remap, int* wide_keys) {
-  __shared__ uint32_t hist[kMaxBuckets];
-  const int64_t tile = unit_of_block(max_tiles, remap);
-  if (tile >= max_tiles) return;
-  TileInfo t;
-  if (!tile_info(tile, tile_batch, batch, &t)) return;  // uniform per work-group
-  const uint32_t buckets = (uint32_t)t.b.buckets;
-  if (buckets == 1 && threadIdx.x == 0)
-    atomicAdd((unsigned long long*)&bucket_cnt[t.b.bucket0],
-              (unsigned long long)(t.end - t.begin));
-  uint32_t key[kPartItems];
-  bool wide = false;
-#pragma unroll
-  for (int i = 0; i < kPartItems; ++i) {  // all loads in flight before any use
-    const int64_t l = t.begin + i * kBlock + threadIdx.x;
-    const uint64_t full = l < t.end ? key_at(k, t.b, l) : 0ull;
-    wide |= full > kMaxPackedKey;  // negative ids land here too
-    key[i] = key_tag(full);
-  }
-  if (wide) *wide_keys = 1;  // every writer stores the same value
-  if (buckets == 1) return;  // nothing to choose
-  for (uint32_t i = threadIdx.x; i < buckets; i += kBlock) hist[i] = 0;
-  __syncthreads();
-#pragma unroll
-  for (int i = 0; i < kPartItems; ++i)
-    if (t.begin + i * kBlock + threadIdx.x < t.end)
-      atomicAdd(&hist[bucket_of(key[i], buckets)], 1u);
-  __syncthreads();
-  for (uint32_t i = threadIdx.x; i < buckets; i += kBlock) {
-    const uint32_t c = hist[i];
-    if (c)
-      atomicAdd((unsigned long long*)&bucket_cnt[t.b.bucket0 + i],
-                (unsigned long long)c);
-  }
-}
-
 // ---------------------------------------------------------------- scatter
-// The buckets of a batch tile its range of the flat space in bucket order, so
-// every work-group gets the bucket offsets of its batch from a scan of the
-// batch's bucket counts in LDS (at most kMaxBuckets of them; the first tile of
-// a batch also leaves them in bucket_off for the dedup pass).  A tile that
-// brings c entries to a bucket takes the next c places at the bucket's cursor.
-// The tile is first ordered by bucket in LDS so that every run leaves as one
-// contiguous write instead of one line per entry.
+// Bucket j of a batch owns entries [region0 + j cap, region0 + (j + 1) cap) of
+// `packed`.  A tile that brings c entries to a bucket takes the next c places at
+// the bucket's cursor; places past the region's capacity are on the batch's
+// overflow list instead (the cursor still counts them, which is how the dedup
+// pass knows).  The tile is first ordered by bucket in LDS so that every run
+// leaves as one contiguous write instead of one line per entry.
 // 48 KB of LDS per work-group lets three share a compute unit: with 512 threads
 // each they fill three quarters of its wavefront slots (256 threads: 11 % slower
 // on 21 M keys; 1024, two work-groups per unit: 45 % slower).
@@ -425,12 +432,12 @@ constexpr int kScatterThreads = 512;
 constexpr int kScatterItems = kPartTile / kScatterThreads;
 __global__ __launch_bounds__(kScatterThreads) void unique_scatter_kernel(
     Keys k, const int32_t* __restrict__ tile_batch,
-    const BatchInfo* __restrict__ batch, const int64_t* __restrict__ bucket_cnt,
-    int64_t* bucket_cur, int64_t* __restrict__ bucket_off,
-    uint64_t* __restrict__ packed, uint32_t* __restrict__ first, int64_t max_tiles,
-    int remap) {
+    const BatchInfo* __restrict__ batch, int64_t* bucket_cur, int64_t* ovf_cur,
+    uint64_t* __restrict__ packed, uint64_t* __restrict__ ovf_entry,
+    int32_t* __restrict__ ovf_bucket, uint32_t* __restrict__ first, int64_t max_tiles,
+    int remap, int* wide_keys) {
   __shared__ uint32_t hist[kMaxBuckets];   // counts, then offsets inside the tile
-  __shared__ uint32_t run_at[kMaxBuckets]; // first entry of the bucket, then of the tile's run in it, relative to the batch
+  __shared__ uint32_t run_at[kMaxBuckets]; // where the tile's run starts in the bucket
   __shared__ uint64_t stage[kPartTile];
   __shared__ uint32_t scan_smem[kScatterThreads / kWave + 1];
   const int64_t tile = unit_of_block(max_tiles, remap);
@@ -438,16 +445,20 @@ __global__ __launch_bounds__(kScatterThreads) void unique_scatter_kernel(
   TileInfo t;
   if (!tile_info(tile, tile_batch, batch, &t)) return;  // uniform per work-group
   const uint32_t buckets = (uint32_t)t.b.buckets;
-  uint64_t* out = packed + t.b.fb;
-  const bool first_tile = tile == t.b.tile0;
+  uint64_t* out = packed + t.b.region0;
   if (buckets == 1) {  // the bucket is the batch, in order
-    if (first_tile && threadIdx.x == 0) bucket_off[t.b.bucket0] = t.b.fb;
+    if (tile == t.b.tile0 && threadIdx.x == 0) bucket_cur[t.b.bucket0] = t.b.n;
+    bool wide = false;
     for (int64_t l = t.begin + threadIdx.x; l < t.end; l += kScatterThreads) {
-      out[l] = ((uint64_t)key_tag(key_at(k, t.b, l)) << 32) | (uint64_t)l;
+      const uint64_t full = key_at(k, t.b, l);
+      wide |= full > kMaxPackedKey;  // negative ids land here too
+      out[l] = ((uint64_t)key_tag(full) << 32) | (uint64_t)l;
       first[t.b.fb + l] = (uint32_t)l;
     }
+    if (wide) *wide_keys = 1;  // every writer stores the same value
     return;
   }
+  uint64_t full[kScatterItems];
   uint32_t key[kScatterItems], place[kScatterItems];
 #pragma unroll
   for (int i = 0; i < kScatterItems; ++i) {
@@ -456,38 +467,26 @@ __global__ __launch_bounds__(kScatterThreads) void unique_scatter_kernel(
     // otherwise moves the first use of the key into that branch and waits
     // there, one load at a time).
     const int64_t l = t.begin + i * kScatterThreads + threadIdx.x;
-    key[i] = (uint32_t)key_at(k, t.b, l < t.end ? l : t.end - 1);
+    full[i] = key_at(k, t.b, l < t.end ? l : t.end - 1);
   }
   constexpr int kBins = kMaxBuckets / kScatterThreads;
-  {
-    const uint32_t bin0 = threadIdx.x * kBins;
-    uint32_t c[kBins], sum = 0;
 #pragma unroll
-    for (int j = 0; j < kBins; ++j) {
-      c[j] = bin0 + j < buckets ? (uint32_t)bucket_cnt[t.b.bucket0 + bin0 + j] : 0u;
-      sum += c[j];
-    }
-    uint32_t total;
-    uint32_t run = block_exclusive_sum<uint32_t, kScatterThreads>(sum, scan_smem, &total);
-#pragma unroll
-    for (int j = 0; j < kBins; ++j) {
-      if (bin0 + j < buckets) {
-        run_at[bin0 + j] = run;
-        hist[bin0 + j] = 0;
-        if (first_tile) bucket_off[t.b.bucket0 + bin0 + j] = t.b.fb + run;
-      }
-      run += c[j];
-    }
+  for (int r = 0; r < kBins; ++r) {
+    const uint32_t bin = threadIdx.x + r * kScatterThreads;
+    if (bin < buckets) hist[bin] = 0;
   }
   __syncthreads();
+  bool wide = false;
 #pragma unroll
   for (int i = 0; i < kScatterItems; ++i) {
     const int64_t l = t.begin + i * kScatterThreads + threadIdx.x;
-    key[i] = key_tag(key[i]);
+    wide |= full[i] > kMaxPackedKey;
+    key[i] = key_tag(full[i]);
     // every position starts as its own first occurrence; the dedup pass only
     // writes the positions that are not (half as many scattered stores)
     if (l < t.end) first[t.b.fb + l] = (uint32_t)l;
   }
+  if (wide) *wide_keys = 1;
 #pragma unroll
   for (int i = 0; i < kScatterItems; ++i)
     if (t.begin + i * kScatterThreads + threadIdx.x < t.end)
@@ -514,16 +513,17 @@ __global__ __launch_bounds__(kScatterThreads) void unique_scatter_kernel(
   // One bin per thread and round; all reservations are sent off before the tile
   // is ordered in LDS, and their answers (a trip to the L2 and back) are only
   // looked at after that.
-  uint32_t taken[kBins];
+  const uint32_t cap = (uint32_t)t.b.cap;
+  uint32_t taken[kBins], mine[kBins];
 #pragma unroll
   for (int r = 0; r < kBins; ++r) {
     const uint32_t bin = threadIdx.x + r * kScatterThreads;
-    taken[r] = 0;
+    taken[r] = mine[r] = 0;
     if (bin < buckets) {
-      const uint32_t c = (bin + 1 < buckets ? hist[bin + 1] : count) - hist[bin];
-      if (c)
+      mine[r] = (bin + 1 < buckets ? hist[bin + 1] : count) - hist[bin];
+      if (mine[r])
         taken[r] = (uint32_t)atomicAdd((unsigned long long*)&bucket_cur[t.b.bucket0 + bin],
-                                       (unsigned long long)c);
+                                       (unsigned long long)mine[r]);
     }
   }
 #pragma unroll
@@ -536,13 +536,29 @@ __global__ __launch_bounds__(kScatterThreads) void unique_scatter_kernel(
 #pragma unroll
   for (int r = 0; r < kBins; ++r) {
     const uint32_t bin = threadIdx.x + r * kScatterThreads;
-    if (bin < buckets) run_at[bin] += taken[r];
+    if (bin < buckets) run_at[bin] = taken[r];
   }
   __syncthreads();
   for (uint32_t j = threadIdx.x; j < count; j += kScatterThreads) {
     const uint64_t e = stage[j];
     const uint32_t bk = bucket_of(e >> 32, buckets);
-    out[run_at[bk] + (j - hist[bk])] = e;
+    const uint32_t at = run_at[bk] + (j - hist[bk]);
+    if (at < cap) out[(uint64_t)bk * cap + at] = e;
+  }
+  // The part of a run that found the region full: the thread that reserved the
+  // run moves it to the batch's overflow list.
+#pragma unroll
+  for (int r = 0; r < kBins; ++r) {
+    if (taken[r] + mine[r] <= cap) continue;
+    const uint32_t bin = threadIdx.x + r * kScatterThreads;
+    const uint32_t fits = taken[r] < cap ? cap - taken[r] : 0u;
+    const uint32_t over = mine[r] - fits;
+    const int64_t at = t.b.fb + (int64_t)atomicAdd((unsigned long long*)&ovf_cur[tile_batch[tile]],
+                                                   (unsigned long long)over);
+    for (uint32_t i = 0; i < over; ++i) {
+      ovf_entry[at + i] = stage[hist[bin] + fits + i];
+      ovf_bucket[at + i] = (int32_t)bin;
+    }
   }
 }
 
@@ -670,14 +686,28 @@ __device__ __forceinline__ void lds_insert_min_counted(uint64_t* tab,
   }
 }
 
+// The entries of a bucket: the first `fit` in its region, the rest (what the
+// region had no room for) in a run of the spill pool.
+struct BucketEntries {
+  const uint64_t* region;
+  const uint64_t* extra;
+  int64_t fit;
+  // (one load either way, so that a thread's loads of a round go out together;
+  // the run of the pool was written by this work-group a moment ago and is
+  // read past the compute unit's own cache)
+  __device__ __forceinline__ uint64_t operator[](int64_t i) const {
+    return load_l2(i < fit ? region + i : extra + (i - fit));
+  }
+};
+
 template <int kThreads, bool kWide>
 __device__ __forceinline__ void dedup_bucket(
-    const Keys& k, const BatchInfo& info, int64_t g, int64_t lo, int64_t hi,
-    const uint64_t* __restrict__ packed, uint64_t* spill, uint32_t* __restrict__ first,
-    uint64_t* tab, uint32_t* distinct_ptr, uint32_t* overflow_ptr) {
+    const Keys& k, const BatchInfo& info, int64_t n, const BucketEntries& entries,
+    uint64_t* spill, unsigned long long* pool_cur, uint32_t* __restrict__ first,
+    uint64_t* tab, uint32_t* distinct_ptr, uint32_t* overflow_ptr,
+    unsigned long long* pool_at) {
   uint32_t& distinct = *distinct_ptr;
   uint32_t& overflow = *overflow_ptr;
-  const int64_t n = hi - lo;
   const SameKey<kWide> same{&k, &info};
   uint32_t* first_b = first + info.fb;
   // table of two slots per entry, a power of two, at most kLdsSlots
@@ -693,8 +723,8 @@ __device__ __forceinline__ void dedup_bucket(
     uint64_t mine[kKeep];
 #pragma unroll
     for (int j = 0; j < kKeep; ++j) {
-      const int64_t i = lo + j * kThreads + threadIdx.x;
-      mine[j] = i < hi ? packed[i] : kEmptySlot;
+      const int64_t i = j * kThreads + threadIdx.x;
+      mine[j] = i < n ? entries[i] : kEmptySlot;
     }
 #pragma unroll
     for (int j = 0; j < kKeep; ++j)
@@ -715,12 +745,12 @@ __device__ __forceinline__ void dedup_bucket(
   // claimed after it rises to one per thread.
   constexpr int kDeep = 8;
   volatile uint32_t* over = &overflow;
-  for (int64_t base = lo; base < hi && !*over; base += (int64_t)kThreads * kDeep) {
+  for (int64_t base = 0; base < n && !*over; base += (int64_t)kThreads * kDeep) {
     uint64_t e[kDeep];
 #pragma unroll
     for (int j = 0; j < kDeep; ++j) {
       const int64_t i = base + j * kThreads + threadIdx.x;
-      e[j] = i < hi ? packed[i] : kEmptySlot;
+      e[j] = i < n ? entries[i] : kEmptySlot;
     }
 #pragma unroll
     for (int j = 0; j < kDeep; ++j)
@@ -729,12 +759,12 @@ __device__ __forceinline__ void dedup_bucket(
   }
   __syncthreads();
   if (!overflow) {
-    for (int64_t base = lo; base < hi; base += (int64_t)kThreads * kDeep) {
+    for (int64_t base = 0; base < n; base += (int64_t)kThreads * kDeep) {
       uint64_t e[kDeep];
 #pragma unroll
       for (int j = 0; j < kDeep; ++j) {
         const int64_t i = base + j * kThreads + threadIdx.x;
-        e[j] = i < hi ? packed[i] : kEmptySlot;
+        e[j] = i < n ? entries[i] : kEmptySlot;
       }
 #pragma unroll
       for (int j = 0; j < kDeep; ++j)
@@ -745,18 +775,21 @@ __device__ __forceinline__ void dedup_bucket(
     }
     return;
   }
-  // too many distinct keys: a private table in global memory, two slots per entry
-  uint64_t* gt = spill + 2 * lo + g;
+  // too many distinct keys: a table of its own from the pool, two slots per entry
   const uint64_t cap = (uint64_t)(2 * n + 1);
+  if (threadIdx.x == 0) *pool_at = atomicAdd(pool_cur, (unsigned long long)cap);
+  __syncthreads();
+  uint64_t* gt = spill + *pool_at;
+  // The table is private to this work-group: the barrier orders its stores and
+  // atomics for the work-group's own wavefronts.  (A fence for the whole device
+  // makes the die write its L2 back, tens of microseconds each time.)
   for (uint64_t i = threadIdx.x; i < cap; i += kThreads) gt[i] = kEmptySlot;
-  __threadfence();
   __syncthreads();
-  for (int64_t i = lo + threadIdx.x; i < hi; i += kThreads)
-    spill_insert_min(gt, cap, packed[i], same);
-  __threadfence();
+  for (int64_t i = threadIdx.x; i < n; i += kThreads)
+    spill_insert_min(gt, cap, entries[i], same);
   __syncthreads();
-  for (int64_t i = lo + threadIdx.x; i < hi; i += kThreads) {
-    const uint64_t e = packed[i];
+  for (int64_t i = threadIdx.x; i < n; i += kThreads) {
+    const uint64_t e = entries[i];
     const uint32_t f = spill_first_of(gt, cap, e, same);
     if (f != (uint32_t)e) first_b[(uint32_t)e] = f;
   }
@@ -776,22 +809,28 @@ template <int kThreads>
 __global__ __launch_bounds__(kThreads) void unique_dedup_kernel(
     Keys k, const int* __restrict__ wide_keys,
     const int32_t* __restrict__ bucket_batch, const BatchInfo* __restrict__ batch,
-    const int64_t* __restrict__ bucket_cnt, const int64_t* __restrict__ bucket_off,
-    const uint64_t* __restrict__ packed, uint64_t* spill, uint32_t* __restrict__ first,
-    int64_t max_buckets, int remap) {
+    const int64_t* __restrict__ bucket_cur, const int64_t* __restrict__ bucket_base,
+    const int32_t* __restrict__ bucket_cap, const int64_t* __restrict__ ovf_cur,
+    const uint64_t* __restrict__ packed, const uint64_t* __restrict__ ovf_entry,
+    const int32_t* __restrict__ ovf_bucket, uint64_t* spill, unsigned long long* pool_cur,
+    uint32_t* __restrict__ first, int64_t max_buckets, int remap) {
   __shared__ uint64_t tab[kLdsSlots];
   __shared__ uint32_t distinct;
   __shared__ uint32_t overflow;
+  __shared__ unsigned long long pool_at;
   const int64_t g = unit_of_block(max_buckets, remap);
   if (g >= max_buckets) return;
   // Everything the bucket needs to know is asked for at once, and its entries
   // right behind (two round trips to memory, not one per early exit): an unused
   // bucket has count 0, and entries are only read below that count.
   const int32_t b = bucket_batch[g];
-  const int64_t lo = bucket_off[g], n = bucket_cnt[g];
+  const int64_t lo = bucket_base[g], n = bucket_cur[g];
+  const int64_t region_cap = bucket_cap[g];
   const bool wide = *wide_keys != 0;
   constexpr int kKeep = kLdsMaxEntries / kThreads;
   uint64_t mine[kKeep];
+  // (a region holds every entry of a bucket this small: it has room for
+  // kBucketCap entries, or for as many as the batch has keys)
   const bool small = n <= kLdsMaxEntries;
 #pragma unroll
   for (int j = 0; j < kKeep; ++j) {
@@ -800,14 +839,49 @@ __global__ __launch_bounds__(kThreads) void unique_dedup_kernel(
   }
   if (b < 0 || n == 0) return;  // uniform per work-group
   const BatchInfo info = batch[b];
-  if (wide) {
-    dedup_bucket<kThreads, true>(k, info, g, lo, lo + n, packed, spill, first, tab, &distinct,
-                                 &overflow);
-    return;
-  }
-  if (!small) {
-    dedup_bucket<kThreads, false>(k, info, g, lo, lo + n, packed, spill, first, tab,
-                                  &distinct, &overflow);
+  if (wide || !small) {
+    BucketEntries entries{packed + lo, nullptr, n < region_cap ? n : region_cap};
+    if (n > region_cap) {
+      // collect what the partition pass left on the batch's overflow list
+      if (threadIdx.x == 0) {
+        pool_at = atomicAdd(pool_cur, (unsigned long long)(n - region_cap));
+        distinct = 0;
+      }
+      __syncthreads();
+      uint64_t* extra = spill + pool_at;
+      const int32_t bin = (int32_t)(g - info.bucket0);
+      const int64_t listed = ovf_cur[b];
+      // (several loads per thread in flight, one LDS atomic per wavefront)
+      constexpr int kDeep = 8;
+      for (int64_t base = 0; base < listed; base += (int64_t)kThreads * kDeep) {
+        int32_t of[kDeep];
+        uint64_t e[kDeep];
+#pragma unroll
+        for (int j = 0; j < kDeep; ++j) {
+          const int64_t i = base + j * kThreads + threadIdx.x;
+          of[j] = i < listed ? ovf_bucket[info.fb + i] : -1;
+          e[j] = ovf_entry[info.fb + (i < listed ? i : listed - 1)];
+        }
+#pragma unroll
+        for (int j = 0; j < kDeep; ++j) {
+          const bool hit = of[j] == bin;
+          const uint64_t peers = __ballot(hit);
+          if (peers == 0) continue;
+          uint32_t at = 0;
+          if (lane_id() == 0) at = atomicAdd(&distinct, (uint32_t)__popcll(peers));
+          at = __shfl(at, 0);
+          if (hit) extra[at + __popcll(peers & ((1ull << lane_id()) - 1ull))] = e[j];
+        }
+      }
+      __syncthreads();  // (read back by this work-group only: no wider fence)
+      entries.extra = extra;
+    }
+    if (wide)
+      dedup_bucket<kThreads, true>(k, info, n, entries, spill, pool_cur, first, tab,
+                                   &distinct, &overflow, &pool_at);
+    else
+      dedup_bucket<kThreads, false>(k, info, n, entries, spill, pool_cur, first, tab,
+                                    &distinct, &overflow, &pool_at);
     return;
   }
   uint32_t* tags = (uint32_t*)tab;          // [slots]
@@ -959,7 +1033,6 @@ __global__ __launch_bounds__(kOffsetsThreads) void unique_offsets_kernel(
     carry += total;
   }
   if (threadIdx.x == 0) group_off[groups] = carry;
-  __threadfence();
   __syncthreads();
   for (int64_t b = threadIdx.x; b <= B; b += kOffsetsThreads) {
     const int64_t p = flat_ptr[b];
@@ -1266,39 +1339,38 @@ int gs_unique_count(const int64_t* seeds, const int64_t* seeds_ptr,
     return GS_OK;
   }
   const Keys k{seeds, seeds_ptr, S, rows, rows_ptr, E, B};
-  const UnitTables units{w.max_tiles, w.max_buckets, w.groups,      w.etiles,
-                         w.tile_batch, w.bucket_batch, w.group_batch, w.etile_batch};
+  const UnitTables units{w.max_tiles,  w.max_buckets,  w.groups,      w.etiles,
+                         w.tile_batch, w.bucket_batch, w.group_batch, w.etile_batch,
+                         w.bucket_base, w.bucket_cap};
   const dim3 unit_grid((unsigned)ceil_div(units.units(), kBlock));
   if (B <= kPlanMaxBatches) {
     GS_LAUNCH("unique_plan", s,
               unique_plan_kernel<<<unit_grid, dim3(kBlock), 0, s>>>(
                   k, N, tn.bucket_keys, w.batch, w.flat_ptr, w.tile_ptr, w.bucket_ptr,
-                  w.bucket_cnt, w.bucket_cur, w.wide_keys, units));
+                  w.region_ptr, w.bucket_cur, w.ovf_cur, w.pool_cur, w.wide_keys, units));
   } else {
     int64_t blocks = ceil_div(w.max_buckets + 1, kBlock * 4);
     if (blocks > 1024) blocks = 1024;
     GS_LAUNCH("unique_plan", s,
               unique_prep_kernel<<<dim3((unsigned)blocks), dim3(kBlock), 0, s>>>(
-                  k, tn.bucket_keys, w.batch, w.flat_ptr, w.tile_ptr,
-                  w.bucket_ptr, w.bucket_cnt, w.bucket_cur, w.max_buckets, w.wide_keys));
+                  k, tn.bucket_keys, w.batch, w.flat_ptr, w.tile_ptr, w.bucket_ptr,
+                  w.region_ptr, w.bucket_cur, w.max_buckets, w.ovf_cur, w.pool_cur,
+                  w.wide_keys));
     GS_LAUNCH("unique_units", s,
               unique_units_kernel<<<unit_grid, dim3(kBlock), 0, s>>>(
-                  k, N, w.flat_ptr, w.tile_ptr, w.bucket_ptr, units));
+                  k, N, w.flat_ptr, w.tile_ptr, w.bucket_ptr, w.region_ptr, units));
   }
   const dim3 tile_grid((unsigned)grid_for_units(w.max_tiles, tn.remap));
-  GS_LAUNCH("unique_hist", s,
-            unique_hist_kernel<<<tile_grid, dim3(kBlock), 0, s>>>(
-                k, w.tile_batch, w.batch, w.bucket_cnt, w.max_tiles, tn.remap,
-                w.wide_keys));
   GS_LAUNCH("unique_scatter", s,
             unique_scatter_kernel<<<tile_grid, dim3(kScatterThreads), 0, s>>>(
-                k, w.tile_batch, w.batch, w.bucket_cnt, w.bucket_cur, w.bucket_off,
-                w.packed, w.first, w.max_tiles, tn.remap));
+                k, w.tile_batch, w.batch, w.bucket_cur, w.ovf_cur, w.packed, w.ovf_entry,
+                w.ovf_bucket, w.first, w.max_tiles, tn.remap, w.wide_keys));
   GS_LAUNCH("unique_dedup", s,
             unique_dedup_kernel<512><<<dim3((unsigned)grid_for_units(w.max_buckets, tn.remap)),
                                        dim3(512), 0, s>>>(
-                k, w.wide_keys, w.bucket_batch, w.batch, w.bucket_cnt, w.bucket_off, w.packed,
-                w.spill, w.first, w.max_buckets, tn.remap));
+                k, w.wide_keys, w.bucket_batch, w.batch, w.bucket_cur, w.bucket_base,
+                w.bucket_cap, w.ovf_cur, w.packed, w.ovf_entry, w.ovf_bucket, w.spill,
+                w.pool_cur, w.first, w.max_buckets, tn.remap));
   GS_LAUNCH("unique_flag", s,
             unique_flag_kernel<<<dim3((unsigned)w.groups), dim3(kBlock), 0, s>>>(
                 w.flat_ptr, w.group_batch, N, w.first, w.words, w.group_cnt));

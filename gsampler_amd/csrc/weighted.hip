@@ -223,7 +223,7 @@ __global__ __launch_bounds__(kBlock) void sample_weighted_replace_kernel(
     carry += __shfl(q, kWave - 1, kWave);
   }
   const uint64_t total = carry;
-  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
   __builtin_amdgcn_wave_barrier();
   for (int64_t j = lane; j < fanout; j += kWave) {
     const uint64_t t = total > 0 ? philox_bounded(key, (uint64_t)item, (uint64_t)j, total) : 0ull;
@@ -722,7 +722,7 @@ __global__ __launch_bounds__(kBlock) void list_replace_kernel(
     carry += __shfl(q, kWave - 1, kWave);
   }
   const uint64_t total = carry;
-  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
   __builtin_amdgcn_wave_barrier();
   const int64_t out_start = out_range[b];
   for (int64_t k = lane; k < num_picks; k += kWave) {

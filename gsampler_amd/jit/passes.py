@@ -145,8 +145,9 @@ def _merge_batch_blocks_and_all_nodes(gm: fx.GraphModule) -> fx.GraphModule:
     for node in gm.graph.nodes:
         if _is_method(node, "_CAPI_BatchGetValidNodes") or _is_method(node, "_CAPI_BatchBlocks"):
             by_graph.setdefault(node.args[0], []).append(node)
-    order = {n: i for i, n in enumerate(gm.graph.nodes)}
     for group in by_graph.values():
+        # (numbered anew for every group: the rewrite of an earlier layer added nodes)
+        order = {n: i for i, n in enumerate(gm.graph.nodes)}
         builders = [n for n in group if n.target == "_CAPI_BatchBlocks"]
         valid = [n for n in group if n.target == "_CAPI_BatchGetValidNodes"]
         if not builders or not valid:

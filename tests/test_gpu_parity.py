@@ -179,6 +179,35 @@ def test_unique_relabel_hubs_and_ragged_batches():
                 orc.unique_relabel(seeds, rows, sp, rp, edge_col))
 
 
+@pytest.mark.parametrize("B", [1, 3])
+def test_unique_relabel_buckets_beyond_their_regions(B):
+    """The partition pass gives every bucket a region of at most 8192 entries.  Ids
+    that repeat 9000 to 150000 times in one batch run over it (several buckets of
+    one batch at once), next to a million ordinary keys; a last batch is all one id."""
+    rng = np.random.default_rng(40 + B)
+    n_r = 1_200_000
+    rows = rng.integers(0, 10**6, size=n_r)
+    for hub, times in [(3, 9000), (77777, 30000), (999_999, 150000), (5, 8193), (123, 8192)]:
+        rows[rng.choice(n_r, size=times, replace=False)] = hub
+    seeds = rng.integers(0, 10**6, size=500 * B)
+    sp = rp = None
+    if B > 1:
+        rows = np.concatenate([rows, np.full(20000, 42), rng.integers(0, 300, size=100000)])
+        sp = np.arange(B + 1) * 500
+        rp = np.array([0, n_r, n_r + 20000, rows.size])
+        edge_col = np.concatenate([rng.integers(sp[b], sp[b + 1], size=rp[b + 1] - rp[b])
+                                   for b in range(B)]).astype(np.int64)
+    else:
+        edge_col = rng.integers(0, seeds.size, size=rows.size)
+    got = capi.unique_relabel(T(seeds), T(rows), T(sp) if B > 1 else None,
+                              T(rp) if B > 1 else None, T(edge_col))
+    assert_same(got, orc.unique_relabel(seeds, rows, sp, rp, edge_col))
+    if B == 1:
+        keys = np.concatenate([seeds, rows])
+        _, idx = np.unique(keys, return_index=True)
+        assert np.array_equal(N(got[0]), keys[np.sort(idx)])
+
+
 def _grouped_case(rng, counts, B, id_range):
     """Edges grouped by seed position: counts[c] edges for seed c, B batches of seeds."""
     S = counts.size

@@ -96,10 +96,12 @@ def test_batch_graphsage_rewrites():
     bm = gs.BatchMatrix()
     bm.load_from_matrix(m, False)
     c = gs.jit.compile(func=batch_graphsage_sampler,
-                       args=(bm, torch.arange(4), torch.tensor([0, 2, 4]), [5, 5]),
+                       args=(bm, torch.arange(4), torch.tensor([0, 2, 4]), [5, 5, 5]),
                        try_compact=False, format_select=False)
     t = targets(c.gm)
-    assert t.count("_CAPI_BatchFusedSlicingSampling") == 2
+    assert t.count("_CAPI_BatchFusedSlicingSampling") == 3
+    # every layer's frontier is read off its block batch
+    assert t.count("_CAPI_BatchBlocks") == 3 and "_CAPI_BatchGetValidNodes" not in t
     assert "_CAPI_BatchColSlicing" not in t and "_CAPI_BatchRowSampling" not in t
     # encoded batches are not fused (rows are renumbered between the two steps)
     bm2 = gs.BatchMatrix()
