@@ -126,6 +126,8 @@ def kernel_bytes(name, sizes):
             "unique_flag": 4 * N + N // 4,       # first positions in, rank words out
             "unique_fill": N // 4 + 16 * U,      # rank words + first keys in, frontier out
             "unique_relabel": 20 * E + 8 * S,    # first position + column pointer in, row + col out
+            # frontier and labels from one launch: the two lines above together
+            "unique_fill_relabel": N // 4 + 16 * U + 20 * E + 8 * S,
         }.get(name, 0)
     return total
 

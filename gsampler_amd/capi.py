@@ -59,6 +59,8 @@ SIGNATURES = {
     "gs_unique_fill": (_int, [_p, _p, _i64, _p, _p, _i64, _i64, _p, _p, _p, _sz, _p]),
     "gs_unique_relabel": (_int, [_p, _p, _i64, _p, _p, _i64, _i64, _p, _p, _p, _p, _p,
                                  _sz, _p]),
+    "gs_unique_fill_relabel": (_int, [_p, _p, _i64, _p, _p, _i64, _i64, _p, _p, _p, _p, _p, _p,
+                                      _p, _sz, _p]),
     "gs_csc2coo": (_int, [_p, _i64, _i64, _p, _p]),
     "gs_sorted_to_indptr": (_int, [_p, _i64, _i64, _p, _p]),
     "gs_decode_batch_ids": (_int, [_p, _i64, _i64, _p, _p, _p]),
@@ -360,11 +362,13 @@ def sample_uniform(indptr, indices, column_ids, fanout, replace=False,
 
 
 def unique_relabel(seeds, rows, seeds_ptr=None, rows_ptr=None, edge_col=None,
-                   want_row=True, want_col=True, col_indptr=None):
+                   want_row=True, want_col=True, col_indptr=None, fused=True):
     """First-occurrence unique of seeds_b ++ rows_b per batch, plus relabel.
 
     The column of an edge comes from `edge_col` (a position into `seeds` per
     edge) or, for edges grouped by column, from `col_indptr` (len(seeds) + 1).
+    `fused`: frontier and labels from one launch (gs_unique_fill_relabel) instead
+    of gs_unique_fill followed by gs_unique_relabel; same outputs.
 
     -> (unique, unique_ptr, out_row | None, out_col | None)
     """
@@ -400,13 +404,19 @@ def unique_relabel(seeds, rows, seeds_ptr=None, rows_ptr=None, edge_col=None,
         if col_indptr.numel() != S + 1:
             raise ValueError(f"unique_relabel: col_indptr has {col_indptr.numel()} entries "
                              f"for {S} seeds")
-    check(l.gs_unique_fill(_ptr(seeds), sp, S, _ptr(rows), rp, E, B,
-                           unique_ptr.data_ptr(), _ptr(unique), ws.data_ptr(),
-                           ws.numel(), _stream()))
-    if want_row or want_col:
-        check(l.gs_unique_relabel(_ptr(seeds), sp, S, _ptr(rows), rp, E, B,
-                                  _ptr(edge_col), _ptr(col_indptr), _ptr(out_row),
-                                  _ptr(out_col), ws.data_ptr(), ws.numel(), _stream()))
+    if (want_row or want_col) and fused:
+        check(l.gs_unique_fill_relabel(_ptr(seeds), sp, S, _ptr(rows), rp, E, B,
+                                       unique_ptr.data_ptr(), _ptr(unique), _ptr(edge_col),
+                                       _ptr(col_indptr), _ptr(out_row), _ptr(out_col),
+                                       ws.data_ptr(), ws.numel(), _stream()))
+    else:
+        check(l.gs_unique_fill(_ptr(seeds), sp, S, _ptr(rows), rp, E, B,
+                               unique_ptr.data_ptr(), _ptr(unique), ws.data_ptr(),
+                               ws.numel(), _stream()))
+        if want_row or want_col:
+            check(l.gs_unique_relabel(_ptr(seeds), sp, S, _ptr(rows), rp, E, B,
+                                      _ptr(edge_col), _ptr(col_indptr), _ptr(out_row),
+                                      _ptr(out_col), ws.data_ptr(), ws.numel(), _stream()))
     total = count.get()
     return unique[:total], unique_ptr, out_row, out_col
 

@@ -202,17 +202,19 @@ Graph::Frontier& Graph::batch_relabel_launch(torch::Tensor& col_seeds,
                 "BatchGraphRelabel: ", col_seeds.numel(), " seeds for a matrix of ",
                 edges.col_indptr.numel() - 1, " columns");
   torch::Tensor rows = batch_rows_for_relabel(edges.row, row_ids);
-  Frontier& f = frontier_for(col_seeds, rows, col_bptr_, edge_bptr_);
-  const int64_t E = rows.numel(), B = f.num_batches;
+  const int64_t E = rows.numel();
   *out_row = new_ids(E, rows);
   *out_col = new_ids(E, rows);
-  GS_CALL(gs_unique_relabel(cptr(col_seeds), cptr(col_bptr_), col_seeds.numel(),
-                            cptr(rows), cptr(edge_bptr_), E, B,
-                            edges.col.defined() ? cptr(edges.col) : nullptr,
-                            edges.col_indptr.defined() ? cptr(edges.col_indptr) : nullptr,
-                            mptr(*out_row), mptr(*out_col),
-                            f.workspace.data_ptr(), f.workspace.numel(),
-                            cur_stream()));
+  LabelRequest labels{edges.col.defined() ? cptr(edges.col) : nullptr,
+                      edges.col_indptr.defined() ? cptr(edges.col_indptr) : nullptr,
+                      mptr(*out_row), mptr(*out_col)};
+  Frontier& f = frontier_for(col_seeds, rows, col_bptr_, edge_bptr_, &labels);
+  if (!labels.done)
+    GS_CALL(gs_unique_relabel(cptr(col_seeds), cptr(col_bptr_), col_seeds.numel(),
+                              cptr(rows), cptr(edge_bptr_), E, f.num_batches,
+                              labels.edge_col, labels.col_indptr, labels.out_row,
+                              labels.out_col, f.workspace.data_ptr(), f.workspace.numel(),
+                              cur_stream()));
   if (e_ids) *e_ids = edges.e_ids;
   return f;
 }

@@ -468,7 +468,8 @@ bool Graph::Frontier::matches(const torch::Tensor& s, const torch::Tensor& r,
 Graph::Frontier& Graph::frontier_for(const torch::Tensor& seeds,
                                      const torch::Tensor& rows,
                                      const torch::Tensor& seeds_ptr,
-                                     const torch::Tensor& rows_ptr) {
+                                     const torch::Tensor& rows_ptr,
+                                     LabelRequest* labels) {
   if (frontier_ && frontier_->matches(seeds, rows, seeds_ptr, rows_ptr))
     return *frontier_;
   auto f = std::make_unique<Frontier>();
@@ -498,10 +499,20 @@ Graph::Frontier& Graph::frontier_for(const torch::Tensor& seeds,
   // at most S + E unique keys
   f->unique_buffer =
       new_ids(S + E <= kBoundLimit ? S + E : f->total(), rows);
-  GS_CALL(gs_unique_fill(cptr(seeds), cptr(seeds_ptr), S, cptr(rows),
-                         cptr(rows_ptr), E, B, cptr(f->unique_ptr),
-                         mptr(f->unique_buffer), f->workspace.data_ptr(),
-                         f->workspace.numel(), cur_stream()));
+  if (labels) {
+    GS_CALL(gs_unique_fill_relabel(cptr(seeds), cptr(seeds_ptr), S, cptr(rows),
+                                   cptr(rows_ptr), E, B, cptr(f->unique_ptr),
+                                   mptr(f->unique_buffer), labels->edge_col,
+                                   labels->col_indptr, labels->out_row, labels->out_col,
+                                   f->workspace.data_ptr(), f->workspace.numel(),
+                                   cur_stream()));
+    labels->done = true;
+  } else {
+    GS_CALL(gs_unique_fill(cptr(seeds), cptr(seeds_ptr), S, cptr(rows),
+                           cptr(rows_ptr), E, B, cptr(f->unique_ptr),
+                           mptr(f->unique_buffer), f->workspace.data_ptr(),
+                           f->workspace.numel(), cur_stream()));
+  }
   frontier_ = std::move(f);
   return *frontier_;
 }
@@ -606,14 +617,16 @@ Graph::GraphRelabel(torch::Tensor col_seeds, torch::Tensor row_ids) {
     return {l.frontier(), out_row, out_col, coo_->e_ids};
   }
   torch::Tensor rows = mapped_rows(coo_->row, row_ids);
-  Frontier& f = frontier_for(col_seeds, rows, {}, {});
   const int64_t E = rows.numel();
   torch::Tensor out_row = new_ids(E, rows), out_col = new_ids(E, rows);
-  GS_CALL(gs_unique_relabel(cptr(col_seeds), nullptr, col_seeds.numel(),
-                            cptr(rows), nullptr, E, 1, cptr(coo_->col), nullptr,
-                            mptr(out_row), mptr(out_col),
-                            f.workspace.data_ptr(), f.workspace.numel(),
-                            cur_stream()));
+  LabelRequest labels{cptr(coo_->col), nullptr, mptr(out_row), mptr(out_col)};
+  Frontier& f = frontier_for(col_seeds, rows, {}, {}, &labels);
+  if (!labels.done)
+    GS_CALL(gs_unique_relabel(cptr(col_seeds), nullptr, col_seeds.numel(),
+                              cptr(rows), nullptr, E, 1, cptr(coo_->col), nullptr,
+                              mptr(out_row), mptr(out_col),
+                              f.workspace.data_ptr(), f.workspace.numel(),
+                              cur_stream()));
   return {f.frontier(), out_row, out_col, coo_->e_ids};
 }
 

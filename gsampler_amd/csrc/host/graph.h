@@ -273,9 +273,19 @@ class Graph : public torch::CustomClassHolder {
    private:
     torch::Tensor unique_;
   };
+  // Labels wanted together with a frontier: when the frontier has to be built,
+  // both come from one launch and `done` is set; a frontier that is already there
+  // leaves `done` false and the caller labels on its own.
+  struct LabelRequest {
+    const int64_t* edge_col = nullptr;
+    const int64_t* col_indptr = nullptr;
+    int64_t* out_row = nullptr;
+    int64_t* out_col = nullptr;
+    bool done = false;
+  };
   Frontier& frontier_for(const torch::Tensor& seeds, const torch::Tensor& rows,
                          const torch::Tensor& seeds_ptr,
-                         const torch::Tensor& rows_ptr);
+                         const torch::Tensor& rows_ptr, LabelRequest* labels = nullptr);
   Frontier& batch_relabel_launch(torch::Tensor& col_seeds, const torch::Tensor& row_ids,
                                  torch::Tensor* out_row, torch::Tensor* out_col,
                                  c10::optional<torch::Tensor>* e_ids);

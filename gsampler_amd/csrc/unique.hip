@@ -1056,12 +1056,18 @@ __global__ __launch_bounds__(kOffsetsThreads) void unique_offsets_kernel(
 // the keys of its kWordsPerWave rows of 64 positions in one go (whole rows:
 // about half of the positions are first occurrences, so every line is needed
 // anyway) and then stores the flagged ones.
-__global__ __launch_bounds__(kBlock) void unique_fill_kernel(
-    Keys k, const int64_t* __restrict__ flat_ptr,
+struct FillArgs {
+  const int64_t* flat_ptr;
+  const int32_t* group_batch;
+  int64_t N;
+  int64_t* out_unique;
+};
+
+__device__ __forceinline__ void fill_group(
+    int64_t group, const Keys& k, const int64_t* __restrict__ flat_ptr,
     const int32_t* __restrict__ group_batch, const BatchInfo* __restrict__ batch,
     int64_t N, const RankWord* __restrict__ words,
     const int64_t* __restrict__ group_off, int64_t* __restrict__ out_unique) {
-  const int64_t group = blockIdx.x;
   const int wave = threadIdx.x / kWave, lane = lane_id();
   const int64_t word0 = group * kGroupWords + wave * kWordsPerWave;
   if (wave_uniform(word0 * kWave) >= N) return;
@@ -1088,6 +1094,13 @@ __global__ __launch_bounds__(kBlock) void unique_fill_kernel(
     if ((bits >> lane) & 1ull)
       out[before + __popcll(bits & ((1ull << lane) - 1ull))] = (int64_t)key[j];
   }
+}
+
+__global__ __launch_bounds__(kBlock) void unique_fill_kernel(
+    Keys k, FillArgs f, const BatchInfo* __restrict__ batch,
+    const RankWord* __restrict__ words, const int64_t* __restrict__ group_off) {
+  fill_group(blockIdx.x, k, f.flat_ptr, f.group_batch, batch, f.N, words, group_off,
+             f.out_unique);
 }
 
 // ---------------------------------------------------------------- relabel
@@ -1172,9 +1185,20 @@ __device__ __forceinline__ int64_t tile_columns(const int64_t* __restrict__ col_
 
 // kByIndptr: the edges are grouped by column and col_indptr (k.S + 1 entries)
 // says where each column's edges start; edge_col is not read.
+struct LabelArgs {
+  const int32_t* etile_batch;
+  const uint32_t* first;
+  const int64_t* unique_ptr;
+  const int64_t* edge_col;
+  const int64_t* col_indptr;
+  int64_t* out_row;
+  int64_t* out_col;
+  int remap;
+};
+
 template <bool kByIndptr>
-__global__ __launch_bounds__(kBlock) void unique_relabel_kernel(
-    Keys k, const int32_t* __restrict__ etile_batch,
+__device__ __forceinline__ void relabel_tile(
+    const Keys& k, const int32_t* __restrict__ etile_batch,
     const BatchInfo* __restrict__ batch, const uint32_t* __restrict__ first,
     const RankWord* __restrict__ words, const int64_t* __restrict__ group_off,
     const int64_t* __restrict__ unique_ptr, const int64_t* __restrict__ edge_col,
@@ -1268,6 +1292,31 @@ __global__ __launch_bounds__(kBlock) void unique_relabel_kernel(
         }
     }
   }
+}
+
+template <bool kByIndptr>
+__global__ __launch_bounds__(kBlock) void unique_relabel_kernel(
+    Keys k, LabelArgs l, const BatchInfo* __restrict__ batch,
+    const RankWord* __restrict__ words, const int64_t* __restrict__ group_off) {
+  relabel_tile<kByIndptr>(k, l.etile_batch, batch, l.first, words, group_off, l.unique_ptr,
+                          l.edge_col, l.col_indptr, l.out_row, l.out_col, l.remap);
+}
+
+// Both of the above in one launch: the first `label_blocks` work-groups label
+// tiles of edges, the rest write the frontier.  Neither reads what the other
+// writes; the short frontier work-groups fill the machine while the last
+// labelling ones drain.
+template <bool kByIndptr>
+__global__ __launch_bounds__(kBlock) void unique_fill_relabel_kernel(
+    Keys k, FillArgs f, LabelArgs l, unsigned label_blocks,
+    const BatchInfo* __restrict__ batch, const RankWord* __restrict__ words,
+    const int64_t* __restrict__ group_off) {
+  if (blockIdx.x < label_blocks)
+    relabel_tile<kByIndptr>(k, l.etile_batch, batch, l.first, words, group_off, l.unique_ptr,
+                            l.edge_col, l.col_indptr, l.out_row, l.out_col, l.remap);
+  else
+    fill_group(blockIdx.x - label_blocks, k, f.flat_ptr, f.group_batch, batch, f.N, words,
+               group_off, f.out_unique);
 }
 
 // No keys at all: every batch is empty.
@@ -1381,6 +1430,48 @@ int gs_unique_count(const int64_t* seeds, const int64_t* seeds_ptr,
   return GS_OK;
 }
 
+// The launches behind gs_unique_fill, gs_unique_relabel and gs_unique_fill_relabel.
+static int launch_fill_relabel(const gs::Keys& k, const gs::UniqueWs& w, int64_t* out_unique,
+                               const int64_t* edge_col, const int64_t* col_indptr,
+                               int64_t* out_row, int64_t* out_col, hipStream_t s) {
+  using namespace gs;
+  const UniqueTuning tn = tuning();
+  const int64_t N = k.S + k.E;
+  const bool fill = out_unique != nullptr && N > 0;
+  const bool label = k.E > 0 && (out_row || out_col);
+  const bool by_indptr = out_col && col_indptr;
+  const FillArgs f{w.flat_ptr, w.group_batch, N, out_unique};
+  const LabelArgs l{w.etile_batch, w.first, w.unique_ptr, by_indptr ? nullptr : edge_col,
+                    by_indptr ? col_indptr : nullptr, out_row, out_col, tn.remap};
+  const unsigned label_blocks =
+      label ? (unsigned)grid_for_units(ceil_div(k.E, kRelabelTile), tn.remap) : 0u;
+  if (fill && label) {
+    const dim3 grid(label_blocks + (unsigned)w.groups);
+    if (by_indptr)
+      GS_LAUNCH("unique_fill_relabel", s,
+                unique_fill_relabel_kernel<true><<<grid, dim3(kBlock), 0, s>>>(
+                    k, f, l, label_blocks, w.batch, w.words, w.group_off));
+    else
+      GS_LAUNCH("unique_fill_relabel", s,
+                unique_fill_relabel_kernel<false><<<grid, dim3(kBlock), 0, s>>>(
+                    k, f, l, label_blocks, w.batch, w.words, w.group_off));
+  } else if (fill) {
+    GS_LAUNCH("unique_fill", s,
+              unique_fill_kernel<<<dim3((unsigned)w.groups), dim3(kBlock), 0, s>>>(
+                  k, f, w.batch, w.words, w.group_off));
+  } else if (label) {
+    if (by_indptr)
+      GS_LAUNCH("unique_relabel", s,
+                unique_relabel_kernel<true><<<dim3(label_blocks), dim3(kBlock), 0, s>>>(
+                    k, l, w.batch, w.words, w.group_off));
+    else
+      GS_LAUNCH("unique_relabel", s,
+                unique_relabel_kernel<false><<<dim3(label_blocks), dim3(kBlock), 0, s>>>(
+                    k, l, w.batch, w.words, w.group_off));
+  }
+  return GS_OK;
+}
+
 int gs_unique_fill(const int64_t* seeds, const int64_t* seeds_ptr,
                    int64_t num_seeds, const int64_t* rows,
                    const int64_t* rows_ptr, int64_t num_rows_keys,
@@ -1394,15 +1485,19 @@ int gs_unique_fill(const int64_t* seeds, const int64_t* seeds_ptr,
   GS_REQUIRE(unique_ptr, "unique_fill: null unique_ptr");
   UniqueWs w = carve_unique(workspace, S, E, B);
   if ((rc = check_workspace(w, workspace, workspace_bytes)) != GS_OK) return rc;
-  const int64_t N = S + E;
-  if (N == 0) return GS_OK;
+  if (S + E == 0) return GS_OK;
   GS_REQUIRE(out_unique, "unique_fill: null out_unique");
-  hipStream_t s = as_stream(stream);
   const Keys k{seeds, seeds_ptr, S, rows, rows_ptr, E, B};
-  GS_LAUNCH("unique_fill", s,
-            unique_fill_kernel<<<dim3((unsigned)w.groups), dim3(kBlock), 0, s>>>(
-                k, w.flat_ptr, w.group_batch, w.batch, N, w.words, w.group_off,
-                out_unique));
+  return launch_fill_relabel(k, w, out_unique, nullptr, nullptr, nullptr, nullptr,
+                             as_stream(stream));
+}
+
+static int check_label_args(int64_t S, int64_t E, const int64_t* edge_col,
+                            const int64_t* col_indptr, const int64_t* out_col) {
+  GS_REQUIRE(out_col == nullptr || E == 0 || (edge_col != nullptr) != (col_indptr != nullptr),
+             "unique_relabel: out_col needs edge_col or col_indptr (one of them)");
+  GS_REQUIRE(col_indptr == nullptr || E == 0 || S > 0,
+             "unique_relabel: %lld edges grouped by column but no seeds", (long long)E);
   return GS_OK;
 }
 
@@ -1416,30 +1511,33 @@ int gs_unique_relabel(const int64_t* seeds, const int64_t* seeds_ptr,
   const int64_t S = num_seeds, E = num_rows_keys, B = num_batches;
   int rc = check_unique_args(seeds, seeds_ptr, S, rows, rows_ptr, E, B);
   if (rc != GS_OK) return rc;
-  GS_REQUIRE(out_col == nullptr || E == 0 || (edge_col != nullptr) != (col_indptr != nullptr),
-             "unique_relabel: out_col needs edge_col or col_indptr (one of them)");
-  GS_REQUIRE(col_indptr == nullptr || E == 0 || S > 0,
-             "unique_relabel: %lld edges grouped by column but no seeds", (long long)E);
+  if ((rc = check_label_args(S, E, edge_col, col_indptr, out_col)) != GS_OK) return rc;
   UniqueWs w = carve_unique(workspace, S, E, B);
   if ((rc = check_workspace(w, workspace, workspace_bytes)) != GS_OK) return rc;
-  hipStream_t s = as_stream(stream);
-  const UniqueTuning tn = tuning();
-  if (E > 0 && (out_row || out_col)) {
-    const Keys k{seeds, seeds_ptr, S, rows, rows_ptr, E, B};
-    const dim3 grid((unsigned)grid_for_units(ceil_div(E, kRelabelTile), tn.remap));
-    if (out_col && col_indptr) {
-      GS_LAUNCH("unique_relabel", s,
-                unique_relabel_kernel<true><<<grid, dim3(kBlock), 0, s>>>(
-                    k, w.etile_batch, w.batch, w.first, w.words, w.group_off, w.unique_ptr,
-                    nullptr, col_indptr, out_row, out_col, tn.remap));
-    } else {
-      GS_LAUNCH("unique_relabel", s,
-                unique_relabel_kernel<false><<<grid, dim3(kBlock), 0, s>>>(
-                    k, w.etile_batch, w.batch, w.first, w.words, w.group_off, w.unique_ptr,
-                    edge_col, nullptr, out_row, out_col, tn.remap));
-    }
-  }
-  return GS_OK;
+  const Keys k{seeds, seeds_ptr, S, rows, rows_ptr, E, B};
+  return launch_fill_relabel(k, w, nullptr, edge_col, col_indptr, out_row, out_col,
+                             as_stream(stream));
+}
+
+int gs_unique_fill_relabel(const int64_t* seeds, const int64_t* seeds_ptr,
+                           int64_t num_seeds, const int64_t* rows,
+                           const int64_t* rows_ptr, int64_t num_rows_keys,
+                           int64_t num_batches, const int64_t* unique_ptr,
+                           int64_t* out_unique, const int64_t* edge_col,
+                           const int64_t* col_indptr, int64_t* out_row, int64_t* out_col,
+                           void* workspace, size_t workspace_bytes, gs_stream_t stream) {
+  using namespace gs;
+  const int64_t S = num_seeds, E = num_rows_keys, B = num_batches;
+  int rc = check_unique_args(seeds, seeds_ptr, S, rows, rows_ptr, E, B);
+  if (rc != GS_OK) return rc;
+  GS_REQUIRE(unique_ptr, "unique_fill_relabel: null unique_ptr");
+  if ((rc = check_label_args(S, E, edge_col, col_indptr, out_col)) != GS_OK) return rc;
+  UniqueWs w = carve_unique(workspace, S, E, B);
+  if ((rc = check_workspace(w, workspace, workspace_bytes)) != GS_OK) return rc;
+  GS_REQUIRE(S + E == 0 || out_unique, "unique_fill_relabel: null out_unique");
+  const Keys k{seeds, seeds_ptr, S, rows, rows_ptr, E, B};
+  return launch_fill_relabel(k, w, out_unique, edge_col, col_indptr, out_row, out_col,
+                             as_stream(stream));
 }
 
 }  // extern "C"

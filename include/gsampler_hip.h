@@ -324,6 +324,10 @@ int gs_list_sample_weighted_fill(const float* probs, const int64_t* range,
  *   src/cuda/batch/batch_relabel.cu:480-498 takes coo_col).  Give one of the
  *   two, the other NULL.  May be called any number of times while the
  *   workspace is kept.
+ * fill_relabel: fill and relabel in one launch (the two read the same state and
+ *   write different outputs), for the caller that wants both at once, as
+ *   BatchGraphRelabel does (src/cuda/batch/batch_relabel.cu:480-498 returns the
+ *   frontier and both label arrays from one call).
  * Keys are any int64 values; one call takes at most 2^31 - 1 keys.  While all
  * keys of a call lie in [0, 2^32 - 2] a packed table entry holds the key itself;
  * when one does not (ids of a very large graph, ids encoded as id + batch *
@@ -354,6 +358,13 @@ int gs_unique_relabel(const int64_t* seeds, const int64_t* seeds_ptr,
                       int64_t num_batches, const int64_t* edge_col,
                       const int64_t* col_indptr, int64_t* out_row, int64_t* out_col,
                       void* workspace, size_t workspace_bytes, gs_stream_t stream);
+int gs_unique_fill_relabel(const int64_t* seeds, const int64_t* seeds_ptr,
+                           int64_t num_seeds, const int64_t* rows,
+                           const int64_t* rows_ptr, int64_t num_rows_keys,
+                           int64_t num_batches, const int64_t* unique_ptr,
+                           int64_t* out_unique, const int64_t* edge_col,
+                           const int64_t* col_indptr, int64_t* out_row, int64_t* out_col,
+                           void* workspace, size_t workspace_bytes, gs_stream_t stream);
 
 /* ------------------------------------------------------------------------
  * out_first[r] = smallest position e with ids[e] == r, INT64_MAX when r does

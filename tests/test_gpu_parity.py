@@ -208,6 +208,25 @@ def test_unique_relabel_buckets_beyond_their_regions(B):
         assert np.array_equal(N(got[0]), keys[np.sort(idx)])
 
 
+@pytest.mark.parametrize("by_pointer", [False, True])
+def test_unique_frontier_and_labels_from_one_launch(by_pointer):
+    """gs_unique_fill_relabel writes what gs_unique_fill and gs_unique_relabel write."""
+    rng = np.random.default_rng(77)
+    counts = rng.integers(0, 9, size=30000)
+    seeds, rows, sp, rp, edge_col, col_indptr = _grouped_case(rng, counts, 16, 10**5)
+    how = dict(col_indptr=T(col_indptr)) if by_pointer else dict(edge_col=T(edge_col))
+    one = capi.unique_relabel(T(seeds), T(rows), T(sp), T(rp), fused=True, **how)
+    two = capi.unique_relabel(T(seeds), T(rows), T(sp), T(rp), fused=False, **how)
+    assert_same(one, tuple(None if x is None else N(x) for x in two))
+    assert_same(one, orc.unique_relabel(seeds, rows, sp, rp, edge_col))
+    # rows only / no edges at all
+    one = capi.unique_relabel(T(seeds), T(rows), T(sp), T(rp), want_col=False, fused=True)
+    assert_same(one, orc.unique_relabel(seeds, rows, sp, rp))
+    e = np.empty(0, dtype=np.int64)
+    assert_same(capi.unique_relabel(T(seeds[:50]), T(e), edge_col=T(e), fused=True),
+                orc.unique_relabel(seeds[:50], e, edge_col=e))
+
+
 def _grouped_case(rng, counts, B, id_range):
     """Edges grouped by seed position: counts[c] edges for seed c, B batches of seeds."""
     S = counts.size
