@@ -1,8 +1,10 @@
 // sort.hip -- per-segment key sort (row ids inside every column), the
 // prerequisite of node2vec's connectivity test, and the stable sort of edges by
-// column (or row) id that turns an edge list into a compressed format.  The
-// sorts themselves are rocPRIM's radix sorts; this file adapts them to the
-// workspace convention and limits the sorted bits to what the ids need.
+// column (or row) id that turns an edge list into a compressed format.  Ids
+// below 2^32 (every graph's row ids) are sorted per segment by the kernels of
+// segsort.hip; for wider or unbounded keys, and for the edge-list sort, this
+// file adapts rocPRIM's radix sorts to the workspace convention and limits the
+// sorted bits to what the ids need.
 #include "common.h"
 
 #include <cstring>
@@ -11,6 +13,11 @@
 #include <rocprim/iterator/counting_iterator.hpp>
 
 namespace gs {
+
+// segsort.hip
+size_t segsort_workspace_bytes(int64_t nnz, int64_t num_segments, int key_bits);
+int segsort_run(const int64_t* indptr, int64_t num_segments, const int64_t* keys_in,
+                int64_t* keys_out, int64_t nnz, int key_bits, void* workspace, hipStream_t s);
 
 static int id_bits(int64_t num_ids) {
   int bits = 1;
@@ -58,6 +65,12 @@ static int packed_bits(int64_t num_segments, int64_t key_bound, int* key_bits) {
   return total <= 64 ? total : 0;
 }
 
+// Whether the kernels of segsort.hip take the call: ids known to lie below 2^32,
+// positions inside a segment that fit 32 bits.
+static bool native_segment_sort(int64_t nnz, int64_t key_bound) {
+  return key_bound > 0 && key_bound <= (int64_t(1) << 32) && nnz < (int64_t(1) << 32);
+}
+
 static size_t segmented_temp_bytes(int64_t nnz, int64_t num_segments) {
   size_t bytes = 0;
   const int64_t* k = nullptr;
@@ -84,6 +97,8 @@ extern "C" {
 size_t gs_segment_sort_workspace_bytes(int64_t nnz, int64_t num_segments, int64_t key_bound) {
   using namespace gs;
   if (nnz < 0 || num_segments < 0) return 0;
+  if (native_segment_sort(nnz, key_bound))
+    return segsort_workspace_bytes(nnz, num_segments, id_bits(key_bound));
   int key_bits = 0;
   const int bits = packed_bits(num_segments, key_bound, &key_bits);
   if (bits == 0) return segmented_temp_bytes(nnz, num_segments);
@@ -109,6 +124,9 @@ int gs_segment_sort_i64(const int64_t* indptr, int64_t num_segments,
     return GS_ERR_WORKSPACE;
   }
   hipStream_t s = as_stream(stream);
+  if (native_segment_sort(nnz, key_bound))
+    return segsort_run(indptr, num_segments, keys_in, keys_out, nnz, id_bits(key_bound),
+                       workspace, s);
   int key_bits = 0;
   const int bits = packed_bits(num_segments, key_bound, &key_bits);
   if (bits == 0) {

@@ -520,9 +520,13 @@ int gs_sorted_to_indptr(const int64_t* sorted_ids, int64_t nnz, int64_t num_cols
  *    ids sorted inside every column.  FusedNode2VecCUDA,
  *    src/cuda/fusion/node2vec.cu:139-162.
  *  gs_segment_sort_i64: sorts the ids of every segment (column).  key_bound:
- *    every key lies in [0, key_bound) (0 = not known).  With it, segment and
- *    key are sorted as one word over the bits they use; without it (or when
- *    the two do not fit 64 bits) a segmented sort over all 64 bits runs.
+ *    every key lies in [0, key_bound) (0 = not known).  For key_bound <= 2^32
+ *    (the row ids of any matrix) the library's own kernels run: segments of up
+ *    to 2048 ids are sorted in LDS in one read and one write, longer ones are
+ *    first split by 11 bits of the ids at a time.  For a wider key_bound segment
+ *    and key are radix-sorted as one word over the bits they use, and without
+ *    one (or when the two do not fit 64 bits) a segmented radix sort over all 64
+ *    bits runs (both rocPRIM).  keys_in and keys_out must not overlap.
  *    SortIndicesCUDA, src/cuda/sort_indices.cu:11-37.
  * ---------------------------------------------------------------------- */
 int gs_random_walk(const int64_t* indptr, const int64_t* indices, int64_t num_cols,
