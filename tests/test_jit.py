@@ -491,3 +491,33 @@ def test_try_compact_runs_the_search_and_leaves_the_random_state_alone():
     assert bool(found.all())
     d = gs.jit.compile(func=graphsage_sampler, args=(m, seeds, [10, 5]))
     assert d.compact is False and d.compact_search_ms is None
+
+
+@pytest.mark.gpu
+def test_a_searched_compile_that_keeps_the_plain_variant_draws_the_same_samples(monkeypatch):
+    """try_compact=True really runs both variants on the example arguments; when the
+    plain one is kept, the compiled sampler returns what an unsearched compile
+    returns from the same random state (nothing the search ran is left behind in
+    the matrix's caches)."""
+    m = _graph()
+    seeds = torch.arange(3, 3000, 7, device=DEV)
+    real = gs.jit.compile._time
+    verdict = iter([1.0, 2.0])                     # plain, then compact: plain wins
+
+    def timed(self, gm, args, runs=3):
+        real(self, gm, args, runs)
+        return next(verdict)
+
+    monkeypatch.setattr(gs.jit.compile, "_time", timed)
+    gs.manual_seed(77)
+    c = gs.jit.compile(func=graphsage_sampler, args=(m, seeds, [10, 5]), try_compact=True)
+    assert c.compact is False and c.compact_search_ms == (1.0, 2.0)
+    assert gs.random_state() == (77, 0)
+    s_in, s_out, s_blocks = c(m, seeds, [10, 5])
+    monkeypatch.undo()
+    gs.manual_seed(77)
+    d = gs.jit.compile(func=graphsage_sampler, args=(m, seeds, [10, 5]))   # try_compact=None
+    p_in, p_out, p_blocks = d(m, seeds, [10, 5])
+    assert torch.equal(s_in, p_in) and torch.equal(s_out, p_out)
+    for a, b in zip(s_blocks, p_blocks):
+        _blocks_equal(a, b)
