@@ -91,7 +91,10 @@ def graphsage_step(be, indptr, indices, seeds, ptr, fanouts, seed, call_base, pr
             sub_indptr, coo_col, rows, sel = be.sample_weighted(
                 indptr, indices, probs, seeds, fanout, False, seed, call_base + layer,
                 with_coo=not by_pointer, cdf=cdf)
-        edge_ptr = sub_indptr[ptr]
+        # (a plain index_select on the device: advanced indexing costs the host three
+        # times as long per call, and the first two layers are bound by the host)
+        edge_ptr = sub_indptr.index_select(0, ptr) if hasattr(sub_indptr, "index_select") \
+            else sub_indptr[ptr]
         if by_pointer:
             uniq, uniq_ptr, out_row, out_col = be.unique_relabel(
                 seeds, rows, ptr, edge_ptr, col_indptr=sub_indptr)
