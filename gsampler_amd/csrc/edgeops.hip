@@ -609,6 +609,7 @@ static RowRangePlan row_range_plan(int format, int64_t nnz, int64_t num_out) {
 // the range that holds the hubs' rows draws most of them): the first lane of a
 // set of peers sends one atomic for all of them, where 64 single ones to the
 // same LDS word are taken one after another.  Every lane must call this.
+constexpr int kPeerBits = 6;  // up to 64 ranges: worth the ballots (one per bit of the range)
 __device__ __forceinline__ uint64_t wave_peers(int value, int bits, bool valid) {
   uint64_t peers = __ballot(valid);
   for (int b = 0; b < bits; ++b) {
@@ -663,6 +664,10 @@ __global__ __launch_bounds__(kPartThreads) void rowsum_hist_kernel(
     for (int i = 0; i < kPartItems; ++i) {
       const bool valid = dst[i] >= 0 && dst[i] < num_out;
       const int range = valid ? (int)(dst[i] >> kRangeShift) : 0;
+      if (range_bits > kPeerBits) {  // many ranges: lanes rarely meet, one atomic each
+        if (valid) atomicAdd(&hist[range], 1);
+        continue;
+      }
       const uint64_t peers = wave_peers(range, range_bits, valid);
       if (valid && (peers & ((1ull << lane_id()) - 1ull)) == 0)  // the first of its peers
         atomicAdd(&hist[range], __popcll(peers));
@@ -728,6 +733,12 @@ __global__ __launch_bounds__(kPartThreads) void rowsum_scatter_kernel(
     for (int i = 0; i < kPartItems; ++i) {
       const bool valid = dst[i] >= 0 && dst[i] < num_out;
       const int range = valid ? (int)(dst[i] >> kRangeShift) : 0;
+      if (range_bits > kPeerBits) {
+        if (valid)
+          entries[atomicAdd(&cursor[range], 1u)] =
+              make_uint2((unsigned)dst[i], __float_as_uint(val[i]));
+        continue;
+      }
       const uint64_t peers = wave_peers(range, range_bits, valid);
       const uint64_t before = peers & ((1ull << lane_id()) - 1ull);
       unsigned base = 0;

@@ -340,7 +340,8 @@ struct BucketTable {
 // kThreads: work-group size.  A large one shares a staged table among more
 // edges; a small one spreads a short edge list over all compute units.
 // IdT: int64_t, or int32_t when the ids are read from a matrix's narrow copy.
-template <bool kInLds, int kThreads, typename IdT>
+// kView: the edges are those of a column slice read in place.
+template <bool kInLds, int kThreads, typename IdT, bool kView>
 __global__ __launch_bounds__(kThreads) void member_flag_kernel(
     const IdT* __restrict__ ids, int64_t nnz,
     const uint64_t* __restrict__ global_table, uint32_t cap,
@@ -383,7 +384,7 @@ __global__ __launch_bounds__(kThreads) void member_flag_kernel(
   SliceView::Run vrun{};
   vrun.split = INT64_MAX;  // no view: every edge at distance 0, offset 0
   bool scattered = false;  // the same in every lane
-  if (view.on()) {
+  if (kView) {
     const int64_t e_first = run * kMemberChunksPerWave * kBlock;
     const int64_t e_stop = e_first + kMemberChunksPerWave * kBlock;
     vrun = view.run(e_first, (e_stop < nnz ? e_stop : nnz) - 1);
@@ -393,6 +394,7 @@ __global__ __launch_bounds__(kThreads) void member_flag_kernel(
   // run the look-up shuffles, so all lanes go through it together
   auto id_of = [&](int64_t e) -> uint64_t {
     if (e >= nnz) e = nnz - 1;
+    if (!kView) return (uint64_t)(int64_t)ids[e];
     if (!scattered) return (uint64_t)((int64_t)ids[vrun.place(e)] + vrun.id_offset(e));
     int64_t c, offset;
     const int64_t p = view.position(vrun, e, &c, &offset);
@@ -402,15 +404,16 @@ __global__ __launch_bounds__(kThreads) void member_flag_kernel(
     const int64_t chunk0 = run * kMemberChunksPerWave + part * kMemberAhead;
     if (chunk0 >= num_chunks) break;
     uint32_t keys[kMemberAhead][kMemberWords];
-    if (!scattered) {
+    if (!kView || !scattered) {
 #pragma unroll
       for (int c = 0; c < kMemberAhead; ++c)
 #pragma unroll
         for (int j = 0; j < kMemberWords; ++j) {
           const int64_t e = (chunk0 + c) * kBlock + j * kWave + lane;
           keys[c][j] =
-              e < nnz ? member_key((uint64_t)((int64_t)ids[vrun.place(e)] + vrun.id_offset(e)))
-                      : kNoKey;
+              e >= nnz ? kNoKey
+              : kView  ? member_key((uint64_t)((int64_t)ids[vrun.place(e)] + vrun.id_offset(e)))
+                       : member_key((uint64_t)(int64_t)ids[e]);
         }
     } else {
 #pragma unroll
@@ -526,7 +529,9 @@ __global__ __launch_bounds__(kBlock) void member_indptr_kernel(
 // chunks of a part are requested together, and only then anything is stored.
 // kEdgeMajor: the id on the other axis comes from edge_major (an edge list)
 // instead of the compressed pointer.
-template <bool kEdgeMajor>
+// kView: the edges are those of a column slice read in place (without it none of
+// the view's look-ups is compiled in).
+template <bool kEdgeMajor, bool kView>
 __global__ __launch_bounds__(kBlock) void member_fill_kernel(
     int64_t nnz, const uint64_t* __restrict__ flags, const int64_t* __restrict__ chunk_off,
     const uint32_t* __restrict__ staged, const int64_t* __restrict__ indptr,
@@ -552,7 +557,7 @@ __global__ __launch_bounds__(kBlock) void member_fill_kernel(
                                                           : nnz;
   SegmentSpan span{0, 0};
   SliceView::Run vrun{};
-  if (view.on()) {  // indptr is the view's column pointer: one look-up serves both
+  if (kView) {  // indptr is the view's column pointer: one look-up serves both
     vrun = view.run(e_first, e_end - 1);
     span = vrun.span;
   } else if (out_major && !kEdgeMajor) {
@@ -594,7 +599,7 @@ __global__ __launch_bounds__(kBlock) void member_fill_kernel(
         // with a view: the edge's place in the parent and its column in the slice
         // (on a scattered run the look-up shuffles: all lanes take it, kept or not)
         int64_t parent_pos = 0, slice_col = 0;
-        if (view.on()) {
+        if (kView) {
           const int64_t ec = e < nnz ? e : nnz - 1;
           if (vrun.near()) {
             parent_pos = vrun.place(ec);
@@ -607,7 +612,7 @@ __global__ __launch_bounds__(kBlock) void member_fill_kernel(
         if ((word >> lane) & 1ull) {
           const int64_t pos = out0 + before + __popcll(word & ((1ull << lane) - 1));
           out_minor[pos] = (int64_t)minor[c][j];
-          if (view.on()) {
+          if (kView) {
             out_select[pos] = parent_pos;
             if (out_major) out_major[pos] = slice_col;
           } else {
@@ -679,24 +684,25 @@ static int minor_slice_count_impl(const int64_t* ids, const int32_t* ids32, int6
     const int64_t resident = (int64_t)(kFilterGroupsPerCu * kMemberThreads / threads) * num_compute_units();
     if (filter && blocks > resident) blocks = resident;
     const dim3 grid((unsigned)blocks);
+#define GS_MEMBER_FLAG_AS(LDS, THREADS, IDT, IDS, VIEW)                                       \
+  GS_LAUNCH("member_flag", s,                                                                 \
+            (member_flag_kernel<LDS, THREADS, IDT, VIEW>)<<<grid, dim3(THREADS), 0, s>>>(     \
+                IDS, nnz, w.table, cap, picked, w.wide, w.flags, w.chunk_off, w.staged,       \
+                filter, view))
 #define GS_MEMBER_FLAG(LDS, THREADS)                                                          \
   do {                                                                                        \
-    if (ids32)                                                                                \
-      GS_LAUNCH("member_flag", s,                                                             \
-                (member_flag_kernel<LDS, THREADS, int32_t>)<<<grid, dim3(THREADS), 0, s>>>(   \
-                    ids32, nnz, w.table, cap, picked, w.wide, w.flags, w.chunk_off, w.staged, \
-                    filter, view));                                                           \
-    else                                                                                      \
-      GS_LAUNCH("member_flag", s,                                                             \
-                (member_flag_kernel<LDS, THREADS, int64_t>)<<<grid, dim3(THREADS), 0, s>>>(   \
-                    ids, nnz, w.table, cap, picked, w.wide, w.flags, w.chunk_off, w.staged,   \
-                    filter, view));                                                           \
+    const bool in_place = view.sub_indptr != nullptr;                                         \
+    if (ids32 && in_place) GS_MEMBER_FLAG_AS(LDS, THREADS, int32_t, ids32, true);             \
+    else if (ids32) GS_MEMBER_FLAG_AS(LDS, THREADS, int32_t, ids32, false);                   \
+    else if (in_place) GS_MEMBER_FLAG_AS(LDS, THREADS, int64_t, ids, true);                   \
+    else GS_MEMBER_FLAG_AS(LDS, THREADS, int64_t, ids, false);                                \
   } while (0)
     if (in_lds && small) GS_MEMBER_FLAG(true, kBlock);
     else if (in_lds) GS_MEMBER_FLAG(true, kMemberThreads);
     else if (small) GS_MEMBER_FLAG(false, kBlock);
     else GS_MEMBER_FLAG(false, kMemberThreads);
 #undef GS_MEMBER_FLAG
+#undef GS_MEMBER_FLAG_AS
     int rc = exclusive_scan_i64(w.chunk_off, w.chunk_off, w.chunks + 1, w.scan_ws,
                                 w.scan_ws_bytes, s);
     if (rc != GS_OK) return rc;
@@ -730,16 +736,20 @@ static int minor_slice_fill_impl(const int64_t* ids, int64_t nnz, int64_t num_pi
   }
   hipStream_t s = as_stream(stream);
   const dim3 grid((unsigned)ceil_div(w.chunks, (kBlock / kWave) * kMemberChunksPerWave));
-  if (edge_major)
-    GS_LAUNCH("member_fill", s,
-              member_fill_kernel<true><<<grid, dim3(kBlock), 0, s>>>(
-                  nnz, w.flags, w.chunk_off, w.staged, indptr, num_major, edge_major,
-                  out_major, out_minor, out_select, view));
-  else
-    GS_LAUNCH("member_fill", s,
-              member_fill_kernel<false><<<grid, dim3(kBlock), 0, s>>>(
-                  nnz, w.flags, w.chunk_off, w.staged, indptr, num_major, edge_major,
-                  out_major, out_minor, out_select, view));
+#define GS_MEMBER_FILL(MAJOR, VIEW)                                                    \
+  GS_LAUNCH("member_fill", s,                                                          \
+            (member_fill_kernel<MAJOR, VIEW>)<<<grid, dim3(kBlock), 0, s>>>(           \
+                nnz, w.flags, w.chunk_off, w.staged, indptr, num_major, edge_major,    \
+                out_major, out_minor, out_select, view))
+  if (view.sub_indptr != nullptr) {
+    GS_REQUIRE(!edge_major, "minor_slice_fill: a slice read in place has no edge list");
+    GS_MEMBER_FILL(false, true);
+  } else if (edge_major) {
+    GS_MEMBER_FILL(true, false);
+  } else {
+    GS_MEMBER_FILL(false, false);
+  }
+#undef GS_MEMBER_FILL
   return GS_OK;
 }
 
