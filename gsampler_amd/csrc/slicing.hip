@@ -73,6 +73,48 @@ __global__ __launch_bounds__(kCountThreads) void col_count_kernel(
   if (threadIdx.x == 0) tile_sums[blockIdx.x] = total;
 }
 
+// Up to kSmallCountItems columns: one work-group counts and scans in a single
+// launch (every thread asks for its eight columns' pointers at once), where the
+// tiled pair of launches above costs a small sampling step one launch more per
+// layer than it has work for.
+constexpr int kSmallCountPer = 8;
+constexpr int64_t kSmallCountItems = (int64_t)kCountThreads * kSmallCountPer - 1;
+__global__ __launch_bounds__(kCountThreads) void col_count_small_kernel(
+    const int64_t* __restrict__ indptr, int64_t num_cols,
+    const int64_t* __restrict__ column_ids, int64_t num_items, int64_t fanout,
+    int replace, int64_t* __restrict__ sub_indptr, int64_t* total_mirror) {
+  __shared__ int64_t smem[kCountThreads / kWave + 1];
+  // thread t owns columns t * 8 .. t * 8 + 7: its prefix sums leave in one run
+  const int64_t base = (int64_t)threadIdx.x * kSmallCountPer;
+  int64_t cnt[kSmallCountPer], sum = 0;
+#pragma unroll
+  for (int k = 0; k < kSmallCountPer; ++k) {
+    const int64_t i = base + k;
+    cnt[k] = 0;
+    if (i < num_items) {
+      int64_t in_start;
+      const int64_t deg =
+          column_degree(indptr, num_cols, column_ids ? column_ids[i] : i, &in_start);
+      if (fanout < 0)
+        cnt[k] = deg;
+      else if (replace)
+        cnt[k] = deg == 0 ? 0 : fanout;
+      else
+        cnt[k] = deg < fanout ? deg : fanout;
+    }
+    sum += cnt[k];
+  }
+  int64_t total;
+  int64_t run = block_exclusive_sum<int64_t, kCountThreads>(sum, smem, &total);
+#pragma unroll
+  for (int k = 0; k < kSmallCountPer; ++k) {
+    const int64_t i = base + k;
+    if (i <= num_items) sub_indptr[i] = run;
+    run += cnt[k];
+  }
+  if (threadIdx.x == 0 && total_mirror) *total_mirror = total;
+}
+
 // Edge-parallel slice: thread e owns output edge e, finds its column by binary
 // search in sub_indptr (L2-resident; skipped when its whole tile lies in one
 // column) and copies one row id.  Load balance is
@@ -265,6 +307,13 @@ int gs_csc_col_count(const int64_t* indptr, int64_t num_cols,
     set_error("col_count: workspace too small: %zu < %zu", workspace_bytes,
               scan_workspace_bytes(n));
     return GS_ERR_WORKSPACE;
+  }
+  if (num_items <= kSmallCountItems) {
+    GS_LAUNCH("col_count", s,
+              col_count_small_kernel<<<dim3(1), dim3(kCountThreads), 0, s>>>(
+                  indptr, num_cols, column_ids, num_items, fanout, replace, sub_indptr,
+                  total_mirror));
+    return GS_OK;
   }
   GS_LAUNCH("col_count", s,
             col_count_kernel<<<dim3((unsigned)ceil_div(n, kScanTile)), dim3(kCountThreads),

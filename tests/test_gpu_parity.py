@@ -422,6 +422,21 @@ def test_coo_to_csc_parity(num_cols, nnz):
     assert_same(got, want)
 
 
+@pytest.mark.parametrize("n", [0, 1, 1023, 8190, 8191, 8192, 8193, 20000])
+@pytest.mark.parametrize("fanout,replace", [(-1, False), (5, False), (3, True)])
+def test_col_count_sizes_around_the_single_launch_path(n, fanout, replace):
+    """Up to 8191 columns one work-group counts and scans in a single launch; beyond,
+    tiles and a down sweep.  Both against the oracle, total in pinned host memory included."""
+    rng = np.random.default_rng(n + 7)
+    indptr, _ = random_csc(rng, 3000, 10**5, 30, hub_deg=5000)
+    cols = rng.integers(-2, 3003, size=n)                   # a few ids outside the matrix
+    count = capi._Count()
+    got = capi.col_count(T(indptr), T(cols), fanout, replace, count=count)
+    want = orc.col_count(indptr, cols, fanout, replace)
+    assert np.array_equal(N(got), want)
+    assert count.get() == want[-1]
+
+
 def test_count_mirrors_in_pinned_host_memory():
     """The optional mirror arguments of the two count entry points: the kernel that
     computes the edge total / the per-batch offsets stores them to pinned host memory
