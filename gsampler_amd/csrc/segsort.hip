@@ -124,17 +124,33 @@ __global__ __launch_bounds__(kSortThreads) void segsort_leaf_kernel(
   }
   const int64_t e_lo = list.ptr[j_lo];
   __syncthreads();
-  for (int64_t j = j_lo + threadIdx.x; j < j_hi; j += kSortThreads) {
-    const int64_t s = list.ptr[j], t = list.ptr[j + 1];
-    if (t <= s) continue;
-    const uint32_t ls = (uint32_t)(s - e_lo);  // < 2048: s and e_lo lie in the window
-    const bool skip = list.is_gap(j) || t - s > kSortSmall;
-    mark[ls] = (uint16_t)(ls << 1 | (skip ? 1u : 0u));
-    if (!skip) {
-      const uint32_t le = (uint32_t)(t - e_lo);  // <= 4096
-      end_at[ls] = (uint16_t)le;
-      atomicMax(&tile_end, le);
-      if (le - ls > kRankMax) atomicMax(&max_phase, bits_for(le - ls));
+  {
+    // (the tile's end and the longest network go to LDS once per wavefront: a
+    // window of short segments would otherwise send hundreds of atomics to the
+    // same two words, which LDS takes one after another)
+    uint32_t my_end = 0;
+    int my_phase = 0;
+    for (int64_t j = j_lo + threadIdx.x; j < j_hi; j += kSortThreads) {
+      const int64_t s = list.ptr[j], t = list.ptr[j + 1];
+      if (t <= s) continue;
+      const uint32_t ls = (uint32_t)(s - e_lo);  // < 2048: s and e_lo lie in the window
+      const bool skip = list.is_gap(j) || t - s > kSortSmall;
+      mark[ls] = (uint16_t)(ls << 1 | (skip ? 1u : 0u));
+      if (!skip) {
+        const uint32_t le = (uint32_t)(t - e_lo);  // <= 4096
+        end_at[ls] = (uint16_t)le;
+        my_end = max(my_end, le);
+        if (le - ls > kRankMax) my_phase = max(my_phase, bits_for(le - ls));
+      }
+    }
+#pragma unroll
+    for (int d = kWave / 2; d > 0; d >>= 1) {
+      my_end = max(my_end, (uint32_t)__shfl_xor((int)my_end, d, kWave));
+      my_phase = max(my_phase, __shfl_xor(my_phase, d, kWave));
+    }
+    if (lane_id() == 0 && my_end != 0) {
+      atomicMax(&tile_end, my_end);
+      if (my_phase != 0) atomicMax(&max_phase, my_phase);
     }
   }
   __syncthreads();
