@@ -521,3 +521,45 @@ def test_a_searched_compile_that_keeps_the_plain_variant_draws_the_same_samples(
     assert torch.equal(s_in, p_in) and torch.equal(s_out, p_out)
     for a, b in zip(s_blocks, p_blocks):
         _blocks_equal(a, b)
+
+
+def _batch_relabel_graph(ids_for_blocks_late: bool, same_ids: bool):
+    """A hand-made trace: all_nodes() first, the block builder after it, with the
+    builder's id tensor either the same node or another one (made before or after
+    the all_nodes() call)."""
+    import operator
+    from torch import fx
+    g = fx.Graph()
+    graph, seeds, rows = g.placeholder("graph"), g.placeholder("seeds"), g.placeholder("rows")
+    other = seeds if same_ids else None
+    if not same_ids and not ids_for_blocks_late:
+        other = g.call_function(operator.add, args=(seeds, 1))
+    valid = g.call_method("_CAPI_BatchGetValidNodes", args=(graph, seeds, rows))
+    frontier = g.call_function(operator.getitem, args=(valid, 0))
+    ptr = g.call_function(operator.getitem, args=(valid, 1))
+    if other is None:
+        other = g.call_function(operator.add, args=(seeds, 1))
+    blocks = g.call_method("_CAPI_BatchBlocks", args=(graph, other, rows))
+    g.output((frontier, ptr, blocks))
+    return fx.GraphModule(torch.nn.Module(), g)
+
+
+@pytest.mark.parametrize("late", [False, True])
+def test_all_nodes_is_not_read_off_a_block_batch_built_from_other_ids(late):
+    """The builder's frontier stands in for all_nodes() only when both were given the
+    same id tensors; with other ids nothing moves (in particular not the builder in
+    front of an argument that is made later) and the graph stays well-formed."""
+    from gsampler_amd.jit import passes
+    gm = passes.merge_relabel_and_all_nodes(_batch_relabel_graph(late, same_ids=False))
+    gm.graph.lint()
+    t = targets(gm)
+    assert t == ["_CAPI_BatchGetValidNodes", "_CAPI_BatchBlocks"]
+
+
+def test_all_nodes_is_read_off_the_block_batch_built_from_the_same_ids():
+    from gsampler_amd.jit import passes
+    gm = passes.merge_relabel_and_all_nodes(_batch_relabel_graph(False, same_ids=True))
+    gm.graph.lint()
+    t = targets(gm)
+    assert "_CAPI_BatchGetValidNodes" not in t
+    assert t == ["_CAPI_BatchBlocks", "frontier", "frontier_ptr"]   # the builder came first
