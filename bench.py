@@ -78,26 +78,29 @@ def graphsage_step(be, indptr, indices, seeds, ptr, fanouts, seed, call_base, pr
     on torch CUDA tensors or oracle.binding on numpy arrays).  With `probs`
     (fp32 per edge) neighbours are drawn by weight instead of uniformly, through
     the matrix's persistent CDF when `cdf` is given.  `by_pointer`: the relabel
-    pass takes the column of an edge from the sampled matrix's column pointer,
-    and the sampler does not write a column per edge (same outputs).
+    pass takes the column of an edge from the sampled matrix's column pointer; the
+    sampler, told where the batches of its columns begin, writes every column's
+    place inside its batch, which is the column's label while the seeds of a batch
+    are distinct, so that the relabel pass only rewrites batches where they are not
+    (same outputs).
     Returns per-layer (S, E, U) and the last layer's outputs."""
     sizes, last = [], None
     for layer, fanout in enumerate(fanouts):
+        how = dict(col_batch_ptr=ptr) if by_pointer else {}
         if probs is None:
             sub_indptr, coo_col, rows, sel = be.sample_uniform(
-                indptr, indices, seeds, fanout, False, 0, seed, call_base + layer,
-                with_coo=not by_pointer)
+                indptr, indices, seeds, fanout, False, 0, seed, call_base + layer, **how)
         else:
             sub_indptr, coo_col, rows, sel = be.sample_weighted(
                 indptr, indices, probs, seeds, fanout, False, seed, call_base + layer,
-                with_coo=not by_pointer, cdf=cdf)
+                cdf=cdf, **how)
         # (a plain index_select on the device: advanced indexing costs the host three
         # times as long per call, and the first two layers are bound by the host)
         edge_ptr = sub_indptr.index_select(0, ptr) if hasattr(sub_indptr, "index_select") \
             else sub_indptr[ptr]
         if by_pointer:
             uniq, uniq_ptr, out_row, out_col = be.unique_relabel(
-                seeds, rows, ptr, edge_ptr, col_indptr=sub_indptr)
+                seeds, rows, ptr, edge_ptr, col_indptr=sub_indptr, out_col=coo_col)
         else:
             uniq, uniq_ptr, out_row, out_col = be.unique_relabel(
                 seeds, rows, ptr, edge_ptr, coo_col)
@@ -119,8 +122,8 @@ def kernel_bytes(name, sizes):
         N = S + E
         total += {
             # the operator's interface: seeds, indptr pair, sub_indptr, gather, and row id,
-            # edge position and column of every edge (the column is delivered as the
-            # column pointer when the caller relabels by pointer: sampler_bytes_moved)
+            # edge position and column of every edge (the column is stored as the column's
+            # place inside its batch, which the relabel pass then leaves alone)
             "sample_uniform": 32 * S + 32 * E,
             "sample_weighted_cdf": 32 * S + 32 * E,  # the same interface as the uniform sampler
             "col_count": 32 * S,                 # seeds, indptr pair, counts
@@ -128,18 +131,11 @@ def kernel_bytes(name, sizes):
             "unique_dedup": 12 * N,              # packed entries in, first positions out
             "unique_flag": 4 * N + N // 4,       # first positions in, rank words out
             "unique_fill": N // 4 + 16 * U,      # rank words + first keys in, frontier out
-            "unique_relabel": 20 * E + 8 * S,    # first position + column pointer in, row + col out
+            "unique_relabel": 12 * E,            # first position in, row label out
             # frontier and labels from one launch: the two lines above together
-            "unique_fill_relabel": N // 4 + 16 * U + 20 * E + 8 * S,
+            "unique_fill_relabel": N // 4 + 16 * U + 12 * E,
         }.get(name, 0)
     return total
-
-
-def sampler_bytes_moved(sizes):
-    """What the sampler launches of one step read and write when no column per edge is
-    stored (the relabel pass reads the column pointer instead): 8 bytes per edge less than
-    the operator's interface of kernel_bytes."""
-    return sum(32 * S + 24 * E for S, E, _ in sizes)
 
 
 def batch_graphsage_sampler(A, seeds, seeds_ptr, fanouts):
@@ -428,8 +424,9 @@ def run_linerate(args, wl, capi, dev):
             torch.empty(bound, dtype=torch.int64, device=dev))
     avg_deg = int(indices.numel() // wl["nodes"])
     variants = [
-        ("as shipped: row id, edge position and column of every edge stored", 0, True),
-        ("as on the benched path: row id and edge position stored", 0, False),
+        ("as shipped: row id, edge position and column of every edge stored (the benched "
+         "path also looks up the batch of the column)", 0, True),
+        ("row id and edge position stored", 0, False),
         ("a multiplicative hash in place of Philox", 1, False),
         ("no exchange among a column's lanes", 2, False),
         ("column pointer not read (every column %d long)" % avg_deg, 4, False),
@@ -446,7 +443,7 @@ def run_linerate(args, wl, capi, dev):
                                                          o, probe_degree=avg_deg,
                                                          seed=args.seed, call_id=2), reps)
         table.append({"variant": name, "bits": variant, "us": round(ms * 1e3, 1)})
-    benched = table[1]["us"] * 1e-6
+    benched = table[0]["us"] * 1e-6
     # Lines the launch visits: per column one line of the column pointer (two when the pair
     # straddles a line) and the distinct lines of int32 row ids under its picks, counted from
     # the picks themselves; the 8-byte seed, offset and output streams come on top as bytes.
@@ -456,13 +453,13 @@ def run_linerate(args, wl, capi, dev):
     row_lines = int(torch.unique(col * (1 << 32) + sel // 32).numel())
     ptr_lines = S + int(((f % 16) == 15).sum().item())
     lines = row_lines + ptr_lines
-    stream_bytes = 16 * S + 16 * E            # seeds and offsets in, row id and edge position out
+    stream_bytes = 16 * S + 24 * E   # seeds and offsets in; row id, edge position, column out
     floor_us = lines / lines_per_s * 1e6 + stream_bytes / (2 * gib / (copy_ms * 1e-3)) * 1e6
     sampler = {
         "columns": S, "picks": E, "fanout": K, "variants": table,
-        "moved_bytes": 32 * S + 24 * E,
-        "moved_gbs": round((32 * S + 24 * E) / benched / 1e9, 1),
-        "frac_of_hbm_peak_by_bytes_moved": round((32 * S + 24 * E) / benched / 1e9 / HBM_PEAK_GBS, 4),
+        "moved_bytes": 32 * S + 32 * E,
+        "moved_gbs": round((32 * S + 32 * E) / benched / 1e9, 1),
+        "frac_of_hbm_peak_by_bytes_moved": round((32 * S + 32 * E) / benched / 1e9 / HBM_PEAK_GBS, 4),
         "lines_visited": lines, "row_id_lines": row_lines, "column_pointer_lines": ptr_lines,
         "streamed_bytes": stream_bytes,
         "time_of_those_lines_and_streams_at_the_measured_rates_us": round(floor_us, 1),
@@ -887,17 +884,8 @@ def main():
                     peak=HBM_PEAK_GBS, unit="GB/s", frac=round(dom["gbs"] / HBM_PEAK_GBS, 4),
                     traffic=traffic, avg_launch_ms=round(dom["avg_ms"], 4),
                     launches=dom["launches"])
-    if dom["kernel"] in ("sample_uniform", "sample_weighted_cdf") and dom["total_ms"] > 0:
-        # The operator's interface (32S + 32E) counts a column per edge that this path does
-        # not store (the relabel pass reads the column pointer): `achieved` / `frac` are the
-        # bytes the launch moves, 32S + 24E; the interface figure is kept by name.
-        moved = sum(sampler_bytes_moved(s) for s in prof_sizes)
-        roofline["achieved_interface"] = roofline["achieved"]
-        roofline["frac_interface"] = roofline["frac"]
-        roofline["achieved"] = round(moved / (dom["total_ms"] * 1e-3) / 1e9, 1)
-        roofline["frac"] = round(roofline["achieved"] / HBM_PEAK_GBS, 4)
-        roofline["frac_moved"] = roofline["frac"]
-        roofline["bytes"] = "32S + 24E per launch (frac, frac_moved); 32S + 32E (frac_interface)"
+    if dom["kernel"] in ("sample_uniform", "sample_weighted_cdf"):
+        roofline["bytes"] = "32S + 32E per launch: the operator's interface, all of it moved"
     if sum(S + E for S, E, _ in sizes) < (1 << 20):
         # a step this small is a chain of launches, not of bytes: say how many
         roofline["launches_per_step"] = round(

@@ -50,17 +50,17 @@ SIGNATURES = {
                                      _i64, _p, _p, _p, _p]),
     "gs_csc_col_sample_uniform_fill": (_int, [_p, _i64, _p, _p, _i64, _i64, _int,
                                               _int, _u64, _u64, _p, _p, _p, _p,
-                                              _p]),
+                                              _p, _i64, _p]),
     "gs_csc_col_sample_uniform_fill_i32": (_int, [_p, _i64, _p, _p, _i64, _i64, _int,
                                                   _int, _u64, _u64, _p, _p, _p, _p,
-                                                  _p]),
+                                                  _p, _i64, _p]),
     "gs_unique_workspace_bytes": (_sz, [_i64, _i64, _i64]),
     "gs_unique_count": (_int, [_p, _p, _i64, _p, _p, _i64, _i64, _p, _p, _p, _sz, _p]),
     "gs_unique_fill": (_int, [_p, _p, _i64, _p, _p, _i64, _i64, _p, _p, _p, _sz, _p]),
-    "gs_unique_relabel": (_int, [_p, _p, _i64, _p, _p, _i64, _i64, _p, _p, _p, _p, _p,
+    "gs_unique_relabel": (_int, [_p, _p, _i64, _p, _p, _i64, _i64, _p, _p, _p, _p, _int, _p,
                                  _sz, _p]),
     "gs_unique_fill_relabel": (_int, [_p, _p, _i64, _p, _p, _i64, _i64, _p, _p, _p, _p, _p, _p,
-                                      _p, _sz, _p]),
+                                      _int, _p, _sz, _p]),
     "gs_csc2coo": (_int, [_p, _i64, _i64, _p, _p]),
     "gs_sorted_to_indptr": (_int, [_p, _i64, _i64, _p, _p]),
     "gs_decode_batch_ids": (_int, [_p, _i64, _i64, _p, _p, _p]),
@@ -99,7 +99,7 @@ SIGNATURES = {
     "gs_weight_cdf_workspace_bytes": (_sz, [_i64, _i64]),
     "gs_weight_cdf_build": (_int, [_p, _i64, _p, _i64, _p, _i64, _p, _p, _sz, _p]),
     "gs_csc_col_sample_weighted_fill": (_int, [_p, _i64, _p, _p, _p, _p, _i64, _i64, _int, _u64,
-                                               _u64, _p, _p, _p, _p, _p, _p, _p]),
+                                               _u64, _p, _p, _p, _p, _p, _p, _p, _i64, _p]),
     "gs_weighted_key_probe": (_int, [_u64, _u64, _u64, _u64, C.c_float, _u64, _p, _p]),
     "gs_list_sample_uniform": (_int, [_i64, _i64, _int, _int, _u64, _u64, _p, _p]),
     "gs_list_sample_workspace_bytes": (_sz, [_i64, _i64]),
@@ -325,10 +325,12 @@ def col_slice_values(indptr, column_ids, sub_indptr, values):
 
 
 def sample_uniform(indptr, indices, column_ids, fanout, replace=False,
-                   algo=ALGO_AUTO, seed=7777, call_id=0, with_coo=True):
+                   algo=ALGO_AUTO, seed=7777, call_id=0, with_coo=True, col_batch_ptr=None):
     """Uniform per-column sampling, fused with the slice when column_ids is given.
 
     `indices` may be the matrix's int32 copy of the row ids (same outputs).
+    `col_batch_ptr` (offsets that cut the columns into batches): coo_col then holds
+    every column's place inside its batch instead of its place in the call.
 
     -> (sub_indptr, coo_col | None, sub_indices, select_index)
     """
@@ -344,6 +346,8 @@ def sample_uniform(indptr, indices, column_ids, fanout, replace=False,
         n = column_ids.numel()
     else:
         n = num_cols
+    if col_batch_ptr is not None:
+        col_batch_ptr = _i64t(col_batch_ptr, "col_batch_ptr")
     count = _Count()
     sub_indptr = col_count(indptr, column_ids, fanout, replace, n, count)
     bound = n * fanout                       # no column yields more than fanout edges
@@ -356,19 +360,23 @@ def sample_uniform(indptr, indices, column_ids, fanout, replace=False,
         check(fill(
             _ptr(indptr), num_cols, _ptr(indices), _ptr(column_ids), n, fanout,
             int(replace), algo, seed, call_id, sub_indptr.data_ptr(),
-            _ptr(out_col), out_idx.data_ptr(), out_sel.data_ptr(), _stream()))
+            _ptr(out_col), out_idx.data_ptr(), out_sel.data_ptr(), _ptr(col_batch_ptr),
+            col_batch_ptr.numel() - 1 if col_batch_ptr is not None else 0, _stream()))
     nnz = count.get()
     return (sub_indptr, out_col[:nnz] if with_coo else None, out_idx[:nnz], out_sel[:nnz])
 
 
 def unique_relabel(seeds, rows, seeds_ptr=None, rows_ptr=None, edge_col=None,
-                   want_row=True, want_col=True, col_indptr=None, fused=True):
+                   want_row=True, want_col=True, col_indptr=None, fused=True, out_col=None):
     """First-occurrence unique of seeds_b ++ rows_b per batch, plus relabel.
 
     The column of an edge comes from `edge_col` (a position into `seeds` per
     edge) or, for edges grouped by column, from `col_indptr` (len(seeds) + 1).
     `fused`: frontier and labels from one launch (gs_unique_fill_relabel) instead
     of gs_unique_fill followed by gs_unique_relabel; same outputs.
+    `out_col` (with col_indptr): the column labels as a sampler wrote them when it was
+    given the batch offsets of its columns (every column's place inside its batch);
+    batches with distinct seeds keep them, the others are rewritten in place.
 
     -> (unique, unique_ptr, out_row | None, out_col | None)
     """
@@ -394,7 +402,16 @@ def unique_relabel(seeds, rows, seeds_ptr=None, rows_ptr=None, edge_col=None,
     unique = torch.empty(size, dtype=torch.int64, device=dev)
     want_col = want_col and (edge_col is not None or col_indptr is not None)
     out_row = torch.empty(E, dtype=torch.int64, device=dev) if want_row else None
-    out_col = torch.empty(E, dtype=torch.int64, device=dev) if want_col else None
+    prefilled = 0
+    if out_col is not None:
+        if col_indptr is None or not want_col:
+            raise ValueError("unique_relabel: out_col goes with col_indptr")
+        out_col = _i64t(out_col, "out_col")
+        if out_col.numel() != E:
+            raise ValueError(f"unique_relabel: out_col has {out_col.numel()} entries for {E} edges")
+        prefilled = 1
+    else:
+        out_col = torch.empty(E, dtype=torch.int64, device=dev) if want_col else None
     if edge_col is not None:
         edge_col = _i64t(edge_col, "edge_col")
     if col_indptr is not None:
@@ -407,7 +424,7 @@ def unique_relabel(seeds, rows, seeds_ptr=None, rows_ptr=None, edge_col=None,
     if (want_row or want_col) and fused:
         check(l.gs_unique_fill_relabel(_ptr(seeds), sp, S, _ptr(rows), rp, E, B,
                                        unique_ptr.data_ptr(), _ptr(unique), _ptr(edge_col),
-                                       _ptr(col_indptr), _ptr(out_row), _ptr(out_col),
+                                       _ptr(col_indptr), _ptr(out_row), _ptr(out_col), prefilled,
                                        ws.data_ptr(), ws.numel(), _stream()))
     else:
         check(l.gs_unique_fill(_ptr(seeds), sp, S, _ptr(rows), rp, E, B,
@@ -416,7 +433,8 @@ def unique_relabel(seeds, rows, seeds_ptr=None, rows_ptr=None, edge_col=None,
         if want_row or want_col:
             check(l.gs_unique_relabel(_ptr(seeds), sp, S, _ptr(rows), rp, E, B,
                                       _ptr(edge_col), _ptr(col_indptr), _ptr(out_row),
-                                      _ptr(out_col), ws.data_ptr(), ws.numel(), _stream()))
+                                      _ptr(out_col), prefilled, ws.data_ptr(), ws.numel(),
+                                      _stream()))
     total = count.get()
     return unique[:total], unique_ptr, out_row, out_col
 
@@ -794,14 +812,16 @@ def weight_cdf(indptr, probs, indices=None, num_rows=None):
 
 
 def sample_weighted(indptr, indices, probs, column_ids, fanout, replace=False, seed=7777,
-                    call_id=0, with_coo=True, cdf=None):
+                    call_id=0, with_coo=True, cdf=None, col_batch_ptr=None):
     """Weighted per-column sampling -> (sub_indptr, coo_col | None, sub_indices, select).
     With `cdf` (from weight_cdf) draws are searches in the CDF instead of passes
-    over the weights."""
+    over the weights.  `col_batch_ptr`: as for sample_uniform."""
     indptr, indices = _i64t(indptr, "indptr"), _i64t(indices, "indices")
+    if col_batch_ptr is not None:
+        col_batch_ptr = _i64t(col_batch_ptr, "col_batch_ptr")
     if cdf is not None:
         return _sample_weighted_cdf(indptr, indices, _i64t(cdf, "cdf"), column_ids, fanout,
-                                    replace, seed, call_id, with_coo)
+                                    replace, seed, call_id, with_coo, col_batch_ptr)
     probs = probs.contiguous()
     if probs.dtype != torch.float32:
         raise GsError("probs must be float32")
@@ -828,12 +848,14 @@ def sample_weighted(indptr, indices, probs, column_ids, fanout, replace=False, s
         check(lib().gs_csc_col_sample_weighted_fill(
             _ptr(indptr), num_cols, _ptr(indices), probs.data_ptr(), None, _ptr(column_ids),
             n, fanout, int(replace), seed, call_id, sub_indptr.data_ptr(), _ptr(cdf_off),
-            _ptr(scratch), _ptr(out_col), out_idx.data_ptr(), out_sel.data_ptr(), _stream()))
+            _ptr(scratch), _ptr(out_col), out_idx.data_ptr(), out_sel.data_ptr(),
+            _ptr(col_batch_ptr), col_batch_ptr.numel() - 1 if col_batch_ptr is not None else 0,
+            _stream()))
     return sub_indptr, out_col, out_idx, out_sel
 
 
 def _sample_weighted_cdf(indptr, indices, cdf, column_ids, fanout, replace, seed, call_id,
-                         with_coo):
+                         with_coo, col_batch_ptr=None):
     num_cols = indptr.numel() - 1
     dev = indptr.device
     if column_ids is not None:
@@ -852,7 +874,8 @@ def _sample_weighted_cdf(indptr, indices, cdf, column_ids, fanout, replace, seed
         check(lib().gs_csc_col_sample_weighted_fill(
             _ptr(indptr), num_cols, _ptr(indices), None, cdf.data_ptr(), _ptr(column_ids), n,
             fanout, int(replace), seed, call_id, sub_indptr.data_ptr(), None, None,
-            _ptr(out_col), out_idx.data_ptr(), out_sel.data_ptr(), _stream()))
+            _ptr(out_col), out_idx.data_ptr(), out_sel.data_ptr(), _ptr(col_batch_ptr),
+            col_batch_ptr.numel() - 1 if col_batch_ptr is not None else 0, _stream()))
     nnz = count.get()
     return (sub_indptr, out_col[:nnz] if with_coo else None, out_idx[:nnz], out_sel[:nnz])
 

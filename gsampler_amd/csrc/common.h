@@ -223,6 +223,29 @@ __device__ __forceinline__ SegmentSpan segment_span(const int64_t* __restrict__ 
   return s;
 }
 
+// What a sampler stores as the column of an edge: the column's position among
+// the call's columns or, with the offsets of the call's batches of columns, its
+// position inside its batch -- which is the label the column gets in a block
+// whose batch has distinct seeds, so that the relabel pass has nothing left to do
+// for the column side.
+struct ColumnLabels {
+  const int64_t* batch_ptr;  // [num_batches + 1], null: positions in the call
+  int64_t num_batches;
+  __device__ __forceinline__ int64_t of(int64_t item) const {
+    return batch_ptr ? item - batch_ptr[segment_of(batch_ptr, num_batches, item)] : item;
+  }
+  // The same for a wavefront whose lanes hold neighbouring columns, the first of
+  // them `wave_first` (the same value in every lane): the batch of that column is
+  // searched once, on the scalar unit, and a lane walks on from there -- nearly
+  // always not at all.
+  __device__ __forceinline__ int64_t of_near(int64_t item, int64_t wave_first) const {
+    if (batch_ptr == nullptr) return item;
+    int64_t b = segment_of(batch_ptr, num_batches, wave_uniform_first(wave_first));
+    while (b + 1 < num_batches && batch_ptr[b + 1] <= item) ++b;
+    return item - batch_ptr[b];
+  }
+};
+
 // A column slice that is not written out.  Edge v of the slice A[:, cols] is
 // edge  indptr[cols[c]] + (v - sub_indptr[c])  of the parent, where c is the
 // position with sub_indptr[c] <= v < sub_indptr[c + 1] (sub_indptr = the

@@ -272,8 +272,12 @@ class OffsetMirror {
 class EdgeCount {
  public:
   struct Hint {
-    torch::Tensor col_bptr;   // set by the caller
-    torch::Tensor edge_bptr;  // left by the sampler
+    torch::Tensor col_bptr;    // set by the caller
+    torch::Tensor edge_bptr;   // left by the sampler
+    // also left by the sampler: for every edge the place of its column inside its
+    // batch, which is the column's label in the batch's block while the batch's
+    // seeds are distinct (the relabel pass then has nothing to do on that side)
+    torch::Tensor col_labels;
   };
   static Hint& hint() {
     static thread_local Hint h;
@@ -283,6 +287,7 @@ class EdgeCount {
     explicit HintScope(const torch::Tensor& col_bptr) {
       hint().col_bptr = col_bptr;
       hint().edge_bptr = torch::Tensor();
+      hint().col_labels = torch::Tensor();
     }
     ~HintScope() { hint() = Hint(); }
   };

@@ -147,6 +147,7 @@ GraphAndIndex Graph::BatchFusedSlicingSampling(torch::Tensor seeds,
   // the coordinate form is expanded from it if somebody asks
   auto ret = FusedSlicingSampling(1, seeds, fanout, replace, kCSC, kCSC);
   Graph& g = *std::get<0>(ret);
+  g.col_labels_ = EdgeCount::hint().col_labels;
   g.col_bptr_ = col_bptr;
   g.orig_col_ids_ = ids(seeds, "seeds");
   g.edge_bptr_ = EdgeCount::hint().edge_bptr;
@@ -204,16 +205,21 @@ Graph::Frontier& Graph::batch_relabel_launch(torch::Tensor& col_seeds,
   torch::Tensor rows = batch_rows_for_relabel(edges.row, row_ids);
   const int64_t E = rows.numel();
   *out_row = new_ids(E, rows);
-  *out_col = new_ids(E, rows);
+  // the column labels that the sampler left go out as they are wherever a batch
+  // has distinct seeds (the relabel pass rewrites the other batches in place)
+  const bool prefilled = edges.col_indptr.defined() && col_labels_.defined() &&
+                         col_labels_.numel() == E && E > 0;
+  *out_col = prefilled ? col_labels_ : new_ids(E, rows);
   LabelRequest labels{edges.col.defined() ? cptr(edges.col) : nullptr,
                       edges.col_indptr.defined() ? cptr(edges.col_indptr) : nullptr,
-                      mptr(*out_row), mptr(*out_col)};
+                      mptr(*out_row), mptr(*out_col), prefilled};
   Frontier& f = frontier_for(col_seeds, rows, col_bptr_, edge_bptr_, &labels);
   if (!labels.done)
     GS_CALL(gs_unique_relabel(cptr(col_seeds), cptr(col_bptr_), col_seeds.numel(),
                               cptr(rows), cptr(edge_bptr_), E, f.num_batches,
                               labels.edge_col, labels.col_indptr, labels.out_row,
-                              labels.out_col, f.workspace.data_ptr(), f.workspace.numel(),
+                              labels.out_col, prefilled ? 1 : 0, f.workspace.data_ptr(),
+                              f.workspace.numel(),
                               cur_stream()));
   if (e_ids) *e_ids = edges.e_ids;
   return f;

@@ -253,24 +253,31 @@ MajorResult major_sample_uniform(const Compressed& m,
   r.minor_ids = new_ids(size, m.indptr);
   r.select = new_ids(size, m.indptr);
   if (with_coo) r.major_ids = new_ids(size, m.indptr);
+  // a super-batched caller that asked for no coordinate form gets the columns'
+  // places inside their batches instead (EdgeCount::Hint)
+  EdgeCount::Hint& hint = EdgeCount::hint();
+  const bool label_cols = !with_coo && fused && hint.col_bptr.defined();
+  torch::Tensor col_labels = label_cols ? new_ids(size, m.indptr) : torch::Tensor();
+  int64_t* out_col = with_coo ? mptr(r.major_ids) : label_cols ? mptr(col_labels) : nullptr;
+  const int64_t* col_batch_ptr = label_cols ? cptr(hint.col_bptr) : nullptr;
+  const int64_t col_batches = label_cols ? hint.col_bptr.numel() - 1 : 0;
   const RandomState& rs = random_state();
   const torch::Tensor& narrow = m.narrow_indices();
   if (narrow.defined()) {
     GS_CALL(gs_csc_col_sample_uniform_fill_i32(
         cptr(m.indptr), num_major, narrow.data_ptr<int32_t>(),
         fused ? cptr(picked) : nullptr, n, fanout, replace ? 1 : 0, (int)rs.algo,
-        rs.seed, next_call_id(), cptr(r.indptr),
-        with_coo ? mptr(r.major_ids) : nullptr, mptr(r.minor_ids), mptr(r.select),
-        cur_stream()));
+        rs.seed, next_call_id(), cptr(r.indptr), out_col, mptr(r.minor_ids), mptr(r.select),
+        col_batch_ptr, col_batches, cur_stream()));
   } else {
     GS_CALL(gs_csc_col_sample_uniform_fill(
         cptr(m.indptr), num_major, cptr(m.indices),
         fused ? cptr(picked) : nullptr, n, fanout, replace ? 1 : 0, (int)rs.algo,
-        rs.seed, next_call_id(), cptr(r.indptr),
-        with_coo ? mptr(r.major_ids) : nullptr, mptr(r.minor_ids), mptr(r.select),
-        cur_stream()));
+        rs.seed, next_call_id(), cptr(r.indptr), out_col, mptr(r.minor_ids), mptr(r.select),
+        col_batch_ptr, col_batches, cur_stream()));
   }
   const int64_t nnz = count.get();
+  if (label_cols) hint.col_labels = col_labels.narrow(0, 0, nnz);
   r.minor_ids = r.minor_ids.narrow(0, 0, nnz);
   r.select = r.select.narrow(0, 0, nnz);
   if (with_coo) r.major_ids = r.major_ids.narrow(0, 0, nnz);
@@ -504,8 +511,8 @@ Graph::Frontier& Graph::frontier_for(const torch::Tensor& seeds,
                                    cptr(rows_ptr), E, B, cptr(f->unique_ptr),
                                    mptr(f->unique_buffer), labels->edge_col,
                                    labels->col_indptr, labels->out_row, labels->out_col,
-                                   f->workspace.data_ptr(), f->workspace.numel(),
-                                   cur_stream()));
+                                   labels->col_prefilled ? 1 : 0, f->workspace.data_ptr(),
+                                   f->workspace.numel(), cur_stream()));
     labels->done = true;
   } else {
     GS_CALL(gs_unique_fill(cptr(seeds), cptr(seeds_ptr), S, cptr(rows),
@@ -592,7 +599,7 @@ Graph::ListLabels& Graph::list_labels_for(const torch::Tensor& col_seeds,
   Frontier& f = frontier_for(col_seeds, rows, {}, {});
   torch::Tensor labels = new_ids(R + S, base);
   GS_CALL(gs_unique_relabel(cptr(col_seeds), nullptr, S, cptr(rows), nullptr, R + S, 1,
-                            nullptr, nullptr, mptr(labels), nullptr, f.workspace.data_ptr(),
+                            nullptr, nullptr, mptr(labels), nullptr, 0, f.workspace.data_ptr(),
                             f.workspace.numel(), cur_stream()));
   out->label_by_local = new_ids(R, base);
   out->label_by_local.index_copy_(0, order, labels.narrow(0, 0, R));
@@ -624,7 +631,7 @@ Graph::GraphRelabel(torch::Tensor col_seeds, torch::Tensor row_ids) {
   if (!labels.done)
     GS_CALL(gs_unique_relabel(cptr(col_seeds), nullptr, col_seeds.numel(),
                               cptr(rows), nullptr, E, 1, cptr(coo_->col), nullptr,
-                              mptr(out_row), mptr(out_col),
+                              mptr(out_row), mptr(out_col), 0,
                               f.workspace.data_ptr(), f.workspace.numel(),
                               cur_stream()));
   return {f.frontier(), out_row, out_col, coo_->e_ids};

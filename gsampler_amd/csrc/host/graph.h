@@ -281,6 +281,7 @@ class Graph : public torch::CustomClassHolder {
     const int64_t* col_indptr = nullptr;
     int64_t* out_row = nullptr;
     int64_t* out_col = nullptr;
+    bool col_prefilled = false;  // out_col holds the samplers' column labels
     bool done = false;
   };
   Frontier& frontier_for(const torch::Tensor& seeds, const torch::Tensor& rows,
@@ -334,6 +335,9 @@ class Graph : public torch::CustomClassHolder {
   std::shared_ptr<Compressed> csc_, csr_;
   std::shared_ptr<Coordinate> coo_;
   torch::Tensor col_bptr_, row_bptr_, edge_bptr_;
+  // per edge, the place of its column inside its batch, as the super-batched
+  // samplers write it (see EdgeCount::Hint); undefined for any other matrix
+  torch::Tensor col_labels_;
   torch::Tensor orig_row_ids_, orig_col_ids_;
   int64_t row_encoding_size_ = 0;
   std::unique_ptr<Frontier> frontier_;

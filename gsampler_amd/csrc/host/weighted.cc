@@ -52,7 +52,7 @@ GraphAndIndex Graph::SamplingProbs(int64_t axis, torch::Tensor edge_probs,
       nullptr,
       replace ? scratch.data_ptr() : nullptr,
       with_coo ? mptr(r.major_ids) : nullptr, mptr(r.minor_ids), mptr(r.select),
-      cur_stream()));
+      nullptr, 0, cur_stream()));
   GraphPtr g = derive(on_format, output_format, r, num_rows_, num_cols_);
   return {g, edge_index(m.e_ids, r.select)};
 }
@@ -115,13 +115,20 @@ GraphAndIndex Graph::FusedSlicingSamplingProbs(int64_t axis, torch::Tensor seeds
   r.minor_ids = new_ids(size, m.indptr);
   r.select = new_ids(size, m.indptr);
   if (with_coo) r.major_ids = new_ids(size, m.indptr);
+  // (as in the uniform sampler: a super-batched caller without a coordinate form
+  // gets the columns' places inside their batches)
+  EdgeCount::Hint& hint = EdgeCount::hint();
+  const bool label_cols = !with_coo && hint.col_bptr.defined();
+  torch::Tensor col_labels = label_cols ? new_ids(size, m.indptr) : torch::Tensor();
   const RandomState& rs = random_state();
   GS_CALL(gs_csc_col_sample_weighted_fill(
       cptr(m.indptr), num_major, cptr(m.indices), nullptr, cptr(cdf), cptr(seeds), n,
       fanout, replace ? 1 : 0, rs.seed, take_call_id(), cptr(r.indptr), nullptr, nullptr,
-      with_coo ? mptr(r.major_ids) : nullptr, mptr(r.minor_ids), mptr(r.select),
-      cur_stream()));
+      with_coo ? mptr(r.major_ids) : label_cols ? mptr(col_labels) : nullptr,
+      mptr(r.minor_ids), mptr(r.select), label_cols ? cptr(hint.col_bptr) : nullptr,
+      label_cols ? hint.col_bptr.numel() - 1 : 0, cur_stream()));
   const int64_t nnz = count.get();
+  if (label_cols) hint.col_labels = col_labels.narrow(0, 0, nnz);
   r.minor_ids = r.minor_ids.narrow(0, 0, nnz);
   r.select = r.select.narrow(0, 0, nnz);
   if (with_coo) r.major_ids = r.major_ids.narrow(0, 0, nnz);
@@ -138,9 +145,11 @@ GraphAndIndex Graph::BatchFusedSlicingSamplingProbs(torch::Tensor seeds,
   col_bptr = ids(col_bptr, "col_bptr");
   BatchOffsets::check(col_bptr, seeds.numel(), "BatchFusedSlicingSamplingProbs");
   EdgeCount::HintScope batch(col_bptr);  // the sampler leaves the edge pointer here
-  auto ret = FusedSlicingSamplingProbs(1, seeds, edge_probs, fanout, replace, kCSC,
-                                       kCSC | kCOO);
+  // compressed by column only, as the uniform twin: the relabel pass reads the
+  // column pointer and the labels the sampler left
+  auto ret = FusedSlicingSamplingProbs(1, seeds, edge_probs, fanout, replace, kCSC, kCSC);
   Graph& g = *std::get<0>(ret);
+  g.col_labels_ = EdgeCount::hint().col_labels;
   g.col_bptr_ = col_bptr;
   g.orig_col_ids_ = ids(seeds, "seeds");
   g.edge_bptr_ = EdgeCount::hint().edge_bptr;

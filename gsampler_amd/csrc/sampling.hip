@@ -22,7 +22,7 @@ __device__ __forceinline__ int64_t load_coherent(const int64_t* p) {
 // lanes.  The path of the reservoir algorithm and of fanouts above 64.
 template <int G, typename IdxT>
 __device__ __forceinline__ void sample_column_generic(
-    int lane, int64_t item, int64_t in_start, int64_t deg, int64_t out_start,
+    int lane, int64_t item, int64_t col_label, int64_t in_start, int64_t deg, int64_t out_start,
     const IdxT* __restrict__ indices, int64_t fanout, int replace,
     PhiloxKey key, int64_t* __restrict__ out_coo_col,
     int64_t* __restrict__ out_indices, int64_t* __restrict__ out_select) {
@@ -34,7 +34,7 @@ __device__ __forceinline__ void sample_column_generic(
                                                       (uint64_t)deg);
       out_indices[out_start + j] = indices ? (int64_t)indices[p] : p;
       out_select[out_start + j] = p;
-      if (out_coo_col) out_coo_col[out_start + j] = item;
+      if (out_coo_col) out_coo_col[out_start + j] = col_label;
     }
     return;
   }
@@ -44,7 +44,7 @@ __device__ __forceinline__ void sample_column_generic(
       int64_t p = in_start + j;
       out_indices[out_start + j] = indices ? (int64_t)indices[p] : p;
       out_select[out_start + j] = p;
-      if (out_coo_col) out_coo_col[out_start + j] = item;
+      if (out_coo_col) out_coo_col[out_start + j] = col_label;
     }
     return;
   }
@@ -69,7 +69,7 @@ __device__ __forceinline__ void sample_column_generic(
     int64_t p = in_start + load_coherent(out_select + out_start + jj);
     out_indices[out_start + jj] = indices ? (int64_t)indices[p] : p;
     out_select[out_start + jj] = p;
-    if (out_coo_col) out_coo_col[out_start + jj] = item;
+    if (out_coo_col) out_coo_col[out_start + jj] = col_label;
   }
 }
 
@@ -120,7 +120,7 @@ __global__ __launch_bounds__(kBlock) void sample_uniform_packed_kernel(
     int64_t num_items, int fanout, int cols_per_wave, int replace, PhiloxKey key,
     const int64_t* __restrict__ sub_indptr, int64_t* __restrict__ out_coo_col,
     int64_t* __restrict__ out_indices, int64_t* __restrict__ out_select,
-    int64_t probe_degree = 0) {
+    ColumnLabels labels, int64_t probe_degree = 0) {
   const int wave_lane = threadIdx.x & (kWave - 1);
   const int group = wave_lane / fanout;
   const int lane = wave_lane - group * fanout;
@@ -131,6 +131,8 @@ __global__ __launch_bounds__(kBlock) void sample_uniform_packed_kernel(
   const int64_t item = wave * cols_per_wave + group;
   if (group >= cols_per_wave || item >= num_items) return;  // whole groups leave together
   const int64_t c = column_ids ? column_ids[item] : item;
+  // (asked for here, so that its loads travel with the ones below)
+  const int64_t col_label = out_coo_col ? labels.of_near(item, wave * cols_per_wave) : item;
   int64_t in_start;
   int64_t deg;
   if (kProbe & kProbeNoIndptr) {
@@ -185,7 +187,7 @@ __global__ __launch_bounds__(kBlock) void sample_uniform_packed_kernel(
   out_indices[out_start + lane] = v;
   if (kProbe & kProbeOneStore) return;
   out_select[out_start + lane] = p;
-  if (out_coo_col) out_coo_col[out_start + lane] = item;
+  if (out_coo_col) out_coo_col[out_start + lane] = col_label;
 }
 
 // Any fanout, any algorithm: a group of G lanes (a power of two) owns a column
@@ -197,7 +199,7 @@ __global__ __launch_bounds__(kBlock) void sample_uniform_strided_kernel(
     const IdxT* __restrict__ indices, const int64_t* __restrict__ column_ids,
     int64_t num_items, int64_t fanout, int replace, PhiloxKey key,
     const int64_t* __restrict__ sub_indptr, int64_t* __restrict__ out_coo_col,
-    int64_t* __restrict__ out_indices, int64_t* __restrict__ out_select) {
+    int64_t* __restrict__ out_indices, int64_t* __restrict__ out_select, ColumnLabels labels) {
   const int lane = threadIdx.x & (G - 1);
   const int64_t item = ((int64_t)blockIdx.x * kBlock + threadIdx.x) / G;
   if (item >= num_items) return;  // whole groups leave together
@@ -205,8 +207,9 @@ __global__ __launch_bounds__(kBlock) void sample_uniform_strided_kernel(
   int64_t in_start;
   const int64_t deg = column_degree(indptr, num_cols, c, &in_start);
   if (deg == 0) return;
-  sample_column_generic<G, IdxT>(lane, item, in_start, deg, sub_indptr[item], indices, fanout,
-                                 replace, key, out_coo_col, out_indices, out_select);
+  sample_column_generic<G, IdxT>(lane, item, out_coo_col ? labels.of(item) : item, in_start, deg,
+                                 sub_indptr[item], indices, fanout, replace, key, out_coo_col,
+                                 out_indices, out_select);
 }
 
 template <int G, typename IdxT>
@@ -214,13 +217,13 @@ static int launch_sample_strided(const int64_t* indptr, int64_t num_cols, const 
                                  const int64_t* column_ids, int64_t num_items, int64_t fanout,
                                  int replace, PhiloxKey key, const int64_t* sub_indptr,
                                  int64_t* out_coo_col, int64_t* out_indices, int64_t* out_select,
-                                 hipStream_t stream) {
+                                 ColumnLabels labels, hipStream_t stream) {
   const int64_t blocks = ceil_div(num_items * G, kBlock);
   GS_LAUNCH("sample_uniform", stream,
             (sample_uniform_strided_kernel<G, IdxT>)<<<dim3((unsigned)blocks), dim3(kBlock), 0,
                                                       stream>>>(
                 indptr, num_cols, indices, column_ids, num_items, fanout, replace, key,
-                sub_indptr, out_coo_col, out_indices, out_select));
+                sub_indptr, out_coo_col, out_indices, out_select, labels));
   return GS_OK;
 }
 
@@ -232,8 +235,14 @@ static int sample_uniform_fill(const int64_t* indptr, int64_t num_cols, const Id
                                const int64_t* column_ids, int64_t num_items, int64_t fanout,
                                int replace, int algo, uint64_t seed, uint64_t call_id,
                                const int64_t* sub_indptr, int64_t* out_coo_col,
-                               int64_t* out_indices, int64_t* out_select, gs_stream_t stream) {
+                               int64_t* out_indices, int64_t* out_select,
+                               const int64_t* col_batch_ptr, int64_t num_col_batches,
+                               gs_stream_t stream) {
   GS_REQUIRE(num_items >= 0 && num_cols >= 0, "sample_uniform: negative size");
+  GS_REQUIRE(col_batch_ptr == nullptr || num_col_batches >= 1,
+             "sample_uniform: col_batch_ptr given but num_col_batches = %lld",
+             (long long)num_col_batches);
+  const ColumnLabels labels{col_batch_ptr, num_col_batches};
   GS_REQUIRE(fanout >= 0, "sample_uniform: negative fanout %lld",
              (long long)fanout);
   GS_REQUIRE(algo == GS_ALGO_AUTO || algo == GS_ALGO_RESERVOIR ||
@@ -259,12 +268,12 @@ static int sample_uniform_fill(const int64_t* indptr, int64_t num_cols, const Id
               sample_uniform_packed_kernel<IdxT><<<dim3((unsigned)(ceil_div(ceil_div(waves * kWave, kBlock), 8) * 8)),
                                                    dim3(kBlock), 0, s>>>(
                   indptr, num_cols, indices, column_ids, num_items, (int)fanout, cols_per_wave,
-                  replace, key, sub_indptr, out_coo_col, out_indices, out_select));
+                  replace, key, sub_indptr, out_coo_col, out_indices, out_select, labels));
     return GS_OK;
   }
 #define GS_SAMPLE_ARGS                                                          \
   indptr, num_cols, indices, column_ids, num_items, fanout, replace, key, sub_indptr, \
-      out_coo_col, out_indices, out_select, s
+      out_coo_col, out_indices, out_select, labels, s
   if (fanout <= 8) return launch_sample_strided<8, IdxT>(GS_SAMPLE_ARGS);
   if (fanout <= 16) return launch_sample_strided<16, IdxT>(GS_SAMPLE_ARGS);
   if (fanout <= 32) return launch_sample_strided<32, IdxT>(GS_SAMPLE_ARGS);
@@ -278,10 +287,11 @@ extern "C" int gs_csc_col_sample_uniform_fill(
     const int64_t* column_ids, int64_t num_items, int64_t fanout, int replace,
     int algo, uint64_t seed, uint64_t call_id, const int64_t* sub_indptr,
     int64_t* out_coo_col, int64_t* out_indices, int64_t* out_select,
-    gs_stream_t stream) {
+    const int64_t* col_batch_ptr, int64_t num_col_batches, gs_stream_t stream) {
   return gs::sample_uniform_fill<int64_t>(indptr, num_cols, indices, column_ids, num_items,
                                           fanout, replace, algo, seed, call_id, sub_indptr,
-                                          out_coo_col, out_indices, out_select, stream);
+                                          out_coo_col, out_indices, out_select, col_batch_ptr,
+                                          num_col_batches, stream);
 }
 
 extern "C" int gs_csc_col_sample_uniform_fill_i32(
@@ -289,11 +299,12 @@ extern "C" int gs_csc_col_sample_uniform_fill_i32(
     const int64_t* column_ids, int64_t num_items, int64_t fanout, int replace,
     int algo, uint64_t seed, uint64_t call_id, const int64_t* sub_indptr,
     int64_t* out_coo_col, int64_t* out_indices, int64_t* out_select,
-    gs_stream_t stream) {
+    const int64_t* col_batch_ptr, int64_t num_col_batches, gs_stream_t stream) {
   GS_REQUIRE(indices32 != nullptr, "sample_uniform_i32: null indices");
   return gs::sample_uniform_fill<int32_t>(indptr, num_cols, indices32, column_ids, num_items,
                                           fanout, replace, algo, seed, call_id, sub_indptr,
-                                          out_coo_col, out_indices, out_select, stream);
+                                          out_coo_col, out_indices, out_select, col_batch_ptr,
+                                          num_col_batches, stream);
 }
 
 // One launch of the packed sampler with parts switched off (`variant` = a sum of
@@ -323,7 +334,7 @@ extern "C" int gs_probe_sample_uniform(
               (sample_uniform_packed_kernel<int32_t, V>)<<<grid, dim3(kBlock), 0, s>>>(       \
                   indptr, num_cols, indices32, column_ids, num_items, (int)fanout,            \
                   cols_per_wave, 0, key, sub_indptr, out_coo_col, out_indices, out_select,    \
-                  probe_degree));                                                             \
+                  ColumnLabels{nullptr, 0}, probe_degree));                                   \
     return GS_OK;
   switch (variant) {
     GS_PROBE_CASE(0)

@@ -1194,6 +1194,7 @@ struct LabelArgs {
   int64_t* out_row;
   int64_t* out_col;
   int remap;
+  int col_prefilled;  // out_col holds every column's place inside its batch already
 };
 
 template <bool kByIndptr>
@@ -1203,7 +1204,7 @@ __device__ __forceinline__ void relabel_tile(
     const RankWord* __restrict__ words, const int64_t* __restrict__ group_off,
     const int64_t* __restrict__ unique_ptr, const int64_t* __restrict__ edge_col,
     const int64_t* __restrict__ col_indptr, int64_t* __restrict__ out_row,
-    int64_t* __restrict__ out_col, int remap) {
+    int64_t* __restrict__ out_col_or_null, int remap, int col_prefilled) {
   const int64_t num_tiles = ceil_div_dev(k.E, kRelabelTile);
   const int64_t tile = unit_of_block(num_tiles, remap);
   if (tile >= num_tiles) return;
@@ -1220,11 +1221,15 @@ __device__ __forceinline__ void relabel_tile(
   // rank ns - 1; the label of seed c is then its place among the seeds.
   const bool one_batch = span.lo == span.hi;
   bool seeds_distinct = false;
-  if (one_batch && out_col && info.ns > 0) {
+  if (one_batch && out_col_or_null && info.ns > 0) {
     const int64_t q = info.fb + info.ns - 1;
     seeds_distinct = ((words[q / kWave].bits >> (int)(q % kWave)) & 1ull) &&
                      rank_of(q, words, group_off) - rank0 == info.ns - 1;
   }
+  // Column labels that the sampler wrote already (a column's place inside its
+  // batch) are the labels of a batch with distinct seeds: nothing to do for the
+  // column side of such a tile.  Any other tile writes them as usual.
+  int64_t* out_col = col_prefilled && seeds_distinct ? nullptr : out_col_or_null;
   // A lane takes pairs of neighbouring edges, so that its labels leave as
   // 16-byte stores: item i is edge  e0 + (i / 2) * 2 * kBlock + 2 * lane + i % 2.
   auto edge_of = [e0](int i) {
@@ -1299,7 +1304,8 @@ __global__ __launch_bounds__(kBlock) void unique_relabel_kernel(
     Keys k, LabelArgs l, const BatchInfo* __restrict__ batch,
     const RankWord* __restrict__ words, const int64_t* __restrict__ group_off) {
   relabel_tile<kByIndptr>(k, l.etile_batch, batch, l.first, words, group_off, l.unique_ptr,
-                          l.edge_col, l.col_indptr, l.out_row, l.out_col, l.remap);
+                          l.edge_col, l.col_indptr, l.out_row, l.out_col, l.remap,
+                          l.col_prefilled);
 }
 
 // Both of the above in one launch: the first `label_blocks` work-groups label
@@ -1313,7 +1319,8 @@ __global__ __launch_bounds__(kBlock) void unique_fill_relabel_kernel(
     const int64_t* __restrict__ group_off) {
   if (blockIdx.x < label_blocks)
     relabel_tile<kByIndptr>(k, l.etile_batch, batch, l.first, words, group_off, l.unique_ptr,
-                            l.edge_col, l.col_indptr, l.out_row, l.out_col, l.remap);
+                            l.edge_col, l.col_indptr, l.out_row, l.out_col, l.remap,
+                            l.col_prefilled);
   else
     fill_group(blockIdx.x - label_blocks, k, f.flat_ptr, f.group_batch, batch, f.N, words,
                group_off, f.out_unique);
@@ -1433,7 +1440,8 @@ int gs_unique_count(const int64_t* seeds, const int64_t* seeds_ptr,
 // The launches behind gs_unique_fill, gs_unique_relabel and gs_unique_fill_relabel.
 static int launch_fill_relabel(const gs::Keys& k, const gs::UniqueWs& w, int64_t* out_unique,
                                const int64_t* edge_col, const int64_t* col_indptr,
-                               int64_t* out_row, int64_t* out_col, hipStream_t s) {
+                               int64_t* out_row, int64_t* out_col, int col_prefilled,
+                               hipStream_t s) {
   using namespace gs;
   const UniqueTuning tn = tuning();
   const int64_t N = k.S + k.E;
@@ -1442,7 +1450,8 @@ static int launch_fill_relabel(const gs::Keys& k, const gs::UniqueWs& w, int64_t
   const bool by_indptr = out_col && col_indptr;
   const FillArgs f{w.flat_ptr, w.group_batch, N, out_unique};
   const LabelArgs l{w.etile_batch, w.first, w.unique_ptr, by_indptr ? nullptr : edge_col,
-                    by_indptr ? col_indptr : nullptr, out_row, out_col, tn.remap};
+                    by_indptr ? col_indptr : nullptr, out_row, out_col, tn.remap,
+                    col_prefilled && by_indptr ? 1 : 0};
   const unsigned label_blocks =
       label ? (unsigned)grid_for_units(ceil_div(k.E, kRelabelTile), tn.remap) : 0u;
   if (fill && label) {
@@ -1488,7 +1497,7 @@ int gs_unique_fill(const int64_t* seeds, const int64_t* seeds_ptr,
   if (S + E == 0) return GS_OK;
   GS_REQUIRE(out_unique, "unique_fill: null out_unique");
   const Keys k{seeds, seeds_ptr, S, rows, rows_ptr, E, B};
-  return launch_fill_relabel(k, w, out_unique, nullptr, nullptr, nullptr, nullptr,
+  return launch_fill_relabel(k, w, out_unique, nullptr, nullptr, nullptr, nullptr, 0,
                              as_stream(stream));
 }
 
@@ -1506,7 +1515,8 @@ int gs_unique_relabel(const int64_t* seeds, const int64_t* seeds_ptr,
                       const int64_t* rows_ptr, int64_t num_rows_keys,
                       int64_t num_batches, const int64_t* edge_col,
                       const int64_t* col_indptr, int64_t* out_row, int64_t* out_col,
-                      void* workspace, size_t workspace_bytes, gs_stream_t stream) {
+                      int out_col_prefilled, void* workspace, size_t workspace_bytes,
+                      gs_stream_t stream) {
   using namespace gs;
   const int64_t S = num_seeds, E = num_rows_keys, B = num_batches;
   int rc = check_unique_args(seeds, seeds_ptr, S, rows, rows_ptr, E, B);
@@ -1516,7 +1526,7 @@ int gs_unique_relabel(const int64_t* seeds, const int64_t* seeds_ptr,
   if ((rc = check_workspace(w, workspace, workspace_bytes)) != GS_OK) return rc;
   const Keys k{seeds, seeds_ptr, S, rows, rows_ptr, E, B};
   return launch_fill_relabel(k, w, nullptr, edge_col, col_indptr, out_row, out_col,
-                             as_stream(stream));
+                             out_col_prefilled, as_stream(stream));
 }
 
 int gs_unique_fill_relabel(const int64_t* seeds, const int64_t* seeds_ptr,
@@ -1525,7 +1535,8 @@ int gs_unique_fill_relabel(const int64_t* seeds, const int64_t* seeds_ptr,
                            int64_t num_batches, const int64_t* unique_ptr,
                            int64_t* out_unique, const int64_t* edge_col,
                            const int64_t* col_indptr, int64_t* out_row, int64_t* out_col,
-                           void* workspace, size_t workspace_bytes, gs_stream_t stream) {
+                           int out_col_prefilled, void* workspace, size_t workspace_bytes,
+                           gs_stream_t stream) {
   using namespace gs;
   const int64_t S = num_seeds, E = num_rows_keys, B = num_batches;
   int rc = check_unique_args(seeds, seeds_ptr, S, rows, rows_ptr, E, B);
@@ -1537,7 +1548,7 @@ int gs_unique_fill_relabel(const int64_t* seeds, const int64_t* seeds_ptr,
   GS_REQUIRE(S + E == 0 || out_unique, "unique_fill_relabel: null out_unique");
   const Keys k{seeds, seeds_ptr, S, rows, rows_ptr, E, B};
   return launch_fill_relabel(k, w, out_unique, edge_col, col_indptr, out_row, out_col,
-                             as_stream(stream));
+                             out_col_prefilled, as_stream(stream));
 }
 
 }  // extern "C"

@@ -91,7 +91,7 @@ __global__ __launch_bounds__(kBlock) void sample_weighted_kernel(
     const int64_t* __restrict__ column_ids, int64_t num_items, int fanout,
     PhiloxKey key, const int64_t* __restrict__ sub_indptr,
     int64_t* __restrict__ out_coo_col, int64_t* __restrict__ out_indices,
-    int64_t* __restrict__ out_select) {
+    int64_t* __restrict__ out_select, ColumnLabels labels) {
   extern __shared__ __align__(8) unsigned char smem[];
   const int nthreads = blockDim.x;
   double* lkey = (double*)smem;                               // [fanout][nthreads]
@@ -112,7 +112,7 @@ __global__ __launch_bounds__(kBlock) void sample_weighted_kernel(
       const int64_t p = in_start + j;
       out_indices[out_start + j] = indices ? indices[p] : p;
       out_select[out_start + j] = p;
-      if (out_coo_col) out_coo_col[out_start + j] = item;
+      if (out_coo_col) out_coo_col[out_start + j] = labels.of(item);
     }
     return;
   }
@@ -160,7 +160,7 @@ __global__ __launch_bounds__(kBlock) void sample_weighted_kernel(
     const int64_t p = in_start + mine;
     out_indices[out_start + lane] = indices ? indices[p] : p;
     out_select[out_start + lane] = p;
-    if (out_coo_col) out_coo_col[out_start + lane] = item;
+    if (out_coo_col) out_coo_col[out_start + lane] = labels.of(item);
   }
 }
 
@@ -192,7 +192,7 @@ __global__ __launch_bounds__(kBlock) void sample_weighted_replace_kernel(
     PhiloxKey key, const int64_t* __restrict__ sub_indptr,
     const int64_t* __restrict__ cdf_offsets, uint64_t* cdf_scratch,
     int64_t* __restrict__ out_coo_col, int64_t* __restrict__ out_indices,
-    int64_t* __restrict__ out_select) {
+    int64_t* __restrict__ out_select, ColumnLabels labels) {
   const int lane = lane_id();
   const int64_t item = ((int64_t)blockIdx.x * kBlock + threadIdx.x) / kWave;
   if (item >= num_items) return;
@@ -240,7 +240,7 @@ __global__ __launch_bounds__(kBlock) void sample_weighted_replace_kernel(
     const int64_t p = in_start + (lo < deg ? lo : deg - 1);
     out_indices[out_start + j] = indices ? indices[p] : p;
     out_select[out_start + j] = p;
-    if (out_coo_col) out_coo_col[out_start + j] = item;
+    if (out_coo_col) out_coo_col[out_start + j] = labels.of(item);
   }
 }
 
@@ -474,9 +474,12 @@ __global__ __launch_bounds__(kBlock) void sample_weighted_cdf_kernel(
     const int64_t* __restrict__ column_ids, int64_t num_items, int fanout,
     int replace, PhiloxKey key, const int64_t* __restrict__ sub_indptr,
     int64_t* __restrict__ out_coo_col, int64_t* __restrict__ out_indices,
-    int64_t* __restrict__ out_select, int mode) {
+    int64_t* __restrict__ out_select, ColumnLabels labels, int mode) {
   const int64_t item = (int64_t)blockIdx.x * kBlock + threadIdx.x;
   if (item >= num_items) return;
+  // (asked for here, so that its loads travel with the ones below)
+  const int64_t col_label =
+      out_coo_col ? labels.of_near(item, item - lane_id()) : item;
   const int row_bits = (int)cdf[0];  // the same word for every lane: a scalar load
   const uint64_t row_mask = row_bits ? (~0ull >> (64 - row_bits)) : 0ull;
   const int64_t c = column_ids ? column_ids[item] : item;
@@ -513,7 +516,7 @@ __global__ __launch_bounds__(kBlock) void sample_weighted_cdf_kernel(
       const int64_t p = in_start + off;
       out_indices[out_start + taken] = row_of(off, entry);
       out_select[out_start + taken] = p;
-      if (out_coo_col) out_coo_col[out_start + taken] = item;
+      if (out_coo_col) out_coo_col[out_start + taken] = col_label;
     }
 #pragma unroll
     for (int i = 0; i < KMAX; ++i)
@@ -603,7 +606,7 @@ __global__ __launch_bounds__(kBlock) void sample_weighted_cdf_kernel(
   if (out_coo_col) {
 #pragma unroll
     for (int i = 0; i < KMAX; ++i)
-      if (i < taken) out_coo_col[out_start + i] = item;
+      if (i < taken) out_coo_col[out_start + i] = col_label;
   }
 }
 
@@ -618,12 +621,12 @@ static int launch_weighted_cdf(const int64_t* indptr, int64_t num_cols,
                                int fanout, int replace, PhiloxKey key,
                                const int64_t* sub_indptr, int64_t* out_coo_col,
                                int64_t* out_indices, int64_t* out_select,
-                               hipStream_t s) {
+                               ColumnLabels labels, hipStream_t s) {
   GS_LAUNCH("sample_weighted_cdf", s,
             sample_weighted_cdf_kernel<KMAX><<<dim3((unsigned)ceil_div(num_items, kBlock)),
                                                dim3(kBlock), 0, s>>>(
                 indptr, num_cols, indices, (const uint64_t*)cdf, column_ids, num_items,
-                fanout, replace, key, sub_indptr, out_coo_col, out_indices, out_select,
+                fanout, replace, key, sub_indptr, out_coo_col, out_indices, out_select, labels,
                 kCdfSearchMode));
   return GS_OK;
 }
@@ -1217,9 +1220,13 @@ int gs_csc_col_sample_weighted_fill(
     int64_t fanout, int replace, uint64_t seed, uint64_t call_id,
     const int64_t* sub_indptr, const int64_t* cdf_offsets, void* cdf_scratch,
     int64_t* out_coo_col, int64_t* out_indices, int64_t* out_select,
-    gs_stream_t stream) {
+    const int64_t* col_batch_ptr, int64_t num_col_batches, gs_stream_t stream) {
   using namespace gs;
   GS_REQUIRE(num_items >= 0 && num_cols >= 0, "sample_weighted: negative size");
+  GS_REQUIRE(col_batch_ptr == nullptr || num_col_batches >= 1,
+             "sample_weighted: col_batch_ptr given but num_col_batches = %lld",
+             (long long)num_col_batches);
+  const ColumnLabels labels{col_batch_ptr, num_col_batches};
   GS_REQUIRE(fanout >= 0, "sample_weighted: negative fanout %lld", (long long)fanout);
   if (num_items == 0 || fanout == 0) return GS_OK;
   GS_REQUIRE(indptr && (probs || cdf) && sub_indptr && out_indices && out_select,
@@ -1236,7 +1243,7 @@ int gs_csc_col_sample_weighted_fill(
     GS_REQUIRE(fanout <= INT32_MAX, "sample_weighted: fanout too large");
 #define GS_CDF_ARGS                                                              \
   indptr, num_cols, indices, cdf, column_ids, num_items, (int)fanout, replace, \
-      key, sub_indptr, out_coo_col, out_indices, out_select, s
+      key, sub_indptr, out_coo_col, out_indices, out_select, labels, s
     if (fanout <= 8) return launch_weighted_cdf<8>(GS_CDF_ARGS);
     if (fanout <= 16) return launch_weighted_cdf<16>(GS_CDF_ARGS);
     if (fanout <= 32) return launch_weighted_cdf<32>(GS_CDF_ARGS);
@@ -1253,7 +1260,7 @@ int gs_csc_col_sample_weighted_fill(
                                                dim3(kBlock), 0, s>>>(
                   indptr, num_cols, indices, probs, column_ids, num_items, fanout,
                   key, sub_indptr, cdf_offsets, (uint64_t*)cdf_scratch, out_coo_col,
-                  out_indices, out_select));
+                  out_indices, out_select, labels));
     return GS_OK;
   }
   GS_REQUIRE(fanout <= 64,
@@ -1272,7 +1279,7 @@ int gs_csc_col_sample_weighted_fill(
             sample_weighted_kernel<<<dim3((unsigned)blocks), dim3(threads), lds, s>>>(
                 indptr, num_cols, indices, probs, column_ids, num_items,
                 (int)fanout, key, sub_indptr, out_coo_col, out_indices,
-                out_select));
+                out_select, labels));
   return GS_OK;
 }
 

@@ -178,7 +178,15 @@ int gs_csc_col_slice_values(const int64_t* indptr, const int64_t* column_ids,
  * the same fanout / replace.  Columns with degree <= fanout are copied in
  * their original order (no replace).  `algo` is one of GS_ALGO_*.  `indices`
  * may be NULL, meaning "the edge position itself" (out_indices then repeats
- * out_select).
+ * out_select).  out_coo_col (nullable) receives the column of every edge: the
+ * position i of its column among the call's columns or, when col_batch_ptr
+ * (num_col_batches + 1 offsets that cut the call's columns into batches, nullable)
+ * is given, i - col_batch_ptr[batch of i], the column's position inside its
+ * batch.  That is the label the column gets in the batch's block whenever the
+ * batch's seeds are distinct, so gs_unique_relabel / gs_unique_fill_relabel with
+ * out_col_prefilled leave such labels as they are and only rewrite the batches
+ * whose seeds repeat (the super-batched samplers of the reference relabel every
+ * edge's column, src/cuda/batch/batch_relabel.cu:379-466).
  * Stands in for CSCColSamplingCUDA (src/cuda/sampling.cu:161-172) and
  * FusedCSCColSlicingSamplingCUDA (src/cuda/fusion/slice_sampling.cu:164-177).
  * ---------------------------------------------------------------------- */
@@ -189,7 +197,9 @@ int gs_csc_col_sample_uniform_fill(const int64_t* indptr, int64_t num_cols,
                                    uint64_t seed, uint64_t call_id,
                                    const int64_t* sub_indptr,
                                    int64_t* out_coo_col, int64_t* out_indices,
-                                   int64_t* out_select, gs_stream_t stream);
+                                   int64_t* out_select,
+                                   const int64_t* col_batch_ptr,
+                                   int64_t num_col_batches, gs_stream_t stream);
 
 /* The same with the row ids read from a 32-bit copy of `indices`
  * (indices32[e] == indices[e] for every edge, all ids < 2^31): identical
@@ -204,7 +214,10 @@ int gs_csc_col_sample_uniform_fill_i32(const int64_t* indptr, int64_t num_cols,
                                        const int64_t* sub_indptr,
                                        int64_t* out_coo_col,
                                        int64_t* out_indices,
-                                       int64_t* out_select, gs_stream_t stream);
+                                       int64_t* out_select,
+                                       const int64_t* col_batch_ptr,
+                                       int64_t num_col_batches,
+                                       gs_stream_t stream);
 
 /* ------------------------------------------------------------------------
  * Weighted per-column sampling (fill phase; counts come from
@@ -230,6 +243,8 @@ int gs_csc_col_sample_uniform_fill_i32(const int64_t* indptr, int64_t num_cols,
  *    draw order; when fewer than fanout edges have positive (quantised)
  *    weight, zero-weight edges follow in index order.  Stream: pos = column
  *    position, draw = output slot.
+ *  out_coo_col, col_batch_ptr, num_col_batches: as for the uniform sampler
+ *    above (the column's position in the call, or inside its batch).
  * Stands in for CSCColSamplingProbsCUDA (src/cuda/sampling_probs.cu:268-281).
  * ---------------------------------------------------------------------- */
 /* Persistent packed CDF of a matrix's edge weights, the input of the fast
@@ -260,7 +275,7 @@ int gs_csc_col_sample_weighted_fill(
     int64_t fanout, int replace, uint64_t seed, uint64_t call_id,
     const int64_t* sub_indptr, const int64_t* cdf_offsets, void* cdf_scratch,
     int64_t* out_coo_col, int64_t* out_indices, int64_t* out_select,
-    gs_stream_t stream);
+    const int64_t* col_batch_ptr, int64_t num_col_batches, gs_stream_t stream);
 
 /* Evaluates the key arithmetic on the device: out2[0] = -log2((r64>>12)+1)/2^52),
  * out2[1] = key of weight w at stream (seed, call_id, pos, draw).  Test hook. */
@@ -323,7 +338,11 @@ int gs_list_sample_weighted_fill(const float* probs, const int64_t* range,
  *   a matrix then need not exist: the reference expands it first,
  *   src/cuda/batch/batch_relabel.cu:480-498 takes coo_col).  Give one of the
  *   two, the other NULL.  May be called any number of times while the
- *   workspace is kept.
+ *   workspace is kept.  out_col_prefilled != 0 (with col_indptr): out_col already
+ *   holds, for every edge, the place of its column inside its batch, as a sampler
+ *   that was given col_batch_ptr writes it; those are the labels wherever the
+ *   seeds of a batch are distinct, and only the edges of other batches are
+ *   rewritten.
  * fill_relabel: fill and relabel in one launch (the two read the same state and
  *   write different outputs), for the caller that wants both at once, as
  *   BatchGraphRelabel does (src/cuda/batch/batch_relabel.cu:480-498 returns the
@@ -357,14 +376,16 @@ int gs_unique_relabel(const int64_t* seeds, const int64_t* seeds_ptr,
                       const int64_t* rows_ptr, int64_t num_rows_keys,
                       int64_t num_batches, const int64_t* edge_col,
                       const int64_t* col_indptr, int64_t* out_row, int64_t* out_col,
-                      void* workspace, size_t workspace_bytes, gs_stream_t stream);
+                      int out_col_prefilled, void* workspace, size_t workspace_bytes,
+                      gs_stream_t stream);
 int gs_unique_fill_relabel(const int64_t* seeds, const int64_t* seeds_ptr,
                            int64_t num_seeds, const int64_t* rows,
                            const int64_t* rows_ptr, int64_t num_rows_keys,
                            int64_t num_batches, const int64_t* unique_ptr,
                            int64_t* out_unique, const int64_t* edge_col,
                            const int64_t* col_indptr, int64_t* out_row, int64_t* out_col,
-                           void* workspace, size_t workspace_bytes, gs_stream_t stream);
+                           int out_col_prefilled, void* workspace, size_t workspace_bytes,
+                           gs_stream_t stream);
 
 /* ------------------------------------------------------------------------
  * out_first[r] = smallest position e with ids[e] == r, INT64_MAX when r does

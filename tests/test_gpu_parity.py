@@ -227,6 +227,57 @@ def test_unique_frontier_and_labels_from_one_launch(by_pointer):
                 orc.unique_relabel(seeds[:50], e, edge_col=e))
 
 
+@pytest.mark.parametrize("weighted", [False, True])
+@pytest.mark.parametrize("fanout", [5, 70])
+def test_samplers_write_the_place_of_a_column_inside_its_batch(weighted, fanout):
+    """With the offsets of the batches of its columns a sampler stores, for every edge,
+    its column's place inside the batch (the packed, the strided and the weighted
+    kernels); without them the column's place in the call."""
+    rng = np.random.default_rng(fanout + weighted)
+    indptr, indices = random_csc(rng, 3000, 10**5, 40, hub_deg=4000)
+    cols = rng.integers(0, 3000, size=900)
+    ptr = np.array([0, 1, 1, 300, 640, 900])
+    if weighted:
+        probs = rng.random(indices.size).astype(np.float32)
+        k = min(fanout, 64)
+        cdf = capi.weight_cdf(T(indptr), torch.as_tensor(probs, device=DEV), T(indices), 3000)
+        plain = capi.sample_weighted(T(indptr), T(indices), None, T(cols), k, cdf=cdf, call_id=3)
+        local = capi.sample_weighted(T(indptr), T(indices), None, T(cols), k, cdf=cdf, call_id=3,
+                                     col_batch_ptr=T(ptr))
+    else:
+        plain = capi.sample_uniform(T(indptr), T(indices), T(cols), fanout, call_id=3)
+        local = capi.sample_uniform(T(indptr), T(indices), T(cols), fanout, call_id=3,
+                                    col_batch_ptr=T(ptr))
+    for a, b in zip((plain[0], plain[2], plain[3]), (local[0], local[2], local[3])):
+        assert torch.equal(a, b)
+    col = N(plain[1])
+    batch = np.searchsorted(ptr, col, side="right") - 1
+    assert np.array_equal(N(local[1]), col - ptr[batch])
+
+
+@pytest.mark.parametrize("repeat_seeds_in", [(), (2,), (0, 1, 2, 3)])
+def test_unique_relabel_with_column_labels_from_the_sampler(repeat_seeds_in):
+    """out_col handed in with every column's place inside its batch: batches with
+    distinct seeds keep it, batches in which a seed repeats are rewritten -- the
+    result is what the pass computes on its own, and what the oracle computes."""
+    rng = np.random.default_rng(len(repeat_seeds_in))
+    counts = rng.integers(0, 7, size=6000)
+    seeds, rows, sp, rp, edge_col, col_indptr = _grouped_case(rng, counts, 4, 10**5)
+    for b in repeat_seeds_in:                       # a repeated seed: labels are no longer places
+        if sp[b + 1] - sp[b] >= 2:
+            seeds[sp[b + 1] - 1] = seeds[sp[b]]
+    batch = np.searchsorted(sp, edge_col, side="right") - 1
+    places = edge_col - sp[batch]
+    own = capi.unique_relabel(T(seeds), T(rows), T(sp), T(rp), col_indptr=T(col_indptr))
+    for fused in (True, False):
+        handed = T(places.copy())
+        got = capi.unique_relabel(T(seeds), T(rows), T(sp), T(rp), col_indptr=T(col_indptr),
+                                  out_col=handed, fused=fused)
+        assert got[3].data_ptr() == handed.data_ptr()            # written in place
+        assert_same(got, tuple(N(x) for x in own))
+    assert_same(own, orc.unique_relabel(seeds, rows, sp, rp, edge_col))
+
+
 def _grouped_case(rng, counts, B, id_range):
     """Edges grouped by seed position: counts[c] edges for seed c, B batches of seeds."""
     S = counts.size
