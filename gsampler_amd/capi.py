@@ -71,6 +71,7 @@ SIGNATURES = {
     "gs_list_labels": (_int, [_p, _i64, _p, _p, _i64, _p, _p, _p, _p, _p, _p]),
     "gs_gather_rows": (_int, [_p, _i64, _i64, _p, _i64, _p, _p, _p]),
     "gs_coo_sort_workspace_bytes": (_sz, [_i64, _i64]),
+    "gs_coo_sort_flag_offset": (_i64, [_i64, _i64]),
     "gs_coo_sort": (_int, [_p, _i64, _i64, _p, _p, _p, _sz, _p]),
     "gs_sddmm": (_int, [_int, _p, _p, _i64, _i64, _p, _int, _int, _p, _p, _p, _int, _int,
                         _i64, _i64, _i64, _i64, _p, _p, _p]),
@@ -492,15 +493,20 @@ def list_labels(seeds, list_ids, first_pos):
     return frontier[:count.get()], list_label, seed_label
 
 
-def coo_sort(major: torch.Tensor, num_major: int):
+def coo_sort(major: torch.Tensor, num_major: int, verify: bool = True):
     """Stable sort of edge positions by their id on the axis to compress:
-    (sorted ids, positions)."""
+    (sorted ids, positions).  `verify` waits for the call and raises when the
+    sort's gave-up flag is set (a pass stopped waiting for another tile's counts:
+    the result is then not fully sorted)."""
     major = _i64t(major, "major")
     n = major.numel()
     out, perm = torch.empty_like(major), torch.empty_like(major)
     ws = _workspace(lib().gs_coo_sort_workspace_bytes(n, num_major), major.device)
     check(lib().gs_coo_sort(_ptr(major), n, num_major, _ptr(out), _ptr(perm), ws.data_ptr(),
                             ws.numel(), _stream()))
+    at = lib().gs_coo_sort_flag_offset(n, num_major)
+    if verify and n > 0 and at >= 0 and int(ws[at:at + 4].view(torch.int32).item()) != 0:
+        raise GsError("coo_sort: a pass gave up waiting for the counts of an earlier tile")
     return out, perm
 
 

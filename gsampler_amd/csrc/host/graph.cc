@@ -116,6 +116,14 @@ static std::shared_ptr<Compressed> compress(const Coordinate& coo, bool by_col,
                         ws.data_ptr(), (size_t)ws.numel(), cur_stream()));
     out->indices = GatherRows(minor, perm);
     out->e_ids = coo.e_ids.has_value() ? GatherRows(coo.e_ids.value(), perm) : perm;
+    // A format conversion is no part of a sampling step: it can afford to wait for
+    // the sort and look at its gave-up flag.
+    const int64_t flag_at = gs_coo_sort_flag_offset(nnz, num_major);
+    if (nnz > 0 && flag_at >= 0) {
+      const torch::Tensor flag = ws.narrow(0, flag_at, 4).view(torch::kInt32).cpu();
+      TORCH_CHECK(flag.item<int32_t>() == 0,
+                  "coo_sort: a pass gave up waiting for the counts of an earlier tile");
+    }
   }
   out->indptr = new_ids(num_major + 1, major);
   GS_CALL(gs_sorted_to_indptr(cptr(sorted_major), sorted_major.numel(),

@@ -1,10 +1,11 @@
 // sort.hip -- per-segment key sort (row ids inside every column), the
 // prerequisite of node2vec's connectivity test, and the stable sort of edges by
 // column (or row) id that turns an edge list into a compressed format.  Ids
-// below 2^32 (every graph's row ids) are sorted per segment by the kernels of
-// segsort.hip; for wider or unbounded keys, and for the edge-list sort, this
-// file adapts rocPRIM's radix sorts to the workspace convention and limits the
-// sorted bits to what the ids need.
+// below 2^32 (every graph's ids) are sorted per segment by the kernels of
+// segsort.hip and over an edge list by those of coosort.hip; for wider or
+// unbounded keys and for lists of 2^32 edges and more this file adapts rocPRIM's
+// radix sorts to the workspace convention and limits the sorted bits to what
+// the ids need.
 #include "common.h"
 
 #include <cstring>
@@ -18,6 +19,11 @@ namespace gs {
 size_t segsort_workspace_bytes(int64_t nnz, int64_t num_segments, int key_bits);
 int segsort_run(const int64_t* indptr, int64_t num_segments, const int64_t* keys_in,
                 int64_t* keys_out, int64_t nnz, int key_bits, void* workspace, hipStream_t s);
+
+// coosort.hip
+size_t coosort_workspace_bytes(int64_t nnz, int id_bits);
+int coosort_run(const int64_t* major, int64_t nnz, int id_bits, int64_t* sorted_major,
+                int64_t* perm, void* workspace, hipStream_t s);
 
 static int id_bits(int64_t num_ids) {
   int bits = 1;
@@ -69,6 +75,11 @@ static int packed_bits(int64_t num_segments, int64_t key_bound, int* key_bits) {
 // positions inside a segment that fit 32 bits.
 static bool native_segment_sort(int64_t nnz, int64_t key_bound) {
   return key_bound > 0 && key_bound <= (int64_t(1) << 32) && nnz < (int64_t(1) << 32);
+}
+
+// Whether the kernels of coosort.hip take the call: ids and positions of 32 bits.
+static bool native_coo_sort(int64_t nnz, int64_t num_major) {
+  return nnz > 0 && nnz < (int64_t(1) << 32) && num_major <= (int64_t(1) << 32);
 }
 
 static size_t segmented_temp_bytes(int64_t nnz, int64_t num_segments) {
@@ -158,12 +169,21 @@ int gs_segment_sort_i64(const int64_t* indptr, int64_t num_segments,
 
 size_t gs_coo_sort_workspace_bytes(int64_t nnz, int64_t num_major) {
   if (nnz < 0) return 0;
+  if (gs::native_coo_sort(nnz, num_major))
+    return gs::coosort_workspace_bytes(nnz, gs::id_bits(num_major));
   size_t bytes = 0;
   const int64_t* k = nullptr;
   int64_t* o = nullptr;
   (void)rocprim::radix_sort_pairs(nullptr, bytes, k, o, rocprim::counting_iterator<int64_t>(0), o,
                                   (size_t)(nnz > 0 ? nnz : 1), 0u, (unsigned)gs::id_bits(num_major));
   return gs::align_up(bytes, 256);
+}
+
+// Where in the workspace of gs_coo_sort, in bytes, the 32-bit gave-up flag of the
+// library's own sort kernels sits for a call of these sizes, or -1 when the call
+// is served by rocPRIM, which has none.
+int64_t gs_coo_sort_flag_offset(int64_t nnz, int64_t num_major) {
+  return gs::native_coo_sort(nnz, num_major) ? 0 : -1;
 }
 
 // Stable sort of the edge positions 0..nnz-1 by major[position]: sorted_major
@@ -185,6 +205,8 @@ int gs_coo_sort(const int64_t* major, int64_t nnz, int64_t num_major,
     return GS_ERR_WORKSPACE;
   }
   hipStream_t s = as_stream(stream);
+  if (native_coo_sort(nnz, num_major))
+    return coosort_run(major, nnz, id_bits(num_major), sorted_major, perm, workspace, s);
   size_t bytes = workspace_bytes;
   ProfScope ps("coo_sort", s);
   GS_HIP(rocprim::radix_sort_pairs(workspace, bytes, major, sorted_major,

@@ -428,8 +428,20 @@ int gs_list_labels(const int64_t* seeds, int64_t num_seeds, const int64_t* list_
  * (the e_ids of the new format); gs_sorted_to_indptr and two gathers by perm
  * finish the conversion.  COOSort / COO2CSCCUDA,
  * src/cuda/format_transform.cu:65-84,121-142.
+ * Fewer than 2^32 edges with num_major <= 2^32 are sorted by the library's own
+ * kernels: least significant digit first, 8 bits a pass over the bits that ids
+ * below num_major need, 8 bytes per edge between the passes.  Tiles of a pass
+ * learn the counts of the tiles before them from words those publish; a wait
+ * for such a word is bounded, and a pass that reaches the bound goes on without
+ * it (the outputs are then a permutation that is not fully sorted) and sets a
+ * 32-bit flag in the workspace, at byte gs_coo_sort_flag_offset(nnz, num_major)
+ * (-1: this call has no flag; rocPRIM's radix sort serves it).  The bound is
+ * 65 536 polls of a word that another running work-group is about to write and
+ * has never been reached; a caller that reads the flag after the call has
+ * completed knows.
  * ---------------------------------------------------------------------- */
 size_t gs_coo_sort_workspace_bytes(int64_t nnz, int64_t num_major);
+int64_t gs_coo_sort_flag_offset(int64_t nnz, int64_t num_major);
 int gs_coo_sort(const int64_t* major, int64_t nnz, int64_t num_major,
                 int64_t* sorted_major, int64_t* perm, void* workspace,
                 size_t workspace_bytes, gs_stream_t stream);
