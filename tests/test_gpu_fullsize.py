@@ -149,6 +149,26 @@ def _check_walk_trace(indptr, indices, start, trace, length, steps):
         assert bool((indptr[ps + 1] == indptr[ps]).all())
 
 
+def test_edge_list_sort_at_full_size(graph):
+    """The 124 M column ids of the headline graph in shuffled order (15 137 tiles a pass, three
+    passes): positions and ids against torch's stable sort, and what holds at any size --
+    the positions are a permutation, ids ascend, equal ids keep their order."""
+    indptr, _, _, _ = graph
+    col = capi.csc2coo(indptr, EDGES)
+    g = torch.Generator(device=col.device)
+    g.manual_seed(9)
+    shuffled = col[torch.randperm(EDGES, generator=g, device=col.device)]
+    ids, perm = capi.coo_sort(shuffled, NODES)
+    assert torch.equal(ids, col)                               # the ids in order are the CSC's columns
+    assert torch.equal(shuffled[perm], ids)
+    assert bool(((ids[1:] > ids[:-1]) | (perm[1:] > perm[:-1])).all())   # stable
+    seen = torch.zeros(EDGES, dtype=torch.bool, device=col.device)
+    seen[perm] = True
+    assert bool(seen.all())
+    want = torch.sort(shuffled, stable=True)
+    assert torch.equal(perm, want.indices)
+
+
 def test_node2vec_walks(graph):
     indptr, indices, _, _ = graph
     indices = capi.segment_sort(indptr, indices, NODES)
