@@ -121,12 +121,12 @@ def kernel_bytes(name, sizes):
     for S, E, U in sizes:
         N = S + E
         total += {
-            # the operator's interface: seeds, indptr pair, sub_indptr, gather, and row id,
-            # edge position and column of every edge (the column is stored as the column's
-            # place inside its batch, which the relabel pass then leaves alone)
-            "sample_uniform": 32 * S + 32 * E,
-            "sample_weighted_cdf": 32 * S + 32 * E,  # the same interface as the uniform sampler
-            "col_count": 32 * S,                 # seeds, indptr pair, counts
+            # the fill pass's interface: span and sub_indptr of every column, gather, and
+            # row id, edge position and column of every edge (the column is stored as the
+            # column's place inside its batch, which the relabel pass then leaves alone)
+            "sample_uniform": 16 * S + 32 * E,
+            "sample_weighted_cdf": 16 * S + 32 * E,  # the same interface as the uniform sampler
+            "col_count": 40 * S,                 # seeds, indptr pair in; counts and spans out
             "unique_scatter": 16 * N,            # keys in, packed entries out
             "unique_dedup": 12 * N,              # packed entries in, first positions out
             "unique_flag": 4 * N + N // 4,       # first positions in, rank words out
@@ -416,7 +416,8 @@ def run_linerate(args, wl, capi, dev):
         f, fp = r_[0], r_[1]
     K = wl["fanouts"][-1]
     S = int(f.numel())
-    sub_indptr = capi.col_count(indptr, f, K, False)
+    col_span = torch.empty(S, dtype=torch.int64, device=dev)
+    sub_indptr = capi.col_count(indptr, f, K, False, col_span=col_span)
     E = int(sub_indptr[-1].item())
     bound = S * K
     outs = (torch.empty(bound, dtype=torch.int64, device=dev),
@@ -424,8 +425,9 @@ def run_linerate(args, wl, capi, dev):
             torch.empty(bound, dtype=torch.int64, device=dev))
     avg_deg = int(indices.numel() // wl["nodes"])
     variants = [
-        ("as shipped: row id, edge position and column of every edge stored (the benched "
-         "path also looks up the batch of the column)", 0, True),
+        ("as shipped: column spans from the count pass; row id, edge position and column of "
+         "every edge stored (the benched path also looks up the batch of the column)", 0, True),
+        ("column pointer looked up again instead (no spans)", -1, True),
         ("row id and edge position stored", 0, False),
         ("a multiplicative hash in place of Philox", 1, False),
         ("no exchange among a column's lanes", 2, False),
@@ -439,28 +441,33 @@ def run_linerate(args, wl, capi, dev):
     table = []
     for name, variant, with_col in variants:
         o = (outs[0] if with_col else None, outs[1], outs[2])
-        ms = _event_ms(lambda: capi.probe_sample_uniform(indptr, idx32, f, K, variant, sub_indptr,
-                                                         o, probe_degree=avg_deg,
-                                                         seed=args.seed, call_id=2), reps)
-        table.append({"variant": name, "bits": variant, "us": round(ms * 1e3, 1)})
+        spans = col_span if variant >= 0 else None
+        ms = _event_ms(lambda: capi.probe_sample_uniform(indptr, idx32, f, K, max(variant, 0),
+                                                         sub_indptr, o, probe_degree=avg_deg,
+                                                         seed=args.seed, call_id=2,
+                                                         col_span=spans), reps)
+        table.append({"variant": name, "bits": max(variant, 0), "spans": spans is not None,
+                      "us": round(ms * 1e3, 1)})
     benched = table[0]["us"] * 1e-6
-    # Lines the launch visits: per column one line of the column pointer (two when the pair
-    # straddles a line) and the distinct lines of int32 row ids under its picks, counted from
-    # the picks themselves; the 8-byte seed, offset and output streams come on top as bytes.
+    # Lines the launch visits: the distinct lines of int32 row ids under its picks, counted
+    # from the picks themselves (without spans also one line of the column pointer per column,
+    # two when the pair straddles a line: column_pointer_lines); the 8-byte span, offset and
+    # output streams come on top as bytes.
     capi.probe_sample_uniform(indptr, idx32, f, K, 0, sub_indptr, (outs[0], outs[1], outs[2]),
-                              seed=args.seed, call_id=2)
+                              seed=args.seed, call_id=2, col_span=col_span)
     col, sel = outs[0][:E], outs[2][:E]
     row_lines = int(torch.unique(col * (1 << 32) + sel // 32).numel())
     ptr_lines = S + int(((f % 16) == 15).sum().item())
-    lines = row_lines + ptr_lines
-    stream_bytes = 16 * S + 24 * E   # seeds and offsets in; row id, edge position, column out
+    lines = row_lines
+    stream_bytes = 16 * S + 24 * E   # spans and offsets in; row id, edge position, column out
     floor_us = lines / lines_per_s * 1e6 + stream_bytes / (2 * gib / (copy_ms * 1e-3)) * 1e6
     sampler = {
         "columns": S, "picks": E, "fanout": K, "variants": table,
-        "moved_bytes": 32 * S + 32 * E,
-        "moved_gbs": round((32 * S + 32 * E) / benched / 1e9, 1),
-        "frac_of_hbm_peak_by_bytes_moved": round((32 * S + 32 * E) / benched / 1e9 / HBM_PEAK_GBS, 4),
-        "lines_visited": lines, "row_id_lines": row_lines, "column_pointer_lines": ptr_lines,
+        "moved_bytes": 16 * S + 32 * E,
+        "moved_gbs": round((16 * S + 32 * E) / benched / 1e9, 1),
+        "frac_of_hbm_peak_by_bytes_moved": round((16 * S + 32 * E) / benched / 1e9 / HBM_PEAK_GBS, 4),
+        "lines_visited": lines, "row_id_lines": row_lines,
+        "column_pointer_lines_without_spans": ptr_lines,
         "streamed_bytes": stream_bytes,
         "time_of_those_lines_and_streams_at_the_measured_rates_us": round(floor_us, 1),
         "frac_of_measured_rates": round(floor_us * 1e-6 / benched, 4),
@@ -885,7 +892,8 @@ def main():
                     traffic=traffic, avg_launch_ms=round(dom["avg_ms"], 4),
                     launches=dom["launches"])
     if dom["kernel"] in ("sample_uniform", "sample_weighted_cdf"):
-        roofline["bytes"] = "32S + 32E per launch: the operator's interface, all of it moved"
+        roofline["bytes"] = ("16S + 32E per launch: the fill pass's interface (column spans from "
+                             "the count pass, which reads the seeds and the indptr pairs: 40S)")
     if sum(S + E for S, E, _ in sizes) < (1 << 20):
         # a step this small is a chain of launches, not of bytes: say how many
         roofline["launches_per_step"] = round(

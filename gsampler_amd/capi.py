@@ -44,15 +44,15 @@ SIGNATURES = {
     "gs_copy_i64": (_int, [_p, _i64, _p, _p]),
     "gs_scan_workspace_bytes": (_sz, [_i64]),
     "gs_exclusive_scan_i64": (_int, [_p, _p, _i64, _p, _sz, _p]),
-    "gs_csc_col_count": (_int, [_p, _i64, _p, _i64, _i64, _int, _p, _p, _p, _sz, _p]),
+    "gs_csc_col_count": (_int, [_p, _i64, _p, _i64, _i64, _int, _p, _p, _p, _p, _sz, _p]),
     "gs_csc_col_count_static": (_int, [_p, _i64, _p, _i64, _i64, _int, _p, _p]),
     "gs_csc_col_slice_fill": (_int, [_p, _i64, _p, _p, _i64, _p, _i64, _p, _i64,
                                      _i64, _p, _p, _p, _p]),
     "gs_csc_col_sample_uniform_fill": (_int, [_p, _i64, _p, _p, _i64, _i64, _int,
-                                              _int, _u64, _u64, _p, _p, _p, _p,
+                                              _int, _u64, _u64, _p, _p, _p, _p, _p,
                                               _p, _i64, _p]),
     "gs_csc_col_sample_uniform_fill_i32": (_int, [_p, _i64, _p, _p, _i64, _i64, _int,
-                                                  _int, _u64, _u64, _p, _p, _p, _p,
+                                                  _int, _u64, _u64, _p, _p, _p, _p, _p,
                                                   _p, _i64, _p]),
     "gs_unique_workspace_bytes": (_sz, [_i64, _i64, _i64]),
     "gs_unique_count": (_int, [_p, _p, _i64, _p, _p, _i64, _i64, _p, _p, _p, _sz, _p]),
@@ -93,14 +93,14 @@ SIGNATURES = {
     "gs_probe_stream_copy": (_int, [_p, _p, _i64, _p]),
     "gs_probe_line_gather": (_int, [_p, _i64, _i64, _u64, _int, _p, _p]),
     "gs_probe_sample_uniform": (_int, [_p, _i64, _p, _p, _i64, _i64, _int, _i64, _u64, _u64, _p,
-                                       _p, _p, _p, _p]),
+                                       _p, _p, _p, _p, _p]),
     "gs_sliced_e_square_sum_workspace_bytes": (_sz, [_i64, _i64]),
     "gs_sliced_e_square_sum": (_int, [_p, _p, _p, _p, _i64, _p, _i64, _p, _p, _p, _i64, _p, _sz,
                                       _p]),
     "gs_weight_cdf_workspace_bytes": (_sz, [_i64, _i64]),
     "gs_weight_cdf_build": (_int, [_p, _i64, _p, _i64, _p, _i64, _p, _p, _sz, _p]),
     "gs_csc_col_sample_weighted_fill": (_int, [_p, _i64, _p, _p, _p, _p, _i64, _i64, _int, _u64,
-                                               _u64, _p, _p, _p, _p, _p, _p, _p, _i64, _p]),
+                                               _u64, _p, _p, _p, _p, _p, _p, _p, _p, _i64, _p]),
     "gs_weighted_key_probe": (_int, [_u64, _u64, _u64, _u64, C.c_float, _u64, _p, _p]),
     "gs_list_sample_uniform": (_int, [_i64, _i64, _int, _int, _u64, _u64, _p, _p]),
     "gs_list_sample_workspace_bytes": (_sz, [_i64, _i64]),
@@ -263,9 +263,12 @@ def exclusive_scan(x: torch.Tensor) -> torch.Tensor:
 
 def col_count(indptr: torch.Tensor, column_ids: Optional[torch.Tensor],
               fanout: int, replace: bool,
-              num_items: Optional[int] = None, count: Optional[_Count] = None) -> torch.Tensor:
+              num_items: Optional[int] = None, count: Optional[_Count] = None,
+              col_span: Optional[torch.Tensor] = None) -> torch.Tensor:
     """sub_indptr[num_items + 1] for slicing (fanout < 0) or sampling.  With
-    `count` the edge total is also on its way to the host when this returns."""
+    `count` the edge total is also on its way to the host when this returns;
+    `col_span` (int64[num_items]) receives every column's start and degree in one
+    word, which the sampler fills take in place of the column pointer."""
     indptr = _i64t(indptr, "indptr")
     num_cols = indptr.numel() - 1
     if column_ids is not None:
@@ -278,7 +281,7 @@ def col_count(indptr: torch.Tensor, column_ids: Optional[torch.Tensor],
     check(lib().gs_csc_col_count(_ptr(indptr), num_cols, _ptr(column_ids),
                                  num_items, fanout, int(replace),
                                  sub_indptr.data_ptr(), count.mirror() if count else None,
-                                 ws.data_ptr(), ws.numel(), _stream()))
+                                 _ptr(col_span), ws.data_ptr(), ws.numel(), _stream()))
     if count:
         count.arm()
     return sub_indptr
@@ -326,12 +329,15 @@ def col_slice_values(indptr, column_ids, sub_indptr, values):
 
 
 def sample_uniform(indptr, indices, column_ids, fanout, replace=False,
-                   algo=ALGO_AUTO, seed=7777, call_id=0, with_coo=True, col_batch_ptr=None):
+                   algo=ALGO_AUTO, seed=7777, call_id=0, with_coo=True, col_batch_ptr=None,
+                   spans=True):
     """Uniform per-column sampling, fused with the slice when column_ids is given.
 
     `indices` may be the matrix's int32 copy of the row ids (same outputs).
     `col_batch_ptr` (offsets that cut the columns into batches): coo_col then holds
     every column's place inside its batch instead of its place in the call.
+    `spans`: the count pass leaves every column's start and degree for the fill
+    pass, which then does not look the column pointer up again (same outputs).
 
     -> (sub_indptr, coo_col | None, sub_indices, select_index)
     """
@@ -350,17 +356,18 @@ def sample_uniform(indptr, indices, column_ids, fanout, replace=False,
     if col_batch_ptr is not None:
         col_batch_ptr = _i64t(col_batch_ptr, "col_batch_ptr")
     count = _Count()
-    sub_indptr = col_count(indptr, column_ids, fanout, replace, n, count)
+    dev = indptr.device
+    col_span = torch.empty(n, dtype=torch.int64, device=dev) if spans else None
+    sub_indptr = col_count(indptr, column_ids, fanout, replace, n, count, col_span)
     bound = n * fanout                       # no column yields more than fanout edges
     size = bound if bound <= _BOUND_LIMIT else count.get()
-    dev = indptr.device
     out_idx = torch.empty(size, dtype=torch.int64, device=dev)
     out_sel = torch.empty(size, dtype=torch.int64, device=dev)
     out_col = torch.empty(size, dtype=torch.int64, device=dev) if with_coo else None
     if size > 0:
         check(fill(
             _ptr(indptr), num_cols, _ptr(indices), _ptr(column_ids), n, fanout,
-            int(replace), algo, seed, call_id, sub_indptr.data_ptr(),
+            int(replace), algo, seed, call_id, sub_indptr.data_ptr(), _ptr(col_span),
             _ptr(out_col), out_idx.data_ptr(), out_sel.data_ptr(), _ptr(col_batch_ptr),
             col_batch_ptr.numel() - 1 if col_batch_ptr is not None else 0, _stream()))
     nnz = count.get()
@@ -777,13 +784,13 @@ def probe_line_gather(table, num_picks, salt=0, ordered=False, out=None):
 
 
 def probe_sample_uniform(indptr, indices32, column_ids, fanout, variant, sub_indptr, outs,
-                         probe_degree=0, seed=7777, call_id=0):
+                         probe_degree=0, seed=7777, call_id=0, col_span=None):
     """One launch of the packed uniform sampler with parts switched off (see
     gs_probe_sample_uniform); outs = (coo_col | None, rows, select) preallocated."""
     check(lib().gs_probe_sample_uniform(
         _ptr(indptr), indptr.numel() - 1, indices32.data_ptr(), _ptr(column_ids),
         column_ids.numel(), fanout, variant, probe_degree, seed, call_id, _ptr(sub_indptr),
-        _ptr(outs[0]), outs[1].data_ptr(), outs[2].data_ptr(), _stream()))
+        _ptr(col_span), _ptr(outs[0]), outs[1].data_ptr(), outs[2].data_ptr(), _stream()))
 
 
 # --------------------------------------------------------- weighted sampling
@@ -853,7 +860,7 @@ def sample_weighted(indptr, indices, probs, column_ids, fanout, replace=False, s
     if nnz > 0:
         check(lib().gs_csc_col_sample_weighted_fill(
             _ptr(indptr), num_cols, _ptr(indices), probs.data_ptr(), None, _ptr(column_ids),
-            n, fanout, int(replace), seed, call_id, sub_indptr.data_ptr(), _ptr(cdf_off),
+            n, fanout, int(replace), seed, call_id, sub_indptr.data_ptr(), None, _ptr(cdf_off),
             _ptr(scratch), _ptr(out_col), out_idx.data_ptr(), out_sel.data_ptr(),
             _ptr(col_batch_ptr), col_batch_ptr.numel() - 1 if col_batch_ptr is not None else 0,
             _stream()))
@@ -861,7 +868,7 @@ def sample_weighted(indptr, indices, probs, column_ids, fanout, replace=False, s
 
 
 def _sample_weighted_cdf(indptr, indices, cdf, column_ids, fanout, replace, seed, call_id,
-                         with_coo, col_batch_ptr=None):
+                         with_coo, col_batch_ptr=None, spans=True):
     num_cols = indptr.numel() - 1
     dev = indptr.device
     if column_ids is not None:
@@ -870,7 +877,8 @@ def _sample_weighted_cdf(indptr, indices, cdf, column_ids, fanout, replace, seed
     else:
         n = num_cols
     count = _Count()
-    sub_indptr = col_count(indptr, column_ids, fanout, replace, n, count)
+    col_span = torch.empty(n, dtype=torch.int64, device=dev) if spans else None
+    sub_indptr = col_count(indptr, column_ids, fanout, replace, n, count, col_span)
     bound = n * fanout
     size = bound if bound <= _BOUND_LIMIT else count.get()
     out_idx = torch.empty(size, dtype=torch.int64, device=dev)
@@ -879,8 +887,8 @@ def _sample_weighted_cdf(indptr, indices, cdf, column_ids, fanout, replace, seed
     if size > 0:
         check(lib().gs_csc_col_sample_weighted_fill(
             _ptr(indptr), num_cols, _ptr(indices), None, cdf.data_ptr(), _ptr(column_ids), n,
-            fanout, int(replace), seed, call_id, sub_indptr.data_ptr(), None, None,
-            _ptr(out_col), out_idx.data_ptr(), out_sel.data_ptr(), _ptr(col_batch_ptr),
+            fanout, int(replace), seed, call_id, sub_indptr.data_ptr(), _ptr(col_span), None,
+            None, _ptr(out_col), out_idx.data_ptr(), out_sel.data_ptr(), _ptr(col_batch_ptr),
             col_batch_ptr.numel() - 1 if col_batch_ptr is not None else 0, _stream()))
     nnz = count.get()
     return (sub_indptr, out_col[:nnz] if with_coo else None, out_idx[:nnz], out_sel[:nnz])

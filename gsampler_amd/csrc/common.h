@@ -366,6 +366,35 @@ __device__ __forceinline__ int64_t column_degree(const int64_t* indptr,
   return indptr[c + 1] - b;
 }
 
+// What the count pass of a slice or a sampler can leave behind for the fill pass
+// of the same columns, one word per requested column: where the column starts
+// (low 40 bits) and how long it is (24 bits above), so that the fill pass reads
+// its columns' spans in a stream instead of looking up each column's pointer pair
+// again -- a 128-byte line of the matrix's column pointer per column.  A start or
+// a length that does not fit is kSpanLookUp: look the pair up after all.
+constexpr int kSpanStartBits = 40;
+constexpr uint64_t kSpanLookUp = ~0ull;
+__device__ __forceinline__ int64_t pack_span(int64_t start, int64_t deg) {
+  const bool fits = ((uint64_t)start >> kSpanStartBits) == 0 && deg >= 0 && deg < (1 << 24) - 1;
+  return (int64_t)(fits ? ((uint64_t)deg << kSpanStartBits) | (uint64_t)start : kSpanLookUp);
+}
+// Degree and start of requested column `item`: from its span when there is one,
+// else from the column pointer.
+__device__ __forceinline__ int64_t column_span(const int64_t* __restrict__ col_span,
+                                               const int64_t* __restrict__ column_ids,
+                                               const int64_t* __restrict__ indptr,
+                                               int64_t num_cols, int64_t item,
+                                               int64_t* in_start) {
+  if (col_span != nullptr) {
+    const uint64_t span = (uint64_t)col_span[item];
+    if (span != kSpanLookUp) {
+      *in_start = (int64_t)(span & ((1ull << kSpanStartBits) - 1ull));
+      return (int64_t)(span >> kSpanStartBits);
+    }
+  }
+  return column_degree(indptr, num_cols, column_ids ? column_ids[item] : item, in_start);
+}
+
 }  // namespace gs
 
 #endif  // GSAMPLER_CSRC_COMMON_H_

@@ -82,7 +82,6 @@ __global__ __launch_bounds__(kCooThreads) void coosort_count_kernel(
   if ((reinterpret_cast<uintptr_t>(major) & 15) == 0) {  // two ids a load
     const longlong2* pairs = reinterpret_cast<const longlong2*>(major);
     const int64_t num_pairs = n >> 1;
-#pragma unroll 4
     for (int64_t q = first; q < num_pairs; q += stride) {
       const longlong2 v = pairs[q];
       count((uint32_t)v.x);
@@ -90,7 +89,6 @@ __global__ __launch_bounds__(kCooThreads) void coosort_count_kernel(
     }
     if (first == 0 && (n & 1)) count((uint32_t)major[n - 1]);
   } else {
-#pragma unroll 4
     for (int64_t e = first; e < n; e += stride) count((uint32_t)major[e]);
   }
   for (int64_t q = first; q < clear_quads; q += stride) clear[q] = make_uint4(0, 0, 0, 0);

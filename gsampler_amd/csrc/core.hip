@@ -280,7 +280,7 @@ int gs_copy_i64(const int64_t* src, int64_t n, int64_t* dst, gs_stream_t stream)
 
 const char* gs_last_error(void) { return gs::g_last_error.c_str(); }
 
-int gs_abi_version(void) { return 6; }
+int gs_abi_version(void) { return 7; }
 
 void gs_profile_enable(int on) {
   std::lock_guard<std::mutex> lock(gs::g_prof_mutex);

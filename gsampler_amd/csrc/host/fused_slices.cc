@@ -30,7 +30,7 @@ const Graph::SliceOffsets& Graph::slice_offsets_for(const torch::Tensor& cols) {
   torch::Tensor ws = new_workspace(gs_scan_workspace_bytes(n + 1), m.indptr);
   AsyncCount count = AsyncCount::mirrored();
   GS_CALL(gs_csc_col_count(cptr(m.indptr), num_major, cptr(cols), n, -1, 0,
-                           mptr(so->sub_indptr), count.mirror(), ws.data_ptr(), ws.numel(),
+                           mptr(so->sub_indptr), count.mirror(), nullptr, ws.data_ptr(), ws.numel(),
                            cur_stream()));
   count.arm();
   so->nnz = count.get();

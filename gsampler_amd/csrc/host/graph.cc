@@ -198,7 +198,7 @@ MajorResult major_slice(const Compressed& m, const torch::Tensor& picked,
   r.indptr = new_ids(n + 1, m.indptr);
   torch::Tensor ws = new_workspace(gs_scan_workspace_bytes(n + 1), m.indptr);
   GS_CALL(gs_csc_col_count(cptr(m.indptr), num_major, cptr(picked), n, -1, 0,
-                           mptr(r.indptr), nullptr, ws.data_ptr(), ws.numel(),
+                           mptr(r.indptr), nullptr, nullptr, ws.data_ptr(), ws.numel(),
                            cur_stream()));
   const int64_t nnz = read_last(r.indptr);
   r.minor_ids = new_ids(nnz, m.indptr);
@@ -251,9 +251,12 @@ MajorResult major_sample_uniform(const Compressed& m,
   // No column yields more than fanout edges: size the outputs by that bound,
   // launch, and trim when the count has arrived.
   EdgeCount count;
+  // the count pass leaves every column's start and degree for the fill pass, which
+  // then does not look the column pointer up a second time
+  torch::Tensor col_span = new_ids(n, m.indptr);
   GS_CALL(gs_csc_col_count(cptr(m.indptr), num_major,
                            fused ? cptr(picked) : nullptr, n, fanout,
-                           replace ? 1 : 0, mptr(r.indptr), count.mirror(),
+                           replace ? 1 : 0, mptr(r.indptr), count.mirror(), mptr(col_span),
                            ws.data_ptr(), ws.numel(), cur_stream()));
   count.arm(r.indptr);
   const int64_t bound = n * fanout;
@@ -275,13 +278,15 @@ MajorResult major_sample_uniform(const Compressed& m,
     GS_CALL(gs_csc_col_sample_uniform_fill_i32(
         cptr(m.indptr), num_major, narrow.data_ptr<int32_t>(),
         fused ? cptr(picked) : nullptr, n, fanout, replace ? 1 : 0, (int)rs.algo,
-        rs.seed, next_call_id(), cptr(r.indptr), out_col, mptr(r.minor_ids), mptr(r.select),
+        rs.seed, next_call_id(), cptr(r.indptr), cptr(col_span), out_col, mptr(r.minor_ids),
+        mptr(r.select),
         col_batch_ptr, col_batches, cur_stream()));
   } else {
     GS_CALL(gs_csc_col_sample_uniform_fill(
         cptr(m.indptr), num_major, cptr(m.indices),
         fused ? cptr(picked) : nullptr, n, fanout, replace ? 1 : 0, (int)rs.algo,
-        rs.seed, next_call_id(), cptr(r.indptr), out_col, mptr(r.minor_ids), mptr(r.select),
+        rs.seed, next_call_id(), cptr(r.indptr), cptr(col_span), out_col, mptr(r.minor_ids),
+        mptr(r.select),
         col_batch_ptr, col_batches, cur_stream()));
   }
   const int64_t nnz = count.get();

@@ -37,7 +37,7 @@ GraphAndIndex Graph::SamplingProbs(int64_t axis, torch::Tensor edge_probs,
   r.indptr = new_ids(n + 1, m.indptr);
   torch::Tensor ws = new_workspace(gs_scan_workspace_bytes(n + 1), m.indptr);
   GS_CALL(gs_csc_col_count(cptr(m.indptr), n, nullptr, n, fanout, replace ? 1 : 0,
-                           mptr(r.indptr), nullptr, ws.data_ptr(), ws.numel(),
+                           mptr(r.indptr), nullptr, nullptr, ws.data_ptr(), ws.numel(),
                            cur_stream()));
   const int64_t nnz = read_last(r.indptr);
   r.minor_ids = new_ids(nnz, m.indptr);
@@ -49,7 +49,7 @@ GraphAndIndex Graph::SamplingProbs(int64_t axis, torch::Tensor edge_probs,
   GS_CALL(gs_csc_col_sample_weighted_fill(
       cptr(m.indptr), n, cptr(m.indices), probs.data_ptr<float>(), nullptr,
       nullptr, n, fanout, replace ? 1 : 0, rs.seed, take_call_id(), cptr(r.indptr),
-      nullptr,
+      nullptr, nullptr,
       replace ? scratch.data_ptr() : nullptr,
       with_coo ? mptr(r.major_ids) : nullptr, mptr(r.minor_ids), mptr(r.select),
       nullptr, 0, cur_stream()));
@@ -106,9 +106,10 @@ GraphAndIndex Graph::FusedSlicingSamplingProbs(int64_t axis, torch::Tensor seeds
   r.indptr = new_ids(n + 1, m.indptr);
   torch::Tensor ws = new_workspace(gs_scan_workspace_bytes(n + 1), m.indptr);
   EdgeCount count;
+  torch::Tensor col_span = new_ids(n, m.indptr);  // the columns' starts and degrees, for the fill pass
   GS_CALL(gs_csc_col_count(cptr(m.indptr), num_major, cptr(seeds), n, fanout,
-                           replace ? 1 : 0, mptr(r.indptr), count.mirror(), ws.data_ptr(),
-                           ws.numel(), cur_stream()));
+                           replace ? 1 : 0, mptr(r.indptr), count.mirror(), mptr(col_span),
+                           ws.data_ptr(), ws.numel(), cur_stream()));
   count.arm(r.indptr);
   const int64_t bound = n * fanout;
   const int64_t size = bound <= kBoundLimit ? bound : count.get();
@@ -123,7 +124,8 @@ GraphAndIndex Graph::FusedSlicingSamplingProbs(int64_t axis, torch::Tensor seeds
   const RandomState& rs = random_state();
   GS_CALL(gs_csc_col_sample_weighted_fill(
       cptr(m.indptr), num_major, cptr(m.indices), nullptr, cptr(cdf), cptr(seeds), n,
-      fanout, replace ? 1 : 0, rs.seed, take_call_id(), cptr(r.indptr), nullptr, nullptr,
+      fanout, replace ? 1 : 0, rs.seed, take_call_id(), cptr(r.indptr), cptr(col_span),
+      nullptr, nullptr,
       with_coo ? mptr(r.major_ids) : label_cols ? mptr(col_labels) : nullptr,
       mptr(r.minor_ids), mptr(r.select), label_cols ? cptr(hint.col_bptr) : nullptr,
       label_cols ? hint.col_bptr.numel() - 1 : 0, cur_stream()));

@@ -120,7 +120,7 @@ __global__ __launch_bounds__(kBlock) void sample_uniform_packed_kernel(
     int64_t num_items, int fanout, int cols_per_wave, int replace, PhiloxKey key,
     const int64_t* __restrict__ sub_indptr, int64_t* __restrict__ out_coo_col,
     int64_t* __restrict__ out_indices, int64_t* __restrict__ out_select,
-    ColumnLabels labels, int64_t probe_degree = 0) {
+    ColumnLabels labels, const int64_t* __restrict__ col_span, int64_t probe_degree = 0) {
   const int wave_lane = threadIdx.x & (kWave - 1);
   const int group = wave_lane / fanout;
   const int lane = wave_lane - group * fanout;
@@ -130,16 +130,15 @@ __global__ __launch_bounds__(kBlock) void sample_uniform_packed_kernel(
   const int64_t wave = (block * kBlock + threadIdx.x) / kWave;
   const int64_t item = wave * cols_per_wave + group;
   if (group >= cols_per_wave || item >= num_items) return;  // whole groups leave together
-  const int64_t c = column_ids ? column_ids[item] : item;
   // (asked for here, so that its loads travel with the ones below)
   const int64_t col_label = out_coo_col ? labels.of_near(item, wave * cols_per_wave) : item;
   int64_t in_start;
   int64_t deg;
   if (kProbe & kProbeNoIndptr) {
     deg = probe_degree;
-    in_start = c * probe_degree;
+    in_start = (column_ids ? column_ids[item] : item) * probe_degree;
   } else {
-    deg = column_degree(indptr, num_cols, c, &in_start);
+    deg = column_span(col_span, column_ids, indptr, num_cols, item, &in_start);
   }
   if (deg == 0) return;
   const int64_t out_start = (kProbe & kProbeNoIndptr) ? item * fanout : sub_indptr[item];
@@ -199,13 +198,13 @@ __global__ __launch_bounds__(kBlock) void sample_uniform_strided_kernel(
     const IdxT* __restrict__ indices, const int64_t* __restrict__ column_ids,
     int64_t num_items, int64_t fanout, int replace, PhiloxKey key,
     const int64_t* __restrict__ sub_indptr, int64_t* __restrict__ out_coo_col,
-    int64_t* __restrict__ out_indices, int64_t* __restrict__ out_select, ColumnLabels labels) {
+    int64_t* __restrict__ out_indices, int64_t* __restrict__ out_select, ColumnLabels labels,
+    const int64_t* __restrict__ col_span) {
   const int lane = threadIdx.x & (G - 1);
   const int64_t item = ((int64_t)blockIdx.x * kBlock + threadIdx.x) / G;
   if (item >= num_items) return;  // whole groups leave together
-  const int64_t c = column_ids ? column_ids[item] : item;
   int64_t in_start;
-  const int64_t deg = column_degree(indptr, num_cols, c, &in_start);
+  const int64_t deg = column_span(col_span, column_ids, indptr, num_cols, item, &in_start);
   if (deg == 0) return;
   sample_column_generic<G, IdxT>(lane, item, out_coo_col ? labels.of(item) : item, in_start, deg,
                                  sub_indptr[item], indices, fanout, replace, key, out_coo_col,
@@ -217,13 +216,14 @@ static int launch_sample_strided(const int64_t* indptr, int64_t num_cols, const 
                                  const int64_t* column_ids, int64_t num_items, int64_t fanout,
                                  int replace, PhiloxKey key, const int64_t* sub_indptr,
                                  int64_t* out_coo_col, int64_t* out_indices, int64_t* out_select,
-                                 ColumnLabels labels, hipStream_t stream) {
+                                 ColumnLabels labels, const int64_t* col_span,
+                                 hipStream_t stream) {
   const int64_t blocks = ceil_div(num_items * G, kBlock);
   GS_LAUNCH("sample_uniform", stream,
             (sample_uniform_strided_kernel<G, IdxT>)<<<dim3((unsigned)blocks), dim3(kBlock), 0,
                                                       stream>>>(
                 indptr, num_cols, indices, column_ids, num_items, fanout, replace, key,
-                sub_indptr, out_coo_col, out_indices, out_select, labels));
+                sub_indptr, out_coo_col, out_indices, out_select, labels, col_span));
   return GS_OK;
 }
 
@@ -234,10 +234,10 @@ template <typename IdxT>
 static int sample_uniform_fill(const int64_t* indptr, int64_t num_cols, const IdxT* indices,
                                const int64_t* column_ids, int64_t num_items, int64_t fanout,
                                int replace, int algo, uint64_t seed, uint64_t call_id,
-                               const int64_t* sub_indptr, int64_t* out_coo_col,
-                               int64_t* out_indices, int64_t* out_select,
-                               const int64_t* col_batch_ptr, int64_t num_col_batches,
-                               gs_stream_t stream) {
+                               const int64_t* sub_indptr, const int64_t* col_span,
+                               int64_t* out_coo_col, int64_t* out_indices,
+                               int64_t* out_select, const int64_t* col_batch_ptr,
+                               int64_t num_col_batches, gs_stream_t stream) {
   GS_REQUIRE(num_items >= 0 && num_cols >= 0, "sample_uniform: negative size");
   GS_REQUIRE(col_batch_ptr == nullptr || num_col_batches >= 1,
              "sample_uniform: col_batch_ptr given but num_col_batches = %lld",
@@ -268,12 +268,13 @@ static int sample_uniform_fill(const int64_t* indptr, int64_t num_cols, const Id
               sample_uniform_packed_kernel<IdxT><<<dim3((unsigned)(ceil_div(ceil_div(waves * kWave, kBlock), 8) * 8)),
                                                    dim3(kBlock), 0, s>>>(
                   indptr, num_cols, indices, column_ids, num_items, (int)fanout, cols_per_wave,
-                  replace, key, sub_indptr, out_coo_col, out_indices, out_select, labels));
+                  replace, key, sub_indptr, out_coo_col, out_indices, out_select, labels,
+                  col_span));
     return GS_OK;
   }
 #define GS_SAMPLE_ARGS                                                          \
   indptr, num_cols, indices, column_ids, num_items, fanout, replace, key, sub_indptr, \
-      out_coo_col, out_indices, out_select, labels, s
+      out_coo_col, out_indices, out_select, labels, col_span, s
   if (fanout <= 8) return launch_sample_strided<8, IdxT>(GS_SAMPLE_ARGS);
   if (fanout <= 16) return launch_sample_strided<16, IdxT>(GS_SAMPLE_ARGS);
   if (fanout <= 32) return launch_sample_strided<32, IdxT>(GS_SAMPLE_ARGS);
@@ -286,11 +287,11 @@ extern "C" int gs_csc_col_sample_uniform_fill(
     const int64_t* indptr, int64_t num_cols, const int64_t* indices,
     const int64_t* column_ids, int64_t num_items, int64_t fanout, int replace,
     int algo, uint64_t seed, uint64_t call_id, const int64_t* sub_indptr,
-    int64_t* out_coo_col, int64_t* out_indices, int64_t* out_select,
+    const int64_t* col_span, int64_t* out_coo_col, int64_t* out_indices, int64_t* out_select,
     const int64_t* col_batch_ptr, int64_t num_col_batches, gs_stream_t stream) {
   return gs::sample_uniform_fill<int64_t>(indptr, num_cols, indices, column_ids, num_items,
                                           fanout, replace, algo, seed, call_id, sub_indptr,
-                                          out_coo_col, out_indices, out_select, col_batch_ptr,
+                                          col_span, out_coo_col, out_indices, out_select, col_batch_ptr,
                                           num_col_batches, stream);
 }
 
@@ -298,12 +299,12 @@ extern "C" int gs_csc_col_sample_uniform_fill_i32(
     const int64_t* indptr, int64_t num_cols, const int32_t* indices32,
     const int64_t* column_ids, int64_t num_items, int64_t fanout, int replace,
     int algo, uint64_t seed, uint64_t call_id, const int64_t* sub_indptr,
-    int64_t* out_coo_col, int64_t* out_indices, int64_t* out_select,
+    const int64_t* col_span, int64_t* out_coo_col, int64_t* out_indices, int64_t* out_select,
     const int64_t* col_batch_ptr, int64_t num_col_batches, gs_stream_t stream) {
   GS_REQUIRE(indices32 != nullptr, "sample_uniform_i32: null indices");
   return gs::sample_uniform_fill<int32_t>(indptr, num_cols, indices32, column_ids, num_items,
                                           fanout, replace, algo, seed, call_id, sub_indptr,
-                                          out_coo_col, out_indices, out_select, col_batch_ptr,
+                                          col_span, out_coo_col, out_indices, out_select, col_batch_ptr,
                                           num_col_batches, stream);
 }
 
@@ -316,7 +317,8 @@ extern "C" int gs_probe_sample_uniform(
     const int64_t* indptr, int64_t num_cols, const int32_t* indices32,
     const int64_t* column_ids, int64_t num_items, int64_t fanout, int variant,
     int64_t probe_degree, uint64_t seed, uint64_t call_id, const int64_t* sub_indptr,
-    int64_t* out_coo_col, int64_t* out_indices, int64_t* out_select, gs_stream_t stream) {
+    const int64_t* col_span, int64_t* out_coo_col, int64_t* out_indices, int64_t* out_select,
+    gs_stream_t stream) {
   using namespace gs;
   GS_REQUIRE(num_items > 0 && fanout >= 1 && fanout <= kWave, "probe_sample_uniform: bad size");
   GS_REQUIRE(indptr && indices32 && column_ids && sub_indptr && out_indices && out_select,
@@ -334,7 +336,7 @@ extern "C" int gs_probe_sample_uniform(
               (sample_uniform_packed_kernel<int32_t, V>)<<<grid, dim3(kBlock), 0, s>>>(       \
                   indptr, num_cols, indices32, column_ids, num_items, (int)fanout,            \
                   cols_per_wave, 0, key, sub_indptr, out_coo_col, out_indices, out_select,    \
-                  ColumnLabels{nullptr, 0}, probe_degree));                                   \
+                  ColumnLabels{nullptr, 0}, col_span, probe_degree));                         \
     return GS_OK;
   switch (variant) {
     GS_PROBE_CASE(0)

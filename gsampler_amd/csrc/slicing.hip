@@ -42,7 +42,8 @@ constexpr int kCountItems = kScanTile / kCountThreads;
 __global__ __launch_bounds__(kCountThreads) void col_count_kernel(
     const int64_t* __restrict__ indptr, int64_t num_cols,
     const int64_t* __restrict__ column_ids, int64_t num_items, int64_t fanout,
-    int replace, int64_t* __restrict__ counts, int64_t* __restrict__ tile_sums) {
+    int replace, int64_t* __restrict__ counts, int64_t* __restrict__ tile_sums,
+    int64_t* __restrict__ col_span) {
   __shared__ int64_t smem[kCountThreads / kWave + 1];
   const int64_t base = (int64_t)blockIdx.x * kScanTile + threadIdx.x;
   int64_t cnt[kCountItems], sum = 0;
@@ -54,6 +55,7 @@ __global__ __launch_bounds__(kCountThreads) void col_count_kernel(
       int64_t in_start;
       const int64_t deg =
           column_degree(indptr, num_cols, column_ids ? column_ids[i] : i, &in_start);
+      if (col_span) col_span[i] = pack_span(in_start, deg);
       if (fanout < 0)
         cnt[k] = deg;
       else if (replace)
@@ -82,7 +84,8 @@ constexpr int64_t kSmallCountItems = (int64_t)kCountThreads * kSmallCountPer - 1
 __global__ __launch_bounds__(kCountThreads) void col_count_small_kernel(
     const int64_t* __restrict__ indptr, int64_t num_cols,
     const int64_t* __restrict__ column_ids, int64_t num_items, int64_t fanout,
-    int replace, int64_t* __restrict__ sub_indptr, int64_t* total_mirror) {
+    int replace, int64_t* __restrict__ sub_indptr, int64_t* total_mirror,
+    int64_t* __restrict__ col_span) {
   __shared__ int64_t smem[kCountThreads / kWave + 1];
   // thread t owns columns t * 8 .. t * 8 + 7: its prefix sums leave in one run
   const int64_t base = (int64_t)threadIdx.x * kSmallCountPer;
@@ -95,6 +98,7 @@ __global__ __launch_bounds__(kCountThreads) void col_count_small_kernel(
       int64_t in_start;
       const int64_t deg =
           column_degree(indptr, num_cols, column_ids ? column_ids[i] : i, &in_start);
+      if (col_span) col_span[i] = pack_span(in_start, deg);
       if (fanout < 0)
         cnt[k] = deg;
       else if (replace)
@@ -293,7 +297,7 @@ int gs_csc_col_slice_values(const int64_t* indptr, const int64_t* column_ids, in
 int gs_csc_col_count(const int64_t* indptr, int64_t num_cols,
                      const int64_t* column_ids, int64_t num_items,
                      int64_t fanout, int replace, int64_t* sub_indptr,
-                     int64_t* total_mirror, void* workspace,
+                     int64_t* total_mirror, int64_t* out_col_span, void* workspace,
                      size_t workspace_bytes, gs_stream_t stream) {
   using namespace gs;
   GS_REQUIRE(num_items >= 0 && num_cols >= 0, "col_count: negative size");
@@ -312,14 +316,14 @@ int gs_csc_col_count(const int64_t* indptr, int64_t num_cols,
     GS_LAUNCH("col_count", s,
               col_count_small_kernel<<<dim3(1), dim3(kCountThreads), 0, s>>>(
                   indptr, num_cols, column_ids, num_items, fanout, replace, sub_indptr,
-                  total_mirror));
+                  total_mirror, out_col_span));
     return GS_OK;
   }
   GS_LAUNCH("col_count", s,
             col_count_kernel<<<dim3((unsigned)ceil_div(n, kScanTile)), dim3(kCountThreads),
                                0, s>>>(indptr, num_cols, column_ids, num_items,
                                        fanout, replace, sub_indptr,
-                                       (int64_t*)workspace));
+                                       (int64_t*)workspace, out_col_span));
   return exclusive_scan_i64(sub_indptr, sub_indptr, n, workspace,
                             workspace_bytes, s, /*sums_ready=*/true, total_mirror);
 }
@@ -338,7 +342,7 @@ int gs_csc_col_count_static(const int64_t* indptr, int64_t num_cols,
   const int rc = static_scratch(&ws);
   if (rc != GS_OK) return rc;
   return gs_csc_col_count(indptr, num_cols, column_ids, num_items, fanout, replace,
-                          sub_indptr, nullptr, ws,
+                          sub_indptr, nullptr, nullptr, ws,
                           (size_t)kStaticScanTiles * sizeof(int64_t), stream);
 }
 

@@ -474,7 +474,8 @@ __global__ __launch_bounds__(kBlock) void sample_weighted_cdf_kernel(
     const int64_t* __restrict__ column_ids, int64_t num_items, int fanout,
     int replace, PhiloxKey key, const int64_t* __restrict__ sub_indptr,
     int64_t* __restrict__ out_coo_col, int64_t* __restrict__ out_indices,
-    int64_t* __restrict__ out_select, ColumnLabels labels, int mode) {
+    int64_t* __restrict__ out_select, ColumnLabels labels,
+    const int64_t* __restrict__ col_span, int mode) {
   const int64_t item = (int64_t)blockIdx.x * kBlock + threadIdx.x;
   if (item >= num_items) return;
   // (asked for here, so that its loads travel with the ones below)
@@ -482,9 +483,8 @@ __global__ __launch_bounds__(kBlock) void sample_weighted_cdf_kernel(
       out_coo_col ? labels.of_near(item, item - lane_id()) : item;
   const int row_bits = (int)cdf[0];  // the same word for every lane: a scalar load
   const uint64_t row_mask = row_bits ? (~0ull >> (64 - row_bits)) : 0ull;
-  const int64_t c = column_ids ? column_ids[item] : item;
   int64_t in_start;
-  const int64_t deg = column_degree(indptr, num_cols, c, &in_start);
+  const int64_t deg = column_span(col_span, column_ids, indptr, num_cols, item, &in_start);
   if (deg == 0) return;
   const int64_t out_start = sub_indptr[item];
   const uint64_t* col = cdf + in_start;  // col[j], 1 <= j <= deg: entry of item j - 1
@@ -621,13 +621,13 @@ static int launch_weighted_cdf(const int64_t* indptr, int64_t num_cols,
                                int fanout, int replace, PhiloxKey key,
                                const int64_t* sub_indptr, int64_t* out_coo_col,
                                int64_t* out_indices, int64_t* out_select,
-                               ColumnLabels labels, hipStream_t s) {
+                               ColumnLabels labels, const int64_t* col_span, hipStream_t s) {
   GS_LAUNCH("sample_weighted_cdf", s,
             sample_weighted_cdf_kernel<KMAX><<<dim3((unsigned)ceil_div(num_items, kBlock)),
                                                dim3(kBlock), 0, s>>>(
                 indptr, num_cols, indices, (const uint64_t*)cdf, column_ids, num_items,
                 fanout, replace, key, sub_indptr, out_coo_col, out_indices, out_select, labels,
-                kCdfSearchMode));
+                col_span, kCdfSearchMode));
   return GS_OK;
 }
 
@@ -1218,7 +1218,8 @@ int gs_csc_col_sample_weighted_fill(
     const float* probs, const int64_t* cdf,
     const int64_t* column_ids, int64_t num_items,
     int64_t fanout, int replace, uint64_t seed, uint64_t call_id,
-    const int64_t* sub_indptr, const int64_t* cdf_offsets, void* cdf_scratch,
+    const int64_t* sub_indptr, const int64_t* col_span, const int64_t* cdf_offsets,
+    void* cdf_scratch,
     int64_t* out_coo_col, int64_t* out_indices, int64_t* out_select,
     const int64_t* col_batch_ptr, int64_t num_col_batches, gs_stream_t stream) {
   using namespace gs;
@@ -1243,7 +1244,7 @@ int gs_csc_col_sample_weighted_fill(
     GS_REQUIRE(fanout <= INT32_MAX, "sample_weighted: fanout too large");
 #define GS_CDF_ARGS                                                              \
   indptr, num_cols, indices, cdf, column_ids, num_items, (int)fanout, replace, \
-      key, sub_indptr, out_coo_col, out_indices, out_select, labels, s
+      key, sub_indptr, out_coo_col, out_indices, out_select, labels, col_span, s
     if (fanout <= 8) return launch_weighted_cdf<8>(GS_CDF_ARGS);
     if (fanout <= 16) return launch_weighted_cdf<16>(GS_CDF_ARGS);
     if (fanout <= 32) return launch_weighted_cdf<32>(GS_CDF_ARGS);

@@ -112,6 +112,13 @@ int gs_exclusive_scan_i64(const int64_t* in, int64_t* out, int64_t n,
  * which the kernel that produces it also stores to *total_mirror when that is
  * given (a word of pinned host memory: the host then has the total as soon as
  * the stream reaches that point, without a copy of its own).
+ * out_col_span (nullable, num_items words): where each requested column starts
+ * in the matrix and how long it is, in one word (start in the low 40 bits, degree
+ * in the 24 above; all ones when either does not fit).  The sampler fills below
+ * take it as `col_span` and then read their columns' spans in a stream instead
+ * of looking up every column's pointer pair a second time -- a 128-byte line of
+ * `indptr` per column, a quarter of all lines a uniform fan-out-5 layer visits.
+ * It is valid for the same indptr and column_ids only.
  * Stands in for the degree lambda + scan of
  *   src/cuda/slicing.cu:133-141, src/cuda/sampling.cu:112-124,
  *   src/cuda/fusion/slice_sampling.cu:111-124, src/cuda/sampling_probs.cu:201-216.
@@ -120,7 +127,7 @@ int gs_exclusive_scan_i64(const int64_t* in, int64_t* out, int64_t n,
 int gs_csc_col_count(const int64_t* indptr, int64_t num_cols,
                      const int64_t* column_ids, int64_t num_items,
                      int64_t fanout, int replace, int64_t* sub_indptr,
-                     int64_t* total_mirror, void* workspace,
+                     int64_t* total_mirror, int64_t* out_col_span, void* workspace,
                      size_t workspace_bytes, gs_stream_t stream);
 
 /* ------------------------------------------------------------------------
@@ -178,7 +185,10 @@ int gs_csc_col_slice_values(const int64_t* indptr, const int64_t* column_ids,
  * the same fanout / replace.  Columns with degree <= fanout are copied in
  * their original order (no replace).  `algo` is one of GS_ALGO_*.  `indices`
  * may be NULL, meaning "the edge position itself" (out_indices then repeats
- * out_select).  out_coo_col (nullable) receives the column of every edge: the
+ * out_select).  col_span (nullable) is what gs_csc_col_count left in
+ * out_col_span for the same indptr and column_ids: with it neither of the two is
+ * read (except for columns whose span did not fit a word); results are the same.
+ * out_coo_col (nullable) receives the column of every edge: the
  * position i of its column among the call's columns or, when col_batch_ptr
  * (num_col_batches + 1 offsets that cut the call's columns into batches, nullable)
  * is given, i - col_batch_ptr[batch of i], the column's position inside its
@@ -195,7 +205,7 @@ int gs_csc_col_sample_uniform_fill(const int64_t* indptr, int64_t num_cols,
                                    const int64_t* column_ids, int64_t num_items,
                                    int64_t fanout, int replace, int algo,
                                    uint64_t seed, uint64_t call_id,
-                                   const int64_t* sub_indptr,
+                                   const int64_t* sub_indptr, const int64_t* col_span,
                                    int64_t* out_coo_col, int64_t* out_indices,
                                    int64_t* out_select,
                                    const int64_t* col_batch_ptr,
@@ -212,6 +222,7 @@ int gs_csc_col_sample_uniform_fill_i32(const int64_t* indptr, int64_t num_cols,
                                        int replace, int algo, uint64_t seed,
                                        uint64_t call_id,
                                        const int64_t* sub_indptr,
+                                       const int64_t* col_span,
                                        int64_t* out_coo_col,
                                        int64_t* out_indices,
                                        int64_t* out_select,
@@ -245,6 +256,7 @@ int gs_csc_col_sample_uniform_fill_i32(const int64_t* indptr, int64_t num_cols,
  *    position, draw = output slot.
  *  out_coo_col, col_batch_ptr, num_col_batches: as for the uniform sampler
  *    above (the column's position in the call, or inside its batch).
+ *  col_span: as for the uniform sampler; read by the CDF form only.
  * Stands in for CSCColSamplingProbsCUDA (src/cuda/sampling_probs.cu:268-281).
  * ---------------------------------------------------------------------- */
 /* Persistent packed CDF of a matrix's edge weights, the input of the fast
@@ -273,8 +285,8 @@ int gs_csc_col_sample_weighted_fill(
     const int64_t* indptr, int64_t num_cols, const int64_t* indices,
     const float* probs, const int64_t* cdf, const int64_t* column_ids, int64_t num_items,
     int64_t fanout, int replace, uint64_t seed, uint64_t call_id,
-    const int64_t* sub_indptr, const int64_t* cdf_offsets, void* cdf_scratch,
-    int64_t* out_coo_col, int64_t* out_indices, int64_t* out_select,
+    const int64_t* sub_indptr, const int64_t* col_span, const int64_t* cdf_offsets,
+    void* cdf_scratch, int64_t* out_coo_col, int64_t* out_indices, int64_t* out_select,
     const int64_t* col_batch_ptr, int64_t num_col_batches, gs_stream_t stream);
 
 /* Evaluates the key arithmetic on the device: out2[0] = -log2((r64>>12)+1)/2^52),
@@ -696,7 +708,7 @@ int gs_e_div_u_sum(int format, const int64_t* a, const int64_t* b,
  *    column's lanes), 4 (column pointer not read: every column probe_degree
  *    long, outputs sized num_items * fanout), 8 (row ids not read), 16 (only
  *    the row id stored), 32 (nothing stored).  Built: 0, 1, 2, 4, 8, 24, 16,
- *    32, 40.
+ *    32, 40.  col_span (nullable) as for the sampler fills.
  * ---------------------------------------------------------------------- */
 int gs_probe_stream_copy(const void* src, void* dst, int64_t bytes, gs_stream_t stream);
 int gs_probe_line_gather(const void* table, int64_t table_bytes, int64_t num_picks,
@@ -705,7 +717,8 @@ int gs_probe_sample_uniform(
     const int64_t* indptr, int64_t num_cols, const int32_t* indices32,
     const int64_t* column_ids, int64_t num_items, int64_t fanout, int variant,
     int64_t probe_degree, uint64_t seed, uint64_t call_id, const int64_t* sub_indptr,
-    int64_t* out_coo_col, int64_t* out_indices, int64_t* out_select, gs_stream_t stream);
+    const int64_t* col_span, int64_t* out_coo_col, int64_t* out_indices, int64_t* out_select,
+    gs_stream_t stream);
 
 #ifdef __cplusplus
 }

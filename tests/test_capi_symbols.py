@@ -39,10 +39,10 @@ def test_argument_errors_are_reported_without_a_gpu():
     l = capi.lib()
     # negative fanout is rejected before any HIP call
     rc = l.gs_csc_col_sample_uniform_fill(None, 0, None, None, 0, -1, 0, 0, 0, 0,
-                                          None, None, None, None, None, 0, None)
+                                          None, None, None, None, None, None, 0, None)
     assert rc == 1 and b"fanout" in l.gs_last_error()
     rc = l.gs_csc_col_sample_uniform_fill(None, 0, None, None, 0, 100, 0, 2, 0, 0,
-                                          None, None, None, None, None, 0, None)
+                                          None, None, None, None, None, None, 0, None)
     assert rc == 1 and b"Floyd" in l.gs_last_error()
     rc = l.gs_unique_count(None, None, 0, None, None, 0, 0, None, None, None, 0, None)
     assert rc == 1

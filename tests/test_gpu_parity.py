@@ -505,7 +505,7 @@ def test_count_mirrors_in_pinned_host_memory():
         sub = torch.empty(n + 1, dtype=torch.int64, device=DEV)
         capi.check(l.gs_csc_col_count(d_indptr.data_ptr(), indptr.size - 1, d_cols.data_ptr(), n, 5, 0,
                                       sub.data_ptr(), mirror.data_ptr() if use_mirror else None,
-                                      ws.data_ptr(), ws.numel(), None))
+                                      None, ws.data_ptr(), ws.numel(), None))
         torch.cuda.synchronize()
         outs.append(sub.cpu().numpy())
     assert np.array_equal(outs[0], outs[1])
@@ -558,3 +558,46 @@ def test_outputs_that_are_only_8_byte_aligned(monkeypatch):
     assert by_pointer[2].data_ptr() % 16 == 8 and by_pointer[3].data_ptr() % 16 == 8
     assert_same(by_pointer, want)
     assert_same(capi.unique_relabel(T(seeds), T(rows), T(sp), T(rp), edge_col=T(edge_col)), want)
+
+
+@pytest.mark.parametrize("fanout,replace", [(5, False), (15, False), (3, True), (100, False)])
+def test_samplers_read_column_spans_left_by_the_count_pass(fanout, replace):
+    """The count pass can leave every column's start and degree in one word; the fill passes
+    that take it give the picks they give from the column pointer (oracle included), for
+    requested columns with repeats, empty columns and ids outside the matrix."""
+    rng = np.random.default_rng(fanout)
+    indptr, indices = random_csc(rng, 3000, 3000, 40)
+    cols = rng.integers(-2, 3004, size=5000)
+    args = (fanout, replace, 0, 11, 3)
+    with_spans = capi.sample_uniform(T(indptr), T(indices), T(cols), *args, spans=True)
+    without = capi.sample_uniform(T(indptr), T(indices), T(cols), *args, spans=False)
+    want = orc.sample_uniform(indptr, indices, cols, *args)
+    for a, b in zip(with_spans, without):
+        assert torch.equal(a, b)
+    assert_same(with_spans, want)
+    if fanout <= 64:
+        probs = rng.random(indices.size).astype(np.float32)
+        cdf = capi.weight_cdf(T(indptr), torch.as_tensor(probs, device=DEV), T(indices), 3000)
+        a = capi._sample_weighted_cdf(T(indptr), T(indices), cdf, T(cols), fanout, replace, 11, 3,
+                                      True, spans=True)
+        b = capi._sample_weighted_cdf(T(indptr), T(indices), cdf, T(cols), fanout, replace, 11, 3,
+                                      True, spans=False)
+        for x, y in zip(a, b):
+            assert torch.equal(x, y)
+
+
+def test_a_column_too_long_for_a_span_is_looked_up():
+    """Degrees from 2^24 - 1 on do not fit a span word: the count pass writes the look-up mark
+    and the fill pass reads the column pointer for that column, and only for it."""
+    long_deg = (1 << 24) + 5
+    indptr = np.array([0, 3, 3 + long_deg, 3 + long_deg + 4], dtype=np.int64)
+    rng = np.random.default_rng(1)
+    indices = rng.integers(0, 1000, size=int(indptr[-1]))
+    cols = np.array([1, 0, 2, 1], dtype=np.int64)
+    d_indptr, d_cols = T(indptr), T(cols)
+    span = torch.empty(4, dtype=torch.int64, device=DEV)
+    capi.col_count(d_indptr, d_cols, 5, False, col_span=span)
+    assert span.cpu().tolist() == [-1, 3 << 40, (4 << 40) | (3 + long_deg), -1]
+    got = capi.sample_uniform(d_indptr, T(indices), d_cols, 5, False, 0, 7, 1, spans=True)
+    want = orc.sample_uniform(indptr, indices, cols, 5, False, 0, 7, 1)
+    assert_same(got, want)
