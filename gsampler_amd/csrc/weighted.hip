@@ -392,6 +392,9 @@ __global__ __launch_bounds__(kBlock) void cdf_pack_kernel(
 // that last lowered `hi` stays at hand: when the search ends it is the entry
 // of the item found, row id included.
 constexpr int kInterpolations = 8;
+// Search mode of the CDF sampler: 0 bisection, 1 alternating, 2 interpolation
+// first (the fastest on prefix sums of real weights, which are nearly linear).
+constexpr int kCdfSearchMode = 2;
 struct CdfSearch {
   int64_t lo, hi;
   uint64_t a_lo, a_hi, x, e_hi;
@@ -408,7 +411,8 @@ struct CdfSearch {
     flip = true;
   }
   __device__ __forceinline__ bool done() const { return hi - lo <= 1; }
-  __device__ __forceinline__ int64_t probe_at(int mode) {
+  __device__ __forceinline__ int64_t probe_at() {
+    constexpr int mode = kCdfSearchMode;
     bool interpolate = false;
     if (hi - lo > 8) {
       if (mode == 1) interpolate = flip;
@@ -417,7 +421,9 @@ struct CdfSearch {
     flip = !flip;
     if (!interpolate) return (lo + hi) >> 1;
     ++guesses;
-    const double frac = (double)(x - a_lo) / (double)(a_hi - a_lo);
+    // (a guess: the hardware's approximate reciprocal will do, and where a probe
+    // lands never changes which item the search ends at)
+    const double frac = (double)(x - a_lo) * __builtin_amdgcn_rcp((double)(a_hi - a_lo));
     int64_t mid = lo + (int64_t)(frac * (double)(hi - lo));
     if (mid <= lo) mid = lo + 1;
     if (mid >= hi) mid = hi - 1;
@@ -441,10 +447,10 @@ struct CdfSearch {
 // looked at it (s.hi == deg).  `mass` is what the column's shares add up to.
 __device__ __forceinline__ void cdf_locate(CdfSearch& s, const uint64_t* __restrict__ col,
                                            int64_t deg, uint64_t mass, int row_bits,
-                                           uint64_t x, int mode) {
+                                           uint64_t x) {
   s.begin(deg, mass, x);
   while (!s.done()) {
-    const int64_t mid = s.probe_at(mode);
+    const int64_t mid = s.probe_at();
     s.narrow(mid, col[mid], row_bits);
   }
 }
@@ -475,7 +481,7 @@ __global__ __launch_bounds__(kBlock) void sample_weighted_cdf_kernel(
     int replace, PhiloxKey key, const int64_t* __restrict__ sub_indptr,
     int64_t* __restrict__ out_coo_col, int64_t* __restrict__ out_indices,
     int64_t* __restrict__ out_select, ColumnLabels labels,
-    const int64_t* __restrict__ col_span, int mode) {
+    const int64_t* __restrict__ col_span) {
   const int64_t item = (int64_t)blockIdx.x * kBlock + threadIdx.x;
   if (item >= num_items) return;
   // (asked for here, so that its loads travel with the ones below)
@@ -532,7 +538,7 @@ __global__ __launch_bounds__(kBlock) void sample_weighted_cdf_kernel(
     for (int j = 0; j < fanout; ++j) {
       if (mass) {
         cdf_locate(s, col, deg, full, row_bits,
-                   philox_bounded(key, (uint64_t)item, (uint64_t)j, full), mode);
+                   philox_bounded(key, (uint64_t)item, (uint64_t)j, full));
         if (s.hi == deg) {
           s.e_hi = col[deg];
           mass = (s.e_hi >> row_bits) != 0;
@@ -562,7 +568,7 @@ __global__ __launch_bounds__(kBlock) void sample_weighted_cdf_kernel(
         if (r + skipped == x) break;
         x = r + skipped;
       }
-      cdf_locate(s, col, deg, full, row_bits, x, mode);
+      cdf_locate(s, col, deg, full, row_bits, x);
       if (s.hi == deg) {  // ended at the last item without having read its entry
         s.e_hi = col[deg];
         if ((s.e_hi >> row_bits) == 0) break;  // a column without mass
@@ -610,10 +616,6 @@ __global__ __launch_bounds__(kBlock) void sample_weighted_cdf_kernel(
   }
 }
 
-// Search mode of the CDF sampler: 0 bisection, 1 alternating, 2 interpolation
-// first (the fastest on prefix sums of real weights, which are nearly linear).
-constexpr int kCdfSearchMode = 2;
-
 template <int KMAX>
 static int launch_weighted_cdf(const int64_t* indptr, int64_t num_cols,
                                const int64_t* indices, const int64_t* cdf,
@@ -627,7 +629,7 @@ static int launch_weighted_cdf(const int64_t* indptr, int64_t num_cols,
                                                dim3(kBlock), 0, s>>>(
                 indptr, num_cols, indices, (const uint64_t*)cdf, column_ids, num_items,
                 fanout, replace, key, sub_indptr, out_coo_col, out_indices, out_select, labels,
-                col_span, kCdfSearchMode));
+                col_span));
   return GS_OK;
 }
 
@@ -1245,8 +1247,16 @@ int gs_csc_col_sample_weighted_fill(
 #define GS_CDF_ARGS                                                              \
   indptr, num_cols, indices, cdf, column_ids, num_items, (int)fanout, replace, \
       key, sub_indptr, out_coo_col, out_indices, out_select, labels, col_span, s
+    // (every slot of the register arrays costs instructions in every draw whether it is
+    // used or not: the common fan-outs get arrays of their own size)
+    if (fanout <= 4) return launch_weighted_cdf<4>(GS_CDF_ARGS);
+    if (fanout == 5) return launch_weighted_cdf<5>(GS_CDF_ARGS);
     if (fanout <= 8) return launch_weighted_cdf<8>(GS_CDF_ARGS);
+    if (fanout <= 10) return launch_weighted_cdf<10>(GS_CDF_ARGS);
+    if (fanout <= 12) return launch_weighted_cdf<12>(GS_CDF_ARGS);
+    if (fanout <= 15) return launch_weighted_cdf<15>(GS_CDF_ARGS);
     if (fanout <= 16) return launch_weighted_cdf<16>(GS_CDF_ARGS);
+    if (fanout <= 24) return launch_weighted_cdf<24>(GS_CDF_ARGS);
     if (fanout <= 32) return launch_weighted_cdf<32>(GS_CDF_ARGS);
     return launch_weighted_cdf<64>(GS_CDF_ARGS);
 #undef GS_CDF_ARGS
