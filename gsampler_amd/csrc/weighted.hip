@@ -473,8 +473,11 @@ constexpr int kMaxCdfFanout = 64;
 // Streams: pos = column position, draw = output slot.
 // The taken intervals live in registers: every access runs over all KMAX slots
 // with a predicate instead of indexing.
+// (Fan-out 10 takes 134 registers left alone: capped at 128 it runs four wavefronts
+// per SIMD instead of three, 342 against 362 us on 592 K columns; the same cap for 15
+// and 16 spills more than it gains.)
 template <int KMAX>
-__global__ __launch_bounds__(kBlock) void sample_weighted_cdf_kernel(
+__global__ __launch_bounds__(kBlock, KMAX <= 10 ? 4 : 1) void sample_weighted_cdf_kernel(
     const int64_t* __restrict__ indptr, int64_t num_cols,
     const int64_t* __restrict__ indices, const uint64_t* __restrict__ cdf,
     const int64_t* __restrict__ column_ids, int64_t num_items, int fanout,
